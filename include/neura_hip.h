@@ -1,0 +1,186 @@
+/*
+ * neura_hip.h -- C ABI of libneura_hip.so: the MI355X (gfx950) implementation of the
+ * quantized-GGUF decoder path of formetaohy/Neura.
+ *
+ * The reference has no C ABI: the path sits behind its Rust crates neura-runtime /
+ * neura-gpu (dispatch), neura-decoder (model helpers) and neura-generate (generation loop).
+ * Each entry point below names the reference interface it stands in for, as path:line under
+ * the reference root.  A Rust `neura-hip-sys` crate binds these symbols one to one.
+ *
+ * Conventions
+ *   - every function that returns int32_t returns 0 on success and a negative NH_E_* code on
+ *     failure; nh_last_error() then returns a thread-local message.  The reference panics
+ *     with a prose message in the same situations (a binding turns the code into a panic).
+ *   - handles are opaque; one nh_device owns one HIP stream and is used from one thread at a
+ *     time (the reference's Runtime is used through `&mut Batch`, one thread).
+ *   - "dev" pointers are device memory of that nh_device; "host" pointers are caller memory.
+ *   - matrices are GGUF tensors in place: W is [N][K] row-major, K contiguous, stored as raw
+ *     ggml blocks (crates/neura-decoder/src/parameter.rs:5-15, crates/neura-runtime/src/store.rs:77-141).
+ *   - element ids are ggml type ids (crates/neura-gguf/src/header.rs:150-162).
+ *   - all work is enqueued on the device's stream; host-visible results are complete when the
+ *     call that returns them (nh_download, nh_decode_step, nh_timer_stop, nh_sync) returns.
+ */
+#ifndef NEURA_HIP_H
+#define NEURA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct nh_device nh_device;
+typedef struct nh_weights nh_weights;
+typedef struct nh_model nh_model;
+
+enum {
+    NH_F32 = 0,   /* Element::Single   */
+    NH_F16 = 1,   /* Element::Half     */
+    NH_Q8_0 = 8,  /* Element::Q8_0: 32 elements / 34 bytes  (crates/neura-abi/src/element.rs:155-158) */
+    NH_Q4_K = 12  /* Element::Q4K: 256 elements / 144 bytes (crates/neura-abi/src/element.rs:159-162) */
+};
+
+enum {
+    NH_OK = 0,
+    NH_E_ARGUMENT = -1, /* a shape, pointer or element the call cannot take */
+    NH_E_DEVICE = -2,   /* a HIP call failed (GpuUnavailable, crates/neura-runtime/src/runtime.rs:183) */
+    NH_E_MEMORY = -3,   /* device allocation failed */
+    NH_E_REFUSAL = -4   /* the device refused an index or origin (crates/neura-abi/src/refusal.rs:73-96) */
+};
+
+/* Epilogue of a product: the reference fuses these through `chained`
+ * (crates/neura-kernel/src/pointwise.rs:90-104). */
+typedef struct nh_epilogue {
+    const float *residual; /* dev, [rows][N] or NULL: y = residual + W·x (residual add, examples/qwen/mlp.rs:35) */
+    int32_t swiglu;        /* 1: W holds gate rows [0,N/2) then up rows [N/2,N); y[rows][N/2] = silu(gate)·up
+                              (examples/qwen/mlp.rs:31-33, crates/neura-pointwise/src/op.rs:163) */
+} nh_epilogue;
+
+/* ---- device, memory, timing : replaces crates/neura-gpu/src/native.rs:231-425 -------------- */
+
+/* Runtime::open (crates/neura-runtime/src/runtime.rs:183).  NULL when no usable gfx950 device. */
+nh_device *nh_open(int32_t device_index);
+void nh_close(nh_device *device);
+/* thread-local message of the last failed call on this thread ("" if none) */
+const char *nh_last_error(void);
+/* NativeDevice::create_buffer (crates/neura-gpu/src/native.rs:231); contents are zeroed */
+void *nh_alloc(nh_device *device, size_t bytes);
+int32_t nh_free(nh_device *device, void *dev);
+/* NativeDevice::write_host / read_host (crates/neura-gpu/src/native.rs:231-425); both are
+ * complete on return */
+int32_t nh_upload(nh_device *device, void *dev_dst, const void *host_src, size_t bytes);
+int32_t nh_download(nh_device *device, void *host_dst, const void *dev_src, size_t bytes);
+/* Command::Clear (crates/neura-gpu/src/submission.rs:17-35) */
+int32_t nh_clear(nh_device *device, void *dev, size_t bytes);
+/* NativeDevice::wait (crates/neura-gpu/src/native.rs:231-425) */
+int32_t nh_sync(nh_device *device);
+/* Run::seconds (crates/neura-runtime/src/runtime.rs:130-135): device time between the two
+ * calls, taken with HIP events on the device's own stream */
+int32_t nh_timer_start(nh_device *device);
+int32_t nh_timer_stop(nh_device *device, double *seconds_out);
+
+/* ---- weight arena : replaces Runtime::load (crates/neura-runtime/src/runtime.rs:356-367) ---- */
+
+/* one arena of `bytes`; tensors are poured verbatim at 256-byte aligned offsets the caller
+ * picks (crates/neura-plan/src/layout.rs:29-36) */
+nh_weights *nh_weights_create(nh_device *device, size_t bytes);
+void nh_weights_destroy(nh_weights *weights);
+/* pour_one (crates/neura-runtime/src/store.rs:77-141): raw ggml bytes, no repacking */
+int32_t nh_weights_put(nh_weights *weights, size_t at, const void *host_bytes, size_t bytes);
+/* device address of arena offset `at` */
+void *nh_weights_at(nh_weights *weights, size_t at);
+size_t nh_weights_bytes(const nh_weights *weights);
+
+/* ---- operators : replace the run_<kind> bodies of crates/neura-kernel ---------------------- */
+
+/* fetch_q8_0 / fetch_q4_k / fetch_half (crates/neura-kernel/src/fetch.rs:236-267, :95-98) ==
+ * unpack (crates/neura-precision/src/ggml.rs:211-216, :336-350): bit-exact fp32 values */
+int32_t nh_dequant(nh_device *device, int32_t element, const void *dev_src, uint64_t elements, float *dev_dst);
+/* run_convert_half (crates/neura-kernel/src/task/convert.rs:229-249): fp32 -> fp16 RNE */
+int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elements, uint16_t *dev_dst);
+/* narrow product, rows <= 8 (template_run_matmul_folded{,_fused,_quad},
+ * crates/neura-kernel/src/task/matmul.rs:376-803): y[r][n] = sum_k x[r][k]·W[n][k], fp32 */
+int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
+                float *dev_y, const nh_epilogue *epilogue);
+/* wide product (template_run_matmul_codes / _run, crates/neura-kernel/src/task/matmul.rs:943-1221):
+ * X [M][K] in x_element (NH_F32 or NH_F16), Y fp32 [M][N] */
+int32_t nh_gemm(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const void *dev_X, int32_t x_element,
+                uint32_t M, float *dev_Y, const nh_epilogue *epilogue);
+/* run_norm NORM_RMS (crates/neura-kernel/src/task/norm.rs:55-130, :350-369):
+ * v = x (+ residual); out = v / sqrt(mean(v^2) + eps) * w.  sum_out (may be NULL) receives v. */
+int32_t nh_rmsnorm(nh_device *device, const float *dev_x, const float *dev_residual, const float *dev_w, float eps, uint32_t rows,
+                   uint32_t C, float *dev_out, float *dev_sum_out);
+/* run_rope (crates/neura-kernel/src/task/rope.rs:52-123): rotate-half over all `width`
+ * channels of x [planes][batch][rows][width]; position = cursor[plane of batch] + row */
+int32_t nh_rope(nh_device *device, const float *dev_x, uint32_t planes, uint32_t batch, uint32_t rows, uint32_t width,
+                const uint32_t *dev_cursor, float base, float *dev_out);
+/* Cache::write / write_masked (crates/neura-decoder/src/cache.rs:267-352): cast to fp16 then
+ * scatter rows.  k, v are fp32 [kv_heads][batch][rows][width]; the caches are fp16
+ * [kv_heads][batch][capacity][width]; row index = cursor[b] + row, or window + row for a
+ * plane whose dev_mask byte is 0 (dev_mask may be NULL = all active). */
+int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v, uint16_t *dev_cache_k, uint16_t *dev_cache_v,
+                       uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
+                       const uint32_t *dev_cursor, const uint8_t *dev_mask);
+/* Cache::attend -> run_attention (+ run_attention_fold) (crates/neura-decoder/src/cache.rs:366-406,
+ * crates/neura-kernel/src/task/attention.rs:309-671): causal GQA attention of q
+ * [heads][batch][rows][width] over fp16 caches [kv_heads][batch][capacity][width], the first
+ * `keys` rows visible; key `at` is weighed iff at <= cursor[b] + row.  out like q. */
+int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
+                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                     const uint32_t *dev_cursor, float scale, float *dev_out);
+/* run_gather (crates/neura-kernel/src/task/select.rs:29-49): out[t][:] = dequant(table[token[t]]),
+ * times mask[t % batch] when dev_mask != NULL.  A token id >= vocab is refused. */
+int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uint32_t vocab, uint32_t width, const uint32_t *dev_tokens,
+                  uint32_t count, uint32_t batch, const uint8_t *dev_mask, float *dev_out);
+/* run_argmax (crates/neura-kernel/src/task/choice.rs:355-368): per row, lowest index wins ties */
+int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out);
+
+/* ---- decoder model : replaces the compiled answer / fill programs of Batch ------------------ */
+
+/* Qwen2-style decoder (composition of examples/qwen/model.rs:92-103, attention.rs:98-154,
+ * mlp.rs:29-36 without the qwen35 q-gate and q/k norms). */
+typedef struct nh_model_config {
+    uint32_t layers, hidden, heads, kv_heads, head_dim, ffn, vocab;
+    uint32_t context;    /* BatchSpec.context */
+    uint32_t batch;      /* BatchSpec.batch (planes) */
+    uint32_t max_rows;   /* widest fill chunk (BatchSpec.chunks[0]), 1 if none */
+    float rope_base;     /* <arch>.rope.freq_base */
+    float eps;           /* <arch>.attention.layer_norm_rms_epsilon */
+} nh_model_config;
+
+/* where each tensor sits in the arena (byte offsets) and its element.  Per layer arrays have
+ * `layers` entries.  output == UINT64_MAX ties the head to token_embd (examples/qwen/model.rs:81-84). */
+typedef struct nh_tensor_table {
+    int32_t matrix_element; /* element of every matrix: NH_Q8_0, NH_Q4_K (or NH_F16 / NH_F32) */
+    uint64_t token_embd, output, output_norm;
+    const uint64_t *attn_norm, *attn_q, *attn_k, *attn_v, *attn_output, *ffn_norm, *ffn_gate, *ffn_up, *ffn_down;
+} nh_tensor_table;
+
+/* Batch::new (crates/neura-generate/src/batch.rs:279-465): allocates fp16 K/V caches of
+ * capacity = context + max_rows per (layer, kv head, plane) and every activation buffer. */
+nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_weights *weights, const nh_tensor_table *table);
+void nh_model_destroy(nh_model *model);
+/* the answer program (crates/neura-generate/src/batch.rs:1716-1725): one token per plane.
+ * host arrays of `batch` entries; mask 0 = inactive plane.  chosen_out[b] = argmax of the logits. */
+int32_t nh_decode_step(nh_model *model, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                       uint32_t *chosen_out);
+/* a fill program (crates/neura-generate/src/batch.rs:1434-1517): `rows` tokens per plane,
+ * tokens[row * batch + plane]; no logits, no readback. */
+int32_t nh_prefill(nh_model *model, const uint32_t *tokens, uint32_t rows, const uint32_t *cursors, const uint8_t *mask, uint32_t batch);
+/* the reset program (crates/neura-generate/src/batch.rs:1094-1100): zero the caches of planes
+ * whose reset byte is non-zero */
+int32_t nh_model_reset(nh_model *model, const uint8_t *reset, uint32_t batch);
+/* Runtime::read of the logits value (crates/neura-runtime/src/runtime.rs:1064-1067): logits of
+ * the last decode step, [batch][vocab] */
+int32_t nh_model_logits(nh_model *model, float *host_out);
+/* Runtime::restore_state / save_state of "blk.{i}.cache.key|value"
+ * (crates/neura-decoder/src/cache.rs:135-137): raw fp16 [kv_heads][batch][capacity][head_dim] */
+int32_t nh_model_cache_write(nh_model *model, uint32_t layer, int32_t value_not_key, const uint16_t *host_src);
+int32_t nh_model_cache_read(nh_model *model, uint32_t layer, int32_t value_not_key, uint16_t *host_dst);
+uint32_t nh_model_capacity(const nh_model *model);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NEURA_HIP_H */

@@ -1,0 +1,56 @@
+"""Builds libneura_hip.so (gfx950 only) in-tree with hipcc.
+
+    python -m neura_amd.build          # compile every .hip file and link
+
+-ffp-contract=off: every fused multiply-add in the kernels is written as fmaf(); plain
+a*b+c stays two roundings, which the bit-exact dequantisation and the norm's sum of squares
+depend on.  Packed fp32 arithmetic is switched off for the device pass.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIBRARY = os.path.join(HERE, "libneura_hip.so")
+SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "model.hip"]
+FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+]
+
+
+def hipcc():
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(source):
+    obj = os.path.join(CSRC, source.replace(".hip", ".o"))
+    cmd = [hipcc(), *FLAGS, "-c", os.path.join(CSRC, source), "-o", obj]
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s\n%s" % (source, " ".join(cmd), done.stderr))
+    noise = "'-packed-fp32-ops' is not a recognized feature"
+    warnings = "\n".join(line for line in done.stderr.splitlines() if noise not in line)
+    return obj, warnings
+
+
+def build_library(verbose=True):
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        results = list(pool.map(_compile, SOURCES))
+    objects = [obj for obj, _ in results]
+    if verbose:
+        for source, (_, warnings) in zip(SOURCES, results):
+            if warnings.strip():
+                print("[%s]\n%s" % (source, warnings), file=sys.stderr)
+    cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIBRARY, *objects]
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError("link failed:\n%s\n%s" % (" ".join(cmd), done.stderr))
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    print(build_library())

@@ -1,0 +1,86 @@
+// Greedy choice: per row the largest value, the lowest index on ties
+// (crates/neura-kernel/src/task/choice.rs:46-51, :355-368; sectioned + fold :331-353).
+#include "common.hpp"
+
+namespace nh {
+
+__device__ __forceinline__ bool precedes(float value, uint32_t index, float other_value, uint32_t other_index) {
+    // true when (other_value, other_index) beats (value, index)
+    return other_value > value || (other_value == value && other_index < index);
+}
+
+__device__ __forceinline__ void wave_choice(float &value, uint32_t &index) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        float other_value = __shfl_xor(value, offset, 64);
+        uint32_t other_index = __shfl_xor(index, offset, 64);
+        if (precedes(value, index, other_value, other_index)) value = other_value, index = other_index;
+    }
+}
+
+__device__ void block_choice(float &value, uint32_t &index, float *values, uint32_t *indices) {
+    wave_choice(value, index);
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    if (lane == 0) values[wave] = value, indices[wave] = index;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < blockDim.x / 64; w++)
+            if (precedes(value, index, values[w], indices[w])) value = values[w], index = indices[w];
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_sections_kernel(const float *__restrict__ values, uint32_t n, uint32_t sections,
+                                                              float *__restrict__ best_values, uint32_t *__restrict__ best_indices) {
+    __shared__ float held_values[4];
+    __shared__ uint32_t held_indices[4];
+    const uint32_t row = blockIdx.y, section = blockIdx.x;
+    const uint32_t chunk = (n + sections - 1) / sections;
+    const uint32_t first = section * chunk, last = min(n, first + chunk);
+    const float *src = values + (size_t)row * n;
+    float value = -INFINITY;
+    uint32_t index = first < n ? first : 0u;
+    for (uint32_t i = first + threadIdx.x; i < last; i += 256) {
+        float held = src[i];
+        if (precedes(value, index, held, i)) value = held, index = i;
+    }
+    block_choice(value, index, held_values, held_indices);
+    if (threadIdx.x == 0) {
+        best_values[(size_t)row * sections + section] = value;
+        best_indices[(size_t)row * sections + section] = index;
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_fold_kernel(const float *__restrict__ best_values, const uint32_t *__restrict__ best_indices,
+                                                          uint32_t sections, uint32_t *__restrict__ out) {
+    __shared__ float held_values[4];
+    __shared__ uint32_t held_indices[4];
+    const uint32_t row = blockIdx.x;
+    float value = -INFINITY;
+    uint32_t index = 0xffffffffu;
+    for (uint32_t s = threadIdx.x; s < sections; s += 256) {
+        float held = best_values[(size_t)row * sections + s];
+        uint32_t at = best_indices[(size_t)row * sections + s];
+        if (index == 0xffffffffu || precedes(value, index, held, at)) value = held, index = at;
+    }
+    block_choice(value, index, held_values, held_indices);
+    if (threadIdx.x == 0) out[row] = index == 0xffffffffu ? 0u : index;
+}
+
+int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out) {
+    if (!rows) return NH_OK;
+    uint32_t sections = (n + 2047) / 2048;
+    if (sections < 1) sections = 1;
+    if (sections > 1024) sections = 1024;
+    size_t bytes = (size_t)rows * sections * (sizeof(float) + sizeof(uint32_t));
+    uint8_t *held = static_cast<uint8_t *>(scratch(d, bytes));
+    if (!held) return NH_E_MEMORY;
+    float *best_values = reinterpret_cast<float *>(held);
+    uint32_t *best_indices = reinterpret_cast<uint32_t *>(held + (size_t)rows * sections * sizeof(float));
+    hipLaunchKernelGGL(argmax_sections_kernel, dim3(sections, rows), dim3(256), 0, d->stream, values, n, sections, best_values, best_indices);
+    NH_HIP(hipGetLastError());
+    hipLaunchKernelGGL(argmax_fold_kernel, dim3(rows), dim3(256), 0, d->stream, best_values, best_indices, sections, out);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+}  // namespace nh

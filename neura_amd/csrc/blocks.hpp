@@ -1,0 +1,68 @@
+// Device-side readers of raw ggml blocks and fp16 helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace nh {
+
+__device__ __forceinline__ float half_to_float(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);  // exact
+}
+
+// fp32 -> fp16, round to nearest even, subnormals kept, NaN -> sign|0x7e00
+// (crates/neura-kernel/src/task/convert.rs:57-84)
+__device__ __forceinline__ uint16_t float_to_half(float value) {
+    uint32_t bits = __builtin_bit_cast(uint32_t, value);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) return (uint16_t)(((bits >> 16) & 0x8000u) | 0x7e00u);
+    return __builtin_bit_cast(uint16_t, (_Float16)value);
+}
+
+__device__ __forceinline__ uint16_t load_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
+
+// 6-bit scale and min `j` (0..7) of a Q4_K super-block from its 12 scale bytes
+// (crates/neura-precision/src/ggml.rs:127-136)
+__device__ __forceinline__ void scale_min_k4(const uint8_t *s, uint32_t j, uint32_t &scale, uint32_t &min) {
+    if (j < 4) {
+        scale = s[j] & 63u;
+        min = s[j + 4] & 63u;
+    } else {
+        scale = (uint32_t)(s[j + 4] & 0x0fu) | ((uint32_t)(s[j - 4] >> 6) << 4);
+        min = (uint32_t)(s[j + 4] >> 4) | ((uint32_t)(s[j] >> 6) << 4);
+    }
+}
+
+// element `i` of a row of Q8_0 blocks (crates/neura-precision/src/ggml.rs:211-216)
+__device__ __forceinline__ float q8_0_element(const uint8_t *row, uint64_t i) {
+    const uint8_t *block = row + (i / 32) * 34;
+    float quantum = half_to_float(load_u16(block));
+    return (float)(int8_t)block[2 + (i % 32)] * quantum;
+}
+
+// element `i` of a row of Q4_K blocks (crates/neura-precision/src/ggml.rs:336-350): the product
+// scale*code and the product min*offset are each rounded before the subtract
+__device__ __forceinline__ float q4_k_element(const uint8_t *row, uint64_t i) {
+    const uint8_t *block = row + (i / 256) * 144;
+    uint32_t within = (uint32_t)(i % 256);
+    uint32_t group = within / 64, seat = (within % 64) / 32, lane = within % 32;
+    uint32_t code, offset;
+    scale_min_k4(block + 4, group * 2 + seat, code, offset);
+    float quantum = __fmul_rn(half_to_float(load_u16(block)), (float)code);
+    float low = __fmul_rn(half_to_float(load_u16(block + 2)), (float)offset);
+    uint8_t byte = block[16 + group * 32 + lane];
+    uint32_t quant = seat ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f);
+    return __fsub_rn(__fmul_rn(quantum, (float)quant), low);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, 64));
+    return v;
+}
+
+}  // namespace nh

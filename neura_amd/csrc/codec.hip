@@ -1,0 +1,115 @@
+// Element-wise readers: bit-exact dequantisation of raw ggml blocks, fp32 -> fp16 conversion
+// and the embedding gather.  Compiled with -ffp-contract=off: the reference rounds every
+// product before the next operation.
+#include "blocks.hpp"
+#include "common.hpp"
+
+namespace nh {
+
+template <int ELEMENT>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ src, uint64_t elements, float *__restrict__ dst) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < elements; i += (uint64_t)gridDim.x * blockDim.x) {
+        float value;
+        if (ELEMENT == NH_Q8_0)
+            value = q8_0_element(src, i);
+        else if (ELEMENT == NH_Q4_K)
+            value = q4_k_element(src, i);
+        else if (ELEMENT == NH_F16)
+            value = half_to_float(reinterpret_cast<const uint16_t *>(src)[i]);
+        else
+            value = reinterpret_cast<const float *>(src)[i];
+        dst[i] = value;
+    }
+}
+
+static uint32_t grid_for(nh_device *d, uint64_t items, uint32_t block) {
+    uint64_t wanted = (items + block - 1) / block;
+    uint64_t most = (uint64_t)d->compute_units * 16;
+    return (uint32_t)(wanted < 1 ? 1 : (wanted > most ? most : wanted));
+}
+
+int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t elements, float *dst) {
+    if (!elements) return NH_OK;
+    uint32_t grid = grid_for(d, elements, 256);
+    const uint8_t *bytes = static_cast<const uint8_t *>(src);
+    switch (element) {
+    case NH_Q8_0: hipLaunchKernelGGL(dequant_kernel<NH_Q8_0>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_Q4_K: hipLaunchKernelGGL(dequant_kernel<NH_Q4_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_F16: hipLaunchKernelGGL(dequant_kernel<NH_F16>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_F32: hipLaunchKernelGGL(dequant_kernel<NH_F32>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    default: return fail(NH_E_ARGUMENT, "element %d carries no reader", element);
+    }
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+__global__ __launch_bounds__(256) void convert_half_kernel(const float *__restrict__ src, uint64_t elements, uint16_t *__restrict__ dst) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < elements; i += (uint64_t)gridDim.x * blockDim.x)
+        dst[i] = float_to_half(src[i]);
+}
+
+int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, uint16_t *dst) {
+    if (!elements) return NH_OK;
+    hipLaunchKernelGGL(convert_half_kernel, dim3(grid_for(d, elements, 256)), dim3(256), 0, d->stream, src, elements, dst);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// out[t][c] = dequant(table[token[t]])[c] * mask[t % batch]   (crates/neura-kernel/src/task/select.rs:29-49,
+// examples/qwen/model.rs:94).  One workgroup per token row.
+template <int ELEMENT>
+__global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__ table, uint32_t vocab, uint32_t width, uint64_t row_bytes,
+                                                     const uint32_t *__restrict__ tokens, uint32_t batch,
+                                                     const uint8_t *__restrict__ mask, float *__restrict__ out, uint32_t *refusal) {
+    uint32_t t = blockIdx.x;
+    uint32_t token = tokens[t];
+    float keep = (mask == nullptr || mask[t % batch]) ? 1.0f : 0.0f;
+    if (token >= vocab) {
+        if (threadIdx.x == 0) atomicMax(refusal, (uint32_t)REFUSAL_INDEX);
+        for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) out[(uint64_t)t * width + c] = 0.0f;
+        return;
+    }
+    const uint8_t *row = table + (uint64_t)token * row_bytes;
+    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+        float value;
+        if (ELEMENT == NH_Q8_0)
+            value = q8_0_element(row, c);
+        else if (ELEMENT == NH_Q4_K)
+            value = q4_k_element(row, c);
+        else if (ELEMENT == NH_F16)
+            value = half_to_float(reinterpret_cast<const uint16_t *>(row)[c]);
+        else
+            value = reinterpret_cast<const float *>(row)[c];
+        out[(uint64_t)t * width + c] = value * keep;
+    }
+}
+
+int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
+                      uint32_t count, uint32_t batch, const uint8_t *mask, float *out) {
+    if (!count) return NH_OK;
+    const uint8_t *bytes = static_cast<const uint8_t *>(table);
+    uint64_t row_bytes = payload_bytes(element, width);
+    switch (element) {
+    case NH_Q8_0:
+        hipLaunchKernelGGL(gather_kernel<NH_Q8_0>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_Q4_K:
+        hipLaunchKernelGGL(gather_kernel<NH_Q4_K>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_F16:
+        hipLaunchKernelGGL(gather_kernel<NH_F16>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_F32:
+        hipLaunchKernelGGL(gather_kernel<NH_F32>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    default: return fail(NH_E_ARGUMENT, "element %d carries no reader", element);
+    }
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+}  // namespace nh

@@ -1,0 +1,145 @@
+// Shared declarations of libneura_hip.so: the device handle, error reporting and the
+// launcher prototypes each kernel file exports to the C ABI layer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/neura_hip.h"
+
+namespace nh {
+
+constexpr uint32_t Q8_0_BLOCK = 32, Q8_0_BYTES = 34;
+constexpr uint32_t Q4_K_BLOCK = 256, Q4_K_BYTES = 144;
+constexpr uint32_t WAVE = 64;
+
+int32_t fail(int32_t code, const char *format, ...) __attribute__((format(printf, 2, 3)));
+int32_t hip_fail(hipError_t error, const char *what);
+
+#define NH_HIP(call)                                              \
+    do {                                                          \
+        hipError_t nh_hip_error_ = (call);                        \
+        if (nh_hip_error_ != hipSuccess) return ::nh::hip_fail(nh_hip_error_, #call); \
+    } while (0)
+
+#define NH_REQUIRE(condition, ...)                                \
+    do {                                                          \
+        if (!(condition)) return ::nh::fail(NH_E_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+inline uint64_t payload_bytes(int32_t element, uint64_t elements) {
+    switch (element) {
+    case NH_Q8_0: return (elements + Q8_0_BLOCK - 1) / Q8_0_BLOCK * Q8_0_BYTES;
+    case NH_Q4_K: return (elements + Q4_K_BLOCK - 1) / Q4_K_BLOCK * Q4_K_BYTES;
+    case NH_F16: return elements * 2;
+    case NH_F32: return elements * 4;
+    default: return 0;
+    }
+}
+
+inline uint32_t block_elements(int32_t element) {
+    switch (element) {
+    case NH_Q8_0: return Q8_0_BLOCK;
+    case NH_Q4_K: return Q4_K_BLOCK;
+    case NH_F16:
+    case NH_F32: return 1;
+    default: return 0;
+    }
+}
+
+}  // namespace nh
+
+// One device = one HIP stream, a pair of timing events and a few scratch buffers that
+// grow on demand (split-K / split-context partials, argmax partials, the refusal word).
+struct nh_device {
+    int32_t index = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t started = nullptr, stopped = nullptr;
+    int32_t compute_units = 0;
+    void *scratch = nullptr;  // device scratch, `scratch_bytes` long
+    size_t scratch_bytes = 0;
+    uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
+    float *rope_table = nullptr;  // device inverse frequencies of the last (base, width)
+    float rope_base = 0.0f;
+    uint32_t rope_width = 0;
+};
+
+namespace nh {
+
+// grows the device scratch to at least `bytes`; returns nullptr on failure (error recorded)
+void *scratch(nh_device *device, size_t bytes);
+// device table of pow(base, -2c/width), c < width/2, computed on the host in fp32
+const float *rope_frequencies(nh_device *device, float base, uint32_t width);
+// reads and clears the refusal word; returns NH_OK or NH_E_REFUSAL with a message
+int32_t check_refusal(nh_device *device, const char *what);
+
+enum Refusal : uint32_t { REFUSAL_NONE = 0, REFUSAL_INDEX = 1, REFUSAL_ORIGIN = 2 };
+
+// ---- launchers (each validates nothing: the C ABI layer checks shapes first) ----
+int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t elements, float *dst);
+int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, uint16_t *dst);
+
+struct GemvArgs {
+    int32_t element;
+    const void *W[3];  // up to three matrices stacked along N; unused entries are nullptr
+    uint32_t end[3];   // first output row past each matrix (end[2] == N); with swiglu W[0] = gate, W[1] = up
+    uint32_t N, K;
+    const float *x;    // [rows][K]
+    uint32_t rows;
+    float *y;          // [rows][N] (or [rows][N/2] with swiglu)
+    const float *residual;
+    int32_t swiglu;
+    // optional fused RMSNorm of x: x' = x / sqrt(mean(x^2)+eps) * norm_w
+    const float *norm_w;
+    float eps;
+};
+int32_t launch_gemv(nh_device *d, const GemvArgs &args);
+
+struct GemmArgs {
+    int32_t element;
+    const void *W;
+    uint32_t N, K;
+    const void *X;  // [M][K]
+    int32_t x_element;
+    uint32_t M;
+    float *Y;                // [M][ldy], the first N of every row are written
+    const float *residual;   // [M][ldy] or nullptr
+    uint32_t ldy;
+};
+int32_t launch_gemm(nh_device *d, const GemmArgs &args);
+
+int32_t launch_rmsnorm(nh_device *d, const float *x, const float *residual, const float *w, float eps, uint32_t rows, uint32_t C,
+                       float *out, float *sum_out);
+int32_t launch_rope(nh_device *d, const float *x, uint32_t planes, uint32_t batch, uint32_t rows, uint32_t width,
+                    const uint32_t *cursor, float base, float *out);
+int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
+                           uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask);
+
+// q / out addressing: element (head, plane, row, c) at head*sh + plane*sb + row*sr + c
+struct AttentionArgs {
+    const float *q;
+    float *out;
+    uint64_t q_sh, q_sb, q_sr, o_sh, o_sb, o_sr;
+    const uint16_t *cache_k, *cache_v;
+    uint32_t heads, kv_heads, batch, rows, width, capacity, keys;
+    const uint32_t *cursor;
+    float scale;
+};
+int32_t launch_attention(nh_device *d, const AttentionArgs &args);
+
+// fused decode-side step: rope(q,k) + fp16 cache append from a token-major qkv buffer
+// qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane; q is roped in place.
+int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
+                           uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask, float base);
+
+int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
+                      uint32_t count, uint32_t batch, const uint8_t *mask, float *out);
+int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);
+int32_t launch_silu_mul(nh_device *d, const float *gate, const float *up, uint64_t n, float *out);
+int32_t launch_mask_rows(nh_device *d, float *x, uint32_t rows, uint32_t batch, uint32_t width, const uint8_t *mask);
+
+}  // namespace nh

@@ -1,0 +1,461 @@
+// The decoder: the hand-scheduled kernel sequence that stands where the reference compiles
+// its answer / fill / reset programs, and the C ABI operator entry points.
+#include "common.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+using namespace nh;
+
+struct nh_model {
+    nh_device *d = nullptr;
+    nh_weights *weights = nullptr;
+    nh_model_config c{};
+    int32_t element = 0;
+    uint32_t capacity = 0, window = 0;
+    const uint8_t *token_embd = nullptr, *output = nullptr;
+    const float *output_norm = nullptr;
+    std::vector<const float *> attn_norm, ffn_norm;
+    std::vector<const uint8_t *> attn_q, attn_k, attn_v, attn_o, ffn_gate, ffn_up, ffn_down;
+    std::vector<uint16_t *> cache_k, cache_v;
+    size_t cache_elements = 0;  // per layer and per K or V
+    // activations; T = rows * batch flattened token rows, t = row * batch + plane
+    float *h = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr, *act = nullptr, *up = nullptr, *logits = nullptr;
+    uint32_t *inputs_dev = nullptr;  // [tokens T_max | cursors B | mask bytes B]
+    uint32_t *chosen_dev = nullptr;
+    uint8_t *inputs_host = nullptr;  // pinned mirror of inputs_dev
+    uint32_t *chosen_host = nullptr; // pinned [B + 1]: chosen tokens, then the refusal word
+    uint32_t max_tokens = 0;
+};
+
+namespace {
+
+uint32_t qkv_width(const nh_model *m) { return (m->c.heads + 2 * m->c.kv_heads) * m->c.head_dim; }
+
+void release(nh_model *m) {
+    if (!m) return;
+    (void)hipStreamSynchronize(m->d->stream);
+    for (auto p : m->cache_k) (void)hipFree(p);
+    for (auto p : m->cache_v) (void)hipFree(p);
+    float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits};
+    for (float *p : buffers)
+        if (p) (void)hipFree(p);
+    if (m->inputs_dev) (void)hipFree(m->inputs_dev);
+    if (m->chosen_dev) (void)hipFree(m->chosen_dev);
+    if (m->inputs_host) (void)hipHostFree(m->inputs_host);
+    if (m->chosen_host) (void)hipHostFree(m->chosen_host);
+    delete m;
+}
+
+template <typename T>
+bool device_array(T *&out, size_t count) {
+    void *held = nullptr;
+    if (hipMalloc(&held, (count ? count : 1) * sizeof(T)) != hipSuccess) return false;
+    out = static_cast<T *>(held);
+    return true;
+}
+
+// writes tokens / cursors / mask through the pinned staging buffer in one copy
+int32_t stage_inputs(nh_model *m, const uint32_t *tokens, uint32_t count, const uint32_t *cursors, const uint8_t *mask, uint32_t batch) {
+    uint32_t *words = reinterpret_cast<uint32_t *>(m->inputs_host);
+    memcpy(words, tokens, (size_t)count * 4);
+    memcpy(words + m->max_tokens, cursors, (size_t)batch * 4);
+    uint8_t *mask_bytes = reinterpret_cast<uint8_t *>(words + m->max_tokens + batch);
+    for (uint32_t b = 0; b < batch; b++) mask_bytes[b] = mask ? (mask[b] ? 1 : 0) : 1;
+    size_t bytes = ((size_t)m->max_tokens + batch) * 4 + batch;
+    NH_HIP(hipMemcpyAsync(m->inputs_dev, m->inputs_host, bytes, hipMemcpyHostToDevice, m->d->stream));
+    return NH_OK;
+}
+
+const uint32_t *dev_tokens(const nh_model *m) { return m->inputs_dev; }
+const uint32_t *dev_cursor(const nh_model *m) { return m->inputs_dev + m->max_tokens; }
+const uint8_t *dev_mask(const nh_model *m) { return reinterpret_cast<const uint8_t *>(m->inputs_dev + m->max_tokens + m->c.batch); }
+
+GemvArgs narrow(const nh_model *m, const uint8_t *W, uint32_t N, uint32_t K, const float *x, uint32_t rows, float *y) {
+    GemvArgs a{};
+    a.element = m->element;
+    a.W[0] = W, a.W[1] = nullptr, a.W[2] = nullptr;
+    a.end[0] = a.end[1] = a.end[2] = N;
+    a.N = N, a.K = K, a.x = x, a.rows = rows, a.y = y;
+    return a;
+}
+
+// all layers over T = rows * batch token rows whose inputs are already staged on the device
+int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
+    nh_device *d = m->d;
+    const nh_model_config &c = m->c;
+    const uint32_t B = c.batch, T = rows * B, H = c.hidden, hd = c.head_dim;
+    const uint32_t QW = c.heads * hd, KW = c.kv_heads * hd, QKV = QW + 2 * KW, F = c.ffn;
+    const uint8_t *mask = any_inactive ? dev_mask(m) : nullptr;
+    const bool wide = T > 8;  // more rows than the narrow product takes
+    int32_t status;
+    if ((status = launch_gather(d, m->element, m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK) return status;
+    const float scale = 1.0f / sqrtf((float)hd);
+    for (uint32_t L = 0; L < c.layers; L++) {
+        if (wide) {
+            if ((status = launch_rmsnorm(d, m->h, nullptr, m->attn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
+            const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
+            const uint32_t widths[3] = {QW, KW, KW};
+            uint32_t column = 0;
+            for (int s = 0; s < 3; s++) {
+                GemmArgs g{m->element, mats[s], widths[s], H, m->xn, NH_F32, T, m->qkv + column, nullptr, QKV};
+                if ((status = launch_gemm(d, g)) != NH_OK) return status;
+                column += widths[s];
+            }
+        } else {
+            GemvArgs a = narrow(m, m->attn_q[L], QKV, H, m->h, T, m->qkv);
+            a.W[1] = m->attn_k[L], a.W[2] = m->attn_v[L];
+            a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
+            a.norm_w = m->attn_norm[L], a.eps = c.eps;
+            if ((status = launch_gemv(d, a)) != NH_OK) return status;
+        }
+        if ((status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L], m->capacity, m->window,
+                                         dev_cursor(m), mask, c.rope_base)) != NH_OK)
+            return status;
+        AttentionArgs at{};
+        at.q = m->qkv, at.out = m->att;
+        at.q_sh = hd, at.q_sb = QKV, at.q_sr = (uint64_t)B * QKV;
+        at.o_sh = hd, at.o_sb = QW, at.o_sr = (uint64_t)B * QW;
+        at.cache_k = m->cache_k[L], at.cache_v = m->cache_v[L];
+        at.heads = c.heads, at.kv_heads = c.kv_heads, at.batch = B, at.rows = rows, at.width = hd;
+        at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
+        if ((status = launch_attention(d, at)) != NH_OK) return status;
+        if (wide) {
+            GemmArgs o{m->element, m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
+            if ((status = launch_gemm(d, o)) != NH_OK) return status;
+            if ((status = launch_rmsnorm(d, m->h, nullptr, m->ffn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
+            GemmArgs g{m->element, m->ffn_gate[L], F, H, m->xn, NH_F32, T, m->act, nullptr, F};
+            GemmArgs u{m->element, m->ffn_up[L], F, H, m->xn, NH_F32, T, m->up, nullptr, F};
+            if ((status = launch_gemm(d, g)) != NH_OK) return status;
+            if ((status = launch_gemm(d, u)) != NH_OK) return status;
+            if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
+            GemmArgs dn{m->element, m->ffn_down[L], H, F, m->act, NH_F32, T, m->h, m->h, H};
+            if ((status = launch_gemm(d, dn)) != NH_OK) return status;
+        } else {
+            GemvArgs o = narrow(m, m->attn_o[L], H, QW, m->att, T, m->h);
+            o.residual = m->h;
+            if ((status = launch_gemv(d, o)) != NH_OK) return status;
+            GemvArgs gu = narrow(m, m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
+            gu.W[1] = m->ffn_up[L];
+            gu.end[0] = F, gu.end[1] = gu.end[2] = 2 * F;
+            gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
+            if ((status = launch_gemv(d, gu)) != NH_OK) return status;
+            GemvArgs dn = narrow(m, m->ffn_down[L], H, F, m->act, T, m->h);
+            dn.residual = m->h;
+            if ((status = launch_gemv(d, dn)) != NH_OK) return status;
+        }
+        if (mask && (status = launch_mask_rows(d, m->h, rows, B, H, mask)) != NH_OK) return status;
+    }
+    return NH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_weights *weights, const nh_tensor_table *table) {
+    if (!device || !config || !weights || !table) {
+        fail(NH_E_ARGUMENT, "a model names no device, config, arena or tensor table");
+        return nullptr;
+    }
+    const nh_model_config &c = *config;
+    if (!c.layers || !c.hidden || !c.heads || !c.kv_heads || !c.head_dim || !c.ffn || !c.vocab || !c.context || !c.batch ||
+        c.heads % c.kv_heads || c.head_dim % 8) {
+        fail(NH_E_ARGUMENT, "a decoder of %u layers, %u hidden, %u/%u heads of %u, %u ffn, %u vocab, %u context, %u planes holds no model",
+             c.layers, c.hidden, c.heads, c.kv_heads, c.head_dim, c.ffn, c.vocab, c.context, c.batch);
+        return nullptr;
+    }
+    if (table->matrix_element != NH_Q8_0 && table->matrix_element != NH_Q4_K) {
+        fail(NH_E_ARGUMENT, "a decoder multiplies Q8_0 or Q4_K matrices, and this table names element %d", table->matrix_element);
+        return nullptr;
+    }
+    uint32_t block = block_elements(table->matrix_element);
+    if (c.hidden % block || c.ffn % block || (c.heads * c.head_dim) % block) {
+        fail(NH_E_ARGUMENT, "rows of %u, %u and %u numbers are not whole blocks of %u", c.hidden, c.ffn, c.heads * c.head_dim, block);
+        return nullptr;
+    }
+    if (!(c.rope_base > 1.0f) || !std::isfinite(c.rope_base)) {  // refusal::KNOB, crates/neura-kernel/src/task/rope.rs:33-36
+        fail(NH_E_ARGUMENT, "a rope base of %f turns nothing", (double)c.rope_base);
+        return nullptr;
+    }
+    nh_model *m = new nh_model();
+    m->d = device, m->weights = weights, m->c = c, m->element = table->matrix_element;
+    uint32_t widest = c.max_rows ? c.max_rows : 1;
+    m->window = c.context;               // crates/neura-generate/src/batch.rs:314
+    m->capacity = c.context + widest;    // crates/neura-generate/src/batch.rs:323-325
+    m->max_tokens = widest * c.batch;
+    size_t arena = nh_weights_bytes(weights);
+    auto at = [&](uint64_t offset, uint64_t bytes, const char *name) -> const uint8_t * {
+        if (offset % 16 || offset > arena || bytes > arena - offset) {
+            fail(NH_E_ARGUMENT, "the tensor %s of %llu bytes at %llu does not sit 16-byte aligned inside an arena of %zu bytes", name,
+                 (unsigned long long)bytes, (unsigned long long)offset, arena);
+            return nullptr;
+        }
+        return static_cast<const uint8_t *>(nh_weights_at(weights, offset));
+    };
+    const uint32_t H = c.hidden, QW = c.heads * c.head_dim, KW = c.kv_heads * c.head_dim, F = c.ffn;
+    auto matrix_bytes = [&](uint64_t n, uint64_t k) { return n * payload_bytes(m->element, k); };
+    bool ok = true;
+    ok = ok && (m->token_embd = at(table->token_embd, matrix_bytes(c.vocab, H), "token_embd.weight"));
+    m->output = m->token_embd;  // tied head unless the table names one (examples/qwen/model.rs:81-84)
+    if (ok && table->output != UINT64_MAX) ok = (m->output = at(table->output, matrix_bytes(c.vocab, H), "output.weight")) != nullptr;
+    ok = ok && (m->output_norm = reinterpret_cast<const float *>(at(table->output_norm, (uint64_t)H * 4, "output_norm.weight")));
+    for (uint32_t L = 0; ok && L < c.layers; L++) {
+        const uint8_t *p;
+        ok = ok && (p = at(table->attn_norm[L], (uint64_t)H * 4, "attn_norm.weight"));
+        if (ok) m->attn_norm.push_back(reinterpret_cast<const float *>(p));
+        ok = ok && (p = at(table->ffn_norm[L], (uint64_t)H * 4, "ffn_norm.weight"));
+        if (ok) m->ffn_norm.push_back(reinterpret_cast<const float *>(p));
+        ok = ok && (p = at(table->attn_q[L], matrix_bytes(QW, H), "attn_q.weight"));
+        if (ok) m->attn_q.push_back(p);
+        ok = ok && (p = at(table->attn_k[L], matrix_bytes(KW, H), "attn_k.weight"));
+        if (ok) m->attn_k.push_back(p);
+        ok = ok && (p = at(table->attn_v[L], matrix_bytes(KW, H), "attn_v.weight"));
+        if (ok) m->attn_v.push_back(p);
+        ok = ok && (p = at(table->attn_output[L], matrix_bytes(H, QW), "attn_output.weight"));
+        if (ok) m->attn_o.push_back(p);
+        ok = ok && (p = at(table->ffn_gate[L], matrix_bytes(F, H), "ffn_gate.weight"));
+        if (ok) m->ffn_gate.push_back(p);
+        ok = ok && (p = at(table->ffn_up[L], matrix_bytes(F, H), "ffn_up.weight"));
+        if (ok) m->ffn_up.push_back(p);
+        ok = ok && (p = at(table->ffn_down[L], matrix_bytes(H, F), "ffn_down.weight"));
+        if (ok) m->ffn_down.push_back(p);
+    }
+    if (!ok) {
+        release(m);
+        return nullptr;
+    }
+    if (hipSetDevice(device->index) != hipSuccess) {
+        fail(NH_E_DEVICE, "device %d cannot be made current", device->index);
+        release(m);
+        return nullptr;
+    }
+    const size_t T = m->max_tokens;
+    m->cache_elements = (size_t)c.kv_heads * c.batch * m->capacity * c.head_dim;
+    ok = device_array(m->h, T * H) && device_array(m->xn, T * H) && device_array(m->qkv, T * (QW + 2 * KW)) &&
+         device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T > 8 ? T * F : 1) &&
+         device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 2 * c.batch + 4) &&
+         device_array(m->chosen_dev, c.batch);
+    for (uint32_t L = 0; ok && L < c.layers; L++) {
+        uint16_t *k = nullptr, *v = nullptr;
+        ok = device_array(k, m->cache_elements);
+        if (ok) m->cache_k.push_back(k);
+        ok = ok && device_array(v, m->cache_elements);
+        if (ok && v) m->cache_v.push_back(v);
+        if (ok) ok = hipMemsetAsync(k, 0, m->cache_elements * 2, device->stream) == hipSuccess &&
+                     hipMemsetAsync(v, 0, m->cache_elements * 2, device->stream) == hipSuccess;
+    }
+    ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 2 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
+         hipHostMalloc((void **)&m->chosen_host, ((size_t)c.batch + 1) * 4, hipHostMallocDefault) == hipSuccess;
+    ok = ok && hipStreamSynchronize(device->stream) == hipSuccess;
+    if (!ok) {
+        fail(NH_E_MEMORY, "device %d holds no caches and activations of this decoder", device->index);
+        release(m);
+        return nullptr;
+    }
+    return m;
+}
+
+void nh_model_destroy(nh_model *model) { release(model); }
+
+uint32_t nh_model_capacity(const nh_model *model) { return model ? model->capacity : 0; }
+
+int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                       uint32_t *chosen_out) {
+    NH_REQUIRE(m && tokens && cursors && chosen_out, "a decode step names no model, tokens, cursors or result");
+    NH_REQUIRE(batch == m->c.batch, "a decode step of %u planes feeds a model of %u planes", batch, m->c.batch);
+    bool any_inactive = false;
+    for (uint32_t b = 0; b < batch; b++) {
+        bool active = !mask || mask[b];
+        any_inactive |= !active;
+        // crates/neura-generate/src/batch.rs:1627-1632: a plane answers only below its context
+        NH_REQUIRE(!active || cursors[b] < m->c.context, "plane %u at cursor %u of a context of %u no longer answers", b, cursors[b],
+                   m->c.context);
+    }
+    nh_device *d = m->d;
+    int32_t status;
+    if ((status = stage_inputs(m, tokens, batch, cursors, mask, batch)) != NH_OK) return status;
+    if ((status = forward(m, 1, any_inactive)) != NH_OK) return status;
+    // logits = rms(hidden) . head^T, then the greedy choice (examples/qwen/model.rs:81-84,
+    // crates/neura-generate/src/sampling.rs:69-71)
+    GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, batch, m->logits);
+    head.norm_w = m->output_norm, head.eps = m->c.eps;
+    if ((status = launch_gemv(d, head)) != NH_OK) return status;
+    if ((status = launch_argmax(d, m->logits, batch, m->c.vocab, m->chosen_dev)) != NH_OK) return status;
+    NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
+    NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
+    NH_HIP(hipStreamSynchronize(d->stream));
+    if (m->chosen_host[batch] != REFUSAL_NONE) return check_refusal(d, "a decode step");
+    memcpy(chosen_out, m->chosen_host, (size_t)batch * 4);
+    return NH_OK;
+}
+
+int32_t nh_prefill(nh_model *m, const uint32_t *tokens, uint32_t rows, const uint32_t *cursors, const uint8_t *mask, uint32_t batch) {
+    NH_REQUIRE(m && tokens && cursors, "a fill names no model, tokens or cursors");
+    NH_REQUIRE(batch == m->c.batch, "a fill of %u planes feeds a model of %u planes", batch, m->c.batch);
+    NH_REQUIRE(rows >= 1 && rows * batch <= m->max_tokens, "a fill of %u rows feeds a model built for chunks of %u rows", rows,
+               m->max_tokens / m->c.batch);
+    bool any_inactive = false;
+    for (uint32_t b = 0; b < batch; b++) {
+        bool active = !mask || mask[b];
+        any_inactive |= !active;
+        NH_REQUIRE(!active || (uint64_t)cursors[b] + rows <= m->c.context, "plane %u at cursor %u fills %u rows past a context of %u", b,
+                   cursors[b], rows, m->c.context);
+    }
+    int32_t status;
+    if ((status = stage_inputs(m, tokens, rows * batch, cursors, mask, batch)) != NH_OK) return status;
+    if ((status = forward(m, rows, any_inactive)) != NH_OK) return status;
+    return check_refusal(m->d, "a fill");
+}
+
+int32_t nh_model_reset(nh_model *m, const uint8_t *reset, uint32_t batch) {
+    NH_REQUIRE(m && reset && batch == m->c.batch, "a reset names no model, no flags or another plane count");
+    const size_t plane = (size_t)m->capacity * m->c.head_dim;
+    for (uint32_t L = 0; L < m->c.layers; L++)
+        for (uint32_t head = 0; head < m->c.kv_heads; head++)
+            for (uint32_t b = 0; b < batch; b++) {
+                if (!reset[b]) continue;
+                size_t at = ((size_t)head * batch + b) * plane;
+                NH_HIP(hipMemsetAsync(m->cache_k[L] + at, 0, plane * 2, m->d->stream));
+                NH_HIP(hipMemsetAsync(m->cache_v[L] + at, 0, plane * 2, m->d->stream));
+            }
+    return NH_OK;
+}
+
+int32_t nh_model_logits(nh_model *m, float *host_out) {
+    NH_REQUIRE(m && host_out, "a logits read names no model or no result");
+    return nh_download(m->d, host_out, m->logits, (size_t)m->c.batch * m->c.vocab * 4);
+}
+
+int32_t nh_model_cache_write(nh_model *m, uint32_t layer, int32_t value_not_key, const uint16_t *host_src) {
+    NH_REQUIRE(m && host_src && layer < m->c.layers, "a cache write names no model, no bytes or no layer %u", layer);
+    return nh_upload(m->d, value_not_key ? m->cache_v[layer] : m->cache_k[layer], host_src, m->cache_elements * 2);
+}
+
+int32_t nh_model_cache_read(nh_model *m, uint32_t layer, int32_t value_not_key, uint16_t *host_dst) {
+    NH_REQUIRE(m && host_dst && layer < m->c.layers, "a cache read names no model, no bytes or no layer %u", layer);
+    return nh_download(m->d, host_dst, value_not_key ? m->cache_v[layer] : m->cache_k[layer], m->cache_elements * 2);
+}
+
+// ---- operator entry points ---------------------------------------------------------------
+
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15u) == 0; }
+
+int32_t nh_dequant(nh_device *device, int32_t element, const void *dev_src, uint64_t elements, float *dev_dst) {
+    NH_REQUIRE(device && dev_src && dev_dst, "a dequantisation names no device or no buffer");
+    uint32_t block = block_elements(element);
+    NH_REQUIRE(block, "element %d carries no reader", element);
+    NH_REQUIRE(elements % block == 0, "%llu numbers are not whole blocks of %u", (unsigned long long)elements, block);
+    return launch_dequant(device, element, dev_src, elements, dev_dst);
+}
+
+int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elements, uint16_t *dev_dst) {
+    NH_REQUIRE(device && dev_src && dev_dst, "a conversion names no device or no buffer");
+    return launch_convert_half(device, dev_src, elements, dev_dst);
+}
+
+int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
+                float *dev_y, const nh_epilogue *epilogue) {
+    NH_REQUIRE(device && dev_W && dev_x && dev_y, "a product names no device or no buffer");
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K, "a narrow product walks Q8_0 or Q4_K weights, not element %d", element);
+    NH_REQUIRE(N > 0 && K > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K, block_elements(element));
+    NH_REQUIRE(rows >= 1 && rows <= 8, "a narrow product takes one to eight rows, not %u", rows);
+    NH_REQUIRE(aligned16(dev_W) && aligned16(dev_x), "a product reads its weights and activations from 16-byte aligned addresses");
+    GemvArgs a{};
+    a.element = element;
+    a.W[0] = dev_W, a.W[1] = nullptr, a.W[2] = nullptr;
+    a.end[0] = a.end[1] = a.end[2] = N;
+    a.N = N, a.K = K, a.x = dev_x, a.rows = rows, a.y = dev_y;
+    if (epilogue) {
+        a.residual = epilogue->residual;
+        a.swiglu = epilogue->swiglu;
+        NH_REQUIRE(!(a.swiglu && a.residual), "a product fuses swiglu or a residual, not both");
+        if (a.swiglu) {
+            NH_REQUIRE(N % 2 == 0, "a swiglu product halves %u rows", N);
+            a.W[1] = static_cast<const uint8_t *>(dev_W) + (size_t)(N / 2) * payload_bytes(element, K);
+            a.end[0] = N / 2;
+            NH_REQUIRE(aligned16(a.W[1]), "the up half of a swiglu product starts off a 16-byte boundary");
+        }
+    }
+    return launch_gemv(device, a);
+}
+
+int32_t nh_gemm(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const void *dev_X, int32_t x_element,
+                uint32_t M, float *dev_Y, const nh_epilogue *epilogue) {
+    NH_REQUIRE(device && dev_W && dev_X && dev_Y, "a product names no device or no buffer");
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K, "a wide product walks Q8_0 or Q4_K weights, not element %d", element);
+    NH_REQUIRE(x_element == NH_F32 || x_element == NH_F16, "a wide product takes fp32 or fp16 activations, not element %d", x_element);
+    NH_REQUIRE(N > 0 && K > 0 && M > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K,
+               block_elements(element));
+    NH_REQUIRE(aligned16(dev_W) && aligned16(dev_X), "a product reads its weights and activations from 16-byte aligned addresses");
+    NH_REQUIRE(!(epilogue && epilogue->swiglu), "a wide product fuses no swiglu");
+    GemmArgs a{element, dev_W, N, K, dev_X, x_element, M, dev_Y, epilogue ? epilogue->residual : nullptr, N};
+    return launch_gemm(device, a);
+}
+
+int32_t nh_rmsnorm(nh_device *device, const float *dev_x, const float *dev_residual, const float *dev_w, float eps, uint32_t rows,
+                   uint32_t C, float *dev_out, float *dev_sum_out) {
+    NH_REQUIRE(device && dev_x && dev_out && C > 0, "a norm names no device, no buffer or no column");
+    return launch_rmsnorm(device, dev_x, dev_residual, dev_w, eps, rows, C, dev_out, dev_sum_out);
+}
+
+int32_t nh_rope(nh_device *device, const float *dev_x, uint32_t planes, uint32_t batch, uint32_t rows, uint32_t width,
+                const uint32_t *dev_cursor, float base, float *dev_out) {
+    NH_REQUIRE(device && dev_x && dev_out, "a rope names no device or no buffer");
+    NH_REQUIRE(width >= 2 && width % 2 == 0, "a rope turns pairs, and %u numbers leave one over", width);
+    NH_REQUIRE(std::isfinite(base) && base > 1.0f, "a rope base of %f turns nothing", (double)base);
+    return launch_rope(device, dev_x, planes, batch, rows, width, dev_cursor, base, dev_out);
+}
+
+int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v, uint16_t *dev_cache_k, uint16_t *dev_cache_v,
+                       uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
+                       const uint32_t *dev_cursor, const uint8_t *dev_mask) {
+    NH_REQUIRE(device && dev_k && dev_v && dev_cache_k && dev_cache_v && dev_cursor, "a cache write names no device or no buffer");
+    // crates/neura-decoder/src/cache.rs:113-125, :328-335
+    NH_REQUIRE(kv_heads > 0 && width > 0 && batch > 0, "a cache of %u planes of %u heads of %u numbers holds no key", batch, kv_heads, width);
+    NH_REQUIRE(window > 0 && window <= capacity, "a cache of %u positions keeps a window of %u positions", capacity, window);
+    NH_REQUIRE(rows > 0 && rows <= window, "a cache of a %u position window takes %u rows at a time", window, rows);
+    NH_REQUIRE(!dev_mask || rows <= capacity - window, "a masked chunk of %u rows holds only %u scratch rows", rows, capacity - window);
+    int32_t status = launch_cache_write(device, dev_k, dev_v, dev_cache_k, dev_cache_v, kv_heads, batch, rows, width, capacity, window,
+                                        dev_cursor, dev_mask);
+    return status != NH_OK ? status : check_refusal(device, "a cache write");
+}
+
+int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
+                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                     const uint32_t *dev_cursor, float scale, float *dev_out) {
+    NH_REQUIRE(device && dev_q && dev_cache_k && dev_cache_v && dev_out, "an attention names no device or no buffer");
+    // crates/neura-decoder/src/cache.rs:383-388
+    NH_REQUIRE(kv_heads > 0 && heads % kv_heads == 0, "a query of %u heads reads a cache of %u key heads", heads, kv_heads);
+    NH_REQUIRE(keys > 0 && keys <= capacity && rows > 0 && rows <= keys, "%u rows weigh %u keys of a cache of %u positions", rows, keys, capacity);
+    NH_REQUIRE(std::isfinite(scale) && scale != 0.0f, "an attention scale of %f weighs nothing", (double)scale);  // attention.rs:128-132
+    NH_REQUIRE(aligned16(dev_cache_k) && aligned16(dev_cache_v), "an attention reads its caches from 16-byte aligned addresses");
+    AttentionArgs a{};
+    a.q = dev_q, a.out = dev_out;
+    a.q_sh = a.o_sh = (uint64_t)batch * rows * width;
+    a.q_sb = a.o_sb = (uint64_t)rows * width;
+    a.q_sr = a.o_sr = width;
+    a.cache_k = dev_cache_k, a.cache_v = dev_cache_v;
+    a.heads = heads, a.kv_heads = kv_heads, a.batch = batch, a.rows = rows, a.width = width, a.capacity = capacity, a.keys = keys;
+    a.cursor = dev_cursor, a.scale = scale;
+    int32_t status = launch_attention(device, a);
+    return status != NH_OK ? status : check_refusal(device, "an attention");
+}
+
+int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uint32_t vocab, uint32_t width, const uint32_t *dev_tokens,
+                  uint32_t count, uint32_t batch, const uint8_t *dev_mask, float *dev_out) {
+    NH_REQUIRE(device && dev_table && dev_tokens && dev_out, "a gather names no device or no buffer");
+    uint32_t block = block_elements(element);
+    NH_REQUIRE(block && width % block == 0, "a row of %u numbers is not whole blocks of element %d", width, element);
+    NH_REQUIRE(batch > 0, "a gather spreads its mask over no plane");
+    int32_t status = launch_gather(device, element, dev_table, vocab, width, dev_tokens, count, batch, dev_mask, dev_out);
+    return status != NH_OK ? status : check_refusal(device, "a gather");
+}
+
+int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out) {
+    NH_REQUIRE(device && dev_values && dev_out && n > 0, "a choice names no device, no buffer or no value");
+    return launch_argmax(device, dev_values, rows, n, dev_out);
+}
+
+}  // extern "C"

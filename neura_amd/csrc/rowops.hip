@@ -1,0 +1,222 @@
+// Row operators around the products: RMSNorm, rotary embedding, fp16 cache append,
+// SwiGLU and plane masking.
+#include "blocks.hpp"
+#include "common.hpp"
+
+namespace nh {
+
+// One workgroup per row; the sum of squares follows the reference's order (thread t adds
+// columns t, t+256, ..., then a 256-wide tree: crates/neura-kernel/src/task/norm.rs:69-104,
+// reduce.rs:21-38) so the scale is the same fp32 number.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x, const float *__restrict__ residual,
+                                                      const float *__restrict__ w, float eps, uint32_t C, float *__restrict__ out,
+                                                      float *__restrict__ sum_out) {
+    __shared__ float red[256];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const float *xr = x + (size_t)row * C;
+    const float *rr = residual ? residual + (size_t)row * C : nullptr;
+    float square = 0.0f;
+    for (uint32_t c = tid; c < C; c += 256) {
+        float value = rr ? __fadd_rn(xr[c], rr[c]) : xr[c];
+        square = __fadd_rn(square, __fmul_rn(value, value));
+    }
+    red[tid] = square;
+    __syncthreads();
+    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+        if (tid < stride) red[tid] = __fadd_rn(red[tid], red[tid + stride]);
+        __syncthreads();
+    }
+    float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(red[0], (float)C), eps)));
+    for (uint32_t c = tid; c < C; c += 256) {
+        float value = rr ? __fadd_rn(xr[c], rr[c]) : xr[c];
+        if (sum_out) sum_out[(size_t)row * C + c] = value;
+        float result = __fmul_rn(value, scale);
+        if (w) result = __fmul_rn(result, w[c]);
+        out[(size_t)row * C + c] = result;
+    }
+}
+
+int32_t launch_rmsnorm(nh_device *d, const float *x, const float *residual, const float *w, float eps, uint32_t rows, uint32_t C,
+                       float *out, float *sum_out) {
+    if (!rows) return NH_OK;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, d->stream, x, residual, w, eps, C, out, sum_out);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// rotate-half (crates/neura-kernel/src/task/rope.rs:95-122); the angle is
+// f32(position) * table[channel], the table holding pow(base, -2c/width) (rope.rs:48-50)
+__device__ __forceinline__ void rotate(float low, float high, uint32_t position, float frequency, float &out_low, float &out_high) {
+    float angle = __fmul_rn((float)position, frequency);
+    float cosine = cosf(angle), sine = sinf(angle);
+    out_low = low * cosine - high * sine;
+    out_high = high * cosine + low * sine;
+}
+
+__global__ __launch_bounds__(256) void rope_kernel(const float *__restrict__ x, uint32_t planes, uint32_t batch, uint32_t rows,
+                                                   uint32_t width, const uint32_t *__restrict__ cursor,
+                                                   const float *__restrict__ table, float *__restrict__ out) {
+    const uint32_t half = width / 2;
+    const uint64_t pairs = (uint64_t)planes * batch * rows * half;
+    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < pairs; index += (uint64_t)gridDim.x * blockDim.x) {
+        uint32_t c = (uint32_t)(index % half);
+        uint64_t vector = index / half;  // (plane, b, row)
+        uint32_t row = (uint32_t)(vector % rows);
+        uint32_t b = (uint32_t)((vector / rows) % batch);
+        const float *src = x + vector * width;
+        float low, high;
+        rotate(src[c], src[c + half], (cursor ? cursor[b] : 0u) + row, table[c], low, high);
+        out[vector * width + c] = low;
+        out[vector * width + c + half] = high;
+    }
+}
+
+int32_t launch_rope(nh_device *d, const float *x, uint32_t planes, uint32_t batch, uint32_t rows, uint32_t width,
+                    const uint32_t *cursor, float base, float *out) {
+    const float *table = rope_frequencies(d, base, width);
+    if (!table) return NH_E_DEVICE;
+    uint64_t pairs = (uint64_t)planes * batch * rows * (width / 2);
+    if (!pairs) return NH_OK;
+    uint32_t grid = (uint32_t)((pairs + 255) / 256 < 65535 ? (pairs + 255) / 256 : 65535);
+    hipLaunchKernelGGL(rope_kernel, dim3(grid), dim3(256), 0, d->stream, x, planes, batch, rows, width, cursor, table, out);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// cast to fp16 and scatter whole rows (crates/neura-decoder/src/cache.rs:311-351,
+// crates/neura-kernel/src/task/scatter.rs:149-171); an inactive plane writes the scratch rows
+__global__ __launch_bounds__(256) void cache_write_kernel(const float *__restrict__ k, const float *__restrict__ v,
+                                                          uint16_t *__restrict__ cache_k, uint16_t *__restrict__ cache_v,
+                                                          uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width,
+                                                          uint32_t capacity, uint32_t window, const uint32_t *__restrict__ cursor,
+                                                          const uint8_t *__restrict__ mask, uint32_t *refusal) {
+    const uint64_t total = (uint64_t)kv_heads * batch * rows * width;
+    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < total; index += (uint64_t)gridDim.x * blockDim.x) {
+        uint32_t c = (uint32_t)(index % width);
+        uint64_t vector = index / width;
+        uint32_t row = (uint32_t)(vector % rows);
+        uint32_t b = (uint32_t)((vector / rows) % batch);
+        uint32_t head = (uint32_t)(vector / rows / batch);
+        bool active = mask == nullptr || mask[b];
+        uint32_t slot = active ? cursor[b] + row : window + row;
+        if (slot >= capacity) {
+            atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
+            continue;
+        }
+        uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width + c;
+        cache_k[at] = float_to_half(k[index]);
+        cache_v[at] = float_to_half(v[index]);
+    }
+}
+
+int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
+                           uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask) {
+    uint64_t total = (uint64_t)kv_heads * batch * rows * width;
+    if (!total) return NH_OK;
+    uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    hipLaunchKernelGGL(cache_write_kernel, dim3(grid), dim3(256), 0, d->stream, k, v, cache_k, cache_v, kv_heads, batch, rows, width,
+                       capacity, window, cursor, mask, d->refusal);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// The decoder's fused form of the two kernels above on a token-major buffer
+// qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane: q is roped in place, k is
+// roped, k and v are cast to fp16 and appended to the caches.
+__global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qkv, uint32_t heads, uint32_t kv_heads, uint32_t width,
+                                                          uint32_t batch, uint32_t rows, uint16_t *__restrict__ cache_k,
+                                                          uint16_t *__restrict__ cache_v, uint32_t capacity, uint32_t window,
+                                                          const uint32_t *__restrict__ cursor, const uint8_t *__restrict__ mask,
+                                                          const float *__restrict__ table, uint32_t *refusal) {
+    const uint32_t half = width / 2;
+    const uint32_t vectors = heads + 2 * kv_heads;  // per token: q heads, k heads, v heads
+    const uint32_t stride = vectors * width;
+    const uint64_t total = (uint64_t)batch * rows * vectors * half;
+    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < total; index += (uint64_t)gridDim.x * blockDim.x) {
+        uint32_t c = (uint32_t)(index % half);
+        uint32_t vector = (uint32_t)((index / half) % vectors);
+        uint32_t t = (uint32_t)(index / half / vectors);
+        uint32_t row = t / batch, b = t % batch;
+        float *src = qkv + (size_t)t * stride + (size_t)vector * width;
+        uint32_t position = cursor[b] + row;
+        if (vector < heads) {
+            float low, high;
+            rotate(src[c], src[c + half], position, table[c], low, high);
+            src[c] = low;
+            src[c + half] = high;
+            continue;
+        }
+        bool active = mask == nullptr || mask[b];
+        uint32_t slot = active ? position : window + row;
+        if (slot >= capacity) {
+            atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
+            continue;
+        }
+        if (vector < heads + kv_heads) {
+            uint32_t head = vector - heads;
+            float low, high;
+            rotate(src[c], src[c + half], position, table[c], low, high);
+            uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
+            cache_k[at + c] = float_to_half(low);
+            cache_k[at + c + half] = float_to_half(high);
+        } else {
+            uint32_t head = vector - heads - kv_heads;
+            uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
+            cache_v[at + c] = float_to_half(src[c]);
+            cache_v[at + c + half] = float_to_half(src[c + half]);
+        }
+    }
+}
+
+int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
+                           uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask, float base) {
+    const float *table = rope_frequencies(d, base, width);
+    if (!table) return NH_E_DEVICE;
+    uint64_t total = (uint64_t)batch * rows * (heads + 2 * kv_heads) * (width / 2);
+    if (!total) return NH_OK;
+    uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    hipLaunchKernelGGL(rope_append_kernel, dim3(grid), dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k,
+                       cache_v, capacity, window, cursor, mask, table, d->refusal);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// silu(gate) * up (examples/qwen/mlp.rs:33; crates/neura-pointwise/src/op.rs:163)
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up, uint64_t n,
+                                                       float *__restrict__ out) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+        float a = gate[i];
+        out[i] = a * (1.0f / (1.0f + expf(-a))) * up[i];
+    }
+}
+
+int32_t launch_silu_mul(nh_device *d, const float *gate, const float *up, uint64_t n, float *out) {
+    if (!n) return NH_OK;
+    uint32_t grid = (uint32_t)((n + 255) / 256 < 65535 ? (n + 255) / 256 : 65535);
+    hipLaunchKernelGGL(silu_mul_kernel, dim3(grid), dim3(256), 0, d->stream, gate, up, n, out);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+// hidden *= mask of its plane (examples/qwen/model.rs:100); rows are t = row * batch + plane
+__global__ __launch_bounds__(256) void mask_rows_kernel(float *__restrict__ x, uint32_t rows, uint32_t batch, uint32_t width,
+                                                        const uint8_t *__restrict__ mask) {
+    const uint64_t total = (uint64_t)rows * batch * width;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+        uint32_t b = (uint32_t)((i / width) % batch);
+        if (!mask[b]) x[i] = 0.0f;
+    }
+}
+
+int32_t launch_mask_rows(nh_device *d, float *x, uint32_t rows, uint32_t batch, uint32_t width, const uint8_t *mask) {
+    uint64_t total = (uint64_t)rows * batch * width;
+    if (!total || !mask) return NH_OK;
+    uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    hipLaunchKernelGGL(mask_rows_kernel, dim3(grid), dim3(256), 0, d->stream, x, rows, batch, width, mask);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+}  // namespace nh

@@ -1,0 +1,177 @@
+"""Seeded synthetic GGUF payloads of the benchmark configurations, and vectorised numpy
+codecs of the two block formats.
+
+The numpy codecs restate ggml's published Q8_0 / Q4_K layouts independently of the C oracle
+(they are how the tests pin it) and quantize random-init model weights fast enough for the
+0.5B-shape configuration.  They run on the host only.
+"""
+import numpy as np
+
+Q8_0_BLOCK, Q8_0_BYTES = 32, 34
+Q4_K_BLOCK, Q4_K_BYTES = 256, 144
+
+
+def q8_0_random(rng, elements):
+    """Blocks of 32 int8 drawn uniformly from [-127, 127] with fp16 scale |N(0, 0.02)|."""
+    blocks = elements // Q8_0_BLOCK
+    raw = np.empty((blocks, Q8_0_BYTES), dtype=np.uint8)
+    scale = np.abs(rng.normal(0.0, 0.02, blocks)).astype(np.float16)
+    raw[:, 0:2] = scale.view(np.uint8).reshape(blocks, 2)
+    raw[:, 2:] = rng.integers(-127, 128, (blocks, 32), dtype=np.int8).view(np.uint8)
+    return raw.reshape(-1)
+
+
+def q4_k_random(rng, elements):
+    """Super-blocks of random nibbles, uniform 6-bit sub-scales / mins (any scale byte is a
+    valid packing) and fp16 d, dmin drawn |N(0, 0.01)|."""
+    blocks = elements // Q4_K_BLOCK
+    raw = np.empty((blocks, Q4_K_BYTES), dtype=np.uint8)
+    d = np.abs(rng.normal(0.0, 0.01, (blocks, 2))).astype(np.float16)
+    raw[:, 0:4] = d.view(np.uint8).reshape(blocks, 4)
+    raw[:, 4:] = rng.integers(0, 256, (blocks, 140), dtype=np.uint8)
+    return raw.reshape(-1)
+
+
+def q8_0_dequant(raw, elements):
+    blocks = np.asarray(raw, dtype=np.uint8).reshape(-1, Q8_0_BYTES)[: elements // Q8_0_BLOCK]
+    d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32)  # [blocks, 1]
+    q = blocks[:, 2:].view(np.int8).astype(np.float32)
+    return (q * d).reshape(-1)
+
+
+def scale_min_k4(scales):
+    """[blocks, 12] uint8 -> (sc [blocks, 8], m [blocks, 8]) as ggml's get_scale_min_k4."""
+    s = scales.astype(np.uint32)
+    sc = np.empty((s.shape[0], 8), dtype=np.uint32)
+    mn = np.empty((s.shape[0], 8), dtype=np.uint32)
+    sc[:, :4] = s[:, 0:4] & 63
+    mn[:, :4] = s[:, 4:8] & 63
+    sc[:, 4:] = (s[:, 8:12] & 0x0F) | ((s[:, 0:4] >> 6) << 4)
+    mn[:, 4:] = (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)
+    return sc, mn
+
+
+def q4_k_dequant(raw, elements):
+    blocks = np.asarray(raw, dtype=np.uint8).reshape(-1, Q4_K_BYTES)[: elements // Q4_K_BLOCK]
+    d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32)    # [blocks, 1]
+    dmin = blocks[:, 2:4].copy().view(np.float16).astype(np.float32)
+    sc, mn = scale_min_k4(blocks[:, 4:16])
+    quantum = d * sc.astype(np.float32)                              # rounded fp32 product
+    low = dmin * mn.astype(np.float32)
+    qs = blocks[:, 16:].reshape(-1, 4, 32)
+    codes = np.stack([qs & 0x0F, qs >> 4], axis=2).astype(np.float32)  # [blocks, group, seat, 32]
+    quantum = quantum.reshape(-1, 4, 2, 1)
+    low = low.reshape(-1, 4, 2, 1)
+    return (quantum * codes - low).astype(np.float32).reshape(-1)
+
+
+def _round_away(values):
+    return np.sign(values) * np.floor(np.abs(values) + np.float32(0.5))
+
+
+def q8_0_quantize(values):
+    """ggml.rs:201-209: d = max|x| / 127 in fp32, codes from the fp32 d, fp16 d stored."""
+    x = np.asarray(values, dtype=np.float32).reshape(-1, Q8_0_BLOCK)
+    size = np.abs(x).max(axis=1, keepdims=True)
+    quantum = (size / np.float32(127.0)).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        inverse = np.where(quantum == 0, np.float32(0), np.float32(1.0) / quantum).astype(np.float32)
+    codes = np.clip(_round_away((x * inverse).astype(np.float32)), -127, 127).astype(np.int8)
+    raw = np.empty((x.shape[0], Q8_0_BYTES), dtype=np.uint8)
+    raw[:, 0:2] = quantum.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    raw[:, 2:] = codes.view(np.uint8)
+    return raw.reshape(-1)
+
+
+def q4_k_quantize(values):
+    """ggml.rs:149-199 (affine_block with 15 steps over 32-element sub-blocks)."""
+    f32 = np.float32
+    x = np.asarray(values, dtype=f32).reshape(-1, 8, 32)
+    lows = np.minimum(f32(0), x.min(axis=2))
+    highs = np.maximum(f32(0), x.max(axis=2))
+    quantums = ((highs - lows) / f32(15)).astype(f32)
+    scale = (quantums.max(axis=1, keepdims=True) / f32(63)).astype(f32)
+    minimum = ((-lows).max(axis=1, keepdims=True) / f32(63)).astype(f32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        codes = np.where(scale == 0, f32(0), quantums / scale).astype(f32)
+        mins = np.where(minimum == 0, f32(0), -lows / minimum).astype(f32)
+    codes = np.clip(_round_away(codes), 0, 63).astype(np.uint32)
+    mins = np.clip(_round_away(mins), 0, 63).astype(np.uint32)
+    raw = np.zeros((x.shape[0], Q4_K_BYTES), dtype=np.uint8)
+    raw[:, 0:2] = scale.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    raw[:, 2:4] = minimum.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    s = raw[:, 4:16]
+    s[:, 0:4] = (codes[:, 0:4] | ((codes[:, 4:8] >> 4) << 6)).astype(np.uint8)
+    s[:, 4:8] = (mins[:, 0:4] | ((mins[:, 4:8] >> 4) << 6)).astype(np.uint8)
+    s[:, 8:12] = ((codes[:, 4:8] & 0x0F) | ((mins[:, 4:8] & 0x0F) << 4)).astype(np.uint8)
+    quantum = (scale * codes.astype(f32)).astype(f32)[:, :, None]
+    low = (minimum * mins.astype(f32)).astype(f32)[:, :, None]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(quantum == 0, f32(0), ((x + low).astype(f32) / quantum).astype(f32))
+    q = np.clip(_round_away(q.astype(f32)), 0, 15).astype(np.uint8).reshape(-1, 4, 2, 32)
+    raw[:, 16:] = (q[:, :, 0, :] | (q[:, :, 1, :] << 4)).reshape(-1, 128)
+    return raw.reshape(-1)
+
+
+QUANTIZE = {8: q8_0_quantize, 12: q4_k_quantize}
+RANDOM = {8: q8_0_random, 12: q4_k_random}
+DEQUANT = {8: q8_0_dequant, 12: q4_k_dequant}
+BLOCK_BYTES = {8: (Q8_0_BLOCK, Q8_0_BYTES), 12: (Q4_K_BLOCK, Q4_K_BYTES)}
+
+
+def matrix_bytes(element, rows, columns):
+    per, size = BLOCK_BYTES[element]
+    return rows * (columns // per) * size
+
+
+# ---- decoder shapes of the benchmark configurations --------------------------------------
+
+SHAPES = {
+    # name: layers, hidden, heads, kv_heads, head_dim, ffn, vocab, tied head
+    "qwen2.5-0.5b": dict(layers=24, hidden=896, heads=14, kv_heads=2, head_dim=64, ffn=4864, vocab=151936, tied=True),
+    "qwen2.5-1.5b": dict(layers=28, hidden=1536, heads=12, kv_heads=2, head_dim=128, ffn=8960, vocab=151936, tied=True),
+    "qwen2.5-7b": dict(layers=28, hidden=3584, heads=28, kv_heads=4, head_dim=128, ffn=18944, vocab=152064, tied=False),
+}
+
+
+def layer_matrices(shape):
+    """(name, rows N, columns K) of the seven matrices of one layer."""
+    H, QW, KW, F = shape["hidden"], shape["heads"] * shape["head_dim"], shape["kv_heads"] * shape["head_dim"], shape["ffn"]
+    return [("attn_q", QW, H), ("attn_k", KW, H), ("attn_v", KW, H), ("attn_output", H, QW), ("ffn_gate", F, H), ("ffn_up", F, H),
+            ("ffn_down", H, F)]
+
+
+def model_tensors(shape, element, rng, mode="blocks", layers=None):
+    """Yields (name, element, dims (GGUF order: K first), raw bytes) of a random-init decoder.
+
+    mode "blocks": matrices are random raw blocks (the Q4_K distribution of the GEMV
+    configurations); mode "normal": N(0, 0.02) weights quantized with the reference's encoder.
+    Norm weights are fp32.
+    """
+    H = shape["hidden"]
+    count = shape["layers"] if layers is None else layers
+
+    def matrix(rows, columns):
+        if mode == "blocks":
+            return RANDOM[element](rng, rows * columns)
+        out = np.empty(matrix_bytes(element, rows, columns), dtype=np.uint8)
+        step = max(1, (1 << 24) // columns)
+        row_bytes = matrix_bytes(element, 1, columns)
+        for first in range(0, rows, step):
+            n = min(step, rows - first)
+            values = rng.normal(0.0, 0.02, (n, columns)).astype(np.float32)
+            out[first * row_bytes:(first + n) * row_bytes] = QUANTIZE[element](values)
+        return out
+
+    def norm():
+        return (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32).view(np.uint8)
+
+    yield "token_embd.weight", element, (H, shape["vocab"]), matrix(shape["vocab"], H)
+    for layer in range(count):
+        yield "blk.%d.attn_norm.weight" % layer, 0, (H,), norm()
+        yield "blk.%d.ffn_norm.weight" % layer, 0, (H,), norm()
+        for name, rows, columns in layer_matrices(shape):
+            yield "blk.%d.%s.weight" % (layer, name), element, (columns, rows), matrix(rows, columns)
+    yield "output_norm.weight", 0, (H,), norm()
+    if not shape["tied"]:
+        yield "output.weight", element, (H, shape["vocab"]), matrix(shape["vocab"], H)

@@ -1,0 +1,157 @@
+"""Pins the CPU oracle's codecs (f16, PRNG, Q8_0, Q4_K) against what fixes them without the
+reference binary: IEEE binary16 (numpy), the published ggml layouts restated in numpy,
+hand-built blocks, and encode/decode invariants."""
+import numpy as np
+import pytest
+
+import oracle
+from neura_amd import synth
+
+
+def test_f16_to_f32_matches_ieee_for_every_code():
+    bits = np.arange(65536, dtype=np.uint16)
+    ours = oracle.f16_to_f32(bits)
+    theirs = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(ours.view(np.uint32)[~np.isnan(theirs)], theirs.view(np.uint32)[~np.isnan(theirs)])
+    assert np.all(np.isnan(ours[np.isnan(theirs)]))
+
+
+def test_f32_to_f16_is_round_to_nearest_even():
+    rng = np.random.default_rng(1)
+    values = np.concatenate([
+        rng.standard_normal(1 << 18).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 1 << 18).astype(np.float32),
+        rng.integers(0, 1 << 32, 1 << 18, dtype=np.uint64).astype(np.uint32).view(np.float32),  # any bit pattern
+        np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, np.inf, -np.inf, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5], dtype=np.float32),
+    ])
+    # every exact midpoint between neighbouring halves (ties) and both neighbours of it
+    halves = np.arange(0, 0x7c00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = ((halves[:-1] + halves[1:]) / 2).astype(np.float32)
+    values = np.concatenate([values, mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9)), -mids])
+    ours = oracle.f32_to_f16(values)
+    with np.errstate(over="ignore"):
+        theirs = values.astype(np.float16).view(np.uint16)
+    nan = np.isnan(values)
+    assert np.array_equal(ours[~nan], theirs[~nan])
+    assert np.all((ours[nan] & 0x7fff) == 0x7e00)  # convert.rs:61-63: NaN -> sign | 0x7e00
+
+
+def test_xorshift_unit_is_the_closed_form():
+    entropy = 23 | 1
+    expected = []
+    for _ in range(1000):
+        entropy ^= (entropy << 13) & 0xFFFFFFFF
+        entropy ^= entropy >> 17
+        entropy ^= (entropy << 5) & 0xFFFFFFFF
+        expected.append(np.float32(-1.0) + np.float32(2.0) * (np.float32(entropy >> 8) / np.float32(1 << 24)))
+    assert np.array_equal(oracle.random(1000, 23), np.array(expected, dtype=np.float32))
+    assert np.array_equal(oracle.random(10, 22), oracle.random(10, 23))  # seed | 1
+    held = oracle.random(100000, 29)
+    assert held.min() >= -1.0 and held.max() < 1.0 and abs(float(held.mean())) < 0.01
+
+
+def test_scale_min_k4_put_then_get_is_identity_everywhere():
+    for at in range(8):
+        for scale in range(64):
+            for minimum in range(64):
+                scales = np.zeros(12, dtype=np.uint8)
+                oracle.put_scale_min_k4(scales, at, scale, minimum)
+                assert oracle.scale_min_k4(scales, at) == (scale, minimum)
+
+
+def test_scale_min_k4_matches_the_published_layout_on_random_bytes():
+    rng = np.random.default_rng(2)
+    scales = rng.integers(0, 256, (200, 12), dtype=np.uint8)
+    sc, mn = synth.scale_min_k4(scales)
+    for row in range(200):
+        for at in range(8):
+            assert oracle.scale_min_k4(scales[row], at) == (int(sc[row, at]), int(mn[row, at]))
+
+
+def test_q8_0_unpack_every_code_is_the_closed_form():
+    # all 256 codes under a spread of scales, block laid out by hand
+    for scale in (np.float16(1.0), np.float16(0.0123), np.float16(6e-8), np.float16(65504.0), np.float16(0.0)):
+        for first in range(0, 256, 32):
+            codes = np.arange(first, first + 32, dtype=np.uint8)
+            raw = np.concatenate([np.array([scale]).view(np.uint8), codes])
+            got = oracle.unpack(oracle.EL_Q8_0, raw, 32)
+            want = codes.view(np.int8).astype(np.float32) * np.float32(scale)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q4_k_unpack_hand_built_block():
+    # byte pattern in the manner of the reference's Q3_K known-answer test
+    # (crates/neura-precision/tests/format.rs:221-234): quants (at*37+11), scales (at*53+7)
+    raw = np.zeros(144, dtype=np.uint8)
+    raw[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+    raw[2:4] = np.array([np.float16(0.25)]).view(np.uint8)
+    raw[4:16] = [(at * 53 + 7) & 0xFF for at in range(12)]
+    raw[16:] = [(at * 37 + 11) & 0xFF for at in range(128)]
+    got = oracle.unpack(oracle.EL_Q4_K, raw, 256)
+    s = raw[4:16].astype(int)
+    expected = []
+    for j in range(8):
+        if j < 4:
+            sc, mn = s[j] & 63, s[j + 4] & 63
+        else:
+            sc, mn = (s[j + 4] & 15) | ((s[j - 4] >> 6) << 4), (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+        for lane in range(32):
+            byte = int(raw[16 + (j // 2) * 32 + lane])
+            q = (byte >> 4) if j % 2 else (byte & 15)
+            expected.append(np.float32(np.float32(0.5) * np.float32(sc)) * np.float32(q) - np.float32(np.float32(0.25) * np.float32(mn)))
+    assert np.array_equal(got, np.array(expected, dtype=np.float32))
+    # element order: 32 low nibbles then 32 high nibbles per 64-group (ggml.rs:339-348)
+    assert got[0] == np.float32(0.5 * (s[0] & 63)) * np.float32(raw[16] & 15) - np.float32(0.25 * (s[4] & 63))
+    assert got[32] == np.float32(0.5 * (s[1] & 63)) * np.float32(raw[16] >> 4) - np.float32(0.25 * (s[5] & 63))
+
+
+@pytest.mark.parametrize("element", [8, 12])
+def test_unpack_matches_the_numpy_restatement_on_random_blocks(element):
+    rng = np.random.default_rng(3 + element)
+    elements = 256 * 300
+    raw = synth.RANDOM[element](rng, elements)
+    got = oracle.unpack(element, raw, elements)
+    want = synth.DEQUANT[element](raw, elements)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("element", [8, 12])
+def test_pack_matches_the_numpy_restatement(element):
+    rng = np.random.default_rng(5 + element)
+    values = np.concatenate([
+        rng.normal(0, 0.02, 256 * 64), rng.uniform(-1, 1, 256 * 64), np.zeros(256), np.full(256, 0.3), -np.abs(rng.normal(0, 1, 256)),
+        np.abs(rng.normal(0, 1, 256)),
+    ]).astype(np.float32)
+    assert np.array_equal(oracle.pack(element, values), synth.QUANTIZE[element](values))
+
+
+def test_q8_0_pack_invariants():
+    values = oracle.random(32 * 500, 7)  # the reference's own packing test draws seed 7 (runtime.rs:727)
+    raw = oracle.pack(oracle.EL_Q8_0, values)
+    back = oracle.unpack(oracle.EL_Q8_0, raw, values.size)
+    blocks = raw.reshape(-1, 34)
+    d = blocks[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)
+    codes = blocks[:, 2:].view(np.int8)
+    assert codes.min() >= -127 and codes.max() <= 127
+    # every block holds a +-127 code: the scale is max|x| / 127
+    assert np.all(np.abs(codes).max(axis=1) == 127)
+    error = np.abs(back - values).reshape(-1, 32).max(axis=1)
+    assert np.all(error <= d * 0.5 + np.abs(values).reshape(-1, 32).max(axis=1) * 2.0 ** -10)  # half a step + fp16 rounding of d
+
+
+def test_q4_k_pack_invariants():
+    values = oracle.random(256 * 200, 23)  # runtime.rs:24 draws seed 23
+    raw = oracle.pack(oracle.EL_Q4_K, values)
+    back = oracle.unpack(oracle.EL_Q4_K, raw, values.size)
+    # 4-bit affine codes over a range of <= 2: step <= 2/15; error within a step
+    assert np.abs(back - values).max() <= 2.0 / 15.0
+    assert np.abs(back - values).mean() < 0.03
+    assert oracle.lib().oracle_payload_bytes(12, 256 * 200) == raw.size == 200 * 144
+
+
+def test_block_geometry():
+    # crates/neura-abi/tests/layout.rs:147-158
+    assert oracle.lib().oracle_payload_bytes(8, 32) == 34
+    assert oracle.lib().oracle_payload_bytes(12, 256) == 144
+    assert oracle.lib().oracle_payload_bytes(8, 4864 * 896) == 4630528
+    assert oracle.lib().oracle_payload_bytes(12, 46792704) == 26320896
+    assert oracle.lib().oracle_payload_bytes(12, 512 * 0 + 3584 * 18944) == 38191104
