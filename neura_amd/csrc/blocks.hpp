@@ -53,6 +53,16 @@ __device__ __forceinline__ float q4_k_element(const uint8_t *row, uint64_t i) {
     return __fsub_rn(__fmul_rn(quantum, (float)quant), low);
 }
 
+// 1 / sqrt(total / columns + eps) with every step rounded to fp32 exactly as IEEE does
+// (crates/neura-kernel/src/task/norm.rs:102-104).  Each step runs in fp64 and is rounded
+// once more to fp32, which for /, + and sqrt equals the correctly rounded fp32 operation.
+__device__ __forceinline__ float rms_scale_of(float total, uint32_t columns, float eps) {
+    float mean = (float)((double)total / (double)(float)columns);
+    float shifted = (float)((double)mean + (double)eps);
+    float root = (float)sqrt((double)shifted);
+    return (float)(1.0 / (double)root);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);

@@ -57,7 +57,7 @@ __device__ float rms_scale(const float *__restrict__ x, uint32_t K, float eps, f
     }
     float total = red[0];
     __syncthreads();
-    return __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)K), eps)));
+    return rms_scale_of(total, K, eps);
 }
 
 __device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ 
         if (tid < stride) red[tid] = __fadd_rn(red[tid], red[tid + stride]);
         __syncthreads();
     }
-    float scale = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(red[0], (float)C), eps)));
+    float scale = rms_scale_of(red[0], C, eps);
     for (uint32_t c = tid; c < C; c += 256) {
         float value = rr ? __fadd_rn(xr[c], rr[c]) : xr[c];
         if (sum_out) sum_out[(size_t)row * C + c] = value;

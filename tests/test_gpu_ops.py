@@ -1,0 +1,315 @@
+"""GPU parity of every operator against the CPU oracle, through the C ABI.
+
+Bars: dequantised weights and fp16 conversion bit-exact; products, norm, rope and attention
+within 1e-3 relative or 1e-2 absolute of the oracle's fp32 accumulation (the tests assert much
+tighter bounds where the arithmetic allows); argmax and gather exact."""
+import numpy as np
+import pytest
+
+import oracle
+from neura_amd import NH_Q4_K, NH_Q8_0, NeuraError, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want, rel=1e-3, abs_=1e-2):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    bad = np.abs(got - want) > np.maximum(abs_, rel * np.abs(want))
+    assert not bad.any(), "%d of %d outside tolerance, worst %g" % (bad.sum(), bad.size, np.abs(got - want).max())
+
+
+def tight(got, want, scale=1e-5):
+    """within `scale` of the largest expected magnitude: what fp32 reordering allows"""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    bound = scale * max(1.0, np.abs(want).max())
+    assert np.abs(got - want).max() <= bound, (np.abs(got - want).max(), bound)
+
+
+# ------------------------------------------------------------------ codecs
+
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+def test_dequant_is_bit_exact(device, element):
+    rng = np.random.default_rng(100 + element)
+    elements = 256 * 4000
+    raw = synth.RANDOM[element](rng, elements)
+    got = device.dequant(element, raw, elements)
+    want = oracle.unpack(element, raw, elements)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # packed real weights too (the reference's seeds)
+    values = oracle.random(256 * 64, 23)
+    raw = oracle.pack(element, values)
+    assert np.array_equal(device.dequant(element, raw, values.size).view(np.uint32), oracle.unpack(element, raw, values.size).view(np.uint32))
+
+
+def test_dequant_refuses_ragged_and_unknown(device):
+    raw = np.zeros(144, dtype=np.uint8)
+    with pytest.raises(NeuraError):
+        device.dequant(NH_Q4_K, raw, 100)
+    with pytest.raises(NeuraError):
+        device.dequant(11, raw, 256)
+
+
+def test_convert_half_is_bit_exact(device):
+    rng = np.random.default_rng(101)
+    values = np.concatenate([
+        rng.standard_normal(100000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 100000).astype(np.float32),
+        rng.integers(0, 1 << 32, 100000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        np.array([0.0, -0.0, 65504.0, 65520.0, 65519.9, np.inf, -np.inf, np.nan, 5.96e-8, 2.98e-8, 6.1e-5], dtype=np.float32),
+    ])
+    assert np.array_equal(device.convert_half(values), oracle.f32_to_f16(values))
+
+
+@pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536)])
+def test_gather_is_the_dequantised_row_times_mask(device, element, width):
+    rng = np.random.default_rng(102)
+    vocab = 50
+    raw = synth.RANDOM[element](rng, vocab * width)
+    table = oracle.unpack(element, raw, vocab * width).reshape(vocab, width)
+    tokens = np.array([0, 49, 7, 7, 13, 21], dtype=np.uint32)
+    got = device.gather(element, raw, vocab, width, tokens, batch=2, mask=[1, 0])
+    want = table[tokens] * np.array([1, 0, 1, 0, 1, 0], dtype=np.float32)[:, None]
+    assert np.array_equal(got, want)
+    with pytest.raises(NeuraError) as refused:  # refusal::INDEX (select.rs:38)
+        device.gather(element, raw, vocab, width, np.array([50], dtype=np.uint32))
+    assert refused.value.code == -4
+    assert np.array_equal(device.gather(element, raw, vocab, width, tokens[:1]), table[:1])  # the refusal word was cleared
+
+
+# ------------------------------------------------------------------ narrow products
+
+def test_config1_q8_0_gemv_4864x896_seed0(device):
+    rng = np.random.default_rng(0)
+    N, K = 4864, 896
+    raw = synth.q8_0_random(rng, N * K)
+    x = rng.standard_normal(K).astype(np.float32)
+    got = device.gemv(NH_Q8_0, raw, N, K, x)[0]
+    want = oracle.gemv(NH_Q8_0, raw, N, K, x, threads=8)[0]
+    close(got, want)
+    tight(got, want, 2e-6)
+
+
+@pytest.mark.parametrize("name,N,K", [("q", 1536, 1536), ("k", 256, 1536), ("o", 1536, 1536), ("gate", 8960, 1536), ("down", 1536, 8960)])
+def test_config2_q4_k_gemvs_of_a_1_5b_layer(device, name, N, K):
+    rng = np.random.default_rng(hash(name) % 1000)
+    raw = synth.q4_k_random(rng, N * K)
+    x = rng.standard_normal(K).astype(np.float32)
+    got = device.gemv(NH_Q4_K, raw, N, K, x)[0]
+    want = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)[0]
+    close(got, want)
+    tight(got, want, 2e-6)
+
+
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+@pytest.mark.parametrize("rows", [1, 2, 3, 4, 7, 8])
+def test_reference_narrow_product_test(device, element, rows):
+    # crates/neura-runtime/tests/runtime.rs:12-86 at its own shape and seeds
+    depth, columns = 2048, 1024
+    payload = oracle.pack(element, oracle.random(columns * depth, 23))
+    inputs = oracle.random(rows * depth, 29).reshape(rows, depth)
+    got = device.gemv(element, payload, columns, depth, inputs)
+    want = oracle.gemv(element, payload, columns, depth, inputs, threads=8)
+    assert np.abs(got - want).max() <= 1e-3  # the reference's own bar
+    tight(got, want, 2e-6)
+
+
+@pytest.mark.parametrize("element,N,K", [(NH_Q8_0, 5, 32), (NH_Q8_0, 33, 96), (NH_Q8_0, 1, 2048 + 32), (NH_Q8_0, 130, 4864), (NH_Q4_K, 3, 256),
+                                         (NH_Q4_K, 17, 512), (NH_Q4_K, 1, 4096 + 256), (NH_Q4_K, 66, 18944), (NH_Q4_K, 9, 3584)])
+def test_gemv_ragged_shapes(device, element, N, K):
+    rng = np.random.default_rng(N * 7 + K)
+    raw = synth.RANDOM[element](rng, N * K)
+    for rows in (1, 2, 5):
+        x = rng.standard_normal((rows, K)).astype(np.float32)
+        got = device.gemv(element, raw, N, K, x)
+        want = oracle.gemv(element, raw, N, K, x, threads=8)
+        close(got, want)
+        tight(got, want, 3e-6)
+
+
+@pytest.mark.parametrize("element,N,K", [(NH_Q8_0, 64, 896), (NH_Q4_K, 64, 1536), (NH_Q4_K, 32, 8960)])
+def test_gemv_epilogues(device, element, N, K):
+    rng = np.random.default_rng(5)
+    raw = synth.RANDOM[element](rng, N * K)
+    for rows in (1, 4):
+        x = rng.standard_normal((rows, K)).astype(np.float32)
+        r = rng.standard_normal((rows, N)).astype(np.float32)
+        plain = oracle.gemv(element, raw, N, K, x, threads=8)
+        tight(device.gemv(element, raw, N, K, x, residual=r), r + plain, 3e-6)
+        gate, up = plain[:, : N // 2], plain[:, N // 2:]
+        want = gate * (np.float32(1) / (np.float32(1) + np.exp(-gate))) * up
+        close(device.gemv(element, raw, N, K, x, swiglu=True), want, rel=1e-4, abs_=1e-4 * np.abs(want).max())
+
+
+def test_gemv_is_linear_and_matches_at_full_size(device):
+    # size-independent properties at the 7B FFN shape: W(a x + b z) = a W x + b W z
+    rng = np.random.default_rng(6)
+    N, K = 18944, 3584
+    raw = device.upload(synth.q4_k_random(rng, N * K))
+    x, z = rng.standard_normal(K).astype(np.float32), rng.standard_normal(K).astype(np.float32)
+    yx, yz = device.gemv(NH_Q4_K, raw, N, K, x)[0], device.gemv(NH_Q4_K, raw, N, K, z)[0]
+    both = device.gemv(NH_Q4_K, raw, N, K, np.float32(0.5) * x - np.float32(2.0) * z)[0]
+    tight(both, 0.5 * yx - 2.0 * yz, 1e-5)
+    batched = device.gemv(NH_Q4_K, raw, N, K, np.stack([x, z]))
+    tight(batched[0], yx, 2e-6)
+    tight(batched[1], yz, 2e-6)
+    assert np.array_equal(yx, device.gemv(NH_Q4_K, raw, N, K, x)[0])  # deterministic
+
+
+def test_gemv_refuses_bad_shapes(device):
+    raw = np.zeros(34 * 4, dtype=np.uint8)
+    for args in ((NH_Q8_0, raw, 4, 33), (11, raw, 4, 32)):
+        with pytest.raises(NeuraError):
+            device.gemv(args[0], args[1], args[2], args[3], np.zeros(args[3], dtype=np.float32))
+    with pytest.raises(NeuraError):
+        device.gemv(NH_Q8_0, raw, 4, 32, np.zeros((9, 32), dtype=np.float32))
+
+
+# ------------------------------------------------------------------ wide products
+
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+def test_reference_wide_product_test(device, element):
+    # crates/neura-runtime/tests/runtime.rs:88-144: 8 x 512 x 4096, seeds 23 / 29, tolerance 1e-3
+    rows, depth, columns = 8, 512, 4096
+    payload = oracle.pack(element, oracle.random(columns * depth, 23))
+    inputs = oracle.random(rows * depth, 29).reshape(rows, depth)
+    want = oracle.gemm(element, payload, columns, depth, inputs, threads=8)
+    got = device.gemm(element, payload, columns, depth, inputs)
+    assert np.abs(got - want).max() <= 1e-3
+
+
+@pytest.mark.parametrize("element,M,N,K,half", [(NH_Q4_K, 70, 130, 512, True), (NH_Q4_K, 512, 256, 3584, True), (NH_Q4_K, 33, 64, 256, False),
+                                                (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True)])
+def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
+    rng = np.random.default_rng(M + N + K)
+    raw = synth.RANDOM[element](rng, N * K)
+    X = rng.standard_normal((M, K)).astype(np.float16 if half else np.float32)
+    want = oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8)
+    got = device.gemm(element, raw, N, K, X)
+    close(got, want)
+    r = rng.standard_normal((M, N)).astype(np.float32)
+    close(device.gemm(element, raw, N, K, X, residual=r), want + r)
+
+
+# ------------------------------------------------------------------ row operators
+
+@pytest.mark.parametrize("C", [896, 1536, 3584, 100])
+def test_rmsnorm_matches_bit_for_bit(device, C):
+    rng = np.random.default_rng(C)
+    x = rng.standard_normal((5, C)).astype(np.float32)
+    w = rng.standard_normal(C).astype(np.float32)
+    r = rng.standard_normal((5, C)).astype(np.float32)
+    want, _ = oracle.rmsnorm(x, w, 1e-6)
+    assert np.array_equal(device.rmsnorm(x, w, 1e-6), want)  # same summation order, same roundings
+    want, total = oracle.rmsnorm(x, w, 1e-6, residual=r)
+    got, got_total = device.rmsnorm(x, w, 1e-6, residual=r, want_sum=True)
+    assert np.array_equal(got, want) and np.array_equal(got_total, total)
+
+
+def test_gemv_with_fused_norm_equals_norm_then_gemv(device):
+    # the decoder fuses the norm into the product's prologue; the C ABI exposes both halves
+    rng = np.random.default_rng(8)
+    N, K = 64, 3584
+    raw = synth.q4_k_random(rng, N * K)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    w = rng.standard_normal(K).astype(np.float32)
+    normed = device.rmsnorm(x, w, 1e-6)
+    want = oracle.gemv(NH_Q4_K, raw, N, K, oracle.rmsnorm(x, w, 1e-6)[0])
+    tight(device.gemv(NH_Q4_K, raw, N, K, normed), want, 2e-6)
+
+
+@pytest.mark.parametrize("width,base,origin", [(64, 1e6, 0), (128, 1e6, 1023), (128, 1e6, 4095), (8, 10000.0, 3)])
+def test_rope_matches_oracle(device, width, base, origin):
+    rng = np.random.default_rng(71)  # runtime.rs:539 draws seed 71
+    x = rng.standard_normal((3, 2, 4, width)).astype(np.float32)
+    cursor = np.array([origin, origin // 2], dtype=np.uint32)
+    got = device.rope(x, cursor, base)
+    for plane in range(3):
+        for b in range(2):
+            want = oracle.rope(x[plane, b], int(cursor[b]), base)
+            assert np.abs(got[plane, b] - want).max() <= 1e-4  # the reference's bar (runtime.rs:468-549)
+            assert np.abs(got[plane, b] - want).max() <= 4e-6 * max(1.0, np.abs(want).max())
+
+
+def test_cache_write_casts_and_scatters(device):
+    rng = np.random.default_rng(9)
+    kv_heads, batch, rows, width, capacity, window = 2, 3, 2, 64, 12, 10
+    k = rng.standard_normal((kv_heads, batch, rows, width)).astype(np.float32)
+    v = rng.standard_normal((kv_heads, batch, rows, width)).astype(np.float32)
+    ck = device.alloc(kv_heads * batch * capacity * width * 2)
+    cv = device.alloc(kv_heads * batch * capacity * width * 2)
+    cursor = [0, 5, 8]
+    device.cache_write(k, v, ck, cv, capacity, window, cursor, mask=[1, 1, 0])
+    gk = ck.numpy(np.uint16, (kv_heads, batch, capacity, width))
+    gv = cv.numpy(np.uint16, (kv_heads, batch, capacity, width))
+    wk, wv = np.zeros_like(gk), np.zeros_like(gv)
+    for b, (at, active) in enumerate(zip(cursor, [1, 1, 0])):
+        first = at if active else window  # an inactive plane writes the scratch rows (cache.rs:336, :360-364)
+        wk[:, b, first:first + rows] = oracle.f32_to_f16(k[:, b])
+        wv[:, b, first:first + rows] = oracle.f32_to_f16(v[:, b])
+    assert np.array_equal(gk, wk) and np.array_equal(gv, wv)
+    with pytest.raises(NeuraError) as refused:  # a cursor past the capacity: refusal::ORIGIN
+        device.cache_write(k, v, ck, cv, capacity, window, [0, 11, 0])
+    assert refused.value.code == -4
+    with pytest.raises(NeuraError):  # rows <= window <= capacity (cache.rs:117-125)
+        device.cache_write(k, v, ck, cv, capacity, capacity + 1, cursor)
+
+
+# ------------------------------------------------------------------ attention, choice
+
+@pytest.mark.parametrize("heads,kv_heads,batch,rows,keys,width,origins", [
+    (4, 2, 2, 3, 12, 32, [9, 4]),
+    (14, 2, 1, 1, 1100, 64, [1024]),       # config 4 decode shape
+    (28, 4, 1, 1, 4200, 128, [4095]),      # config 5 decode shape
+    (28, 4, 8, 1, 600, 128, [0, 1, 63, 64, 65, 300, 511, 599]),
+    (12, 2, 1, 17, 300, 128, [200]),       # a fill chunk
+    (8, 8, 2, 5, 40, 256, [35, 0]),
+    (6, 1, 1, 2, 70, 64, [3]),
+])
+def test_attention_matches_oracle_and_f64(device, heads, kv_heads, batch, rows, keys, width, origins):
+    rng = np.random.default_rng(17)  # runtime.rs:594-605 draws seeds 17 / 29 / 43
+    capacity = keys + 3
+    q = rng.standard_normal((heads, batch, rows, width)).astype(np.float32)
+    K = rng.standard_normal((kv_heads, batch, capacity, width)).astype(np.float16)
+    V = rng.standard_normal((kv_heads, batch, capacity, width)).astype(np.float16)
+    scale = 1.0 / np.sqrt(width)
+    got = device.attention(q, K.view(np.uint16), V.view(np.uint16), kv_heads, capacity, keys, origins, scale)
+    want = oracle.attention(q, K.view(np.uint16), V.view(np.uint16), kv_heads, capacity, keys, origins, scale)
+    close(got, want)
+    assert np.abs(got - want).max() <= 1e-5
+    if batch == 1:
+        exact = oracle.attention_f64(q, K[:, :, :keys].astype(np.float32), V[:, :, :keys].astype(np.float32), kv_heads, origins[0], True, scale)
+        assert np.abs(got - exact).max() <= 1e-5  # the reference's bar against fp64 (runtime.rs:551-619)
+
+
+def test_attention_of_equal_scores_is_the_running_mean(device):
+    # crates/neura-runtime/tests/runtime.rs:813-875
+    rng = np.random.default_rng(43)
+    V = rng.standard_normal((2, 1, 100, 64)).astype(np.float16)
+    q = np.zeros((4, 1, 1, 64), dtype=np.float32)
+    for origin in (0, 7, 99):
+        got = device.attention(q, np.zeros_like(V).view(np.uint16), V.view(np.uint16), 2, 100, 100, [origin], 0.125)
+        for head in range(4):
+            assert np.allclose(got[head, 0, 0], V[head // 2, 0, : origin + 1].astype(np.float32).mean(axis=0), atol=1e-5)
+
+
+def test_attention_refuses_a_cursor_past_its_keys(device):
+    q = np.zeros((2, 1, 1, 64), dtype=np.float32)
+    K = np.zeros((2, 1, 8, 64), dtype=np.uint16)
+    with pytest.raises(NeuraError) as refused:  # attention.rs:250-252
+        device.attention(q, K, K, 2, 8, 8, [8], 1.0)
+    assert refused.value.code == -4
+    with pytest.raises(NeuraError):
+        device.attention(q, K, K, 2, 8, 8, [0], 0.0)  # refusal::KNOB (attention.rs:128-132)
+
+
+def test_argmax_lowest_index_on_ties(device):
+    rng = np.random.default_rng(10)
+    values = rng.integers(0, 1000, (3, 151936)).astype(np.float32)  # many exact ties
+    got = device.argmax(values)
+    assert list(got) == [oracle.argmax(row) for row in values] == [int(np.argmax(row)) for row in values]
+    values = rng.standard_normal((8, 152064)).astype(np.float32)
+    assert list(device.argmax(values)) == [int(np.argmax(row)) for row in values]
+    assert list(device.argmax(np.full((1, 5000), -np.inf, dtype=np.float32))) == [0]
+    assert list(device.argmax(np.array([[1.0]], dtype=np.float32))) == [0]
+    edge = np.zeros((1, 4097), dtype=np.float32)
+    edge[0, 4096] = 1.0
+    assert list(device.argmax(edge)) == [4096]
