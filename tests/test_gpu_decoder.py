@@ -1,0 +1,125 @@
+"""GPU parity of the decoder (decode step, fill, greedy loop) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle
+from neura_amd import NH_Q4_K, NH_Q8_0, NeuraError, synth
+from neura_amd.loader import Model, Weights
+
+pytestmark = pytest.mark.gpu
+
+TINY = dict(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=320, tied=True)
+SMALL_Q4 = dict(layers=3, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=1000, tied=False)
+
+
+def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None):
+    rng = np.random.default_rng(seed)
+    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
+    host = {name: raw for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers)
+    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers)
+    return model, ref, weights
+
+
+def margins(logits):
+    top = np.sort(logits, axis=1)[:, -2:]
+    return top[:, 1] - top[:, 0]
+
+
+@pytest.mark.parametrize("shape,element", [(TINY, NH_Q8_0), (SMALL_Q4, NH_Q4_K)])
+def test_decode_steps_match_oracle_logits_and_tokens(device, shape, element):
+    model, ref, weights = build(device, shape, element, batch=2, context=32)
+    rng = np.random.default_rng(1)
+    tokens = rng.integers(0, shape["vocab"], 2)
+    for step in range(6):
+        cursors = [step, step]
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        got = model.decode_step(tokens, cursors)
+        logits = model.logits()
+        scale = np.abs(want_logits).max()
+        # a 1e-6 reordering difference now and then flips the fp16 rounding of a cached key or
+        # value (one half ulp = 5e-4 relative); the oracle sits as far from an fp64 forward pass
+        assert np.abs(logits - want_logits).max() <= 1e-3 * scale, step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens = got
+    for layer in range(shape["layers"]):  # the caches hold the same halves
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_cache = oracle.f16_to_f32(model.cache_read(layer, which).reshape(-1))
+            want_cache = oracle.f16_to_f32(held[layer])
+            assert np.abs(got_cache - want_cache).max() <= 2e-3 * max(1.0, np.abs(want_cache).max())
+    model.release(), weights.release()
+
+
+def test_masked_planes_and_chunked_fill(device):
+    shape = SMALL_Q4
+    model, ref, weights = build(device, shape, NH_Q4_K, batch=2, context=40, max_rows=16, seed=3)
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, shape["vocab"], (16, 2))  # tokens[row * batch + plane]
+    # plane 0 fills 16 rows at cursor 0 while plane 1 is inactive
+    model.prefill(prompt.reshape(-1), 16, [0, 0], mask=[1, 0])
+    ref.forward(prompt.reshape(-1), 16, [0, 0], mask=[1, 0], want_logits=False)
+    # then both planes decode: plane 0 at cursor 16, plane 1 starts at 0
+    tokens = [7, 9]
+    for step in range(3):
+        cursors = [16 + step, step]
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        got = model.decode_step(tokens, cursors)
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max()
+        assert list(got) == list(want)
+        tokens = got
+    k = model.cache_read(0, 0)
+    assert np.any(k[:, 0, :16]) and not np.any(k[:, 1, 3:40])  # the inactive plane wrote scratch rows only
+    # chunked fill == token by token (generation.rs:458-470): replay plane 0 alone, one token at a time
+    model.reset([1, 1])
+    assert not np.any(model.cache_read(0, 0)[:, :, :40])
+    for at in range(16):
+        model.decode_step([prompt[at, 0], 0], [at, 0], mask=[1, 0])
+    k_single = oracle.f16_to_f32(model.cache_read(0, 0)[:, 0, :16].reshape(-1))
+    k_chunk = oracle.f16_to_f32(k[:, 0, :16].reshape(-1))
+    assert np.abs(k_single - k_chunk).max() <= 2e-3 * max(1.0, np.abs(k_chunk).max())
+    model.release(), weights.release()
+
+
+def test_decode_refuses_what_the_reference_refuses(device):
+    model, ref, weights = build(device, TINY, NH_Q8_0, batch=1, context=8)
+    with pytest.raises(NeuraError):   # cursor at the context (batch.rs:1627-1632)
+        model.decode_step([1], [8])
+    with pytest.raises(NeuraError) as refused:  # token id past the vocabulary: refusal::INDEX
+        model.decode_step([TINY["vocab"]], [0])
+    assert refused.value.code == -4
+    assert model.decode_step([1], [0])[0] == ref.forward([1], 1, [0])[1][0]  # and the model still answers
+    with pytest.raises(NeuraError):
+        model.prefill([1, 2], 2, [0])  # built for chunks of one row
+    model.release(), weights.release()
+
+
+def test_config4_greedy_64_steps_qwen2_5_0_5b_shape_q8_0(device):
+    """Random-init 0.5B-shape Q8_0 decoder, fp16 caches prefilled to 1024 random tokens' worth
+    of N(0,1) halves, 64 greedy steps from a random prompt id: token ids identical to the
+    oracle.  The oracle follows the reference's summation order; identity against the
+    reference binary itself is unpinned (it cannot be run here)."""
+    shape = synth.SHAPES["qwen2.5-0.5b"]
+    context, filled, steps = 1024 + 64, 1024, 64
+    model, ref, weights = build(device, shape, NH_Q8_0, batch=1, context=context, seed=0)
+    rng = np.random.default_rng(40)
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            halves = np.zeros(model.cache_shape, dtype=np.float16)
+            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
+            held[layer][:] = halves.view(np.uint16).reshape(-1)
+            model.cache_write(layer, which, halves.view(np.uint16))
+    token = int(rng.integers(0, shape["vocab"]))
+    got_tokens, want_tokens, gaps = [], [], []
+    got = want = token
+    for step in range(steps):
+        want_logits, chosen = ref.forward([want], 1, [filled + step], threads=16)
+        want = int(chosen[0])
+        got = int(model.decode_step([got], [filled + step])[0])
+        want_tokens.append(want), got_tokens.append(got)
+        gaps.append(float(margins(want_logits)[0]))
+        if got != want:
+            break
+    print("greedy margins (top1 - top2): min %.3g median %.3g" % (min(gaps), float(np.median(gaps))))
+    assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
+    model.release(), weights.release()
