@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Headline benchmark: batch-1 greedy decode of a random-init Qwen2.5-7B-shaped decoder with
+Q4_K weights and an fp16 KV cache at context 4096, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step (one token): input upload, every kernel of the 28 layers, the
+output head, the greedy choice and the read-back of the chosen token.  Weights and caches are
+resident in HBM before the timed region.  Prints ONE JSON line:
+  value        tokens/s over the K timed steps (host clock around device-synchronised steps)
+  roofline     the Q4_K narrow product: weight bytes each launch walks / its device time,
+               measured with HIP event pairs around every launch (a profiled pass of the same
+               steps on the same stream), against MI355X's 8 TB/s HBM peak
+  cpu_baseline the CPU oracle (a port of the reference path, OpenMP over output columns) on
+               the host cores, timed on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def workload(name):
+    from neura_amd import synth
+
+    if name == "qwen2.5-7b-q4k":
+        return synth.SHAPES["qwen2.5-7b"], 12, 4096
+    if name == "qwen2.5-0.5b-q8_0":
+        return synth.SHAPES["qwen2.5-0.5b"], 8, 1088
+    raise SystemExit("unknown workload %s" % name)
+
+
+def weight_bytes_per_token(shape, element, layers):
+    from neura_amd import synth
+
+    per_layer = sum(synth.matrix_bytes(element, rows, columns) for _, rows, columns in synth.layer_matrices(shape))
+    head = synth.matrix_bytes(element, shape["vocab"], shape["hidden"])
+    return layers * per_layer + head
+
+
+def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=20.0):
+    """Times the oracle's decode step (the checker, used here only as the reported CPU baseline)
+    on a bounded sample: a decoder cut to `sample_layers` layers plus the output head, at the
+    same context length; the full-depth rate is extrapolated from the per-layer and head times."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle
+
+    cores = min(os.cpu_count() or 1, 16)
+    sample_layers = min(layers, 4)
+    model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=sample_layers)
+    rng = np.random.default_rng(7)
+    for held in model.cache_k + model.cache_v:  # a filled cache, as on the device
+        held[:] = rng.standard_normal(held.size).astype(np.float16).view(np.uint16)
+    cursor = context - 1
+    model.forward([1], 1, [cursor], threads=cores)  # warm-up
+    began = time.perf_counter()
+    runs = 0
+    while runs < 3 or (time.perf_counter() - began < seconds_budget and runs < 50):
+        model.forward([1], 1, [cursor], threads=cores)
+        runs += 1
+    with_head = (time.perf_counter() - began) / runs
+    # head alone: a zero-layer model
+    head_model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=0)
+    head_model.forward([1], 1, [cursor], threads=cores)
+    began = time.perf_counter()
+    for _ in range(3):
+        head_model.forward([1], 1, [cursor], threads=cores)
+    head = (time.perf_counter() - began) / 3
+    per_layer = max(with_head - head, 0.0) / sample_layers
+    step = head + per_layer * layers
+    return {
+        "value": 1.0 / step,
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": "%d decode steps of a %d-layer cut of the %d-layer decoder plus the output head at context %d; "
+                  "full depth extrapolated as head + %d x per-layer time (%.3f s/step)" % (runs, sample_layers, layers, context, layers, step),
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--workload", default="qwen2.5-7b-q4k")
+    parser.add_argument("--layers", type=int, default=None, help="cut the decoder (for quick checks; the result is then not the headline)")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import neura_amd
+    from neura_amd import synth
+    from neura_amd.loader import Model, Weights
+
+    shape, element, context = workload(args.workload)
+    layers = shape["layers"] if args.layers is None else args.layers
+    rng = np.random.default_rng(0)
+    mode = "blocks" if element == 12 else "normal"
+    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
+    device = neura_amd.Device(0)
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, element, batch=1, context=context, layers=layers)
+    # fp16 caches filled up to the context with N(0,1) halves
+    for layer in range(layers):
+        for which in (0, 1):
+            model.cache_write(layer, which, rng.standard_normal(model.cache_shape).astype(np.float16).view(np.uint16))
+
+    total = args.warmup + args.steps
+    first_cursor = context - total  # the last timed step sits at cursor context - 1
+    assert first_cursor >= 0, "more steps than the context holds"
+    token = 1
+    for step in range(args.warmup):
+        token = int(model.decode_step([token], [first_cursor + step])[0])
+    device.sync()
+    began = time.perf_counter()
+    for step in range(args.steps):
+        token = int(model.decode_step([token], [first_cursor + args.warmup + step])[0])
+    device.sync()
+    elapsed = time.perf_counter() - began
+
+    # profiled pass: the same steps again with an event pair around every narrow product
+    profiled = min(args.steps, 16)
+    device.profile_begin()
+    for step in range(profiled):
+        token = int(model.decode_step([token], [context - profiled + step])[0])
+    gemv_seconds, launches, walked = device.profile_end()
+    per_launch_bytes = walked / launches
+    per_launch_seconds = gemv_seconds / launches
+    achieved = per_launch_bytes / per_launch_seconds / 1e9
+
+    result = {
+        "metric": "decode tok/s (bs=1) Qwen2.5-7B-shape Q4_K; quant-GEMV HBM GB/s (% peak)",
+        "value": args.steps / elapsed,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s decode, batch 1, %d layers, fp16 KV cache at context %d, random-init %s weights" %
+                        (args.workload, layers, context, "Q4_K" if element == 12 else "Q8_0"),
+            "weight_bytes_per_token": weight_bytes_per_token(shape, element, layers),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_q4k_kernel" if element == 12 else "gemv_q8_0_kernel",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "bytes_per_launch": per_launch_bytes,
+            "us_per_launch": per_launch_seconds * 1e6,
+            "launches_per_step": launches / profiled,
+            "gemv_ms_per_step": gemv_seconds / profiled * 1e3,
+        },
+    }
+    if not args.no_cpu:
+        host = {name: raw for name, _, _, raw in tensors}
+        result["cpu_baseline"] = cpu_baseline(shape, element, host, context, layers)
+    else:
+        result["cpu_baseline"] = None
+    model.release()
+    weights.release()
+    device.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

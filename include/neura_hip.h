@@ -80,6 +80,15 @@ int32_t nh_sync(nh_device *device);
 int32_t nh_timer_start(nh_device *device);
 int32_t nh_timer_stop(nh_device *device, double *seconds_out);
 
+/* Per-kernel timing as the reference's benchmark takes it (GPU timestamps around each
+ * submission, crates/neura-gpu/src/native/vulkan.rs:1234-1276; examples/benchmark/measure.rs:4-33):
+ * between begin and end every narrow-product launch on this device is bracketed by a HIP event
+ * pair on the device's stream.  end returns the summed device seconds of those launches, their
+ * count and the weight bytes they walked (payload bytes, counted once per launch:
+ * examples/benchmark/product.rs:103-105). */
+int32_t nh_profile_begin(nh_device *device);
+int32_t nh_profile_end(nh_device *device, double *seconds_out, uint64_t *launches_out, uint64_t *bytes_out);
+
 /* ---- weight arena : replaces Runtime::load (crates/neura-runtime/src/runtime.rs:356-367) ---- */
 
 /* one arena of `bytes`; tensors are poured verbatim at 256-byte aligned offsets the caller

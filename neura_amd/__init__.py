@@ -99,6 +99,15 @@ class Device:
         _check(self.lib.nh_timer_stop(self.handle, ctypes.byref(seconds)))
         return seconds.value
 
+    def profile_begin(self):
+        _check(self.lib.nh_profile_begin(self.handle))
+
+    def profile_end(self):
+        """(device seconds, launches, weight bytes) of the narrow products since profile_begin"""
+        seconds, launches, nbytes = ctypes.c_double(), ctypes.c_uint64(), ctypes.c_uint64()
+        _check(self.lib.nh_profile_end(self.handle, ctypes.byref(seconds), ctypes.byref(launches), ctypes.byref(nbytes)))
+        return seconds.value, launches.value, nbytes.value
+
     # ---- operators (numpy in, numpy out unless a Buffer is passed)
     def _dev(self, value):
         return value if isinstance(value, Buffer) else self.upload(value)

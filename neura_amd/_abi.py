@@ -44,6 +44,8 @@ SIGNATURES = {
     "nh_sync": (c_int32, [c_void_p]),
     "nh_timer_start": (c_int32, [c_void_p]),
     "nh_timer_stop": (c_int32, [c_void_p, POINTER(c_double)]),
+    "nh_profile_begin": (c_int32, [c_void_p]),
+    "nh_profile_end": (c_int32, [c_void_p, POINTER(c_double), POINTER(c_uint64), POINTER(c_uint64)]),
     "nh_weights_create": (c_void_p, [c_void_p, c_size_t]),
     "nh_weights_destroy": (None, [c_void_p]),
     "nh_weights_put": (c_int32, [c_void_p, c_size_t, c_void_p, c_size_t]),

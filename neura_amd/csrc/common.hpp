@@ -6,6 +6,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <cstdio>
+#include <vector>
 
 #include "../../include/neura_hip.h"
 
@@ -64,6 +65,11 @@ struct nh_device {
     float *rope_table = nullptr;  // device inverse frequencies of the last (base, width)
     float rope_base = 0.0f;
     uint32_t rope_width = 0;
+    // per-launch timing of the narrow products (nh_profile_*): event pairs on the stream
+    bool profile = false;
+    std::vector<hipEvent_t> profile_events;  // start, stop, start, stop, ...
+    size_t profile_used = 0;
+    uint64_t profile_bytes = 0;              // weight bytes the timed launches walked
 };
 
 namespace nh {
@@ -74,6 +80,9 @@ void *scratch(nh_device *device, size_t bytes);
 const float *rope_frequencies(nh_device *device, float base, uint32_t width);
 // reads and clears the refusal word; returns NH_OK or NH_E_REFUSAL with a message
 int32_t check_refusal(nh_device *device, const char *what);
+
+// records the next profiling event on the stream (no-op unless profiling is on)
+void profile_mark(nh_device *device);
 
 enum Refusal : uint32_t { REFUSAL_NONE = 0, REFUSAL_INDEX = 1, REFUSAL_ORIGIN = 2 };
 

@@ -502,6 +502,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     }
     if (lds > 64 * 1024) return fail(NH_E_ARGUMENT, "a product of depth %u stages %zu bytes where a workgroup holds 65536", a.K, lds);
     dim3 grid(blocks_x, p.splits), block(256);
+    profile_mark(d);
 #define NH_LAUNCH(KERNEL, RR) hipLaunchKernelGGL((KERNEL<RR, RB>), grid, block, lds, d->stream, p)
     if (q4) {
         if (R == 4) NH_LAUNCH(gemv_q4k_kernel, 4);
@@ -518,6 +519,8 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
                            residual, a.swiglu, y);
         NH_HIP(hipGetLastError());
     }
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
     return NH_OK;
 }
 

@@ -85,6 +85,16 @@ int32_t check_refusal(nh_device *device, const char *what) {
     }
 }
 
+void profile_mark(nh_device *device) {
+    if (!device->profile) return;
+    if (device->profile_used == device->profile_events.size()) {
+        hipEvent_t event;
+        if (hipEventCreate(&event) != hipSuccess) return;
+        device->profile_events.push_back(event);
+    }
+    (void)hipEventRecord(device->profile_events[device->profile_used++], device->stream);
+}
+
 }  // namespace nh
 
 using namespace nh;
@@ -133,6 +143,7 @@ void nh_close(nh_device *device) {
     if (device->scratch) (void)hipFree(device->scratch);
     if (device->refusal) (void)hipFree(device->refusal);
     if (device->rope_table) (void)hipFree(device->rope_table);
+    for (hipEvent_t event : device->profile_events) (void)hipEventDestroy(event);
     if (device->started) (void)hipEventDestroy(device->started);
     if (device->stopped) (void)hipEventDestroy(device->stopped);
     if (device->stream) (void)hipStreamDestroy(device->stream);
@@ -208,6 +219,31 @@ int32_t nh_timer_stop(nh_device *device, double *seconds_out) {
     float milliseconds = 0.0f;
     NH_HIP(hipEventElapsedTime(&milliseconds, device->started, device->stopped));
     *seconds_out = (double)milliseconds * 1e-3;
+    return NH_OK;
+}
+
+int32_t nh_profile_begin(nh_device *device) {
+    NH_REQUIRE(device, "a profile names no device");
+    NH_HIP(hipStreamSynchronize(device->stream));
+    device->profile = true;
+    device->profile_used = 0;
+    device->profile_bytes = 0;
+    return NH_OK;
+}
+
+int32_t nh_profile_end(nh_device *device, double *seconds_out, uint64_t *launches_out, uint64_t *bytes_out) {
+    NH_REQUIRE(device && seconds_out && launches_out && bytes_out, "a profile names no device or no result");
+    device->profile = false;
+    NH_HIP(hipStreamSynchronize(device->stream));
+    double total = 0.0;
+    for (size_t at = 0; at + 1 < device->profile_used; at += 2) {
+        float milliseconds = 0.0f;
+        NH_HIP(hipEventElapsedTime(&milliseconds, device->profile_events[at], device->profile_events[at + 1]));
+        total += (double)milliseconds * 1e-3;
+    }
+    *seconds_out = total;
+    *launches_out = device->profile_used / 2;
+    *bytes_out = device->profile_bytes;
     return NH_OK;
 }
 
