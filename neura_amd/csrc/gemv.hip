@@ -44,12 +44,14 @@ __device__ __forceinline__ uint32_t skew32(uint32_t i) { return i + (i >> 5) * 4
 // (crates/neura-kernel/src/task/norm.rs:69-83 + reduce.rs:21-38): thread t adds columns
 // t, t+256, ...; then a 256-wide tree.  Returns 1/sqrt(mean + eps) to every thread.
 __device__ float rms_scale(const float *__restrict__ x, uint32_t K, float eps, float *red) {
-    float square = 0.0f;
-    for (uint32_t c = threadIdx.x; c < K; c += 256) {
-        float value = x[c];
-        square = __fadd_rn(square, __fmul_rn(value, value));
+    if (threadIdx.x < 256) {  // larger workgroups leave the sum to their first 256 threads
+        float square = 0.0f;
+        for (uint32_t c = threadIdx.x; c < K; c += 256) {
+            float value = x[c];
+            square = __fadd_rn(square, __fmul_rn(value, value));
+        }
+        red[threadIdx.x] = square;
     }
-    red[threadIdx.x] = square;
     __syncthreads();
     for (uint32_t stride = 128; stride > 0; stride >>= 1) {
         if (threadIdx.x < stride) red[threadIdx.x] = __fadd_rn(red[threadIdx.x], red[threadIdx.x + stride]);
@@ -68,12 +70,18 @@ __device__ __forceinline__ uint32_t weight_row(uint32_t i, uint32_t N, int32_t s
     return swiglu ? ((i & 1u) ? N / 2 + (i >> 1) : (i >> 1)) : i;
 }
 
-// first byte of output row n and the end of the matrix that holds it
+// first byte of output row n and the end of the matrix that holds it.  Written with selects
+// over scalars: indexing the parameter arrays by a per-lane segment would turn into loads
+// from the kernel argument block and serialise the weight loads behind them.
 __device__ __forceinline__ const uint8_t *row_start(const GemvParams &p, uint32_t n, const uint8_t *&matrix_end) {
-    uint32_t segment = n < p.end[0] ? 0u : (n < p.end[1] ? 1u : 2u);
-    uint32_t before = segment == 0 ? 0u : p.end[segment - 1];
-    matrix_end = p.W[segment] + (size_t)(p.end[segment] - before) * p.row_bytes;
-    return p.W[segment] + (size_t)(n - before) * p.row_bytes;
+    const uint8_t *w0 = p.W[0], *w1 = p.W[1], *w2 = p.W[2];
+    const uint32_t e0 = p.end[0], e1 = p.end[1], e2 = p.end[2];
+    const bool first = n < e0, second = n < e1;
+    const uint8_t *base = first ? w0 : (second ? w1 : w2);
+    const uint32_t before = first ? 0u : (second ? e0 : e1);
+    const uint32_t rows = first ? e0 : (second ? e1 - e0 : e2 - e1);
+    matrix_end = base + (size_t)rows * p.row_bytes;
+    return base + (size_t)(n - before) * p.row_bytes;
 }
 
 template <int R, int RB>
@@ -114,26 +122,37 @@ __device__ __forceinline__ void publish(const GemvParams &p, uint32_t first, uin
 
 // ---------------------------------------------------------------------------- Q4_K -------
 
-// sum over the 32 low-nibble and the 32 high-nibble weights of 8 words against xl / xh
-__device__ __forceinline__ void nibble_dots(const uint4 &qa, const uint4 &qb, const float (&xl)[32], const float (&xh)[32], float &low,
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Sum over the 32 low-nibble and the 32 high-nibble weights of 8 words against xl / xh.
+// A nibble masked in place inside a 16-bit lane IS a half-precision subnormal: bits 0..3 read
+// as code * 2^-24 and bits 4..7 as code * 2^-20, both exact.  The mixed-precision multiply-add
+// (v_fma_mix_f32) widens the half operand on the fly, so a nibble costs one mask per pair and
+// one multiply-add; the powers of two are folded into the block scales by the caller.
+template <typename V4>
+__device__ __forceinline__ void nibble_dots(const V4 &qa, const V4 &qb, const float (&xl)[32], const float (&xh)[32], float &low,
                                             float &high) {
     const uint32_t words[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
     float l = 0.0f, h = 0.0f;
 #pragma unroll
     for (int w = 0; w < 8; w++) {
-        uint32_t lo = words[w] & 0x0f0f0f0fu;
-        uint32_t hi = (words[w] >> 4) & 0x0f0f0f0fu;
-        l = fmaf(xl[4 * w + 0], (float)(lo & 0xffu), l);
-        l = fmaf(xl[4 * w + 1], (float)((lo >> 8) & 0xffu), l);
-        l = fmaf(xl[4 * w + 2], (float)((lo >> 16) & 0xffu), l);
-        l = fmaf(xl[4 * w + 3], (float)(lo >> 24), l);
-        h = fmaf(xh[4 * w + 0], (float)(hi & 0xffu), h);
-        h = fmaf(xh[4 * w + 1], (float)((hi >> 8) & 0xffu), h);
-        h = fmaf(xh[4 * w + 2], (float)((hi >> 16) & 0xffu), h);
-        h = fmaf(xh[4 * w + 3], (float)(hi >> 24), h);
+        const uint32_t even = words[w], odd = words[w] >> 8;  // bytes (0, 2) and bytes (1, 3) in the 16-bit lanes
+        const half2_t l02 = __builtin_bit_cast(half2_t, even & 0x000f000fu);
+        const half2_t h02 = __builtin_bit_cast(half2_t, even & 0x00f000f0u);
+        const half2_t l13 = __builtin_bit_cast(half2_t, odd & 0x000f000fu);
+        const half2_t h13 = __builtin_bit_cast(half2_t, odd & 0x00f000f0u);
+        l = fmaf((float)l02.x, xl[4 * w + 0], l);
+        l = fmaf((float)l13.x, xl[4 * w + 1], l);
+        l = fmaf((float)l02.y, xl[4 * w + 2], l);
+        l = fmaf((float)l13.y, xl[4 * w + 3], l);
+        h = fmaf((float)h02.x, xh[4 * w + 0], h);
+        h = fmaf((float)h13.x, xh[4 * w + 1], h);
+        h = fmaf((float)h02.y, xh[4 * w + 2], h);
+        h = fmaf((float)h13.y, xh[4 * w + 3], h);
     }
-    low = l;
-    high = h;
+    low = l;   // scaled by 2^-24: the caller folds 2^24 into xl or the block scale
+    high = h;  // scaled by 2^-20
 }
 
 // the two (scale, min) pairs of group g (sub-blocks 2g and 2g+1) from a block header
@@ -160,6 +179,217 @@ __device__ __forceinline__ void group_scales(const uint4 &hdr, uint32_t g, float
     m1 = dmin * (float)mn1;
 }
 
+// ---- cross-lane sums without LDS round trips ---------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;  // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;
+
+// Sums R per-lane partials over the G lanes of a row group.  The first log2(R) steps fold two
+// rows into one register (each lane keeps the row its own index selects), so R rows cost
+// R - 1 + log2(G / R) exchanges instead of R log2(G); steps inside a row of 16 lanes are DPP
+// adds, only the steps across 16 and 32 lanes go through the LDS crossbar.  On return lane u
+// (u < R, u = lane % G) of every group holds the total of row u.
+template <int R, int G>
+__device__ __forceinline__ float fold_rows(float (&acc)[R], uint32_t lane) {
+    static_assert(R == 2 || R == 4, "rows per pass");
+    static_assert(G == 16 || G == 32 || G == 64, "lanes per row group");
+    float v;
+    const bool odd = lane & 1u;
+    if (R == 4) {
+        const bool upper = lane & 2u;
+        float keep01 = odd ? acc[1] : acc[0], send01 = odd ? acc[0] : acc[1];
+        float keep23 = odd ? acc[3] : acc[2], send23 = odd ? acc[2] : acc[3];
+        float v01 = keep01 + dpp<DPP_QUAD_XOR1>(send01);
+        float v23 = keep23 + dpp<DPP_QUAD_XOR1>(send23);
+        float keep = upper ? v23 : v01, send = upper ? v01 : v23;
+        v = keep + dpp<DPP_QUAD_XOR2>(send);
+    } else {
+        float keep = odd ? acc[1] : acc[0], send = odd ? acc[0] : acc[1];
+        v = keep + dpp<DPP_QUAD_XOR1>(send);
+        v += dpp<DPP_QUAD_XOR2>(v);
+    }
+    v += dpp<DPP_ROW_ROR4>(v);  // rotations inside a row of 16 lanes keep lane % 4
+    v += dpp<DPP_ROW_ROR8>(v);
+    if (G >= 32) v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+    if (G >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// Per-lane constants of the branch-free scale decode (they depend on the lane's group only).
+struct ScaleLane {
+    uint32_t pick;    // byte selector: the two bytes of this group from the low or the high scale word
+    uint32_t pick_q;  // byte selector: the two bytes that carry the top bits (groups 2, 3)
+    uint32_t mask_p, mask_q;
+    uint32_t shift_m;  // 4 for groups 2, 3: their minimums sit in the high nibbles
+};
+
+__device__ __forceinline__ ScaleLane scale_lane(uint32_t g) {
+    const uint32_t j = 2u * (g & 1u);
+    ScaleLane s;
+    s.pick_q = 0x0c000c00u | j | ((j + 1u) << 16);
+    s.pick = g < 2 ? s.pick_q : (0x0c000c00u | (4u + j) | ((5u + j) << 16));
+    s.mask_p = g < 2 ? 0x003f003fu : 0x000f000fu;
+    s.mask_q = g < 2 ? 0u : 0x00300030u;
+    s.shift_m = g < 2 ? 0u : 4u;
+    return s;
+}
+
+// The 6-bit scales (sc) and minimums (mn) of sub-blocks 2g, 2g+1 as pairs of half-precision
+// subnormals (value * 2^-24 in each 16-bit lane), straight from the header words:
+// crates/neura-precision/src/ggml.rs:127-136 without a branch or an int -> float conversion.
+__device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s, half2_t &sc, half2_t &mn) {
+    const uint32_t p_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick), q_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick_q);
+    const uint32_t p_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick) >> s.shift_m, q_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick_q);
+    sc = __builtin_bit_cast(half2_t, (p_sc & s.mask_p) | ((q_sc >> 2) & s.mask_q));
+    mn = __builtin_bit_cast(half2_t, (p_mn & s.mask_p) | ((q_mn >> 2) & s.mask_q));
+}
+
+// One pass of the decode kernel over R rows: the raw blocks a lane owns.
+template <int R>
+struct DecodeTile {
+    u32x4 hdr[R], qa[R], qb[R];
+};
+
+// Decode path (one activation row).  G = lanes per output row (64: one row group per wave
+// pass, the hot case; 32 / 16: short rows, several row groups side by side in a wave).
+//
+// A lane owns one 64-element group of one super-block for the whole kernel and keeps its 64
+// activations in registers.  Every integer field is consumed as a half-precision subnormal by
+// mixed-precision multiply-adds (nibbles: * 2^-24 / 2^-20, undone by scaling the activations
+// once; scales: * 2^-24, undone once per pass), so a weight costs 1.6 vector instructions.
+template <int R, int G, bool PIPE, int NW>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) {
+    extern __shared__ float xs[];  // skew64(slice)
+    __shared__ float red[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t split = blockIdx.y;
+    const uint32_t blk0 = split * p.blocks_per_split;
+    const uint32_t nb = min(p.blocks_per_split, p.nblk - blk0);
+    const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
+
+    constexpr uint32_t RS = 64u / G;
+    constexpr uint32_t rows_per_pass = R * RS;
+    const uint32_t u = lane & (G - 1u), rs = lane / G;
+    const bool active = u < nb * 4u;
+    const uint32_t unit = active ? u : 0u;  // an idle lane re-reads unit 0 against zero activations
+    const uint32_t g = unit & 3u;
+    const uint32_t lane_offset = (blk0 + (unit >> 2)) * 144u + g * 32u;
+    const ScaleLane lane_scales = scale_lane(g);
+
+    auto load = [&](DecodeTile<R> &t, uint32_t rg) {
+        const uint32_t first = rg * rows_per_pass + rs * R;  // first logical row of this lane group (a multiple of R)
+        // R rows of one matrix: rows never straddle a matrix (every end is a multiple of R)
+        const uint8_t *base[R];
+        if (p.swiglu) {
+            const uint32_t pair = min(first, p.N - R) >> 1;  // logical rows 2q, 2q+1 = gate row q, up row q
+#pragma unroll
+            for (int r = 0; r < R; r++) base[r] = ((r & 1) ? p.W[1] : p.W[0]) + (size_t)(pair + (r >> 1)) * p.row_bytes;
+        } else {
+            const uint32_t n = min(first, p.N - R);
+            const bool in0 = n < p.end[0], in1 = n < p.end[1];
+            const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
+            const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
+#pragma unroll
+            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r) * p.row_bytes;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            typedef const __attribute__((address_space(1))) u32x4 *global_uint4;  // the arena is global memory
+            const uint8_t *at = base[r] + lane_offset;
+            t.hdr[r] = *(global_uint4)(uintptr_t)(at - g * 32u);
+            t.qa[r] = *(global_uint4)(uintptr_t)(at + 16u);
+            t.qb[r] = *(global_uint4)(uintptr_t)(at + 32u);
+        }
+    };
+
+    const uint32_t stride = gridDim.x * NW;
+    uint32_t rg = blockIdx.x * NW + wave;
+    DecodeTile<R> ta, tb;
+    if (rg < p.row_groups) load(ta, rg);  // in flight while the activations are staged
+
+    {
+        float scale = 1.0f;
+        if (p.norm_w) scale = rms_scale(p.x, p.K, p.eps, red);
+        for (uint32_t i = tid; i < kn; i += NW * 64) {
+            float value = p.x[k0 + i];
+            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, scale), p.norm_w[k0 + i]);
+            xs[skew64(i)] = value;
+        }
+    }
+    __syncthreads();
+
+    float xl[32], xh[32];
+    float xsl = 0.0f, xsh = 0.0f;  // plain sums of this lane's activations (for the block minimums)
+    {
+        const float4 *src = reinterpret_cast<const float4 *>(xs + skew64(unit * 64u));
+        const float keep = active ? 1.0f : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            // sum and scale each chunk as it arrives: raw and scaled copies never coexist
+            float4 a = src[j], c = src[8 + j];
+            xsl += (a.x + a.y) + (a.z + a.w);
+            xsh += (c.x + c.y) + (c.z + c.w);
+            const float sl = keep * 16777216.0f, sh = keep * 1048576.0f;  // nibbles arrive * 2^-24 / * 2^-20
+            xl[4 * j] = a.x * sl, xl[4 * j + 1] = a.y * sl, xl[4 * j + 2] = a.z * sl, xl[4 * j + 3] = a.w * sl;
+            xh[4 * j] = c.x * sh, xh[4 * j + 1] = c.y * sh, xh[4 * j + 2] = c.z * sh, xh[4 * j + 3] = c.w * sh;
+        }
+        xsl *= keep, xsh *= keep;
+    }
+
+    auto compute = [&](const DecodeTile<R> &t, uint32_t rg) {
+        const uint32_t first = rg * rows_per_pass + rs * R;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float low, high;
+            nibble_dots(t.qa[r], t.qb[r], xl, xh, low, high);
+            half2_t sc, mn;
+            scale_pairs(t.hdr[r], lane_scales, sc, mn);
+            const half2_t dd = __builtin_bit_cast(half2_t, t.hdr[r].x);  // (d, dmin)
+            const float weighed = fmaf((float)sc.y, high, (float)sc.x * low);
+            const float floor_ = fmaf((float)mn.y, xsh, (float)mn.x * xsl);
+            acc[r] = fmaf((float)dd.x, weighed, -((float)dd.y * floor_));
+        }
+        float total = fold_rows<R, G>(acc, lane) * 16777216.0f;  // the scales arrived * 2^-24
+        const uint32_t i = first + u;                             // lane u < R holds row first + u
+        if (p.splits > 1) {
+            if (u < R && i < p.N) p.partial[(size_t)split * p.N + weight_row(i, p.N, p.swiglu)] = total;
+        } else if (p.swiglu) {
+            float up = dpp<DPP_QUAD_XOR1>(total);
+            if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(total) * up;
+        } else if (u < R && i < p.N) {
+            p.y[i] = p.residual ? p.residual[i] + total : total;
+        }
+    };
+
+    if (PIPE) {
+        while (rg < p.row_groups) {
+            uint32_t next = rg + stride;
+            if (next < p.row_groups) load(tb, next);
+            compute(ta, rg);
+            rg = next;
+            if (rg >= p.row_groups) break;
+            next = rg + stride;
+            if (next < p.row_groups) load(ta, next);
+            compute(tb, rg);
+            rg = next;
+        }
+    } else {
+        while (rg < p.row_groups) {
+            compute(ta, rg);
+            rg += stride;
+            __builtin_amdgcn_sched_barrier(0);  // the next loads reuse this tile's registers: keep them behind the arithmetic
+            if (rg < p.row_groups) load(ta, rg);
+        }
+    }
+}
+
+// General narrow product: RB activation rows (2 or 4) staged in LDS and re-read per row group.
 template <int R, int RB>
 __global__ __launch_bounds__(256) void gemv_q4k_kernel(GemvParams p) {
     extern __shared__ float xs[];  // [RB][skew64(slice)]
@@ -188,21 +418,7 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(GemvParams p) {
     const uint32_t u = lane & (G - 1u), rs = lane / G, RS = 64u / G;
     const bool active = u < nb * 4u;
     const uint32_t blk = active ? (u >> 2) : 0u, g = u & 3u;
-
     float xl[32], xh[32];
-    float xsl = 0.0f, xsh = 0.0f;
-    if (RB == 1) {
-        const float4 *src = reinterpret_cast<const float4 *>(xs + skew64((blk * 4u + g) * 64u));
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            float4 a = active ? src[j] : make_float4(0.f, 0.f, 0.f, 0.f);
-            float4 c = active ? src[8 + j] : make_float4(0.f, 0.f, 0.f, 0.f);
-            xl[4 * j] = a.x, xl[4 * j + 1] = a.y, xl[4 * j + 2] = a.z, xl[4 * j + 3] = a.w;
-            xh[4 * j] = c.x, xh[4 * j + 1] = c.y, xh[4 * j + 2] = c.z, xh[4 * j + 3] = c.w;
-        }
-#pragma unroll
-        for (int j = 0; j < 32; j++) xsl += xl[j], xsh += xh[j];
-    }
 
     const uint32_t rows_per_pass = R * RS;
     for (uint32_t rg = blockIdx.x * 4u + wave; rg < p.row_groups; rg += gridDim.x * 4u) {
@@ -214,44 +430,30 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(GemvParams p) {
             uint32_t n = weight_row(i < p.N ? i : 0u, p.N, p.swiglu);
             const uint8_t *matrix_end;
             const uint8_t *base = row_start(p, n, matrix_end) + (size_t)(blk0 + blk) * 144u;
-            if (active) {
-                hdr[r] = *reinterpret_cast<const uint4 *>(base);
-                qa[r] = *reinterpret_cast<const uint4 *>(base + 16u + g * 32u);
-                qb[r] = *reinterpret_cast<const uint4 *>(base + 32u + g * 32u);
-            } else {
-                hdr[r] = qa[r] = qb[r] = make_uint4(0u, 0u, 0u, 0u);
-            }
+            hdr[r] = *reinterpret_cast<const uint4 *>(base);
+            qa[r] = *reinterpret_cast<const uint4 *>(base + 16u + g * 32u);
+            qb[r] = *reinterpret_cast<const uint4 *>(base + 32u + g * 32u);
         }
         float acc[R][RB];
-        if (RB == 1) {
+#pragma unroll
+        for (int b = 0; b < RB; b++) {
+            const float4 *src = reinterpret_cast<const float4 *>(xs + b * xstride + skew64((blk * 4u + g) * 64u));
+            float xsl = 0.0f, xsh = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float4 a = active ? src[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+                float4 c = active ? src[8 + j] : make_float4(0.f, 0.f, 0.f, 0.f);
+                xl[4 * j] = a.x, xl[4 * j + 1] = a.y, xl[4 * j + 2] = a.z, xl[4 * j + 3] = a.w;
+                xh[4 * j] = c.x, xh[4 * j + 1] = c.y, xh[4 * j + 2] = c.z, xh[4 * j + 3] = c.w;
+            }
+#pragma unroll
+            for (int j = 0; j < 32; j++) xsl += xl[j], xsh += xh[j];
 #pragma unroll
             for (int r = 0; r < R; r++) {
                 float d0, d1, m0, m1, low, high;
                 group_scales(hdr[r], g, d0, d1, m0, m1);
                 nibble_dots(qa[r], qb[r], xl, xh, low, high);
-                acc[r][0] = (d0 * low + d1 * high) - (m0 * xsl + m1 * xsh);
-            }
-        } else {
-#pragma unroll
-            for (int b = 0; b < RB; b++) {
-                const float4 *src = reinterpret_cast<const float4 *>(xs + b * xstride + skew64((blk * 4u + g) * 64u));
-                xsl = 0.0f, xsh = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    float4 a = active ? src[j] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    float4 c = active ? src[8 + j] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    xl[4 * j] = a.x, xl[4 * j + 1] = a.y, xl[4 * j + 2] = a.z, xl[4 * j + 3] = a.w;
-                    xh[4 * j] = c.x, xh[4 * j + 1] = c.y, xh[4 * j + 2] = c.z, xh[4 * j + 3] = c.w;
-                }
-#pragma unroll
-                for (int j = 0; j < 32; j++) xsl += xl[j], xsh += xh[j];
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    float d0, d1, m0, m1, low, high;
-                    group_scales(hdr[r], g, d0, d1, m0, m1);
-                    nibble_dots(qa[r], qb[r], xl, xh, low, high);
-                    acc[r][b] = (d0 * low + d1 * high) - (m0 * xsl + m1 * xsh);
-                }
+                acc[r][b] = (d0 * (low * 16777216.0f) + d1 * (high * 1048576.0f)) - (m0 * xsl + m1 * xsh);
             }
         }
         // sum over the G lanes of the group
@@ -470,21 +672,28 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * RB * a.N * sizeof(float)));
         if (!p.partial) return NH_E_MEMORY;
     }
-    // rows per lane group and pass: more rows amortise the activation registers, fewer give
-    // more waves; keep at least ~8 waves per compute unit busy
-    int R = 4;
-    uint64_t waves_at_4 = (uint64_t)((a.N + 4 * RS - 1) / (4 * RS)) * p.splits;
-    if (waves_at_4 < (uint64_t)d->compute_units * 8) R = 2;
+    // rows per lane group and pass: four rows amortise the cross-lane sum and keep more bytes
+    // in flight per wave, two rows give twice the waves; tall matrices take four
+    int R = (a.N >= 16384u && RB == 1) ? 4 : 2;
     R = env_int("NEURA_HIP_GEMV_ROWS", R);
     if (R != 2 && R != 4) R = 2;
     if (RB >= 4) R = 2;
+    // the decode kernel walks R rows of ONE matrix per lane group: every matrix boundary must be a
+    // multiple of R (with swiglu the halves interleave, so N/2 must be a multiple of R/2)
+    auto whole = [&](int rows) {
+        if (a.swiglu) return a.N % (uint32_t)rows == 0 && a.end[0] == a.N / 2;
+        return a.end[0] % (uint32_t)rows == 0 && a.end[1] % (uint32_t)rows == 0 && a.N % (uint32_t)rows == 0;
+    };
+    if (R == 4 && !whole(4)) R = 2;
+    const bool fast = whole(R) && a.N >= (uint32_t)R && (uint64_t)a.N * p.row_bytes < (1ull << 32);
     uint32_t rows_per_pass = (uint32_t)R * RS;
     p.row_groups = (a.N + rows_per_pass - 1) / rows_per_pass;
     uint32_t blocks_x;
     size_t lds;
     if (q4) {
         blocks_x = (p.row_groups + 3) / 4;
-        uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_GEMV_WGS", 4) / p.splits;
+        // one resident round of workgroups: 3 per compute unit at four rows (136 registers), 4 at two
+        uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_GEMV_WGS", R == 4 ? 3 : 4) / p.splits;
         if (most < 1) most = 1;
         if (blocks_x > most) blocks_x = most;
         uint32_t slice = p.blocks_per_split * 256u;
@@ -502,9 +711,28 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     }
     if (lds > 64 * 1024) return fail(NH_E_ARGUMENT, "a product of depth %u stages %zu bytes where a workgroup holds 65536", a.K, lds);
     dim3 grid(blocks_x, p.splits), block(256);
+    const bool pipe = env_int("NEURA_HIP_GEMV_PIPE", 0) != 0;
+    const int nw = env_int("NEURA_HIP_GEMV_WAVES", 4);
     profile_mark(d);
 #define NH_LAUNCH(KERNEL, RR) hipLaunchKernelGGL((KERNEL<RR, RB>), grid, block, lds, d->stream, p)
-    if (q4) {
+#define NH_DECODE(RR, GG)                                                                                              \
+    do {                                                                                                               \
+        if (pipe) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, true, 4>), grid, block, lds, d->stream, p);       \
+        else if (nw == 16) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 16>), dim3((blocks_x + 3) / 4, p.splits), dim3(1024), lds, d->stream, p); \
+        else if (nw == 8) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 8>), dim3((blocks_x + 1) / 2, p.splits), dim3(512), lds, d->stream, p); \
+        else hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p);           \
+    } while (0)
+    if (q4 && RB == 1 && fast) {
+        if (R == 4) {
+            if (p.group == 64) NH_DECODE(4, 64);
+            else if (p.group == 32) NH_DECODE(4, 32);
+            else NH_DECODE(4, 16);
+        } else {
+            if (p.group == 64) NH_DECODE(2, 64);
+            else if (p.group == 32) NH_DECODE(2, 32);
+            else NH_DECODE(2, 16);
+        }
+    } else if (q4) {
         if (R == 4) NH_LAUNCH(gemv_q4k_kernel, 4);
         else NH_LAUNCH(gemv_q4k_kernel, 2);
     } else {
@@ -512,6 +740,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         else NH_LAUNCH(gemv_q8_0_kernel, 2);
     }
 #undef NH_LAUNCH
+#undef NH_DECODE
     NH_HIP(hipGetLastError());
     if (p.splits > 1) {
         uint32_t outputs = (a.swiglu ? a.N / 2 : a.N) * RB;
