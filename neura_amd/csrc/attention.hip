@@ -7,6 +7,7 @@
 // Every lane keeps a running (max, sum, accumulator) for its own key stream; streams are
 // merged with shuffles inside a wave, through LDS across waves, and across sections by a
 // second kernel (crates/neura-kernel/src/task/attention.rs:619-671 does the same fold).
+// The K/V rows of two steps ahead are always in flight.
 #include "blocks.hpp"
 #include "common.hpp"
 
@@ -17,7 +18,7 @@ constexpr int MAX_GROUPS = 8;
 struct AttentionParams {
     const float *q;
     float *out;
-    float *partial;  // [sections][heads][batch][rows][width + 2] when sections > 1
+    float *partial;      // [unit][section][group][width + 2] when sections > 1
     uint64_t q_sh, q_sb, q_sr, o_sh, o_sb, o_sr;
     const uint16_t *cache_k, *cache_v;
     uint32_t heads, kv_heads, groups, batch, rows, capacity, keys, sections;
@@ -38,6 +39,18 @@ __device__ __forceinline__ void unpack8(const uint4 &raw, float (&out)[8]) {
 // exp(max(argument, -104)) (crates/neura-kernel/src/substrate.rs:110-116)
 __device__ __forceinline__ float softmax_exp(float argument) { return expf(fmaxf(argument, -104.0f)); }
 
+// sum over the LPK lanes that share a key: DPP adds inside a row of 16 lanes
+template <int LPK>
+__device__ __forceinline__ float key_sum(float v) {
+    static_assert(LPK == 4 || LPK == 8 || LPK == 16 || LPK == 32, "lanes per key");
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));  // lane ^ 1
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));  // lane ^ 2
+    if (LPK >= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // half mirror: the other quad of 8
+    if (LPK >= 16) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // mirror: the other half of 16
+    if (LPK >= 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     constexpr int LPK = WIDTH / 8;   // lanes per key
@@ -45,10 +58,9 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     __shared__ float merged[4][MAX_GROUPS][WIDTH + 2];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t sub = lane / LPK, dl = lane % LPK;
-    uint32_t unit = blockIdx.x;  // (kv head, plane, row)
+    const uint32_t unit = blockIdx.x;  // (kv head, plane, row)
     const uint32_t row = unit % p.rows;
-    unit /= p.rows;
-    const uint32_t b = unit % p.batch, kvh = unit / p.batch;
+    const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
     const uint32_t section = blockIdx.y;
     const uint32_t G = p.groups;
 
@@ -60,6 +72,19 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     const uint32_t visible = min(p.keys, origin + row + 1u);  // key `at` counts iff at <= origin + row
     const uint32_t chunk = (visible + p.sections - 1u) / p.sections;
     const uint32_t first = min(visible, section * chunk), last = min(visible, first + chunk);
+
+    // K and V rows of the first two steps go out before anything else
+    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
+    const uint32_t step = 4u * KPW;
+    uint32_t key = first + wave * KPW + sub;
+    uint4 kraw[2], vraw[2];
+#pragma unroll
+    for (int ahead = 0; ahead < 2; ahead++) {
+        const uint32_t at_key = min(key + ahead * step, p.capacity - 1u);
+        const uint64_t at = (plane + at_key) * WIDTH + dl * 8u;
+        kraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_k + at);
+        vraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_v + at);
+    }
 
     float qr[MAX_GROUPS][8], acc[MAX_GROUPS][8], top[MAX_GROUPS], mass[MAX_GROUPS];
 #pragma unroll
@@ -74,30 +99,36 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
             for (int j = 0; j < 8; j++) qr[g][j] = src[j];
         }
     }
-    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
-    for (uint32_t key = first + wave * KPW + sub; key < last; key += 4u * KPW) {
-        const uint64_t at = (plane + key) * WIDTH + dl * 8u;
-        uint4 kraw = *reinterpret_cast<const uint4 *>(p.cache_k + at);
-        uint4 vraw = *reinterpret_cast<const uint4 *>(p.cache_v + at);
-        float kf[8], vf[8];
-        unpack8(kraw, kf);
-        unpack8(vraw, vf);
+    for (; key < last; key += 2u * step) {
 #pragma unroll
-        for (int g = 0; g < MAX_GROUPS; g++) {
-            if (g >= (int)G) break;
-            float score = 0.0f;
+        for (int phase = 0; phase < 2; phase++) {
+            const uint32_t now = key + phase * step;
+            float kf[8], vf[8];
+            unpack8(kraw[phase], kf);
+            unpack8(vraw[phase], vf);
+            {  // the loads of two steps ahead reuse this phase's registers
+                const uint32_t at_key = min(now + 2u * step, p.capacity - 1u);
+                const uint64_t at = (plane + at_key) * WIDTH + dl * 8u;
+                kraw[phase] = *reinterpret_cast<const uint4 *>(p.cache_k + at);
+                vraw[phase] = *reinterpret_cast<const uint4 *>(p.cache_v + at);
+            }
+            if (now < last) {
 #pragma unroll
-            for (int j = 0; j < 8; j++) score = fmaf(qr[g][j], kf[j], score);
+                for (int g = 0; g < MAX_GROUPS; g++) {
+                    if (g >= (int)G) break;
+                    float score = 0.0f;
 #pragma unroll
-            for (int offset = LPK / 2; offset > 0; offset >>= 1) score += __shfl_xor(score, offset, 64);
-            score *= p.scale;
-            float next = fmaxf(top[g], score);
-            float rescale = top[g] == -INFINITY ? 0.0f : softmax_exp(top[g] - next);
-            float weight = softmax_exp(score - next);
-            top[g] = next;
-            mass[g] = mass[g] * rescale + weight;
+                    for (int j = 0; j < 8; j++) score = fmaf(qr[g][j], kf[j], score);
+                    score = key_sum<LPK>(score) * p.scale;
+                    float next = fmaxf(top[g], score);
+                    float rescale = top[g] == -INFINITY ? 0.0f : softmax_exp(top[g] - next);
+                    float weight = softmax_exp(score - next);
+                    top[g] = next;
+                    mass[g] = fmaf(mass[g], rescale, weight);
 #pragma unroll
-            for (int j = 0; j < 8; j++) acc[g][j] = acc[g][j] * rescale + weight * vf[j];
+                    for (int j = 0; j < 8; j++) acc[g][j] = fmaf(acc[g][j], rescale, weight * vf[j]);
+                }
+            }
         }
     }
     // merge the KPW key streams of a wave: lanes with the same dl
@@ -142,7 +173,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
         }
         const uint32_t head = kvh * G + g;
         if (p.sections > 1) {
-            float *dst = p.partial + ((((uint64_t)section * p.heads + head) * p.batch + b) * p.rows + row) * (WIDTH + 2);
+            float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (WIDTH + 2);
             dst[c] = value;
             if (c == 0) {
                 dst[WIDTH] = largest;
@@ -155,28 +186,49 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     }
 }
 
-// combine the sections of one (head, plane, row): crates/neura-kernel/src/task/attention.rs:619-671
+// Fold of the sections of one (unit, query head): crates/neura-kernel/src/task/attention.rs:619-671.
+// One workgroup per (unit, group).  Thread s first turns the statistics of section s into its
+// weight, then thread c sums channel c over the sections with eight loads in flight.
 __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, uint32_t width) {
-    const uint32_t words = width + 2;
-    const uint64_t vectors = (uint64_t)p.heads * p.batch * p.rows;
-    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < vectors * width;
-         index += (uint64_t)gridDim.x * blockDim.x) {
-        uint64_t vector = index / width;
-        uint32_t c = (uint32_t)(index % width);
-        float largest = -INFINITY;
-        for (uint32_t s = 0; s < p.sections; s++) largest = fmaxf(largest, p.partial[(s * vectors + vector) * words + width]);
-        float total = 0.0f, value = 0.0f;
-        for (uint32_t s = 0; s < p.sections; s++) {
-            const float *src = p.partial + (s * vectors + vector) * words;
-            float weight = src[width] == -INFINITY ? 0.0f : softmax_exp(src[width] - largest);
-            total += src[width + 1] * weight;
-            value += src[c] * weight;
+    __shared__ float weights[256], masses[256], held[256];
+    const uint32_t G = p.groups, tid = threadIdx.x;
+    const uint32_t unit = blockIdx.x / G, g = blockIdx.x % G;
+    const uint32_t row = unit % p.rows;
+    const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
+    const float *src = p.partial + ((uint64_t)unit * p.sections * G + g) * (width + 2);
+    const uint64_t hop = (uint64_t)G * (width + 2);  // one section further
+    float top = -INFINITY, mass = 0.0f;
+    if (tid < p.sections) {
+        top = src[tid * hop + width];
+        mass = src[tid * hop + width + 1];
+    }
+    held[tid] = top;
+    __syncthreads();
+    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+        if (tid < stride) held[tid] = fmaxf(held[tid], held[tid + stride]);
+        __syncthreads();
+    }
+    const float largest = held[0];
+    const float weight = top == -INFINITY ? 0.0f : softmax_exp(top - largest);
+    weights[tid] = weight;
+    masses[tid] = mass * weight;
+    __syncthreads();
+    float total = 0.0f;
+    for (uint32_t s = 0; s < p.sections; s++) total += masses[s];
+    const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
+    for (uint32_t c = tid; c < width; c += 256) {
+        float sums[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        uint32_t s = 0;
+        for (; s + 8 <= p.sections; s += 8) {
+            float values[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) values[j] = src[(s + j) * hop + c];
+#pragma unroll
+            for (int j = 0; j < 8; j++) sums[j] = fmaf(values[j], weights[s + j], sums[j]);
         }
-        float normalized = total > 0.0f ? 1.0f / total : 0.0f;
-        uint32_t row = (uint32_t)(vector % p.rows);
-        uint32_t b = (uint32_t)((vector / p.rows) % p.batch);
-        uint32_t head = (uint32_t)(vector / p.rows / p.batch);
-        p.out[(uint64_t)head * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr + c] = value * normalized;
+        for (; s < p.sections; s++) sums[0] = fmaf(src[s * hop + c], weights[s], sums[0]);
+        float value = ((sums[0] + sums[1]) + (sums[2] + sums[3])) + ((sums[4] + sums[5]) + (sums[6] + sums[7]));
+        p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr + c] = value * normalized;
     }
 }
 
@@ -191,10 +243,12 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
-    // enough sections to put ~2 workgroups on every compute unit, none thinner than 64 keys
-    uint32_t wanted = ((uint32_t)d->compute_units * 2 + units - 1) / units;
-    uint32_t most = (a.keys + 63) / 64;
+    // sections of the context: enough workgroups to fill the chip four times over, none thinner
+    // than 32 keys
+    uint32_t wanted = ((uint32_t)d->compute_units * 4 + units - 1) / units;
+    uint32_t most = (a.keys + 31) / 32;
     p.sections = wanted < 1 ? 1 : (wanted > most ? most : wanted);
+    if (p.sections > 256) p.sections = 256;
     if (p.sections > 1) {
         p.partial = static_cast<float *>(scratch(d, (size_t)p.sections * a.heads * a.batch * a.rows * (a.width + 2) * sizeof(float)));
         if (!p.partial) return NH_E_MEMORY;
@@ -209,9 +263,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     NH_HIP(hipGetLastError());
     if (p.sections > 1) {
-        uint64_t outputs = (uint64_t)a.heads * a.batch * a.rows * a.width;
-        uint32_t blocks = (uint32_t)((outputs + 255) / 256 < 65535 ? (outputs + 255) / 256 : 65535);
-        hipLaunchKernelGGL(attention_fold_kernel, dim3(blocks), dim3(256), 0, d->stream, p, a.width);
+        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups), dim3(256), 0, d->stream, p, a.width);
         NH_HIP(hipGetLastError());
     }
     return NH_OK;
