@@ -9,8 +9,8 @@ output head, the greedy choice and the read-back of the chosen token.  Weights a
 resident in HBM before the timed region.  Prints ONE JSON line:
   value        tokens/s over the K timed steps (host clock around device-synchronised steps)
   roofline     the Q4_K narrow product: weight bytes each launch walks / its device time,
-               measured with HIP event pairs around every launch (a profiled pass of the same
-               steps on the same stream), against MI355X's 8 TB/s HBM peak
+               measured with HIP events around back-to-back passes over the 113 product
+               launches of a decode step on the same stream, against MI355X's 8 TB/s HBM peak
   cpu_baseline the CPU oracle (a port of the reference path, OpenMP over output columns) on
                the host cores, timed on a bounded sample of the same workload
 """
@@ -26,6 +26,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one Q4_K product launch of the 7B-shape decode step moves on average, from the
+# rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_q4k_decode_hbm_counters.md
+# (each counter scaled by its reading for a plain 1 GiB copy); not measurable inside this script
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 36.06e6}
 
 
 def workload(name):
@@ -94,6 +98,8 @@ def main():
     parser.add_argument("--workload", default="qwen2.5-7b-q4k")
     parser.add_argument("--layers", type=int, default=None, help="cut the decoder (for quick checks; the result is then not the headline)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                        help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -115,6 +121,13 @@ def main():
         for which in (0, 1):
             model.cache_write(layer, which, rng.standard_normal(model.cache_shape).astype(np.float16).view(np.uint16))
 
+    if args.calibrate_copy:
+        nbytes = args.calibrate_copy << 20
+        source, target = device.alloc(nbytes), device.alloc(nbytes)
+        for _ in range(4):
+            assert device.lib.nh_copy(device.handle, target.pointer, source.pointer, nbytes) == 0
+        device.sync()
+
     total = args.warmup + args.steps
     first_cursor = context - total  # the last timed step sits at cursor context - 1
     assert first_cursor >= 0, "more steps than the context holds"
@@ -128,12 +141,10 @@ def main():
     device.sync()
     elapsed = time.perf_counter() - began
 
-    # profiled pass: the same steps again with an event pair around every narrow product
-    profiled = min(args.steps, 16)
-    device.profile_begin()
-    for step in range(profiled):
-        token = int(model.decode_step([token], [context - profiled + step])[0])
-    gemv_seconds, launches, walked = device.profile_end()
+    # the dominant kernel alone: every narrow product of a decode step (same matrices, shapes
+    # and buffers), launched back to back between one pair of HIP events on the same stream
+    profiled = min(args.steps, 32)
+    gemv_seconds, launches, walked = model.time_products(profiled)
     per_launch_bytes = walked / launches
     per_launch_seconds = gemv_seconds / launches
     achieved = per_launch_bytes / per_launch_seconds / 1e9
@@ -163,7 +174,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if args.layers is None else None,
             "bytes_per_launch": per_launch_bytes,
             "us_per_launch": per_launch_seconds * 1e6,
             "launches_per_step": launches / profiled,

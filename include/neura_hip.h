@@ -71,6 +71,8 @@ int32_t nh_free(nh_device *device, void *dev);
  * complete on return */
 int32_t nh_upload(nh_device *device, void *dev_dst, const void *host_src, size_t bytes);
 int32_t nh_download(nh_device *device, void *host_dst, const void *dev_src, size_t bytes);
+/* Command::Copy (crates/neura-gpu/src/submission.rs:17-35): device to device, enqueued */
+int32_t nh_copy(nh_device *device, void *dev_dst, const void *dev_src, size_t bytes);
 /* Command::Clear (crates/neura-gpu/src/submission.rs:17-35) */
 int32_t nh_clear(nh_device *device, void *dev, size_t bytes);
 /* NativeDevice::wait (crates/neura-gpu/src/native.rs:231-425) */
@@ -177,6 +179,12 @@ int32_t nh_decode_step(nh_model *model, const uint32_t *tokens, const uint32_t *
 /* a fill program (crates/neura-generate/src/batch.rs:1434-1517): `rows` tokens per plane,
  * tokens[row * batch + plane]; no logits, no readback. */
 int32_t nh_prefill(nh_model *model, const uint32_t *tokens, uint32_t rows, const uint32_t *cursors, const uint8_t *mask, uint32_t batch);
+/* Runtime::measure restricted to the products (crates/neura-runtime/src/runtime.rs:807-816,
+ * examples/benchmark/product.rs:19-107): launches every narrow product of one decode step
+ * (same matrices, shapes and buffers, nothing else) `steps` times back to back on the device's
+ * stream between one pair of HIP events.  Returns the device seconds, the number of product
+ * launches and the weight payload bytes they walked. */
+int32_t nh_model_time_products(nh_model *model, uint32_t steps, double *seconds_out, uint64_t *launches_out, uint64_t *bytes_out);
 /* the reset program (crates/neura-generate/src/batch.rs:1094-1100): zero the caches of planes
  * whose reset byte is non-zero */
 int32_t nh_model_reset(nh_model *model, const uint8_t *reset, uint32_t batch);

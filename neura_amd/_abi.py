@@ -40,6 +40,7 @@ SIGNATURES = {
     "nh_free": (c_int32, [c_void_p, c_void_p]),
     "nh_upload": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "nh_download": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "nh_copy": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "nh_clear": (c_int32, [c_void_p, c_void_p, c_size_t]),
     "nh_sync": (c_int32, [c_void_p]),
     "nh_timer_start": (c_int32, [c_void_p]),
@@ -67,6 +68,7 @@ SIGNATURES = {
     "nh_model_destroy": (None, [c_void_p]),
     "nh_decode_step": (c_int32, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint8), c_uint32, POINTER(c_uint32)]),
     "nh_prefill": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32, POINTER(c_uint32), POINTER(c_uint8), c_uint32]),
+    "nh_model_time_products": (c_int32, [c_void_p, c_uint32, POINTER(c_double), POINTER(c_uint64), POINTER(c_uint64)]),
     "nh_model_reset": (c_int32, [c_void_p, POINTER(c_uint8), c_uint32]),
     "nh_model_logits": (c_int32, [c_void_p, c_void_p]),
     "nh_model_cache_write": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),

@@ -3,6 +3,7 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -27,6 +28,9 @@ struct nh_model {
     uint8_t *inputs_host = nullptr;  // pinned mirror of inputs_dev
     uint32_t *chosen_host = nullptr; // pinned [B + 1]: chosen tokens, then the refusal word
     uint32_t max_tokens = 0;
+    // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked
+    hipGraphExec_t decode_graph[2] = {nullptr, nullptr};
+    bool use_graph = true;
 };
 
 namespace {
@@ -36,6 +40,8 @@ uint32_t qkv_width(const nh_model *m) { return (m->c.heads + 2 * m->c.kv_heads) 
 void release(nh_model *m) {
     if (!m) return;
     (void)hipStreamSynchronize(m->d->stream);
+    for (hipGraphExec_t graph : m->decode_graph)
+        if (graph) (void)hipGraphExecDestroy(graph);
     for (auto p : m->cache_k) (void)hipFree(p);
     for (auto p : m->cache_v) (void)hipFree(p);
     float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits};
@@ -82,7 +88,7 @@ GemvArgs narrow(const nh_model *m, const uint8_t *W, uint32_t N, uint32_t K, con
 }
 
 // all layers over T = rows * batch token rows whose inputs are already staged on the device
-int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
+int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_only = false) {
     nh_device *d = m->d;
     const nh_model_config &c = m->c;
     const uint32_t B = c.batch, T = rows * B, H = c.hidden, hd = c.head_dim;
@@ -90,7 +96,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
     const uint8_t *mask = any_inactive ? dev_mask(m) : nullptr;
     const bool wide = T > 8;  // more rows than the narrow product takes
     int32_t status;
-    if ((status = launch_gather(d, m->element, m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK) return status;
+    if (!products_only && (status = launch_gather(d, m->element, m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK)
+        return status;
     const float scale = 1.0f / sqrtf((float)hd);
     for (uint32_t L = 0; L < c.layers; L++) {
         if (wide) {
@@ -110,8 +117,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
             if ((status = launch_gemv(d, a)) != NH_OK) return status;
         }
-        if ((status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L], m->capacity, m->window,
-                                         dev_cursor(m), mask, c.rope_base)) != NH_OK)
+        if (!products_only && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
+                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base)) != NH_OK)
             return status;
         AttentionArgs at{};
         at.q = m->qkv, at.out = m->att;
@@ -120,7 +127,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
         at.cache_k = m->cache_k[L], at.cache_v = m->cache_v[L];
         at.heads = c.heads, at.kv_heads = c.kv_heads, at.batch = B, at.rows = rows, at.width = hd;
         at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
-        if ((status = launch_attention(d, at)) != NH_OK) return status;
+        if (!products_only && (status = launch_attention(d, at)) != NH_OK) return status;
         if (wide) {
             GemmArgs o{m->element, m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
             if ((status = launch_gemm(d, o)) != NH_OK) return status;
@@ -145,9 +152,20 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive) {
             dn.residual = m->h;
             if ((status = launch_gemv(d, dn)) != NH_OK) return status;
         }
-        if (mask && (status = launch_mask_rows(d, m->h, rows, B, H, mask)) != NH_OK) return status;
+        if (!products_only && mask && (status = launch_mask_rows(d, m->h, rows, B, H, mask)) != NH_OK) return status;
     }
     return NH_OK;
+}
+
+// every kernel of one decode step: the layers, then logits = rms(hidden) . head^T and the greedy
+// choice (examples/qwen/model.rs:81-84, crates/neura-generate/src/sampling.rs:69-71)
+int32_t decode_kernels(nh_model *m, bool any_inactive) {
+    int32_t status;
+    if ((status = forward(m, 1, any_inactive)) != NH_OK) return status;
+    GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+    head.norm_w = m->output_norm, head.eps = m->c.eps;
+    if ((status = launch_gemv(m->d, head)) != NH_OK) return status;
+    return launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
 }
 
 }  // namespace
@@ -248,6 +266,22 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     }
     ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 2 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
          hipHostMalloc((void **)&m->chosen_host, ((size_t)c.batch + 1) * 4, hipHostMallocDefault) == hipSuccess;
+    // everything a captured step touches exists before the capture: the split partials of the
+    // products (at most 5 slices x 4 rows), of the attention (at most 256 sections) and of the
+    // greedy choice, and the rope table
+    {
+        size_t widest = (size_t)(2 * F > c.vocab ? 2 * F : c.vocab);
+        size_t products = 8 * 4 * widest * sizeof(float);
+        size_t sections = (size_t)256 * c.heads * T * (c.head_dim + 2) * sizeof(float);
+        size_t choice = (size_t)c.batch * 1024 * 8;
+        size_t wanted = products > sections ? products : sections;
+        if (choice > wanted) wanted = choice;
+        ok = ok && scratch(device, wanted) != nullptr && rope_frequencies(device, c.rope_base, c.head_dim) != nullptr;
+    }
+    {
+        const char *held = getenv("NEURA_HIP_GRAPH");
+        m->use_graph = !(held && held[0] == '0');
+    }
     ok = ok && hipStreamSynchronize(device->stream) == hipSuccess;
     if (!ok) {
         fail(NH_E_MEMORY, "device %d holds no caches and activations of this decoder", device->index);
@@ -276,13 +310,32 @@ int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *curs
     nh_device *d = m->d;
     int32_t status;
     if ((status = stage_inputs(m, tokens, batch, cursors, mask, batch)) != NH_OK) return status;
-    if ((status = forward(m, 1, any_inactive)) != NH_OK) return status;
-    // logits = rms(hidden) . head^T, then the greedy choice (examples/qwen/model.rs:81-84,
-    // crates/neura-generate/src/sampling.rs:69-71)
-    GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, batch, m->logits);
-    head.norm_w = m->output_norm, head.eps = m->c.eps;
-    if ((status = launch_gemv(d, head)) != NH_OK) return status;
-    if ((status = launch_argmax(d, m->logits, batch, m->c.vocab, m->chosen_dev)) != NH_OK) return status;
+    // Every kernel of the step reads its token, cursor and mask from device memory and no launch
+    // shape depends on them, so the step is captured once per mask variant and replayed.
+    // Profiled steps run eagerly (event records do not belong in a graph).
+    hipGraphExec_t &graph = m->decode_graph[any_inactive ? 1 : 0];
+    if (m->use_graph && !d->profile) {
+        if (!graph) {
+            NH_HIP(hipStreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal));
+            status = decode_kernels(m, any_inactive);
+            hipGraph_t recorded = nullptr;
+            hipError_t ended = hipStreamEndCapture(d->stream, &recorded);
+            if (status != NH_OK) {
+                if (recorded) (void)hipGraphDestroy(recorded);
+                return status;
+            }
+            if (ended != hipSuccess) return hip_fail(ended, "hipStreamEndCapture");
+            hipError_t built = hipGraphInstantiate(&graph, recorded, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(recorded);
+            if (built != hipSuccess) {
+                graph = nullptr;
+                return hip_fail(built, "hipGraphInstantiate");
+            }
+        }
+        NH_HIP(hipGraphLaunch(graph, d->stream));
+    } else if ((status = decode_kernels(m, any_inactive)) != NH_OK) {
+        return status;
+    }
     NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
     NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
     NH_HIP(hipStreamSynchronize(d->stream));
@@ -307,6 +360,36 @@ int32_t nh_prefill(nh_model *m, const uint32_t *tokens, uint32_t rows, const uin
     if ((status = stage_inputs(m, tokens, rows * batch, cursors, mask, batch)) != NH_OK) return status;
     if ((status = forward(m, rows, any_inactive)) != NH_OK) return status;
     return check_refusal(m->d, "a fill");
+}
+
+int32_t nh_model_time_products(nh_model *m, uint32_t steps, double *seconds_out, uint64_t *launches_out, uint64_t *bytes_out) {
+    NH_REQUIRE(m && steps && seconds_out && launches_out && bytes_out, "a product timing names no model, no step or no result");
+    nh_device *d = m->d;
+    // count launches and bytes with the per-launch profile of one untimed pass, then time
+    // `steps` passes of the same launches between one pair of events
+    int32_t status;
+    if ((status = nh_profile_begin(d)) != NH_OK) return status;
+    status = forward(m, 1, false, true);
+    if (status == NH_OK) {
+        GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+        head.norm_w = m->output_norm, head.eps = m->c.eps;
+        status = launch_gemv(d, head);
+    }
+    double ignored = 0.0;
+    int32_t ended = nh_profile_end(d, &ignored, launches_out, bytes_out);
+    if (status != NH_OK) return status;
+    if (ended != NH_OK) return ended;
+    if ((status = nh_timer_start(d)) != NH_OK) return status;
+    for (uint32_t step = 0; step < steps; step++) {
+        if ((status = forward(m, 1, false, true)) != NH_OK) return status;
+        GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+        head.norm_w = m->output_norm, head.eps = m->c.eps;
+        if ((status = launch_gemv(d, head)) != NH_OK) return status;
+    }
+    if ((status = nh_timer_stop(d, seconds_out)) != NH_OK) return status;
+    *launches_out *= steps;
+    *bytes_out *= steps;
+    return NH_OK;
 }
 
 int32_t nh_model_reset(nh_model *m, const uint8_t *reset, uint32_t batch) {

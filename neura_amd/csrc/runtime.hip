@@ -193,6 +193,13 @@ int32_t nh_download(nh_device *device, void *host_dst, const void *dev_src, size
     return NH_OK;
 }
 
+int32_t nh_copy(nh_device *device, void *dev_dst, const void *dev_src, size_t bytes) {
+    NH_REQUIRE(device && (bytes == 0 || (dev_dst && dev_src)), "a copy of %zu bytes names no buffer", bytes);
+    if (!bytes) return NH_OK;
+    NH_HIP(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, device->stream));
+    return NH_OK;
+}
+
 int32_t nh_clear(nh_device *device, void *dev, size_t bytes) {
     NH_REQUIRE(device && (bytes == 0 || dev), "a clear of %zu bytes names no buffer", bytes);
     if (!bytes) return NH_OK;

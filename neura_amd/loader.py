@@ -104,6 +104,12 @@ class Model:
         _check(self.lib.nh_prefill(self.handle, tokens.ctypes.data_as(u32), rows, cursors.ctypes.data_as(u32), mask.ctypes.data_as(u8),
                                    self.batch))
 
+    def time_products(self, steps):
+        """(device seconds, launches, weight bytes) of `steps` back-to-back passes over the narrow products of a decode step"""
+        seconds, launches, nbytes = ctypes.c_double(), ctypes.c_uint64(), ctypes.c_uint64()
+        _check(self.lib.nh_model_time_products(self.handle, steps, ctypes.byref(seconds), ctypes.byref(launches), ctypes.byref(nbytes)))
+        return seconds.value, launches.value, nbytes.value
+
     def reset(self, flags):
         flags = np.ascontiguousarray(flags, dtype=np.uint8)
         _check(self.lib.nh_model_reset(self.handle, flags.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), self.batch))
