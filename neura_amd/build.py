@@ -52,5 +52,23 @@ def build_library(verbose=True):
     return LIBRARY
 
 
+HOST_LIBRARY = os.path.join(HERE, "libneura_host.so")
+
+
+def build_host(verbose=True):
+    """The C++ host layer (GGUF reader, decoder declarations, generation batch) over the C ABI,
+    with its flat C surface; plain g++, no device code.  Links against libneura_hip.so."""
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared",
+           os.path.join(HERE, "host", "capi.cpp"), "-o", HOST_LIBRARY,
+           "-L" + HERE, "-lneura_hip", "-Wl,-rpath,$ORIGIN"]
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError("host build failed:\n%s\n%s" % (" ".join(cmd), done.stderr))
+    if verbose and done.stderr.strip():
+        print(done.stderr, file=sys.stderr)
+    return HOST_LIBRARY
+
+
 if __name__ == "__main__":
     print(build_library())
+    print(build_host())

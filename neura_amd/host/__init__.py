@@ -1,0 +1,356 @@
+"""ctypes face of libneura_host.so: the C++ host layer (neura.hpp) behind a flat C surface.
+
+The classes here read like the reference's own (Gguf, GgufFile, Batch); a refusal of the
+C++ layer -- a panic of the reference -- surfaces as `Panic` carrying the same sentence.
+Loading touches no GPU; only Runtime() does.
+"""
+import ctypes
+import os
+from ctypes import POINTER, byref, c_char_p, c_double, c_float, c_int32, c_int64, c_size_t, c_uint32, c_uint64, c_void_p
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY = os.path.join(os.path.dirname(HERE), "libneura_host.so")
+
+
+class Panic(RuntimeError):
+    pass
+
+
+class TensorInfo(ctypes.Structure):
+    _fields_ = [("element", c_int32), ("rank", c_uint32), ("elements", c_uint64), ("shape", c_uint64 * 4), ("at", c_uint64), ("bytes", c_uint64)]
+
+
+SIGNATURES = {
+    "nhost_last_error": (c_char_p, []),
+    "nhost_gguf_decode": (c_void_p, [c_void_p, c_size_t]),
+    "nhost_gguf_open": (c_void_p, [c_char_p]),
+    "nhost_gguf_close": (None, [c_void_p]),
+    "nhost_gguf_tensors": (c_uint64, [c_void_p]),
+    "nhost_gguf_reads": (c_uint64, [c_void_p]),
+    "nhost_gguf_tensor": (c_int32, [c_void_p, c_char_p, POINTER(TensorInfo)]),
+    "nhost_gguf_has": (c_int32, [c_void_p, c_char_p]),
+    "nhost_gguf_word": (c_int32, [c_void_p, c_char_p, POINTER(c_uint32)]),
+    "nhost_gguf_single": (c_int32, [c_void_p, c_char_p, POINTER(c_float)]),
+    "nhost_gguf_flag": (c_int32, [c_void_p, c_char_p, POINTER(c_int32)]),
+    "nhost_gguf_text": (c_int64, [c_void_p, c_char_p, c_void_p, c_size_t]),
+    "nhost_gguf_integer": (c_int32, [c_void_p, c_char_p, POINTER(c_uint64)]),
+    "nhost_gguf_array_len": (c_int64, [c_void_p, c_char_p]),
+    "nhost_gguf_array_text": (c_int64, [c_void_p, c_char_p, c_uint64, c_void_p, c_size_t]),
+    "nhost_gguf_array_number": (c_int64, [c_void_p, c_char_p, c_uint64, POINTER(c_double)]),
+    "nhost_gguf_payload": (c_int64, [c_void_p, c_char_p, c_void_p, c_size_t]),
+    "nhost_gguf_placed": (c_int32, [c_void_p, c_char_p, POINTER(c_int32), POINTER(c_uint64), POINTER(c_float), POINTER(c_uint64), POINTER(c_uint64)]),
+    "nhost_writer_new": (c_void_p, [c_uint64]),
+    "nhost_writer_free": (None, [c_void_p]),
+    "nhost_writer_u32": (None, [c_void_p, c_char_p, c_uint32]),
+    "nhost_writer_f32": (None, [c_void_p, c_char_p, c_float]),
+    "nhost_writer_text": (None, [c_void_p, c_char_p, c_char_p]),
+    "nhost_writer_tensor": (None, [c_void_p, c_char_p, c_int32, POINTER(c_uint64), c_uint32, c_void_p, c_size_t]),
+    "nhost_writer_save": (c_int32, [c_void_p, c_char_p]),
+    "nhost_matrix": (c_int32, [c_void_p, c_char_p, c_uint32, c_uint32, POINTER(c_int32)]),
+    "nhost_vector": (c_int32, [c_void_p, c_char_p, c_uint32, POINTER(c_int32)]),
+    "nhost_cache_validate": (c_int32, [c_char_p] + [c_uint32] * 6 + [c_int32]),
+    "nhost_payload_bytes": (c_uint64, [c_int32, c_uint64]),
+    "nhost_runtime_open": (c_void_p, [c_int32]),
+    "nhost_runtime_close": (None, [c_void_p]),
+    "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_close": (None, [c_void_p]),
+    "nhost_batch_admit": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_restart": (c_int32, [c_void_p, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_resume": (c_int32, [c_void_p, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_suspend": (c_int32, [c_void_p, c_uint32]),
+    "nhost_batch_finish": (c_int32, [c_void_p, c_uint32]),
+    "nhost_batch_step": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_cursor": (c_int64, [c_void_p, c_uint32]),
+    "nhost_batch_remaining": (c_int64, [c_void_p, c_uint32]),
+    "nhost_batch_planes": (c_uint64, [c_void_p]),
+    "nhost_batch_logits": (c_int32, [c_void_p, c_void_p]),
+}
+
+_lib = None
+
+
+def library():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIBRARY):
+            raise RuntimeError("%s is not built: run `python -m neura_amd.build`" % LIBRARY)
+        lib = ctypes.CDLL(LIBRARY)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            entry = getattr(lib, name)
+            entry.restype, entry.argtypes = restype, argtypes
+        _lib = lib
+    return _lib
+
+
+def _refused():
+    return Panic(library().nhost_last_error().decode("utf-8", "replace"))
+
+
+def _words(values):
+    held = (c_uint32 * max(len(values), 1))(*[int(v) for v in values])
+    return held, len(values)
+
+
+class _Archive:
+    """What Gguf and GgufFile share: metadata accessors, the tensor table, Source."""
+
+    handle = None
+
+    def close(self):
+        if self.handle:
+            library().nhost_gguf_close(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        self.close()
+
+    def tensors(self):
+        return int(library().nhost_gguf_tensors(self.handle))
+
+    def tensor(self, name):
+        info = TensorInfo()
+        if not library().nhost_gguf_tensor(self.handle, name.encode(), byref(info)):
+            return None
+        return {"element": info.element, "elements": info.elements, "shape": list(info.shape), "rank": info.rank, "at": info.at, "bytes": info.bytes}
+
+    def has(self, key):
+        return bool(library().nhost_gguf_has(self.handle, key.encode()))
+
+    def word(self, key):
+        out = c_uint32()
+        if library().nhost_gguf_word(self.handle, key.encode(), byref(out)) != 0:
+            raise _refused()
+        return out.value
+
+    def optional_word(self, key):
+        return self.word(key) if self.has(key) else None
+
+    def single(self, key):
+        out = c_float()
+        if library().nhost_gguf_single(self.handle, key.encode(), byref(out)) != 0:
+            raise _refused()
+        return out.value
+
+    def flag(self, key):
+        out = c_int32()
+        if library().nhost_gguf_flag(self.handle, key.encode(), byref(out)) != 0:
+            raise _refused()
+        return bool(out.value)
+
+    def text(self, key):
+        room = ctypes.create_string_buffer(1 << 16)
+        length = library().nhost_gguf_text(self.handle, key.encode(), room, len(room))
+        if length < 0:
+            raise _refused()
+        return room.raw[:length].decode()
+
+    def integer(self, key):
+        out = c_uint64()
+        status = library().nhost_gguf_integer(self.handle, key.encode(), byref(out))
+        if status < 0:
+            raise _refused()
+        return out.value if status else None
+
+    def array_len(self, key):
+        length = library().nhost_gguf_array_len(self.handle, key.encode())
+        if length < 0:
+            raise _refused()
+        return length
+
+    def texts(self, key):
+        out = []
+        room = ctypes.create_string_buffer(1 << 12)
+        for index in range(self.array_len(key)):
+            length = library().nhost_gguf_array_text(self.handle, key.encode(), index, room, len(room))
+            if length < 0:
+                raise _refused()
+            out.append(room.raw[:length].decode())
+        return out
+
+    def numbers(self, key):
+        out = []
+        for index in range(self.array_len(key)):
+            held = c_double()
+            status = library().nhost_gguf_array_number(self.handle, key.encode(), index, byref(held))
+            if status < 0:
+                raise _refused()
+            out.append(held.value if status else None)
+        return out
+
+    def placed(self, name):
+        element, elements, scale, payload, table = c_int32(), c_uint64(), c_float(), c_uint64(), c_uint64()
+        if not library().nhost_gguf_placed(self.handle, name.encode(), byref(element), byref(elements), byref(scale), byref(payload), byref(table)):
+            return None
+        return {"element": element.value, "elements": elements.value, "scale": scale.value, "payload_bytes": payload.value, "table_bytes": table.value}
+
+    def payload(self, name):
+        placed = self.placed(name)
+        room = np.empty(placed["payload_bytes"] if placed else 0, dtype=np.uint8)
+        length = library().nhost_gguf_payload(self.handle, name.encode(), room.ctypes.data, room.size)
+        if length < 0:
+            raise _refused()
+        return room.tobytes()
+
+    def matrix(self, name, rows, columns):
+        element = c_int32()
+        if library().nhost_matrix(self.handle, name.encode(), rows, columns, byref(element)) != 0:
+            raise _refused()
+        return element.value
+
+    def vector(self, name, width):
+        element = c_int32()
+        if library().nhost_vector(self.handle, name.encode(), width, byref(element)) != 0:
+            raise _refused()
+        return element.value
+
+
+class Gguf(_Archive):
+    @classmethod
+    def decode(cls, data):
+        held = np.frombuffer(bytes(data), dtype=np.uint8)
+        out = cls()
+        out.handle = library().nhost_gguf_decode(held.ctypes.data if held.size else None, held.size)
+        if not out.handle:
+            raise _refused()
+        return out
+
+
+class GgufFile(_Archive):
+    @classmethod
+    def open(cls, path):
+        out = cls()
+        out.handle = library().nhost_gguf_open(os.fspath(path).encode())
+        if not out.handle:
+            raise _refused()
+        return out
+
+    def reads(self):
+        return int(library().nhost_gguf_reads(self.handle))
+
+
+class Writer:
+    def __init__(self, alignment=32):
+        self.handle = library().nhost_writer_new(alignment)
+
+    def u32(self, key, value):
+        library().nhost_writer_u32(self.handle, key.encode(), value)
+
+    def f32(self, key, value):
+        library().nhost_writer_f32(self.handle, key.encode(), value)
+
+    def text(self, key, value):
+        library().nhost_writer_text(self.handle, key.encode(), value.encode())
+
+    def tensor(self, name, element, shape, payload):
+        held = np.frombuffer(bytes(payload), dtype=np.uint8)
+        dims = (c_uint64 * len(shape))(*shape)
+        library().nhost_writer_tensor(self.handle, name.encode(), element, dims, len(shape), held.ctypes.data if held.size else None, held.size)
+
+    def save(self, path):
+        if library().nhost_writer_save(self.handle, os.fspath(path).encode()) != 0:
+            raise _refused()
+
+    def __del__(self):
+        if self.handle:
+            library().nhost_writer_free(self.handle)
+            self.handle = None
+
+
+def cache_validate(name, heads, width, capacity, window, batch, rows, element=1):
+    if library().nhost_cache_validate(name.encode(), heads, width, capacity, window, batch, rows, element) != 0:
+        raise _refused()
+
+
+def batch_spec_check(context, batch, chunks):
+    held, count = _words(chunks)
+    if library().nhost_batch_spec_check(context, batch, held, count) != 0:
+        raise _refused()
+
+
+def payload_bytes(element, elements):
+    return int(library().nhost_payload_bytes(element, elements))
+
+
+class Runtime:
+    def __init__(self, index=0):
+        self.handle = library().nhost_runtime_open(index)
+        if not self.handle:
+            raise _refused()
+
+    def close(self):
+        if self.handle:
+            library().nhost_runtime_close(self.handle)
+            self.handle = None
+
+
+class Batch:
+    """A Qwen2 GGUF loaded onto a runtime with a greedy generation batch above it."""
+
+    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=()):
+        held, count = _words(chunks)
+        self.planes = batch
+        self.vocabulary = vocabulary
+        self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count)
+        if not self.handle:
+            raise _refused()
+
+    def close(self):
+        if self.handle:
+            library().nhost_batch_close(self.handle)
+            self.handle = None
+
+    def _status(self, status):
+        if status < 0:
+            raise _refused()
+        return status
+
+    def admit(self, tokens):
+        held, count = _words(tokens)
+        return self._status(library().nhost_batch_admit(self.handle, held, count))
+
+    def restart(self, slot, tokens):
+        held, count = _words(tokens)
+        self._status(library().nhost_batch_restart(self.handle, slot, held, count))
+
+    def resume(self, slot, tokens):
+        held, count = _words(tokens)
+        self._status(library().nhost_batch_resume(self.handle, slot, held, count))
+
+    def suspend(self, slot):
+        self._status(library().nhost_batch_suspend(self.handle, slot))
+
+    def finish(self, slot):
+        self._status(library().nhost_batch_finish(self.handle, slot))
+
+    def step(self):
+        room = (c_uint32 * (2 * self.planes))()
+        count = self._status(library().nhost_batch_step(self.handle, room, self.planes))
+        return [(room[2 * i], room[2 * i + 1]) for i in range(count)]
+
+    def cursor(self, slot):
+        at = library().nhost_batch_cursor(self.handle, slot)
+        if at == -2:
+            raise _refused()
+        return None if at < 0 else at
+
+    def remaining(self, slot):
+        left = library().nhost_batch_remaining(self.handle, slot)
+        if left == -2:
+            raise _refused()
+        return None if left < 0 else left
+
+    def active(self):
+        planes = library().nhost_batch_planes(self.handle)
+        return [slot for slot in range(self.planes) if planes >> slot & 1]
+
+    def occupied(self):
+        planes = library().nhost_batch_planes(self.handle)
+        return [slot for slot in range(self.planes) if planes >> (32 + slot) & 1]
+
+    def logits(self):
+        out = np.empty((self.planes, self.vocabulary), dtype=np.float32)
+        self._status(library().nhost_batch_logits(self.handle, out.ctypes.data))
+        return out

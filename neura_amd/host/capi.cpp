@@ -1,0 +1,254 @@
+// capi.cpp -- a flat C surface over neura.hpp so the host layer can be driven from scripts and
+// tests without a C++ compiler in the loop.  Every call that can be refused returns a status
+// (0 done, -1 refused) or a null handle, and nhost_last_error() then holds the sentence the
+// reference would have panicked with.
+#include "neura.hpp"
+
+#include <cstdlib>
+
+using namespace neura;
+
+namespace {
+thread_local std::string last_error;
+
+template <typename F>
+auto guarded(F &&body, decltype(body()) refused) -> decltype(body()) {
+    try {
+        return body();
+    } catch (const std::exception &held) {
+        last_error = held.what();
+        return refused;
+    }
+}
+
+struct Opened {
+    std::unique_ptr<gguf::Gguf> whole;
+    std::unique_ptr<gguf::GgufFile> file;
+    const gguf::Archive &archive() const { return whole ? static_cast<const gguf::Archive &>(*whole) : *file; }
+    const gguf::Source &source() const { return whole ? static_cast<const gguf::Source &>(*whole) : *file; }
+};
+
+struct Loaded {
+    std::unique_ptr<generate::Model> model;
+    std::unique_ptr<generate::Batch> batch;
+};
+}  // namespace
+
+struct nhost_tensor {
+    int32_t element;
+    uint32_t rank;
+    uint64_t elements, shape[4], at, bytes;
+};
+
+extern "C" {
+
+const char *nhost_last_error(void) { return last_error.c_str(); }
+
+// ---- GGUF ---------------------------------------------------------------------------------------
+void *nhost_gguf_decode(const uint8_t *bytes, size_t size) {
+    return guarded([&]() -> void * {
+        auto out = std::make_unique<Opened>();
+        out->whole = std::make_unique<gguf::Gguf>(gguf::Gguf::decode(bytes, size));
+        return out.release();
+    }, nullptr);
+}
+void *nhost_gguf_open(const char *path) {
+    return guarded([&]() -> void * {
+        auto out = std::make_unique<Opened>();
+        out->file = gguf::GgufFile::open(path);
+        return out.release();
+    }, nullptr);
+}
+void nhost_gguf_close(void *held) { delete static_cast<Opened *>(held); }
+uint64_t nhost_gguf_tensors(void *held) {
+    auto *opened = static_cast<Opened *>(held);
+    return opened->whole ? opened->whole->tensors() : opened->file->tensors();
+}
+uint64_t nhost_gguf_reads(void *held) {
+    auto *opened = static_cast<Opened *>(held);
+    return opened->file ? opened->file->reads() : 0;
+}
+// 1 found, 0 absent
+int32_t nhost_gguf_tensor(void *held, const char *name, nhost_tensor *out) {
+    auto found = static_cast<Opened *>(held)->archive().tensor(name);
+    if (!found) return 0;
+    out->element = (int32_t)found->element, out->rank = found->rank, out->elements = found->elements;
+    for (int d = 0; d < 4; d++) out->shape[d] = found->shape[d];
+    out->at = found->at, out->bytes = found->bytes;
+    return 1;
+}
+int32_t nhost_gguf_has(void *held, const char *key) { return static_cast<Opened *>(held)->archive().metadata().has(key); }
+int32_t nhost_gguf_word(void *held, const char *key, uint32_t *out) {
+    return guarded([&] { return *out = static_cast<Opened *>(held)->archive().metadata().word(key), 0; }, -1);
+}
+int32_t nhost_gguf_single(void *held, const char *key, float *out) {
+    return guarded([&] { return *out = static_cast<Opened *>(held)->archive().metadata().single(key), 0; }, -1);
+}
+int32_t nhost_gguf_flag(void *held, const char *key, int32_t *out) {
+    return guarded([&] { return *out = static_cast<Opened *>(held)->archive().metadata().flag(key), 0; }, -1);
+}
+// the bytes of the string, at most `room` of them; returns its length or -1
+int64_t nhost_gguf_text(void *held, const char *key, char *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        std::string text = static_cast<Opened *>(held)->archive().metadata().text(key);
+        memcpy(out, text.data(), std::min(room, text.size()));
+        return (int64_t)text.size();
+    }, -1);
+}
+// integer(): 1 and *out when the value is a whole number, 0 when it is another type, -1 absent
+int32_t nhost_gguf_integer(void *held, const char *key, uint64_t *out) {
+    return guarded([&] {
+        auto found = static_cast<Opened *>(held)->archive().metadata().value(key).integer();
+        if (found) *out = *found;
+        return found ? 1 : 0;
+    }, -1);
+}
+// length of an array value and, for arrays of strings, the text of entry `index`
+int64_t nhost_gguf_array_len(void *held, const char *key) {
+    return guarded([&]() -> int64_t { return (int64_t) static_cast<Opened *>(held)->archive().metadata().array(key).size(); }, -1);
+}
+int64_t nhost_gguf_array_text(void *held, const char *key, uint64_t index, char *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto &items = static_cast<Opened *>(held)->archive().metadata().array(key);
+        auto text = items.at(index).text();
+        if (!text) panic("entry %llu of the %s of this gguf is %s where a string stands", (unsigned long long)index, key, items.at(index).name());
+        memcpy(out, text->data(), std::min(room, text->size()));
+        return (int64_t)text->size();
+    }, -1);
+}
+int64_t nhost_gguf_array_number(void *held, const char *key, uint64_t index, double *out) {
+    return guarded([&]() -> int64_t {
+        auto number = static_cast<Opened *>(held)->archive().metadata().array(key).at(index).number();
+        if (!number) return 0;
+        *out = *number;
+        return 1;
+    }, -1);
+}
+// Source::placed + Source::payload: streams the tensor into out (room bytes), returns its bytes
+int64_t nhost_gguf_payload(void *held, const char *name, uint8_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto &source = static_cast<Opened *>(held)->source();
+        size_t at = 0;
+        source.payload(name, [&](const uint8_t *chunk, size_t bytes) {
+            if (at + bytes <= room) memcpy(out + at, chunk, bytes);
+            at += bytes;
+        });
+        return (int64_t)at;
+    }, -1);
+}
+int32_t nhost_gguf_placed(void *held, const char *name, int32_t *element, uint64_t *elements, float *scale, uint64_t *payload, uint64_t *table) {
+    auto found = static_cast<Opened *>(held)->source().placed(name);
+    if (!found) return 0;
+    *element = (int32_t)found->element, *elements = found->elements, *scale = found->scale;
+    *payload = found->payload_bytes, *table = found->table_bytes;
+    return 1;
+}
+
+// ---- writer -------------------------------------------------------------------------------------
+void *nhost_writer_new(uint64_t alignment) { return new gguf::Writer(alignment); }
+void nhost_writer_free(void *writer) { delete static_cast<gguf::Writer *>(writer); }
+void nhost_writer_u32(void *writer, const char *key, uint32_t value) { static_cast<gguf::Writer *>(writer)->meta_u32(key, value); }
+void nhost_writer_f32(void *writer, const char *key, float value) { static_cast<gguf::Writer *>(writer)->meta_f32(key, value); }
+void nhost_writer_text(void *writer, const char *key, const char *value) { static_cast<gguf::Writer *>(writer)->meta_text(key, value); }
+void nhost_writer_tensor(void *writer, const char *name, int32_t element, const uint64_t *shape, uint32_t rank, const uint8_t *payload, size_t bytes) {
+    static_cast<gguf::Writer *>(writer)->tensor(name, (Element)element, std::vector<uint64_t>(shape, shape + rank), payload, bytes);
+}
+int32_t nhost_writer_save(void *writer, const char *path) {
+    return guarded([&] {
+        auto bytes = static_cast<gguf::Writer *>(writer)->bytes();
+        std::ofstream out(path, std::ios::binary);
+        out.write(reinterpret_cast<const char *>(bytes.data()), (std::streamsize)bytes.size());
+        if (!out) panic("a gguf could not be written at %s", path);
+        return 0;
+    }, -1);
+}
+
+// ---- decoder declarations -----------------------------------------------------------------------
+int32_t nhost_matrix(void *held, const char *name, uint32_t rows, uint32_t columns, int32_t *element) {
+    return guarded([&] { return *element = (int32_t)decoder::matrix(static_cast<Opened *>(held)->archive(), name, rows, columns).element, 0; }, -1);
+}
+int32_t nhost_vector(void *held, const char *name, uint32_t width, int32_t *element) {
+    return guarded([&] { return *element = (int32_t)decoder::vector(static_cast<Opened *>(held)->archive(), name, width).element, 0; }, -1);
+}
+int32_t nhost_cache_validate(const char *name, uint32_t heads, uint32_t width, uint32_t capacity, uint32_t window, uint32_t batch, uint32_t rows,
+                             int32_t element) {
+    return guarded([&] { return decoder::Cache::validate(name, decoder::CacheShape(heads, width, capacity, window, batch, rows), (Element)element), 0; }, -1);
+}
+uint64_t nhost_payload_bytes(int32_t element, uint64_t elements) { return payload_bytes((Element)element, elements); }
+
+// ---- runtime, model, batch ----------------------------------------------------------------------
+void *nhost_runtime_open(int32_t index) {
+    return guarded([&]() -> void * { return new runtime::Runtime(index); }, nullptr);
+}
+void nhost_runtime_close(void *runtime) { delete static_cast<runtime::Runtime *>(runtime); }
+
+// a Qwen2 GGUF (whole or file) becomes a model and a greedy batch over it
+void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count) {
+    return guarded([&]() -> void * {
+        auto *opened = static_cast<Opened *>(held);
+        generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
+        auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
+        auto out = std::make_unique<Loaded>();
+        out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
+        out->batch = std::make_unique<generate::Batch>(*out->model, spec);
+        return out.release();
+    }, nullptr);
+}
+// BatchSpec's refusals alone, with no device: a batch over no model
+int32_t nhost_batch_spec_check(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count) {
+    return guarded([&] {
+        generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
+        generate::Batch::validate(spec);
+        return 0;
+    }, -1);
+}
+void nhost_batch_close(void *held) { delete static_cast<Loaded *>(held); }
+int32_t nhost_batch_admit(void *held, const uint32_t *tokens, uint32_t count) {
+    return guarded([&] { return (int32_t) static_cast<Loaded *>(held)->batch->admit(std::vector<uint32_t>(tokens, tokens + count)); }, -1);
+}
+int32_t nhost_batch_restart(void *held, uint32_t slot, const uint32_t *tokens, uint32_t count) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->restart(slot, std::vector<uint32_t>(tokens, tokens + count)), 0; }, -1);
+}
+int32_t nhost_batch_resume(void *held, uint32_t slot, const uint32_t *tokens, uint32_t count) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->resume(slot, std::vector<uint32_t>(tokens, tokens + count)), 0; }, -1);
+}
+int32_t nhost_batch_suspend(void *held, uint32_t slot) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->suspend(slot), 0; }, -1);
+}
+int32_t nhost_batch_finish(void *held, uint32_t slot) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->finish(slot), 0; }, -1);
+}
+// emitted pairs (slot, token) into out, at most `room` pairs; returns their count or -1
+int32_t nhost_batch_step(void *held, uint32_t *out, uint32_t room) {
+    return guarded([&] {
+        auto emitted = static_cast<Loaded *>(held)->batch->step();
+        for (size_t i = 0; i < emitted.size() && i < room; i++) out[2 * i] = emitted[i].slot, out[2 * i + 1] = emitted[i].token;
+        return (int32_t)emitted.size();
+    }, -1);
+}
+// -1 when the plane holds no sequence
+int64_t nhost_batch_cursor(void *held, uint32_t slot) {
+    return guarded([&]() -> int64_t {
+        auto at = static_cast<Loaded *>(held)->batch->cursor(slot);
+        return at ? (int64_t)*at : -1;
+    }, -2);
+}
+int64_t nhost_batch_remaining(void *held, uint32_t slot) {
+    return guarded([&]() -> int64_t {
+        auto left = static_cast<Loaded *>(held)->batch->remaining(slot);
+        return left ? (int64_t)*left : -1;
+    }, -2);
+}
+// bit i set: plane i is active (low word) / occupied (high word)
+uint64_t nhost_batch_planes(void *held) {
+    auto &batch = *static_cast<Loaded *>(held)->batch;
+    uint64_t out = 0;
+    for (uint32_t slot : batch.active()) out |= 1ull << slot;
+    for (uint32_t slot : batch.occupied()) out |= 1ull << (32 + slot);
+    return out;
+}
+int32_t nhost_batch_logits(void *held, float *out) {
+    return guarded([&] { return runtime::check(nh_model_logits(static_cast<Loaded *>(held)->model->handle(), out)), 0; }, -1);
+}
+
+}  // extern "C"

@@ -1,0 +1,1057 @@
+// neura.hpp -- C++ host layer over the C ABI of libneura_hip.so.
+//
+// The reference's host side is Rust (neura-gguf, neura-source, neura-decoder, neura-generate,
+// neura-runtime); no Rust toolchain exists in this build, so the same interfaces are written
+// in C++ with the same names, argument meaning and error behaviour.  Where the reference
+// panics with a prose message this layer throws neura::Panic carrying the same sentence.
+// Everything below the classes goes through include/neura_hip.h only.
+#pragma once
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <deque>
+#include <fstream>
+#include <functional>
+#include <map>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/neura_hip.h"
+
+namespace neura {
+
+struct Panic : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+
+template <typename... Args>
+[[noreturn]] inline void panic(const char *format, Args... args) {
+    char text[1024];
+    if constexpr (sizeof...(Args) == 0)
+        snprintf(text, sizeof(text), "%s", format);
+    else
+        snprintf(text, sizeof(text), format, args...);
+    throw Panic(text);
+}
+
+#define NEURA_ASSERT(condition, ...) \
+    do {                             \
+        if (!(condition)) ::neura::panic(__VA_ARGS__); \
+    } while (0)
+
+// ---- neura-abi: storage formats (crates/neura-abi/src/element.rs:3-17, :145-178, :231-240) ----
+
+enum class Element : int32_t { Single = 0, Half = 1, Q8_0 = 8, Q3K = 11, Q4K = 12, Q5K = 13, Q6K = 14, Bfloat16 = 30 };
+
+struct Block {
+    uint32_t elements, bytes;
+};
+
+inline const char *name(Element element) {
+    switch (element) {
+    case Element::Single: return "single";
+    case Element::Half: return "half";
+    case Element::Q8_0: return "q8_0";
+    case Element::Q3K: return "q3_k";
+    case Element::Q4K: return "q4_k";
+    case Element::Q5K: return "q5_k";
+    case Element::Q6K: return "q6_k";
+    case Element::Bfloat16: return "bfloat16";
+    }
+    return "unknown";
+}
+
+inline std::optional<Block> block(Element element) {
+    switch (element) {
+    case Element::Q8_0: return Block{32, 34};
+    case Element::Q4K: return Block{256, 144};
+    case Element::Q5K: return Block{256, 176};
+    case Element::Q6K: return Block{256, 210};
+    case Element::Q3K: return Block{256, 110};
+    default: return std::nullopt;
+    }
+}
+
+inline uint32_t bits_per_element(Element element) { return element == Element::Single ? 32 : 16; }
+
+inline uint64_t payload_bytes(Element element, uint64_t elements) {
+    if (auto held = block(element)) return (elements + held->elements - 1) / held->elements * held->bytes;
+    return (elements * bits_per_element(element) + 7) / 8;
+}
+
+// ---- neura-gguf (crates/neura-gguf/src/{value,metadata,header,lib}.rs) ------------------------
+
+namespace gguf {
+
+struct Value {
+    enum Kind { Unsigned8, Signed8, Unsigned16, Signed16, Unsigned32, Signed32, Single, Flag, Text, Array, Unsigned64, Signed64, Double };
+    Kind kind = Unsigned8;
+    uint64_t bits = 0;  // integers (two's complement for signed), flag
+    double real = 0.0;  // Single, Double
+    std::string string;
+    std::vector<Value> items;
+
+    const char *name() const {
+        static const char *names[] = {"u8", "i8", "u16", "i16", "u32", "i32", "f32", "bool", "string", "array", "u64", "i64", "f64"};
+        return names[kind];
+    }
+    std::optional<std::string> text() const { return kind == Text ? std::optional<std::string>(string) : std::nullopt; }
+    // whole numbers; signed ones travel as their two's complement (crates/neura-gguf/tests/gguf.rs:83-86)
+    std::optional<uint64_t> integer() const {
+        switch (kind) {
+        case Unsigned8: case Signed8: case Unsigned16: case Signed16: case Unsigned32: case Signed32: case Unsigned64: case Signed64:
+            return bits;
+        default: return std::nullopt;
+        }
+    }
+    std::optional<double> number() const {
+        if (kind == Single || kind == Double) return real;
+        if (auto held = integer()) {
+            bool is_signed = kind == Signed8 || kind == Signed16 || kind == Signed32 || kind == Signed64;
+            return is_signed ? (double)(int64_t)*held : (double)*held;
+        }
+        return std::nullopt;
+    }
+    std::optional<bool> flag() const { return kind == Flag ? std::optional<bool>(bits != 0) : std::nullopt; }
+    const std::vector<Value> *array() const { return kind == Array ? &items : nullptr; }
+};
+
+struct Tensor {
+    Element element;
+    uint64_t elements;
+    uint64_t shape[4];
+    uint32_t rank;
+    uint64_t at;
+    uint64_t bytes;
+    bool operator==(const Tensor &o) const {
+        return element == o.element && elements == o.elements && rank == o.rank && at == o.at && bytes == o.bytes &&
+               std::equal(shape, shape + 4, o.shape);
+    }
+};
+
+class Metadata {
+  public:
+    explicit Metadata(const std::map<std::string, Value> *held) : held_(held) {}
+    bool has(const std::string &key) const { return held_->count(key) != 0; }
+    const Value &value(const std::string &key) const {
+        auto found = held_->find(key);
+        if (found == held_->end()) panic("this gguf holds no %s", key.c_str());
+        return found->second;
+    }
+    std::string text(const std::string &key) const {
+        auto held = value(key).text();
+        if (!held) panic("the %s of this gguf is %s where a string stands", key.c_str(), value(key).name());
+        return *held;
+    }
+    bool flag(const std::string &key) const {
+        auto held = value(key).flag();
+        if (!held) panic("the %s of this gguf is %s where a flag stands", key.c_str(), value(key).name());
+        return *held;
+    }
+    uint32_t word(const std::string &key) const {
+        auto held = value(key).integer();
+        if (!held) panic("the %s of this gguf is %s where a whole number stands", key.c_str(), value(key).name());
+        if (*held > 0xffffffffull) panic("the %s of this gguf holds %llu where a word holds what fits one", key.c_str(), (unsigned long long)*held);
+        return (uint32_t)*held;
+    }
+    float single(const std::string &key) const {
+        auto held = value(key).number();
+        if (!held) panic("the %s of this gguf is %s where a number stands", key.c_str(), value(key).name());
+        return (float)*held;
+    }
+    std::optional<uint32_t> optional_word(const std::string &key) const { return has(key) ? std::optional<uint32_t>(word(key)) : std::nullopt; }
+    const std::vector<Value> &array(const std::string &key) const {
+        auto held = value(key).array();
+        if (!held) panic("the %s of this gguf is %s where an array stands", key.c_str(), value(key).name());
+        return *held;
+    }
+
+  private:
+    const std::map<std::string, Value> *held_;
+};
+
+// crates/neura-source/src/lib.rs:7-22
+struct Placed {
+    Element element;
+    uint64_t elements;
+    float scale;
+    uint64_t payload_bytes, table_bytes;
+};
+
+using Sink = std::function<void(const uint8_t *, size_t)>;
+
+class Source {
+  public:
+    virtual ~Source() = default;
+    virtual std::optional<Placed> placed(const std::string &name) const = 0;
+    virtual void payload(const std::string &name, const Sink &sink) const = 0;
+    virtual void table(const std::string &name, const Sink &sink) const = 0;
+};
+
+// crates/neura-gguf/src/archive.rs:3-7
+class Archive {
+  public:
+    virtual ~Archive() = default;
+    virtual Metadata metadata() const = 0;
+    virtual std::optional<Tensor> tensor(const std::string &name) const = 0;
+};
+
+namespace detail {
+
+constexpr uint64_t DEFAULT_ALIGNMENT = 32;  // crates/neura-gguf/src/header.rs:6
+constexpr size_t COPY_CHUNK = 1 << 16;      // crates/neura-gguf/src/lib.rs:20
+constexpr size_t HEADER_STEP = 1 << 20;     // crates/neura-gguf/src/lib.rs:21
+
+struct Truncated {};
+
+struct Header {
+    std::map<std::string, Value> metadata;
+    std::vector<std::pair<std::string, Tensor>> tensors;
+    uint64_t data = 0;
+};
+
+inline const char *type_name(uint32_t kind) {  // crates/neura-gguf/src/header.rs:164-204
+    static const char *names[] = {"F32", "F16", "Q4_0", "Q4_1", "removed four bit", "removed four bit", "Q5_0", "Q5_1", "Q8_0", "Q8_1",
+                                  "Q2_K", "Q3_K", "Q4_K", "Q5_K", "Q6_K", "Q8_K", "IQ2_XXS", "IQ2_XS", "IQ3_XXS", "IQ1_S", "IQ4_NL",
+                                  "IQ3_S", "IQ2_S", "IQ4_XS", "I8", "I16", "I32", "I64", "F64", "IQ1_M", "BF16"};
+    if (kind <= 30) return names[kind];
+    if (kind <= 33 || (kind >= 36 && kind <= 38)) return "removed four bit plane";
+    if (kind == 34) return "TQ1_0";
+    if (kind == 35) return "TQ2_0";
+    if (kind == 39) return "MXFP4";
+    return "unknown";
+}
+
+inline std::optional<Element> type_element(uint32_t kind) {  // crates/neura-gguf/src/header.rs:150-162
+    switch (kind) {
+    case 0: return Element::Single;
+    case 1: return Element::Half;
+    case 8: return Element::Q8_0;
+    case 11: return Element::Q3K;
+    case 12: return Element::Q4K;
+    case 13: return Element::Q5K;
+    case 14: return Element::Q6K;
+    case 30: return Element::Bfloat16;
+    default: return std::nullopt;
+    }
+}
+
+class Reader {  // crates/neura-gguf/src/header.rs:206-299
+  public:
+    Reader(const uint8_t *bytes, size_t size) : bytes_(bytes), size_(size) {}
+    size_t at = 0;
+    const uint8_t *take(size_t count) {
+        if (count > size_ - at || at > size_) throw Truncated{};
+        const uint8_t *held = bytes_ + at;
+        at += count;
+        return held;
+    }
+    template <typename T>
+    T plain() {
+        T out;
+        memcpy(&out, take(sizeof(T)), sizeof(T));
+        return out;
+    }
+    std::string text() {
+        uint64_t length = plain<uint64_t>();
+        if (length > size_) throw Truncated{};
+        const uint8_t *held = take((size_t)length);
+        return std::string(reinterpret_cast<const char *>(held), (size_t)length);
+    }
+    Value value(int depth) { return body(plain<uint32_t>(), depth); }
+    Value body(uint32_t kind, int depth) {
+        if (depth > 8) panic("this gguf nests arrays deeper than eight deep");
+        Value v;
+        switch (kind) {
+        case 0: v.kind = Value::Unsigned8, v.bits = plain<uint8_t>(); break;
+        case 1: v.kind = Value::Signed8, v.bits = (uint64_t)(int64_t)plain<int8_t>(); break;
+        case 2: v.kind = Value::Unsigned16, v.bits = plain<uint16_t>(); break;
+        case 3: v.kind = Value::Signed16, v.bits = (uint64_t)(int64_t)plain<int16_t>(); break;
+        case 4: v.kind = Value::Unsigned32, v.bits = plain<uint32_t>(); break;
+        case 5: v.kind = Value::Signed32, v.bits = (uint64_t)(int64_t)plain<int32_t>(); break;
+        case 6: v.kind = Value::Single, v.real = plain<float>(); break;
+        case 7: {
+            uint8_t held = plain<uint8_t>();
+            if (held > 1) panic("this gguf holds %u where a flag holds zero or one", held);
+            v.kind = Value::Flag, v.bits = held;
+            break;
+        }
+        case 8: v.kind = Value::Text, v.string = text(); break;
+        case 9: {
+            uint32_t held = plain<uint32_t>();
+            uint64_t count = plain<uint64_t>();
+            v.kind = Value::Array;
+            for (uint64_t i = 0; i < count; i++) v.items.push_back(body(held, depth + 1));
+            break;
+        }
+        case 10: v.kind = Value::Unsigned64, v.bits = plain<uint64_t>(); break;
+        case 11: v.kind = Value::Signed64, v.bits = (uint64_t)plain<int64_t>(); break;
+        case 12: v.kind = Value::Double, v.real = plain<double>(); break;
+        default: panic("this gguf holds a metadata value of type %u, and a gguf declares thirteen of them", kind);
+        }
+        return v;
+    }
+
+  private:
+    const uint8_t *bytes_;
+    size_t size_;
+};
+
+// crates/neura-gguf/src/header.rs:43-148; throws Truncated when the bytes stop inside the header
+inline Header parse(const uint8_t *bytes, size_t size) {
+    Reader reader(bytes, size);
+    const uint8_t *magic = reader.take(4);
+    if (memcmp(magic, "GGUF", 4) != 0)
+        panic("this file opens with [%02x, %02x, %02x, %02x] where a gguf opens with GGUF", magic[0], magic[1], magic[2], magic[3]);
+    uint32_t version = reader.plain<uint32_t>();
+    if (version != 2 && version != 3)
+        panic("this gguf declares version %u, and this reader holds the versions [2, 3] whose layout it follows", version);
+    uint64_t tensors = reader.plain<uint64_t>(), pairs = reader.plain<uint64_t>();
+    Header header;
+    for (uint64_t i = 0; i < pairs; i++) {
+        std::string key = reader.text();
+        Value value = reader.value(0);
+        if (!header.metadata.emplace(key, std::move(value)).second) panic("two entries of this gguf carry the metadata key %s", key.c_str());
+    }
+    uint64_t alignment = DEFAULT_ALIGNMENT;
+    auto declared = header.metadata.find("general.alignment");
+    if (declared != header.metadata.end()) {
+        auto held = declared->second.integer();
+        if (!held) panic("this gguf measures its alignment by a value that is not an integer");
+        alignment = *held;
+    }
+    if (alignment == 0 || alignment % 8 != 0)
+        panic("this gguf aligns its tensors by %llu, and a gguf aligns them by a multiple of eight", (unsigned long long)alignment);
+    for (uint64_t i = 0; i < tensors; i++) {
+        std::string name = reader.text();
+        uint32_t rank = reader.plain<uint32_t>();
+        if (rank == 0 || rank > 4) panic("the tensor %s declares %u dimensions, and a gguf tensor carries one to four", name.c_str(), rank);
+        Tensor tensor{};
+        tensor.rank = rank;
+        tensor.elements = 1;
+        for (int d = 0; d < 4; d++) tensor.shape[d] = 1;
+        for (uint32_t d = 0; d < rank; d++) {
+            uint64_t held = reader.plain<uint64_t>();
+            tensor.shape[d] = held;
+            if (held != 0 && tensor.elements > UINT64_MAX / held) panic("the tensor %s spans more numbers than a gguf counts", name.c_str());
+            tensor.elements *= held;
+        }
+        uint32_t kind = reader.plain<uint32_t>();
+        tensor.at = reader.plain<uint64_t>();
+        if (tensor.at % alignment != 0)
+            panic("the tensor %s begins at byte %llu of the tensor data, and a gguf aligns it by %llu", name.c_str(),
+                  (unsigned long long)tensor.at, (unsigned long long)alignment);
+        auto element = type_element(kind);
+        if (!element)
+            panic("the tensor %s holds numbers of ggml type %u (%s), which this framework does not read", name.c_str(), kind, type_name(kind));
+        tensor.element = *element;
+        if (auto held = block(*element)) {
+            if (tensor.elements % held->elements != 0)
+                panic("the tensor %s holds %llu numbers of %s storage, and a %s block packs %u of them", name.c_str(),
+                      (unsigned long long)tensor.elements, neura::name(*element), neura::name(*element), held->elements);
+            tensor.bytes = tensor.elements / held->elements * held->bytes;
+        } else {
+            tensor.bytes = tensor.elements * bits_per_element(*element) / 8;
+        }
+        header.tensors.emplace_back(std::move(name), tensor);
+    }
+    header.data = (reader.at + alignment - 1) / alignment * alignment;
+    return header;
+}
+
+inline void bounds(const Header &header, uint64_t held, const std::string &what) {  // crates/neura-gguf/src/lib.rs:225-233
+    for (auto &entry : header.tensors) {
+        uint64_t end = header.data + entry.second.at + entry.second.bytes;
+        if (end > held)
+            panic("%s holds %llu bytes where the tensor %s runs to byte %llu", what.c_str(), (unsigned long long)held, entry.first.c_str(),
+                  (unsigned long long)end);
+    }
+}
+
+inline std::unordered_map<std::string, size_t> index_of(const Header &header) {  // crates/neura-gguf/src/lib.rs:235-244
+    std::unordered_map<std::string, size_t> index;
+    for (size_t at = 0; at < header.tensors.size(); at++)
+        if (!index.emplace(header.tensors[at].first, at).second)
+            panic("two tensors of one gguf carry the name %s, and a name identifies one tensor", header.tensors[at].first.c_str());
+    return index;
+}
+
+inline Placed placed_of(const Tensor &tensor) { return Placed{tensor.element, tensor.elements, 1.0f, tensor.bytes, 0}; }
+
+}  // namespace detail
+
+// A whole GGUF held in memory (crates/neura-gguf/src/lib.rs:23-91)
+class Gguf : public Source, public Archive {
+  public:
+    static Gguf decode(const uint8_t *bytes, size_t size) {
+        Gguf out;
+        try {
+            out.header_ = detail::parse(bytes, size);
+        } catch (const detail::Truncated &) {
+            panic("a gguf header runs past the bytes this file holds, and a gguf opens with its metadata and its tensor table");
+        }
+        detail::bounds(out.header_, size, "a gguf");
+        out.index_ = detail::index_of(out.header_);
+        out.bytes_.assign(bytes, bytes + size);
+        return out;
+    }
+    static Gguf decode(const std::vector<uint8_t> &bytes) { return decode(bytes.data(), bytes.size()); }
+
+    const std::vector<uint8_t> &bytes() const { return bytes_; }
+    Metadata metadata() const override { return Metadata(&header_.metadata); }
+    const Value *value(const std::string &key) const {
+        auto found = header_.metadata.find(key);
+        return found == header_.metadata.end() ? nullptr : &found->second;
+    }
+    size_t tensors() const { return header_.tensors.size(); }
+    std::vector<std::string> names() const {
+        std::vector<std::string> out;
+        for (auto &entry : header_.tensors) out.push_back(entry.first);
+        return out;
+    }
+    std::optional<Tensor> tensor(const std::string &name) const override {
+        auto found = index_.find(name);
+        if (found == index_.end()) return std::nullopt;
+        return header_.tensors[found->second].second;
+    }
+    uint64_t data() const { return header_.data; }
+
+    std::optional<Placed> placed(const std::string &name) const override {
+        auto held = tensor(name);
+        return held ? std::optional<Placed>(detail::placed_of(*held)) : std::nullopt;
+    }
+    void payload(const std::string &name, const Sink &sink) const override {
+        auto held = tensor(name);
+        if (!held) panic("this gguf holds no tensor named %s", name.c_str());
+        size_t start = (size_t)(header_.data + held->at), left = (size_t)held->bytes;
+        while (left) {
+            size_t take = std::min(left, detail::COPY_CHUNK);
+            sink(bytes_.data() + start, take);
+            start += take, left -= take;
+        }
+    }
+    void table(const std::string &name, const Sink &) const override {
+        if (!index_.count(name)) panic("this gguf holds no tensor named %s", name.c_str());
+    }
+
+  private:
+    std::vector<uint8_t> bytes_;
+    detail::Header header_;
+    std::unordered_map<std::string, size_t> index_;
+};
+
+// A GGUF read from a file: the header only, payloads streamed on demand
+// (crates/neura-gguf/src/lib.rs:93-213)
+class GgufFile : public Source, public Archive {
+  public:
+    static std::unique_ptr<GgufFile> open(const std::string &path) {
+        std::unique_ptr<GgufFile> out(new GgufFile());
+        out->path_ = path;
+        out->file_.open(path, std::ios::binary);
+        if (!out->file_) panic("a gguf at %s could not be opened: no such file or no access", path.c_str());
+        out->file_.seekg(0, std::ios::end);
+        uint64_t len = (uint64_t)out->file_.tellg();
+        size_t held = std::min<uint64_t>(detail::HEADER_STEP, std::max<uint64_t>(len, 1));
+        for (;;) {
+            std::vector<uint8_t> bytes(held);
+            out->read_at(0, bytes.data(), bytes.size());
+            try {
+                out->header_ = detail::parse(bytes.data(), bytes.size());
+                break;
+            } catch (const detail::Truncated &) {
+                if (held >= len)
+                    panic("a gguf at %s holds %llu bytes where its metadata and its tensor table run past them, and a header closes before the first tensor of a gguf",
+                          path.c_str(), (unsigned long long)len);
+                held = (size_t)std::min<uint64_t>((uint64_t)held * 2, len);
+            } catch (const Panic &refused) {
+                panic("a gguf at %s holds %s", path.c_str(), refused.what());
+            }
+        }
+        detail::bounds(out->header_, len, "a gguf at " + path);
+        out->index_ = detail::index_of(out->header_);
+        return out;
+    }
+    uint64_t reads() const { return reads_; }
+    const std::string &path() const { return path_; }
+    Metadata metadata() const override { return Metadata(&header_.metadata); }
+    size_t tensors() const { return header_.tensors.size(); }
+    std::optional<Tensor> tensor(const std::string &name) const override {
+        auto found = index_.find(name);
+        if (found == index_.end()) return std::nullopt;
+        return header_.tensors[found->second].second;
+    }
+    std::optional<Placed> placed(const std::string &name) const override {
+        auto held = tensor(name);
+        return held ? std::optional<Placed>(detail::placed_of(*held)) : std::nullopt;
+    }
+    void payload(const std::string &name, const Sink &sink) const override {
+        auto held = tensor(name);
+        if (!held) panic("this gguf holds no tensor named %s", name.c_str());
+        uint64_t at = header_.data + held->at, left = held->bytes;
+        std::vector<uint8_t> chunk;
+        while (left) {
+            size_t take = (size_t)std::min<uint64_t>(left, detail::COPY_CHUNK);
+            chunk.resize(take);
+            read_at(at, chunk.data(), take);
+            reads_++;
+            sink(chunk.data(), take);
+            at += take, left -= take;
+        }
+    }
+    void table(const std::string &name, const Sink &) const override {
+        if (!index_.count(name)) panic("this gguf holds no tensor named %s", name.c_str());
+    }
+
+  private:
+    GgufFile() = default;
+    void read_at(uint64_t at, uint8_t *bytes, size_t count) const {
+        file_.clear();
+        file_.seekg((std::streamoff)at);
+        file_.read(reinterpret_cast<char *>(bytes), (std::streamsize)count);
+        if ((size_t)file_.gcount() != count) panic("a gguf at %s could not be read at %llu: the file ends early", path_.c_str(), (unsigned long long)at);
+    }
+    mutable std::ifstream file_;
+    std::string path_;
+    detail::Header header_;
+    std::unordered_map<std::string, size_t> index_;
+    mutable uint64_t reads_ = 0;
+};
+
+// Writes a GGUF v3 (the layout of the reference's fixture builder, crates/neura-gguf/tests/support/mod.rs:21-64)
+class Writer {
+  public:
+    explicit Writer(uint64_t alignment = 32) : alignment_(alignment) {}
+    void meta_u32(const std::string &key, uint32_t value) { key_kind(key, 4), put(value); }
+    void meta_f32(const std::string &key, float value) { key_kind(key, 6), put(value); }
+    void meta_text(const std::string &key, const std::string &value) { key_kind(key, 8), text(meta_, value); }
+    void tensor(const std::string &name, Element element, const std::vector<uint64_t> &shape, const uint8_t *payload, size_t bytes) {
+        tensors_.push_back({name, (uint32_t)element, shape, std::vector<uint8_t>(payload, payload + bytes)});
+    }
+    std::vector<uint8_t> bytes() const {
+        std::vector<uint8_t> out;
+        out.insert(out.end(), {'G', 'G', 'U', 'F'});
+        append(out, (uint32_t)3), append(out, (uint64_t)tensors_.size()), append(out, (uint64_t)pairs_);
+        out.insert(out.end(), meta_.begin(), meta_.end());
+        uint64_t cursor = 0;
+        for (auto &t : tensors_) {
+            text(out, t.name);
+            append(out, (uint32_t)t.shape.size());
+            for (uint64_t dim : t.shape) append(out, dim);
+            append(out, t.kind), append(out, cursor);
+            cursor = (cursor + t.payload.size() + alignment_ - 1) / alignment_ * alignment_;
+        }
+        while (out.size() % alignment_) out.push_back(0);
+        for (auto &t : tensors_) {
+            out.insert(out.end(), t.payload.begin(), t.payload.end());
+            while (out.size() % alignment_) out.push_back(0);
+        }
+        return out;
+    }
+
+  private:
+    struct Held {
+        std::string name;
+        uint32_t kind;
+        std::vector<uint64_t> shape;
+        std::vector<uint8_t> payload;
+    };
+    template <typename T>
+    static void append(std::vector<uint8_t> &out, T value) {
+        const uint8_t *raw = reinterpret_cast<const uint8_t *>(&value);
+        out.insert(out.end(), raw, raw + sizeof(T));
+    }
+    static void text(std::vector<uint8_t> &out, const std::string &held) {
+        append(out, (uint64_t)held.size());
+        out.insert(out.end(), held.begin(), held.end());
+    }
+    void key_kind(const std::string &key, uint32_t kind) { text(meta_, key), append(meta_, kind), pairs_++; }
+    template <typename T>
+    void put(T value) { append(meta_, value); }
+    uint64_t alignment_;
+    uint64_t pairs_ = 0;
+    std::vector<uint8_t> meta_;
+    std::vector<Held> tensors_;
+};
+
+}  // namespace gguf
+
+// ---- neura-runtime: the device and the weight arena ------------------------------------------
+
+namespace runtime {
+
+inline void check(int32_t status) {
+    if (status != NH_OK) panic("%s", nh_last_error());
+}
+
+// Runtime::open (crates/neura-runtime/src/runtime.rs:183): the only error VALUE of the reference
+// is GpuUnavailable at open; here open throws Panic carrying the library's message.
+class Runtime {
+  public:
+    explicit Runtime(int32_t index = 0) : device_(nh_open(index)) {
+        if (!device_) panic("%s", nh_last_error());
+    }
+    ~Runtime() { nh_close(device_); }
+    Runtime(const Runtime &) = delete;
+    Runtime &operator=(const Runtime &) = delete;
+    nh_device *device() const { return device_; }
+
+  private:
+    nh_device *device_;
+};
+
+// Runtime::load (crates/neura-runtime/src/runtime.rs:356-367): every named tensor of a Source
+// poured verbatim into one arena at 256-byte aligned starts (crates/neura-plan/src/layout.rs:29-36)
+class Weights {
+  public:
+    Weights(const Runtime &runtime, const gguf::Source &source, const std::vector<std::string> &names) {
+        uint64_t total = 0;
+        for (auto &name : names) {
+            auto placed = source.placed(name);
+            if (!placed) panic("this gguf holds no tensor named %s", name.c_str());
+            offsets_[name] = total;
+            placed_.emplace(name, *placed);
+            total += (placed->payload_bytes + 255) / 256 * 256;
+        }
+        arena_ = nh_weights_create(runtime.device(), (size_t)std::max<uint64_t>(total, 256));
+        if (!arena_) panic("%s", nh_last_error());
+        for (auto &name : names) {
+            uint64_t at = offsets_[name];
+            source.payload(name, [&](const uint8_t *chunk, size_t bytes) {
+                check(nh_weights_put(arena_, (size_t)at, chunk, bytes));
+                at += bytes;
+            });
+        }
+    }
+    ~Weights() { nh_weights_destroy(arena_); }
+    Weights(const Weights &) = delete;
+    Weights &operator=(const Weights &) = delete;
+    nh_weights *arena() const { return arena_; }
+    uint64_t offset(const std::string &name) const {
+        auto found = offsets_.find(name);
+        if (found == offsets_.end()) panic("this store holds no tensor named %s", name.c_str());
+        return found->second;
+    }
+    const gguf::Placed &placed(const std::string &name) const { return placed_.at(name); }
+
+  private:
+    nh_weights *arena_ = nullptr;
+    std::map<std::string, uint64_t> offsets_;
+    std::map<std::string, gguf::Placed> placed_;
+};
+
+}  // namespace runtime
+
+// ---- neura-decoder: declarations and the KV cache ---------------------------------------------
+
+namespace decoder {
+
+struct Parameter {
+    std::string name;
+    uint32_t rows, columns;
+    Element element;
+};
+
+// crates/neura-decoder/src/parameter.rs:5-15: GGUF dim0 = columns (contiguous), dim1 = rows
+inline Parameter matrix(const gguf::Archive &source, const std::string &name, uint32_t rows, uint32_t columns) {
+    auto held = source.tensor(name);
+    if (!held) panic("this gguf holds no tensor named %s", name.c_str());
+    if (!(held->rank == 2 && held->shape[0] == columns && held->shape[1] == rows))
+        panic("the tensor %s of this gguf walks %u dimensions of [%llu, %llu, %llu, %llu] where %u rows of %u numbers walk [1, 1, %u, %u]", name.c_str(),
+              held->rank, (unsigned long long)held->shape[0], (unsigned long long)held->shape[1], (unsigned long long)held->shape[2],
+              (unsigned long long)held->shape[3], rows, columns, rows, columns);
+    return Parameter{name, rows, columns, held->element};
+}
+
+// crates/neura-decoder/src/parameter.rs:17-27
+inline Parameter vector(const gguf::Archive &source, const std::string &name, uint32_t width) {
+    auto held = source.tensor(name);
+    if (!held) panic("this gguf holds no tensor named %s", name.c_str());
+    if (!(held->rank == 1 && held->shape[0] == width))
+        panic("the tensor %s of this gguf walks %u dimensions of [%llu, %llu, %llu, %llu] where %u numbers walk [1, 1, 1, %u]", name.c_str(), held->rank,
+              (unsigned long long)held->shape[0], (unsigned long long)held->shape[1], (unsigned long long)held->shape[2],
+              (unsigned long long)held->shape[3], width, width);
+    return Parameter{name, 1, width, held->element};
+}
+
+// crates/neura-decoder/src/cache.rs:19-39
+struct CacheShape {
+    uint32_t heads, width, capacity, window, batch, rows;
+    CacheShape(uint32_t heads, uint32_t width, uint32_t capacity, uint32_t window, uint32_t batch, uint32_t rows)
+        : heads(heads), width(width), capacity(capacity), window(window), batch(batch), rows(rows) {}
+};
+
+// An fp16 KV cache of one layer with the reference's write / attend / reset surface
+// (crates/neura-decoder/src/cache.rs:63-65, :92-195, :223-250, :267-352, :366-406); eager: each
+// call enqueues the kernels on the runtime's stream.
+class Cache {
+  public:
+    // the constructor's refusals, callable without a device
+    static void validate(const std::string &name, const CacheShape &shape, Element element) {
+        NEURA_ASSERT(!name.empty(), "a cache names the state it keeps so a checkpoint can hold it");
+        NEURA_ASSERT(shape.heads > 0 && shape.width > 0 && shape.batch > 0, "a cache of %u planes of %u heads of %u numbers holds no key",
+                     shape.batch, shape.heads, shape.width);
+        NEURA_ASSERT(shape.capacity > 0, "a cache of %u positions holds no key", shape.capacity);
+        NEURA_ASSERT(shape.window > 0 && shape.window <= shape.capacity, "a cache of %u positions keeps a window of %u positions",
+                     shape.capacity, shape.window);
+        NEURA_ASSERT(shape.rows > 0 && shape.rows <= shape.window,
+                     "a cache of a %u position window takes %u rows at a time, and a chunk of more rows than the window holds walks past the slots it fills",
+                     shape.window, shape.rows);
+        NEURA_ASSERT(element == Element::Single || element == Element::Half || element == Element::Bfloat16,
+                     "a cache holds keys and values in single, half or bfloat16 storage, and %s storage carries another grid", neura::name(element));
+        NEURA_ASSERT(element == Element::Half, "this build keeps caches in half storage, and %s storage is not built", neura::name(element));
+    }
+    Cache(const runtime::Runtime &runtime, const std::string &name, CacheShape shape, Element element = Element::Half)
+        : device_(runtime.device()), name_(name), shape_(shape) {
+        validate(name, shape, element);
+        size_t bytes = (size_t)shape.heads * shape.batch * shape.capacity * shape.width * 2;
+        keys_ = static_cast<uint16_t *>(nh_alloc(device_, bytes));
+        values_ = static_cast<uint16_t *>(nh_alloc(device_, bytes));
+        if (!keys_ || !values_) panic("%s", nh_last_error());
+    }
+    ~Cache() {
+        nh_free(device_, keys_);
+        nh_free(device_, values_);
+    }
+    Cache(const Cache &) = delete;
+    Cache &operator=(const Cache &) = delete;
+
+    uint32_t rows() const { return shape_.rows; }
+    uint32_t batch() const { return shape_.batch; }
+    uint32_t window() const { return shape_.window; }
+    std::pair<uint16_t *, uint16_t *> states() const { return {keys_, values_}; }  // "{name}.key", "{name}.value"
+    std::string key_name() const { return name_ + ".key"; }
+    std::string value_name() const { return name_ + ".value"; }
+
+    // keys / values: device fp32 [heads][batch][rows][width]; cursor: device u32 [batch]
+    void write(const uint32_t *cursor, const float *keys, const float *values) { store(cursor, keys, values, nullptr); }
+    void write_masked(const uint32_t *cursor, const float *keys, const float *values, const uint8_t *active) {
+        NEURA_ASSERT(shape_.rows <= shape_.capacity - shape_.window,
+                     "a cache of %u positions keeps a %u position window, and a masked chunk of %u rows holds only %u scratch rows", shape_.capacity,
+                     shape_.window, shape_.rows, shape_.capacity - shape_.window);
+        store(cursor, keys, values, active);
+    }
+    // query / out: device fp32 [query_heads][batch][rows][width]
+    void attend(const float *query, uint32_t query_heads, const uint32_t *cursor, float scale, float *out) {
+        NEURA_ASSERT(query_heads % shape_.heads == 0,
+                     "a query of %u heads reads a cache of %u key heads, and every key head serves a whole group of queries", query_heads, shape_.heads);
+        runtime::check(nh_attention(device_, query, keys_, values_, query_heads, shape_.heads, shape_.batch, shape_.rows, shape_.width,
+                                    shape_.capacity, shape_.window, cursor, scale, out));
+    }
+    // reset: host flags, one per plane; a set flag zeroes the plane's keys and values
+    void reset(const std::vector<uint8_t> &reset) {
+        NEURA_ASSERT(reset.size() == shape_.batch, "a cache of %u planes resets by %zu flags", shape_.batch, reset.size());
+        size_t plane = (size_t)shape_.capacity * shape_.width;
+        for (uint32_t head = 0; head < shape_.heads; head++)
+            for (uint32_t b = 0; b < shape_.batch; b++)
+                if (reset[b]) {
+                    size_t at = ((size_t)head * shape_.batch + b) * plane;
+                    runtime::check(nh_clear(device_, keys_ + at, plane * 2));
+                    runtime::check(nh_clear(device_, values_ + at, plane * 2));
+                }
+    }
+
+  private:
+    void store(const uint32_t *cursor, const float *keys, const float *values, const uint8_t *active) {
+        runtime::check(nh_cache_write(device_, keys, values, keys_, values_, shape_.heads, shape_.batch, shape_.rows, shape_.width, shape_.capacity,
+                                      shape_.window, cursor, active));
+    }
+    nh_device *device_;
+    std::string name_;
+    CacheShape shape_;
+    uint16_t *keys_ = nullptr, *values_ = nullptr;
+};
+
+}  // namespace decoder
+
+// ---- the Qwen2-style decoder and neura-generate ------------------------------------------------
+
+namespace generate {
+
+// examples/qwen/config.rs:21-60 for the qwen2 architecture keys
+struct Config {
+    uint32_t layers, hidden, feed_forward, heads, key_heads, head_width, vocabulary, context;
+    float rope_base, floor;
+    static Config read(const gguf::Metadata &metadata, uint32_t vocabulary) {
+        std::string arch = metadata.text("general.architecture");
+        NEURA_ASSERT(arch == "qwen2",
+                     "this model weighs the tensors of the qwen2 architecture, and this gguf names %s as its general.architecture", arch.c_str());
+        auto key = [&](const char *suffix) { return arch + "." + suffix; };
+        Config c;
+        c.layers = metadata.word(key("block_count"));
+        c.hidden = metadata.word(key("embedding_length"));
+        c.feed_forward = metadata.word(key("feed_forward_length"));
+        c.heads = metadata.word(key("attention.head_count"));
+        c.key_heads = metadata.word(key("attention.head_count_kv"));
+        c.head_width = metadata.optional_word(key("attention.key_length")).value_or(c.hidden / c.heads);
+        c.rope_base = metadata.single(key("rope.freq_base"));
+        c.context = metadata.word(key("context_length"));
+        c.floor = metadata.single(key("attention.layer_norm_rms_epsilon"));
+        c.vocabulary = vocabulary;
+        return c;
+    }
+};
+
+// crates/neura-generate/src/batch.rs:110-153 (greedy; sampling, tuning, sharing and windows are not built)
+struct BatchSpec {
+    uint32_t context, batch;
+    std::vector<uint32_t> chunks;
+    BatchSpec(uint32_t context, uint32_t batch, std::vector<uint32_t> chunks) : context(context), batch(batch), chunks(std::move(chunks)) {}
+};
+
+struct Emitted {  // crates/neura-generate/src/batch.rs:155-159
+    uint32_t slot, token;
+    bool operator==(const Emitted &o) const { return slot == o.slot && token == o.token; }
+};
+
+// The decoder of one GGUF on one device: weights poured into an arena, nh_model above them.
+class Model {
+  public:
+    Model(const runtime::Runtime &runtime, const gguf::Archive &archive, const gguf::Source &source, const Config &config, const BatchSpec &spec)
+        : config_(config) {
+        const uint32_t H = config.hidden, QW = config.heads * config.head_width, KW = config.key_heads * config.head_width, F = config.feed_forward;
+        std::vector<std::string> names;
+        // tensor names of a Qwen2 GGUF (the reference's qwen35 example names them alike, examples/qwen/attention.rs:40-78, mlp.rs:22-25)
+        Element element = decoder::matrix(archive, "token_embd.weight", config.vocabulary, H).element;
+        NEURA_ASSERT(element == Element::Q8_0 || element == Element::Q4K,
+                     "this decoder multiplies q8_0 and q4_k matrices, and token_embd.weight holds %s storage", name(element));
+        auto declare = [&](const decoder::Parameter &parameter) {
+            if (parameter.rows == 1)
+                NEURA_ASSERT(parameter.element == Element::Single, "this decoder reads norm weights in single storage, and %s holds %s storage",
+                             parameter.name.c_str(), name(parameter.element));
+            else
+                NEURA_ASSERT(parameter.element == element, "this decoder multiplies matrices of one storage, and %s holds %s storage beside %s",
+                             parameter.name.c_str(), name(parameter.element), name(element));
+            names.push_back(parameter.name);
+            return parameter;
+        };
+        declare(decoder::matrix(archive, "token_embd.weight", config.vocabulary, H));
+        declare(decoder::vector(archive, "output_norm.weight", H));
+        bool separate_head = archive.tensor("output.weight").has_value();
+        if (separate_head) declare(decoder::matrix(archive, "output.weight", config.vocabulary, H));
+        for (uint32_t layer = 0; layer < config.layers; layer++) {
+            auto at = [&](const char *suffix) { return "blk." + std::to_string(layer) + "." + suffix; };
+            declare(decoder::vector(archive, at("attn_norm.weight"), H));
+            declare(decoder::matrix(archive, at("attn_q.weight"), QW, H));
+            declare(decoder::matrix(archive, at("attn_k.weight"), KW, H));
+            declare(decoder::matrix(archive, at("attn_v.weight"), KW, H));
+            declare(decoder::matrix(archive, at("attn_output.weight"), H, QW));
+            declare(decoder::vector(archive, at("ffn_norm.weight"), H));
+            declare(decoder::matrix(archive, at("ffn_gate.weight"), F, H));
+            declare(decoder::matrix(archive, at("ffn_up.weight"), F, H));
+            declare(decoder::matrix(archive, at("ffn_down.weight"), H, F));
+        }
+        weights_ = std::make_unique<runtime::Weights>(runtime, source, names);
+        std::vector<uint64_t> columns[9];
+        const char *suffixes[9] = {"attn_norm", "attn_q", "attn_k", "attn_v", "attn_output", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down"};
+        for (uint32_t layer = 0; layer < config.layers; layer++)
+            for (int s = 0; s < 9; s++) columns[s].push_back(weights_->offset("blk." + std::to_string(layer) + "." + suffixes[s] + ".weight"));
+        nh_tensor_table table{};
+        table.matrix_element = (int32_t)element;
+        table.token_embd = weights_->offset("token_embd.weight");
+        table.output = separate_head ? weights_->offset("output.weight") : UINT64_MAX;
+        table.output_norm = weights_->offset("output_norm.weight");
+        table.attn_norm = columns[0].data(), table.attn_q = columns[1].data(), table.attn_k = columns[2].data(), table.attn_v = columns[3].data();
+        table.attn_output = columns[4].data(), table.ffn_norm = columns[5].data(), table.ffn_gate = columns[6].data();
+        table.ffn_up = columns[7].data(), table.ffn_down = columns[8].data();
+        nh_model_config c{};
+        c.layers = config.layers, c.hidden = H, c.heads = config.heads, c.kv_heads = config.key_heads, c.head_dim = config.head_width;
+        c.ffn = F, c.vocab = config.vocabulary, c.context = spec.context, c.batch = spec.batch;
+        c.max_rows = spec.chunks.empty() ? 1 : spec.chunks.front();
+        c.rope_base = config.rope_base, c.eps = config.floor;
+        model_ = nh_model_create(runtime.device(), &c, weights_->arena(), &table);
+        if (!model_) panic("%s", nh_last_error());
+    }
+    ~Model() { nh_model_destroy(model_); }
+    Model(const Model &) = delete;
+    Model &operator=(const Model &) = delete;
+    nh_model *handle() const { return model_; }
+    const Config &config() const { return config_; }
+
+  private:
+    Config config_;
+    std::unique_ptr<runtime::Weights> weights_;
+    nh_model *model_ = nullptr;
+};
+
+// The greedy generation state machine (crates/neura-generate/src/batch.rs:279-465, :1000-1172,
+// :1401-1517, :1595-1725): admit / restart / resume / suspend / finish / step with chunked
+// prompt fill.  Single threaded, one model, like `&mut Batch`.
+class Batch {
+  public:
+    // the constructor's refusals, callable without a model
+    static void validate(const BatchSpec &spec) {
+        NEURA_ASSERT(spec.batch > 0, "a batch of no plane answers nothing");
+        NEURA_ASSERT(spec.context > 0, "a context of no token holds no batch");
+        for (size_t i = 0; i + 1 < spec.chunks.size(); i++)
+            NEURA_ASSERT(spec.chunks[i] > spec.chunks[i + 1], "a batch fills the largest chunk first, and fills %u then %u", spec.chunks[i],
+                         spec.chunks[i + 1]);
+        for (uint32_t chunk : spec.chunks)
+            NEURA_ASSERT(chunk > 1 && chunk < spec.context,
+                         "a batch fills %u rows of a context of %u, and a chunk holds between two rows and the rows a prompt leaves for the answer",
+                         chunk, spec.context);
+    }
+    Batch(Model &model, BatchSpec spec) : model_(model), batch_(spec.batch), context_(spec.context), chunks_(spec.chunks), slots_(spec.batch) {
+        validate(spec);
+    }
+    uint32_t batch() const { return batch_; }
+    uint32_t context() const { return context_; }
+
+    uint32_t admit(const std::vector<uint32_t> &tokens) {  // batch.rs:1000-1013
+        for (uint32_t slot = 0; slot < batch_; slot++)
+            if (!slots_[slot]) {
+                restart(slot, tokens);
+                return slot;
+            }
+        panic("all %u planes of this batch hold a sequence", batch_);
+    }
+    void restart(uint32_t slot, const std::vector<uint32_t> &tokens) {  // batch.rs:1056-1105
+        NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot);
+        NEURA_ASSERT(!tokens.empty(), "a batch admits a prompt of at least one token");
+        NEURA_ASSERT(tokens.size() < context_, "the prompt holds %zu tokens where this batch holds %u of context", tokens.size(), context_);
+        std::vector<uint8_t> reset(batch_, 0);
+        reset[slot] = 1;
+        runtime::check(nh_model_reset(model_.handle(), reset.data(), batch_));
+        slots_[slot] = Slot{0, Prompting, std::deque<uint32_t>(tokens.begin(), tokens.end()), 0};
+    }
+    void resume(uint32_t slot, const std::vector<uint32_t> &tokens) {  // batch.rs:1015-1054
+        auto &held = slots_.at(slot);
+        NEURA_ASSERT(held.has_value(), "plane %u of this batch holds no sequence", slot);
+        NEURA_ASSERT(held->phase == Suspended, "plane %u resumes only after it is suspended, and it is %s its sequence", slot,
+                     held->phase == Prompting ? "still feeding" : "still answering");
+        NEURA_ASSERT(!tokens.empty(), "a sequence resumes with at least one token");
+        NEURA_ASSERT(held->cursor < context_, "a sequence at cursor %u of a context of %u resumes only after the application restarts or releases it",
+                     held->cursor, context_);
+        NEURA_ASSERT(tokens.size() < context_ - held->cursor, "a sequence at cursor %u resumes with %zu tokens where this batch holds %u of context",
+                     held->cursor, tokens.size(), context_);
+        held->phase = Prompting;
+        held->prompt.assign(tokens.begin(), tokens.end());
+    }
+    void suspend(uint32_t slot) {  // batch.rs:1107-1123
+        auto &held = slots_.at(slot);
+        NEURA_ASSERT(held.has_value(), "plane %u of this batch holds no sequence", slot);
+        if (held->phase == Prompting)
+            panic("a sequence suspends after it has fed its prompt, and plane %u still holds %zu prompt tokens", slot, held->prompt.size());
+        if (held->phase == Suspended) panic("plane %u of this batch is already suspended", slot);
+        held->phase = Suspended;
+    }
+    void finish(uint32_t slot) {  // batch.rs:1137-1148
+        NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot);
+        slots_[slot].reset();
+    }
+    std::vector<uint32_t> active() const {
+        std::vector<uint32_t> out;
+        for (uint32_t slot = 0; slot < batch_; slot++)
+            if (slots_[slot] && slots_[slot]->phase != Suspended) out.push_back(slot);
+        return out;
+    }
+    std::vector<uint32_t> occupied() const {
+        std::vector<uint32_t> out;
+        for (uint32_t slot = 0; slot < batch_; slot++)
+            if (slots_[slot]) out.push_back(slot);
+        return out;
+    }
+    std::optional<uint32_t> cursor(uint32_t slot) const { return slots_.at(slot) ? std::optional<uint32_t>(slots_[slot]->cursor) : std::nullopt; }
+    std::optional<uint32_t> remaining(uint32_t slot) const {
+        auto held = cursor(slot);
+        return held ? std::optional<uint32_t>(context_ - *held) : std::nullopt;
+    }
+
+    std::vector<Emitted> step() {  // batch.rs:1125-1135
+        if (active().empty()) return {};
+        prefill();
+        return answer();
+    }
+
+  private:
+    enum Phase { Prompting, Generating, Suspended };
+    struct Slot {
+        uint32_t cursor;
+        Phase phase;
+        std::deque<uint32_t> prompt;
+        uint32_t feed;
+    };
+
+    // batch.rs:1401-1432: the first (largest) chunk some prompt still exceeds, and the planes it serves
+    bool next_fill(size_t &index, std::vector<uint32_t> &group) const {
+        std::vector<std::vector<uint32_t>> groups(chunks_.size());
+        for (uint32_t slot = 0; slot < batch_; slot++) {
+            if (!slots_[slot] || slots_[slot]->phase != Prompting) continue;
+            size_t left = slots_[slot]->prompt.size();
+            if (left <= 1) continue;
+            NEURA_ASSERT(slots_[slot]->cursor < context_, "a sequence at cursor %u of a context of %u no longer reaches the prompt it holds",
+                         slots_[slot]->cursor, context_);
+            for (size_t i = 0; i < chunks_.size(); i++)
+                if (chunks_[i] < left) {
+                    groups[i].push_back(slot);
+                    break;
+                }
+        }
+        for (size_t i = 0; i < groups.size(); i++)
+            if (!groups[i].empty()) {
+                index = i, group = groups[i];
+                return true;
+            }
+        return false;
+    }
+    void prefill() {  // batch.rs:1595-1599, :1434-1501
+        size_t index;
+        std::vector<uint32_t> group;
+        while (next_fill(index, group)) {
+            const uint32_t rows = chunks_[index];
+            std::vector<uint32_t> tokens((size_t)rows * batch_, 0), cursors(batch_, 0);
+            std::vector<uint8_t> mask(batch_, 0);
+            for (uint32_t slot : group) {
+                auto &held = *slots_[slot];
+                cursors[slot] = held.cursor, mask[slot] = 1;
+                for (uint32_t row = 0; row < rows; row++) tokens[(size_t)row * batch_ + slot] = held.prompt[row];
+            }
+            runtime::check(nh_prefill(model_.handle(), tokens.data(), rows, cursors.data(), mask.data(), batch_));
+            for (uint32_t slot : group) {
+                auto &held = *slots_[slot];
+                held.cursor += rows;
+                held.prompt.erase(held.prompt.begin(), held.prompt.begin() + rows);
+            }
+        }
+    }
+    std::vector<Emitted> answer() {  // batch.rs:1601-1644, :1681-1725
+        std::vector<uint32_t> tokens(batch_, 0), cursors(batch_, 0), chosen(batch_, 0);
+        std::vector<uint8_t> mask(batch_, 0);
+        for (uint32_t slot = 0; slot < batch_; slot++) {
+            if (!slots_[slot] || slots_[slot]->phase == Suspended) continue;
+            auto &held = *slots_[slot];
+            NEURA_ASSERT(held.cursor < context_, "a sequence at cursor %u of a context of %u no longer %s", held.cursor, context_,
+                         held.phase == Prompting ? "feeds the prompt it holds" : "answers; suspend or release it");
+            tokens[slot] = held.phase == Prompting ? held.prompt.front() : held.feed;
+            cursors[slot] = held.cursor, mask[slot] = 1;
+        }
+        runtime::check(nh_decode_step(model_.handle(), tokens.data(), cursors.data(), mask.data(), batch_, chosen.data()));
+        std::vector<Emitted> emitted;
+        for (uint32_t slot = 0; slot < batch_; slot++) {
+            if (!slots_[slot]) continue;
+            auto &held = *slots_[slot];
+            if (held.phase == Prompting) {
+                held.prompt.pop_front();
+                if (held.prompt.empty()) held.phase = Generating, held.feed = chosen[slot];
+            } else if (held.phase == Generating) {
+                emitted.push_back(Emitted{slot, held.feed});  // a token is emitted on the step after it was chosen
+                held.feed = chosen[slot];
+            }
+            if (held.phase != Suspended) held.cursor += 1;
+        }
+        return emitted;
+    }
+
+    Model &model_;
+    uint32_t batch_, context_;
+    std::vector<uint32_t> chunks_;
+    std::vector<std::optional<Slot>> slots_;
+};
+
+}  // namespace generate
+}  // namespace neura
