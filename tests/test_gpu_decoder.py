@@ -123,3 +123,41 @@ def test_config4_greedy_64_steps_qwen2_5_0_5b_shape_q8_0(device):
     print("greedy margins (top1 - top2): min %.3g median %.3g" % (min(gaps), float(np.median(gaps))))
     assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
     model.release(), weights.release()
+
+
+def test_graph_replays_match_eager_steps(device, monkeypatch):
+    """The decode step replayed from its captured HIP graph gives, on every replay, exactly the
+    logits and tokens of the same step launched eagerly -- with eager work (fills, operator
+    calls, synchronisations) between the replays, masked and unmasked variants interleaved."""
+    shape = SMALL_Q4
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "1")
+    replayed, _, weights_a = build(device, shape, NH_Q4_K, batch=2, context=48, max_rows=8, seed=5)
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")
+    eager, _, weights_b = build(device, shape, NH_Q4_K, batch=2, context=48, max_rows=8, seed=5)
+    rng = np.random.default_rng(6)
+    prompt = rng.integers(0, shape["vocab"], (8, 2)).reshape(-1)
+    tokens_a = tokens_b = [3, 4]
+    cursor = [0, 0]
+    for step in range(12):
+        if step == 4:  # a chunked fill between replays moves both cursors on by 8
+            for model in (replayed, eager):
+                model.prefill(prompt, 8, cursor)
+            cursor = [cursor[0] + 8, cursor[1] + 8]
+        mask = [1, 0] if step % 3 == 2 else None
+        got_a = replayed.decode_step(tokens_a, cursor, mask=mask)
+        got_b = eager.decode_step(tokens_b, cursor, mask=mask)
+        logits_a, logits_b = replayed.logits(), eager.logits()
+        rows = [0] if mask else [0, 1]
+        assert np.array_equal(logits_a[rows], logits_b[rows]), step
+        assert list(got_a[rows]) == list(got_b[rows]), step
+        # eager operator work on the same stream before the next replay
+        x = rng.standard_normal((1, shape["hidden"])).astype(np.float32)
+        device.rmsnorm(x, np.ones(shape["hidden"], np.float32), 1e-6)
+        device.sync()
+        tokens_a, tokens_b = [int(got_a[0]), 4], [int(got_b[0]), 4]
+        cursor = [cursor[0] + 1, cursor[1] + (0 if mask else 1)]
+    for layer in range(shape["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(replayed.cache_read(layer, which)[:, :, :40], eager.cache_read(layer, which)[:, :, :40])
+    for held in (replayed, eager, weights_a, weights_b):
+        held.release()
