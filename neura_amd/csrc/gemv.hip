@@ -607,6 +607,274 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     }
 }
 
+// ------------------------------------------------------------------- Q4_K on MFMA --------
+//
+// The same product with the multiply-adds on the matrix cores, in exact integer arithmetic.
+// A wave owns a tile of 16 output rows; lane (r, g) = (lane % 16, lane / 16) loads the header
+// and the 32 nibble bytes of 64-element group g of one super-block of row r.
+// v_mfma_i32_4x4x4_16B_i8 runs sixteen independent 4x4x4 products, one per four neighbouring
+// lanes: lane j of a quad supplies column j of B (four weights of its own row and group, one per
+// byte) and row j of A (four activations of column j), and receives C[0..3][j] -- the dot
+// products of its own weights with four activation columns.  Sums never mix groups, and the
+// lane that holds a partial sum also holds the block header that scales it.
+//
+// Unpacking is two masks and a shift per 8 weights: word & 0x0f0f0f0f is four weights of
+// sub-block 2g, (word >> 4) & 0x0f0f0f0f four of sub-block 2g+1, each already one per byte.
+// The activations are staged once per workgroup in LDS as integers: a row slice is scaled by a
+// power of two so its largest magnitude lies in [2^29, 2^30), rounded to an integer, and cut
+// into four signed base-256 digits (the four columns of the A operand), so every activation
+// within 2^-6 of the row's largest keeps its whole fp32 mantissa and every product and sum on the matrix cores is exact.
+// Per super-block, lane and activation row: 8 MFMAs over the low nibbles and 8 over the high
+// nibbles; the eight integer sums are joined in fp32, weighed by d*sc, and the minimums take the
+// integer sum of the sub-block's activations: d*sc*sum(q*x) - dmin*m*sum(x), the reference's
+// value (crates/neura-kernel/src/dot.rs:583-619) regrouped per sub-block.
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+struct MfmaParams {
+    const uint8_t *W[3];
+    uint32_t end[3];
+    const float *x;
+    float *y;
+    const float *residual;
+    const float *norm_w;
+    float *partial;
+    uint32_t N, K, row_bytes;
+    uint32_t nblk, slice_blocks, splits;
+    uint32_t rows;   // activation rows of this launch, 1..4
+    uint32_t tiles;  // 16-row tiles
+    int32_t swiglu;
+    float eps;
+};
+
+struct MfmaUnit {
+    u32x4 hdr, qa, qb;
+};
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+
+// KS waves share one tile (each takes every KS-th super-block of the slice); NW waves per
+// workgroup; P activation rows.
+template <int KS, int NW, int P>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
+    extern __shared__ uint32_t xop[];  // [block][16 steps][4 groups][4 P digit columns] of 4 bytes; then sums; then tile partials
+    __shared__ float red[256];
+    __shared__ uint32_t wave_top[NW];
+    __shared__ float unscale[P];
+    constexpr uint32_t NT = NW * 64, TPW = NW / KS, NCW = 4 * P;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t split = blockIdx.y;
+    const uint32_t blk0 = split * p.slice_blocks;
+    const uint32_t nb = min(p.slice_blocks, p.nblk - blk0);
+    const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
+    float *xsum = reinterpret_cast<float *>(xop + (size_t)p.slice_blocks * 64u * NCW);  // [block][group][P][2 sub-blocks]
+    float *part = xsum + (size_t)p.slice_blocks * 8u * P;                               // [2][TPW][KS][P][16]
+
+    // ---- activations -> integer digits in operand order
+    for (uint32_t row = 0; row < P; row++) {
+        const float *xr = p.x + (size_t)min(row, p.rows - 1u) * p.K;
+        float rms = 1.0f;
+        if (p.norm_w) rms = rms_scale(xr, p.K, p.eps, red);
+        uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
+        for (uint32_t i = tid; i < kn; i += NT) {
+            float value = xr[k0 + i];
+            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, rms), p.norm_w[k0 + i]);
+            top = max(top, __builtin_bit_cast(uint32_t, value) & 0x7fffffffu);
+        }
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
+        if (lane == 0) wave_top[wave] = top;
+        __syncthreads();
+        top = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) top = max(top, wave_top[w]);
+        __syncthreads();  // the next row overwrites wave_top
+        // a power of two that puts the largest magnitude in [2^29, 2^30)
+        const uint32_t raw_exponent = top >> 23;
+        const uint32_t exponent = min(max(raw_exponent, 30u), 254u);
+        const float scale = __builtin_bit_cast(float, (283u - exponent) << 23);
+        if (tid == 0) unscale[row] = raw_exponent == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 29u) << 23);
+        const uint32_t chunks = nb * 32u;  // 8 activations each; 8 consecutive chunks = one 64-element group
+        for (uint32_t first = 0; first < chunks; first += NT) {
+            const uint32_t q = first + tid;
+            const bool held = q < chunks;
+            float t[8];
+            if (held) {
+                const float4 a = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q), b = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q + 4u);
+                t[0] = a.x, t[1] = a.y, t[2] = a.z, t[3] = a.w, t[4] = b.x, t[5] = b.y, t[6] = b.z, t[7] = b.w;
+                if (p.norm_w) {
+                    const float4 wa = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q), wb = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q + 4u);
+                    const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) t[i] = __fmul_rn(__fmul_rn(t[i], rms), w[i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) t[i] = 0.0f;
+            }
+            uint32_t digits[4][2] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};  // [digit, most significant first][word of four elements]
+            float total = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float rounded = rintf(t[i] * scale);
+                const int whole = (int)rounded;
+                const int d3 = (whole << 24) >> 24, upper = (whole - d3) >> 8;
+                const int d2 = (upper << 24) >> 24, top2 = (upper - d2) >> 8;
+                const int d1 = (top2 << 24) >> 24, d0 = (top2 - d1) >> 8;
+                total += rounded;
+                const int shift = 8 * (i & 3);
+                digits[0][i >> 2] |= ((uint32_t)d0 & 0xffu) << shift;
+                digits[1][i >> 2] |= ((uint32_t)d1 & 0xffu) << shift;
+                digits[2][i >> 2] |= ((uint32_t)d2 & 0xffu) << shift;
+                digits[3][i >> 2] |= ((uint32_t)d3 & 0xffu) << shift;
+            }
+            // sum of the 32 activations of this chunk's sub-block: 4 chunks = 4 neighbouring lanes
+            total += dpp<DPP_QUAD_XOR1>(total);
+            total += dpp<DPP_QUAD_XOR2>(total);
+            if (held) {
+                // chunk q = elements 8m..8m+7 of half `upper` of group g: nibble words 2m, 2m+1 of that half
+                const uint32_t b = q >> 5, g = (q >> 3) & 3u, upper = (q >> 2) & 1u, step = 8u * upper + 2u * (q & 3u);
+                uint32_t *slot = xop + ((size_t)(b * 16u + step) * 4u + g) * NCW + 4u * row;
+#pragma unroll
+                for (int digit = 0; digit < 4; digit++) {
+                    slot[digit] = digits[digit][0];
+                    slot[4u * NCW + digit] = digits[digit][1];
+                }
+                if ((q & 3u) == 0) xsum[((size_t)(b * 4u + g) * P + row) * 2u + upper] = total;
+            }
+        }
+    }
+    __syncthreads();
+
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t ks = KS == 1 ? 0u : wave % KS, tslot = wave / KS;
+    const ScaleLane lane_scales = scale_lane(g);
+    // lane i of a quad supplies digit column i of an activation row
+    const uint32_t *xlane = xop + (size_t)g * NCW + (lane & 3u);
+    const float2 *slane = reinterpret_cast<const float2 *>(xsum) + (size_t)g * P;
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+
+    uint32_t parity = 0;
+    for (uint32_t base = blockIdx.x * TPW; base < p.tiles; base += gridDim.x * TPW, parity ^= 1u) {
+        const uint32_t tile = base + tslot;
+        const bool live = tile < p.tiles;
+        float acc[P];
+#pragma unroll
+        for (int pass = 0; pass < P; pass++) acc[pass] = 0.0f;
+        if (live) {
+            const uint8_t *rowp;
+            if (p.swiglu) {
+                rowp = (r < 8u ? p.W[0] : p.W[1]) + (size_t)(tile * 8u + (r & 7u)) * p.row_bytes;
+            } else {
+                const uint32_t n0 = tile * 16u;
+                const bool in0 = n0 < p.end[0], in1 = n0 < p.end[1];
+                const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
+                const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
+                rowp = matrix + (size_t)(n0 - before + r) * p.row_bytes;
+            }
+            rowp += (size_t)blk0 * 144u + g * 32u;
+            auto load = [&](MfmaUnit &u, uint32_t b) {
+                const uint8_t *at = rowp + (size_t)b * 144u;
+                u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
+                u.qa = *(global_uint4)(uintptr_t)(at + 16u);
+                u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+            };
+            auto compute = [&](const MfmaUnit &u, uint32_t b) {
+                const uint32_t *xb = xlane + (size_t)b * 64u * NCW;
+                const uint32_t words[8] = {u.qa.x, u.qa.y, u.qa.z, u.qa.w, u.qb.x, u.qb.y, u.qb.z, u.qb.w};
+                i32x4 cl[P], ch[P];
+#pragma unroll
+                for (int pass = 0; pass < P; pass++) cl[pass] = ch[pass] = i32x4{0, 0, 0, 0};
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    const int low = (int)(words[w] & 0x0f0f0f0fu), high = (int)((words[w] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+                    for (int pass = 0; pass < P; pass++) {
+                        const int xl = (int)xb[(size_t)w * 4u * NCW + 4 * pass], xh = (int)xb[(size_t)(8 + w) * 4u * NCW + 4 * pass];
+                        cl[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xl, low, cl[pass], 0, 0, 0);
+                        ch[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xh, high, ch[pass], 0, 0, 0);
+                    }
+                }
+                half2_t sc, mn;
+                scale_pairs(u.hdr, lane_scales, sc, mn);                  // integers as half subnormals: value * 2^-24
+                const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
+                const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * 16777216.0f;
+                const float s0 = d24 * (float)sc.x, s1 = d24 * (float)sc.y, m0 = m24 * (float)mn.x, m1 = m24 * (float)mn.y;
+#pragma unroll
+                for (int pass = 0; pass < P; pass++) {
+                    const float fl = fmaf(fmaf(fmaf((float)cl[pass][0], 256.0f, (float)cl[pass][1]), 256.0f, (float)cl[pass][2]), 256.0f, (float)cl[pass][3]);
+                    const float fh = fmaf(fmaf(fmaf((float)ch[pass][0], 256.0f, (float)ch[pass][1]), 256.0f, (float)ch[pass][2]), 256.0f, (float)ch[pass][3]);
+                    const float2 sums = slane[(size_t)b * 4u * P + pass];
+                    acc[pass] += fmaf(s0, fl, s1 * fh) - fmaf(m0, sums.x, m1 * sums.y);
+                }
+            };
+            uint32_t b = ks;
+            MfmaUnit ua, ub;
+            if (b < nb) load(ua, b);
+            if (b + KS < nb) load(ub, b + KS);
+            while (b < nb) {
+                compute(ua, b);
+                if (b + 2 * KS < nb) load(ua, b + 2 * KS);
+                b += KS;
+                if (b >= nb) break;
+                compute(ub, b);
+                if (b + 2 * KS < nb) load(ub, b + 2 * KS);
+                b += KS;
+            }
+        }
+        // lane (r, g) holds group g's share of output row r for every activation row; the four groups are summed across lanes
+        float value[P];
+#pragma unroll
+        for (int j = 0; j < P; j++) {
+            float v = acc[j];
+            v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+            v += __shfl_xor(v, 32, 64);
+            value[j] = v * unscale[j];
+        }
+        auto publish_one = [&](uint32_t t, uint32_t rr, uint32_t brow, float total, float up) {
+            // (t, rr): tile and row inside it; `up` is the up-projection partner when swiglu folds here
+            if (p.splits > 1) {
+                const uint32_t n = p.swiglu ? (rr < 8u ? t * 8u + rr : p.N / 2 + t * 8u + (rr - 8u)) : t * 16u + rr;
+                p.partial[((size_t)split * p.rows + brow) * p.N + n] = total;
+            } else if (p.swiglu) {
+                if (rr < 8u) p.y[(size_t)brow * (p.N / 2) + t * 8u + rr] = silu(total) * up;
+            } else {
+                const size_t at = (size_t)brow * p.N + t * 16u + rr;
+                p.y[at] = p.residual ? p.residual[at] + total : total;
+            }
+        };
+        if (KS == 1) {
+#pragma unroll
+            for (int j = 0; j < P; j++) {
+                const float up = dpp<DPP_ROW_ROR8>(value[j]);
+                if (live && g == 0 && (uint32_t)j < p.rows) publish_one(tile, r, (uint32_t)j, value[j], up);
+            }
+        } else {
+            float *mine = part + ((size_t)(parity * TPW + tslot) * KS + ks) * P * 16u;
+#pragma unroll
+            for (int j = 0; j < P; j++)
+                if (g == 0) mine[j * 16u + r] = live ? value[j] : 0.0f;
+            __syncthreads();
+            for (uint32_t o = tid; o < TPW * p.rows * 16u; o += NT) {
+                const uint32_t rr = o & 15u, brow = (o >> 4) % p.rows, ts = (o >> 4) / p.rows;
+                const float *from = part + (size_t)(parity * TPW + ts) * KS * P * 16u + brow * 16u;
+                float total = 0.0f, up = 0.0f;
+#pragma unroll
+                for (int k = 0; k < KS; k++) total += from[(size_t)k * P * 16u + rr];
+                if (p.swiglu && p.splits == 1 && rr < 8u) {
+#pragma unroll
+                    for (int k = 0; k < KS; k++) up += from[(size_t)k * P * 16u + rr + 8u];
+                }
+                if (base + ts < p.tiles) publish_one(base + ts, rr, brow, total, up);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------- fold ----------
 
 // sums the slice partials in slice order and applies the epilogue
@@ -753,7 +1021,116 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     return NH_OK;
 }
 
+// The MFMA kernel takes a product when every matrix boundary falls on a 16-row tile and the
+// activations can be read with 128-bit loads.
+static bool mfma_takes(const GemvArgs &a) {
+    if (a.element != NH_Q4_K || env_int("NEURA_HIP_MFMA", 1) == 0) return false;
+    if (a.N < 16 || a.N % 16 != 0) return false;
+    if (a.swiglu) {
+        if (a.end[0] != a.N / 2 || (a.N / 2) % 8 != 0) return false;
+    } else if (a.end[0] % 16 != 0 || a.end[1] % 16 != 0) {
+        return false;
+    }
+    if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
+    return true;
+}
+
+template <int KS, int NW, int P>
+static hipError_t launch_mfma_instance(nh_device *d, const MfmaParams &p, uint32_t blocks_x, size_t lds) {
+    static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
+    if (lds > 64 * 1024 && !widened) {
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma_kernel<KS, NW, P>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024);  // the static arrays take the rest of the 160 KiB
+        if (status != hipSuccess) return status;
+        widened = true;
+    }
+    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<KS, NW, P>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    return hipGetLastError();
+}
+
+template <int KS, int NW>
+static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t P, uint32_t blocks_x, size_t lds) {
+    if (P == 1) return launch_mfma_instance<KS, NW, 1>(d, p, blocks_x, lds);
+    if (P == 2) return launch_mfma_instance<KS, NW, 2>(d, p, blocks_x, lds);
+    return launch_mfma_instance<KS, NW, 4>(d, p, blocks_x, lds);
+}
+
+// LDS bytes of the staged activations of `blocks` super-blocks for P activation rows: digits + sums
+static size_t mfma_staged(uint32_t blocks, uint32_t P) { return (size_t)blocks * (1024u + 32u) * P; }
+
+static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
+    const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
+    const uint32_t nblk = a.K / 256u;
+    const size_t room = 140 * 1024;  // a gfx950 workgroup may take all 160 KiB of a compute unit; tile partials and static arrays need the rest
+    for (uint32_t done = 0; done < a.rows;) {
+        // activation rows per launch: 4, 2 or 1 (the kernel's instantiations), fewer when a whole row would not fit beside them
+        uint32_t left = a.rows - done, P = left >= 3 ? 4u : left;
+        while (P > 1 && mfma_staged(nblk, P) > room) P /= 2;
+        MfmaParams p{};
+        for (int s = 0; s < 3; s++) {
+            p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+            p.end[s] = a.end[s];
+        }
+        p.rows = min(P, left);
+        p.x = a.x + (size_t)done * a.K;
+        p.y = a.y + (size_t)done * outputs;
+        p.residual = a.residual ? a.residual + (size_t)done * a.N : nullptr;
+        p.norm_w = a.norm_w;
+        p.N = a.N;
+        p.K = a.K;
+        p.row_bytes = nblk * 144u;
+        p.nblk = nblk;
+        p.swiglu = a.swiglu;
+        p.eps = a.eps;
+        p.tiles = a.N / 16u;
+        p.splits = (uint32_t)((mfma_staged(nblk, P) + room - 1) / room);
+        p.slice_blocks = (nblk + p.splits - 1) / p.splits;
+        p.splits = (nblk + p.slice_blocks - 1) / p.slice_blocks;
+        if (p.splits > 1) {
+            p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * p.rows * a.N * sizeof(float)));
+            if (!p.partial) return NH_E_MEMORY;
+        }
+        // waves that share a tile: enough of them to fill the device when the matrix is short
+        const uint32_t slots = (uint32_t)d->compute_units * 16u;
+        uint32_t ks = 1;
+        while (ks < 16 && p.tiles * p.splits * ks < slots && ks * 2 <= p.slice_blocks) ks *= 2;
+        ks = (uint32_t)env_int("NEURA_HIP_MFMA_KS", (int)ks);
+        if (ks != 1 && ks != 2 && ks != 4 && ks != 8 && ks != 16) ks = 1;
+        const uint32_t nw = ks > 4 ? ks : 4u, tiles_per_group = nw / ks;
+        const size_t staged = mfma_staged(p.slice_blocks, P);
+        const size_t lds = staged + (ks > 1 ? (size_t)2 * nw * P * 64u : 0);
+        uint32_t blocks_x = (p.tiles + tiles_per_group - 1) / tiles_per_group;
+        // resident waves per compute unit by register use: 6 per SIMD for one activation row, 4 for two, 3 for four
+        uint32_t resident = (uint32_t)env_int("NEURA_HIP_MFMA_WAVES", P == 1 ? 24 : (P == 2 ? 16 : 12)) / nw;
+        const uint32_t by_lds = (uint32_t)((160 * 1024) / (lds + 1536));
+        if (resident > by_lds) resident = by_lds;
+        uint32_t most = (uint32_t)d->compute_units * (resident ? resident : 1u) / p.splits;
+        if (most < 1) most = 1;
+        if (blocks_x > most) blocks_x = most;
+        profile_mark(d);
+        hipError_t launched;
+        switch (ks) {
+        case 1: launched = launch_mfma_kernel<1, 4>(d, p, P, blocks_x, lds); break;
+        case 2: launched = launch_mfma_kernel<2, 4>(d, p, P, blocks_x, lds); break;
+        case 4: launched = launch_mfma_kernel<4, 4>(d, p, P, blocks_x, lds); break;
+        case 8: launched = launch_mfma_kernel<8, 8>(d, p, P, blocks_x, lds); break;
+        default: launched = launch_mfma_kernel<16, 16>(d, p, P, blocks_x, lds); break;
+        }
+        NH_HIP(launched);
+        if (p.splits > 1) {
+            hipLaunchKernelGGL(gemv_fold_kernel, dim3((outputs * p.rows + 255) / 256), dim3(256), 0, d->stream, p.partial, p.splits, p.rows, a.N,
+                               p.residual, a.swiglu, p.y);
+            NH_HIP(hipGetLastError());
+        }
+        profile_mark(d);
+        if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+        done += p.rows;
+    }
+    return NH_OK;
+}
+
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
+    if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
     uint32_t done = 0;
