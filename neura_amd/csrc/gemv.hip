@@ -657,8 +657,9 @@ __device__ __forceinline__ int dpp_int(int v) {
 }
 
 // KS waves share one tile (each takes every KS-th super-block of the slice); NW waves per
-// workgroup; P activation rows.
-template <int KS, int NW, int P>
+// workgroup; P activation rows; D super-blocks in flight per wave (the loads run ahead of the
+// arithmetic across tile boundaries, and the first ones are issued before the activations are staged).
+template <int KS, int NW, int P, int D>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
     extern __shared__ uint32_t xop[];  // [block][16 steps][4 groups][4 P digit columns] of 4 bytes; then sums; then tile partials
     __shared__ float red[256];
@@ -673,6 +674,51 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
     const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
     float *xsum = reinterpret_cast<float *>(xop + (size_t)p.slice_blocks * 64u * NCW);  // [block][group][P][2 sub-blocks]
     float *part = xsum + (size_t)p.slice_blocks * 8u * P;                               // [2][TPW][KS][P][16]
+
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t ks = KS == 1 ? 0u : wave % KS, tslot = wave / KS;
+    const uint32_t stride = gridDim.x * TPW;
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    // first byte this lane reads of super-block 0 of the slice in `tile`
+    // selects over scalars: indexing the parameter arrays by a computed segment would copy them to scratch memory
+    const uint8_t *const w0 = p.W[0], *const w1 = p.W[1], *const w2 = p.W[2];
+    const uint32_t end0 = p.end[0], end1 = p.end[1];
+    const uint8_t *const swiglu_base = r < 8u ? w0 : w1;
+    const bool gated = p.swiglu != 0;
+    const uint32_t row_bytes = p.row_bytes;
+    // captured by value: a by-reference closure would select between the addresses of w0, w1, w2 in memory
+    auto lane_row = [w0, w1, w2, end0, end1, swiglu_base, gated, row_bytes, blk0, g, r](uint32_t tile) -> const uint8_t * {
+        const uint8_t *rowp;
+        if (gated) {
+            rowp = swiglu_base + (size_t)(tile * 8u + (r & 7u)) * row_bytes;
+        } else {
+            const uint32_t n0 = tile * 16u;
+            const bool in0 = n0 < end0, in1 = n0 < end1;
+            const uint8_t *matrix = in0 ? w0 : (in1 ? w1 : w2);
+            const uint32_t before = in0 ? 0u : (in1 ? end0 : end1);
+            rowp = matrix + (size_t)(n0 - before + r) * row_bytes;
+        }
+        return rowp + (size_t)blk0 * 144u + g * 32u;
+    };
+    // the loads run D super-blocks ahead of the arithmetic: (ahead_base, ahead_b) is the next one to fetch
+    MfmaUnit ring[D];
+    uint32_t ahead_base = blockIdx.x * TPW, ahead_b = ks;
+    const uint8_t *ahead_row = ahead_base + tslot < p.tiles ? lane_row(ahead_base + tslot) : nullptr;
+    auto fetch = [&](MfmaUnit &u) {
+        if (ahead_base + tslot >= p.tiles) return;  // past the last tile (stays so)
+        const uint8_t *at = ahead_row + (size_t)ahead_b * 144u;
+        u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
+        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
+        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+        ahead_b += KS;
+        if (ahead_b >= nb) {
+            ahead_b = ks;
+            ahead_base += stride;
+            if (ahead_base + tslot < p.tiles) ahead_row = lane_row(ahead_base + tslot);
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < D; i++) fetch(ring[i]);
 
     // ---- activations -> integer digits in operand order
     for (uint32_t row = 0; row < P; row++) {
@@ -716,22 +762,28 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) t[i] = 0.0f;
             }
-            uint32_t digits[4][2] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};  // [digit, most significant first][word of four elements]
+            // four signed base-256 digits of each rounded activation, most significant first, one byte per element
             float total = 0.0f;
+            auto digits_of = [&](float v0, float v1, float v2, float v3, uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3) {
+                const float in[4] = {v0, v1, v2, v3};
+                w0 = w1 = w2 = w3 = 0u;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float rounded = rintf(t[i] * scale);
-                const int whole = (int)rounded;
-                const int d3 = (whole << 24) >> 24, upper = (whole - d3) >> 8;
-                const int d2 = (upper << 24) >> 24, top2 = (upper - d2) >> 8;
-                const int d1 = (top2 << 24) >> 24, d0 = (top2 - d1) >> 8;
-                total += rounded;
-                const int shift = 8 * (i & 3);
-                digits[0][i >> 2] |= ((uint32_t)d0 & 0xffu) << shift;
-                digits[1][i >> 2] |= ((uint32_t)d1 & 0xffu) << shift;
-                digits[2][i >> 2] |= ((uint32_t)d2 & 0xffu) << shift;
-                digits[3][i >> 2] |= ((uint32_t)d3 & 0xffu) << shift;
-            }
+                for (int i = 0; i < 4; i++) {
+                    const float rounded = rintf(in[i] * scale);
+                    const int whole = (int)rounded;
+                    const int d3 = (whole << 24) >> 24, upper = (whole - d3) >> 8;
+                    const int d2 = (upper << 24) >> 24, top2 = (upper - d2) >> 8;
+                    const int d1 = (top2 << 24) >> 24, d0 = (top2 - d1) >> 8;
+                    total += rounded;
+                    w0 |= ((uint32_t)d0 & 0xffu) << (8 * i);
+                    w1 |= ((uint32_t)d1 & 0xffu) << (8 * i);
+                    w2 |= ((uint32_t)d2 & 0xffu) << (8 * i);
+                    w3 |= ((uint32_t)d3 & 0xffu) << (8 * i);
+                }
+            };
+            uint32_t a0, a1, a2, a3, b0, b1, b2, b3;
+            digits_of(t[0], t[1], t[2], t[3], a0, a1, a2, a3);
+            digits_of(t[4], t[5], t[6], t[7], b0, b1, b2, b3);
             // sum of the 32 activations of this chunk's sub-block: 4 chunks = 4 neighbouring lanes
             total += dpp<DPP_QUAD_XOR1>(total);
             total += dpp<DPP_QUAD_XOR2>(total);
@@ -739,138 +791,118 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
                 // chunk q = elements 8m..8m+7 of half `upper` of group g: nibble words 2m, 2m+1 of that half
                 const uint32_t b = q >> 5, g = (q >> 3) & 3u, upper = (q >> 2) & 1u, step = 8u * upper + 2u * (q & 3u);
                 uint32_t *slot = xop + ((size_t)(b * 16u + step) * 4u + g) * NCW + 4u * row;
-#pragma unroll
-                for (int digit = 0; digit < 4; digit++) {
-                    slot[digit] = digits[digit][0];
-                    slot[4u * NCW + digit] = digits[digit][1];
-                }
+                slot[0] = a0, slot[1] = a1, slot[2] = a2, slot[3] = a3;
+                slot[4u * NCW] = b0, slot[4u * NCW + 1u] = b1, slot[4u * NCW + 2u] = b2, slot[4u * NCW + 3u] = b3;
                 if ((q & 3u) == 0) xsum[((size_t)(b * 4u + g) * P + row) * 2u + upper] = total;
             }
         }
     }
     __syncthreads();
 
-    const uint32_t r = lane & 15u, g = lane >> 4;
-    const uint32_t ks = KS == 1 ? 0u : wave % KS, tslot = wave / KS;
     const ScaleLane lane_scales = scale_lane(g);
     // lane i of a quad supplies digit column i of an activation row
     const uint32_t *xlane = xop + (size_t)g * NCW + (lane & 3u);
     const float2 *slane = reinterpret_cast<const float2 *>(xsum) + (size_t)g * P;
-    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
 
-    uint32_t parity = 0;
-    for (uint32_t base = blockIdx.x * TPW; base < p.tiles; base += gridDim.x * TPW, parity ^= 1u) {
-        const uint32_t tile = base + tslot;
-        const bool live = tile < p.tiles;
-        float acc[P];
+    float acc[P];
 #pragma unroll
-        for (int pass = 0; pass < P; pass++) acc[pass] = 0.0f;
-        if (live) {
-            const uint8_t *rowp;
-            if (p.swiglu) {
-                rowp = (r < 8u ? p.W[0] : p.W[1]) + (size_t)(tile * 8u + (r & 7u)) * p.row_bytes;
-            } else {
-                const uint32_t n0 = tile * 16u;
-                const bool in0 = n0 < p.end[0], in1 = n0 < p.end[1];
-                const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
-                const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
-                rowp = matrix + (size_t)(n0 - before + r) * p.row_bytes;
+    for (int pass = 0; pass < P; pass++) acc[pass] = 0.0f;
+    auto compute = [&](const MfmaUnit &u, uint32_t b) {
+        const uint32_t *xb = xlane + (size_t)b * 64u * NCW;
+        const uint32_t words[8] = {u.qa.x, u.qa.y, u.qa.z, u.qa.w, u.qb.x, u.qb.y, u.qb.z, u.qb.w};
+        i32x4 cl[P], ch[P];
+#pragma unroll
+        for (int pass = 0; pass < P; pass++) cl[pass] = ch[pass] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const int low = (int)(words[w] & 0x0f0f0f0fu), high = (int)((words[w] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int pass = 0; pass < P; pass++) {
+                const int xl = (int)xb[(size_t)w * 4u * NCW + 4 * pass], xh = (int)xb[(size_t)(8 + w) * 4u * NCW + 4 * pass];
+                cl[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xl, low, cl[pass], 0, 0, 0);
+                ch[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xh, high, ch[pass], 0, 0, 0);
             }
-            rowp += (size_t)blk0 * 144u + g * 32u;
-            auto load = [&](MfmaUnit &u, uint32_t b) {
-                const uint8_t *at = rowp + (size_t)b * 144u;
-                u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
-                u.qa = *(global_uint4)(uintptr_t)(at + 16u);
-                u.qb = *(global_uint4)(uintptr_t)(at + 32u);
-            };
-            auto compute = [&](const MfmaUnit &u, uint32_t b) {
-                const uint32_t *xb = xlane + (size_t)b * 64u * NCW;
-                const uint32_t words[8] = {u.qa.x, u.qa.y, u.qa.z, u.qa.w, u.qb.x, u.qb.y, u.qb.z, u.qb.w};
-                i32x4 cl[P], ch[P];
+        }
+        half2_t sc, mn;
+        scale_pairs(u.hdr, lane_scales, sc, mn);                  // integers as half subnormals: value * 2^-24
+        const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
+        const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * 16777216.0f;
+        const float s0 = d24 * (float)sc.x, s1 = d24 * (float)sc.y, m0 = m24 * (float)mn.x, m1 = m24 * (float)mn.y;
 #pragma unroll
-                for (int pass = 0; pass < P; pass++) cl[pass] = ch[pass] = i32x4{0, 0, 0, 0};
+        for (int pass = 0; pass < P; pass++) {
+            const float fl = fmaf(fmaf(fmaf((float)cl[pass][0], 256.0f, (float)cl[pass][1]), 256.0f, (float)cl[pass][2]), 256.0f, (float)cl[pass][3]);
+            const float fh = fmaf(fmaf(fmaf((float)ch[pass][0], 256.0f, (float)ch[pass][1]), 256.0f, (float)ch[pass][2]), 256.0f, (float)ch[pass][3]);
+            const float2 sums = slane[(size_t)b * 4u * P + pass];
+            acc[pass] += fmaf(s0, fl, s1 * fh) - fmaf(m0, sums.x, m1 * sums.y);
+        }
+    };
+
+    // one tile of this workgroup's round is finished by this wave: publish it (with its K partners) and start the next
+    uint32_t parity = 0, base = blockIdx.x * TPW, b = ks;
+    while (base < p.tiles) {
 #pragma unroll
-                for (int w = 0; w < 8; w++) {
-                    const int low = (int)(words[w] & 0x0f0f0f0fu), high = (int)((words[w] >> 4) & 0x0f0f0f0fu);
-#pragma unroll
-                    for (int pass = 0; pass < P; pass++) {
-                        const int xl = (int)xb[(size_t)w * 4u * NCW + 4 * pass], xh = (int)xb[(size_t)(8 + w) * 4u * NCW + 4 * pass];
-                        cl[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xl, low, cl[pass], 0, 0, 0);
-                        ch[pass] = __builtin_amdgcn_mfma_i32_4x4x4i8(xh, high, ch[pass], 0, 0, 0);
+        for (int slot = 0; slot < D; slot++) {
+            if (base >= p.tiles) break;
+            const uint32_t tile = base + tslot;
+            const bool live = tile < p.tiles;
+            if (live) {
+                compute(ring[slot], b);
+                fetch(ring[slot]);
+            }
+            b += KS;
+            if (b < nb) continue;
+                // lane (r, g) holds group g's share of output row r for every activation row; the four groups are summed across lanes
+                float value[P];
+        #pragma unroll
+                for (int j = 0; j < P; j++) {
+                    float v = acc[j];
+                    v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+                    v += __shfl_xor(v, 32, 64);
+                    value[j] = v * unscale[j];
+                }
+                auto publish_one = [&](uint32_t t, uint32_t rr, uint32_t brow, float total, float up) {
+                    // (t, rr): tile and row inside it; `up` is the up-projection partner when swiglu folds here
+                    if (p.splits > 1) {
+                        const uint32_t n = p.swiglu ? (rr < 8u ? t * 8u + rr : p.N / 2 + t * 8u + (rr - 8u)) : t * 16u + rr;
+                        p.partial[((size_t)split * p.rows + brow) * p.N + n] = total;
+                    } else if (p.swiglu) {
+                        if (rr < 8u) p.y[(size_t)brow * (p.N / 2) + t * 8u + rr] = silu(total) * up;
+                    } else {
+                        const size_t at = (size_t)brow * p.N + t * 16u + rr;
+                        p.y[at] = p.residual ? p.residual[at] + total : total;
+                    }
+                };
+                if (KS == 1) {
+        #pragma unroll
+                    for (int j = 0; j < P; j++) {
+                        const float up = dpp<DPP_ROW_ROR8>(value[j]);
+                        if (live && g == 0 && (uint32_t)j < p.rows) publish_one(tile, r, (uint32_t)j, value[j], up);
+                    }
+                } else {
+                    float *mine = part + ((size_t)(parity * TPW + tslot) * KS + ks) * P * 16u;
+        #pragma unroll
+                    for (int j = 0; j < P; j++)
+                        if (g == 0) mine[j * 16u + r] = live ? value[j] : 0.0f;
+                    __syncthreads();
+                    for (uint32_t o = tid; o < TPW * p.rows * 16u; o += NT) {
+                        const uint32_t rr = o & 15u, brow = (o >> 4) % p.rows, ts = (o >> 4) / p.rows;
+                        const float *from = part + (size_t)(parity * TPW + ts) * KS * P * 16u + brow * 16u;
+                        float total = 0.0f, up = 0.0f;
+        #pragma unroll
+                        for (int k = 0; k < KS; k++) total += from[(size_t)k * P * 16u + rr];
+                        if (p.swiglu && p.splits == 1 && rr < 8u) {
+        #pragma unroll
+                            for (int k = 0; k < KS; k++) up += from[(size_t)k * P * 16u + rr + 8u];
+                        }
+                        if (base + ts < p.tiles) publish_one(base + ts, rr, brow, total, up);
                     }
                 }
-                half2_t sc, mn;
-                scale_pairs(u.hdr, lane_scales, sc, mn);                  // integers as half subnormals: value * 2^-24
-                const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
-                const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * 16777216.0f;
-                const float s0 = d24 * (float)sc.x, s1 = d24 * (float)sc.y, m0 = m24 * (float)mn.x, m1 = m24 * (float)mn.y;
+            // the next tile of this wave
 #pragma unroll
-                for (int pass = 0; pass < P; pass++) {
-                    const float fl = fmaf(fmaf(fmaf((float)cl[pass][0], 256.0f, (float)cl[pass][1]), 256.0f, (float)cl[pass][2]), 256.0f, (float)cl[pass][3]);
-                    const float fh = fmaf(fmaf(fmaf((float)ch[pass][0], 256.0f, (float)ch[pass][1]), 256.0f, (float)ch[pass][2]), 256.0f, (float)ch[pass][3]);
-                    const float2 sums = slane[(size_t)b * 4u * P + pass];
-                    acc[pass] += fmaf(s0, fl, s1 * fh) - fmaf(m0, sums.x, m1 * sums.y);
-                }
-            };
-            uint32_t b = ks;
-            MfmaUnit ua, ub;
-            if (b < nb) load(ua, b);
-            if (b + KS < nb) load(ub, b + KS);
-            while (b < nb) {
-                compute(ua, b);
-                if (b + 2 * KS < nb) load(ua, b + 2 * KS);
-                b += KS;
-                if (b >= nb) break;
-                compute(ub, b);
-                if (b + 2 * KS < nb) load(ub, b + 2 * KS);
-                b += KS;
-            }
-        }
-        // lane (r, g) holds group g's share of output row r for every activation row; the four groups are summed across lanes
-        float value[P];
-#pragma unroll
-        for (int j = 0; j < P; j++) {
-            float v = acc[j];
-            v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
-            v += __shfl_xor(v, 32, 64);
-            value[j] = v * unscale[j];
-        }
-        auto publish_one = [&](uint32_t t, uint32_t rr, uint32_t brow, float total, float up) {
-            // (t, rr): tile and row inside it; `up` is the up-projection partner when swiglu folds here
-            if (p.splits > 1) {
-                const uint32_t n = p.swiglu ? (rr < 8u ? t * 8u + rr : p.N / 2 + t * 8u + (rr - 8u)) : t * 16u + rr;
-                p.partial[((size_t)split * p.rows + brow) * p.N + n] = total;
-            } else if (p.swiglu) {
-                if (rr < 8u) p.y[(size_t)brow * (p.N / 2) + t * 8u + rr] = silu(total) * up;
-            } else {
-                const size_t at = (size_t)brow * p.N + t * 16u + rr;
-                p.y[at] = p.residual ? p.residual[at] + total : total;
-            }
-        };
-        if (KS == 1) {
-#pragma unroll
-            for (int j = 0; j < P; j++) {
-                const float up = dpp<DPP_ROW_ROR8>(value[j]);
-                if (live && g == 0 && (uint32_t)j < p.rows) publish_one(tile, r, (uint32_t)j, value[j], up);
-            }
-        } else {
-            float *mine = part + ((size_t)(parity * TPW + tslot) * KS + ks) * P * 16u;
-#pragma unroll
-            for (int j = 0; j < P; j++)
-                if (g == 0) mine[j * 16u + r] = live ? value[j] : 0.0f;
-            __syncthreads();
-            for (uint32_t o = tid; o < TPW * p.rows * 16u; o += NT) {
-                const uint32_t rr = o & 15u, brow = (o >> 4) % p.rows, ts = (o >> 4) / p.rows;
-                const float *from = part + (size_t)(parity * TPW + ts) * KS * P * 16u + brow * 16u;
-                float total = 0.0f, up = 0.0f;
-#pragma unroll
-                for (int k = 0; k < KS; k++) total += from[(size_t)k * P * 16u + rr];
-                if (p.swiglu && p.splits == 1 && rr < 8u) {
-#pragma unroll
-                    for (int k = 0; k < KS; k++) up += from[(size_t)k * P * 16u + rr + 8u];
-                }
-                if (base + ts < p.tiles) publish_one(base + ts, rr, brow, total, up);
-            }
+            for (int pass = 0; pass < P; pass++) acc[pass] = 0.0f;
+            b = ks;
+            base += stride;
+            parity ^= 1u;
         }
     }
 }
@@ -1024,7 +1056,11 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
 // The MFMA kernel takes a product when every matrix boundary falls on a 16-row tile and the
 // activations can be read with 128-bit loads.
 static bool mfma_takes(const GemvArgs &a) {
-    if (a.element != NH_Q4_K || env_int("NEURA_HIP_MFMA", 1) == 0) return false;
+    // 2: always; 1: where it measured faster than the vector kernels -- several activation rows (they ride on
+    // the same unpacked weights) or rows deeper than one wave spans (no second launch to fold slices); 0: never
+    const int mode = env_int("NEURA_HIP_MFMA", 1);
+    if (a.element != NH_Q4_K || mode == 0) return false;
+    if (mode == 1 && a.rows == 1 && a.K <= 4096) return false;
     if (a.N < 16 || a.N % 16 != 0) return false;
     if (a.swiglu) {
         if (a.end[0] != a.N / 2 || (a.N / 2) % 8 != 0) return false;
@@ -1035,24 +1071,28 @@ static bool mfma_takes(const GemvArgs &a) {
     return true;
 }
 
-template <int KS, int NW, int P>
+template <int KS, int NW, int P, int D>
 static hipError_t launch_mfma_instance(nh_device *d, const MfmaParams &p, uint32_t blocks_x, size_t lds) {
     static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
     if (lds > 64 * 1024 && !widened) {
-        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma_kernel<KS, NW, P>),
+        hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma_kernel<KS, NW, P, D>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024);  // the static arrays take the rest of the 160 KiB
         if (status != hipSuccess) return status;
         widened = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<KS, NW, P>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<KS, NW, P, D>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
     return hipGetLastError();
 }
 
 template <int KS, int NW>
 static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t P, uint32_t blocks_x, size_t lds) {
-    if (P == 1) return launch_mfma_instance<KS, NW, 1>(d, p, blocks_x, lds);
-    if (P == 2) return launch_mfma_instance<KS, NW, 2>(d, p, blocks_x, lds);
-    return launch_mfma_instance<KS, NW, 4>(d, p, blocks_x, lds);
+    if (P == 1) {
+        const int depth = env_int("NEURA_HIP_MFMA_DEPTH", 4);
+        if (depth == 2) return launch_mfma_instance<KS, NW, 1, 2>(d, p, blocks_x, lds);
+        return launch_mfma_instance<KS, NW, 1, 4>(d, p, blocks_x, lds);
+    }
+    if (P == 2) return launch_mfma_instance<KS, NW, 2, 3>(d, p, blocks_x, lds);
+    return launch_mfma_instance<KS, NW, 4, 2>(d, p, blocks_x, lds);
 }
 
 // LDS bytes of the staged activations of `blocks` super-blocks for P activation rows: digits + sums
@@ -1096,12 +1136,16 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
         while (ks < 16 && p.tiles * p.splits * ks < slots && ks * 2 <= p.slice_blocks) ks *= 2;
         ks = (uint32_t)env_int("NEURA_HIP_MFMA_KS", (int)ks);
         if (ks != 1 && ks != 2 && ks != 4 && ks != 8 && ks != 16) ks = 1;
-        const uint32_t nw = ks > 4 ? ks : 4u, tiles_per_group = nw / ks;
+        // waves per workgroup: four measured best (larger workgroups stage the activations less often but stream slower)
+        uint32_t nw = (uint32_t)env_int("NEURA_HIP_MFMA_NW", 4);
+        if (nw != 4 && nw != 8 && nw != 16) nw = 4;
+        if (nw < ks) nw = ks;
+        const uint32_t tiles_per_group = nw / ks;
         const size_t staged = mfma_staged(p.slice_blocks, P);
         const size_t lds = staged + (ks > 1 ? (size_t)2 * nw * P * 64u : 0);
         uint32_t blocks_x = (p.tiles + tiles_per_group - 1) / tiles_per_group;
-        // resident waves per compute unit by register use: 6 per SIMD for one activation row, 4 for two, 3 for four
-        uint32_t resident = (uint32_t)env_int("NEURA_HIP_MFMA_WAVES", P == 1 ? 24 : (P == 2 ? 16 : 12)) / nw;
+        // resident waves per compute unit, by register use: 4 per SIMD (one or two activation rows), 3 for four
+        uint32_t resident = (uint32_t)env_int("NEURA_HIP_MFMA_WAVES", P == 4 ? 12 : 16) / nw;
         const uint32_t by_lds = (uint32_t)((160 * 1024) / (lds + 1536));
         if (resident > by_lds) resident = by_lds;
         uint32_t most = (uint32_t)d->compute_units * (resident ? resident : 1u) / p.splits;
@@ -1109,13 +1153,12 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
         if (blocks_x > most) blocks_x = most;
         profile_mark(d);
         hipError_t launched;
-        switch (ks) {
-        case 1: launched = launch_mfma_kernel<1, 4>(d, p, P, blocks_x, lds); break;
-        case 2: launched = launch_mfma_kernel<2, 4>(d, p, P, blocks_x, lds); break;
-        case 4: launched = launch_mfma_kernel<4, 4>(d, p, P, blocks_x, lds); break;
-        case 8: launched = launch_mfma_kernel<8, 8>(d, p, P, blocks_x, lds); break;
-        default: launched = launch_mfma_kernel<16, 16>(d, p, P, blocks_x, lds); break;
-        }
+#define NH_MFMA_CASE(KK, WW) if (ks == KK && nw == WW) launched = launch_mfma_kernel<KK, WW>(d, p, P, blocks_x, lds); else
+        NH_MFMA_CASE(1, 4) NH_MFMA_CASE(2, 4) NH_MFMA_CASE(4, 4)
+        NH_MFMA_CASE(1, 8) NH_MFMA_CASE(2, 8) NH_MFMA_CASE(4, 8) NH_MFMA_CASE(8, 8)
+        NH_MFMA_CASE(1, 16) NH_MFMA_CASE(2, 16) NH_MFMA_CASE(4, 16) NH_MFMA_CASE(8, 16)
+        launched = launch_mfma_kernel<16, 16>(d, p, P, blocks_x, lds);
+#undef NH_MFMA_CASE
         NH_HIP(launched);
         if (p.splits > 1) {
             hipLaunchKernelGGL(gemv_fold_kernel, dim3((outputs * p.rows + 255) / 256), dim3(256), 0, d->stream, p.partial, p.splits, p.rows, a.N,
