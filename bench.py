@@ -90,6 +90,48 @@ def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=2
     }
 
 
+def extras(device, weights, shape, element, context, layers, rng):
+    """The other two measurements the workload names, on the same resident weights: decode at
+    batch 8 (eight sequences at the end of their context) and a 512-token prompt fill."""
+    from neura_amd.loader import Model
+
+    out = {}
+    batch = 8
+    model = Model(device, weights, shape, element, batch=batch, context=context, layers=layers)
+    steps, warm = 16, 4
+    tokens = list(range(1, batch + 1))
+    first = context - (steps + warm)
+    for step in range(warm):
+        tokens = [int(t) for t in model.decode_step(tokens, [first + step] * batch)]
+    device.sync()
+    began = time.perf_counter()
+    for step in range(steps):
+        tokens = [int(t) for t in model.decode_step(tokens, [first + warm + step] * batch)]
+    device.sync()
+    elapsed = time.perf_counter() - began
+    out["decode_batch8"] = {"value": batch * steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
+                            "note": "8 planes, caches not pre-filled (zeros), cursors at the end of context %d" % context}
+    model.release()
+    rows = 512
+    model = Model(device, weights, shape, element, batch=1, context=context, max_rows=rows, layers=layers)
+    prompt = rng.integers(0, shape["vocab"], rows)
+    model.prefill(prompt, rows, [0])
+    device.sync()
+    began = time.perf_counter()
+    repeats = 3
+    for _ in range(repeats):
+        model.prefill(prompt, rows, [0])
+    device.sync()
+    elapsed = (time.perf_counter() - began) / repeats
+    per_layer = sum(2.0 * rows * n * k for _, n, k in __import__("neura_amd").synth.layer_matrices(shape))
+    out["prefill_512"] = {"value": rows / elapsed, "unit": "tokens/s", "ms": elapsed * 1e3,
+                          "product_tflops": layers * per_layer / elapsed / 1e12,
+                          "note": "one 512-row fill at cursor 0, all products on f16 MFMA with fp32 activations as (value, residue) half rows; "
+                                  "product_tflops counts 2*M*N*K of the products over the whole fill time"}
+    model.release()
+    return out
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -98,6 +140,7 @@ def main():
     parser.add_argument("--workload", default="qwen2.5-7b-q4k")
     parser.add_argument("--layers", type=int, default=None, help="cut the decoder (for quick checks; the result is then not the headline)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode and 512-token fill measurements")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()
@@ -181,6 +224,8 @@ def main():
             "gemv_ms_per_step": gemv_seconds / profiled * 1e3,
         },
     }
+    if not args.no_extras:
+        result["extras"] = extras(device, weights, shape, element, context, layers, rng)
     if not args.no_cpu:
         host = {name: raw for name, _, _, raw in tensors}
         result["cpu_baseline"] = cpu_baseline(shape, element, host, context, layers)

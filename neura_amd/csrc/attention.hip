@@ -11,6 +11,8 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <cstdlib>
+
 namespace nh {
 
 constexpr int MAX_GROUPS = 8;
@@ -244,9 +246,11 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
     // sections of the context: enough workgroups to fill the chip four times over, none thinner
-    // than 32 keys
+    // than 64 keys (thinner sections cost more in the fold than they gain in the walk)
+    const char *held = getenv("NEURA_HIP_ATTENTION_KEYS");
+    const uint32_t thinnest = held && atoi(held) > 0 ? (uint32_t)atoi(held) : 64u;
     uint32_t wanted = ((uint32_t)d->compute_units * 4 + units - 1) / units;
-    uint32_t most = (a.keys + 31) / 32;
+    uint32_t most = (a.keys + thinnest - 1) / thinnest;
     p.sections = wanted < 1 ? 1 : (wanted > most ? most : wanted);
     if (p.sections > 256) p.sections = 256;
     if (p.sections > 1) {

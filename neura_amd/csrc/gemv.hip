@@ -40,25 +40,23 @@ struct GemvParams {
 __device__ __forceinline__ uint32_t skew64(uint32_t i) { return i + (i >> 6) * 4; }
 __device__ __forceinline__ uint32_t skew32(uint32_t i) { return i + (i >> 5) * 4; }
 
-// sum of squares of one activation row in the order of the reference's norm kernel
-// (crates/neura-kernel/src/task/norm.rs:69-83 + reduce.rs:21-38): thread t adds columns
-// t, t+256, ...; then a 256-wide tree.  Returns 1/sqrt(mean + eps) to every thread.
+// 1 / sqrt(mean(x^2) + eps) of one activation row, to every thread.  Thread t adds columns t, t+256, ...
+// as the reference's norm kernel does (crates/neura-kernel/src/task/norm.rs:69-83); the 256 partial
+// sums are then joined inside each wave by shuffles and across waves through LDS with one barrier,
+// not by the reference's eight-level tree (reduce.rs:21-38): a different order of the same fp32 adds.
 __device__ float rms_scale(const float *__restrict__ x, uint32_t K, float eps, float *red) {
+    float square = 0.0f;
     if (threadIdx.x < 256) {  // larger workgroups leave the sum to their first 256 threads
-        float square = 0.0f;
         for (uint32_t c = threadIdx.x; c < K; c += 256) {
             float value = x[c];
             square = __fadd_rn(square, __fmul_rn(value, value));
         }
-        red[threadIdx.x] = square;
     }
+    square = wave_sum(square);
+    if ((threadIdx.x & 63u) == 0 && threadIdx.x < 256) red[threadIdx.x >> 6] = square;
     __syncthreads();
-    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
-        if (threadIdx.x < stride) red[threadIdx.x] = __fadd_rn(red[threadIdx.x], red[threadIdx.x + stride]);
-        __syncthreads();
-    }
-    float total = red[0];
-    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    __syncthreads();  // red is reused by the next row
     return rms_scale_of(total, K, eps);
 }
 
