@@ -189,12 +189,15 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 }
 
 // Fold of the sections of one (unit, query head): crates/neura-kernel/src/task/attention.rs:619-671.
-// One workgroup per (unit, group).  Thread s first turns the statistics of section s into its
-// weight, then thread c sums channel c over the sections with eight loads in flight.
+// One workgroup per (unit, group, block of 32 channels).  Thread s first turns the statistics of
+// section s into its weight; then thread (channel, stripe) sums its channel over every eighth
+// section -- all of its loads in flight at once -- and the eight stripes meet in LDS.
 __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, uint32_t width) {
-    __shared__ float weights[256], masses[256], held[256];
+    __shared__ float weights[256], masses[256], held[256], stripes[8][32];
     const uint32_t G = p.groups, tid = threadIdx.x;
-    const uint32_t unit = blockIdx.x / G, g = blockIdx.x % G;
+    const uint32_t blocks = (width + 31u) / 32u;
+    const uint32_t cblock = blockIdx.x % blocks, ug = blockIdx.x / blocks;
+    const uint32_t unit = ug / G, g = ug % G;
     const uint32_t row = unit % p.rows;
     const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
     const float *src = p.partial + ((uint64_t)unit * p.sections * G + g) * (width + 2);
@@ -203,6 +206,14 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, 
     if (tid < p.sections) {
         top = src[tid * hop + width];
         mass = src[tid * hop + width + 1];
+    }
+    // the channel sums do not wait for the weights: fetch first
+    const uint32_t c = cblock * 32u + (tid & 31u), stripe = tid >> 5;
+    float values[32];
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+        const uint32_t s = stripe + 8u * j;
+        values[j] = (s < p.sections && c < width) ? src[s * hop + c] : 0.0f;
     }
     held[tid] = top;
     __syncthreads();
@@ -218,18 +229,17 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, 
     float total = 0.0f;
     for (uint32_t s = 0; s < p.sections; s++) total += masses[s];
     const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
-    for (uint32_t c = tid; c < width; c += 256) {
-        float sums[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        uint32_t s = 0;
-        for (; s + 8 <= p.sections; s += 8) {
-            float values[8];
+    float sum = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 8; j++) values[j] = src[(s + j) * hop + c];
-#pragma unroll
-            for (int j = 0; j < 8; j++) sums[j] = fmaf(values[j], weights[s + j], sums[j]);
-        }
-        for (; s < p.sections; s++) sums[0] = fmaf(src[s * hop + c], weights[s], sums[0]);
-        float value = ((sums[0] + sums[1]) + (sums[2] + sums[3])) + ((sums[4] + sums[5]) + (sums[6] + sums[7]));
+    for (int j = 0; j < 32; j++) {
+        const uint32_t s = stripe + 8u * j;
+        if (s < p.sections) sum = fmaf(values[j], weights[s], sum);
+    }
+    stripes[stripe][tid & 31u] = sum;
+    __syncthreads();
+    if (tid < 32 && c < width) {
+        float value = ((stripes[0][tid] + stripes[1][tid]) + (stripes[2][tid] + stripes[3][tid])) +
+                      ((stripes[4][tid] + stripes[5][tid]) + (stripes[6][tid] + stripes[7][tid]));
         p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr + c] = value * normalized;
     }
 }
@@ -267,7 +277,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     NH_HIP(hipGetLastError());
     if (p.sections > 1) {
-        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups), dim3(256), 0, d->stream, p, a.width);
+        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
         NH_HIP(hipGetLastError());
     }
     return NH_OK;

@@ -90,6 +90,16 @@ enum Refusal : uint32_t { REFUSAL_NONE = 0, REFUSAL_INDEX = 1, REFUSAL_ORIGIN = 
 int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t elements, float *dst);
 int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, uint16_t *dst);
 
+// Rotation and cache append folded into the q|k|v product of one token (one activation row, one plane):
+// output rows [0, q_rows) are rotated and written to y, rows [q_rows, k_rows) are rotated, rounded to fp16 and
+// written to the key cache at the cursor, the rest are rounded to fp16 into the value cache.
+struct RopeFusion {
+    const float *table;      // pow(base, -2c/width), c < width/2
+    const uint32_t *cursor;  // device, one plane
+    uint16_t *cache_k, *cache_v;
+    uint32_t width, q_rows, k_rows, capacity;
+};
+
 struct GemvArgs {
     int32_t element;
     const void *W[3];  // up to three matrices stacked along N; unused entries are nullptr
@@ -103,8 +113,11 @@ struct GemvArgs {
     // optional fused RMSNorm of x: x' = x / sqrt(mean(x^2)+eps) * norm_w
     const float *norm_w;
     float eps;
+    const RopeFusion *rope = nullptr;  // only where gemv_fuses_rope() says so
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
+// whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)
+bool gemv_fuses_rope(const GemvArgs &args, const RopeFusion &rope);
 
 struct GemmArgs {
     int32_t element;

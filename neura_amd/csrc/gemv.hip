@@ -33,6 +33,12 @@ struct GemvParams {
     uint32_t chunks_per_row;    // Q8_0: 16-byte chunks of a staged row slice
     int32_t swiglu;
     float eps;
+    // rotation folded into the product (decode kernel only): see RopeFusion
+    const float *rope_table;
+    const uint32_t *rope_cursor;
+    uint16_t *rope_k, *rope_v;
+    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity;
+    uint32_t *refusal;
 };
 
 // skewed LDS index of activation i: 4 floats of padding per 64 keep 128-bit reads of
@@ -288,12 +294,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
 #pragma unroll
             for (int r = 0; r < R; r++) base[r] = ((r & 1) ? p.W[1] : p.W[0]) + (size_t)(pair + (r >> 1)) * p.row_bytes;
         } else {
-            const uint32_t n = min(first, p.N - R);
+            // with the rotation folded in, logical rows 2t, 2t+1 are channels t and t + width/2 of one head
+            const uint32_t logical = min(first, p.N - R);
+            const uint32_t half = p.rope_width >> 1, pair = logical >> 1;
+            const uint32_t n = p.rope_table ? (pair / half) * p.rope_width + pair % half : logical;
+            const uint32_t hop = p.rope_table ? half : 1u;
             const bool in0 = n < p.end[0], in1 = n < p.end[1];
             const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
             const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
 #pragma unroll
-            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r) * p.row_bytes;
+            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r * hop) * p.row_bytes;
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -360,6 +370,31 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
         } else if (p.swiglu) {
             float up = dpp<DPP_QUAD_XOR1>(total);
             if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(total) * up;
+        } else if (p.rope_table) {
+            // lanes 0 and 1 hold channels c and c + width/2 of one head (crates/neura-kernel/src/task/rope.rs:95-122)
+            const float other = dpp<DPP_QUAD_XOR1>(total);
+            if (u < R && i < p.N) {
+                const uint32_t half = p.rope_width >> 1, pair = i >> 1, c = pair % half;
+                const uint32_t n = (pair / half) * p.rope_width + c + (i & 1u) * half;
+                const uint32_t position = p.rope_cursor[0];
+                float value = total;
+                if (n < p.rope_k_rows) {
+                    const float angle = __fmul_rn((float)position, p.rope_table[c]);
+                    const float cosine = cosf(angle), sine = sinf(angle);
+                    value = (i & 1u) ? total * cosine + other * sine : total * cosine - other * sine;
+                }
+                if (n < p.rope_q_rows) {
+                    p.y[n] = value;
+                } else if (position >= p.rope_capacity) {
+                    atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+                } else {
+                    const bool key = n < p.rope_k_rows;
+                    const uint32_t within = n - (key ? p.rope_q_rows : p.rope_k_rows);  // head * width + channel
+                    const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
+                    uint16_t *cache = key ? p.rope_k : p.rope_v;
+                    cache[((size_t)head * p.rope_capacity + position) * p.rope_width + channel] = float_to_half(value);
+                }
+            }
         } else if (u < R && i < p.N) {
             p.y[i] = p.residual ? p.residual[i] + total : total;
         }
@@ -955,6 +990,11 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     p.K = a.K;
     p.swiglu = a.swiglu;
     p.eps = a.eps;
+    if (a.rope) {
+        p.rope_table = a.rope->table, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
+        p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
+        p.refusal = d->refusal;
+    }
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     const bool q4 = a.element == NH_Q4_K;
     p.nblk = a.K / (q4 ? 256u : 32u);
@@ -1020,6 +1060,8 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         else if (nw == 8) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 8>), dim3((blocks_x + 1) / 2, p.splits), dim3(512), lds, d->stream, p); \
         else hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p);           \
     } while (0)
+    if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1))
+        return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (q4 && RB == 1 && fast) {
         if (R == 4) {
             if (p.group == 64) NH_DECODE(4, 64);
@@ -1170,7 +1212,21 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
     return NH_OK;
 }
 
+// mirrors the conditions under which launch_rows<1> takes the decode kernel with two rows per pass
+bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
+    if (env_int("NEURA_HIP_FUSE_ROPE", 1) == 0) return false;
+    if (a.element != NH_Q4_K || a.rows != 1 || a.swiglu || a.residual || a.K % 256u != 0 || a.K > 4096u) return false;
+    if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 256u * 144u) >= (1ull << 32)) return false;
+    if (env_int("NEURA_HIP_GEMV_ROWS", 2) != 2 || env_int("NEURA_HIP_MFMA", 1) == 2) return false;
+    const uint32_t width = rope.width;
+    if (width < 2 || (width & (width - 1u)) != 0) return false;
+    if (rope.q_rows % width || rope.k_rows % width || a.N % width || rope.q_rows > rope.k_rows || rope.k_rows > a.N) return false;
+    // a head never straddles two matrices
+    return a.end[0] % width == 0 && a.end[1] % width == 0 && a.end[2] == a.N;
+}
+
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
+    if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;

@@ -100,6 +100,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         return status;
     const float scale = 1.0f / sqrtf((float)hd);
     for (uint32_t L = 0; L < c.layers; L++) {
+        bool roped = false;
         if (wide) {
             if ((status = launch_rmsnorm(d, m->h, nullptr, m->attn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
             const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
@@ -115,9 +116,15 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             a.W[1] = m->attn_k[L], a.W[2] = m->attn_v[L];
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
+            // one token of one active plane: the rotation and the cache append ride in the product's epilogue
+            RopeFusion rope{rope_frequencies(d, c.rope_base, hd), dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
+            if (!products_only && T == 1 && !mask && rope.table && gemv_fuses_rope(a, rope)) {
+                a.rope = &rope;
+                roped = true;
+            }
             if ((status = launch_gemv(d, a)) != NH_OK) return status;
         }
-        if (!products_only && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
+        if (!products_only && !roped && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
                                                            m->capacity, m->window, dev_cursor(m), mask, c.rope_base)) != NH_OK)
             return status;
         AttentionArgs at{};

@@ -161,3 +161,35 @@ def test_graph_replays_match_eager_steps(device, monkeypatch):
             assert np.array_equal(replayed.cache_read(layer, which)[:, :, :40], eager.cache_read(layer, which)[:, :, :40])
     for held in (replayed, eager, weights_a, weights_b):
         held.release()
+
+
+def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, monkeypatch):
+    """At batch 1 the q|k|v product of a Q4_K decoder rotates q and k and appends k and v to the
+    caches in its epilogue; the same steps with the rotation as its own kernel give the same
+    bits in the caches and the logits."""
+    shape = SMALL_Q4
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    folded, ref, weights_a = build(device, shape, NH_Q4_K, batch=1, context=24, seed=9)
+    apart, _, weights_b = build(device, shape, NH_Q4_K, batch=1, context=24, seed=9)
+    token_a = token_b = 5
+    for step in range(8):
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1")
+        got_a = folded.decode_step([token_a], [step])
+        logits_a = folded.logits()
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "0")
+        got_b = apart.decode_step([token_b], [step])
+        logits_b = apart.logits()
+        assert np.array_equal(logits_a, logits_b), step
+        want_logits, want = ref.forward([token_a], 1, [step])
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * np.abs(want_logits).max()
+        assert list(got_a) == list(got_b) == list(want), step
+        token_a = token_b = int(got_a[0])
+    for layer in range(shape["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(folded.cache_read(layer, which), apart.cache_read(layer, which)), (layer, which)
+    # a cursor past the window is refused by the folded form as by the separate kernel
+    monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1")
+    with pytest.raises(NeuraError):
+        folded.decode_step([1], [folded.capacity + 3])
+    for held in (folded, apart, weights_a, weights_b):
+        held.release()
