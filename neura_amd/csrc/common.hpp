@@ -61,6 +61,9 @@ struct nh_device {
     int32_t compute_units = 0;
     void *scratch = nullptr;  // device scratch, `scratch_bytes` long
     size_t scratch_bytes = 0;
+    // counts the times the scratch or the rope table moved: a captured graph holds their addresses and is
+    // recorded again when this no longer matches the count at its capture
+    uint64_t moved = 0;
     uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
     float *rope_table = nullptr;  // device inverse frequencies of the last (base, width)
     float rope_base = 0.0f;
@@ -94,8 +97,8 @@ int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, u
 // output rows [0, q_rows) are rotated and written to y, rows [q_rows, k_rows) are rotated, rounded to fp16 and
 // written to the key cache at the cursor, the rest are rounded to fp16 into the value cache.
 struct RopeFusion {
-    const float *table;      // pow(base, -2c/width), c < width/2
-    const uint32_t *cursor;  // device, one plane
+    const float *cosines, *sines;  // [capacity][width / 2]: cos and sin of f32(position) * pow(base, -2c/width)
+    const uint32_t *cursor;        // device, one plane
     uint16_t *cache_k, *cache_v;
     uint32_t width, q_rows, k_rows, capacity;
 };
@@ -154,6 +157,8 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 
 // fused decode-side step: rope(q,k) + fp16 cache append from a token-major qkv buffer
 // qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane; q is roped in place.
+// cos / sin of every (position, channel pair) the rotation can meet, computed as the rotation kernels compute them
+int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t positions, float *cosines, float *sines);
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
                            const uint8_t *mask, float base);

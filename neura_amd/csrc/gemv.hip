@@ -34,7 +34,7 @@ struct GemvParams {
     int32_t swiglu;
     float eps;
     // rotation folded into the product (decode kernel only): see RopeFusion
-    const float *rope_table;
+    const float *rope_cosines, *rope_sines;  // [position][width / 2]
     const uint32_t *rope_cursor;
     uint16_t *rope_k, *rope_v;
     uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity;
@@ -265,7 +265,7 @@ struct DecodeTile {
 // activations in registers.  Every integer field is consumed as a half-precision subnormal by
 // mixed-precision multiply-adds (nibbles: * 2^-24 / 2^-20, undone by scaling the activations
 // once; scales: * 2^-24, undone once per pass), so a weight costs 1.6 vector instructions.
-template <int R, int G, bool PIPE, int NW>
+template <int R, int G, bool PIPE, int NW, bool ROPE = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) {
     extern __shared__ float xs[];  // skew64(slice)
     __shared__ float red[256];
@@ -297,8 +297,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
             // with the rotation folded in, logical rows 2t, 2t+1 are channels t and t + width/2 of one head
             const uint32_t logical = min(first, p.N - R);
             const uint32_t half = p.rope_width >> 1, pair = logical >> 1;
-            const uint32_t n = p.rope_table ? (pair / half) * p.rope_width + pair % half : logical;
-            const uint32_t hop = p.rope_table ? half : 1u;
+            const uint32_t n = ROPE ? (pair / half) * p.rope_width + pair % half : logical;
+            const uint32_t hop = ROPE ? half : 1u;
             const bool in0 = n < p.end[0], in1 = n < p.end[1];
             const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
             const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
         } else if (p.swiglu) {
             float up = dpp<DPP_QUAD_XOR1>(total);
             if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(total) * up;
-        } else if (p.rope_table) {
+        } else if (ROPE) {
             // lanes 0 and 1 hold channels c and c + width/2 of one head (crates/neura-kernel/src/task/rope.rs:95-122)
             const float other = dpp<DPP_QUAD_XOR1>(total);
             if (u < R && i < p.N) {
@@ -379,8 +379,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
                 const uint32_t position = p.rope_cursor[0];
                 float value = total;
                 if (n < p.rope_k_rows) {
-                    const float angle = __fmul_rn((float)position, p.rope_table[c]);
-                    const float cosine = cosf(angle), sine = sinf(angle);
+                    // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
+                    const float cosine = p.rope_cosines[(size_t)min(position, p.rope_capacity - 1u) * half + c];
+                    const float sine = p.rope_sines[(size_t)min(position, p.rope_capacity - 1u) * half + c];
                     value = (i & 1u) ? total * cosine + other * sine : total * cosine - other * sine;
                 }
                 if (n < p.rope_q_rows) {
@@ -991,7 +992,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     p.swiglu = a.swiglu;
     p.eps = a.eps;
     if (a.rope) {
-        p.rope_table = a.rope->table, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
+        p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
         p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
         p.refusal = d->refusal;
     }
@@ -1062,7 +1063,11 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     } while (0)
     if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1))
         return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
-    if (q4 && RB == 1 && fast) {
+    if (q4 && RB == 1 && fast && a.rope) {
+        if (p.group == 64) hipLaunchKernelGGL((gemv_q4k_decode_kernel<2, 64, false, 4, true>), grid, block, lds, d->stream, p);
+        else if (p.group == 32) hipLaunchKernelGGL((gemv_q4k_decode_kernel<2, 32, false, 4, true>), grid, block, lds, d->stream, p);
+        else hipLaunchKernelGGL((gemv_q4k_decode_kernel<2, 16, false, 4, true>), grid, block, lds, d->stream, p);
+    } else if (q4 && RB == 1 && fast) {
         if (R == 4) {
             if (p.group == 64) NH_DECODE(4, 64);
             else if (p.group == 32) NH_DECODE(4, 32);

@@ -23,6 +23,7 @@ struct nh_model {
     size_t cache_elements = 0;  // per layer and per K or V
     // activations; T = rows * batch flattened token rows, t = row * batch + plane
     float *h = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr, *act = nullptr, *up = nullptr, *logits = nullptr;
+    float *rope_cos = nullptr, *rope_sin = nullptr;  // [capacity][head_dim / 2], for the rotation folded into the q|k|v product
     uint32_t *inputs_dev = nullptr;  // [tokens T_max | cursors B | mask bytes B]
     uint32_t *chosen_dev = nullptr;
     uint8_t *inputs_host = nullptr;  // pinned mirror of inputs_dev
@@ -30,6 +31,7 @@ struct nh_model {
     uint32_t max_tokens = 0;
     // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked
     hipGraphExec_t decode_graph[2] = {nullptr, nullptr};
+    uint64_t graph_moved[2] = {0, 0};  // nh_device::moved when each graph was recorded
     bool use_graph = true;
 };
 
@@ -44,7 +46,7 @@ void release(nh_model *m) {
         if (graph) (void)hipGraphExecDestroy(graph);
     for (auto p : m->cache_k) (void)hipFree(p);
     for (auto p : m->cache_v) (void)hipFree(p);
-    float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits};
+    float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits, m->rope_cos, m->rope_sin};
     for (float *p : buffers)
         if (p) (void)hipFree(p);
     if (m->inputs_dev) (void)hipFree(m->inputs_dev);
@@ -117,8 +119,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
             // one token of one active plane: the rotation and the cache append ride in the product's epilogue
-            RopeFusion rope{rope_frequencies(d, c.rope_base, hd), dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
-            if (!products_only && T == 1 && !mask && rope.table && gemv_fuses_rope(a, rope)) {
+            RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
+            if (!products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
                 roped = true;
             }
@@ -261,7 +263,8 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     ok = device_array(m->h, T * H) && device_array(m->xn, T * H) && device_array(m->qkv, T * (QW + 2 * KW)) &&
          device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T > 8 ? T * F : 1) &&
          device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 2 * c.batch + 4) &&
-         device_array(m->chosen_dev, c.batch);
+         device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->capacity * (c.head_dim / 2)) &&
+         device_array(m->rope_sin, (size_t)m->capacity * (c.head_dim / 2));
     for (uint32_t L = 0; ok && L < c.layers; L++) {
         uint16_t *k = nullptr, *v = nullptr;
         ok = device_array(k, m->cache_elements);
@@ -281,9 +284,15 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         size_t products = 8 * 4 * widest * sizeof(float);
         size_t sections = (size_t)256 * c.heads * T * (c.head_dim + 2) * sizeof(float);
         size_t choice = (size_t)c.batch * 1024 * 8;
+        // the wide product keeps its fp32 activations as two half rows each, plus a scale per row
+        size_t deepest = (size_t)(F > QW ? F : QW);
+        if (H > deepest) deepest = H;
+        size_t split_rows = T > 8 ? (size_t)2 * T * deepest * 2 + T * sizeof(float) : 0;
         size_t wanted = products > sections ? products : sections;
         if (choice > wanted) wanted = choice;
-        ok = ok && scratch(device, wanted) != nullptr && rope_frequencies(device, c.rope_base, c.head_dim) != nullptr;
+        if (split_rows > wanted) wanted = split_rows;
+        ok = ok && scratch(device, wanted) != nullptr && rope_frequencies(device, c.rope_base, c.head_dim) != nullptr &&
+             launch_rope_angles(device, c.rope_base, c.head_dim, m->capacity, m->rope_cos, m->rope_sin) == NH_OK;
     }
     {
         const char *held = getenv("NEURA_HIP_GRAPH");
@@ -322,7 +331,13 @@ int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *curs
     // Profiled steps run eagerly (event records do not belong in a graph).
     hipGraphExec_t &graph = m->decode_graph[any_inactive ? 1 : 0];
     if (m->use_graph && !d->profile) {
+        if (graph && m->graph_moved[any_inactive ? 1 : 0] != d->moved) {
+            // the device scratch or rope table moved since the capture (another model or operator call grew it)
+            (void)hipGraphExecDestroy(graph);
+            graph = nullptr;
+        }
         if (!graph) {
+            m->graph_moved[any_inactive ? 1 : 0] = d->moved;
             NH_HIP(hipStreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal));
             status = decode_kernels(m, any_inactive);
             hipGraph_t recorded = nullptr;

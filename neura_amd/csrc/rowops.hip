@@ -121,6 +121,27 @@ int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_
     return NH_OK;
 }
 
+__global__ __launch_bounds__(256) void rope_angles_kernel(const float *__restrict__ table, uint32_t half, uint32_t positions,
+                                                          float *__restrict__ cosines, float *__restrict__ sines) {
+    const uint64_t total = (uint64_t)positions * half;
+    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < total; index += (uint64_t)gridDim.x * blockDim.x) {
+        const float angle = __fmul_rn((float)(uint32_t)(index / half), table[index % half]);  // as rotate() forms it
+        cosines[index] = cosf(angle);
+        sines[index] = sinf(angle);
+    }
+}
+
+int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t positions, float *cosines, float *sines) {
+    const float *table = rope_frequencies(d, base, width);
+    if (!table) return NH_E_DEVICE;
+    const uint64_t total = (uint64_t)positions * (width / 2);
+    if (!total) return NH_OK;
+    uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    hipLaunchKernelGGL(rope_angles_kernel, dim3(grid), dim3(256), 0, d->stream, table, width / 2, positions, cosines, sines);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
 // The decoder's fused form of the two kernels above on a token-major buffer
 // qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane: q is roped in place, k is
 // roped, k and v are cast to fp16 and appended to the caches.

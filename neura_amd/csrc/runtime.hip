@@ -41,6 +41,7 @@ void *scratch(nh_device *device, size_t bytes) {
     }
     device->scratch = held;
     device->scratch_bytes = wanted;
+    device->moved++;
     return held;
 }
 
@@ -66,6 +67,7 @@ const float *rope_frequencies(nh_device *device, float base, uint32_t width) {
         return nullptr;
     }
     device->rope_table = held;
+    device->moved++;
     device->rope_base = base;
     device->rope_width = width;
     return held;

@@ -193,3 +193,25 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         folded.decode_step([1], [folded.capacity + 3])
     for held in (folded, apart, weights_a, weights_b):
         held.release()
+
+
+def test_a_recorded_step_survives_a_scratch_that_moves(device):
+    """The recorded decode step holds addresses inside the device scratch; an operator call that makes the
+    scratch grow (and move) in between must not leave the replay reading freed memory."""
+    shape = SMALL_Q4
+    model, ref, weights = build(device, shape, NH_Q4_K, batch=2, context=16, seed=13)
+    tokens = [3, 4]
+    for step in range(2):
+        want_logits, want = ref.forward(tokens, 1, [step, step])
+        tokens = list(model.decode_step(tokens, [step, step]))
+        assert tokens == list(want)
+    # a wide product with fp32 activations large enough to outgrow whatever scratch the device holds now
+    rng = np.random.default_rng(1)
+    M, N, K = 2048, 128, 16384
+    device.gemm(NH_Q4_K, synth.q4_k_random(rng, N * K), N, K, rng.standard_normal((M, K)).astype(np.float32))
+    for step in range(2, 5):
+        want_logits, want = ref.forward(tokens, 1, [step, step])
+        tokens = list(model.decode_step(tokens, [step, step]))
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max()
+        assert tokens == list(want)
+    model.release(), weights.release()
