@@ -320,7 +320,33 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
     DecodeTile<R> ta, tb;
     if (rg < p.row_groups) load(ta, rg);  // in flight while the activations are staged
 
-    {
+    if (NW == 4 && p.splits == 1 && p.K <= 4096u) {
+        // a whole row is at most 16 values per thread: every load goes out before the first is used (a loop
+        // that adds each value as it arrives spends a memory round trip per value), and the row is read once
+        float held[16], weight[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t c = tid + 256u * j;
+            held[j] = c < p.K ? p.x[c] : 0.0f;
+            weight[j] = (p.norm_w && c < p.K) ? p.norm_w[c] : 0.0f;
+        }
+        if (p.norm_w) {
+            float square = 0.0f;  // thread t adds columns t, t + 256, ... in order (crates/neura-kernel/src/task/norm.rs:69-83)
+#pragma unroll
+            for (int j = 0; j < 16; j++) square = __fadd_rn(square, __fmul_rn(held[j], held[j]));
+            square = wave_sum(square);
+            if (lane == 0) red[wave] = square;
+            __syncthreads();
+            const float scale = rms_scale_of((red[0] + red[1]) + (red[2] + red[3]), p.K, p.eps);
+#pragma unroll
+            for (int j = 0; j < 16; j++) held[j] = __fmul_rn(__fmul_rn(held[j], scale), weight[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t c = tid + 256u * j;
+            if (c < kn) xs[skew64(c)] = held[j];
+        }
+    } else {
         float scale = 1.0f;
         if (p.norm_w) scale = rms_scale(p.x, p.K, p.eps, red);
         for (uint32_t i = tid; i < kn; i += NW * 64) {
