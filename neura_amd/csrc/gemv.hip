@@ -781,15 +781,64 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
     for (int i = 0; i < D; i++) fetch(ring[i]);
 
     // ---- activations -> integer digits in operand order
+    // A thread takes chunks of 8 activations (8 consecutive chunks = one 64-element group).  When the slice is at most
+    // four chunks per thread, every load goes out before the first value is used and the row is read once; a deeper
+    // slice is walked twice (largest magnitude, then digits) with its loads one after the other.
+    const uint32_t chunks = nb * 32u;
+    const bool resident = chunks <= 4u * NT && (!p.norm_w || p.K == kn);
     for (uint32_t row = 0; row < P; row++) {
         const float *xr = p.x + (size_t)min(row, p.rows - 1u) * p.K;
+        float t[4][8];
         float rms = 1.0f;
-        if (p.norm_w) rms = rms_scale(xr, p.K, p.eps, red);
         uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
-        for (uint32_t i = tid; i < kn; i += NT) {
-            float value = xr[k0 + i];
-            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, rms), p.norm_w[k0 + i]);
-            top = max(top, __builtin_bit_cast(uint32_t, value) & 0x7fffffffu);
+        if (resident) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t q = tid + NT * j;
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+                if (q < chunks) a = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q), b = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q + 4u);
+                t[j][0] = a.x, t[j][1] = a.y, t[j][2] = a.z, t[j][3] = a.w, t[j][4] = b.x, t[j][5] = b.y, t[j][6] = b.z, t[j][7] = b.w;
+            }
+            if (p.norm_w) {
+                // the whole row is in registers: sum of squares (thread order differs from the reference's strided sum), then scale and weight
+                float4 wa[4], wb[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t q = tid + NT * j;
+                    wa[j] = wb[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (q < chunks) wa[j] = *reinterpret_cast<const float4 *>(p.norm_w + 8u * q), wb[j] = *reinterpret_cast<const float4 *>(p.norm_w + 8u * q + 4u);
+                }
+                float square = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int i = 0; i < 8; i++) square = __fadd_rn(square, __fmul_rn(t[j][i], t[j][i]));
+                square = wave_sum(square);
+                if (lane == 0) red[wave] = square;
+                __syncthreads();
+                float total = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NW; w++) total += red[w];
+                __syncthreads();
+                rms = rms_scale_of(total, p.K, p.eps);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float w[8] = {wa[j].x, wa[j].y, wa[j].z, wa[j].w, wb[j].x, wb[j].y, wb[j].z, wb[j].w};
+#pragma unroll
+                    for (int i = 0; i < 8; i++) t[j][i] = __fmul_rn(__fmul_rn(t[j][i], rms), w[i]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) top = max(top, __builtin_bit_cast(uint32_t, t[j][i]) & 0x7fffffffu);
+        } else {
+            if (p.norm_w) rms = rms_scale(xr, p.K, p.eps, red);
+            for (uint32_t i = tid; i < kn; i += NT) {
+                float value = xr[k0 + i];
+                if (p.norm_w) value = __fmul_rn(__fmul_rn(value, rms), p.norm_w[k0 + i]);
+                top = max(top, __builtin_bit_cast(uint32_t, value) & 0x7fffffffu);
+            }
         }
 #pragma unroll
         for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
@@ -804,56 +853,64 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
         const uint32_t exponent = min(max(raw_exponent, 30u), 254u);
         const float scale = __builtin_bit_cast(float, (283u - exponent) << 23);
         if (tid == 0) unscale[row] = raw_exponent == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 29u) << 23);
-        const uint32_t chunks = nb * 32u;  // 8 activations each; 8 consecutive chunks = one 64-element group
-        for (uint32_t first = 0; first < chunks; first += NT) {
-            const uint32_t q = first + tid;
-            const bool held = q < chunks;
-            float t[8];
-            if (held) {
-                const float4 a = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q), b = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q + 4u);
-                t[0] = a.x, t[1] = a.y, t[2] = a.z, t[3] = a.w, t[4] = b.x, t[5] = b.y, t[6] = b.z, t[7] = b.w;
-                if (p.norm_w) {
-                    const float4 wa = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q), wb = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q + 4u);
-                    const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
-#pragma unroll
-                    for (int i = 0; i < 8; i++) t[i] = __fmul_rn(__fmul_rn(t[i], rms), w[i]);
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; i++) t[i] = 0.0f;
-            }
-            // four signed base-256 digits of each rounded activation, most significant first, one byte per element
+        // one chunk: four signed base-256 digits of each rounded activation, most significant first, one byte per element
+        auto stage = [&](uint32_t q, bool held, const float (&v)[8]) {
             float total = 0.0f;
-            auto digits_of = [&](float v0, float v1, float v2, float v3, uint32_t &w0, uint32_t &w1, uint32_t &w2, uint32_t &w3) {
-                const float in[4] = {v0, v1, v2, v3};
-                w0 = w1 = w2 = w3 = 0u;
+            uint32_t word[2][4];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                word[h][0] = word[h][1] = word[h][2] = word[h][3] = 0u;
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float rounded = rintf(in[i] * scale);
+                    const float rounded = rintf(v[4 * h + i] * scale);
                     const int whole = (int)rounded;
                     const int d3 = (whole << 24) >> 24, upper = (whole - d3) >> 8;
                     const int d2 = (upper << 24) >> 24, top2 = (upper - d2) >> 8;
                     const int d1 = (top2 << 24) >> 24, d0 = (top2 - d1) >> 8;
                     total += rounded;
-                    w0 |= ((uint32_t)d0 & 0xffu) << (8 * i);
-                    w1 |= ((uint32_t)d1 & 0xffu) << (8 * i);
-                    w2 |= ((uint32_t)d2 & 0xffu) << (8 * i);
-                    w3 |= ((uint32_t)d3 & 0xffu) << (8 * i);
+                    word[h][0] |= ((uint32_t)d0 & 0xffu) << (8 * i);
+                    word[h][1] |= ((uint32_t)d1 & 0xffu) << (8 * i);
+                    word[h][2] |= ((uint32_t)d2 & 0xffu) << (8 * i);
+                    word[h][3] |= ((uint32_t)d3 & 0xffu) << (8 * i);
                 }
-            };
-            uint32_t a0, a1, a2, a3, b0, b1, b2, b3;
-            digits_of(t[0], t[1], t[2], t[3], a0, a1, a2, a3);
-            digits_of(t[4], t[5], t[6], t[7], b0, b1, b2, b3);
+            }
             // sum of the 32 activations of this chunk's sub-block: 4 chunks = 4 neighbouring lanes
             total += dpp<DPP_QUAD_XOR1>(total);
             total += dpp<DPP_QUAD_XOR2>(total);
             if (held) {
                 // chunk q = elements 8m..8m+7 of half `upper` of group g: nibble words 2m, 2m+1 of that half
                 const uint32_t b = q >> 5, g = (q >> 3) & 3u, upper = (q >> 2) & 1u, step = 8u * upper + 2u * (q & 3u);
-                uint32_t *slot = xop + ((size_t)(b * 16u + step) * 4u + g) * NCW + 4u * row;
-                slot[0] = a0, slot[1] = a1, slot[2] = a2, slot[3] = a3;
-                slot[4u * NCW] = b0, slot[4u * NCW + 1u] = b1, slot[4u * NCW + 2u] = b2, slot[4u * NCW + 3u] = b3;
+                uint4 *slot = reinterpret_cast<uint4 *>(xop + ((size_t)(b * 16u + step) * 4u + g) * NCW + 4u * row);
+                slot[0] = make_uint4(word[0][0], word[0][1], word[0][2], word[0][3]);
+                slot[NCW] = make_uint4(word[1][0], word[1][1], word[1][2], word[1][3]);  // the next step: 4 groups * NCW words further
                 if ((q & 3u) == 0) xsum[((size_t)(b * 4u + g) * P + row) * 2u + upper] = total;
+            }
+        };
+        if (resident) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (NT * j >= chunks) break;  // uniform over the workgroup
+                stage(tid + NT * j, tid + NT * j < chunks, t[j]);
+            }
+        } else {
+            for (uint32_t first = 0; first < chunks; first += NT) {
+                const uint32_t q = first + tid;
+                const bool held = q < chunks;
+                float v[8];
+                if (held) {
+                    const float4 a = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q), b = *reinterpret_cast<const float4 *>(xr + k0 + 8u * q + 4u);
+                    v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+                    if (p.norm_w) {
+                        const float4 wa = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q), wb = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 8u * q + 4u);
+                        const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+                        for (int i = 0; i < 8; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) v[i] = 0.0f;
+                }
+                stage(q, held, v);
             }
         }
     }
@@ -1158,11 +1215,12 @@ static hipError_t launch_mfma_instance(nh_device *d, const MfmaParams &p, uint32
 template <int KS, int NW>
 static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t P, uint32_t blocks_x, size_t lds) {
     if (P == 1) {
-        const int depth = env_int("NEURA_HIP_MFMA_DEPTH", 4);
-        if (depth == 2) return launch_mfma_instance<KS, NW, 1, 2>(d, p, blocks_x, lds);
+        // sixteen waves leave 128 registers a lane: two super-blocks in flight fit, four would spill
+        const int depth = env_int("NEURA_HIP_MFMA_DEPTH", NW == 16 ? 2 : 4);
+        if (depth == 2 || NW == 16) return launch_mfma_instance<KS, NW, 1, 2>(d, p, blocks_x, lds);
         return launch_mfma_instance<KS, NW, 1, 4>(d, p, blocks_x, lds);
     }
-    if (P == 2) return launch_mfma_instance<KS, NW, 2, 3>(d, p, blocks_x, lds);
+    if (P == 2) return launch_mfma_instance<KS, NW, 2, 2>(d, p, blocks_x, lds);
     return launch_mfma_instance<KS, NW, 4, 2>(d, p, blocks_x, lds);
 }
 
@@ -1207,6 +1265,7 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
         while (ks < 16 && p.tiles * p.splits * ks < slots && ks * 2 <= p.slice_blocks) ks *= 2;
         ks = (uint32_t)env_int("NEURA_HIP_MFMA_KS", (int)ks);
         if (ks != 1 && ks != 2 && ks != 4 && ks != 8 && ks != 16) ks = 1;
+        if (P > 1 && ks > 8) ks = 8;  // sixteen-wave workgroups leave 128 registers a lane, too few for several activation rows
         // waves per workgroup: four measured best (larger workgroups stage the activations less often but stream slower)
         uint32_t nw = (uint32_t)env_int("NEURA_HIP_MFMA_NW", 4);
         if (nw != 4 && nw != 8 && nw != 16) nw = 4;
