@@ -66,19 +66,13 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     const uint32_t section = blockIdx.y;
     const uint32_t G = p.groups;
 
-    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
-    if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
-        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-        origin = p.keys - p.rows;
-    }
-    const uint32_t visible = min(p.keys, origin + row + 1u);  // key `at` counts iff at <= origin + row
-    const uint32_t chunk = (visible + p.sections - 1u) / p.sections;
-    const uint32_t first = min(visible, section * chunk), last = min(visible, first + chunk);
-
-    // K and V rows of the first two steps go out before anything else
+    // A section is a fixed span of the window, whatever the cursor says: the K and V rows of its first two
+    // steps go out before the cursor has even arrived (rows past the visible keys are fetched and dropped).
+    const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
+    const uint32_t begin = min(p.keys, section * chunk);
     const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
     const uint32_t step = 4u * KPW;
-    uint32_t key = first + wave * KPW + sub;
+    uint32_t key = begin + wave * KPW + sub;
     uint4 kraw[2], vraw[2];
 #pragma unroll
     for (int ahead = 0; ahead < 2; ahead++) {
@@ -87,6 +81,14 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
         kraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_k + at);
         vraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_v + at);
     }
+
+    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
+    if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        origin = p.keys - p.rows;
+    }
+    const uint32_t visible = min(p.keys, origin + row + 1u);  // key `at` counts iff at <= origin + row
+    const uint32_t last = min(visible, begin + chunk);
 
     float qr[MAX_GROUPS][8], acc[MAX_GROUPS][8], top[MAX_GROUPS], mass[MAX_GROUPS];
 #pragma unroll

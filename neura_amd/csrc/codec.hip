@@ -56,7 +56,7 @@ int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, u
 }
 
 // out[t][c] = dequant(table[token[t]])[c] * mask[t % batch]   (crates/neura-kernel/src/task/select.rs:29-49,
-// examples/qwen/model.rs:94).  One workgroup per token row.
+// examples/qwen/model.rs:94).  One thread per element: blockIdx.y walks the row in spans of 256.
 template <int ELEMENT>
 __global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__ table, uint32_t vocab, uint32_t width, uint64_t row_bytes,
                                                      const uint32_t *__restrict__ tokens, uint32_t batch,
@@ -65,12 +65,12 @@ __global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__
     uint32_t token = tokens[t];
     float keep = (mask == nullptr || mask[t % batch]) ? 1.0f : 0.0f;
     if (token >= vocab) {
-        if (threadIdx.x == 0) atomicMax(refusal, (uint32_t)REFUSAL_INDEX);
-        for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) out[(uint64_t)t * width + c] = 0.0f;
+        if (threadIdx.x == 0 && blockIdx.y == 0) atomicMax(refusal, (uint32_t)REFUSAL_INDEX);
+        for (uint32_t c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) out[(uint64_t)t * width + c] = 0.0f;
         return;
     }
     const uint8_t *row = table + (uint64_t)token * row_bytes;
-    for (uint32_t c = threadIdx.x; c < width; c += blockDim.x) {
+    for (uint32_t c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
         float value;
         if (ELEMENT == NH_Q8_0)
             value = q8_0_element(row, c);
@@ -89,21 +89,23 @@ int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t
     if (!count) return NH_OK;
     const uint8_t *bytes = static_cast<const uint8_t *>(table);
     uint64_t row_bytes = payload_bytes(element, width);
+    uint32_t spans = (width + 255) / 256;
+    const dim3 grid(count, spans < 64 ? spans : 64);
     switch (element) {
     case NH_Q8_0:
-        hipLaunchKernelGGL(gather_kernel<NH_Q8_0>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+        hipLaunchKernelGGL(gather_kernel<NH_Q8_0>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     case NH_Q4_K:
-        hipLaunchKernelGGL(gather_kernel<NH_Q4_K>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+        hipLaunchKernelGGL(gather_kernel<NH_Q4_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     case NH_F16:
-        hipLaunchKernelGGL(gather_kernel<NH_F16>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+        hipLaunchKernelGGL(gather_kernel<NH_F16>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     case NH_F32:
-        hipLaunchKernelGGL(gather_kernel<NH_F32>, dim3(count), dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+        hipLaunchKernelGGL(gather_kernel<NH_F32>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     default: return fail(NH_E_ARGUMENT, "element %d carries no reader", element);
