@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one Q4_K product launch of the 7B-shape decode step moves on average, from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_q4k_decode_hbm_counters.md
 # (each counter scaled by its reading for a plain 1 GiB copy); not measurable inside this script
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 36.06e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.79e6}
 
 
 def workload(name):
@@ -90,6 +90,35 @@ def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=2
     }
 
 
+def gemm_config3(device, rng, repeats=10):
+    """BASELINE config 3: the Q4_K wide product M=512, K=3584, N=18944 (the 7B-shape FFN up projection), with half
+    activations as the configuration states them and with fp32 activations as the decoder's fill passes them."""
+    import ctypes
+
+    from neura_amd import synth
+
+    M, K, N = 512, 3584, 18944
+    raw = device.upload(synth.q4_k_random(rng, N * K))
+    y = device.alloc(M * N * 4)
+    out = {"workload": "Q4_K wide product M=%d K=%d N=%d, random blocks, N(0,1) activations" % (M, K, N), "flop": 2.0 * M * N * K,
+           "mfma_peak_tflops": 2500.0}
+    for name, dtype, code in (("half_activations", np.float16, 1), ("fp32_activations", np.float32, 0)):
+        x = device.upload(rng.standard_normal((M, K)).astype(dtype))
+        for timed in (False, True):
+            if timed:
+                device.sync()
+                device.timer_start()
+            for _ in range(repeats if timed else 3):
+                status = device.lib.nh_gemm(device.handle, 12, raw.pointer, N, K, x.pointer, code, M, y.pointer, None)
+                assert status == 0, device.lib.nh_last_error()
+        seconds = device.timer_stop() / repeats
+        out[name] = {"us": seconds * 1e6, "tflops": 2.0 * M * N * K / seconds / 1e12, "frac_of_mfma_peak": 2.0 * M * N * K / seconds / 2.5e15}
+        x.release()
+    raw.release()
+    y.release()
+    return out
+
+
 def extras(device, weights, shape, element, context, layers, rng):
     """The other two measurements the workload names, on the same resident weights: decode at
     batch 8 (eight sequences at the end of their context) and a 512-token prompt fill."""
@@ -129,6 +158,7 @@ def extras(device, weights, shape, element, context, layers, rng):
                           "note": "one 512-row fill at cursor 0, all products on f16 MFMA with fp32 activations as (value, residue) half rows; "
                                   "product_tflops counts 2*M*N*K of the products over the whole fill time"}
     model.release()
+    out["gemm_config3"] = gemm_config3(device, rng)
     return out
 
 
@@ -140,7 +170,8 @@ def main():
     parser.add_argument("--workload", default="qwen2.5-7b-q4k")
     parser.add_argument("--layers", type=int, default=None, help="cut the decoder (for quick checks; the result is then not the headline)")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode and 512-token fill measurements")
+    parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode, 512-token fill and wide-product measurements")
+    parser.add_argument("--gemm-only", action="store_true", help="run only the wide product of BASELINE config 3 and print its line")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()
@@ -151,6 +182,11 @@ def main():
     from neura_amd import synth
     from neura_amd.loader import Model, Weights
 
+    if args.gemm_only:
+        device = neura_amd.Device(0)
+        print(json.dumps({"gemm_config3": gemm_config3(device, np.random.default_rng(0))}))
+        device.close()
+        return
     shape, element, context = workload(args.workload)
     layers = shape["layers"] if args.layers is None else args.layers
     rng = np.random.default_rng(0)
@@ -212,7 +248,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q4k_kernel" if element == 12 else "gemv_q8_0_kernel",
+            "kernel": "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_kernel (down)" if element == 12 else "gemv_q8_0_kernel",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -1232,9 +1232,8 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
     const uint32_t nblk = a.K / 256u;
     const size_t room = 140 * 1024;  // a gfx950 workgroup may take all 160 KiB of a compute unit; tile partials and static arrays need the rest
     for (uint32_t done = 0; done < a.rows;) {
-        // activation rows per launch: 4, 2 or 1 (the kernel's instantiations), fewer when a whole row would not fit beside them
+        // activation rows per launch: 4, 2 or 1 (the kernel's instantiations); rows too deep to stage whole are cut into K slices
         uint32_t left = a.rows - done, P = left >= 3 ? 4u : left;
-        while (P > 1 && mfma_staged(nblk, P) > room) P /= 2;
         MfmaParams p{};
         for (int s = 0; s < 3; s++) {
             p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
