@@ -2,12 +2,16 @@
 //
 // One workgroup serves one (kv head, plane, query row, key section): the `groups` query
 // heads that share the kv head ride along, so every K/V row is fetched once for all of them.
-// A key row of `WIDTH` halves is read by WIDTH/8 lanes with one 128-bit load each; a wave
-// therefore walks 64/(WIDTH/8) keys per step and the four waves of a workgroup interleave.
-// Every lane keeps a running (max, sum, accumulator) for its own key stream; streams are
-// merged with shuffles inside a wave, through LDS across waves, and across sections by a
-// second kernel (crates/neura-kernel/src/task/attention.rs:619-671 does the same fold).
-// The K/V rows of two steps ahead are always in flight.
+// A section is walked in tiles of 64 keys, three passes per tile:
+//   scores  a key row of `WIDTH` halves is read by WIDTH/8 lanes with one 128-bit load each and
+//           dotted with the query heads in registers (DPP sums across the lanes of a key); the
+//           value rows of the tile go to LDS as they arrive;
+//   weights one wave per query head, one lane per key: tile maximum, exp, running (top, mass);
+//   values  every thread owns a few channels and a slice of the tile's keys and adds
+//           weight * value from LDS, so no accumulator ever crosses lanes.
+// Rescaling happens once per tile, not per key.  The slices meet in LDS at the end; sections
+// are merged by a second kernel (crates/neura-kernel/src/task/attention.rs:619-671 does the
+// same fold).  The next tile's K/V rows are in flight during the weight and value passes.
 #include "blocks.hpp"
 #include "common.hpp"
 
@@ -29,7 +33,9 @@ struct AttentionParams {
     uint32_t *refusal;
 };
 
-__device__ __forceinline__ void unpack8(const uint4 &raw, float (&out)[8]) {
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void unpack8(const u32x4 &raw, float (&out)[8]) {
     const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -53,11 +59,35 @@ __device__ __forceinline__ float key_sum(float v) {
     return v;
 }
 
+// the K and V rows (8 halves per lane) of the T steps of one tile; `first` is this lane's key in step 0
+template <int T, int STEP, int WIDTH>
+__device__ __forceinline__ void fetch_tile(u32x4 (&kraw)[T], u32x4 (&vraw)[T], const uint16_t *__restrict__ cache_k,
+                                           const uint16_t *__restrict__ cache_v, uint64_t plane, uint32_t first, uint32_t capacity, uint32_t dl) {
+#pragma unroll
+    for (int s = 0; s < T; s++) {
+        const uint32_t at_key = min(first + s * STEP, capacity - 1u);
+        const uint64_t at = (plane + at_key) * WIDTH + dl * 8u;
+        kraw[s] = *reinterpret_cast<const u32x4 *>(cache_k + at);
+        vraw[s] = *reinterpret_cast<const u32x4 *>(cache_v + at);
+    }
+}
+
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
-    constexpr int LPK = WIDTH / 8;   // lanes per key
-    constexpr int KPW = 64 / LPK;    // keys per wave step
-    __shared__ float merged[4][MAX_GROUPS][WIDTH + 2];
+    constexpr int LPK = WIDTH / 8;                       // lanes per key in the score pass
+    constexpr int KPW = 64 / LPK, STEP = 4 * KPW;        // keys per wave and per workgroup step
+    constexpr int TK = 64, T = TK / STEP;                // keys and steps per tile
+    constexpr int DPT = WIDTH >= 64 ? WIDTH / 64 : 1;    // channels per thread in the value pass
+    constexpr int TPS = WIDTH / DPT;                     // threads per key slice in the value pass
+    constexpr int SLICES = 256 / TPS, KPS = TK / SLICES; // key slices of a tile and keys per slice
+    // the tile's value rows, and once the last tile is done the slices' sums, share one buffer
+    constexpr size_t VT_BYTES = sizeof(uint16_t) * TK * WIDTH, MERGED_BYTES = sizeof(float) * SLICES * MAX_GROUPS * WIDTH;
+    __shared__ __attribute__((aligned(16))) uint8_t shared_rows[VT_BYTES > MERGED_BYTES ? VT_BYTES : MERGED_BYTES];
+    uint16_t(*vt)[WIDTH] = reinterpret_cast<uint16_t(*)[WIDTH]>(shared_rows);
+    float(*merged)[MAX_GROUPS][WIDTH] = reinterpret_cast<float(*)[MAX_GROUPS][WIDTH]>(shared_rows);
+    __shared__ __attribute__((aligned(16))) float scores[TK][MAX_GROUPS];  // scores, then weights, of the tile's keys
+    __shared__ float tile_scale[MAX_GROUPS];                               // exp(old top - new top) per query head
+    __shared__ float stat_top[MAX_GROUPS], stat_mass[MAX_GROUPS];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t sub = lane / LPK, dl = lane % LPK;
     const uint32_t unit = blockIdx.x;  // (kv head, plane, row)
@@ -66,21 +96,14 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     const uint32_t section = blockIdx.y;
     const uint32_t G = p.groups;
 
-    // A section is a fixed span of the window, whatever the cursor says: the K and V rows of its first two
-    // steps go out before the cursor has even arrived (rows past the visible keys are fetched and dropped).
+    // A section is a fixed span of the window, whatever the cursor says: the K and V rows of its first tile
+    // go out before the cursor has even arrived (rows past the visible keys are fetched and dropped).
     const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
     const uint32_t begin = min(p.keys, section * chunk);
     const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
-    const uint32_t step = 4u * KPW;
-    uint32_t key = begin + wave * KPW + sub;
-    uint4 kraw[2], vraw[2];
-#pragma unroll
-    for (int ahead = 0; ahead < 2; ahead++) {
-        const uint32_t at_key = min(key + ahead * step, p.capacity - 1u);
-        const uint64_t at = (plane + at_key) * WIDTH + dl * 8u;
-        kraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_k + at);
-        vraw[ahead] = *reinterpret_cast<const uint4 *>(p.cache_v + at);
-    }
+    const uint32_t mine = wave * KPW + sub;  // this lane's key inside a step
+    u32x4 kraw[T], vraw[T];
+    fetch_tile<T, STEP, WIDTH>(kraw, vraw, p.cache_k, p.cache_v, plane, begin + mine, p.capacity, dl);
 
     uint32_t origin = p.cursor ? p.cursor[b] : 0u;
     if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
@@ -90,91 +113,117 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     const uint32_t visible = min(p.keys, origin + row + 1u);  // key `at` counts iff at <= origin + row
     const uint32_t last = min(visible, begin + chunk);
 
-    float qr[MAX_GROUPS][8], acc[MAX_GROUPS][8], top[MAX_GROUPS], mass[MAX_GROUPS];
+    float qr[MAX_GROUPS][8];
 #pragma unroll
     for (int g = 0; g < MAX_GROUPS; g++) {
-        top[g] = -INFINITY;
-        mass[g] = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 8; j++) acc[g][j] = 0.0f, qr[g][j] = 0.0f;
+        for (int j = 0; j < 8; j++) qr[g][j] = 0.0f;
         if (g < (int)G) {
             const float *src = p.q + (uint64_t)(kvh * G + g) * p.q_sh + (uint64_t)b * p.q_sb + (uint64_t)row * p.q_sr + dl * 8u;
 #pragma unroll
             for (int j = 0; j < 8; j++) qr[g][j] = src[j];
         }
     }
-    for (; key < last; key += 2u * step) {
+    // value pass: this thread sums DPT channels over the keys of one slice of every tile
+    const uint32_t slice = tid / TPS, channel = (tid % TPS) * DPT;
+    float acc[MAX_GROUPS][DPT];
 #pragma unroll
-        for (int phase = 0; phase < 2; phase++) {
-            const uint32_t now = key + phase * step;
-            float kf[8], vf[8];
-            unpack8(kraw[phase], kf);
-            unpack8(vraw[phase], vf);
-            {  // the loads of two steps ahead reuse this phase's registers
-                const uint32_t at_key = min(now + 2u * step, p.capacity - 1u);
-                const uint64_t at = (plane + at_key) * WIDTH + dl * 8u;
-                kraw[phase] = *reinterpret_cast<const uint4 *>(p.cache_k + at);
-                vraw[phase] = *reinterpret_cast<const uint4 *>(p.cache_v + at);
-            }
-            if (now < last) {
+    for (int g = 0; g < MAX_GROUPS; g++)
 #pragma unroll
-                for (int g = 0; g < MAX_GROUPS; g++) {
-                    if (g >= (int)G) break;
+        for (int d = 0; d < DPT; d++) acc[g][d] = 0.0f;
+    // softmax statistics: wave w keeps the running top and mass of query heads w and w + 4 (the same in all its lanes)
+    float top[2] = {-INFINITY, -INFINITY}, mass[2] = {0.0f, 0.0f};
+
+    for (uint32_t tile = begin; tile < last; tile += TK) {
+        // ---- scores of the tile's 64 keys; its value rows go to LDS as they are
+#pragma unroll
+        for (int s = 0; s < T; s++) {
+            const uint32_t local = s * STEP + mine, key = tile + local;
+            *reinterpret_cast<u32x4 *>(&vt[local][dl * 8u]) = vraw[s];
+            float kf[8];
+            unpack8(kraw[s], kf);
+#pragma unroll
+            for (int g = 0; g < MAX_GROUPS; g++) {
+                if (g < (int)G) {
                     float score = 0.0f;
 #pragma unroll
                     for (int j = 0; j < 8; j++) score = fmaf(qr[g][j], kf[j], score);
                     score = key_sum<LPK>(score) * p.scale;
-                    float next = fmaxf(top[g], score);
-                    float rescale = top[g] == -INFINITY ? 0.0f : softmax_exp(top[g] - next);
-                    float weight = softmax_exp(score - next);
-                    top[g] = next;
-                    mass[g] = fmaf(mass[g], rescale, weight);
-#pragma unroll
-                    for (int j = 0; j < 8; j++) acc[g][j] = fmaf(acc[g][j], rescale, weight * vf[j]);
+                    if (dl == 0) scores[local][g] = key < last ? score : -INFINITY;
                 }
             }
         }
-    }
-    // merge the KPW key streams of a wave: lanes with the same dl
+        if (tile + TK < last) fetch_tile<T, STEP, WIDTH>(kraw, vraw, p.cache_k, p.cache_v, plane, tile + TK + mine, p.capacity, dl);  // in flight during the rest of this tile
+        __syncthreads();
+        // ---- weights: one lane per key, one wave per query head
 #pragma unroll
-    for (int g = 0; g < MAX_GROUPS; g++) {
-        if (g >= (int)G) break;
-#pragma unroll
-        for (int offset = LPK; offset < 64; offset <<= 1) {
-            float other_top = __shfl_xor(top[g], offset, 64);
-            float other_mass = __shfl_xor(mass[g], offset, 64);
-            float next = fmaxf(top[g], other_top);
-            float mine = top[g] == -INFINITY ? 0.0f : softmax_exp(top[g] - next);
-            float theirs = other_top == -INFINITY ? 0.0f : softmax_exp(other_top - next);
-            mass[g] = mass[g] * mine + other_mass * theirs;
-#pragma unroll
-            for (int j = 0; j < 8; j++) acc[g][j] = acc[g][j] * mine + __shfl_xor(acc[g][j], offset, 64) * theirs;
-            top[g] = next;
-        }
-        if (sub == 0) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) merged[wave][g][dl * 8 + j] = acc[g][j];
-            if (dl == 0) {
-                merged[wave][g][WIDTH] = top[g];
-                merged[wave][g][WIDTH + 1] = mass[g];
+        for (int gi = 0; gi < 2; gi++) {
+            const uint32_t g = wave + 4u * gi;
+            if (g < G) {
+                const float score = scores[lane][g];
+                const float next = fmaxf(top[gi], wave_max(score));
+                const float weight = score == -INFINITY ? 0.0f : softmax_exp(score - next);
+                const float rescale = top[gi] == -INFINITY ? 0.0f : softmax_exp(top[gi] - next);
+                mass[gi] = fmaf(mass[gi], rescale, wave_sum(weight));
+                top[gi] = next;
+                scores[lane][g] = weight;
+                if (lane == 0) tile_scale[g] = rescale;
             }
         }
+        __syncthreads();
+        // ---- values: acc = acc * rescale + sum over this slice's keys of weight * value
+#pragma unroll
+        for (int g = 0; g < MAX_GROUPS; g++) {
+            const float rescale = g < (int)G ? tile_scale[g] : 0.0f;
+#pragma unroll
+            for (int d = 0; d < DPT; d++) acc[g][d] *= rescale;
+        }
+#pragma unroll
+        for (int kk = 0; kk < KPS; kk++) {
+            const uint32_t local = slice * KPS + kk;
+            float v[DPT];
+            if (DPT == 1) {
+                v[0] = half_to_float(vt[local][channel]);
+            } else if (DPT == 2) {
+                const uint32_t pair = *reinterpret_cast<const uint32_t *>(&vt[local][channel]);
+                v[0] = half_to_float((uint16_t)(pair & 0xffffu)), v[1 % DPT] = half_to_float((uint16_t)(pair >> 16));
+            } else {
+                const uint2 quad = *reinterpret_cast<const uint2 *>(&vt[local][channel]);
+                v[0] = half_to_float((uint16_t)(quad.x & 0xffffu)), v[1 % DPT] = half_to_float((uint16_t)(quad.x >> 16));
+                v[2 % DPT] = half_to_float((uint16_t)(quad.y & 0xffffu)), v[3 % DPT] = half_to_float((uint16_t)(quad.y >> 16));
+            }
+            const float4 w0 = *reinterpret_cast<const float4 *>(&scores[local][0]), w1 = *reinterpret_cast<const float4 *>(&scores[local][4]);
+            // heads past G hold stale weights: their sums are never read
+#pragma unroll
+            for (int d = 0; d < DPT; d++) {
+                acc[0][d] = fmaf(w0.x, v[d], acc[0][d]), acc[1][d] = fmaf(w0.y, v[d], acc[1][d]);
+                acc[2][d] = fmaf(w0.z, v[d], acc[2][d]), acc[3][d] = fmaf(w0.w, v[d], acc[3][d]);
+                acc[4][d] = fmaf(w1.x, v[d], acc[4][d]), acc[5][d] = fmaf(w1.y, v[d], acc[5][d]);
+                acc[6][d] = fmaf(w1.z, v[d], acc[6][d]), acc[7][d] = fmaf(w1.w, v[d], acc[7][d]);
+            }
+        }
+        __syncthreads();  // the next tile overwrites vt and scores
+    }
+    // ---- the slices meet in LDS
+#pragma unroll
+    for (int g = 0; g < MAX_GROUPS; g++) {
+        if (g < (int)G) {
+#pragma unroll
+            for (int d = 0; d < DPT; d++) merged[slice][g][channel + d] = acc[g][d];
+        }
+    }
+#pragma unroll
+    for (int gi = 0; gi < 2; gi++) {
+        const uint32_t g = wave + 4u * gi;
+        if (g < G && lane == 0) stat_top[g] = top[gi], stat_mass[g] = mass[gi];
     }
     __syncthreads();
-    // merge the four waves; thread -> (group, channel)
     for (uint32_t index = tid; index < G * WIDTH; index += 256) {
-        uint32_t g = index / WIDTH, c = index % WIDTH;
-        float largest = -INFINITY;
+        const uint32_t g = index / WIDTH, c = index % WIDTH;
+        float value = 0.0f;
 #pragma unroll
-        for (int w = 0; w < 4; w++) largest = fmaxf(largest, merged[w][g][WIDTH]);
-        float total = 0.0f, value = 0.0f;
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            float held = merged[w][g][WIDTH];
-            float weight = held == -INFINITY ? 0.0f : softmax_exp(held - largest);
-            total += merged[w][g][WIDTH + 1] * weight;
-            value += merged[w][g][c] * weight;
-        }
+        for (int s = 0; s < SLICES; s++) value += merged[s][g][c];
+        const float largest = stat_top[g], total = stat_mass[g];
         const uint32_t head = kvh * G + g;
         if (p.sections > 1) {
             float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (WIDTH + 2);
