@@ -66,6 +66,50 @@ __device__ float rms_scale(const float *__restrict__ x, uint32_t K, float eps, f
     return rms_scale_of(total, K, eps);
 }
 
+// Stages x[k0 .. k0 + kn) of one activation row into LDS at dst[skew(i)], RMS-normalised over the whole row and
+// weighed when norm_w is given.  With 256 threads and at most 16 values per thread every load goes out before the
+// first value is used and the row is read once: a loop that handles each value as it arrives spends one memory
+// round trip per value (6 us on a 3584-wide row).  Deeper slices take the looped form.
+template <typename Skew>
+__device__ __forceinline__ void stage_row(const float *__restrict__ x, uint32_t K, uint32_t k0, uint32_t kn, const float *__restrict__ norm_w,
+                                          float eps, float *dst, float *red, Skew skew) {
+    const uint32_t tid = threadIdx.x;
+    if (blockDim.x == 256 && kn <= 4096u && (!norm_w || (k0 == 0 && kn == K))) {
+        float held[16], weight[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t c = tid + 256u * j;
+            held[j] = c < kn ? x[k0 + c] : 0.0f;
+            weight[j] = (norm_w && c < kn) ? norm_w[k0 + c] : 0.0f;
+        }
+        if (norm_w) {
+            float square = 0.0f;  // thread t adds columns t, t + 256, ... in order (crates/neura-kernel/src/task/norm.rs:69-83)
+#pragma unroll
+            for (int j = 0; j < 16; j++) square = __fadd_rn(square, __fmul_rn(held[j], held[j]));
+            square = wave_sum(square);
+            if ((tid & 63u) == 0) red[tid >> 6] = square;
+            __syncthreads();
+            const float scale = rms_scale_of((red[0] + red[1]) + (red[2] + red[3]), K, eps);
+            __syncthreads();  // red is reused by the next row
+#pragma unroll
+            for (int j = 0; j < 16; j++) held[j] = __fmul_rn(__fmul_rn(held[j], scale), weight[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t c = tid + 256u * j;
+            if (c < kn) dst[skew(c)] = held[j];
+        }
+    } else {
+        float scale = 1.0f;
+        if (norm_w) scale = rms_scale(x, K, eps, red);
+        for (uint32_t i = tid; i < kn; i += blockDim.x) {
+            float value = x[k0 + i];
+            if (norm_w) value = __fmul_rn(__fmul_rn(value, scale), norm_w[k0 + i]);
+            dst[skew(i)] = value;
+        }
+    }
+}
+
 __device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
 
 // logical row i of a pass -> output row.  With swiglu, even i walk the gate rows and odd i the
@@ -320,41 +364,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
     DecodeTile<R> ta, tb;
     if (rg < p.row_groups) load(ta, rg);  // in flight while the activations are staged
 
-    if (NW == 4 && p.splits == 1 && p.K <= 4096u) {
-        // a whole row is at most 16 values per thread: every load goes out before the first is used (a loop
-        // that adds each value as it arrives spends a memory round trip per value), and the row is read once
-        float held[16], weight[16];
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t c = tid + 256u * j;
-            held[j] = c < p.K ? p.x[c] : 0.0f;
-            weight[j] = (p.norm_w && c < p.K) ? p.norm_w[c] : 0.0f;
-        }
-        if (p.norm_w) {
-            float square = 0.0f;  // thread t adds columns t, t + 256, ... in order (crates/neura-kernel/src/task/norm.rs:69-83)
-#pragma unroll
-            for (int j = 0; j < 16; j++) square = __fadd_rn(square, __fmul_rn(held[j], held[j]));
-            square = wave_sum(square);
-            if (lane == 0) red[wave] = square;
-            __syncthreads();
-            const float scale = rms_scale_of((red[0] + red[1]) + (red[2] + red[3]), p.K, p.eps);
-#pragma unroll
-            for (int j = 0; j < 16; j++) held[j] = __fmul_rn(__fmul_rn(held[j], scale), weight[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t c = tid + 256u * j;
-            if (c < kn) xs[skew64(c)] = held[j];
-        }
-    } else {
-        float scale = 1.0f;
-        if (p.norm_w) scale = rms_scale(p.x, p.K, p.eps, red);
-        for (uint32_t i = tid; i < kn; i += NW * 64) {
-            float value = p.x[k0 + i];
-            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, scale), p.norm_w[k0 + i]);
-            xs[skew64(i)] = value;
-        }
-    }
+    stage_row(p.x, p.K, k0, kn, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew64(i); });
     __syncthreads();
 
     float xl[32], xh[32];
@@ -462,16 +472,8 @@ __global__ __launch_bounds__(256) void gemv_q4k_kernel(GemvParams p) {
     const uint32_t xstride = skew64(p.blocks_per_split * 256u);
 
 #pragma unroll
-    for (int b = 0; b < RB; b++) {
-        const float *xb = p.x + (size_t)b * p.K;
-        float scale = 1.0f;
-        if (p.norm_w) scale = rms_scale(xb, p.K, p.eps, red);
-        for (uint32_t i = tid; i < kn; i += 256) {
-            float value = xb[k0 + i];
-            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, scale), p.norm_w[k0 + i]);
-            xs[b * xstride + skew64(i)] = value;
-        }
-    }
+    for (int b = 0; b < RB; b++)
+        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew64(i); });
     __syncthreads();
 
     const uint32_t G = p.group;  // lanes per output row
@@ -546,16 +548,8 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     const uint32_t lrow = p.chunks_per_row * 16u;
 
 #pragma unroll
-    for (int b = 0; b < RB; b++) {
-        const float *xb = p.x + (size_t)b * p.K;
-        float scale = 1.0f;
-        if (p.norm_w) scale = rms_scale(xb, p.K, p.eps, red);
-        for (uint32_t i = tid; i < kn; i += 256) {
-            float value = xb[k0 + i];
-            if (p.norm_w) value = __fmul_rn(__fmul_rn(value, scale), p.norm_w[k0 + i]);
-            xs[b * xstride + skew32(i)] = value;
-        }
-    }
+    for (int b = 0; b < RB; b++)
+        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew32(i); });
     __syncthreads();
 
     const uint32_t G = p.group;
