@@ -139,6 +139,43 @@ def test_gemv_epilogues(device, element, N, K):
         close(device.gemv(element, raw, N, K, x, swiglu=True), want, rel=1e-4, abs_=1e-4 * np.abs(want).max())
 
 
+@pytest.mark.parametrize("mode", ["0", "2"])
+@pytest.mark.parametrize("N,K,rows", [(16, 256, 1), (48, 512, 3), (272, 3584, 1), (64, 1536, 8), (32, 18944, 1), (32, 18944, 5), (1040, 768, 2)])
+def test_q4_k_products_agree_in_every_form(device, monkeypatch, mode, N, K, rows):
+    """NEURA_HIP_MFMA=0 forces the vector kernels, =2 the matrix-core kernel (integer MFMA over four-digit activations);
+    both sit within fp32 reordering of the order-faithful oracle, plain, with a residual and with SwiGLU, for 1..8
+    activation rows, rows deeper than one LDS stage, and activations that span many orders of magnitude."""
+    monkeypatch.setenv("NEURA_HIP_MFMA", mode)
+    rng = np.random.default_rng(N + K + rows)
+    raw = synth.q4_k_random(rng, N * K)
+    x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-6, 6, (rows, K)))).astype(np.float32)  # wide dynamic range
+    r = rng.standard_normal((rows, N)).astype(np.float32)
+    plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+    exact = oracle.unpack(NH_Q4_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+    scale = max(1.0, np.abs(exact).max())
+    got = device.gemv(NH_Q4_K, raw, N, K, x)
+    close(got, plain)
+    # as close to the exact product as the oracle's own fp32 sums are, up to a small factor
+    assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * scale)
+    tight(device.gemv(NH_Q4_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2:].astype(np.float64)
+    want = gate / (1.0 + np.exp(-gate)) * up
+    close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+
+
+def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device, monkeypatch):
+    monkeypatch.setenv("NEURA_HIP_MFMA", "2")
+    rng = np.random.default_rng(2)
+    N, K = 32, 512
+    raw = synth.q4_k_random(rng, N * K)
+    x = rng.standard_normal((2, K)).astype(np.float32)
+    x[1, 77] = np.inf
+    got = device.gemv(NH_Q4_K, raw, N, K, x)
+    assert np.isfinite(got[0]).all() and not np.isfinite(got[1]).any()
+    assert not np.isfinite(device.gemv(NH_Q4_K, raw, N, K, np.full((1, K), np.nan, np.float32))).any()
+    assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
+
+
 def test_gemv_is_linear_and_matches_at_full_size(device):
     # size-independent properties at the 7B FFN shape: W(a x + b z) = a W x + b W z
     rng = np.random.default_rng(6)
