@@ -134,6 +134,8 @@ struct GemmArgs {
     uint32_t ldy;
 };
 int32_t launch_gemm(nh_device *d, const GemmArgs &args);
+// device scratch a Q4_K wide product over M rows of K activations packs them into
+size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows);
 
 int32_t launch_rmsnorm(nh_device *d, const float *x, const float *residual, const float *w, float eps, uint32_t rows, uint32_t C,
                        float *out, float *sum_out);

@@ -106,8 +106,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint8_t *__restrict__ W
 //
 // A nibble masked in place in a 16-bit lane is the half subnormal code * 2^-24 (or 2^-20);
 // one packed half multiply by sc * 2^10 (or 2^6) turns it into the normal half code*sc*2^-14.
+//
+// Everything that does not depend on the weights is done once per activation row by a kernel
+// of its own (gemm_pack_rows_kernel): the halves in the element order the unpacked nibbles come
+// out in, and the sub-block sums the minimums are weighed by, already cut into the operand of
+// their MFMA.  The tile loop is left with copies for the activations and four instructions
+// per eight weights, and stages step s + 1 into the other half of LDS while the matrix cores
+// walk step s: one barrier per step.
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -119,7 +127,9 @@ constexpr int GS = GK + 8;        // LDS row stride in halves: 144 B keeps 128-b
 struct GemmQ4Params {
     const uint8_t *W;
     uint32_t N, K, row_bytes;
-    const _Float16 *A;   // [rows][K] halves; with `split`, row 2m is the rounded value of activation row m and row 2m+1 its residue * 2^11
+    const _Float16 *A;   // [rows][K] halves, every four k in the order 0, 2, 1, 3; with `split`, row 2m is the rounded value of
+                         // activation row m and row 2m+1 its residue * 2^11
+    const _Float16 *S;   // [rows][K / 256][16]: the eight sub-block sums / 64 of a super-block as halves, then their residues * 2^11
     uint32_t rows;       // rows of A
     float *Y;
     const float *residual;
@@ -128,37 +138,88 @@ struct GemmQ4Params {
     const float *unscale;  // [M] with split: undoes the row scale
 };
 
-// fp32 activations -> scaled (value, residue) half rows
-__global__ __launch_bounds__(256) void gemm_split_rows_kernel(const float *__restrict__ X, uint32_t K, _Float16 *__restrict__ A, float *__restrict__ unscale) {
+// One workgroup per activation row: the row as MFMA-ready halves (and, for fp32 rows, its residue row and scale).
+template <bool HALF_IN>
+__global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restrict__ X, uint32_t K, _Float16 *__restrict__ A,
+                                                             _Float16 *__restrict__ S, float *__restrict__ unscale) {
     __shared__ uint32_t wave_top[4];
     const uint32_t m = blockIdx.x, tid = threadIdx.x;
-    const float *x = X + (size_t)m * K;
-    uint32_t top = 0;
-    for (uint32_t k = tid; k < K; k += 256) top = max(top, __builtin_bit_cast(uint32_t, x[k]) & 0x7fffffffu);
+    const uint32_t nsb = K / 256u;
+    float scale = 1.0f;
+    if (!HALF_IN) {
+        const float *x = static_cast<const float *>(X) + (size_t)m * K;
+        uint32_t top = 0;
+        for (uint32_t k = tid * 4u; k < K; k += 1024u) {
+            const float4 v = *reinterpret_cast<const float4 *>(x + k);
+            top = max(max(top, __builtin_bit_cast(uint32_t, v.x) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.y) & 0x7fffffffu);
+            top = max(max(top, __builtin_bit_cast(uint32_t, v.z) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.w) & 0x7fffffffu);
+        }
 #pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
-    if ((tid & 63u) == 0) wave_top[tid >> 6] = top;
-    __syncthreads();
-    top = max(max(wave_top[0], wave_top[1]), max(wave_top[2], wave_top[3]));
-    // a power of two that puts the largest magnitude in [2^13, 2^14)
-    const uint32_t raw = top >> 23, exponent = min(max(raw, 27u), 254u);
-    const float scale = __builtin_bit_cast(float, (267u - exponent) << 23);
-    if (tid == 0) unscale[m] = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 13u) << 23);
-    _Float16 *hi = A + (size_t)(2 * m) * K, *lo = hi + K;
-    for (uint32_t k = tid; k < K; k += 256) {
-        const float t = x[k] * scale;
-        const _Float16 h = (_Float16)t;
-        hi[k] = h;
-        lo[k] = (_Float16)((t - (float)h) * 2048.0f);
+        for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
+        if ((tid & 63u) == 0) wave_top[tid >> 6] = top;
+        __syncthreads();
+        top = max(max(wave_top[0], wave_top[1]), max(wave_top[2], wave_top[3]));
+        // a power of two that puts the largest magnitude in [2^13, 2^14)
+        const uint32_t raw = top >> 23, exponent = min(max(raw, 27u), 254u);
+        scale = __builtin_bit_cast(float, (267u - exponent) << 23);
+        if (tid == 0) unscale[m] = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 13u) << 23);
+    }
+    const uint32_t row = HALF_IN ? m : 2u * m;
+    for (uint32_t k = tid * 4u; k < K; k += 1024u) {
+        _Float16 hi[4], lo[4];
+        if (HALF_IN) {
+            const half4_t v = *reinterpret_cast<const half4_t *>(static_cast<const _Float16 *>(X) + (size_t)m * K + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) hi[e] = v[e], lo[e] = (_Float16)0.0f;
+        } else {
+            const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(X) + (size_t)m * K + k);
+            const float t[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                hi[e] = (_Float16)t[e];
+                lo[e] = (_Float16)((t[e] - (float)hi[e]) * 2048.0f);
+            }
+        }
+        // the nibbles of four weight bytes unpack as bytes 0, 2, 1, 3
+        const half4_t out_hi = {hi[0], hi[2], hi[1], hi[3]}, out_lo = {lo[0], lo[2], lo[1], lo[3]};
+        *reinterpret_cast<half4_t *>(A + (size_t)row * K + k) = out_hi;
+        if (!HALF_IN) *reinterpret_cast<half4_t *>(A + (size_t)(row + 1u) * K + k) = out_lo;
+        // sums of the 32 halves of a sub-block: eight neighbouring lanes
+        float sum_hi = ((float)hi[0] + (float)hi[1]) + ((float)hi[2] + (float)hi[3]);
+        float sum_lo = ((float)lo[0] + (float)lo[1]) + ((float)lo[2] + (float)lo[3]);
+#pragma unroll
+        for (int offset = 1; offset < 8; offset <<= 1) {
+            sum_hi += __shfl_xor(sum_hi, offset, 64);
+            sum_lo += __shfl_xor(sum_lo, offset, 64);
+        }
+        if ((tid & 7u) == 0) {
+            const uint32_t sb = k >> 8, slot = (k >> 5) & 7u;
+            {
+                const float v = sum_hi * 0.015625f;
+                const _Float16 h = (_Float16)v;
+                _Float16 *dst = S + ((size_t)row * nsb + sb) * 16u;
+                dst[slot] = h;
+                dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
+            }
+            if (!HALF_IN) {
+                const float v = sum_lo * 0.015625f;
+                const _Float16 h = (_Float16)v;
+                _Float16 *dst = S + ((size_t)(row + 1u) * nsb + sb) * 16u;
+                dst[slot] = h;
+                dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
+            }
+        }
     }
 }
 
+constexpr size_t GEMM_Q4K_LDS = sizeof(_Float16) * (2 * GT * GS + 2 * GT * GS + 2 * GT * 8) + sizeof(uint32_t) * 2 * GT;
+
 __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
-    __shared__ __attribute__((aligned(16))) _Float16 As[GT][GS];
-    __shared__ __attribute__((aligned(16))) _Float16 Bs[GT][GS];
-    __shared__ __attribute__((aligned(16))) float xs[GT][8];        // sub-block sums of the activation rows of this super-block, / 64
-    __shared__ __attribute__((aligned(16))) _Float16 mns[GT][8];    // the eight minimums of every weight row
-    __shared__ uint32_t dds[GT];                                    // (d, dmin) of every weight row
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);                                           // [2]
+    _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);          // [2]
+    _Float16(*mns)[GT][8] = reinterpret_cast<_Float16(*)[GT][8]>(gemm_lds + sizeof(_Float16) * 4 * GT * GS);           // [2] by super-block parity: the eight minimums of every weight row
+    uint32_t(*dds)[GT] = reinterpret_cast<uint32_t(*)[GT]>(gemm_lds + sizeof(_Float16) * (4 * GT * GS + 2 * GT * 8));  // [2]: (d, dmin) of every weight row
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
     // staging role: one row of each tile, one half (32 k) of the step
@@ -167,6 +228,10 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
     const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
     // compute role: wave (wm, wn) owns rows 64 wm.. of A' and weight rows 64 wn..
     const uint32_t wm = wave >> 1, wn = wave & 1u, l32 = lane & 31u, part = lane >> 5;
+    const uint32_t nsb = p.K / 256u;
+    const _Float16 *sums[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) sums[i] = p.S + (size_t)min(m0 + 64u * wm + 32u * i + l32, p.rows - 1u) * nsb * 16u + 8u * part;
 
     f32x16 acc[2][2], tmp[2][2];
 #pragma unroll
@@ -187,71 +252,74 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
 #pragma unroll
         for (int i = 0; i < 4; i++) av[i] = *(global_uint4)(uintptr_t)(at + 8 * i);
     };
+    // the fetched step into half `buf` of LDS
+    auto stage = [&](uint32_t step) {
+        const uint32_t g = step & 3u, buf = step & 1u, sbuf = (step >> 2) & 1u;
+        // 6-bit fields of sub-blocks 2g, 2g+1 (crates/neura-precision/src/ggml.rs:127-136); 0x6400 | v is the half 1024 + v
+        const uint32_t shift = 16u * (g & 1u);
+        const uint32_t ya = (hdr.y >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
+        const uint32_t sc = g < 2 ? (ya & 0x3f3fu) : ((wa & 0x0f0fu) | ((ya >> 2) & 0x3030u));
+        const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;  // (1024 + sc0, 1024 + sc1)
+        const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
+        const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;     // (sc0 * 2^10, sc1 * 2^6)
+        const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
+        const uint32_t words[4] = {qs.x, qs.y, qs.z, qs.w};
+        uint32_t low[8], high[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t even = words[w], odd = words[w] >> 8;
+            // element order inside a word: 0, 2 then 1, 3 (the byte lanes); the activations were packed in the same order
+            low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
+            low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
+            high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
+            high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+        }
+        u32x4 *blow = reinterpret_cast<u32x4 *>(&Bs[buf][srow][16u * sh]), *bhigh = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u + 16u * sh]);
+        blow[0] = u32x4{low[0], low[1], low[2], low[3]};
+        blow[1] = u32x4{low[4], low[5], low[6], low[7]};
+        bhigh[0] = u32x4{high[0], high[1], high[2], high[3]};
+        bhigh[1] = u32x4{high[4], high[5], high[6], high[7]};
+        if (g == 0 && sh == 0) {
+            // the eight minimums of the super-block, as halves
+            const uint32_t lo4 = hdr.z & 0x3f3f3f3fu;                                         // m0..m3
+            const uint32_t hi4 = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);  // m4..m7
+            const half2_t m01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c010c00u) | 0x64006400u) - offset;
+            const half2_t m23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c030c02u) | 0x64006400u) - offset;
+            const half2_t m45 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c010c00u) | 0x64006400u) - offset;
+            const half2_t m67 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c030c02u) | 0x64006400u) - offset;
+            *reinterpret_cast<u32x4 *>(mns[sbuf][srow]) = u32x4{__builtin_bit_cast(uint32_t, m01), __builtin_bit_cast(uint32_t, m23),
+                                                                __builtin_bit_cast(uint32_t, m45), __builtin_bit_cast(uint32_t, m67)};
+            dds[sbuf][srow] = hdr.x;
+        }
+        u32x4 *adst = reinterpret_cast<u32x4 *>(&As[buf][srow][32u * sh]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) adst[i] = av[i];
+    };
+
     const uint32_t steps = p.K / 64u;
     fetch(0);
+    stage(0);
+    if (steps > 1) fetch(1);
+    __syncthreads();
+    u32x4 sraw[2];
     for (uint32_t step = 0; step < steps; step++) {
-        const uint32_t g = step & 3u;
-        __syncthreads();  // the previous step's operands have been read
-        {
-            // ---- weights: 16 bytes = 16 low nibbles (sub-block 2g) and 16 high nibbles (sub-block 2g+1)
-            const uint32_t shift = 16u * (g & 1u);
-            const uint32_t ya = (hdr.y >> shift) & 0xffffu, za = (hdr.z >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
-            uint32_t sc0, sc1, mn0, mn1;  // crates/neura-precision/src/ggml.rs:127-136
-            if (g < 2) {
-                sc0 = ya & 63u, sc1 = (ya >> 8) & 63u, mn0 = za & 63u, mn1 = (za >> 8) & 63u;
-            } else {
-                sc0 = (wa & 0x0fu) | (((ya >> 6) & 3u) << 4);
-                sc1 = ((wa >> 8) & 0x0fu) | (((ya >> 14) & 3u) << 4);
-                mn0 = ((wa >> 4) & 0x0fu) | (((za >> 6) & 3u) << 4);
-                mn1 = ((wa >> 12) & 0x0fu) | (((za >> 14) & 3u) << 4);
-            }
-            const _Float16 s_low = (_Float16)(float)(sc0 << 10), s_high = (_Float16)(float)(sc1 << 6);
-            const half2_t low_scale = {s_low, s_low}, high_scale = {s_high, s_high};
-            const uint32_t words[4] = {qs.x, qs.y, qs.z, qs.w};
-            uint32_t low[8], high[8];
+        const uint32_t g = step & 3u, buf = step & 1u, sbuf = (step >> 2) & 1u;
+        if (g == 0) {
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const uint32_t even = words[w], odd = words[w] >> 8;
-                // element order inside a word: 0, 2 then 1, 3 (the byte lanes); the activations are staged in the same order
-                low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
-                low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
-                high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
-                high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
-            }
-            uint4 *blow = reinterpret_cast<uint4 *>(&Bs[srow][16u * sh]), *bhigh = reinterpret_cast<uint4 *>(&Bs[srow][32u + 16u * sh]);
-            blow[0] = make_uint4(low[0], low[1], low[2], low[3]);
-            blow[1] = make_uint4(low[4], low[5], low[6], low[7]);
-            bhigh[0] = make_uint4(high[0], high[1], high[2], high[3]);
-            bhigh[1] = make_uint4(high[4], high[5], high[6], high[7]);
-            if (sh == 0) {
-                mns[srow][2 * g] = (_Float16)(float)mn0;
-                mns[srow][2 * g + 1] = (_Float16)(float)mn1;
-                if (g == 0) dds[srow] = hdr.x;
-            }
-            // ---- activations: 32 halves of sub-block 2g + sh, reordered like the weights; their sum for the minimums
-            float total = 0.0f;
-            const half2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
-            uint4 *adst = reinterpret_cast<uint4 *>(&As[srow][32u * sh]);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t d[4] = {av[i].x, av[i].y, av[i].z, av[i].w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) total = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, d[e]), ones, total, false);
-                adst[i] = make_uint4(__builtin_amdgcn_perm(d[1], d[0], 0x05040100u), __builtin_amdgcn_perm(d[1], d[0], 0x07060302u),
-                                     __builtin_amdgcn_perm(d[3], d[2], 0x05040100u), __builtin_amdgcn_perm(d[3], d[2], 0x07060302u));
-            }
-            xs[srow][2 * g + sh] = total * 0.015625f;
+            for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(step >> 2) * 16u);  // wanted three steps from here
         }
-        __syncthreads();
-        if (step + 1 < steps) fetch(step + 1);
+        if (step + 1 < steps) {
+            stage(step + 1);
+            if (step + 2 < steps) fetch(step + 2);
+        }
         // ---- 64 x 64 x 64 per wave
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             half8_t a[2], b[2];
 #pragma unroll
-            for (int i = 0; i < 2; i++) a[i] = *reinterpret_cast<const half8_t *>(&As[64u * wm + 32u * i + l32][16u * kk + 8u * part]);
+            for (int i = 0; i < 2; i++) a[i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
 #pragma unroll
-            for (int j = 0; j < 2; j++) b[j] = *reinterpret_cast<const half8_t *>(&Bs[64u * wn + 32u * j + l32][16u * kk + 8u * part]);
+            for (int j = 0; j < 2; j++) b[j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -260,31 +328,18 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
         if (g == 3) {
             // ---- the super-block is complete: weigh by d, then take the minimums off
             float dscale[2], mscale[2];
+            half8_t b2[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const half2_t dd = __builtin_bit_cast(half2_t, dds[64u * wn + 32u * j + l32]);
+                const half2_t dd = __builtin_bit_cast(half2_t, dds[sbuf][64u * wn + 32u * j + l32]);
                 dscale[j] = (float)dd.x * 16384.0f;  // the weights were staged * 2^-14
-                mscale[j] = (float)dd.y * -64.0f;    // the sums were staged / 64
+                mscale[j] = (float)dd.y * -64.0f;    // the sums were packed / 64
+                b2[j] = *reinterpret_cast<const half8_t *>(mns[sbuf][64u * wn + 32u * j + l32]);
+                if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11 against the residues * 2^11
             }
-            half8_t a2[2], b2[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                const float4 *sums = reinterpret_cast<const float4 *>(xs[64u * wm + 32u * i + l32]);
-                const float4 s0 = sums[0], s1 = sums[1];
-                const float v[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const _Float16 h = (_Float16)v[e];
-                    a2[i][e] = part ? (_Float16)((v[e] - (float)h) * 2048.0f) : h;  // k 0..7: the sums; k 8..15: their residues * 2^11
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                b2[j] = *reinterpret_cast<const half8_t *>(mns[64u * wn + 32u * j + l32]);
-                if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11
-            }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
+                const half8_t a2 = __builtin_bit_cast(half8_t, sraw[i]);  // k 0..7: the sums; k 8..15: their residues
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
 #pragma unroll
@@ -292,11 +347,13 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
                     f32x16 zero;
 #pragma unroll
                     for (int e = 0; e < 16; e++) zero[e] = 0.0f;
-                    const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2[i], b2[j], zero, 0, 0, 0);
+                    const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[j], zero, 0, 0, 0);
 #pragma unroll
                     for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(mscale[j], mins[e], acc[i][j][e]), tmp[i][j][e] = 0.0f;
                 }
+            }
         }
+        __syncthreads();  // step + 1 is staged; every wave is done with this step's half of LDS
     }
     // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
 #pragma unroll
@@ -330,6 +387,12 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
         }
 }
 
+// bytes of device scratch a Q4_K wide product over M activation rows of K numbers packs into
+size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows) {
+    const size_t rows = half_rows ? M : (size_t)2 * M;
+    return rows * K * sizeof(_Float16) + rows * (K / 256u) * 16u * sizeof(_Float16) + (size_t)M * sizeof(float);
+}
+
 static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     GemmQ4Params p{};
     p.W = static_cast<const uint8_t *>(a.W);
@@ -340,26 +403,28 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     p.residual = a.residual;
     p.ldy = a.ldy;
     p.M = a.M;
-    if (a.x_element == NH_F16) {
-        p.A = static_cast<const _Float16 *>(a.X);
-        p.rows = a.M;
-        p.split = 0;
-    } else {
-        // scratch: [2M][K] halves, then M row scales
-        const size_t halves = (size_t)2 * a.M * a.K * sizeof(_Float16);
-        uint8_t *room = static_cast<uint8_t *>(scratch(d, halves + (size_t)a.M * sizeof(float)));
-        if (!room) return NH_E_MEMORY;
-        _Float16 *A = reinterpret_cast<_Float16 *>(room);
-        float *unscale = reinterpret_cast<float *>(room + halves);
-        hipLaunchKernelGGL(gemm_split_rows_kernel, dim3(a.M), dim3(256), 0, d->stream, static_cast<const float *>(a.X), a.K, A, unscale);
-        NH_HIP(hipGetLastError());
-        p.A = A;
-        p.rows = 2 * a.M;
-        p.split = 1;
-        p.unscale = unscale;
+    const bool half_rows = a.x_element == NH_F16;
+    p.rows = half_rows ? a.M : 2 * a.M;
+    p.split = half_rows ? 0 : 1;
+    // scratch: [rows][K] halves, [rows][K / 256][16] sums, M row scales
+    const size_t halves = (size_t)p.rows * a.K * sizeof(_Float16), sums = (size_t)p.rows * (a.K / 256u) * 16u * sizeof(_Float16);
+    uint8_t *room = static_cast<uint8_t *>(scratch(d, gemm_q4k_scratch_bytes(a.M, a.K, half_rows)));
+    if (!room) return NH_E_MEMORY;
+    _Float16 *A = reinterpret_cast<_Float16 *>(room), *S = reinterpret_cast<_Float16 *>(room + halves);
+    float *unscale = reinterpret_cast<float *>(room + halves + sums);
+    if (half_rows)
+        hipLaunchKernelGGL(gemm_pack_rows_kernel<true>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
+    else
+        hipLaunchKernelGGL(gemm_pack_rows_kernel<false>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
+    NH_HIP(hipGetLastError());
+    p.A = A, p.S = S, p.unscale = unscale;
+    static bool sized = false;
+    if (!sized) {
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
+        sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
-    hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(256), 0, d->stream, p);
+    hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(256), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }

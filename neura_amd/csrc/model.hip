@@ -284,10 +284,10 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         size_t products = 8 * 4 * widest * sizeof(float);
         size_t sections = (size_t)256 * c.heads * T * (c.head_dim + 2) * sizeof(float);
         size_t choice = (size_t)c.batch * 1024 * 8;
-        // the wide product keeps its fp32 activations as two half rows each, plus a scale per row
+        // the wide product packs its fp32 activations as two half rows each, with their sub-block sums and a scale per row
         size_t deepest = (size_t)(F > QW ? F : QW);
         if (H > deepest) deepest = H;
-        size_t split_rows = T > 8 ? (size_t)2 * T * deepest * 2 + T * sizeof(float) : 0;
+        size_t split_rows = T > 8 ? gemm_q4k_scratch_bytes(T, (uint32_t)deepest, false) : 0;
         size_t wanted = products > sections ? products : sections;
         if (choice > wanted) wanted = choice;
         if (split_rows > wanted) wanted = split_rows;
