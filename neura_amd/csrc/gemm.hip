@@ -214,146 +214,169 @@ __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restr
 
 constexpr size_t GEMM_Q4K_LDS = sizeof(_Float16) * (2 * GT * GS + 2 * GT * GS + 2 * GT * 8) + sizeof(uint32_t) * 2 * GT;
 
-__global__ __launch_bounds__(256, 2) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
+// The eight waves of a workgroup split the work by kind.  Waves 4..7 (the stagers) fetch raw blocks and packed
+// activations four steps ahead into registers, unpack step s + 1 into LDS; waves 0..3 (the multipliers) do nothing
+// but read operands and drive the matrix cores over step s.  One stager and one multiplier share each SIMD, so
+// unpacking and memory latency hide behind the MFMAs instead of taking turns with them.
+__global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);                                           // [2]
     _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);          // [2]
     _Float16(*mns)[GT][8] = reinterpret_cast<_Float16(*)[GT][8]>(gemm_lds + sizeof(_Float16) * 4 * GT * GS);           // [2] by super-block parity: the eight minimums of every weight row
     uint32_t(*dds)[GT] = reinterpret_cast<uint32_t(*)[GT]>(gemm_lds + sizeof(_Float16) * (4 * GT * GS + 2 * GT * 8));  // [2]: (d, dmin) of every weight row
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
-    // staging role: one row of each tile, one half (32 k) of the step
-    const uint32_t srow = tid >> 1, sh = tid & 1u;
-    const uint8_t *wrow = p.W + (size_t)min(n0 + srow, p.N - 1u) * p.row_bytes;
-    const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
-    // compute role: wave (wm, wn) owns rows 64 wm.. of A' and weight rows 64 wn..
+    const uint32_t steps = p.K / 64u;  // a multiple of 4: K is whole super-blocks
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------ stagers
+        // one row of each tile, one half (32 k) of the step
+        const uint32_t tid = threadIdx.x - 256u;
+        const uint32_t srow = tid >> 1, sh = tid & 1u;
+        const uint8_t *wrow = p.W + (size_t)min(n0 + srow, p.N - 1u) * p.row_bytes;
+        const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
+        u32x4 ahead, qs[4], av[4][4];  // the next super-block's header; groups and activations by slot = step % 4
+        const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
+        ahead = *(global_uint4)(uintptr_t)wrow;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {  // steps 0..3 = super-block 0
+            qs[g] = *(global_uint4)(uintptr_t)(wrow + 16u + 32u * g + 16u * sh);
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[g][i] = *(global_uint4)(uintptr_t)(arow + (size_t)g * 64u + 8 * i);
+            __builtin_amdgcn_sched_barrier(0);  // slot 0 goes out first: the loop waits for the oldest slot only
+        }
+        for (uint32_t first = 0; first < steps; first += 4) {
+            const u32x4 hdr = ahead;
+            const uint32_t next = min((first >> 2) + 1u, (steps >> 2) - 1u);
+            ahead = *(global_uint4)(uintptr_t)(wrow + (size_t)next * 144u);
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint32_t buf = g & 1u, sbuf = (first >> 2) & 1u;
+                // 6-bit fields of sub-blocks 2g, 2g+1 (crates/neura-precision/src/ggml.rs:127-136); 0x6400 | v is the half 1024 + v
+                const uint32_t shift = 16u * (g & 1u);
+                const uint32_t ya = (hdr.y >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
+                const uint32_t sc = g < 2 ? (ya & 0x3f3fu) : ((wa & 0x0f0fu) | ((ya >> 2) & 0x3030u));
+                const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;  // (1024 + sc0, 1024 + sc1)
+                const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;     // (sc0 * 2^10, sc1 * 2^6)
+                const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
+                const uint32_t words[4] = {qs[g].x, qs[g].y, qs[g].z, qs[g].w};
+                uint32_t low[8], high[8];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t even = words[w], odd = words[w] >> 8;
+                    // element order inside a word: 0, 2 then 1, 3 (the byte lanes); the activations were packed in the same order
+                    low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
+                    low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
+                    high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
+                    high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+                }
+                u32x4 *blow = reinterpret_cast<u32x4 *>(&Bs[buf][srow][16u * sh]), *bhigh = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u + 16u * sh]);
+                blow[0] = u32x4{low[0], low[1], low[2], low[3]};
+                blow[1] = u32x4{low[4], low[5], low[6], low[7]};
+                bhigh[0] = u32x4{high[0], high[1], high[2], high[3]};
+                bhigh[1] = u32x4{high[4], high[5], high[6], high[7]};
+                if (g == 0 && sh == 0) {
+                    // the eight minimums of the super-block, as halves
+                    const uint32_t lo4 = hdr.z & 0x3f3f3f3fu;                                         // m0..m3
+                    const uint32_t hi4 = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);  // m4..m7
+                    const half2_t m01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c010c00u) | 0x64006400u) - offset;
+                    const half2_t m23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c030c02u) | 0x64006400u) - offset;
+                    const half2_t m45 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c010c00u) | 0x64006400u) - offset;
+                    const half2_t m67 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c030c02u) | 0x64006400u) - offset;
+                    *reinterpret_cast<u32x4 *>(mns[sbuf][srow]) = u32x4{__builtin_bit_cast(uint32_t, m01), __builtin_bit_cast(uint32_t, m23),
+                                                                        __builtin_bit_cast(uint32_t, m45), __builtin_bit_cast(uint32_t, m67)};
+                    dds[sbuf][srow] = hdr.x;
+                }
+                u32x4 *adst = reinterpret_cast<u32x4 *>(&As[buf][srow][32u * sh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) adst[i] = av[g][i];
+                // the slot is free: the same group of the next super-block goes out.  Past the end the last super-block is
+                // fetched again and dropped: with the same loads in every round the waits count exactly how many are newer
+                {
+                    const uint8_t *block = wrow + (size_t)next * 144u;
+                    qs[g] = *(global_uint4)(uintptr_t)(block + 16u + 32u * g + 16u * sh);
+                    const _Float16 *at = arow + (size_t)(4u * next + g) * 64u;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) av[g][i] = *(global_uint4)(uintptr_t)(at + 8 * i);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();  // step is staged; the multipliers are done with the step before it
+            }
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- multipliers
+    // wave (wm, wn) owns rows 64 wm.. of A' and weight rows 64 wn..
     const uint32_t wm = wave >> 1, wn = wave & 1u, l32 = lane & 31u, part = lane >> 5;
     const uint32_t nsb = p.K / 256u;
     const _Float16 *sums[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) sums[i] = p.S + (size_t)min(m0 + 64u * wm + 32u * i + l32, p.rows - 1u) * nsb * 16u + 8u * part;
 
-    f32x16 acc[2][2], tmp[2][2];
+    f32x16 acc[2][2], tmp[2][2], zero;
+#pragma unroll
+    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f, tmp[i][j][e] = 0.0f;
+        for (int j = 0; j < 2; j++) acc[i][j] = zero, tmp[i][j] = zero;
 
-    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
-    u32x4 hdr, qs, av[4];
-    auto fetch = [&](uint32_t step) {
-        const uint32_t b = step >> 2, g = step & 3u;
-        const uint8_t *block = wrow + (size_t)b * 144u;
-        hdr = *(global_uint4)(uintptr_t)block;
-        qs = *(global_uint4)(uintptr_t)(block + 16u + 32u * g + 16u * sh);
-        const _Float16 *at = arow + (size_t)step * 64u;
+    for (uint32_t first = 0; first < steps; first += 4) {
+        const uint32_t sbuf = (first >> 2) & 1u;
+        u32x4 sraw[2];
 #pragma unroll
-        for (int i = 0; i < 4; i++) av[i] = *(global_uint4)(uintptr_t)(at + 8 * i);
-    };
-    // the fetched step into half `buf` of LDS
-    auto stage = [&](uint32_t step) {
-        const uint32_t g = step & 3u, buf = step & 1u, sbuf = (step >> 2) & 1u;
-        // 6-bit fields of sub-blocks 2g, 2g+1 (crates/neura-precision/src/ggml.rs:127-136); 0x6400 | v is the half 1024 + v
-        const uint32_t shift = 16u * (g & 1u);
-        const uint32_t ya = (hdr.y >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
-        const uint32_t sc = g < 2 ? (ya & 0x3f3fu) : ((wa & 0x0f0fu) | ((ya >> 2) & 0x3030u));
-        const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;  // (1024 + sc0, 1024 + sc1)
-        const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
-        const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;     // (sc0 * 2^10, sc1 * 2^6)
-        const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
-        const uint32_t words[4] = {qs.x, qs.y, qs.z, qs.w};
-        uint32_t low[8], high[8];
+        for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(first >> 2) * 16u);  // wanted at the end of the super-block
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const uint32_t even = words[w], odd = words[w] >> 8;
-            // element order inside a word: 0, 2 then 1, 3 (the byte lanes); the activations were packed in the same order
-            low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
-            low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
-            high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
-            high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+        for (int g = 0; g < 4; g++) {
+            const uint32_t buf = g & 1u;
+            __syncthreads();  // the step is staged
+            // ---- 64 x 64 x 64 per wave; the operands of the next 16 k are on their way while the matrix cores walk these
+            half8_t a[2][2], b[2][2];
+            auto operands = [&](int kk) {
+#pragma unroll
+                for (int i = 0; i < 2; i++) a[kk & 1][i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
+#pragma unroll
+                for (int j = 0; j < 2; j++) b[kk & 1][j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
+            };
+            operands(0);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                if (kk < 3) operands(kk + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        tmp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk & 1][i], b[kk & 1][j], (g == 0 && kk == 0) ? zero : tmp[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        u32x4 *blow = reinterpret_cast<u32x4 *>(&Bs[buf][srow][16u * sh]), *bhigh = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u + 16u * sh]);
-        blow[0] = u32x4{low[0], low[1], low[2], low[3]};
-        blow[1] = u32x4{low[4], low[5], low[6], low[7]};
-        bhigh[0] = u32x4{high[0], high[1], high[2], high[3]};
-        bhigh[1] = u32x4{high[4], high[5], high[6], high[7]};
-        if (g == 0 && sh == 0) {
-            // the eight minimums of the super-block, as halves
-            const uint32_t lo4 = hdr.z & 0x3f3f3f3fu;                                         // m0..m3
-            const uint32_t hi4 = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);  // m4..m7
-            const half2_t m01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c010c00u) | 0x64006400u) - offset;
-            const half2_t m23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c030c02u) | 0x64006400u) - offset;
-            const half2_t m45 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c010c00u) | 0x64006400u) - offset;
-            const half2_t m67 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c030c02u) | 0x64006400u) - offset;
-            *reinterpret_cast<u32x4 *>(mns[sbuf][srow]) = u32x4{__builtin_bit_cast(uint32_t, m01), __builtin_bit_cast(uint32_t, m23),
-                                                                __builtin_bit_cast(uint32_t, m45), __builtin_bit_cast(uint32_t, m67)};
-            dds[sbuf][srow] = hdr.x;
+        // ---- the super-block is complete: weigh by d, then take the minimums off
+        float dscale[2], mscale[2];
+        half8_t b2[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const half2_t dd = __builtin_bit_cast(half2_t, dds[sbuf][64u * wn + 32u * j + l32]);
+            dscale[j] = (float)dd.x * 16384.0f;  // the weights were staged * 2^-14
+            mscale[j] = (float)dd.y * -64.0f;    // the sums were packed / 64
+            b2[j] = *reinterpret_cast<const half8_t *>(mns[sbuf][64u * wn + 32u * j + l32]);
+            if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11 against the residues * 2^11
         }
-        u32x4 *adst = reinterpret_cast<u32x4 *>(&As[buf][srow][32u * sh]);
 #pragma unroll
-        for (int i = 0; i < 4; i++) adst[i] = av[i];
-    };
-
-    const uint32_t steps = p.K / 64u;
-    fetch(0);
-    stage(0);
-    if (steps > 1) fetch(1);
-    __syncthreads();
-    u32x4 sraw[2];
-    for (uint32_t step = 0; step < steps; step++) {
-        const uint32_t g = step & 3u, buf = step & 1u, sbuf = (step >> 2) & 1u;
-        if (g == 0) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(step >> 2) * 16u);  // wanted three steps from here
-        }
-        if (step + 1 < steps) {
-            stage(step + 1);
-            if (step + 2 < steps) fetch(step + 2);
-        }
-        // ---- 64 x 64 x 64 per wave
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            half8_t a[2], b[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) a[i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
-#pragma unroll
-            for (int j = 0; j < 2; j++) b[j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) tmp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], tmp[i][j], 0, 0, 0);
-        }
-        if (g == 3) {
-            // ---- the super-block is complete: weigh by d, then take the minimums off
-            float dscale[2], mscale[2];
-            half8_t b2[2];
+        for (int i = 0; i < 2; i++) {
+            const half8_t a2 = __builtin_bit_cast(half8_t, sraw[i]);  // k 0..7: the sums; k 8..15: their residues
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const half2_t dd = __builtin_bit_cast(half2_t, dds[sbuf][64u * wn + 32u * j + l32]);
-                dscale[j] = (float)dd.x * 16384.0f;  // the weights were staged * 2^-14
-                mscale[j] = (float)dd.y * -64.0f;    // the sums were packed / 64
-                b2[j] = *reinterpret_cast<const half8_t *>(mns[sbuf][64u * wn + 32u * j + l32]);
-                if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11 against the residues * 2^11
-            }
+                const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[j], zero, 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const half8_t a2 = __builtin_bit_cast(half8_t, sraw[i]);  // k 0..7: the sums; k 8..15: their residues
+                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(dscale[j], tmp[i][j][e], acc[i][j][e]);
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-#pragma unroll
-                    for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(dscale[j], tmp[i][j][e], acc[i][j][e]);
-                    f32x16 zero;
-#pragma unroll
-                    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
-                    const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[j], zero, 0, 0, 0);
-#pragma unroll
-                    for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(mscale[j], mins[e], acc[i][j][e]), tmp[i][j][e] = 0.0f;
-                }
+                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(mscale[j], mins[e], acc[i][j][e]);
             }
         }
-        __syncthreads();  // step + 1 is staged; every wave is done with this step's half of LDS
     }
     // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
 #pragma unroll
@@ -424,7 +447,7 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
         sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
-    hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(256), GEMM_Q4K_LDS, d->stream, p);
+    hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
