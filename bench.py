@@ -248,7 +248,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_kernel (down)" if element == 12 else "gemv_q8_0_kernel",
+            "kernel": "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_deep_kernel (down)" if element == 12 else "gemv_q8_0_kernel",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

@@ -713,6 +713,21 @@ __device__ __forceinline__ int dpp_int(int v) {
 // KS waves share one tile (each takes every KS-th super-block of the slice); NW waves per
 // workgroup; P activation rows; D super-blocks in flight per wave (the loads run ahead of the
 // arithmetic across tile boundaries, and the first ones are issued before the activations are staged).
+// The four signed base-256 digits of an integer below 2^30 in magnitude, one per byte, least significant in byte 0:
+// adding 128 at the three low byte positions makes every low byte the digit plus 128 (the carries are the ones the
+// signed digits need), and flipping bit 7 takes the 128 off again.
+__device__ __forceinline__ uint32_t signed_digits(int whole) { return ((uint32_t)whole + 0x00808080u) ^ 0x00808080u; }
+
+// Digit planes of four elements: plane[0] holds their most significant digits (element e in byte e), plane[3] the least.
+__device__ __forceinline__ void digit_planes(uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3, uint32_t (&plane)[4]) {
+    const uint32_t lo01 = __builtin_amdgcn_perm(d1, d0, 0x05010400u), hi01 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(d3, d2, 0x05010400u), hi23 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+    plane[3] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    plane[2] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    plane[1] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    plane[0] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
 template <int KS, int NW, int P, int D>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
     extern __shared__ uint32_t xop[];  // [block][16 steps][4 groups][4 P digit columns] of 4 bytes; then sums; then tile partials
@@ -754,21 +769,24 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
         }
         return rowp + (size_t)blk0 * 144u + g * 32u;
     };
-    // the loads run D super-blocks ahead of the arithmetic: (ahead_base, ahead_b) is the next one to fetch
+    // The loads run D super-blocks ahead of the arithmetic: (ahead_base, ahead_b) is the next one to fetch.  Every fetch
+    // issues its three loads, whatever is left: past the last super-block of this wave the last one is fetched again and
+    // never used.  A fetch that could be skipped would make the compiler, which counts the loads in flight along every
+    // path, wait for the newest load before each use of the oldest, and the ring would hide nothing.
     MfmaUnit ring[D];
     uint32_t ahead_base = blockIdx.x * TPW, ahead_b = ks;
-    const uint8_t *ahead_row = ahead_base + tslot < p.tiles ? lane_row(ahead_base + tslot) : nullptr;
+    const uint8_t *ahead_row = lane_row(min(ahead_base + tslot, p.tiles - 1u));
     auto fetch = [&](MfmaUnit &u) {
-        if (ahead_base + tslot >= p.tiles) return;  // past the last tile (stays so)
         const uint8_t *at = ahead_row + (size_t)ahead_b * 144u;
         u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
         u.qa = *(global_uint4)(uintptr_t)(at + 16u);
         u.qb = *(global_uint4)(uintptr_t)(at + 32u);
-        ahead_b += KS;
-        if (ahead_b >= nb) {
+        if (ahead_b + KS < nb) {
+            ahead_b += KS;
+        } else if (ahead_base + stride + tslot < p.tiles) {
             ahead_b = ks;
             ahead_base += stride;
-            if (ahead_base + tslot < p.tiles) ahead_row = lane_row(ahead_base + tslot);
+            ahead_row = lane_row(ahead_base + tslot);
         }
     };
 #pragma unroll
@@ -853,20 +871,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
             uint32_t word[2][4];
 #pragma unroll
             for (int h = 0; h < 2; h++) {
-                word[h][0] = word[h][1] = word[h][2] = word[h][3] = 0u;
+                uint32_t digits[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float rounded = rintf(v[4 * h + i] * scale);
-                    const int whole = (int)rounded;
-                    const int d3 = (whole << 24) >> 24, upper = (whole - d3) >> 8;
-                    const int d2 = (upper << 24) >> 24, top2 = (upper - d2) >> 8;
-                    const int d1 = (top2 << 24) >> 24, d0 = (top2 - d1) >> 8;
                     total += rounded;
-                    word[h][0] |= ((uint32_t)d0 & 0xffu) << (8 * i);
-                    word[h][1] |= ((uint32_t)d1 & 0xffu) << (8 * i);
-                    word[h][2] |= ((uint32_t)d2 & 0xffu) << (8 * i);
-                    word[h][3] |= ((uint32_t)d3 & 0xffu) << (8 * i);
+                    digits[i] = signed_digits((int)rounded);
                 }
+                digit_planes(digits[0], digits[1], digits[2], digits[3], word[h]);
             }
             // sum of the 32 activations of this chunk's sub-block: 4 chunks = 4 neighbouring lanes
             total += dpp<DPP_QUAD_XOR1>(total);
@@ -956,10 +968,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
             if (base >= p.tiles) break;
             const uint32_t tile = base + tslot;
             const bool live = tile < p.tiles;
-            if (live) {
-                compute(ring[slot], b);
-                fetch(ring[slot]);
-            }
+            compute(ring[slot], b);  // a wave past the last tile multiplies what it fetched again; nothing of it is published
+            fetch(ring[slot]);
             b += KS;
             if (b < nb) continue;
                 // lane (r, g) holds group g's share of output row r for every activation row; the four groups are summed across lanes
@@ -1015,6 +1025,129 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
             base += stride;
             parity ^= 1u;
         }
+    }
+}
+
+// One activation row against a short, deep matrix (a down projection: few output rows, long rows).  One 16-row tile
+// per workgroup, its super-blocks dealt to the NW waves in turn, and no shared staging at all: a wave turns the 256
+// activations of a super-block into digits itself, right before it multiplies them, in a corner of LDS nobody else
+// reads.  The digits are scaled per sub-block of 32 (a power of two that puts the sub-block's largest magnitude in
+// [2^29, 2^30)), which is exact, finer than one scale per row, and needs no pass over the whole row first: nothing
+// in the kernel waits for anything but its own loads until the sixteen partial sums of a row meet at the end.
+// Loads are issued whether or not a super-block is left (the last one again, its product dropped), so that the
+// waits count exactly how many loads are newer than the one needed.
+template <int NW, int D>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MfmaParams p) {
+    static_assert(D % 2 == 0, "the activation ring alternates between two slots");
+    __shared__ __attribute__((aligned(16))) uint32_t digits[NW][256];  // [step][group][digit plane] per wave
+    __shared__ float sums[NW][16];                                    // per wave: 8 sub-block sums, 8 sub-block unscales
+    __shared__ float part[NW][16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t tile = blockIdx.x;
+    const uint32_t r = lane & 15u, g = lane >> 4;
+    const uint32_t nb = p.nblk;
+    const uint32_t count = wave < nb ? (nb - wave + NW - 1u) / NW : 0u;  // super-blocks wave, wave + NW, ...
+    const uint32_t last = count ? count - 1u : 0u;
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(1))) f32x4 *global_float4;
+
+    float residual = 0.0f;
+    if (wave == 0 && lane < 16u && p.residual) residual = p.residual[(size_t)tile * 16u + lane];
+
+    const uint8_t *const rowp = p.W[0] + (size_t)(tile * 16u + r) * p.row_bytes + g * 32u;
+    const float *const xp = p.x + 4u * lane;
+    auto block_of = [&](uint32_t i) { return min(wave + NW * min(i, last), nb - 1u); };
+    MfmaUnit ring[D];
+    f32x4 xring[2];
+    auto fetch_x = [&](f32x4 &x, uint32_t i) { x = *(global_float4)(uintptr_t)(xp + (size_t)block_of(i) * 256u); };
+    auto fetch_w = [&](MfmaUnit &u, uint32_t i) {
+        const uint8_t *at = rowp + (size_t)block_of(i) * 144u;
+        u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
+        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
+        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+    };
+    fetch_x(xring[0], 0);
+    fetch_x(xring[1], 1);
+#pragma unroll
+    for (int i = 0; i < D; i++) fetch_w(ring[i], i);
+
+    const ScaleLane lane_scales = scale_lane(g);
+    uint32_t *const mine = digits[wave];
+    float *const mysums = sums[wave];
+    const uint32_t *const xlane = mine + g * 4u + (lane & 3u);
+    float acc = 0.0f;
+    for (uint32_t first = 0; first < count; first += D) {
+#pragma unroll
+        for (int slot = 0; slot < D; slot++) {
+            const uint32_t i = first + slot;
+            // ---- this super-block's 256 activations -> digits: lane l holds elements 4l..4l+3, eight lanes a sub-block
+            const f32x4 xv = xring[slot & 1];
+            fetch_x(xring[slot & 1], i + 2u);
+            const float v[4] = {xv.x, xv.y, xv.z, xv.w};
+            uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
+#pragma unroll
+            for (int e = 0; e < 4; e++) top = max(top, __builtin_bit_cast(uint32_t, v[e]) & 0x7fffffffu);
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+            top = max(top, (uint32_t)dpp_int<0x141>((int)top));  // half mirror: the other quad of the eight
+            const uint32_t raw_exponent = top >> 23;
+            const uint32_t exponent = min(max(raw_exponent, 30u), 254u);
+            const float scale = __builtin_bit_cast(float, (283u - exponent) << 23);
+            const float unscale = raw_exponent == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 29u) << 23);
+            float total = 0.0f;
+            uint32_t word[4], each[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float rounded = rintf(v[e] * scale);
+                total += rounded;
+                each[e] = signed_digits((int)rounded);
+            }
+            digit_planes(each[0], each[1], each[2], each[3], word);
+            total += dpp<DPP_QUAD_XOR1>(total);
+            total += dpp<DPP_QUAD_XOR2>(total);
+            total += dpp<0x141>(total);
+            // elements 4l..4l+3 are nibble word l % 16 of group l / 16 (words 0..7: the low sub-block, 8..15: the high one)
+            *reinterpret_cast<u32x4 *>(mine + ((lane & 15u) * 4u + (lane >> 4)) * 4u) = u32x4{word[0], word[1], word[2], word[3]};
+            if ((lane & 7u) == 0) mysums[lane >> 3] = total, mysums[8u + (lane >> 3)] = unscale;
+            __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
+
+            // ---- the super-block against them
+            const MfmaUnit &u = ring[slot];
+            const uint32_t words[8] = {u.qa.x, u.qa.y, u.qa.z, u.qa.w, u.qb.x, u.qb.y, u.qb.z, u.qb.w};
+            i32x4 cl = {0, 0, 0, 0}, ch = {0, 0, 0, 0};
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                const int low = (int)(words[w] & 0x0f0f0f0fu), high = (int)((words[w] >> 4) & 0x0f0f0f0fu);
+                const int xl = (int)xlane[w * 16], xh = (int)xlane[(8 + w) * 16];
+                cl = __builtin_amdgcn_mfma_i32_4x4x4i8(xl, low, cl, 0, 0, 0);
+                ch = __builtin_amdgcn_mfma_i32_4x4x4i8(xh, high, ch, 0, 0, 0);
+            }
+            half2_t sc, mn;
+            scale_pairs(u.hdr, lane_scales, sc, mn);                  // integers as half subnormals: value * 2^-24
+            const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
+            const float ul = mysums[8u + 2u * g], uh = mysums[9u + 2u * g];
+            const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * 16777216.0f;
+            const float s0 = d24 * (float)sc.x * ul, s1 = d24 * (float)sc.y * uh, m0 = m24 * (float)mn.x * ul, m1 = m24 * (float)mn.y * uh;
+            const float fl = fmaf(fmaf(fmaf((float)cl[0], 256.0f, (float)cl[1]), 256.0f, (float)cl[2]), 256.0f, (float)cl[3]);
+            const float fh = fmaf(fmaf(fmaf((float)ch[0], 256.0f, (float)ch[1]), 256.0f, (float)ch[2]), 256.0f, (float)ch[3]);
+            const float product = fmaf(s0, fl, s1 * fh) - fmaf(m0, mysums[2u * g], m1 * mysums[2u * g + 1u]);
+            acc += i < count ? product : 0.0f;
+            __builtin_amdgcn_wave_barrier();  // the next super-block's digits overwrite these
+            fetch_w(ring[slot], i + D);
+        }
+    }
+    // lane (r, g) holds group g's share of output row r: the four groups, then the waves
+    acc += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, acc), 0x401F));  // lane ^ 16
+    acc += __shfl_xor(acc, 32, 64);
+    if (g == 0) part[wave][r] = acc;
+    __syncthreads();
+    if (wave == 0 && lane < 16u) {
+        float total = 0.0f;
+#pragma unroll
+        for (int k = 0; k < NW; k++) total += part[k][lane];
+        p.y[(size_t)tile * 16u + lane] = p.residual ? residual + total : total;
     }
 }
 
@@ -1221,9 +1354,29 @@ static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t
 // LDS bytes of the staged activations of `blocks` super-blocks for P activation rows: digits + sums
 static size_t mfma_staged(uint32_t blocks, uint32_t P) { return (size_t)blocks * (1024u + 32u) * P; }
 
+// whether the deep kernel (one tile per workgroup, sixteen waves along K) serves this product
+static bool mfma_goes_deep(const nh_device *d, const GemvArgs &a) {
+    const int mode = env_int("NEURA_HIP_MFMA_DEEP", 1);
+    if (mode == 0 || a.rows != 1 || a.swiglu || a.norm_w || a.W[1] || a.W[2]) return false;
+    // a matrix short enough that its tiles do not even fill the device once, and rows deep enough to feed sixteen waves
+    return mode == 2 || (a.N / 16u <= (uint32_t)d->compute_units && a.K / 256u >= 32u);
+}
+
 static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
     const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
     const uint32_t nblk = a.K / 256u;
+    if (mfma_goes_deep(d, a)) {
+        MfmaParams p{};
+        p.W[0] = static_cast<const uint8_t *>(a.W[0]);
+        p.x = a.x, p.y = a.y, p.residual = a.residual;
+        p.N = a.N, p.K = a.K, p.row_bytes = nblk * 144u, p.nblk = nblk, p.rows = 1, p.tiles = a.N / 16u;
+        profile_mark(d);
+        hipLaunchKernelGGL((gemv_q4k_mfma_deep_kernel<16, 2>), dim3(p.tiles), dim3(1024), 0, d->stream, p);
+        NH_HIP(hipGetLastError());
+        profile_mark(d);
+        if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+        return NH_OK;
+    }
     const size_t room = 140 * 1024;  // a gfx950 workgroup may take all 160 KiB of a compute unit; tile partials and static arrays need the rest
     for (uint32_t done = 0; done < a.rows;) {
         // activation rows per launch: 4, 2 or 1 (the kernel's instantiations); rows too deep to stage whole are cut into K slices
