@@ -10,7 +10,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int32, c_size_t, c_ui
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY = os.path.join(HERE, "libneura_hip.so")
 
-NH_F32, NH_F16, NH_Q8_0, NH_Q4_K = 0, 1, 8, 12
+NH_F32, NH_F16, NH_Q8_0, NH_Q4_K, NH_Q6_K = 0, 1, 8, 12, 14
 NH_OK, NH_E_ARGUMENT, NH_E_DEVICE, NH_E_MEMORY, NH_E_REFUSAL = 0, -1, -2, -3, -4
 UINT64_MAX = (1 << 64) - 1
 

@@ -53,6 +53,19 @@ __device__ __forceinline__ float q4_k_element(const uint8_t *row, uint64_t i) {
     return __fsub_rn(__fmul_rn(quantum, (float)quant), low);
 }
 
+// element `i` of a row of Q6_K blocks (crates/neura-precision/src/ggml.rs:394-407): d * scale, rounded, times (code - 32)
+__device__ __forceinline__ float q6_k_element(const uint8_t *row, uint64_t i) {
+    const uint8_t *block = row + (i / 256) * 210;
+    uint32_t within = (uint32_t)(i % 256);
+    uint32_t half = within / 128, group = (within % 128) / 32, lane = within % 32;
+    uint8_t packed = block[half * 64 + (group % 2) * 32 + lane];
+    uint32_t low = group >= 2 ? (uint32_t)(packed >> 4) : (uint32_t)(packed & 0x0f);
+    uint32_t high = ((uint32_t)block[128 + half * 32 + lane] >> (2 * group)) & 3u;
+    float scale = (float)(int8_t)block[192 + half * 8 + group * 2 + lane / 16];
+    float quantum = __fmul_rn(half_to_float(load_u16(block + 208)), scale);
+    return __fmul_rn(quantum, (float)(low | (high << 4)) - 32.0f);
+}
+
 // 1 / sqrt(total / columns + eps) with every step rounded to fp32 exactly as IEEE does
 // (crates/neura-kernel/src/task/norm.rs:102-104).  Each step runs in fp64 and is rounded
 // once more to fp32, which for /, + and sqrt equals the correctly rounded fp32 operation.

@@ -14,6 +14,8 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
             value = q8_0_element(src, i);
         else if (ELEMENT == NH_Q4_K)
             value = q4_k_element(src, i);
+        else if (ELEMENT == NH_Q6_K)
+            value = q6_k_element(src, i);
         else if (ELEMENT == NH_F16)
             value = half_to_float(reinterpret_cast<const uint16_t *>(src)[i]);
         else
@@ -35,6 +37,7 @@ int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t 
     switch (element) {
     case NH_Q8_0: hipLaunchKernelGGL(dequant_kernel<NH_Q8_0>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_Q4_K: hipLaunchKernelGGL(dequant_kernel<NH_Q4_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_Q6_K: hipLaunchKernelGGL(dequant_kernel<NH_Q6_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_F16: hipLaunchKernelGGL(dequant_kernel<NH_F16>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_F32: hipLaunchKernelGGL(dequant_kernel<NH_F32>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     default: return fail(NH_E_ARGUMENT, "element %d carries no reader", element);
@@ -76,6 +79,8 @@ __global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__
             value = q8_0_element(row, c);
         else if (ELEMENT == NH_Q4_K)
             value = q4_k_element(row, c);
+        else if (ELEMENT == NH_Q6_K)
+            value = q6_k_element(row, c);
         else if (ELEMENT == NH_F16)
             value = half_to_float(reinterpret_cast<const uint16_t *>(row)[c]);
         else
@@ -98,6 +103,10 @@ int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t
         break;
     case NH_Q4_K:
         hipLaunchKernelGGL(gather_kernel<NH_Q4_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_Q6_K:
+        hipLaunchKernelGGL(gather_kernel<NH_Q6_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     case NH_F16:

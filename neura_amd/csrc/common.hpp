@@ -14,6 +14,7 @@ namespace nh {
 
 constexpr uint32_t Q8_0_BLOCK = 32, Q8_0_BYTES = 34;
 constexpr uint32_t Q4_K_BLOCK = 256, Q4_K_BYTES = 144;
+constexpr uint32_t Q6_K_BLOCK = 256, Q6_K_BYTES = 210;
 constexpr uint32_t WAVE = 64;
 
 int32_t fail(int32_t code, const char *format, ...) __attribute__((format(printf, 2, 3)));
@@ -34,6 +35,7 @@ inline uint64_t payload_bytes(int32_t element, uint64_t elements) {
     switch (element) {
     case NH_Q8_0: return (elements + Q8_0_BLOCK - 1) / Q8_0_BLOCK * Q8_0_BYTES;
     case NH_Q4_K: return (elements + Q4_K_BLOCK - 1) / Q4_K_BLOCK * Q4_K_BYTES;
+    case NH_Q6_K: return (elements + Q6_K_BLOCK - 1) / Q6_K_BLOCK * Q6_K_BYTES;
     case NH_F16: return elements * 2;
     case NH_F32: return elements * 4;
     default: return 0;
@@ -44,6 +46,7 @@ inline uint32_t block_elements(int32_t element) {
     switch (element) {
     case NH_Q8_0: return Q8_0_BLOCK;
     case NH_Q4_K: return Q4_K_BLOCK;
+    case NH_Q6_K: return Q6_K_BLOCK;
     case NH_F16:
     case NH_F32: return 1;
     default: return 0;

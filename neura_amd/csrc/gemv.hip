@@ -661,6 +661,101 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------- Q6_K -------
+//
+// 210-byte super-blocks leave rows on 2-byte boundaries.  A wave copies the two rows it is about to walk into LDS with
+// aligned 128-bit loads -- a row is contiguous, the copy fully coalesced -- and its lanes pick the fields out of LDS
+// two bytes at a time.  A lane takes 16 weights of a super-block: four neighbouring elements of each of the four
+// 32-element groups of one half, which share two words of nibbles and one word of bit pairs
+// (crates/neura-precision/src/ggml.rs:394-407).  The weight is (d * scale) * (code - 32) as in
+// crates/neura-kernel/src/dot.rs:663-797; the sums run in lane order, not in the reference's run order.
+template <int RB>
+__global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
+    extern __shared__ float xs[];  // [RB][slice]; then the raw row slices, two per wave
+    __shared__ float red[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t split = blockIdx.y;
+    const uint32_t blk0 = split * p.blocks_per_split;
+    const uint32_t nb = min(p.blocks_per_split, p.nblk - blk0);
+    const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
+    const uint32_t xstride = p.blocks_per_split * 256u;
+    for (uint32_t b = 0; b < RB; b++) {
+        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return i; });
+    }
+    __syncthreads();
+    const uint32_t raw_stride = p.chunks_per_row * 16u;  // bytes of one staged row slice
+    uint8_t *const mine = reinterpret_cast<uint8_t *>(xs + RB * xstride) + (size_t)wave * 2u * raw_stride;
+    const uint32_t units = nb * 16u;
+
+    for (uint32_t first = 2u * (blockIdx.x * 4u + wave); first < p.N; first += 2u * gridDim.x * 4u) {
+        uint32_t lead[2];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const uint32_t i = min(first + r, p.N - 1u);
+            const uint8_t *matrix_end;
+            const uint8_t *src = row_start(p, weight_row(i, p.N, p.swiglu), matrix_end) + (size_t)blk0 * 210u;
+            lead[r] = (uint32_t)((uintptr_t)src & 15u);
+            const uint8_t *from = src - lead[r];
+            const uint32_t bytes = lead[r] + nb * 210u;
+            for (uint32_t c = lane; c * 16u < bytes; c += 64u) {
+                uint4 held;
+                if (from + 16u * c + 16u <= matrix_end) {
+                    held = *reinterpret_cast<const uint4 *>(from + 16u * c);
+                } else {  // the last bytes of the tensor: never read past its end
+                    uint8_t tail[16];
+#pragma unroll
+                    for (int j = 0; j < 16; j++) tail[j] = (from + 16u * c + j < matrix_end) ? from[16u * c + j] : (uint8_t)0;
+                    held = *reinterpret_cast<uint4 *>(tail);
+                }
+                *reinterpret_cast<uint4 *>(mine + r * raw_stride + 16u * c) = held;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
+
+        float acc[2][RB];
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int b = 0; b < RB; b++) acc[r][b] = 0.0f;
+        for (uint32_t u = lane; u < units; u += 64u) {
+            const uint32_t blk = u >> 4, half = (u >> 3) & 1u, j = u & 7u;
+            float4 xv[RB][4];
+#pragma unroll
+            for (int b = 0; b < RB; b++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) xv[b][g] = *reinterpret_cast<const float4 *>(xs + b * xstride + blk * 256u + half * 128u + g * 32u + 4u * j);
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                const uint8_t *block = mine + r * raw_stride + lead[r] + blk * 210u;
+                auto word = [&](uint32_t at) { return (uint32_t)*reinterpret_cast<const uint16_t *>(block + at) | ((uint32_t)*reinterpret_cast<const uint16_t *>(block + at + 2u) << 16); };
+                const uint32_t lows = word(half * 64u + 4u * j), highs = word(half * 64u + 32u + 4u * j), pairs = word(128u + half * 32u + 4u * j);
+                const float d = half_to_float(*reinterpret_cast<const uint16_t *>(block + 208u));
+                const uint8_t *scales = block + 192u + half * 8u + (j >> 2);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t nibbles = ((g & 1) ? highs : lows) >> (g >= 2 ? 4 : 0);
+                    const uint32_t codes = (nibbles & 0x0f0f0f0fu) | (((pairs >> (2 * g)) & 0x03030303u) << 4);
+                    const float weight = d * (float)(int8_t)scales[2 * g];
+                    const float c0 = (float)(codes & 0xffu) - 32.0f, c1 = (float)((codes >> 8) & 0xffu) - 32.0f;
+                    const float c2 = (float)((codes >> 16) & 0xffu) - 32.0f, c3 = (float)(codes >> 24) - 32.0f;
+#pragma unroll
+                    for (int b = 0; b < RB; b++) {
+                        const float dot = fmaf(xv[b][g].w, c3, fmaf(xv[b][g].z, c2, fmaf(xv[b][g].y, c1, xv[b][g].x * c0)));
+                        acc[r][b] = fmaf(weight, dot, acc[r][b]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int b = 0; b < RB; b++) acc[r][b] = wave_sum(acc[r][b]);
+        if (lane == 0) publish<2, RB>(p, first, split, acc);
+        __builtin_amdgcn_wave_barrier();  // the next rows overwrite the staged ones
+    }
+}
+
 // ------------------------------------------------------------------- Q4_K on MFMA --------
 //
 // The same product with the multiply-adds on the matrix cores, in exact integer arithmetic.
@@ -1461,12 +1556,65 @@ bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     return a.end[0] % width == 0 && a.end[1] % width == 0 && a.end[2] == a.N;
 }
 
+// Q6_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
+template <int RB>
+static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
+    GemvParams p{};
+    for (int s = 0; s < 3; s++) {
+        p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+        p.end[s] = a.end[s];
+    }
+    p.x = x, p.y = y, p.residual = residual, p.norm_w = a.norm_w;
+    p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps;
+    p.row_bytes = (uint32_t)payload_bytes(NH_Q6_K, a.K);
+    p.nblk = a.K / 256u;
+    const uint32_t most_blocks = 16u;
+    p.splits = (p.nblk + most_blocks - 1) / most_blocks;
+    p.blocks_per_split = (p.nblk + p.splits - 1) / p.splits;
+    p.splits = (p.nblk + p.blocks_per_split - 1) / p.blocks_per_split;
+    if (p.splits > 1) {
+        p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * RB * a.N * sizeof(float)));
+        if (!p.partial) return NH_E_MEMORY;
+    }
+    p.chunks_per_row = (15u + p.blocks_per_split * 210u + 15u) / 16u;
+    const size_t lds = (size_t)RB * p.blocks_per_split * 256u * sizeof(float) + (size_t)8 * p.chunks_per_row * 16u;
+    uint32_t blocks_x = (a.N + 7u) / 8u;
+    uint32_t most = (uint32_t)d->compute_units * 2u / p.splits;
+    if (most < 1) most = 1;
+    if (blocks_x > most) blocks_x = most;
+    profile_mark(d);
+    hipLaunchKernelGGL((gemv_q6_k_kernel<RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, p);
+    NH_HIP(hipGetLastError());
+    if (p.splits > 1) {
+        uint32_t outputs = (a.swiglu ? a.N / 2 : a.N) * RB;
+        hipLaunchKernelGGL(gemv_fold_kernel, dim3((outputs + 255) / 256), dim3(256), 0, d->stream, p.partial, p.splits, (uint32_t)RB, a.N,
+                           residual, a.swiglu, y);
+        NH_HIP(hipGetLastError());
+    }
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
+}
+
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
     uint32_t done = 0;
+    if (a.element == NH_Q6_K) {
+        if (a.swiglu && (a.N % 2u || a.end[0] != a.N / 2)) return fail(NH_E_ARGUMENT, "a swiglu product halves %u rows", a.N);
+        while (done < a.rows) {
+            const float *x = a.x + (size_t)done * a.K;
+            float *y = a.y + (size_t)done * outputs;
+            const float *residual = a.residual ? a.residual + (size_t)done * a.N : nullptr;
+            const bool pair = a.rows - done >= 2;
+            int32_t status = pair ? launch_q6k_rows<2>(d, a, x, y, residual) : launch_q6k_rows<1>(d, a, x, y, residual);
+            if (status != NH_OK) return status;
+            done += pair ? 2 : 1;
+        }
+        return NH_OK;
+    }
     while (done < a.rows) {
         uint32_t left = a.rows - done;
         const float *x = a.x + (size_t)done * a.K;

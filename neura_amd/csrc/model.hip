@@ -463,7 +463,7 @@ int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elemen
 int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
                 float *dev_y, const nh_epilogue *epilogue) {
     NH_REQUIRE(device && dev_W && dev_x && dev_y, "a product names no device or no buffer");
-    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K, "a narrow product walks Q8_0 or Q4_K weights, not element %d", element);
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || element == NH_Q6_K, "a narrow product walks Q8_0, Q4_K or Q6_K weights, not element %d", element);
     NH_REQUIRE(N > 0 && K > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K, block_elements(element));
     NH_REQUIRE(rows >= 1 && rows <= 8, "a narrow product takes one to eight rows, not %u", rows);
     NH_REQUIRE(aligned16(dev_W) && aligned16(dev_x), "a product reads its weights and activations from 16-byte aligned addresses");
@@ -480,7 +480,8 @@ int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t 
             NH_REQUIRE(N % 2 == 0, "a swiglu product halves %u rows", N);
             a.W[1] = static_cast<const uint8_t *>(dev_W) + (size_t)(N / 2) * payload_bytes(element, K);
             a.end[0] = N / 2;
-            NH_REQUIRE(aligned16(a.W[1]), "the up half of a swiglu product starts off a 16-byte boundary");
+            // Q6_K rows are read through aligned copies whatever their own alignment
+            NH_REQUIRE(element == NH_Q6_K || aligned16(a.W[1]), "the up half of a swiglu product starts off a 16-byte boundary");
         }
     }
     return launch_gemv(device, a);
@@ -489,7 +490,7 @@ int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t 
 int32_t nh_gemm(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const void *dev_X, int32_t x_element,
                 uint32_t M, float *dev_Y, const nh_epilogue *epilogue) {
     NH_REQUIRE(device && dev_W && dev_X && dev_Y, "a product names no device or no buffer");
-    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K, "a wide product walks Q8_0 or Q4_K weights, not element %d", element);
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || element == NH_Q6_K, "a wide product walks Q8_0, Q4_K or Q6_K weights, not element %d", element);
     NH_REQUIRE(x_element == NH_F32 || x_element == NH_F16, "a wide product takes fp32 or fp16 activations, not element %d", x_element);
     NH_REQUIRE(N > 0 && K > 0 && M > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K,
                block_elements(element));

@@ -1,7 +1,7 @@
 """Seeded synthetic GGUF payloads of the benchmark configurations, and vectorised numpy
-codecs of the two block formats.
+codecs of the block formats.
 
-The numpy codecs restate ggml's published Q8_0 / Q4_K layouts independently of the C oracle
+The numpy codecs restate ggml's published Q8_0 / Q4_K / Q6_K layouts independently of the C oracle
 (they are how the tests pin it) and quantize random-init model weights fast enough for the
 0.5B-shape configuration.  They run on the host only.
 """
@@ -9,6 +9,7 @@ import numpy as np
 
 Q8_0_BLOCK, Q8_0_BYTES = 32, 34
 Q4_K_BLOCK, Q4_K_BYTES = 256, 144
+Q6_K_BLOCK, Q6_K_BYTES = 256, 210
 
 
 def q8_0_random(rng, elements):
@@ -30,6 +31,35 @@ def q4_k_random(rng, elements):
     raw[:, 0:4] = d.view(np.uint8).reshape(blocks, 4)
     raw[:, 4:] = rng.integers(0, 256, (blocks, 140), dtype=np.uint8)
     return raw.reshape(-1)
+
+
+def q6_k_random(rng, elements):
+    """Super-blocks of random 6-bit codes (128 nibble bytes, 64 bytes of bit pairs), int8 sub-scales drawn uniformly
+    from [-64, 63] and fp16 d drawn |N(0, 0.001)| (weights of the order of 0.01..1, as d * scale * (code - 32))."""
+    blocks = elements // Q6_K_BLOCK
+    raw = np.empty((blocks, Q6_K_BYTES), dtype=np.uint8)
+    raw[:, 0:192] = rng.integers(0, 256, (blocks, 192), dtype=np.uint8)
+    raw[:, 192:208] = rng.integers(-64, 64, (blocks, 16), dtype=np.int8).view(np.uint8)
+    raw[:, 208:210] = np.abs(rng.normal(0.0, 0.001, (blocks, 1))).astype(np.float16).view(np.uint8).reshape(blocks, 2)
+    return raw.reshape(-1)
+
+
+def q6_k_dequant(raw, elements):
+    """ggml's dequantize_row_q6_K, vectorised: per half of 128, element l of groups 0..3 takes nibble ql[l] & 15,
+    ql[l + 32] & 15, ql[l] >> 4, ql[l + 32] >> 4 and bit pairs 0, 2, 4, 6 of qh[l]; scale sc[l // 16 + 2 * group]."""
+    f32 = np.float32
+    blocks = np.asarray(raw, dtype=np.uint8).reshape(-1, Q6_K_BYTES)[: elements // Q6_K_BLOCK]
+    d = blocks[:, 208:210].copy().view(np.float16).astype(f32)              # [blocks, 1]
+    sc = blocks[:, 192:208].view(np.int8).astype(f32).reshape(-1, 2, 8)      # [blocks, half, 8]
+    ql = blocks[:, 0:128].reshape(-1, 2, 2, 32)                              # [blocks, half, low/high 32, l]
+    qh = blocks[:, 128:192].reshape(-1, 2, 32)
+    out = np.empty((blocks.shape[0], 2, 4, 32), dtype=f32)
+    for group in range(4):
+        nibble = (ql[:, :, group % 2, :] >> 4) if group >= 2 else (ql[:, :, group % 2, :] & 0x0F)
+        code = (nibble | (((qh >> (2 * group)) & 3) << 4)).astype(f32) - f32(32)
+        scale = np.repeat(sc[:, :, 2 * group:2 * group + 2], 16, axis=2)      # [blocks, half, 32]
+        out[:, :, group, :] = (d[:, :, None] * scale).astype(f32) * code
+    return out.reshape(-1)
 
 
 def q8_0_dequant(raw, elements):
@@ -114,9 +144,9 @@ def q4_k_quantize(values):
 
 
 QUANTIZE = {8: q8_0_quantize, 12: q4_k_quantize}
-RANDOM = {8: q8_0_random, 12: q4_k_random}
-DEQUANT = {8: q8_0_dequant, 12: q4_k_dequant}
-BLOCK_BYTES = {8: (Q8_0_BLOCK, Q8_0_BYTES), 12: (Q4_K_BLOCK, Q4_K_BYTES)}
+RANDOM = {8: q8_0_random, 12: q4_k_random, 14: q6_k_random}
+DEQUANT = {8: q8_0_dequant, 12: q4_k_dequant, 14: q6_k_dequant}
+BLOCK_BYTES = {8: (Q8_0_BLOCK, Q8_0_BYTES), 12: (Q4_K_BLOCK, Q4_K_BYTES), 14: (Q6_K_BLOCK, Q6_K_BYTES)}
 
 
 def matrix_bytes(element, rows, columns):

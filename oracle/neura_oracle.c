@@ -40,13 +40,15 @@
 #define Q8_0_BYTES 34
 #define Q4_K_BLOCK 256
 #define Q4_K_BYTES 144
+#define Q6_K_BLOCK 256
+#define Q6_K_BYTES 210 /* 128 low nibbles, 64 bytes of high bit pairs, 16 int8 scales, f16 d: neura-abi/src/element.rs:167-170 */
 #define SUB_BLOCK 32
 #define FOLDED_LANES 32   /* neura-profile/src/profile.rs:1327 */
 #define FOLDED_STAGE 1024 /* neura-profile/src/profile.rs:1358 */
 #define WORKGROUP 256     /* neura-profile/src/profile.rs:2086-2089 */
 #define ATTN_KEYS 16      /* neura-profile/src/profile.rs:70 */
 
-enum { EL_F32 = 0, EL_F16 = 1, EL_Q8_0 = 8, EL_Q4_K = 12 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
+enum { EL_F32 = 0, EL_F16 = 1, EL_Q8_0 = 8, EL_Q4_K = 12, EL_Q6_K = 14 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
 
 /* ---------------------------------------------------------------- f16 ---- */
 
@@ -176,6 +178,27 @@ static void q4_k_values(const uint8_t *field, float *out) {
     }
 }
 
+/* crates/neura-precision/src/ggml.rs:394-407: two halves of 128, four groups of 32 in each; the 6-bit code is a
+ * nibble (groups 0, 1 low and 2, 3 high of bytes half*64 + (group%2)*32 + within) plus two bits
+ * (byte 128 + half*32 + within, shifted by 2*group); one int8 scale per 16 elements; value = d * scale * (code - 32),
+ * left to right, every product rounded. */
+static void q6_k_values(const uint8_t *field, float *out) {
+    uint16_t h;
+    memcpy(&h, field + 208, 2);
+    float scale = oracle_f16_to_f32(h);
+    for (uint32_t seat = 0; seat < 2; seat++)
+        for (uint32_t group = 0; group < 4; group++)
+            for (uint32_t within = 0; within < 32; within++) {
+                uint32_t index = group * 2 + within / 16;
+                int8_t sub = (int8_t)field[192 + seat * 8 + index];
+                uint8_t byte = field[seat * 64 + (group % 2) * 32 + within];
+                uint32_t nibble = group >= 2 ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f);
+                uint32_t quant = nibble | (((uint32_t)(field[128 + seat * 32 + within] >> (2 * group)) & 3u) << 4);
+                float product = scale * (float)sub;
+                *out++ = product * ((float)quant - 32.0f);
+            }
+}
+
 /* crates/neura-precision/src/ggml.rs:22-38 (unpack); elements must be whole blocks */
 int oracle_unpack(int element, const uint8_t *bytes, uint64_t elements, float *out) {
     if (element == EL_Q8_0) {
@@ -186,6 +209,11 @@ int oracle_unpack(int element, const uint8_t *bytes, uint64_t elements, float *o
     if (element == EL_Q4_K) {
         if (elements % Q4_K_BLOCK) return -1;
         for (uint64_t b = 0; b < elements / Q4_K_BLOCK; b++) q4_k_values(bytes + b * Q4_K_BYTES, out + b * Q4_K_BLOCK);
+        return 0;
+    }
+    if (element == EL_Q6_K) {
+        if (elements % Q6_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < elements / Q6_K_BLOCK; b++) q6_k_values(bytes + b * Q6_K_BYTES, out + b * Q6_K_BLOCK);
         return 0;
     }
     if (element == EL_F16) {
@@ -263,6 +291,50 @@ static void q4_k_encode(const float *values, uint8_t *field) {
     }
 }
 
+/* crates/neura-precision/src/ggml.rs:352-392.  Sixteen sub-blocks of 16: factor = largest magnitude / 32, super scale =
+ * largest factor / 127 stored as f16 while the f32 value quantizes.  `quantized` (ggml.rs:120-125) converts the
+ * rounded, clamped quotient to an unsigned integer, which in Rust saturates: every negative quotient becomes 0, so
+ * negative values pack as code 32 (zero).  This follows the reference; a decoder never notices. */
+static void q6_k_encode(const float *values, uint8_t *field) {
+    float factors[16];
+    for (int at = 0; at < 16; at++) {
+        float size = 0.0f;
+        for (int i = 0; i < 16; i++) {
+            float a = fabsf(values[at * 16 + i]);
+            if (size < a) size = a;
+        }
+        factors[at] = size / 32.0f;
+    }
+    float scale = 0.0f;
+    for (int at = 0; at < 16; at++) scale = greatest(scale, fabsf(factors[at]));
+    scale = scale / 127.0f;
+    memset(field, 0, Q6_K_BYTES);
+    uint16_t h = oracle_f32_to_f16(scale);
+    memcpy(field + 208, &h, 2);
+    for (int at = 0; at < 16; at++) {
+        int8_t code = 0;
+        if (scale != 0.0f) code = (int8_t)clampf(round_away(factors[at] / scale), -127.0f, 127.0f);
+        field[192 + at] = (uint8_t)code;
+        float factor = scale * (float)code;
+        for (int within = 0; within < 16; within++) {
+            int element = at * 16 + within;
+            int half = element / 128, group = (element % 128) / 32, seat = element % 32;
+            uint32_t quant = 0;
+            if (factor != 0.0f) {
+                float q = clampf(round_away(values[element] / factor), -32.0f, 31.0f);
+                quant = q < 0.0f ? 0u : (uint32_t)q; /* a saturating float -> u32 cast */
+            }
+            quant += 32;
+            uint8_t *byte = &field[half * 64 + (group % 2) * 32 + seat];
+            if (group >= 2)
+                *byte = (uint8_t)((*byte & 0x0f) | ((quant & 15u) << 4));
+            else
+                *byte = (uint8_t)((*byte & 0xf0) | (quant & 15u));
+            field[128 + half * 32 + seat] |= (uint8_t)(((quant >> 4) & 3u) << (2 * group));
+        }
+    }
+}
+
 /* crates/neura-precision/src/ggml.rs:8-20 (pack); n must be whole blocks here */
 int oracle_pack(int element, const float *values, uint64_t n, uint8_t *out) {
     if (element == EL_Q8_0) {
@@ -273,6 +345,11 @@ int oracle_pack(int element, const float *values, uint64_t n, uint8_t *out) {
     if (element == EL_Q4_K) {
         if (n % Q4_K_BLOCK) return -1;
         for (uint64_t b = 0; b < n / Q4_K_BLOCK; b++) q4_k_encode(values + b * Q4_K_BLOCK, out + b * Q4_K_BYTES);
+        return 0;
+    }
+    if (element == EL_Q6_K) {
+        if (n % Q6_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < n / Q6_K_BLOCK; b++) q6_k_encode(values + b * Q6_K_BLOCK, out + b * Q6_K_BYTES);
         return 0;
     }
     if (element == EL_F16) {
@@ -290,6 +367,7 @@ uint64_t oracle_payload_bytes(int element, uint64_t elements) { /* neura-abi/src
     switch (element) {
     case EL_Q8_0: return (elements + Q8_0_BLOCK - 1) / Q8_0_BLOCK * Q8_0_BYTES;
     case EL_Q4_K: return (elements + Q4_K_BLOCK - 1) / Q4_K_BLOCK * Q4_K_BYTES;
+    case EL_Q6_K: return (elements + Q6_K_BLOCK - 1) / Q6_K_BLOCK * Q6_K_BYTES;
     case EL_F16: return elements * 2;
     case EL_F32: return elements * 4;
     default: return 0;
@@ -326,6 +404,24 @@ static float run_dot(int element, const uint8_t *w_row, uint32_t k0, const float
             uint8_t byte = field[16 + group * 32 + at];
             uint32_t quant = seat ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f);
             total = total + x[k0 + at] * (scale * (float)quant - min);
+        }
+        return total;
+    }
+    if (element == EL_Q6_K) { /* crates/neura-kernel/src/dot.rs:663-797: weight = (d * scale) * (code - 32), one scale per 16 */
+        const uint8_t *field = w_row + (size_t)(k0 / Q6_K_BLOCK) * Q6_K_BYTES;
+        uint32_t within = k0 % Q6_K_BLOCK;
+        uint32_t side = within / 128u, group = (within % 128u) / SUB_BLOCK;
+        uint16_t h;
+        memcpy(&h, field + 208, 2);
+        float width = oracle_f16_to_f32(h);
+        float lower = width * (float)(int8_t)field[192 + side * 8 + group * 2];
+        float upper = width * (float)(int8_t)field[192 + side * 8 + group * 2 + 1];
+        for (uint32_t at = 0; at < last; at++) {
+            uint8_t byte = field[side * 64 + (group % 2) * 32 + at];
+            uint32_t nibble = group >= 2 ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f);
+            uint32_t quant = nibble | (((uint32_t)(field[128 + side * 32 + at] >> (2 * group)) & 3u) << 4);
+            float weight = at >= 16 ? upper : lower;
+            total = total + x[k0 + at] * (weight * ((float)quant - 32.0f));
         }
         return total;
     }
@@ -377,7 +473,7 @@ static float folded_dot(int element, const uint8_t *w_row, uint32_t K, const flo
 /* y[r][n] = Σ_k x[r][k]·W[n][k], W row-major [N][K] in `element` storage, order as above.
  * threads > 1 splits the N loop (every output keeps its own serial order). */
 int oracle_gemv(int element, const uint8_t *W, uint32_t N, uint32_t K, const float *x, uint32_t rows, float *y, int threads) {
-    if (element != EL_Q8_0 && element != EL_Q4_K && element != EL_F16 && element != EL_F32) return -2;
+    if (element != EL_Q8_0 && element != EL_Q4_K && element != EL_Q6_K && element != EL_F16 && element != EL_F32) return -2;
     size_t stride = row_bytes(element, K);
     (void)threads;
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)

@@ -10,7 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 LIBRARY = os.path.join(ORACLE_DIR, "libneura_oracle.so")
 
-EL_F32, EL_F16, EL_Q8_0, EL_Q4_K = 0, 1, 8, 12
+EL_F32, EL_F16, EL_Q8_0, EL_Q4_K, EL_Q6_K = 0, 1, 8, 12, 14
 
 
 class OracleModel(ctypes.Structure):

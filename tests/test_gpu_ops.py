@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle
-from neura_amd import NH_Q4_K, NH_Q8_0, NeuraError, synth
+from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -27,7 +27,7 @@ def tight(got, want, scale=1e-5):
 
 # ------------------------------------------------------------------ codecs
 
-@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K, NH_Q6_K])
 def test_dequant_is_bit_exact(device, element):
     rng = np.random.default_rng(100 + element)
     elements = 256 * 4000
@@ -59,7 +59,7 @@ def test_convert_half_is_bit_exact(device):
     assert np.array_equal(device.convert_half(values), oracle.f32_to_f16(values))
 
 
-@pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536)])
+@pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536), (NH_Q6_K, 768)])
 def test_gather_is_the_dequantised_row_times_mask(device, element, width):
     rng = np.random.default_rng(102)
     vocab = 50
@@ -176,6 +176,35 @@ def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device
     assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
 
 
+@pytest.mark.parametrize("N,K,rows", [(2, 256, 1), (7, 512, 3), (272, 3584, 1), (64, 1536, 8), (32, 18944, 1), (33, 18944, 5), (1040, 768, 2)])
+def test_q6_k_products(device, N, K, rows):
+    """Q6_K rows start on 2-byte boundaries (210-byte blocks): every alignment of a row, odd row counts, rows deeper than
+    one LDS stage (K slices folded by a second kernel), 1..8 activation rows, plain, residual and SwiGLU."""
+    rng = np.random.default_rng(N + K + rows)
+    raw = synth.q6_k_random(rng, N * K)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    r = rng.standard_normal((rows, N)).astype(np.float32)
+    plain = oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8)
+    exact = oracle.unpack(NH_Q6_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+    got = device.gemv(NH_Q6_K, raw, N, K, x)
+    close(got, plain)
+    tight(got, plain, 3e-6)
+    assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * max(1.0, np.abs(exact).max()))
+    tight(device.gemv(NH_Q6_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    if N % 2 == 0:
+        gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2:].astype(np.float64)
+        want = gate / (1.0 + np.exp(-gate)) * up
+        close(device.gemv(NH_Q6_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+
+
+def test_q6_k_product_reads_packed_weights_and_fuses_the_norm(device):
+    rng = np.random.default_rng(14)
+    N, K = 96, 2048
+    raw = oracle.pack(NH_Q6_K, np.abs(oracle.random(N * K, 23)))  # the reference's packing keeps non-negative values
+    x = oracle.random(K, 29).reshape(1, K)
+    tight(device.gemv(NH_Q6_K, raw, N, K, x), oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8), 2e-6)
+
+
 def test_gemv_is_linear_and_matches_at_full_size(device):
     # size-independent properties at the 7B FFN shape: W(a x + b z) = a W x + b W z
     rng = np.random.default_rng(6)
@@ -214,7 +243,8 @@ def test_reference_wide_product_test(device, element):
 
 
 @pytest.mark.parametrize("element,M,N,K,half", [(NH_Q4_K, 70, 130, 512, True), (NH_Q4_K, 512, 256, 3584, True), (NH_Q4_K, 33, 64, 256, False),
-                                                (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True)])
+                                                (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q6_K, 70, 130, 512, False),
+                                                (NH_Q6_K, 40, 64, 3584, True)])
 def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
     rng = np.random.default_rng(M + N + K)
     raw = synth.RANDOM[element](rng, N * K)

@@ -104,7 +104,42 @@ def test_q4_k_unpack_hand_built_block():
     assert got[32] == np.float32(0.5 * (s[1] & 63)) * np.float32(raw[16] >> 4) - np.float32(0.25 * (s[5] & 63))
 
 
-@pytest.mark.parametrize("element", [8, 12])
+def test_q6_k_unpack_hand_built_block():
+    # one super-block whose element e carries code (7 e + 3) % 64 and whose sub-block s carries scale 5 s - 40, packed
+    # here by ggml's published layout (crates/neura-precision/src/ggml.rs:394-407 reads it back)
+    raw = np.zeros(210, dtype=np.uint8)
+    codes = [(7 * e + 3) % 64 for e in range(256)]
+    scales = [5 * s - 40 for s in range(16)]
+    for e, code in enumerate(codes):
+        half, group, seat = e // 128, (e % 128) // 32, e % 32
+        at = half * 64 + (group % 2) * 32 + seat
+        raw[at] |= (code & 15) << (4 if group >= 2 else 0)
+        raw[128 + half * 32 + seat] |= (code >> 4) << (2 * group)
+    raw[192:208] = np.array(scales, dtype=np.int8).view(np.uint8)
+    raw[208:210] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    got = oracle.unpack(oracle.EL_Q6_K, raw, 256)
+    want = np.array([np.float32(np.float32(0.25) * np.float32(scales[e // 16])) * np.float32(codes[e] - 32) for e in range(256)], dtype=np.float32)
+    assert np.array_equal(got, want)
+
+
+def test_q6_k_pack_invariants():
+    # non-negative values survive within a step and a half of their sub-block (step = largest / 32, the largest itself
+    # clamps to code 31, the int8 sub-scale rounds the step by up to a percent); the reference's unsigned conversion
+    # (ggml.rs:120-125) drops every negative value to zero, and the restatement keeps that
+    rng = np.random.default_rng(11)
+    values = np.abs(rng.normal(0, 1, 256 * 40)).astype(np.float32)
+    raw = oracle.pack(oracle.EL_Q6_K, values)
+    assert raw.size == 40 * 210 == oracle.lib().oracle_payload_bytes(14, 256 * 40)
+    back = oracle.unpack(oracle.EL_Q6_K, raw, values.size)
+    step = np.abs(values).reshape(-1, 16).max(axis=1) / 32.0
+    error = np.abs(back - values).reshape(-1, 16).max(axis=1)
+    assert np.all(error <= step * 1.5)
+    assert np.median(error / step) < 1.05  # the largest of sixteen draws usually sits on the clamped code
+    negative = oracle.unpack(oracle.EL_Q6_K, oracle.pack(oracle.EL_Q6_K, -values), values.size)
+    assert np.all(negative == 0.0)
+
+
+@pytest.mark.parametrize("element", [8, 12, 14])
 def test_unpack_matches_the_numpy_restatement_on_random_blocks(element):
     rng = np.random.default_rng(3 + element)
     elements = 256 * 300
@@ -152,6 +187,7 @@ def test_block_geometry():
     # crates/neura-abi/tests/layout.rs:147-158
     assert oracle.lib().oracle_payload_bytes(8, 32) == 34
     assert oracle.lib().oracle_payload_bytes(12, 256) == 144
+    assert oracle.lib().oracle_payload_bytes(14, 256) == 210
     assert oracle.lib().oracle_payload_bytes(8, 4864 * 896) == 4630528
     assert oracle.lib().oracle_payload_bytes(12, 46792704) == 26320896
     assert oracle.lib().oracle_payload_bytes(12, 512 * 0 + 3584 * 18944) == 38191104
