@@ -28,7 +28,8 @@ class ModelConfig(ctypes.Structure):
 class TensorTable(ctypes.Structure):
     _fields_ = [("matrix_element", c_int32), ("token_embd", c_uint64), ("output", c_uint64), ("output_norm", c_uint64)] + \
                [(name, POINTER(c_uint64)) for name in
-                ("attn_norm", "attn_q", "attn_k", "attn_v", "attn_output", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down")]
+                ("attn_norm", "attn_q", "attn_k", "attn_v", "attn_output", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down")] + \
+               [("matrix_elements", POINTER(c_int32))] + [(name, POINTER(c_uint64)) for name in ("attn_q_bias", "attn_k_bias", "attn_v_bias")]
 
 
 # name -> (restype, argtypes); the single list of what the header declares

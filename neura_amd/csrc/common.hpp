@@ -120,6 +120,7 @@ struct GemvArgs {
     const float *norm_w;
     float eps;
     const RopeFusion *rope = nullptr;  // only where gemv_fuses_rope() says so
+    const float *bias[3] = {nullptr, nullptr, nullptr};  // one per stacked matrix, added before the rotation: only together with `rope`
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
 // whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)
@@ -167,6 +168,8 @@ int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t po
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
                            const uint8_t *mask, float base);
+
+int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n);
 
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
                       uint32_t count, uint32_t batch, const uint8_t *mask, float *out);

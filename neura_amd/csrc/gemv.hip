@@ -39,6 +39,7 @@ struct GemvParams {
     uint16_t *rope_k, *rope_v;
     uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity;
     uint32_t *refusal;
+    const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
 };
 
 // skewed LDS index of activation i: 4 floats of padding per 64 keep 128-bit reads of
@@ -408,10 +409,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
             if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(total) * up;
         } else if (ROPE) {
             // lanes 0 and 1 hold channels c and c + width/2 of one head (crates/neura-kernel/src/task/rope.rs:95-122)
+            const uint32_t half = p.rope_width >> 1, pair = min(i, p.N - 1u) >> 1, c = pair % half;
+            const uint32_t n = (pair / half) * p.rope_width + c + (i & 1u) * half;
+            if (u < R && i < p.N) {
+                // the projection's bias, if it has one, comes before the rotation
+                const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
+                const uint32_t e0 = p.end[0], e1 = p.end[1];
+                const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
+                const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
+                if (bias) total += bias[n - before];
+            }
             const float other = dpp<DPP_QUAD_XOR1>(total);
             if (u < R && i < p.N) {
-                const uint32_t half = p.rope_width >> 1, pair = i >> 1, c = pair % half;
-                const uint32_t n = (pair / half) * p.rope_width + c + (i & 1u) * half;
                 const uint32_t position = p.rope_cursor[0];
                 float value = total;
                 if (n < p.rope_k_rows) {
@@ -1300,6 +1309,9 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
         p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
         p.refusal = d->refusal;
+        for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
+    } else if (a.bias[0] || a.bias[1] || a.bias[2]) {
+        return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
     }
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     const bool q4 = a.element == NH_Q4_K;
@@ -1598,6 +1610,7 @@ static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, 
 
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
+    if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
     if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;

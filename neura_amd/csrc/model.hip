@@ -19,6 +19,9 @@ struct nh_model {
     const float *output_norm = nullptr;
     std::vector<const float *> attn_norm, ffn_norm;
     std::vector<const uint8_t *> attn_q, attn_k, attn_v, attn_o, ffn_gate, ffn_up, ffn_down;
+    // the element of every matrix: [token_embd, output, then per layer q, k, v, o, gate, up, down]
+    std::vector<int32_t> elements;
+    std::vector<const float *> bias_q, bias_k, bias_v;  // per layer, nullptr where a projection has none
     std::vector<uint16_t *> cache_k, cache_v;
     size_t cache_elements = 0;  // per layer and per K or V
     // activations; T = rows * batch flattened token rows, t = row * batch + plane
@@ -80,9 +83,12 @@ const uint32_t *dev_tokens(const nh_model *m) { return m->inputs_dev; }
 const uint32_t *dev_cursor(const nh_model *m) { return m->inputs_dev + m->max_tokens; }
 const uint8_t *dev_mask(const nh_model *m) { return reinterpret_cast<const uint8_t *>(m->inputs_dev + m->max_tokens + m->c.batch); }
 
-GemvArgs narrow(const nh_model *m, const uint8_t *W, uint32_t N, uint32_t K, const float *x, uint32_t rows, float *y) {
+enum { EMBD = 0, HEAD = 1, Q = 0, K_ = 1, V = 2, O = 3, GATE = 4, UP = 5, DOWN = 6 };
+int32_t element_at(const nh_model *m, uint32_t layer, int which) { return m->elements[2 + 7 * layer + which]; }
+
+GemvArgs narrow(const nh_model *m, int32_t element, const uint8_t *W, uint32_t N, uint32_t K, const float *x, uint32_t rows, float *y) {
     GemvArgs a{};
-    a.element = m->element;
+    a.element = element;
     a.W[0] = W, a.W[1] = nullptr, a.W[2] = nullptr;
     a.end[0] = a.end[1] = a.end[2] = N;
     a.N = N, a.K = K, a.x = x, a.rows = rows, a.y = y;
@@ -98,7 +104,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
     const uint8_t *mask = any_inactive ? dev_mask(m) : nullptr;
     const bool wide = T > 8;  // more rows than the narrow product takes
     int32_t status;
-    if (!products_only && (status = launch_gather(d, m->element, m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK)
+    if (!products_only && (status = launch_gather(d, m->elements[EMBD], m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK)
         return status;
     const float scale = 1.0f / sqrtf((float)hd);
     for (uint32_t L = 0; L < c.layers; L++) {
@@ -106,25 +112,45 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         if (wide) {
             if ((status = launch_rmsnorm(d, m->h, nullptr, m->attn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
             const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
+            const float *biases[3] = {m->bias_q[L], m->bias_k[L], m->bias_v[L]};
             const uint32_t widths[3] = {QW, KW, KW};
             uint32_t column = 0;
             for (int s = 0; s < 3; s++) {
-                GemmArgs g{m->element, mats[s], widths[s], H, m->xn, NH_F32, T, m->qkv + column, nullptr, QKV};
+                GemmArgs g{element_at(m, L, Q + s), mats[s], widths[s], H, m->xn, NH_F32, T, m->qkv + column, nullptr, QKV};
                 if ((status = launch_gemm(d, g)) != NH_OK) return status;
+                if (biases[s] && (status = launch_columns(d, m->qkv + column, QKV, biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
                 column += widths[s];
             }
         } else {
-            GemvArgs a = narrow(m, m->attn_q[L], QKV, H, m->h, T, m->qkv);
+            const bool biased = m->bias_q[L] || m->bias_k[L] || m->bias_v[L];
+            const bool alike = element_at(m, L, Q) == element_at(m, L, K_) && element_at(m, L, Q) == element_at(m, L, V);
+            GemvArgs a = narrow(m, element_at(m, L, Q), m->attn_q[L], QKV, H, m->h, T, m->qkv);
             a.W[1] = m->attn_k[L], a.W[2] = m->attn_v[L];
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
-            // one token of one active plane: the rotation and the cache append ride in the product's epilogue
+            // one token of one active plane: the rotation, the biases and the cache append ride in the product's epilogue
             RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
-            if (!products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
+            if (alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
+                a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];
                 roped = true;
             }
-            if ((status = launch_gemv(d, a)) != NH_OK) return status;
+            if (roped || (alike && (!biased || products_only))) {
+                if ((status = launch_gemv(d, a)) != NH_OK) return status;
+            } else {
+                // matrices of different elements, or biases outside the folded rotation: one product each, placed side by side
+                const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
+                const float *biases[3] = {m->bias_q[L], m->bias_k[L], m->bias_v[L]};
+                const uint32_t widths[3] = {QW, KW, KW};
+                uint32_t column = 0;
+                for (int s = 0; s < 3; s++) {
+                    GemvArgs one = narrow(m, element_at(m, L, Q + s), mats[s], widths[s], H, m->h, T, m->xn);
+                    one.norm_w = m->attn_norm[L], one.eps = c.eps;
+                    if ((status = launch_gemv(d, one)) != NH_OK) return status;
+                    if ((status = launch_columns(d, m->xn, widths[s], products_only ? nullptr : biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
+                    column += widths[s];
+                }
+            }
         }
         if (!products_only && !roped && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
                                                            m->capacity, m->window, dev_cursor(m), mask, c.rope_base)) != NH_OK)
@@ -138,26 +164,35 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
         if (!products_only && (status = launch_attention(d, at)) != NH_OK) return status;
         if (wide) {
-            GemmArgs o{m->element, m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
+            GemmArgs o{element_at(m, L, O), m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
             if ((status = launch_gemm(d, o)) != NH_OK) return status;
             if ((status = launch_rmsnorm(d, m->h, nullptr, m->ffn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
-            GemmArgs g{m->element, m->ffn_gate[L], F, H, m->xn, NH_F32, T, m->act, nullptr, F};
-            GemmArgs u{m->element, m->ffn_up[L], F, H, m->xn, NH_F32, T, m->up, nullptr, F};
+            GemmArgs g{element_at(m, L, GATE), m->ffn_gate[L], F, H, m->xn, NH_F32, T, m->act, nullptr, F};
+            GemmArgs u{element_at(m, L, UP), m->ffn_up[L], F, H, m->xn, NH_F32, T, m->up, nullptr, F};
             if ((status = launch_gemm(d, g)) != NH_OK) return status;
             if ((status = launch_gemm(d, u)) != NH_OK) return status;
             if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
-            GemmArgs dn{m->element, m->ffn_down[L], H, F, m->act, NH_F32, T, m->h, m->h, H};
+            GemmArgs dn{element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, NH_F32, T, m->h, m->h, H};
             if ((status = launch_gemm(d, dn)) != NH_OK) return status;
         } else {
-            GemvArgs o = narrow(m, m->attn_o[L], H, QW, m->att, T, m->h);
+            GemvArgs o = narrow(m, element_at(m, L, O), m->attn_o[L], H, QW, m->att, T, m->h);
             o.residual = m->h;
             if ((status = launch_gemv(d, o)) != NH_OK) return status;
-            GemvArgs gu = narrow(m, m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
-            gu.W[1] = m->ffn_up[L];
-            gu.end[0] = F, gu.end[1] = gu.end[2] = 2 * F;
-            gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
-            if ((status = launch_gemv(d, gu)) != NH_OK) return status;
-            GemvArgs dn = narrow(m, m->ffn_down[L], H, F, m->act, T, m->h);
+            if (element_at(m, L, GATE) == element_at(m, L, UP)) {
+                GemvArgs gu = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
+                gu.W[1] = m->ffn_up[L];
+                gu.end[0] = F, gu.end[1] = gu.end[2] = 2 * F;
+                gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
+                if ((status = launch_gemv(d, gu)) != NH_OK) return status;
+            } else {
+                GemvArgs g = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], F, H, m->h, T, m->act);
+                GemvArgs u = narrow(m, element_at(m, L, UP), m->ffn_up[L], F, H, m->h, T, m->up);
+                g.norm_w = u.norm_w = m->ffn_norm[L], g.eps = u.eps = c.eps;
+                if ((status = launch_gemv(d, g)) != NH_OK) return status;
+                if ((status = launch_gemv(d, u)) != NH_OK) return status;
+                if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
+            }
+            GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
             dn.residual = m->h;
             if ((status = launch_gemv(d, dn)) != NH_OK) return status;
         }
@@ -171,7 +206,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
 int32_t decode_kernels(nh_model *m, bool any_inactive) {
     int32_t status;
     if ((status = forward(m, 1, any_inactive)) != NH_OK) return status;
-    GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+    GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
     head.norm_w = m->output_norm, head.eps = m->c.eps;
     if ((status = launch_gemv(m->d, head)) != NH_OK) return status;
     return launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
@@ -193,14 +228,18 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
              c.layers, c.hidden, c.heads, c.kv_heads, c.head_dim, c.ffn, c.vocab, c.context, c.batch);
         return nullptr;
     }
-    if (table->matrix_element != NH_Q8_0 && table->matrix_element != NH_Q4_K) {
-        fail(NH_E_ARGUMENT, "a decoder multiplies Q8_0 or Q4_K matrices, and this table names element %d", table->matrix_element);
-        return nullptr;
-    }
-    uint32_t block = block_elements(table->matrix_element);
-    if (c.hidden % block || c.ffn % block || (c.heads * c.head_dim) % block) {
-        fail(NH_E_ARGUMENT, "rows of %u, %u and %u numbers are not whole blocks of %u", c.hidden, c.ffn, c.heads * c.head_dim, block);
-        return nullptr;
+    std::vector<int32_t> elements(2 + 7 * (size_t)c.layers, table->matrix_element);
+    if (table->matrix_elements) elements.assign(table->matrix_elements, table->matrix_elements + elements.size());
+    for (int32_t element : elements) {
+        if (element != NH_Q8_0 && element != NH_Q4_K && element != NH_Q6_K) {
+            fail(NH_E_ARGUMENT, "a decoder multiplies Q8_0, Q4_K or Q6_K matrices, and this table names element %d", element);
+            return nullptr;
+        }
+        uint32_t block = block_elements(element);
+        if (c.hidden % block || c.ffn % block || (c.heads * c.head_dim) % block) {
+            fail(NH_E_ARGUMENT, "rows of %u, %u and %u numbers are not whole blocks of %u", c.hidden, c.ffn, c.heads * c.head_dim, block);
+            return nullptr;
+        }
     }
     if (!(c.rope_base > 1.0f) || !std::isfinite(c.rope_base)) {  // refusal::KNOB, crates/neura-kernel/src/task/rope.rs:33-36
         fail(NH_E_ARGUMENT, "a rope base of %f turns nothing", (double)c.rope_base);
@@ -208,6 +247,7 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     }
     nh_model *m = new nh_model();
     m->d = device, m->weights = weights, m->c = c, m->element = table->matrix_element;
+    m->elements = elements;
     uint32_t widest = c.max_rows ? c.max_rows : 1;
     m->window = c.context;               // crates/neura-generate/src/batch.rs:314
     m->capacity = c.context + widest;    // crates/neura-generate/src/batch.rs:323-325
@@ -222,11 +262,11 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         return static_cast<const uint8_t *>(nh_weights_at(weights, offset));
     };
     const uint32_t H = c.hidden, QW = c.heads * c.head_dim, KW = c.kv_heads * c.head_dim, F = c.ffn;
-    auto matrix_bytes = [&](uint64_t n, uint64_t k) { return n * payload_bytes(m->element, k); };
+    auto matrix_bytes = [&](int32_t element, uint64_t n, uint64_t k) { return n * payload_bytes(element, k); };
     bool ok = true;
-    ok = ok && (m->token_embd = at(table->token_embd, matrix_bytes(c.vocab, H), "token_embd.weight"));
+    ok = ok && (m->token_embd = at(table->token_embd, matrix_bytes(elements[EMBD], c.vocab, H), "token_embd.weight"));
     m->output = m->token_embd;  // tied head unless the table names one (examples/qwen/model.rs:81-84)
-    if (ok && table->output != UINT64_MAX) ok = (m->output = at(table->output, matrix_bytes(c.vocab, H), "output.weight")) != nullptr;
+    if (ok && table->output != UINT64_MAX) ok = (m->output = at(table->output, matrix_bytes(elements[HEAD], c.vocab, H), "output.weight")) != nullptr;
     ok = ok && (m->output_norm = reinterpret_cast<const float *>(at(table->output_norm, (uint64_t)H * 4, "output_norm.weight")));
     for (uint32_t L = 0; ok && L < c.layers; L++) {
         const uint8_t *p;
@@ -234,20 +274,32 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         if (ok) m->attn_norm.push_back(reinterpret_cast<const float *>(p));
         ok = ok && (p = at(table->ffn_norm[L], (uint64_t)H * 4, "ffn_norm.weight"));
         if (ok) m->ffn_norm.push_back(reinterpret_cast<const float *>(p));
-        ok = ok && (p = at(table->attn_q[L], matrix_bytes(QW, H), "attn_q.weight"));
+        ok = ok && (p = at(table->attn_q[L], matrix_bytes(element_at(m, L, Q), QW, H), "attn_q.weight"));
         if (ok) m->attn_q.push_back(p);
-        ok = ok && (p = at(table->attn_k[L], matrix_bytes(KW, H), "attn_k.weight"));
+        ok = ok && (p = at(table->attn_k[L], matrix_bytes(element_at(m, L, K_), KW, H), "attn_k.weight"));
         if (ok) m->attn_k.push_back(p);
-        ok = ok && (p = at(table->attn_v[L], matrix_bytes(KW, H), "attn_v.weight"));
+        ok = ok && (p = at(table->attn_v[L], matrix_bytes(element_at(m, L, V), KW, H), "attn_v.weight"));
         if (ok) m->attn_v.push_back(p);
-        ok = ok && (p = at(table->attn_output[L], matrix_bytes(H, QW), "attn_output.weight"));
+        ok = ok && (p = at(table->attn_output[L], matrix_bytes(element_at(m, L, O), H, QW), "attn_output.weight"));
         if (ok) m->attn_o.push_back(p);
-        ok = ok && (p = at(table->ffn_gate[L], matrix_bytes(F, H), "ffn_gate.weight"));
+        ok = ok && (p = at(table->ffn_gate[L], matrix_bytes(element_at(m, L, GATE), F, H), "ffn_gate.weight"));
         if (ok) m->ffn_gate.push_back(p);
-        ok = ok && (p = at(table->ffn_up[L], matrix_bytes(F, H), "ffn_up.weight"));
+        ok = ok && (p = at(table->ffn_up[L], matrix_bytes(element_at(m, L, UP), F, H), "ffn_up.weight"));
         if (ok) m->ffn_up.push_back(p);
-        ok = ok && (p = at(table->ffn_down[L], matrix_bytes(H, F), "ffn_down.weight"));
+        ok = ok && (p = at(table->ffn_down[L], matrix_bytes(element_at(m, L, DOWN), H, F), "ffn_down.weight"));
         if (ok) m->ffn_down.push_back(p);
+        const uint64_t *bias_tables[3] = {table->attn_q_bias, table->attn_k_bias, table->attn_v_bias};
+        std::vector<const float *> *held[3] = {&m->bias_q, &m->bias_k, &m->bias_v};
+        const uint32_t bias_rows[3] = {QW, KW, KW};
+        const char *bias_names[3] = {"attn_q.bias", "attn_k.bias", "attn_v.bias"};
+        for (int s = 0; ok && s < 3; s++) {
+            const float *bias = nullptr;
+            if (bias_tables[s] && bias_tables[s][L] != UINT64_MAX) {
+                ok = (p = at(bias_tables[s][L], (uint64_t)bias_rows[s] * 4, bias_names[s])) != nullptr;
+                bias = reinterpret_cast<const float *>(p);
+            }
+            held[s]->push_back(bias);
+        }
     }
     if (!ok) {
         release(m);
@@ -260,8 +312,8 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     }
     const size_t T = m->max_tokens;
     m->cache_elements = (size_t)c.kv_heads * c.batch * m->capacity * c.head_dim;
-    ok = device_array(m->h, T * H) && device_array(m->xn, T * H) && device_array(m->qkv, T * (QW + 2 * KW)) &&
-         device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T > 8 ? T * F : 1) &&
+    ok = device_array(m->h, T * H) && device_array(m->xn, T * (H > QW ? H : QW)) && device_array(m->qkv, T * (QW + 2 * KW)) &&
+         device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T * F) &&
          device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 2 * c.batch + 4) &&
          device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->capacity * (c.head_dim / 2)) &&
          device_array(m->rope_sin, (size_t)m->capacity * (c.head_dim / 2));
@@ -393,7 +445,7 @@ int32_t nh_model_time_products(nh_model *m, uint32_t steps, double *seconds_out,
     if ((status = nh_profile_begin(d)) != NH_OK) return status;
     status = forward(m, 1, false, true);
     if (status == NH_OK) {
-        GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+        GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
         head.norm_w = m->output_norm, head.eps = m->c.eps;
         status = launch_gemv(d, head);
     }
@@ -404,7 +456,7 @@ int32_t nh_model_time_products(nh_model *m, uint32_t steps, double *seconds_out,
     if ((status = nh_timer_start(d)) != NH_OK) return status;
     for (uint32_t step = 0; step < steps; step++) {
         if ((status = forward(m, 1, false, true)) != NH_OK) return status;
-        GemvArgs head = narrow(m, m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
+        GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
         head.norm_w = m->output_norm, head.eps = m->c.eps;
         if ((status = launch_gemv(d, head)) != NH_OK) return status;
     }

@@ -205,6 +205,24 @@ int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv
 }
 
 // silu(gate) * up (examples/qwen/mlp.rs:33; crates/neura-pointwise/src/op.rs:163)
+// dst[r][c] = src[r][c] + bias[c]: places the columns of one projection in a wider row, or adds a bias where it stands
+__global__ __launch_bounds__(256) void columns_kernel(const float *__restrict__ src, uint32_t lds, const float *__restrict__ bias,
+                                                      float *__restrict__ dst, uint32_t ldd, uint32_t rows, uint32_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (uint64_t)rows * n; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t r = (uint32_t)(i / n), c = (uint32_t)(i % n);
+        const float value = src[(size_t)r * lds + c];
+        dst[(size_t)r * ldd + c] = bias ? value + bias[c] : value;
+    }
+}
+
+int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n) {
+    if (!rows || !n) return NH_OK;
+    const uint64_t wanted = ((uint64_t)rows * n + 255) / 256, most = (uint64_t)d->compute_units * 8;
+    hipLaunchKernelGGL(columns_kernel, dim3((uint32_t)(wanted < most ? wanted : most)), dim3(256), 0, d->stream, src, lds, bias, dst, ldd, rows, n);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float *__restrict__ gate, const float *__restrict__ up, uint64_t n,
                                                        float *__restrict__ out) {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {

@@ -12,6 +12,7 @@ from ._abi import ModelConfig, TensorTable, UINT64_MAX
 
 ALIGNMENT = 256
 LAYER_TENSORS = ("attn_norm", "attn_q", "attn_k", "attn_v", "attn_output", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down")
+MATRICES = ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")
 
 
 def _check(status):
@@ -71,6 +72,19 @@ class Model:
             array = (ctypes.c_uint64 * L)(*[weights.offsets["blk.%d.%s.weight" % (i, name)] for i in range(L)])
             self._arrays.append(array)
             setattr(table, name, ctypes.cast(array, ctypes.POINTER(ctypes.c_uint64)))
+        # every matrix keeps the element it was stored with (a Q4_K_M file mixes Q4_K and Q6_K); Qwen2's q/k/v biases ride along
+        names = ["token_embd.weight", "output.weight"] + ["blk.%d.%s.weight" % (i, n) for i in range(L) for n in MATRICES]
+        held = [weights.elements.get(n, element) for n in names]
+        if any(e != element for e in held):
+            array = (ctypes.c_int32 * len(held))(*held)
+            self._arrays.append(array)
+            table.matrix_elements = ctypes.cast(array, ctypes.POINTER(ctypes.c_int32))
+        for which in ("q", "k", "v"):
+            offsets = [weights.offsets.get("blk.%d.attn_%s.bias" % (i, which), UINT64_MAX) for i in range(L)]
+            if any(o != UINT64_MAX for o in offsets):
+                array = (ctypes.c_uint64 * L)(*offsets)
+                self._arrays.append(array)
+                setattr(table, "attn_%s_bias" % which, ctypes.cast(array, ctypes.POINTER(ctypes.c_uint64)))
         self.handle = self.lib.nh_model_create(device.handle, ctypes.byref(self.config), weights.handle, ctypes.byref(table))
         if not self.handle:
             from . import NeuraError

@@ -143,7 +143,36 @@ def q4_k_quantize(values):
     return raw.reshape(-1)
 
 
-QUANTIZE = {8: q8_0_quantize, 12: q4_k_quantize}
+def q6_k_quantize(values):
+    """Symmetric 6-bit codes in ggml's Q6_K layout: per 16 elements a step of largest / 31, int8 sub-scales against a
+    super scale of largest step / 127, codes round(x / step) + 32.  (Test data only: the reference's own Q6_K packer,
+    ggml.rs:352-392, keeps non-negative values alone, which no model's weights are.)"""
+    f32 = np.float32
+    x = np.asarray(values, dtype=f32).reshape(-1, 16, 16)
+    steps = (np.abs(x).max(axis=2) / f32(31)).astype(f32)                      # [blocks, 16]
+    d = (steps.max(axis=1, keepdims=True) / f32(127)).astype(f32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sc = np.where(d == 0, f32(0), steps / d)
+    sc = np.clip(_round_away(sc.astype(f32)), 0, 127).astype(np.int8)
+    d16 = d.astype(np.float16)
+    step = (d16.astype(f32) * sc.astype(f32)).astype(f32)[:, :, None]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(step == 0, f32(0), x / step)
+    codes = (np.clip(_round_away(q.astype(f32)), -32, 31) + 32).astype(np.uint8).reshape(-1, 2, 4, 32)  # [blocks, half, group, l]
+    raw = np.zeros((codes.shape[0], Q6_K_BYTES), dtype=np.uint8)
+    low = codes & 0x0F
+    ql = np.empty((codes.shape[0], 2, 2, 32), dtype=np.uint8)
+    ql[:, :, 0, :] = low[:, :, 0, :] | (low[:, :, 2, :] << 4)
+    ql[:, :, 1, :] = low[:, :, 1, :] | (low[:, :, 3, :] << 4)
+    raw[:, 0:128] = ql.reshape(-1, 128)
+    high = codes >> 4
+    raw[:, 128:192] = (high[:, :, 0, :] | (high[:, :, 1, :] << 2) | (high[:, :, 2, :] << 4) | (high[:, :, 3, :] << 6)).reshape(-1, 64)
+    raw[:, 192:208] = sc.view(np.uint8)
+    raw[:, 208:210] = d16.view(np.uint8).reshape(-1, 2)
+    return raw.reshape(-1)
+
+
+QUANTIZE = {8: q8_0_quantize, 12: q4_k_quantize, 14: q6_k_quantize}
 RANDOM = {8: q8_0_random, 12: q4_k_random, 14: q6_k_random}
 DEQUANT = {8: q8_0_dequant, 12: q4_k_dequant, 14: q6_k_dequant}
 BLOCK_BYTES = {8: (Q8_0_BLOCK, Q8_0_BYTES), 12: (Q4_K_BLOCK, Q4_K_BYTES), 14: (Q6_K_BLOCK, Q6_K_BYTES)}
@@ -171,8 +200,11 @@ def layer_matrices(shape):
             ("ffn_down", H, F)]
 
 
-def model_tensors(shape, element, rng, mode="blocks", layers=None):
+def model_tensors(shape, element, rng, mode="blocks", layers=None, elements=None, biases=()):
     """Yields (name, element, dims (GGUF order: K first), raw bytes) of a random-init decoder.
+
+    `elements`: name -> element of the matrices stored otherwise than `element` (a Q4_K_M file keeps some in Q6_K);
+    `biases`: layers whose q, k and v projections carry an fp32 bias (Qwen2 checkpoints do).
 
     mode "blocks": matrices are random raw blocks (the Q4_K distribution of the GEMV
     configurations); mode "normal": N(0, 0.02) weights quantized with the reference's encoder.
@@ -181,27 +213,35 @@ def model_tensors(shape, element, rng, mode="blocks", layers=None):
     H = shape["hidden"]
     count = shape["layers"] if layers is None else layers
 
-    def matrix(rows, columns):
+    elements = elements or {}
+
+    def matrix(name, rows, columns):
+        held = elements.get(name, element)
         if mode == "blocks":
-            return RANDOM[element](rng, rows * columns)
-        out = np.empty(matrix_bytes(element, rows, columns), dtype=np.uint8)
+            return held, RANDOM[held](rng, rows * columns)
+        out = np.empty(matrix_bytes(held, rows, columns), dtype=np.uint8)
         step = max(1, (1 << 24) // columns)
-        row_bytes = matrix_bytes(element, 1, columns)
+        row_bytes = matrix_bytes(held, 1, columns)
         for first in range(0, rows, step):
             n = min(step, rows - first)
             values = rng.normal(0.0, 0.02, (n, columns)).astype(np.float32)
-            out[first * row_bytes:(first + n) * row_bytes] = QUANTIZE[element](values)
-        return out
+            out[first * row_bytes:(first + n) * row_bytes] = QUANTIZE[held](values)
+        return held, out
 
     def norm():
         return (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32).view(np.uint8)
 
-    yield "token_embd.weight", element, (H, shape["vocab"]), matrix(shape["vocab"], H)
+    held, raw = matrix("token_embd.weight", shape["vocab"], H)
+    yield "token_embd.weight", held, (H, shape["vocab"]), raw
     for layer in range(count):
         yield "blk.%d.attn_norm.weight" % layer, 0, (H,), norm()
         yield "blk.%d.ffn_norm.weight" % layer, 0, (H,), norm()
         for name, rows, columns in layer_matrices(shape):
-            yield "blk.%d.%s.weight" % (layer, name), element, (columns, rows), matrix(rows, columns)
+            held, raw = matrix("blk.%d.%s.weight" % (layer, name), rows, columns)
+            yield "blk.%d.%s.weight" % (layer, name), held, (columns, rows), raw
+            if layer in biases and name in ("attn_q", "attn_k", "attn_v"):
+                yield "blk.%d.%s.bias" % (layer, name), 0, (rows,), rng.normal(0.0, 0.5, rows).astype(np.float32).view(np.uint8)
     yield "output_norm.weight", 0, (H,), norm()
     if not shape["tied"]:
-        yield "output.weight", element, (H, shape["vocab"]), matrix(shape["vocab"], H)
+        held, raw = matrix("output.weight", shape["vocab"], H)
+        yield "output.weight", held, (H, shape["vocab"]), raw

@@ -716,7 +716,20 @@ typedef struct {
     const float **ffn_norm;
     const uint8_t **ffn_gate, **ffn_up, **ffn_down;
     uint16_t **cache_k, **cache_v; /* [layers] -> f16 [kv_heads][batch][capacity][head_dim] */
+    /* optional (NULL = absent).  matrix_elements: the element of each matrix where they differ -- [token_embd, output, then per
+     * layer attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down].  attn_*_bias [layers] -> f32 [rows] or NULL entries:
+     * Qwen2 checkpoints add a bias to q, k and v before the rotation; the reference's qwen example has none
+     * (examples/qwen/attention.rs:98-154). */
+    const int *matrix_elements;
+    const float **attn_q_bias, **attn_k_bias, **attn_v_bias;
 } oracle_model;
+
+static int element_of(const oracle_model *m, uint32_t slot) { return m->matrix_elements ? m->matrix_elements[slot] : m->matrix_element; }
+static void add_bias(float *y, const float *bias, uint32_t rows, uint32_t n) {
+    if (!bias) return;
+    for (uint32_t r = 0; r < rows; r++)
+        for (uint32_t c = 0; c < n; c++) y[(size_t)r * n + c] = y[(size_t)r * n + c] + bias[c];
+}
 
 /* crates/neura-kernel/src/pointwise.rs:66-68 and neura-pointwise/src/op.rs:163 */
 static float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
@@ -731,8 +744,8 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
                          float *logits_out, uint32_t *chosen_out, int threads) {
     const uint32_t H = m->hidden, B = m->batch, hd = m->head_dim, QW = m->heads * hd, KW = m->kv_heads * hd, F = m->ffn;
     const uint32_t T = rows * B; /* flattened rows: index t = row*B + plane */
-    const int el = m->matrix_element;
-    const size_t embd_stride = row_bytes(el, H);
+    const int el_embd = element_of(m, 0), el_head = m->output ? element_of(m, 1) : element_of(m, 0);
+    const size_t embd_stride = row_bytes(el_embd, H);
     float *h = (float *)calloc((size_t)T * H, 4), *xn = (float *)malloc((size_t)T * H * 4);
     float *q = (float *)malloc((size_t)T * QW * 4), *k = (float *)malloc((size_t)T * KW * 4), *v = (float *)malloc((size_t)T * KW * 4);
     float *qh = (float *)malloc((size_t)T * QW * 4), *att = (float *)malloc((size_t)T * QW * 4), *attj = (float *)malloc((size_t)T * QW * 4);
@@ -742,7 +755,7 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
     for (uint32_t t = 0; t < T; t++) {
         uint32_t b = t % B;
         if (tokens[t] >= m->vocab) return -3; /* refusal::INDEX, select.rs:38 */
-        oracle_unpack(el, m->token_embd + (size_t)tokens[t] * embd_stride, H, tmp);
+        oracle_unpack(el_embd, m->token_embd + (size_t)tokens[t] * embd_stride, H, tmp);
         for (uint32_t c = 0; c < H; c++) h[(size_t)t * H + c] = tmp[c] * (mask[b] ? 1.0f : 0.0f);
     }
     for (uint32_t b = 0; b < B; b++)
@@ -750,9 +763,13 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
     float scale = 1.0f / sqrtf((float)hd);
     for (uint32_t L = 0; L < m->layers; L++) {
         oracle_rmsnorm(h, NULL, m->attn_norm[L], m->eps, T, H, xn, NULL);
-        oracle_gemv(el, m->attn_q[L], QW, H, xn, T, q, threads);
-        oracle_gemv(el, m->attn_k[L], KW, H, xn, T, k, threads);
-        oracle_gemv(el, m->attn_v[L], KW, H, xn, T, v, threads);
+        const uint32_t slot0 = 2 + 7 * L;
+        oracle_gemv(element_of(m, slot0 + 0), m->attn_q[L], QW, H, xn, T, q, threads);
+        oracle_gemv(element_of(m, slot0 + 1), m->attn_k[L], KW, H, xn, T, k, threads);
+        oracle_gemv(element_of(m, slot0 + 2), m->attn_v[L], KW, H, xn, T, v, threads);
+        add_bias(q, m->attn_q_bias ? m->attn_q_bias[L] : NULL, T, QW);
+        add_bias(k, m->attn_k_bias ? m->attn_k_bias[L] : NULL, T, KW);
+        add_bias(v, m->attn_v_bias ? m->attn_v_bias[L] : NULL, T, KW);
         /* heads + as_planes: q [T][heads*hd] -> qh [heads][B][rows][hd], roped at cursor+row */
         for (uint32_t t = 0; t < T; t++) {
             uint32_t row = t / B, b = t % B;
@@ -775,20 +792,20 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
             for (uint32_t head = 0; head < m->heads; head++)
                 memcpy(attj + (size_t)t * QW + head * hd, att + (((size_t)head * B + b) * rows + row) * hd, hd * 4);
         }
-        oracle_gemv(el, m->attn_o[L], H, QW, attj, T, proj, threads);
+        oracle_gemv(element_of(m, slot0 + 3), m->attn_o[L], H, QW, attj, T, proj, threads);
         for (size_t i = 0; i < (size_t)T * H; i++) h[i] = h[i] + proj[i];
         oracle_rmsnorm(h, NULL, m->ffn_norm[L], m->eps, T, H, xn, NULL);
-        oracle_gemv(el, m->ffn_gate[L], F, H, xn, T, g, threads);
-        oracle_gemv(el, m->ffn_up[L], F, H, xn, T, u, threads);
+        oracle_gemv(element_of(m, slot0 + 4), m->ffn_gate[L], F, H, xn, T, g, threads);
+        oracle_gemv(element_of(m, slot0 + 5), m->ffn_up[L], F, H, xn, T, u, threads);
         for (size_t i = 0; i < (size_t)T * F; i++) g[i] = silu(g[i]) * u[i];
-        oracle_gemv(el, m->ffn_down[L], H, F, g, T, proj, threads);
+        oracle_gemv(element_of(m, slot0 + 6), m->ffn_down[L], H, F, g, T, proj, threads);
         for (size_t i = 0; i < (size_t)T * H; i++) h[i] = (h[i] + proj[i]) * (mask[(i / H) % B] ? 1.0f : 0.0f);
     }
     if (logits_out || chosen_out) {
         float *logits = logits_out ? logits_out : (float *)malloc((size_t)B * m->vocab * 4);
         const float *last = h + (size_t)(rows - 1) * B * H;
         oracle_rmsnorm(last, NULL, m->output_norm, m->eps, B, H, xn, NULL);
-        oracle_gemv(el, m->output ? m->output : m->token_embd, m->vocab, H, xn, B, logits, threads);
+        oracle_gemv(el_head, m->output ? m->output : m->token_embd, m->vocab, H, xn, B, logits, threads);
         if (chosen_out)
             for (uint32_t b = 0; b < B; b++) chosen_out[b] = oracle_argmax(logits + (size_t)b * m->vocab, m->vocab);
         if (!logits_out) free(logits);

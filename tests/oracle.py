@@ -20,6 +20,8 @@ class OracleModel(ctypes.Structure):
         ("attn_norm", POINTER(c_void_p)), ("attn_q", POINTER(c_void_p)), ("attn_k", POINTER(c_void_p)), ("attn_v", POINTER(c_void_p)),
         ("attn_o", POINTER(c_void_p)), ("ffn_norm", POINTER(c_void_p)), ("ffn_gate", POINTER(c_void_p)), ("ffn_up", POINTER(c_void_p)),
         ("ffn_down", POINTER(c_void_p)), ("cache_k", POINTER(c_void_p)), ("cache_v", POINTER(c_void_p)),
+        ("matrix_elements", POINTER(c_int)), ("attn_q_bias", POINTER(c_void_p)), ("attn_k_bias", POINTER(c_void_p)),
+        ("attn_v_bias", POINTER(c_void_p)),
     ]
 
 
@@ -173,7 +175,9 @@ def argmax(values):
 class Model:
     """The oracle's decoder over host copies of the same GGUF tensors the device gets."""
 
-    def __init__(self, shape, element, tensors, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None):
+    def __init__(self, shape, element, tensors, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, elements=None):
+        """`elements`: name -> element of the matrices that differ from `element`; tensors named blk.N.attn_{q,k,v}.bias
+        are added to the projections before the rotation."""
         self.keep = []
         L = shape["layers"] if layers is None else layers
         self.capacity, self.window = context + max_rows, context
@@ -199,9 +203,21 @@ class Model:
         m.attn_norm, m.attn_q, m.attn_k, m.attn_v = table("attn_norm"), table("attn_q"), table("attn_k"), table("attn_v")
         m.attn_o, m.ffn_norm = table("attn_output"), table("ffn_norm")
         m.ffn_gate, m.ffn_up, m.ffn_down = table("ffn_gate"), table("ffn_up"), table("ffn_down")
-        elements = shape["kv_heads"] * batch * self.capacity * shape["head_dim"]
-        self.cache_k = [np.zeros(elements, dtype=np.uint16) for _ in range(L)]
-        self.cache_v = [np.zeros(elements, dtype=np.uint16) for _ in range(L)]
+        if elements:
+            names = ["token_embd.weight", "output.weight"] + ["blk.%d.%s.weight" % (i, n) for i in range(L) for n in
+                                                              ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")]
+            held = (c_int * len(names))(*[elements.get(n, element) for n in names])
+            self.keep.append(held)
+            m.matrix_elements = ctypes.cast(held, POINTER(c_int))
+        for which in ("q", "k", "v"):
+            if any("blk.%d.attn_%s.bias" % (i, which) in tensors for i in range(L)):
+                pointers = (c_void_p * L)(*[hold(np.asarray(tensors["blk.%d.attn_%s.bias" % (i, which)], dtype=np.float32))
+                                            if "blk.%d.attn_%s.bias" % (i, which) in tensors else None for i in range(L)])
+                self.keep.append(pointers)
+                setattr(m, "attn_%s_bias" % which, ctypes.cast(pointers, POINTER(c_void_p)))
+        cache_elements = shape["kv_heads"] * batch * self.capacity * shape["head_dim"]
+        self.cache_k = [np.zeros(cache_elements, dtype=np.uint16) for _ in range(L)]
+        self.cache_v = [np.zeros(cache_elements, dtype=np.uint16) for _ in range(L)]
         ks = (c_void_p * L)(*[a.ctypes.data for a in self.cache_k])
         vs = (c_void_p * L)(*[a.ctypes.data for a in self.cache_v])
         self.keep += [ks, vs]

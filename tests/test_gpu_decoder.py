@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 import oracle
-from neura_amd import NH_Q4_K, NH_Q8_0, NeuraError, synth
+from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
 from neura_amd.loader import Model, Weights
 
 pytestmark = pytest.mark.gpu
@@ -78,6 +78,41 @@ def test_masked_planes_and_chunked_fill(device):
     k_single = oracle.f16_to_f32(model.cache_read(0, 0)[:, 0, :16].reshape(-1))
     k_chunk = oracle.f16_to_f32(k[:, 0, :16].reshape(-1))
     assert np.abs(k_single - k_chunk).max() <= 2e-3 * max(1.0, np.abs(k_chunk).max())
+    model.release(), weights.release()
+
+
+MIXED = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.2.ffn_down.weight": NH_Q6_K, "blk.2.ffn_gate.weight": NH_Q6_K}
+
+
+@pytest.mark.parametrize("batch", [1, 2])
+def test_mixed_elements_and_projection_biases(device, batch):
+    """A decoder stored the way Q4_K_M files are (Q6_K for some matrices, Q4_K for the rest) whose q, k and v projections
+    carry Qwen2's biases: layer 0 (a Q6_K value projection, biases) takes one product per matrix, layer 1 (one element,
+    biases) folds rotation and biases into the stacked product at batch 1, layer 2 (gate and up stored differently) runs
+    the two halves apart.  Decode steps, a 16-row fill and the caches against the oracle."""
+    shape = SMALL_Q4
+    rng = np.random.default_rng(21)
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="normal", elements=MIXED, biases=(0, 1)))
+    host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, NH_Q4_K, batch, 40, 16)
+    ref = oracle.Model(shape, NH_Q4_K, host, batch, 40, 16, elements=MIXED)
+    prompt = rng.integers(0, shape["vocab"], (16, batch))
+    model.prefill(prompt.reshape(-1), 16, [0] * batch)
+    ref.forward(prompt.reshape(-1), 16, [0] * batch, want_logits=False)
+    tokens = rng.integers(0, shape["vocab"], batch)
+    for step in range(5):
+        cursors = [16 + step] * batch
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        got = model.decode_step(tokens, cursors)
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens = got
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_cache = oracle.f16_to_f32(model.cache_read(layer, which).reshape(-1))
+            want_cache = oracle.f16_to_f32(held[layer])
+            assert np.abs(got_cache - want_cache).max() <= 2e-3 * max(1.0, np.abs(want_cache).max())
     model.release(), weights.release()
 
 

@@ -122,6 +122,17 @@ def test_q6_k_unpack_hand_built_block():
     assert np.array_equal(got, want)
 
 
+def test_q6_k_symmetric_quantizer_of_the_test_data_round_trips():
+    # synth.q6_k_quantize makes the Q6_K matrices of the synthetic decoders; the oracle reads them back within half a step
+    rng = np.random.default_rng(12)
+    values = rng.normal(0, 0.02, 256 * 50).astype(np.float32)
+    back = oracle.unpack(oracle.EL_Q6_K, synth.q6_k_quantize(values), values.size)
+    step = np.abs(values).reshape(-1, 16).max(axis=1) / 31.0
+    error = np.abs(back - values).reshape(-1, 16).max(axis=1)
+    assert np.all(error <= step * 0.55 + np.abs(values).reshape(-1, 256).max(axis=1).repeat(16) * 2.0 ** -9)
+    assert np.sign(back[np.abs(values) > 0.01]).tolist() == np.sign(values[np.abs(values) > 0.01]).tolist()
+
+
 def test_q6_k_pack_invariants():
     # non-negative values survive within a step and a half of their sub-block (step = largest / 32, the largest itself
     # clamps to code 31, the int8 sub-scale rounds the step by up to a percent); the reference's unsigned conversion
