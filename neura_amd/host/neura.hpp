@@ -817,42 +817,63 @@ class Model {
         const uint32_t H = config.hidden, QW = config.heads * config.head_width, KW = config.key_heads * config.head_width, F = config.feed_forward;
         std::vector<std::string> names;
         // tensor names of a Qwen2 GGUF (the reference's qwen35 example names them alike, examples/qwen/attention.rs:40-78, mlp.rs:22-25)
+        // every matrix keeps the storage the file gives it (a Q4_K_M file mixes q4_k and q6_k); the q, k and v projections of
+        // Qwen2 checkpoints carry biases the reference's own example has no tensors for
         Element element = decoder::matrix(archive, "token_embd.weight", config.vocabulary, H).element;
-        NEURA_ASSERT(element == Element::Q8_0 || element == Element::Q4K,
-                     "this decoder multiplies q8_0 and q4_k matrices, and token_embd.weight holds %s storage", name(element));
+        std::vector<int32_t> elements;
         auto declare = [&](const decoder::Parameter &parameter) {
-            if (parameter.rows == 1)
-                NEURA_ASSERT(parameter.element == Element::Single, "this decoder reads norm weights in single storage, and %s holds %s storage",
+            if (parameter.rows == 1) {
+                NEURA_ASSERT(parameter.element == Element::Single, "this decoder reads norm weights and biases in single storage, and %s holds %s storage",
                              parameter.name.c_str(), name(parameter.element));
-            else
-                NEURA_ASSERT(parameter.element == element, "this decoder multiplies matrices of one storage, and %s holds %s storage beside %s",
-                             parameter.name.c_str(), name(parameter.element), name(element));
+            } else {
+                NEURA_ASSERT(parameter.element == Element::Q8_0 || parameter.element == Element::Q4K || parameter.element == Element::Q6K,
+                             "this decoder multiplies q8_0, q4_k and q6_k matrices, and %s holds %s storage", parameter.name.c_str(),
+                             name(parameter.element));
+                elements.push_back((int32_t)parameter.element);
+            }
             names.push_back(parameter.name);
             return parameter;
         };
         declare(decoder::matrix(archive, "token_embd.weight", config.vocabulary, H));
-        declare(decoder::vector(archive, "output_norm.weight", H));
         bool separate_head = archive.tensor("output.weight").has_value();
-        if (separate_head) declare(decoder::matrix(archive, "output.weight", config.vocabulary, H));
+        if (separate_head)
+            declare(decoder::matrix(archive, "output.weight", config.vocabulary, H));
+        else
+            elements.push_back((int32_t)element);
+        declare(decoder::vector(archive, "output_norm.weight", H));
+        std::vector<uint64_t> biases[3];
         for (uint32_t layer = 0; layer < config.layers; layer++) {
             auto at = [&](const char *suffix) { return "blk." + std::to_string(layer) + "." + suffix; };
-            declare(decoder::vector(archive, at("attn_norm.weight"), H));
             declare(decoder::matrix(archive, at("attn_q.weight"), QW, H));
             declare(decoder::matrix(archive, at("attn_k.weight"), KW, H));
             declare(decoder::matrix(archive, at("attn_v.weight"), KW, H));
             declare(decoder::matrix(archive, at("attn_output.weight"), H, QW));
-            declare(decoder::vector(archive, at("ffn_norm.weight"), H));
             declare(decoder::matrix(archive, at("ffn_gate.weight"), F, H));
             declare(decoder::matrix(archive, at("ffn_up.weight"), F, H));
             declare(decoder::matrix(archive, at("ffn_down.weight"), H, F));
+            declare(decoder::vector(archive, at("attn_norm.weight"), H));
+            declare(decoder::vector(archive, at("ffn_norm.weight"), H));
+            const char *projections[3] = {"attn_q.bias", "attn_k.bias", "attn_v.bias"};
+            const uint32_t widths[3] = {QW, KW, KW};
+            for (int s = 0; s < 3; s++)
+                if (archive.tensor(at(projections[s])).has_value()) declare(decoder::vector(archive, at(projections[s]), widths[s]));
         }
         weights_ = std::make_unique<runtime::Weights>(runtime, source, names);
         std::vector<uint64_t> columns[9];
         const char *suffixes[9] = {"attn_norm", "attn_q", "attn_k", "attn_v", "attn_output", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down"};
         for (uint32_t layer = 0; layer < config.layers; layer++)
             for (int s = 0; s < 9; s++) columns[s].push_back(weights_->offset("blk." + std::to_string(layer) + "." + suffixes[s] + ".weight"));
+        for (uint32_t layer = 0; layer < config.layers; layer++) {
+            const char *projections[3] = {"attn_q.bias", "attn_k.bias", "attn_v.bias"};
+            for (int s = 0; s < 3; s++) {
+                const std::string bias = "blk." + std::to_string(layer) + "." + projections[s];
+                biases[s].push_back(archive.tensor(bias).has_value() ? weights_->offset(bias) : UINT64_MAX);
+            }
+        }
         nh_tensor_table table{};
         table.matrix_element = (int32_t)element;
+        table.matrix_elements = elements.data();
+        table.attn_q_bias = biases[0].data(), table.attn_k_bias = biases[1].data(), table.attn_v_bias = biases[2].data();
         table.token_embd = weights_->offset("token_embd.weight");
         table.output = separate_head ? weights_->offset("output.weight") : UINT64_MAX;
         table.output_norm = weights_->offset("output_norm.weight");

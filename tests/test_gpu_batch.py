@@ -8,7 +8,7 @@ import pytest
 
 import oracle
 from gguf_fixture import build as build_gguf
-from neura_amd import NH_Q4_K, NH_Q8_0, host, synth
+from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, host, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -17,9 +17,9 @@ SHAPE_Q4 = dict(layers=2, hidden=512, heads=4, kv_heads=2, head_dim=128, ffn=102
 CONTEXT = 96
 
 
-def qwen2_gguf(path, shape, element, seed):
+def qwen2_gguf(path, shape, element, seed, elements=None, biases=()):
     rng = np.random.default_rng(seed)
-    tensors = list(synth.model_tensors(shape, element, rng, mode="normal"))
+    tensors = list(synth.model_tensors(shape, element, rng, mode="normal", elements=elements, biases=biases))
     metadata = [("general.alignment", "u32", 32), ("general.architecture", "string", "qwen2"),
                 ("qwen2.block_count", "u32", shape["layers"]), ("qwen2.embedding_length", "u32", shape["hidden"]),
                 ("qwen2.feed_forward_length", "u32", shape["ffn"]), ("qwen2.attention.head_count", "u32", shape["heads"]),
@@ -29,12 +29,12 @@ def qwen2_gguf(path, shape, element, seed):
         metadata.append(("qwen2.attention.key_length", "u32", shape["head_dim"]))
     data, _, _ = build_gguf(32, metadata, [(name, kind, list(dims), raw.tobytes()) for name, kind, dims, raw in tensors])
     path.write_bytes(data)
-    return {name: raw for name, _, _, raw in tensors}
+    return {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
 
 
-def alone(shape, element, tensors, prompt, count):
+def alone(shape, element, tensors, prompt, count, elements=None):
     """The oracle's greedy answer to one prompt: fed token by token, then `count` choices."""
-    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT)
+    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT, elements=elements)
     margins = []
     for at, token in enumerate(prompt):
         logits, chosen = ref.forward([token], 1, [at])
@@ -80,6 +80,24 @@ def test_a_batched_sequence_answers_as_it_does_alone(runtime, tmp_path, shape, e
     got = run(batch, {slot: 8 for slot in slots})
     for slot, prompt in zip(slots, prompts):
         want, margin = alone(shape, element, tensors, prompt, 8)
+        assert got[slot] == want, (slot, margin)
+    batch.close()
+    archive.close()
+
+
+def test_a_file_of_mixed_storage_with_projection_biases_generates(runtime, tmp_path):
+    # the way Q4_K_M files of Qwen2 checkpoints come: q6_k for the head, some value and down projections; biases on q, k, v
+    shape = SHAPE_Q4
+    mixed = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.1.ffn_down.weight": NH_Q6_K}
+    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, NH_Q4_K, seed=31, elements=mixed, biases=(0, 1))
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [16])
+    rng = np.random.default_rng(32)
+    prompts = [list(rng.integers(0, shape["vocab"], n)) for n in (5, 21)]
+    slots = [batch.admit(prompt) for prompt in prompts]
+    got = run(batch, {slot: 6 for slot in slots})
+    for slot, prompt in zip(slots, prompts):
+        want, margin = alone(shape, NH_Q4_K, tensors, prompt, 6, elements=mixed)
         assert got[slot] == want, (slot, margin)
     batch.close()
     archive.close()
