@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes one Q4_K product launch of the 7B-shape decode step moves on average, from the
 # rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_q4k_decode_hbm_counters.md
 # (each counter scaled by its reading for a plain 1 GiB copy); not measurable inside this script
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.79e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.76e6}
 
 
 def workload(name):
