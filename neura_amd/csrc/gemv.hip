@@ -1255,6 +1255,228 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MfmaParams 
     }
 }
 
+// The Q4_K product on 32 x 32 x 32 integer MFMAs (v_mfma_i32_32x32x32_i8): weights are the B operand -- lane (n, q) =
+// (lane % 32, lane / 32) supplies 16 nibbles of row n, one per byte, straight from its 16-byte load of half a group --
+// and the digit planes of up to eight activation rows are the A operand (row m = 4 * activation row + plane, read from
+// LDS as they were staged).  C comes back with lane n holding the sums of ITS OWN weight row against every plane: no
+// sum ever crosses lanes, the lane that holds a sum holds the header that scales it, and one instruction multiplies
+// 1024 weights by eight activation rows.  Against the vector kernel that is about half the vector instructions per
+// weight for one activation row, and eight rows cost little more than one.  Digits are scaled per sub-block of 32
+// (no pass over the row).  Four waves share a tile of 32 rows, each walking every fourth super-block; their partial
+// sums meet lane by lane in LDS.  J: row pairs of C in use (activation rows 2j + q), NW: waves per workgroup.
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+struct Tile32Unit {
+    u32x4 hdr, g[4];
+};
+
+template <int J, int NW, int KS>
+__global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_kernel(MfmaParams p) {  // second bound: waves per SIMD
+
+    constexpr uint32_t M8 = 8 * J, R2 = 2 * J, TPW = NW / KS, NT = NW * 64;
+    constexpr bool STAGED = J == 1;  // raw blocks through LDS; with eight activation rows the digits leave no room for them
+    extern __shared__ __attribute__((aligned(16))) uint32_t staged[];  // digits [block][sub-block][q][M8] of 16 bytes
+    __shared__ float red[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t nb = p.nblk;
+    float2 *const sums = reinterpret_cast<float2 *>(staged + (size_t)nb * 64u * M8);  // [block][sub-block][R2]: (unscale, sub-block sum * unscale)
+    float *const part = reinterpret_cast<float *>(sums + (size_t)nb * 8u * R2);        // [2][TPW][KS][J][64]
+    u32x4 *const raw = reinterpret_cast<u32x4 *>(part + (size_t)2 * TPW * KS * J * 64u) + (size_t)wave * 288u;  // per wave: one super-block of the tile, raw
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+
+    // ---- activations -> digit planes, 16 elements (half a sub-block) per thread; a row takes at most 256 threads
+    // (K <= 4096), so a workgroup of sixteen waves stages four rows side by side
+    constexpr uint32_t GROUPS = NT / 256u;
+    const uint32_t chunks = nb * 16u;
+    const uint32_t rg = tid >> 8, t = tid & 255u;
+    for (uint32_t row0 = 0; row0 < R2; row0 += GROUPS) {
+        const uint32_t row = row0 + rg;  // groups past the staged rows only keep the barriers company
+        const bool real = row < p.rows;
+        const float *xr = p.x + (size_t)min(row, p.rows - 1u) * p.K;
+        {
+            const bool held = t < chunks && row < R2;
+            float v[16];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (held && real) a = *reinterpret_cast<const float4 *>(xr + 16u * t + 4u * c);
+                v[4 * c] = a.x, v[4 * c + 1] = a.y, v[4 * c + 2] = a.z, v[4 * c + 3] = a.w;
+            }
+            if (p.norm_w) {
+                // the whole row is in registers across its 256 threads
+                float4 w[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++) w[c] = held ? *reinterpret_cast<const float4 *>(p.norm_w + 16u * t + 4u * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+                float square = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
+                square = wave_sum(square);
+                if (lane == 0) red[wave] = square;
+                __syncthreads();
+                const float total = (red[4u * rg] + red[4u * rg + 1u]) + (red[4u * rg + 2u] + red[4u * rg + 3u]);
+                __syncthreads();  // red is reused by the next rows
+                const float rms = rms_scale_of(total, p.K, p.eps);
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    v[4 * c] = __fmul_rn(__fmul_rn(v[4 * c], rms), w[c].x), v[4 * c + 1] = __fmul_rn(__fmul_rn(v[4 * c + 1], rms), w[c].y);
+                    v[4 * c + 2] = __fmul_rn(__fmul_rn(v[4 * c + 2], rms), w[c].z), v[4 * c + 3] = __fmul_rn(__fmul_rn(v[4 * c + 3], rms), w[c].w);
+                }
+            }
+            uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
+#pragma unroll
+            for (int i = 0; i < 16; i++) top = max(top, __builtin_bit_cast(uint32_t, v[i]) & 0x7fffffffu);
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));  // the other half of the sub-block
+            const uint32_t raw_exponent = top >> 23;
+            const uint32_t exponent = min(max(raw_exponent, 30u), 254u);
+            const float scale = __builtin_bit_cast(float, (283u - exponent) << 23);
+            const float unscale = raw_exponent == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 29u) << 23);
+            float total = 0.0f;
+            uint32_t plane[4][4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                uint32_t each[4], out[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float rounded = rintf(v[4 * c + e] * scale);
+                    total += rounded;
+                    each[e] = signed_digits((int)rounded);
+                }
+                digit_planes(each[0], each[1], each[2], each[3], out);
+#pragma unroll
+                for (int d = 0; d < 4; d++) plane[d][c] = out[d];
+            }
+            total += dpp<DPP_QUAD_XOR1>(total);
+            if (held) {
+                const uint32_t sub = t >> 1, q = t & 1u;  // sub-block of the row (block * 8 + sub-block), half of it
+                u32x4 *at = reinterpret_cast<u32x4 *>(staged) + ((size_t)sub * 2u + q) * M8 + 4u * row;
+#pragma unroll
+                for (int d = 0; d < 4; d++) at[d] = real ? u32x4{plane[d][0], plane[d][1], plane[d][2], plane[d][3]} : u32x4{0u, 0u, 0u, 0u};
+                if (q == 0) sums[(size_t)sub * R2 + row] = real ? make_float2(unscale, total * unscale) : make_float2(0.0f, 0.0f);
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- tiles of 32 weight rows
+    const uint32_t n = lane & 31u, q = lane >> 5;
+    const uint32_t ts = wave / KS, ks = wave % KS;
+    const uint32_t count = ks < nb ? (nb - ks + KS - 1u) / KS : 0u;  // super-blocks ks, ks + KS, ...
+    const uint32_t last_step = count ? count - 1u : 0u;
+    const uint8_t *const w0 = p.W[0], *const w1 = p.W[1], *const w2 = p.W[2];
+    const uint32_t end0 = p.end[0], end1 = p.end[1];
+    const bool gated = p.swiglu != 0;
+    const u32x4 *const a_lane = reinterpret_cast<const u32x4 *>(staged) + (size_t)q * M8 + (lane & 31u);
+    const bool a_held = (lane & 31u) < M8;
+    uint32_t parity = 0;
+    for (uint32_t base = blockIdx.x * TPW; base < p.tiles; base += gridDim.x * TPW) {
+        const uint32_t tile = base + ts;
+        const bool live = tile < p.tiles;
+        const uint32_t at_tile = live ? tile : p.tiles - 1u;
+        // first byte of row `r` of the tile
+        const uint32_t r0 = at_tile * 32u;
+        const bool in0 = r0 < end0, in1 = r0 < end1;
+        const uint8_t *const plain_base = (in0 ? w0 : (in1 ? w1 : w2)) + (size_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1))) * p.row_bytes;
+        auto row_base = [&](uint32_t r) -> const uint8_t * {
+            if (gated) return (r < 16u ? w0 : w1) + (size_t)(at_tile * 16u + (r & 15u)) * p.row_bytes;
+            return plain_base + (size_t)r * p.row_bytes;
+        };
+        // A super-block of the tile is 32 rows x 144 bytes = 288 pieces of 16 bytes.  Lane l fetches pieces l, l + 64, ...: nine
+        // neighbouring lanes read one row's block end to end (a load instruction touches 15 cache lines where one lane per
+        // row would touch 32), and the pieces go through LDS to the lanes that multiply them.
+        const uint8_t *src[5];
+#pragma unroll
+        for (int i = 0; i < 5; i++) {
+            if (STAGED) {
+                const uint32_t c = lane + 64u * i < 288u ? lane + 64u * i : lane;  // the last 32 pieces do not exist: fetched twice, dropped
+                src[i] = row_base(c / 9u) + (c % 9u) * 16u;
+            } else {
+                src[i] = row_base(n) + (i == 0 ? 0u : 16u + 32u * (i - 1) + 16u * q);  // this lane's own header and half groups
+            }
+        }
+        u32x4 ahead[5];
+        auto fetch = [&](uint32_t step) {
+            // past the wave's last super-block the last one is fetched again: the waits count on every step issuing its loads
+            const size_t off = (size_t)min(ks + KS * min(step, last_step), nb - 1u) * 144u;
+#pragma unroll
+            for (int i = 0; i < 5; i++) ahead[i] = *(global_uint4)(uintptr_t)(src[i] + off);
+        };
+        float acc[J];
+#pragma unroll
+        for (int j = 0; j < J; j++) acc[j] = 0.0f;
+        fetch(0);
+        for (uint32_t step = 0; step < count; step++) {
+            const uint32_t b = min(ks + KS * step, nb - 1u);
+            Tile32Unit u;
+            if (STAGED) {
+#pragma unroll
+                for (int i = 0; i < 5; i++)
+                    if (i < 4 || lane < 32u) raw[lane + 64u * i] = ahead[i];
+                fetch(step + 1u);
+                __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
+                u.hdr = raw[n * 9u];
+#pragma unroll
+                for (int g = 0; g < 4; g++) u.g[g] = raw[n * 9u + 1u + 2u * g + q];
+            } else {
+                u.hdr = ahead[0];
+#pragma unroll
+                for (int g = 0; g < 4; g++) u.g[g] = ahead[1 + g];
+                fetch(step + 1u);
+            }
+            // the eight 6-bit scales and minimums (crates/neura-precision/src/ggml.rs:127-136), four to a word
+            const uint32_t sc_lo = u.hdr.y & 0x3f3f3f3fu, sc_hi = (u.hdr.w & 0x0f0f0f0fu) | ((u.hdr.y >> 2) & 0x30303030u);
+            const uint32_t mn_lo = u.hdr.z & 0x3f3f3f3fu, mn_hi = ((u.hdr.w >> 4) & 0x0f0f0f0fu) | ((u.hdr.z >> 2) & 0x30303030u);
+            const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
+            const float d = (float)dd.x, dmin = (float)dd.y;
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const u32x4 words = u.g[s >> 1];
+                const u32x4 nibbles = ((s & 1) ? (words >> 4) : words) & 0x0f0f0f0fu;
+                u32x4 digits = {0u, 0u, 0u, 0u};
+                if (a_held) digits = a_lane[((size_t)b * 8u + s) * 2u * M8];
+                i32x16 zero;
+#pragma unroll
+                for (int e = 0; e < 16; e++) zero[e] = 0;
+                const i32x16 c = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(i32x4, digits), __builtin_bit_cast(i32x4, nibbles), zero, 0, 0, 0);
+                const uint32_t sc_word = s < 4 ? sc_lo : sc_hi, mn_word = s < 4 ? mn_lo : mn_hi;
+                const float weigh = d * (float)((sc_word >> (8 * (s & 3))) & 0xffu), floor_ = dmin * (float)((mn_word >> (8 * (s & 3))) & 0xffu);
+#pragma unroll
+                for (int j = 0; j < J; j++) {
+                    const float joined = fmaf(fmaf(fmaf((float)c[4 * j], 256.0f, (float)c[4 * j + 1]), 256.0f, (float)c[4 * j + 2]), 256.0f, (float)c[4 * j + 3]);
+                    const float2 xs = sums[((size_t)b * 8u + s) * R2 + 2u * j + q];
+                    acc[j] += fmaf(weigh * xs.x, joined, -(floor_ * xs.y));
+                }
+                if (s & 1) __builtin_amdgcn_sched_barrier(0);  // two sub-blocks' sums live at a time, not eight
+            }
+            __builtin_amdgcn_wave_barrier();  // the next super-block overwrites the raw pieces
+        }
+        // ---- the four waves of the tile meet lane by lane
+        float *mine = part + ((size_t)(parity * TPW + ts) * KS + ks) * J * 64u;
+#pragma unroll
+        for (int j = 0; j < J; j++) mine[j * 64 + lane] = acc[j];
+        __syncthreads();
+        if (ks == 0) {
+            const float *from = part + (size_t)(parity * TPW + ts) * KS * J * 64u;
+#pragma unroll
+            for (int j = 0; j < J; j++) {
+                float total = 0.0f;
+#pragma unroll
+                for (int k = 0; k < KS; k++) total += from[(size_t)k * J * 64u + j * 64 + lane];
+                const uint32_t arow = 2u * j + q;
+                const float up = __shfl_xor(total, 16, 64);
+                if (!live || arow >= p.rows) continue;
+                if (gated) {
+                    if (n < 16u) p.y[(size_t)arow * (p.N / 2) + tile * 16u + n] = silu(total) * up;
+                } else {
+                    const size_t at = (size_t)arow * p.N + tile * 32u + n;
+                    p.y[at] = p.residual ? p.residual[at] + total : total;
+                }
+            }
+        }
+        parity ^= 1u;
+    }
+}
+
 // ------------------------------------------------------------------------- fold ----------
 
 // sums the slice partials in slice order and applies the epilogue
@@ -1568,6 +1790,76 @@ bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     return a.end[0] % width == 0 && a.end[1] % width == 0 && a.end[2] == a.N;
 }
 
+// LDS of the 32-row tile kernel: digits, (unscale, sum) pairs, two rounds of partial sums, a raw super-block per wave
+static size_t mfma32_lds(uint32_t nblk, uint32_t J, uint32_t NW) {
+    return (size_t)nblk * 64u * 8u * J * 4u + (size_t)nblk * 8u * 2u * J * 8u + (size_t)2 * NW * J * 64u * 4u + (J == 1 ? (size_t)NW * 288u * 16u : 0u);
+}
+
+// whether the 32-row tile kernel serves this product: NEURA_HIP_MFMA32 = 0 never, 2 wherever it can, 1 (default) where
+// it measured faster -- several activation rows, or one row against a tall matrix
+static bool mfma32_takes(const nh_device *d, const GemvArgs &a) {
+    const int mode = env_int("NEURA_HIP_MFMA32", 1);
+    if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.K > 4096u || a.rows > 8) return false;
+    if (a.swiglu) {
+        if (a.N % 2u || a.end[0] != a.N / 2 || (a.N / 2) % 16u != 0) return false;
+    } else if (a.N % 32u != 0 || a.end[0] % 32u != 0 || a.end[1] % 32u != 0) {
+        return false;
+    }
+    if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
+    const uint32_t J = a.rows <= 2 ? 1u : 4u;
+    if (mfma32_lds(a.K / 256u, J, 16u) > 156u * 1024u) return false;  // eight rows of 4096 activations leave no room
+    if (mode == 2) return true;
+    // measured on the 7B shapes against the vector and 4 x 4 x 4 kernels: two rows win everywhere, five to eight rows
+    // win everywhere, three and four rows (which pay for eight) win on short and on very tall matrices only; one row
+    // never does (the vector kernel keeps its activations in registers)
+    if (a.rows == 2 || a.rows >= 5) return true;
+    return a.rows >= 3 && (a.N >= 65536u || a.N <= 8192u);
+}
+
+template <int J, int NW, int KS>
+static int32_t launch_mfma32_instance(nh_device *d, const MfmaParams &p, size_t lds) {
+    static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
+    if (lds > 64 * 1024 && !widened) {
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma32_kernel<J, NW, KS>), hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024));
+        widened = true;
+    }
+    // one resident round of workgroups, as many as LDS and registers let a compute unit hold
+    uint32_t resident = (uint32_t)((159 * 1024) / (lds + 1280));
+    const uint32_t by_waves = NW == 16 ? 1u : 12u / NW;
+    if (resident > by_waves) resident = by_waves;
+    if (resident < 1) resident = 1;
+    uint32_t blocks_x = (p.tiles + NW / KS - 1) / (NW / KS);
+    const uint32_t most = (uint32_t)d->compute_units * resident;
+    if (blocks_x > most) blocks_x = most;
+    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x), dim3(NW * 64), lds, d->stream, p);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
+    MfmaParams p{};
+    for (int s = 0; s < 3; s++) {
+        p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+        p.end[s] = a.end[s];
+    }
+    p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
+    p.N = a.N, p.K = a.K, p.nblk = a.K / 256u, p.row_bytes = p.nblk * 144u, p.rows = a.rows;
+    p.swiglu = a.swiglu, p.eps = a.eps;
+    p.tiles = a.swiglu ? a.N / 32u : a.N / 32u;
+    const uint32_t J = a.rows <= 2 ? 1u : 4u;  // a two-pair form spilled at 128 registers; three and four rows take the four-pair one
+    profile_mark(d);
+    int32_t status;
+    // with eight staged rows, a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
+    const bool few = p.tiles < 2u * (uint32_t)d->compute_units;
+    if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.nblk, 1, 4));
+    else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.nblk, 4, 16));
+    else status = launch_mfma32_instance<4, 16, 4>(d, p, mfma32_lds(p.nblk, 4, 16));
+    if (status != NH_OK) return status;
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
+}
+
 // Q6_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
 template <int RB>
 static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
@@ -1611,6 +1903,7 @@ static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, 
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (mfma32_takes(d, a)) return launch_mfma32(d, a);
     if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;

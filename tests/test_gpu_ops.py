@@ -163,6 +163,29 @@ def test_q4_k_products_agree_in_every_form(device, monkeypatch, mode, N, K, rows
     close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
 
 
+@pytest.mark.parametrize("N,K,rows", [(64, 3584, 1), (96, 2048, 4), (128, 256, 2), (2048, 3584, 7), (64, 4096, 3), (64, 1536, 8), (160, 768, 5)])
+def test_q4_k_product_on_32_row_tiles(device, monkeypatch, N, K, rows):
+    """NEURA_HIP_MFMA32=2 forces the 32 x 32 x 32 integer MFMA kernel (weights as the B operand, the digit planes of up to
+    eight activation rows as A, digits scaled per sub-block): plain, with a residual and with SwiGLU, for every count of
+    activation rows, against the oracle and an fp64 product (the decoder tests run it with the fused norm)."""
+    monkeypatch.setenv("NEURA_HIP_MFMA32", "2")
+    rng = np.random.default_rng(N + K + rows)
+    raw = synth.q4_k_random(rng, N * K)
+    x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-6, 6, (rows, K)))).astype(np.float32)  # wide dynamic range
+    r = rng.standard_normal((rows, N)).astype(np.float32)
+    plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+    exact = oracle.unpack(NH_Q4_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+    got = device.gemv(NH_Q4_K, raw, N, K, x)
+    close(got, plain)
+    assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * max(1.0, np.abs(exact).max()))
+    tight(device.gemv(NH_Q4_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2:].astype(np.float64)
+    want = gate / (1.0 + np.exp(-gate)) * up
+    close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+    x[0, 5] = np.inf
+    assert not np.isfinite(device.gemv(NH_Q4_K, raw, N, K, x)[0]).any()
+
+
 def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device, monkeypatch):
     monkeypatch.setenv("NEURA_HIP_MFMA", "2")
     rng = np.random.default_rng(2)
