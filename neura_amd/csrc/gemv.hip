@@ -1279,7 +1279,10 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
     __shared__ float red[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nb = p.nblk;
+    // rows too deep to stage whole are cut into K slices (blockIdx.y), whose partial sums a second kernel folds
+    const uint32_t split = blockIdx.y, blk0 = split * p.slice_blocks;
+    const uint32_t nb = min(p.slice_blocks, p.nblk - blk0);
+    const uint32_t k0 = blk0 * 256u;
     float2 *const sums = reinterpret_cast<float2 *>(staged + (size_t)nb * 64u * M8);  // [block][sub-block][R2]: (unscale, sub-block sum * unscale)
     float *const part = reinterpret_cast<float *>(sums + (size_t)nb * 8u * R2);        // [2][TPW][KS][J][64]
     u32x4 *const raw = reinterpret_cast<u32x4 *>(part + (size_t)2 * TPW * KS * J * 64u) + (size_t)wave * 288u;  // per wave: one super-block of the tile, raw
@@ -1300,14 +1303,14 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (held && real) a = *reinterpret_cast<const float4 *>(xr + 16u * t + 4u * c);
+                if (held && real) a = *reinterpret_cast<const float4 *>(xr + k0 + 16u * t + 4u * c);
                 v[4 * c] = a.x, v[4 * c + 1] = a.y, v[4 * c + 2] = a.z, v[4 * c + 3] = a.w;
             }
             if (p.norm_w) {
                 // the whole row is in registers across its 256 threads
                 float4 w[4];
 #pragma unroll
-                for (int c = 0; c < 4; c++) w[c] = held ? *reinterpret_cast<const float4 *>(p.norm_w + 16u * t + 4u * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+                for (int c = 0; c < 4; c++) w[c] = held ? *reinterpret_cast<const float4 *>(p.norm_w + k0 + 16u * t + 4u * c) : make_float4(0.f, 0.f, 0.f, 0.f);
                 float square = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 16; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
@@ -1389,9 +1392,9 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
         for (int i = 0; i < 5; i++) {
             if (STAGED) {
                 const uint32_t c = lane + 64u * i < 288u ? lane + 64u * i : lane;  // the last 32 pieces do not exist: fetched twice, dropped
-                src[i] = row_base(c / 9u) + (c % 9u) * 16u;
+                src[i] = row_base(c / 9u) + (size_t)blk0 * 144u + (c % 9u) * 16u;
             } else {
-                src[i] = row_base(n) + (i == 0 ? 0u : 16u + 32u * (i - 1) + 16u * q);  // this lane's own header and half groups
+                src[i] = row_base(n) + (size_t)blk0 * 144u + (i == 0 ? 0u : 16u + 32u * (i - 1) + 16u * q);  // this lane's own header and half groups
             }
         }
         u32x4 ahead[5];
@@ -1465,7 +1468,10 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
                 const uint32_t arow = 2u * j + q;
                 const float up = __shfl_xor(total, 16, 64);
                 if (!live || arow >= p.rows) continue;
-                if (gated) {
+                if (p.splits > 1) {
+                    const uint32_t column = gated ? (n < 16u ? tile * 16u + n : p.N / 2 + tile * 16u + (n - 16u)) : tile * 32u + n;
+                    p.partial[((size_t)split * p.rows + arow) * p.N + column] = total;
+                } else if (gated) {
                     if (n < 16u) p.y[(size_t)arow * (p.N / 2) + tile * 16u + n] = silu(total) * up;
                 } else {
                     const size_t at = (size_t)arow * p.N + tile * 32u + n;
@@ -1799,7 +1805,9 @@ static size_t mfma32_lds(uint32_t nblk, uint32_t J, uint32_t NW) {
 // it measured faster -- several activation rows, or one row against a tall matrix
 static bool mfma32_takes(const nh_device *d, const GemvArgs &a) {
     const int mode = env_int("NEURA_HIP_MFMA32", 1);
-    if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.K > 4096u || a.rows > 8) return false;
+    if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.rows > 8) return false;
+    // deeper rows go in K slices with a fold behind them: worth it from five activation rows on, and never with a fused norm
+    if (a.K > 4096u && (a.norm_w || (mode != 2 && a.rows < 5))) return false;
     if (a.swiglu) {
         if (a.N % 2u || a.end[0] != a.N / 2 || (a.N / 2) % 16u != 0) return false;
     } else if (a.N % 32u != 0 || a.end[0] % 32u != 0 || a.end[1] % 32u != 0) {
@@ -1807,7 +1815,7 @@ static bool mfma32_takes(const nh_device *d, const GemvArgs &a) {
     }
     if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
     const uint32_t J = a.rows <= 2 ? 1u : 4u;
-    if (mfma32_lds(a.K / 256u, J, 16u) > 156u * 1024u) return false;  // eight rows of 4096 activations leave no room
+    if (a.K <= 4096u && mfma32_lds(a.K / 256u, J, 16u) > 156u * 1024u) return false;  // eight rows of 4096 activations leave no room
     if (mode == 2) return true;
     // measured on the 7B shapes against the vector and 4 x 4 x 4 kernels: two rows win everywhere, five to eight rows
     // win everywhere, three and four rows (which pay for eight) win on short and on very tall matrices only; one row
@@ -1829,9 +1837,10 @@ static int32_t launch_mfma32_instance(nh_device *d, const MfmaParams &p, size_t 
     if (resident > by_waves) resident = by_waves;
     if (resident < 1) resident = 1;
     uint32_t blocks_x = (p.tiles + NW / KS - 1) / (NW / KS);
-    const uint32_t most = (uint32_t)d->compute_units * resident;
+    uint32_t most = (uint32_t)d->compute_units * resident / p.splits;
+    if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
-    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -1845,16 +1854,32 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
     p.N = a.N, p.K = a.K, p.nblk = a.K / 256u, p.row_bytes = p.nblk * 144u, p.rows = a.rows;
     p.swiglu = a.swiglu, p.eps = a.eps;
-    p.tiles = a.swiglu ? a.N / 32u : a.N / 32u;
+    p.tiles = a.N / 32u;
     const uint32_t J = a.rows <= 2 ? 1u : 4u;  // a two-pair form spilled at 128 registers; three and four rows take the four-pair one
+    // K slices: at most 14 super-blocks with eight staged rows (the digits of 3584 activations x 8 rows fill 112 KiB), 16 otherwise
+    const uint32_t most_blocks = J == 4 ? 14u : 16u;
+    p.splits = (p.nblk + most_blocks - 1) / most_blocks;
+    p.slice_blocks = (p.nblk + p.splits - 1) / p.splits;
+    p.splits = (p.nblk + p.slice_blocks - 1) / p.slice_blocks;
+    if (p.splits > 1) {
+        p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * p.rows * a.N * sizeof(float)));
+        if (!p.partial) return NH_E_MEMORY;
+    }
     profile_mark(d);
     int32_t status;
     // with eight staged rows, a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
-    const bool few = p.tiles < 2u * (uint32_t)d->compute_units;
-    if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.nblk, 1, 4));
-    else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.nblk, 4, 16));
-    else status = launch_mfma32_instance<4, 16, 4>(d, p, mfma32_lds(p.nblk, 4, 16));
+    const int forced = env_int("NEURA_HIP_MFMA32_KS", 0);
+    const bool few = forced ? forced == 16 : p.tiles * p.splits < 2u * (uint32_t)d->compute_units;
+    if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.slice_blocks, 1, 4));
+    else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
+    else status = launch_mfma32_instance<4, 16, 4>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
     if (status != NH_OK) return status;
+    if (p.splits > 1) {
+        const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
+        hipLaunchKernelGGL(gemv_fold_kernel, dim3((outputs * p.rows + 255) / 256), dim3(256), 0, d->stream, p.partial, p.splits, p.rows, a.N,
+                           p.residual, a.swiglu, p.y);
+        NH_HIP(hipGetLastError());
+    }
     profile_mark(d);
     if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
     return NH_OK;

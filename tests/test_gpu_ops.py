@@ -163,7 +163,8 @@ def test_q4_k_products_agree_in_every_form(device, monkeypatch, mode, N, K, rows
     close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
 
 
-@pytest.mark.parametrize("N,K,rows", [(64, 3584, 1), (96, 2048, 4), (128, 256, 2), (2048, 3584, 7), (64, 4096, 3), (64, 1536, 8), (160, 768, 5)])
+@pytest.mark.parametrize("N,K,rows", [(64, 3584, 1), (96, 2048, 4), (128, 256, 2), (2048, 3584, 7), (64, 4096, 3), (64, 1536, 8), (160, 768, 5),
+                                      (64, 18944, 8), (96, 8960, 2), (32, 18944, 5)])
 def test_q4_k_product_on_32_row_tiles(device, monkeypatch, N, K, rows):
     """NEURA_HIP_MFMA32=2 forces the 32 x 32 x 32 integer MFMA kernel (weights as the B operand, the digit planes of up to
     eight activation rows as A, digits scaled per sub-block): plain, with a residual and with SwiGLU, for every count of
