@@ -697,29 +697,51 @@ __global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
     uint8_t *const mine = reinterpret_cast<uint8_t *>(xs + RB * xstride) + (size_t)wave * 2u * raw_stride;
     const uint32_t units = nb * 16u;
 
-    for (uint32_t first = 2u * (blockIdx.x * 4u + wave); first < p.N; first += 2u * gridDim.x * 4u) {
-        uint32_t lead[2];
+    // the 16-byte pieces of the two rows `first`, `first + 1` this lane copies: fetched one pair of rows ahead, so the copy
+    // of the next pair is in flight while this pair is multiplied (a slice is at most 16 blocks: four pieces a lane and row)
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    u32x4 ahead[2][4];
+    uint32_t ahead_lead[2] = {0u, 0u};
+    auto fetch = [&](uint32_t first) {
 #pragma unroll
         for (int r = 0; r < 2; r++) {
             const uint32_t i = min(first + r, p.N - 1u);
             const uint8_t *matrix_end;
             const uint8_t *src = row_start(p, weight_row(i, p.N, p.swiglu), matrix_end) + (size_t)blk0 * 210u;
-            lead[r] = (uint32_t)((uintptr_t)src & 15u);
-            const uint8_t *from = src - lead[r];
-            const uint32_t bytes = lead[r] + nb * 210u;
-            for (uint32_t c = lane; c * 16u < bytes; c += 64u) {
-                uint4 held;
-                if (from + 16u * c + 16u <= matrix_end) {
-                    held = *reinterpret_cast<const uint4 *>(from + 16u * c);
-                } else {  // the last bytes of the tensor: never read past its end
-                    uint8_t tail[16];
+            ahead_lead[r] = (uint32_t)((uintptr_t)src & 15u);
+            const uint8_t *from = src - ahead_lead[r];
+            const uint32_t bytes = ahead_lead[r] + nb * 210u;
 #pragma unroll
-                    for (int j = 0; j < 16; j++) tail[j] = (from + 16u * c + j < matrix_end) ? from[16u * c + j] : (uint8_t)0;
-                    held = *reinterpret_cast<uint4 *>(tail);
+            for (int k = 0; k < 4; k++) {
+                const uint32_t c = lane + 64u * k;
+                u32x4 held = {0u, 0u, 0u, 0u};
+                if (c * 16u < bytes) {
+                    if (from + 16u * c + 16u <= matrix_end) {
+                        held = *(global_uint4)(uintptr_t)(from + 16u * c);
+                    } else {  // the last bytes of the tensor: never read past its end
+                        uint8_t tail[16];
+#pragma unroll
+                        for (int j = 0; j < 16; j++) tail[j] = (from + 16u * c + j < matrix_end) ? from[16u * c + j] : (uint8_t)0;
+                        held = *reinterpret_cast<u32x4 *>(tail);
+                    }
                 }
-                *reinterpret_cast<uint4 *>(mine + r * raw_stride + 16u * c) = held;
+                ahead[r][k] = held;
             }
         }
+    };
+    const uint32_t stride = 2u * gridDim.x * 4u;
+    uint32_t first = 2u * (blockIdx.x * 4u + wave);
+    if (first < p.N) fetch(first);
+    for (; first < p.N; first += stride) {
+        uint32_t lead[2];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            lead[r] = ahead_lead[r];
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                if ((lane + 64u * k) < p.chunks_per_row) *reinterpret_cast<u32x4 *>(mine + r * raw_stride + 16u * (lane + 64u * k)) = ahead[r][k];
+        }
+        if (first + stride < p.N) fetch(first + stride);
         __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
 
         float acc[2][RB];
