@@ -38,7 +38,9 @@ enum {
     NH_F32 = 0,   /* Element::Single   */
     NH_F16 = 1,   /* Element::Half     */
     NH_Q8_0 = 8,  /* Element::Q8_0: 32 elements / 34 bytes  (crates/neura-abi/src/element.rs:155-158) */
+    NH_Q3_K = 11, /* Element::Q3K: 256 elements / 110 bytes (crates/neura-abi/src/element.rs:171-174) */
     NH_Q4_K = 12, /* Element::Q4K: 256 elements / 144 bytes (crates/neura-abi/src/element.rs:159-162) */
+    NH_Q5_K = 13, /* Element::Q5K: 256 elements / 176 bytes (crates/neura-abi/src/element.rs:163-166) */
     NH_Q6_K = 14  /* Element::Q6K: 256 elements / 210 bytes (crates/neura-abi/src/element.rs:167-170) */
 };
 

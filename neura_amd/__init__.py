@@ -7,9 +7,9 @@ import ctypes
 import numpy as np
 
 from . import _abi
-from ._abi import NH_F16, NH_F32, NH_Q4_K, NH_Q6_K, NH_Q8_0, UINT64_MAX, Epilogue, ModelConfig, TensorTable
+from ._abi import NH_F16, NH_F32, NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K, NH_Q8_0, UINT64_MAX, Epilogue, ModelConfig, TensorTable
 
-BLOCK = {NH_Q8_0: (32, 34), NH_Q4_K: (256, 144), NH_Q6_K: (256, 210), NH_F16: (1, 2), NH_F32: (1, 4)}  # elements, bytes
+BLOCK = {NH_Q8_0: (32, 34), NH_Q3_K: (256, 110), NH_Q4_K: (256, 144), NH_Q5_K: (256, 176), NH_Q6_K: (256, 210), NH_F16: (1, 2), NH_F32: (1, 4)}  # elements, bytes
 
 
 class NeuraError(RuntimeError):
@@ -217,5 +217,5 @@ class Device:
         return out.numpy(np.uint32)
 
 
-__all__ = ["Device", "Buffer", "NeuraError", "payload_bytes", "NH_F32", "NH_F16", "NH_Q8_0", "NH_Q4_K", "NH_Q6_K", "UINT64_MAX", "Epilogue",
+__all__ = ["Device", "Buffer", "NeuraError", "payload_bytes", "NH_F32", "NH_F16", "NH_Q8_0", "NH_Q3_K", "NH_Q4_K", "NH_Q5_K", "NH_Q6_K", "UINT64_MAX", "Epilogue",
            "ModelConfig", "TensorTable"]

@@ -11,6 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY = os.path.join(HERE, "libneura_hip.so")
 
 NH_F32, NH_F16, NH_Q8_0, NH_Q4_K, NH_Q6_K = 0, 1, 8, 12, 14
+NH_Q3_K, NH_Q5_K = 11, 13
 NH_OK, NH_E_ARGUMENT, NH_E_DEVICE, NH_E_MEMORY, NH_E_REFUSAL = 0, -1, -2, -3, -4
 UINT64_MAX = (1 << 64) - 1
 

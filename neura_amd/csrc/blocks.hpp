@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <cstdint>
 
+#include "../../include/neura_hip.h"
+
 namespace nh {
 
 __device__ __forceinline__ float half_to_float(uint16_t bits) {
@@ -64,6 +66,53 @@ __device__ __forceinline__ float q6_k_element(const uint8_t *row, uint64_t i) {
     float scale = (float)(int8_t)block[192 + half * 8 + group * 2 + lane / 16];
     float quantum = __fmul_rn(half_to_float(load_u16(block + 208)), scale);
     return __fmul_rn(quantum, (float)(low | (high << 4)) - 32.0f);
+}
+
+// element `i` of a row of Q5_K blocks (crates/neura-precision/src/ggml.rs:321-335): Q4_K's walk with a fifth bit per code
+__device__ __forceinline__ float q5_k_element(const uint8_t *row, uint64_t i) {
+    const uint8_t *block = row + (i / 256) * 176;
+    uint32_t within = (uint32_t)(i % 256);
+    uint32_t group = within / 64, seat = (within % 64) / 32, lane = within % 32;
+    uint32_t code, offset;
+    scale_min_k4(block + 4, group * 2 + seat, code, offset);
+    float quantum = __fmul_rn(half_to_float(load_u16(block)), (float)code);
+    float low = __fmul_rn(half_to_float(load_u16(block + 2)), (float)offset);
+    uint8_t byte = block[48 + group * 32 + lane];
+    uint32_t quant = (seat ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f)) | ((((uint32_t)block[16 + lane] >> (2 * group + seat)) & 1u) << 4);
+    return __fsub_rn(__fmul_rn(quantum, (float)quant), low);
+}
+
+// 6-bit scale `at` (0..15) of a Q3_K super-block, as stored (32 too large): crates/neura-precision/src/ggml.rs:224-229
+__device__ __forceinline__ uint32_t q3_k_scale(const uint8_t *block, uint32_t at) {
+    uint32_t low = block[96 + at % 8];
+    uint32_t nibble = at < 8 ? (low & 0x0fu) : (low >> 4);
+    uint32_t high = block[104 + at % 4];
+    return nibble | (((high >> (2 * (at / 4))) & 3u) << 4);
+}
+
+// element `i` of a row of Q3_K blocks (crates/neura-precision/src/ggml.rs:291-306): d * (scale - 32), rounded, times the
+// code: the bit pair, less 4 unless the third bit is set
+__device__ __forceinline__ float q3_k_element(const uint8_t *row, uint64_t i) {
+    const uint8_t *block = row + (i / 256) * 110;
+    uint32_t within = (uint32_t)(i % 256);
+    uint32_t sub = within / 16, lane = within % 16;
+    uint32_t half = sub / 8, j = (sub % 8) / 2, second = sub % 2;
+    uint32_t low = ((uint32_t)block[32 + half * 32 + second * 16 + lane] >> (2 * j)) & 3u;
+    uint32_t high = ((uint32_t)block[second * 16 + lane] >> (half * 4 + j)) & 1u;
+    float quantum = __fmul_rn(half_to_float(load_u16(block + 108)), (float)q3_k_scale(block, sub) - 32.0f);
+    return __fmul_rn(quantum, (float)low - (high ? 0.0f : 4.0f));
+}
+
+// element `i` of a row stored as ELEMENT
+template <int ELEMENT>
+__device__ __forceinline__ float stored_element(const uint8_t *row, uint64_t i) {
+    if (ELEMENT == NH_Q8_0) return q8_0_element(row, i);
+    if (ELEMENT == NH_Q3_K) return q3_k_element(row, i);
+    if (ELEMENT == NH_Q4_K) return q4_k_element(row, i);
+    if (ELEMENT == NH_Q5_K) return q5_k_element(row, i);
+    if (ELEMENT == NH_Q6_K) return q6_k_element(row, i);
+    if (ELEMENT == NH_F16) return half_to_float(reinterpret_cast<const uint16_t *>(row)[i]);
+    return reinterpret_cast<const float *>(row)[i];
 }
 
 // 1 / sqrt(total / columns + eps) with every step rounded to fp32 exactly as IEEE does

@@ -9,18 +9,7 @@ namespace nh {
 template <int ELEMENT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ src, uint64_t elements, float *__restrict__ dst) {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < elements; i += (uint64_t)gridDim.x * blockDim.x) {
-        float value;
-        if (ELEMENT == NH_Q8_0)
-            value = q8_0_element(src, i);
-        else if (ELEMENT == NH_Q4_K)
-            value = q4_k_element(src, i);
-        else if (ELEMENT == NH_Q6_K)
-            value = q6_k_element(src, i);
-        else if (ELEMENT == NH_F16)
-            value = half_to_float(reinterpret_cast<const uint16_t *>(src)[i]);
-        else
-            value = reinterpret_cast<const float *>(src)[i];
-        dst[i] = value;
+        dst[i] = stored_element<ELEMENT>(src, i);
     }
 }
 
@@ -38,6 +27,8 @@ int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t 
     case NH_Q8_0: hipLaunchKernelGGL(dequant_kernel<NH_Q8_0>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_Q4_K: hipLaunchKernelGGL(dequant_kernel<NH_Q4_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_Q6_K: hipLaunchKernelGGL(dequant_kernel<NH_Q6_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_Q5_K: hipLaunchKernelGGL(dequant_kernel<NH_Q5_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
+    case NH_Q3_K: hipLaunchKernelGGL(dequant_kernel<NH_Q3_K>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_F16: hipLaunchKernelGGL(dequant_kernel<NH_F16>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     case NH_F32: hipLaunchKernelGGL(dequant_kernel<NH_F32>, dim3(grid), dim3(256), 0, d->stream, bytes, elements, dst); break;
     default: return fail(NH_E_ARGUMENT, "element %d carries no reader", element);
@@ -74,18 +65,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__
     }
     const uint8_t *row = table + (uint64_t)token * row_bytes;
     for (uint32_t c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
-        float value;
-        if (ELEMENT == NH_Q8_0)
-            value = q8_0_element(row, c);
-        else if (ELEMENT == NH_Q4_K)
-            value = q4_k_element(row, c);
-        else if (ELEMENT == NH_Q6_K)
-            value = q6_k_element(row, c);
-        else if (ELEMENT == NH_F16)
-            value = half_to_float(reinterpret_cast<const uint16_t *>(row)[c]);
-        else
-            value = reinterpret_cast<const float *>(row)[c];
-        out[(uint64_t)t * width + c] = value * keep;
+        out[(uint64_t)t * width + c] = stored_element<ELEMENT>(row, c) * keep;
     }
 }
 
@@ -107,6 +87,14 @@ int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t
         break;
     case NH_Q6_K:
         hipLaunchKernelGGL(gather_kernel<NH_Q6_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_Q5_K:
+        hipLaunchKernelGGL(gather_kernel<NH_Q5_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
+                           out, d->refusal);
+        break;
+    case NH_Q3_K:
+        hipLaunchKernelGGL(gather_kernel<NH_Q3_K>, grid, dim3(256), 0, d->stream, bytes, vocab, width, row_bytes, tokens, batch, mask,
                            out, d->refusal);
         break;
     case NH_F16:

@@ -15,6 +15,8 @@ namespace nh {
 constexpr uint32_t Q8_0_BLOCK = 32, Q8_0_BYTES = 34;
 constexpr uint32_t Q4_K_BLOCK = 256, Q4_K_BYTES = 144;
 constexpr uint32_t Q6_K_BLOCK = 256, Q6_K_BYTES = 210;
+constexpr uint32_t Q5_K_BLOCK = 256, Q5_K_BYTES = 176;
+constexpr uint32_t Q3_K_BLOCK = 256, Q3_K_BYTES = 110;
 constexpr uint32_t WAVE = 64;
 
 int32_t fail(int32_t code, const char *format, ...) __attribute__((format(printf, 2, 3)));
@@ -36,16 +38,23 @@ inline uint64_t payload_bytes(int32_t element, uint64_t elements) {
     case NH_Q8_0: return (elements + Q8_0_BLOCK - 1) / Q8_0_BLOCK * Q8_0_BYTES;
     case NH_Q4_K: return (elements + Q4_K_BLOCK - 1) / Q4_K_BLOCK * Q4_K_BYTES;
     case NH_Q6_K: return (elements + Q6_K_BLOCK - 1) / Q6_K_BLOCK * Q6_K_BYTES;
+    case NH_Q5_K: return (elements + Q5_K_BLOCK - 1) / Q5_K_BLOCK * Q5_K_BYTES;
+    case NH_Q3_K: return (elements + Q3_K_BLOCK - 1) / Q3_K_BLOCK * Q3_K_BYTES;
     case NH_F16: return elements * 2;
     case NH_F32: return elements * 4;
     default: return 0;
     }
 }
 
+// the super-block formats whose rows the narrow product stages raw in LDS
+inline bool staged_super_block(int32_t element) { return element == NH_Q6_K || element == NH_Q5_K || element == NH_Q3_K; }
+
 inline uint32_t block_elements(int32_t element) {
     switch (element) {
     case NH_Q8_0: return Q8_0_BLOCK;
     case NH_Q4_K: return Q4_K_BLOCK;
+    case NH_Q3_K:
+    case NH_Q5_K:
     case NH_Q6_K: return Q6_K_BLOCK;
     case NH_F16:
     case NH_F32: return 1;

@@ -1,7 +1,7 @@
 // Wide products (prefill): Y[m][n] = sum_k X[m][k] * W[n][k], W in raw GGUF blocks.
 //
 // Tile 64 (m) x 64 (n) x 32 (k) per 256-thread workgroup.  The weight tile is dequantised
-// into LDS once per k step (one Q8_0 block / one Q4_K or Q6_K sub-block deep) and reused by all 64
+// into LDS once per k step (one Q8_0 block / one sub-block of a super-block format deep) and reused by all 64
 // activation rows; each thread owns a 4 x 4 patch of the output in registers.
 #include "blocks.hpp"
 #include "common.hpp"
@@ -52,14 +52,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint8_t *__restrict__ W
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 float value = 0.0f;
-                if (n < N && k0 + kk + j < K) {
-                    if (ELEMENT == NH_Q8_0)
-                        value = q8_0_element(row, k0 + kk + j);
-                    else if (ELEMENT == NH_Q6_K)
-                        value = q6_k_element(row, k0 + kk + j);
-                    else
-                        value = q4_k_element(row, k0 + kk + j);
-                }
+                if (n < N && k0 + kk + j < K) value = stored_element<ELEMENT>(row, k0 + kk + j);
                 ws[kk + j][r] = value;
             }
         }
@@ -476,6 +469,12 @@ int32_t launch_gemm(nh_device *d, const GemmArgs &a) {
     } else if (a.element == NH_Q6_K) {
         if (half) NH_GEMM(NH_Q6_K, true);
         else NH_GEMM(NH_Q6_K, false);
+    } else if (a.element == NH_Q5_K) {
+        if (half) NH_GEMM(NH_Q5_K, true);
+        else NH_GEMM(NH_Q5_K, false);
+    } else if (a.element == NH_Q3_K) {
+        if (half) NH_GEMM(NH_Q3_K, true);
+        else NH_GEMM(NH_Q3_K, false);
     } else {
         return fail(NH_E_ARGUMENT, "element %d carries no wide product", a.element);
     }

@@ -670,16 +670,120 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     }
 }
 
-// ---------------------------------------------------------------------------- Q6_K -------
+// ------------------------------------------------------------ Q6_K, Q5_K, Q3_K -------
 //
-// 210-byte super-blocks leave rows on 2-byte boundaries.  A wave copies the two rows it is about to walk into LDS with
-// aligned 128-bit loads -- a row is contiguous, the copy fully coalesced -- and its lanes pick the fields out of LDS
-// two bytes at a time.  A lane takes 16 weights of a super-block: four neighbouring elements of each of the four
-// 32-element groups of one half, which share two words of nibbles and one word of bit pairs
-// (crates/neura-precision/src/ggml.rs:394-407).  The weight is (d * scale) * (code - 32) as in
-// crates/neura-kernel/src/dot.rs:663-797; the sums run in lane order, not in the reference's run order.
-template <int RB>
-__global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
+// 210-, 176- and 110-byte super-blocks; the first and the last leave rows on 2-byte boundaries.  A wave copies the two
+// rows it is about to walk into LDS with aligned 128-bit loads -- a row is contiguous, the copy fully coalesced -- and its
+// lanes pick the fields out of LDS.  A lane takes 32 weights of a super-block: eight neighbouring elements
+// (8j .. 8j + 7) of each of the four 32-element runs of one half.  In all three formats those share one or two 8-byte
+// pieces of low bits and one of high bits, and each run has one scale for the eight:
+//   Q6_K (crates/neura-precision/src/ggml.rs:394-407, crates/neura-kernel/src/dot.rs:663-797): (d * scale) * (code - 32)
+//   Q5_K (ggml.rs:321-335, dot.rs:621-661): d * sc * code - dmin * m
+//   Q3_K (ggml.rs:291-306, dot.rs:544-581): (d * (scale - 32)) * (code - 4), the third bit being the code's top bit
+// Every run contributes weight * sum(x * code) - (weight * offset + minimum) * sum(x): the stored codes convert to fp32
+// with one instruction each, and the offset and the minimum cost one multiply-add per eight weights.  The sums run in
+// lane order, not in the reference's run order.
+__device__ __forceinline__ uint32_t byte_of(uint32_t word, uint32_t at) { return (word >> (8u * at)) & 0xffu; }
+
+template <int ELEMENT>
+struct Staged;
+
+template <>
+struct Staged<NH_Q6_K> {
+    static constexpr uint32_t BYTES = 210u;
+    static constexpr float OFFSET = 32.0f;
+    static constexpr bool FLOORS = false;
+    // codes[g][h]: elements 8j + 4h .. + 3 of run g, one code a byte
+    template <typename Word>
+    static __device__ __forceinline__ void unit(const uint8_t *block, Word word, uint32_t half, uint32_t j, uint32_t (&codes)[4][2], float (&weight)[4],
+                                                float (&floor)[4]) {
+        const float d = half_to_float(*reinterpret_cast<const uint16_t *>(block + 208u));
+        const uint32_t scales[2] = {word(192u + half * 8u), word(196u + half * 8u)};  // run g, elements 16c ..: byte 2g + c
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t lows = word(half * 64u + 8u * j + 4u * h), highs = word(half * 64u + 32u + 8u * j + 4u * h);
+            const uint32_t pairs = word(128u + half * 32u + 8u * j + 4u * h);
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint32_t nibbles = ((g & 1) ? highs : lows) >> (g >= 2 ? 4 : 0);
+                codes[g][h] = (nibbles & 0x0f0f0f0fu) | (((pairs >> (2 * g)) & 0x03030303u) << 4);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            weight[g] = d * (float)(int8_t)byte_of(scales[g >> 1], 2u * (g & 1) + (j >> 1));
+            floor[g] = 0.0f;
+        }
+    }
+};
+
+template <>
+struct Staged<NH_Q5_K> {
+    static constexpr uint32_t BYTES = 176u;
+    static constexpr float OFFSET = 0.0f;
+    static constexpr bool FLOORS = true;
+    template <typename Word>
+    static __device__ __forceinline__ void unit(const uint8_t *block, Word word, uint32_t half, uint32_t j, uint32_t (&codes)[4][2], float (&weight)[4],
+                                                float (&floor)[4]) {
+        // runs 0..3 of a half are sub-blocks 4 half + t: nibble group 2 half + t / 2, low nibbles for even t
+        const uint32_t header = word(0u);
+        const float d = half_to_float((uint16_t)header), dmin = half_to_float((uint16_t)(header >> 16));
+        const uint32_t s0 = word(4u), s1 = word(8u), s2 = word(12u);  // the twelve scale bytes (ggml.rs:127-136)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t first = word(48u + half * 64u + 8u * j + 4u * h), second = word(48u + half * 64u + 32u + 8u * j + 4u * h);
+            const uint32_t fifths = word(16u + 8u * j + 4u * h);
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint32_t nibbles = ((t & 2) ? second : first) >> ((t & 1) ? 4 : 0);
+                codes[t][h] = (nibbles & 0x0f0f0f0fu) | (((fifths >> (4u * half + t)) & 0x01010101u) << 4);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t a = byte_of(s0, t), b = byte_of(s1, t), c = byte_of(s2, t);
+            const uint32_t sc = half ? ((c & 15u) | ((a >> 6) << 4)) : (a & 63u);
+            const uint32_t mn = half ? ((c >> 4) | ((b >> 6) << 4)) : (b & 63u);
+            weight[t] = d * (float)sc;
+            floor[t] = dmin * (float)mn;
+        }
+    }
+};
+
+template <>
+struct Staged<NH_Q3_K> {
+    static constexpr uint32_t BYTES = 110u;
+    static constexpr float OFFSET = 4.0f;
+    static constexpr bool FLOORS = false;
+    template <typename Word>
+    static __device__ __forceinline__ void unit(const uint8_t *block, Word word, uint32_t half, uint32_t j, uint32_t (&codes)[4][2], float (&weight)[4],
+                                                float (&floor)[4]) {
+        const float d = half_to_float(*reinterpret_cast<const uint16_t *>(block + 108u));
+        const uint32_t lows[2] = {word(96u), word(100u)}, highs = word(104u);  // six-bit scales (ggml.rs:224-229)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t pairs = word(32u + half * 32u + 8u * j + 4u * h), thirds = word(8u * j + 4u * h);
+#pragma unroll
+            for (int t = 0; t < 4; t++) codes[t][h] = ((pairs >> (2 * t)) & 0x03030303u) | (((thirds >> (4u * half + t)) & 0x01010101u) << 2);
+        }
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            // scale 8 half + 2t + c, c = 1 for elements 16 .. 31 of the run: a nibble of byte 2t + c, two bits of byte 8 + (2t + c) % 4
+            const uint32_t at = 2u * (t & 1) + (j >> 1);
+            const uint32_t low = byte_of(lows[t >> 1], at);
+            const uint32_t nibble = half ? (low >> 4) : (low & 15u);
+            const uint32_t top = (byte_of(highs, at) >> (2u * (2u * half + (t >> 1)))) & 3u;
+            weight[t] = d * ((float)(nibble | (top << 4)) - 32.0f);
+            floor[t] = 0.0f;
+        }
+    }
+};
+
+__device__ __forceinline__ uint32_t skew128(uint32_t i) { return i + (i >> 7) * 4; }
+
+template <int ELEMENT, int RB>
+__global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
+    typedef Staged<ELEMENT> Format;
     extern __shared__ float xs[];  // [RB][slice]; then the raw row slices, two per wave
     __shared__ float red[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -688,14 +792,15 @@ __global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
     const uint32_t blk0 = split * p.blocks_per_split;
     const uint32_t nb = min(p.blocks_per_split, p.nblk - blk0);
     const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
-    const uint32_t xstride = p.blocks_per_split * 256u;
+    // halves of 128 activations sit 16 bytes apart: the lanes of a wave read eight of them at once
+    const uint32_t xstride = skew128(p.blocks_per_split * 256u);
     for (uint32_t b = 0; b < RB; b++) {
-        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return i; });
+        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew128(i); });
     }
     __syncthreads();
     const uint32_t raw_stride = p.chunks_per_row * 16u;  // bytes of one staged row slice
     uint8_t *const mine = reinterpret_cast<uint8_t *>(xs + RB * xstride) + (size_t)wave * 2u * raw_stride;
-    const uint32_t units = nb * 16u;
+    const uint32_t units = nb * 8u;
 
     // the 16-byte pieces of the two rows `first`, `first + 1` this lane copies: fetched one pair of rows ahead, so the copy
     // of the next pair is in flight while this pair is multiplied (a slice is at most 16 blocks: four pieces a lane and row)
@@ -707,10 +812,10 @@ __global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
         for (int r = 0; r < 2; r++) {
             const uint32_t i = min(first + r, p.N - 1u);
             const uint8_t *matrix_end;
-            const uint8_t *src = row_start(p, weight_row(i, p.N, p.swiglu), matrix_end) + (size_t)blk0 * 210u;
+            const uint8_t *src = row_start(p, weight_row(i, p.N, p.swiglu), matrix_end) + (size_t)blk0 * Format::BYTES;
             ahead_lead[r] = (uint32_t)((uintptr_t)src & 15u);
             const uint8_t *from = src - ahead_lead[r];
-            const uint32_t bytes = ahead_lead[r] + nb * 210u;
+            const uint32_t bytes = ahead_lead[r] + nb * Format::BYTES;
 #pragma unroll
             for (int k = 0; k < 4; k++) {
                 const uint32_t c = lane + 64u * k;
@@ -750,30 +855,42 @@ __global__ __launch_bounds__(256) void gemv_q6_k_kernel(GemvParams p) {
 #pragma unroll
             for (int b = 0; b < RB; b++) acc[r][b] = 0.0f;
         for (uint32_t u = lane; u < units; u += 64u) {
-            const uint32_t blk = u >> 4, half = (u >> 3) & 1u, j = u & 7u;
-            float4 xv[RB][4];
+            const uint32_t blk = u >> 3, half = (u >> 2) & 1u, j = u & 3u;
+            float4 xv[RB][4][2];
+            float xsum[RB][4];  // a code's offset and a run's minimum weigh the plain sum of the eight activations
 #pragma unroll
             for (int b = 0; b < RB; b++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) xv[b][g] = *reinterpret_cast<const float4 *>(xs + b * xstride + blk * 256u + half * 128u + g * 32u + 4u * j);
+                for (int g = 0; g < 4; g++) {
+                    const float4 *at = reinterpret_cast<const float4 *>(xs + b * xstride + skew128(blk * 256u + half * 128u) + g * 32u + 8u * j);
+                    xv[b][g][0] = at[0], xv[b][g][1] = at[1];
+                    xsum[b][g] = ((xv[b][g][0].x + xv[b][g][0].y) + (xv[b][g][0].z + xv[b][g][0].w)) +
+                                 ((xv[b][g][1].x + xv[b][g][1].y) + (xv[b][g][1].z + xv[b][g][1].w));
+                }
 #pragma unroll
             for (int r = 0; r < 2; r++) {
-                const uint8_t *block = mine + r * raw_stride + lead[r] + blk * 210u;
+                const uint8_t *block = mine + r * raw_stride + lead[r] + blk * Format::BYTES;
                 auto word = [&](uint32_t at) { return (uint32_t)*reinterpret_cast<const uint16_t *>(block + at) | ((uint32_t)*reinterpret_cast<const uint16_t *>(block + at + 2u) << 16); };
-                const uint32_t lows = word(half * 64u + 4u * j), highs = word(half * 64u + 32u + 4u * j), pairs = word(128u + half * 32u + 4u * j);
-                const float d = half_to_float(*reinterpret_cast<const uint16_t *>(block + 208u));
-                const uint8_t *scales = block + 192u + half * 8u + (j >> 2);
+                uint32_t codes[4][2];
+                float weight[4], floor[4];
+                Format::unit(block, word, half, j, codes, weight, floor);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const uint32_t nibbles = ((g & 1) ? highs : lows) >> (g >= 2 ? 4 : 0);
-                    const uint32_t codes = (nibbles & 0x0f0f0f0fu) | (((pairs >> (2 * g)) & 0x03030303u) << 4);
-                    const float weight = d * (float)(int8_t)scales[2 * g];
-                    const float c0 = (float)(codes & 0xffu) - 32.0f, c1 = (float)((codes >> 8) & 0xffu) - 32.0f;
-                    const float c2 = (float)((codes >> 16) & 0xffu) - 32.0f, c3 = (float)(codes >> 24) - 32.0f;
+                    const float low = Format::FLOORS ? fmaf(weight[g], Format::OFFSET, floor[g]) : weight[g] * Format::OFFSET;
 #pragma unroll
                     for (int b = 0; b < RB; b++) {
-                        const float dot = fmaf(xv[b][g].w, c3, fmaf(xv[b][g].z, c2, fmaf(xv[b][g].y, c1, xv[b][g].x * c0)));
-                        acc[r][b] = fmaf(weight, dot, acc[r][b]);
+                        float dot = 0.0f;
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            // the codes go to fp32 as they are stored, one conversion each; their offset leaves with the sum
+                            const uint32_t c = codes[g][h];
+                            dot = fmaf(xv[b][g][h].x, (float)(c & 0xffu), dot);
+                            dot = fmaf(xv[b][g][h].y, (float)((c >> 8) & 0xffu), dot);
+                            dot = fmaf(xv[b][g][h].z, (float)((c >> 16) & 0xffu), dot);
+                            dot = fmaf(xv[b][g][h].w, (float)(c >> 24), dot);
+                        }
+                        acc[r][b] = fmaf(weight[g], dot, acc[r][b]);
+                        acc[r][b] = fmaf(-low, xsum[b][g], acc[r][b]);
                     }
                 }
             }
@@ -1907,9 +2024,9 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     return NH_OK;
 }
 
-// Q6_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
-template <int RB>
-static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
+// Q6_K, Q5_K, Q3_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
+template <int ELEMENT, int RB>
+static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
     GemvParams p{};
     for (int s = 0; s < 3; s++) {
         p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
@@ -1917,7 +2034,7 @@ static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, 
     }
     p.x = x, p.y = y, p.residual = residual, p.norm_w = a.norm_w;
     p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps;
-    p.row_bytes = (uint32_t)payload_bytes(NH_Q6_K, a.K);
+    p.row_bytes = (uint32_t)payload_bytes(ELEMENT, a.K);
     p.nblk = a.K / 256u;
     const uint32_t most_blocks = 16u;
     p.splits = (p.nblk + most_blocks - 1) / most_blocks;
@@ -1927,14 +2044,14 @@ static int32_t launch_q6k_rows(nh_device *d, const GemvArgs &a, const float *x, 
         p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * RB * a.N * sizeof(float)));
         if (!p.partial) return NH_E_MEMORY;
     }
-    p.chunks_per_row = (15u + p.blocks_per_split * 210u + 15u) / 16u;
-    const size_t lds = (size_t)RB * p.blocks_per_split * 256u * sizeof(float) + (size_t)8 * p.chunks_per_row * 16u;
+    p.chunks_per_row = (15u + p.blocks_per_split * Staged<ELEMENT>::BYTES + 15u) / 16u;
+    const size_t lds = (size_t)RB * p.blocks_per_split * 264u * sizeof(float) + (size_t)8 * p.chunks_per_row * 16u;  // slices, 8 floats of skew a block
     uint32_t blocks_x = (a.N + 7u) / 8u;
-    uint32_t most = (uint32_t)d->compute_units * 2u / p.splits;
+    uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_STAGED_WGS", 2) / p.splits;
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
     profile_mark(d);
-    hipLaunchKernelGGL((gemv_q6_k_kernel<RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_staged_kernel<ELEMENT, RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, p);
     NH_HIP(hipGetLastError());
     if (p.splits > 1) {
         uint32_t outputs = (a.swiglu ? a.N / 2 : a.N) * RB;
@@ -1955,14 +2072,20 @@ int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     // activation rows are taken four, two or one at a time
     uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
     uint32_t done = 0;
-    if (a.element == NH_Q6_K) {
+    if (staged_super_block(a.element)) {
         if (a.swiglu && (a.N % 2u || a.end[0] != a.N / 2)) return fail(NH_E_ARGUMENT, "a swiglu product halves %u rows", a.N);
         while (done < a.rows) {
             const float *x = a.x + (size_t)done * a.K;
             float *y = a.y + (size_t)done * outputs;
             const float *residual = a.residual ? a.residual + (size_t)done * a.N : nullptr;
             const bool pair = a.rows - done >= 2;
-            int32_t status = pair ? launch_q6k_rows<2>(d, a, x, y, residual) : launch_q6k_rows<1>(d, a, x, y, residual);
+            int32_t status;
+            if (a.element == NH_Q6_K)
+                status = pair ? launch_staged_rows<NH_Q6_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q6_K, 1>(d, a, x, y, residual);
+            else if (a.element == NH_Q5_K)
+                status = pair ? launch_staged_rows<NH_Q5_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q5_K, 1>(d, a, x, y, residual);
+            else
+                status = pair ? launch_staged_rows<NH_Q3_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q3_K, 1>(d, a, x, y, residual);
             if (status != NH_OK) return status;
             done += pair ? 2 : 1;
         }

@@ -231,8 +231,8 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     std::vector<int32_t> elements(2 + 7 * (size_t)c.layers, table->matrix_element);
     if (table->matrix_elements) elements.assign(table->matrix_elements, table->matrix_elements + elements.size());
     for (int32_t element : elements) {
-        if (element != NH_Q8_0 && element != NH_Q4_K && element != NH_Q6_K) {
-            fail(NH_E_ARGUMENT, "a decoder multiplies Q8_0, Q4_K or Q6_K matrices, and this table names element %d", element);
+        if (element != NH_Q8_0 && element != NH_Q4_K && !staged_super_block(element)) {
+            fail(NH_E_ARGUMENT, "a decoder multiplies Q8_0, Q3_K, Q4_K, Q5_K or Q6_K matrices, and this table names element %d", element);
             return nullptr;
         }
         uint32_t block = block_elements(element);
@@ -515,7 +515,8 @@ int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elemen
 int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
                 float *dev_y, const nh_epilogue *epilogue) {
     NH_REQUIRE(device && dev_W && dev_x && dev_y, "a product names no device or no buffer");
-    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || element == NH_Q6_K, "a narrow product walks Q8_0, Q4_K or Q6_K weights, not element %d", element);
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || staged_super_block(element),
+               "a narrow product walks Q8_0, Q3_K, Q4_K, Q5_K or Q6_K weights, not element %d", element);
     NH_REQUIRE(N > 0 && K > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K, block_elements(element));
     NH_REQUIRE(rows >= 1 && rows <= 8, "a narrow product takes one to eight rows, not %u", rows);
     NH_REQUIRE(aligned16(dev_W) && aligned16(dev_x), "a product reads its weights and activations from 16-byte aligned addresses");
@@ -532,8 +533,8 @@ int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t 
             NH_REQUIRE(N % 2 == 0, "a swiglu product halves %u rows", N);
             a.W[1] = static_cast<const uint8_t *>(dev_W) + (size_t)(N / 2) * payload_bytes(element, K);
             a.end[0] = N / 2;
-            // Q6_K rows are read through aligned copies whatever their own alignment
-            NH_REQUIRE(element == NH_Q6_K || aligned16(a.W[1]), "the up half of a swiglu product starts off a 16-byte boundary");
+            // Q6_K, Q5_K and Q3_K rows are read through aligned copies whatever their own alignment
+            NH_REQUIRE(staged_super_block(element) || aligned16(a.W[1]), "the up half of a swiglu product starts off a 16-byte boundary");
         }
     }
     return launch_gemv(device, a);
@@ -542,7 +543,8 @@ int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t 
 int32_t nh_gemm(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const void *dev_X, int32_t x_element,
                 uint32_t M, float *dev_Y, const nh_epilogue *epilogue) {
     NH_REQUIRE(device && dev_W && dev_X && dev_Y, "a product names no device or no buffer");
-    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || element == NH_Q6_K, "a wide product walks Q8_0, Q4_K or Q6_K weights, not element %d", element);
+    NH_REQUIRE(element == NH_Q8_0 || element == NH_Q4_K || staged_super_block(element),
+               "a wide product walks Q8_0, Q3_K, Q4_K, Q5_K or Q6_K weights, not element %d", element);
     NH_REQUIRE(x_element == NH_F32 || x_element == NH_F16, "a wide product takes fp32 or fp16 activations, not element %d", x_element);
     NH_REQUIRE(N > 0 && K > 0 && M > 0 && K % block_elements(element) == 0, "a row of %u numbers is not whole blocks of %u", K,
                block_elements(element));

@@ -817,7 +817,7 @@ class Model {
         const uint32_t H = config.hidden, QW = config.heads * config.head_width, KW = config.key_heads * config.head_width, F = config.feed_forward;
         std::vector<std::string> names;
         // tensor names of a Qwen2 GGUF (the reference's qwen35 example names them alike, examples/qwen/attention.rs:40-78, mlp.rs:22-25)
-        // every matrix keeps the storage the file gives it (a Q4_K_M file mixes q4_k and q6_k); the q, k and v projections of
+        // every matrix keeps the storage the file gives it (a Q4_K_M file mixes q4_k and q6_k, a Q3_K_M file q3_k, q4_k and q5_k); the q, k and v projections of
         // Qwen2 checkpoints carry biases the reference's own example has no tensors for
         Element element = decoder::matrix(archive, "token_embd.weight", config.vocabulary, H).element;
         std::vector<int32_t> elements;
@@ -826,8 +826,9 @@ class Model {
                 NEURA_ASSERT(parameter.element == Element::Single, "this decoder reads norm weights and biases in single storage, and %s holds %s storage",
                              parameter.name.c_str(), name(parameter.element));
             } else {
-                NEURA_ASSERT(parameter.element == Element::Q8_0 || parameter.element == Element::Q4K || parameter.element == Element::Q6K,
-                             "this decoder multiplies q8_0, q4_k and q6_k matrices, and %s holds %s storage", parameter.name.c_str(),
+                NEURA_ASSERT(parameter.element == Element::Q8_0 || parameter.element == Element::Q3K || parameter.element == Element::Q4K ||
+                                 parameter.element == Element::Q5K || parameter.element == Element::Q6K,
+                             "this decoder multiplies q8_0, q3_k, q4_k, q5_k and q6_k matrices, and %s holds %s storage", parameter.name.c_str(),
                              name(parameter.element));
                 elements.push_back((int32_t)parameter.element);
             }

@@ -20,6 +20,11 @@
  *                            dequantize_row_q8_0 / dequantize_row_q4_K + hand-built blocks
  *   q8_0 / q4_k pack ....... pinned: invariants (|unpack(pack(x)) - x| <= d/2, codes in
  *                            range) + independent numpy restatement
+ *   q3_k unpack ............ pinned: the reference's own known-answer block (bytes at*37+11, at*53+7, at*19+3,
+ *                            d = 0.25: crates/neura-precision/tests/format.rs:221-234) walked by a numpy
+ *                            restatement of ggml's published dequantize_row_q3_K, + its round-trip bound (:236-245)
+ *   q5_k / q6_k unpack ..... pinned: numpy restatements of ggml's published dequantize_row_q5_K / _q6_K + hand-built blocks
+ *   q3_k / q5_k / q6_k pack  pinned: round-trip bounds and field invariants
  *   gemv / gemm ............ pinned: the reference's own test definition (fp32 triple
  *                            loop over unpack, runtime.rs:72-83) + fp64 numpy
  *   rmsnorm ................ pinned: composed form tests/norm.rs:21-26
@@ -42,13 +47,17 @@
 #define Q4_K_BYTES 144
 #define Q6_K_BLOCK 256
 #define Q6_K_BYTES 210 /* 128 low nibbles, 64 bytes of high bit pairs, 16 int8 scales, f16 d: neura-abi/src/element.rs:167-170 */
+#define Q5_K_BLOCK 256
+#define Q5_K_BYTES 176 /* f16 d, f16 dmin, 12 scale bytes, 32 bytes of fifth bits, 128 nibble bytes: neura-abi/src/element.rs:163-166 */
+#define Q3_K_BLOCK 256
+#define Q3_K_BYTES 110 /* 32 bytes of third bits, 64 bytes of bit pairs, 12 scale bytes, f16 d: neura-abi/src/element.rs:171-174 */
 #define SUB_BLOCK 32
 #define FOLDED_LANES 32   /* neura-profile/src/profile.rs:1327 */
 #define FOLDED_STAGE 1024 /* neura-profile/src/profile.rs:1358 */
 #define WORKGROUP 256     /* neura-profile/src/profile.rs:2086-2089 */
 #define ATTN_KEYS 16      /* neura-profile/src/profile.rs:70 */
 
-enum { EL_F32 = 0, EL_F16 = 1, EL_Q8_0 = 8, EL_Q4_K = 12, EL_Q6_K = 14 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
+enum { EL_F32 = 0, EL_F16 = 1, EL_Q8_0 = 8, EL_Q3_K = 11, EL_Q4_K = 12, EL_Q5_K = 13, EL_Q6_K = 14 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
 
 /* ---------------------------------------------------------------- f16 ---- */
 
@@ -199,6 +208,54 @@ static void q6_k_values(const uint8_t *field, float *out) {
             }
 }
 
+/* crates/neura-precision/src/ggml.rs:321-335: Q4_K's walk with a fifth bit per code, bit 2*group + seat of byte 16 + within */
+static void q5_k_values(const uint8_t *field, float *out) {
+    uint16_t h0, h1;
+    memcpy(&h0, field, 2);
+    memcpy(&h1, field + 2, 2);
+    float scale = oracle_f16_to_f32(h0);
+    float min = oracle_f16_to_f32(h1);
+    for (uint32_t group = 0; group < 4; group++) {
+        for (uint32_t seat = 0; seat < 2; seat++) {
+            uint32_t code, offset;
+            oracle_scale_min_k4(field + 4, group * 2 + seat, &code, &offset);
+            float quantum = scale * (float)code;
+            float low = min * (float)offset;
+            for (uint32_t within = 0; within < SUB_BLOCK; within++) {
+                uint32_t high = ((uint32_t)field[16 + within] >> (2 * group + seat)) & 1u;
+                uint8_t byte = field[48 + group * 32 + within];
+                uint32_t quant = (seat ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f)) | (high << 4);
+                *out++ = quantum * (float)quant - low;
+            }
+        }
+    }
+}
+
+/* 6-bit scale `at` (0..15) of a Q3_K super-block: crates/neura-precision/src/ggml.rs:224-229 */
+static uint32_t q3_k_scale(const uint8_t *field, uint32_t at) {
+    uint8_t low = field[96 + at % 8];
+    uint32_t nibble = at < 8 ? (uint32_t)(low & 0x0f) : (uint32_t)(low >> 4);
+    uint8_t high = field[96 + 8 + at % 4];
+    return nibble | ((((uint32_t)high >> (2 * (at / 4))) & 3u) << 4);
+}
+
+/* crates/neura-precision/src/ggml.rs:291-306: sixteen sub-blocks of 16; code = two bits minus 4 unless the third bit is set;
+ * value = d * (scale - 32) * code, left to right */
+static void q3_k_values(const uint8_t *field, float *out) {
+    uint16_t h;
+    memcpy(&h, field + 108, 2);
+    float d = oracle_f16_to_f32(h);
+    for (uint32_t at = 0; at < Q3_K_BLOCK; at++) {
+        uint32_t sub = at / 16, lane = at % 16;
+        uint32_t half = sub / 8, within = sub % 8, j = within / 2, second = within % 2;
+        uint32_t low = ((uint32_t)field[32 + half * 32 + second * 16 + lane] >> (2 * j)) & 3u;
+        int high = (field[second * 16 + lane] & (1u << (half * 4 + j))) != 0;
+        int quant = (int)low - (high ? 0 : 4);
+        float product = d * ((float)(uint8_t)q3_k_scale(field, sub) - 32.0f);
+        out[at] = product * (float)quant;
+    }
+}
+
 /* crates/neura-precision/src/ggml.rs:22-38 (unpack); elements must be whole blocks */
 int oracle_unpack(int element, const uint8_t *bytes, uint64_t elements, float *out) {
     if (element == EL_Q8_0) {
@@ -214,6 +271,16 @@ int oracle_unpack(int element, const uint8_t *bytes, uint64_t elements, float *o
     if (element == EL_Q6_K) {
         if (elements % Q6_K_BLOCK) return -1;
         for (uint64_t b = 0; b < elements / Q6_K_BLOCK; b++) q6_k_values(bytes + b * Q6_K_BYTES, out + b * Q6_K_BLOCK);
+        return 0;
+    }
+    if (element == EL_Q5_K) {
+        if (elements % Q5_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < elements / Q5_K_BLOCK; b++) q5_k_values(bytes + b * Q5_K_BYTES, out + b * Q5_K_BLOCK);
+        return 0;
+    }
+    if (element == EL_Q3_K) {
+        if (elements % Q3_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < elements / Q3_K_BLOCK; b++) q3_k_values(bytes + b * Q3_K_BYTES, out + b * Q3_K_BLOCK);
         return 0;
     }
     if (element == EL_F16) {
@@ -246,10 +313,11 @@ static void q8_0_encode(const float *values, uint8_t *out) {
 static float least(float a, float b) { return a < b ? a : b; }
 static float greatest(float a, float b) { return a > b ? a : b; }
 
-/* crates/neura-precision/src/ggml.rs:149-199 (affine_block for Q4K: steps 15, sub 32) */
-static void q4_k_encode(const float *values, uint8_t *field) {
+/* crates/neura-precision/src/ggml.rs:149-199 (affine_block; Q4K: steps 15, nibbles at 16; Q5K: steps 31, fifth bits at 16, nibbles at 48) */
+static void affine_encode(const float *values, uint8_t *field, int fifth) {
     const int count = Q4_K_BLOCK / SUB_BLOCK;
-    const float steps = 15.0f;
+    const float steps = fifth ? 31.0f : 15.0f;
+    const int quants = fifth ? 48 : 16;
     float lows[8], quantums[8];
     for (int at = 0; at < count; at++) {
         float low = 0.0f, high = 0.0f; /* span folds from (0,0): ggml.rs:110-114 */
@@ -272,7 +340,7 @@ static void q4_k_encode(const float *values, uint8_t *field) {
         codes[at] = (uint8_t)clampf(round_away(c), 0.0f, 63.0f);
         mins[at] = (uint8_t)clampf(round_away(m), 0.0f, 63.0f);
     }
-    memset(field, 0, Q4_K_BYTES);
+    memset(field, 0, fifth ? Q5_K_BYTES : Q4_K_BYTES);
     for (int at = 0; at < count; at++) oracle_put_scale_min_k4(field + 4, (uint32_t)at, codes[at], mins[at]);
     uint16_t h = oracle_f32_to_f16(scale);
     memcpy(field, &h, 2);
@@ -286,9 +354,50 @@ static void q4_k_encode(const float *values, uint8_t *field) {
             if (quantum != 0.0f) code = (uint32_t)clampf(round_away((values[at * SUB_BLOCK + within] + low) / quantum), 0.0f, steps);
             int group = at / 2;
             int seat = at % 2;
-            field[16 + group * SUB_BLOCK + within] |= (uint8_t)((code & 0x0f) << (seat ? 4 : 0));
+            field[quants + group * SUB_BLOCK + within] |= (uint8_t)((code & 0x0f) << (seat ? 4 : 0));
+            if (fifth && (code & 0x10)) field[16 + within] |= (uint8_t)(1u << (2 * group + seat));
         }
     }
+}
+
+static void q4_k_encode(const float *values, uint8_t *field) { affine_encode(values, field, 0); }
+static void q5_k_encode(const float *values, uint8_t *field) { affine_encode(values, field, 1); } /* ggml.rs:313-315 */
+
+/* crates/neura-precision/src/ggml.rs:242-289: sixteen sub-blocks of 16, d = widest / 4 / 31, scale codes 32..63
+ * (stored six bits: four in a nibble of bytes 96..103, two in bytes 104..107), codes round(x / (d * scale)) in -4..3 */
+static void q3_k_encode(const float *values, uint8_t *field) {
+    float peaks[16];
+    for (int at = 0; at < 16; at++) {
+        float peak = 0.0f;
+        for (int i = 0; i < 16; i++) peak = greatest(peak, fabsf(values[at * 16 + i]));
+        peaks[at] = peak;
+    }
+    float widest = 0.0f;
+    for (int at = 0; at < 16; at++) widest = greatest(widest, peaks[at]);
+    if (!(widest >= 1.17549435e-38f)) widest = 1.17549435e-38f; /* f32::max(MIN_POSITIVE) */
+    float d = widest / 4.0f / 31.0f;
+    uint32_t codes[16];
+    for (int at = 0; at < 16; at++) codes[at] = (uint32_t)clampf(round_away(peaks[at] / 4.0f / d), 0.0f, 31.0f) + 32u;
+    memset(field, 0, Q3_K_BYTES);
+    for (uint32_t at = 0; at < 16; at++) { /* put_q3_k_scale, ggml.rs:231-240 */
+        uint8_t low = (uint8_t)(codes[at] & 0x0f), high = (uint8_t)((codes[at] >> 4) & 3u);
+        if (at < 8)
+            field[96 + at] |= low;
+        else
+            field[96 + at - 8] |= (uint8_t)(low << 4);
+        field[96 + 8 + at % 4] |= (uint8_t)(high << (2 * (at / 4)));
+    }
+    for (uint32_t at = 0; at < Q3_K_BLOCK; at++) {
+        uint32_t sub = at / 16, lane = at % 16;
+        float quantum = d * (float)(codes[sub] - 32u);
+        int quant = 0;
+        if (quantum != 0.0f) quant = (int)clampf(round_away(values[at] / quantum), -4.0f, 3.0f);
+        uint32_t half = sub / 8, within = sub % 8, j = within / 2, second = within % 2;
+        field[32 + half * 32 + second * 16 + lane] |= (uint8_t)(((uint32_t)quant & 3u) << (2 * j));
+        if (quant >= 0) field[second * 16 + lane] |= (uint8_t)(1u << (half * 4 + j));
+    }
+    uint16_t h = oracle_f32_to_f16(d);
+    memcpy(field + 108, &h, 2);
 }
 
 /* crates/neura-precision/src/ggml.rs:352-392.  Sixteen sub-blocks of 16: factor = largest magnitude / 32, super scale =
@@ -352,6 +461,16 @@ int oracle_pack(int element, const float *values, uint64_t n, uint8_t *out) {
         for (uint64_t b = 0; b < n / Q6_K_BLOCK; b++) q6_k_encode(values + b * Q6_K_BLOCK, out + b * Q6_K_BYTES);
         return 0;
     }
+    if (element == EL_Q5_K) {
+        if (n % Q5_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < n / Q5_K_BLOCK; b++) q5_k_encode(values + b * Q5_K_BLOCK, out + b * Q5_K_BYTES);
+        return 0;
+    }
+    if (element == EL_Q3_K) {
+        if (n % Q3_K_BLOCK) return -1;
+        for (uint64_t b = 0; b < n / Q3_K_BLOCK; b++) q3_k_encode(values + b * Q3_K_BLOCK, out + b * Q3_K_BYTES);
+        return 0;
+    }
     if (element == EL_F16) {
         oracle_f32_to_f16_many(values, n, (uint16_t *)out);
         return 0;
@@ -368,6 +487,8 @@ uint64_t oracle_payload_bytes(int element, uint64_t elements) { /* neura-abi/src
     case EL_Q8_0: return (elements + Q8_0_BLOCK - 1) / Q8_0_BLOCK * Q8_0_BYTES;
     case EL_Q4_K: return (elements + Q4_K_BLOCK - 1) / Q4_K_BLOCK * Q4_K_BYTES;
     case EL_Q6_K: return (elements + Q6_K_BLOCK - 1) / Q6_K_BLOCK * Q6_K_BYTES;
+    case EL_Q5_K: return (elements + Q5_K_BLOCK - 1) / Q5_K_BLOCK * Q5_K_BYTES;
+    case EL_Q3_K: return (elements + Q3_K_BLOCK - 1) / Q3_K_BLOCK * Q3_K_BYTES;
     case EL_F16: return elements * 2;
     case EL_F32: return elements * 4;
     default: return 0;
@@ -425,6 +546,43 @@ static float run_dot(int element, const uint8_t *w_row, uint32_t k0, const float
         }
         return total;
     }
+    if (element == EL_Q5_K) { /* crates/neura-kernel/src/dot.rs:621-661: weight = scale * f32(nibble | fifth << 4) - min */
+        const uint8_t *field = w_row + (size_t)(k0 / Q5_K_BLOCK) * Q5_K_BYTES;
+        uint32_t within = k0 % Q5_K_BLOCK;
+        uint32_t group = within / 64u, seat = (within % 64u) / SUB_BLOCK;
+        uint32_t sc, m;
+        oracle_scale_min_k4(field + 4, group * 2 + seat, &sc, &m);
+        uint16_t h0, h1;
+        memcpy(&h0, field, 2);
+        memcpy(&h1, field + 2, 2);
+        float scale = oracle_f16_to_f32(h0) * (float)sc;
+        float min = oracle_f16_to_f32(h1) * (float)m;
+        for (uint32_t at = 0; at < last; at++) {
+            uint8_t byte = field[48 + group * 32 + at];
+            uint32_t nibble = seat ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 0x0f);
+            uint32_t quant = nibble | ((((uint32_t)field[16 + at] >> (2 * group + seat)) & 1u) << 4);
+            total = total + x[k0 + at] * (scale * (float)quant - min);
+        }
+        return total;
+    }
+    if (element == EL_Q3_K) { /* crates/neura-kernel/src/dot.rs:544-581: weight = (d * (scale - 32)) * (pair - 4 unless the third bit is set) */
+        const uint8_t *field = w_row + (size_t)(k0 / Q3_K_BLOCK) * Q3_K_BYTES;
+        uint32_t within = k0 % Q3_K_BLOCK;
+        uint32_t group = within / SUB_BLOCK, half = group / 4u, j = group % 4u;
+        uint16_t h;
+        memcpy(&h, field + 108, 2);
+        float width = oracle_f16_to_f32(h);
+        float scale0 = width * ((float)q3_k_scale(field, half * 8 + j * 2) - 32.0f);
+        float scale1 = width * ((float)q3_k_scale(field, half * 8 + j * 2 + 1) - 32.0f);
+        for (uint32_t at = 0; at < last; at++) {
+            uint32_t low = ((uint32_t)field[32 + half * 32 + at] >> (2 * j)) & 3u;
+            uint32_t high = ((uint32_t)field[at] >> (half * 4 + j)) & 1u;
+            float scale = at >= 16 ? scale1 : scale0;
+            float weight = scale * ((float)low - (high == 0u ? 4.0f : 0.0f));
+            total = total + x[k0 + at] * weight;
+        }
+        return total;
+    }
     if (element == EL_F16) {
         const uint16_t *w = (const uint16_t *)w_row;
         for (uint32_t at = 0; at < last; at++) total = total + x[k0 + at] * oracle_f16_to_f32(w[k0 + at]);
@@ -473,7 +631,7 @@ static float folded_dot(int element, const uint8_t *w_row, uint32_t K, const flo
 /* y[r][n] = Σ_k x[r][k]·W[n][k], W row-major [N][K] in `element` storage, order as above.
  * threads > 1 splits the N loop (every output keeps its own serial order). */
 int oracle_gemv(int element, const uint8_t *W, uint32_t N, uint32_t K, const float *x, uint32_t rows, float *y, int threads) {
-    if (element != EL_Q8_0 && element != EL_Q4_K && element != EL_Q6_K && element != EL_F16 && element != EL_F32) return -2;
+    if (element != EL_Q8_0 && element != EL_Q4_K && element != EL_Q6_K && element != EL_Q5_K && element != EL_Q3_K && element != EL_F16 && element != EL_F32) return -2;
     size_t stride = row_bytes(element, K);
     (void)threads;
 #pragma omp parallel for num_threads(threads > 0 ? threads : 1) schedule(static)

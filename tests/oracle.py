@@ -11,6 +11,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 LIBRARY = os.path.join(ORACLE_DIR, "libneura_oracle.so")
 
 EL_F32, EL_F16, EL_Q8_0, EL_Q4_K, EL_Q6_K = 0, 1, 8, 12, 14
+EL_Q3_K, EL_Q5_K = 11, 13
 
 
 class OracleModel(ctypes.Structure):

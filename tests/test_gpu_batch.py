@@ -8,7 +8,7 @@ import pytest
 
 import oracle
 from gguf_fixture import build as build_gguf
-from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, host, synth
+from neura_amd import NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K, NH_Q8_0, host, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -85,11 +85,19 @@ def test_a_batched_sequence_answers_as_it_does_alone(runtime, tmp_path, shape, e
     archive.close()
 
 
-def test_a_file_of_mixed_storage_with_projection_biases_generates(runtime, tmp_path):
+MIXED_FILES = {
     # the way Q4_K_M files of Qwen2 checkpoints come: q6_k for the head, some value and down projections; biases on q, k, v
+    "q4_k_m": (NH_Q4_K, {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.1.ffn_down.weight": NH_Q6_K}),
+    # and Q3_K_M files: q3_k for most, q5_k and q4_k for some projections, a q6_k head
+    "q3_k_m": (NH_Q3_K, {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.ffn_down.weight": NH_Q5_K, "blk.1.attn_output.weight": NH_Q4_K}),
+}
+
+
+@pytest.mark.parametrize("kind", sorted(MIXED_FILES))
+def test_a_file_of_mixed_storage_with_projection_biases_generates(runtime, tmp_path, kind):
     shape = SHAPE_Q4
-    mixed = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.1.ffn_down.weight": NH_Q6_K}
-    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, NH_Q4_K, seed=31, elements=mixed, biases=(0, 1))
+    base, mixed = MIXED_FILES[kind]
+    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, base, seed=31, elements=mixed, biases=(0, 1))
     archive = host.GgufFile.open(tmp_path / "model.gguf")
     batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [16])
     rng = np.random.default_rng(32)
@@ -97,7 +105,7 @@ def test_a_file_of_mixed_storage_with_projection_biases_generates(runtime, tmp_p
     slots = [batch.admit(prompt) for prompt in prompts]
     got = run(batch, {slot: 6 for slot in slots})
     for slot, prompt in zip(slots, prompts):
-        want, margin = alone(shape, NH_Q4_K, tensors, prompt, 6, elements=mixed)
+        want, margin = alone(shape, base, tensors, prompt, 6, elements=mixed)
         assert got[slot] == want, (slot, margin)
     batch.close()
     archive.close()

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 
 import oracle
-from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
+from neura_amd import NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
 from neura_amd.loader import Model, Weights
 
 pytestmark = pytest.mark.gpu
@@ -82,21 +82,25 @@ def test_masked_planes_and_chunked_fill(device):
 
 
 MIXED = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.2.ffn_down.weight": NH_Q6_K, "blk.2.ffn_gate.weight": NH_Q6_K}
+# the way Q3_K_M files are: Q3_K for most, Q5_K and Q4_K for some projections, a Q6_K head
+MIXED_3 = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.ffn_down.weight": NH_Q5_K, "blk.1.attn_output.weight": NH_Q4_K,
+           "blk.2.attn_q.weight": NH_Q4_K, "blk.2.attn_k.weight": NH_Q4_K, "blk.2.attn_v.weight": NH_Q4_K, "blk.2.ffn_up.weight": NH_Q5_K}
 
 
+@pytest.mark.parametrize("base,mixed", [(NH_Q4_K, MIXED), (NH_Q3_K, MIXED_3)], ids=["q4_k_m", "q3_k_m"])
 @pytest.mark.parametrize("batch", [1, 2])
-def test_mixed_elements_and_projection_biases(device, batch):
+def test_mixed_elements_and_projection_biases(device, batch, base, mixed):
     """A decoder stored the way Q4_K_M files are (Q6_K for some matrices, Q4_K for the rest) whose q, k and v projections
     carry Qwen2's biases: layer 0 (a Q6_K value projection, biases) takes one product per matrix, layer 1 (one element,
     biases) folds rotation and biases into the stacked product at batch 1, layer 2 (gate and up stored differently) runs
     the two halves apart.  Decode steps, a 16-row fill and the caches against the oracle."""
     shape = SMALL_Q4
     rng = np.random.default_rng(21)
-    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="normal", elements=MIXED, biases=(0, 1)))
+    tensors = list(synth.model_tensors(shape, base, rng, mode="normal", elements=mixed, biases=(0, 1)))
     host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
-    model = Model(device, weights, shape, NH_Q4_K, batch, 40, 16)
-    ref = oracle.Model(shape, NH_Q4_K, host, batch, 40, 16, elements=MIXED)
+    model = Model(device, weights, shape, base, batch, 40, 16)
+    ref = oracle.Model(shape, base, host, batch, 40, 16, elements=mixed)
     prompt = rng.integers(0, shape["vocab"], (16, batch))
     model.prefill(prompt.reshape(-1), 16, [0] * batch)
     ref.forward(prompt.reshape(-1), 16, [0] * batch, want_logits=False)

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle
-from neura_amd import NH_Q4_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
+from neura_amd import NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -27,7 +27,7 @@ def tight(got, want, scale=1e-5):
 
 # ------------------------------------------------------------------ codecs
 
-@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K, NH_Q6_K])
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K])
 def test_dequant_is_bit_exact(device, element):
     rng = np.random.default_rng(100 + element)
     elements = 256 * 4000
@@ -46,7 +46,7 @@ def test_dequant_refuses_ragged_and_unknown(device):
     with pytest.raises(NeuraError):
         device.dequant(NH_Q4_K, raw, 100)
     with pytest.raises(NeuraError):
-        device.dequant(11, raw, 256)
+        device.dequant(10, raw, 256)  # Q2_K: the reference reads it neither (crates/neura-gguf/src/header.rs:150-162)
 
 
 def test_convert_half_is_bit_exact(device):
@@ -59,7 +59,7 @@ def test_convert_half_is_bit_exact(device):
     assert np.array_equal(device.convert_half(values), oracle.f32_to_f16(values))
 
 
-@pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536), (NH_Q6_K, 768)])
+@pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536), (NH_Q6_K, 768), (NH_Q5_K, 512), (NH_Q3_K, 768)])
 def test_gather_is_the_dequantised_row_times_mask(device, element, width):
     rng = np.random.default_rng(102)
     vocab = 50
@@ -99,10 +99,10 @@ def test_config2_q4_k_gemvs_of_a_1_5b_layer(device, name, N, K):
     tight(got, want, 2e-6)
 
 
-@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K])
 @pytest.mark.parametrize("rows", [1, 2, 3, 4, 7, 8])
 def test_reference_narrow_product_test(device, element, rows):
-    # crates/neura-runtime/tests/runtime.rs:12-86 at its own shape and seeds
+    # crates/neura-runtime/tests/runtime.rs:12-86 at its own shape, seeds and elements
     depth, columns = 2048, 1024
     payload = oracle.pack(element, oracle.random(columns * depth, 23))
     inputs = oracle.random(rows * depth, 29).reshape(rows, depth)
@@ -200,33 +200,38 @@ def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device
     assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
 
 
+@pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K, NH_Q3_K])
 @pytest.mark.parametrize("N,K,rows", [(2, 256, 1), (7, 512, 3), (272, 3584, 1), (64, 1536, 8), (32, 18944, 1), (33, 18944, 5), (1040, 768, 2)])
-def test_q6_k_products(device, N, K, rows):
-    """Q6_K rows start on 2-byte boundaries (210-byte blocks): every alignment of a row, odd row counts, rows deeper than
-    one LDS stage (K slices folded by a second kernel), 1..8 activation rows, plain, residual and SwiGLU."""
-    rng = np.random.default_rng(N + K + rows)
-    raw = synth.q6_k_random(rng, N * K)
+def test_staged_super_block_products(device, element, N, K, rows):
+    """Q6_K and Q3_K rows start on 2-byte boundaries (210- and 110-byte blocks), Q5_K rows on 16-byte ones: every alignment
+    of a row, odd row counts, rows deeper than one LDS stage (K slices folded by a second kernel), 1..8 activation rows,
+    plain, residual and SwiGLU."""
+    rng = np.random.default_rng(N + K + rows + element)
+    raw = synth.RANDOM[element](rng, N * K)
     x = rng.standard_normal((rows, K)).astype(np.float32)
     r = rng.standard_normal((rows, N)).astype(np.float32)
-    plain = oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8)
-    exact = oracle.unpack(NH_Q6_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
-    got = device.gemv(NH_Q6_K, raw, N, K, x)
+    plain = oracle.gemv(element, raw, N, K, x, threads=8)
+    exact = oracle.unpack(element, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+    got = device.gemv(element, raw, N, K, x)
     close(got, plain)
     tight(got, plain, 3e-6)
     assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * max(1.0, np.abs(exact).max()))
-    tight(device.gemv(NH_Q6_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    tight(device.gemv(element, raw, N, K, x, residual=r), r + plain, 1e-5)
     if N % 2 == 0:
         gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2:].astype(np.float64)
         want = gate / (1.0 + np.exp(-gate)) * up
-        close(device.gemv(NH_Q6_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+        close(device.gemv(element, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
 
 
-def test_q6_k_product_reads_packed_weights_and_fuses_the_norm(device):
-    rng = np.random.default_rng(14)
+@pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K, NH_Q3_K])
+def test_staged_super_block_product_reads_packed_weights(device, element):
     N, K = 96, 2048
-    raw = oracle.pack(NH_Q6_K, np.abs(oracle.random(N * K, 23)))  # the reference's packing keeps non-negative values
+    values = oracle.random(N * K, 23)
+    if element == NH_Q6_K:
+        values = np.abs(values)  # the reference's Q6_K packing keeps non-negative values alone
+    raw = oracle.pack(element, values)
     x = oracle.random(K, 29).reshape(1, K)
-    tight(device.gemv(NH_Q6_K, raw, N, K, x), oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8), 2e-6)
+    tight(device.gemv(element, raw, N, K, x), oracle.gemv(element, raw, N, K, x, threads=8), 2e-6)
 
 
 def test_gemv_is_linear_and_matches_at_full_size(device):
@@ -255,7 +260,7 @@ def test_gemv_refuses_bad_shapes(device):
 
 # ------------------------------------------------------------------ wide products
 
-@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K])
+@pytest.mark.parametrize("element", [NH_Q8_0, NH_Q4_K, NH_Q5_K, NH_Q3_K])
 def test_reference_wide_product_test(device, element):
     # crates/neura-runtime/tests/runtime.rs:88-144: 8 x 512 x 4096, seeds 23 / 29, tolerance 1e-3
     rows, depth, columns = 8, 512, 4096
@@ -268,7 +273,8 @@ def test_reference_wide_product_test(device, element):
 
 @pytest.mark.parametrize("element,M,N,K,half", [(NH_Q4_K, 70, 130, 512, True), (NH_Q4_K, 512, 256, 3584, True), (NH_Q4_K, 33, 64, 256, False),
                                                 (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q6_K, 70, 130, 512, False),
-                                                (NH_Q6_K, 40, 64, 3584, True)])
+                                                (NH_Q6_K, 40, 64, 3584, True), (NH_Q5_K, 70, 130, 512, True), (NH_Q5_K, 33, 64, 3584, False),
+                                                (NH_Q3_K, 70, 130, 512, False), (NH_Q3_K, 40, 64, 3584, True)])
 def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
     rng = np.random.default_rng(M + N + K)
     raw = synth.RANDOM[element](rng, N * K)

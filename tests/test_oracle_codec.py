@@ -150,7 +150,100 @@ def test_q6_k_pack_invariants():
     assert np.all(negative == 0.0)
 
 
-@pytest.mark.parametrize("element", [8, 12, 14])
+def q3_k_walk(field):
+    """ggml's published dequantize_row_q3_K as a scalar walk (the form the reference's own test checks its codec
+    against, crates/neura-precision/tests/format.rs:173-219): scales through the three-word shuffle, then per half four
+    shifts of two runs of 16, the mask bit moving up once per 32."""
+    aux = [int.from_bytes(bytes(field[96 + 4 * at:100 + 4 * at]), "little") for at in range(3)] + [0]
+    tmp = aux[2]
+    k1, k2 = 0x03030303, 0x0F0F0F0F
+    packed = [(aux[0] & k2) | ((tmp & k1) << 4), (aux[1] & k2) | (((tmp >> 2) & k1) << 4),
+              ((aux[0] >> 4) & k2) | (((tmp >> 4) & k1) << 4), ((aux[1] >> 4) & k2) | (((tmp >> 6) & k1) << 4)]
+    scales = [((packed[at // 4] >> ((at % 4) * 8)) & 0xFF) - 32 for at in range(16)]
+    d = np.float32(np.array(field[108:110], dtype=np.uint8).view(np.float16)[0])
+    out, walk, m = [], 0, 1
+    for half in range(2):
+        q = field[32 + half * 32:64 + half * 32]
+        for shift in (0, 2, 4, 6):
+            for run in range(2):
+                dl = np.float32(d * np.float32(scales[walk]))
+                walk += 1
+                for l in range(16):
+                    at = l + 16 * run
+                    quant = ((int(q[at]) >> shift) & 3) - (0 if int(field[at]) & m else 4)
+                    out.append(np.float32(dl * np.float32(quant)))
+            m <<= 1
+    return np.array(out, dtype=np.float32)
+
+
+def test_q3_k_known_answer_block_of_the_reference():
+    # the block of crates/neura-precision/tests/format.rs:221-234: third bits at*37+11, bit pairs at*53+7, scales at*19+3,
+    # d = 0.25; the reference asserts its codec equals ggml's walk on it, bit for bit
+    field = np.zeros(110, dtype=np.uint8)
+    field[0:32] = [(at * 37 + 11) & 0xFF for at in range(32)]
+    field[32:96] = [(at * 53 + 7) & 0xFF for at in range(64)]
+    field[96:108] = [(at * 19 + 3) & 0xFF for at in range(12)]
+    field[108:110] = np.array([0.25], dtype=np.float16).view(np.uint8)
+    got = oracle.unpack(oracle.EL_Q3_K, field, 256)
+    want = q3_k_walk(field)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(synth.q3_k_dequant(field, 256).view(np.uint32), want.view(np.uint32))
+    # spot values worked by hand: element 0 has pair (7 >> 0) & 3 = 3, third bit 11 & 1 = 1 -> code 3; its scale is
+    # (3 & 15) | ((155 & 3) << 4) = 51 - 32 = 19
+    assert got[0] == np.float32(0.25 * 19 * 3)
+    # element 16: pair (byte 32+16 = 16*53+7 = 855 & 255 = 87) & 3 = 3, third bit (16*37+11 = 603 & 255 = 91) & 1 = 1 -> 3;
+    # scale 1 = (22 & 15) | ((174 & 3) << 4) = 6 | 32 = 38 - 32 = 6
+    assert got[16] == np.float32(0.25 * 6 * 3)
+
+
+def test_q3_k_round_trip_of_the_reference():
+    # crates/neura-precision/tests/format.rs:236-245: a slow sine of amplitude 0.75 comes back within 0.25
+    values = (np.sin(np.arange(256, dtype=np.float32) * np.float32(0.031)) * np.float32(0.75)).astype(np.float32)
+    raw = oracle.pack(oracle.EL_Q3_K, values)
+    assert raw.size == 110 == oracle.lib().oracle_payload_bytes(11, 256)
+    back = oracle.unpack(oracle.EL_Q3_K, raw, 256)
+    assert np.abs(back - values).max() <= 0.25
+    # the scales are stored as codes 32..63 and every code is a pair plus a third bit
+    scales = synth.q3_k_scales(raw[96:108].reshape(1, 12))
+    assert scales.min() >= 0 and scales.max() <= 31
+
+
+def test_q5_k_unpack_hand_built_block():
+    # element e of sub-block s carries code (11 e + 5) % 32; scales and minimums through put_scale_min_k4's layout
+    raw = np.zeros(176, dtype=np.uint8)
+    raw[0:2] = np.array([np.float16(0.5)]).view(np.uint8)
+    raw[2:4] = np.array([np.float16(0.125)]).view(np.uint8)
+    raw[4:16] = [(at * 53 + 7) & 0xFF for at in range(12)]
+    codes = [(11 * e + 5) % 32 for e in range(256)]
+    for e, code in enumerate(codes):
+        sub, l = e // 32, e % 32
+        raw[48 + (sub // 2) * 32 + l] |= (code & 15) << (4 if sub % 2 else 0)
+        raw[16 + l] |= (code >> 4) << sub
+    got = oracle.unpack(oracle.EL_Q5_K, raw, 256)
+    s = raw[4:16].astype(int)
+    want = []
+    for e, code in enumerate(codes):
+        j = e // 32
+        if j < 4:
+            sc, mn = s[j] & 63, s[j + 4] & 63
+        else:
+            sc, mn = (s[j + 4] & 15) | ((s[j - 4] >> 6) << 4), (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+        want.append(np.float32(np.float32(0.5) * np.float32(sc)) * np.float32(code) - np.float32(np.float32(0.125) * np.float32(mn)))
+    assert np.array_equal(got, np.array(want, dtype=np.float32))
+
+
+def test_q5_k_pack_invariants():
+    values = oracle.random(256 * 200, 23)
+    raw = oracle.pack(oracle.EL_Q5_K, values)
+    assert oracle.lib().oracle_payload_bytes(13, 256 * 200) == raw.size == 200 * 176
+    back = oracle.unpack(oracle.EL_Q5_K, raw, values.size)
+    # 5-bit affine codes over a range of <= 2: step <= 2/31, and twice as fine as Q4_K on the same values
+    assert np.abs(back - values).max() <= 2.0 / 31.0
+    coarse = oracle.unpack(oracle.EL_Q4_K, oracle.pack(oracle.EL_Q4_K, values), values.size)
+    assert np.abs(back - values).mean() < 0.6 * np.abs(coarse - values).mean()
+
+
+@pytest.mark.parametrize("element", [8, 11, 12, 13, 14])
 def test_unpack_matches_the_numpy_restatement_on_random_blocks(element):
     rng = np.random.default_rng(3 + element)
     elements = 256 * 300
@@ -160,7 +253,7 @@ def test_unpack_matches_the_numpy_restatement_on_random_blocks(element):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("element", [8, 12])
+@pytest.mark.parametrize("element", [8, 11, 12, 13])
 def test_pack_matches_the_numpy_restatement(element):
     rng = np.random.default_rng(5 + element)
     values = np.concatenate([
@@ -198,6 +291,9 @@ def test_block_geometry():
     # crates/neura-abi/tests/layout.rs:147-158
     assert oracle.lib().oracle_payload_bytes(8, 32) == 34
     assert oracle.lib().oracle_payload_bytes(12, 256) == 144
+    assert oracle.lib().oracle_payload_bytes(11, 256) == 110
+    assert oracle.lib().oracle_payload_bytes(13, 256) == 176
+    assert oracle.lib().oracle_payload_bytes(14, 256) == 210
     assert oracle.lib().oracle_payload_bytes(14, 256) == 210
     assert oracle.lib().oracle_payload_bytes(8, 4864 * 896) == 4630528
     assert oracle.lib().oracle_payload_bytes(12, 46792704) == 26320896
