@@ -166,14 +166,14 @@ typedef struct nh_model_config {
 /* where each tensor sits in the arena (byte offsets) and its element.  Per layer arrays have
  * `layers` entries.  output == UINT64_MAX ties the head to token_embd (examples/qwen/model.rs:81-84). */
 typedef struct nh_tensor_table {
-    int32_t matrix_element; /* element of every matrix: NH_Q8_0, NH_Q4_K or NH_Q6_K */
+    int32_t matrix_element; /* element of every matrix: NH_Q8_0, NH_Q3_K, NH_Q4_K, NH_Q5_K or NH_Q6_K */
     uint64_t token_embd, output, output_norm;
     const uint64_t *attn_norm, *attn_q, *attn_k, *attn_v, *attn_output, *ffn_norm, *ffn_gate, *ffn_up, *ffn_down;
     /* Optional, NULL = absent.
      * matrix_elements: the element of each matrix where a file mixes them (a Q4_K_M file keeps some matrices in Q6_K;
      * neura-gguf hands every tensor over with its own element, crates/neura-gguf/src/header.rs:10-17):
      * [token_embd, output, then per layer attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down], 2 + 7 * layers
-     * entries of NH_Q8_0 / NH_Q4_K / NH_Q6_K.  NULL: every matrix is `matrix_element`.
+     * entries of NH_Q8_0 / NH_Q3_K / NH_Q4_K / NH_Q5_K / NH_Q6_K.  NULL: every matrix is `matrix_element`.
      * attn_{q,k,v}_bias: byte offsets of f32 [rows] vectors per layer, UINT64_MAX = none, added to the projection before the
      * rotation.  Qwen2 checkpoints carry them (blk.N.attn_q.bias ...); the reference's own qwen example has none
      * (examples/qwen/attention.rs:98-154), so they have no counterpart there. */

@@ -680,9 +680,9 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
 //   Q6_K (crates/neura-precision/src/ggml.rs:394-407, crates/neura-kernel/src/dot.rs:663-797): (d * scale) * (code - 32)
 //   Q5_K (ggml.rs:321-335, dot.rs:621-661): d * sc * code - dmin * m
 //   Q3_K (ggml.rs:291-306, dot.rs:544-581): (d * (scale - 32)) * (code - 4), the third bit being the code's top bit
-// Every run contributes weight * sum(x * code) - (weight * offset + minimum) * sum(x): the stored codes convert to fp32
-// with one instruction each, and the offset and the minimum cost one multiply-add per eight weights.  The sums run in
-// lane order, not in the reference's run order.
+// Every run contributes weight * (sum(x * code) - offset * sum(x)) - minimum * sum(x): the stored codes convert to fp32
+// with one instruction each, and sum(x) per eight activations is worked out once per workgroup.  The sums run in lane
+// order, not in the reference's run order.
 __device__ __forceinline__ uint32_t byte_of(uint32_t word, uint32_t at) { return (word >> (8u * at)) & 0xffu; }
 
 template <int ELEMENT>
@@ -781,10 +781,20 @@ struct Staged<NH_Q3_K> {
 
 __device__ __forceinline__ uint32_t skew128(uint32_t i) { return i + (i >> 7) * 4; }
 
+// sixteen bytes from `at`, those at and past `end` read as zero without being touched.  Out of line: only the last rows of a
+// tensor come here, and the byte loads would otherwise sit in every caller's loop.
+__device__ __noinline__ u32x4 piece_before(const uint8_t *at, const uint8_t *end) {
+    uint32_t words[4] = {0u, 0u, 0u, 0u};
+    for (uint32_t j = 0; j < 16u; j++)
+        if (at + j < end) words[j >> 2] |= (uint32_t)at[j] << (8u * (j & 3u));
+    u32x4 held = {words[0], words[1], words[2], words[3]};
+    return held;
+}
+
 template <int ELEMENT, int RB>
 __global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
     typedef Staged<ELEMENT> Format;
-    extern __shared__ float xs[];  // [RB][slice]; then the raw row slices, two per wave
+    extern __shared__ float xs[];  // [RB][slice]; the sums per eight activations; then the raw row slices, two per wave
     __shared__ float red[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -798,8 +808,21 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
         stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew128(i); });
     }
     __syncthreads();
+    // what the codes' offset (or a run's minimum) multiplies, once for all rows: per unit and run the sum of the eight
+    // activations, times the offset where the format has one
+    float *const sums = xs + RB * xstride;
+    const uint32_t sstride = p.blocks_per_split * 32u;
+    for (uint32_t b = 0; b < RB; b++)
+        for (uint32_t q = tid; q < nb * 32u; q += 256u) {
+            const uint32_t u = q >> 2, g = q & 3u;
+            const float4 *at = reinterpret_cast<const float4 *>(xs + b * xstride + skew128((u >> 2) * 128u) + g * 32u + 8u * (u & 3u));
+            const float4 lo = at[0], hi = at[1];
+            const float total = ((lo.x + lo.y) + (lo.z + lo.w)) + ((hi.x + hi.y) + (hi.z + hi.w));
+            sums[b * sstride + q] = Format::FLOORS ? total : -Format::OFFSET * total;
+        }
+    __syncthreads();
     const uint32_t raw_stride = p.chunks_per_row * 16u;  // bytes of one staged row slice
-    uint8_t *const mine = reinterpret_cast<uint8_t *>(xs + RB * xstride) + (size_t)wave * 2u * raw_stride;
+    uint8_t *const mine = reinterpret_cast<uint8_t *>(sums + RB * sstride) + (size_t)wave * 2u * raw_stride;
     const uint32_t units = nb * 8u;
 
     // the 16-byte pieces of the two rows `first`, `first + 1` this lane copies: fetched one pair of rows ahead, so the copy
@@ -816,21 +839,23 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
             ahead_lead[r] = (uint32_t)((uintptr_t)src & 15u);
             const uint8_t *from = src - ahead_lead[r];
             const uint32_t bytes = ahead_lead[r] + nb * Format::BYTES;
+            const uint32_t pieces = (bytes + 15u) / 16u;
+            if (from + 16u * pieces <= matrix_end) {  // the same for every lane of the wave
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const uint32_t c = lane + 64u * k;
-                u32x4 held = {0u, 0u, 0u, 0u};
-                if (c * 16u < bytes) {
-                    if (from + 16u * c + 16u <= matrix_end) {
-                        held = *(global_uint4)(uintptr_t)(from + 16u * c);
-                    } else {  // the last bytes of the tensor: never read past its end
-                        uint8_t tail[16];
-#pragma unroll
-                        for (int j = 0; j < 16; j++) tail[j] = (from + 16u * c + j < matrix_end) ? from[16u * c + j] : (uint8_t)0;
-                        held = *reinterpret_cast<u32x4 *>(tail);
-                    }
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t c = lane + 64u * k;
+                    u32x4 held = {0u, 0u, 0u, 0u};
+                    if (c < pieces) held = *(global_uint4)(uintptr_t)(from + 16u * c);
+                    ahead[r][k] = held;
                 }
-                ahead[r][k] = held;
+            } else {  // the last bytes of the tensor: never read past its end
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t c = lane + 64u * k;
+                    u32x4 held = {0u, 0u, 0u, 0u};
+                    if (c < pieces) held = piece_before(from + 16u * c, matrix_end);
+                    ahead[r][k] = held;
+                }
             }
         }
     };
@@ -857,32 +882,39 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
         for (uint32_t u = lane; u < units; u += 64u) {
             const uint32_t blk = u >> 3, half = (u >> 2) & 1u, j = u & 3u;
             float4 xv[RB][4][2];
-            float xsum[RB][4];  // a code's offset and a run's minimum weigh the plain sum of the eight activations
+            float base[RB][4];
 #pragma unroll
-            for (int b = 0; b < RB; b++)
+            for (int b = 0; b < RB; b++) {
+                const float4 held = *reinterpret_cast<const float4 *>(sums + b * sstride + 4u * u);
+                base[b][0] = held.x, base[b][1] = held.y, base[b][2] = held.z, base[b][3] = held.w;
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const float4 *at = reinterpret_cast<const float4 *>(xs + b * xstride + skew128(blk * 256u + half * 128u) + g * 32u + 8u * j);
                     xv[b][g][0] = at[0], xv[b][g][1] = at[1];
-                    xsum[b][g] = ((xv[b][g][0].x + xv[b][g][0].y) + (xv[b][g][0].z + xv[b][g][0].w)) +
-                                 ((xv[b][g][1].x + xv[b][g][1].y) + (xv[b][g][1].z + xv[b][g][1].w));
                 }
+            }
 #pragma unroll
             for (int r = 0; r < 2; r++) {
                 const uint8_t *block = mine + r * raw_stride + lead[r] + blk * Format::BYTES;
-                auto word = [&](uint32_t at) { return (uint32_t)*reinterpret_cast<const uint16_t *>(block + at) | ((uint32_t)*reinterpret_cast<const uint16_t *>(block + at + 2u) << 16); };
+                // a block sits on a 2-byte boundary: its words are cut out of the aligned words around them (LDS serves a
+                // misaligned read at a fraction of its rate)
+                const uint32_t off = Format::BYTES % 4u ? (uint32_t)(uintptr_t)block & 3u : 0u;
+                const uint32_t *words = reinterpret_cast<const uint32_t *>(block - off);
+                auto word = [&](uint32_t at) {
+                    if (Format::BYTES % 4u == 0) return words[at / 4u];
+                    return __builtin_amdgcn_alignbit(words[at / 4u + 1u], words[at / 4u], off * 8u);
+                };
                 uint32_t codes[4][2];
                 float weight[4], floor[4];
                 Format::unit(block, word, half, j, codes, weight, floor);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const float low = Format::FLOORS ? fmaf(weight[g], Format::OFFSET, floor[g]) : weight[g] * Format::OFFSET;
 #pragma unroll
                     for (int b = 0; b < RB; b++) {
-                        float dot = 0.0f;
+                        // the codes go to fp32 as they are stored, one conversion each; their offset came with the sum
+                        float dot = Format::FLOORS ? 0.0f : base[b][g];
 #pragma unroll
                         for (int h = 0; h < 2; h++) {
-                            // the codes go to fp32 as they are stored, one conversion each; their offset leaves with the sum
                             const uint32_t c = codes[g][h];
                             dot = fmaf(xv[b][g][h].x, (float)(c & 0xffu), dot);
                             dot = fmaf(xv[b][g][h].y, (float)((c >> 8) & 0xffu), dot);
@@ -890,7 +922,7 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
                             dot = fmaf(xv[b][g][h].w, (float)(c >> 24), dot);
                         }
                         acc[r][b] = fmaf(weight[g], dot, acc[r][b]);
-                        acc[r][b] = fmaf(-low, xsum[b][g], acc[r][b]);
+                        if (Format::FLOORS) acc[r][b] = fmaf(-floor[g], base[b][g], acc[r][b]);
                     }
                 }
             }
@@ -2044,10 +2076,12 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
         p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * RB * a.N * sizeof(float)));
         if (!p.partial) return NH_E_MEMORY;
     }
-    p.chunks_per_row = (15u + p.blocks_per_split * Staged<ELEMENT>::BYTES + 15u) / 16u;
-    const size_t lds = (size_t)RB * p.blocks_per_split * 264u * sizeof(float) + (size_t)8 * p.chunks_per_row * 16u;  // slices, 8 floats of skew a block
+    p.chunks_per_row = (15u + p.blocks_per_split * Staged<ELEMENT>::BYTES + 15u) / 16u + 1u;  // a lead, the blocks, and the word past the last field
+    // activation slices (8 floats of skew a block), their sums per eight, the raw rows
+    const size_t lds = (size_t)RB * p.blocks_per_split * (264u + 32u) * sizeof(float) + (size_t)8 * p.chunks_per_row * 16u;
     uint32_t blocks_x = (a.N + 7u) / 8u;
-    uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_STAGED_WGS", 2) / p.splits;
+    // three workgroups a compute unit: their LDS (about 41 KiB each at 14 blocks) and registers fit, and a fourth measured slower
+    uint32_t most = (uint32_t)d->compute_units * 3u / p.splits;
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
     profile_mark(d);
