@@ -33,21 +33,36 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.76e6}
 
 
 def workload(name):
+    """(shape, element of the matrices, context, matrices stored otherwise, layers whose q/k/v carry biases)"""
     from neura_amd import synth
 
     if name == "qwen2.5-7b-q4k":
-        return synth.SHAPES["qwen2.5-7b"], 12, 4096
+        return synth.SHAPES["qwen2.5-7b"], 12, 4096, {}, ()
     if name == "qwen2.5-0.5b-q8_0":
-        return synth.SHAPES["qwen2.5-0.5b"], 8, 1088
+        return synth.SHAPES["qwen2.5-0.5b"], 8, 1088, {}, ()
+    if name == "qwen2.5-7b-q4_k_m":
+        # the mix llama.cpp's Q4_K_M recipe gives a Qwen2.5-7B file: the head and, in the first and last eighth of the layers
+        # and every third between, the value and down projections in Q6_K, the rest Q4_K; q, k and v biases everywhere
+        shape = synth.SHAPES["qwen2.5-7b"]
+        count = shape["layers"]
+        more_bits = [i for i in range(count) if i < count // 8 or i >= 7 * count // 8 or (i - count // 8) % 3 == 2]
+        mixed = {"output.weight": 14}
+        for i in more_bits:
+            mixed["blk.%d.attn_v.weight" % i] = 14
+            mixed["blk.%d.ffn_down.weight" % i] = 14
+        return shape, 12, 4096, mixed, tuple(range(count))
     raise SystemExit("unknown workload %s" % name)
 
 
-def weight_bytes_per_token(shape, element, layers):
+def weight_bytes_per_token(shape, element, layers, mixed=None):
     from neura_amd import synth
 
-    per_layer = sum(synth.matrix_bytes(element, rows, columns) for _, rows, columns in synth.layer_matrices(shape))
-    head = synth.matrix_bytes(element, shape["vocab"], shape["hidden"])
-    return layers * per_layer + head
+    mixed = mixed or {}
+    total = synth.matrix_bytes(mixed.get("output.weight", element), shape["vocab"], shape["hidden"])
+    for layer in range(layers):
+        for name, rows, columns in synth.layer_matrices(shape):
+            total += synth.matrix_bytes(mixed.get("blk.%d.%s.weight" % (layer, name), element), rows, columns)
+    return total
 
 
 def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=20.0):
@@ -187,11 +202,11 @@ def main():
         print(json.dumps({"gemm_config3": gemm_config3(device, np.random.default_rng(0))}))
         device.close()
         return
-    shape, element, context = workload(args.workload)
+    shape, element, context, mixed, biases = workload(args.workload)
     layers = shape["layers"] if args.layers is None else args.layers
     rng = np.random.default_rng(0)
     mode = "blocks" if element == 12 else "normal"
-    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
+    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers, elements=mixed, biases=biases))
     device = neura_amd.Device(0)
     weights = Weights(device, tensors)
     model = Model(device, weights, shape, element, batch=1, context=context, layers=layers)
@@ -243,12 +258,13 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "%s decode, batch 1, %d layers, fp16 KV cache at context %d, random-init %s weights" %
-                        (args.workload, layers, context, "Q4_K" if element == 12 else "Q8_0"),
-            "weight_bytes_per_token": weight_bytes_per_token(shape, element, layers),
+                        (args.workload, layers, context, ("Q4_K" if element == 12 else "Q8_0") + (" and Q6_K" if mixed else "")),
+            "weight_bytes_per_token": weight_bytes_per_token(shape, element, layers, mixed),
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_deep_kernel (down)" if element == 12 else "gemv_q8_0_kernel",
+            "kernel": ("all narrow products: gemv_q4k_decode_kernel, gemv_q4k_mfma_deep_kernel, gemv_staged_kernel<Q6_K>" if mixed else
+                       "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_deep_kernel (down)" if element == 12 else "gemv_q8_0_kernel"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
@@ -262,7 +278,7 @@ def main():
     }
     if not args.no_extras:
         result["extras"] = extras(device, weights, shape, element, context, layers, rng)
-    if not args.no_cpu:
+    if not args.no_cpu and not mixed:
         host = {name: raw for name, _, _, raw in tensors}
         result["cpu_baseline"] = cpu_baseline(shape, element, host, context, layers)
     else:

@@ -108,17 +108,19 @@ size_t nh_weights_bytes(const nh_weights *weights);
 
 /* ---- operators : replace the run_<kind> bodies of crates/neura-kernel ---------------------- */
 
-/* fetch_q8_0 / fetch_q4_k / fetch_half (crates/neura-kernel/src/fetch.rs:236-267, :95-98) ==
- * unpack (crates/neura-precision/src/ggml.rs:211-216, :336-350): bit-exact fp32 values */
+/* fetch_q8_0 / fetch_q3_k / fetch_q4_k / fetch_q5_k / fetch_q6_k / fetch_half (crates/neura-kernel/src/fetch.rs:236-303, :95-98) ==
+ * unpack (crates/neura-precision/src/ggml.rs:211-216, :291-350, :394-407): bit-exact fp32 values of NH_Q8_0, NH_Q3_K, NH_Q4_K,
+ * NH_Q5_K, NH_Q6_K, NH_F16 or NH_F32 storage */
 int32_t nh_dequant(nh_device *device, int32_t element, const void *dev_src, uint64_t elements, float *dev_dst);
 /* run_convert_half (crates/neura-kernel/src/task/convert.rs:229-249): fp32 -> fp16 RNE */
 int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elements, uint16_t *dev_dst);
 /* narrow product, rows <= 8 (template_run_matmul_folded{,_fused,_quad},
- * crates/neura-kernel/src/task/matmul.rs:376-803): y[r][n] = sum_k x[r][k]·W[n][k], fp32 */
+ * crates/neura-kernel/src/task/matmul.rs:376-803): y[r][n] = sum_k x[r][k]·W[n][k], fp32; W in NH_Q8_0, NH_Q3_K, NH_Q4_K,
+ * NH_Q5_K or NH_Q6_K blocks (the dots of crates/neura-kernel/src/dot.rs:471-797) */
 int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
                 float *dev_y, const nh_epilogue *epilogue);
 /* wide product (template_run_matmul_codes / _run, crates/neura-kernel/src/task/matmul.rs:943-1221):
- * X [M][K] in x_element (NH_F32 or NH_F16), Y fp32 [M][N] */
+ * X [M][K] in x_element (NH_F32 or NH_F16), Y fp32 [M][N]; W in the same five block formats */
 int32_t nh_gemm(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const void *dev_X, int32_t x_element,
                 uint32_t M, float *dev_Y, const nh_epilogue *epilogue);
 /* run_norm NORM_RMS (crates/neura-kernel/src/task/norm.rs:55-130, :350-369):
