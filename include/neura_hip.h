@@ -152,6 +152,23 @@ int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uin
 /* run_argmax (crates/neura-kernel/src/task/choice.rs:355-368): per row, lowest index wins ties */
 int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out);
 
+/* What one row draws with (Sampling::Sampled and the per-plane states of a sampled batch,
+ * crates/neura-generate/src/sampling.rs:3-36, crates/neura-generate/src/batch.rs:383-386): the seed's 32 bits as the
+ * kernel hashes them, the temperature the logits are divided by, the number of largest logits kept (1..64) and the
+ * cumulative softmax mass the kept ones are cut at (0 < cumulative <= 1). */
+typedef struct nh_draw {
+    uint32_t seed;
+    float temperature;
+    uint32_t keep;
+    float cumulative;
+} nh_draw;
+/* graph.sample over logits * recip(temperature) (crates/neura-generate/src/sampling.rs:69-94; run_sample / run_sample_fold,
+ * crates/neura-kernel/src/task/choice.rs:933-989, :1109-1123, :1270-1359): per row the `keep` largest values, cut where
+ * their running softmax mass plus the mass outside them reaches cumulative * total, then the largest of
+ * value + gumbel_noise(seed, column) (choice.rs:81-89), the lowest column among equals.  keep == 1 is the argmax.
+ * `host_draws`: rows entries of caller memory.  A row holds at most 262144 columns. */
+int32_t nh_sample(nh_device *device, const float *dev_logits, uint32_t rows, uint32_t n, const nh_draw *host_draws, uint32_t *dev_out);
+
 /* ---- decoder model : replaces the compiled answer / fill programs of Batch ------------------ */
 
 /* Qwen2-style decoder (composition of examples/qwen/model.rs:92-103, attention.rs:98-154,
@@ -191,6 +208,10 @@ void nh_model_destroy(nh_model *model);
  * host arrays of `batch` entries; mask 0 = inactive plane.  chosen_out[b] = argmax of the logits. */
 int32_t nh_decode_step(nh_model *model, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
                        uint32_t *chosen_out);
+/* the answer program of a sampled batch (crates/neura-generate/src/batch.rs:330-398, sampling.rs:69-94): as nh_decode_step,
+ * with chosen_out[b] drawn from plane b's logits as nh_sample draws it with host_draws[b]. */
+int32_t nh_decode_step_sampled(nh_model *model, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                               const nh_draw *host_draws, uint32_t *chosen_out);
 /* a fill program (crates/neura-generate/src/batch.rs:1434-1517): `rows` tokens per plane,
  * tokens[row * batch + plane]; no logits, no readback. */
 int32_t nh_prefill(nh_model *model, const uint32_t *tokens, uint32_t rows, const uint32_t *cursors, const uint8_t *mask, uint32_t batch);

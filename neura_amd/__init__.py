@@ -216,6 +216,20 @@ class Device:
         _check(self.lib.nh_argmax(self.handle, vd.pointer, rows, n, out.pointer))
         return out.numpy(np.uint32)
 
+    def sample(self, values, draws):
+        """one column per row of `values`, drawn with the records of `draws` (dtype DRAW)"""
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        draws = np.ascontiguousarray(draws, dtype=DRAW)
+        rows, n = values.shape
+        assert draws.size == rows
+        vd = self.upload(values)
+        out = self.alloc(max(rows, 1) * 4)
+        _check(self.lib.nh_sample(self.handle, vd.pointer, rows, n, draws.ctypes.data, out.pointer))
+        return out.numpy(np.uint32)[:rows]
 
-__all__ = ["Device", "Buffer", "NeuraError", "payload_bytes", "NH_F32", "NH_F16", "NH_Q8_0", "NH_Q3_K", "NH_Q4_K", "NH_Q5_K", "NH_Q6_K", "UINT64_MAX", "Epilogue",
+
+# one row's draw, laid out as nh_draw: seed bits, temperature, candidates kept, cumulative mass
+DRAW = np.dtype([("seed", np.uint32), ("temperature", np.float32), ("keep", np.uint32), ("cumulative", np.float32)])
+
+__all__ = ["Device", "DRAW", "Buffer", "NeuraError", "payload_bytes", "NH_F32", "NH_F16", "NH_Q8_0", "NH_Q3_K", "NH_Q4_K", "NH_Q5_K", "NH_Q6_K", "UINT64_MAX", "Epilogue",
            "ModelConfig", "TensorTable"]

@@ -66,9 +66,11 @@ SIGNATURES = {
                                c_uint32, c_void_p, c_float, c_void_p]),
     "nh_gather": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_argmax": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
+    "nh_sample": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_model_create": (c_void_p, [c_void_p, POINTER(ModelConfig), c_void_p, POINTER(TensorTable)]),
     "nh_model_destroy": (None, [c_void_p]),
     "nh_decode_step": (c_int32, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint8), c_uint32, POINTER(c_uint32)]),
+    "nh_decode_step_sampled": (c_int32, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint8), c_uint32, c_void_p, POINTER(c_uint32)]),
     "nh_prefill": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32, POINTER(c_uint32), POINTER(c_uint8), c_uint32]),
     "nh_model_time_products": (c_int32, [c_void_p, c_uint32, POINTER(c_double), POINTER(c_uint64), POINTER(c_uint64)]),
     "nh_model_reset": (c_int32, [c_void_p, POINTER(c_uint8), c_uint32]),

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBRARY = os.path.join(HERE, "libneura_hip.so")
-SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "model.hip"]
+SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "sample.hip", "model.hip"]
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

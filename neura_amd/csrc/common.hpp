@@ -183,6 +183,9 @@ int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
                       uint32_t count, uint32_t batch, const uint8_t *mask, float *out);
 int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);
+// sampled choice: `draws` is device memory, one entry a row; check_draws refuses what the reference's host asserts refuse
+int32_t launch_sample(nh_device *d, const float *logits, uint32_t rows, uint32_t n, const nh_draw *draws, uint32_t *out);
+int32_t check_draws(const nh_draw *draws, uint32_t rows);
 int32_t launch_silu_mul(nh_device *d, const float *gate, const float *up, uint64_t n, float *out);
 int32_t launch_mask_rows(nh_device *d, float *x, uint32_t rows, uint32_t batch, uint32_t width, const uint8_t *mask);
 

@@ -27,14 +27,14 @@ struct nh_model {
     // activations; T = rows * batch flattened token rows, t = row * batch + plane
     float *h = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr, *act = nullptr, *up = nullptr, *logits = nullptr;
     float *rope_cos = nullptr, *rope_sin = nullptr;  // [capacity][head_dim / 2], for the rotation folded into the q|k|v product
-    uint32_t *inputs_dev = nullptr;  // [tokens T_max | cursors B | mask bytes B]
+    uint32_t *inputs_dev = nullptr;  // [tokens T_max | cursors B | draws B x 4 words | mask bytes B]
     uint32_t *chosen_dev = nullptr;
     uint8_t *inputs_host = nullptr;  // pinned mirror of inputs_dev
     uint32_t *chosen_host = nullptr; // pinned [B + 1]: chosen tokens, then the refusal word
     uint32_t max_tokens = 0;
-    // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked
-    hipGraphExec_t decode_graph[2] = {nullptr, nullptr};
-    uint64_t graph_moved[2] = {0, 0};  // nh_device::moved when each graph was recorded
+    // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked, [2], [3] the same with a sampled choice
+    hipGraphExec_t decode_graph[4] = {nullptr, nullptr, nullptr, nullptr};
+    uint64_t graph_moved[4] = {0, 0, 0, 0};  // nh_device::moved when each graph was recorded
     bool use_graph = true;
 };
 
@@ -67,21 +67,25 @@ bool device_array(T *&out, size_t count) {
     return true;
 }
 
-// writes tokens / cursors / mask through the pinned staging buffer in one copy
-int32_t stage_inputs(nh_model *m, const uint32_t *tokens, uint32_t count, const uint32_t *cursors, const uint8_t *mask, uint32_t batch) {
+// writes tokens / cursors / draws / mask through the pinned staging buffer in one copy
+int32_t stage_inputs(nh_model *m, const uint32_t *tokens, uint32_t count, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                     const nh_draw *draws = nullptr) {
+    static_assert(sizeof(nh_draw) == 16, "a draw is four words");
     uint32_t *words = reinterpret_cast<uint32_t *>(m->inputs_host);
     memcpy(words, tokens, (size_t)count * 4);
     memcpy(words + m->max_tokens, cursors, (size_t)batch * 4);
-    uint8_t *mask_bytes = reinterpret_cast<uint8_t *>(words + m->max_tokens + batch);
+    if (draws) memcpy(words + m->max_tokens + batch, draws, (size_t)batch * sizeof(nh_draw));
+    uint8_t *mask_bytes = reinterpret_cast<uint8_t *>(words + m->max_tokens + 5 * (size_t)batch);
     for (uint32_t b = 0; b < batch; b++) mask_bytes[b] = mask ? (mask[b] ? 1 : 0) : 1;
-    size_t bytes = ((size_t)m->max_tokens + batch) * 4 + batch;
+    size_t bytes = ((size_t)m->max_tokens + 5 * (size_t)batch) * 4 + batch;
     NH_HIP(hipMemcpyAsync(m->inputs_dev, m->inputs_host, bytes, hipMemcpyHostToDevice, m->d->stream));
     return NH_OK;
 }
 
 const uint32_t *dev_tokens(const nh_model *m) { return m->inputs_dev; }
 const uint32_t *dev_cursor(const nh_model *m) { return m->inputs_dev + m->max_tokens; }
-const uint8_t *dev_mask(const nh_model *m) { return reinterpret_cast<const uint8_t *>(m->inputs_dev + m->max_tokens + m->c.batch); }
+const nh_draw *dev_draws(const nh_model *m) { return reinterpret_cast<const nh_draw *>(m->inputs_dev + m->max_tokens + m->c.batch); }
+const uint8_t *dev_mask(const nh_model *m) { return reinterpret_cast<const uint8_t *>(m->inputs_dev + m->max_tokens + 5 * (size_t)m->c.batch); }
 
 enum { EMBD = 0, HEAD = 1, Q = 0, K_ = 1, V = 2, O = 3, GATE = 4, UP = 5, DOWN = 6 };
 int32_t element_at(const nh_model *m, uint32_t layer, int which) { return m->elements[2 + 7 * layer + which]; }
@@ -203,12 +207,13 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
 
 // every kernel of one decode step: the layers, then logits = rms(hidden) . head^T and the greedy
 // choice (examples/qwen/model.rs:81-84, crates/neura-generate/src/sampling.rs:69-71)
-int32_t decode_kernels(nh_model *m, bool any_inactive) {
+int32_t decode_kernels(nh_model *m, bool any_inactive, bool sampled) {
     int32_t status;
     if ((status = forward(m, 1, any_inactive)) != NH_OK) return status;
     GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
     head.norm_w = m->output_norm, head.eps = m->c.eps;
     if ((status = launch_gemv(m->d, head)) != NH_OK) return status;
+    if (sampled) return launch_sample(m->d, m->logits, m->c.batch, m->c.vocab, dev_draws(m), m->chosen_dev);
     return launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
 }
 
@@ -314,7 +319,7 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     m->cache_elements = (size_t)c.kv_heads * c.batch * m->capacity * c.head_dim;
     ok = device_array(m->h, T * H) && device_array(m->xn, T * (H > QW ? H : QW)) && device_array(m->qkv, T * (QW + 2 * KW)) &&
          device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T * F) &&
-         device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 2 * c.batch + 4) &&
+         device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 6 * c.batch + 4) &&
          device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->capacity * (c.head_dim / 2)) &&
          device_array(m->rope_sin, (size_t)m->capacity * (c.head_dim / 2));
     for (uint32_t L = 0; ok && L < c.layers; L++) {
@@ -326,7 +331,7 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         if (ok) ok = hipMemsetAsync(k, 0, m->cache_elements * 2, device->stream) == hipSuccess &&
                      hipMemsetAsync(v, 0, m->cache_elements * 2, device->stream) == hipSuccess;
     }
-    ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 2 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
+    ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 6 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
          hipHostMalloc((void **)&m->chosen_host, ((size_t)c.batch + 1) * 4, hipHostMallocDefault) == hipSuccess;
     // everything a captured step touches exists before the capture: the split partials of the
     // products (at most 5 slices x 4 rows), of the attention (at most 256 sections) and of the
@@ -363,8 +368,8 @@ void nh_model_destroy(nh_model *model) { release(model); }
 
 uint32_t nh_model_capacity(const nh_model *model) { return model ? model->capacity : 0; }
 
-int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
-                       uint32_t *chosen_out) {
+static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                           const nh_draw *draws, uint32_t *chosen_out) {
     NH_REQUIRE(m && tokens && cursors && chosen_out, "a decode step names no model, tokens, cursors or result");
     NH_REQUIRE(batch == m->c.batch, "a decode step of %u planes feeds a model of %u planes", batch, m->c.batch);
     bool any_inactive = false;
@@ -377,21 +382,23 @@ int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *curs
     }
     nh_device *d = m->d;
     int32_t status;
-    if ((status = stage_inputs(m, tokens, batch, cursors, mask, batch)) != NH_OK) return status;
+    if (draws && (status = check_draws(draws, batch)) != NH_OK) return status;
+    if ((status = stage_inputs(m, tokens, batch, cursors, mask, batch, draws)) != NH_OK) return status;
     // Every kernel of the step reads its token, cursor and mask from device memory and no launch
     // shape depends on them, so the step is captured once per mask variant and replayed.
     // Profiled steps run eagerly (event records do not belong in a graph).
-    hipGraphExec_t &graph = m->decode_graph[any_inactive ? 1 : 0];
+    const int variant = (any_inactive ? 1 : 0) + (draws ? 2 : 0);
+    hipGraphExec_t &graph = m->decode_graph[variant];
     if (m->use_graph && !d->profile) {
-        if (graph && m->graph_moved[any_inactive ? 1 : 0] != d->moved) {
+        if (graph && m->graph_moved[variant] != d->moved) {
             // the device scratch or rope table moved since the capture (another model or operator call grew it)
             (void)hipGraphExecDestroy(graph);
             graph = nullptr;
         }
         if (!graph) {
-            m->graph_moved[any_inactive ? 1 : 0] = d->moved;
+            m->graph_moved[variant] = d->moved;
             NH_HIP(hipStreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal));
-            status = decode_kernels(m, any_inactive);
+            status = decode_kernels(m, any_inactive, draws != nullptr);
             hipGraph_t recorded = nullptr;
             hipError_t ended = hipStreamEndCapture(d->stream, &recorded);
             if (status != NH_OK) {
@@ -407,7 +414,7 @@ int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *curs
             }
         }
         NH_HIP(hipGraphLaunch(graph, d->stream));
-    } else if ((status = decode_kernels(m, any_inactive)) != NH_OK) {
+    } else if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) {
         return status;
     }
     NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
@@ -416,6 +423,17 @@ int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *curs
     if (m->chosen_host[batch] != REFUSAL_NONE) return check_refusal(d, "a decode step");
     memcpy(chosen_out, m->chosen_host, (size_t)batch * 4);
     return NH_OK;
+}
+
+int32_t nh_decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                       uint32_t *chosen_out) {
+    return decode_step(m, tokens, cursors, mask, batch, nullptr, chosen_out);
+}
+
+int32_t nh_decode_step_sampled(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
+                               const nh_draw *host_draws, uint32_t *chosen_out) {
+    NH_REQUIRE(host_draws, "a sampled decode step names no draws");
+    return decode_step(m, tokens, cursors, mask, batch, host_draws, chosen_out);
 }
 
 int32_t nh_prefill(nh_model *m, const uint32_t *tokens, uint32_t rows, const uint32_t *cursors, const uint8_t *mask, uint32_t batch) {
@@ -611,6 +629,23 @@ int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uin
     NH_REQUIRE(batch > 0, "a gather spreads its mask over no plane");
     int32_t status = launch_gather(device, element, dev_table, vocab, width, dev_tokens, count, batch, dev_mask, dev_out);
     return status != NH_OK ? status : check_refusal(device, "a gather");
+}
+
+int32_t nh_sample(nh_device *device, const float *dev_logits, uint32_t rows, uint32_t n, const nh_draw *host_draws, uint32_t *dev_out) {
+    NH_REQUIRE(device && dev_logits && host_draws && dev_out, "a sample names no device, logits, draws or result");
+    NH_REQUIRE(rows <= 4096, "a sample draws at most 4096 rows a call, not %u", rows);
+    int32_t status = check_draws(host_draws, rows);
+    if (status != NH_OK) return status;
+    if (!rows) return NH_OK;
+    // the draws ride in a small buffer of their own: the scratch belongs to the kernels
+    nh_draw *draws = nullptr;
+    NH_HIP(hipMalloc((void **)&draws, (size_t)rows * sizeof(nh_draw)));
+    hipError_t copied = hipMemcpyAsync(draws, host_draws, (size_t)rows * sizeof(nh_draw), hipMemcpyHostToDevice, device->stream);
+    if (copied == hipSuccess) status = launch_sample(device, dev_logits, rows, n, draws, dev_out);
+    (void)hipStreamSynchronize(device->stream);
+    (void)hipFree(draws);
+    if (copied != hipSuccess) return hip_fail(copied, "hipMemcpyAsync");
+    return status;
 }
 
 int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out) {

@@ -111,6 +111,20 @@ class Model:
                                        self.batch, chosen.ctypes.data_as(u32)))
         return chosen
 
+    def decode_step_sampled(self, tokens, cursors, draws, mask=None):
+        """a decode step whose chosen tokens are drawn: `draws` holds one record (dtype neura_amd.DRAW) a plane"""
+        from . import DRAW
+
+        tokens, cursors = self._u32(tokens), self._u32(cursors)
+        draws = np.ascontiguousarray(draws, dtype=DRAW)
+        assert draws.size == self.batch
+        mask = np.ones(self.batch, dtype=np.uint8) if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)
+        chosen = np.empty(self.batch, dtype=np.uint32)
+        u32, u8 = ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint8)
+        _check(self.lib.nh_decode_step_sampled(self.handle, tokens.ctypes.data_as(u32), cursors.ctypes.data_as(u32), mask.ctypes.data_as(u8),
+                                               self.batch, draws.ctypes.data, chosen.ctypes.data_as(u32)))
+        return chosen
+
     def prefill(self, tokens, rows, cursors, mask=None):
         tokens, cursors = self._u32(tokens), self._u32(cursors)
         mask = np.ones(self.batch, dtype=np.uint8) if mask is None else np.ascontiguousarray(mask, dtype=np.uint8)

@@ -31,6 +31,10 @@
  *   rope ................... pinned: closed form runtime.rs:468-494 (rotate-half)
  *   attention .............. pinned: f64 reference tests/support/attention.rs:38-109
  *   argmax ................. pinned: ties -> lowest index, brute force
+ *   sample ................. pinned: the hash against a numpy restatement; keep == 1 is the argmax and a row draws by
+ *                            its own seed (the reference's own tests, crates/neura-runtime/tests/choice.rs:41-126); the
+ *                            draw frequencies against the softmax over the kept nucleus (Gumbel-max); a nucleus worked
+ *                            by hand.  The rounding of the shader's log and exp is PARITY UNPINNED (no fixture holds it).
  *   decode step / greedy ... PARITY UNPINNED against the reference binary (no reference
  *                            test runs a transformer); pinned only by composition of the
  *                            pinned parts above plus an independent numpy forward pass.
@@ -853,6 +857,101 @@ void oracle_top2(const float *values, uint32_t n, float *first, float *second) {
     *first = a;
     *second = b;
 }
+
+/* ------------------------------------------------------------- sample ---- */
+
+typedef struct {
+    uint32_t seed;     /* the 32 bits the kernel hashes (a batch writes seed_bits(seed), crates/neura-generate/src/batch.rs:1845-1847) */
+    float temperature; /* logits * recip(temperature), crates/neura-generate/src/sampling.rs:82 */
+    uint32_t keep;     /* 1..64 */
+    float cumulative;  /* (0, 1] */
+} oracle_draw;
+
+/* crates/neura-kernel/src/task/choice.rs:81-89 over element_key((0, 0, 0, column)) (substrate.rs:146-152;
+ * coordinates(column, dims) of a [1, 1, rows, columns] value puts the column in w and zero elsewhere, choice.rs:102-107) */
+float oracle_gumbel_noise(uint32_t seed, uint32_t column) {
+    uint32_t key = 0u * 0x9e3779b9u;
+    key = (key ^ 0u) * 0x85ebca6bu;
+    key = (key ^ 0u) * 0xc2b2ae35u;
+    key = (key ^ column) * 0x27d4eb2fu;
+    uint32_t hash = seed ^ (key * 0x9e3779b9u);
+    hash = hash ^ (hash >> 16);
+    hash = hash * 0x7feb352du;
+    hash = hash ^ (hash >> 15);
+    hash = hash * 0x846ca68bu;
+    hash = hash ^ (hash >> 16);
+    return -logf(-logf((float)(hash >> 8) * (1.0f / 16777216.0f)));
+}
+
+/* One row of crates/neura-kernel/src/task/choice.rs:933-989 (sample_row): the keep largest values (larger first, lower
+ * column first among equals, :396-404), the nucleus boundary against cumulative * total, then the largest
+ * value + noise (choice_precedes, :46-51).  The row's mass is summed in column order here; the reference sums it
+ * over a workgroup tree (:891-931), which differs in the last bits only. */
+static uint32_t sample_row(const float *logits, uint32_t n, oracle_draw draw) {
+    float scale = 1.0f / draw.temperature;
+    float *values = (float *)malloc((size_t)n * 4);
+    for (uint32_t i = 0; i < n; i++) values[i] = logits[i] * scale;
+    uint32_t chosen = 0xffffffffu;
+    if (draw.keep == 1 && draw.cumulative == 1.0f) { /* :943-947 */
+        chosen = oracle_argmax(values, n);
+        free(values);
+        return chosen;
+    }
+    float row_max = -INFINITY;
+    for (uint32_t i = 0; i < n; i++)
+        if (values[i] > row_max) row_max = values[i];
+    float total = 0.0f;
+    for (uint32_t i = 0; i < n; i++) total = total + softmax_exp(values[i] - row_max);
+    /* rank_row: the next candidate is the best of those that rank after the previous one */
+    float kept_value[64];
+    uint32_t kept_index[64];
+    uint32_t count = 0;
+    float previous_value = INFINITY;
+    uint32_t previous_index = 0xffffffffu;
+    while (count < draw.keep && count < 64) {
+        uint32_t best = 0xffffffffu;
+        for (uint32_t i = 0; i < n; i++) {
+            int after = previous_index == 0xffffffffu || values[i] < previous_value || (values[i] == previous_value && i > previous_index);
+            if (!after) continue;
+            if (best == 0xffffffffu || values[i] > values[best]) best = i; /* equal values: the lower index stays */
+        }
+        if (best == 0xffffffffu) break;
+        kept_value[count] = values[best], kept_index[count] = best;
+        previous_value = values[best], previous_index = best;
+        count++;
+    }
+    float mass = 0.0f;
+    for (uint32_t c = 0; c < count; c++) mass = mass + softmax_exp(kept_value[c] - row_max);
+    float tail = total - mass;
+    float threshold = draw.cumulative * total;
+    uint32_t boundary = count;
+    float running = 0.0f;
+    for (uint32_t c = 0; c < count; c++) {
+        running = running + softmax_exp(kept_value[c] - row_max);
+        if (running + tail >= threshold && c + 1 < boundary) boundary = c + 1;
+    }
+    float best = -INFINITY;
+    for (uint32_t c = 0; c < boundary; c++) {
+        float weight = kept_value[c] + oracle_gumbel_noise(draw.seed, kept_index[c]);
+        if (chosen == 0xffffffffu || weight > best || (weight == best && kept_index[c] < chosen)) best = weight, chosen = kept_index[c];
+    }
+    free(values);
+    return chosen == 0xffffffffu ? 0u : chosen;
+}
+
+/* graph.sample over rows of n logits: out[r] drawn with draws[r] */
+int oracle_sample(const float *logits, uint32_t rows, uint32_t n, const oracle_draw *draws, uint32_t *out) {
+    for (uint32_t r = 0; r < rows; r++) {
+        oracle_draw d = draws[r];
+        if (!(d.temperature > 0.0f) || isinf(d.temperature) || d.keep < 1 || d.keep > 64 || !(d.cumulative > 0.0f) || !(d.cumulative <= 1.0f)) return -1;
+        out[r] = sample_row(logits + (size_t)r * n, n, d);
+    }
+    return 0;
+}
+
+/* crates/neura-generate/src/batch.rs:1841-1847: the seed of plane `slot` under a batch seed, and the bits a batch writes */
+uint32_t oracle_plane_seed(uint32_t seed, uint32_t slot) { return seed ^ ((slot + 1u) * 0x9e3779b9u); }
+uint32_t oracle_seed_bits(uint32_t seed) { return 0x3f800000u | ((seed ^ (seed >> 23)) & 0x007fffffu); }
 
 /* -------------------------------------------------------------- model ---- */
 

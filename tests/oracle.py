@@ -47,6 +47,12 @@ def lib():
         held.oracle_payload_bytes.argtypes = [c_int, c_uint64]
         held.oracle_argmax.restype = c_uint32
         held.oracle_argmax.argtypes = [c_void_p, c_uint32]
+        held.oracle_gumbel_noise.restype = c_float
+        held.oracle_gumbel_noise.argtypes = [c_uint32, c_uint32]
+        held.oracle_plane_seed.restype = c_uint32
+        held.oracle_plane_seed.argtypes = [c_uint32, c_uint32]
+        held.oracle_seed_bits.restype = c_uint32
+        held.oracle_seed_bits.argtypes = [c_uint32]
         _lib = held
     return _lib
 
@@ -171,6 +177,26 @@ def attention_f64(q, K, V, kv_heads, origin, causal, scale):
 def argmax(values):
     values = np.ascontiguousarray(values, dtype=np.float32)
     return lib().oracle_argmax(_p(values), c_uint32(values.size))
+
+
+DRAW = np.dtype([("seed", np.uint32), ("temperature", np.float32), ("keep", np.uint32), ("cumulative", np.float32)])
+
+
+def draws(entries):
+    """[(seed, temperature, keep, cumulative), ...] as the records both libraries take"""
+    return np.array([tuple(entry) for entry in entries], dtype=DRAW)
+
+
+def sample(logits, drawn):
+    """one column per row of `logits`, drawn as graph.sample draws it (oracle_sample)"""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    logits = logits.reshape(-1, logits.shape[-1])
+    drawn = np.ascontiguousarray(drawn, dtype=DRAW)
+    assert drawn.size == logits.shape[0]
+    out = np.empty(logits.shape[0], dtype=np.uint32)
+    status = lib().oracle_sample(_p(logits), c_uint32(logits.shape[0]), c_uint32(logits.shape[1]), _p(drawn), _p(out))
+    assert status == 0, status
+    return out
 
 
 class Model:

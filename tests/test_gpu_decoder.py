@@ -120,6 +120,38 @@ def test_mixed_elements_and_projection_biases(device, batch, base, mixed):
     model.release(), weights.release()
 
 
+def test_sampled_decode_steps_draw_as_the_oracle_draws(device):
+    """A sampled answer program: the same forward pass, the choice drawn per plane with its own seed, temperature,
+    candidate count and nucleus, all written by the host before each step (the recorded graph is replayed with new
+    draws).  The draw is checked on the device's own logits, the logits against the oracle's as in the greedy test."""
+    shape = SMALL_Q4
+    model, ref, weights = build(device, shape, NH_Q4_K, batch=3, context=40)
+    rng = np.random.default_rng(9)
+    tokens = rng.integers(0, shape["vocab"], 3)
+    seeds = [oracle.lib().oracle_plane_seed(1234, slot) for slot in range(3)]
+    for step in range(8):
+        cursors = [step] * 3
+        mask = [1, 1, 1] if step % 3 else [1, 0, 1]
+        drawn = oracle.draws([(oracle.lib().oracle_seed_bits((seeds[slot] + step) & 0xFFFFFFFF), [0.8, 1.0, 1.3][slot], [40, 1, 64][slot],
+                               [0.9, 1.0, 0.5][slot]) for slot in range(3)])
+        want_logits, greedy = ref.forward(tokens, 1, cursors, mask=mask)
+        got = model.decode_step_sampled(tokens, cursors, drawn, mask=mask)
+        logits = model.logits()
+        live = [slot for slot in range(3) if mask[slot]]
+        assert np.abs(logits[live] - want_logits[live]).max() <= 1e-3 * np.abs(want_logits[live]).max(), step
+        want = oracle.sample(logits, drawn)
+        assert [got[slot] for slot in live] == [want[slot] for slot in live], step
+        if mask[1]:
+            assert got[1] == greedy[1]  # a plane that keeps one candidate answers greedily
+        tokens = [int(got[slot]) if mask[slot] else int(tokens[slot]) for slot in range(3)]
+    # a greedy step after sampled ones still answers with the argmax
+    want_logits, greedy = ref.forward(tokens, 1, [8] * 3)
+    assert list(model.decode_step(tokens, [8] * 3)) == list(greedy)
+    with pytest.raises(NeuraError):
+        model.decode_step_sampled(tokens, [9] * 3, oracle.draws([(1, 1.0, 70, 1.0)] * 3))
+    model.release(), weights.release()
+
+
 def test_decode_refuses_what_the_reference_refuses(device):
     model, ref, weights = build(device, TINY, NH_Q8_0, batch=1, context=8)
     with pytest.raises(NeuraError):   # cursor at the context (batch.rs:1627-1632)

@@ -398,6 +398,68 @@ def test_attention_refuses_a_cursor_past_its_keys(device):
         device.attention(q, K, K, 2, 8, 8, [0], 0.0)  # refusal::KNOB (attention.rs:128-132)
 
 
+@pytest.mark.parametrize("n", [1, 32, 1000, 4096, 4097, 20000, 152064])
+def test_sample_matches_the_oracle(device, n):
+    """nh_sample against the oracle's restatement of sample_row on the same logits: every keep from 1 to 64, tight and open
+    nuclei, temperatures either side of one, many seeds.  Columns can only differ where two candidates' value + noise tie
+    within the last bits of the device's and the host's logarithms, which these seeds do not meet."""
+    rng = np.random.default_rng(n)
+    rows = 96
+    logits = (rng.standard_normal((rows, n)) * 3.0).astype(np.float32)
+    drawn = oracle.draws([(int(rng.integers(0, 2 ** 32)), float(rng.choice([0.25, 0.7, 1.0, 1.5, 4.0])), int(rng.integers(1, 65)),
+                           float(rng.choice([0.05, 0.5, 0.85, 0.95, 1.0]))) for _ in range(rows)])
+    got = device.sample(logits, drawn)
+    want = oracle.sample(logits, drawn)
+    assert list(got) == list(want)
+    # the reference's own properties (crates/neura-runtime/tests/choice.rs:41-126)
+    first = oracle.draws([(s, 1.0, 1, 1.0) for s in range(rows)])
+    assert list(device.sample(logits, first)) == [int(np.argmax(row)) for row in logits]
+    if n >= 32:
+        pair = oracle.draws([(0x2F0F1A3B, 1.0, 6, 0.85), (0x91E10D57, 1.0, 6, 0.85)])
+        alone = [int(device.sample(logits[r:r + 1], pair[r:r + 1])[0]) for r in range(2)]
+        assert list(device.sample(logits[:2], pair)) == alone
+
+
+def test_sample_ranks_ties_by_column_and_refuses_what_the_reference_refuses(device):
+    # equal logits rank by column: keep 4 of 5000 equal columns leaves the first four, in any section
+    flat = np.zeros((256, 5000), dtype=np.float32)
+    got = device.sample(flat, oracle.draws([(seed, 1.0, 4, 1.0) for seed in range(256)]))
+    assert set(got) == {0, 1, 2, 3}
+    assert list(got) == list(oracle.sample(flat, oracle.draws([(seed, 1.0, 4, 1.0) for seed in range(256)])))
+    # integers in a narrow range: many exact ties across sections
+    rng = np.random.default_rng(3)
+    tied = rng.integers(0, 40, (64, 152064)).astype(np.float32)
+    drawn = oracle.draws([(seed * 977, 1.0, 64, 1.0) for seed in range(64)])
+    assert list(device.sample(tied, drawn)) == list(oracle.sample(tied, drawn))
+    one = np.zeros((1, 8), dtype=np.float32)
+    for bad in ((1, 0.0, 4, 1.0), (1, np.inf, 4, 1.0), (1, np.nan, 4, 1.0), (1, 1.0, 0, 1.0), (1, 1.0, 65, 1.0), (1, 1.0, 4, 0.0), (1, 1.0, 4, 1.5)):
+        with pytest.raises(NeuraError):  # crates/neura-generate/src/sampling.rs:16-29
+            device.sample(one, oracle.draws([bad]))
+    with pytest.raises(NeuraError):
+        device.sample(np.zeros((1, 262145), dtype=np.float32), oracle.draws([(1, 1.0, 4, 1.0)]))
+
+
+def test_sample_frequencies_follow_the_softmax_of_the_kept_candidates(device):
+    # Gumbel-max on the device: 4096 rows of the same logits under 4096 seeds
+    rng = np.random.default_rng(5)
+    row = rng.normal(0, 1.5, 12).astype(np.float32)
+    logits = np.tile(row, (4096, 1))
+    for temperature, keep in ((1.0, 12), (0.5, 12), (2.0, 5)):
+        scaled = row.astype(np.float64) / temperature
+        kept = np.argsort(-scaled, kind="stable")[:keep]
+        p = np.zeros(12)
+        p[kept] = np.exp(scaled[kept] - scaled.max())
+        p /= p.sum()
+        counts = np.zeros(12)
+        for batch in range(5):
+            drawn = oracle.draws([((batch * 4096 + seed) * 2654435761 % 2 ** 32, temperature, keep, 1.0) for seed in range(4096)])
+            counts += np.bincount(device.sample(logits, drawn), minlength=12)
+        assert counts[p == 0].sum() == 0
+        expected = p * counts.sum()
+        chi2 = ((counts - expected) ** 2 / np.maximum(expected, 1e-9))[p > 0].sum()
+        assert chi2 < 45, (temperature, keep, chi2)
+
+
 def test_argmax_lowest_index_on_ties(device):
     rng = np.random.default_rng(10)
     values = rng.integers(0, 1000, (3, 151936)).astype(np.float32)  # many exact ties
