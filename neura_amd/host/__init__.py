@@ -55,6 +55,15 @@ SIGNATURES = {
     "nhost_runtime_open": (c_void_p, [c_int32]),
     "nhost_runtime_close": (None, [c_void_p]),
     "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_open_sampled": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_float, c_uint32, c_float]),
+    "nhost_sampling_check": (c_int32, [c_float, c_uint32, c_float]),
+    "nhost_plane_seed": (c_uint32, [c_uint32, c_uint32]),
+    "nhost_seed_bits": (c_uint32, [c_uint32]),
+    "nhost_batch_set_seed": (c_int32, [c_void_p, c_int32, c_uint32]),
+    "nhost_batch_seed_of": (c_int64, [c_void_p, c_uint32]),
+    "nhost_batch_set_temperature": (c_int32, [c_void_p, c_int32, c_float]),
+    "nhost_batch_set_keep": (c_int32, [c_void_p, c_int32, c_uint32]),
+    "nhost_batch_set_cumulative": (c_int32, [c_void_p, c_int32, c_float]),
     "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
     "nhost_batch_close": (None, [c_void_p]),
     "nhost_batch_admit": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
@@ -270,6 +279,20 @@ def batch_spec_check(context, batch, chunks):
         raise _refused()
 
 
+def sampling_check(temperature, keep, cumulative):
+    """Sampling::sampled's refusals (crates/neura-generate/src/sampling.rs:16-29), with no device"""
+    if library().nhost_sampling_check(temperature, keep, cumulative) != 0:
+        raise _refused()
+
+
+def plane_seed(seed, slot):
+    return int(library().nhost_plane_seed(seed, slot))
+
+
+def seed_bits(seed):
+    return int(library().nhost_seed_bits(seed))
+
+
 def payload_bytes(element, elements):
     return int(library().nhost_payload_bytes(element, elements))
 
@@ -287,15 +310,37 @@ class Runtime:
 
 
 class Batch:
-    """A Qwen2 GGUF loaded onto a runtime with a greedy generation batch above it."""
+    """A Qwen2 GGUF loaded onto a runtime with a generation batch above it: greedy, or drawing with
+    `sampling` = (temperature, keep, cumulative) as BatchSpec::sampled(Sampling::sampled(..)) does."""
 
-    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=()):
+    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None):
         held, count = _words(chunks)
         self.planes = batch
         self.vocabulary = vocabulary
-        self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count)
+        if sampling is None:
+            self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count)
+        else:
+            temperature, keep, cumulative = sampling
+            self.handle = library().nhost_batch_open_sampled(runtime.handle, archive.handle, vocabulary, context, batch, held, count,
+                                                             temperature, keep, cumulative)
         if not self.handle:
             raise _refused()
+
+    # what a sampled batch draws with (crates/neura-generate/src/batch.rs:643-732, :829-864); slot None names every plane
+    def set_seed(self, seed, slot=None):
+        self._status(library().nhost_batch_set_seed(self.handle, -1 if slot is None else slot, seed))
+
+    def seed_of(self, slot):
+        return self._status(library().nhost_batch_seed_of(self.handle, slot))
+
+    def set_temperature(self, value, slot=None):
+        self._status(library().nhost_batch_set_temperature(self.handle, -1 if slot is None else slot, value))
+
+    def set_keep(self, keep, slot=None):
+        self._status(library().nhost_batch_set_keep(self.handle, -1 if slot is None else slot, keep))
+
+    def set_cumulative(self, value, slot=None):
+        self._status(library().nhost_batch_set_cumulative(self.handle, -1 if slot is None else slot, value))
 
     def close(self):
         if self.handle:

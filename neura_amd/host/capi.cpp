@@ -194,6 +194,62 @@ void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t 
         return out.release();
     }, nullptr);
 }
+// the same with a sampled answer (BatchSpec::sampled(Sampling::sampled(temperature, keep, cumulative)))
+void *nhost_batch_open_sampled(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
+                               float temperature, uint32_t keep, float cumulative) {
+    return guarded([&]() -> void * {
+        auto *opened = static_cast<Opened *>(held);
+        generate::BatchSpec spec =
+            generate::BatchSpec(context, batch, std::vector<uint32_t>(chunks, chunks + count)).sampled(generate::Sampling::sampled(temperature, keep, cumulative));
+        auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
+        auto out = std::make_unique<Loaded>();
+        out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
+        out->batch = std::make_unique<generate::Batch>(*out->model, spec);
+        return out.release();
+    }, nullptr);
+}
+// Sampling::sampled's refusals alone, with no device
+int32_t nhost_sampling_check(float temperature, uint32_t keep, float cumulative) {
+    return guarded([&] { return generate::Sampling::sampled(temperature, keep, cumulative), 0; }, -1);
+}
+uint32_t nhost_plane_seed(uint32_t seed, uint32_t slot) { return generate::Batch::plane_seed(seed, slot); }
+uint32_t nhost_seed_bits(uint32_t seed) { return generate::Batch::seed_bits(seed); }
+// what a sampled batch draws with; slot < 0 names every plane
+int32_t nhost_batch_set_seed(void *held, int32_t slot, uint32_t seed) {
+    return guarded([&] {
+        auto &batch = *static_cast<Loaded *>(held)->batch;
+        if (slot < 0) batch.set_seed(seed);
+        else batch.set_seed_of((uint32_t)slot, seed);
+        return 0;
+    }, -1);
+}
+int64_t nhost_batch_seed_of(void *held, uint32_t slot) {
+    return guarded([&]() -> int64_t { return (int64_t) static_cast<Loaded *>(held)->batch->seed_of(slot); }, -1);
+}
+int32_t nhost_batch_set_temperature(void *held, int32_t slot, float value) {
+    return guarded([&] {
+        auto &batch = *static_cast<Loaded *>(held)->batch;
+        if (slot < 0) batch.set_temperature(value);
+        else batch.set_temperature_of((uint32_t)slot, value);
+        return 0;
+    }, -1);
+}
+int32_t nhost_batch_set_keep(void *held, int32_t slot, uint32_t keep) {
+    return guarded([&] {
+        auto &batch = *static_cast<Loaded *>(held)->batch;
+        if (slot < 0) batch.set_keep(keep);
+        else batch.set_keep_of((uint32_t)slot, keep);
+        return 0;
+    }, -1);
+}
+int32_t nhost_batch_set_cumulative(void *held, int32_t slot, float value) {
+    return guarded([&] {
+        auto &batch = *static_cast<Loaded *>(held)->batch;
+        if (slot < 0) batch.set_cumulative(value);
+        else batch.set_cumulative_of((uint32_t)slot, value);
+        return 0;
+    }, -1);
+}
 // BatchSpec's refusals alone, with no device: a batch over no model
 int32_t nhost_batch_spec_check(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count) {
     return guarded([&] {

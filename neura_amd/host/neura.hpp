@@ -8,6 +8,7 @@
 #pragma once
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
@@ -798,10 +799,40 @@ struct Config {
 };
 
 // crates/neura-generate/src/batch.rs:110-153 (greedy; sampling, tuning, sharing and windows are not built)
+// crates/neura-generate/src/sampling.rs:3-57: a batch answers with the largest logit, or draws among the `keep` largest
+// cut at a cumulative mass after dividing the logits by a temperature
+struct Sampling {
+    bool greedy = true;
+    float temperature = 1.0f;
+    uint32_t keep = 1;
+    float cumulative = 1.0f;
+    static constexpr uint32_t CANDIDATES = 64;  // crates/neura-abi/src/lib.rs:39
+    static Sampling sampled(float temperature, uint32_t keep, float cumulative) {
+        check_temperature(temperature);
+        NEURA_ASSERT(keep >= 1 && keep <= CANDIDATES, "a sample keeps %u candidates where a row holds between one and %u", keep, CANDIDATES);
+        check_cumulative(cumulative);
+        Sampling out;
+        out.greedy = false, out.temperature = temperature, out.keep = keep, out.cumulative = cumulative;
+        return out;
+    }
+    static void check_temperature(float value) {
+        NEURA_ASSERT(value > 0.0f && std::isfinite(value), "a sampling temperature of %g spreads no logits", (double)value);
+    }
+    static void check_cumulative(float value) {
+        NEURA_ASSERT(value > 0.0f && value <= 1.0f, "a cumulative mass of %g keeps no candidate or names more than every candidate", (double)value);
+    }
+};
+
 struct BatchSpec {
     uint32_t context, batch;
     std::vector<uint32_t> chunks;
+    Sampling sampling;
     BatchSpec(uint32_t context, uint32_t batch, std::vector<uint32_t> chunks) : context(context), batch(batch), chunks(std::move(chunks)) {}
+    BatchSpec sampled(Sampling held) const {  // crates/neura-generate/src/batch.rs:133-136
+        BatchSpec out = *this;
+        out.sampling = held;
+        return out;
+    }
 };
 
 struct Emitted {  // crates/neura-generate/src/batch.rs:155-159
@@ -901,9 +932,10 @@ class Model {
     nh_model *model_ = nullptr;
 };
 
-// The greedy generation state machine (crates/neura-generate/src/batch.rs:279-465, :1000-1172,
+// The generation state machine (crates/neura-generate/src/batch.rs:279-465, :1000-1172,
 // :1401-1517, :1595-1725): admit / restart / resume / suspend / finish / step with chunked
-// prompt fill.  Single threaded, one model, like `&mut Batch`.
+// prompt fill; greedy, or sampled with per-plane seeds, temperatures, candidate counts and nuclei
+// (:643-732, :829-864).  Single threaded, one model, like `&mut Batch`.
 class Batch {
   public:
     // the constructor's refusals, callable without a model
@@ -918,9 +950,66 @@ class Batch {
                          "a batch fills %u rows of a context of %u, and a chunk holds between two rows and the rows a prompt leaves for the answer",
                          chunk, spec.context);
     }
-    Batch(Model &model, BatchSpec spec) : model_(model), batch_(spec.batch), context_(spec.context), chunks_(spec.chunks), slots_(spec.batch) {
+    Batch(Model &model, BatchSpec spec)
+        : model_(model), batch_(spec.batch), context_(spec.context), chunks_(spec.chunks), slots_(spec.batch), seeded_(!spec.sampling.greedy),
+          temperatures_(spec.batch, spec.sampling.temperature), keeps_(spec.batch, spec.sampling.keep), cumulatives_(spec.batch, spec.sampling.cumulative) {
         validate(spec);
+        for (uint32_t slot = 0; slot < batch_; slot++) seeds_.push_back(plane_seed(0, slot));  // batch.rs:426-428
     }
+
+    // ---- what a sampled batch draws with (crates/neura-generate/src/batch.rs:643-732, :829-864): written by the host
+    // between steps, per plane or for every plane
+    bool sampled() const { return seeded_; }
+    uint32_t seed_of(uint32_t slot) const {
+        plane(slot);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no seed");
+        return seeds_[slot];
+    }
+    void set_seed(uint32_t seed) {
+        NEURA_ASSERT(seeded_, "a greedy batch draws no seed");
+        for (uint32_t slot = 0; slot < batch_; slot++) seeds_[slot] = plane_seed(seed, slot);
+    }
+    void set_seed_of(uint32_t slot, uint32_t seed) {
+        plane(slot);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no seed");
+        seeds_[slot] = seed;
+    }
+    void set_temperature(float value) {
+        Sampling::check_temperature(value);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no temperature");
+        std::fill(temperatures_.begin(), temperatures_.end(), value);
+    }
+    void set_temperature_of(uint32_t slot, float value) {
+        plane(slot);
+        Sampling::check_temperature(value);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no temperature");
+        temperatures_[slot] = value;
+    }
+    void set_keep(uint32_t keep) {
+        check_keep(keep);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no candidate count");
+        std::fill(keeps_.begin(), keeps_.end(), keep);
+    }
+    void set_keep_of(uint32_t slot, uint32_t keep) {
+        plane(slot);
+        check_keep(keep);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no candidate count");
+        keeps_[slot] = keep;
+    }
+    void set_cumulative(float value) {
+        Sampling::check_cumulative(value);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no cumulative mass");
+        std::fill(cumulatives_.begin(), cumulatives_.end(), value);
+    }
+    void set_cumulative_of(uint32_t slot, float value) {
+        plane(slot);
+        Sampling::check_cumulative(value);
+        NEURA_ASSERT(seeded_, "a greedy batch draws no cumulative mass");
+        cumulatives_[slot] = value;
+    }
+    // crates/neura-generate/src/batch.rs:1841-1847: the seed of a plane under a batch seed, and the bits a batch writes for it
+    static uint32_t plane_seed(uint32_t seed, uint32_t slot) { return seed ^ ((slot + 1u) * 0x9e3779b9u); }
+    static uint32_t seed_bits(uint32_t seed) { return 0x3f800000u | ((seed ^ (seed >> 23)) & 0x007fffffu); }
     uint32_t batch() const { return batch_; }
     uint32_t context() const { return context_; }
 
@@ -1052,11 +1141,21 @@ class Batch {
             tokens[slot] = held.phase == Prompting ? held.prompt.front() : held.feed;
             cursors[slot] = held.cursor, mask[slot] = 1;
         }
-        runtime::check(nh_decode_step(model_.handle(), tokens.data(), cursors.data(), mask.data(), batch_, chosen.data()));
+        if (seeded_) {
+            std::vector<nh_draw> draws(batch_);
+            for (uint32_t slot = 0; slot < batch_; slot++)
+                draws[slot] = nh_draw{seed_bits(seeds_[slot]), temperatures_[slot], keeps_[slot], cumulatives_[slot]};
+            runtime::check(nh_decode_step_sampled(model_.handle(), tokens.data(), cursors.data(), mask.data(), batch_, draws.data(), chosen.data()));
+        } else {
+            runtime::check(nh_decode_step(model_.handle(), tokens.data(), cursors.data(), mask.data(), batch_, chosen.data()));
+        }
         std::vector<Emitted> emitted;
         for (uint32_t slot = 0; slot < batch_; slot++) {
             if (!slots_[slot]) continue;
             auto &held = *slots_[slot];
+            // a plane draws when it answers: on the last token of its prompt and on every token after (batch.rs:1688-1709)
+            const bool drew = held.phase == Generating || (held.phase == Prompting && held.prompt.size() == 1);
+            if (drew) seeds_[slot] += 1u;
             if (held.phase == Prompting) {
                 held.prompt.pop_front();
                 if (held.prompt.empty()) held.phase = Generating, held.feed = chosen[slot];
@@ -1069,10 +1168,21 @@ class Batch {
         return emitted;
     }
 
+    void plane(uint32_t slot) const { NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot); }
+    static void check_keep(uint32_t keep) {
+        NEURA_ASSERT(keep >= 1 && keep <= Sampling::CANDIDATES, "a batch keeps %u candidates where a row holds between one and %u", keep,
+                     Sampling::CANDIDATES);
+    }
+
     Model &model_;
     uint32_t batch_, context_;
     std::vector<uint32_t> chunks_;
     std::vector<std::optional<Slot>> slots_;
+    bool seeded_;
+    std::vector<uint32_t> seeds_;
+    std::vector<float> temperatures_;
+    std::vector<uint32_t> keeps_;
+    std::vector<float> cumulatives_;
 };
 
 }  // namespace generate

@@ -111,6 +111,96 @@ def test_a_file_of_mixed_storage_with_projection_biases_generates(runtime, tmp_p
     archive.close()
 
 
+def test_a_sampled_batch_draws_by_plane_seeds_the_host_can_write(runtime, tmp_path):
+    """BatchSpec::sampled: every plane draws with its own seed (plane_seed of the batch seed, one further per draw),
+    temperature, candidate count and nucleus (crates/neura-generate/src/batch.rs:643-732, :829-864, :1688-1709).  Each
+    emitted token is checked against the oracle's draw from the logits the device answered with one step earlier."""
+    shape, element = SHAPE, NH_Q8_0
+    qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=41)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], sampling=(0.9, 40, 0.95))
+    assert [batch.seed_of(slot) for slot in range(2)] == [host.plane_seed(0, slot) for slot in range(2)]
+    batch.set_seed(1234)
+    batch.set_temperature(1.4, slot=1)
+    batch.set_cumulative(0.8, slot=1)
+    batch.set_keep(17, slot=1)
+    settings = [(0.9, 40, 0.95), (1.4, 17, 0.8)]
+    rng = np.random.default_rng(42)
+    prompts = [list(rng.integers(0, shape["vocab"], n)) for n in (3, 12)]
+    slots = [batch.admit(prompt) for prompt in prompts]
+    draws = [0, 0]
+    pending = {}  # slot -> the token the oracle expects the plane to emit next
+    emitted = {0: [], 1: []}
+    for step in range(30):
+        before = [batch.seed_of(slot) for slot in slots]
+        out = batch.step()
+        for slot, token in out:
+            assert token == pending[slot], (step, slot)
+            emitted[slot].append(token)
+        logits = batch.logits()
+        for slot in slots:
+            if batch.seed_of(slot) != before[slot]:  # the plane drew on this step
+                assert batch.seed_of(slot) == (before[slot] + 1) & 0xFFFFFFFF
+                assert before[slot] == (host.plane_seed(1234, slot) + draws[slot]) & 0xFFFFFFFF
+                draws[slot] += 1
+                temperature, keep, cumulative = settings[slot]
+                pending[slot] = int(oracle.sample(logits[slot:slot + 1], oracle.draws([(host.seed_bits(before[slot]), temperature, keep, cumulative)]))[0])
+    assert len(emitted[0]) >= 20 and len(emitted[1]) >= 15
+    assert len(set(emitted[0])) > 3  # a temperature near one spreads the answers of a random-init decoder
+    batch.close()
+
+    # the same seed answers the same; another seed answers otherwise
+    streams = []
+    for seed in (1234, 1234, 99):
+        again = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], sampling=(0.9, 40, 0.95))
+        again.set_seed(seed)
+        again.set_temperature(1.4, slot=1), again.set_cumulative(0.8, slot=1), again.set_keep(17, slot=1)
+        for prompt in prompts:
+            again.admit(prompt)
+        streams.append(run(again, {0: 20, 1: 15}))
+        again.close()
+    assert streams[0] == {0: emitted[0][:20], 1: emitted[1][:15]} == streams[1]
+    assert streams[2] != streams[0]
+    archive.close()
+
+
+def test_a_temperature_and_a_candidate_count_the_host_writes_steer_the_draws(runtime, tmp_path):
+    # crates/neura-generate/tests/generation.rs:564-627 and the test after it, on a decoder instead of constant logits
+    shape, element = SHAPE, NH_Q8_0
+    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=43)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    prompt = [5, 9, 2, 77]
+    greedy, margin = alone(shape, element, tensors, prompt, 12)
+    batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [], sampling=(1.0, 64, 1.0))
+    batch.set_temperature(1e-4)  # logits 10^4 apart leave the noise nothing to move
+    batch.admit(prompt), batch.admit(prompt)
+    assert run(batch, {0: 12, 1: 12}) == {0: greedy, 1: greedy}, margin
+    # plane 0 hot, plane 1 keeping one candidate: the one stays greedy while the other spreads
+    batch.restart(0, prompt), batch.restart(1, prompt)
+    batch.set_temperature(1000.0)
+    batch.set_keep(1, slot=1)
+    got = run(batch, {0: 40, 1: 12})
+    assert got[1] == greedy, margin
+    assert len(set(got[0])) > 10 and got[0][:12] != greedy
+    with pytest.raises(host.Panic, match="a batch of 2 planes names no plane 2"):
+        batch.set_keep(3, slot=2)
+    with pytest.raises(host.Panic, match="a batch keeps 65 candidates where a row holds between one and 64"):
+        batch.set_keep(65)
+    with pytest.raises(host.Panic, match="a sampling temperature of 0 spreads no logits"):
+        batch.set_temperature(0.0)
+    with pytest.raises(host.Panic, match="a cumulative mass of 2 keeps no candidate"):
+        batch.set_cumulative(2.0)
+    batch.close()
+    plain = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 1, [])
+    for refused, sentence in ((lambda: plain.set_temperature(1.0), "a greedy batch draws no temperature"), (lambda: plain.set_keep(4), "a greedy batch draws no candidate count"),
+                              (lambda: plain.set_cumulative(0.5), "a greedy batch draws no cumulative mass"), (lambda: plain.set_seed(1), "a greedy batch draws no seed"),
+                              (lambda: plain.seed_of(0), "a greedy batch draws no seed")):
+        with pytest.raises(host.Panic, match=sentence):
+            refused()
+    plain.close()
+    archive.close()
+
+
 def test_a_batch_keeps_the_planes_it_is_told_to(runtime, tmp_path):
     shape, element = SHAPE, NH_Q8_0
     tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=21)

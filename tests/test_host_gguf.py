@@ -209,3 +209,26 @@ def test_a_batch_refuses_a_spec_it_cannot_fill():
     refuses(lambda: host.batch_spec_check(128, 1, [8, 8]), "fills 8 then 8")
     refuses(lambda: host.batch_spec_check(128, 1, [8, 1]), "a batch fills 1 rows of a context of 128")
     refuses(lambda: host.batch_spec_check(64, 1, [64]), "a batch fills 64 rows of a context of 64")
+
+
+def test_a_sampling_refuses_what_spreads_or_keeps_nothing():
+    # crates/neura-generate/src/sampling.rs:16-29
+    host.sampling_check(1.0, 1, 1.0)
+    host.sampling_check(0.01, 64, 0.05)
+    refuses(lambda: host.sampling_check(0.0, 4, 1.0), "a sampling temperature of 0 spreads no logits")
+    refuses(lambda: host.sampling_check(float("inf"), 4, 1.0), "a sampling temperature of inf spreads no logits")
+    refuses(lambda: host.sampling_check(1.0, 0, 1.0), "a sample keeps 0 candidates where a row holds between one and 64")
+    refuses(lambda: host.sampling_check(1.0, 65, 1.0), "a sample keeps 65 candidates where a row holds between one and 64")
+    refuses(lambda: host.sampling_check(1.0, 4, 0.0), "a cumulative mass of 0 keeps no candidate or names more than every candidate")
+    refuses(lambda: host.sampling_check(1.0, 4, 1.5), "a cumulative mass of 1.5 keeps no candidate")
+
+
+def test_plane_seeds_and_the_bits_a_batch_writes():
+    # crates/neura-generate/src/batch.rs:1841-1847, against the oracle's restatement and by hand
+    import oracle
+
+    assert host.plane_seed(0, 0) == 0x9E3779B9 and host.plane_seed(0, 1) == (2 * 0x9E3779B9) & 0xFFFFFFFF
+    for seed in (0, 1, 77, 0x9E3779B9, 0xFFFFFFFF):
+        for slot in (0, 1, 7):
+            assert host.plane_seed(seed, slot) == oracle.lib().oracle_plane_seed(seed, slot)
+        assert host.seed_bits(seed) == oracle.lib().oracle_seed_bits(seed) == 0x3F800000 | ((seed ^ (seed >> 23)) & 0x7FFFFF)
