@@ -65,6 +65,16 @@ SIGNATURES = {
     "nhost_batch_set_keep": (c_int32, [c_void_p, c_int32, c_uint32]),
     "nhost_batch_set_cumulative": (c_int32, [c_void_p, c_int32, c_float]),
     "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_tokenizer_open": (c_void_p, [c_void_p, c_char_p]),
+    "nhost_tokenizer_close": (None, [c_void_p]),
+    "nhost_tokenizer_vocabulary": (c_uint64, [c_void_p]),
+    "nhost_tokenizer_id": (c_int64, [c_void_p, c_char_p]),
+    "nhost_tokenizer_encode": (c_int64, [c_void_p, c_char_p, c_size_t, POINTER(c_uint32), c_size_t]),
+    "nhost_tokenizer_piece": (c_int64, [c_void_p, c_uint32, c_void_p, c_size_t]),
+    "nhost_rule_pieces": (c_int64, [c_char_p, c_char_p, c_size_t, POINTER(c_uint64), c_size_t]),
+    "nhost_text_open": (c_void_p, []),
+    "nhost_text_close": (None, [c_void_p]),
+    "nhost_text_push": (c_int64, [c_void_p, c_void_p, c_size_t, c_int32, c_void_p, c_size_t]),
     "nhost_batch_close": (None, [c_void_p]),
     "nhost_batch_admit": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
     "nhost_batch_restart": (c_int32, [c_void_p, c_uint32, POINTER(c_uint32), c_uint32]),
@@ -277,6 +287,87 @@ def batch_spec_check(context, batch, chunks):
     held, count = _words(chunks)
     if library().nhost_batch_spec_check(context, batch, held, count) != 0:
         raise _refused()
+
+
+class Tokenizer:
+    """crates/neura-tokenizer: the byte level bpe a gpt2 GGUF holds under a split rule ("qwen", or "per_character",
+    "per_space", "whole" as the reference's own tests define them)."""
+
+    def __init__(self, archive, rule="qwen"):
+        self.handle = library().nhost_tokenizer_open(archive.handle, rule.encode())
+        if not self.handle:
+            raise _refused()
+
+    def close(self):
+        if self.handle:
+            library().nhost_tokenizer_close(self.handle)
+            self.handle = None
+
+    def vocabulary(self):
+        return int(library().nhost_tokenizer_vocabulary(self.handle))
+
+    def id(self, token):
+        held = library().nhost_tokenizer_id(self.handle, token.encode())
+        return None if held < 0 else int(held)
+
+    def encode(self, text):
+        raw = text.encode() if isinstance(text, str) else bytes(text)
+        room = (c_uint32 * max(1, len(raw)))()  # a token spells at least one byte
+        count = library().nhost_tokenizer_encode(self.handle, raw, len(raw), room, len(room))
+        if count < 0:
+            raise _refused()
+        return list(room[:count])
+
+    def piece(self, id):
+        room = ctypes.create_string_buffer(1024)
+        length = library().nhost_tokenizer_piece(self.handle, id, room, len(room))
+        if length < 0:
+            raise _refused()
+        return room.raw[:length]
+
+    def decode(self, ids):
+        """the text the pieces of `ids` spell (through Text: ill-formed bytes read as U+FFFD)"""
+        text = Text()
+        out = "".join(text.push(self.piece(id)) for id in ids) + text.flush()
+        text.close()
+        return out
+
+
+def rule_pieces(rule, text):
+    """the pieces a split rule cuts a text into"""
+    raw = text.encode()
+    ends = (c_uint64 * max(1, len(raw)))()
+    count = library().nhost_rule_pieces(rule.encode(), raw, len(raw), ends, len(ends))
+    if count < 0:
+        raise _refused()
+    out, at = [], 0
+    for end in ends[:count]:
+        out.append(raw[at:end].decode())
+        at = end
+    return out
+
+
+class Text:
+    """crates/neura-tokenizer/src/text.rs: pieces in, whole characters out"""
+
+    def __init__(self):
+        self.handle = library().nhost_text_open()
+
+    def close(self):
+        if self.handle:
+            library().nhost_text_close(self.handle)
+            self.handle = None
+
+    def _call(self, raw, flush):
+        room = ctypes.create_string_buffer(4 * len(raw) + 64)
+        length = library().nhost_text_push(self.handle, raw, len(raw), flush, room, len(room))
+        return room.raw[:length].decode()
+
+    def push(self, piece):
+        return self._call(bytes(piece), 0)
+
+    def flush(self):
+        return self._call(b"", 1)
 
 
 def sampling_check(temperature, keep, cumulative):

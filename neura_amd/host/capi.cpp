@@ -3,6 +3,7 @@
 // (0 done, -1 refused) or a null handle, and nhost_last_error() then holds the sentence the
 // reference would have panicked with.
 #include "neura.hpp"
+#include "tokenizer.hpp"
 
 #include <cstdlib>
 
@@ -32,6 +33,14 @@ struct Loaded {
     std::unique_ptr<generate::Model> model;
     std::unique_ptr<generate::Batch> batch;
 };
+
+std::unique_ptr<tokenizer::Rule> rule_named(const std::string &name) {
+    if (name == "qwen") return std::make_unique<tokenizer::Qwen>();
+    if (name == "per_character") return std::make_unique<tokenizer::PerCharacter>();
+    if (name == "per_space") return std::make_unique<tokenizer::PerSpace>();
+    if (name == "whole") return std::make_unique<tokenizer::Whole>();
+    panic("no split rule is named %s", name.c_str());
+}
 }  // namespace
 
 struct nhost_tensor {
@@ -305,6 +314,55 @@ uint64_t nhost_batch_planes(void *held) {
 }
 int32_t nhost_batch_logits(void *held, float *out) {
     return guarded([&] { return runtime::check(nh_model_logits(static_cast<Loaded *>(held)->model->handle(), out)), 0; }, -1);
+}
+
+// ---- tokenizer ------------------------------------------------------------------------------------
+// the byte level bpe of a gguf under a split rule: "qwen", or the rules of the reference's own tests
+void *nhost_tokenizer_open(void *held, const char *rule) {
+    return guarded([&]() -> void * {
+        return new tokenizer::Tokenizer(tokenizer::Vocabulary::read(static_cast<Opened *>(held)->archive()), rule_named(rule));
+    }, nullptr);
+}
+void nhost_tokenizer_close(void *held) { delete static_cast<tokenizer::Tokenizer *>(held); }
+uint64_t nhost_tokenizer_vocabulary(void *held) { return static_cast<tokenizer::Tokenizer *>(held)->vocabulary(); }
+// -1 when no token is spelled so
+int64_t nhost_tokenizer_id(void *held, const char *token) {
+    auto id = static_cast<tokenizer::Tokenizer *>(held)->id(token);
+    return id ? (int64_t)*id : -1;
+}
+// the ids of `size` bytes of text into out (at most `room`); returns their count, or -1 refused
+int64_t nhost_tokenizer_encode(void *held, const char *text, size_t size, uint32_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto ids = static_cast<tokenizer::Tokenizer *>(held)->encode(std::string_view(text, size));
+        for (size_t i = 0; i < ids.size() && i < room; i++) out[i] = ids[i];
+        return (int64_t)ids.size();
+    }, -1);
+}
+// the bytes of token `id` into out (at most `room`); returns their count, or -1 refused
+int64_t nhost_tokenizer_piece(void *held, uint32_t id, uint8_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto bytes = static_cast<tokenizer::Tokenizer *>(held)->piece(id);
+        for (size_t i = 0; i < bytes.size() && i < room; i++) out[i] = bytes[i];
+        return (int64_t)bytes.size();
+    }, -1);
+}
+// the ends of the pieces a rule cuts `size` bytes of text into (byte offsets, at most `room`); returns their count
+int64_t nhost_rule_pieces(const char *rule, const char *text, size_t size, uint64_t *ends, size_t room) {
+    return guarded([&]() -> int64_t {
+        std::string_view held(text, size);
+        auto pieces = rule_named(rule)->pieces(held);
+        for (size_t i = 0; i < pieces.size() && i < room; i++) ends[i] = (uint64_t)(pieces[i].data() + pieces[i].size() - held.data());
+        return (int64_t)pieces.size();
+    }, -1);
+}
+void *nhost_text_open(void) { return new tokenizer::Text(); }
+void nhost_text_close(void *held) { delete static_cast<tokenizer::Text *>(held); }
+// feeds `size` bytes (flush: size 0 and flush != 0) and copies the text that became whole into out; returns its length
+int64_t nhost_text_push(void *held, const uint8_t *bytes, size_t size, int32_t flush, char *out, size_t room) {
+    auto *text = static_cast<tokenizer::Text *>(held);
+    const std::string whole = flush ? text->flush() : text->push(std::vector<uint8_t>(bytes, bytes + size));
+    for (size_t i = 0; i < whole.size() && i < room; i++) out[i] = whole[i];
+    return (int64_t)whole.size();
 }
 
 }  // extern "C"
