@@ -65,6 +65,11 @@ SIGNATURES = {
     "nhost_batch_set_keep": (c_int32, [c_void_p, c_int32, c_uint32]),
     "nhost_batch_set_cumulative": (c_int32, [c_void_p, c_int32, c_float]),
     "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_snapshot_round_trip": (c_int64, [c_char_p, c_size_t, c_void_p, c_size_t]),
+    "nhost_batch_snapshot": (c_int64, [c_void_p, c_void_p, c_size_t]),
+    "nhost_batch_restore": (c_int32, [c_void_p, c_char_p, c_size_t]),
+    "nhost_batch_save_state": (c_int32, [c_void_p, c_char_p]),
+    "nhost_batch_restore_state": (c_int32, [c_void_p, c_char_p, c_char_p, c_size_t]),
     "nhost_tokenizer_open": (c_void_p, [c_void_p, c_char_p]),
     "nhost_tokenizer_close": (None, [c_void_p]),
     "nhost_tokenizer_vocabulary": (c_uint64, [c_void_p]),
@@ -370,6 +375,15 @@ class Text:
         return self._call(b"", 1)
 
 
+def snapshot_round_trip(raw):
+    """BatchSnapshot::from_bytes then to_bytes (crates/neura-generate/src/snapshot.rs), with no device"""
+    room = ctypes.create_string_buffer(len(raw) + 64)
+    length = library().nhost_snapshot_round_trip(bytes(raw), len(raw), room, len(room))
+    if length < 0:
+        raise _refused()
+    return room.raw[:length]
+
+
 def sampling_check(temperature, keep, cumulative):
     """Sampling::sampled's refusals (crates/neura-generate/src/sampling.rs:16-29), with no device"""
     if library().nhost_sampling_check(temperature, keep, cumulative) != 0:
@@ -460,6 +474,24 @@ class Batch:
 
     def finish(self, slot):
         self._status(library().nhost_batch_finish(self.handle, slot))
+
+    # what the batch holds between steps (crates/neura-generate/src/batch.rs:484-628): the host side as "NBS1" bytes,
+    # the key and value states of the device as a container file
+    def snapshot(self):
+        room = ctypes.create_string_buffer(1 << 20)
+        length = library().nhost_batch_snapshot(self.handle, room, len(room))
+        if length < 0 or length > len(room):
+            raise _refused()
+        return room.raw[:length]
+
+    def restore(self, snapshot):
+        self._status(library().nhost_batch_restore(self.handle, bytes(snapshot), len(snapshot)))
+
+    def save_state(self, path):
+        self._status(library().nhost_batch_save_state(self.handle, str(path).encode()))
+
+    def restore_state(self, path, snapshot):
+        self._status(library().nhost_batch_restore_state(self.handle, str(path).encode(), bytes(snapshot), len(snapshot)))
 
     def step(self):
         room = (c_uint32 * (2 * self.planes))()

@@ -316,6 +316,37 @@ int32_t nhost_batch_logits(void *held, float *out) {
     return guarded([&] { return runtime::check(nh_model_logits(static_cast<Loaded *>(held)->model->handle(), out)), 0; }, -1);
 }
 
+// ---- snapshots --------------------------------------------------------------------------------------
+// BatchSnapshot::from_bytes then to_bytes: the bytes a reader that accepts them would write back (out, at most room);
+// returns their count, or -1 refused
+int64_t nhost_snapshot_round_trip(const uint8_t *bytes, size_t size, uint8_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto written = generate::BatchSnapshot::from_bytes(std::vector<uint8_t>(bytes, bytes + size)).to_bytes();
+        for (size_t i = 0; i < written.size() && i < room; i++) out[i] = written[i];
+        return (int64_t)written.size();
+    }, -1);
+}
+int64_t nhost_batch_snapshot(void *held, uint8_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto written = static_cast<Loaded *>(held)->batch->snapshot().to_bytes();
+        for (size_t i = 0; i < written.size() && i < room; i++) out[i] = written[i];
+        return (int64_t)written.size();
+    }, -1);
+}
+int32_t nhost_batch_restore(void *held, const uint8_t *bytes, size_t size) {
+    return guarded([&] {
+        return static_cast<Loaded *>(held)->batch->restore(generate::BatchSnapshot::from_bytes(std::vector<uint8_t>(bytes, bytes + size))), 0;
+    }, -1);
+}
+int32_t nhost_batch_save_state(void *held, const char *path) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->save_state(path), 0; }, -1);
+}
+int32_t nhost_batch_restore_state(void *held, const char *path, const uint8_t *bytes, size_t size) {
+    return guarded([&] {
+        return static_cast<Loaded *>(held)->batch->restore_state(path, generate::BatchSnapshot::from_bytes(std::vector<uint8_t>(bytes, bytes + size))), 0;
+    }, -1);
+}
+
 // ---- tokenizer ------------------------------------------------------------------------------------
 // the byte level bpe of a gguf under a split rule: "qwen", or the rules of the reference's own tests
 void *nhost_tokenizer_open(void *held, const char *rule) {

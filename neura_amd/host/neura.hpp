@@ -932,6 +932,139 @@ class Model {
     nh_model *model_ = nullptr;
 };
 
+// crates/neura-generate/src/snapshot.rs: what a batch holds between steps on the host -- planes, cursors, phases,
+// seeds and draw settings -- and its wire format "NBS1": little-endian words, counted lists, floats by their bits.
+struct SlotSnapshot {
+    uint32_t cursor;
+    uint32_t phase;  // 1 prompting (prompt tokens follow), 2 generating (the token to feed follows), 3 suspended
+    std::vector<uint32_t> prompt;
+    uint32_t feed;
+};
+
+struct BatchSnapshot {
+    uint32_t batch = 0, context = 0, window = 0;
+    bool sampled = false;
+    std::optional<std::vector<uint32_t>> prefix;
+    std::vector<std::optional<SlotSnapshot>> slots;
+    std::vector<uint32_t> seeds;
+    std::vector<float> temperatures, keeps, cumulatives;
+    std::vector<std::string> state_names;
+    std::vector<std::vector<float>> states;
+
+    std::vector<uint8_t> to_bytes() const {  // snapshot.rs:47-130
+        std::vector<uint8_t> bytes{'N', 'B', 'S', '1'};
+        auto word = [&](uint32_t value) {
+            for (int k = 0; k < 4; k++) bytes.push_back((uint8_t)(value >> (8 * k)));
+        };
+        auto words = [&](const std::vector<uint32_t> &values) {
+            word((uint32_t)values.size());
+            for (uint32_t value : values) word(value);
+        };
+        auto floats = [&](const std::vector<float> &values) {
+            word((uint32_t)values.size());
+            for (float value : values) {
+                uint32_t bits;
+                memcpy(&bits, &value, 4);
+                word(bits);
+            }
+        };
+        word(batch), word(context), word(window), word(sampled ? 1 : 0);
+        if (prefix) word(1), words(*prefix);
+        else word(0);
+        word((uint32_t)slots.size());
+        for (const auto &slot : slots) {
+            if (!slot) {
+                word(0);
+                continue;
+            }
+            word(slot->phase), word(slot->cursor);
+            if (slot->phase == 1) words(slot->prompt);
+            else if (slot->phase == 2) word(slot->feed);
+        }
+        words(seeds);
+        floats(temperatures), floats(keeps), floats(cumulatives);
+        word((uint32_t)state_names.size());
+        for (const std::string &name : state_names) {
+            word((uint32_t)name.size());
+            bytes.insert(bytes.end(), name.begin(), name.end());
+        }
+        word((uint32_t)states.size());
+        for (const auto &values : states) floats(values);
+        return bytes;
+    }
+
+    static BatchSnapshot from_bytes(const std::vector<uint8_t> &bytes) {  // snapshot.rs:132-236
+        size_t at = 0;
+        auto take = [&](size_t count) {
+            NEURA_ASSERT(count <= bytes.size() - at, "a snapshot holds %zu bytes where its reader asks for %zu", bytes.size(), at + count);
+            const uint8_t *held = bytes.data() + at;
+            at += count;
+            return held;
+        };
+        auto word = [&]() {
+            const uint8_t *held = take(4);
+            return (uint32_t)held[0] | ((uint32_t)held[1] << 8) | ((uint32_t)held[2] << 16) | ((uint32_t)held[3] << 24);
+        };
+        auto count = [&]() {
+            const uint32_t held = word();
+            NEURA_ASSERT(held <= bytes.size(), "a snapshot counts %u values in %zu bytes", held, bytes.size());
+            return held;
+        };
+        auto words = [&]() {
+            std::vector<uint32_t> out(count());
+            for (uint32_t &value : out) value = word();
+            return out;
+        };
+        auto floats = [&]() {
+            std::vector<float> out(count());
+            for (float &value : out) {
+                const uint32_t bits = word();
+                memcpy(&value, &bits, 4);
+            }
+            return out;
+        };
+        NEURA_ASSERT(bytes.size() >= 4 && memcmp(take(4), "NBS1", 4) == 0, "a batch snapshot opens with the four bytes NBS1");
+        BatchSnapshot out;
+        out.batch = word(), out.context = word(), out.window = word();
+        const uint32_t sampled = word();
+        NEURA_ASSERT(sampled <= 1, "a batch snapshot samples by %u", sampled);
+        out.sampled = sampled == 1;
+        if (word() != 0) out.prefix = words();
+        const uint32_t planes = count();
+        NEURA_ASSERT(planes == out.batch, "a snapshot of %u planes names %u slots", out.batch, planes);
+        for (uint32_t plane = 0; plane < planes; plane++) {
+            const uint32_t tag = word();
+            if (tag == 0) {
+                out.slots.push_back(std::nullopt);
+                continue;
+            }
+            SlotSnapshot slot{word(), tag, {}, 0};
+            if (tag == 1) slot.prompt = words();
+            else if (tag == 2) slot.feed = word();
+            else NEURA_ASSERT(tag == 3, "a slot snapshot holds phase %u", tag);
+            out.slots.push_back(slot);
+        }
+        out.seeds = words();
+        out.temperatures = floats(), out.keeps = floats(), out.cumulatives = floats();
+        const uint32_t names = count();
+        for (uint32_t i = 0; i < names; i++) {
+            const uint32_t length = word();
+            const uint8_t *held = take(length);
+            out.state_names.emplace_back(reinterpret_cast<const char *>(held), length);
+        }
+        const uint32_t held = count();
+        NEURA_ASSERT(held == names, "a snapshot names %u states and holds %u of them", names, held);
+        for (uint32_t i = 0; i < held; i++) out.states.push_back(floats());
+        NEURA_ASSERT(at == bytes.size(), "a snapshot holds %zu bytes where its reader stops at %zu", bytes.size(), at);
+        NEURA_ASSERT(out.seeds.size() == out.batch, "a snapshot of %u planes carries %zu seeds", out.batch, out.seeds.size());
+        for (const auto *values : {&out.temperatures, &out.keeps, &out.cumulatives})
+            NEURA_ASSERT(values->size() == out.batch, "a snapshot of %u planes carries %zu values", out.batch, values->size());
+        for (const auto &values : out.states)
+            NEURA_ASSERT(values.size() == out.batch, "a state of %u planes carries %zu values", out.batch, values.size());
+        return out;
+    }
+};
+
 // The generation state machine (crates/neura-generate/src/batch.rs:279-465, :1000-1172,
 // :1401-1517, :1595-1725): admit / restart / resume / suspend / finish / step with chunked
 // prompt fill; greedy, or sampled with per-plane seeds, temperatures, candidate counts and nuclei
@@ -1073,6 +1206,133 @@ class Batch {
         return held ? std::optional<uint32_t>(context_ - *held) : std::nullopt;
     }
 
+    // ---- what a batch holds between steps (crates/neura-generate/src/batch.rs:484-628) ----------------------------
+    BatchSnapshot snapshot() const {
+        BatchSnapshot out;
+        out.batch = batch_, out.context = context_, out.window = context_, out.sampled = seeded_;
+        for (const auto &slot : slots_) {
+            if (!slot) {
+                out.slots.push_back(std::nullopt);
+                continue;
+            }
+            out.slots.push_back(SlotSnapshot{slot->cursor, slot->phase == Prompting ? 1u : slot->phase == Generating ? 2u : 3u,
+                                             std::vector<uint32_t>(slot->prompt.begin(), slot->prompt.end()), slot->feed});
+        }
+        out.seeds = seeds_, out.temperatures = temperatures_, out.cumulatives = cumulatives_;
+        for (uint32_t keep : keeps_) out.keeps.push_back((float)keep);
+        return out;
+    }
+    void restore(const BatchSnapshot &snapshot) {
+        NEURA_ASSERT(snapshot.batch == batch_, "a batch of %u planes restores a snapshot of %u planes", batch_, snapshot.batch);
+        NEURA_ASSERT(snapshot.context == context_, "a batch of %u tokens of context restores a snapshot of %u", context_, snapshot.context);
+        NEURA_ASSERT(snapshot.window == context_, "a batch of a %u token window restores a snapshot of a %u token window", context_, snapshot.window);
+        NEURA_ASSERT(snapshot.sampled == seeded_, "a batch draws %s restores a snapshot of a batch that draws %s", seeded_ ? "true" : "false",
+                     snapshot.sampled ? "true" : "false");
+        NEURA_ASSERT(snapshot.slots.size() == batch_, "a snapshot of %u planes holds %zu slots", batch_, snapshot.slots.size());
+        NEURA_ASSERT(!snapshot.prefix, "a snapshot holds a shared prefix where this batch declares none");
+        NEURA_ASSERT(snapshot.state_names.empty(), "a snapshot names %zu states where this batch registers 0", snapshot.state_names.size());
+        NEURA_ASSERT(snapshot.states.size() == snapshot.state_names.size(), "a snapshot names %zu states and holds %zu of them",
+                     snapshot.state_names.size(), snapshot.states.size());
+        NEURA_ASSERT(snapshot.seeds.size() == batch_, "a batch of %u planes restores %zu seeds", batch_, snapshot.seeds.size());
+        NEURA_ASSERT(snapshot.temperatures.size() == batch_, "a batch of %u planes restores %zu temperatures", batch_, snapshot.temperatures.size());
+        NEURA_ASSERT(snapshot.keeps.size() == batch_, "a batch of %u planes restores %zu keeps", batch_, snapshot.keeps.size());
+        NEURA_ASSERT(snapshot.cumulatives.size() == batch_, "a batch of %u planes restores %zu cumulatives", batch_, snapshot.cumulatives.size());
+        for (uint32_t slot = 0; slot < batch_; slot++) {
+            const auto &held = snapshot.slots[slot];
+            if (!held) {
+                slots_[slot].reset();
+                continue;
+            }
+            slots_[slot] = Slot{held->cursor, held->phase == 1 ? Prompting : held->phase == 2 ? Generating : Suspended,
+                                std::deque<uint32_t>(held->prompt.begin(), held->prompt.end()), held->feed};
+        }
+        seeds_ = snapshot.seeds, temperatures_ = snapshot.temperatures, cumulatives_ = snapshot.cumulatives;
+        for (uint32_t slot = 0; slot < batch_; slot++) keeps_[slot] = (uint32_t)snapshot.keeps[slot];
+    }
+    // The device side of a batch between steps: the key and value states of every layer, written as the container the
+    // reference's Runtime::save_state writes (crates/neura-runtime/src/checkpoint/container.rs:129-246: an 8-byte
+    // length, a JSON header padded with blanks to a multiple of 8, then the tensors back to back in header order --
+    // the layout of a safetensors file).  States are named as the decoder's caches name them (blk.N.cache.key / .value,
+    // crates/neura-decoder/src/cache.rs:136-137) and shaped [key heads, planes, capacity, width] in half storage.
+    void save_state(const std::string &path) const {
+        const Config &c = model_.config();
+        const uint32_t capacity = nh_model_capacity(model_.handle());
+        const size_t elements = (size_t)c.key_heads * batch_ * capacity * c.head_width;
+        std::vector<std::string> names;
+        for (uint32_t layer = 0; layer < c.layers; layer++)
+            for (const char *which : {"key", "value"}) names.push_back("blk." + std::to_string(layer) + ".cache." + which);
+        std::sort(names.begin(), names.end());  // one storage width: the header orders by name
+        std::string header = "{";
+        size_t at = 0;
+        for (size_t i = 0; i < names.size(); i++) {
+            if (i) header += ',';
+            header += '"' + names[i] + "\":{\"dtype\":\"F16\",\"shape\":[" + std::to_string(c.key_heads) + ',' + std::to_string(batch_) + ',' +
+                      std::to_string(capacity) + ',' + std::to_string(c.head_width) + "],\"data_offsets\":[" + std::to_string(at) + ',';
+            at += elements * 2;
+            header += std::to_string(at) + "]}";
+        }
+        header += '}';
+        header.resize((header.size() + 7) / 8 * 8, ' ');
+        std::ofstream out(path, std::ios::binary);
+        if (!out) panic("a container at %s could not be created", path.c_str());
+        const uint64_t length = header.size();
+        for (int k = 0; k < 8; k++) out.put((char)(length >> (8 * k)));
+        out.write(header.data(), (std::streamsize)header.size());
+        std::vector<uint16_t> held(elements);
+        for (const std::string &name : names) {
+            uint32_t layer;
+            bool value;
+            parse_state_name(name, layer, value);
+            runtime::check(nh_model_cache_read(model_.handle(), layer, value ? 1 : 0, held.data()));
+            out.write(reinterpret_cast<const char *>(held.data()), (std::streamsize)(elements * 2));
+        }
+        out.flush();
+        if (!out) panic("a container at %s could not be written", path.c_str());
+    }
+    // Batch::restore_state (batch.rs:519-532): the device states out of a container, then the host bookkeeping
+    void restore_state(const std::string &path, const BatchSnapshot &snapshot) {
+        const Config &c = model_.config();
+        const uint32_t capacity = nh_model_capacity(model_.handle());
+        const size_t elements = (size_t)c.key_heads * batch_ * capacity * c.head_width;
+        std::ifstream in(path, std::ios::binary);
+        if (!in) panic("a container at %s could not be opened", path.c_str());
+        uint8_t framed[8];
+        in.read(reinterpret_cast<char *>(framed), 8);
+        NEURA_ASSERT(in.gcount() == 8, "a container at %s holds no header length", path.c_str());
+        uint64_t length = 0;
+        for (int k = 0; k < 8; k++) length |= (uint64_t)framed[k] << (8 * k);
+        NEURA_ASSERT(length > 0 && length < (1ull << 26), "a container at %s frames a header of %llu bytes", path.c_str(), (unsigned long long)length);
+        std::string header(length, ' ');
+        in.read(header.data(), (std::streamsize)length);
+        NEURA_ASSERT((uint64_t)in.gcount() == length, "a container at %s ends inside its header", path.c_str());
+        const std::string shape = "[" + std::to_string(c.key_heads) + ',' + std::to_string(batch_) + ',' + std::to_string(capacity) + ',' +
+                                  std::to_string(c.head_width) + "]";
+        std::vector<uint16_t> held(elements);
+        for (uint32_t layer = 0; layer < c.layers; layer++)
+            for (int value = 0; value < 2; value++) {
+                const std::string name = "blk." + std::to_string(layer) + ".cache." + (value ? "value" : "key");
+                const size_t found = header.find('"' + name + "\":{");
+                NEURA_ASSERT(found != std::string::npos, "the container at %s holds no state named %s", path.c_str(), name.c_str());
+                const size_t close = header.find('}', found);
+                const std::string entry = compact(header.substr(found, close - found));
+                NEURA_ASSERT(entry.find("\"dtype\":\"F16\"") != std::string::npos, "state %s of the container at %s is not in half storage", name.c_str(),
+                             path.c_str());
+                NEURA_ASSERT(entry.find("\"shape\":" + shape) != std::string::npos, "state %s of the container at %s is not shaped %s", name.c_str(),
+                             path.c_str(), shape.c_str());
+                const size_t offsets = entry.find("\"data_offsets\":[");
+                NEURA_ASSERT(offsets != std::string::npos, "state %s of the container at %s names no bytes", name.c_str(), path.c_str());
+                const uint64_t begin = std::stoull(entry.substr(offsets + 16));
+                const uint64_t end = std::stoull(entry.substr(entry.find(',', offsets + 16) + 1));
+                NEURA_ASSERT(end - begin == elements * 2, "state %s of the container at %s holds %llu bytes where the cache holds %zu", name.c_str(),
+                             path.c_str(), (unsigned long long)(end - begin), elements * 2);
+                in.seekg((std::streamoff)(8 + length + begin));
+                in.read(reinterpret_cast<char *>(held.data()), (std::streamsize)(elements * 2));
+                NEURA_ASSERT((size_t)in.gcount() == elements * 2, "the container at %s ends inside state %s", path.c_str(), name.c_str());
+                runtime::check(nh_model_cache_write(model_.handle(), layer, value, held.data()));
+            }
+        restore(snapshot);
+    }
+
     std::vector<Emitted> step() {  // batch.rs:1125-1135
         if (active().empty()) return {};
         prefill();
@@ -1169,6 +1429,16 @@ class Batch {
     }
 
     void plane(uint32_t slot) const { NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot); }
+    static void parse_state_name(const std::string &name, uint32_t &layer, bool &value) {  // blk.N.cache.key / blk.N.cache.value
+        layer = (uint32_t)std::stoul(name.substr(4));
+        value = name.size() >= 6 && name.compare(name.size() - 6, 6, ".value") == 0;
+    }
+    static std::string compact(const std::string &text) {  // a header entry without the blanks a writer may have put between its parts
+        std::string out;
+        for (char held : text)
+            if (held != ' ' && held != '\n' && held != '\t') out.push_back(held);
+        return out;
+    }
     static void check_keep(uint32_t keep) {
         NEURA_ASSERT(keep >= 1 && keep <= Sampling::CANDIDATES, "a batch keeps %u candidates where a row holds between one and %u", keep,
                      Sampling::CANDIDATES);

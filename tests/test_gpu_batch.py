@@ -201,6 +201,61 @@ def test_a_temperature_and_a_candidate_count_the_host_writes_steer_the_draws(run
     archive.close()
 
 
+@pytest.mark.parametrize("sampling", [None, (0.9, 40, 0.95)], ids=["greedy", "sampled"])
+def test_a_batch_restored_from_its_snapshot_and_state_file_answers_on(runtime, tmp_path, sampling):
+    """Batch::snapshot + save_state, then restore_state into another batch (crates/neura-generate/src/batch.rs:484-628):
+    the second batch goes on with the tokens the first would have answered with.  The state file is a container any
+    safetensors reader opens; its tensors are the caches as the C ABI reads them."""
+    from safetensors.numpy import load_file
+
+    shape, element = SHAPE, NH_Q8_0
+    qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=51)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    first = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [8], sampling=sampling)
+    if sampling:
+        first.set_seed(77)
+        first.set_temperature(1.3, slot=2)
+    rng = np.random.default_rng(52)
+    prompts = [list(rng.integers(0, shape["vocab"], n)) for n in (4, 30)]
+    for prompt in prompts:
+        first.admit(prompt)
+    for _ in range(9):   # plane 0 answers already, plane 1 still feeds its prompt, plane 2 is empty
+        first.step()
+    first.suspend(0)
+    snapshot = first.snapshot()
+    assert snapshot[:4] == b"NBS1" and host.snapshot_round_trip(snapshot) == snapshot
+    first.save_state(tmp_path / "state.safetensors")
+    held = load_file(str(tmp_path / "state.safetensors"))
+    capacity = CONTEXT + 8
+    assert sorted(held) == sorted("blk.%d.cache.%s" % (layer, which) for layer in range(shape["layers"]) for which in ("key", "value"))
+    assert all(tensor.dtype == np.float16 and tensor.shape == (shape["kv_heads"], 3, capacity, shape["head_dim"]) for tensor in held.values())
+    assert np.abs(held["blk.1.cache.key"][:, 1, :20].astype(np.float32)).max() > 0  # plane 1 has written twenty-odd keys
+    assert not held["blk.1.cache.key"][:, 2].any()                                    # plane 2 none
+
+    second = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [8], sampling=sampling)
+    second.restore_state(tmp_path / "state.safetensors", snapshot)
+    assert second.active() == [1] and second.occupied() == [0, 1]
+    assert [second.cursor(slot) for slot in range(3)] == [first.cursor(slot) for slot in range(3)]
+    if sampling:
+        assert [second.seed_of(slot) for slot in range(3)] == [first.seed_of(slot) for slot in range(3)]
+    for batch in (first, second):
+        batch.resume(0, [3, 1, 4])
+    want = run(first, {0: 10, 1: 10})
+    assert run(second, {0: 10, 1: 10}) == want
+    # a batch of another shape refuses the snapshot, and a file that misses a state is refused
+    other = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], sampling=sampling)
+    with pytest.raises(host.Panic, match="a batch of 2 planes restores a snapshot of 3 planes"):
+        other.restore(snapshot)
+    if sampling is None:
+        drawing = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [8], sampling=(1.0, 4, 1.0))
+        with pytest.raises(host.Panic, match="a batch draws true restores a snapshot of a batch that draws false"):
+            drawing.restore(snapshot)
+        drawing.close()
+    for batch in (first, second, other):
+        batch.close()
+    archive.close()
+
+
 def test_a_batch_keeps_the_planes_it_is_told_to(runtime, tmp_path):
     shape, element = SHAPE, NH_Q8_0
     tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=21)

@@ -232,3 +232,37 @@ def test_plane_seeds_and_the_bits_a_batch_writes():
         for slot in (0, 1, 7):
             assert host.plane_seed(seed, slot) == oracle.lib().oracle_plane_seed(seed, slot)
         assert host.seed_bits(seed) == oracle.lib().oracle_seed_bits(seed) == 0x3F800000 | ((seed ^ (seed >> 23)) & 0x7FFFFF)
+
+
+def test_a_batch_snapshot_reads_and_writes_the_nbs1_wire_format():
+    # crates/neura-generate/src/snapshot.rs:47-236, the bytes laid out here by hand: little-endian words, counted lists
+    import struct
+
+    def words(*values):
+        return struct.pack("<%dI" % len(values), *values)
+
+    def floats(*values):
+        return struct.pack("<I", len(values)) + struct.pack("<%df" % len(values), *values)
+
+    raw = (b"NBS1" + words(3, 96, 96) + words(1)            # batch, context, window; sampled
+           + words(0)                                        # no shared prefix
+           + words(3)                                        # three slots
+           + words(1, 7) + words(2, 41, 42)                  # prompting at cursor 7 with two tokens left
+           + words(0)                                        # an empty plane
+           + words(2, 19, 555)                               # generating at cursor 19, feeding token 555
+           + words(3, 11, 22, 33)                            # seeds
+           + floats(0.5, 1.0, 1.5) + floats(40.0, 1.0, 64.0) + floats(0.9, 1.0, 0.25)
+           + words(1) + words(4) + b"gate"                   # one named state ...
+           + words(1) + floats(0.0, 1.0, 0.0))               # ... of a value a plane
+    assert host.snapshot_round_trip(raw) == raw
+    suspended = raw.replace(words(2, 19, 555), words(3, 19))
+    assert host.snapshot_round_trip(suspended) == suspended
+    prefixed = raw.replace(b"NBS1" + words(3, 96, 96) + words(1) + words(0), b"NBS1" + words(3, 96, 96) + words(1) + words(1) + words(2, 5, 6))
+    assert host.snapshot_round_trip(prefixed) == prefixed
+    refuses(lambda: host.snapshot_round_trip(b"NBS2" + raw[4:]), "a batch snapshot opens with the four bytes NBS1")
+    refuses(lambda: host.snapshot_round_trip(raw[:-2]), "bytes where its reader asks for")
+    refuses(lambda: host.snapshot_round_trip(raw + b"\0\0\0\0"), "bytes where its reader stops at")
+    refuses(lambda: host.snapshot_round_trip(raw.replace(words(3, 96, 96) + words(1), words(3, 96, 96) + words(2))), "a batch snapshot samples by 2")
+    refuses(lambda: host.snapshot_round_trip(raw.replace(words(3, 96, 96), words(2, 96, 96))), "a snapshot of 2 planes names 3 slots")
+    refuses(lambda: host.snapshot_round_trip(raw.replace(words(2, 19, 555), words(4, 19, 555))), "a slot snapshot holds phase 4")
+    refuses(lambda: host.snapshot_round_trip(raw.replace(words(3, 11, 22, 33), words(2, 11, 22))), "a snapshot of 3 planes carries 2 seeds")
