@@ -139,7 +139,24 @@ def extras(device, weights, shape, element, context, layers, rng):
     batch 8 (eight sequences at the end of their context) and a 512-token prompt fill."""
     from neura_amd.loader import Model
 
+    import neura_amd
+
     out = {}
+    # batch 1 again with a sampled choice (temperature 0.8, 40 candidates, nucleus 0.95; the seed one further a step)
+    model = Model(device, weights, shape, element, batch=1, context=context, layers=layers)
+    steps, warm = 32, 4
+    first, token = context - (steps + warm), 1
+    for step in range(warm + steps):
+        if step == warm:
+            device.sync()
+            began = time.perf_counter()
+        draws = np.array([(0x3F800000 | (step & 0x7FFFFF), 0.8, 40, 0.95)], dtype=neura_amd.DRAW)
+        token = int(model.decode_step_sampled([token], [first + step], draws)[0])
+    device.sync()
+    elapsed = time.perf_counter() - began
+    out["decode_sampled_batch1"] = {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
+                                    "note": "as the headline step with the greedy choice replaced by the sampled one; caches not pre-filled (zeros)"}
+    model.release()
     batch = 8
     model = Model(device, weights, shape, element, batch=batch, context=context, layers=layers)
     steps, warm = 16, 4
