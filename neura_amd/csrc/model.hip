@@ -35,6 +35,7 @@ struct nh_model {
     // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked, [2], [3] the same with a sampled choice
     hipGraphExec_t decode_graph[4] = {nullptr, nullptr, nullptr, nullptr};
     uint64_t graph_moved[4] = {0, 0, 0, 0};  // nh_device::moved when each graph was recorded
+    bool graph_warmed[4] = {false, false, false, false};  // the variant has run once outside a capture
     bool use_graph = true;
 };
 
@@ -389,7 +390,9 @@ static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *
     // Profiled steps run eagerly (event records do not belong in a graph).
     const int variant = (any_inactive ? 1 : 0) + (draws ? 2 : 0);
     hipGraphExec_t &graph = m->decode_graph[variant];
-    if (m->use_graph && !d->profile) {
+    // The first step of a variant runs eagerly: its launchers grow the device scratch to what the variant needs (a
+    // synchronize, a free and an allocation), none of which belongs inside a stream capture.
+    if (m->use_graph && !d->profile && m->graph_warmed[variant]) {
         if (graph && m->graph_moved[variant] != d->moved) {
             // the device scratch or rope table moved since the capture (another model or operator call grew it)
             (void)hipGraphExecDestroy(graph);
@@ -414,8 +417,9 @@ static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *
             }
         }
         NH_HIP(hipGraphLaunch(graph, d->stream));
-    } else if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) {
-        return status;
+    } else {
+        if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) return status;
+        m->graph_warmed[variant] = true;
     }
     NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
     NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
