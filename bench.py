@@ -201,6 +201,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--workload", default="qwen2.5-7b-q4k")
     parser.add_argument("--layers", type=int, default=None, help="cut the decoder (for quick checks; the result is then not the headline)")
+    parser.add_argument("--sampled", action="store_true",
+                        help="draw every token (temperature 0.8, 40 candidates, nucleus 0.95) instead of taking the largest logit; not the headline")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode, 512-token fill and wide-product measurements")
     parser.add_argument("--gemm-only", action="store_true", help="run only the wide product of BASELINE config 3 and print its line")
@@ -243,12 +245,19 @@ def main():
     first_cursor = context - total  # the last timed step sits at cursor context - 1
     assert first_cursor >= 0, "more steps than the context holds"
     token = 1
+
+    def one_step(token, step):
+        if args.sampled:
+            draws = np.array([(0x3F800000 | (step & 0x7FFFFF), 0.8, 40, 0.95)], dtype=neura_amd.DRAW)
+            return int(model.decode_step_sampled([token], [first_cursor + step], draws)[0])
+        return int(model.decode_step([token], [first_cursor + step])[0])
+
     for step in range(args.warmup):
-        token = int(model.decode_step([token], [first_cursor + step])[0])
+        token = one_step(token, step)
     device.sync()
     began = time.perf_counter()
     for step in range(args.steps):
-        token = int(model.decode_step([token], [first_cursor + args.warmup + step])[0])
+        token = one_step(token, args.warmup + step)
     device.sync()
     elapsed = time.perf_counter() - began
 
@@ -274,8 +283,9 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "%s decode, batch 1, %d layers, fp16 KV cache at context %d, random-init %s weights" %
-                        (args.workload, layers, context, ("Q4_K" if element == 12 else "Q8_0") + (" and Q6_K" if mixed else "")),
+            "workload": "%s decode, batch 1, %d layers, fp16 KV cache at context %d, random-init %s weights%s" %
+                        (args.workload, layers, context, ("Q4_K" if element == 12 else "Q8_0") + (" and Q6_K" if mixed else ""),
+                         ", sampled choice" if args.sampled else ""),
             "weight_bytes_per_token": weight_bytes_per_token(shape, element, layers, mixed),
         },
         "roofline": {
