@@ -178,6 +178,9 @@ int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv
                            uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
                            const uint8_t *mask, float base);
 
+// one token of one plane: v (+ bias) as halves into the value state at cursor[0]
+int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
+                            const uint32_t *cursor);
 int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n);
 
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,

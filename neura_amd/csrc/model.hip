@@ -140,8 +140,27 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];
                 roped = true;
             }
+            // the same with a value projection stored otherwise (a Q4_K_M file keeps some in Q6_K): q|k go out rotated from
+            // one product, the value row follows from its own product through a small append
+            GemvArgs qk = narrow(m, element_at(m, L, Q), m->attn_q[L], QW + KW, H, m->h, T, m->qkv);
+            qk.W[1] = m->attn_k[L];
+            qk.end[0] = QW, qk.end[1] = QW + KW, qk.end[2] = QW + KW;
+            qk.norm_w = m->attn_norm[L], qk.eps = c.eps;
+            RopeFusion rope_qk{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
+            const bool split_value = !alike && element_at(m, L, Q) == element_at(m, L, K_) && !products_only && T == 1 && !mask &&
+                                     gemv_fuses_rope(qk, rope_qk);
             if (roped || (alike && (!biased || products_only))) {
                 if ((status = launch_gemv(d, a)) != NH_OK) return status;
+            } else if (split_value) {
+                qk.rope = &rope_qk;
+                qk.bias[0] = m->bias_q[L], qk.bias[1] = m->bias_k[L];
+                if ((status = launch_gemv(d, qk)) != NH_OK) return status;
+                GemvArgs value = narrow(m, element_at(m, L, V), m->attn_v[L], KW, H, m->h, T, m->xn);
+                value.norm_w = m->attn_norm[L], value.eps = c.eps;
+                if ((status = launch_gemv(d, value)) != NH_OK) return status;
+                if ((status = launch_value_append(d, m->xn, m->bias_v[L], m->cache_v[L], c.kv_heads, hd, m->capacity, dev_cursor(m))) != NH_OK)
+                    return status;
+                roped = true;
             } else {
                 // matrices of different elements, or biases outside the folded rotation: one product each, placed side by side
                 const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};

@@ -121,6 +121,33 @@ int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_
     return NH_OK;
 }
 
+// one token of one plane: value + bias cast to fp16 into the value state at the cursor (what cache_write_kernel does for
+// a value row whose key went out with the product that rotated it)
+__global__ __launch_bounds__(256) void value_append_kernel(const float *__restrict__ v, const float *__restrict__ bias, uint16_t *__restrict__ cache_v,
+                                                           uint32_t kv_heads, uint32_t width, uint32_t capacity, const uint32_t *__restrict__ cursor,
+                                                           uint32_t *refusal) {
+    const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= kv_heads * width) return;
+    const uint32_t slot = cursor[0];
+    if (slot >= capacity) {
+        atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
+        return;
+    }
+    const uint32_t head = index / width, c = index % width;
+    const float value = bias ? v[index] + bias[index] : v[index];
+    cache_v[((uint64_t)head * capacity + slot) * width + c] = float_to_half(value);
+}
+
+int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
+                            const uint32_t *cursor) {
+    const uint32_t total = kv_heads * width;
+    if (!total) return NH_OK;
+    hipLaunchKernelGGL(value_append_kernel, dim3((total + 255) / 256), dim3(256), 0, d->stream, v, bias, cache_v, kv_heads, width, capacity, cursor,
+                       d->refusal);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
 __global__ __launch_bounds__(256) void rope_angles_kernel(const float *__restrict__ table, uint32_t half, uint32_t positions,
                                                           float *__restrict__ cosines, float *__restrict__ sines) {
     const uint64_t total = (uint64_t)positions * half;
