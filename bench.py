@@ -106,7 +106,7 @@ def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=2
 
 
 def gemm_config3(device, rng, repeats=10):
-    """BASELINE config 3: the Q4_K wide product M=512, K=3584, N=18944 (the 7B-shape FFN up projection), with half
+    """The wide-product configuration of the benchmark: the Q4_K product M=512, K=3584, N=18944 (the 7B-shape FFN up projection), with half
     activations as the configuration states them and with fp32 activations as the decoder's fill passes them."""
     import ctypes
 
@@ -205,7 +205,7 @@ def main():
                         help="draw every token (temperature 0.8, 40 candidates, nucleus 0.95) instead of taking the largest logit; not the headline")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode, 512-token fill and wide-product measurements")
-    parser.add_argument("--gemm-only", action="store_true", help="run only the wide product of BASELINE config 3 and print its line")
+    parser.add_argument("--gemm-only", action="store_true", help="run only the wide product (M=512, K=3584, N=18944) and print its line")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()

@@ -354,8 +354,8 @@ def test_cache_write_casts_and_scatters(device):
 
 @pytest.mark.parametrize("heads,kv_heads,batch,rows,keys,width,origins", [
     (4, 2, 2, 3, 12, 32, [9, 4]),
-    (14, 2, 1, 1, 1100, 64, [1024]),       # config 4 decode shape
-    (28, 4, 1, 1, 4200, 128, [4095]),      # config 5 decode shape
+    (14, 2, 1, 1, 1100, 64, [1024]),       # the 0.5B decode shape at context 1024
+    (28, 4, 1, 1, 4200, 128, [4095]),      # the 7B decode shape at context 4096
     (28, 4, 8, 1, 600, 128, [0, 1, 63, 64, 65, 300, 511, 599]),
     (12, 2, 1, 17, 300, 128, [200]),       # a fill chunk
     (8, 8, 2, 5, 40, 256, [35, 0]),
