@@ -295,6 +295,175 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, 
     }
 }
 
+
+// ---------------------------------------------------------------- several query rows: the matrix cores --------
+//
+// A chunk of query rows (a fill) against the same cache, on v_mfma_f32_32x32x16_f16.  One workgroup serves one
+// (kv head, plane) and a block of query rows; each of its four waves owns 32 "columns" -- RPW = 32 / groups query
+// rows times the query heads of the group -- and all four share the key and value tiles of 32 keys the workgroup
+// stages in LDS.  Per tile and wave:
+//   scores  S^T[key][column] = K[key][:] . q[column][:]: the key rows are the A operand as they lie (a lane reads 8
+//           halves of its key), the queries the B operand, held in registers as two half planes (value and residue, so
+//           fp32 queries lose nothing).  C hands lane (column, half) sixteen of the tile's 32 keys: a column's maximum
+//           and sum never leave its two lanes.
+//   values  O^T[channel][column] += V^T[channel][key] . P^T[key][column]: the weights go back in as the B operand
+//           straight from the registers C left them in (again as value and residue planes), and the value tile, which
+//           the workgroup wrote to LDS transposed, is the A operand in that same key order.
+// The running maximum, sum and the 32 x 64 accumulators of a column live in its two lanes; nothing is folded afterwards.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int WIDTH>
+__global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, uint32_t rows_per_wave) {
+    constexpr int TK = 32;                       // keys per tile
+    constexpr int STEPS = WIDTH / 16;            // MFMA steps over the channels of a score
+    constexpr int BLOCKS = WIDTH / 32;           // 32-channel blocks of the output
+    constexpr int KPITCH = WIDTH + 8;            // halves per staged key row (the pad spreads the banks)
+    constexpr int VPITCH = TK + 4;               // halves per staged value channel
+    __shared__ __attribute__((aligned(16))) uint16_t kt[TK][KPITCH];
+    __shared__ __attribute__((aligned(16))) uint16_t vt[WIDTH][VPITCH];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t n = lane & 31u, h = lane >> 5;
+    const uint32_t G = p.groups;
+    const uint32_t b = blockIdx.x % p.batch, kvh = blockIdx.x / p.batch;
+    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
+
+    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
+    if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        origin = p.keys - p.rows;
+    }
+    // this lane's column: a query row and a query head of the group
+    const uint32_t block_row = blockIdx.y * 4u * rows_per_wave;
+    const uint32_t row = block_row + wave * rows_per_wave + n / G, g = n % G;
+    const bool held = n < rows_per_wave * G && row < p.rows;
+    const uint32_t limit = origin + min(row, p.rows - 1u);  // the last key this column sees
+    // the workgroup walks up to the last key its last row sees
+    const uint32_t last_row = min(p.rows, block_row + 4u * rows_per_wave) - 1u;
+    const uint32_t span = min(p.keys, origin + last_row + 1u);
+    const uint32_t wave_first = block_row + wave * rows_per_wave;
+    const uint32_t wave_span = wave_first < p.rows ? min(p.keys, origin + min(p.rows, wave_first + rows_per_wave)) : 0u;
+
+    // queries as two half planes: q = value + residue, both halves
+    half8_t q_value[STEPS], q_residue[STEPS];
+    {
+        const float *src = p.q + (uint64_t)(kvh * G + g) * p.q_sh + (uint64_t)b * p.q_sb + (uint64_t)min(row, p.rows - 1u) * p.q_sr;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float value = held ? src[16 * s + 8 * h + i] : 0.0f;
+                const _Float16 high = (_Float16)value;
+                q_value[s][i] = high;
+                q_residue[s][i] = (_Float16)((value - (float)high) * 2048.0f);  // scaled up, clear of the subnormal halves
+            }
+        }
+    }
+    f32x16 acc[BLOCKS];
+#pragma unroll
+    for (int d = 0; d < BLOCKS; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[d][r] = 0.0f;
+    float top = -INFINITY, mass = 0.0f;
+
+    // the pieces of a tile this thread stages: 16 bytes of a key row and of a value row each
+    constexpr int PIECES = TK * WIDTH / 8 / 256;  // per thread and tile
+    u32x4 kraw[PIECES], vraw[PIECES];
+    auto fetch = [&](uint32_t tile) {
+#pragma unroll
+        for (int k = 0; k < PIECES; k++) {
+            const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
+            const uint64_t at = (plane + min(tile + key, p.capacity - 1u)) * WIDTH + chunk * 8u;
+            kraw[k] = *reinterpret_cast<const u32x4 *>(p.cache_k + at);
+            vraw[k] = *reinterpret_cast<const u32x4 *>(p.cache_v + at);
+        }
+    };
+    fetch(0);
+    for (uint32_t tile = 0; tile < span; tile += TK) {
+        __syncthreads();  // the last tile's readers are done
+#pragma unroll
+        for (int k = 0; k < PIECES; k++) {
+            const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
+            *reinterpret_cast<u32x4 *>(&kt[key][chunk * 8u]) = kraw[k];
+            // rows past the written keys may hold anything, and a weight of zero does not silence a NaN
+            const uint32_t keep = tile + key < p.keys ? 0xffffffffu : 0u;
+            const uint32_t words[4] = {vraw[k].x & keep, vraw[k].y & keep, vraw[k].z & keep, vraw[k].w & keep};
+#pragma unroll
+            for (int i = 0; i < 8; i++) vt[chunk * 8u + i][key] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
+        }
+        if (tile + TK < span) fetch(tile + TK);  // in flight while this tile is multiplied
+        __syncthreads();
+        if (tile >= wave_span) continue;  // keys none of this wave's rows see (every wave still meets the barriers)
+
+        // ---- scores
+        f32x16 scores, fine;
+#pragma unroll
+        for (int r = 0; r < 16; r++) scores[r] = 0.0f, fine[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const half8_t keys = *reinterpret_cast<const half8_t *>(&kt[n][16 * s + 8 * h]);
+            scores = __builtin_amdgcn_mfma_f32_32x32x16_f16(keys, q_value[s], scores, 0, 0, 0);
+            fine = __builtin_amdgcn_mfma_f32_32x32x16_f16(keys, q_residue[s], fine, 0, 0, 0);
+        }
+        // ---- weights: register 4j + e of lane (column, h) is key 8j + 4h + e of the tile
+        float tile_top = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t key = tile + 8u * (r >> 2) + 4u * h + (r & 3);
+            const bool seen = held && key <= limit && key < p.keys;
+            scores[r] = seen ? fmaf(fine[r], 1.0f / 2048.0f, scores[r]) * p.scale : -INFINITY;
+            tile_top = fmaxf(tile_top, scores[r]);
+        }
+        tile_top = fmaxf(tile_top, __shfl_xor(tile_top, 32, 64));
+        const float next = fmaxf(top, tile_top);
+        const float rescale = top == -INFINITY ? 0.0f : softmax_exp(top - next);
+        float tile_mass = 0.0f;
+        half8_t w_value[2], w_residue[2];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float weight = scores[r] == -INFINITY ? 0.0f : softmax_exp(scores[r] - next);
+            tile_mass += weight;
+            // the weights ride 2^10 up (undone with the mass at the end): their residues stay normal halves
+            const float raised = weight * 1024.0f;
+            const _Float16 high = (_Float16)raised;
+            // key slots of the second product: step t takes registers 8t .. 8t + 7 in order
+            w_value[r >> 3][r & 7] = high;
+            w_residue[r >> 3][r & 7] = (_Float16)(raised - (float)high);
+        }
+        tile_mass += __shfl_xor(tile_mass, 32, 64);
+        mass = fmaf(mass, rescale, tile_mass);
+        top = next;
+        // ---- values
+#pragma unroll
+        for (int d = 0; d < BLOCKS; d++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[d][r] *= rescale;
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                // slots 8h + i of step t: keys 16t + 4h + i (i < 4) and 16t + 8 + 4h + (i - 4), as the weights lie
+                half8_t values;
+                const uint2 low = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][16 * t + 4 * h]);
+                const uint2 high = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][16 * t + 8 + 4 * h]);
+                const u32x4 joined = {low.x, low.y, high.x, high.y};
+                values = __builtin_bit_cast(half8_t, joined);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(values, w_value[t], acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(values, w_residue[t], acc[d], 0, 0, 0);
+            }
+        }
+    }
+    if (!held) return;
+    // register 4j + e of block d is channel 32d + 8j + 4h + e of this lane's column
+    const float normalized = mass > 0.0f ? 1.0f / (mass * 1024.0f) : 0.0f;
+    float *dst = p.out + (uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr;
+#pragma unroll
+    for (int d = 0; d < BLOCKS; d++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float4 out4 = {acc[d][4 * j] * normalized, acc[d][4 * j + 1] * normalized, acc[d][4 * j + 2] * normalized, acc[d][4 * j + 3] * normalized};
+            *reinterpret_cast<float4 *>(dst + 32 * d + 8 * j + 4 * h) = out4;
+        }
+}
+
 int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     AttentionParams p{};
     p.q = a.q, p.out = a.out;
@@ -306,6 +475,22 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
+    // a chunk of query rows goes to the matrix cores (NEURA_HIP_ATTENTION_TILE=0 keeps the row-at-a-time kernel)
+    {
+        const char *held = getenv("NEURA_HIP_ATTENTION_TILE");
+        const bool wanted = !(held && held[0] == '0');
+        const bool aligned = ((uintptr_t)a.out & 15u) == 0 && a.o_sh % 4 == 0 && a.o_sb % 4 == 0 && a.o_sr % 4 == 0 && ((uintptr_t)a.cache_k & 15u) == 0 &&
+                             ((uintptr_t)a.cache_v & 15u) == 0;
+        if (wanted && aligned && a.rows >= 4 && (a.width == 64 || a.width == 128) && p.groups >= 1) {
+            const uint32_t rows_per_wave = 32u / p.groups;
+            dim3 grid(a.kv_heads * a.batch, (a.rows + 4u * rows_per_wave - 1u) / (4u * rows_per_wave));
+            p.sections = 1;
+            if (a.width == 64) hipLaunchKernelGGL(attention_tile_kernel<64>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
+            else hipLaunchKernelGGL(attention_tile_kernel<128>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
+            NH_HIP(hipGetLastError());
+            return NH_OK;
+        }
+    }
     // sections of the context: enough workgroups to fill the chip four times over, none thinner
     // than 64 keys (thinner sections cost more in the fold than they gain in the walk)
     const char *held = getenv("NEURA_HIP_ATTENTION_KEYS");
