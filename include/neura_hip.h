@@ -134,16 +134,20 @@ int32_t nh_rope(nh_device *device, const float *dev_x, uint32_t planes, uint32_t
 /* Cache::write / write_masked (crates/neura-decoder/src/cache.rs:267-352): cast to fp16 then
  * scatter rows.  k, v are fp32 [kv_heads][batch][rows][width]; the caches are fp16
  * [kv_heads][batch][capacity][width]; row index = cursor[b] + row, or window + row for a
- * plane whose dev_mask byte is 0 (dev_mask may be NULL = all active). */
+ * plane whose dev_mask byte is 0 (dev_mask may be NULL = all active).  ring != 0 is Cache::windowed (cache.rs:67-69,
+ * :311-317; crates/neura-decoder/src/layout.rs:32-36): the window is a ring, row index = (cursor[b] + row) mod window. */
 int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v, uint16_t *dev_cache_k, uint16_t *dev_cache_v,
                        uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
-                       const uint32_t *dev_cursor, const uint8_t *dev_mask);
+                       const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring);
 /* Cache::attend -> run_attention (+ run_attention_fold) (crates/neura-decoder/src/cache.rs:366-406,
  * crates/neura-kernel/src/task/attention.rs:309-671): causal GQA attention of q
  * [heads][batch][rows][width] over fp16 caches [kv_heads][batch][capacity][width], the first
- * `keys` rows visible; key `at` is weighed iff at <= cursor[b] + row.  out like q. */
+ * `keys` rows visible; key `at` is weighed iff at <= cursor[b] + row.  out like q.
+ * reach (AttentionOptions::reach, cache.rs:391-394; key_position / weighed, attention.rs:103-108, :136-144): 0, or the
+ * span of a ring of `keys` slots -- slot `at` then holds the latest position below cursor[b] + rows that lands on it, a query
+ * weighs the `reach` positions up to its own, and a cursor past `keys` is no refusal. */
 int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
-                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach,
                      const uint32_t *dev_cursor, float scale, float *dev_out);
 /* run_gather (crates/neura-kernel/src/task/select.rs:29-49): out[t][:] = dequant(table[token[t]]),
  * times mask[t % batch] when dev_mask != NULL.  A token id >= vocab is refused. */
@@ -178,6 +182,8 @@ typedef struct nh_model_config {
     uint32_t context;    /* BatchSpec.context */
     uint32_t batch;      /* BatchSpec.batch (planes) */
     uint32_t max_rows;   /* widest fill chunk (BatchSpec.chunks[0]), 1 if none */
+    uint32_t window;     /* BatchSpec.window (crates/neura-generate/src/batch.rs:148-152): 0 = none; else the caches are rings of
+                            `window` positions (+ max_rows scratch rows) and a sequence attends to its last `window` tokens */
     float rope_base;     /* <arch>.rope.freq_base */
     float eps;           /* <arch>.attention.layer_norm_rms_epsilon */
 } nh_model_config;
@@ -201,7 +207,7 @@ typedef struct nh_tensor_table {
 } nh_tensor_table;
 
 /* Batch::new (crates/neura-generate/src/batch.rs:279-465): allocates fp16 K/V caches of
- * capacity = context + max_rows per (layer, kv head, plane) and every activation buffer. */
+ * capacity = (window, or context without one) + max_rows per (layer, kv head, plane) and every activation buffer. */
 nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_weights *weights, const nh_tensor_table *table);
 void nh_model_destroy(nh_model *model);
 /* the answer program (crates/neura-generate/src/batch.rs:1716-1725): one token per plane.

@@ -22,7 +22,7 @@ class Epilogue(ctypes.Structure):
 
 class ModelConfig(ctypes.Structure):
     _fields_ = [(name, c_uint32) for name in
-                ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "context", "batch", "max_rows")] + \
+                ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "context", "batch", "max_rows", "window")] + \
                [("rope_base", c_float), ("eps", c_float)]
 
 
@@ -61,9 +61,9 @@ SIGNATURES = {
     "nh_rmsnorm": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_rope": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_float, c_void_p]),
     "nh_cache_write": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
-                                 c_uint32, c_void_p, c_void_p]),
+                                 c_uint32, c_void_p, c_void_p, c_int32]),
     "nh_attention": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
-                               c_uint32, c_void_p, c_float, c_void_p]),
+                               c_uint32, c_uint32, c_void_p, c_float, c_void_p]),
     "nh_gather": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_argmax": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
     "nh_sample": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),

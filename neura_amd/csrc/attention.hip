@@ -31,6 +31,27 @@ struct AttentionParams {
     const uint32_t *cursor;
     float scale;
     uint32_t *refusal;
+    uint32_t reach;  // 0, or the span of a ring of `keys` slots
+};
+
+// A ring cache (Cache::windowed, crates/neura-decoder/src/cache.rs:311-317, :391-394): once `written` positions have gone
+// in, slot `at` holds the latest position below `written` that lands on it (key_position,
+// crates/neura-kernel/src/task/attention.rs:103-108), and a query weighs the `reach` positions up to its own
+// (weighed, :136-144).  The one division is done once: the slots up to `last` hold base + at, the others base - keys + at.
+struct Ring {
+    uint32_t base, last, keys, reach;
+    __device__ Ring(uint32_t keys, uint32_t written, uint32_t reach) : keys(keys), reach(reach) {
+        if (written <= keys) {
+            base = 0u, last = keys - 1u;
+        } else {
+            last = (written - 1u) % keys;
+            base = written - 1u - last;
+        }
+    }
+    __device__ __forceinline__ bool seen(uint32_t at, uint32_t position) const {
+        const uint32_t held = at <= last ? base + at : base - keys + at;
+        return held <= position && position - held < reach;
+    }
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -106,12 +127,15 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
     fetch_tile<T, STEP, WIDTH>(kraw, vraw, p.cache_k, p.cache_v, plane, begin + mine, p.capacity, dl);
 
     uint32_t origin = p.cursor ? p.cursor[b] : 0u;
-    if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+    if (!p.reach && origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
         if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
         origin = p.keys - p.rows;
     }
-    const uint32_t visible = min(p.keys, origin + row + 1u);  // key `at` counts iff at <= origin + row
+    // key `at` counts iff at <= origin + row; in a ring every written slot is walked and asked what it holds
+    const uint32_t position = origin + row;
+    const uint32_t visible = min(p.keys, p.reach ? origin + p.rows : position + 1u);
     const uint32_t last = min(visible, begin + chunk);
+    const Ring ring(p.keys, origin + p.rows, p.reach);
 
     float qr[MAX_GROUPS][8];
 #pragma unroll
@@ -149,7 +173,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 #pragma unroll
                     for (int j = 0; j < 8; j++) score = fmaf(qr[g][j], kf[j], score);
                     score = key_sum<LPK>(score) * p.scale;
-                    if (dl == 0) scores[local][g] = key < last ? score : -INFINITY;
+                    if (dl == 0) scores[local][g] = key < last && (!p.reach || ring.seen(key, position)) ? score : -INFINITY;
                 }
             }
         }
@@ -329,20 +353,21 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
     const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
 
     uint32_t origin = p.cursor ? p.cursor[b] : 0u;
-    if (origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+    if (!p.reach && origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
         if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
         origin = p.keys - p.rows;
     }
+    const Ring ring(p.keys, origin + p.rows, p.reach);
     // this lane's column: a query row and a query head of the group
     const uint32_t block_row = blockIdx.y * 4u * rows_per_wave;
     const uint32_t row = block_row + wave * rows_per_wave + n / G, g = n % G;
     const bool held = n < rows_per_wave * G && row < p.rows;
-    const uint32_t limit = origin + min(row, p.rows - 1u);  // the last key this column sees
-    // the workgroup walks up to the last key its last row sees
+    const uint32_t limit = origin + min(row, p.rows - 1u);  // the last key this column sees (its own position)
+    // the workgroup walks up to the last key its last row sees; a ring is walked whole, every slot asked what it holds
     const uint32_t last_row = min(p.rows, block_row + 4u * rows_per_wave) - 1u;
-    const uint32_t span = min(p.keys, origin + last_row + 1u);
+    const uint32_t span = min(p.keys, p.reach ? origin + p.rows : origin + last_row + 1u);
     const uint32_t wave_first = block_row + wave * rows_per_wave;
-    const uint32_t wave_span = wave_first < p.rows ? min(p.keys, origin + min(p.rows, wave_first + rows_per_wave)) : 0u;
+    const uint32_t wave_span = wave_first >= p.rows ? 0u : (p.reach ? span : min(p.keys, origin + min(p.rows, wave_first + rows_per_wave)));
 
     // queries as two half planes: q = value + residue, both halves
     half8_t q_value[STEPS], q_residue[STEPS];
@@ -386,7 +411,7 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
             *reinterpret_cast<u32x4 *>(&kt[key][chunk * 8u]) = kraw[k];
             // rows past the written keys may hold anything, and a weight of zero does not silence a NaN
-            const uint32_t keep = tile + key < p.keys ? 0xffffffffu : 0u;
+            const uint32_t keep = tile + key < span ? 0xffffffffu : 0u;
             const uint32_t words[4] = {vraw[k].x & keep, vraw[k].y & keep, vraw[k].z & keep, vraw[k].w & keep};
 #pragma unroll
             for (int i = 0; i < 8; i++) vt[chunk * 8u + i][key] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
@@ -410,7 +435,7 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const uint32_t key = tile + 8u * (r >> 2) + 4u * h + (r & 3);
-            const bool seen = held && key <= limit && key < p.keys;
+            const bool seen = held && key < p.keys && (p.reach ? ring.seen(key, limit) : key <= limit);
             scores[r] = seen ? fmaf(fine[r], 1.0f / 2048.0f, scores[r]) * p.scale : -INFINITY;
             tile_top = fmaxf(tile_top, scores[r]);
         }
@@ -471,7 +496,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     p.cache_k = a.cache_k, p.cache_v = a.cache_v;
     p.heads = a.heads, p.kv_heads = a.kv_heads, p.groups = a.heads / a.kv_heads;
     p.batch = a.batch, p.rows = a.rows, p.capacity = a.capacity, p.keys = a.keys;
-    p.cursor = a.cursor, p.scale = a.scale, p.refusal = d->refusal;
+    p.cursor = a.cursor, p.scale = a.scale, p.refusal = d->refusal, p.reach = a.reach;
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;

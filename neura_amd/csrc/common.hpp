@@ -109,10 +109,12 @@ int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, u
 // output rows [0, q_rows) are rotated and written to y, rows [q_rows, k_rows) are rotated, rounded to fp16 and
 // written to the key cache at the cursor, the rest are rounded to fp16 into the value cache.
 struct RopeFusion {
-    const float *cosines, *sines;  // [capacity][width / 2]: cos and sin of f32(position) * pow(base, -2c/width)
+    const float *cosines, *sines;  // [positions][width / 2]: cos and sin of f32(position) * pow(base, -2c/width)
     const uint32_t *cursor;        // device, one plane
     uint16_t *cache_k, *cache_v;
     uint32_t width, q_rows, k_rows, capacity;
+    uint32_t positions;  // rows of the two tables
+    uint32_t ring;       // 0, or the span of a ring cache: position p is written to slot p % ring
 };
 
 struct GemvArgs {
@@ -156,7 +158,7 @@ int32_t launch_rope(nh_device *d, const float *x, uint32_t planes, uint32_t batc
                     const uint32_t *cursor, float base, float *out);
 int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
                            uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask);
+                           const uint8_t *mask, bool ring);
 
 // q / out addressing: element (head, plane, row, c) at head*sh + plane*sb + row*sr + c
 struct AttentionArgs {
@@ -167,6 +169,7 @@ struct AttentionArgs {
     uint32_t heads, kv_heads, batch, rows, width, capacity, keys;
     const uint32_t *cursor;
     float scale;
+    uint32_t reach = 0;  // 0, or the span of a ring cache of `keys` slots (Cache::windowed): the last `reach` positions are weighed
 };
 int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 
@@ -176,11 +179,11 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t positions, float *cosines, float *sines);
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base);
+                           const uint8_t *mask, float base, bool ring);
 
-// one token of one plane: v (+ bias) as halves into the value state at cursor[0]
+// one token of one plane: v (+ bias) as halves into the value state at cursor[0] (at cursor[0] % ring when the cache is a ring)
 int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
-                            const uint32_t *cursor);
+                            const uint32_t *cursor, uint32_t ring);
 int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n);
 
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,

@@ -37,7 +37,7 @@ struct GemvParams {
     const float *rope_cosines, *rope_sines;  // [position][width / 2]
     const uint32_t *rope_cursor;
     uint16_t *rope_k, *rope_v;
-    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity;
+    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
     uint32_t *refusal;
     const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
 };
@@ -425,20 +425,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
                 float value = total;
                 if (n < p.rope_k_rows) {
                     // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
-                    const float cosine = p.rope_cosines[(size_t)min(position, p.rope_capacity - 1u) * half + c];
-                    const float sine = p.rope_sines[(size_t)min(position, p.rope_capacity - 1u) * half + c];
+                    const float cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+                    const float sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
                     value = (i & 1u) ? total * cosine + other * sine : total * cosine - other * sine;
                 }
                 if (n < p.rope_q_rows) {
                     p.y[n] = value;
-                } else if (position >= p.rope_capacity) {
+                } else if (position >= p.rope_positions || (!p.rope_ring && position >= p.rope_capacity)) {
                     atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
                 } else {
                     const bool key = n < p.rope_k_rows;
                     const uint32_t within = n - (key ? p.rope_q_rows : p.rope_k_rows);  // head * width + channel
                     const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
                     uint16_t *cache = key ? p.rope_k : p.rope_v;
-                    cache[((size_t)head * p.rope_capacity + position) * p.rope_width + channel] = float_to_half(value);
+                    const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
+                    cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
                 }
             }
         } else if (u < R && i < p.N) {
@@ -1707,6 +1708,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     if (a.rope) {
         p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
         p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
+        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring;
         p.refusal = d->refusal;
         for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
     } else if (a.bias[0] || a.bias[1] || a.bias[2]) {

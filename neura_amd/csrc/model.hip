@@ -15,6 +15,8 @@ struct nh_model {
     nh_model_config c{};
     int32_t element = 0;
     uint32_t capacity = 0, window = 0;
+    uint32_t positions = 0;  // rows of the rotation's tables: every position a cursor can name
+    bool ring = false;       // the window is a ring (a bounded batch, crates/neura-generate/src/batch.rs:313-325)
     const uint8_t *token_embd = nullptr, *output = nullptr;
     const float *output_norm = nullptr;
     std::vector<const float *> attn_norm, ffn_norm;
@@ -134,7 +136,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
             // one token of one active plane: the rotation, the biases and the cache append ride in the product's epilogue
-            RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
+            RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity, m->positions,
+                            m->ring ? m->window : 0u};
             if (alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
                 a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];
@@ -146,7 +149,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             qk.W[1] = m->attn_k[L];
             qk.end[0] = QW, qk.end[1] = QW + KW, qk.end[2] = QW + KW;
             qk.norm_w = m->attn_norm[L], qk.eps = c.eps;
-            RopeFusion rope_qk{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity};
+            RopeFusion rope_qk = rope;
             const bool split_value = !alike && element_at(m, L, Q) == element_at(m, L, K_) && !products_only && T == 1 && !mask &&
                                      gemv_fuses_rope(qk, rope_qk);
             if (roped || (alike && (!biased || products_only))) {
@@ -158,7 +161,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 GemvArgs value = narrow(m, element_at(m, L, V), m->attn_v[L], KW, H, m->h, T, m->xn);
                 value.norm_w = m->attn_norm[L], value.eps = c.eps;
                 if ((status = launch_gemv(d, value)) != NH_OK) return status;
-                if ((status = launch_value_append(d, m->xn, m->bias_v[L], m->cache_v[L], c.kv_heads, hd, m->capacity, dev_cursor(m))) != NH_OK)
+                if ((status = launch_value_append(d, m->xn, m->bias_v[L], m->cache_v[L], c.kv_heads, hd, m->capacity, dev_cursor(m), m->ring ? m->window : 0u)) != NH_OK)
                     return status;
                 roped = true;
             } else {
@@ -177,7 +180,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             }
         }
         if (!products_only && !roped && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
-                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base)) != NH_OK)
+                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base, m->ring)) != NH_OK)
             return status;
         AttentionArgs at{};
         at.q = m->qkv, at.out = m->att;
@@ -186,6 +189,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         at.cache_k = m->cache_k[L], at.cache_v = m->cache_v[L];
         at.heads = c.heads, at.kv_heads = c.kv_heads, at.batch = B, at.rows = rows, at.width = hd;
         at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
+        at.reach = m->ring ? m->window : 0u;
         if (!products_only && (status = launch_attention(d, at)) != NH_OK) return status;
         if (wide) {
             GemmArgs o{element_at(m, L, O), m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
@@ -270,12 +274,23 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         fail(NH_E_ARGUMENT, "a rope base of %f turns nothing", (double)c.rope_base);
         return nullptr;
     }
+    // crates/neura-generate/src/batch.rs:315-322
+    if (c.window > c.context) {
+        fail(NH_E_ARGUMENT, "a batch keeps a window of %u tokens over a context of %u", c.window, c.context);
+        return nullptr;
+    }
+    if (c.window && (c.max_rows ? c.max_rows : 1u) > c.window) {
+        fail(NH_E_ARGUMENT, "a batch fills chunks of %u rows into a window of %u tokens", c.max_rows, c.window);
+        return nullptr;
+    }
     nh_model *m = new nh_model();
     m->d = device, m->weights = weights, m->c = c, m->element = table->matrix_element;
     m->elements = elements;
     uint32_t widest = c.max_rows ? c.max_rows : 1;
-    m->window = c.context;               // crates/neura-generate/src/batch.rs:314
-    m->capacity = c.context + widest;    // crates/neura-generate/src/batch.rs:323-325
+    m->ring = c.window != 0;                          // BatchSpec::window names one: the caches are rings of it
+    m->window = c.window ? c.window : c.context;      // crates/neura-generate/src/batch.rs:313-314
+    m->capacity = m->window + widest;                 // crates/neura-generate/src/batch.rs:323-325
+    m->positions = c.context + widest;
     m->max_tokens = widest * c.batch;
     size_t arena = nh_weights_bytes(weights);
     auto at = [&](uint64_t offset, uint64_t bytes, const char *name) -> const uint8_t * {
@@ -340,8 +355,8 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     ok = device_array(m->h, T * H) && device_array(m->xn, T * (H > QW ? H : QW)) && device_array(m->qkv, T * (QW + 2 * KW)) &&
          device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T * F) &&
          device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 6 * c.batch + 4) &&
-         device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->capacity * (c.head_dim / 2)) &&
-         device_array(m->rope_sin, (size_t)m->capacity * (c.head_dim / 2));
+         device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->positions * (c.head_dim / 2)) &&
+         device_array(m->rope_sin, (size_t)m->positions * (c.head_dim / 2));
     for (uint32_t L = 0; ok && L < c.layers; L++) {
         uint16_t *k = nullptr, *v = nullptr;
         ok = device_array(k, m->cache_elements);
@@ -369,7 +384,7 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         if (choice > wanted) wanted = choice;
         if (split_rows > wanted) wanted = split_rows;
         ok = ok && scratch(device, wanted) != nullptr && rope_frequencies(device, c.rope_base, c.head_dim) != nullptr &&
-             launch_rope_angles(device, c.rope_base, c.head_dim, m->capacity, m->rope_cos, m->rope_sin) == NH_OK;
+             launch_rope_angles(device, c.rope_base, c.head_dim, m->positions, m->rope_cos, m->rope_sin) == NH_OK;
     }
     {
         const char *held = getenv("NEURA_HIP_GRAPH");
@@ -611,7 +626,7 @@ int32_t nh_rope(nh_device *device, const float *dev_x, uint32_t planes, uint32_t
 
 int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v, uint16_t *dev_cache_k, uint16_t *dev_cache_v,
                        uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
-                       const uint32_t *dev_cursor, const uint8_t *dev_mask) {
+                       const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring) {
     NH_REQUIRE(device && dev_k && dev_v && dev_cache_k && dev_cache_v && dev_cursor, "a cache write names no device or no buffer");
     // crates/neura-decoder/src/cache.rs:113-125, :328-335
     NH_REQUIRE(kv_heads > 0 && width > 0 && batch > 0, "a cache of %u planes of %u heads of %u numbers holds no key", batch, kv_heads, width);
@@ -619,12 +634,12 @@ int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v
     NH_REQUIRE(rows > 0 && rows <= window, "a cache of a %u position window takes %u rows at a time", window, rows);
     NH_REQUIRE(!dev_mask || rows <= capacity - window, "a masked chunk of %u rows holds only %u scratch rows", rows, capacity - window);
     int32_t status = launch_cache_write(device, dev_k, dev_v, dev_cache_k, dev_cache_v, kv_heads, batch, rows, width, capacity, window,
-                                        dev_cursor, dev_mask);
+                                        dev_cursor, dev_mask, ring != 0);
     return status != NH_OK ? status : check_refusal(device, "a cache write");
 }
 
 int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
-                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                     uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach,
                      const uint32_t *dev_cursor, float scale, float *dev_out) {
     NH_REQUIRE(device && dev_q && dev_cache_k && dev_cache_v && dev_out, "an attention names no device or no buffer");
     // crates/neura-decoder/src/cache.rs:383-388
@@ -639,7 +654,7 @@ int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_
     a.q_sr = a.o_sr = width;
     a.cache_k = dev_cache_k, a.cache_v = dev_cache_v;
     a.heads = heads, a.kv_heads = kv_heads, a.batch = batch, a.rows = rows, a.width = width, a.capacity = capacity, a.keys = keys;
-    a.cursor = dev_cursor, a.scale = scale;
+    a.cursor = dev_cursor, a.scale = scale, a.reach = reach;
     int32_t status = launch_attention(device, a);
     return status != NH_OK ? status : check_refusal(device, "an attention");
 }

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void cache_write_kernel(const float *__restric
                                                           uint16_t *__restrict__ cache_k, uint16_t *__restrict__ cache_v,
                                                           uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width,
                                                           uint32_t capacity, uint32_t window, const uint32_t *__restrict__ cursor,
-                                                          const uint8_t *__restrict__ mask, uint32_t *refusal) {
+                                                          const uint8_t *__restrict__ mask, uint32_t *refusal, bool ring) {
     const uint64_t total = (uint64_t)kv_heads * batch * rows * width;
     for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < total; index += (uint64_t)gridDim.x * blockDim.x) {
         uint32_t c = (uint32_t)(index % width);
@@ -98,7 +98,9 @@ __global__ __launch_bounds__(256) void cache_write_kernel(const float *__restric
         uint32_t b = (uint32_t)((vector / rows) % batch);
         uint32_t head = (uint32_t)(vector / rows / batch);
         bool active = mask == nullptr || mask[b];
-        uint32_t slot = active ? cursor[b] + row : window + row;
+        // a ring seats position p at p mod window (crates/neura-decoder/src/layout.rs:32-36)
+        uint32_t seat = ring ? (cursor[b] + row) % window : cursor[b] + row;
+        uint32_t slot = active ? seat : window + row;
         if (slot >= capacity) {
             atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
             continue;
@@ -111,12 +113,12 @@ __global__ __launch_bounds__(256) void cache_write_kernel(const float *__restric
 
 int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
                            uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask) {
+                           const uint8_t *mask, bool ring) {
     uint64_t total = (uint64_t)kv_heads * batch * rows * width;
     if (!total) return NH_OK;
     uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     hipLaunchKernelGGL(cache_write_kernel, dim3(grid), dim3(256), 0, d->stream, k, v, cache_k, cache_v, kv_heads, batch, rows, width,
-                       capacity, window, cursor, mask, d->refusal);
+                       capacity, window, cursor, mask, d->refusal, ring);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -125,10 +127,10 @@ int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_
 // a value row whose key went out with the product that rotated it)
 __global__ __launch_bounds__(256) void value_append_kernel(const float *__restrict__ v, const float *__restrict__ bias, uint16_t *__restrict__ cache_v,
                                                            uint32_t kv_heads, uint32_t width, uint32_t capacity, const uint32_t *__restrict__ cursor,
-                                                           uint32_t *refusal) {
+                                                           uint32_t *refusal, uint32_t ring) {
     const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
     if (index >= kv_heads * width) return;
-    const uint32_t slot = cursor[0];
+    const uint32_t slot = ring ? cursor[0] % ring : cursor[0];
     if (slot >= capacity) {
         atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
         return;
@@ -139,11 +141,11 @@ __global__ __launch_bounds__(256) void value_append_kernel(const float *__restri
 }
 
 int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
-                            const uint32_t *cursor) {
+                            const uint32_t *cursor, uint32_t ring) {
     const uint32_t total = kv_heads * width;
     if (!total) return NH_OK;
     hipLaunchKernelGGL(value_append_kernel, dim3((total + 255) / 256), dim3(256), 0, d->stream, v, bias, cache_v, kv_heads, width, capacity, cursor,
-                       d->refusal);
+                       d->refusal, ring);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qk
                                                           uint32_t batch, uint32_t rows, uint16_t *__restrict__ cache_k,
                                                           uint16_t *__restrict__ cache_v, uint32_t capacity, uint32_t window,
                                                           const uint32_t *__restrict__ cursor, const uint8_t *__restrict__ mask,
-                                                          const float *__restrict__ table, uint32_t *refusal) {
+                                                          const float *__restrict__ table, uint32_t *refusal, bool ring) {
     const uint32_t half = width / 2;
     const uint32_t vectors = heads + 2 * kv_heads;  // per token: q heads, k heads, v heads
     const uint32_t stride = vectors * width;
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qk
             continue;
         }
         bool active = mask == nullptr || mask[b];
-        uint32_t slot = active ? position : window + row;
+        uint32_t slot = active ? (ring ? position % window : position) : window + row;
         if (slot >= capacity) {
             atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
             continue;
@@ -219,14 +221,14 @@ __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qk
 
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base) {
+                           const uint8_t *mask, float base, bool ring) {
     const float *table = rope_frequencies(d, base, width);
     if (!table) return NH_E_DEVICE;
     uint64_t total = (uint64_t)batch * rows * (heads + 2 * kv_heads) * (width / 2);
     if (!total) return NH_OK;
     uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     hipLaunchKernelGGL(rope_append_kernel, dim3(grid), dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k,
-                       cache_v, capacity, window, cursor, mask, table, d->refusal);
+                       cache_v, capacity, window, cursor, mask, table, d->refusal, ring);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }

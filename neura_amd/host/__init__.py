@@ -54,8 +54,11 @@ SIGNATURES = {
     "nhost_payload_bytes": (c_uint64, [c_int32, c_uint64]),
     "nhost_runtime_open": (c_void_p, [c_int32]),
     "nhost_runtime_close": (None, [c_void_p]),
-    "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
-    "nhost_batch_open_sampled": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_float, c_uint32, c_float]),
+    "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32]),
+    "nhost_batch_open_sampled": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_float, c_uint32, c_float,
+                                            c_uint32]),
+    "nhost_batch_window_check": (c_int32, [c_uint32]),
+    "nhost_batch_window": (c_int64, [c_void_p]),
     "nhost_sampling_check": (c_int32, [c_float, c_uint32, c_float]),
     "nhost_plane_seed": (c_uint32, [c_uint32, c_uint32]),
     "nhost_seed_bits": (c_uint32, [c_uint32]),
@@ -64,7 +67,7 @@ SIGNATURES = {
     "nhost_batch_set_temperature": (c_int32, [c_void_p, c_int32, c_float]),
     "nhost_batch_set_keep": (c_int32, [c_void_p, c_int32, c_uint32]),
     "nhost_batch_set_cumulative": (c_int32, [c_void_p, c_int32, c_float]),
-    "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_spec_check": (c_int32, [c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32]),
     "nhost_snapshot_round_trip": (c_int64, [c_char_p, c_size_t, c_void_p, c_size_t]),
     "nhost_batch_snapshot": (c_int64, [c_void_p, c_void_p, c_size_t]),
     "nhost_batch_restore": (c_int32, [c_void_p, c_char_p, c_size_t]),
@@ -288,9 +291,12 @@ def cache_validate(name, heads, width, capacity, window, batch, rows, element=1)
         raise _refused()
 
 
-def batch_spec_check(context, batch, chunks):
+def batch_spec_check(context, batch, chunks, window=None):
+    """BatchSpec::new(context, batch, chunks)[.window(window)] as Batch::new checks it, with no device"""
     held, count = _words(chunks)
-    if library().nhost_batch_spec_check(context, batch, held, count) != 0:
+    if window is not None and library().nhost_batch_window_check(window) != 0:
+        raise _refused()
+    if library().nhost_batch_spec_check(context, batch, held, count, window or 0) != 0:
         raise _refused()
 
 
@@ -418,16 +424,19 @@ class Batch:
     """A Qwen2 GGUF loaded onto a runtime with a generation batch above it: greedy, or drawing with
     `sampling` = (temperature, keep, cumulative) as BatchSpec::sampled(Sampling::sampled(..)) does."""
 
-    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None):
+    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None, window=None):
+        """`window`: BatchSpec::window -- the caches are rings of that many tokens and a sequence attends to its last `window`"""
         held, count = _words(chunks)
         self.planes = batch
         self.vocabulary = vocabulary
+        if window is not None and library().nhost_batch_window_check(window) != 0:
+            raise _refused()
         if sampling is None:
-            self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count)
+            self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count, window or 0)
         else:
             temperature, keep, cumulative = sampling
             self.handle = library().nhost_batch_open_sampled(runtime.handle, archive.handle, vocabulary, context, batch, held, count,
-                                                             temperature, keep, cumulative)
+                                                             temperature, keep, cumulative, window or 0)
         if not self.handle:
             raise _refused()
 
@@ -503,6 +512,9 @@ class Batch:
         if at == -2:
             raise _refused()
         return None if at < 0 else at
+
+    def window(self):
+        return self._status(library().nhost_batch_window(self.handle))
 
     def remaining(self, slot):
         left = library().nhost_batch_remaining(self.handle, slot)

@@ -191,11 +191,17 @@ void *nhost_runtime_open(int32_t index) {
 }
 void nhost_runtime_close(void *runtime) { delete static_cast<runtime::Runtime *>(runtime); }
 
+// BatchSpec::new(context, batch, chunks), and .window(window) when window is not 0
+static generate::BatchSpec spec_of(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count, uint32_t window) {
+    generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
+    return window ? spec.window(window) : spec;
+}
 // a Qwen2 GGUF (whole or file) becomes a model and a greedy batch over it
-void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count) {
+void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
+                       uint32_t window) {
     return guarded([&]() -> void * {
         auto *opened = static_cast<Opened *>(held);
-        generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
+        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window);
         auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
         auto out = std::make_unique<Loaded>();
         out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
@@ -205,11 +211,10 @@ void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t 
 }
 // the same with a sampled answer (BatchSpec::sampled(Sampling::sampled(temperature, keep, cumulative)))
 void *nhost_batch_open_sampled(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
-                               float temperature, uint32_t keep, float cumulative) {
+                               float temperature, uint32_t keep, float cumulative, uint32_t window) {
     return guarded([&]() -> void * {
         auto *opened = static_cast<Opened *>(held);
-        generate::BatchSpec spec =
-            generate::BatchSpec(context, batch, std::vector<uint32_t>(chunks, chunks + count)).sampled(generate::Sampling::sampled(temperature, keep, cumulative));
+        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window).sampled(generate::Sampling::sampled(temperature, keep, cumulative));
         auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
         auto out = std::make_unique<Loaded>();
         out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
@@ -260,12 +265,18 @@ int32_t nhost_batch_set_cumulative(void *held, int32_t slot, float value) {
     }, -1);
 }
 // BatchSpec's refusals alone, with no device: a batch over no model
-int32_t nhost_batch_spec_check(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count) {
+int32_t nhost_batch_spec_check(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count, uint32_t window) {
     return guarded([&] {
-        generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
-        generate::Batch::validate(spec);
+        generate::Batch::validate(spec_of(context, batch, chunks, count, window));
         return 0;
     }, -1);
+}
+// BatchSpec::window's own refusal
+int32_t nhost_batch_window_check(uint32_t window) {
+    return guarded([&] { return generate::BatchSpec(8, 1, {}).window(window), 0; }, -1);
+}
+int64_t nhost_batch_window(void *held) {
+    return guarded([&]() -> int64_t { return (int64_t) static_cast<Loaded *>(held)->batch->window(); }, -1);
 }
 void nhost_batch_close(void *held) { delete static_cast<Loaded *>(held); }
 int32_t nhost_batch_admit(void *held, const uint32_t *tokens, uint32_t count) {

@@ -707,8 +707,8 @@ class Cache {
                      "a cache holds keys and values in single, half or bfloat16 storage, and %s storage carries another grid", neura::name(element));
         NEURA_ASSERT(element == Element::Half, "this build keeps caches in half storage, and %s storage is not built", neura::name(element));
     }
-    Cache(const runtime::Runtime &runtime, const std::string &name, CacheShape shape, Element element = Element::Half)
-        : device_(runtime.device()), name_(name), shape_(shape) {
+    Cache(const runtime::Runtime &runtime, const std::string &name, CacheShape shape, Element element = Element::Half, bool ring = false)
+        : device_(runtime.device()), name_(name), shape_(shape), ring_(ring) {
         validate(name, shape, element);
         size_t bytes = (size_t)shape.heads * shape.batch * shape.capacity * shape.width * 2;
         keys_ = static_cast<uint16_t *>(nh_alloc(device_, bytes));
@@ -722,9 +722,15 @@ class Cache {
     Cache(const Cache &) = delete;
     Cache &operator=(const Cache &) = delete;
 
+    // crates/neura-decoder/src/cache.rs:67-69: the window is a ring -- position p is written to slot p mod window and a
+    // query weighs the last `window` positions
+    static std::unique_ptr<Cache> windowed(const runtime::Runtime &runtime, const std::string &name, CacheShape shape, Element element = Element::Half) {
+        return std::make_unique<Cache>(runtime, name, shape, element, true);
+    }
     uint32_t rows() const { return shape_.rows; }
     uint32_t batch() const { return shape_.batch; }
     uint32_t window() const { return shape_.window; }
+    bool ring() const { return ring_; }
     std::pair<uint16_t *, uint16_t *> states() const { return {keys_, values_}; }  // "{name}.key", "{name}.value"
     std::string key_name() const { return name_ + ".key"; }
     std::string value_name() const { return name_ + ".value"; }
@@ -742,7 +748,7 @@ class Cache {
         NEURA_ASSERT(query_heads % shape_.heads == 0,
                      "a query of %u heads reads a cache of %u key heads, and every key head serves a whole group of queries", query_heads, shape_.heads);
         runtime::check(nh_attention(device_, query, keys_, values_, query_heads, shape_.heads, shape_.batch, shape_.rows, shape_.width,
-                                    shape_.capacity, shape_.window, cursor, scale, out));
+                                    shape_.capacity, shape_.window, ring_ ? shape_.window : 0u, cursor, scale, out));
     }
     // reset: host flags, one per plane; a set flag zeroes the plane's keys and values
     void reset(const std::vector<uint8_t> &reset) {
@@ -760,11 +766,12 @@ class Cache {
   private:
     void store(const uint32_t *cursor, const float *keys, const float *values, const uint8_t *active) {
         runtime::check(nh_cache_write(device_, keys, values, keys_, values_, shape_.heads, shape_.batch, shape_.rows, shape_.width, shape_.capacity,
-                                      shape_.window, cursor, active));
+                                      shape_.window, cursor, active, ring_ ? 1 : 0));
     }
     nh_device *device_;
     std::string name_;
     CacheShape shape_;
+    bool ring_ = false;
     uint16_t *keys_ = nullptr, *values_ = nullptr;
 };
 
@@ -798,7 +805,7 @@ struct Config {
     }
 };
 
-// crates/neura-generate/src/batch.rs:110-153 (greedy; sampling, tuning, sharing and windows are not built)
+// crates/neura-generate/src/batch.rs:110-153 (tuning and sharing are not built)
 // crates/neura-generate/src/sampling.rs:3-57: a batch answers with the largest logit, or draws among the `keep` largest
 // cut at a cumulative mass after dividing the logits by a temperature
 struct Sampling {
@@ -827,7 +834,14 @@ struct BatchSpec {
     uint32_t context, batch;
     std::vector<uint32_t> chunks;
     Sampling sampling;
+    std::optional<uint32_t> window_tokens;  // BatchSpec::window: the caches are rings of that many tokens
     BatchSpec(uint32_t context, uint32_t batch, std::vector<uint32_t> chunks) : context(context), batch(batch), chunks(std::move(chunks)) {}
+    BatchSpec window(uint32_t tokens) const {  // crates/neura-generate/src/batch.rs:148-152
+        NEURA_ASSERT(tokens > 0, "a batch keeps a window of no token");
+        BatchSpec out = *this;
+        out.window_tokens = tokens;
+        return out;
+    }
     BatchSpec sampled(Sampling held) const {  // crates/neura-generate/src/batch.rs:133-136
         BatchSpec out = *this;
         out.sampling = held;
@@ -916,6 +930,7 @@ class Model {
         c.layers = config.layers, c.hidden = H, c.heads = config.heads, c.kv_heads = config.key_heads, c.head_dim = config.head_width;
         c.ffn = F, c.vocab = config.vocabulary, c.context = spec.context, c.batch = spec.batch;
         c.max_rows = spec.chunks.empty() ? 1 : spec.chunks.front();
+        c.window = spec.window_tokens.value_or(0);
         c.rope_base = config.rope_base, c.eps = config.floor;
         model_ = nh_model_create(runtime.device(), &c, weights_->arena(), &table);
         if (!model_) panic("%s", nh_last_error());
@@ -1082,9 +1097,14 @@ class Batch {
             NEURA_ASSERT(chunk > 1 && chunk < spec.context,
                          "a batch fills %u rows of a context of %u, and a chunk holds between two rows and the rows a prompt leaves for the answer",
                          chunk, spec.context);
+        // crates/neura-generate/src/batch.rs:313-322
+        const uint32_t widest = spec.chunks.empty() ? 1 : spec.chunks.front(), window = spec.window_tokens.value_or(spec.context);
+        NEURA_ASSERT(window <= spec.context, "a batch keeps a window of %u tokens over a context of %u", window, spec.context);
+        NEURA_ASSERT(widest <= window, "a batch fills chunks of %u rows into a window of %u tokens", widest, window);
     }
     Batch(Model &model, BatchSpec spec)
-        : model_(model), batch_(spec.batch), context_(spec.context), chunks_(spec.chunks), slots_(spec.batch), seeded_(!spec.sampling.greedy),
+        : model_(model), batch_(spec.batch), context_(spec.context), window_(spec.window_tokens.value_or(spec.context)), chunks_(spec.chunks),
+          slots_(spec.batch), seeded_(!spec.sampling.greedy),
           temperatures_(spec.batch, spec.sampling.temperature), keeps_(spec.batch, spec.sampling.keep), cumulatives_(spec.batch, spec.sampling.cumulative) {
         validate(spec);
         for (uint32_t slot = 0; slot < batch_; slot++) seeds_.push_back(plane_seed(0, slot));  // batch.rs:426-428
@@ -1145,6 +1165,7 @@ class Batch {
     static uint32_t seed_bits(uint32_t seed) { return 0x3f800000u | ((seed ^ (seed >> 23)) & 0x007fffffu); }
     uint32_t batch() const { return batch_; }
     uint32_t context() const { return context_; }
+    uint32_t window() const { return window_; }  // crates/neura-generate/src/batch.rs:635-637
 
     uint32_t admit(const std::vector<uint32_t> &tokens) {  // batch.rs:1000-1013
         for (uint32_t slot = 0; slot < batch_; slot++)
@@ -1209,7 +1230,7 @@ class Batch {
     // ---- what a batch holds between steps (crates/neura-generate/src/batch.rs:484-628) ----------------------------
     BatchSnapshot snapshot() const {
         BatchSnapshot out;
-        out.batch = batch_, out.context = context_, out.window = context_, out.sampled = seeded_;
+        out.batch = batch_, out.context = context_, out.window = window_, out.sampled = seeded_;
         for (const auto &slot : slots_) {
             if (!slot) {
                 out.slots.push_back(std::nullopt);
@@ -1225,7 +1246,7 @@ class Batch {
     void restore(const BatchSnapshot &snapshot) {
         NEURA_ASSERT(snapshot.batch == batch_, "a batch of %u planes restores a snapshot of %u planes", batch_, snapshot.batch);
         NEURA_ASSERT(snapshot.context == context_, "a batch of %u tokens of context restores a snapshot of %u", context_, snapshot.context);
-        NEURA_ASSERT(snapshot.window == context_, "a batch of a %u token window restores a snapshot of a %u token window", context_, snapshot.window);
+        NEURA_ASSERT(snapshot.window == window_, "a batch of a %u token window restores a snapshot of a %u token window", window_, snapshot.window);
         NEURA_ASSERT(snapshot.sampled == seeded_, "a batch draws %s restores a snapshot of a batch that draws %s", seeded_ ? "true" : "false",
                      snapshot.sampled ? "true" : "false");
         NEURA_ASSERT(snapshot.slots.size() == batch_, "a snapshot of %u planes holds %zu slots", batch_, snapshot.slots.size());
@@ -1445,7 +1466,7 @@ class Batch {
     }
 
     Model &model_;
-    uint32_t batch_, context_;
+    uint32_t batch_, context_, window_;
     std::vector<uint32_t> chunks_;
     std::vector<std::optional<Slot>> slots_;
     bool seeded_;

@@ -57,11 +57,11 @@ class Weights:
 class Model:
     """nh_model over a Weights arena; tokens / cursors / mask are host arrays."""
 
-    def __init__(self, device, weights, shape, element, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None):
+    def __init__(self, device, weights, shape, element, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, window=None):
         self.device, self.lib, self.weights = device, device.lib, weights
         L = shape["layers"] if layers is None else layers
         self.config = ModelConfig(L, shape["hidden"], shape["heads"], shape["kv_heads"], shape["head_dim"], shape["ffn"], shape["vocab"],
-                                  context, batch, max_rows, rope_base, eps)
+                                  context, batch, max_rows, window or 0, rope_base, eps)
         table = TensorTable()
         table.matrix_element = element
         table.token_embd = weights.offsets["token_embd.weight"]

@@ -730,15 +730,34 @@ void oracle_rope(const float *in, uint32_t rows, uint32_t width, uint32_t origin
 
 static float softmax_exp(float a) { return expf(a > -104.0f ? a : -104.0f); } /* substrate.rs:110-116 */
 
+/* crates/neura-kernel/src/task/attention.rs:103-108: the position the key in slot `at` of a ring of `keys` slots holds
+ * once `written` positions have gone in -- the latest one below `written` that lands on the slot */
+static uint32_t key_position(uint32_t at, uint32_t keys, uint32_t written) {
+    if (written <= keys) return at;
+    return at + keys * ((written - 1u - at) / keys);
+}
+
+/* crates/neura-kernel/src/task/attention.rs:136-163 (causal): the key in slot `at` is weighed by the query at `position` */
+static int key_seen(uint32_t at, uint32_t keys, uint32_t written, uint32_t position, uint32_t reach) {
+    if (at >= keys) return 0;
+    uint32_t held = reach > 0 ? key_position(at, keys, written) : at;
+    if (held > position) return 0;
+    if (reach > 0 && position - held >= reach) return 0;
+    return 1;
+}
+
 /* Causal GQA attention over an fp16 or fp32 KV cache, fp32 online softmax in key blocks of 16
  * (crates/neura-kernel/src/task/attention.rs:309-617; visible :151-163; GQA head :327-334).
  *   q    [heads][batch][rows][width] f32
  *   K,V  [kv_heads][batch][capacity][width]  (kv_element: EL_F16 or EL_F32)
  *   cursor[batch] = origin of each plane; key `at` visible iff at <= origin+row and at < keys
+ *   reach: 0, or the span of a ring (Cache::windowed, crates/neura-decoder/src/cache.rs:366-406): slot `at` then holds
+ *          position key_position(at), and a query weighs the last `reach` positions up to its own
  *   out  [heads][batch][rows][width]
  */
 int oracle_attention(const float *q, const void *K, const void *V, int kv_element, uint32_t heads, uint32_t kv_heads, uint32_t batch,
-                     uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, const uint32_t *cursor, float scale, float *out) {
+                     uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach, const uint32_t *cursor, float scale,
+                     float *out) {
     if (kv_element != EL_F16 && kv_element != EL_F32) return -2;
     if (heads % kv_heads || width > 512) return -1;
     uint32_t groups = heads / kv_heads;
@@ -748,7 +767,7 @@ int oracle_attention(const float *q, const void *K, const void *V, int kv_elemen
                 const float *qr = q + (((size_t)h * batch + b) * rows + row) * width;
                 size_t plane = ((size_t)(h / groups) * batch + b) * capacity;
                 uint32_t origin = cursor[b];
-                uint32_t position = origin + row;
+                uint32_t position = origin + row, written = origin + rows;
                 uint32_t walked_keys = origin + rows < keys ? origin + rows : keys;
                 float acc[512];
                 for (uint32_t d = 0; d < width; d++) acc[d] = 0.0f;
@@ -759,7 +778,7 @@ int oracle_attention(const float *q, const void *K, const void *V, int kv_elemen
                     uint32_t block_keys = 0;
                     for (uint32_t s = 0; s < ATTN_KEYS; s++) {
                         uint32_t at = block * ATTN_KEYS + s;
-                        int seen = at < keys && at <= position;
+                        int seen = key_seen(at, keys, written, position, reach);
                         weights[s] = -INFINITY;
                         if (!seen) continue;
                         float score = 0.0f;
@@ -779,7 +798,7 @@ int oracle_attention(const float *q, const void *K, const void *V, int kv_elemen
                     for (uint32_t d = 0; d < width; d++) acc[d] = acc[d] * rescale;
                     for (uint32_t s = 0; s < ATTN_KEYS; s++) {
                         uint32_t at = block * ATTN_KEYS + s;
-                        if (!(at < keys && at <= position)) continue; /* an unseen key weighs exp(-104) ~ 0 there */
+                        if (!key_seen(at, keys, written, position, reach)) continue; /* an unseen key weighs exp(-104) ~ 0 there */
                         float weight = block_keys > 0 ? softmax_exp(weights[s] - largest) : 0.0f;
                         total = total + weight;
                         for (uint32_t d = 0; d < width; d++) {
@@ -963,6 +982,7 @@ typedef struct {
     uint32_t capacity; /* cache rows per (head, plane) */
     uint32_t window;   /* visible keys; scratch rows start at `window` */
     uint32_t batch;
+    uint32_t ring;     /* 1: the window is a ring (Cache::windowed): position p sits in slot p % window */
     float rope_base, eps;
     int matrix_element;          /* element of every matrix (EL_Q8_0 / EL_Q4_K / EL_F16 / EL_F32) */
     const uint8_t *token_embd;   /* [vocab][hidden] in matrix_element */
@@ -1016,7 +1036,7 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
         for (uint32_t c = 0; c < H; c++) h[(size_t)t * H + c] = tmp[c] * (mask[b] ? 1.0f : 0.0f);
     }
     for (uint32_t b = 0; b < B; b++)
-        if (mask[b] && cursor[b] + rows > m->window) return -4; /* refusal::ORIGIN, attention.rs:250-252 */
+        if (mask[b] && !m->ring && cursor[b] + rows > m->window) return -4; /* refusal::ORIGIN, attention.rs:250-252 (reach == 0) */
     float scale = 1.0f / sqrtf((float)hd);
     for (uint32_t L = 0; L < m->layers; L++) {
         oracle_rmsnorm(h, NULL, m->attn_norm[L], m->eps, T, H, xn, NULL);
@@ -1036,13 +1056,15 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
             }
             for (uint32_t head = 0; head < m->kv_heads; head++) {
                 /* slot math crates/neura-decoder/src/cache.rs:311-337, layout.rs:10-24 */
-                size_t slot = ((size_t)head * B + b) * m->capacity + (mask[b] ? cursor[b] + row : m->window + row);
+                /* a ring seats position p at p - window * floor(p / window) (layout.rs:32-36) */
+                uint32_t seat = m->ring ? (cursor[b] + row) % m->window : cursor[b] + row;
+                size_t slot = ((size_t)head * B + b) * m->capacity + (mask[b] ? seat : m->window + row);
                 oracle_rope(k + (size_t)t * KW + head * hd, 1, hd, cursor[b] + row, m->rope_base, tmp);
                 oracle_f32_to_f16_many(tmp, hd, m->cache_k[L] + slot * hd);
                 oracle_f32_to_f16_many(v + (size_t)t * KW + head * hd, hd, m->cache_v[L] + slot * hd);
             }
         }
-        oracle_attention(qh, m->cache_k[L], m->cache_v[L], EL_F16, m->heads, m->kv_heads, B, rows, hd, m->capacity, m->window, cursor, scale, att);
+        oracle_attention(qh, m->cache_k[L], m->cache_v[L], EL_F16, m->heads, m->kv_heads, B, rows, hd, m->capacity, m->window, m->ring ? m->window : 0u, cursor, scale, att);
         /* joined + as_rows: [heads][B][rows][hd] -> [T][heads*hd] */
         for (uint32_t t = 0; t < T; t++) {
             uint32_t row = t / B, b = t % B;

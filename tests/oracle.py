@@ -15,7 +15,7 @@ EL_Q3_K, EL_Q5_K = 11, 13
 
 
 class OracleModel(ctypes.Structure):
-    _fields_ = [(n, c_uint32) for n in ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "capacity", "window", "batch")] + [
+    _fields_ = [(n, c_uint32) for n in ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "capacity", "window", "batch", "ring")] + [
         ("rope_base", c_float), ("eps", c_float), ("matrix_element", c_int),
         ("token_embd", c_void_p), ("output", c_void_p), ("output_norm", c_void_p),
         ("attn_norm", POINTER(c_void_p)), ("attn_q", POINTER(c_void_p)), ("attn_k", POINTER(c_void_p)), ("attn_v", POINTER(c_void_p)),
@@ -146,7 +146,7 @@ def rope(x, origin, base):
     return out
 
 
-def attention(q, K, V, kv_heads, capacity, keys, cursor, scale):
+def attention(q, K, V, kv_heads, capacity, keys, cursor, scale, reach=0):
     q = np.ascontiguousarray(q, dtype=np.float32)
     heads, batch, rows, width = q.shape
     if K.dtype == np.uint16:
@@ -158,7 +158,7 @@ def attention(q, K, V, kv_heads, capacity, keys, cursor, scale):
     cursor = np.ascontiguousarray(cursor, dtype=np.uint32)
     out = np.empty_like(q)
     status = lib().oracle_attention(_p(q), _p(K), _p(V), c_int(el), c_uint32(heads), c_uint32(kv_heads), c_uint32(batch), c_uint32(rows),
-                                    c_uint32(width), c_uint32(capacity), c_uint32(keys), _p(cursor), c_float(scale), _p(out))
+                                    c_uint32(width), c_uint32(capacity), c_uint32(keys), c_uint32(reach), _p(cursor), c_float(scale), _p(out))
     assert status == 0, status
     return out
 
@@ -202,13 +202,17 @@ def sample(logits, drawn):
 class Model:
     """The oracle's decoder over host copies of the same GGUF tensors the device gets."""
 
-    def __init__(self, shape, element, tensors, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, elements=None):
+    def __init__(self, shape, element, tensors, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, elements=None,
+                 window=None):
         """`elements`: name -> element of the matrices that differ from `element`; tensors named blk.N.attn_{q,k,v}.bias
-        are added to the projections before the rotation."""
+        are added to the projections before the rotation.  `window`: the caches are rings of that many positions
+        (BatchSpec::window, crates/neura-generate/src/batch.rs:148-152, :313-325)."""
         self.keep = []
         L = shape["layers"] if layers is None else layers
-        self.capacity, self.window = context + max_rows, context
+        self.window = context if window is None else window
+        self.capacity = self.window + max_rows
         m = OracleModel()
+        m.ring = 0 if window is None else 1
         m.layers, m.hidden, m.heads, m.kv_heads = L, shape["hidden"], shape["heads"], shape["kv_heads"]
         m.head_dim, m.ffn, m.vocab = shape["head_dim"], shape["ffn"], shape["vocab"]
         m.capacity, m.window, m.batch = self.capacity, self.window, batch

@@ -32,9 +32,9 @@ def qwen2_gguf(path, shape, element, seed, elements=None, biases=()):
     return {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
 
 
-def alone(shape, element, tensors, prompt, count, elements=None):
+def alone(shape, element, tensors, prompt, count, elements=None, window=None):
     """The oracle's greedy answer to one prompt: fed token by token, then `count` choices."""
-    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT, elements=elements)
+    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT, elements=elements, window=window)
     margins = []
     for at, token in enumerate(prompt):
         logits, chosen = ref.forward([token], 1, [at])
@@ -83,6 +83,37 @@ def test_a_batched_sequence_answers_as_it_does_alone(runtime, tmp_path, shape, e
         assert got[slot] == want, (slot, margin)
     batch.close()
     archive.close()
+
+
+@pytest.mark.parametrize("chunks", [[], [8, 4]])
+def test_a_batch_keeps_only_the_window_of_tokens_it_declares(runtime, tmp_path, chunks):
+    """crates/neura-generate/tests/generation.rs:521-560 on the real decoder: a batch of a 10 token window answers as the
+    oracle's ring of 10 does, alone or beside another plane, with prompts longer than the window (the fill wraps)."""
+    WINDOW = 10
+    tensors = qwen2_gguf(tmp_path / "model.gguf", SHAPE, NH_Q8_0, seed=21)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    batch = host.Batch(runtime, archive, SHAPE["vocab"], CONTEXT, 2, chunks, window=WINDOW)
+    assert batch.window() == WINDOW
+    rng = np.random.default_rng(22)
+    prompts = [list(rng.integers(0, SHAPE["vocab"], n)) for n in (27, 5)]
+    slots = [batch.admit(prompt) for prompt in prompts]
+    got = run(batch, {slot: 14 for slot in slots})
+    for slot, prompt in zip(slots, prompts):
+        want, margin = alone(SHAPE, NH_Q8_0, tensors, prompt, 14, window=WINDOW)
+        assert got[slot] == want, (slot, margin)
+    unbounded, _ = alone(SHAPE, NH_Q8_0, tensors, prompts[0], 14)
+    assert unbounded != got[slots[0]]  # the window is felt: 27 prompt tokens in, only 10 are weighed
+    batch.close()
+    archive.close()
+    with pytest.raises(host.Panic) as refused:  # batch.rs:149, :315-322
+        host.batch_spec_check(16, 1, [], window=0)
+    assert "a batch keeps a window of no token" in str(refused.value)
+    with pytest.raises(host.Panic) as refused:
+        host.batch_spec_check(16, 1, [], window=17)
+    assert "a batch keeps a window of 17 tokens over a context of 16" in str(refused.value)
+    with pytest.raises(host.Panic) as refused:
+        host.batch_spec_check(16, 1, [8, 4], window=6)
+    assert "a batch fills chunks of 8 rows into a window of 6 tokens" in str(refused.value)
 
 
 MIXED_FILES = {

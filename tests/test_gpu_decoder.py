@@ -12,13 +12,13 @@ TINY = dict(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512, voc
 SMALL_Q4 = dict(layers=3, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=1000, tied=False)
 
 
-def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None):
+def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None, window=None):
     rng = np.random.default_rng(seed)
     tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
     host = {name: raw for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
-    model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers)
-    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers)
+    model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers, window=window)
+    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers, window=window)
     return model, ref, weights
 
 
@@ -150,6 +150,57 @@ def test_sampled_decode_steps_draw_as_the_oracle_draws(device):
     with pytest.raises(NeuraError):
         model.decode_step_sampled(tokens, [9] * 3, oracle.draws([(1, 1.0, 70, 1.0)] * 3))
     model.release(), weights.release()
+
+
+@pytest.mark.parametrize("shape,element,batch", [(TINY, NH_Q8_0, 2), (SMALL_Q4, NH_Q4_K, 1)])
+def test_a_windowed_model_keeps_a_ring_of_its_last_tokens(device, shape, element, batch):
+    """BatchSpec::window (crates/neura-generate/src/batch.rs:148-152, :313-325): caches of window + chunk rows written as
+    rings, attention over the last `window` positions.  A chunked fill that wraps inside a chunk, then decode steps two
+    turns round the ring (batch 1 folds the rotation and the ring seat into the q|k|v product), against the oracle."""
+    window, rows, context = 12, 8, 64
+    model, ref, weights = build(device, shape, element, batch=batch, context=context, max_rows=rows, seed=5, window=window)
+    assert model.capacity == window + rows
+    rng = np.random.default_rng(6)
+    cursor = 0
+    for chunk in range(2):  # the second chunk wraps: positions 8..15 over a ring of 12
+        prompt = rng.integers(0, shape["vocab"], (rows, batch))
+        model.prefill(prompt.reshape(-1), rows, [cursor] * batch)
+        ref.forward(prompt.reshape(-1), rows, [cursor] * batch, want_logits=False)
+        cursor += rows
+    tokens = rng.integers(0, shape["vocab"], batch)
+    for step in range(2 * window + 3):
+        want_logits, want = ref.forward(tokens, 1, [cursor] * batch)
+        got = model.decode_step(tokens, [cursor] * batch)
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens = got
+        cursor += 1
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_cache = oracle.f16_to_f32(model.cache_read(layer, which)[:, :, :window].reshape(-1))
+            want_cache = oracle.f16_to_f32(held[layer].reshape(shape["kv_heads"], batch, window + rows, shape["head_dim"])[:, :, :window].reshape(-1))
+            assert np.abs(got_cache - want_cache).max() <= 2e-3 * max(1.0, np.abs(want_cache).max())
+    with pytest.raises(NeuraError) as refused:  # batch.rs:315-318
+        Model(device, weights, shape, element, batch, 8, 1, window=9)
+    assert "a batch keeps a window of 9 tokens over a context of 8" in str(refused.value)
+    with pytest.raises(NeuraError) as refused:  # batch.rs:319-322
+        Model(device, weights, shape, element, batch, 32, 8, window=6)
+    assert "a batch fills chunks of 8 rows into a window of 6 tokens" in str(refused.value)
+    model.release(), weights.release()
+
+
+def test_a_window_as_wide_as_what_was_fed_changes_nothing(device):
+    """Until the ring wraps a windowed model holds every key an unbounded one holds: the same tokens."""
+    shape = TINY
+    bounded, _, held = build(device, shape, NH_Q8_0, batch=1, context=32, seed=7, window=16)
+    open_, _, held2 = build(device, shape, NH_Q8_0, batch=1, context=32, seed=7)
+    token_a = token_b = [3]
+    for step in range(16):
+        token_a = bounded.decode_step(token_a, [step])
+        token_b = open_.decode_step(token_b, [step])
+        assert list(token_a) == list(token_b), step
+        assert np.array_equal(bounded.logits(), open_.logits())
+    bounded.release(), open_.release(), held.release(), held2.release()
 
 
 def test_decode_refuses_what_the_reference_refuses(device):

@@ -388,6 +388,81 @@ def test_attention_of_equal_scores_is_the_running_mean(device):
             assert np.allclose(got[head, 0, 0], V[head // 2, 0, : origin + 1].astype(np.float32).mean(axis=0), atol=1e-5)
 
 
+def test_a_ring_cache_weighs_the_last_window_of_keys(device):
+    # crates/neura-decoder/tests/cache.rs:11-51 in half storage: equal scores, value = step -> the mean of the last WINDOW steps
+    WINDOW, CAPACITY, WIDTH = 5, 7, 32
+    ck = device.alloc(CAPACITY * WIDTH * 2)
+    cv = device.alloc(CAPACITY * WIDTH * 2)
+    q = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
+    q[..., 0] = 1.0
+    key = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
+    key[..., 0] = 1.0
+    for step in range(2 * WINDOW + 2):
+        value = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
+        value[..., 0] = float(step)
+        device.cache_write(key, value, ck, cv, CAPACITY, WINDOW, [step], ring=True)
+        got = device.attention(q, ck, cv, 1, CAPACITY, WINDOW, [step], 1.0, reach=WINDOW)
+        first = max(0, step - (WINDOW - 1))
+        expected = sum(range(first, step + 1)) / (step - first + 1)
+        assert abs(got[0, 0, 0, 0] - expected) < 1e-5 and got[0, 0, 0, 1] == 0.0, (step, got[0, 0, 0, :2])
+
+
+def test_a_masked_chunk_leaves_the_ring_it_wraps_into_alone(device):
+    # crates/neura-decoder/tests/cache.rs:53-95: an inactive plane whose cursor wraps onto slot 0 writes the scratch row
+    WINDOW, WIDTH = 4, 32
+    ck = device.alloc((WINDOW + 1) * WIDTH * 2)
+    cv = device.alloc((WINDOW + 1) * WIDTH * 2)
+    key = np.ones((1, 1, 1, WIDTH), dtype=np.float32)
+    values = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
+    values[..., 0] = 7.0
+    masked = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
+    masked[..., 0] = 9.0
+    device.cache_write(key, values, ck, cv, WINDOW + 1, WINDOW, [0], ring=True)
+    device.cache_write(key, masked, ck, cv, WINDOW + 1, WINDOW, [WINDOW], mask=[0], ring=True)
+    got = device.attention(np.zeros((1, 1, 1, WIDTH), dtype=np.float32), ck, cv, 1, WINDOW + 1, WINDOW, [0], 1.0, reach=WINDOW)
+    assert abs(got[0, 0, 0, 0] - 7.0) < 1e-5
+
+
+@pytest.mark.parametrize("heads,kv_heads,batch,width,window,chunks", [
+    (4, 2, 1, 32, 6, (1, 3, 2, 6, 1, 1, 4, 5, 2)),         # the row-at-a-time kernel
+    (12, 2, 2, 128, 40, (1, 17, 30, 1, 40, 8, 1, 1, 25)),  # chunks of four rows and more: the matrix cores
+    (14, 2, 1, 64, 100, (64, 1, 50, 1, 1, 100, 7)),
+    (28, 4, 1, 128, 300, (250, 1, 1, 120, 1, 1)),          # several sections of the ring, folded
+])
+def test_ring_attention_matches_the_oracle(device, heads, kv_heads, batch, width, window, chunks):
+    """Chunks of rows written into a ring and attended as they go, planes at different cursors: device against oracle on
+    the same cache bytes, before the ring wraps, as it wraps inside a chunk, and several turns in."""
+    rng = np.random.default_rng(29)
+    widest = max(chunks)
+    capacity = window + widest
+    scale = 1.0 / np.sqrt(width)
+    K = np.zeros((kv_heads, batch, capacity, width), dtype=np.uint16)
+    V = np.zeros_like(K)
+    origins = np.array([0] + [3 * b + 2 for b in range(1, batch)], dtype=np.uint32)
+    for rows in chunks:
+        k = rng.standard_normal((kv_heads, batch, rows, width)).astype(np.float32)
+        v = rng.standard_normal((kv_heads, batch, rows, width)).astype(np.float32)
+        q = rng.standard_normal((heads, batch, rows, width)).astype(np.float32)
+        for b in range(batch):
+            for row in range(rows):
+                K[:, b, (origins[b] + row) % window] = oracle.f32_to_f16(k[:, b, row])
+                V[:, b, (origins[b] + row) % window] = oracle.f32_to_f16(v[:, b, row])
+        ck, cv = device.upload(K), device.upload(V)
+        got = device.attention(q, ck, cv, kv_heads, capacity, window, origins, scale, reach=window)
+        want = oracle.attention(q, K, V, kv_heads, capacity, window, origins, scale, reach=window)
+        assert np.abs(got - want).max() <= 1e-5, (rows, origins)
+        # the device's own ring write lands on the same slots
+        dk, dv = device.upload(np.zeros_like(K)), device.upload(np.zeros_like(V))
+        device.cache_write(k, v, dk, dv, capacity, window, origins, ring=True)
+        mine = dk.numpy(np.uint16, K.shape)
+        for b in range(batch):
+            for row in range(rows):
+                if origins[b] + row + window >= origins[b] + rows:  # not overwritten by a later row of the same chunk
+                    assert np.array_equal(mine[:, b, (origins[b] + row) % window], oracle.f32_to_f16(k[:, b, row]))
+        ck.release(), cv.release(), dk.release(), dv.release()
+        origins = origins + rows
+
+
 def test_attention_refuses_a_cursor_past_its_keys(device):
     q = np.zeros((2, 1, 1, 64), dtype=np.float32)
     K = np.zeros((2, 1, 8, 64), dtype=np.uint16)

@@ -115,6 +115,59 @@ def test_attention_over_equal_scores_is_the_running_mean_of_the_values():
             assert np.allclose(got[head, 0, 0], V[head // 2, 0, : origin + 1].mean(axis=0), atol=1e-6)
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_a_ring_weighs_the_last_window_of_keys(half):
+    # crates/neura-decoder/tests/cache.rs:11-51: equal scores, value = step -> the mean of the last WINDOW steps
+    WINDOW, CAPACITY, WIDTH = 5, 7, 2
+    K = np.zeros((1, 1, CAPACITY, WIDTH), dtype=np.float32)
+    V = np.zeros((1, 1, CAPACITY, WIDTH), dtype=np.float32)
+    q = np.array([1.0, 0.0], dtype=np.float32).reshape(1, 1, 1, WIDTH)
+    for step in range(2 * WINDOW + 3):
+        K[0, 0, step % WINDOW] = [1.0, 0.0]
+        V[0, 0, step % WINDOW] = [float(step), 0.0]
+        if half:
+            got = oracle.attention(q, K.astype(np.float16).view(np.uint16), V.astype(np.float16).view(np.uint16), 1, CAPACITY, WINDOW, [step], 1.0, reach=WINDOW)
+        else:
+            got = oracle.attention(q, K, V, 1, CAPACITY, WINDOW, [step], 1.0, reach=WINDOW)
+        first = max(0, step - (WINDOW - 1))
+        expected = sum(range(first, step + 1)) / (step - first + 1)
+        assert abs(got[0, 0, 0, 0] - expected) < 1e-5 and got[0, 0, 0, 1] == 0.0, (step, got)
+
+
+def test_a_ring_equals_attention_over_the_positions_it_still_holds():
+    # An independent reading of the ring: keep every position ever written; the query at position p weighs positions
+    # p - reach + 1 .. p that no later row of the same chunk has overwritten (position j leaves when j + window is written).
+    rng = np.random.default_rng(31)
+    heads, kv_heads, width, window, capacity = 4, 2, 8, 6, 9
+    scale = 1.0 / np.sqrt(width)
+    K = np.zeros((kv_heads, 1, capacity, width), dtype=np.float32)
+    V = np.zeros_like(K)
+    history_k, history_v = [], []
+    origin = 0
+    for rows in (1, 3, 2, 6, 1, 1, 4, 5, 2):
+        k = rng.standard_normal((kv_heads, rows, width)).astype(np.float32)
+        v = rng.standard_normal((kv_heads, rows, width)).astype(np.float32)
+        q = rng.standard_normal((heads, 1, rows, width)).astype(np.float32)
+        for row in range(rows):
+            K[:, 0, (origin + row) % window] = k[:, row]
+            V[:, 0, (origin + row) % window] = v[:, row]
+            history_k.append(k[:, row])
+            history_v.append(v[:, row])
+        got = oracle.attention(q, K, V, kv_heads, capacity, window, [origin], scale, reach=window)
+        written = origin + rows
+        for head in range(heads):
+            for row in range(rows):
+                position = origin + row
+                seen = [j for j in range(max(0, position - window + 1), position + 1) if j + window >= written]
+                keys = np.array([history_k[j][head // 2] for j in seen], dtype=np.float64)
+                values = np.array([history_v[j][head // 2] for j in seen], dtype=np.float64)
+                scores = keys @ q[head, 0, row].astype(np.float64) * scale
+                weights = np.exp(scores - scores.max())
+                want = (weights / weights.sum()) @ values
+                assert np.abs(got[head, 0, row] - want).max() <= 1e-5, (origin, rows, head, row)
+        origin += rows
+
+
 def test_argmax_breaks_ties_toward_the_lowest_index():
     assert oracle.argmax([1.0, 3.0, 3.0, 2.0]) == 1
     assert oracle.argmax([5.0]) == 0
