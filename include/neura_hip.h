@@ -238,6 +238,18 @@ int32_t nh_model_logits(nh_model *model, float *host_out);
 int32_t nh_model_cache_write(nh_model *model, uint32_t layer, int32_t value_not_key, const uint16_t *host_src);
 int32_t nh_model_cache_read(nh_model *model, uint32_t layer, int32_t value_not_key, uint16_t *host_dst);
 uint32_t nh_model_capacity(const nh_model *model);
+/* The shared prefix of a batch that declares one (Cache::with_shared / Cache::shared, crates/neura-decoder/src/cache.rs:71-90,
+ * :138-161; Batch::prefix, crates/neura-generate/src/batch.rs:885-994): one more plane of keys and values per layer,
+ * fp16 [kv_heads][1][capacity][head_dim], zero until kept.
+ * nh_model_keep_prefix: the shared plane becomes a copy of plane `plane` -- the prefix program's result, once the caller has
+ *   fed the prefix to that plane with nh_prefill / nh_decode_step while no plane holds a sequence.
+ * nh_model_reset_shared: the reset program with its share input (cache.rs:223-250, batch.rs:1094-1100): a plane whose share
+ *   byte is set becomes a copy of the shared plane, else a plane whose reset byte is set is zeroed.
+ * nh_model_shared_write / _read: Runtime::restore_state / save_state of "blk.{i}.cache.shared.key|value". */
+int32_t nh_model_keep_prefix(nh_model *model, uint32_t plane);
+int32_t nh_model_reset_shared(nh_model *model, const uint8_t *reset, const uint8_t *share, uint32_t batch);
+int32_t nh_model_shared_write(nh_model *model, uint32_t layer, int32_t value_not_key, const uint16_t *host_src);
+int32_t nh_model_shared_read(nh_model *model, uint32_t layer, int32_t value_not_key, uint16_t *host_dst);
 
 #ifdef __cplusplus
 }

@@ -77,6 +77,10 @@ SIGNATURES = {
     "nh_model_logits": (c_int32, [c_void_p, c_void_p]),
     "nh_model_cache_write": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
     "nh_model_cache_read": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
+    "nh_model_keep_prefix": (c_int32, [c_void_p, c_uint32]),
+    "nh_model_reset_shared": (c_int32, [c_void_p, POINTER(c_uint8), POINTER(c_uint8), c_uint32]),
+    "nh_model_shared_write": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
+    "nh_model_shared_read": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
     "nh_model_capacity": (c_uint32, [c_void_p]),
 }
 

@@ -26,6 +26,9 @@ struct nh_model {
     std::vector<const float *> bias_q, bias_k, bias_v;  // per layer, nullptr where a projection has none
     std::vector<uint16_t *> cache_k, cache_v;
     size_t cache_elements = 0;  // per layer and per K or V
+    // the shared prefix (Cache::with_shared, crates/neura-decoder/src/cache.rs:138-161): one plane per layer,
+    // [kv_heads][1][capacity][head_dim], allocated when a prefix is first kept
+    std::vector<uint16_t *> shared_k, shared_v;
     // activations; T = rows * batch flattened token rows, t = row * batch + plane
     float *h = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr, *act = nullptr, *up = nullptr, *logits = nullptr;
     float *rope_cos = nullptr, *rope_sin = nullptr;  // [capacity][head_dim / 2], for the rotation folded into the q|k|v product
@@ -52,6 +55,8 @@ void release(nh_model *m) {
         if (graph) (void)hipGraphExecDestroy(graph);
     for (auto p : m->cache_k) (void)hipFree(p);
     for (auto p : m->cache_v) (void)hipFree(p);
+    for (auto p : m->shared_k) (void)hipFree(p);
+    for (auto p : m->shared_v) (void)hipFree(p);
     float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits, m->rope_cos, m->rope_sin};
     for (float *p : buffers)
         if (p) (void)hipFree(p);
@@ -534,6 +539,73 @@ int32_t nh_model_reset(nh_model *m, const uint8_t *reset, uint32_t batch) {
                 NH_HIP(hipMemsetAsync(m->cache_v[L] + at, 0, plane * 2, m->d->stream));
             }
     return NH_OK;
+}
+
+// the shared planes, zeroed, on first use
+static int32_t shared_planes(nh_model *m) {
+    if (!m->shared_k.empty()) return NH_OK;
+    const size_t bytes = (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2;
+    for (uint32_t L = 0; L < m->c.layers; L++) {
+        uint16_t *k = nullptr, *v = nullptr;
+        if (hipMalloc((void **)&k, bytes) != hipSuccess || hipMalloc((void **)&v, bytes) != hipSuccess) {
+            if (k) (void)hipFree(k);
+            return fail(NH_E_MEMORY, "no room for the %zu bytes a shared prefix of layer %u holds", 2 * bytes, L);
+        }
+        m->shared_k.push_back(k), m->shared_v.push_back(v);
+        NH_HIP(hipMemsetAsync(k, 0, bytes, m->d->stream));
+        NH_HIP(hipMemsetAsync(v, 0, bytes, m->d->stream));
+    }
+    return NH_OK;
+}
+
+int32_t nh_model_keep_prefix(nh_model *m, uint32_t plane_index) {
+    NH_REQUIRE(m && plane_index < m->c.batch, "a prefix is kept from a plane of the model");
+    int32_t status = shared_planes(m);
+    if (status != NH_OK) return status;
+    const size_t plane = (size_t)m->capacity * m->c.head_dim;
+    for (uint32_t L = 0; L < m->c.layers; L++)
+        for (uint32_t head = 0; head < m->c.kv_heads; head++) {
+            const size_t from = ((size_t)head * m->c.batch + plane_index) * plane, to = (size_t)head * plane;
+            NH_HIP(hipMemcpyAsync(m->shared_k[L] + to, m->cache_k[L] + from, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+            NH_HIP(hipMemcpyAsync(m->shared_v[L] + to, m->cache_v[L] + from, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+        }
+    return NH_OK;
+}
+
+int32_t nh_model_reset_shared(nh_model *m, const uint8_t *reset, const uint8_t *share, uint32_t batch) {
+    NH_REQUIRE(m && reset && share && batch == m->c.batch, "a reset names no model, no flags or another plane count");
+    bool any = false;
+    for (uint32_t b = 0; b < batch; b++) any |= share[b] != 0;
+    int32_t status = any ? shared_planes(m) : NH_OK;
+    if (status != NH_OK) return status;
+    const size_t plane = (size_t)m->capacity * m->c.head_dim;
+    for (uint32_t L = 0; L < m->c.layers; L++)
+        for (uint32_t head = 0; head < m->c.kv_heads; head++)
+            for (uint32_t b = 0; b < batch; b++) {
+                const size_t at = ((size_t)head * batch + b) * plane;
+                if (share[b]) {  // select(share, prefix, blank): the prefix wins over the reset (cache.rs:231-238)
+                    NH_HIP(hipMemcpyAsync(m->cache_k[L] + at, m->shared_k[L] + (size_t)head * plane, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+                    NH_HIP(hipMemcpyAsync(m->cache_v[L] + at, m->shared_v[L] + (size_t)head * plane, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+                } else if (reset[b]) {
+                    NH_HIP(hipMemsetAsync(m->cache_k[L] + at, 0, plane * 2, m->d->stream));
+                    NH_HIP(hipMemsetAsync(m->cache_v[L] + at, 0, plane * 2, m->d->stream));
+                }
+            }
+    return NH_OK;
+}
+
+int32_t nh_model_shared_write(nh_model *m, uint32_t layer, int32_t value_not_key, const uint16_t *host_src) {
+    NH_REQUIRE(m && host_src && layer < m->c.layers, "a shared prefix write names no model, no bytes or no layer %u", layer);
+    int32_t status = shared_planes(m);
+    if (status != NH_OK) return status;
+    return nh_upload(m->d, value_not_key ? m->shared_v[layer] : m->shared_k[layer], host_src, (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2);
+}
+
+int32_t nh_model_shared_read(nh_model *m, uint32_t layer, int32_t value_not_key, uint16_t *host_dst) {
+    NH_REQUIRE(m && host_dst && layer < m->c.layers, "a shared prefix read names no model, no bytes or no layer %u", layer);
+    int32_t status = shared_planes(m);
+    if (status != NH_OK) return status;
+    return nh_download(m->d, host_dst, value_not_key ? m->shared_v[layer] : m->shared_k[layer], (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2);
 }
 
 int32_t nh_model_logits(nh_model *m, float *host_out) {

@@ -54,9 +54,11 @@ SIGNATURES = {
     "nhost_payload_bytes": (c_uint64, [c_int32, c_uint64]),
     "nhost_runtime_open": (c_void_p, [c_int32]),
     "nhost_runtime_close": (None, [c_void_p]),
-    "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32]),
+    "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32, c_int32]),
     "nhost_batch_open_sampled": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_float, c_uint32, c_float,
-                                            c_uint32]),
+                                            c_uint32, c_int32]),
+    "nhost_batch_prefix": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
+    "nhost_batch_forget_prefix": (c_int32, [c_void_p]),
     "nhost_batch_window_check": (c_int32, [c_uint32]),
     "nhost_batch_window": (c_int64, [c_void_p]),
     "nhost_sampling_check": (c_int32, [c_float, c_uint32, c_float]),
@@ -424,19 +426,21 @@ class Batch:
     """A Qwen2 GGUF loaded onto a runtime with a generation batch above it: greedy, or drawing with
     `sampling` = (temperature, keep, cumulative) as BatchSpec::sampled(Sampling::sampled(..)) does."""
 
-    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None, window=None):
-        """`window`: BatchSpec::window -- the caches are rings of that many tokens and a sequence attends to its last `window`"""
+    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None, window=None, shared=False):
+        """`window`: BatchSpec::window -- the caches are rings of that many tokens and a sequence attends to its last `window`;
+        `shared`: BatchSpec::shared -- the batch can keep one prefix (`prefix`) every prompt then starts from"""
         held, count = _words(chunks)
         self.planes = batch
         self.vocabulary = vocabulary
         if window is not None and library().nhost_batch_window_check(window) != 0:
             raise _refused()
         if sampling is None:
-            self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count, window or 0)
+            self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count, window or 0,
+                                                     1 if shared else 0)
         else:
             temperature, keep, cumulative = sampling
             self.handle = library().nhost_batch_open_sampled(runtime.handle, archive.handle, vocabulary, context, batch, held, count,
-                                                             temperature, keep, cumulative, window or 0)
+                                                             temperature, keep, cumulative, window or 0, 1 if shared else 0)
         if not self.handle:
             raise _refused()
 
@@ -515,6 +519,14 @@ class Batch:
 
     def window(self):
         return self._status(library().nhost_batch_window(self.handle))
+
+    def prefix(self, tokens):
+        """Batch::prefix (crates/neura-generate/src/batch.rs:885-994)"""
+        held, count = _words(tokens)
+        self._status(library().nhost_batch_prefix(self.handle, held, count))
+
+    def forget_prefix(self):
+        self._status(library().nhost_batch_forget_prefix(self.handle))
 
     def remaining(self, slot):
         left = library().nhost_batch_remaining(self.handle, slot)

@@ -192,16 +192,17 @@ void *nhost_runtime_open(int32_t index) {
 void nhost_runtime_close(void *runtime) { delete static_cast<runtime::Runtime *>(runtime); }
 
 // BatchSpec::new(context, batch, chunks), and .window(window) when window is not 0
-static generate::BatchSpec spec_of(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count, uint32_t window) {
+static generate::BatchSpec spec_of(uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count, uint32_t window, int32_t shared = 0) {
     generate::BatchSpec spec(context, batch, std::vector<uint32_t>(chunks, chunks + count));
+    if (shared) spec = spec.shared();
     return window ? spec.window(window) : spec;
 }
 // a Qwen2 GGUF (whole or file) becomes a model and a greedy batch over it
 void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
-                       uint32_t window) {
+                       uint32_t window, int32_t shared) {
     return guarded([&]() -> void * {
         auto *opened = static_cast<Opened *>(held);
-        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window);
+        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window, shared);
         auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
         auto out = std::make_unique<Loaded>();
         out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
@@ -211,10 +212,10 @@ void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t 
 }
 // the same with a sampled answer (BatchSpec::sampled(Sampling::sampled(temperature, keep, cumulative)))
 void *nhost_batch_open_sampled(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
-                               float temperature, uint32_t keep, float cumulative, uint32_t window) {
+                               float temperature, uint32_t keep, float cumulative, uint32_t window, int32_t shared) {
     return guarded([&]() -> void * {
         auto *opened = static_cast<Opened *>(held);
-        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window).sampled(generate::Sampling::sampled(temperature, keep, cumulative));
+        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window, shared).sampled(generate::Sampling::sampled(temperature, keep, cumulative));
         auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
         auto out = std::make_unique<Loaded>();
         out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec);
@@ -274,6 +275,13 @@ int32_t nhost_batch_spec_check(uint32_t context, uint32_t batch, const uint32_t 
 // BatchSpec::window's own refusal
 int32_t nhost_batch_window_check(uint32_t window) {
     return guarded([&] { return generate::BatchSpec(8, 1, {}).window(window), 0; }, -1);
+}
+// Batch::prefix / forget_prefix (crates/neura-generate/src/batch.rs:885-998)
+int32_t nhost_batch_prefix(void *held, const uint32_t *tokens, uint32_t count) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->prefix(std::vector<uint32_t>(tokens, tokens + count)), 0; }, -1);
+}
+int32_t nhost_batch_forget_prefix(void *held) {
+    return guarded([&] { return static_cast<Loaded *>(held)->batch->forget_prefix(), 0; }, -1);
 }
 int64_t nhost_batch_window(void *held) {
     return guarded([&]() -> int64_t { return (int64_t) static_cast<Loaded *>(held)->batch->window(); }, -1);

@@ -805,7 +805,7 @@ struct Config {
     }
 };
 
-// crates/neura-generate/src/batch.rs:110-153 (tuning and sharing are not built)
+// crates/neura-generate/src/batch.rs:110-153 (tuning is not built: there is no compiler to tune)
 // crates/neura-generate/src/sampling.rs:3-57: a batch answers with the largest logit, or draws among the `keep` largest
 // cut at a cumulative mass after dividing the logits by a temperature
 struct Sampling {
@@ -835,6 +835,12 @@ struct BatchSpec {
     std::vector<uint32_t> chunks;
     Sampling sampling;
     std::optional<uint32_t> window_tokens;  // BatchSpec::window: the caches are rings of that many tokens
+    bool shares = false;                    // BatchSpec::shared: the planes can start from one prefix fed once
+    BatchSpec shared() const {              // crates/neura-generate/src/batch.rs:143-146
+        BatchSpec out = *this;
+        out.shares = true;
+        return out;
+    }
     BatchSpec(uint32_t context, uint32_t batch, std::vector<uint32_t> chunks) : context(context), batch(batch), chunks(std::move(chunks)) {}
     BatchSpec window(uint32_t tokens) const {  // crates/neura-generate/src/batch.rs:148-152
         NEURA_ASSERT(tokens > 0, "a batch keeps a window of no token");
@@ -1104,7 +1110,7 @@ class Batch {
     }
     Batch(Model &model, BatchSpec spec)
         : model_(model), batch_(spec.batch), context_(spec.context), window_(spec.window_tokens.value_or(spec.context)), chunks_(spec.chunks),
-          slots_(spec.batch), seeded_(!spec.sampling.greedy),
+          slots_(spec.batch), shared_(spec.shares), seeded_(!spec.sampling.greedy),
           temperatures_(spec.batch, spec.sampling.temperature), keeps_(spec.batch, spec.sampling.keep), cumulatives_(spec.batch, spec.sampling.cumulative) {
         validate(spec);
         for (uint32_t slot = 0; slot < batch_; slot++) seeds_.push_back(plane_seed(0, slot));  // batch.rs:426-428
@@ -1179,11 +1185,56 @@ class Batch {
         NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot);
         NEURA_ASSERT(!tokens.empty(), "a batch admits a prompt of at least one token");
         NEURA_ASSERT(tokens.size() < context_, "the prompt holds %zu tokens where this batch holds %u of context", tokens.size(), context_);
-        std::vector<uint8_t> reset(batch_, 0);
+        std::vector<uint8_t> reset(batch_, 0), share(batch_, 0);
         reset[slot] = 1;
-        runtime::check(nh_model_reset(model_.handle(), reset.data(), batch_));
-        slots_[slot] = Slot{0, Prompting, std::deque<uint32_t>(tokens.begin(), tokens.end()), 0};
+        size_t fed = 0;
+        if (prefix_) {  // batch.rs:1076-1093: the plane starts from the keys and values the prefix left, at the cursor behind it
+            NEURA_ASSERT(tokens.size() >= prefix_->size() && std::equal(prefix_->begin(), prefix_->end(), tokens.begin()),
+                         "a batch shares a prefix of %zu tokens, and this prompt does not start with it", prefix_->size());
+            NEURA_ASSERT(tokens.size() > prefix_->size(), "a prompt of %zu tokens holds no token after the shared prefix of %zu tokens", tokens.size(),
+                         prefix_->size());
+            fed = prefix_->size(), share[slot] = 1;
+        }
+        if (shared_)
+            runtime::check(nh_model_reset_shared(model_.handle(), reset.data(), share.data(), batch_));
+        else
+            runtime::check(nh_model_reset(model_.handle(), reset.data(), batch_));
+        slots_[slot] = Slot{(uint32_t)fed, Prompting, std::deque<uint32_t>(tokens.begin() + (std::ptrdiff_t)fed, tokens.end()), 0};
     }
+    // Batch::prefix (batch.rs:885-994): the tokens every prompt of this batch will start with, fed once -- in the largest
+    // chunk while it fits, then token by token -- into the shared plane the reset copies into a plane that starts a sequence
+    void prefix(const std::vector<uint32_t> &tokens) {
+        NEURA_ASSERT(shared_, "a batch fills a shared prefix only when it declares one");
+        for (const auto &slot : slots_) NEURA_ASSERT(!slot.has_value(), "a batch fills a shared prefix while no plane holds a sequence");
+        NEURA_ASSERT(!tokens.empty(), "a shared prefix holds at least one token");
+        NEURA_ASSERT(tokens.size() < context_,
+                     "a shared prefix holds %zu tokens where this batch holds %u of context, and the prompt after it holds at least one token",
+                     tokens.size(), context_);
+        if (prefix_ && *prefix_ == tokens) return;
+        // no plane holds a sequence: plane 0 stands in for the one-plane program the reference compiles for the prefix
+        std::vector<uint8_t> reset(batch_, 0), mask(batch_, 0);
+        reset[0] = 1, mask[0] = 1;
+        runtime::check(nh_model_reset(model_.handle(), reset.data(), batch_));
+        const uint32_t bulk = chunks_.empty() ? 1 : chunks_.front();
+        size_t at = 0;
+        std::vector<uint32_t> cursors(batch_, 0), chosen(batch_, 0);
+        while (bulk > 1 && tokens.size() - at >= bulk) {
+            std::vector<uint32_t> rows((size_t)bulk * batch_, 0);
+            for (uint32_t row = 0; row < bulk; row++) rows[(size_t)row * batch_] = tokens[at + row];
+            cursors[0] = (uint32_t)at;
+            runtime::check(nh_prefill(model_.handle(), rows.data(), bulk, cursors.data(), mask.data(), batch_));
+            at += bulk;
+        }
+        for (; at < tokens.size(); at++) {
+            std::vector<uint32_t> row(batch_, 0);
+            row[0] = tokens[at], cursors[0] = (uint32_t)at;
+            runtime::check(nh_decode_step(model_.handle(), row.data(), cursors.data(), mask.data(), batch_, chosen.data()));
+        }
+        runtime::check(nh_model_keep_prefix(model_.handle(), 0));
+        prefix_ = tokens;
+    }
+    void forget_prefix() { prefix_.reset(); }  // batch.rs:996-998
+    const std::optional<std::vector<uint32_t>> &shared_prefix() const { return prefix_; }
     void resume(uint32_t slot, const std::vector<uint32_t> &tokens) {  // batch.rs:1015-1054
         auto &held = slots_.at(slot);
         NEURA_ASSERT(held.has_value(), "plane %u of this batch holds no sequence", slot);
@@ -1231,6 +1282,7 @@ class Batch {
     BatchSnapshot snapshot() const {
         BatchSnapshot out;
         out.batch = batch_, out.context = context_, out.window = window_, out.sampled = seeded_;
+        out.prefix = prefix_;
         for (const auto &slot : slots_) {
             if (!slot) {
                 out.slots.push_back(std::nullopt);
@@ -1250,7 +1302,7 @@ class Batch {
         NEURA_ASSERT(snapshot.sampled == seeded_, "a batch draws %s restores a snapshot of a batch that draws %s", seeded_ ? "true" : "false",
                      snapshot.sampled ? "true" : "false");
         NEURA_ASSERT(snapshot.slots.size() == batch_, "a snapshot of %u planes holds %zu slots", batch_, snapshot.slots.size());
-        NEURA_ASSERT(!snapshot.prefix, "a snapshot holds a shared prefix where this batch declares none");
+        NEURA_ASSERT(!snapshot.prefix || shared_, "a snapshot holds a shared prefix where this batch declares none");
         NEURA_ASSERT(snapshot.state_names.empty(), "a snapshot names %zu states where this batch registers 0", snapshot.state_names.size());
         NEURA_ASSERT(snapshot.states.size() == snapshot.state_names.size(), "a snapshot names %zu states and holds %zu of them",
                      snapshot.state_names.size(), snapshot.states.size());
@@ -1269,6 +1321,7 @@ class Batch {
         }
         seeds_ = snapshot.seeds, temperatures_ = snapshot.temperatures, cumulatives_ = snapshot.cumulatives;
         for (uint32_t slot = 0; slot < batch_; slot++) keeps_[slot] = (uint32_t)snapshot.keeps[slot];
+        prefix_ = snapshot.prefix;  // batch.rs:621
     }
     // The device side of a batch between steps: the key and value states of every layer, written as the container the
     // reference's Runtime::save_state writes (crates/neura-runtime/src/checkpoint/container.rs:129-246: an 8-byte
@@ -1276,20 +1329,13 @@ class Batch {
     // the layout of a safetensors file).  States are named as the decoder's caches name them (blk.N.cache.key / .value,
     // crates/neura-decoder/src/cache.rs:136-137) and shaped [key heads, planes, capacity, width] in half storage.
     void save_state(const std::string &path) const {
-        const Config &c = model_.config();
-        const uint32_t capacity = nh_model_capacity(model_.handle());
-        const size_t elements = (size_t)c.key_heads * batch_ * capacity * c.head_width;
-        std::vector<std::string> names;
-        for (uint32_t layer = 0; layer < c.layers; layer++)
-            for (const char *which : {"key", "value"}) names.push_back("blk." + std::to_string(layer) + ".cache." + which);
-        std::sort(names.begin(), names.end());  // one storage width: the header orders by name
+        const std::vector<State> states = device_states();
         std::string header = "{";
         size_t at = 0;
-        for (size_t i = 0; i < names.size(); i++) {
+        for (size_t i = 0; i < states.size(); i++) {
             if (i) header += ',';
-            header += '"' + names[i] + "\":{\"dtype\":\"F16\",\"shape\":[" + std::to_string(c.key_heads) + ',' + std::to_string(batch_) + ',' +
-                      std::to_string(capacity) + ',' + std::to_string(c.head_width) + "],\"data_offsets\":[" + std::to_string(at) + ',';
-            at += elements * 2;
+            header += '"' + states[i].name + "\":{\"dtype\":\"F16\",\"shape\":" + states[i].shape + ",\"data_offsets\":[" + std::to_string(at) + ',';
+            at += states[i].elements * 2;
             header += std::to_string(at) + "]}";
         }
         header += '}';
@@ -1299,22 +1345,20 @@ class Batch {
         const uint64_t length = header.size();
         for (int k = 0; k < 8; k++) out.put((char)(length >> (8 * k)));
         out.write(header.data(), (std::streamsize)header.size());
-        std::vector<uint16_t> held(elements);
-        for (const std::string &name : names) {
-            uint32_t layer;
-            bool value;
-            parse_state_name(name, layer, value);
-            runtime::check(nh_model_cache_read(model_.handle(), layer, value ? 1 : 0, held.data()));
-            out.write(reinterpret_cast<const char *>(held.data()), (std::streamsize)(elements * 2));
+        std::vector<uint16_t> held;
+        for (const State &state : states) {
+            held.resize(state.elements);
+            if (state.shared)
+                runtime::check(nh_model_shared_read(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
+            else
+                runtime::check(nh_model_cache_read(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
+            out.write(reinterpret_cast<const char *>(held.data()), (std::streamsize)(state.elements * 2));
         }
         out.flush();
         if (!out) panic("a container at %s could not be written", path.c_str());
     }
     // Batch::restore_state (batch.rs:519-532): the device states out of a container, then the host bookkeeping
     void restore_state(const std::string &path, const BatchSnapshot &snapshot) {
-        const Config &c = model_.config();
-        const uint32_t capacity = nh_model_capacity(model_.handle());
-        const size_t elements = (size_t)c.key_heads * batch_ * capacity * c.head_width;
         std::ifstream in(path, std::ios::binary);
         if (!in) panic("a container at %s could not be opened", path.c_str());
         uint8_t framed[8];
@@ -1326,31 +1370,33 @@ class Batch {
         std::string header(length, ' ');
         in.read(header.data(), (std::streamsize)length);
         NEURA_ASSERT((uint64_t)in.gcount() == length, "a container at %s ends inside its header", path.c_str());
-        const std::string shape = "[" + std::to_string(c.key_heads) + ',' + std::to_string(batch_) + ',' + std::to_string(capacity) + ',' +
-                                  std::to_string(c.head_width) + "]";
-        std::vector<uint16_t> held(elements);
-        for (uint32_t layer = 0; layer < c.layers; layer++)
-            for (int value = 0; value < 2; value++) {
-                const std::string name = "blk." + std::to_string(layer) + ".cache." + (value ? "value" : "key");
-                const size_t found = header.find('"' + name + "\":{");
-                NEURA_ASSERT(found != std::string::npos, "the container at %s holds no state named %s", path.c_str(), name.c_str());
-                const size_t close = header.find('}', found);
-                const std::string entry = compact(header.substr(found, close - found));
-                NEURA_ASSERT(entry.find("\"dtype\":\"F16\"") != std::string::npos, "state %s of the container at %s is not in half storage", name.c_str(),
-                             path.c_str());
-                NEURA_ASSERT(entry.find("\"shape\":" + shape) != std::string::npos, "state %s of the container at %s is not shaped %s", name.c_str(),
-                             path.c_str(), shape.c_str());
-                const size_t offsets = entry.find("\"data_offsets\":[");
-                NEURA_ASSERT(offsets != std::string::npos, "state %s of the container at %s names no bytes", name.c_str(), path.c_str());
-                const uint64_t begin = std::stoull(entry.substr(offsets + 16));
-                const uint64_t end = std::stoull(entry.substr(entry.find(',', offsets + 16) + 1));
-                NEURA_ASSERT(end - begin == elements * 2, "state %s of the container at %s holds %llu bytes where the cache holds %zu", name.c_str(),
-                             path.c_str(), (unsigned long long)(end - begin), elements * 2);
-                in.seekg((std::streamoff)(8 + length + begin));
-                in.read(reinterpret_cast<char *>(held.data()), (std::streamsize)(elements * 2));
-                NEURA_ASSERT((size_t)in.gcount() == elements * 2, "the container at %s ends inside state %s", path.c_str(), name.c_str());
-                runtime::check(nh_model_cache_write(model_.handle(), layer, value, held.data()));
-            }
+        std::vector<uint16_t> held;
+        for (const State &state : device_states()) {
+            const std::string &name = state.name;
+            const size_t elements = state.elements;
+            const size_t found = header.find('"' + name + "\":{");
+            NEURA_ASSERT(found != std::string::npos, "the container at %s holds no state named %s", path.c_str(), name.c_str());
+            const size_t close = header.find('}', found);
+            const std::string entry = compact(header.substr(found, close - found));
+            NEURA_ASSERT(entry.find("\"dtype\":\"F16\"") != std::string::npos, "state %s of the container at %s is not in half storage", name.c_str(),
+                         path.c_str());
+            NEURA_ASSERT(entry.find("\"shape\":" + state.shape) != std::string::npos, "state %s of the container at %s is not shaped %s", name.c_str(),
+                         path.c_str(), state.shape.c_str());
+            const size_t offsets = entry.find("\"data_offsets\":[");
+            NEURA_ASSERT(offsets != std::string::npos, "state %s of the container at %s names no bytes", name.c_str(), path.c_str());
+            const uint64_t begin = std::stoull(entry.substr(offsets + 16));
+            const uint64_t end = std::stoull(entry.substr(entry.find(',', offsets + 16) + 1));
+            NEURA_ASSERT(end - begin == elements * 2, "state %s of the container at %s holds %llu bytes where the cache holds %zu", name.c_str(),
+                         path.c_str(), (unsigned long long)(end - begin), elements * 2);
+            held.resize(elements);
+            in.seekg((std::streamoff)(8 + length + begin));
+            in.read(reinterpret_cast<char *>(held.data()), (std::streamsize)(elements * 2));
+            NEURA_ASSERT((size_t)in.gcount() == elements * 2, "the container at %s ends inside state %s", path.c_str(), name.c_str());
+            if (state.shared)
+                runtime::check(nh_model_shared_write(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
+            else
+                runtime::check(nh_model_cache_write(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
+        }
         restore(snapshot);
     }
 
@@ -1450,9 +1496,29 @@ class Batch {
     }
 
     void plane(uint32_t slot) const { NEURA_ASSERT(slot < batch_, "a batch of %u planes names no plane %u", batch_, slot); }
-    static void parse_state_name(const std::string &name, uint32_t &layer, bool &value) {  // blk.N.cache.key / blk.N.cache.value
-        layer = (uint32_t)std::stoul(name.substr(4));
-        value = name.size() >= 6 && name.compare(name.size() - 6, 6, ".value") == 0;
+    // the device states of this batch in the order a container holds them (one storage width: by name): blk.N.cache.key / .value,
+    // and blk.N.cache.shared.key / .value of one plane where the batch declares a shared prefix (cache.rs:136-137, :140-143)
+    struct State {
+        std::string name, shape;
+        uint32_t layer;
+        bool value, shared;
+        size_t elements;
+    };
+    std::vector<State> device_states() const {
+        const Config &c = model_.config();
+        const uint32_t capacity = nh_model_capacity(model_.handle());
+        std::vector<State> out;
+        for (uint32_t layer = 0; layer < c.layers; layer++)
+            for (int shared = 0; shared < (shared_ ? 2 : 1); shared++)
+                for (int value = 0; value < 2; value++) {
+                    const uint32_t planes = shared ? 1 : batch_;
+                    out.push_back(State{"blk." + std::to_string(layer) + ".cache." + (shared ? "shared." : "") + (value ? "value" : "key"),
+                                        "[" + std::to_string(c.key_heads) + ',' + std::to_string(planes) + ',' + std::to_string(capacity) + ',' +
+                                            std::to_string(c.head_width) + "]",
+                                        layer, value != 0, shared != 0, (size_t)c.key_heads * planes * capacity * c.head_width});
+                }
+        std::sort(out.begin(), out.end(), [](const State &a, const State &b) { return a.name < b.name; });
+        return out;
     }
     static std::string compact(const std::string &text) {  // a header entry without the blanks a writer may have put between its parts
         std::string out;
@@ -1469,6 +1535,8 @@ class Batch {
     uint32_t batch_, context_, window_;
     std::vector<uint32_t> chunks_;
     std::vector<std::optional<Slot>> slots_;
+    bool shared_ = false;
+    std::optional<std::vector<uint32_t>> prefix_;
     bool seeded_;
     std::vector<uint32_t> seeds_;
     std::vector<float> temperatures_;

@@ -287,6 +287,95 @@ def test_a_batch_restored_from_its_snapshot_and_state_file_answers_on(runtime, t
     archive.close()
 
 
+@pytest.mark.parametrize("chunks", [[], [4, 2]])
+@pytest.mark.parametrize("sampling", [None, (1.0, 4, 1.0)], ids=["greedy", "sampled"])
+def test_a_batch_reuses_the_prefix_its_planes_share(runtime, tmp_path, chunks, sampling):
+    """crates/neura-generate/tests/generation.rs:379-405: two prompts that start alike answer the same whether each feeds its
+    whole prompt or the batch keeps their common start as a shared prefix (fed once, copied into a plane as it starts);
+    the greedy answers are also the oracle's answers to the whole prompts."""
+    shape, element = SHAPE, NH_Q8_0
+    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=61)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    rng = np.random.default_rng(62)
+    common = list(rng.integers(0, shape["vocab"], 7))
+    prompts = [common + list(rng.integers(0, shape["vocab"], n)) for n in (3, 5)]
+
+    def batched(prefix):
+        batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, chunks, sampling=sampling, shared=prefix is not None)
+        if prefix is not None:
+            batch.prefix(prefix)
+            batch.prefix(prefix)  # the prefix it already keeps: nothing to do (batch.rs:913-915)
+        slots = [batch.admit(prompt) for prompt in prompts]
+        if prefix is not None:
+            assert [batch.cursor(slot) for slot in slots] == [len(prefix)] * 2
+        got = run(batch, {slot: 6 for slot in slots})
+        batch.close()
+        return [got[slot] for slot in slots]
+
+    plain = batched(None)
+    assert batched(common) == plain
+    if sampling is None:
+        assert plain == [alone(shape, element, tensors, prompt, 6)[0] for prompt in prompts]
+    archive.close()
+
+
+def test_a_shared_prefix_is_refused_where_the_reference_refuses_it_and_travels_in_a_state_file(runtime, tmp_path):
+    from safetensors.numpy import load_file
+
+    shape, element = SHAPE, NH_Q8_0
+    qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=63)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    rng = np.random.default_rng(64)
+    common = list(rng.integers(0, shape["vocab"], 9))
+    plain = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [4])
+    with pytest.raises(host.Panic, match="a batch fills a shared prefix only when it declares one"):  # batch.rs:895-898
+        plain.prefix(common)
+    plain.close()
+    first = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [4], shared=True)
+    with pytest.raises(host.Panic, match="a shared prefix holds at least one token"):
+        first.prefix([])
+    with pytest.raises(host.Panic, match="a shared prefix holds 96 tokens where this batch holds 96 of context"):
+        first.prefix([1] * CONTEXT)
+    first.prefix(common)
+    with pytest.raises(host.Panic, match="a batch shares a prefix of 9 tokens, and this prompt does not start with it"):  # batch.rs:1078-1082
+        first.admit([common[0] + 1] + common[1:] + [5])
+    with pytest.raises(host.Panic, match="a prompt of 9 tokens holds no token after the shared prefix of 9 tokens"):
+        first.admit(common)
+    first.admit(common + [5, 6, 7])
+    with pytest.raises(host.Panic, match="a batch fills a shared prefix while no plane holds a sequence"):  # batch.rs:899-902
+        first.prefix(common + [1])
+    first.admit(common + [8])
+    for _ in range(5):
+        first.step()
+    # the prefix and the shared plane travel with the snapshot and the state file
+    snapshot = first.snapshot()
+    assert host.snapshot_round_trip(snapshot) == snapshot
+    first.save_state(tmp_path / "state.safetensors")
+    held = load_file(str(tmp_path / "state.safetensors"))
+    assert sorted(held) == sorted("blk.%d.cache.%s%s" % (layer, shared, which) for layer in range(shape["layers"]) for shared in ("", "shared.")
+                                  for which in ("key", "value"))
+    capacity = CONTEXT + 4
+    assert held["blk.0.cache.shared.key"].shape == (shape["kv_heads"], 1, capacity, shape["head_dim"])
+    assert held["blk.1.cache.shared.value"][:, 0, :9].any() and not held["blk.1.cache.shared.value"][:, 0, 9:].any()
+    assert np.array_equal(held["blk.1.cache.key"][:, 1, :9], held["blk.1.cache.shared.key"][:, 0, :9])  # a plane started from it
+    second = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [4], shared=True)
+    second.restore_state(tmp_path / "state.safetensors", snapshot)
+    for batch in (first, second):
+        assert batch.admit(common + [11, 12]) == 2  # starts from the prefix the state file brought
+    want = run(first, {0: 6, 1: 6, 2: 6})
+    assert run(second, {0: 6, 1: 6, 2: 6}) == want
+    undeclared = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 3, [4])
+    with pytest.raises(host.Panic, match="a snapshot holds a shared prefix where this batch declares none"):  # batch.rs:564-567
+        undeclared.restore(snapshot)
+    # a forgotten prefix: prompts are whole again
+    second.finish(0)
+    second.forget_prefix()
+    assert second.admit([4, 5]) == 0 and second.cursor(0) == 0
+    for batch in (first, second, undeclared):
+        batch.close()
+    archive.close()
+
+
 def test_a_batch_keeps_the_planes_it_is_told_to(runtime, tmp_path):
     shape, element = SHAPE, NH_Q8_0
     tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=21)
