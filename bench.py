@@ -173,6 +173,15 @@ def extras(device, weights, shape, element, context, layers, rng):
     out["decode_batch8"] = {"value": batch * steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
                             "note": "8 planes, caches not pre-filled (zeros), cursors at the end of context %d" % context}
     model.release()
+    out["prefill_512"] = fill_512(device, weights, shape, element, context, layers, rng)
+    out["gemm_config3"] = gemm_config3(device, rng)
+    return out
+
+
+def fill_512(device, weights, shape, element, context, layers, rng):
+    """One 512-token prompt filled into an empty cache at cursor 0: a warm-up, then the mean of three."""
+    from neura_amd.loader import Model
+
     rows = 512
     model = Model(device, weights, shape, element, batch=1, context=context, max_rows=rows, layers=layers)
     prompt = rng.integers(0, shape["vocab"], rows)
@@ -185,13 +194,10 @@ def extras(device, weights, shape, element, context, layers, rng):
     device.sync()
     elapsed = (time.perf_counter() - began) / repeats
     per_layer = sum(2.0 * rows * n * k for _, n, k in __import__("neura_amd").synth.layer_matrices(shape))
-    out["prefill_512"] = {"value": rows / elapsed, "unit": "tokens/s", "ms": elapsed * 1e3,
-                          "product_tflops": layers * per_layer / elapsed / 1e12,
-                          "note": "one 512-row fill at cursor 0, all products on f16 MFMA with fp32 activations as (value, residue) half rows; "
-                                  "product_tflops counts 2*M*N*K of the products over the whole fill time"}
     model.release()
-    out["gemm_config3"] = gemm_config3(device, rng)
-    return out
+    return {"value": rows / elapsed, "unit": "tokens/s", "ms": elapsed * 1e3, "product_tflops": layers * per_layer / elapsed / 1e12,
+            "note": "one 512-row fill at cursor 0, all products on f16 MFMA with fp32 activations as (value, residue) half rows; "
+                    "product_tflops counts 2*M*N*K of the products over the whole fill time"}
 
 
 def main():
@@ -206,6 +212,7 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode, 512-token fill and wide-product measurements")
     parser.add_argument("--gemm-only", action="store_true", help="run only the wide product (M=512, K=3584, N=18944) and print its line")
+    parser.add_argument("--fill-only", action="store_true", help="run only the 512-token fill of the workload and print its line")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()
@@ -228,6 +235,11 @@ def main():
     tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers, elements=mixed, biases=biases))
     device = neura_amd.Device(0)
     weights = Weights(device, tensors)
+    if args.fill_only:
+        print(json.dumps({"prefill_512": fill_512(device, weights, shape, element, context, layers, rng)}))
+        weights.release()
+        device.close()
+        return
     model = Model(device, weights, shape, element, batch=1, context=context, layers=layers)
     # fp16 caches filled up to the context with N(0,1) halves
     for layer in range(layers):
