@@ -147,8 +147,18 @@ struct GemmArgs {
     float *Y;                // [M][ldy], the first N of every row are written
     const float *residual;   // [M][ldy] or nullptr
     uint32_t ldy;
+    // Optional, Q4_K on the matrix cores only (gemm_stacks() says when): two more matrices stacked along N behind W, as the
+    // narrow product stacks q|k|v.  end[s] = first output column past matrix s (end[2] == N); unused entries: W_more nullptr.
+    const void *W_more[2] = {nullptr, nullptr};
+    uint32_t end[2] = {0, 0};
+    // the activations were packed by the launch before this one (same X, M, K, nothing else launched on the device's
+    // scratch in between): skip the packing pass
+    bool packed = false;
 };
 int32_t launch_gemm(nh_device *d, const GemmArgs &args);
+// whether launch_gemm takes a product of this element and depth with matrices stacked along N at these boundaries, or with
+// activations the launch before packed
+bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1);
 // device scratch a Q4_K wide product over M rows of K activations packs them into
 size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows);
 

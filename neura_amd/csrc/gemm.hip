@@ -121,6 +121,8 @@ constexpr int GS = GK + 8;        // LDS row stride in halves: 144 B keeps 128-b
 
 struct GemmQ4Params {
     const uint8_t *W;
+    const uint8_t *W1, *W2;  // matrices stacked along N behind W: columns [end0, end1) and [end1, N); both ends are multiples of the tile
+    uint32_t end0, end1;
     uint32_t N, K, row_bytes;
     const _Float16 *A;   // [rows][K] halves, every four k in the order 0, 2, 1, 3; with `split`, row 2m is the rounded value of
                          // activation row m and row 2m+1 its residue * 2^11
@@ -230,7 +232,11 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
         // one row of each tile, one half (32 k) of the step
         const uint32_t tid = threadIdx.x - 256u;
         const uint32_t srow = tid >> 1, sh = tid & 1u;
-        const uint8_t *wrow = p.W + (size_t)min(n0 + srow, p.N - 1u) * p.row_bytes;
+        // a tile lies in one matrix: the boundaries between stacked matrices are multiples of the tile
+        const uint32_t column = min(n0 + srow, p.N - 1u);
+        const uint8_t *wrow = column < p.end0   ? p.W + (size_t)column * p.row_bytes
+                              : column < p.end1 ? p.W1 + (size_t)(column - p.end0) * p.row_bytes
+                                                : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
         const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
         u32x4 ahead, qs[4], av[4][4];  // the next super-block's header; groups and activations by slot = step % 4
         const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
@@ -414,6 +420,10 @@ size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows) {
 static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     GemmQ4Params p{};
     p.W = static_cast<const uint8_t *>(a.W);
+    p.W1 = static_cast<const uint8_t *>(a.W_more[0]), p.W2 = static_cast<const uint8_t *>(a.W_more[1]);
+    p.end0 = p.W1 ? a.end[0] : a.N, p.end1 = p.W2 ? a.end[1] : a.N;
+    if ((p.W1 && (p.end0 % GT || p.end0 > a.N)) || (p.W2 && (!p.W1 || p.end1 % GT || p.end1 < p.end0 || p.end1 > a.N)))
+        return fail(NH_E_ARGUMENT, "matrices stacked at columns %u and %u of %u do not fall on tiles of %d", a.end[0], a.end[1], a.N, GT);
     p.N = a.N;
     p.K = a.K;
     p.row_bytes = (uint32_t)payload_bytes(NH_Q4_K, a.K);
@@ -430,10 +440,13 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     if (!room) return NH_E_MEMORY;
     _Float16 *A = reinterpret_cast<_Float16 *>(room), *S = reinterpret_cast<_Float16 *>(room + halves);
     float *unscale = reinterpret_cast<float *>(room + halves + sums);
-    if (half_rows)
+    if (a.packed) {
+        // what the launch before left in the scratch is this launch's operand
+    } else if (half_rows) {
         hipLaunchKernelGGL(gemm_pack_rows_kernel<true>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
-    else
+    } else {
         hipLaunchKernelGGL(gemm_pack_rows_kernel<false>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
+    }
     NH_HIP(hipGetLastError());
     p.A = A, p.S = S, p.unscale = unscale;
     static bool sized = false;
@@ -447,14 +460,26 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     return NH_OK;
 }
 
+// the matrix-core form takes Q4_K rows of whole super-blocks read from 16-byte aligned addresses
+static bool mfma_takes(int32_t element, uint32_t K, const void *X, const void *W) {
+    const char *held = getenv("NEURA_HIP_GEMM_MFMA");
+    const bool wanted = !(held && held[0] == '0');
+    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & 15u) == 0;
+    return wanted && aligned && element == NH_Q4_K && K % 256u == 0;
+}
+
+bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1) {
+    if (!mfma_takes(element, K, X, W0)) return false;
+    if (W1 && (((uintptr_t)W1 & 15u) || end0 % GT)) return false;
+    if (W2 && (((uintptr_t)W2 & 15u) || end1 % GT || !W1)) return false;
+    return true;
+}
+
 int32_t launch_gemm(nh_device *d, const GemmArgs &a) {
     if (!a.M || !a.N) return NH_OK;
-    {
-        const char *held = getenv("NEURA_HIP_GEMM_MFMA");
-        const bool wanted = !(held && held[0] == '0');
-        const bool aligned = ((uintptr_t)a.X & 15u) == 0 && ((uintptr_t)a.W & 15u) == 0;
-        if (wanted && aligned && a.element == NH_Q4_K && a.K % 256u == 0) return launch_gemm_q4k_mfma(d, a);
-    }
+    if (mfma_takes(a.element, a.K, a.X, a.W)) return launch_gemm_q4k_mfma(d, a);
+    if (a.W_more[0] || a.W_more[1] || a.packed)
+        return fail(NH_E_ARGUMENT, "this wide product stacks no matrices and reuses no packed activations (ask gemm_stacks first)");
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM), block(256);
     uint32_t row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     const uint8_t *W = static_cast<const uint8_t *>(a.W);

@@ -126,12 +126,24 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
             const float *biases[3] = {m->bias_q[L], m->bias_k[L], m->bias_v[L]};
             const uint32_t widths[3] = {QW, KW, KW};
+            const bool alike = element_at(m, L, Q) == element_at(m, L, K_) && element_at(m, L, Q) == element_at(m, L, V);
             uint32_t column = 0;
-            for (int s = 0; s < 3; s++) {
-                GemmArgs g{element_at(m, L, Q + s), mats[s], widths[s], H, m->xn, NH_F32, T, m->qkv + column, nullptr, QKV};
+            if (alike && gemm_stacks(element_at(m, L, Q), H, m->xn, mats[0], mats[1], mats[2], QW, QW + KW)) {
+                // q|k|v as one product: the key and value projections alone are a few dozen workgroups each
+                GemmArgs g{element_at(m, L, Q), mats[0], QKV, H, m->xn, NH_F32, T, m->qkv, nullptr, QKV};
+                g.W_more[0] = mats[1], g.W_more[1] = mats[2], g.end[0] = QW, g.end[1] = QW + KW;
                 if ((status = launch_gemm(d, g)) != NH_OK) return status;
-                if (biases[s] && (status = launch_columns(d, m->qkv + column, QKV, biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
-                column += widths[s];
+                for (int s = 0; s < 3; s++) {
+                    if (biases[s] && (status = launch_columns(d, m->qkv + column, QKV, biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
+                    column += widths[s];
+                }
+            } else {
+                for (int s = 0; s < 3; s++) {
+                    GemmArgs g{element_at(m, L, Q + s), mats[s], widths[s], H, m->xn, NH_F32, T, m->qkv + column, nullptr, QKV};
+                    if ((status = launch_gemm(d, g)) != NH_OK) return status;
+                    if (biases[s] && (status = launch_columns(d, m->qkv + column, QKV, biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
+                    column += widths[s];
+                }
             }
         } else {
             const bool biased = m->bias_q[L] || m->bias_k[L] || m->bias_v[L];
@@ -203,6 +215,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             GemmArgs g{element_at(m, L, GATE), m->ffn_gate[L], F, H, m->xn, NH_F32, T, m->act, nullptr, F};
             GemmArgs u{element_at(m, L, UP), m->ffn_up[L], F, H, m->xn, NH_F32, T, m->up, nullptr, F};
             if ((status = launch_gemm(d, g)) != NH_OK) return status;
+            // the up projection multiplies the rows the gate projection just packed
+            u.packed = element_at(m, L, GATE) == element_at(m, L, UP) && gemm_stacks(element_at(m, L, UP), H, m->xn, m->ffn_up[L], nullptr, nullptr, 0, 0);
             if ((status = launch_gemm(d, u)) != NH_OK) return status;
             if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
             GemmArgs dn{element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, NH_F32, T, m->h, m->h, H};
