@@ -154,6 +154,12 @@ struct GemmArgs {
     // the activations were packed by the launch before this one (same X, M, K, nothing else launched on the device's
     // scratch in between): skip the packing pass
     bool packed = false;
+    // what the packing pass works on, instead of X as it lies (fp32 X only; the results are the ones the separate kernels give):
+    //   norm_w: the rows of X normalised as launch_rmsnorm(X, nullptr, norm_w, eps) writes them;
+    //   gate:   silu(gate) * X, element by element, as launch_silu_mul(gate, X) writes it (gate: [M][K] like X).
+    const float *norm_w = nullptr;
+    float eps = 0.0f;
+    const float *gate = nullptr;
 };
 int32_t launch_gemm(nh_device *d, const GemmArgs &args);
 // whether launch_gemm takes a product of this element and depth with matrices stacked along N at these boundaries, or with

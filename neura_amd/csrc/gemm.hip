@@ -136,18 +136,50 @@ struct GemmQ4Params {
 };
 
 // One workgroup per activation row: the row as MFMA-ready halves (and, for fp32 rows, its residue row and scale).
-template <bool HALF_IN>
+// PRELUDE: what a row is before it is packed -- 0: X as it lies; 1: X normalised (rmsnorm_kernel's arithmetic, so the same
+// fp32 numbers: thread t adds the squares of columns t, t + 256, ..., then a 256-wide tree); 2: silu(gate) * X as
+// silu_mul_kernel forms it.  `aux` is the norm's weight vector or the gate rows.
+constexpr int PACK_PLAIN = 0, PACK_NORM = 1, PACK_SWIGLU = 2;
+template <bool HALF_IN, int PRELUDE = PACK_PLAIN>
 __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restrict__ X, uint32_t K, _Float16 *__restrict__ A,
-                                                             _Float16 *__restrict__ S, float *__restrict__ unscale) {
+                                                             _Float16 *__restrict__ S, float *__restrict__ unscale,
+                                                             const float *__restrict__ aux = nullptr, float eps = 0.0f) {
+    static_assert(!(HALF_IN && PRELUDE != PACK_PLAIN), "half rows are packed as they lie");
     __shared__ uint32_t wave_top[4];
+    __shared__ float red[256];
     const uint32_t m = blockIdx.x, tid = threadIdx.x;
     const uint32_t nsb = K / 256u;
-    float scale = 1.0f;
+    float scale = 1.0f, norm = 1.0f;
+    if (PRELUDE == PACK_NORM) {
+        const float *xr = static_cast<const float *>(X) + (size_t)m * K;
+        float square = 0.0f;
+        for (uint32_t c = tid; c < K; c += 256) square = __fadd_rn(square, __fmul_rn(xr[c], xr[c]));
+        red[tid] = square;
+        __syncthreads();
+        for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+            if (tid < stride) red[tid] = __fadd_rn(red[tid], red[tid + stride]);
+            __syncthreads();
+        }
+        norm = rms_scale_of(red[0], K, eps);
+    }
+    // four neighbouring numbers of the row as the packing sees them
+    auto fetch = [&](uint32_t k) -> float4 {
+        float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(X) + (size_t)m * K + k);
+        if (PRELUDE == PACK_NORM) {
+            const float4 w = *reinterpret_cast<const float4 *>(aux + k);
+            v.x = __fmul_rn(__fmul_rn(v.x, norm), w.x), v.y = __fmul_rn(__fmul_rn(v.y, norm), w.y);
+            v.z = __fmul_rn(__fmul_rn(v.z, norm), w.z), v.w = __fmul_rn(__fmul_rn(v.w, norm), w.w);
+        } else if (PRELUDE == PACK_SWIGLU) {
+            const float4 g = *reinterpret_cast<const float4 *>(aux + (size_t)m * K + k);
+            v.x = g.x * (1.0f / (1.0f + expf(-g.x))) * v.x, v.y = g.y * (1.0f / (1.0f + expf(-g.y))) * v.y;
+            v.z = g.z * (1.0f / (1.0f + expf(-g.z))) * v.z, v.w = g.w * (1.0f / (1.0f + expf(-g.w))) * v.w;
+        }
+        return v;
+    };
     if (!HALF_IN) {
-        const float *x = static_cast<const float *>(X) + (size_t)m * K;
         uint32_t top = 0;
         for (uint32_t k = tid * 4u; k < K; k += 1024u) {
-            const float4 v = *reinterpret_cast<const float4 *>(x + k);
+            const float4 v = fetch(k);
             top = max(max(top, __builtin_bit_cast(uint32_t, v.x) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.y) & 0x7fffffffu);
             top = max(max(top, __builtin_bit_cast(uint32_t, v.z) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.w) & 0x7fffffffu);
         }
@@ -169,7 +201,7 @@ __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restr
 #pragma unroll
             for (int e = 0; e < 4; e++) hi[e] = v[e], lo[e] = (_Float16)0.0f;
         } else {
-            const float4 v = *reinterpret_cast<const float4 *>(static_cast<const float *>(X) + (size_t)m * K + k);
+            const float4 v = fetch(k);
             const float t[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -440,12 +472,18 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     if (!room) return NH_E_MEMORY;
     _Float16 *A = reinterpret_cast<_Float16 *>(room), *S = reinterpret_cast<_Float16 *>(room + halves);
     float *unscale = reinterpret_cast<float *>(room + halves + sums);
+    if ((a.norm_w || a.gate) && (half_rows || (a.norm_w && a.gate) || ((uintptr_t)(a.norm_w ? a.norm_w : a.gate) & 15u)))
+        return fail(NH_E_ARGUMENT, "a wide product normalises or gates fp32 rows read from 16-byte aligned addresses, one of the two");
     if (a.packed) {
         // what the launch before left in the scratch is this launch's operand
     } else if (half_rows) {
-        hipLaunchKernelGGL(gemm_pack_rows_kernel<true>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
+        hipLaunchKernelGGL(gemm_pack_rows_kernel<true>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, nullptr, 0.0f);
+    } else if (a.norm_w) {
+        hipLaunchKernelGGL((gemm_pack_rows_kernel<false, PACK_NORM>), dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, a.norm_w, a.eps);
+    } else if (a.gate) {
+        hipLaunchKernelGGL((gemm_pack_rows_kernel<false, PACK_SWIGLU>), dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, a.gate, 0.0f);
     } else {
-        hipLaunchKernelGGL(gemm_pack_rows_kernel<false>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale);
+        hipLaunchKernelGGL(gemm_pack_rows_kernel<false>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, nullptr, 0.0f);
     }
     NH_HIP(hipGetLastError());
     p.A = A, p.S = S, p.unscale = unscale;
@@ -478,8 +516,8 @@ bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, con
 int32_t launch_gemm(nh_device *d, const GemmArgs &a) {
     if (!a.M || !a.N) return NH_OK;
     if (mfma_takes(a.element, a.K, a.X, a.W)) return launch_gemm_q4k_mfma(d, a);
-    if (a.W_more[0] || a.W_more[1] || a.packed)
-        return fail(NH_E_ARGUMENT, "this wide product stacks no matrices and reuses no packed activations (ask gemm_stacks first)");
+    if (a.W_more[0] || a.W_more[1] || a.packed || a.norm_w || a.gate)
+        return fail(NH_E_ARGUMENT, "this wide product stacks no matrices, reuses no packed activations and packs rows as they lie (ask gemm_stacks first)");
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM), block(256);
     uint32_t row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     const uint8_t *W = static_cast<const uint8_t *>(a.W);

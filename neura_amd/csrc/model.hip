@@ -122,16 +122,19 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
     for (uint32_t L = 0; L < c.layers; L++) {
         bool roped = false;
         if (wide) {
-            if ((status = launch_rmsnorm(d, m->h, nullptr, m->attn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
             const uint8_t *mats[3] = {m->attn_q[L], m->attn_k[L], m->attn_v[L]};
             const float *biases[3] = {m->bias_q[L], m->bias_k[L], m->bias_v[L]};
             const uint32_t widths[3] = {QW, KW, KW};
             const bool alike = element_at(m, L, Q) == element_at(m, L, K_) && element_at(m, L, Q) == element_at(m, L, V);
+            const bool stacked = alike && gemm_stacks(element_at(m, L, Q), H, m->h, mats[0], mats[1], mats[2], QW, QW + KW);
             uint32_t column = 0;
-            if (alike && gemm_stacks(element_at(m, L, Q), H, m->xn, mats[0], mats[1], mats[2], QW, QW + KW)) {
-                // q|k|v as one product: the key and value projections alone are a few dozen workgroups each
-                GemmArgs g{element_at(m, L, Q), mats[0], QKV, H, m->xn, NH_F32, T, m->qkv, nullptr, QKV};
+            if (!stacked && (status = launch_rmsnorm(d, m->h, nullptr, m->attn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
+            if (stacked) {
+                // q|k|v as one product (the key and value projections alone are a few dozen workgroups each), the norm
+                // done by the pass that packs the rows
+                GemmArgs g{element_at(m, L, Q), mats[0], QKV, H, m->h, NH_F32, T, m->qkv, nullptr, QKV};
                 g.W_more[0] = mats[1], g.W_more[1] = mats[2], g.end[0] = QW, g.end[1] = QW + KW;
+                g.norm_w = m->attn_norm[L], g.eps = c.eps;
                 if ((status = launch_gemm(d, g)) != NH_OK) return status;
                 for (int s = 0; s < 3; s++) {
                     if (biases[s] && (status = launch_columns(d, m->qkv + column, QKV, biases[s], m->qkv + column, QKV, T, widths[s])) != NH_OK) return status;
@@ -211,15 +214,22 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         if (wide) {
             GemmArgs o{element_at(m, L, O), m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
             if ((status = launch_gemm(d, o)) != NH_OK) return status;
-            if ((status = launch_rmsnorm(d, m->h, nullptr, m->ffn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
-            GemmArgs g{element_at(m, L, GATE), m->ffn_gate[L], F, H, m->xn, NH_F32, T, m->act, nullptr, F};
-            GemmArgs u{element_at(m, L, UP), m->ffn_up[L], F, H, m->xn, NH_F32, T, m->up, nullptr, F};
+            // where the matrix cores take both projections the norm rides in the pass that packs the rows for the gate
+            // projection, and the up projection multiplies those same packed rows
+            const bool paired = element_at(m, L, GATE) == element_at(m, L, UP) &&
+                                gemm_stacks(element_at(m, L, GATE), H, m->h, m->ffn_gate[L], nullptr, nullptr, 0, 0) &&
+                                gemm_stacks(element_at(m, L, UP), H, m->h, m->ffn_up[L], nullptr, nullptr, 0, 0);
+            if (!paired && (status = launch_rmsnorm(d, m->h, nullptr, m->ffn_norm[L], c.eps, T, H, m->xn, nullptr)) != NH_OK) return status;
+            GemmArgs g{element_at(m, L, GATE), m->ffn_gate[L], F, H, paired ? m->h : m->xn, NH_F32, T, m->act, nullptr, F};
+            GemmArgs u{element_at(m, L, UP), m->ffn_up[L], F, H, paired ? m->h : m->xn, NH_F32, T, m->up, nullptr, F};
+            if (paired) g.norm_w = m->ffn_norm[L], g.eps = c.eps, u.packed = true;
             if ((status = launch_gemm(d, g)) != NH_OK) return status;
-            // the up projection multiplies the rows the gate projection just packed
-            u.packed = element_at(m, L, GATE) == element_at(m, L, UP) && gemm_stacks(element_at(m, L, UP), H, m->xn, m->ffn_up[L], nullptr, nullptr, 0, 0);
             if ((status = launch_gemm(d, u)) != NH_OK) return status;
-            if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
-            GemmArgs dn{element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, NH_F32, T, m->h, m->h, H};
+            // silu(gate) * up is formed as the down projection packs its rows, or by a kernel of its own
+            const bool gated = gemm_stacks(element_at(m, L, DOWN), F, m->up, m->ffn_down[L], nullptr, nullptr, 0, 0);
+            if (!gated && (status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
+            GemmArgs dn{element_at(m, L, DOWN), m->ffn_down[L], H, F, gated ? m->up : m->act, NH_F32, T, m->h, m->h, H};
+            if (gated) dn.gate = m->act;
             if ((status = launch_gemm(d, dn)) != NH_OK) return status;
         } else {
             GemvArgs o = narrow(m, element_at(m, L, O), m->attn_o[L], H, QW, m->att, T, m->h);
