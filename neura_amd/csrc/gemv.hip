@@ -1655,6 +1655,253 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
     }
 }
 
+
+// ------------------------------------------------- several activation rows on half-precision matrix cores ------
+//
+// Two to eight activation rows against 16-row tiles on v_mfma_f32_16x16x32_f16.  The weights are the B operand as exact
+// normal halves code * sc * 2^-14 (a nibble masked in place in a 16-bit lane is the half subnormal code * 2^-24 or
+// code * 2^-20; one packed multiply by sc * 2^10 or sc * 2^6 makes it normal), so the scale of a sub-block rides in
+// the operand and a whole super-block accumulates on the matrix cores before anything is weighed: four instructions per
+// eight weights and eight multiply-adds per super-block and lane, where the integer tiles convert and join digit sums
+// per sub-block.  An fp32 activation enters as two half rows (the value rounded to half after a power-of-two row scale,
+// and the rounding residue * 2^11): A row m < 8 is activation row m, A row 8 + m its residue, 22 bits of each take part.
+// The minimums come off with one more MFMA per super-block over (minimum, sub-block sum) pairs, as in the wide product.
+//
+// Operand slots: one MFMA takes 32 k.  Lane (n, kq) = (lane % 16, lane / 16) loads, per super-block, its row's header and
+// the 16 bytes at 16 + 64 j + 16 kq (j = 0, 1): half a 64-element group g = 2j + kq / 2, whose 16 low nibbles are elements
+// 16 (kq & 1) .. + 15 of sub-block 2g and whose high nibbles are the same elements of sub-block 2g + 1.  MFMA (j, i),
+// i = 2h + half, multiplies, in lane kq's eight slots, elements 16 (kq & 1) + 8 half + {0, 2, 1, 3, 4, 6, 5, 7} of
+// sub-block 2g + h -- the order the masks leave them in -- and the activations are staged in LDS in that same order, so a
+// lane's A operand is one 16-byte read.  Sub-blocks mix inside an MFMA; only d and dmin wait for the super-block's end.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t F16_BLOCK_PIECES = 8u * 4u * 16u + 2u * 16u;  // 16-byte pieces of LDS per staged super-block: operands, then sums
+
+template <int NW, int KS>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
+    constexpr uint32_t TPW = NW / KS, NT = NW * 64;
+    static_assert(NT == 1024, "eight row groups of 128 threads stage the activations");
+    extern __shared__ __attribute__((aligned(16))) uint32_t staged[];  // [block][F16_BLOCK_PIECES] pieces
+    __shared__ float red[NW];
+    __shared__ uint32_t tops[8];
+    __shared__ float unscale[8];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t split = blockIdx.y, blk0 = split * p.slice_blocks;
+    const uint32_t nb = min(p.slice_blocks, p.nblk - blk0);
+    const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
+    u32x4 *const pieces = reinterpret_cast<u32x4 *>(staged);
+    float *const part = reinterpret_cast<float *>(pieces + (size_t)nb * F16_BLOCK_PIECES);  // [TPW][KS][4][64]
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+
+    // ---- activations -> half planes in operand order: row r by threads 128 r .. 128 r + 127, eight neighbours a thread
+    {
+        const uint32_t r = tid >> 7, t = tid & 127u;
+        const bool real = r < p.rows;
+        const float *xr = p.x + (size_t)min(r, p.rows - 1u) * p.K + k0;
+        float v[4][8];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t k = 8u * t + 1024u * c;
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+            if (real && k < kn) a = *reinterpret_cast<const float4 *>(xr + k), b = *reinterpret_cast<const float4 *>(xr + k + 4u);
+            v[c][0] = a.x, v[c][1] = a.y, v[c][2] = a.z, v[c][3] = a.w, v[c][4] = b.x, v[c][5] = b.y, v[c][6] = b.z, v[c][7] = b.w;
+        }
+        if (p.norm_w) {  // one slice holds the whole row (the launcher sees to it)
+            float square = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) square = __fadd_rn(square, __fmul_rn(v[c][i], v[c][i]));
+            square = wave_sum(square);
+            if (lane == 0) red[wave] = square;
+            __syncthreads();
+            const float rms = rms_scale_of(red[2u * r] + red[2u * r + 1u], p.K, p.eps);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t k = 8u * t + 1024u * c;
+                float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+                if (k < kn) a = *reinterpret_cast<const float4 *>(p.norm_w + k0 + k), b = *reinterpret_cast<const float4 *>(p.norm_w + k0 + k + 4u);
+                const float w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[c][i] = __fmul_rn(__fmul_rn(v[c][i], rms), w[i]);
+            }
+        }
+        uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) top = max(top, __builtin_bit_cast(uint32_t, v[c][i]) & 0x7fffffffu);
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
+        if (tid < 8) tops[tid] = 0u;
+        __syncthreads();
+        if (lane == 0) atomicMax(&tops[r], top);
+        __syncthreads();
+        top = tops[r];
+        // a power of two that puts the row's largest magnitude in [2^13, 2^14)
+        const uint32_t raw = top >> 23, exponent = min(max(raw, 27u), 254u);
+        const float scale = __builtin_bit_cast(float, (267u - exponent) << 23);
+        if (t == 0) unscale[r] = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 13u) << 23);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t k = 8u * t + 1024u * c;
+            _Float16 hi[8], lo[8];
+            float sum_hi = 0.0f, sum_lo = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float scaled = v[c][i] * scale;
+                hi[i] = (_Float16)scaled;
+                lo[i] = (_Float16)((scaled - (float)hi[i]) * 2048.0f);
+                sum_hi += (float)hi[i], sum_lo += (float)lo[i];
+            }
+            // the 32 halves of a sub-block: four neighbouring threads
+            sum_hi += dpp<DPP_QUAD_XOR1>(sum_hi), sum_lo += dpp<DPP_QUAD_XOR1>(sum_lo);
+            sum_hi += dpp<DPP_QUAD_XOR2>(sum_hi), sum_lo += dpp<DPP_QUAD_XOR2>(sum_lo);
+            if (k < kn) {
+                const uint32_t b = k >> 8, g = (k >> 6) & 3u, h = (k >> 5) & 1u, e = k & 31u;
+                const uint32_t kq = 2u * (g & 1u) + (e >> 4), jj = 4u * (g >> 1) + 2u * h + ((e >> 3) & 1u);
+                u32x4 *at = pieces + (size_t)b * F16_BLOCK_PIECES + (jj * 4u + kq) * 16u;
+                typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+                auto pair = [](_Float16 a, _Float16 c) { return __builtin_bit_cast(uint32_t, half2v{a, c}); };
+                // slots 0..7 take elements 0, 2, 1, 3, 4, 6, 5, 7
+                at[r] = u32x4{pair(hi[0], hi[2]), pair(hi[1], hi[3]), pair(hi[4], hi[6]), pair(hi[5], hi[7])};
+                at[8u + r] = u32x4{pair(lo[0], lo[2]), pair(lo[1], lo[3]), pair(lo[4], lo[6]), pair(lo[5], lo[7])};
+                if ((t & 3u) == 0) {
+                    // sums / 64 as a half and its residue * 2^11: slots s (kq = 0) and s (kq = 1) of the minimums' operand
+                    const uint32_t sub = (k >> 5) & 7u;
+                    _Float16 *sums = reinterpret_cast<_Float16 *>(pieces + (size_t)b * F16_BLOCK_PIECES + 8u * 4u * 16u);
+                    const float a = sum_hi * 0.015625f, c2 = sum_lo * 0.015625f;
+                    const _Float16 ah = (_Float16)a, ch = (_Float16)c2;
+                    sums[(0u * 16u + r) * 8u + sub] = ah, sums[(1u * 16u + r) * 8u + sub] = (_Float16)((a - (float)ah) * 2048.0f);
+                    sums[(0u * 16u + 8u + r) * 8u + sub] = ch, sums[(1u * 16u + 8u + r) * 8u + sub] = (_Float16)((c2 - (float)ch) * 2048.0f);
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- tiles of 16 weight rows
+    const uint32_t n = lane & 15u, kq = lane >> 4;
+    const uint32_t ts = wave / KS, ks = wave % KS;
+    const uint32_t count = ks < nb ? (nb - ks + KS - 1u) / KS : 0u;  // super-blocks ks, ks + KS, ...
+    const uint32_t last_step = count ? count - 1u : 0u;
+    const uint8_t *const w0 = p.W[0], *const w1 = p.W[1], *const w2 = p.W[2];
+    const uint32_t end0 = p.end[0], end1 = p.end[1];
+    const bool gated = p.swiglu != 0;
+    const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
+    const uint32_t shift = 16u * (kq >> 1);  // the group's pair of 6-bit fields inside its scale words
+    for (uint32_t base = blockIdx.x * TPW; base < p.tiles; base += gridDim.x * TPW) {
+        const uint32_t tile = base + ts;
+        const bool live = tile < p.tiles;
+        const uint32_t at_tile = live ? tile : p.tiles - 1u;
+        const uint32_t r0 = at_tile * 16u;
+        const bool in0 = r0 < end0, in1 = r0 < end1;
+        const uint8_t *row = gated ? (n < 8u ? w0 : w1) + (size_t)(at_tile * 8u + (n & 7u)) * p.row_bytes
+                                   : (in0 ? w0 : (in1 ? w1 : w2)) + (size_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1)) + n) * p.row_bytes;
+        row += (size_t)blk0 * 144u;
+        u32x4 ahead[3];
+        auto fetch = [&](uint32_t step) {
+            // past the wave's last super-block the last one is fetched again: the waits count on every step issuing its loads
+            const uint8_t *block = row + (size_t)min(ks + KS * min(step, last_step), nb - 1u) * 144u;
+            ahead[0] = *(global_uint4)(uintptr_t)block;
+            ahead[1] = *(global_uint4)(uintptr_t)(block + 16u + 16u * kq);
+            ahead[2] = *(global_uint4)(uintptr_t)(block + 80u + 16u * kq);
+        };
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        fetch(0);
+        for (uint32_t step = 0; step < count; step++) {
+            const uint32_t b = min(ks + KS * step, nb - 1u);
+            const u32x4 hdr = ahead[0], q0 = ahead[1], q1 = ahead[2];
+            fetch(step + 1u);
+            const u32x4 *a_block = pieces + (size_t)b * F16_BLOCK_PIECES + kq * 16u + n;
+            f32x4_t tmp = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                // 6-bit scales of sub-blocks 2g, 2g + 1, g = 2j + kq / 2 (crates/neura-precision/src/ggml.rs:127-136); 0x6400 | v is the half 1024 + v
+                const uint32_t ya = (hdr.y >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
+                const uint32_t sc = j == 0 ? (ya & 0x3f3fu) : ((wa & 0x0f0fu) | ((ya >> 2) & 0x3030u));
+                const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;
+                const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;  // (sc0 * 2^10, sc1 * 2^6)
+                const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
+                const u32x4 q = j == 0 ? q0 : q1;
+                const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+                uint32_t low[8], high[8];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t even = words[w], odd = words[w] >> 8;
+                    low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
+                    low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
+                    high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
+                    high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t *from = (i < 2 ? low : high) + 4 * (i & 1);
+                    const half8_t weights = __builtin_bit_cast(half8_t, u32x4{from[0], from[1], from[2], from[3]});
+                    const half8_t rows = __builtin_bit_cast(half8_t, a_block[(4u * j + i) * 64u]);
+                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(rows, weights, tmp, 0, 0, 0);
+                }
+            }
+            // ---- the super-block is complete: weigh by d, take the minimums off
+            u32x4 mins = {0u, 0u, 0u, 0u}, sums = {0u, 0u, 0u, 0u};
+            if (kq < 2u) {
+                const uint32_t lo4 = hdr.z & 0x3f3f3f3fu;                                         // m0..m3
+                const uint32_t hi4 = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);  // m4..m7
+                half2_t m01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c010c00u) | 0x64006400u) - offset;
+                half2_t m23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c030c02u) | 0x64006400u) - offset;
+                half2_t m45 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c010c00u) | 0x64006400u) - offset;
+                half2_t m67 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c030c02u) | 0x64006400u) - offset;
+                if (kq == 1u) {  // the minimums * 2^-11 against the residues * 2^11
+                    const half2_t down = {(_Float16)0.00048828125f, (_Float16)0.00048828125f};
+                    m01 = m01 * down, m23 = m23 * down, m45 = m45 * down, m67 = m67 * down;
+                }
+                mins = u32x4{__builtin_bit_cast(uint32_t, m01), __builtin_bit_cast(uint32_t, m23), __builtin_bit_cast(uint32_t, m45),
+                             __builtin_bit_cast(uint32_t, m67)};
+                sums = pieces[(size_t)b * F16_BLOCK_PIECES + 8u * 4u * 16u + kq * 16u + n];
+            }
+            const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            const f32x4_t floors = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, sums), __builtin_bit_cast(half8_t, mins), zero, 0, 0, 0);
+            const half2_t dd = __builtin_bit_cast(half2_t, hdr.x);  // (d, dmin)
+            const float dscale = (float)dd.x * 16384.0f;  // the weights were staged * 2^-14
+            const float mscale = (float)dd.y * -64.0f;    // the sums were staged / 64
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] = fmaf(mscale, floors[e], fmaf(dscale, tmp[e], acc[e]));
+        }
+        // ---- the waves of the tile meet lane by lane
+        float *mine = part + ((size_t)ts * KS + ks) * 4u * 64u;
+#pragma unroll
+        for (int e = 0; e < 4; e++) mine[e * 64 + lane] = acc[e];
+        __syncthreads();
+        if (ks == 0) {
+            const float *from = part + (size_t)ts * KS * 4u * 64u;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float total = 0.0f;
+#pragma unroll
+                for (int k = 0; k < KS; k++) total += from[(size_t)k * 4u * 64u + e * 64 + lane];
+                // C row 4 kq + e: activation row 4 kq + e for kq < 2, its residue plane for kq >= 2 (32 lanes on)
+                const float residue = __shfl_xor(total, 32, 64);
+                const uint32_t arow = 4u * (kq & 1u) + e;
+                float value = fmaf(residue, 0.00048828125f, total) * unscale[arow];
+                const float up = __shfl_xor(value, 8, 64);
+                if (!live || kq >= 2u || arow >= p.rows) continue;
+                if (p.splits > 1) {
+                    const uint32_t column = gated ? (n < 8u ? tile * 8u + n : p.N / 2 + tile * 8u + (n - 8u)) : tile * 16u + n;
+                    p.partial[((size_t)split * p.rows + arow) * p.N + column] = value;
+                } else if (gated) {
+                    if (n < 8u) p.y[(size_t)arow * (p.N / 2) + tile * 8u + n] = silu(value) * up;
+                } else {
+                    const size_t at = (size_t)arow * p.N + tile * 16u + n;
+                    p.y[at] = p.residual ? p.residual[at] + value : value;
+                }
+            }
+        }
+        __syncthreads();  // the next tile's partial sums take the same places
+    }
+}
+
 // ------------------------------------------------------------------------- fold ----------
 
 // sums the slice partials in slice order and applies the epilogue
@@ -2058,6 +2305,83 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     return NH_OK;
 }
 
+// whether the half-precision tile kernel serves this product: NEURA_HIP_F16_TILES = 0 never, 2 wherever it can (two to eight
+// activation rows), 1 (default) where it measured faster than the integer tiles on the 7B shapes -- five to eight rows
+// against a matrix of enough tiles to give every wave several super-blocks (gate|up 36.6 against 42 us, the head 91 against
+// 110, ffn_down 29 against 27 with its fold; q|k|v and the output projection, one super-block a wave, are slower: 16.2 and
+// 12.5 against 11.4 and 11.2)
+static size_t f16_tiles_lds(uint32_t blocks, uint32_t NW) { return (size_t)blocks * F16_BLOCK_PIECES * 16u + (size_t)NW * 4u * 64u * sizeof(float); }
+static bool f16_tiles_take(const nh_device *d, const GemvArgs &a) {
+    const int mode = env_int("NEURA_HIP_F16_TILES", 1);
+    if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.rows < 2 || a.rows > 8) return false;
+    if (mode != 2 && (a.rows < 5 || a.K > 4096u || a.N / 16u < 4u * (uint32_t)d->compute_units)) return false;
+    if (a.K > 4096u && a.norm_w) return false;  // a fused norm wants the whole row in one slice
+    if (a.swiglu) {
+        if (a.N % 2u || a.end[0] != a.N / 2 || (a.N / 2) % 8u != 0) return false;
+    } else if (a.N % 16u != 0 || a.end[0] % 16u != 0 || a.end[1] % 16u != 0) {
+        return false;
+    }
+    for (int s = 0; s < 3; s++)
+        if (a.W[s] && ((uintptr_t)a.W[s] & 15u)) return false;
+    return !(((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u)));
+}
+
+template <int NW, int KS>
+static int32_t launch_f16_tiles_instance(nh_device *d, const MfmaParams &p, size_t lds) {
+    static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
+    if (lds > 64 * 1024 && !widened) {
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_f16_kernel<NW, KS>), hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024));
+        widened = true;
+    }
+    uint32_t resident = (uint32_t)((159 * 1024) / (lds + 1280));
+    if (resident > 1) resident = 1;  // sixteen waves a workgroup
+    if (resident < 1) resident = 1;
+    uint32_t blocks_x = (p.tiles + NW / KS - 1) / (NW / KS);
+    uint32_t most = (uint32_t)d->compute_units * resident / p.splits;
+    if (most < 1) most = 1;
+    if (blocks_x > most) blocks_x = most;
+    hipLaunchKernelGGL((gemv_q4k_f16_kernel<NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
+static int32_t launch_f16_tiles(nh_device *d, const GemvArgs &a) {
+    MfmaParams p{};
+    for (int s = 0; s < 3; s++) {
+        p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+        p.end[s] = a.end[s];
+    }
+    p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
+    p.N = a.N, p.K = a.K, p.nblk = a.K / 256u, p.row_bytes = p.nblk * 144u, p.rows = a.rows;
+    p.swiglu = a.swiglu, p.eps = a.eps;
+    p.tiles = a.N / 16u;
+    // K slices: 16 super-blocks stage in 136 KiB
+    const uint32_t most_blocks = 16u;
+    p.splits = (p.nblk + most_blocks - 1) / most_blocks;
+    p.slice_blocks = (p.nblk + p.splits - 1) / p.splits;
+    p.splits = (p.nblk + p.slice_blocks - 1) / p.slice_blocks;
+    if (p.splits > 1) {
+        p.partial = static_cast<float *>(scratch(d, (size_t)p.splits * p.rows * a.N * sizeof(float)));
+        if (!p.partial) return NH_E_MEMORY;
+    }
+    profile_mark(d);
+    // a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
+    const int forced = env_int("NEURA_HIP_F16_TILES_KS", 0);
+    const bool few = forced ? forced == 16 : p.tiles * p.splits < 4u * (uint32_t)d->compute_units;
+    const size_t lds = f16_tiles_lds(p.slice_blocks, 16);
+    int32_t status = few ? launch_f16_tiles_instance<16, 16>(d, p, lds) : launch_f16_tiles_instance<16, 4>(d, p, lds);
+    if (status != NH_OK) return status;
+    if (p.splits > 1) {
+        const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
+        hipLaunchKernelGGL(gemv_fold_kernel, dim3((outputs * p.rows + 255) / 256), dim3(256), 0, d->stream, p.partial, p.splits, p.rows, a.N,
+                           p.residual, a.swiglu, p.y);
+        NH_HIP(hipGetLastError());
+    }
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
+}
+
 // Q6_K, Q5_K, Q3_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
 template <int ELEMENT, int RB>
 static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
@@ -2103,6 +2427,7 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (f16_tiles_take(d, a)) return launch_f16_tiles(d, a);
     if (mfma32_takes(d, a)) return launch_mfma32(d, a);
     if (mfma_takes(a)) return launch_mfma(d, a);
     // activation rows are taken four, two or one at a time

@@ -203,6 +203,25 @@ def test_a_window_as_wide_as_what_was_fed_changes_nothing(device):
     bounded.release(), open_.release(), held.release(), held2.release()
 
 
+@pytest.mark.parametrize("batch", [2, 6, 8])
+def test_decode_on_half_precision_tiles_matches_the_oracle(device, monkeypatch, batch):
+    """NEURA_HIP_F16_TILES=2 sends every product of a 2..8 plane step to the 16-row half-precision tiles: stacked q|k|v and
+    gate|up with the fused norm, the residual epilogues, SwiGLU, against the oracle's logits and tokens."""
+    monkeypatch.setenv("NEURA_HIP_F16_TILES", "2")
+    shape = SMALL_Q4
+    model, ref, weights = build(device, shape, NH_Q4_K, batch=batch, context=24, seed=8)
+    rng = np.random.default_rng(9)
+    tokens = rng.integers(0, shape["vocab"], batch)
+    for step in range(5):
+        cursors = [step] * batch
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        got = model.decode_step(tokens, cursors)
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens = got
+    model.release(), weights.release()
+
+
 def test_decode_refuses_what_the_reference_refuses(device):
     model, ref, weights = build(device, TINY, NH_Q8_0, batch=1, context=8)
     with pytest.raises(NeuraError):   # cursor at the context (batch.rs:1627-1632)

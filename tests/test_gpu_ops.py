@@ -165,11 +165,14 @@ def test_q4_k_products_agree_in_every_form(device, monkeypatch, mode, N, K, rows
 
 @pytest.mark.parametrize("N,K,rows", [(64, 3584, 1), (96, 2048, 4), (128, 256, 2), (2048, 3584, 7), (64, 4096, 3), (64, 1536, 8), (160, 768, 5),
                                       (64, 18944, 8), (96, 8960, 2), (32, 18944, 5)])
-def test_q4_k_product_on_32_row_tiles(device, monkeypatch, N, K, rows):
+@pytest.mark.parametrize("forced", ["NEURA_HIP_MFMA32", "NEURA_HIP_F16_TILES"])
+def test_q4_k_product_on_32_row_tiles(device, monkeypatch, forced, N, K, rows):
     """NEURA_HIP_MFMA32=2 forces the 32 x 32 x 32 integer MFMA kernel (weights as the B operand, the digit planes of up to
     eight activation rows as A, digits scaled per sub-block): plain, with a residual and with SwiGLU, for every count of
-    activation rows, against the oracle and an fp64 product (the decoder tests run it with the fused norm)."""
-    monkeypatch.setenv("NEURA_HIP_MFMA32", "2")
+    activation rows, against the oracle and an fp64 product (the decoder tests run it with the fused norm).
+    NEURA_HIP_F16_TILES=2 forces, for two rows and more, the 16-row tiles on half-precision MFMA (weights as exact halves
+    code * sc, activations as value and residue half rows) through the same cases."""
+    monkeypatch.setenv(forced, "2")
     rng = np.random.default_rng(N + K + rows)
     raw = synth.q4_k_random(rng, N * K)
     x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-6, 6, (rows, K)))).astype(np.float32)  # wide dynamic range
