@@ -413,8 +413,10 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             // rows past the written keys may hold anything, and a weight of zero does not silence a NaN
             const uint32_t keep = tile + key < span ? 0xffffffffu : 0u;
             const uint32_t words[4] = {vraw[k].x & keep, vraw[k].y & keep, vraw[k].z & keep, vraw[k].w & keep};
+            // groups of four keys change places by the channel block (chunk / 4), or the chunks a store instruction touches share four banks
+            const uint32_t column = (((key >> 2) ^ (chunk >> 2)) << 2) | (key & 3u);
 #pragma unroll
-            for (int i = 0; i < 8; i++) vt[chunk * 8u + i][key] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
+            for (int i = 0; i < 8; i++) vt[chunk * 8u + i][column] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
         }
         if (tile + TK < span) fetch(tile + TK);  // in flight while this tile is multiplied
         __syncthreads();
@@ -467,8 +469,9 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             for (int t = 0; t < 2; t++) {
                 // slots 8h + i of step t: keys 16t + 4h + i (i < 4) and 16t + 8 + 4h + (i - 4), as the weights lie
                 half8_t values;
-                const uint2 low = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][16 * t + 4 * h]);
-                const uint2 high = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][16 * t + 8 + 4 * h]);
+                // channels 32 d + n lie in chunks 4 d .. 4 d + 3: their key groups sit d places off
+                const uint2 low = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][4 * ((4 * t + h) ^ d)]);
+                const uint2 high = *reinterpret_cast<const uint2 *>(&vt[32 * d + n][4 * ((4 * t + 2 + h) ^ d)]);
                 const u32x4 joined = {low.x, low.y, high.x, high.y};
                 values = __builtin_bit_cast(half8_t, joined);
                 acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(values, w_value[t], acc[d], 0, 0, 0);
@@ -487,6 +490,202 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             float4 out4 = {acc[d][4 * j] * normalized, acc[d][4 * j + 1] * normalized, acc[d][4 * j + 2] * normalized, acc[d][4 * j + 3] * normalized};
             *reinterpret_cast<float4 *>(dst + 32 * d + 8 * j + 4 * h) = out4;
         }
+}
+
+
+// ---------------------------------------------------------------- one query row, many planes: the matrix cores ------
+//
+// A decode step of several planes walks as many key tiles as a long fill, one query row each; the row-at-a-time kernel
+// spends its time in the multiply-adds of the scores and the value sums.  Here the ≤16 query heads of a group are the 16
+// columns of v_mfma_f32_16x16x32_f16.  A workgroup serves one (kv head, plane, section of the window); each of its four
+// waves walks every fourth tile of 32 keys on its own -- no barrier inside the walk -- and the four meet once in LDS.
+// Per tile and wave:
+//   scores  S[key][column]: the key rows are the A operand straight from the cache (lane (key % 16, kq) loads the 8 halves
+//           32 s + 8 kq .. of its key), the queries the B operand as value and residue * 2^11 half planes in registers.
+//           C hands lane (column, kq) the keys 4 kq + e and 16 + 4 kq + e of the tile: a column's statistics live in four lanes.
+//   values  O^T[channel][column] += V^T[channel][key] . P^T[key][column]: the weights (* 2^10, value and residue planes) go
+//           back in as the B operand from the registers C left them in -- slots 0..3 the keys 4 kq + e, slots 4..7 the keys
+//           16 + 4 kq + e -- and the value rows, which the wave wrote to its own corner of LDS transposed, are the A operand in
+//           that same key order (two 8-byte reads a lane).
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int WIDTH>
+__global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionParams p) {
+    constexpr int TK = 32;                  // keys per tile
+    constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
+    constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output
+    constexpr int VPITCH = TK + 4;          // halves per staged value channel
+    constexpr int PIECES = TK * WIDTH / 8 / 64;  // 16-byte pieces of a value tile per lane
+    // the waves' value corners and, once every wave has left the walk, their sums share one buffer
+    constexpr size_t VT_BYTES = sizeof(uint16_t) * 4 * WIDTH * VPITCH, MERGED_BYTES = sizeof(float) * 4 * 16 * (WIDTH + 2);
+    __shared__ __attribute__((aligned(16))) uint8_t shared_rows[VT_BYTES > MERGED_BYTES ? VT_BYTES : MERGED_BYTES];
+    uint16_t(*vt)[WIDTH][VPITCH] = reinterpret_cast<uint16_t(*)[WIDTH][VPITCH]>(shared_rows);
+    float(*merged)[16][WIDTH + 2] = reinterpret_cast<float(*)[16][WIDTH + 2]>(shared_rows);  // per wave and column: the channel sums, then the running top and mass
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n = lane & 15u, kq = lane >> 4;
+    const uint32_t G = p.groups;
+    const uint32_t unit = blockIdx.x, section = blockIdx.y;
+    const uint32_t b = unit % p.batch, kvh = unit / p.batch;
+    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
+
+    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
+    if (!p.reach && origin + 1u > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        origin = p.keys - 1u;
+    }
+    const Ring ring(p.keys, origin + 1u, p.reach);
+    const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
+    const uint32_t begin = min(p.keys, section * chunk);
+    const uint32_t visible = min(p.keys, origin + 1u);  // a ring too: the slots written so far
+    const uint32_t last = min(visible, begin + chunk);
+    const bool held = n < G;
+
+    // the queries of this lane's column as two half planes
+    half8_t q_value[STEPS], q_residue[STEPS];
+    {
+        const float *src = p.q + (uint64_t)(kvh * G + min(n, G - 1u)) * p.q_sh + (uint64_t)b * p.q_sb;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float value = held ? src[32 * s + 8 * kq + i] : 0.0f;
+                const _Float16 high = (_Float16)value;
+                q_value[s][i] = high;
+                q_residue[s][i] = (_Float16)((value - (float)high) * 2048.0f);
+            }
+    }
+    f32x4_t acc[BLOCKS];
+#pragma unroll
+    for (int d = 0; d < BLOCKS; d++) acc[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float top = -INFINITY, mass = 0.0f;
+
+    u32x4 kraw[2][STEPS], vraw[PIECES];
+    auto fetch_keys = [&](uint32_t tile) {
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const uint64_t at = (plane + min(tile + 16u * kb + n, p.capacity - 1u)) * WIDTH + 32u * s + 8u * kq;
+                kraw[kb][s] = *reinterpret_cast<const u32x4 *>(p.cache_k + at);
+            }
+    };
+    auto fetch_values = [&](uint32_t tile) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
+            vraw[i] = *reinterpret_cast<const u32x4 *>(p.cache_v + (plane + min(tile + key, p.capacity - 1u)) * WIDTH + part * 8u);
+        }
+    };
+    uint32_t tile = begin + wave * TK;
+    if (tile < last) fetch_keys(tile), fetch_values(tile);
+    for (; tile < last; tile += 4 * TK) {
+        // ---- scores
+        f32x4_t scores[2], fine[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            scores[kb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, fine[kb] = scores[kb];
+#pragma unroll
+            for (int s = 0; s < STEPS; s++) {
+                const half8_t keys = __builtin_bit_cast(half8_t, kraw[kb][s]);
+                scores[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(keys, q_value[s], scores[kb], 0, 0, 0);
+                fine[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(keys, q_residue[s], fine[kb], 0, 0, 0);
+            }
+        }
+        const uint32_t next = tile + 4 * TK;
+        if (next < last) fetch_keys(next);  // in flight during the rest of this tile
+        // ---- weights: register e of block kb is key 16 kb + 4 kq + e of the tile, for this lane's column
+        float tile_top = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t key = tile + 16u * kb + 4u * kq + e;
+                const bool seen = held && key < last && (!p.reach || ring.seen(key, origin));
+                scores[kb][e] = seen ? fmaf(fine[kb][e], 1.0f / 2048.0f, scores[kb][e]) * p.scale : -INFINITY;
+                tile_top = fmaxf(tile_top, scores[kb][e]);
+            }
+        tile_top = fmaxf(tile_top, __shfl_xor(tile_top, 16, 64));
+        tile_top = fmaxf(tile_top, __shfl_xor(tile_top, 32, 64));
+        const float newer = fmaxf(top, tile_top);
+        const float rescale = top == -INFINITY ? 0.0f : softmax_exp(top - newer);
+        float tile_mass = 0.0f;
+        half8_t w_value, w_residue;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float weight = scores[kb][e] == -INFINITY ? 0.0f : softmax_exp(scores[kb][e] - newer);
+                tile_mass += weight;
+                // the weights ride 2^10 up (undone with the mass at the end): their residues stay normal halves
+                const float raised = weight * 1024.0f;
+                const _Float16 high = (_Float16)raised;
+                w_value[4 * kb + e] = high;
+                w_residue[4 * kb + e] = (_Float16)(raised - (float)high);
+            }
+        tile_mass += __shfl_xor(tile_mass, 16, 64);
+        tile_mass += __shfl_xor(tile_mass, 32, 64);
+        mass = fmaf(mass, rescale, tile_mass);
+        top = newer;
+        // ---- the tile's value rows, transposed, into this wave's corner of LDS
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
+            // rows past the walked keys may hold anything, and a weight of zero does not silence a NaN
+            const uint32_t keep = tile + key < last ? 0xffffffffu : 0u;
+            const uint32_t words[4] = {vraw[i].x & keep, vraw[i].y & keep, vraw[i].z & keep, vraw[i].w & keep};
+            // groups of four keys change places by the channel block (part / 4): the sixteen parts a store instruction
+            // touches would otherwise share four banks
+            const uint32_t column = (((key >> 2) ^ (part >> 2)) << 2) | (key & 3u);
+#pragma unroll
+            for (int j = 0; j < 8; j++) vt[wave][part * 8u + j][column] = (uint16_t)(words[j >> 1] >> (16 * (j & 1)));
+        }
+        if (next < last) fetch_values(next);
+        __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
+        // ---- values
+#pragma unroll
+        for (int d = 0; d < BLOCKS; d++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[d][e] *= rescale;
+            // channels 16 d + n lie in parts 2 d and 2 d + 1: their key groups sit d / 2 places off
+            const uint2 low = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * (kq ^ (d >> 1))]);
+            const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
+            const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_value, acc[d], 0, 0, 0);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_residue, acc[d], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();  // the next tile overwrites the corner
+    }
+    // ---- the four waves meet: register e of block d is channel 16 d + 4 kq + e of this lane's column
+    __syncthreads();  // every wave is done with its corner
+#pragma unroll
+    for (int d = 0; d < BLOCKS; d++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) merged[wave][n][16 * d + 4 * kq + e] = acc[d][e] * (1.0f / 1024.0f);
+    if (kq == 0) merged[wave][n][WIDTH] = top, merged[wave][n][WIDTH + 1] = mass;
+    __syncthreads();
+    for (uint32_t index = tid; index < G * WIDTH; index += 256) {
+        const uint32_t g = index / WIDTH, c = index % WIDTH;
+        float largest = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; w++) largest = fmaxf(largest, merged[w][g][WIDTH]);
+        float value = 0.0f, total = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float held_top = merged[w][g][WIDTH];
+            const float weight = held_top == -INFINITY ? 0.0f : softmax_exp(held_top - largest);
+            value = fmaf(merged[w][g][c], weight, value);
+            total = fmaf(merged[w][g][WIDTH + 1], weight, total);
+        }
+        if (p.sections > 1) {
+            float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (WIDTH + 2);
+            dst[c] = value;
+            if (c == 0) dst[WIDTH] = largest, dst[WIDTH + 1] = total;
+        } else {
+            const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
+            p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + c] = value * normalized;
+        }
+    }
 }
 
 int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
@@ -513,6 +712,37 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             if (a.width == 64) hipLaunchKernelGGL(attention_tile_kernel<64>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
             else hipLaunchKernelGGL(attention_tile_kernel<128>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
             NH_HIP(hipGetLastError());
+            return NH_OK;
+        }
+    }
+    // one query row a plane: the group's query heads are the columns of the matrix cores
+    // (NEURA_HIP_ATTENTION_DECODE_TILE=0 keeps the row-at-a-time kernel)
+    {
+        const char *held = getenv("NEURA_HIP_ATTENTION_DECODE_TILE");
+        const bool wanted = !(held && held[0] == '0');
+        const bool aligned = ((uintptr_t)a.cache_k & 15u) == 0 && ((uintptr_t)a.cache_v & 15u) == 0;
+        const uint32_t planes = a.kv_heads * a.batch;
+        if (wanted && aligned && a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16) {
+            // sections of at least 256 keys (two tiles a wave) where the planes alone fill the chip, of 128 (one tile a wave)
+            // where they do not; enough workgroups to fill the chip twice over
+            const char *keys_held = getenv("NEURA_HIP_ATTENTION_DECODE_KEYS");
+            const uint32_t thinnest = keys_held && atoi(keys_held) > 0 ? (uint32_t)atoi(keys_held) : (planes >= 8 ? 256u : 128u);
+            uint32_t wanted_sections = ((uint32_t)d->compute_units * 2 + planes - 1) / planes;
+            const uint32_t most = (a.keys + thinnest - 1) / thinnest;
+            p.sections = wanted_sections < 1 ? 1 : (wanted_sections > most ? most : wanted_sections);
+            if (p.sections > 256) p.sections = 256;
+            if (p.sections > 1) {
+                p.partial = static_cast<float *>(scratch(d, (size_t)p.sections * a.heads * a.batch * (a.width + 2) * sizeof(float)));
+                if (!p.partial) return NH_E_MEMORY;
+            }
+            dim3 grid(planes, p.sections);
+            if (a.width == 64) hipLaunchKernelGGL(attention_decode_tile_kernel<64>, grid, dim3(256), 0, d->stream, p);
+            else hipLaunchKernelGGL(attention_decode_tile_kernel<128>, grid, dim3(256), 0, d->stream, p);
+            NH_HIP(hipGetLastError());
+            if (p.sections > 1) {
+                hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
+                NH_HIP(hipGetLastError());
+            }
             return NH_OK;
         }
     }
