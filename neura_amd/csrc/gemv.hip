@@ -1801,8 +1801,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
         const uint8_t *row = gated ? (n < 8u ? w0 : w1) + (size_t)(at_tile * 8u + (n & 7u)) * p.row_bytes
                                    : (in0 ? w0 : (in1 ? w1 : w2)) + (size_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1)) + n) * p.row_bytes;
         row += (size_t)blk0 * 144u;
-        u32x4 ahead[3];
-        auto fetch = [&](uint32_t step) {
+        // two super-blocks in flight a wave: the loads of step s + 2 go out as step s is taken up
+        u32x4 even[3], odd[3];
+        auto fetch = [&](u32x4 (&ahead)[3], uint32_t step) {
             // past the wave's last super-block the last one is fetched again: the waits count on every step issuing its loads
             const uint8_t *block = row + (size_t)min(ks + KS * min(step, last_step), nb - 1u) * 144u;
             ahead[0] = *(global_uint4)(uintptr_t)block;
@@ -1810,11 +1811,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
             ahead[2] = *(global_uint4)(uintptr_t)(block + 80u + 16u * kq);
         };
         f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        fetch(0);
-        for (uint32_t step = 0; step < count; step++) {
+        auto take = [&](const u32x4 (&ahead)[3], uint32_t step) {
             const uint32_t b = min(ks + KS * step, nb - 1u);
             const u32x4 hdr = ahead[0], q0 = ahead[1], q1 = ahead[2];
-            fetch(step + 1u);
             const u32x4 *a_block = pieces + (size_t)b * F16_BLOCK_PIECES + kq * 16u + n;
             f32x4_t tmp = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -1868,7 +1867,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
             const float mscale = (float)dd.y * -64.0f;    // the sums were staged / 64
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[e] = fmaf(mscale, floors[e], fmaf(dscale, tmp[e], acc[e]));
+        };
+        fetch(even, 0);
+        fetch(odd, 1);
+        uint32_t step = 0;
+        for (; step + 1u < count; step += 2u) {
+            take(even, step);
+            fetch(even, step + 2u);
+            take(odd, step + 1u);
+            fetch(odd, step + 3u);
         }
+        if (step < count) take(even, step);
         // ---- the waves of the tile meet lane by lane
         float *mine = part + ((size_t)ts * KS + ks) * 4u * 64u;
 #pragma unroll
