@@ -266,6 +266,63 @@ def test_config4_greedy_64_steps_qwen2_5_0_5b_shape_q8_0(device):
     model.release(), weights.release()
 
 
+def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
+    """The 7B shape itself (hidden 3584, 28 query heads over 4 key heads of 128, ffn 18944, vocabulary 152064, random Q4_K
+    blocks, separate head) cut to two layers, at context 4096: decode steps at batch 1 on caches filled with N(0,1) halves
+    (the products at their real depths and row counts, the rotation folded in, attention over 4000 keys in sections), a
+    64-row fill (wide products with stacked q|k|v and fused packing passes, attention over a chunk), and a step of eight
+    planes (the half-precision tiles on gate|up and the head, the integer tiles on the rest), each against the oracle."""
+    shape = synth.SHAPES["qwen2.5-7b"]
+    layers, context, filled, rows = 2, 4096, 4000, 64
+    rng = np.random.default_rng(50)
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks", layers=layers))
+    host = {name: raw for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+
+    def pair(batch, max_rows):
+        model = Model(device, weights, shape, NH_Q4_K, batch, context, max_rows, layers=layers)
+        ref = oracle.Model(shape, NH_Q4_K, host, batch, context, max_rows, layers=layers)
+        for layer in range(layers):
+            for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+                halves = np.zeros(model.cache_shape, dtype=np.float16)
+                halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], batch, filled, shape["head_dim"])).astype(np.float16)
+                held[layer][:] = halves.view(np.uint16).reshape(-1)
+                model.cache_write(layer, which, halves.view(np.uint16))
+        return model, ref
+
+    def same(model, ref, tokens, cursors, what):
+        want_logits, want = ref.forward(tokens, 1, cursors, threads=16)
+        got = model.decode_step(tokens, cursors)
+        logits = model.logits()
+        scale = np.abs(want_logits).max()
+        assert np.abs(logits - want_logits).max() <= 1e-3 * scale, what
+        for plane, gap in enumerate(margins(want_logits)):
+            if gap > 2e-3 * scale:
+                assert got[plane] == want[plane], (what, plane, gap)
+        return [int(t) for t in want]
+
+    model, ref = pair(1, rows)
+    token = [int(rng.integers(0, shape["vocab"]))]
+    for step in range(3):
+        token = same(model, ref, token, [filled + step], "batch 1, step %d" % step)
+    # a fill of 64 rows over positions 100 .. 163, then a step that weighs what it wrote
+    prompt = rng.integers(0, shape["vocab"], rows)
+    model.prefill(prompt, rows, [100])
+    ref.forward(prompt, rows, [100], want_logits=False, threads=16)
+    for layer in range(layers):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_rows = oracle.f16_to_f32(model.cache_read(layer, which)[:, :, 100:100 + rows].reshape(-1))
+            want_rows = oracle.f16_to_f32(held[layer].reshape(model.cache_shape)[:, :, 100:100 + rows].reshape(-1))
+            assert np.abs(got_rows - want_rows).max() <= 2e-3 * max(1.0, np.abs(want_rows).max()), (layer, which)
+    same(model, ref, token, [filled + 3], "batch 1 after the fill")
+    model.release()
+    model, ref = pair(8, 1)
+    tokens = [int(t) for t in rng.integers(0, shape["vocab"], 8)]
+    for step in range(2):
+        tokens = same(model, ref, tokens, [filled - 7 * plane + step for plane in range(8)], "batch 8, step %d" % step)
+    model.release(), weights.release()
+
+
 def test_graph_replays_match_eager_steps(device, monkeypatch):
     """The decode step replayed from its captured HIP graph gives, on every replay, exactly the
     logits and tokens of the same step launched eagerly -- with eager work (fills, operator
