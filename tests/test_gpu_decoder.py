@@ -323,6 +323,38 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
     model.release(), weights.release()
 
 
+def test_config5_shape_stored_as_a_q4_k_m_file_stores_it(device):
+    """The 7B shape cut to two layers, stored the way llama.cpp's Q4_K_M recipe stores Qwen2.5-7B: the head and the first
+    layer's value and down projections in Q6_K, q, k and v biases on every layer.  Batch-1 steps at context 4096: the
+    staged Q6_K products at their real shapes (a 152064-row head, a down projection in K slices), q|k rotated from one
+    product with the value row appended behind it, the layer of one element with biases in the folded rotation."""
+    shape = synth.SHAPES["qwen2.5-7b"]
+    layers, context, filled = 2, 4096, 4000
+    mixed = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.0.ffn_down.weight": NH_Q6_K}
+    rng = np.random.default_rng(51)
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks", layers=layers, elements=mixed, biases=(0, 1)))
+    host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, NH_Q4_K, 1, context, 1, layers=layers)
+    ref = oracle.Model(shape, NH_Q4_K, host, 1, context, 1, layers=layers, elements=mixed)
+    for layer in range(layers):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            halves = np.zeros(model.cache_shape, dtype=np.float16)
+            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
+            held[layer][:] = halves.view(np.uint16).reshape(-1)
+            model.cache_write(layer, which, halves.view(np.uint16))
+    token = [int(rng.integers(0, shape["vocab"]))]
+    for step in range(3):
+        want_logits, want = ref.forward(token, 1, [filled + step], threads=16)
+        got = model.decode_step(token, [filled + step])
+        scale = np.abs(want_logits).max()
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * scale, step
+        if margins(want_logits)[0] > 2e-3 * scale:
+            assert int(got[0]) == int(want[0]), (step, margins(want_logits))
+        token = [int(want[0])]
+    model.release(), weights.release()
+
+
 def test_graph_replays_match_eager_steps(device, monkeypatch):
     """The decode step replayed from its captured HIP graph gives, on every replay, exactly the
     logits and tokens of the same step launched eagerly -- with eager work (fills, operator
