@@ -671,6 +671,115 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     }
 }
 
+// Q8_0, one activation row, rows of at most 64 blocks (K <= 2048): the shape of the Q4_K decode kernel.  A lane owns one
+// block column for the whole kernel and keeps its 32 activations in registers; the 34 bytes of a block sit on a 2-byte
+// boundary, so a lane reads the nine words that cover it from the 4-byte boundary below it (the reference's own reading,
+// crates/neura-kernel/src/dot.rs:197-264) and realigns by 16 bits where the block starts on a half word.  No LDS tile and no
+// barrier between the rows: the first pass's words are on their way while the activations are staged.
+typedef uint32_t u32x4_loose __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int R>
+struct Q8Tile {
+    u32x4 a[R], b[R];
+    uint32_t c[R];
+    uint32_t odd[R];  // 2 where the row's block starts on a half word, else 0
+};
+
+template <int R, int G>
+__global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
+    extern __shared__ float xs[];  // skew32(K)
+    __shared__ float red[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr uint32_t RS = 64u / G, rows_per_pass = R * RS;
+    const uint32_t u = lane & (G - 1u), rs = lane / G;
+    const bool active = u < p.nblk;
+    const uint32_t unit = active ? u : 0u;  // an idle lane re-reads block 0 against zero activations
+
+    auto load = [&](Q8Tile<R> &t, uint32_t rg) {
+        const uint32_t first = rg * rows_per_pass + rs * R;  // first logical row of this lane group (a multiple of R)
+        const uint8_t *base[R];
+        if (p.swiglu) {
+            const uint32_t pair = min(first, p.N - R) >> 1;  // logical rows 2q, 2q+1 = gate row q, up row q
+#pragma unroll
+            for (int r = 0; r < R; r++) base[r] = ((r & 1) ? p.W[1] : p.W[0]) + (size_t)(pair + (r >> 1)) * p.row_bytes;
+        } else {
+            const uint32_t n = min(first, p.N - R);  // R rows of one matrix: every matrix end is a multiple of R
+            const bool in0 = n < p.end[0], in1 = n < p.end[1];
+            const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
+            const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
+#pragma unroll
+            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r) * p.row_bytes;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uintptr_t at = (uintptr_t)(base[r] + unit * 34u);
+            const uintptr_t low = at & ~(uintptr_t)3;
+            t.odd[r] = (uint32_t)(at & 2u);
+            t.a[r] = *(const __attribute__((address_space(1))) u32x4_loose *)low;
+            t.b[r] = *(const __attribute__((address_space(1))) u32x4_loose *)(low + 16u);
+            // a block on a word boundary ends two bytes into the ninth word: those two only are read (the last block of a
+            // tensor ends where its allocation may)
+            if (at & 2u) t.c[r] = *(const __attribute__((address_space(1))) uint32_t *)(low + 32u);
+            else t.c[r] = *(const __attribute__((address_space(1))) uint16_t *)(low + 32u);
+        }
+    };
+
+    const uint32_t stride = gridDim.x * 4u;
+    uint32_t rg = blockIdx.x * 4u + wave;
+    Q8Tile<R> held;
+    if (rg < p.row_groups) load(held, rg);  // in flight while the activations are staged
+
+    stage_row(p.x, p.K, 0u, p.K, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew32(i); });
+    __syncthreads();
+
+    float xr[32];
+    float xsum = 0.0f;
+    {
+        const float4 *src = reinterpret_cast<const float4 *>(xs + skew32(unit * 32u));
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float4 a = active ? src[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+            xr[4 * j] = a.x, xr[4 * j + 1] = a.y, xr[4 * j + 2] = a.z, xr[4 * j + 3] = a.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 32; j++) xsum += xr[j];
+    }
+
+    while (rg < p.row_groups) {
+        const uint32_t first = rg * rows_per_pass + rs * R;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t words[9] = {held.a[r].x, held.a[r].y, held.a[r].z, held.a[r].w, held.b[r].x, held.b[r].y, held.b[r].z, held.b[r].w, held.c[r]};
+            const bool odd = held.odd[r] != 0u;
+            // the scale is the half at the block's first two bytes, the 32 codes follow it
+            const float scale = half_to_float((uint16_t)(odd ? words[0] >> 16 : words[0] & 0xffffu));
+            float total = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const uint32_t w = (odd ? words[j + 1] : __funnelshift_r(words[j], words[j + 1], 16)) ^ 0x80808080u;  // q + 128
+                total = fmaf(xr[4 * j + 0], (float)(w & 0xffu), total);
+                total = fmaf(xr[4 * j + 1], (float)((w >> 8) & 0xffu), total);
+                total = fmaf(xr[4 * j + 2], (float)((w >> 16) & 0xffu), total);
+                total = fmaf(xr[4 * j + 3], (float)(w >> 24), total);
+            }
+            acc[r] = scale * (total - 128.0f * xsum);
+        }
+        rg += stride;
+        __builtin_amdgcn_sched_barrier(0);  // the next loads reuse this tile's registers: keep them behind the arithmetic
+        const float sum = fold_rows<R, G>(acc, lane);  // lane u < R holds row first + u
+        if (rg < p.row_groups) load(held, rg);
+        const uint32_t i = first + u;
+        if (p.swiglu) {
+            const float up = dpp<DPP_QUAD_XOR1>(sum);
+            if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(sum) * up;
+        } else if (u < R && i < p.N) {
+            p.y[i] = p.residual ? p.residual[i] + sum : sum;
+        }
+    }
+}
+
 // ------------------------------------------------------------ Q6_K, Q5_K, Q3_K -------
 //
 // 210-, 176- and 110-byte super-blocks; the first and the last leave rows on 2-byte boundaries.  A wave copies the two
@@ -2054,6 +2163,26 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     } else if (q4) {
         if (R == 4) NH_LAUNCH(gemv_q4k_kernel, 4);
         else NH_LAUNCH(gemv_q4k_kernel, 2);
+    } else if (RB == 1 && fast && p.splits == 1 && p.nblk <= 64u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0) {
+        // one activation row, a row of blocks inside one wave: the words of a block straight from memory, no LDS tile
+        const uint32_t passes = (a.N + (uint32_t)R * RS - 1) / ((uint32_t)R * RS);
+        p.row_groups = passes;
+        uint32_t wgs = (passes + 3) / 4;
+        const uint32_t resident = (uint32_t)d->compute_units * 4u;
+        if (wgs > resident) wgs = resident;
+        const size_t staged = (size_t)(a.K + a.K / 32u * 4u) * sizeof(float);
+        const dim3 wide(wgs);
+#define NH_Q8(RR, GG) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<RR, GG>), wide, block, staged, d->stream, p)
+        if (R == 4) {
+            if (p.group == 64) NH_Q8(4, 64);
+            else if (p.group == 32) NH_Q8(4, 32);
+            else NH_Q8(4, 16);
+        } else {
+            if (p.group == 64) NH_Q8(2, 64);
+            else if (p.group == 32) NH_Q8(2, 32);
+            else NH_Q8(2, 16);
+        }
+#undef NH_Q8
     } else {
         if (R == 4) NH_LAUNCH(gemv_q8_0_kernel, 4);
         else NH_LAUNCH(gemv_q8_0_kernel, 2);
