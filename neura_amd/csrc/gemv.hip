@@ -685,16 +685,21 @@ struct Q8Tile {
     uint32_t odd[R];  // 2 where the row's block starts on a half word, else 0
 };
 
-template <int R, int G>
+// DEEP (rows of 65 to 256 blocks, K <= 8192): the four waves of a workgroup walk the same rows, wave w the blocks 64 w ..
+// 64 w + 63, and meet in LDS once a pass.
+template <int R, int G, bool DEEP = false>
 __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
+    static_assert(!DEEP || G == 64, "a deep row fills every wave");
     extern __shared__ float xs[];  // skew32(K)
     __shared__ float red[256];
+    __shared__ float part[2][4][R];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr uint32_t RS = 64u / G, rows_per_pass = R * RS;
     const uint32_t u = lane & (G - 1u), rs = lane / G;
-    const bool active = u < p.nblk;
-    const uint32_t unit = active ? u : 0u;  // an idle lane re-reads block 0 against zero activations
+    const uint32_t block = DEEP ? 64u * wave + u : u;
+    const bool active = block < p.nblk;
+    const uint32_t unit = active ? block : 0u;  // an idle lane re-reads block 0 against zero activations
 
     auto load = [&](Q8Tile<R> &t, uint32_t rg) {
         const uint32_t first = rg * rows_per_pass + rs * R;  // first logical row of this lane group (a multiple of R)
@@ -725,8 +730,9 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
         }
     };
 
-    const uint32_t stride = gridDim.x * 4u;
-    uint32_t rg = blockIdx.x * 4u + wave;
+    const uint32_t stride = DEEP ? gridDim.x : gridDim.x * 4u;
+    uint32_t rg = DEEP ? blockIdx.x : blockIdx.x * 4u + wave;
+    uint32_t parity = 0;
     Q8Tile<R> held;
     if (rg < p.row_groups) load(held, rg);  // in flight while the activations are staged
 
@@ -768,8 +774,15 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
         }
         rg += stride;
         __builtin_amdgcn_sched_barrier(0);  // the next loads reuse this tile's registers: keep them behind the arithmetic
-        const float sum = fold_rows<R, G>(acc, lane);  // lane u < R holds row first + u
+        float sum = fold_rows<R, G>(acc, lane);  // lane u < R holds row first + u
         if (rg < p.row_groups) load(held, rg);
+        if (DEEP) {
+            if (u < R) part[parity][wave][u] = sum;
+            __syncthreads();  // every wave walks the same passes
+            if (u < R) sum = (part[parity][0][u] + part[parity][1][u]) + (part[parity][2][u] + part[parity][3][u]);
+            parity ^= 1u;
+            if (wave != 0) continue;
+        }
         const uint32_t i = first + u;
         if (p.swiglu) {
             const float up = dpp<DPP_QUAD_XOR1>(sum);
@@ -2163,17 +2176,24 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     } else if (q4) {
         if (R == 4) NH_LAUNCH(gemv_q4k_kernel, 4);
         else NH_LAUNCH(gemv_q4k_kernel, 2);
-    } else if (RB == 1 && fast && p.splits == 1 && p.nblk <= 64u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0) {
-        // one activation row, a row of blocks inside one wave: the words of a block straight from memory, no LDS tile
+    } else if (RB == 1 && fast && p.nblk <= 256u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0) {
+        // one activation row, a row of blocks inside one wave (or, deeper, inside the four waves of a workgroup): the words of
+        // a block straight from memory, no LDS tile, no K slices and no fold
+        const bool deep = p.nblk > 64u;
+        if (deep) p.group = 64, RS = 1;
+        p.splits = 1, p.blocks_per_split = p.nblk;
         const uint32_t passes = (a.N + (uint32_t)R * RS - 1) / ((uint32_t)R * RS);
         p.row_groups = passes;
-        uint32_t wgs = (passes + 3) / 4;
+        uint32_t wgs = deep ? passes : (passes + 3) / 4;
         const uint32_t resident = (uint32_t)d->compute_units * 4u;
         if (wgs > resident) wgs = resident;
         const size_t staged = (size_t)(a.K + a.K / 32u * 4u) * sizeof(float);
         const dim3 wide(wgs);
 #define NH_Q8(RR, GG) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<RR, GG>), wide, block, staged, d->stream, p)
-        if (R == 4) {
+        if (deep) {
+            if (R == 4) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<4, 64, true>), wide, block, staged, d->stream, p);
+            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, true>), wide, block, staged, d->stream, p);
+        } else if (R == 4) {
             if (p.group == 64) NH_Q8(4, 64);
             else if (p.group == 32) NH_Q8(4, 32);
             else NH_Q8(4, 16);
