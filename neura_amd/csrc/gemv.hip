@@ -297,6 +297,46 @@ __device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s
     mn = __builtin_bit_cast(half2_t, (p_mn & s.mask_p) | ((q_mn >> 2) & s.mask_q));
 }
 
+// The epilogue of a q|k|v product that folds the rotation in: lane u < R of a lane group holds logical row i = first + u, and
+// logical rows 2t, 2t + 1 are channels c and c + width/2 of one head (crates/neura-kernel/src/task/rope.rs:95-122).  The
+// projection's bias, if it has one, comes before the rotation; q rows go to y, k rows rotated and v rows as they are to the
+// caches as halves, at the cursor (at cursor mod span in a ring).  Every lane of the wave calls it.
+template <int R>
+__device__ __forceinline__ void rotate_and_store(const GemvParams &p, float total, uint32_t i, uint32_t u) {
+    const uint32_t half = p.rope_width >> 1, pair = min(i, p.N - 1u) >> 1, c = pair % half;
+    const uint32_t n = (pair / half) * p.rope_width + c + (i & 1u) * half;
+    if (u < R && i < p.N) {
+        const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
+        const uint32_t e0 = p.end[0], e1 = p.end[1];
+        const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
+        const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
+        if (bias) total += bias[n - before];
+    }
+    const float other = dpp<DPP_QUAD_XOR1>(total);
+    if (u < R && i < p.N) {
+        const uint32_t position = p.rope_cursor[0];
+        float value = total;
+        if (n < p.rope_k_rows) {
+            // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
+            const float cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+            const float sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+            value = (i & 1u) ? total * cosine + other * sine : total * cosine - other * sine;
+        }
+        if (n < p.rope_q_rows) {
+            p.y[n] = value;
+        } else if (position >= p.rope_positions || (!p.rope_ring && position >= p.rope_capacity)) {
+            atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        } else {
+            const bool key = n < p.rope_k_rows;
+            const uint32_t within = n - (key ? p.rope_q_rows : p.rope_k_rows);  // head * width + channel
+            const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
+            uint16_t *cache = key ? p.rope_k : p.rope_v;
+            const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
+            cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
+        }
+    }
+}
+
 // One pass of the decode kernel over R rows: the raw blocks a lane owns.
 template <int R>
 struct DecodeTile {
@@ -408,40 +448,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) 
             float up = dpp<DPP_QUAD_XOR1>(total);
             if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(total) * up;
         } else if (ROPE) {
-            // lanes 0 and 1 hold channels c and c + width/2 of one head (crates/neura-kernel/src/task/rope.rs:95-122)
-            const uint32_t half = p.rope_width >> 1, pair = min(i, p.N - 1u) >> 1, c = pair % half;
-            const uint32_t n = (pair / half) * p.rope_width + c + (i & 1u) * half;
-            if (u < R && i < p.N) {
-                // the projection's bias, if it has one, comes before the rotation
-                const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
-                const uint32_t e0 = p.end[0], e1 = p.end[1];
-                const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
-                const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
-                if (bias) total += bias[n - before];
-            }
-            const float other = dpp<DPP_QUAD_XOR1>(total);
-            if (u < R && i < p.N) {
-                const uint32_t position = p.rope_cursor[0];
-                float value = total;
-                if (n < p.rope_k_rows) {
-                    // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
-                    const float cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
-                    const float sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
-                    value = (i & 1u) ? total * cosine + other * sine : total * cosine - other * sine;
-                }
-                if (n < p.rope_q_rows) {
-                    p.y[n] = value;
-                } else if (position >= p.rope_positions || (!p.rope_ring && position >= p.rope_capacity)) {
-                    atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-                } else {
-                    const bool key = n < p.rope_k_rows;
-                    const uint32_t within = n - (key ? p.rope_q_rows : p.rope_k_rows);  // head * width + channel
-                    const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
-                    uint16_t *cache = key ? p.rope_k : p.rope_v;
-                    const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
-                    cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
-                }
-            }
+            rotate_and_store<R>(p, total, i, u);
         } else if (u < R && i < p.N) {
             p.y[i] = p.residual ? p.residual[i] + total : total;
         }
@@ -687,9 +694,10 @@ struct Q8Tile {
 
 // DEEP (rows of 65 to 256 blocks, K <= 8192): the four waves of a workgroup walk the same rows, wave w the blocks 64 w ..
 // 64 w + 63, and meet in LDS once a pass.
-template <int R, int G, bool DEEP = false>
+template <int R, int G, bool DEEP = false, bool ROPE = false>
 __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
     static_assert(!DEEP || G == 64, "a deep row fills every wave");
+    static_assert(!ROPE || (R == 2 && !DEEP), "the rotation pairs the two rows of a pass");
     extern __shared__ float xs[];  // skew32(K)
     __shared__ float red[256];
     __shared__ float part[2][4][R];
@@ -709,12 +717,17 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
 #pragma unroll
             for (int r = 0; r < R; r++) base[r] = ((r & 1) ? p.W[1] : p.W[0]) + (size_t)(pair + (r >> 1)) * p.row_bytes;
         } else {
-            const uint32_t n = min(first, p.N - R);  // R rows of one matrix: every matrix end is a multiple of R
+            // R rows of one matrix: every matrix end is a multiple of R.  With the rotation folded in, logical rows 2t, 2t+1
+            // are channels t and t + width/2 of one head
+            const uint32_t logical = min(first, p.N - R);
+            const uint32_t half = p.rope_width >> 1, pair = logical >> 1;
+            const uint32_t n = ROPE ? (pair / half) * p.rope_width + pair % half : logical;
+            const uint32_t hop = ROPE ? half : 1u;
             const bool in0 = n < p.end[0], in1 = n < p.end[1];
             const uint8_t *matrix = in0 ? p.W[0] : (in1 ? p.W[1] : p.W[2]);
             const uint32_t before = in0 ? 0u : (in1 ? p.end[0] : p.end[1]);
 #pragma unroll
-            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r) * p.row_bytes;
+            for (int r = 0; r < R; r++) base[r] = matrix + (size_t)(n - before + r * hop) * p.row_bytes;
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -787,6 +800,8 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
         if (p.swiglu) {
             const float up = dpp<DPP_QUAD_XOR1>(sum);
             if (u < R && !(u & 1u) && i + 1 < p.N) p.y[i >> 1] = silu(sum) * up;
+        } else if (ROPE) {
+            rotate_and_store<R>(p, sum, i, u);
         } else if (u < R && i < p.N) {
             p.y[i] = p.residual ? p.residual[i] + sum : sum;
         }
@@ -2157,7 +2172,8 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         else if (nw == 8) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 8>), dim3((blocks_x + 1) / 2, p.splits), dim3(512), lds, d->stream, p); \
         else hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p);           \
     } while (0)
-    if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1))
+    const bool q8_direct = !q4 && RB == 1 && fast && p.nblk <= 256u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0;
+    if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1) && !(q8_direct && R == 2 && p.nblk <= 64u))
         return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (q4 && RB == 1 && fast && a.rope) {
         if (p.group == 64) hipLaunchKernelGGL((gemv_q4k_decode_kernel<2, 64, false, 4, true>), grid, block, lds, d->stream, p);
@@ -2176,7 +2192,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     } else if (q4) {
         if (R == 4) NH_LAUNCH(gemv_q4k_kernel, 4);
         else NH_LAUNCH(gemv_q4k_kernel, 2);
-    } else if (RB == 1 && fast && p.nblk <= 256u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0) {
+    } else if (q8_direct) {
         // one activation row, a row of blocks inside one wave (or, deeper, inside the four waves of a workgroup): the words of
         // a block straight from memory, no LDS tile, no K slices and no fold
         const bool deep = p.nblk > 64u;
@@ -2190,7 +2206,11 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         const size_t staged = (size_t)(a.K + a.K / 32u * 4u) * sizeof(float);
         const dim3 wide(wgs);
 #define NH_Q8(RR, GG) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<RR, GG>), wide, block, staged, d->stream, p)
-        if (deep) {
+        if (a.rope) {
+            if (p.group == 64) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, false, true>), wide, block, staged, d->stream, p);
+            else if (p.group == 32) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 32, false, true>), wide, block, staged, d->stream, p);
+            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 16, false, true>), wide, block, staged, d->stream, p);
+        } else if (deep) {
             if (R == 4) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<4, 64, true>), wide, block, staged, d->stream, p);
             else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, true>), wide, block, staged, d->stream, p);
         } else if (R == 4) {
@@ -2364,8 +2384,16 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
 // mirrors the conditions under which launch_rows<1> takes the decode kernel with two rows per pass
 bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     if (env_int("NEURA_HIP_FUSE_ROPE", 1) == 0) return false;
-    if (a.element != NH_Q4_K || a.rows != 1 || a.swiglu || a.residual || a.K % 256u != 0 || a.K > 4096u) return false;
-    if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 256u * 144u) >= (1ull << 32)) return false;
+    if (a.rows != 1 || a.swiglu || a.residual) return false;
+    if (a.element == NH_Q8_0) {
+        // the direct Q8_0 decode kernel, a row of blocks inside one wave
+        if (a.K % 32u != 0 || a.K > 2048u || env_int("NEURA_HIP_Q8_DECODE", 1) == 0) return false;
+        if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 32u * 34u) >= (1ull << 32)) return false;
+        if (a.end[0] % 2u || a.end[1] % 2u || a.N % 2u) return false;
+    } else {
+        if (a.element != NH_Q4_K || a.K % 256u != 0 || a.K > 4096u) return false;
+        if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 256u * 144u) >= (1ull << 32)) return false;
+    }
     if (env_int("NEURA_HIP_GEMV_ROWS", 2) != 2 || env_int("NEURA_HIP_MFMA", 1) == 2) return false;
     const uint32_t width = rope.width;
     if (width < 2 || (width & (width - 1u)) != 0) return false;

@@ -393,14 +393,14 @@ def test_graph_replays_match_eager_steps(device, monkeypatch):
         held.release()
 
 
-def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, monkeypatch):
-    """At batch 1 the q|k|v product of a Q4_K decoder rotates q and k and appends k and v to the
+@pytest.mark.parametrize("shape,element", [(SMALL_Q4, NH_Q4_K), (TINY, NH_Q8_0)], ids=["q4_k", "q8_0"])
+def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, monkeypatch, shape, element):
+    """At batch 1 the q|k|v product of a Q4_K or Q8_0 decoder rotates q and k and appends k and v to the
     caches in its epilogue; the same steps with the rotation as its own kernel give the same
     bits in the caches and the logits."""
-    shape = SMALL_Q4
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
-    folded, ref, weights_a = build(device, shape, NH_Q4_K, batch=1, context=24, seed=9)
-    apart, _, weights_b = build(device, shape, NH_Q4_K, batch=1, context=24, seed=9)
+    folded, ref, weights_a = build(device, shape, element, batch=1, context=24, seed=9)
+    apart, _, weights_b = build(device, shape, element, batch=1, context=24, seed=9)
     token_a = token_b = 5
     for step in range(8):
         monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1")
