@@ -175,7 +175,39 @@ def extras(device, weights, shape, element, context, layers, rng):
     model.release()
     out["prefill_512"] = fill_512(device, weights, shape, element, context, layers, rng)
     out["gemm_config3"] = gemm_config3(device, rng)
+    if element == 12 and not os.environ.get("NEURA_BENCH_SKIP_Q8"):
+        out["decode_0_5b_q8_0"] = small_q8_0_decode(device)
     return out
+
+
+def small_q8_0_decode(device):
+    """The 0.5B-shape Q8_0 decoder (the model of the reference's own CPU-runnable decode case): batch 1, cache filled to 1024,
+    64 greedy steps after 8."""
+    from neura_amd import synth
+    from neura_amd.loader import Model, Weights
+
+    shape, element, context, _, _ = workload("qwen2.5-0.5b-q8_0")
+    rng = np.random.default_rng(0)
+    tensors = list(synth.model_tensors(shape, element, rng, mode="normal"))
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, element, batch=1, context=context)
+    for layer in range(shape["layers"]):
+        for which in (0, 1):
+            model.cache_write(layer, which, rng.standard_normal(model.cache_shape).astype(np.float16).view(np.uint16))
+    steps, warm = 64, 8
+    first, token = context - (steps + warm), 1
+    for step in range(warm + steps):
+        if step == warm:
+            device.sync()
+            began = time.perf_counter()
+        token = int(model.decode_step([token], [first + step])[0])
+    device.sync()
+    elapsed = time.perf_counter() - began
+    model.release()
+    weights.release()
+    return {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
+            "weight_bytes_per_token": weight_bytes_per_token(shape, element, shape["layers"]),
+            "note": "qwen2.5-0.5b shape, Q8_0, 24 layers, batch 1, fp16 KV cache at context %d" % context}
 
 
 def fill_512(device, weights, shape, element, context, layers, rng):
