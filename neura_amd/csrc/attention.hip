@@ -290,19 +290,17 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, 
         const uint32_t s = stripe + 8u * j;
         values[j] = (s < p.sections && c < width) ? src[s * hop + c] : 0.0f;
     }
-    held[tid] = top;
+    // the largest top and the weighed mass: a wave each, then the four waves' words
+    const float wave_top = wave_max(top);
+    if ((tid & 63u) == 0) held[tid >> 6] = wave_top;
     __syncthreads();
-    for (uint32_t stride = 128; stride > 0; stride >>= 1) {
-        if (tid < stride) held[tid] = fmaxf(held[tid], held[tid + stride]);
-        __syncthreads();
-    }
-    const float largest = held[0];
+    const float largest = fmaxf(fmaxf(held[0], held[1]), fmaxf(held[2], held[3]));
     const float weight = top == -INFINITY ? 0.0f : softmax_exp(top - largest);
     weights[tid] = weight;
-    masses[tid] = mass * weight;
+    const float wave_mass = wave_sum(mass * weight);
+    if ((tid & 63u) == 0) masses[tid >> 6] = wave_mass;
     __syncthreads();
-    float total = 0.0f;
-    for (uint32_t s = 0; s < p.sections; s++) total += masses[s];
+    const float total = (masses[0] + masses[1]) + (masses[2] + masses[3]);
     const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
     float sum = 0.0f;
 #pragma unroll
