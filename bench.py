@@ -32,6 +32,11 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.76e6}
 
 
+def note(text):
+    """progress on stderr (stdout carries the one JSON line): names the leg a failure belongs to"""
+    print("[bench] " + text, file=sys.stderr, flush=True)
+
+
 def workload(name):
     """(shape, element of the matrices, context, matrices stored otherwise, layers whose q/k/v carry biases)"""
     from neura_amd import synth
@@ -142,6 +147,7 @@ def extras(device, weights, shape, element, context, layers, rng):
     import neura_amd
 
     out = {}
+    note("extras: sampled decode, batch 1")
     # batch 1 again with a sampled choice (temperature 0.8, 40 candidates, nucleus 0.95; the seed one further a step)
     model = Model(device, weights, shape, element, batch=1, context=context, layers=layers)
     steps, warm = 32, 4
@@ -157,6 +163,7 @@ def extras(device, weights, shape, element, context, layers, rng):
     out["decode_sampled_batch1"] = {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
                                     "note": "as the headline step with the greedy choice replaced by the sampled one; caches not pre-filled (zeros)"}
     model.release()
+    note("extras: decode, batch 8")
     batch = 8
     model = Model(device, weights, shape, element, batch=batch, context=context, layers=layers)
     steps, warm = 16, 4
@@ -173,9 +180,12 @@ def extras(device, weights, shape, element, context, layers, rng):
     out["decode_batch8"] = {"value": batch * steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
                             "note": "8 planes, caches not pre-filled (zeros), cursors at the end of context %d" % context}
     model.release()
+    note("extras: 512-token fill")
     out["prefill_512"] = fill_512(device, weights, shape, element, context, layers, rng)
+    note("extras: wide product of configuration 3")
     out["gemm_config3"] = gemm_config3(device, rng)
     if element == 12 and not os.environ.get("NEURA_BENCH_SKIP_Q8"):
+        note("extras: 0.5B-shape Q8_0 decode")
         out["decode_0_5b_q8_0"] = small_q8_0_decode(device)
     return out
 
@@ -265,8 +275,10 @@ def main():
     rng = np.random.default_rng(0)
     mode = "blocks" if element == 12 else "normal"
     tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers, elements=mixed, biases=biases))
+    note("weights synthesised; opening the device")
     device = neura_amd.Device(0)
     weights = Weights(device, tensors)
+    note("weights resident")
     if args.fill_only:
         print(json.dumps({"prefill_512": fill_512(device, weights, shape, element, context, layers, rng)}))
         weights.release()
@@ -296,15 +308,19 @@ def main():
             return int(model.decode_step_sampled([token], [first_cursor + step], draws)[0])
         return int(model.decode_step([token], [first_cursor + step])[0])
 
+    note("caches filled; warm-up steps")
     for step in range(args.warmup):
         token = one_step(token, step)
+        note("warm-up step %d done" % step)
     device.sync()
+    note("timed steps")
     began = time.perf_counter()
     for step in range(args.steps):
         token = one_step(token, args.warmup + step)
     device.sync()
     elapsed = time.perf_counter() - began
 
+    note("timed steps done; product-only passes")
     # the dominant kernel alone: every narrow product of a decode step (same matrices, shapes
     # and buffers), launched back to back between one pair of HIP events on the same stream
     profiled = min(args.steps, 32)
@@ -350,6 +366,7 @@ def main():
     if not args.no_extras:
         result["extras"] = extras(device, weights, shape, element, context, layers, rng)
     if not args.no_cpu and not mixed:
+        note("CPU baseline")
         host = {name: raw for name, _, _, raw in tensors}
         result["cpu_baseline"] = cpu_baseline(shape, element, host, context, layers)
     else:

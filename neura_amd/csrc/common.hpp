@@ -73,13 +73,17 @@ struct nh_device {
     int32_t compute_units = 0;
     void *scratch = nullptr;  // device scratch, `scratch_bytes` long
     size_t scratch_bytes = 0;
-    // counts the times the scratch or the rope table moved: a captured graph holds their addresses and is
+    std::vector<void *> retired;  // scratch blocks that were outgrown: released by nh_close, never before
+    // counts the times the scratch was replaced by a larger block: a captured graph holds its address and is
     // recorded again when this no longer matches the count at its capture
     uint64_t moved = 0;
     uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
-    float *rope_table = nullptr;  // device inverse frequencies of the last (base, width)
-    float rope_base = 0.0f;
-    uint32_t rope_width = 0;
+    struct RopeTable {
+        float base;
+        uint32_t width;
+        float *table;  // device inverse frequencies pow(base, -2c/width), c < width / 2
+    };
+    std::vector<RopeTable> rope_tables;  // one per (base, width) met so far; entries never move
     // per-launch timing of the narrow products (nh_profile_*): event pairs on the stream
     bool profile = false;
     std::vector<hipEvent_t> profile_events;  // start, stop, start, stop, ...

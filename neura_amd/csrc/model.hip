@@ -46,6 +46,14 @@ struct nh_model {
 
 namespace {
 
+// whether rocprofv3 launched this process: it names its tool library in the environment of what it runs
+bool traced_by_rocprofiler() {
+    const char *tools = getenv("ROCP_TOOL_LIBRARIES");
+    if (tools && tools[0]) return true;
+    const char *preloaded = getenv("LD_PRELOAD");
+    return preloaded && strstr(preloaded, "rocprofiler-sdk") != nullptr;
+}
+
 uint32_t qkv_width(const nh_model *m) { return (m->c.heads + 2 * m->c.kv_heads) * m->c.head_dim; }
 
 void release(nh_model *m) {
@@ -416,8 +424,12 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
              launch_rope_angles(device, c.rope_base, c.head_dim, m->positions, m->rope_cos, m->rope_sin) == NH_OK;
     }
     {
+        // Decode steps replay a recorded HIP graph unless NEURA_HIP_GRAPH=0 -- or the process runs under rocprofv3: with the
+        // profiler's queue interception in place, hipGraphLaunch has died in a host copy past a page-aligned address (the
+        // same address in every such run) once a few thousand packets had gone through the queue, where eager launches of
+        // the same kernels trace cleanly.  Kernel durations are the same either way, so traced runs step eagerly.
         const char *held = getenv("NEURA_HIP_GRAPH");
-        m->use_graph = !(held && held[0] == '0');
+        m->use_graph = !(held && held[0] == '0') && !(held == nullptr && traced_by_rocprofiler());
     }
     ok = ok && hipStreamSynchronize(device->stream) == hipSuccess;
     if (!ok) {

@@ -25,20 +25,16 @@ int32_t hip_fail(hipError_t error, const char *what) {
 
 void *scratch(nh_device *device, size_t bytes) {
     if (bytes <= device->scratch_bytes) return device->scratch;
-    // the stream may still read the old buffer
-    if (hipStreamSynchronize(device->stream) != hipSuccess) {
-        fail(NH_E_DEVICE, "the stream of device %d does not drain before its scratch grows", device->index);
-        return nullptr;
-    }
-    if (device->scratch) (void)hipFree(device->scratch);
-    device->scratch = nullptr;
-    device->scratch_bytes = 0;
+    // The block that is outgrown is kept until nh_close: work already queued on the stream, and any recorded
+    // decode step that has not been recorded again yet, still holds its address, and nothing is released
+    // in the middle of a process (no synchronize, no free).
     size_t wanted = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
     void *held = nullptr;
     if (hipMalloc(&held, wanted) != hipSuccess) {
         fail(NH_E_MEMORY, "device %d holds no %zu bytes of scratch", device->index, wanted);
         return nullptr;
     }
+    if (device->scratch) device->retired.push_back(device->scratch);
     device->scratch = held;
     device->scratch_bytes = wanted;
     device->moved++;
@@ -46,16 +42,13 @@ void *scratch(nh_device *device, size_t bytes) {
 }
 
 const float *rope_frequencies(nh_device *device, float base, uint32_t width) {
-    if (device->rope_table && device->rope_base == base && device->rope_width == width) return device->rope_table;
+    // one table per (base, width) the device has met, kept until nh_close: a table never moves, so decoders of
+    // different head widths or bases can step in turn, each from its own recorded graph
+    for (const nh_device::RopeTable &known : device->rope_tables)
+        if (known.base == base && known.width == width) return known.table;
     // pow(base, -2c/width) in fp32 on the host: crates/neura-kernel/src/task/rope.rs:48-50
     std::vector<float> table(width / 2);
     for (uint32_t c = 0; c < width / 2; c++) table[c] = powf(base, -2.0f * (float)c / (float)width);
-    if (hipStreamSynchronize(device->stream) != hipSuccess) {
-        fail(NH_E_DEVICE, "the stream of device %d does not drain before its rope table changes", device->index);
-        return nullptr;
-    }
-    if (device->rope_table) (void)hipFree(device->rope_table);
-    device->rope_table = nullptr;
     float *held = nullptr;
     if (hipMalloc((void **)&held, table.size() * sizeof(float)) != hipSuccess) {
         fail(NH_E_MEMORY, "device %d holds no rope table of %u channels", device->index, width);
@@ -66,10 +59,7 @@ const float *rope_frequencies(nh_device *device, float base, uint32_t width) {
         fail(NH_E_DEVICE, "device %d takes no rope table", device->index);
         return nullptr;
     }
-    device->rope_table = held;
-    device->moved++;
-    device->rope_base = base;
-    device->rope_width = width;
+    device->rope_tables.push_back({base, width, held});
     return held;
 }
 
@@ -143,8 +133,9 @@ void nh_close(nh_device *device) {
     (void)hipSetDevice(device->index);
     if (device->stream) (void)hipStreamSynchronize(device->stream);
     if (device->scratch) (void)hipFree(device->scratch);
+    for (void *block : device->retired) (void)hipFree(block);
     if (device->refusal) (void)hipFree(device->refusal);
-    if (device->rope_table) (void)hipFree(device->rope_table);
+    for (const nh_device::RopeTable &known : device->rope_tables) (void)hipFree(known.table);
     for (hipEvent_t event : device->profile_events) (void)hipEventDestroy(event);
     if (device->started) (void)hipEventDestroy(device->started);
     if (device->stopped) (void)hipEventDestroy(device->stopped);

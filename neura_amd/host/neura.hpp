@@ -358,7 +358,10 @@ inline Header parse(const uint8_t *bytes, size_t size) {
                       (unsigned long long)tensor.elements, neura::name(*element), neura::name(*element), held->elements);
             tensor.bytes = tensor.elements / held->elements * held->bytes;
         } else {
-            tensor.bytes = tensor.elements * bits_per_element(*element) / 8;
+            uint64_t bits = 0;
+            if (__builtin_mul_overflow(tensor.elements, (uint64_t)bits_per_element(*element), &bits))
+                panic("the tensor %s spans more bytes than a gguf counts", name.c_str());
+            tensor.bytes = bits / 8;
         }
         header.tensors.emplace_back(std::move(name), tensor);
     }
@@ -368,10 +371,12 @@ inline Header parse(const uint8_t *bytes, size_t size) {
 
 inline void bounds(const Header &header, uint64_t held, const std::string &what) {  // crates/neura-gguf/src/lib.rs:225-233
     for (auto &entry : header.tensors) {
-        uint64_t end = header.data + entry.second.at + entry.second.bytes;
-        if (end > held)
+        // checked sums: an offset near 2^64 must not wrap to an end inside the file
+        uint64_t start = 0, end = 0;
+        const bool wraps = __builtin_add_overflow(header.data, entry.second.at, &start) || __builtin_add_overflow(start, entry.second.bytes, &end);
+        if (wraps || end > held)
             panic("%s holds %llu bytes where the tensor %s runs to byte %llu", what.c_str(), (unsigned long long)held, entry.first.c_str(),
-                  (unsigned long long)end);
+                  (unsigned long long)(wraps ? UINT64_MAX : end));
     }
 }
 

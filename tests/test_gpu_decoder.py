@@ -270,10 +270,11 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
     """The 7B shape itself (hidden 3584, 28 query heads over 4 key heads of 128, ffn 18944, vocabulary 152064, random Q4_K
     blocks, separate head) cut to two layers, at context 4096: decode steps at batch 1 on caches filled with N(0,1) halves
     (the products at their real depths and row counts, the rotation folded in, attention over 4000 keys in sections), a
-    64-row fill (wide products with stacked q|k|v and fused packing passes, attention over a chunk), and a step of eight
-    planes (the half-precision tiles on gate|up and the head, the integer tiles on the rest), each against the oracle."""
+    512-row fill, the prompt chunk of the benchmark (wide products with stacked q|k|v and fused packing passes, attention
+    over a chunk), and a step of eight planes (the half-precision tiles on gate|up and the head, the integer tiles on the
+    rest), each against the oracle: logits within 1e-3 of the largest, the greedy token identical at every step."""
     shape = synth.SHAPES["qwen2.5-7b"]
-    layers, context, filled, rows = 2, 4096, 4000, 64
+    layers, context, filled, rows = 2, 4096, 3500, 512
     rng = np.random.default_rng(50)
     tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks", layers=layers))
     host = {name: raw for name, _, _, raw in tensors}
@@ -296,30 +297,71 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
         logits = model.logits()
         scale = np.abs(want_logits).max()
         assert np.abs(logits - want_logits).max() <= 1e-3 * scale, what
-        for plane, gap in enumerate(margins(want_logits)):
-            if gap > 2e-3 * scale:
-                assert got[plane] == want[plane], (what, plane, gap)
+        gaps = margins(want_logits)
+        print("%s: top-2 margins min %.3g of a largest logit of %.3g, logits within %.3g" % (what, gaps.min(), scale, np.abs(logits - want_logits).max()))
+        assert [int(t) for t in got] == [int(t) for t in want], (what, gaps)
         return [int(t) for t in want]
 
     model, ref = pair(1, rows)
     token = [int(rng.integers(0, shape["vocab"]))]
     for step in range(3):
         token = same(model, ref, token, [filled + step], "batch 1, step %d" % step)
-    # a fill of 64 rows over positions 100 .. 163, then a step that weighs what it wrote
+    # a fill of 512 rows behind the keys already held (positions 3503 .. 4014), then a step that weighs what it wrote
     prompt = rng.integers(0, shape["vocab"], rows)
-    model.prefill(prompt, rows, [100])
-    ref.forward(prompt, rows, [100], want_logits=False, threads=16)
+    first = filled + 3
+    model.prefill(prompt, rows, [first])
+    ref.forward(prompt, rows, [first], want_logits=False, threads=16)
     for layer in range(layers):
         for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-            got_rows = oracle.f16_to_f32(model.cache_read(layer, which)[:, :, 100:100 + rows].reshape(-1))
-            want_rows = oracle.f16_to_f32(held[layer].reshape(model.cache_shape)[:, :, 100:100 + rows].reshape(-1))
+            got_rows = oracle.f16_to_f32(model.cache_read(layer, which)[:, :, first:first + rows].reshape(-1))
+            want_rows = oracle.f16_to_f32(held[layer].reshape(model.cache_shape)[:, :, first:first + rows].reshape(-1))
             assert np.abs(got_rows - want_rows).max() <= 2e-3 * max(1.0, np.abs(want_rows).max()), (layer, which)
-    same(model, ref, token, [filled + 3], "batch 1 after the fill")
+    same(model, ref, token, [first + rows], "batch 1 after the 512-row fill")
     model.release()
     model, ref = pair(8, 1)
     tokens = [int(t) for t in rng.integers(0, shape["vocab"], 8)]
     for step in range(2):
         tokens = same(model, ref, tokens, [filled - 7 * plane + step for plane in range(8)], "batch 8, step %d" % step)
+    model.release(), weights.release()
+
+
+def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device):
+    """The model the benchmark times, whole: 28 layers of the 7B shape, random Q4_K blocks, a separate head, fp16 caches
+    holding 4032 positions of N(0,1) halves, then 64 greedy steps up to the end of the context of 4096 -- every token
+    identical to the oracle's, with no allowance for close calls.  The oracle follows the reference's summation order;
+    identity against the reference binary itself is unpinned (it cannot be run here)."""
+    shape = synth.SHAPES["qwen2.5-7b"]
+    context, steps = 4096, 64
+    filled = context - steps
+    rng = np.random.default_rng(52)
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks"))
+    host = {name: raw for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, NH_Q4_K, 1, context, 1)
+    ref = oracle.Model(shape, NH_Q4_K, host, 1, context, 1)
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            halves = np.zeros(model.cache_shape, dtype=np.float16)
+            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
+            held[layer][:] = halves.view(np.uint16).reshape(-1)
+            model.cache_write(layer, which, halves.view(np.uint16))
+    got = want = int(rng.integers(0, shape["vocab"]))
+    got_tokens, want_tokens, gaps, apart = [], [], [], []
+    for step in range(steps):
+        want_logits, chosen = ref.forward([want], 1, [filled + step], threads=16)
+        want = int(chosen[0])
+        got = int(model.decode_step([got], [filled + step])[0])
+        want_tokens.append(want), got_tokens.append(got)
+        gaps.append(float(margins(want_logits)[0]))
+        apart.append(float(np.abs(model.logits() - want_logits).max() / np.abs(want_logits).max()))
+        if step % 8 == 7:
+            print("step %d: tokens identical so far, smallest top-2 margin %.3g" % (step, min(gaps)), flush=True)
+        if got != want:
+            break
+    print("greedy margins (top1 - top2) over %d steps: min %.3g median %.3g; logits within %.3g of the largest" %
+          (len(gaps), min(gaps), float(np.median(gaps)), max(apart)))
+    assert max(apart) <= 1e-3
+    assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
     model.release(), weights.release()
 
 
@@ -349,8 +391,7 @@ def test_config5_shape_stored_as_a_q4_k_m_file_stores_it(device):
         got = model.decode_step(token, [filled + step])
         scale = np.abs(want_logits).max()
         assert np.abs(model.logits() - want_logits).max() <= 1e-3 * scale, step
-        if margins(want_logits)[0] > 2e-3 * scale:
-            assert int(got[0]) == int(want[0]), (step, margins(want_logits))
+        assert int(got[0]) == int(want[0]), (step, margins(want_logits))
         token = [int(want[0])]
     model.release(), weights.release()
 
@@ -423,6 +464,28 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         folded.decode_step([1], [folded.capacity + 3])
     for held in (folded, apart, weights_a, weights_b):
         held.release()
+
+
+def test_decoders_of_different_rope_bases_step_in_turn(device):
+    """Two decoders of different rope bases and head widths stepping alternately at batch 2 (the rotation as its own
+    kernel, read from the device's table of inverse frequencies): each keeps answering from its own recorded step as the
+    oracle does, whatever table the other one asked for in between."""
+    first, ref_a, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=2, context=24, seed=21)
+    tensors_b = list(synth.model_tensors(TINY, NH_Q8_0, np.random.default_rng(22), mode="normal"))
+    weights_b = Weights(device, tensors_b)
+    second = Model(device, weights_b, TINY, NH_Q8_0, 2, 24, 1, rope_base=1e4)
+    ref_b = oracle.Model(TINY, NH_Q8_0, {name: raw for name, _, _, raw in tensors_b}, 2, 24, 1, rope_base=1e4)
+    tokens_a, tokens_b = [3, 4], [5, 6]
+    for step in range(6):
+        want_logits, want = ref_a.forward(tokens_a, 1, [step, step])
+        tokens_a = list(first.decode_step(tokens_a, [step, step]))
+        assert np.abs(first.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert tokens_a == list(want), step
+        want_logits, want = ref_b.forward(tokens_b, 1, [step, step])
+        tokens_b = list(second.decode_step(tokens_b, [step, step]))
+        assert np.abs(second.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert tokens_b == list(want), step
+    first.release(), second.release(), weights_a.release(), weights_b.release()
 
 
 def test_a_recorded_step_survives_a_scratch_that_moves(device):

@@ -289,6 +289,21 @@ def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
     close(device.gemm(element, raw, N, K, X, residual=r), want + r)
 
 
+def test_config3_wide_product_at_full_size(device):
+    """The wide product of the benchmark as it is timed: M = 512, K = 3584, N = 18944 (148 column tiles by 4 row tiles),
+    random Q4_K blocks, half activations N(0,1), every one of the 9.7 million outputs against fp32 accumulation."""
+    M, K, N = 512, 3584, 18944
+    rng = np.random.default_rng(33)
+    raw = synth.q4_k_random(rng, N * K)
+    X = rng.standard_normal((M, K)).astype(np.float16)
+    want = oracle.gemm(NH_Q4_K, raw, N, K, X.astype(np.float32), threads=16)
+    got = device.gemm(NH_Q4_K, raw, N, K, X)
+    close(got, want)
+    # and with the decoder's fp32 activations
+    X32 = rng.standard_normal((M, K)).astype(np.float32)
+    close(device.gemm(NH_Q4_K, raw, N, K, X32), oracle.gemm(NH_Q4_K, raw, N, K, X32, threads=16))
+
+
 # ------------------------------------------------------------------ row operators
 
 @pytest.mark.parametrize("C", [896, 1536, 3584, 100])

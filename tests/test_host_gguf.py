@@ -117,6 +117,20 @@ def test_a_gguf_refuses_a_file_that_does_not_follow_its_layout():
     refuses(lambda: host.Gguf.decode(flagged), "where a flag holds zero or one")
 
 
+def test_a_gguf_refuses_offsets_and_sizes_that_wrap_around():
+    """A crafted table whose offset sits just below 2^64, or whose tensor spans more bytes than 2^64 counts, must not wrap
+    to an end inside the file: the reader copies payloads with memcpy, where the reference's slices would panic."""
+    good, _, _ = build(32, ALIGN, [("weights", 8, [32], bytes(34))])
+    at = good.index(b"weights") + len(b"weights") + 4 + 8 + 4  # rank, one dimension, ggml type: then the offset
+    assert good[at:at + 8] == bytes(8)
+    far = good[:at] + (2 ** 64 - 32).to_bytes(8, "little") + good[at + 8:]
+    refuses(lambda: host.Gguf.decode(far), "where the tensor weights runs to byte")
+    huge, _, _ = build(32, ALIGN, [("wide", 0, [2 ** 62, 2], bytes(32))])  # 2^63 floats: 2^65 bytes
+    refuses(lambda: host.Gguf.decode(huge), "wide", "more bytes than a gguf counts")
+    big, _, _ = build(32, ALIGN, [("wide", 0, [2 ** 58], bytes(32))])  # 2^60 bytes: counted, but far past the file
+    refuses(lambda: host.Gguf.decode(big), "where the tensor wide runs to byte")
+
+
 def test_a_gguf_without_an_alignment_key_aligns_by_thirty_two_and_reads_version_two():
     data, start, at = build(32, [("general.name", "string", "x")], [("a", 0, [3], bytes(12)), ("b", 0, [2, 2], bytes(range(16)))], version=2)
     gguf = host.Gguf.decode(data)
