@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBRARY = os.path.join(HERE, "libneura_hip.so")
-SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "sample.hip", "model.hip"]
+SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemv_tile16.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "sample.hip", "model.hip"]
 FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -26,9 +26,13 @@ def hipcc():
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
+# per file: the 16-row tile product weighs its matrix-core sums where they land, in vector registers
+EXTRA_FLAGS = {"gemv_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _compile(source):
     obj = os.path.join(CSRC, source.replace(".hip", ".o"))
-    cmd = [hipcc(), *FLAGS, "-c", os.path.join(CSRC, source), "-o", obj]
+    cmd = [hipcc(), *FLAGS, *EXTRA_FLAGS.get(source, []), "-c", os.path.join(CSRC, source), "-o", obj]
     done = subprocess.run(cmd, capture_output=True, text=True)
     if done.returncode != 0:
         raise RuntimeError("hipcc failed on %s:\n%s\n%s" % (source, " ".join(cmd), done.stderr))

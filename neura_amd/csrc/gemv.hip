@@ -11,36 +11,11 @@
 // into LDS with aligned 128-bit loads and each lane then reads its own block from LDS.
 #include "blocks.hpp"
 #include "common.hpp"
+#include "gemv_shared.hpp"
 
 #include <cstdlib>
 
 namespace nh {
-
-struct GemvParams {
-    const uint8_t *W[3];  // up to three matrices stacked along N (q|k|v, or gate|up with swiglu)
-    uint32_t end[3];      // first output row past each matrix
-    const float *x;
-    float *y;
-    const float *residual;
-    const float *norm_w;
-    float *partial;
-    uint32_t N, K, row_bytes;
-    uint32_t nblk;              // blocks per row
-    uint32_t blocks_per_split;  // blocks of one K slice
-    uint32_t splits;
-    uint32_t group;             // lanes that share one output row: 16, 32 or 64
-    uint32_t row_groups;        // passes over the rows
-    uint32_t chunks_per_row;    // Q8_0: 16-byte chunks of a staged row slice
-    int32_t swiglu;
-    float eps;
-    // rotation folded into the product (decode kernel only): see RopeFusion
-    const float *rope_cosines, *rope_sines;  // [position][width / 2]
-    const uint32_t *rope_cursor;
-    uint16_t *rope_k, *rope_v;
-    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
-    uint32_t *refusal;
-    const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
-};
 
 // skewed LDS index of activation i: 4 floats of padding per 64 keep 128-bit reads of
 // neighbouring lanes on different banks
@@ -111,8 +86,6 @@ __device__ __forceinline__ void stage_row(const float *__restrict__ x, uint32_t 
     }
 }
 
-__device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
-
 // logical row i of a pass -> output row.  With swiglu, even i walk the gate rows and odd i the
 // up rows so that one lane group ends up holding both halves of an output.
 __device__ __forceinline__ uint32_t weight_row(uint32_t i, uint32_t N, int32_t swiglu) {
@@ -171,8 +144,6 @@ __device__ __forceinline__ void publish(const GemvParams &p, uint32_t first, uin
 
 // ---------------------------------------------------------------------------- Q4_K -------
 
-typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // Sum over the 32 low-nibble and the 32 high-nibble weights of 8 words against xl / xh.
 // A nibble masked in place inside a 16-bit lane IS a half-precision subnormal: bits 0..3 read
@@ -228,15 +199,6 @@ __device__ __forceinline__ void group_scales(const uint4 &hdr, uint32_t g, float
     m1 = dmin * (float)mn1;
 }
 
-// ---- cross-lane sums without LDS round trips ---------------------------------------------
-template <int CTRL>
-__device__ __forceinline__ float dpp(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
-}
-constexpr int DPP_QUAD_XOR1 = 0xB1;  // quad_perm [1,0,3,2]
-constexpr int DPP_QUAD_XOR2 = 0x4E;  // quad_perm [2,3,0,1]
-constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;
-
 // Sums R per-lane partials over the G lanes of a row group.  The first log2(R) steps fold two
 // rows into one register (each lane keeps the row its own index selects), so R rows cost
 // R - 1 + log2(G / R) exchanges instead of R log2(G); steps inside a row of 16 lanes are DPP
@@ -266,35 +228,6 @@ __device__ __forceinline__ float fold_rows(float (&acc)[R], uint32_t lane) {
     if (G >= 32) v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
     if (G >= 64) v += __shfl_xor(v, 32, 64);
     return v;
-}
-
-// Per-lane constants of the branch-free scale decode (they depend on the lane's group only).
-struct ScaleLane {
-    uint32_t pick;    // byte selector: the two bytes of this group from the low or the high scale word
-    uint32_t pick_q;  // byte selector: the two bytes that carry the top bits (groups 2, 3)
-    uint32_t mask_p, mask_q;
-    uint32_t shift_m;  // 4 for groups 2, 3: their minimums sit in the high nibbles
-};
-
-__device__ __forceinline__ ScaleLane scale_lane(uint32_t g) {
-    const uint32_t j = 2u * (g & 1u);
-    ScaleLane s;
-    s.pick_q = 0x0c000c00u | j | ((j + 1u) << 16);
-    s.pick = g < 2 ? s.pick_q : (0x0c000c00u | (4u + j) | ((5u + j) << 16));
-    s.mask_p = g < 2 ? 0x003f003fu : 0x000f000fu;
-    s.mask_q = g < 2 ? 0u : 0x00300030u;
-    s.shift_m = g < 2 ? 0u : 4u;
-    return s;
-}
-
-// The 6-bit scales (sc) and minimums (mn) of sub-blocks 2g, 2g+1 as pairs of half-precision
-// subnormals (value * 2^-24 in each 16-bit lane), straight from the header words:
-// crates/neura-precision/src/ggml.rs:127-136 without a branch or an int -> float conversion.
-__device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s, half2_t &sc, half2_t &mn) {
-    const uint32_t p_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick), q_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick_q);
-    const uint32_t p_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick) >> s.shift_m, q_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick_q);
-    sc = __builtin_bit_cast(half2_t, (p_sc & s.mask_p) | ((q_sc >> 2) & s.mask_q));
-    mn = __builtin_bit_cast(half2_t, (p_mn & s.mask_p) | ((q_mn >> 2) & s.mask_q));
 }
 
 // The epilogue of a q|k|v product that folds the rotation in: lane u < R of a lane group holds logical row i = first + u, and
@@ -1118,18 +1051,10 @@ struct MfmaUnit {
     u32x4 hdr, qa, qb;
 };
 
-template <int CTRL>
-__device__ __forceinline__ int dpp_int(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
-}
 
 // KS waves share one tile (each takes every KS-th super-block of the slice); NW waves per
 // workgroup; P activation rows; D super-blocks in flight per wave (the loads run ahead of the
 // arithmetic across tile boundaries, and the first ones are issued before the activations are staged).
-// The four signed base-256 digits of an integer below 2^30 in magnitude, one per byte, least significant in byte 0:
-// adding 128 at the three low byte positions makes every low byte the digit plus 128 (the carries are the ones the
-// signed digits need), and flipping bit 7 takes the 128 off again.
-__device__ __forceinline__ uint32_t signed_digits(int whole) { return ((uint32_t)whole + 0x00808080u) ^ 0x00808080u; }
 
 // Digit planes of four elements: plane[0] holds their most significant digits (element e in byte e), plane[3] the least.
 __device__ __forceinline__ void digit_planes(uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3, uint32_t (&plane)[4]) {
@@ -2078,10 +2003,6 @@ static uint32_t pow2_at_least(uint32_t v, uint32_t floor) {
     return p;
 }
 
-static int env_int(const char *name, int fallback) {
-    const char *held = getenv(name);
-    return held && *held ? atoi(held) : fallback;
-}
 
 template <int RB>
 static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
@@ -2385,6 +2306,11 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
 bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     if (env_int("NEURA_HIP_FUSE_ROPE", 1) == 0) return false;
     if (a.rows != 1 || a.swiglu || a.residual) return false;
+    {
+        GemvArgs folded = a;
+        folded.rope = &rope;
+        if (tile16_takes(folded)) return true;
+    }
     if (a.element == NH_Q8_0) {
         // the direct Q8_0 decode kernel, a row of blocks inside one wave
         if (a.K % 32u != 0 || a.K > 2048u || env_int("NEURA_HIP_Q8_DECODE", 1) == 0) return false;
@@ -2611,6 +2537,8 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
 }
 
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
+    if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (tile16_takes(a)) return launch_tile16(d, a);
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
     if (f16_tiles_take(d, a)) return launch_f16_tiles(d, a);

@@ -1,0 +1,136 @@
+// What the narrow-product kernels of gemv.hip and gemv_tile16.hip share: the kernel parameters, the branch-free decode of
+// the Q4_K block scales, lane exchanges and the rotation's epilogue.
+#pragma once
+#include "blocks.hpp"
+#include "common.hpp"
+
+#include <cstdlib>
+
+namespace nh {
+
+struct GemvParams {
+    const uint8_t *W[3];  // up to three matrices stacked along N (q|k|v, or gate|up with swiglu)
+    uint32_t end[3];      // first output row past each matrix
+    const float *x;
+    float *y;
+    const float *residual;
+    const float *norm_w;
+    float *partial;
+    uint32_t N, K, row_bytes;
+    uint32_t nblk;              // blocks per row
+    uint32_t blocks_per_split;  // blocks of one K slice
+    uint32_t splits;
+    uint32_t group;             // lanes that share one output row: 16, 32 or 64
+    uint32_t row_groups;        // passes over the rows
+    uint32_t chunks_per_row;    // Q8_0: 16-byte chunks of a staged row slice
+    int32_t swiglu;
+    float eps;
+    // rotation folded into the product (decode kernel only): see RopeFusion
+    const float *rope_cosines, *rope_sines;  // [position][width / 2]
+    const uint32_t *rope_cursor;
+    uint16_t *rope_k, *rope_v;
+    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
+    uint32_t *refusal;
+    const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
+};
+
+__device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---- cross-lane sums without LDS round trips ---------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;  // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;
+
+// Per-lane constants of the branch-free scale decode (they depend on the lane's group only).
+struct ScaleLane {
+    uint32_t pick;    // byte selector: the two bytes of this group from the low or the high scale word
+    uint32_t pick_q;  // byte selector: the two bytes that carry the top bits (groups 2, 3)
+    uint32_t mask_p, mask_q;
+    uint32_t shift_m;  // 4 for groups 2, 3: their minimums sit in the high nibbles
+};
+
+__device__ __forceinline__ ScaleLane scale_lane(uint32_t g) {
+    const uint32_t j = 2u * (g & 1u);
+    ScaleLane s;
+    s.pick_q = 0x0c000c00u | j | ((j + 1u) << 16);
+    s.pick = g < 2 ? s.pick_q : (0x0c000c00u | (4u + j) | ((5u + j) << 16));
+    s.mask_p = g < 2 ? 0x003f003fu : 0x000f000fu;
+    s.mask_q = g < 2 ? 0u : 0x00300030u;
+    s.shift_m = g < 2 ? 0u : 4u;
+    return s;
+}
+
+// The 6-bit scales (sc) and minimums (mn) of sub-blocks 2g, 2g+1 as pairs of half-precision
+// subnormals (value * 2^-24 in each 16-bit lane), straight from the header words:
+// crates/neura-precision/src/ggml.rs:127-136 without a branch or an int -> float conversion.
+__device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s, half2_t &sc, half2_t &mn) {
+    const uint32_t p_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick), q_sc = __builtin_amdgcn_perm(hdr.w, hdr.y, s.pick_q);
+    const uint32_t p_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick) >> s.shift_m, q_mn = __builtin_amdgcn_perm(hdr.w, hdr.z, s.pick_q);
+    sc = __builtin_bit_cast(half2_t, (p_sc & s.mask_p) | ((q_sc >> 2) & s.mask_q));
+    mn = __builtin_bit_cast(half2_t, (p_mn & s.mask_p) | ((q_mn >> 2) & s.mask_q));
+}
+
+// One rotated output of a q|k|v product that folds the rotation in: `total` is output row n (channel c of its head's first
+// half, or c + width/2 when `second`), the lane 8 further round its row of 16 holds the partner channel.  The projection's
+// bias, if it has one, comes before the rotation; q rows go to y, k rows rotated and v rows as they are to the caches as
+// halves, at the cursor (at cursor mod span in a ring).  Lanes 0..15 of a wave call it together
+// (crates/neura-kernel/src/task/rope.rs:95-122).
+__device__ __forceinline__ void rope_store(const GemvParams &p, float total, uint32_t n, uint32_t c, bool second) {
+    const uint32_t half = p.rope_width >> 1;
+    {
+        const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
+        const uint32_t e0 = p.end[0], e1 = p.end[1];
+        const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
+        const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
+        if (bias) total += bias[n - before];
+    }
+    const float other = dpp<DPP_ROW_ROR8>(total);
+    const uint32_t position = p.rope_cursor[0];
+    float value = total;
+    if (n < p.rope_k_rows) {
+        // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
+        const float cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+        const float sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+        value = second ? total * cosine + other * sine : total * cosine - other * sine;
+    }
+    if (n < p.rope_q_rows) {
+        p.y[n] = value;
+    } else if (position >= p.rope_positions || (!p.rope_ring && position >= p.rope_capacity)) {
+        atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+    } else {
+        const bool key = n < p.rope_k_rows;
+        const uint32_t within = n - (key ? p.rope_q_rows : p.rope_k_rows);  // head * width + channel
+        const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
+        uint16_t *cache = key ? p.rope_k : p.rope_v;
+        const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
+        cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
+    }
+}
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_int(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+
+// The four signed base-256 digits of an integer below 2^30 in magnitude, one per byte, least significant in byte 0:
+// adding 128 at the three low byte positions makes every low byte the digit plus 128 (the carries are the ones the
+// signed digits need), and flipping bit 7 takes the 128 off again.
+__device__ __forceinline__ uint32_t signed_digits(int whole) { return ((uint32_t)whole + 0x00808080u) ^ 0x00808080u; }
+
+inline int env_int(const char *name, int fallback) {
+    const char *held = getenv(name);
+    return held && *held ? atoi(held) : fallback;
+}
+
+// the 16-row tile kernel (gemv_tile16.hip): whether it serves this product, and its launch
+bool tile16_takes(const GemvArgs &args);
+int32_t launch_tile16(nh_device *d, const GemvArgs &args);
+
+}  // namespace nh

@@ -1,0 +1,395 @@
+// The Q4_K product of one activation row on 16-row tiles of the 16x16x64 integer MFMA: kernel and launcher.
+// Built with the matrix-core results in vector registers (-amdgpu-mfma-vgpr-form): the sums are weighed right where they land.
+#include "gemv_shared.hpp"
+
+namespace nh {
+
+// ---------------------------------------------------------------------------------------------------------------------
+// One activation row against a Q4_K matrix on 16-row tiles of v_mfma_i32_16x16x64_i8: the decode step's product.
+//
+// A wave step covers one super-block of 16 rows.  Lane (r, q) = (lane % 16, lane / 16) fetches the 32 nibble bytes of
+// group q of row r (two 128-bit loads) and the block header, and unpacks them with two masks and a shift a word into the B
+// operands of four MFMAs: the sixteen low nibbles of each load are K slice q of one instruction, the high nibbles of
+// another.  The activations are the A operand: row m = 4 * slice + plane holds one of three signed base-256 digit planes of
+// the sixteen activations slice `slice` meets and zeros everywhere else, so C comes back with lane (r, q) holding the three
+// plane sums of ITS OWN weights -- no sum crosses lanes and the lane that holds a sum holds the header that weighs it.  The
+// digits carry 22 bits below a power-of-two scale per 64-element group (exact for the group's largest magnitudes, finer
+// than fp32 rounding of the products for the rest), so the integer arithmetic is exact and what is left to fp32 is
+// d * (sc . sums) - dmin * (m . activation sums) per group, as the reference weighs it (crates/neura-kernel/src/dot.rs:583-619).
+//
+// NW waves share a tile, wave w taking super-blocks w, w + NW, ... (and turning exactly those activations into digits,
+// in its own corner of LDS, so no barrier stands between staging and walking); their sixteen partial sums meet in LDS once
+// a tile.  Loads run D steps ahead across tile boundaries; workgroups take tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+// so that the device as a whole walks one window of the matrix from end to end.
+// 0.9 vector instructions a weight (the vector kernel above: 2.4) with the multiply-adds on the matrix cores.
+// Epilogues: y (+ in-place residual by one fire-and-forget add), SwiGLU over a gate tile and the up tile behind it, or the
+// rotation with the cache append (tile rows = 8 channels c.. and their partners c + width/2.. of one head).
+constexpr uint32_t TILE16_BLOCK_DIGITS = 768;  // 16 chunks of 16 activations x 3 planes x 16 bytes
+constexpr uint32_t TILE16_ZERO_BYTES = 208;    // what an idle A lane reads: four chunk offsets (0, 48, 96, 144) + 16 bytes
+enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2 };
+
+static size_t tile16_lds(uint32_t nblk, uint32_t NW) {
+    return (size_t)nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + (size_t)nblk * 64u + (size_t)2 * NW * 16u * 4u + (size_t)NW * 4u + 64u;
+}
+
+struct Tile16Unit {
+    u32x4 hdr, qa, qb;
+};
+
+template <int NW, int D, int MODE>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
+    constexpr uint32_t NT = NW * 64;
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t nblk = p.nblk;
+    uint8_t *const digits = tile16_lds_bytes;
+    uint8_t *const zeros = tile16_lds_bytes + (size_t)nblk * TILE16_BLOCK_DIGITS + wave * TILE16_ZERO_BYTES;  // a wave's own zeros
+    f32x4 *const sums = reinterpret_cast<f32x4 *>(tile16_lds_bytes + (size_t)nblk * TILE16_BLOCK_DIGITS + NW * TILE16_ZERO_BYTES);
+    float *const part = reinterpret_cast<float *>(sums + (size_t)nblk * 4u);
+    float *const red = part + 2u * NW * 16u;
+
+    const uint32_t r = lane & 15u, q = lane >> 4;
+    // tiles of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
+    const uint32_t tiles = p.row_groups;
+    if (blockIdx.x >= tiles) return;  // the whole workgroup: no barrier has been reached
+    const uint32_t ntiles = (tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;  // super-blocks of one tile this wave walks
+
+    // the weight row lane r reads in tile `tile`; with the rotation folded in a tile holds channels c0 .. c0 + 7 of a head and
+    // their partners half a head further (written with selects over scalars captured by value: nothing here may end up indexed)
+    const uint8_t *const w0 = p.W[0];
+    const int64_t to_w1 = p.W[1] - p.W[0], to_w2 = p.W[2] - p.W[0];
+    const uint32_t end0 = p.end[0], end1 = p.end[1];
+    const uint32_t row_bytes = p.row_bytes;
+    const uint32_t half_width = p.rope_width >> 1, tiles_per_head = max(half_width >> 3, 1u);
+    const uint32_t first_tile = blockIdx.x, hop = gridDim.x;
+    auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, r, q](uint32_t tile) -> const uint8_t * {
+        int64_t offset;
+        if (MODE == TILE16_SWIGLU) {
+            offset = ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((tile >> 1) * 16u + r) * row_bytes;
+        } else {
+            uint32_t n = tile * 16u + r;
+            if (MODE == TILE16_ROPE) n = (tile / tiles_per_head) * (2u * half_width) + (tile % tiles_per_head) * 8u + (r & 7u) + (r >> 3) * half_width;
+            const bool in0 = n < end0, in1 = n < end1;
+            const int64_t matrix = in0 ? (int64_t)0 : (in1 ? to_w1 : to_w2);
+            const uint32_t before = in0 ? 0u : (in1 ? end0 : end1);
+            offset = matrix + (int64_t)(n - before) * row_bytes;
+        }
+        return w0 + offset + q * 32u;
+    };
+    // with SwiGLU the workgroup's unit of work is a pair: tiles 2j (gate) and 2j + 1 (up)
+    auto tile_at = [first_tile, hop](uint32_t i) -> uint32_t {
+        if (MODE == TILE16_SWIGLU) return 2u * (first_tile + (i >> 1) * hop) + (i & 1u);
+        return first_tile + i * hop;
+    };
+    const uint32_t walked = MODE == TILE16_SWIGLU ? 2u * ntiles : ntiles;  // tiles this workgroup walks
+
+    // Loads run D steps ahead of the arithmetic, across tile boundaries.  Every fetch issues its three loads: past the last
+    // step the last unit is fetched again and dropped, so that every path issues the same loads in the same order and the
+    // waits count exactly how many loads are newer than the one needed.
+    Tile16Unit ring[D];
+    uint32_t ahead_tile = 0, ahead_b = wave;
+    const uint8_t *ahead_row = lane_row(tile_at(0));
+    auto fetch = [&](Tile16Unit &u) {
+        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * 144u;
+        u.hdr = *(global_uint4)(uintptr_t)(at - q * 32u);
+        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
+        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+        if (ahead_b + NW < nblk) {
+            ahead_b += NW;
+        } else if (ahead_tile + 1u < walked) {
+            ahead_b = wave;
+            ahead_tile++;
+            ahead_row = lane_row(tile_at(ahead_tile));
+        }
+    };
+
+    // ---- activations -> three signed base-256 digit planes per 16 elements, a power-of-two scale per 64-element group.
+    // Unit e4 = tid + NT * j (four consecutive activations) lies in super-block wave + NW * j: a wave turns into digits
+    // exactly the super-blocks it multiplies.
+    {
+        const uint32_t units = p.K / 4u;
+        constexpr int MAXJ = 5;
+        f32x4 held[MAXJ], weight[MAXJ];
+        const bool resident = units <= MAXJ * NT;
+        float rms = 1.0f;
+        if (lane < TILE16_ZERO_BYTES / 4u) reinterpret_cast<uint32_t *>(zeros)[lane] = 0u;
+        if (resident) {
+#pragma unroll
+            for (int j = 0; j < MAXJ; j++) {
+                const uint32_t e4 = tid + NT * j;
+                held[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(p.x + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            if (p.norm_w) {
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    weight[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+        // the weights' loads go out behind the activations', which everything waits for first
+#pragma unroll
+        for (int i = 0; i < D; i++) fetch(ring[i]);
+        if (p.norm_w) {
+            // sum of squares of the whole row (crates/neura-kernel/src/task/norm.rs:69-83; the same fp32 adds in another order)
+            float square = 0.0f;
+            if (resident) {
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(held[j][i], held[j][i]));
+            } else {
+                for (uint32_t e4 = tid; e4 < units; e4 += NT) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(p.x + 4u * e4);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
+                }
+            }
+            square = wave_sum(square);
+            if (lane == 0) red[wave] = square;
+            __syncthreads();
+            float total = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) total += red[w];
+            rms = rms_scale_of(total, p.K, p.eps);
+        }
+        auto stage = [&](uint32_t e4, f32x4 v, f32x4 w) {
+            if (p.norm_w) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
+            }
+            uint32_t top = 0;  // largest magnitude of the group as bits: infinities and NaNs sort above every finite value
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float element = v[i];  // a copy first: the bits of a vector element taken in place read element 0 every time
+                top = max(top, __builtin_bit_cast(uint32_t, element) & 0x7fffffffu);
+            }
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
+            const uint32_t raw = top >> 23;
+            const uint32_t exponent = min(max(raw, 22u), 254u);
+            const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);  // the group's largest magnitude lands in [2^21, 2^22)
+            const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
+            float total = 0.0f;
+            uint32_t dg[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float rounded = rintf(v[i] * scale);
+                total += rounded;
+                dg[i] = signed_digits((int)rounded);  // bytes 0..2: signed digits, least significant first; byte 3 is zero below 2^23
+            }
+            const uint32_t lo01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x07030602u);
+            const uint32_t plane2 = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);  // digit 0 (least significant) of the four elements
+            const uint32_t plane1 = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+            const uint32_t plane0 = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  // digit 2 (most significant)
+            total += dpp<DPP_QUAD_XOR1>(total);
+            total += dpp<DPP_QUAD_XOR2>(total);
+            total += dpp<0x141>(total);  // half mirror: the other quad of the eight lanes of a sub-block
+            // unit e4: 64 units a super-block, 16 a group, 8 a sub-block, 4 a chunk of 16 elements
+            uint32_t *slot = reinterpret_cast<uint32_t *>(digits + (size_t)(e4 >> 2) * 48u) + (e4 & 3u);
+            slot[0] = plane0, slot[4] = plane1, slot[8] = plane2;
+            float *s = reinterpret_cast<float *>(sums + (e4 >> 4));  // (low sub-block sum, high sub-block sum, unscale, -)
+            if ((e4 & 7u) == 0) s[(e4 >> 3) & 1u] = total * unscale;
+            if ((e4 & 15u) == 0) s[2] = unscale;
+        };
+        if (resident) {
+#pragma unroll
+            for (int j = 0; j < MAXJ; j++) {
+                if (NT * j >= units) break;  // uniform over the workgroup
+                const uint32_t e4 = tid + NT * j;
+                if (e4 < units) stage(e4, held[j], weight[j]);  // whole groups of 16 lanes are in or out together
+            }
+        } else {
+            for (uint32_t e4 = tid; e4 < units; e4 += NT)
+                stage(e4, *reinterpret_cast<const f32x4 *>(p.x + 4u * e4), p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f});
+        }
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see this wave's writes
+
+    // ---- the walk
+    const ScaleLane lane_scales = scale_lane(q);
+    const uint32_t m = lane & 15u;
+    const bool feeds = (m >> 2) == q && (m & 3u) < 3u;  // A row m = 4 * slice + plane meets K slice `slice` only
+    const uint8_t *const abase = feeds ? digits + q * 192u + (m & 3u) * 16u : zeros;
+    const uint32_t astride = feeds ? TILE16_BLOCK_DIGITS : 0u;
+    float acc = 0.0f, gate = 0.0f;
+    uint32_t parity = 0;
+    // One step in two halves with the next fetch between them: everything that reads the fetched registers (nibbles, header)
+    // comes first, so the fetch can reuse them, and the weighing of the sums follows while the loads are under way.
+    struct Step {
+        i32x4 cl, ch;
+        f32x4 s;
+        uint32_t sc, mn, dd;
+    };
+    auto multiply = [&](const Tile16Unit &u, uint32_t b, Step &st) {
+        const uint8_t *at = abase + (size_t)b * astride;
+        const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
+        const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
+        st.s = sums[b * 4u + q];
+        const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+        const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
+        const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
+        half2_t sc, mn;
+        scale_pairs(u.hdr, lane_scales, sc, mn);
+        st.sc = __builtin_bit_cast(uint32_t, sc), st.mn = __builtin_bit_cast(uint32_t, mn), st.dd = u.hdr.x;
+        i32x4 cl = {0, 0, 0, 0}, ch = {0, 0, 0, 0};
+        cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a00, la, cl, 0, 0, 0);
+        ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a10, ha, ch, 0, 0, 0);
+        cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a01, lb, cl, 0, 0, 0);
+        ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a11, hb, ch, 0, 0, 0);
+        st.cl = cl, st.ch = ch;
+        asm volatile("" : "+v"(st.sc), "+v"(st.mn), "+v"(st.dd));  // the header is read by here
+    };
+    auto weigh = [&](const Step &st) {
+        const half2_t sc = __builtin_bit_cast(half2_t, st.sc), mn = __builtin_bit_cast(half2_t, st.mn), dd = __builtin_bit_cast(half2_t, st.dd);
+        // (c0 * 256 + c1) fits 24 bits: one conversion for two planes
+        const float fl = fmaf((float)((st.cl[0] << 8) + st.cl[1]), 256.0f, (float)st.cl[2]);
+        const float fh = fmaf((float)((st.ch[0] << 8) + st.ch[1]), 256.0f, (float)st.ch[2]);
+        const float weighed = fmaf((float)sc.x, fl, (float)sc.y * fh);    // scales and minimums arrive * 2^-24 (half subnormals)
+        const float floor_ = fmaf((float)mn.x, st.s.x, (float)mn.y * st.s.y);
+        const float d24 = (float)dd.x * (16777216.0f * st.s.z), m24 = (float)dd.y * -16777216.0f;
+        acc = fmaf(d24, weighed, fmaf(m24, floor_, acc));
+    };
+    auto tile_end = [&](uint32_t tile) {
+        float v = acc;
+        v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+        v += __shfl_xor(v, 32, 64);
+        if (q == 0) part[(parity * NW + wave) * 16u + r] = v;
+        __syncthreads();
+        if (wave == 0 && lane < 16u) {
+            float total = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) total += part[(parity * NW + w) * 16u + lane];
+            if (MODE == TILE16_SWIGLU) {
+                if (tile & 1u) p.y[(tile >> 1) * 16u + lane] = silu(gate) * total;
+                else gate = total;
+            } else if (MODE == TILE16_ROPE) {
+                const uint32_t c = (tile % tiles_per_head) * 8u + (lane & 7u);
+                const uint32_t n = (tile / tiles_per_head) * (2u * half_width) + c + (lane >> 3) * half_width;
+                rope_store(p, total, n, c, lane >= 8u);
+            } else {
+                const uint32_t n = tile * 16u + lane;
+                // in place (the decoder's residual stream): one add per element, nothing to wait for
+                if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);
+                else p.y[n] = p.residual ? p.residual[n] + total : total;
+            }
+        }
+        parity ^= 1u;
+        acc = 0.0f;
+    };
+    if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
+        for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t));
+        return;
+    }
+    // Every wave walks whole rounds of D steps: the steps past its last tile multiply what was fetched again and publish nothing.
+    uint32_t at_tile = 0, at_b = wave;
+    const uint32_t steps = walked * count;
+    for (uint32_t s0 = 0; s0 < steps; s0 += D) {
+#pragma unroll
+        for (int slot = 0; slot < D; slot++) {
+            Step st;
+            multiply(ring[slot], at_b, st);
+            __builtin_amdgcn_sched_barrier(0);  // the fetch reuses this unit's registers: keep its loads behind their last use
+            fetch(ring[slot]);
+            __builtin_amdgcn_sched_barrier(0);
+            weigh(st);
+            at_b += NW;
+            if (at_b >= nblk) {
+                if (at_tile < walked) tile_end(tile_at(at_tile));
+                at_b = wave;
+                at_tile++;
+            }
+        }
+    }
+}
+
+// ---- the 16-row tile kernel (one activation row, Q4_K)
+// NEURA_HIP_TILE16=0 keeps it out (the vector and the other matrix-core forms then take one row as before), as does a forced
+// NEURA_HIP_MFMA form.  Otherwise it takes every one-row Q4_K product whose matrices end on tile boundaries.
+bool tile16_takes(const GemvArgs &a) {
+    if (a.element != NH_Q4_K || a.rows != 1 || a.K % 256u != 0 || a.K == 0) return false;
+    if (env_int("NEURA_HIP_TILE16", 1) == 0 || env_int("NEURA_HIP_MFMA", 1) != 1) return false;
+    if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
+    if (a.N < 16u || a.N % 16u != 0) return false;
+    if (a.swiglu) {
+        if (a.residual || a.rope || a.end[0] != a.N / 2 || (a.N / 2) % 16u != 0) return false;
+    } else if (a.rope) {
+        const uint32_t width = a.rope->width;
+        if (a.residual || width < 16u || width % 16u != 0) return false;
+        if (a.rope->q_rows % width || a.rope->k_rows % width || a.N % width || a.rope->q_rows > a.rope->k_rows || a.rope->k_rows > a.N) return false;
+        if (a.end[0] % width || a.end[1] % width || a.end[2] != a.N) return false;
+    } else if (a.end[0] % 16u != 0 || a.end[1] % 16u != 0) {
+        return false;
+    }
+    const uint32_t nblk = a.K / 256u;
+    return tile16_lds(nblk, nblk > 32u ? 16u : 8u) <= 160u * 1024u;
+}
+
+template <int NW, int D, int MODE>
+static hipError_t launch_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
+    static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
+    if (!raised && lds > 64u * 1024u) {
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (error != hipSuccess) return error;
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    return hipGetLastError();
+}
+
+template <int MODE>
+static hipError_t launch_tile16_mode(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
+    switch (waves) {
+    case 4: return launch_tile16_instance<4, 2, MODE>(d, p, grid, lds);
+    case 7: return launch_tile16_instance<7, 2, MODE>(d, p, grid, lds);
+    case 8: return launch_tile16_instance<8, 2, MODE>(d, p, grid, lds);
+    default: return launch_tile16_instance<16, 2, MODE>(d, p, grid, lds);
+    }
+}
+
+int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
+    GemvParams p{};
+    for (int s = 0; s < 3; s++) {
+        p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+        p.end[s] = a.end[s];
+    }
+    p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
+    p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps;
+    p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
+    p.nblk = a.K / 256u;
+    p.rope_width = 16;  // the kernel derives a tile's rows from it only where the rotation is folded in
+    if (a.rope) {
+        p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
+        p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
+        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring;
+        p.refusal = d->refusal;
+        for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
+    }
+    // waves of a workgroup share a tile and split its super-blocks: about two steps a wave
+    const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u ? 8u : 16u));
+    // units of work: tiles, or with SwiGLU pairs (a gate tile and the up tile behind it); every workgroup takes the same
+    // number of them, one workgroup a compute unit when there are that many
+    const uint32_t units = a.swiglu ? a.N / 32u : a.N / 16u;
+    p.row_groups = units;
+    const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
+    const uint32_t grid = (units + rounds - 1u) / rounds;
+    const size_t lds = tile16_lds(p.nblk, waves);
+    profile_mark(d);
+    hipError_t launched = a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
+                          : a.rope ? launch_tile16_mode<TILE16_ROPE>(d, p, waves, grid, lds)
+                                   : launch_tile16_mode<TILE16_PLAIN>(d, p, waves, grid, lds);
+    NH_HIP(launched);
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
+}
+
+}  // namespace nh
