@@ -155,6 +155,13 @@ int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uin
                   uint32_t count, uint32_t batch, const uint8_t *dev_mask, float *dev_out);
 /* run_argmax (crates/neura-kernel/src/task/choice.rs:355-368): per row, lowest index wins ties */
 int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out);
+/* No counterpart in the reference.  nh_argmax for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same two kernels and the same result, with the section partials in a
+ * 512 KiB array that is part of the library's device image (one copy per GPU, held until the process ends) instead of the
+ * device scratch that nh_argmax may grow.  It calls no hipMalloc, hipFree or allocating routine.  rows <= 64 (any n); more
+ * is refused with NH_E_ARGUMENT.  Nothing in the array has to start at zero (every partial is written before it is read).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two handles) race. */
+int32_t nh_argmax_static(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out);
 
 /* What one row draws with (Sampling::Sampled and the per-plane states of a sampled batch,
  * crates/neura-generate/src/sampling.rs:3-36, crates/neura-generate/src/batch.rs:383-386): the seed's 32 bits as the

@@ -66,6 +66,7 @@ SIGNATURES = {
                                c_uint32, c_uint32, c_void_p, c_float, c_void_p]),
     "nh_gather": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_argmax": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
+    "nh_argmax_static": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
     "nh_sample": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_model_create": (c_void_p, [c_void_p, POINTER(ModelConfig), c_void_p, POINTER(TensorTable)]),
     "nh_model_destroy": (None, [c_void_p]),

@@ -2,6 +2,14 @@
 // (crates/neura-kernel/src/task/choice.rs:46-51, :355-368; sectioned + fold :331-353).
 #include "common.hpp"
 
+// The section partials of nh_argmax_static, the greedy choice for callers that cannot allocate, live in this array
+// instead of the device scratch (which grows by hipMalloc).  Every GPU the library runs on holds its own copy at its own
+// address until the process ends; in host code the name is only a handle for hipGetSymbolAddress, never an address a
+// kernel could follow.  64 rows of 1024 sections of (value, index): 512 KiB.
+constexpr uint32_t STATIC_ARGMAX_ROWS = 64;
+constexpr size_t STATIC_ARGMAX_BYTES = (size_t)STATIC_ARGMAX_ROWS * 1024u * (sizeof(float) + sizeof(uint32_t));
+static __device__ __align__(256) uint8_t scratch[STATIC_ARGMAX_BYTES];
+
 namespace nh {
 
 __device__ __forceinline__ bool precedes(float value, uint32_t index, float other_value, uint32_t other_index) {
@@ -66,14 +74,15 @@ __global__ __launch_bounds__(256) void argmax_fold_kernel(const float *__restric
     if (threadIdx.x == 0) out[row] = index == 0xffffffffu ? 0u : index;
 }
 
-int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out) {
-    if (!rows) return NH_OK;
+static uint32_t argmax_sections(uint32_t n) {
     uint32_t sections = (n + 2047) / 2048;
     if (sections < 1) sections = 1;
     if (sections > 1024) sections = 1024;
-    size_t bytes = (size_t)rows * sections * (sizeof(float) + sizeof(uint32_t));
-    uint8_t *held = static_cast<uint8_t *>(scratch(d, bytes));
-    if (!held) return NH_E_MEMORY;
+    return sections;
+}
+
+static int32_t launch_argmax_over(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out, uint8_t *held) {
+    const uint32_t sections = argmax_sections(n);
     float *best_values = reinterpret_cast<float *>(held);
     uint32_t *best_indices = reinterpret_cast<uint32_t *>(held + (size_t)rows * sections * sizeof(float));
     hipLaunchKernelGGL(argmax_sections_kernel, dim3(sections, rows), dim3(256), 0, d->stream, values, n, sections, best_values, best_indices);
@@ -81,6 +90,35 @@ int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t
     hipLaunchKernelGGL(argmax_fold_kernel, dim3(rows), dim3(256), 0, d->stream, best_values, best_indices, sections, out);
     NH_HIP(hipGetLastError());
     return NH_OK;
+}
+
+int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out) {
+    if (!rows) return NH_OK;
+    const size_t bytes = (size_t)rows * argmax_sections(n) * (sizeof(float) + sizeof(uint32_t));
+    uint8_t *held = static_cast<uint8_t *>(scratch(d, bytes));
+    if (!held) return NH_E_MEMORY;
+    return launch_argmax_over(d, values, rows, n, out, held);
+}
+
+// ---- the greedy choice for callers that cannot allocate ----------------------------------------------------------
+// once per device, with that device current (nh_open calls it): where this device keeps its copy of the array
+int32_t argmax_static_setup(nh_device *d) {
+    void *address = nullptr;
+    hipError_t found = hipGetSymbolAddress(&address, HIP_SYMBOL(::scratch));
+    if (found != hipSuccess || !address) return hip_fail(found, "hipGetSymbolAddress(scratch)");
+    d->static_scratch = static_cast<uint8_t *>(address);
+    return NH_OK;
+}
+
+int32_t launch_argmax_static(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out) {
+    if (!rows) return NH_OK;
+    if (!d->static_scratch) return fail(NH_E_DEVICE, "device %d holds no address of the static scratch array", d->index);
+    const size_t bytes = (size_t)rows * argmax_sections(n) * (sizeof(float) + sizeof(uint32_t));
+    if (rows > STATIC_ARGMAX_ROWS || bytes > STATIC_ARGMAX_BYTES)
+        return fail(NH_E_ARGUMENT, "a greedy choice over %u rows of %u needs %zu bytes of partials, and the static scratch holds %zu (at most %u rows)",
+                    rows, n, bytes, STATIC_ARGMAX_BYTES, STATIC_ARGMAX_ROWS);
+    // nothing in the array has to start at zero: the first kernel writes every partial the second one reads
+    return launch_argmax_over(d, values, rows, n, out, d->static_scratch);
 }
 
 }  // namespace nh

@@ -78,6 +78,7 @@ struct nh_device {
     // recorded again when this no longer matches the count at its capture
     uint64_t moved = 0;
     uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
+    uint8_t *static_scratch = nullptr;  // this device's copy of the file-scope array nh_argmax_static works in (argmax.hip)
     struct RopeTable {
         float base;
         uint32_t width;
@@ -209,6 +210,9 @@ int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
                       uint32_t count, uint32_t batch, const uint8_t *mask, float *out);
 int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);
+// the same choice with its partials in a file-scope device array: no allocation, at most 64 rows
+int32_t argmax_static_setup(nh_device *d);
+int32_t launch_argmax_static(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);
 // sampled choice: `draws` is device memory, one entry a row; check_draws refuses what the reference's host asserts refuse
 int32_t launch_sample(nh_device *d, const float *logits, uint32_t rows, uint32_t n, const nh_draw *draws, uint32_t *out);
 int32_t check_draws(const nh_draw *draws, uint32_t rows);

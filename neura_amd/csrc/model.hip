@@ -799,4 +799,9 @@ int32_t nh_argmax(nh_device *device, const float *dev_values, uint32_t rows, uin
     return launch_argmax(device, dev_values, rows, n, dev_out);
 }
 
+int32_t nh_argmax_static(nh_device *device, const float *dev_values, uint32_t rows, uint32_t n, uint32_t *dev_out) {
+    NH_REQUIRE(device && dev_values && dev_out && n > 0, "a choice names no device, no buffer or no value");
+    return launch_argmax_static(device, dev_values, rows, n, dev_out);
+}
+
 }  // extern "C"

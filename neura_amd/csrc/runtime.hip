@@ -125,6 +125,10 @@ nh_device *nh_open(int32_t device_index) {
         nh_close(device);
         return nullptr;
     }
+    if (argmax_static_setup(device) != NH_OK) {  // the error names the call that failed
+        nh_close(device);
+        return nullptr;
+    }
     return device;
 }
 
