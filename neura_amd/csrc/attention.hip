@@ -527,31 +527,21 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
     const uint32_t b = unit % p.batch, kvh = unit / p.batch;
     const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
 
-    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
-    if (!p.reach && origin + 1u > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
-        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-        origin = p.keys - 1u;
-    }
-    const Ring ring(p.keys, origin + 1u, p.reach);
+    // what does not need the cursor comes first: the cursor's load, the queries' and the first tile's are then all in flight
+    // together instead of one round trip to memory behind the other
+    const uint32_t origin_read = p.cursor ? p.cursor[b] : 0u;
     const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
     const uint32_t begin = min(p.keys, section * chunk);
-    const uint32_t visible = min(p.keys, origin + 1u);  // a ring too: the slots written so far
-    const uint32_t last = min(visible, begin + chunk);
     const bool held = n < G;
 
-    // the queries of this lane's column as two half planes
-    half8_t q_value[STEPS], q_residue[STEPS];
+    // the queries of this lane's column, as they lie; they become two half planes once the first tile has been asked for
+    float q_raw[STEPS][8];
     {
         const float *src = p.q + (uint64_t)(kvh * G + min(n, G - 1u)) * p.q_sh + (uint64_t)b * p.q_sb;
 #pragma unroll
         for (int s = 0; s < STEPS; s++)
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float value = held ? src[32 * s + 8 * kq + i] : 0.0f;
-                const _Float16 high = (_Float16)value;
-                q_value[s][i] = high;
-                q_residue[s][i] = (_Float16)((value - (float)high) * 2048.0f);
-            }
+            for (int i = 0; i < 8; i++) q_raw[s][i] = held ? src[32 * s + 8 * kq + i] : 0.0f;
     }
     f32x4_t acc[BLOCKS];
 #pragma unroll
@@ -575,8 +565,28 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
             vraw[i] = *reinterpret_cast<const u32x4 *>(p.cache_v + (plane + min(tile + key, p.capacity - 1u)) * WIDTH + part * 8u);
         }
     };
+    // the first tile's rows are asked for whether or not the cursor has reached them (the addresses are clamped to the cache)
     uint32_t tile = begin + wave * TK;
-    if (tile < last) fetch_keys(tile), fetch_values(tile);
+    __builtin_amdgcn_sched_barrier(0);  // the queries' loads stay ahead of the tile's, their first use behind them
+    if (tile < min(p.keys, begin + chunk)) fetch_keys(tile), fetch_values(tile);
+    __builtin_amdgcn_sched_barrier(0);
+    half8_t q_value[STEPS], q_residue[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; s++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const _Float16 high = (_Float16)q_raw[s][i];
+            q_value[s][i] = high;
+            q_residue[s][i] = (_Float16)((q_raw[s][i] - (float)high) * 2048.0f);
+        }
+    uint32_t origin = origin_read;
+    if (!p.reach && origin + 1u > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        origin = p.keys - 1u;
+    }
+    const Ring ring(p.keys, origin + 1u, p.reach);
+    const uint32_t visible = min(p.keys, origin + 1u);  // a ring too: the slots written so far
+    const uint32_t last = min(visible, begin + chunk);
     for (; tile < last; tile += 4 * TK) {
         // ---- scores
         f32x4_t scores[2], fine[2];

@@ -81,25 +81,36 @@ __device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s
 // half, or c + width/2 when `second`), the lane 8 further round its row of 16 holds the partner channel.  The projection's
 // bias, if it has one, comes before the rotation; q rows go to y, k rows rotated and v rows as they are to the caches as
 // halves, at the cursor (at cursor mod span in a ring).  Lanes 0..15 of a wave call it together
-// (crates/neura-kernel/src/task/rope.rs:95-122).
-__device__ __forceinline__ void rope_store(const GemvParams &p, float total, uint32_t n, uint32_t c, bool second) {
+// (crates/neura-kernel/src/task/rope.rs:95-122).  What it reads from memory can be fetched ahead with rope_operands().
+struct RopeOperands {
+    float bias, cosine, sine;
+};
+
+__device__ __forceinline__ RopeOperands rope_operands(const GemvParams &p, uint32_t n, uint32_t c, uint32_t position) {
     const uint32_t half = p.rope_width >> 1;
-    {
-        const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
-        const uint32_t e0 = p.end[0], e1 = p.end[1];
-        const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
-        const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
-        if (bias) total += bias[n - before];
-    }
-    const float other = dpp<DPP_ROW_ROR8>(total);
-    const uint32_t position = p.rope_cursor[0];
-    float value = total;
+    const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
+    const uint32_t e0 = p.end[0], e1 = p.end[1];
+    const float *bias = n < e0 ? b0 : (n < e1 ? b1 : b2);
+    const uint32_t before = n < e0 ? 0u : (n < e1 ? e0 : e1);
+    RopeOperands held{0.0f, 1.0f, 0.0f};
+    if (bias) held.bias = bias[n - before];
     if (n < p.rope_k_rows) {
         // cos and sin of f32(position) * pow(base, -2c/width), tabulated once per model by the rotation's own kernel
-        const float cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
-        const float sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
-        value = second ? total * cosine + other * sine : total * cosine - other * sine;
+        held.cosine = p.rope_cosines[(size_t)min(position, p.rope_positions - 1u) * half + c];
+        held.sine = p.rope_sines[(size_t)min(position, p.rope_positions - 1u) * half + c];
     }
+    return held;
+}
+
+__device__ __forceinline__ void rope_store(const GemvParams &p, float total, uint32_t n, bool second, uint32_t position, const RopeOperands &held) {
+    {
+        const float *b0 = p.bias[0], *b1 = p.bias[1], *b2 = p.bias[2];
+        const float *bias = n < p.end[0] ? b0 : (n < p.end[1] ? b1 : b2);
+        if (bias) total += held.bias;
+    }
+    const float other = dpp<DPP_ROW_ROR8>(total);
+    float value = total;
+    if (n < p.rope_k_rows) value = second ? total * held.cosine + other * held.sine : total * held.cosine - other * held.sine;
     if (n < p.rope_q_rows) {
         p.y[n] = value;
     } else if (position >= p.rope_positions || (!p.rope_ring && position >= p.rope_capacity)) {

@@ -108,6 +108,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         }
     };
 
+    // what the rotation's epilogue reads (the cursor, then cos, sin and bias of a tile's sixteen outputs) is fetched ahead:
+    // the cursor with the activations, a tile's operands a tile early
+    uint32_t rope_position = 0;
+    RopeOperands rope_held{0.0f, 1.0f, 0.0f};
+    auto rope_row = [half_width, tiles_per_head, lane](uint32_t tile, uint32_t &c) -> uint32_t {
+        c = (tile % tiles_per_head) * 8u + (lane & 7u);
+        return (tile / tiles_per_head) * (2u * half_width) + c + ((lane >> 3) & 1u) * half_width;
+    };
+
     // ---- activations -> three signed base-256 digit planes per 16 elements, a power-of-two scale per 64-element group.
     // Unit e4 = tid + NT * j (four consecutive activations) lies in super-block wave + NW * j: a wave turns into digits
     // exactly the super-blocks it multiplies.
@@ -132,6 +141,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
                 }
             }
         }
+        if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
         // the weights' loads go out behind the activations', which everything waits for first
 #pragma unroll
         for (int i = 0; i < D; i++) fetch(ring[i]);
@@ -213,6 +223,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         }
     }
     __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see this wave's writes
+    if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) {
+        uint32_t c;
+        const uint32_t n = rope_row(tile_at(0), c);
+        rope_held = rope_operands(p, n, c, rope_position);
+    }
 
     // ---- the walk
     const ScaleLane lane_scales = scale_lane(q);
@@ -272,9 +287,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
                 if (tile & 1u) p.y[(tile >> 1) * 16u + lane] = silu(gate) * total;
                 else gate = total;
             } else if (MODE == TILE16_ROPE) {
-                const uint32_t c = (tile % tiles_per_head) * 8u + (lane & 7u);
-                const uint32_t n = (tile / tiles_per_head) * (2u * half_width) + c + (lane >> 3) * half_width;
-                rope_store(p, total, n, c, lane >= 8u);
+                uint32_t c;
+                const uint32_t n = rope_row(tile, c);
+                rope_store(p, total, n, lane >= 8u, rope_position, rope_held);
+                if (tile + hop < tiles) {  // the next tile of this workgroup
+                    const uint32_t next = rope_row(tile + hop, c);
+                    rope_held = rope_operands(p, next, c, rope_position);
+                }
             } else {
                 const uint32_t n = tile * 16u + lane;
                 // in place (the decoder's residual stream): one add per element, nothing to wait for
