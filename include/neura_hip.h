@@ -114,6 +114,12 @@ size_t nh_weights_bytes(const nh_weights *weights);
 int32_t nh_dequant(nh_device *device, int32_t element, const void *dev_src, uint64_t elements, float *dev_dst);
 /* run_convert_half (crates/neura-kernel/src/task/convert.rs:229-249): fp32 -> fp16 RNE */
 int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elements, uint16_t *dev_dst);
+/* run_convert_q8_0 with q8_0_quantum and q8_0_code (crates/neura-kernel/src/task/convert.rs:355-430), the device twin of
+ * the host's q8_0 encoder (crates/neura-precision/src/ggml.rs:209-216): `elements` fp32 numbers into ceil(elements / 32) blocks
+ * of 34 bytes (a ragged last block counts zeros behind its numbers).  dev_dst holds the blocks rounded up to a four-byte word;
+ * the two bytes behind an odd number of blocks are written as zero, as the host's pack writes them.  dev_src on a 16-byte
+ * boundary. */
+int32_t nh_pack_q8_0(nh_device *device, const float *dev_src, uint64_t elements, void *dev_dst);
 /* narrow product, rows <= 8 (template_run_matmul_folded{,_fused,_quad},
  * crates/neura-kernel/src/task/matmul.rs:376-803): y[r][n] = sum_k x[r][k]·W[n][k], fp32; W in NH_Q8_0, NH_Q3_K, NH_Q4_K,
  * NH_Q5_K or NH_Q6_K blocks (the dots of crates/neura-kernel/src/dot.rs:471-797) */

@@ -125,6 +125,14 @@ class Device:
         _check(self.lib.nh_convert_half(self.handle, src.pointer, n, out.pointer))
         return out.numpy(np.uint16)
 
+    def pack_q8_0(self, values):
+        """fp32 numbers into Q8_0 blocks on the device; the bytes end on a four-byte word"""
+        src = self._dev(np.asarray(values, dtype=np.float32))
+        n = src.nbytes // 4
+        out = self.alloc(((n + 31) // 32 * 34 + 3) // 4 * 4)
+        _check(self.lib.nh_pack_q8_0(self.handle, src.pointer, n, out.pointer))
+        return out.numpy(np.uint8)
+
     def gemv(self, element, W, N, K, x, residual=None, swiglu=False, out=None):
         W, x = self._dev(W), self._dev(np.asarray(x, dtype=np.float32))
         rows = x.nbytes // 4 // K

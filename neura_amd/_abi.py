@@ -56,6 +56,7 @@ SIGNATURES = {
     "nh_weights_bytes": (c_size_t, [c_void_p]),
     "nh_dequant": (c_int32, [c_void_p, c_int32, c_void_p, c_uint64, c_void_p]),
     "nh_convert_half": (c_int32, [c_void_p, c_void_p, c_uint64, c_void_p]),
+    "nh_pack_q8_0": (c_int32, [c_void_p, c_void_p, c_uint64, c_void_p]),
     "nh_gemv": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_void_p, POINTER(Epilogue)]),
     "nh_gemm": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_int32, c_uint32, c_void_p, POINTER(Epilogue)]),
     "nh_rmsnorm": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_uint32, c_uint32, c_void_p, c_void_p]),

@@ -49,6 +49,56 @@ int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, u
     return NH_OK;
 }
 
+// The device's Q8_0 encoder (run_convert_q8_0, q8_0_quantum, q8_0_code,
+// crates/neura-kernel/src/task/convert.rs:355-430): per block of 32 the quantum is the largest
+// magnitude / 127, stored as a half, and every code is value * (1 / quantum) rounded half away
+// from zero as trunc(scaled +- 0.5), clamped to +-127.  Elements past the end count as zero.
+// Eight lanes share a block: each loads four numbers, the magnitude folds over the eight, and each
+// stores its four codes as two 16-bit halves (a block starts on an even byte, not on a word).
+// The bytes behind an odd number of blocks, up to the four-byte word, are zero.
+__global__ __launch_bounds__(256) void pack_q8_0_kernel(const float *__restrict__ src, uint64_t elements, uint64_t blocks,
+                                                        uint8_t *__restrict__ dst) {
+    const uint64_t lanes = blocks * 8;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < (lanes + 63) / 64 * 64; i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t block = i / 8, first = i * 4;
+        float v[4];
+        if (first + 4 <= elements && i < lanes) {
+            const float4 held = *reinterpret_cast<const float4 *>(src + first);
+            v[0] = held.x, v[1] = held.y, v[2] = held.z, v[3] = held.w;
+        } else {
+            for (int j = 0; j < 4; j++) v[j] = (i < lanes && first + j < elements) ? src[first + j] : 0.0f;
+        }
+        float size = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+        size = fmaxf(size, __shfl_xor(size, 1));
+        size = fmaxf(size, __shfl_xor(size, 2));
+        size = fmaxf(size, __shfl_xor(size, 4));
+        if (i >= lanes) continue;
+        const float quantum = __fdiv_rn(size, 127.0f);
+        const float inverse = quantum != 0.0f ? __fdiv_rn(1.0f, quantum) : 0.0f;
+        uint32_t word = 0;
+        for (int j = 0; j < 4; j++) {
+            const float scaled = __fmul_rn(v[j], inverse);
+            const float rounded = truncf(__fadd_rn(scaled, scaled >= 0.0f ? 0.5f : -0.5f));
+            const int code = (int)fminf(fmaxf(rounded, -127.0f), 127.0f);
+            word |= ((uint32_t)code & 0xffu) << (8 * j);
+        }
+        uint16_t *field = reinterpret_cast<uint16_t *>(dst + block * 34);
+        const uint32_t lane = (uint32_t)(i % 8);
+        if (lane == 0) field[0] = float_to_half(quantum);
+        field[1 + 2 * lane] = (uint16_t)word;
+        field[2 + 2 * lane] = (uint16_t)(word >> 16);
+        if (lane == 7 && block + 1 == blocks && (blocks & 1)) field[17] = 0;
+    }
+}
+
+int32_t launch_pack_q8_0(nh_device *d, const float *src, uint64_t elements, uint8_t *dst) {
+    if (!elements) return NH_OK;
+    const uint64_t blocks = (elements + 31) / 32;
+    hipLaunchKernelGGL(pack_q8_0_kernel, dim3(grid_for(d, blocks * 8, 256)), dim3(256), 0, d->stream, src, elements, blocks, dst);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
+}
+
 // out[t][c] = dequant(table[token[t]])[c] * mask[t % batch]   (crates/neura-kernel/src/task/select.rs:29-49,
 // examples/qwen/model.rs:94).  One thread per element: blockIdx.y walks the row in spans of 256.
 template <int ELEMENT>

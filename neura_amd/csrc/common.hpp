@@ -207,6 +207,7 @@ int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uin
                             const uint32_t *cursor, uint32_t ring);
 int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n);
 
+int32_t launch_pack_q8_0(nh_device *d, const float *src, uint64_t elements, uint8_t *dst);
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
                       uint32_t count, uint32_t batch, const uint8_t *mask, float *out);
 int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);

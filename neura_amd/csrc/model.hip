@@ -676,6 +676,12 @@ int32_t nh_convert_half(nh_device *device, const float *dev_src, uint64_t elemen
     return launch_convert_half(device, dev_src, elements, dev_dst);
 }
 
+int32_t nh_pack_q8_0(nh_device *device, const float *dev_src, uint64_t elements, void *dev_dst) {
+    NH_REQUIRE(device && dev_src && dev_dst, "a packing names no device or no buffer");
+    NH_REQUIRE(aligned16(dev_src) && ((uintptr_t)dev_dst & 3u) == 0, "a packing reads from a 16-byte boundary and writes from a 4-byte one");
+    return launch_pack_q8_0(device, dev_src, elements, static_cast<uint8_t *>(dev_dst));
+}
+
 int32_t nh_gemv(nh_device *device, int32_t element, const void *dev_W, uint32_t N, uint32_t K, const float *dev_x, uint32_t rows,
                 float *dev_y, const nh_epilogue *epilogue) {
     NH_REQUIRE(device && dev_W && dev_x && dev_y, "a product names no device or no buffer");

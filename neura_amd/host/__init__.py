@@ -52,6 +52,10 @@ SIGNATURES = {
     "nhost_vector": (c_int32, [c_void_p, c_char_p, c_uint32, POINTER(c_int32)]),
     "nhost_cache_validate": (c_int32, [c_char_p] + [c_uint32] * 6 + [c_int32]),
     "nhost_payload_bytes": (c_uint64, [c_int32, c_uint64]),
+    "nhost_pack": (c_int64, [c_int32, c_float, c_void_p, c_size_t, c_void_p, c_size_t]),
+    "nhost_unpack": (c_int32, [c_int32, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "nhost_half_bits": (c_uint32, [c_float]),
+    "nhost_half_value": (c_float, [c_uint32]),
     "nhost_runtime_open": (c_void_p, [c_int32]),
     "nhost_runtime_close": (None, [c_void_p]),
     "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32, c_int32]),
@@ -408,6 +412,25 @@ def seed_bits(seed):
 
 def payload_bytes(element, elements):
     return int(library().nhost_payload_bytes(element, elements))
+
+
+def pack(element, values, quantum=0.0):
+    """neura_precision::pack (crates/neura-precision/src/lib.rs:5-24): float32 numbers into the format's bytes"""
+    values = np.ascontiguousarray(values, dtype=np.float32).reshape(-1)
+    room = np.zeros(payload_bytes(element, max(values.size, 1)) + 8, dtype=np.uint8)
+    length = library().nhost_pack(element, quantum, values.ctypes.data, values.size, room.ctypes.data, room.size)
+    if length < 0:
+        raise _refused()
+    return room[:length].copy()
+
+
+def unpack(element, elements, raw):
+    """neura_precision::unpack (crates/neura-precision/src/lib.rs:26-68): the numbers `raw` holds"""
+    raw = np.ascontiguousarray(np.frombuffer(bytes(raw), dtype=np.uint8) if not isinstance(raw, np.ndarray) else raw, dtype=np.uint8)
+    out = np.zeros(max(elements, 1), dtype=np.float32)
+    if library().nhost_unpack(element, elements, raw.ctypes.data, raw.size, out.ctypes.data) != 0:
+        raise _refused()
+    return out[:elements]
 
 
 class Runtime:

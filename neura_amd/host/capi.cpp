@@ -185,6 +185,26 @@ int32_t nhost_cache_validate(const char *name, uint32_t heads, uint32_t width, u
 }
 uint64_t nhost_payload_bytes(int32_t element, uint64_t elements) { return payload_bytes((Element)element, elements); }
 
+// ---- neura-precision --------------------------------------------------------------------------------
+// precision::pack: the bytes `count` numbers pack into (out, at most room); returns their count, or -1 refused
+int64_t nhost_pack(int32_t element, float quantum, const float *values, size_t count, uint8_t *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        auto packed = precision::pack((Element)element, quantum, values, count);
+        for (size_t i = 0; i < packed.size() && i < room; i++) out[i] = packed[i];
+        return (int64_t)packed.size();
+    }, -1);
+}
+// precision::unpack: `elements` numbers out of `size` bytes; 0 done, -1 refused
+int32_t nhost_unpack(int32_t element, size_t elements, const uint8_t *bytes, size_t size, float *out) {
+    return guarded([&] {
+        auto values = precision::unpack((Element)element, elements, bytes, size);
+        for (size_t i = 0; i < values.size(); i++) out[i] = values[i];
+        return 0;
+    }, -1);
+}
+uint32_t nhost_half_bits(float value) { return precision::half_bits(value); }
+float nhost_half_value(uint32_t bits) { return precision::half_value((uint16_t)bits); }
+
 // ---- runtime, model, batch ----------------------------------------------------------------------
 void *nhost_runtime_open(int32_t index) {
     return guarded([&]() -> void * { return new runtime::Runtime(index); }, nullptr);

@@ -86,6 +86,350 @@ inline uint64_t payload_bytes(Element element, uint64_t elements) {
     return (elements * bits_per_element(element) + 7) / 8;
 }
 
+// ---- neura-precision: host encoders and decoders of the storage formats ------------------------
+//
+// pack() lays numbers out in a format's bytes and unpack() reads them back, as
+// crates/neura-precision/src/lib.rs:5-68 does for the formats a GGUF decoder meets: single, half,
+// bfloat16 and the five block formats of crates/neura-precision/src/ggml.rs.  Every product,
+// quotient and rounding below is the reference's, in its order, in IEEE single precision, so the
+// bytes are the reference's bytes.
+
+namespace precision {
+
+// IEEE half from single, round to nearest even (what half::f16::from_f32 does)
+inline uint16_t half_bits(float value) {
+    uint32_t bits;
+    std::memcpy(&bits, &value, 4);
+    const uint32_t sign = (bits >> 16) & 0x8000u;
+    bits &= 0x7fffffffu;
+    if (bits >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (bits > 0x7f800000u ? 0x0200u | ((bits >> 13) & 0x3ffu) : 0u));
+    if (bits >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);  // rounds past the largest half
+    if (bits < 0x33000001u) return (uint16_t)sign;               // at most half of the least subnormal
+    const int32_t exponent = (int32_t)(bits >> 23) - 127;
+    uint32_t mantissa = (bits & 0x7fffffu) | 0x800000u;
+    const int32_t drop = exponent < -14 ? 13 + (-14 - exponent) : 13;
+    const uint32_t kept = mantissa >> drop, rest = mantissa & ((1u << drop) - 1u), middle = 1u << (drop - 1);
+    uint32_t out = exponent < -14 ? kept : (((uint32_t)(exponent + 15) << 10) + (kept & 0x3ffu));
+    if (rest > middle || (rest == middle && (out & 1u))) out++;
+    return (uint16_t)(sign | out);
+}
+
+inline float half_value(uint16_t half) {
+    const uint32_t sign = (uint32_t)(half & 0x8000u) << 16, exponent = (half >> 10) & 31u, mantissa = half & 0x3ffu;
+    uint32_t bits;
+    if (exponent == 31)
+        bits = sign | 0x7f800000u | (mantissa << 13);
+    else if (exponent != 0)
+        bits = sign | ((exponent + 112u) << 23) | (mantissa << 13);
+    else if (mantissa == 0)
+        bits = sign;
+    else {
+        int shift = 0;
+        uint32_t m = mantissa;
+        while (!(m & 0x400u)) m <<= 1, shift++;
+        bits = sign | ((uint32_t)(113 - shift) << 23) | ((m & 0x3ffu) << 13);
+    }
+    float value;
+    std::memcpy(&value, &bits, 4);
+    return value;
+}
+
+// crates/neura-precision/src/lib.rs:325-329
+inline uint16_t bfloat16_bits(float value) {
+    uint32_t bits;
+    std::memcpy(&bits, &value, 4);
+    return (uint16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+
+namespace detail {
+
+inline float least(float value, float other) { return value < other ? value : other; }     // ggml.rs:90-92
+inline float greatest(float value, float other) { return value > other ? value : other; }  // ggml.rs:94-96
+inline float rounded(float value) { return std::round(value); }                            // f32::round: halves away from zero
+inline float clamped(float value, float low, float high) { return value < low ? low : value > high ? high : value; }
+
+inline void put_half(uint8_t *field, size_t at, float value) {
+    const uint16_t bits = half_bits(value);
+    field[at] = (uint8_t)bits, field[at + 1] = (uint8_t)(bits >> 8);
+}
+inline float half_at(const uint8_t *field, size_t at) { return half_value((uint16_t)(field[at] | field[at + 1] << 8)); }
+inline void put_nibble(uint8_t *field, size_t at, bool high, uint32_t value) { field[at] |= (uint8_t)((value & 0x0fu) << (high ? 4 : 0)); }
+inline uint32_t nibble_at(uint8_t byte, bool high) { return high ? byte >> 4 : byte & 0x0fu; }
+
+// ggml.rs:120-125: the quotient rounds, clamps and converts to an unsigned integer, a conversion
+// that saturates: whatever lies below zero after the clamp becomes 0
+inline uint32_t quantized(float value, float quantum, float low, float high) {
+    if (quantum == 0.0f) return 0;
+    const float held = clamped(rounded(value / quantum), low, high);
+    return held < 0.0f ? 0u : (uint32_t)held;
+}
+
+// ggml.rs:127-149: eight six-bit scales and eight six-bit minima in twelve bytes
+inline void scale_min_k4(const uint8_t *scales, size_t at, uint32_t &scale, uint32_t &min) {
+    if (at < 4) {
+        scale = scales[at] & 63u, min = scales[at + 4] & 63u;
+    } else {
+        scale = (scales[at + 4] & 0x0fu) | (uint32_t)(scales[at - 4] >> 6) << 4;
+        min = (uint32_t)(scales[at + 4] >> 4) | (uint32_t)(scales[at] >> 6) << 4;
+    }
+}
+inline void put_scale_min_k4(uint8_t *scales, size_t at, uint32_t scale, uint32_t min) {
+    if (at < 4) {
+        scales[at] = (uint8_t)scale, scales[at + 4] = (uint8_t)min;
+    } else {
+        scales[at + 4] = (uint8_t)((scale & 0x0fu) | (min & 0x0fu) << 4);
+        scales[at - 4] |= (uint8_t)((scale >> 4) << 6);
+        scales[at] |= (uint8_t)((min >> 4) << 6);
+    }
+}
+
+// ggml.rs:209-216: quantum = the largest magnitude / 127, codes round(value * (1 / quantum))
+inline void q8_0(const float *values, uint8_t *field) {
+    float size = 0.0f;
+    for (int at = 0; at < 32; at++)
+        if (size < std::fabs(values[at])) size = std::fabs(values[at]);
+    const float quantum = size / 127.0f;
+    const float inverse = quantum == 0.0f ? 0.0f : 1.0f / quantum;
+    put_half(field, 0, quantum);
+    for (int at = 0; at < 32; at++) field[2 + at] = (uint8_t)(int8_t)clamped(rounded(values[at] * inverse), -127.0f, 127.0f);
+}
+
+// ggml.rs:151-207: Q4_K (steps 15) and Q5_K (steps 31).  Each 32-element sub-block spans from
+// min(0, its least) to its greatest in `steps` steps; the super-block stores the widest step and
+// the deepest low over 63 as halves and each sub-block a six-bit multiple of either.
+inline void affine_block(Element element, const float *values, uint8_t *field, uint32_t steps) {
+    const size_t bytes = element == Element::Q5K ? 176 : 144, quants = element == Element::Q5K ? 48 : 16;
+    float lows[8], quantums[8];
+    for (int at = 0; at < 8; at++) {
+        float low = 0.0f, high = 0.0f;
+        for (int i = 0; i < 32; i++) low = least(low, values[at * 32 + i]), high = greatest(high, values[at * 32 + i]);
+        lows[at] = least(0.0f, low);
+        quantums[at] = (high - lows[at]) / (float)steps;
+    }
+    float scale = 0.0f, min = 0.0f;
+    for (int at = 0; at < 8; at++) scale = greatest(scale, quantums[at]), min = greatest(min, -lows[at]);
+    scale = scale / 63.0f, min = min / 63.0f;
+    uint8_t codes[8], mins[8];
+    for (int at = 0; at < 8; at++) {
+        codes[at] = (uint8_t)clamped(rounded(scale == 0.0f ? 0.0f : quantums[at] / scale), 0.0f, 63.0f);
+        mins[at] = (uint8_t)clamped(rounded(min == 0.0f ? 0.0f : -lows[at] / min), 0.0f, 63.0f);
+    }
+    std::memset(field, 0, bytes);
+    put_half(field, 0, scale);
+    put_half(field, 2, min);
+    for (int at = 0; at < 8; at++) put_scale_min_k4(field + 4, at, codes[at], mins[at]);
+    for (int at = 0; at < 8; at++) {
+        const float quantum = scale * (float)codes[at], low = min * (float)mins[at];
+        const int group = at / 2;
+        const bool seat = at % 2 == 1;
+        for (int within = 0; within < 32; within++) {
+            const uint32_t code = quantized(values[at * 32 + within] + low, quantum, 0.0f, (float)steps);
+            put_nibble(field, quants + group * 32 + within, seat, code);
+            if (element == Element::Q5K && (code & 0x10u)) field[16 + within] |= (uint8_t)(1u << (2 * group + (seat ? 1 : 0)));
+        }
+    }
+}
+
+// ggml.rs:242-289: sixteen sub-blocks of 16; d = the widest magnitude / 4 / 31, six-bit scale
+// codes 32..63, three-bit codes -4..3 whose top bit (set when not negative) lies in bytes 0..31
+inline void q3_k(const float *values, uint8_t *field) {
+    float peaks[16], widest = 0.0f;
+    for (int at = 0; at < 16; at++) {
+        float peak = 0.0f;
+        for (int i = 0; i < 16; i++) peak = greatest(peak, std::fabs(values[at * 16 + i]));
+        peaks[at] = peak;
+        widest = greatest(widest, peak);
+    }
+    if (!(widest >= 1.17549435e-38f)) widest = 1.17549435e-38f;  // f32::max(MIN_POSITIVE)
+    const float d = widest / 4.0f / 31.0f;
+    uint32_t codes[16];
+    for (int at = 0; at < 16; at++) codes[at] = (uint32_t)clamped(rounded(peaks[at] / 4.0f / d), 0.0f, 31.0f) + 32u;
+    std::memset(field, 0, 110);
+    for (uint32_t at = 0; at < 16; at++) {  // put_q3_k_scale, ggml.rs:231-240
+        const uint8_t low = (uint8_t)(codes[at] & 0x0fu), high = (uint8_t)((codes[at] >> 4) & 3u);
+        field[96 + at % 8] |= (uint8_t)(at < 8 ? low : low << 4);
+        field[96 + 8 + at % 4] |= (uint8_t)(high << (2 * (at / 4)));
+    }
+    for (uint32_t at = 0; at < 256; at++) {
+        const uint32_t sub = at / 16, lane = at % 16;
+        const float quantum = d * (float)(codes[sub] - 32u);
+        const int quant = quantum == 0.0f ? 0 : (int)clamped(rounded(values[at] / quantum), -4.0f, 3.0f);
+        const uint32_t half = sub / 8, j = sub % 8 / 2, second = sub % 2;
+        field[32 + half * 32 + second * 16 + lane] |= (uint8_t)(((uint32_t)quant & 3u) << (2 * j));
+        if (quant >= 0) field[second * 16 + lane] |= (uint8_t)(1u << (half * 4 + j));
+    }
+    put_half(field, 108, d);
+}
+
+// ggml.rs:352-392: sixteen sub-blocks of 16; factor = the largest magnitude / 32, the super scale
+// = the largest factor / 127 (stored as a half while the single quantizes), signed byte multiples
+// per sub-block, six-bit codes offset by 32.  `quantized` saturates below zero, so a negative
+// number packs as code 32; this keeps the reference's bytes.
+inline void q6_k(const float *values, uint8_t *field) {
+    float factors[16], scale = 0.0f;
+    for (int at = 0; at < 16; at++) {
+        float size = 0.0f;
+        for (int i = 0; i < 16; i++)
+            if (size < std::fabs(values[at * 16 + i])) size = std::fabs(values[at * 16 + i]);
+        factors[at] = size / 32.0f;
+        scale = greatest(scale, std::fabs(factors[at]));
+    }
+    scale = scale / 127.0f;
+    std::memset(field, 0, 210);
+    put_half(field, 208, scale);
+    for (int at = 0; at < 16; at++) {
+        const int8_t code = scale == 0.0f ? (int8_t)0 : (int8_t)clamped(rounded(factors[at] / scale), -127.0f, 127.0f);
+        field[192 + at] = (uint8_t)code;
+        const float factor = scale * (float)code;
+        for (int within = 0; within < 16; within++) {
+            const int element = at * 16 + within, half = element / 128, group = element % 128 / 32, seat = element % 32;
+            const uint32_t quant = quantized(values[element], factor, -32.0f, 31.0f) + 32u;
+            put_nibble(field, half * 64 + (group % 2) * 32 + seat, group >= 2, quant);
+            field[128 + half * 32 + seat] |= (uint8_t)(((quant >> 4) & 3u) << (2 * group));
+        }
+    }
+}
+
+inline void encode(Element element, const float *values, uint8_t *field) {
+    switch (element) {
+    case Element::Q8_0: return q8_0(values, field);
+    case Element::Q3K: return q3_k(values, field);
+    case Element::Q4K: return affine_block(element, values, field, 15);  // ggml.rs:295-297
+    case Element::Q5K: return affine_block(element, values, field, 31);  // ggml.rs:291-293
+    case Element::Q6K: return q6_k(values, field);
+    default: panic("%s storage packs numbers a host quantizes by its element", neura::name(element));
+    }
+}
+
+// the decoders: ggml.rs:218-223 (Q8_0), :291-309 (Q3_K), :311-350 (Q5_K, Q4_K), :394-408 (Q6_K)
+inline void decode(Element element, const uint8_t *field, float *out) {
+    switch (element) {
+    case Element::Q8_0: {
+        const float quantum = half_at(field, 0);
+        for (int at = 0; at < 32; at++) out[at] = (float)(int8_t)field[2 + at] * quantum;
+        return;
+    }
+    case Element::Q4K:
+    case Element::Q5K: {
+        const float scale = half_at(field, 0), min = half_at(field, 2);
+        const bool five = element == Element::Q5K;
+        for (int group = 0; group < 4; group++)
+            for (int seat = 0; seat < 2; seat++) {
+                uint32_t code, offset;
+                scale_min_k4(field + 4, group * 2 + seat, code, offset);
+                const float quantum = scale * (float)code, low = min * (float)offset;
+                for (int within = 0; within < 32; within++) {
+                    uint32_t quant = nibble_at(field[(five ? 48 : 16) + group * 32 + within], seat == 1);
+                    if (five) quant |= (uint32_t)((field[16 + within] >> (2 * group + seat)) & 1u) << 4;
+                    *out++ = quantum * (float)quant - low;
+                }
+            }
+        return;
+    }
+    case Element::Q3K: {
+        const float d = half_at(field, 108);
+        for (uint32_t at = 0; at < 256; at++) {
+            const uint32_t sub = at / 16, lane = at % 16, half = sub / 8, j = sub % 8 / 2, second = sub % 2;
+            const uint8_t low_byte = field[96 + sub % 8], high_byte = field[96 + 8 + sub % 4];
+            const uint32_t code = (sub < 8 ? low_byte & 0x0fu : low_byte >> 4) | (uint32_t)((high_byte >> (2 * (sub / 4))) & 3u) << 4;
+            const int low = (field[32 + half * 32 + second * 16 + lane] >> (2 * j)) & 3;
+            const bool high = (field[second * 16 + lane] & (1u << (half * 4 + j))) != 0;
+            out[at] = d * ((float)(uint8_t)code - 32.0f) * (float)(low - (high ? 0 : 4));
+        }
+        return;
+    }
+    case Element::Q6K: {
+        const float scale = half_at(field, 208);
+        for (int seat = 0; seat < 2; seat++)
+            for (int group = 0; group < 4; group++)
+                for (int within = 0; within < 32; within++) {
+                    const int8_t sub = (int8_t)field[192 + seat * 8 + group * 2 + within / 16];
+                    const uint32_t quant = nibble_at(field[seat * 64 + (group % 2) * 32 + within], group >= 2) |
+                                           (uint32_t)((field[128 + seat * 32 + within] >> (2 * group)) & 3u) << 4;
+                    *out++ = scale * (float)sub * ((float)quant - 32.0f);
+                }
+        return;
+    }
+    default: panic("%s storage walks numbers a host reads by its element", neura::name(element));
+    }
+}
+
+}  // namespace detail
+
+// crates/neura-precision/src/lib.rs:5-24 and ggml.rs:8-20.  `quantum` only matters to the
+// per-tensor integer formats, which no GGUF holds; it is kept so calls read like the reference's.
+// A ragged last block is packed with zeros behind it, and the bytes end on a four-byte word.
+inline std::vector<uint8_t> pack(Element element, float quantum, const float *values, size_t count) {
+    (void)quantum;
+    std::vector<uint8_t> bytes;
+    if (element == Element::Single) {
+        bytes.resize(count * 4);
+        if (count) std::memcpy(bytes.data(), values, count * 4);
+        return bytes;
+    }
+    if (element == Element::Half || element == Element::Bfloat16) {
+        bytes.assign((count + 1) / 2 * 4, 0);
+        for (size_t at = 0; at < count; at++) {
+            const uint16_t bits = element == Element::Half ? half_bits(values[at]) : bfloat16_bits(values[at]);
+            bytes[2 * at] = (uint8_t)bits, bytes[2 * at + 1] = (uint8_t)(bits >> 8);
+        }
+        return bytes;
+    }
+    const auto layout = block(element);
+    NEURA_ASSERT(layout.has_value(), "%s storage packs numbers a host quantizes by its element", neura::name(element));
+    const size_t blocks = (count + layout->elements - 1) / layout->elements;
+    bytes.assign((blocks * layout->bytes + 3) / 4 * 4, 0);
+    float held[256];
+    for (size_t at = 0; at < blocks; at++) {
+        const size_t first = at * layout->elements, lane = std::min<size_t>(layout->elements, count - first);
+        std::fill(held, held + 256, 0.0f);
+        std::copy(values + first, values + first + lane, held);
+        detail::encode(element, held, bytes.data() + at * layout->bytes);
+    }
+    return bytes;
+}
+inline std::vector<uint8_t> pack(Element element, float quantum, const std::vector<float> &values) {
+    return pack(element, quantum, values.data(), values.size());
+}
+
+// crates/neura-precision/src/lib.rs:26-68 and ggml.rs:22-38
+inline std::vector<float> unpack(Element element, size_t elements, const uint8_t *bytes, size_t size) {
+    const uint64_t held = (payload_bytes(element, elements) + 3) / 4 * 4;
+    NEURA_ASSERT(size >= held, "unpacking %zu %s numbers out of %zu bytes where they pack %llu", elements, neura::name(element), size,
+                 (unsigned long long)held);
+    std::vector<float> values;
+    if (element == Element::Single) {
+        values.resize(elements);
+        if (elements) std::memcpy(values.data(), bytes, elements * 4);
+        return values;
+    }
+    if (element == Element::Half || element == Element::Bfloat16) {
+        values.resize(elements);
+        for (size_t at = 0; at < elements; at++) {
+            const uint16_t bits = (uint16_t)(bytes[2 * at] | bytes[2 * at + 1] << 8);
+            if (element == Element::Half) {
+                values[at] = half_value(bits);
+            } else {
+                const uint32_t word = (uint32_t)bits << 16;
+                std::memcpy(&values[at], &word, 4);
+            }
+        }
+        return values;
+    }
+    const auto layout = block(element);
+    NEURA_ASSERT(layout.has_value(), "%s storage walks numbers a host reads by its element", neura::name(element));
+    const size_t blocks = (elements + layout->elements - 1) / layout->elements;
+    values.resize(blocks * layout->elements);
+    for (size_t at = 0; at < blocks; at++) detail::decode(element, bytes + at * layout->bytes, values.data() + at * layout->elements);
+    values.resize(elements);
+    return values;
+}
+inline std::vector<float> unpack(Element element, size_t elements, const std::vector<uint8_t> &bytes) {
+    return unpack(element, elements, bytes.data(), bytes.size());
+}
+
+}  // namespace precision
+
 // ---- neura-gguf (crates/neura-gguf/src/{value,metadata,header,lib}.rs) ------------------------
 
 namespace gguf {

@@ -59,6 +59,33 @@ def test_convert_half_is_bit_exact(device):
     assert np.array_equal(device.convert_half(values), oracle.f32_to_f16(values))
 
 
+@pytest.mark.parametrize("count", [5 * 96, 3 * 33, 7, 32 * 100000 + 13])
+def test_pack_q8_0_is_the_host_s_blocks(device, count):
+    """the device encoder against the host's on the reference's own data (crates/neura-runtime/tests/runtime.rs:717-736: seed 7,
+    shapes 5x96, 3x33 and 7) and on three million numbers: byte-equal, the padding behind the last block included"""
+    values = oracle.random(count, 7)
+    padded = np.zeros(-(-count // 32) * 32, dtype=np.float32)
+    padded[:count] = values
+    want = oracle.pack(NH_Q8_0, padded)
+    want = np.concatenate([want, np.zeros(-want.size % 4, dtype=np.uint8)])
+    got = device.pack_q8_0(values)
+    assert got.size == want.size and np.array_equal(got, want)
+    # and the blocks read back as the numbers the oracle reads
+    back = device.dequant(NH_Q8_0, got[: padded.size // 32 * 34], padded.size)
+    assert np.array_equal(back.view(np.uint32), oracle.unpack(NH_Q8_0, want, padded.size).view(np.uint32))
+
+
+def test_pack_q8_0_of_hard_blocks(device):
+    rng = np.random.default_rng(41)
+    values = np.concatenate([
+        np.zeros(64), np.full(32, 0.3), rng.normal(0, 1, 3200) * 10.0 ** rng.integers(-30, 30, 3200), np.full(32, -1e-38), np.full(32, 3e38),
+        (rng.integers(-254, 255, 3200) * 0.5 / 127.0),  # quotients that land on halves
+    ]).astype(np.float32)
+    got, want = device.pack_q8_0(values), oracle.pack(NH_Q8_0, values)
+    assert got.size == want.size + 2 and not got[want.size :].any()  # an odd number of blocks ends two bytes short of a word
+    assert np.array_equal(got[: want.size], want)
+
+
 @pytest.mark.parametrize("element,width", [(NH_Q8_0, 896), (NH_Q4_K, 1536), (NH_Q6_K, 768), (NH_Q5_K, 512), (NH_Q3_K, 768)])
 def test_gather_is_the_dequantised_row_times_mask(device, element, width):
     rng = np.random.default_rng(102)
