@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restr
     __shared__ uint32_t wave_top[4];
     __shared__ float red[256];
     const uint32_t m = blockIdx.x, tid = threadIdx.x;
-    const uint32_t nsb = K / 256u;
+    const uint32_t nsb = (K + 255u) / 256u;
     float scale = 1.0f, norm = 1.0f;
     if (PRELUDE == PACK_NORM) {
         const float *xr = static_cast<const float *>(X) + (size_t)m * K;
@@ -443,13 +443,188 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
         }
 }
 
+// ------------------------------------------------------------------- Q8_0 on MFMA --------
+//
+// The same tiles, the same packed activation rows and the same division of the waves.  A step of 64 k is two blocks: a
+// stager owns one row and one block of the step, reads the nine words that cover its 34 bytes from the 4-byte boundary
+// below it (a block starts on a half word as often as not; crates/neura-kernel/src/dot.rs:197-264 reads it the same way),
+// and unpacks the 32 codes into LDS as the halves they are -- a signed byte b is the low byte of the half 1024 + 128 + b
+// once its top bit is flipped, so one byte shuffle, one xor and one packed subtraction make two exact halves.  The block's
+// scale cannot ride in the operand (a half times a byte is no half), so the multipliers close a sum after every block:
+// two MFMAs of depth 16 into a fresh accumulator, then acc += d * sum in fp32 (run_weight_q8_0,
+// crates/neura-kernel/src/task/matmul.rs:309-318, weighs a block the same way).  The weighing of one block runs on the
+// vector unit while the matrix cores walk the next: the second block of a step is weighed behind the first MFMAs of the
+// step after it.  K is a multiple of 64; steps are walked four at a time, the ones past the end as zero codes and zero
+// scales, so every round issues the same loads and the waits count them exactly.
+typedef uint32_t u32x4_loose __attribute__((ext_vector_type(4), aligned(4)));
+constexpr size_t GEMM_Q8_LDS = sizeof(_Float16) * (4 * GT * GS) + sizeof(float) * 2 * 2 * GT;
+
+__global__ __launch_bounds__(512) void gemm_q8_0_mfma_kernel(GemmQ4Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);                                   // [2]
+    _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);  // [2]
+    float(*dds)[2][GT] = reinterpret_cast<float(*)[2][GT]>(gemm_lds + sizeof(_Float16) * 4 * GT * GS);         // [2][block of the step]: d of every weight row
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
+    const uint32_t steps = p.K / 64u, walked = (steps + 3u) & ~3u;
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    typedef const __attribute__((address_space(1))) u32x4_loose *global_loose4;
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------ stagers
+        const uint32_t tid = threadIdx.x - 256u;
+        const uint32_t srow = tid >> 1, sh = tid & 1u;
+        const uint32_t column = min(n0 + srow, p.N - 1u);
+        const uint8_t *wrow = column < p.end0   ? p.W + (size_t)column * p.row_bytes
+                              : column < p.end1 ? p.W1 + (size_t)(column - p.end0) * p.row_bytes
+                                                : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
+        const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
+        u32x4 qa[4], qb[4], av[4][4];  // by slot = step % 4
+        uint32_t qc[4];
+        auto fetch = [&](int g, uint32_t step) {
+            const uint32_t s = min(step, steps - 1u);  // past the end the last step is fetched again and dropped
+            const uintptr_t at = (uintptr_t)(wrow + (size_t)(2u * s + sh) * 34u), low = at & ~(uintptr_t)3;
+            qa[g] = *(global_loose4)low;
+            qb[g] = *(global_loose4)(low + 16u);
+            // a block on a word boundary ends two bytes into the ninth word: those two only are read (the last block of a
+            // tensor ends where its allocation may)
+            if (at & 2u) qc[g] = *(const __attribute__((address_space(1))) uint32_t *)(low + 32u);
+            else qc[g] = *(const __attribute__((address_space(1))) uint16_t *)(low + 32u);
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[g][i] = *(global_uint4)(uintptr_t)(arow + (size_t)s * 64u + 8 * i);
+        };
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            fetch(g, (uint32_t)g);
+            __builtin_amdgcn_sched_barrier(0);  // slot 0 goes out first: the loop waits for the oldest slot only
+        }
+        const half2_t offset = {(_Float16)1152.0f, (_Float16)1152.0f};
+        for (uint32_t first = 0; first < walked; first += 4) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint32_t buf = g & 1u, step = first + g;
+                const bool odd = ((uintptr_t)(wrow + (size_t)(2u * min(step, steps - 1u) + sh) * 34u) & 2u) != 0;
+                const uint32_t live = step < steps ? 0xffffffffu : 0u;
+                const uint32_t words[9] = {qa[g].x, qa[g].y, qa[g].z, qa[g].w, qb[g].x, qb[g].y, qb[g].z, qb[g].w, qc[g]};
+                const uint32_t scale_bits = (odd ? words[0] >> 16 : words[0] & 0xffffu) & live;
+                uint32_t out[16];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const uint32_t codes = (odd ? words[j + 1] : __funnelshift_r(words[j], words[j + 1], 16)) & live;
+                    // element order inside a word: 0, 2 then 1, 3, the order the activations were packed in
+                    const uint32_t even = __builtin_amdgcn_perm(0u, codes, 0x0c020c00u) ^ 0x64806480u;
+                    const uint32_t uneven = __builtin_amdgcn_perm(0u, codes, 0x0c030c01u) ^ 0x64806480u;
+                    out[2 * j] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even) - offset);
+                    out[2 * j + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, uneven) - offset);
+                }
+                u32x4 *bdst = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u * sh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) bdst[i] = u32x4{out[4 * i], out[4 * i + 1], out[4 * i + 2], out[4 * i + 3]};
+                dds[buf][sh][srow] = (float)__builtin_bit_cast(_Float16, (uint16_t)scale_bits);
+                u32x4 *adst = reinterpret_cast<u32x4 *>(&As[buf][srow][32u * sh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) adst[i] = av[g][i];
+                fetch(g, step + 4u);  // the slot is free: the same slot of the next round goes out
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();  // step is staged; the multipliers are done with the step before it
+            }
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- multipliers
+    const uint32_t wm = wave >> 1, wn = wave & 1u, l32 = lane & 31u, part = lane >> 5;
+    f32x16 acc[2][2], tmp[2][2][2], zero;
+#pragma unroll
+    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = zero, tmp[0][i][j] = zero, tmp[1][i][j] = zero;
+    float late[2] = {0.0f, 0.0f};  // the scales of the block whose sums wait in tmp[1]
+
+    auto weigh = [&](int h, const float *scales) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(scales[j], tmp[h][i][j][e], acc[i][j][e]);
+    };
+
+    for (uint32_t step = 0; step < walked; step++) {
+        const uint32_t buf = step & 1u;
+        __syncthreads();  // the step is staged
+        float early[2], next[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) early[j] = dds[buf][0][64u * wn + 32u * j + l32], next[j] = dds[buf][1][64u * wn + 32u * j + l32];
+        half8_t a[2][2], b[2][2];
+        auto operands = [&](int kk) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) a[kk & 1][i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
+#pragma unroll
+            for (int j = 0; j < 2; j++) b[kk & 1][j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
+        };
+        operands(0);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            if (kk < 3) operands(kk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    tmp[kk >> 1][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk & 1][i], b[kk & 1][j], (kk & 1) ? tmp[kk >> 1][i][j] : zero, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // the sums the matrix cores are not writing are weighed meanwhile: the block before this step's first behind
+            // its first MFMAs, this step's first behind the MFMAs of its second
+            if (kk == 0) weigh(1, late);
+            if (kk == 2) weigh(0, early);
+            if (kk == 0 || kk == 2) __builtin_amdgcn_sched_barrier(0);
+        }
+        late[0] = next[0], late[1] = next[1];
+    }
+    weigh(1, late);
+    // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t n = n0 + 64u * wn + 32u * j + l32;
+            if (n >= p.N) continue;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t row = m0 + 64u * wm + 32u * i + 8u * q + 4u * part;  // first of four rows of A'
+                if (p.split) {
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const uint32_t m = (row >> 1) + e;
+                        if (m >= p.M) continue;
+                        float value = fmaf(acc[i][j][4 * q + 2 * e + 1], 0.00048828125f, acc[i][j][4 * q + 2 * e]) * p.unscale[m];
+                        const size_t at = (size_t)m * p.ldy + n;
+                        p.Y[at] = p.residual ? p.residual[at] + value : value;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t m = row + e;
+                        if (m >= p.M) continue;
+                        const size_t at = (size_t)m * p.ldy + n;
+                        p.Y[at] = p.residual ? p.residual[at] + acc[i][j][4 * q + e] : acc[i][j][4 * q + e];
+                    }
+                }
+            }
+        }
+}
+
 // bytes of device scratch a Q4_K wide product over M activation rows of K numbers packs into
 size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows) {
     const size_t rows = half_rows ? M : (size_t)2 * M;
-    return rows * K * sizeof(_Float16) + rows * (K / 256u) * 16u * sizeof(_Float16) + (size_t)M * sizeof(float);
+    return rows * K * sizeof(_Float16) + rows * ((K + 255u) / 256u) * 16u * sizeof(_Float16) + (size_t)M * sizeof(float);
 }
 
-static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
+static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
     GemmQ4Params p{};
     p.W = static_cast<const uint8_t *>(a.W);
     p.W1 = static_cast<const uint8_t *>(a.W_more[0]), p.W2 = static_cast<const uint8_t *>(a.W_more[1]);
@@ -458,7 +633,7 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
         return fail(NH_E_ARGUMENT, "matrices stacked at columns %u and %u of %u do not fall on tiles of %d", a.end[0], a.end[1], a.N, GT);
     p.N = a.N;
     p.K = a.K;
-    p.row_bytes = (uint32_t)payload_bytes(NH_Q4_K, a.K);
+    p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     p.Y = a.Y;
     p.residual = a.residual;
     p.ldy = a.ldy;
@@ -467,7 +642,7 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     p.rows = half_rows ? a.M : 2 * a.M;
     p.split = half_rows ? 0 : 1;
     // scratch: [rows][K] halves, [rows][K / 256][16] sums, M row scales
-    const size_t halves = (size_t)p.rows * a.K * sizeof(_Float16), sums = (size_t)p.rows * (a.K / 256u) * 16u * sizeof(_Float16);
+    const size_t halves = (size_t)p.rows * a.K * sizeof(_Float16), sums = (size_t)p.rows * ((a.K + 255u) / 256u) * 16u * sizeof(_Float16);
     uint8_t *room = static_cast<uint8_t *>(scratch(d, gemm_q4k_scratch_bytes(a.M, a.K, half_rows)));
     if (!room) return NH_E_MEMORY;
     _Float16 *A = reinterpret_cast<_Float16 *>(room), *S = reinterpret_cast<_Float16 *>(room + halves);
@@ -490,32 +665,36 @@ static int32_t launch_gemm_q4k_mfma(nh_device *d, const GemmArgs &a) {
     static bool sized = false;
     if (!sized) {
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q8_LDS));
         sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
-    hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
+    if (a.element == NH_Q8_0) hipLaunchKernelGGL(gemm_q8_0_mfma_kernel, grid, dim3(512), GEMM_Q8_LDS, d->stream, p);
+    else hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
 
-// the matrix-core form takes Q4_K rows of whole super-blocks read from 16-byte aligned addresses
+// the matrix-core forms take Q4_K rows of whole super-blocks and Q8_0 rows of whole pairs of blocks, read from 16-byte
+// aligned addresses (a Q8_0 matrix from a 4-byte one; its rows may start on any half word)
 static bool mfma_takes(int32_t element, uint32_t K, const void *X, const void *W) {
     const char *held = getenv("NEURA_HIP_GEMM_MFMA");
     const bool wanted = !(held && held[0] == '0');
-    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & 15u) == 0;
-    return wanted && aligned && element == NH_Q4_K && K % 256u == 0;
+    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q8_0 ? 3u : 15u)) == 0;
+    return wanted && aligned && K > 0 && ((element == NH_Q4_K && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
 }
 
 bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1) {
     if (!mfma_takes(element, K, X, W0)) return false;
-    if (W1 && (((uintptr_t)W1 & 15u) || end0 % GT)) return false;
-    if (W2 && (((uintptr_t)W2 & 15u) || end1 % GT || !W1)) return false;
+    const uintptr_t loose = element == NH_Q8_0 ? 3u : 15u;
+    if (W1 && (((uintptr_t)W1 & loose) || end0 % GT)) return false;
+    if (W2 && (((uintptr_t)W2 & loose) || end1 % GT || !W1)) return false;
     return true;
 }
 
 int32_t launch_gemm(nh_device *d, const GemmArgs &a) {
     if (!a.M || !a.N) return NH_OK;
-    if (mfma_takes(a.element, a.K, a.X, a.W)) return launch_gemm_q4k_mfma(d, a);
+    if (mfma_takes(a.element, a.K, a.X, a.W)) return launch_gemm_mfma(d, a);
     if (a.W_more[0] || a.W_more[1] || a.packed || a.norm_w || a.gate)
         return fail(NH_E_ARGUMENT, "this wide product stacks no matrices, reuses no packed activations and packs rows as they lie (ask gemm_stacks first)");
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM), block(256);

@@ -302,7 +302,9 @@ def test_reference_wide_product_test(device, element):
 
 
 @pytest.mark.parametrize("element,M,N,K,half", [(NH_Q4_K, 70, 130, 512, True), (NH_Q4_K, 512, 256, 3584, True), (NH_Q4_K, 33, 64, 256, False),
-                                                (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q6_K, 70, 130, 512, False),
+                                                (NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q8_0, 200, 300, 4864, False),
+                                                (NH_Q8_0, 130, 128, 192, True), (NH_Q8_0, 512, 1152, 896, False), (NH_Q8_0, 16, 32, 96, False),
+                                                (NH_Q8_0, 9, 129, 320, False), (NH_Q6_K, 70, 130, 512, False),
                                                 (NH_Q6_K, 40, 64, 3584, True), (NH_Q5_K, 70, 130, 512, True), (NH_Q5_K, 33, 64, 3584, False),
                                                 (NH_Q3_K, 70, 130, 512, False), (NH_Q3_K, 40, 64, 3584, True)])
 def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
