@@ -70,43 +70,80 @@ def weight_bytes_per_token(shape, element, layers, mixed=None):
     return total
 
 
-def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=20.0):
+def host_threads():
+    """(threads the CPU legs use, cores the machine shows): the scheduler's affinity mask, at most the 16 cores a one-GPU
+    job is given on a shared host whatever the machine shows"""
+    shown = os.cpu_count() or 1
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        allowed = shown
+    return max(1, min(allowed, int(os.environ.get("NEURA_BENCH_CPU_THREADS", "16")))), shown
+
+
+def native_oracle():
+    """Compiles the oracle for this machine (-O3 -march=native -ffp-contract=off) and returns the build's flags; the
+    portable build the parity tests use is timed instead where no compiler is at hand."""
+    import subprocess
+
+    directory = os.path.join(ROOT, "oracle")
+    try:
+        subprocess.run(["make", "-B", "-C", directory, "native"], check=True, capture_output=True, timeout=120)
+        os.environ["NEURA_ORACLE_LIBRARY"] = os.path.join(directory, "libneura_oracle_native.so")
+        return "-O3 -march=native -ffp-contract=off"
+    except (OSError, subprocess.SubprocessError):
+        return "-O2 -march=x86-64-v2 -ffp-contract=off (no native build here)"
+
+
+def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=12.0):
     """Times the oracle's decode step (the checker, used here only as the reported CPU baseline)
     on a bounded sample: a decoder cut to `sample_layers` layers plus the output head, at the
-    same context length; the full-depth rate is extrapolated from the per-layer and head times."""
+    same context length; the full-depth rate is extrapolated from the per-layer and head times.
+    Two legs: every core this job may use, and one thread."""
+    flags = native_oracle()
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle
 
-    cores = min(os.cpu_count() or 1, 16)
-    sample_layers = min(layers, 4)
-    model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=sample_layers)
+    cores, shown = host_threads()
     rng = np.random.default_rng(7)
-    for held in model.cache_k + model.cache_v:  # a filled cache, as on the device
-        held[:] = rng.standard_normal(held.size).astype(np.float16).view(np.uint16)
     cursor = context - 1
-    model.forward([1], 1, [cursor], threads=cores)  # warm-up
-    began = time.perf_counter()
-    runs = 0
-    while runs < 3 or (time.perf_counter() - began < seconds_budget and runs < 50):
-        model.forward([1], 1, [cursor], threads=cores)
-        runs += 1
-    with_head = (time.perf_counter() - began) / runs
-    # head alone: a zero-layer model
-    head_model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=0)
-    head_model.forward([1], 1, [cursor], threads=cores)
-    began = time.perf_counter()
-    for _ in range(3):
-        head_model.forward([1], 1, [cursor], threads=cores)
-    head = (time.perf_counter() - began) / 3
-    per_layer = max(with_head - head, 0.0) / sample_layers
-    step = head + per_layer * layers
+
+    def step_seconds(threads, sample_layers, budget, most):
+        model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=sample_layers)
+        for held in model.cache_k + model.cache_v:  # a filled cache, as on the device
+            held[:] = rng.standard_normal(held.size).astype(np.float16).view(np.uint16)
+        model.forward([1], 1, [cursor], threads=threads)  # warm-up
+        began = time.perf_counter()
+        runs = 0
+        while runs < 2 or (time.perf_counter() - began < budget and runs < most):
+            model.forward([1], 1, [cursor], threads=threads)
+            runs += 1
+        with_head = (time.perf_counter() - began) / runs
+        # head alone: a zero-layer model
+        head_model = oracle.Model(shape, element, host_tensors, batch=1, context=context, layers=0)
+        head_model.forward([1], 1, [cursor], threads=threads)
+        began = time.perf_counter()
+        for _ in range(2):
+            head_model.forward([1], 1, [cursor], threads=threads)
+        head = (time.perf_counter() - began) / 2
+        per_layer = max(with_head - head, 0.0) / sample_layers
+        return head + per_layer * layers, runs
+
+    sample_layers = min(layers, 4)
+    step, runs = step_seconds(cores, sample_layers, seconds_budget, 50)
+    single, single_runs = step_seconds(1, 1, seconds_budget / 2, 3)
     return {
         "value": 1.0 / step,
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": "%d decode steps of a %d-layer cut of the %d-layer decoder plus the output head at context %d; "
-                  "full depth extrapolated as head + %d x per-layer time (%.3f s/step)" % (runs, sample_layers, layers, context, layers, step),
+        "single_thread": {"value": 1.0 / single, "unit": "tokens/s", "cores": 1},
+        "host_cores_shown": shown,
+        "build": flags,
+        "sample": "%d decode steps of a %d-layer cut of the %d-layer decoder plus the output head at context %d on %d threads (this job's "
+                  "share of a host that shows %d cores); full depth extrapolated as head + %d x per-layer time (%.3f s/step); the "
+                  "single-thread figure from %d steps of a 1-layer cut the same way (%.2f s/step)" %
+                  (runs, sample_layers, layers, context, cores, shown, layers, step, single_runs, single),
     }
 
 

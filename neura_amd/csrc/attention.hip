@@ -707,13 +707,11 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
-    // a chunk of query rows goes to the matrix cores (NEURA_HIP_ATTENTION_TILE=0 keeps the row-at-a-time kernel)
+    // a chunk of query rows goes to the matrix cores
     {
-        const char *held = getenv("NEURA_HIP_ATTENTION_TILE");
-        const bool wanted = !(held && held[0] == '0');
         const bool aligned = ((uintptr_t)a.out & 15u) == 0 && a.o_sh % 4 == 0 && a.o_sb % 4 == 0 && a.o_sr % 4 == 0 && ((uintptr_t)a.cache_k & 15u) == 0 &&
                              ((uintptr_t)a.cache_v & 15u) == 0;
-        if (wanted && aligned && a.rows >= 4 && (a.width == 64 || a.width == 128) && p.groups >= 1) {
+        if (aligned && a.rows >= 4 && (a.width == 64 || a.width == 128) && p.groups >= 1) {
             const uint32_t rows_per_wave = 32u / p.groups;
             dim3 grid(a.kv_heads * a.batch, (a.rows + 4u * rows_per_wave - 1u) / (4u * rows_per_wave));
             p.sections = 1;
@@ -724,17 +722,13 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
         }
     }
     // one query row a plane: the group's query heads are the columns of the matrix cores
-    // (NEURA_HIP_ATTENTION_DECODE_TILE=0 keeps the row-at-a-time kernel)
     {
-        const char *held = getenv("NEURA_HIP_ATTENTION_DECODE_TILE");
-        const bool wanted = !(held && held[0] == '0');
         const bool aligned = ((uintptr_t)a.cache_k & 15u) == 0 && ((uintptr_t)a.cache_v & 15u) == 0;
         const uint32_t planes = a.kv_heads * a.batch;
-        if (wanted && aligned && a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16) {
+        if (aligned && a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16) {
             // sections of at least 256 keys (two tiles a wave) where the planes alone fill the chip, of 128 (one tile a wave)
             // where they do not; enough workgroups to fill the chip twice over
-            const char *keys_held = getenv("NEURA_HIP_ATTENTION_DECODE_KEYS");
-            const uint32_t thinnest = keys_held && atoi(keys_held) > 0 ? (uint32_t)atoi(keys_held) : (planes >= 8 ? 256u : 128u);
+            const uint32_t thinnest = planes >= 8 ? 256u : 128u;
             uint32_t wanted_sections = ((uint32_t)d->compute_units * 2 + planes - 1) / planes;
             const uint32_t most = (a.keys + thinnest - 1) / thinnest;
             p.sections = wanted_sections < 1 ? 1 : (wanted_sections > most ? most : wanted_sections);
@@ -756,8 +750,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     // sections of the context: enough workgroups to fill the chip four times over, none thinner
     // than 64 keys (thinner sections cost more in the fold than they gain in the walk)
-    const char *held = getenv("NEURA_HIP_ATTENTION_KEYS");
-    const uint32_t thinnest = held && atoi(held) > 0 ? (uint32_t)atoi(held) : 64u;
+    const uint32_t thinnest = 64u;
     uint32_t wanted = ((uint32_t)d->compute_units * 4 + units - 1) / units;
     uint32_t most = (a.keys + thinnest - 1) / thinnest;
     p.sections = wanted < 1 ? 1 : (wanted > most ? most : wanted);

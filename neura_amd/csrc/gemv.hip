@@ -2046,8 +2046,6 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     // rows per lane group and pass: four rows amortise the cross-lane sum and keep more bytes
     // in flight per wave, two rows give twice the waves; tall matrices take four
     int R = (a.N >= 16384u && RB == 1) ? 4 : 2;
-    R = env_int("NEURA_HIP_GEMV_ROWS", R);
-    if (R != 2 && R != 4) R = 2;
     if (RB >= 4) R = 2;
     // the decode kernel walks R rows of ONE matrix per lane group: every matrix boundary must be a
     // multiple of R (with swiglu the halves interleave, so N/2 must be a multiple of R/2)
@@ -2064,7 +2062,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     if (q4) {
         blocks_x = (p.row_groups + 3) / 4;
         // one resident round of workgroups: 3 per compute unit at four rows (136 registers), 4 at two
-        uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_GEMV_WGS", R == 4 ? 3 : 4) / p.splits;
+        uint32_t most = (uint32_t)d->compute_units * (R == 4 ? 3u : 4u) / p.splits;
         if (most < 1) most = 1;
         if (blocks_x > most) blocks_x = most;
         uint32_t slice = p.blocks_per_split * 256u;
@@ -2074,7 +2072,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         p.chunks_per_row = (15u + slice_bytes + 15u) / 16u;
         uint32_t tiles = (p.row_groups + 3) / 4;
         blocks_x = tiles;
-        uint32_t most = (uint32_t)d->compute_units * (uint32_t)env_int("NEURA_HIP_GEMV_WGS", 4) / p.splits;
+        uint32_t most = (uint32_t)d->compute_units * 4u / p.splits;
         if (most < 1) most = 1;
         if (blocks_x > most) blocks_x = most;
         uint32_t slice = p.blocks_per_split * 32u;
@@ -2082,18 +2080,10 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     }
     if (lds > 64 * 1024) return fail(NH_E_ARGUMENT, "a product of depth %u stages %zu bytes where a workgroup holds 65536", a.K, lds);
     dim3 grid(blocks_x, p.splits), block(256);
-    const bool pipe = env_int("NEURA_HIP_GEMV_PIPE", 0) != 0;
-    const int nw = env_int("NEURA_HIP_GEMV_WAVES", 4);
     profile_mark(d);
 #define NH_LAUNCH(KERNEL, RR) hipLaunchKernelGGL((KERNEL<RR, RB>), grid, block, lds, d->stream, p)
-#define NH_DECODE(RR, GG)                                                                                              \
-    do {                                                                                                               \
-        if (pipe) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, true, 4>), grid, block, lds, d->stream, p);       \
-        else if (nw == 16) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 16>), dim3((blocks_x + 3) / 4, p.splits), dim3(1024), lds, d->stream, p); \
-        else if (nw == 8) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 8>), dim3((blocks_x + 1) / 2, p.splits), dim3(512), lds, d->stream, p); \
-        else hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p);           \
-    } while (0)
-    const bool q8_direct = !q4 && RB == 1 && fast && p.nblk <= 256u && env_int("NEURA_HIP_Q8_DECODE", 1) != 0;
+#define NH_DECODE(RR, GG) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p)
+    const bool q8_direct = !q4 && RB == 1 && fast && p.nblk <= 256u;
     if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1) && !(q8_direct && R == 2 && p.nblk <= 64u))
         return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (q4 && RB == 1 && fast && a.rope) {
@@ -2197,8 +2187,7 @@ template <int KS, int NW>
 static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t P, uint32_t blocks_x, size_t lds) {
     if (P == 1) {
         // sixteen waves leave 128 registers a lane: two super-blocks in flight fit, four would spill
-        const int depth = env_int("NEURA_HIP_MFMA_DEPTH", NW == 16 ? 2 : 4);
-        if (depth == 2 || NW == 16) return launch_mfma_instance<KS, NW, 1, 2>(d, p, blocks_x, lds);
+        if (NW == 16) return launch_mfma_instance<KS, NW, 1, 2>(d, p, blocks_x, lds);
         return launch_mfma_instance<KS, NW, 1, 4>(d, p, blocks_x, lds);
     }
     if (P == 2) return launch_mfma_instance<KS, NW, 2, 2>(d, p, blocks_x, lds);
@@ -2210,10 +2199,9 @@ static size_t mfma_staged(uint32_t blocks, uint32_t P) { return (size_t)blocks *
 
 // whether the deep kernel (one tile per workgroup, sixteen waves along K) serves this product
 static bool mfma_goes_deep(const nh_device *d, const GemvArgs &a) {
-    const int mode = env_int("NEURA_HIP_MFMA_DEEP", 1);
-    if (mode == 0 || a.rows != 1 || a.swiglu || a.norm_w || a.W[1] || a.W[2]) return false;
+    if (a.rows != 1 || a.swiglu || a.norm_w || a.W[1] || a.W[2]) return false;
     // a matrix short enough that its tiles do not even fill the device once, and rows deep enough to feed sixteen waves
-    return mode == 2 || (a.N / 16u <= (uint32_t)d->compute_units && a.K / 256u >= 32u);
+    return a.N / 16u <= (uint32_t)d->compute_units && a.K / 256u >= 32u;
 }
 
 static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
@@ -2263,19 +2251,16 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
         const uint32_t slots = (uint32_t)d->compute_units * 16u;
         uint32_t ks = 1;
         while (ks < 16 && p.tiles * p.splits * ks < slots && ks * 2 <= p.slice_blocks) ks *= 2;
-        ks = (uint32_t)env_int("NEURA_HIP_MFMA_KS", (int)ks);
-        if (ks != 1 && ks != 2 && ks != 4 && ks != 8 && ks != 16) ks = 1;
         if (P > 1 && ks > 8) ks = 8;  // sixteen-wave workgroups leave 128 registers a lane, too few for several activation rows
         // waves per workgroup: four measured best (larger workgroups stage the activations less often but stream slower)
-        uint32_t nw = (uint32_t)env_int("NEURA_HIP_MFMA_NW", 4);
-        if (nw != 4 && nw != 8 && nw != 16) nw = 4;
+        uint32_t nw = 4;
         if (nw < ks) nw = ks;
         const uint32_t tiles_per_group = nw / ks;
         const size_t staged = mfma_staged(p.slice_blocks, P);
         const size_t lds = staged + (ks > 1 ? (size_t)2 * nw * P * 64u : 0);
         uint32_t blocks_x = (p.tiles + tiles_per_group - 1) / tiles_per_group;
         // resident waves per compute unit, by register use: 4 per SIMD (one or two activation rows), 3 for four
-        uint32_t resident = (uint32_t)env_int("NEURA_HIP_MFMA_WAVES", P == 4 ? 12 : 16) / nw;
+        uint32_t resident = (P == 4 ? 12u : 16u) / nw;
         const uint32_t by_lds = (uint32_t)((160 * 1024) / (lds + 1536));
         if (resident > by_lds) resident = by_lds;
         uint32_t most = (uint32_t)d->compute_units * (resident ? resident : 1u) / p.splits;
@@ -2313,14 +2298,14 @@ bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     }
     if (a.element == NH_Q8_0) {
         // the direct Q8_0 decode kernel, a row of blocks inside one wave
-        if (a.K % 32u != 0 || a.K > 2048u || env_int("NEURA_HIP_Q8_DECODE", 1) == 0) return false;
+        if (a.K % 32u != 0 || a.K > 2048u ) return false;
         if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 32u * 34u) >= (1ull << 32)) return false;
         if (a.end[0] % 2u || a.end[1] % 2u || a.N % 2u) return false;
     } else {
         if (a.element != NH_Q4_K || a.K % 256u != 0 || a.K > 4096u) return false;
         if (a.N >= 16384u || a.N < 2u || (uint64_t)a.N * (a.K / 256u * 144u) >= (1ull << 32)) return false;
     }
-    if (env_int("NEURA_HIP_GEMV_ROWS", 2) != 2 || env_int("NEURA_HIP_MFMA", 1) == 2) return false;
+    if (env_int("NEURA_HIP_MFMA", 1) == 2) return false;
     const uint32_t width = rope.width;
     if (width < 2 || (width & (width - 1u)) != 0) return false;
     if (rope.q_rows % width || rope.k_rows % width || a.N % width || rope.q_rows > rope.k_rows || rope.k_rows > a.N) return false;
@@ -2400,8 +2385,7 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     profile_mark(d);
     int32_t status;
     // with eight staged rows, a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
-    const int forced = env_int("NEURA_HIP_MFMA32_KS", 0);
-    const bool few = forced ? forced == 16 : p.tiles * p.splits < 2u * (uint32_t)d->compute_units;
+    const bool few = p.tiles * p.splits < 2u * (uint32_t)d->compute_units;
     if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.slice_blocks, 1, 4));
     else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
     else status = launch_mfma32_instance<4, 16, 4>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
@@ -2478,8 +2462,7 @@ static int32_t launch_f16_tiles(nh_device *d, const GemvArgs &a) {
     }
     profile_mark(d);
     // a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
-    const int forced = env_int("NEURA_HIP_F16_TILES_KS", 0);
-    const bool few = forced ? forced == 16 : p.tiles * p.splits < 4u * (uint32_t)d->compute_units;
+    const bool few = p.tiles * p.splits < 4u * (uint32_t)d->compute_units;
     const size_t lds = f16_tiles_lds(p.slice_blocks, 16);
     int32_t status = few ? launch_f16_tiles_instance<16, 16>(d, p, lds) : launch_f16_tiles_instance<16, 4>(d, p, lds);
     if (status != NH_OK) return status;

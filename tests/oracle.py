@@ -34,7 +34,8 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIBRARY):
             subprocess.run(["make", "-C", ORACLE_DIR], check=True, capture_output=True)
-        held = ctypes.CDLL(LIBRARY)
+        # the benchmark's CPU-baseline leg may name another build of the same source (one compiled for the machine it times)
+        held = ctypes.CDLL(os.environ.get("NEURA_ORACLE_LIBRARY") or LIBRARY)
         held.oracle_f32_to_f16.restype = c_uint16
         held.oracle_f32_to_f16.argtypes = [c_float]
         held.oracle_f16_to_f32.restype = c_float

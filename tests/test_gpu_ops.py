@@ -217,6 +217,42 @@ def test_q4_k_product_on_32_row_tiles(device, monkeypatch, forced, N, K, rows):
     assert not np.isfinite(device.gemv(NH_Q4_K, raw, N, K, x)[0]).any()
 
 
+@pytest.mark.parametrize("tile16", ["1", "0"])
+@pytest.mark.parametrize("N,K", [(16, 256), (64, 3584), (4608, 3584), (3584, 18944), (37888, 3584), (1040, 768), (48, 2048), (272, 8960)])
+def test_q4_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K):
+    """One activation row against Q4_K rows: the 16-row tiles on the 16 x 16 x 64 integer MFMA (weights as nibbles, the
+    activation as three signed digit planes scaled per 64 numbers), and with NEURA_HIP_TILE16=0 the kernels that served
+    before it.  Activations over many orders of magnitude, with outliers that set a group's scale from any seat of it;
+    plain, with a residual (added in place), with SwiGLU; non-finite inputs stay visible and zeros give zeros."""
+    monkeypatch.setenv("NEURA_HIP_TILE16", tile16)
+    rng = np.random.default_rng(N + K)
+    raw = synth.q4_k_random(rng, N * K)
+    weights = oracle.unpack(NH_Q4_K, raw, N * K).reshape(N, K).astype(np.float64)
+    r = rng.standard_normal((1, N)).astype(np.float32)
+    for spread, outliers in ((2.0, False), (6.0, False), (6.0, True)):
+        x = (rng.standard_normal((1, K)) * np.exp(rng.uniform(-spread, spread, (1, K)))).astype(np.float32)
+        if outliers:
+            x[0, rng.integers(0, K, 24)] *= 1e4  # at any seat of a group
+        plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+        exact = weights @ x.astype(np.float64).T
+        got = device.gemv(NH_Q4_K, raw, N, K, x)
+        if spread == 2.0:
+            close(got, plain)  # past this spread the oracle's own fp32 sums are the looser side: the exact product judges
+        assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * max(1.0, np.abs(exact).max()))
+        tight(device.gemv(NH_Q4_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    if N % 32 == 0:
+        x = rng.standard_normal((1, K)).astype(np.float32)
+        x[0, rng.integers(0, K, 8)] *= 50.0
+        plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+        gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2 :].astype(np.float64)
+        want = gate / (1.0 + np.exp(-gate)) * up
+        close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+    x[0, 5] = np.inf
+    assert not np.isfinite(device.gemv(NH_Q4_K, raw, N, K, x)).any()
+    assert not np.isfinite(device.gemv(NH_Q4_K, raw, N, K, np.full((1, K), np.nan, np.float32))).any()
+    assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
+
+
 def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device, monkeypatch):
     monkeypatch.setenv("NEURA_HIP_MFMA", "2")
     rng = np.random.default_rng(2)
@@ -316,6 +352,32 @@ def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
     close(got, want)
     r = rng.standard_normal((M, N)).astype(np.float32)
     close(device.gemm(element, raw, N, K, X, residual=r), want + r)
+
+
+@pytest.mark.parametrize("element,M,N,K,half", [(NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q4_K, 70, 130, 512, True),
+                                                (NH_Q4_K, 33, 64, 256, False)])
+def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N, K, half):
+    """NEURA_HIP_GEMM_MFMA=0 keeps Q8_0 and Q4_K wide products on the tiled vector kernel that serves the shapes the matrix
+    cores do not take (rows that are not whole steps, unaligned operands)."""
+    monkeypatch.setenv("NEURA_HIP_GEMM_MFMA", "0")
+    rng = np.random.default_rng(M + N + K)
+    raw = synth.RANDOM[element](rng, N * K)
+    X = rng.standard_normal((M, K)).astype(np.float16 if half else np.float32)
+    close(device.gemm(element, raw, N, K, X), oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8))
+
+
+def test_q8_0_wide_product_of_the_small_decoder_s_shapes(device):
+    """The Q8_0 products of a 512-token fill of the 0.5B-shape decoder (hidden 896, FFN 4864, 14 heads of 64, 2 key heads), weights
+    N(0, 0.02) quantised as a checkpoint's are, fp32 activations over a few orders of magnitude: every output against fp32
+    accumulation."""
+    rng = np.random.default_rng(8)
+    for N, K in [(1152, 896), (896, 896), (4864, 896), (896, 4864)]:
+        raw = oracle.pack(NH_Q8_0, (rng.standard_normal(N * K) * 0.02).astype(np.float32))
+        X = (rng.standard_normal((512, K)) * np.exp(rng.uniform(-3, 3, (512, K)))).astype(np.float32)
+        want = oracle.gemm(NH_Q8_0, raw, N, K, X, threads=16)
+        got = device.gemm(NH_Q8_0, raw, N, K, X)
+        close(got, want, rel=1e-3, abs_=1e-2)
+        tight(got, want, 1e-5)
 
 
 def test_config3_wide_product_at_full_size(device):
