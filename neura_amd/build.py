@@ -26,8 +26,8 @@ def hipcc():
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
-# per file: the 16-row tile product weighs its matrix-core sums where they land, in vector registers
-EXTRA_FLAGS = {"gemv_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+# per file: the 16-row tile product and the attention kernels work on their matrix-core sums where they land, in vector registers
+EXTRA_FLAGS = {"gemv_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _compile(source):

@@ -66,7 +66,16 @@ __device__ __forceinline__ void unpack8(const u32x4 &raw, float (&out)[8]) {
 }
 
 // exp(max(argument, -104)) (crates/neura-kernel/src/substrate.rs:110-116)
-__device__ __forceinline__ float softmax_exp(float argument) { return expf(fmaxf(argument, -104.0f)); }
+// e^argument for the arguments a running softmax meets (never above zero; -inf gives 0, below -104 the result is zero in
+// single precision anyway).  One hardware exp2 of argument * log2(e), the product carried in two parts so the result keeps
+// the accuracy of the instruction; no branches, so a lane's eight weights of a tile stay one straight run of instructions.
+__device__ __forceinline__ float softmax_exp(float argument) {
+    const float x = fmaxf(argument, -104.0f);
+    const float scaled = x * 1.44269502e+00f;
+    const float rest = fmaf(x, 1.44269502e+00f, -scaled) + x * 1.92596299e-08f;  // what the rounded product left out
+    const float power = __builtin_amdgcn_exp2f(scaled);
+    return fmaf(power, rest * 6.93147182e-01f, power);
+}
 
 // sum over the LPK lanes that share a key: DPP adds inside a row of 16 lanes
 template <int LPK>
@@ -515,10 +524,11 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
     constexpr int VPITCH = TK + 4;          // halves per staged value channel
     constexpr int PIECES = TK * WIDTH / 8 / 64;  // 16-byte pieces of a value tile per lane
     // the waves' value corners and, once every wave has left the walk, their sums share one buffer
-    constexpr size_t VT_BYTES = sizeof(uint16_t) * 4 * WIDTH * VPITCH, MERGED_BYTES = sizeof(float) * 4 * 16 * (WIDTH + 2);
-    __shared__ __attribute__((aligned(16))) uint8_t shared_rows[VT_BYTES > MERGED_BYTES ? VT_BYTES : MERGED_BYTES];
+    constexpr size_t VT_BYTES = sizeof(uint16_t) * 4 * WIDTH * VPITCH, MERGED_BYTES = sizeof(float) * 4 * 16 * (WIDTH + 4), STATS_BYTES = sizeof(float) * 8 * 16;
+    constexpr size_t ROWS_BYTES = VT_BYTES > MERGED_BYTES ? VT_BYTES : MERGED_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t shared_rows[ROWS_BYTES + STATS_BYTES];
     uint16_t(*vt)[WIDTH][VPITCH] = reinterpret_cast<uint16_t(*)[WIDTH][VPITCH]>(shared_rows);
-    float(*merged)[16][WIDTH + 2] = reinterpret_cast<float(*)[16][WIDTH + 2]>(shared_rows);  // per wave and column: the channel sums, then the running top and mass
+    float(*merged)[16][WIDTH + 4] = reinterpret_cast<float(*)[16][WIDTH + 4]>(shared_rows);  // per wave and column: the weighed channel sums (rows 16 bytes apart in phase)
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t n = lane & 15u, kq = lane >> 4;
@@ -538,10 +548,13 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
     float q_raw[STEPS][8];
     {
         const float *src = p.q + (uint64_t)(kvh * G + min(n, G - 1u)) * p.q_sh + (uint64_t)b * p.q_sb;
+        // a column past the group reads the group's last head: its scores are masked, and no column reaches another's sums
 #pragma unroll
-        for (int s = 0; s < STEPS; s++)
-#pragma unroll
-            for (int i = 0; i < 8; i++) q_raw[s][i] = held ? src[32 * s + 8 * kq + i] : 0.0f;
+        for (int s = 0; s < STEPS; s++) {
+            const float4 low = *reinterpret_cast<const float4 *>(src + 32 * s + 8 * kq), high = *reinterpret_cast<const float4 *>(src + 32 * s + 8 * kq + 4);
+            q_raw[s][0] = low.x, q_raw[s][1] = low.y, q_raw[s][2] = low.z, q_raw[s][3] = low.w;
+            q_raw[s][4] = high.x, q_raw[s][5] = high.y, q_raw[s][6] = high.z, q_raw[s][7] = high.w;
+        }
     }
     f32x4_t acc[BLOCKS];
 #pragma unroll
@@ -665,30 +678,34 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
         __builtin_amdgcn_wave_barrier();  // the next tile overwrites the corner
     }
     // ---- the four waves meet: register e of block d is channel 16 d + 4 kq + e of this lane's column
-    __syncthreads();  // every wave is done with its corner
+    // a wave's sums are weighed by e^(its top - the largest of the four) before they leave its registers: the four tops and
+    // masses of a column cross in LDS first (lanes kq = 0 hold a column's statistics; every lane of the column reads them back)
+    float(*tops)[16] = reinterpret_cast<float(*)[16]>(shared_rows + ROWS_BYTES);  // [4 waves][16 columns], then the masses
+    float(*masses)[16] = tops + 4;
+    if (kq == 0) tops[wave][n] = top, masses[wave][n] = mass;
+    __syncthreads();  // the statistics are out, and every wave is done with its corner
+    float largest = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; w++) largest = fmaxf(largest, tops[w][n]);
+    const float mine = top == -INFINITY ? 0.0f : softmax_exp(top - largest) * (1.0f / 1024.0f);
 #pragma unroll
     for (int d = 0; d < BLOCKS; d++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) merged[wave][n][16 * d + 4 * kq + e] = acc[d][e] * (1.0f / 1024.0f);
-    if (kq == 0) merged[wave][n][WIDTH] = top, merged[wave][n][WIDTH + 1] = mass;
+        *reinterpret_cast<f32x4_t *>(&merged[wave][n][16 * d + 4 * kq]) = acc[d] * mine;
     __syncthreads();
     for (uint32_t index = tid; index < G * WIDTH; index += 256) {
         const uint32_t g = index / WIDTH, c = index % WIDTH;
-        float largest = -INFINITY;
+        const float value = (merged[0][g][c] + merged[1][g][c]) + (merged[2][g][c] + merged[3][g][c]);
+        float total = 0.0f, highest = -INFINITY;
+        if (c == 0 || p.sections == 1) {
 #pragma unroll
-        for (int w = 0; w < 4; w++) largest = fmaxf(largest, merged[w][g][WIDTH]);
-        float value = 0.0f, total = 0.0f;
+            for (int w = 0; w < 4; w++) highest = fmaxf(highest, tops[w][g]);
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const float held_top = merged[w][g][WIDTH];
-            const float weight = held_top == -INFINITY ? 0.0f : softmax_exp(held_top - largest);
-            value = fmaf(merged[w][g][c], weight, value);
-            total = fmaf(merged[w][g][WIDTH + 1], weight, total);
+            for (int w = 0; w < 4; w++) total = fmaf(masses[w][g], tops[w][g] == -INFINITY ? 0.0f : softmax_exp(tops[w][g] - highest), total);
         }
         if (p.sections > 1) {
             float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (WIDTH + 2);
             dst[c] = value;
-            if (c == 0) dst[WIDTH] = largest, dst[WIDTH + 1] = total;
+            if (c == 0) dst[WIDTH] = highest, dst[WIDTH + 1] = total;
         } else {
             const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
             p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + c] = value * normalized;
@@ -723,7 +740,8 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     // one query row a plane: the group's query heads are the columns of the matrix cores
     {
-        const bool aligned = ((uintptr_t)a.cache_k & 15u) == 0 && ((uintptr_t)a.cache_v & 15u) == 0;
+        const bool aligned = ((uintptr_t)a.cache_k & 15u) == 0 && ((uintptr_t)a.cache_v & 15u) == 0 && ((uintptr_t)a.q & 15u) == 0 && a.q_sh % 4 == 0 &&
+                             a.q_sb % 4 == 0;
         const uint32_t planes = a.kv_heads * a.batch;
         if (aligned && a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16) {
             // sections of at least 256 keys (two tiles a wave) where the planes alone fill the chip, of 128 (one tile a wave)
