@@ -67,12 +67,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     const uint32_t row_bytes = p.row_bytes;
     const uint32_t half_width = p.rope_width >> 1, tiles_per_head = max(half_width >> 3, 1u);
     const uint32_t first_tile = blockIdx.x, hop = gridDim.x;
-    auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, r, q](uint32_t tile) -> const uint8_t * {
+    // a plain tile may hold fewer than 16 rows (a matrix of 3584 rows is 256 tiles of 14, one a compute unit, where it is 224
+    // of 16): the columns past them walk the tile's last row again and are never written
+    const uint32_t tile_rows = MODE == TILE16_PLAIN ? p.tile_rows : 16u;
+    auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, tile_rows, r, q](uint32_t tile) -> const uint8_t * {
         int64_t offset;
         if (MODE == TILE16_SWIGLU) {
             offset = ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((tile >> 1) * 16u + r) * row_bytes;
         } else {
-            uint32_t n = tile * 16u + r;
+            uint32_t n = tile * tile_rows + min(r, tile_rows - 1u);
             if (MODE == TILE16_ROPE) n = (tile / tiles_per_head) * (2u * half_width) + (tile % tiles_per_head) * 8u + (r & 7u) + (r >> 3) * half_width;
             const bool in0 = n < end0, in1 = n < end1;
             const int64_t matrix = in0 ? (int64_t)0 : (in1 ? to_w1 : to_w2);
@@ -294,8 +297,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
                     const uint32_t next = rope_row(tile + hop, c);
                     rope_held = rope_operands(p, next, c, rope_position);
                 }
-            } else {
-                const uint32_t n = tile * 16u + lane;
+            } else if (lane < tile_rows) {
+                const uint32_t n = tile * tile_rows + lane;
                 // in place (the decoder's residual stream): one add per element, nothing to wait for
                 if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);
                 else p.y[n] = p.residual ? p.residual[n] + total : total;
@@ -396,7 +399,20 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u ? 8u : 16u));
     // units of work: tiles, or with SwiGLU pairs (a gate tile and the up tile behind it); every workgroup takes the same
     // number of them, one workgroup a compute unit when there are that many
-    const uint32_t units = a.swiglu ? a.N / 32u : a.N / 16u;
+    // A plain tile holds the number of rows, 16 down to 12, that leaves the fewest compute units idle in the last round.
+    p.tile_rows = 16;
+    if (!a.swiglu && !a.rope) {
+        auto idle = [&](uint32_t rows) {  // share of the rounds' slots left empty, in 1/65536
+            const uint32_t tiles = a.N / rows, rounds = (tiles + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
+            return 65536u - (uint32_t)((uint64_t)tiles * 65536u / ((uint64_t)rounds * (uint32_t)d->compute_units));
+        };
+        for (uint32_t rows = 15; rows >= 12; rows--) {
+            if (a.N % rows || a.end[0] % rows || a.end[1] % rows) continue;
+            // fewer rows a tile stage the activations more often: taken only where they fill at least a twentieth more of the device
+            if (idle(rows) + 3277u < idle(p.tile_rows)) p.tile_rows = rows;
+        }
+    }
+    const uint32_t units = a.swiglu ? a.N / 32u : a.N / p.tile_rows;
     p.row_groups = units;
     const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
     const uint32_t grid = (units + rounds - 1u) / rounds;
