@@ -26,10 +26,23 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one Q4_K product launch of the 7B-shape decode step moves on average, from the
-# rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in profiles/gemv_q4k_decode_hbm_counters.md
-# (each counter scaled by its reading for a plain 1 GiB copy); not measurable inside this script
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"qwen2.5-7b-q4k": 35.76e6}
+# HBM bytes one Q4_K product launch of the 7B-shape decode step moves on average come from the rocprofv3 FETCH_SIZE /
+# WRITE_SIZE runs summarised in this file (each counter scaled by its reading for a plain 1 GiB copy); they cannot be
+# measured inside this script, so the summary carries one machine-readable line and the commit it was measured at
+TRAFFIC_SUMMARY = os.path.join("profiles", "gemv_q4k_tile16_hbm_counters.md")
+
+
+def measured_traffic(name):
+    """(bytes per launch, "file @ commit") from the line `traffic <workload> <bytes> at <commit>` of the summary, or (None, None)"""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_SUMMARY)) as held:
+            for line in held:
+                words = line.strip().strip("`").split()
+                if len(words) == 5 and words[0] == "traffic" and words[1] == name and words[3] == "at":
+                    return float(words[2]), "%s @ %s" % (TRAFFIC_SUMMARY, words[4])
+    except OSError:
+        pass
+    return None, None
 
 
 def note(text):
@@ -149,29 +162,29 @@ def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=1
 
 def gemm_config3(device, rng, repeats=10):
     """The wide-product configuration of the benchmark: the Q4_K product M=512, K=3584, N=18944 (the 7B-shape FFN up projection), with half
-    activations as the configuration states them and with fp32 activations as the decoder's fill passes them."""
-    import ctypes
-
+    activations as the configuration states them and with fp32 activations as the decoder's fill passes them; and the same shape in
+    Q8_0 blocks (the element of the small decoder's fill), half activations."""
     from neura_amd import synth
 
     M, K, N = 512, 3584, 18944
-    raw = device.upload(synth.q4_k_random(rng, N * K))
     y = device.alloc(M * N * 4)
     out = {"workload": "Q4_K wide product M=%d K=%d N=%d, random blocks, N(0,1) activations" % (M, K, N), "flop": 2.0 * M * N * K,
            "mfma_peak_tflops": 2500.0}
-    for name, dtype, code in (("half_activations", np.float16, 1), ("fp32_activations", np.float32, 0)):
+    for name, element, dtype, code in (("half_activations", 12, np.float16, 1), ("fp32_activations", 12, np.float32, 0),
+                                       ("q8_0_half_activations", 8, np.float16, 1)):
+        raw = device.upload(synth.RANDOM[element](rng, N * K))
         x = device.upload(rng.standard_normal((M, K)).astype(dtype))
         for timed in (False, True):
             if timed:
                 device.sync()
                 device.timer_start()
             for _ in range(repeats if timed else 3):
-                status = device.lib.nh_gemm(device.handle, 12, raw.pointer, N, K, x.pointer, code, M, y.pointer, None)
+                status = device.lib.nh_gemm(device.handle, element, raw.pointer, N, K, x.pointer, code, M, y.pointer, None)
                 assert status == 0, device.lib.nh_last_error()
         seconds = device.timer_stop() / repeats
         out[name] = {"us": seconds * 1e6, "tflops": 2.0 * M * N * K / seconds / 1e12, "frac_of_mfma_peak": 2.0 * M * N * K / seconds / 2.5e15}
         x.release()
-    raw.release()
+        raw.release()
     y.release()
     return out
 
@@ -224,6 +237,8 @@ def extras(device, weights, shape, element, context, layers, rng):
     if element == 12 and not os.environ.get("NEURA_BENCH_SKIP_Q8"):
         note("extras: 0.5B-shape Q8_0 decode")
         out["decode_0_5b_q8_0"] = small_q8_0_decode(device)
+        note("extras: Q4_K products of one 1.5B-shape layer")
+        out["layer_products_1_5b_q4k"] = layer_products_1_5b(device)
     return out
 
 
@@ -252,9 +267,38 @@ def small_q8_0_decode(device):
     elapsed = time.perf_counter() - began
     model.release()
     weights.release()
+    walked = weight_bytes_per_token(shape, element, shape["layers"])
     return {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
-            "weight_bytes_per_token": weight_bytes_per_token(shape, element, shape["layers"]),
-            "note": "qwen2.5-0.5b shape, Q8_0, 24 layers, batch 1, fp16 KV cache at context %d" % context}
+            "weight_bytes_per_token": walked, "hbm_frac_whole_step": walked / (elapsed / steps) / 1e9 / HBM_PEAK_GBS,
+            "note": "qwen2.5-0.5b shape, Q8_0, 24 layers, batch 1, fp16 KV cache at context %d; hbm_frac_whole_step = weight bytes of a "
+                    "step over the whole step's time (every kernel and the read-back), against 8 TB/s" % context}
+
+
+def layer_products_1_5b(device):
+    """The Q4_K narrow products of one Qwen2.5-1.5B-shaped layer at batch 1 (hidden 1536, 12 query and 2 key heads of 128,
+    FFN 8960: q|k|v, attn_output, gate|up, ffn_down), launched back to back between one pair of events.  The timed pass of a
+    decoder also walks its output head: a decoder of two such layers and one of one are timed and their difference is the layer."""
+    from neura_amd import synth
+    from neura_amd.loader import Model, Weights
+
+    rng = np.random.default_rng(2)
+    passes = 64
+    measured = []
+    for layers in (2, 1):
+        shape = dict(synth.SHAPES["qwen2.5-1.5b"], layers=layers)
+        weights = Weights(device, list(synth.model_tensors(shape, 12, rng, mode="blocks", layers=layers)))
+        model = Model(device, weights, shape, 12, batch=1, context=64, layers=layers)
+        model.decode_step([1], [0])
+        measured.append(model.time_products(passes))
+        model.release()
+        weights.release()
+    seconds = measured[0][0] - measured[1][0]
+    launches = (measured[0][1] - measured[1][1]) / passes
+    walked = (measured[0][2] - measured[1][2]) / passes
+    return {"us_per_layer": seconds / passes * 1e6, "launches": launches, "weight_bytes": walked, "hbm_gbs": walked * passes / seconds / 1e9,
+            "hbm_frac": walked * passes / seconds / 1e9 / HBM_PEAK_GBS,
+            "note": "q|k|v, attn_output, gate|up and ffn_down of one layer: a pass over a two-layer decoder's products minus a pass over "
+                    "a one-layer decoder's (the output head, which both walk, drops out)"}
 
 
 def fill_512(device, weights, shape, element, context, layers, rng):
@@ -275,7 +319,9 @@ def fill_512(device, weights, shape, element, context, layers, rng):
     per_layer = sum(2.0 * rows * n * k for _, n, k in __import__("neura_amd").synth.layer_matrices(shape))
     model.release()
     return {"value": rows / elapsed, "unit": "tokens/s", "ms": elapsed * 1e3, "product_tflops": layers * per_layer / elapsed / 1e12,
-            "note": "one 512-row fill at cursor 0, all products on f16 MFMA with fp32 activations as (value, residue) half rows; "
+            "note": "one 512-row fill at cursor 0, all products on f16 MFMA; the decoder's fp32 activations enter as two half rows each "
+                    "(the value rounded to half and its residue), 22 bits of every activation, so the matrix cores do twice the work of "
+                    "a half-activation product; "
                     "product_tflops counts 2*M*N*K of the products over the whole fill time"}
 
 
@@ -366,6 +412,7 @@ def main():
     per_launch_seconds = gemv_seconds / launches
     achieved = per_launch_bytes / per_launch_seconds / 1e9
 
+    traffic, traffic_source = measured_traffic(args.workload)
     result = {
         "metric": "decode tok/s (bs=1) Qwen2.5-7B-shape Q4_K; quant-GEMV HBM GB/s (% peak)",
         "value": args.steps / elapsed,
@@ -387,13 +434,15 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": ("all narrow products: gemv_q4k_decode_kernel, gemv_q4k_mfma_deep_kernel, gemv_staged_kernel<Q6_K>" if mixed else
-                       "gemv_q4k_decode_kernel (q|k|v, o, gate|up, head) + gemv_q4k_mfma_deep_kernel (down)" if element == 12 else "gemv_q8_0_kernel"),
+            "kernel": ("all narrow products: gemv_q4k_tile16_kernel, gemv_staged_kernel<Q6_K>" if mixed else
+                       "gemv_q4k_tile16_kernel (q|k|v with the rotation, attn_output, gate|up with SwiGLU, ffn_down, output head)" if element == 12
+                       else "gemv_q8_0_decode_kernel"),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if args.layers is None else None,
+            "traffic": traffic if args.layers is None else None,
+            "traffic_source": traffic_source if args.layers is None else None,
             "bytes_per_launch": per_launch_bytes,
             "us_per_launch": per_launch_seconds * 1e6,
             "launches_per_step": launches / profiled,
