@@ -37,6 +37,7 @@ typedef struct nh_model nh_model;
 enum {
     NH_F32 = 0,   /* Element::Single   */
     NH_F16 = 1,   /* Element::Half     */
+    NH_BF16 = 30, /* Element::Bfloat16: a key / value cache element only (crates/neura-decoder/src/cache.rs:130-134) */
     NH_Q8_0 = 8,  /* Element::Q8_0: 32 elements / 34 bytes  (crates/neura-abi/src/element.rs:155-158) */
     NH_Q3_K = 11, /* Element::Q3K: 256 elements / 110 bytes (crates/neura-abi/src/element.rs:171-174) */
     NH_Q4_K = 12, /* Element::Q4K: 256 elements / 144 bytes (crates/neura-abi/src/element.rs:159-162) */
@@ -155,6 +156,15 @@ int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v
 int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
                      uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach,
                      const uint32_t *dev_cursor, float scale, float *dev_out);
+/* nh_cache_write and nh_attention over states of another element (Cache::new(.., Element::Single | Half | Bfloat16),
+ * crates/neura-decoder/src/cache.rs:130-134; the reference's cache tests run Single and Half, tests/cache.rs:17): the caches
+ * are arrays of `cache_element` (NH_F16, NH_BF16 or NH_F32), everything else as above.  NH_F16 takes the kernels above. */
+int32_t nh_cache_write_element(nh_device *device, const float *dev_k, const float *dev_v, void *dev_cache_k, void *dev_cache_v,
+                               uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
+                               const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring, int32_t cache_element);
+int32_t nh_attention_element(nh_device *device, const float *dev_q, const void *dev_cache_k, const void *dev_cache_v, uint32_t heads,
+                             uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                             uint32_t reach, const uint32_t *dev_cursor, float scale, float *dev_out, int32_t cache_element);
 /* run_gather (crates/neura-kernel/src/task/select.rs:29-49): out[t][:] = dequant(table[token[t]]),
  * times mask[t % batch] when dev_mask != NULL.  A token id >= vocab is refused. */
 int32_t nh_gather(nh_device *device, int32_t element, const void *dev_table, uint32_t vocab, uint32_t width, const uint32_t *dev_tokens,
@@ -199,6 +209,11 @@ typedef struct nh_model_config {
                             `window` positions (+ max_rows scratch rows) and a sequence attends to its last `window` tokens */
     float rope_base;     /* <arch>.rope.freq_base */
     float eps;           /* <arch>.attention.layer_norm_rms_epsilon */
+    int32_t cache_element; /* what the key and value states hold (Cache::new(.., element), crates/neura-decoder/src/cache.rs:63,
+                              :130-134): NH_F16, NH_BF16 or NH_F32 -- NH_F32 is 0, so a config that never names it keeps single
+                              precision states as the reference's own example does (examples/qwen/main.rs:107); the headline
+                              workload names NH_F16.  Keys and values are cast on their way in (graph.cast, cache.rs:347-348;
+                              bfloat16 rounds to nearest even, crates/neura-kernel/src/task/convert.rs:86-89) */
 } nh_model_config;
 
 /* where each tensor sits in the arena (byte offsets) and its element.  Per layer arrays have
@@ -247,9 +262,10 @@ int32_t nh_model_reset(nh_model *model, const uint8_t *reset, uint32_t batch);
  * the last decode step, [batch][vocab] */
 int32_t nh_model_logits(nh_model *model, float *host_out);
 /* Runtime::restore_state / save_state of "blk.{i}.cache.key|value"
- * (crates/neura-decoder/src/cache.rs:135-137): raw fp16 [kv_heads][batch][capacity][head_dim] */
-int32_t nh_model_cache_write(nh_model *model, uint32_t layer, int32_t value_not_key, const uint16_t *host_src);
-int32_t nh_model_cache_read(nh_model *model, uint32_t layer, int32_t value_not_key, uint16_t *host_dst);
+ * (crates/neura-decoder/src/cache.rs:135-137): [kv_heads][batch][capacity][head_dim] numbers of the config's cache_element,
+ * as they lie (2 bytes each for NH_F16 and NH_BF16, 4 for NH_F32) */
+int32_t nh_model_cache_write(nh_model *model, uint32_t layer, int32_t value_not_key, const void *host_src);
+int32_t nh_model_cache_read(nh_model *model, uint32_t layer, int32_t value_not_key, void *host_dst);
 uint32_t nh_model_capacity(const nh_model *model);
 /* The shared prefix of a batch that declares one (Cache::with_shared / Cache::shared, crates/neura-decoder/src/cache.rs:71-90,
  * :138-161; Batch::prefix, crates/neura-generate/src/batch.rs:885-994): one more plane of keys and values per layer,
@@ -261,8 +277,8 @@ uint32_t nh_model_capacity(const nh_model *model);
  * nh_model_shared_write / _read: Runtime::restore_state / save_state of "blk.{i}.cache.shared.key|value". */
 int32_t nh_model_keep_prefix(nh_model *model, uint32_t plane);
 int32_t nh_model_reset_shared(nh_model *model, const uint8_t *reset, const uint8_t *share, uint32_t batch);
-int32_t nh_model_shared_write(nh_model *model, uint32_t layer, int32_t value_not_key, const uint16_t *host_src);
-int32_t nh_model_shared_read(nh_model *model, uint32_t layer, int32_t value_not_key, uint16_t *host_dst);
+int32_t nh_model_shared_write(nh_model *model, uint32_t layer, int32_t value_not_key, const void *host_src);
+int32_t nh_model_shared_read(nh_model *model, uint32_t layer, int32_t value_not_key, void *host_dst);
 
 #ifdef __cplusplus
 }

@@ -185,25 +185,33 @@ class Device:
         _check(self.lib.nh_rope(self.handle, xd.pointer, planes, batch, rows, width, cd.pointer if cd else None, base, out.pointer))
         return out.numpy(np.float32, x.shape)
 
-    def cache_write(self, k, v, cache_k, cache_v, capacity, window, cursor, mask=None, ring=False):
+    def cache_write(self, k, v, cache_k, cache_v, capacity, window, cursor, mask=None, ring=False, element=NH_F16):
         k = np.ascontiguousarray(k, dtype=np.float32)
         v = np.ascontiguousarray(v, dtype=np.float32)
         kv_heads, batch, rows, width = k.shape
         kd, vd = self.upload(k), self.upload(v)
         cd = self.upload(np.asarray(cursor, dtype=np.uint32))
         md = self.upload(np.asarray(mask, dtype=np.uint8)) if mask is not None else None
-        _check(self.lib.nh_cache_write(self.handle, kd.pointer, vd.pointer, cache_k.pointer, cache_v.pointer, kv_heads, batch, rows, width,
-                                       capacity, window, cd.pointer, md.pointer if md else None, 1 if ring else 0))
+        if element == NH_F16:
+            _check(self.lib.nh_cache_write(self.handle, kd.pointer, vd.pointer, cache_k.pointer, cache_v.pointer, kv_heads, batch, rows, width,
+                                           capacity, window, cd.pointer, md.pointer if md else None, 1 if ring else 0))
+        else:
+            _check(self.lib.nh_cache_write_element(self.handle, kd.pointer, vd.pointer, cache_k.pointer, cache_v.pointer, kv_heads, batch, rows,
+                                                   width, capacity, window, cd.pointer, md.pointer if md else None, 1 if ring else 0, element))
 
-    def attention(self, q, cache_k, cache_v, kv_heads, capacity, keys, cursor, scale, reach=0):
+    def attention(self, q, cache_k, cache_v, kv_heads, capacity, keys, cursor, scale, reach=0, element=NH_F16):
         q = np.ascontiguousarray(q, dtype=np.float32)
         heads, batch, rows, width = q.shape
         qd = self.upload(q)
         kd, vd = self._dev(cache_k), self._dev(cache_v)
         cd = self.upload(np.asarray(cursor, dtype=np.uint32))
         out = self.alloc(q.nbytes)
-        _check(self.lib.nh_attention(self.handle, qd.pointer, kd.pointer, vd.pointer, heads, kv_heads, batch, rows, width, capacity, keys, reach,
-                                     cd.pointer, scale, out.pointer))
+        if element == NH_F16:
+            _check(self.lib.nh_attention(self.handle, qd.pointer, kd.pointer, vd.pointer, heads, kv_heads, batch, rows, width, capacity, keys, reach,
+                                         cd.pointer, scale, out.pointer))
+        else:
+            _check(self.lib.nh_attention_element(self.handle, qd.pointer, kd.pointer, vd.pointer, heads, kv_heads, batch, rows, width, capacity, keys,
+                                                 reach, cd.pointer, scale, out.pointer, element))
         return out.numpy(np.float32, q.shape)
 
     def gather(self, element, table, vocab, width, tokens, batch=1, mask=None):

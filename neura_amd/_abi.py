@@ -23,7 +23,7 @@ class Epilogue(ctypes.Structure):
 class ModelConfig(ctypes.Structure):
     _fields_ = [(name, c_uint32) for name in
                 ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "context", "batch", "max_rows", "window")] + \
-               [("rope_base", c_float), ("eps", c_float)]
+               [("rope_base", c_float), ("eps", c_float), ("cache_element", c_int32)]
 
 
 class TensorTable(ctypes.Structure):
@@ -65,6 +65,10 @@ SIGNATURES = {
                                  c_uint32, c_void_p, c_void_p, c_int32]),
     "nh_attention": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
                                c_uint32, c_uint32, c_void_p, c_float, c_void_p]),
+    "nh_cache_write_element": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
+                                         c_uint32, c_void_p, c_void_p, c_int32, c_int32]),
+    "nh_attention_element": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32,
+                                       c_uint32, c_uint32, c_void_p, c_float, c_void_p, c_int32]),
     "nh_gather": (c_int32, [c_void_p, c_int32, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "nh_argmax": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
     "nh_argmax_static": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),

@@ -26,7 +26,7 @@ struct AttentionParams {
     float *out;
     float *partial;      // [unit][section][group][width + 2] when sections > 1
     uint64_t q_sh, q_sb, q_sr, o_sh, o_sb, o_sr;
-    const uint16_t *cache_k, *cache_v;
+    const uint16_t *cache_k, *cache_v;  // as bytes of another element for attention_any_kernel
     uint32_t heads, kv_heads, groups, batch, rows, capacity, keys, sections;
     const uint32_t *cursor;
     float scale;
@@ -713,6 +713,88 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
     }
 }
 
+// ---------------------------------------------------------------- states of any element ------------------------------
+//
+// Keys and values held as single, bfloat16 (or half) numbers (Cache::new(.., element), crates/neura-decoder/src/cache.rs:130-134).
+// One workgroup per (kv head, plane, row, section of the window), three plain passes over the section's keys: the scores of
+// every (query head of the group, key) pair into LDS (a thread a pair, neighbouring threads the heads of one key, so a key
+// row is fetched once and shared); a wave per query head for the largest score, the weights e^(score - largest) and their
+// mass; a thread per (query head, channel) for the weighed sum of the value rows.  The section's sums leave in the layout
+// attention_fold_kernel merges (or normalised, when one section covers the window).  fp32 throughout, no matrix cores: this
+// is the form for elements the tile kernels do not read, built to be right rather than fast.
+constexpr uint32_t ANY_KEYS = 256;  // keys a section holds at most: 16 query heads x 256 scores of LDS
+
+template <int CE>
+__global__ __launch_bounds__(256) void attention_any_kernel(AttentionParams p, uint32_t width) {
+    __shared__ float scores[16 * ANY_KEYS];
+    __shared__ float tops[16], masses[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t unit = blockIdx.x, section = blockIdx.y;
+    const uint32_t row = unit % p.rows;
+    const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
+    const uint32_t G = p.groups;
+    const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
+    const uint32_t begin = min(p.keys, section * chunk);
+    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
+    uint32_t origin = p.cursor ? p.cursor[b] : 0u;
+    if (!p.reach && origin + p.rows > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+        if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+        origin = p.keys - p.rows;
+    }
+    const uint32_t position = origin + row;
+    const uint32_t visible = min(p.keys, p.reach ? origin + p.rows : position + 1u);
+    const uint32_t last = min(visible, begin + chunk);
+    const uint32_t n = last > begin ? last - begin : 0u;
+    const Ring ring(p.keys, origin + p.rows, p.reach);
+    // ---- scores
+    for (uint32_t pair = tid; pair < n * G; pair += 256) {
+        const uint32_t g = pair % G, key = begin + pair / G;
+        float score = -INFINITY;
+        if (!p.reach || ring.seen(key, position)) {
+            const float *q = p.q + (uint64_t)(kvh * G + g) * p.q_sh + (uint64_t)b * p.q_sb + (uint64_t)row * p.q_sr;
+            float total = 0.0f;
+            for (uint32_t c = 0; c < width; c++) total = fmaf(q[c], cache_load<CE>(p.cache_k, (plane + key) * width + c), total);
+            score = total * p.scale;
+        }
+        scores[g * ANY_KEYS + pair / G] = score;
+    }
+    __syncthreads();
+    // ---- weights: wave w takes query heads w, w + 4, ...
+    for (uint32_t g = wave; g < G; g += 4) {
+        float top = -INFINITY;
+        for (uint32_t k = lane; k < n; k += 64) top = fmaxf(top, scores[g * ANY_KEYS + k]);
+        top = wave_max(top);
+        float mass = 0.0f;
+        for (uint32_t k = lane; k < n; k += 64) {
+            const float score = scores[g * ANY_KEYS + k];
+            const float weight = score == -INFINITY ? 0.0f : softmax_exp(score - top);
+            scores[g * ANY_KEYS + k] = weight;
+            mass += weight;
+        }
+        mass = wave_sum(mass);
+        if (lane == 0) tops[g] = top, masses[g] = mass;
+    }
+    __syncthreads();
+    // ---- values
+    for (uint32_t index = tid; index < G * width; index += 256) {
+        const uint32_t g = index / width, c = index % width;
+        float value = 0.0f;
+        for (uint32_t k = 0; k < n; k++) {
+            const float weight = scores[g * ANY_KEYS + k];
+            // a slot no query weighs may hold anything, and a weight of zero does not silence a NaN
+            if (weight != 0.0f) value = fmaf(weight, cache_load<CE>(p.cache_v, (plane + begin + k) * width + c), value);
+        }
+        if (p.sections > 1) {
+            float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (width + 2);
+            dst[c] = value;
+            if (c == 0) dst[width] = tops[g], dst[width + 1] = masses[g];
+        } else {
+            const float normalized = masses[g] > 0.0f ? 1.0f / masses[g] : 0.0f;
+            p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr + c] = value * normalized;
+        }
+    }
+}
+
 int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     AttentionParams p{};
     p.q = a.q, p.out = a.out;
@@ -724,6 +806,31 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
+    if (a.cache_element != NH_F16) {
+        if (a.cache_element != NH_F32 && a.cache_element != NH_BF16)
+            return fail(NH_E_ARGUMENT, "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid", a.cache_element);
+        if (p.groups > 16u) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides 16", p.groups);
+        // sections of at most ANY_KEYS keys, enough of them to fill the device where the units alone do not
+        uint32_t sections = (a.keys + ANY_KEYS - 1u) / ANY_KEYS;
+        const uint32_t wanted = ((uint32_t)d->compute_units * 2u + units - 1u) / units, most = (a.keys + 31u) / 32u;
+        if (sections < wanted) sections = wanted < most ? wanted : most;
+        if (sections < 1u) sections = 1u;
+        if (sections > 256u) return fail(NH_E_ARGUMENT, "a window of %u keys is more than 256 sections of %u", a.keys, ANY_KEYS);
+        p.sections = sections;
+        if (p.sections > 1) {
+            p.partial = static_cast<float *>(scratch(d, (size_t)p.sections * a.heads * a.batch * a.rows * (a.width + 2) * sizeof(float)));
+            if (!p.partial) return NH_E_MEMORY;
+        }
+        dim3 grid(units, p.sections);
+        if (a.cache_element == NH_F32) hipLaunchKernelGGL(attention_any_kernel<NH_F32>, grid, dim3(256), 0, d->stream, p, a.width);
+        else hipLaunchKernelGGL(attention_any_kernel<NH_BF16>, grid, dim3(256), 0, d->stream, p, a.width);
+        NH_HIP(hipGetLastError());
+        if (p.sections > 1) {
+            hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
+            NH_HIP(hipGetLastError());
+        }
+        return NH_OK;
+    }
     // a chunk of query rows goes to the matrix cores
     {
         const bool aligned = ((uintptr_t)a.out & 15u) == 0 && a.o_sh % 4 == 0 && a.o_sb % 4 == 0 && a.o_sr % 4 == 0 && ((uintptr_t)a.cache_k & 15u) == 0 &&

@@ -19,6 +19,26 @@ __device__ __forceinline__ uint16_t float_to_half(float value) {
     return __builtin_bit_cast(uint16_t, (_Float16)value);
 }
 
+// round to nearest even, as the reference's device casts (crates/neura-kernel/src/task/convert.rs:86-89)
+__device__ __forceinline__ uint16_t float_to_bfloat16(float value) {
+    const uint32_t bits = __builtin_bit_cast(uint32_t, value);
+    return (uint16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+}
+
+// one number of a key / value state held in CE = NH_F16, NH_BF16 or NH_F32 (crates/neura-kernel/src/fetch.rs:95-107)
+template <int CE>
+__device__ __forceinline__ void cache_store(void *base, uint64_t at, float value) {
+    if (CE == NH_F32) static_cast<float *>(base)[at] = value;
+    else if (CE == NH_BF16) static_cast<uint16_t *>(base)[at] = float_to_bfloat16(value);
+    else static_cast<uint16_t *>(base)[at] = float_to_half(value);
+}
+template <int CE>
+__device__ __forceinline__ float cache_load(const void *base, uint64_t at) {
+    if (CE == NH_F32) return static_cast<const float *>(base)[at];
+    if (CE == NH_BF16) return __builtin_bit_cast(float, (uint32_t)static_cast<const uint16_t *>(base)[at] << 16);
+    return half_to_float(static_cast<const uint16_t *>(base)[at]);
+}
+
 __device__ __forceinline__ uint16_t load_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
 
 // 6-bit scale and min `j` (0..7) of a Q4_K super-block from its 12 scale bytes

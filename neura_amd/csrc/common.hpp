@@ -177,9 +177,9 @@ int32_t launch_rmsnorm(nh_device *d, const float *x, const float *residual, cons
                        float *out, float *sum_out);
 int32_t launch_rope(nh_device *d, const float *x, uint32_t planes, uint32_t batch, uint32_t rows, uint32_t width,
                     const uint32_t *cursor, float base, float *out);
-int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
+int32_t launch_cache_write(nh_device *d, const float *k, const float *v, void *cache_k, void *cache_v, uint32_t kv_heads,
                            uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, bool ring);
+                           const uint8_t *mask, bool ring, int32_t cache_element = NH_F16);
 
 // q / out addressing: element (head, plane, row, c) at head*sh + plane*sb + row*sr + c
 struct AttentionArgs {
@@ -191,6 +191,7 @@ struct AttentionArgs {
     const uint32_t *cursor;
     float scale;
     uint32_t reach = 0;  // 0, or the span of a ring cache of `keys` slots (Cache::windowed): the last `reach` positions are weighed
+    int32_t cache_element = NH_F16;  // what the caches hold: NH_F16 (the matrix-core kernels), NH_BF16 or NH_F32 (the kernel for any element)
 };
 int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 
@@ -199,12 +200,12 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 // cos / sin of every (position, channel pair) the rotation can meet, computed as the rotation kernels compute them
 int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t positions, float *cosines, float *sines);
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
-                           uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base, bool ring);
+                           void *cache_k, void *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask, float base, bool ring, int32_t cache_element = NH_F16);
 
 // one token of one plane: v (+ bias) as halves into the value state at cursor[0] (at cursor[0] % ring when the cache is a ring)
-int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
-                            const uint32_t *cursor, uint32_t ring);
+int32_t launch_value_append(nh_device *d, const float *v, const float *bias, void *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
+                            const uint32_t *cursor, uint32_t ring, int32_t cache_element = NH_F16);
 int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float *bias, float *dst, uint32_t ldd, uint32_t rows, uint32_t n);
 
 int32_t launch_pack_q8_0(nh_device *d, const float *src, uint64_t elements, uint8_t *dst);

@@ -71,6 +71,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     // of 16): the columns past them walk the tile's last row again and are never written
     const uint32_t tile_rows = MODE == TILE16_PLAIN ? p.tile_rows : 16u;
     auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, tile_rows, r, q](uint32_t tile) -> const uint8_t * {
+        (void)tile_rows;  // the SwiGLU form's tiles are whole
         int64_t offset;
         if (MODE == TILE16_SWIGLU) {
             offset = ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((tile >> 1) * 16u + r) * row_bytes;

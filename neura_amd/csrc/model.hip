@@ -24,11 +24,12 @@ struct nh_model {
     // the element of every matrix: [token_embd, output, then per layer q, k, v, o, gate, up, down]
     std::vector<int32_t> elements;
     std::vector<const float *> bias_q, bias_k, bias_v;  // per layer, nullptr where a projection has none
-    std::vector<uint16_t *> cache_k, cache_v;
+    std::vector<uint8_t *> cache_k, cache_v;  // numbers of c.cache_element, `eb` bytes each
     size_t cache_elements = 0;  // per layer and per K or V
+    size_t eb = 2;
     // the shared prefix (Cache::with_shared, crates/neura-decoder/src/cache.rs:138-161): one plane per layer,
     // [kv_heads][1][capacity][head_dim], allocated when a prefix is first kept
-    std::vector<uint16_t *> shared_k, shared_v;
+    std::vector<uint8_t *> shared_k, shared_v;
     // activations; T = rows * batch flattened token rows, t = row * batch + plane
     float *h = nullptr, *xn = nullptr, *qkv = nullptr, *att = nullptr, *act = nullptr, *up = nullptr, *logits = nullptr;
     float *rope_cos = nullptr, *rope_sin = nullptr;  // [capacity][head_dim / 2], for the rotation folded into the q|k|v product
@@ -164,9 +165,11 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
             // one token of one active plane: the rotation, the biases and the cache append ride in the product's epilogue
-            RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), m->cache_k[L], m->cache_v[L], hd, QW, QW + KW, m->capacity, m->positions,
-                            m->ring ? m->window : 0u};
-            if (alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
+            // (the folded rotation appends halves: states of another element take the rotation's own kernel)
+            const bool halves = c.cache_element == NH_F16;
+            RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), reinterpret_cast<uint16_t *>(m->cache_k[L]), reinterpret_cast<uint16_t *>(m->cache_v[L]),
+                            hd, QW, QW + KW, m->capacity, m->positions, m->ring ? m->window : 0u};
+            if (halves && alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
                 a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];
                 roped = true;
@@ -178,7 +181,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             qk.end[0] = QW, qk.end[1] = QW + KW, qk.end[2] = QW + KW;
             qk.norm_w = m->attn_norm[L], qk.eps = c.eps;
             RopeFusion rope_qk = rope;
-            const bool split_value = !alike && element_at(m, L, Q) == element_at(m, L, K_) && !products_only && T == 1 && !mask &&
+            const bool split_value = halves && !alike && element_at(m, L, Q) == element_at(m, L, K_) && !products_only && T == 1 && !mask &&
                                      gemv_fuses_rope(qk, rope_qk);
             if (roped || (alike && (!biased || products_only))) {
                 if ((status = launch_gemv(d, a)) != NH_OK) return status;
@@ -189,7 +192,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 GemvArgs value = narrow(m, element_at(m, L, V), m->attn_v[L], KW, H, m->h, T, m->xn);
                 value.norm_w = m->attn_norm[L], value.eps = c.eps;
                 if ((status = launch_gemv(d, value)) != NH_OK) return status;
-                if ((status = launch_value_append(d, m->xn, m->bias_v[L], m->cache_v[L], c.kv_heads, hd, m->capacity, dev_cursor(m), m->ring ? m->window : 0u)) != NH_OK)
+                if ((status = launch_value_append(d, m->xn, m->bias_v[L], m->cache_v[L], c.kv_heads, hd, m->capacity, dev_cursor(m), m->ring ? m->window : 0u,
+                                                  c.cache_element)) != NH_OK)
                     return status;
                 roped = true;
             } else {
@@ -208,13 +212,14 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             }
         }
         if (!products_only && !roped && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
-                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base, m->ring)) != NH_OK)
+                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base, m->ring, c.cache_element)) != NH_OK)
             return status;
         AttentionArgs at{};
         at.q = m->qkv, at.out = m->att;
         at.q_sh = hd, at.q_sb = QKV, at.q_sr = (uint64_t)B * QKV;
         at.o_sh = hd, at.o_sb = QW, at.o_sr = (uint64_t)B * QW;
-        at.cache_k = m->cache_k[L], at.cache_v = m->cache_v[L];
+        at.cache_k = reinterpret_cast<const uint16_t *>(m->cache_k[L]), at.cache_v = reinterpret_cast<const uint16_t *>(m->cache_v[L]);
+        at.cache_element = c.cache_element;
         at.heads = c.heads, at.kv_heads = c.kv_heads, at.batch = B, at.rows = rows, at.width = hd;
         at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
         at.reach = m->ring ? m->window : 0u;
@@ -288,6 +293,10 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         return nullptr;
     }
     const nh_model_config &c = *config;
+    if (c.cache_element != NH_F16 && c.cache_element != NH_BF16 && c.cache_element != NH_F32) {  // crates/neura-decoder/src/cache.rs:130-134
+        fail(NH_E_ARGUMENT, "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid", c.cache_element);
+        return nullptr;
+    }
     if (!c.layers || !c.hidden || !c.heads || !c.kv_heads || !c.head_dim || !c.ffn || !c.vocab || !c.context || !c.batch ||
         c.heads % c.kv_heads || c.head_dim % 8) {
         fail(NH_E_ARGUMENT, "a decoder of %u layers, %u hidden, %u/%u heads of %u, %u ffn, %u vocab, %u context, %u planes holds no model",
@@ -389,19 +398,20 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     }
     const size_t T = m->max_tokens;
     m->cache_elements = (size_t)c.kv_heads * c.batch * m->capacity * c.head_dim;
+    m->eb = c.cache_element == NH_F32 ? 4 : 2;
     ok = device_array(m->h, T * H) && device_array(m->xn, T * (H > QW ? H : QW)) && device_array(m->qkv, T * (QW + 2 * KW)) &&
          device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T * F) &&
          device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 6 * c.batch + 4) &&
          device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->positions * (c.head_dim / 2)) &&
          device_array(m->rope_sin, (size_t)m->positions * (c.head_dim / 2));
     for (uint32_t L = 0; ok && L < c.layers; L++) {
-        uint16_t *k = nullptr, *v = nullptr;
-        ok = device_array(k, m->cache_elements);
+        uint8_t *k = nullptr, *v = nullptr;
+        ok = device_array(k, m->cache_elements * m->eb);
         if (ok) m->cache_k.push_back(k);
-        ok = ok && device_array(v, m->cache_elements);
+        ok = ok && device_array(v, m->cache_elements * m->eb);
         if (ok && v) m->cache_v.push_back(v);
-        if (ok) ok = hipMemsetAsync(k, 0, m->cache_elements * 2, device->stream) == hipSuccess &&
-                     hipMemsetAsync(v, 0, m->cache_elements * 2, device->stream) == hipSuccess;
+        if (ok) ok = hipMemsetAsync(k, 0, m->cache_elements * m->eb, device->stream) == hipSuccess &&
+                     hipMemsetAsync(v, 0, m->cache_elements * m->eb, device->stream) == hipSuccess;
     }
     ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 6 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
          hipHostMalloc((void **)&m->chosen_host, ((size_t)c.batch + 1) * 4, hipHostMallocDefault) == hipSuccess;
@@ -571,8 +581,8 @@ int32_t nh_model_reset(nh_model *m, const uint8_t *reset, uint32_t batch) {
             for (uint32_t b = 0; b < batch; b++) {
                 if (!reset[b]) continue;
                 size_t at = ((size_t)head * batch + b) * plane;
-                NH_HIP(hipMemsetAsync(m->cache_k[L] + at, 0, plane * 2, m->d->stream));
-                NH_HIP(hipMemsetAsync(m->cache_v[L] + at, 0, plane * 2, m->d->stream));
+                NH_HIP(hipMemsetAsync(m->cache_k[L] + at * m->eb, 0, plane * m->eb, m->d->stream));
+                NH_HIP(hipMemsetAsync(m->cache_v[L] + at * m->eb, 0, plane * m->eb, m->d->stream));
             }
     return NH_OK;
 }
@@ -580,9 +590,9 @@ int32_t nh_model_reset(nh_model *m, const uint8_t *reset, uint32_t batch) {
 // the shared planes, zeroed, on first use
 static int32_t shared_planes(nh_model *m) {
     if (!m->shared_k.empty()) return NH_OK;
-    const size_t bytes = (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2;
+    const size_t bytes = (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * m->eb;
     for (uint32_t L = 0; L < m->c.layers; L++) {
-        uint16_t *k = nullptr, *v = nullptr;
+        uint8_t *k = nullptr, *v = nullptr;
         if (hipMalloc((void **)&k, bytes) != hipSuccess || hipMalloc((void **)&v, bytes) != hipSuccess) {
             if (k) (void)hipFree(k);
             return fail(NH_E_MEMORY, "no room for the %zu bytes a shared prefix of layer %u holds", 2 * bytes, L);
@@ -602,8 +612,8 @@ int32_t nh_model_keep_prefix(nh_model *m, uint32_t plane_index) {
     for (uint32_t L = 0; L < m->c.layers; L++)
         for (uint32_t head = 0; head < m->c.kv_heads; head++) {
             const size_t from = ((size_t)head * m->c.batch + plane_index) * plane, to = (size_t)head * plane;
-            NH_HIP(hipMemcpyAsync(m->shared_k[L] + to, m->cache_k[L] + from, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
-            NH_HIP(hipMemcpyAsync(m->shared_v[L] + to, m->cache_v[L] + from, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+            NH_HIP(hipMemcpyAsync(m->shared_k[L] + to * m->eb, m->cache_k[L] + from * m->eb, plane * m->eb, hipMemcpyDeviceToDevice, m->d->stream));
+            NH_HIP(hipMemcpyAsync(m->shared_v[L] + to * m->eb, m->cache_v[L] + from * m->eb, plane * m->eb, hipMemcpyDeviceToDevice, m->d->stream));
         }
     return NH_OK;
 }
@@ -620,28 +630,28 @@ int32_t nh_model_reset_shared(nh_model *m, const uint8_t *reset, const uint8_t *
             for (uint32_t b = 0; b < batch; b++) {
                 const size_t at = ((size_t)head * batch + b) * plane;
                 if (share[b]) {  // select(share, prefix, blank): the prefix wins over the reset (cache.rs:231-238)
-                    NH_HIP(hipMemcpyAsync(m->cache_k[L] + at, m->shared_k[L] + (size_t)head * plane, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
-                    NH_HIP(hipMemcpyAsync(m->cache_v[L] + at, m->shared_v[L] + (size_t)head * plane, plane * 2, hipMemcpyDeviceToDevice, m->d->stream));
+                    NH_HIP(hipMemcpyAsync(m->cache_k[L] + at * m->eb, m->shared_k[L] + (size_t)head * plane * m->eb, plane * m->eb, hipMemcpyDeviceToDevice, m->d->stream));
+                    NH_HIP(hipMemcpyAsync(m->cache_v[L] + at * m->eb, m->shared_v[L] + (size_t)head * plane * m->eb, plane * m->eb, hipMemcpyDeviceToDevice, m->d->stream));
                 } else if (reset[b]) {
-                    NH_HIP(hipMemsetAsync(m->cache_k[L] + at, 0, plane * 2, m->d->stream));
-                    NH_HIP(hipMemsetAsync(m->cache_v[L] + at, 0, plane * 2, m->d->stream));
+                    NH_HIP(hipMemsetAsync(m->cache_k[L] + at * m->eb, 0, plane * m->eb, m->d->stream));
+                    NH_HIP(hipMemsetAsync(m->cache_v[L] + at * m->eb, 0, plane * m->eb, m->d->stream));
                 }
             }
     return NH_OK;
 }
 
-int32_t nh_model_shared_write(nh_model *m, uint32_t layer, int32_t value_not_key, const uint16_t *host_src) {
+int32_t nh_model_shared_write(nh_model *m, uint32_t layer, int32_t value_not_key, const void *host_src) {
     NH_REQUIRE(m && host_src && layer < m->c.layers, "a shared prefix write names no model, no bytes or no layer %u", layer);
     int32_t status = shared_planes(m);
     if (status != NH_OK) return status;
-    return nh_upload(m->d, value_not_key ? m->shared_v[layer] : m->shared_k[layer], host_src, (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2);
+    return nh_upload(m->d, value_not_key ? m->shared_v[layer] : m->shared_k[layer], host_src, (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * m->eb);
 }
 
-int32_t nh_model_shared_read(nh_model *m, uint32_t layer, int32_t value_not_key, uint16_t *host_dst) {
+int32_t nh_model_shared_read(nh_model *m, uint32_t layer, int32_t value_not_key, void *host_dst) {
     NH_REQUIRE(m && host_dst && layer < m->c.layers, "a shared prefix read names no model, no bytes or no layer %u", layer);
     int32_t status = shared_planes(m);
     if (status != NH_OK) return status;
-    return nh_download(m->d, host_dst, value_not_key ? m->shared_v[layer] : m->shared_k[layer], (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * 2);
+    return nh_download(m->d, host_dst, value_not_key ? m->shared_v[layer] : m->shared_k[layer], (size_t)m->c.kv_heads * m->capacity * m->c.head_dim * m->eb);
 }
 
 int32_t nh_model_logits(nh_model *m, float *host_out) {
@@ -649,14 +659,14 @@ int32_t nh_model_logits(nh_model *m, float *host_out) {
     return nh_download(m->d, host_out, m->logits, (size_t)m->c.batch * m->c.vocab * 4);
 }
 
-int32_t nh_model_cache_write(nh_model *m, uint32_t layer, int32_t value_not_key, const uint16_t *host_src) {
+int32_t nh_model_cache_write(nh_model *m, uint32_t layer, int32_t value_not_key, const void *host_src) {
     NH_REQUIRE(m && host_src && layer < m->c.layers, "a cache write names no model, no bytes or no layer %u", layer);
-    return nh_upload(m->d, value_not_key ? m->cache_v[layer] : m->cache_k[layer], host_src, m->cache_elements * 2);
+    return nh_upload(m->d, value_not_key ? m->cache_v[layer] : m->cache_k[layer], host_src, m->cache_elements * m->eb);
 }
 
-int32_t nh_model_cache_read(nh_model *m, uint32_t layer, int32_t value_not_key, uint16_t *host_dst) {
+int32_t nh_model_cache_read(nh_model *m, uint32_t layer, int32_t value_not_key, void *host_dst) {
     NH_REQUIRE(m && host_dst && layer < m->c.layers, "a cache read names no model, no bytes or no layer %u", layer);
-    return nh_download(m->d, host_dst, value_not_key ? m->cache_v[layer] : m->cache_k[layer], m->cache_elements * 2);
+    return nh_download(m->d, host_dst, value_not_key ? m->cache_v[layer] : m->cache_k[layer], m->cache_elements * m->eb);
 }
 
 // ---- operator entry points ---------------------------------------------------------------
@@ -738,24 +748,45 @@ int32_t nh_rope(nh_device *device, const float *dev_x, uint32_t planes, uint32_t
     return launch_rope(device, dev_x, planes, batch, rows, width, dev_cursor, base, dev_out);
 }
 
+static bool cache_holds(int32_t element) { return element == NH_F16 || element == NH_BF16 || element == NH_F32; }
+
 int32_t nh_cache_write(nh_device *device, const float *dev_k, const float *dev_v, uint16_t *dev_cache_k, uint16_t *dev_cache_v,
                        uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
                        const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring) {
+    return nh_cache_write_element(device, dev_k, dev_v, dev_cache_k, dev_cache_v, kv_heads, batch, rows, width, capacity, window, dev_cursor, dev_mask,
+                                  ring, NH_F16);
+}
+
+int32_t nh_cache_write_element(nh_device *device, const float *dev_k, const float *dev_v, void *dev_cache_k, void *dev_cache_v,
+                               uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
+                               const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring, int32_t cache_element) {
     NH_REQUIRE(device && dev_k && dev_v && dev_cache_k && dev_cache_v && dev_cursor, "a cache write names no device or no buffer");
+    // crates/neura-decoder/src/cache.rs:130-134
+    NH_REQUIRE(cache_holds(cache_element), "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid",
+               cache_element);
     // crates/neura-decoder/src/cache.rs:113-125, :328-335
     NH_REQUIRE(kv_heads > 0 && width > 0 && batch > 0, "a cache of %u planes of %u heads of %u numbers holds no key", batch, kv_heads, width);
     NH_REQUIRE(window > 0 && window <= capacity, "a cache of %u positions keeps a window of %u positions", capacity, window);
     NH_REQUIRE(rows > 0 && rows <= window, "a cache of a %u position window takes %u rows at a time", window, rows);
     NH_REQUIRE(!dev_mask || rows <= capacity - window, "a masked chunk of %u rows holds only %u scratch rows", rows, capacity - window);
     int32_t status = launch_cache_write(device, dev_k, dev_v, dev_cache_k, dev_cache_v, kv_heads, batch, rows, width, capacity, window,
-                                        dev_cursor, dev_mask, ring != 0);
+                                        dev_cursor, dev_mask, ring != 0, cache_element);
     return status != NH_OK ? status : check_refusal(device, "a cache write");
 }
 
 int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_cache_k, const uint16_t *dev_cache_v, uint32_t heads,
                      uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach,
                      const uint32_t *dev_cursor, float scale, float *dev_out) {
+    return nh_attention_element(device, dev_q, dev_cache_k, dev_cache_v, heads, kv_heads, batch, rows, width, capacity, keys, reach, dev_cursor, scale,
+                                dev_out, NH_F16);
+}
+
+int32_t nh_attention_element(nh_device *device, const float *dev_q, const void *dev_cache_k, const void *dev_cache_v, uint32_t heads,
+                             uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys,
+                             uint32_t reach, const uint32_t *dev_cursor, float scale, float *dev_out, int32_t cache_element) {
     NH_REQUIRE(device && dev_q && dev_cache_k && dev_cache_v && dev_out, "an attention names no device or no buffer");
+    NH_REQUIRE(cache_holds(cache_element), "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid",
+               cache_element);
     // crates/neura-decoder/src/cache.rs:383-388
     NH_REQUIRE(kv_heads > 0 && heads % kv_heads == 0, "a query of %u heads reads a cache of %u key heads", heads, kv_heads);
     NH_REQUIRE(keys > 0 && keys <= capacity && rows > 0 && rows <= keys, "%u rows weigh %u keys of a cache of %u positions", rows, keys, capacity);
@@ -766,9 +797,9 @@ int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_
     a.q_sh = a.o_sh = (uint64_t)batch * rows * width;
     a.q_sb = a.o_sb = (uint64_t)rows * width;
     a.q_sr = a.o_sr = width;
-    a.cache_k = dev_cache_k, a.cache_v = dev_cache_v;
+    a.cache_k = static_cast<const uint16_t *>(dev_cache_k), a.cache_v = static_cast<const uint16_t *>(dev_cache_v);
     a.heads = heads, a.kv_heads = kv_heads, a.batch = batch, a.rows = rows, a.width = width, a.capacity = capacity, a.keys = keys;
-    a.cursor = dev_cursor, a.scale = scale, a.reach = reach;
+    a.cursor = dev_cursor, a.scale = scale, a.reach = reach, a.cache_element = cache_element;
     int32_t status = launch_attention(device, a);
     return status != NH_OK ? status : check_refusal(device, "an attention");
 }

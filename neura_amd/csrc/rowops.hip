@@ -83,10 +83,11 @@ int32_t launch_rope(nh_device *d, const float *x, uint32_t planes, uint32_t batc
     return NH_OK;
 }
 
-// cast to fp16 and scatter whole rows (crates/neura-decoder/src/cache.rs:311-351,
+// cast to the states' element and scatter whole rows (crates/neura-decoder/src/cache.rs:311-351,
 // crates/neura-kernel/src/task/scatter.rs:149-171); an inactive plane writes the scratch rows
+template <int CE>
 __global__ __launch_bounds__(256) void cache_write_kernel(const float *__restrict__ k, const float *__restrict__ v,
-                                                          uint16_t *__restrict__ cache_k, uint16_t *__restrict__ cache_v,
+                                                          void *__restrict__ cache_k, void *__restrict__ cache_v,
                                                           uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width,
                                                           uint32_t capacity, uint32_t window, const uint32_t *__restrict__ cursor,
                                                           const uint8_t *__restrict__ mask, uint32_t *refusal, bool ring) {
@@ -106,26 +107,31 @@ __global__ __launch_bounds__(256) void cache_write_kernel(const float *__restric
             continue;
         }
         uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width + c;
-        cache_k[at] = float_to_half(k[index]);
-        cache_v[at] = float_to_half(v[index]);
+        cache_store<CE>(cache_k, at, k[index]);
+        cache_store<CE>(cache_v, at, v[index]);
     }
 }
 
-int32_t launch_cache_write(nh_device *d, const float *k, const float *v, uint16_t *cache_k, uint16_t *cache_v, uint32_t kv_heads,
+int32_t launch_cache_write(nh_device *d, const float *k, const float *v, void *cache_k, void *cache_v, uint32_t kv_heads,
                            uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, bool ring) {
+                           const uint8_t *mask, bool ring, int32_t cache_element) {
     uint64_t total = (uint64_t)kv_heads * batch * rows * width;
     if (!total) return NH_OK;
     uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
-    hipLaunchKernelGGL(cache_write_kernel, dim3(grid), dim3(256), 0, d->stream, k, v, cache_k, cache_v, kv_heads, batch, rows, width,
-                       capacity, window, cursor, mask, d->refusal, ring);
+#define NH_WRITE(CE) hipLaunchKernelGGL(cache_write_kernel<CE>, dim3(grid), dim3(256), 0, d->stream, k, v, cache_k, cache_v, kv_heads, batch, rows, width, \
+                                        capacity, window, cursor, mask, d->refusal, ring)
+    if (cache_element == NH_F32) NH_WRITE(NH_F32);
+    else if (cache_element == NH_BF16) NH_WRITE(NH_BF16);
+    else NH_WRITE(NH_F16);
+#undef NH_WRITE
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
 
-// one token of one plane: value + bias cast to fp16 into the value state at the cursor (what cache_write_kernel does for
+// one token of one plane: value + bias cast into the value state at the cursor (what cache_write_kernel does for
 // a value row whose key went out with the product that rotated it)
-__global__ __launch_bounds__(256) void value_append_kernel(const float *__restrict__ v, const float *__restrict__ bias, uint16_t *__restrict__ cache_v,
+template <int CE>
+__global__ __launch_bounds__(256) void value_append_kernel(const float *__restrict__ v, const float *__restrict__ bias, void *__restrict__ cache_v,
                                                            uint32_t kv_heads, uint32_t width, uint32_t capacity, const uint32_t *__restrict__ cursor,
                                                            uint32_t *refusal, uint32_t ring) {
     const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
@@ -137,15 +143,19 @@ __global__ __launch_bounds__(256) void value_append_kernel(const float *__restri
     }
     const uint32_t head = index / width, c = index % width;
     const float value = bias ? v[index] + bias[index] : v[index];
-    cache_v[((uint64_t)head * capacity + slot) * width + c] = float_to_half(value);
+    cache_store<CE>(cache_v, ((uint64_t)head * capacity + slot) * width + c, value);
 }
 
-int32_t launch_value_append(nh_device *d, const float *v, const float *bias, uint16_t *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
-                            const uint32_t *cursor, uint32_t ring) {
+int32_t launch_value_append(nh_device *d, const float *v, const float *bias, void *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,
+                            const uint32_t *cursor, uint32_t ring, int32_t cache_element) {
     const uint32_t total = kv_heads * width;
     if (!total) return NH_OK;
-    hipLaunchKernelGGL(value_append_kernel, dim3((total + 255) / 256), dim3(256), 0, d->stream, v, bias, cache_v, kv_heads, width, capacity, cursor,
-                       d->refusal, ring);
+#define NH_APPEND(CE) hipLaunchKernelGGL(value_append_kernel<CE>, dim3((total + 255) / 256), dim3(256), 0, d->stream, v, bias, cache_v, kv_heads, width, capacity, \
+                                         cursor, d->refusal, ring)
+    if (cache_element == NH_F32) NH_APPEND(NH_F32);
+    else if (cache_element == NH_BF16) NH_APPEND(NH_BF16);
+    else NH_APPEND(NH_F16);
+#undef NH_APPEND
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -173,10 +183,11 @@ int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t po
 
 // The decoder's fused form of the two kernels above on a token-major buffer
 // qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane: q is roped in place, k is
-// roped, k and v are cast to fp16 and appended to the caches.
+// roped, k and v are cast to the states' element and appended to the caches.
+template <int CE>
 __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qkv, uint32_t heads, uint32_t kv_heads, uint32_t width,
-                                                          uint32_t batch, uint32_t rows, uint16_t *__restrict__ cache_k,
-                                                          uint16_t *__restrict__ cache_v, uint32_t capacity, uint32_t window,
+                                                          uint32_t batch, uint32_t rows, void *__restrict__ cache_k,
+                                                          void *__restrict__ cache_v, uint32_t capacity, uint32_t window,
                                                           const uint32_t *__restrict__ cursor, const uint8_t *__restrict__ mask,
                                                           const float *__restrict__ table, uint32_t *refusal, bool ring) {
     const uint32_t half = width / 2;
@@ -208,27 +219,31 @@ __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qk
             float low, high;
             rotate(src[c], src[c + half], position, table[c], low, high);
             uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
-            cache_k[at + c] = float_to_half(low);
-            cache_k[at + c + half] = float_to_half(high);
+            cache_store<CE>(cache_k, at + c, low);
+            cache_store<CE>(cache_k, at + c + half, high);
         } else {
             uint32_t head = vector - heads - kv_heads;
             uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
-            cache_v[at + c] = float_to_half(src[c]);
-            cache_v[at + c + half] = float_to_half(src[c + half]);
+            cache_store<CE>(cache_v, at + c, src[c]);
+            cache_store<CE>(cache_v, at + c + half, src[c + half]);
         }
     }
 }
 
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
-                           uint16_t *cache_k, uint16_t *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base, bool ring) {
+                           void *cache_k, void *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
+                           const uint8_t *mask, float base, bool ring, int32_t cache_element) {
     const float *table = rope_frequencies(d, base, width);
     if (!table) return NH_E_DEVICE;
     uint64_t total = (uint64_t)batch * rows * (heads + 2 * kv_heads) * (width / 2);
     if (!total) return NH_OK;
     uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
-    hipLaunchKernelGGL(rope_append_kernel, dim3(grid), dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k,
-                       cache_v, capacity, window, cursor, mask, table, d->refusal, ring);
+#define NH_ROPE(CE) hipLaunchKernelGGL(rope_append_kernel<CE>, dim3(grid), dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k, \
+                                       cache_v, capacity, window, cursor, mask, table, d->refusal, ring)
+    if (cache_element == NH_F32) NH_ROPE(NH_F32);
+    else if (cache_element == NH_BF16) NH_ROPE(NH_BF16);
+    else NH_ROPE(NH_F16);
+#undef NH_ROPE
     NH_HIP(hipGetLastError());
     return NH_OK;
 }

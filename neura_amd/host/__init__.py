@@ -59,6 +59,7 @@ SIGNATURES = {
     "nhost_runtime_open": (c_void_p, [c_int32]),
     "nhost_runtime_close": (None, [c_void_p]),
     "nhost_batch_open": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32, c_int32]),
+    "nhost_batch_open_element": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_uint32, c_int32, c_int32]),
     "nhost_batch_open_sampled": (c_void_p, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, POINTER(c_uint32), c_uint32, c_float, c_uint32, c_float,
                                             c_uint32, c_int32]),
     "nhost_batch_prefix": (c_int32, [c_void_p, POINTER(c_uint32), c_uint32]),
@@ -449,15 +450,19 @@ class Batch:
     """A Qwen2 GGUF loaded onto a runtime with a generation batch above it: greedy, or drawing with
     `sampling` = (temperature, keep, cumulative) as BatchSpec::sampled(Sampling::sampled(..)) does."""
 
-    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None, window=None, shared=False):
+    def __init__(self, runtime, archive, vocabulary, context, batch, chunks=(), sampling=None, window=None, shared=False, cache=None):
         """`window`: BatchSpec::window -- the caches are rings of that many tokens and a sequence attends to its last `window`;
-        `shared`: BatchSpec::shared -- the batch can keep one prefix (`prefix`) every prompt then starts from"""
+        `shared`: BatchSpec::shared -- the batch can keep one prefix (`prefix`) every prompt then starts from;
+        `cache`: the element of the key and value states (0 single, 1 half -- the default --, 30 bfloat16), greedy batches"""
         held, count = _words(chunks)
         self.planes = batch
         self.vocabulary = vocabulary
         if window is not None and library().nhost_batch_window_check(window) != 0:
             raise _refused()
-        if sampling is None:
+        if sampling is None and cache is not None:
+            self.handle = library().nhost_batch_open_element(runtime.handle, archive.handle, vocabulary, context, batch, held, count, window or 0,
+                                                             1 if shared else 0, cache)
+        elif sampling is None:
             self.handle = library().nhost_batch_open(runtime.handle, archive.handle, vocabulary, context, batch, held, count, window or 0,
                                                      1 if shared else 0)
         else:

@@ -230,6 +230,20 @@ void *nhost_batch_open(void *runtime, void *held, uint32_t vocabulary, uint32_t 
         return out.release();
     }, nullptr);
 }
+// the same with the key and value states in `cache_element` (Element::Single, Half or Bfloat16)
+void *nhost_batch_open_element(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks,
+                               uint32_t count, uint32_t window, int32_t shared, int32_t cache_element) {
+    return guarded([&]() -> void * {
+        auto *opened = static_cast<Opened *>(held);
+        generate::BatchSpec spec = spec_of(context, batch, chunks, count, window, shared);
+        auto config = generate::Config::read(opened->archive().metadata(), vocabulary);
+        auto out = std::make_unique<Loaded>();
+        out->model = std::make_unique<generate::Model>(*static_cast<runtime::Runtime *>(runtime), opened->archive(), opened->source(), config, spec,
+                                                       (Element)cache_element);
+        out->batch = std::make_unique<generate::Batch>(*out->model, spec);
+        return out.release();
+    }, nullptr);
+}
 // the same with a sampled answer (BatchSpec::sampled(Sampling::sampled(temperature, keep, cumulative)))
 void *nhost_batch_open_sampled(void *runtime, void *held, uint32_t vocabulary, uint32_t context, uint32_t batch, const uint32_t *chunks, uint32_t count,
                                float temperature, uint32_t keep, float cumulative, uint32_t window, int32_t shared) {

@@ -1054,14 +1054,16 @@ class Cache {
                      shape.window, shape.rows);
         NEURA_ASSERT(element == Element::Single || element == Element::Half || element == Element::Bfloat16,
                      "a cache holds keys and values in single, half or bfloat16 storage, and %s storage carries another grid", neura::name(element));
-        NEURA_ASSERT(element == Element::Half, "this build keeps caches in half storage, and %s storage is not built", neura::name(element));
     }
+    // bytes of one key or value number, and the element as the C ABI names it
+    static size_t width_of(Element element) { return element == Element::Single ? 4 : 2; }
+    static int32_t abi(Element element) { return element == Element::Single ? NH_F32 : element == Element::Bfloat16 ? NH_BF16 : NH_F16; }
     Cache(const runtime::Runtime &runtime, const std::string &name, CacheShape shape, Element element = Element::Half, bool ring = false)
-        : device_(runtime.device()), name_(name), shape_(shape), ring_(ring) {
+        : device_(runtime.device()), name_(name), shape_(shape), ring_(ring), element_(element) {
         validate(name, shape, element);
-        size_t bytes = (size_t)shape.heads * shape.batch * shape.capacity * shape.width * 2;
-        keys_ = static_cast<uint16_t *>(nh_alloc(device_, bytes));
-        values_ = static_cast<uint16_t *>(nh_alloc(device_, bytes));
+        size_t bytes = (size_t)shape.heads * shape.batch * shape.capacity * shape.width * width_of(element);
+        keys_ = static_cast<uint8_t *>(nh_alloc(device_, bytes));
+        values_ = static_cast<uint8_t *>(nh_alloc(device_, bytes));
         if (!keys_ || !values_) panic("%s", nh_last_error());
     }
     ~Cache() {
@@ -1080,7 +1082,8 @@ class Cache {
     uint32_t batch() const { return shape_.batch; }
     uint32_t window() const { return shape_.window; }
     bool ring() const { return ring_; }
-    std::pair<uint16_t *, uint16_t *> states() const { return {keys_, values_}; }  // "{name}.key", "{name}.value"
+    Element element() const { return element_; }  // cache.rs:219-221
+    std::pair<void *, void *> states() const { return {keys_, values_}; }  // "{name}.key", "{name}.value", numbers of element()
     std::string key_name() const { return name_ + ".key"; }
     std::string value_name() const { return name_ + ".value"; }
 
@@ -1096,8 +1099,8 @@ class Cache {
     void attend(const float *query, uint32_t query_heads, const uint32_t *cursor, float scale, float *out) {
         NEURA_ASSERT(query_heads % shape_.heads == 0,
                      "a query of %u heads reads a cache of %u key heads, and every key head serves a whole group of queries", query_heads, shape_.heads);
-        runtime::check(nh_attention(device_, query, keys_, values_, query_heads, shape_.heads, shape_.batch, shape_.rows, shape_.width,
-                                    shape_.capacity, shape_.window, ring_ ? shape_.window : 0u, cursor, scale, out));
+        runtime::check(nh_attention_element(device_, query, keys_, values_, query_heads, shape_.heads, shape_.batch, shape_.rows, shape_.width,
+                                            shape_.capacity, shape_.window, ring_ ? shape_.window : 0u, cursor, scale, out, abi(element_)));
     }
     // reset: host flags, one per plane; a set flag zeroes the plane's keys and values
     void reset(const std::vector<uint8_t> &reset) {
@@ -1106,22 +1109,23 @@ class Cache {
         for (uint32_t head = 0; head < shape_.heads; head++)
             for (uint32_t b = 0; b < shape_.batch; b++)
                 if (reset[b]) {
-                    size_t at = ((size_t)head * shape_.batch + b) * plane;
-                    runtime::check(nh_clear(device_, keys_ + at, plane * 2));
-                    runtime::check(nh_clear(device_, values_ + at, plane * 2));
+                    size_t at = ((size_t)head * shape_.batch + b) * plane * width_of(element_);
+                    runtime::check(nh_clear(device_, keys_ + at, plane * width_of(element_)));
+                    runtime::check(nh_clear(device_, values_ + at, plane * width_of(element_)));
                 }
     }
 
   private:
     void store(const uint32_t *cursor, const float *keys, const float *values, const uint8_t *active) {
-        runtime::check(nh_cache_write(device_, keys, values, keys_, values_, shape_.heads, shape_.batch, shape_.rows, shape_.width, shape_.capacity,
-                                      shape_.window, cursor, active, ring_ ? 1 : 0));
+        runtime::check(nh_cache_write_element(device_, keys, values, keys_, values_, shape_.heads, shape_.batch, shape_.rows, shape_.width,
+                                              shape_.capacity, shape_.window, cursor, active, ring_ ? 1 : 0, abi(element_)));
     }
     nh_device *device_;
     std::string name_;
     CacheShape shape_;
     bool ring_ = false;
-    uint16_t *keys_ = nullptr, *values_ = nullptr;
+    Element element_ = Element::Half;
+    uint8_t *keys_ = nullptr, *values_ = nullptr;
 };
 
 }  // namespace decoder
@@ -1212,8 +1216,13 @@ struct Emitted {  // crates/neura-generate/src/batch.rs:155-159
 // The decoder of one GGUF on one device: weights poured into an arena, nh_model above them.
 class Model {
   public:
-    Model(const runtime::Runtime &runtime, const gguf::Archive &archive, const gguf::Source &source, const Config &config, const BatchSpec &spec)
-        : config_(config) {
+    // `cache`: what the key and value states hold (the element the model function hands Cache::new, examples/qwen/main.rs:107,
+    // attention.rs:77-83): Half unless the caller names Single or Bfloat16
+    Model(const runtime::Runtime &runtime, const gguf::Archive &archive, const gguf::Source &source, const Config &config, const BatchSpec &spec,
+          Element cache = Element::Half)
+        : config_(config), cache_(cache) {
+        NEURA_ASSERT(cache == Element::Single || cache == Element::Half || cache == Element::Bfloat16,
+                     "a cache holds keys and values in single, half or bfloat16 storage, and %s storage carries another grid", neura::name(cache));
         const uint32_t H = config.hidden, QW = config.heads * config.head_width, KW = config.key_heads * config.head_width, F = config.feed_forward;
         std::vector<std::string> names;
         // tensor names of a Qwen2 GGUF (the reference's qwen35 example names them alike, examples/qwen/attention.rs:40-78, mlp.rs:22-25)
@@ -1287,6 +1296,7 @@ class Model {
         c.max_rows = spec.chunks.empty() ? 1 : spec.chunks.front();
         c.window = spec.window_tokens.value_or(0);
         c.rope_base = config.rope_base, c.eps = config.floor;
+        c.cache_element = decoder::Cache::abi(cache);
         model_ = nh_model_create(runtime.device(), &c, weights_->arena(), &table);
         if (!model_) panic("%s", nh_last_error());
     }
@@ -1295,9 +1305,11 @@ class Model {
     Model &operator=(const Model &) = delete;
     nh_model *handle() const { return model_; }
     const Config &config() const { return config_; }
+    Element cache_element() const { return cache_; }
 
   private:
     Config config_;
+    Element cache_ = Element::Half;
     std::unique_ptr<runtime::Weights> weights_;
     nh_model *model_ = nullptr;
 };
@@ -1679,12 +1691,15 @@ class Batch {
     // crates/neura-decoder/src/cache.rs:136-137) and shaped [key heads, planes, capacity, width] in half storage.
     void save_state(const std::string &path) const {
         const std::vector<State> states = device_states();
+        const Element stored = model_.cache_element();
+        const size_t wide = decoder::Cache::width_of(stored);
+        const char *dtype = stored == Element::Single ? "F32" : stored == Element::Bfloat16 ? "BF16" : "F16";
         std::string header = "{";
         size_t at = 0;
         for (size_t i = 0; i < states.size(); i++) {
             if (i) header += ',';
-            header += '"' + states[i].name + "\":{\"dtype\":\"F16\",\"shape\":" + states[i].shape + ",\"data_offsets\":[" + std::to_string(at) + ',';
-            at += states[i].elements * 2;
+            header += '"' + states[i].name + "\":{\"dtype\":\"" + dtype + "\",\"shape\":" + states[i].shape + ",\"data_offsets\":[" + std::to_string(at) + ',';
+            at += states[i].elements * wide;
             header += std::to_string(at) + "]}";
         }
         header += '}';
@@ -1694,14 +1709,14 @@ class Batch {
         const uint64_t length = header.size();
         for (int k = 0; k < 8; k++) out.put((char)(length >> (8 * k)));
         out.write(header.data(), (std::streamsize)header.size());
-        std::vector<uint16_t> held;
+        std::vector<uint8_t> held;
         for (const State &state : states) {
-            held.resize(state.elements);
+            held.resize(state.elements * wide);
             if (state.shared)
                 runtime::check(nh_model_shared_read(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
             else
                 runtime::check(nh_model_cache_read(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
-            out.write(reinterpret_cast<const char *>(held.data()), (std::streamsize)(state.elements * 2));
+            out.write(reinterpret_cast<const char *>(held.data()), (std::streamsize)(state.elements * wide));
         }
         out.flush();
         if (!out) panic("a container at %s could not be written", path.c_str());
@@ -1719,7 +1734,10 @@ class Batch {
         std::string header(length, ' ');
         in.read(header.data(), (std::streamsize)length);
         NEURA_ASSERT((uint64_t)in.gcount() == length, "a container at %s ends inside its header", path.c_str());
-        std::vector<uint16_t> held;
+        const Element stored = model_.cache_element();
+        const size_t wide = decoder::Cache::width_of(stored);
+        const std::string dtype = std::string("\"dtype\":\"") + (stored == Element::Single ? "F32" : stored == Element::Bfloat16 ? "BF16" : "F16") + "\"";
+        std::vector<uint8_t> held;
         for (const State &state : device_states()) {
             const std::string &name = state.name;
             const size_t elements = state.elements;
@@ -1727,20 +1745,20 @@ class Batch {
             NEURA_ASSERT(found != std::string::npos, "the container at %s holds no state named %s", path.c_str(), name.c_str());
             const size_t close = header.find('}', found);
             const std::string entry = compact(header.substr(found, close - found));
-            NEURA_ASSERT(entry.find("\"dtype\":\"F16\"") != std::string::npos, "state %s of the container at %s is not in half storage", name.c_str(),
-                         path.c_str());
+            NEURA_ASSERT(entry.find(dtype) != std::string::npos, "state %s of the container at %s is not in %s storage", name.c_str(),
+                         path.c_str(), neura::name(stored));
             NEURA_ASSERT(entry.find("\"shape\":" + state.shape) != std::string::npos, "state %s of the container at %s is not shaped %s", name.c_str(),
                          path.c_str(), state.shape.c_str());
             const size_t offsets = entry.find("\"data_offsets\":[");
             NEURA_ASSERT(offsets != std::string::npos, "state %s of the container at %s names no bytes", name.c_str(), path.c_str());
             const uint64_t begin = std::stoull(entry.substr(offsets + 16));
             const uint64_t end = std::stoull(entry.substr(entry.find(',', offsets + 16) + 1));
-            NEURA_ASSERT(end - begin == elements * 2, "state %s of the container at %s holds %llu bytes where the cache holds %zu", name.c_str(),
-                         path.c_str(), (unsigned long long)(end - begin), elements * 2);
-            held.resize(elements);
+            NEURA_ASSERT(end - begin == elements * wide, "state %s of the container at %s holds %llu bytes where the cache holds %zu", name.c_str(),
+                         path.c_str(), (unsigned long long)(end - begin), elements * wide);
+            held.resize(elements * wide);
             in.seekg((std::streamoff)(8 + length + begin));
-            in.read(reinterpret_cast<char *>(held.data()), (std::streamsize)(elements * 2));
-            NEURA_ASSERT((size_t)in.gcount() == elements * 2, "the container at %s ends inside state %s", path.c_str(), name.c_str());
+            in.read(reinterpret_cast<char *>(held.data()), (std::streamsize)(elements * wide));
+            NEURA_ASSERT((size_t)in.gcount() == elements * wide, "the container at %s ends inside state %s", path.c_str(), name.c_str());
             if (state.shared)
                 runtime::check(nh_model_shared_write(model_.handle(), state.layer, state.value ? 1 : 0, held.data()));
             else

@@ -57,11 +57,14 @@ class Weights:
 class Model:
     """nh_model over a Weights arena; tokens / cursors / mask are host arrays."""
 
-    def __init__(self, device, weights, shape, element, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, window=None):
+    def __init__(self, device, weights, shape, element, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, window=None,
+                 cache_element=1):
         self.device, self.lib, self.weights = device, device.lib, weights
         L = shape["layers"] if layers is None else layers
         self.config = ModelConfig(L, shape["hidden"], shape["heads"], shape["kv_heads"], shape["head_dim"], shape["ffn"], shape["vocab"],
-                                  context, batch, max_rows, window or 0, rope_base, eps)
+                                  context, batch, max_rows, window or 0, rope_base, eps, cache_element)
+        # what the key and value states hold: NH_F16 (1, two bytes read as uint16), NH_BF16 (30, the same) or NH_F32 (0, float32)
+        self.cache_dtype = np.float32 if cache_element == 0 else np.uint16
         table = TensorTable()
         table.matrix_element = element
         table.token_embd = weights.offsets["token_embd.weight"]
@@ -148,11 +151,11 @@ class Model:
         return out
 
     def cache_write(self, layer, value_not_key, halves):
-        halves = np.ascontiguousarray(halves, dtype=np.uint16)
+        halves = np.ascontiguousarray(halves, dtype=self.cache_dtype)
         assert halves.size == int(np.prod(self.cache_shape))
         _check(self.lib.nh_model_cache_write(self.handle, layer, int(value_not_key), halves.ctypes.data))
 
     def cache_read(self, layer, value_not_key):
-        out = np.empty(self.cache_shape, dtype=np.uint16)
+        out = np.empty(self.cache_shape, dtype=self.cache_dtype)
         _check(self.lib.nh_model_cache_read(self.handle, layer, int(value_not_key), out.ctypes.data))
         return out

@@ -61,7 +61,7 @@
 #define WORKGROUP 256     /* neura-profile/src/profile.rs:2086-2089 */
 #define ATTN_KEYS 16      /* neura-profile/src/profile.rs:70 */
 
-enum { EL_F32 = 0, EL_F16 = 1, EL_Q8_0 = 8, EL_Q3_K = 11, EL_Q4_K = 12, EL_Q5_K = 13, EL_Q6_K = 14 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
+enum { EL_F32 = 0, EL_F16 = 1, EL_BF16 = 30, EL_Q8_0 = 8, EL_Q3_K = 11, EL_Q4_K = 12, EL_Q5_K = 13, EL_Q6_K = 14 }; /* ggml ids, neura-gguf/src/header.rs:150-162 */
 
 /* ---------------------------------------------------------------- f16 ---- */
 
@@ -746,10 +746,38 @@ static int key_seen(uint32_t at, uint32_t keys, uint32_t written, uint32_t posit
     return 1;
 }
 
-/* Causal GQA attention over an fp16 or fp32 KV cache, fp32 online softmax in key blocks of 16
+/* One number of a key / value state (crates/neura-kernel/src/fetch.rs:95-107: a half, the upper half of a single, or a single),
+ * and the cast that puts it there (graph.cast, crates/neura-decoder/src/cache.rs:347-348; bfloat16 rounds to nearest even,
+ * crates/neura-kernel/src/task/convert.rs:86-89 and crates/neura-precision/src/lib.rs:325-329). */
+static float cache_value(const void *held, int element, size_t at) {
+    if (element == EL_F32) return ((const float *)held)[at];
+    if (element == EL_BF16) {
+        uint32_t bits = (uint32_t)((const uint16_t *)held)[at] << 16;
+        float value;
+        memcpy(&value, &bits, 4);
+        return value;
+    }
+    return oracle_f16_to_f32(((const uint16_t *)held)[at]);
+}
+static void cache_put(void *held, int element, size_t at, float value) {
+    if (element == EL_F32) {
+        ((float *)held)[at] = value;
+    } else if (element == EL_BF16) {
+        uint32_t bits;
+        memcpy(&bits, &value, 4);
+        ((uint16_t *)held)[at] = (uint16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+    } else {
+        ((uint16_t *)held)[at] = oracle_f32_to_f16(value);
+    }
+}
+void oracle_cache_put_many(void *held, int element, uint64_t at, const float *values, uint64_t count) {
+    for (uint64_t i = 0; i < count; i++) cache_put(held, element, at + i, values[i]);
+}
+
+/* Causal GQA attention over an fp16, bf16 or fp32 KV cache, fp32 online softmax in key blocks of 16
  * (crates/neura-kernel/src/task/attention.rs:309-617; visible :151-163; GQA head :327-334).
  *   q    [heads][batch][rows][width] f32
- *   K,V  [kv_heads][batch][capacity][width]  (kv_element: EL_F16 or EL_F32)
+ *   K,V  [kv_heads][batch][capacity][width]  (kv_element: EL_F16, EL_BF16 or EL_F32)
  *   cursor[batch] = origin of each plane; key `at` visible iff at <= origin+row and at < keys
  *   reach: 0, or the span of a ring (Cache::windowed, crates/neura-decoder/src/cache.rs:366-406): slot `at` then holds
  *          position key_position(at), and a query weighs the last `reach` positions up to its own
@@ -758,7 +786,7 @@ static int key_seen(uint32_t at, uint32_t keys, uint32_t written, uint32_t posit
 int oracle_attention(const float *q, const void *K, const void *V, int kv_element, uint32_t heads, uint32_t kv_heads, uint32_t batch,
                      uint32_t rows, uint32_t width, uint32_t capacity, uint32_t keys, uint32_t reach, const uint32_t *cursor, float scale,
                      float *out) {
-    if (kv_element != EL_F16 && kv_element != EL_F32) return -2;
+    if (kv_element != EL_F16 && kv_element != EL_F32 && kv_element != EL_BF16) return -2;
     if (heads % kv_heads || width > 512) return -1;
     uint32_t groups = heads / kv_heads;
     for (uint32_t h = 0; h < heads; h++)
@@ -783,8 +811,7 @@ int oracle_attention(const float *q, const void *K, const void *V, int kv_elemen
                         if (!seen) continue;
                         float score = 0.0f;
                         for (uint32_t d = 0; d < width; d++) {
-                            float kv = kv_element == EL_F16 ? oracle_f16_to_f32(((const uint16_t *)K)[(plane + at) * width + d])
-                                                            : ((const float *)K)[(plane + at) * width + d];
+                            float kv = cache_value(K, kv_element, (plane + at) * width + d);
                             score = score + qr[d] * kv;
                         }
                         weights[s] = score * scale;
@@ -802,8 +829,7 @@ int oracle_attention(const float *q, const void *K, const void *V, int kv_elemen
                         float weight = block_keys > 0 ? softmax_exp(weights[s] - largest) : 0.0f;
                         total = total + weight;
                         for (uint32_t d = 0; d < width; d++) {
-                            float vv = kv_element == EL_F16 ? oracle_f16_to_f32(((const uint16_t *)V)[(plane + at) * width + d])
-                                                            : ((const float *)V)[(plane + at) * width + d];
+                            float vv = cache_value(V, kv_element, (plane + at) * width + d);
                             acc[d] = acc[d] + weight * vv;
                         }
                     }
@@ -999,6 +1025,7 @@ typedef struct {
      * (examples/qwen/attention.rs:98-154). */
     const int *matrix_elements;
     const float **attn_q_bias, **attn_k_bias, **attn_v_bias;
+    int cache_element; /* what cache_k / cache_v hold: EL_F16, EL_BF16 or EL_F32 (Cache::new(.., element), cache.rs:130-134) */
 } oracle_model;
 
 static int element_of(const oracle_model *m, uint32_t slot) { return m->matrix_elements ? m->matrix_elements[slot] : m->matrix_element; }
@@ -1060,11 +1087,11 @@ int oracle_model_forward(const oracle_model *m, const uint32_t *tokens, uint32_t
                 uint32_t seat = m->ring ? (cursor[b] + row) % m->window : cursor[b] + row;
                 size_t slot = ((size_t)head * B + b) * m->capacity + (mask[b] ? seat : m->window + row);
                 oracle_rope(k + (size_t)t * KW + head * hd, 1, hd, cursor[b] + row, m->rope_base, tmp);
-                oracle_f32_to_f16_many(tmp, hd, m->cache_k[L] + slot * hd);
-                oracle_f32_to_f16_many(v + (size_t)t * KW + head * hd, hd, m->cache_v[L] + slot * hd);
+                oracle_cache_put_many(m->cache_k[L], m->cache_element, slot * hd, tmp, hd);
+                oracle_cache_put_many(m->cache_v[L], m->cache_element, slot * hd, v + (size_t)t * KW + head * hd, hd);
             }
         }
-        oracle_attention(qh, m->cache_k[L], m->cache_v[L], EL_F16, m->heads, m->kv_heads, B, rows, hd, m->capacity, m->window, m->ring ? m->window : 0u, cursor, scale, att);
+        oracle_attention(qh, m->cache_k[L], m->cache_v[L], m->cache_element, m->heads, m->kv_heads, B, rows, hd, m->capacity, m->window, m->ring ? m->window : 0u, cursor, scale, att);
         /* joined + as_rows: [heads][B][rows][hd] -> [T][heads*hd] */
         for (uint32_t t = 0; t < T; t++) {
             uint32_t row = t / B, b = t % B;

@@ -12,6 +12,7 @@ LIBRARY = os.path.join(ORACLE_DIR, "libneura_oracle.so")
 
 EL_F32, EL_F16, EL_Q8_0, EL_Q4_K, EL_Q6_K = 0, 1, 8, 12, 14
 EL_Q3_K, EL_Q5_K = 11, 13
+EL_BF16 = 30
 
 
 class OracleModel(ctypes.Structure):
@@ -22,7 +23,7 @@ class OracleModel(ctypes.Structure):
         ("attn_o", POINTER(c_void_p)), ("ffn_norm", POINTER(c_void_p)), ("ffn_gate", POINTER(c_void_p)), ("ffn_up", POINTER(c_void_p)),
         ("ffn_down", POINTER(c_void_p)), ("cache_k", POINTER(c_void_p)), ("cache_v", POINTER(c_void_p)),
         ("matrix_elements", POINTER(c_int)), ("attn_q_bias", POINTER(c_void_p)), ("attn_k_bias", POINTER(c_void_p)),
-        ("attn_v_bias", POINTER(c_void_p)),
+        ("attn_v_bias", POINTER(c_void_p)), ("cache_element", c_int),
     ]
 
 
@@ -147,10 +148,22 @@ def rope(x, origin, base):
     return out
 
 
-def attention(q, K, V, kv_heads, capacity, keys, cursor, scale, reach=0):
+def cache_cast(values, element):
+    """float32 numbers as a cache of `element` holds them (halves and bfloat16 as uint16 bits, single as it is)"""
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    if element == EL_F32:
+        return values.copy()
+    out = np.empty(values.size, dtype=np.uint16)
+    lib().oracle_cache_put_many(_p(out), c_int(element), c_uint64(0), _p(values.reshape(-1)), c_uint64(values.size))
+    return out.reshape(values.shape)
+
+
+def attention(q, K, V, kv_heads, capacity, keys, cursor, scale, reach=0, element=None):
     q = np.ascontiguousarray(q, dtype=np.float32)
     heads, batch, rows, width = q.shape
-    if K.dtype == np.uint16:
+    if element is not None and element != EL_F32:
+        el = element
+    elif K.dtype == np.uint16:
         el = EL_F16
     else:
         el = EL_F32
@@ -204,7 +217,7 @@ class Model:
     """The oracle's decoder over host copies of the same GGUF tensors the device gets."""
 
     def __init__(self, shape, element, tensors, batch, context, max_rows=1, rope_base=1e6, eps=1e-6, layers=None, elements=None,
-                 window=None):
+                 window=None, cache_element=EL_F16):
         """`elements`: name -> element of the matrices that differ from `element`; tensors named blk.N.attn_{q,k,v}.bias
         are added to the projections before the rotation.  `window`: the caches are rings of that many positions
         (BatchSpec::window, crates/neura-generate/src/batch.rs:148-152, :313-325)."""
@@ -248,8 +261,10 @@ class Model:
                 self.keep.append(pointers)
                 setattr(m, "attn_%s_bias" % which, ctypes.cast(pointers, POINTER(c_void_p)))
         cache_elements = shape["kv_heads"] * batch * self.capacity * shape["head_dim"]
-        self.cache_k = [np.zeros(cache_elements, dtype=np.uint16) for _ in range(L)]
-        self.cache_v = [np.zeros(cache_elements, dtype=np.uint16) for _ in range(L)]
+        m.cache_element = cache_element
+        held_as = np.float32 if cache_element == EL_F32 else np.uint16
+        self.cache_k = [np.zeros(cache_elements, dtype=held_as) for _ in range(L)]
+        self.cache_v = [np.zeros(cache_elements, dtype=held_as) for _ in range(L)]
         ks = (c_void_p * L)(*[a.ctypes.data for a in self.cache_k])
         vs = (c_void_p * L)(*[a.ctypes.data for a in self.cache_v])
         self.keep += [ks, vs]

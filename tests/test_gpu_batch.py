@@ -32,9 +32,9 @@ def qwen2_gguf(path, shape, element, seed, elements=None, biases=()):
     return {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
 
 
-def alone(shape, element, tensors, prompt, count, elements=None, window=None):
+def alone(shape, element, tensors, prompt, count, elements=None, window=None, cache_element=1):
     """The oracle's greedy answer to one prompt: fed token by token, then `count` choices."""
-    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT, elements=elements, window=window)
+    ref = oracle.Model(shape, element, tensors, batch=1, context=CONTEXT, elements=elements, window=window, cache_element=cache_element)
     margins = []
     for at, token in enumerate(prompt):
         logits, chosen = ref.forward([token], 1, [at])
@@ -82,6 +82,43 @@ def test_a_batched_sequence_answers_as_it_does_alone(runtime, tmp_path, shape, e
         want, margin = alone(shape, element, tensors, prompt, 8)
         assert got[slot] == want, (slot, margin)
     batch.close()
+    archive.close()
+
+
+@pytest.mark.parametrize("cache,dtype", [(0, np.float32), (30, None)], ids=["single", "bfloat16"])
+def test_a_batch_keeps_its_states_in_the_element_it_is_given(runtime, tmp_path, cache, dtype):
+    """The model function hands its caches an element (examples/qwen/main.rs:107 keeps single precision states): a batch over such
+    a model answers as the oracle with the same states does, and its state file holds them in that element."""
+    from safetensors.numpy import load_file
+
+    shape, element = SHAPE, NH_Q8_0
+    tensors = qwen2_gguf(tmp_path / "model.gguf", shape, element, seed=71)
+    archive = host.GgufFile.open(tmp_path / "model.gguf")
+    batch = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], cache=cache)
+    rng = np.random.default_rng(72)
+    prompts = [list(rng.integers(0, shape["vocab"], n)) for n in (5, 21)]
+    slots = [batch.admit(prompt) for prompt in prompts]
+    got = run(batch, {slot: 6 for slot in slots})
+    for slot, prompt in zip(slots, prompts):
+        want, margin = alone(shape, element, tensors, prompt, 6, cache_element=cache)
+        assert got[slot] == want, (slot, margin)
+    batch.save_state(tmp_path / "state.safetensors")
+    raw = open(tmp_path / "state.safetensors", "rb").read()
+    assert (b'"dtype":"F32"' if cache == 0 else b'"dtype":"BF16"') in raw
+    if dtype is not None:  # numpy holds no bfloat16: the single precision file is opened by the package, the other by its header
+        held = load_file(str(tmp_path / "state.safetensors"))
+        assert all(tensor.dtype == dtype and tensor.shape == (shape["kv_heads"], 2, CONTEXT + 8, shape["head_dim"]) for tensor in held.values())
+        assert held["blk.1.cache.key"][:, 1, :20].any()
+    second = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], cache=cache)
+    second.restore_state(tmp_path / "state.safetensors", batch.snapshot())
+    assert run(second, {0: 4, 1: 4}) == run(batch, {0: 4, 1: 4})
+    other = host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8])
+    with pytest.raises(host.Panic, match="is not in half storage"):
+        other.restore_state(tmp_path / "state.safetensors", batch.snapshot())
+    with pytest.raises(host.Panic, match="single, half or bfloat16"):
+        host.Batch(runtime, archive, shape["vocab"], CONTEXT, 2, [8], cache=8)
+    for held_batch in (batch, second, other):
+        held_batch.close()
     archive.close()
 
 

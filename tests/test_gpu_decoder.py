@@ -12,13 +12,13 @@ TINY = dict(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512, voc
 SMALL_Q4 = dict(layers=3, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=1000, tied=False)
 
 
-def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None, window=None):
+def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None, window=None, cache_element=1):
     rng = np.random.default_rng(seed)
     tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
     host = {name: raw for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
-    model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers, window=window)
-    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers, window=window)
+    model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers, window=window, cache_element=cache_element)
+    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers, window=window, cache_element=cache_element)
     return model, ref, weights
 
 
@@ -49,6 +49,46 @@ def test_decode_steps_match_oracle_logits_and_tokens(device, shape, element):
             want_cache = oracle.f16_to_f32(held[layer])
             assert np.abs(got_cache - want_cache).max() <= 2e-3 * max(1.0, np.abs(want_cache).max())
     model.release(), weights.release()
+
+
+@pytest.mark.parametrize("cache_element", [0, 30], ids=["single", "bfloat16"])
+@pytest.mark.parametrize("shape,element", [(TINY, NH_Q8_0), (SMALL_Q4, NH_Q4_K)])
+def test_decoders_keep_their_states_in_single_or_bfloat16(device, shape, element, cache_element):
+    """Cache::new(.., Element::Single | Bfloat16) (crates/neura-decoder/src/cache.rs:130-134; the reference's own example
+    keeps single precision states, examples/qwen/main.rs:107): a fill chunk with one plane masked, then decode steps of
+    both planes -- logits and greedy tokens as the oracle's with the same states, and the states themselves equal."""
+    model, ref, weights = build(device, shape, element, batch=2, context=40, max_rows=8, seed=5, cache_element=cache_element)
+    rng = np.random.default_rng(6)
+    prompt = rng.integers(0, shape["vocab"], (8, 2))
+    model.prefill(prompt.reshape(-1), 8, [0, 0], mask=[1, 0])
+    ref.forward(prompt.reshape(-1), 8, [0, 0], mask=[1, 0], want_logits=False)
+    model.prefill(prompt.reshape(-1), 8, [8, 0], mask=[1, 1])
+    ref.forward(prompt.reshape(-1), 8, [8, 0], mask=[1, 1], want_logits=False)
+    tokens = rng.integers(0, shape["vocab"], 2)
+    for step in range(5):
+        cursors = [16 + step, 8 + step]
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        got = model.decode_step(tokens, cursors)
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens = got
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_cache, want_cache = model.cache_read(layer, which).reshape(-1), held[layer]
+            if cache_element == 30:
+                got_cache, want_cache = (got_cache.astype(np.uint32) << 16).view(np.float32), (want_cache.astype(np.uint32) << 16).view(np.float32)
+            assert got_cache.dtype == np.float32 and np.abs(got_cache - want_cache).max() <= 1e-2 * max(1.0, np.abs(want_cache).max())
+    # a state written through the C ABI reads back as it was written, in the states' element
+    written = (rng.standard_normal(model.cache_shape).astype(np.float32) if cache_element == 0
+               else rng.integers(0, 1 << 15, model.cache_shape).astype(np.uint16))
+    model.cache_write(0, 1, written)
+    assert np.array_equal(model.cache_read(0, 1), written)
+    model.release(), weights.release()
+
+
+def test_a_decoder_names_the_element_of_its_states(device):
+    with pytest.raises(NeuraError, match="single, half or bfloat16"):
+        build(device, TINY, NH_Q8_0, batch=1, context=8, cache_element=12)
 
 
 def test_masked_planes_and_chunked_fill(device):

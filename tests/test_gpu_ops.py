@@ -486,6 +486,46 @@ def test_attention_matches_oracle_and_f64(device, heads, kv_heads, batch, rows, 
         assert np.abs(got - exact).max() <= 1e-5  # the reference's bar against fp64 (runtime.rs:551-619)
 
 
+@pytest.mark.parametrize("element", [0, 30])  # Element::Single, Element::Bfloat16 (crates/neura-decoder/src/cache.rs:130-134)
+@pytest.mark.parametrize("heads,kv_heads,batch,rows,keys,width,origins", [
+    (4, 2, 2, 3, 12, 32, [9, 4]),
+    (14, 2, 1, 1, 1100, 64, [1024]),
+    (28, 4, 2, 1, 600, 128, [63, 599]),
+    (12, 2, 1, 17, 300, 128, [200]),
+    (8, 8, 2, 5, 40, 256, [35, 0]),
+])
+def test_attention_over_single_and_bfloat16_states(device, element, heads, kv_heads, batch, rows, keys, width, origins):
+    """Keys and values cast into states of another element by the device (nh_cache_write_element), bit for bit what the
+    oracle's cast holds, then weighed (nh_attention_element) as the oracle weighs them and within 1e-5 of the f64 reference
+    over the numbers the states hold."""
+    rng = np.random.default_rng(17 + element)
+    capacity = keys + rows
+    wide = 4 if element == 0 else 2
+    stored = np.float32 if element == 0 else np.uint16
+    ck, cv = device.alloc(kv_heads * batch * capacity * width * wide), device.alloc(kv_heads * batch * capacity * width * wide)
+    K = rng.standard_normal((kv_heads, batch, capacity, width)).astype(np.float32)
+    V = rng.standard_normal((kv_heads, batch, capacity, width)).astype(np.float32)
+    want_k, want_v = oracle.cache_cast(K, element), oracle.cache_cast(V, element)
+    for first in range(0, capacity - rows + 1, rows):  # the states are filled a chunk at a time through the writer
+        device.cache_write(K[:, :, first : first + rows], V[:, :, first : first + rows], ck, cv, capacity, keys, [first] * batch, element=element)
+    filled = (capacity - rows) // rows * rows + rows
+    got_k, got_v = ck.numpy(stored, K.shape), cv.numpy(stored, K.shape)
+    assert np.array_equal(got_k[:, :, :filled].view(np.uint8), want_k[:, :, :filled].view(np.uint8))
+    assert np.array_equal(got_v[:, :, :filled].view(np.uint8), want_v[:, :, :filled].view(np.uint8))
+    ck, cv = device.upload(want_k), device.upload(want_v)  # every slot now, the ones no chunk reached too
+    q = rng.standard_normal((heads, batch, rows, width)).astype(np.float32)
+    scale = 1.0 / np.sqrt(width)
+    got = device.attention(q, ck, cv, kv_heads, capacity, keys, origins, scale, element=element)
+    want = oracle.attention(q, want_k, want_v, kv_heads, capacity, keys, origins, scale, element=element)
+    close(got, want)
+    assert np.abs(got - want).max() <= 1e-5
+    if batch == 1:
+        held_k = want_k if element == 0 else (want_k.astype(np.uint32) << 16).view(np.float32)
+        held_v = want_v if element == 0 else (want_v.astype(np.uint32) << 16).view(np.float32)
+        exact = oracle.attention_f64(q, held_k[:, :, :keys], held_v[:, :, :keys], kv_heads, origins[0], True, scale)
+        assert np.abs(got - exact).max() <= 1e-5
+
+
 def test_attention_of_equal_scores_is_the_running_mean(device):
     # crates/neura-runtime/tests/runtime.rs:813-875
     rng = np.random.default_rng(43)
@@ -497,11 +537,13 @@ def test_attention_of_equal_scores_is_the_running_mean(device):
             assert np.allclose(got[head, 0, 0], V[head // 2, 0, : origin + 1].astype(np.float32).mean(axis=0), atol=1e-5)
 
 
-def test_a_ring_cache_weighs_the_last_window_of_keys(device):
-    # crates/neura-decoder/tests/cache.rs:11-51 in half storage: equal scores, value = step -> the mean of the last WINDOW steps
+@pytest.mark.parametrize("element", [1, 0, 30])
+def test_a_ring_cache_weighs_the_last_window_of_keys(device, element):
+    # crates/neura-decoder/tests/cache.rs:11-51 (the reference runs it in single and half storage): equal scores,
+    # value = step -> the mean of the last WINDOW steps
     WINDOW, CAPACITY, WIDTH = 5, 7, 32
-    ck = device.alloc(CAPACITY * WIDTH * 2)
-    cv = device.alloc(CAPACITY * WIDTH * 2)
+    ck = device.alloc(CAPACITY * WIDTH * 4)
+    cv = device.alloc(CAPACITY * WIDTH * 4)
     q = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
     q[..., 0] = 1.0
     key = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
@@ -509,8 +551,8 @@ def test_a_ring_cache_weighs_the_last_window_of_keys(device):
     for step in range(2 * WINDOW + 2):
         value = np.zeros((1, 1, 1, WIDTH), dtype=np.float32)
         value[..., 0] = float(step)
-        device.cache_write(key, value, ck, cv, CAPACITY, WINDOW, [step], ring=True)
-        got = device.attention(q, ck, cv, 1, CAPACITY, WINDOW, [step], 1.0, reach=WINDOW)
+        device.cache_write(key, value, ck, cv, CAPACITY, WINDOW, [step], ring=True, element=element)
+        got = device.attention(q, ck, cv, 1, CAPACITY, WINDOW, [step], 1.0, reach=WINDOW, element=element)
         first = max(0, step - (WINDOW - 1))
         expected = sum(range(first, step + 1)) / (step - first + 1)
         assert abs(got[0, 0, 0, 0] - expected) < 1e-5 and got[0, 0, 0, 1] == 0.0, (step, got[0, 0, 0, :2])
