@@ -52,6 +52,8 @@ SIGNATURES = {
     "nhost_vector": (c_int32, [c_void_p, c_char_p, c_uint32, POINTER(c_int32)]),
     "nhost_cache_validate": (c_int32, [c_char_p] + [c_uint32] * 6 + [c_int32]),
     "nhost_payload_bytes": (c_uint64, [c_int32, c_uint64]),
+    "nhost_template_render": (c_int64, [c_char_p, c_char_p, c_char_p, c_void_p, c_size_t]),
+    "nhost_template_render_gguf": (c_int64, [c_void_p, c_char_p, c_char_p, c_void_p, c_size_t]),
     "nhost_pack": (c_int64, [c_int32, c_float, c_void_p, c_size_t, c_void_p, c_size_t]),
     "nhost_unpack": (c_int32, [c_int32, c_size_t, c_void_p, c_size_t, c_void_p]),
     "nhost_half_bits": (c_uint32, [c_float]),
@@ -413,6 +415,28 @@ def seed_bits(seed):
 
 def payload_bytes(element, elements):
     return int(library().nhost_payload_bytes(element, elements))
+
+
+def render_template(source, messages, values=None):
+    """neura_template::Template::parse(source).render(messages, values) (crates/neura-template/src/template.rs): `source` is the
+    template text, or an opened GGUF whose tokenizer.chat_template is read; messages are mappings with a role and a content"""
+    import json
+
+    listed = json.dumps(list(messages), ensure_ascii=False).encode("utf-8")
+    named = json.dumps(dict(values or {}), ensure_ascii=False).encode("utf-8")
+    room = ctypes.create_string_buffer(1 << 16)
+    for _ in range(2):
+        if isinstance(source, (str, bytes)):
+            text = source.encode("utf-8") if isinstance(source, str) else source
+            length = library().nhost_template_render(text, listed, named, room, len(room))
+        else:
+            length = library().nhost_template_render_gguf(source.handle, listed, named, room, len(room))
+        if length < 0:
+            raise _refused()
+        if length <= len(room):
+            return room.raw[:length].decode("utf-8")
+        room = ctypes.create_string_buffer(length)
+    raise RuntimeError("a rendered template outgrew its room twice")
 
 
 def pack(element, values, quantum=0.0):

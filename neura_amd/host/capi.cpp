@@ -3,6 +3,7 @@
 // (0 done, -1 refused) or a null handle, and nhost_last_error() then holds the sentence the
 // reference would have panicked with.
 #include "neura.hpp"
+#include "template.hpp"
 #include "tokenizer.hpp"
 
 #include <cstdlib>
@@ -40,6 +41,131 @@ std::unique_ptr<tokenizer::Rule> rule_named(const std::string &name) {
     if (name == "per_space") return std::make_unique<tokenizer::PerSpace>();
     if (name == "whole") return std::make_unique<tokenizer::Whole>();
     panic("no split rule is named %s", name.c_str());
+}
+}  // namespace
+
+namespace {
+// what a script hands the template engine: JSON text into chat::Value (objects keep their order; a number without a
+// fraction or exponent is a whole number)
+struct Json {
+    const std::string &text;
+    size_t at = 0;
+    void blanks() {
+        while (at < text.size() && std::isspace((unsigned char)text[at])) at++;
+    }
+    char next() {
+        blanks();
+        if (at >= text.size()) panic("the json handed to a template ends early");
+        return text[at];
+    }
+    void expect(char wanted) {
+        if (next() != wanted) panic("the json handed to a template holds %c where %c stands", text[at], wanted);
+        at++;
+    }
+    static void put(std::string &out, uint32_t code) {
+        if (code < 0x80) out += (char)code;
+        else if (code < 0x800) out += (char)(0xc0 | code >> 6), out += (char)(0x80 | (code & 63));
+        else if (code < 0x10000) out += (char)(0xe0 | code >> 12), out += (char)(0x80 | ((code >> 6) & 63)), out += (char)(0x80 | (code & 63));
+        else out += (char)(0xf0 | code >> 18), out += (char)(0x80 | ((code >> 12) & 63)), out += (char)(0x80 | ((code >> 6) & 63)), out += (char)(0x80 | (code & 63));
+    }
+    uint32_t hex4() {
+        if (at + 4 > text.size()) panic("the json handed to a template ends inside an escape");
+        const uint32_t code = (uint32_t)std::stoul(text.substr(at, 4), nullptr, 16);
+        at += 4;
+        return code;
+    }
+    std::string string() {
+        expect('"');
+        std::string out;
+        while (at < text.size() && text[at] != '"') {
+            char c = text[at++];
+            if (c != '\\') {
+                out += c;
+                continue;
+            }
+            c = text[at++];
+            switch (c) {
+            case 'n': out += '\n'; break;
+            case 't': out += '\t'; break;
+            case 'r': out += '\r'; break;
+            case 'b': out += '\b'; break;
+            case 'f': out += '\f'; break;
+            case 'u': {
+                uint32_t code = hex4();
+                if (code >= 0xd800 && code < 0xdc00 && text.compare(at, 2, "\\u") == 0) {
+                    at += 2;
+                    code = 0x10000 + ((code - 0xd800) << 10) + (hex4() - 0xdc00);
+                }
+                put(out, code);
+                break;
+            }
+            default: out += c;
+            }
+        }
+        expect('"');
+        return out;
+    }
+    chat::Value value() {
+        const char c = next();
+        if (c == '"') return chat::Value::of(string());
+        if (c == '{') {
+            at++;
+            chat::Value::Entries entries;
+            if (next() == '}') return at++, chat::Value::map({});
+            for (;;) {
+                std::string key = string();
+                expect(':');
+                entries.emplace_back(std::move(key), value());
+                if (next() == ',') {
+                    at++;
+                    continue;
+                }
+                expect('}');
+                return chat::Value::map(std::move(entries));
+            }
+        }
+        if (c == '[') {
+            at++;
+            std::vector<chat::Value> items;
+            if (next() == ']') return at++, chat::Value::list({});
+            for (;;) {
+                items.push_back(value());
+                if (next() == ',') {
+                    at++;
+                    continue;
+                }
+                expect(']');
+                return chat::Value::list(std::move(items));
+            }
+        }
+        if (text.compare(at, 4, "true") == 0) return at += 4, chat::Value::of(true);
+        if (text.compare(at, 5, "false") == 0) return at += 5, chat::Value::of(false);
+        if (text.compare(at, 4, "null") == 0) return at += 4, chat::Value::empty();
+        size_t end = at;
+        bool real = false;
+        while (end < text.size() && (std::isdigit((unsigned char)text[end]) || std::strchr("+-.eE", text[end]))) real |= std::strchr(".eE", text[end]) != nullptr, end++;
+        if (end == at) panic("the json handed to a template holds %c where a value stands", c);
+        const std::string digits = text.substr(at, end - at);
+        at = end;
+        return real ? chat::Value::of(std::stod(digits)) : chat::Value::of((int64_t)std::stoll(digits));
+    }
+};
+
+int64_t rendered(const chat::Template &held, const char *messages_json, const char *values_json, char *out, size_t room) {
+    const std::string messages_text = messages_json ? messages_json : "[]", values_text = values_json ? values_json : "{}";
+    const chat::Value listed = Json{messages_text}.value(), named = Json{values_text}.value();
+    if (listed.kind != chat::Value::List || named.kind != chat::Value::Map) panic("a template renders a list of messages and a mapping of values");
+    std::vector<chat::Message> messages;
+    for (const chat::Value &entry : listed.items) {
+        if (entry.kind != chat::Value::Map) panic("a message handed to a template is a mapping");
+        chat::Message message(entry.attribute("role").text(), entry.attribute("content"));
+        for (const auto &field : entry.entries)
+            if (field.first != "role" && field.first != "content") message = std::move(message).with(field.first, field.second);
+        messages.push_back(std::move(message));
+    }
+    const std::string text = held.render(messages, named.entries);
+    for (size_t i = 0; i < text.size() && i < room; i++) out[i] = text[i];
+    return (int64_t)text.size();
 }
 }  // namespace
 
@@ -204,6 +330,19 @@ int32_t nhost_unpack(int32_t element, size_t elements, const uint8_t *bytes, siz
 }
 uint32_t nhost_half_bits(float value) { return precision::half_bits(value); }
 float nhost_half_value(uint32_t bits) { return precision::half_value((uint16_t)bits); }
+
+// ---- neura-template -----------------------------------------------------------------------------------
+// Template::parse(source).render(messages, values): messages and values as JSON text; the rendered bytes (out, at most room);
+// returns their count, or -1 refused
+int64_t nhost_template_render(const char *source, const char *messages_json, const char *values_json, char *out, size_t room) {
+    return guarded([&]() -> int64_t { return rendered(chat::Template::parse(source), messages_json, values_json, out, room); }, -1);
+}
+// Template::read(archive): the template the GGUF carries under tokenizer.chat_template
+int64_t nhost_template_render_gguf(void *held, const char *messages_json, const char *values_json, char *out, size_t room) {
+    return guarded([&]() -> int64_t {
+        return rendered(chat::Template::read(static_cast<Opened *>(held)->archive()), messages_json, values_json, out, room);
+    }, -1);
+}
 
 // ---- runtime, model, batch ----------------------------------------------------------------------
 void *nhost_runtime_open(int32_t index) {
