@@ -23,6 +23,7 @@ struct GemvParams {
     uint32_t group;             // lanes that share one output row: 16, 32 or 64
     uint32_t row_groups;        // passes over the rows
     uint32_t tile_rows;         // 16-row tile kernel, plain epilogue: weight rows a tile holds (12..16)
+    uint32_t rows;              // 16-row tile kernel: activation rows of x (1..8)
     uint32_t chunks_per_row;    // Q8_0: 16-byte chunks of a staged row slice
     int32_t swiglu;
     float eps;

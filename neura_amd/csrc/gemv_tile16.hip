@@ -28,16 +28,21 @@ constexpr uint32_t TILE16_BLOCK_DIGITS = 768;  // 16 chunks of 16 activations x 
 constexpr uint32_t TILE16_ZERO_BYTES = 208;    // what an idle A lane reads: four chunk offsets (0, 48, 96, 144) + 16 bytes
 enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2 };
 
-static size_t tile16_lds(uint32_t nblk, uint32_t NW) {
-    return (size_t)nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + (size_t)nblk * 64u + (size_t)2 * NW * 16u * 4u + (size_t)NW * 4u + 64u;
+static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R) {
+    return (size_t)R * nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + (size_t)R * nblk * 64u + (size_t)2 * NW * R * 16u * 4u + (size_t)NW * R * 4u + 64u;
 }
 
 struct Tile16Unit {
     u32x4 hdr, qa, qb;
 };
 
-template <int NW, int D, int MODE>
+//
+// R > 1: up to R activation rows (p.rows of them) meet the weights in one pass.  Every row has its own digit planes and sums in
+// LDS; a step unpacks its weights once and runs the four MFMAs and the weighing once a row, so the weights are read once for
+// all rows where one launch a row read them `rows` times.
+template <int NW, int D, int MODE, int R>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) {
+    static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
     extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
     constexpr uint32_t NT = NW * 64;
     typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -47,10 +52,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t nblk = p.nblk;
     uint8_t *const digits = tile16_lds_bytes;
-    uint8_t *const zeros = tile16_lds_bytes + (size_t)nblk * TILE16_BLOCK_DIGITS + wave * TILE16_ZERO_BYTES;  // a wave's own zeros
-    f32x4 *const sums = reinterpret_cast<f32x4 *>(tile16_lds_bytes + (size_t)nblk * TILE16_BLOCK_DIGITS + NW * TILE16_ZERO_BYTES);
-    float *const part = reinterpret_cast<float *>(sums + (size_t)nblk * 4u);
-    float *const red = part + 2u * NW * 16u;
+    const uint32_t row_digits = nblk * TILE16_BLOCK_DIGITS;  // digit planes of one activation row
+    uint8_t *const zeros = tile16_lds_bytes + (size_t)R * row_digits + wave * TILE16_ZERO_BYTES;  // a wave's own zeros
+    f32x4 *const sums = reinterpret_cast<f32x4 *>(tile16_lds_bytes + (size_t)R * row_digits + NW * TILE16_ZERO_BYTES);  // [row][block][group]
+    float *const part = reinterpret_cast<float *>(sums + (size_t)R * nblk * 4u);  // [parity][wave][row][16]
+    float *const red = part + 2u * NW * R * 16u;                                  // [wave][row]
 
     const uint32_t r = lane & 15u, q = lane >> 4;
     // tiles of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
@@ -126,11 +132,86 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     // exactly the super-blocks it multiplies.
     {
         const uint32_t units = p.K / 4u;
+        if (lane < TILE16_ZERO_BYTES / 4u) reinterpret_cast<uint32_t *>(zeros)[lane] = 0u;
+        auto stage = [&](uint32_t e4, f32x4 v, f32x4 w, float rms, uint8_t *row_planes, f32x4 *row_sums) {
+            if (p.norm_w) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
+            }
+            uint32_t top = 0;  // largest magnitude of the group as bits: infinities and NaNs sort above every finite value
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float element = v[i];  // a copy first: the bits of a vector element taken in place read element 0 every time
+                top = max(top, __builtin_bit_cast(uint32_t, element) & 0x7fffffffu);
+            }
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
+            const uint32_t raw = top >> 23;
+            const uint32_t exponent = min(max(raw, 22u), 254u);
+            const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);  // the group's largest magnitude lands in [2^21, 2^22)
+            const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
+            float total = 0.0f;
+            uint32_t dg[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float rounded = rintf(v[i] * scale);
+                total += rounded;
+                dg[i] = signed_digits((int)rounded);  // bytes 0..2: signed digits, least significant first; byte 3 is zero below 2^23
+            }
+            const uint32_t lo01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x07030602u);
+            const uint32_t plane2 = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);  // digit 0 (least significant) of the four elements
+            const uint32_t plane1 = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+            const uint32_t plane0 = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  // digit 2 (most significant)
+            total += dpp<DPP_QUAD_XOR1>(total);
+            total += dpp<DPP_QUAD_XOR2>(total);
+            total += dpp<0x141>(total);  // half mirror: the other quad of the eight lanes of a sub-block
+            // unit e4: 64 units a super-block, 16 a group, 8 a sub-block, 4 a chunk of 16 elements
+            uint32_t *slot = reinterpret_cast<uint32_t *>(row_planes + (size_t)(e4 >> 2) * 48u) + (e4 & 3u);
+            slot[0] = plane0, slot[4] = plane1, slot[8] = plane2;
+            float *s = reinterpret_cast<float *>(row_sums + (e4 >> 4));  // (low sub-block sum, high sub-block sum, unscale, -)
+            if ((e4 & 7u) == 0) s[(e4 >> 3) & 1u] = total * unscale;
+            if ((e4 & 15u) == 0) s[2] = unscale;
+        };
+        if constexpr (R > 1) {
+            // the weights' loads go out first; every row's activations follow (twice where the norm is folded in: once for
+            // the row's sum of squares, once for the digits -- the second pass finds them in the cache)
+#pragma unroll
+            for (int i = 0; i < D; i++) fetch(ring[i]);
+            const uint32_t rows = min(p.rows, (uint32_t)R);
+            if (p.norm_w) {
+                for (uint32_t row = 0; row < rows; row++) {
+                    float square = 0.0f;
+                    for (uint32_t e4 = tid; e4 < units; e4 += NT) {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
+                    }
+                    square = wave_sum(square);
+                    if (lane == 0) red[wave * R + row] = square;
+                }
+                __syncthreads();
+            }
+            for (uint32_t row = 0; row < rows; row++) {
+                float rms = 1.0f;
+                if (p.norm_w) {
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < NW; w++) total += red[w * R + row];
+                    rms = rms_scale_of(total, p.K, p.eps);
+                }
+                for (uint32_t e4 = tid; e4 < units; e4 += NT)
+                    stage(e4, *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4),
+                          p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms, digits + (size_t)row * row_digits,
+                          sums + (size_t)row * nblk * 4u);
+            }
+        } else {
         constexpr int MAXJ = 5;
         f32x4 held[MAXJ], weight[MAXJ];
         const bool resident = units <= MAXJ * NT;
         float rms = 1.0f;
-        if (lane < TILE16_ZERO_BYTES / 4u) reinterpret_cast<uint32_t *>(zeros)[lane] = 0u;
         if (resident) {
 #pragma unroll
             for (int j = 0; j < MAXJ; j++) {
@@ -172,58 +253,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             for (int w = 0; w < NW; w++) total += red[w];
             rms = rms_scale_of(total, p.K, p.eps);
         }
-        auto stage = [&](uint32_t e4, f32x4 v, f32x4 w) {
-            if (p.norm_w) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
-            }
-            uint32_t top = 0;  // largest magnitude of the group as bits: infinities and NaNs sort above every finite value
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float element = v[i];  // a copy first: the bits of a vector element taken in place read element 0 every time
-                top = max(top, __builtin_bit_cast(uint32_t, element) & 0x7fffffffu);
-            }
-            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
-            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
-            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
-            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
-            const uint32_t raw = top >> 23;
-            const uint32_t exponent = min(max(raw, 22u), 254u);
-            const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);  // the group's largest magnitude lands in [2^21, 2^22)
-            const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
-            float total = 0.0f;
-            uint32_t dg[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float rounded = rintf(v[i] * scale);
-                total += rounded;
-                dg[i] = signed_digits((int)rounded);  // bytes 0..2: signed digits, least significant first; byte 3 is zero below 2^23
-            }
-            const uint32_t lo01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x07030602u);
-            const uint32_t lo23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x07030602u);
-            const uint32_t plane2 = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);  // digit 0 (least significant) of the four elements
-            const uint32_t plane1 = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
-            const uint32_t plane0 = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  // digit 2 (most significant)
-            total += dpp<DPP_QUAD_XOR1>(total);
-            total += dpp<DPP_QUAD_XOR2>(total);
-            total += dpp<0x141>(total);  // half mirror: the other quad of the eight lanes of a sub-block
-            // unit e4: 64 units a super-block, 16 a group, 8 a sub-block, 4 a chunk of 16 elements
-            uint32_t *slot = reinterpret_cast<uint32_t *>(digits + (size_t)(e4 >> 2) * 48u) + (e4 & 3u);
-            slot[0] = plane0, slot[4] = plane1, slot[8] = plane2;
-            float *s = reinterpret_cast<float *>(sums + (e4 >> 4));  // (low sub-block sum, high sub-block sum, unscale, -)
-            if ((e4 & 7u) == 0) s[(e4 >> 3) & 1u] = total * unscale;
-            if ((e4 & 15u) == 0) s[2] = unscale;
-        };
         if (resident) {
 #pragma unroll
             for (int j = 0; j < MAXJ; j++) {
                 if (NT * j >= units) break;  // uniform over the workgroup
                 const uint32_t e4 = tid + NT * j;
-                if (e4 < units) stage(e4, held[j], weight[j]);  // whole groups of 16 lanes are in or out together
+                if (e4 < units) stage(e4, held[j], weight[j], rms, digits, sums);  // whole groups of 16 lanes are in or out together
             }
         } else {
             for (uint32_t e4 = tid; e4 < units; e4 += NT)
-                stage(e4, *reinterpret_cast<const f32x4 *>(p.x + 4u * e4), p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f});
+                stage(e4, *reinterpret_cast<const f32x4 *>(p.x + 4u * e4), p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
+                      digits, sums);
+        }
         }
     }
     __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see this wave's writes
@@ -239,7 +280,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     const bool feeds = (m >> 2) == q && (m & 3u) < 3u;  // A row m = 4 * slice + plane meets K slice `slice` only
     const uint8_t *const abase = feeds ? digits + q * 192u + (m & 3u) * 16u : zeros;
     const uint32_t astride = feeds ? TILE16_BLOCK_DIGITS : 0u;
-    float acc = 0.0f, gate = 0.0f;
+    const uint32_t arow = feeds ? row_digits : 0u;  // from one activation row's planes to the next one's
+    constexpr int RQ = (R + 3) / 4;                 // rows an epilogue lane finishes: q, q + 4, ...
+    float acc[R], gate[RQ];
+#pragma unroll
+    for (int row = 0; row < R; row++) acc[row] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < RQ; i++) gate[i] = 0.0f;
     uint32_t parity = 0;
     // One step in two halves with the next fetch between them: everything that reads the fetched registers (nibbles, header)
     // comes first, so the fetch can reuse them, and the weighing of the sums follows while the loads are under way.
@@ -275,21 +322,65 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         const float weighed = fmaf((float)sc.x, fl, (float)sc.y * fh);    // scales and minimums arrive * 2^-24 (half subnormals)
         const float floor_ = fmaf((float)mn.x, st.s.x, (float)mn.y * st.s.y);
         const float d24 = (float)dd.x * (16777216.0f * st.s.z), m24 = (float)dd.y * -16777216.0f;
-        acc = fmaf(d24, weighed, fmaf(m24, floor_, acc));
+        acc[0] = fmaf(d24, weighed, fmaf(m24, floor_, acc[0]));
+    };
+    // R > 1: the weights are unpacked once, the next fetch goes out, and every row then runs its four MFMAs and its weighing
+    auto step_rows = [&](Tile16Unit &u, uint32_t b) {
+        const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+        const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
+        const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
+        half2_t sc, mn;
+        scale_pairs(u.hdr, lane_scales, sc, mn);
+        const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);
+        float scx = (float)sc.x, scy = (float)sc.y, mnx = (float)mn.x, mny = (float)mn.y;
+        float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * -16777216.0f;
+        asm volatile("" : "+v"(scx), "+v"(scy), "+v"(mnx), "+v"(mny), "+v"(d24), "+v"(m24));  // the header is read by here
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(u);
+        __builtin_amdgcn_sched_barrier(0);
+        const uint8_t *at = abase + (size_t)b * astride;
+        const f32x4 *s = sums + b * 4u + q;
+#pragma unroll
+        for (int row = 0; row < R; row++) {
+            const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
+            const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
+            const f32x4 rs = *s;
+            i32x4 cl = {0, 0, 0, 0}, ch = {0, 0, 0, 0};
+            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a00, la, cl, 0, 0, 0);
+            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a10, ha, ch, 0, 0, 0);
+            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a01, lb, cl, 0, 0, 0);
+            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a11, hb, ch, 0, 0, 0);
+            const float fl = fmaf((float)((cl[0] << 8) + cl[1]), 256.0f, (float)cl[2]);
+            const float fh = fmaf((float)((ch[0] << 8) + ch[1]), 256.0f, (float)ch[2]);
+            const float weighed = fmaf(scx, fl, scy * fh);
+            const float floor_ = fmaf(mnx, rs.x, mny * rs.y);
+            acc[row] = fmaf(d24 * rs.z, weighed, fmaf(m24, floor_, acc[row]));
+            at += arow;
+            s += nblk * 4u;
+        }
     };
     auto tile_end = [&](uint32_t tile) {
-        float v = acc;
-        v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
-        v += __shfl_xor(v, 32, 64);
-        if (q == 0) part[(parity * NW + wave) * 16u + r] = v;
+#pragma unroll
+        for (int row = 0; row < R; row++) {
+            float v = acc[row];
+            v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+            v += __shfl_xor(v, 32, 64);
+            if (q == 0) part[((parity * NW + wave) * R + row) * 16u + r] = v;
+            acc[row] = 0.0f;
+        }
         __syncthreads();
-        if (wave == 0 && lane < 16u) {
+        if (wave == 0) {
+#pragma unroll
+          for (int i = 0; i < RQ; i++) {
+            // lane (r, q) finishes output r of activation rows q, q + 4, ...
+            const uint32_t row = q + 4u * i;
+            if (row >= min(p.rows, (uint32_t)R)) break;
             float total = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW; w++) total += part[(parity * NW + w) * 16u + lane];
+            for (int w = 0; w < NW; w++) total += part[((parity * NW + w) * R + row) * 16u + r];
             if (MODE == TILE16_SWIGLU) {
-                if (tile & 1u) p.y[(tile >> 1) * 16u + lane] = silu(gate) * total;
-                else gate = total;
+                if (tile & 1u) p.y[(size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r] = silu(gate[i]) * total;
+                else gate[i] = total;
             } else if (MODE == TILE16_ROPE) {
                 uint32_t c;
                 const uint32_t n = rope_row(tile, c);
@@ -298,15 +389,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
                     const uint32_t next = rope_row(tile + hop, c);
                     rope_held = rope_operands(p, next, c, rope_position);
                 }
-            } else if (lane < tile_rows) {
-                const uint32_t n = tile * tile_rows + lane;
+            } else if (r < tile_rows) {
+                const size_t n = (size_t)row * p.N + tile * tile_rows + r;
                 // in place (the decoder's residual stream): one add per element, nothing to wait for
                 if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);
                 else p.y[n] = p.residual ? p.residual[n] + total : total;
             }
+          }
         }
         parity ^= 1u;
-        acc = 0.0f;
     };
     if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
         for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t));
@@ -318,12 +409,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     for (uint32_t s0 = 0; s0 < steps; s0 += D) {
 #pragma unroll
         for (int slot = 0; slot < D; slot++) {
-            Step st;
-            multiply(ring[slot], at_b, st);
-            __builtin_amdgcn_sched_barrier(0);  // the fetch reuses this unit's registers: keep its loads behind their last use
-            fetch(ring[slot]);
-            __builtin_amdgcn_sched_barrier(0);
-            weigh(st);
+            if constexpr (R > 1) {
+                step_rows(ring[slot], at_b);
+            } else {
+                Step st;
+                multiply(ring[slot], at_b, st);
+                __builtin_amdgcn_sched_barrier(0);  // the fetch reuses this unit's registers: keep its loads behind their last use
+                fetch(ring[slot]);
+                __builtin_amdgcn_sched_barrier(0);
+                weigh(st);
+            }
             at_b += NW;
             if (at_b >= nblk) {
                 if (at_tile < walked) tile_end(tile_at(at_tile));
@@ -336,10 +431,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
 
 // ---- the 16-row tile kernel (one activation row, Q4_K)
 // NEURA_HIP_TILE16=0 keeps it out (the vector and the other matrix-core forms then take one row as before), as does a forced
-// NEURA_HIP_MFMA form.  Otherwise it takes every one-row Q4_K product whose matrices end on tile boundaries.
+// NEURA_HIP_MFMA form.  Otherwise it takes every Q4_K product of one row whose matrices end on tile boundaries, and of two
+// to four rows (NEURA_HIP_TILE16_ROWS lowers that) where all their digit planes fit the workgroup's LDS.  From five rows on
+// the MFMAs and the weighing, both paid once a row, cost more than the weights' bytes: the 32-row tiles take those.
+constexpr uint32_t TILE16_MOST_ROWS = 4;
+static uint32_t tile16_row_form(uint32_t rows) { return rows <= 1u ? 1u : (rows <= 2u ? 2u : 4u); }
+
 bool tile16_takes(const GemvArgs &a) {
-    if (a.element != NH_Q4_K || a.rows != 1 || a.K % 256u != 0 || a.K == 0) return false;
+    if (a.element != NH_Q4_K || a.rows < 1 || a.rows > TILE16_MOST_ROWS || a.K % 256u != 0 || a.K == 0) return false;
     if (env_int("NEURA_HIP_TILE16", 1) == 0 || env_int("NEURA_HIP_MFMA", 1) != 1) return false;
+    if (a.rows > 1 && (a.rope || a.rows > (uint32_t)env_int("NEURA_HIP_TILE16_ROWS", (int)TILE16_MOST_ROWS))) return false;
+    if (a.rows > 1 && (env_int("NEURA_HIP_MFMA32", 1) == 2 || env_int("NEURA_HIP_F16_TILES", 1) == 2)) return false;  // another form is forced
     if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
     if (a.N < 16u || a.N % 16u != 0) return false;
     if (a.swiglu) {
@@ -353,29 +455,41 @@ bool tile16_takes(const GemvArgs &a) {
         return false;
     }
     const uint32_t nblk = a.K / 256u;
-    return tile16_lds(nblk, nblk > 32u ? 16u : 8u) <= 160u * 1024u;
+    return tile16_lds(nblk, nblk > 32u ? 16u : 8u, tile16_row_form(a.rows)) <= 160u * 1024u;
 }
 
-template <int NW, int D, int MODE>
+template <int NW, int D, int MODE, int R>
 static hipError_t launch_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
     static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
     return hipGetLastError();
+}
+
+template <int MODE, int R>
+static hipError_t launch_tile16_rows(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
+    switch (waves) {
+    case 4: return launch_tile16_instance<4, 2, MODE, R>(d, p, grid, lds);
+    case 7: return launch_tile16_instance<7, 2, MODE, R>(d, p, grid, lds);
+    case 8: return launch_tile16_instance<8, 2, MODE, R>(d, p, grid, lds);
+    default: return launch_tile16_instance<16, 2, MODE, R>(d, p, grid, lds);
+    }
 }
 
 template <int MODE>
 static hipError_t launch_tile16_mode(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
-    switch (waves) {
-    case 4: return launch_tile16_instance<4, 2, MODE>(d, p, grid, lds);
-    case 7: return launch_tile16_instance<7, 2, MODE>(d, p, grid, lds);
-    case 8: return launch_tile16_instance<8, 2, MODE>(d, p, grid, lds);
-    default: return launch_tile16_instance<16, 2, MODE>(d, p, grid, lds);
+    if constexpr (MODE != TILE16_ROPE) {
+        switch (tile16_row_form(p.rows)) {
+        case 1: break;
+        case 2: return launch_tile16_rows<MODE, 2>(d, p, waves, grid, lds);
+        default: return launch_tile16_rows<MODE, 4>(d, p, waves, grid, lds);
+        }
     }
+    return launch_tile16_rows<MODE, 1>(d, p, waves, grid, lds);
 }
 
 int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
@@ -385,7 +499,7 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
         p.end[s] = a.end[s];
     }
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
-    p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps;
+    p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps, p.rows = a.rows;
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     p.nblk = a.K / 256u;
     p.rope_width = 16;  // the kernel derives a tile's rows from it only where the rotation is folded in
@@ -417,7 +531,7 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     p.row_groups = units;
     const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
     const uint32_t grid = (units + rounds - 1u) / rounds;
-    const size_t lds = tile16_lds(p.nblk, waves);
+    const size_t lds = tile16_lds(p.nblk, waves, tile16_row_form(a.rows));
     profile_mark(d);
     hipError_t launched = a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
                           : a.rope ? launch_tile16_mode<TILE16_ROPE>(d, p, waves, grid, lds)

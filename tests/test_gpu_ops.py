@@ -253,6 +253,38 @@ def test_q4_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K)
     assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
 
 
+@pytest.mark.parametrize("N,K,rows", [(16, 256, 2), (64, 3584, 4), (4608, 3584, 4), (3584, 3584, 3), (4608, 3584, 2), (1040, 768, 4), (48, 2048, 3),
+                                      (272, 8960, 4), (96, 18944, 2), (37888, 3584, 4), (64, 10240, 3), (152064, 3584, 2)])
+def test_q4_k_products_of_a_few_rows_on_16_row_tiles(device, N, K, rows):
+    """Two to four activation rows against Q4_K rows in one pass of the 16-row tiles (every row its own digit planes, the
+    weights unpacked once a step): each row is, bit for bit, what the one-row product gives for it alone, plain, with a
+    residual and with SwiGLU (the decoders' batches run it with the norm folded in); and the whole sits as close to the exact
+    product as the oracle does.  A non-finite number stays in its own row."""
+    rng = np.random.default_rng(N + K + rows)
+    raw = synth.q4_k_random(rng, N * K)
+    x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-2, 2, (rows, K)))).astype(np.float32)
+    r = rng.standard_normal((rows, N)).astype(np.float32)
+    if N * K <= 4608 * 3584:
+        close(device.gemv(NH_Q4_K, raw, N, K, x), oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8))
+    x[rows - 1, rng.integers(0, K, 8)] *= 1e3  # with outliers the oracle's own fp32 sums are the looser side: the exact product judges
+    got = device.gemv(NH_Q4_K, raw, N, K, x)
+    if N * K <= 4608 * 3584:
+        plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+        exact = oracle.unpack(NH_Q4_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+        assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 2e-6 * max(1.0, np.abs(exact).max()))
+    with_residual = device.gemv(NH_Q4_K, raw, N, K, x, residual=r)
+    gated = device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True) if N % 32 == 0 else None
+    for row in range(rows):
+        one = x[row : row + 1]
+        assert np.array_equal(got[row : row + 1], device.gemv(NH_Q4_K, raw, N, K, one)), row
+        assert np.array_equal(with_residual[row : row + 1], device.gemv(NH_Q4_K, raw, N, K, one, residual=r[row : row + 1])), row
+        if gated is not None:
+            assert np.array_equal(gated[row : row + 1], device.gemv(NH_Q4_K, raw, N, K, one, swiglu=True)), row
+    x[0, 5] = np.inf
+    spoilt = device.gemv(NH_Q4_K, raw, N, K, x)
+    assert not np.isfinite(spoilt[0]).any() and np.array_equal(spoilt[1:], got[1:])
+
+
 def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device, monkeypatch):
     monkeypatch.setenv("NEURA_HIP_MFMA", "2")
     rng = np.random.default_rng(2)
