@@ -243,6 +243,122 @@ __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restr
 
 constexpr size_t GEMM_Q4K_LDS = sizeof(_Float16) * (2 * GT * GS + 2 * GT * GS + 2 * GT * 8) + sizeof(uint32_t) * 2 * GT;
 
+// What the multiplier waves of a super-block wide product do (waves 0..3 of the workgroup; the stagers fill As, Bs, mns and dds).
+// FLOORS: the weights have minimums (Q4_K, Q5_K), taken off with one more MFMA per four steps over (minimum, activation sum)
+// pairs; SCALE is what the stagers divided the weights' operand by.  Four steps share one (d, dmin) in dds[(step / 4) & 1].
+template <bool FLOORS>
+__device__ __forceinline__ void gemm_multiply(const GemmQ4Params &p, _Float16 (*As)[GT][GS], _Float16 (*Bs)[GT][GS], _Float16 (*mns)[GT][8], uint32_t (*dds)[GT],
+                                              const uint32_t wave, const uint32_t lane, const uint32_t n0, const uint32_t m0, const uint32_t steps, const float unscale_weights) {
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    // ---------------------------------------------------------------------- multipliers
+    // wave (wm, wn) owns rows 64 wm.. of A' and weight rows 64 wn..
+    const uint32_t wm = wave >> 1, wn = wave & 1u, l32 = lane & 31u, part = lane >> 5;
+    const uint32_t nsb = p.K / 256u;
+    const _Float16 *sums[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) sums[i] = p.S + (size_t)min(m0 + 64u * wm + 32u * i + l32, p.rows - 1u) * nsb * 16u + 8u * part;
+    (void)sums;
+
+    f32x16 acc[2][2], tmp[2][2], zero;
+#pragma unroll
+    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = zero, tmp[i][j] = zero;
+
+    for (uint32_t first = 0; first < steps; first += 4) {
+        const uint32_t sbuf = (first >> 2) & 1u;
+        u32x4 sraw[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
+        if (FLOORS) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(first >> 2) * 16u);  // wanted at the end of the super-block
+        }
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t buf = g & 1u;
+            __syncthreads();  // the step is staged
+            // ---- 64 x 64 x 64 per wave; the operands of the next 16 k are on their way while the matrix cores walk these
+            half8_t a[2][2], b[2][2];
+            auto operands = [&](int kk) {
+#pragma unroll
+                for (int i = 0; i < 2; i++) a[kk & 1][i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
+#pragma unroll
+                for (int j = 0; j < 2; j++) b[kk & 1][j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
+            };
+            operands(0);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                if (kk < 3) operands(kk + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        tmp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk & 1][i], b[kk & 1][j], (g == 0 && kk == 0) ? zero : tmp[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // ---- the super-block is complete: weigh by d, then take the minimums off
+        float dscale[2], mscale[2];
+        half8_t b2[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const half2_t dd = __builtin_bit_cast(half2_t, dds[sbuf][64u * wn + 32u * j + l32]);
+            dscale[j] = (float)dd.x * unscale_weights;
+            mscale[j] = (float)dd.y * -64.0f;  // the sums were packed / 64
+            if (FLOORS) {
+                b2[j] = *reinterpret_cast<const half8_t *>(mns[sbuf][64u * wn + 32u * j + l32]);
+                if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11 against the residues * 2^11
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const half8_t a2 = __builtin_bit_cast(half8_t, sraw[i]);  // k 0..7: the sums; k 8..15: their residues
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(dscale[j], tmp[i][j][e], acc[i][j][e]);
+                if (FLOORS) {
+                    const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[j], zero, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(mscale[j], mins[e], acc[i][j][e]);
+                }
+            }
+        }
+    }
+    // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t n = n0 + 64u * wn + 32u * j + l32;
+            if (n >= p.N) continue;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t row = m0 + 64u * wm + 32u * i + 8u * q + 4u * part;  // first of four rows of A'
+                if (p.split) {
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const uint32_t m = (row >> 1) + e;
+                        if (m >= p.M) continue;
+                        float value = fmaf(acc[i][j][4 * q + 2 * e + 1], 0.00048828125f, acc[i][j][4 * q + 2 * e]) * p.unscale[m];
+                        const size_t at = (size_t)m * p.ldy + n;
+                        p.Y[at] = p.residual ? p.residual[at] + value : value;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t m = row + e;
+                        if (m >= p.M) continue;
+                        const size_t at = (size_t)m * p.ldy + n;
+                        p.Y[at] = p.residual ? p.residual[at] + acc[i][j][4 * q + e] : acc[i][j][4 * q + e];
+                    }
+                }
+            }
+        }
+}
+
 // The eight waves of a workgroup split the work by kind.  Waves 4..7 (the stagers) fetch raw blocks and packed
 // activations four steps ahead into registers, unpack step s + 1 into LDS; waves 0..3 (the multipliers) do nothing
 // but read operands and drive the matrix cores over step s.  One stager and one multiplier share each SIMD, so
@@ -341,106 +457,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
         return;
     }
 
-    // ---------------------------------------------------------------------- multipliers
-    // wave (wm, wn) owns rows 64 wm.. of A' and weight rows 64 wn..
-    const uint32_t wm = wave >> 1, wn = wave & 1u, l32 = lane & 31u, part = lane >> 5;
-    const uint32_t nsb = p.K / 256u;
-    const _Float16 *sums[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) sums[i] = p.S + (size_t)min(m0 + 64u * wm + 32u * i + l32, p.rows - 1u) * nsb * 16u + 8u * part;
-
-    f32x16 acc[2][2], tmp[2][2], zero;
-#pragma unroll
-    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = zero, tmp[i][j] = zero;
-
-    for (uint32_t first = 0; first < steps; first += 4) {
-        const uint32_t sbuf = (first >> 2) & 1u;
-        u32x4 sraw[2];
-#pragma unroll
-        for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(first >> 2) * 16u);  // wanted at the end of the super-block
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const uint32_t buf = g & 1u;
-            __syncthreads();  // the step is staged
-            // ---- 64 x 64 x 64 per wave; the operands of the next 16 k are on their way while the matrix cores walk these
-            half8_t a[2][2], b[2][2];
-            auto operands = [&](int kk) {
-#pragma unroll
-                for (int i = 0; i < 2; i++) a[kk & 1][i] = *reinterpret_cast<const half8_t *>(&As[buf][64u * wm + 32u * i + l32][16u * kk + 8u * part]);
-#pragma unroll
-                for (int j = 0; j < 2; j++) b[kk & 1][j] = *reinterpret_cast<const half8_t *>(&Bs[buf][64u * wn + 32u * j + l32][16u * kk + 8u * part]);
-            };
-            operands(0);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                if (kk < 3) operands(kk + 1);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        tmp[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[kk & 1][i], b[kk & 1][j], (g == 0 && kk == 0) ? zero : tmp[i][j], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        // ---- the super-block is complete: weigh by d, then take the minimums off
-        float dscale[2], mscale[2];
-        half8_t b2[2];
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const half2_t dd = __builtin_bit_cast(half2_t, dds[sbuf][64u * wn + 32u * j + l32]);
-            dscale[j] = (float)dd.x * 16384.0f;  // the weights were staged * 2^-14
-            mscale[j] = (float)dd.y * -64.0f;    // the sums were packed / 64
-            b2[j] = *reinterpret_cast<const half8_t *>(mns[sbuf][64u * wn + 32u * j + l32]);
-            if (part) b2[j] = b2[j] * (_Float16)0.00048828125f;  // k 8..15: the minimums * 2^-11 against the residues * 2^11
-        }
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const half8_t a2 = __builtin_bit_cast(half8_t, sraw[i]);  // k 0..7: the sums; k 8..15: their residues
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b2[j], zero, 0, 0, 0);
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(dscale[j], tmp[i][j][e], acc[i][j][e]);
-#pragma unroll
-                for (int e = 0; e < 16; e++) acc[i][j][e] = fmaf(mscale[j], mins[e], acc[i][j][e]);
-            }
-        }
-    }
-    // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const uint32_t n = n0 + 64u * wn + 32u * j + l32;
-            if (n >= p.N) continue;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const uint32_t row = m0 + 64u * wm + 32u * i + 8u * q + 4u * part;  // first of four rows of A'
-                if (p.split) {
-#pragma unroll
-                    for (int e = 0; e < 2; e++) {
-                        const uint32_t m = (row >> 1) + e;
-                        if (m >= p.M) continue;
-                        float value = fmaf(acc[i][j][4 * q + 2 * e + 1], 0.00048828125f, acc[i][j][4 * q + 2 * e]) * p.unscale[m];
-                        const size_t at = (size_t)m * p.ldy + n;
-                        p.Y[at] = p.residual ? p.residual[at] + value : value;
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const uint32_t m = row + e;
-                        if (m >= p.M) continue;
-                        const size_t at = (size_t)m * p.ldy + n;
-                        p.Y[at] = p.residual ? p.residual[at] + acc[i][j][4 * q + e] : acc[i][j][4 * q + e];
-                    }
-                }
-            }
-        }
+    gemm_multiply<true>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 16384.0f);  // the weights were staged * 2^-14
 }
 
 // ------------------------------------------------------------------- Q8_0 on MFMA --------
@@ -618,6 +635,133 @@ __global__ __launch_bounds__(512) void gemm_q8_0_mfma_kernel(GemmQ4Params p) {
         }
 }
 
+// ------------------------------------------------------------------- Q6_K on MFMA --------
+//
+// A Q6_K weight is d * sc * (q - 32) with q of six bits and sc a signed byte a 16 weights (crates/neura-precision/src/ggml.rs,
+// the Q6_K reader): sc * (q - 32) reaches +-4064, past the integers a half holds exactly.  The byte splits as
+// sc = 16 * (sc >> 4) + (sc & 15), and (q - 32) * (sc & 15) (below 512) and 16 * (q - 32) * (sc >> 4) (a nine-bit integer times
+// 16) are both exact halves: the weights enter as two operand planes and the matrix cores add the two products in fp32, so
+// tmp holds exactly sum a * sc * (q - 32) however the scales fall.  A step is 32 k: its 64 operand columns are plane one
+// then plane two of those 32 weights, against the step's 32 activations written twice; four steps (half a super-block)
+// are weighed by d together.  The same tiles, packed activation rows, division of the waves and multipliers as the Q4_K
+// kernel; there are no minimums.  Blocks are 210 bytes and start on any half word: a stager reads each 16-byte run it
+// needs as the four aligned words below it and the half word above, and shifts the five into place.
+struct Q6Raw {
+    u32x4 ql[4], qh[2], sc;          // this thread's runs of the low nibbles, of the high bit pairs, and the 16 scales
+    uint32_t qle[4], qhe[2], sce, d;  // the half word above each run; d
+};
+
+__global__ __launch_bounds__(512) void gemm_q6k_mfma_kernel(GemmQ4Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);
+    _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);
+    _Float16(*mns)[GT][8] = reinterpret_cast<_Float16(*)[GT][8]>(gemm_lds + sizeof(_Float16) * 4 * GT * GS);  // unused: no minimums
+    uint32_t(*dds)[GT] = reinterpret_cast<uint32_t(*)[GT]>(gemm_lds + sizeof(_Float16) * (4 * GT * GS + 2 * GT * 8));
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
+    const uint32_t steps = p.K / 32u;  // a multiple of 8: K is whole super-blocks
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    typedef const __attribute__((address_space(1))) uint16_t *global_half_word;
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------ stagers
+        // one row of each tile, one half (16 k: one scale) of the step
+        const uint32_t tid = threadIdx.x - 256u;
+        const uint32_t srow = tid >> 1, sh = tid & 1u;
+        const uint32_t column = min(n0 + srow, p.N - 1u);
+        const uint8_t *wrow = column < p.end0   ? p.W + (size_t)column * p.row_bytes
+                              : column < p.end1 ? p.W1 + (size_t)(column - p.end0) * p.row_bytes
+                                                : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
+        const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 16u * sh;
+        const uint32_t nsb = steps >> 3;
+        // 16 bytes from `at` (any half word) as the aligned 16 below and the half word at + 14
+        auto run = [&](const uint8_t *at, u32x4 &low, uint32_t &above) {
+            low = *(global_uint4)((uintptr_t)at & ~(uintptr_t)3);
+            above = *(global_half_word)(uintptr_t)(at + 14u);
+        };
+        auto fetch = [&](Q6Raw &raw, uint32_t sb) {
+            const uint8_t *block = wrow + (size_t)min(sb, nsb - 1u) * 210u;  // past the end the last super-block again, dropped
+#pragma unroll
+            for (int r = 0; r < 4; r++) run(block + 64u * (r >> 1) + 32u * (r & 1) + 16u * sh, raw.ql[r], raw.qle[r]);
+#pragma unroll
+            for (int n = 0; n < 2; n++) run(block + 128u + 32u * n + 16u * sh, raw.qh[n], raw.qhe[n]);
+            run(block + 192u, raw.sc, raw.sce);
+            raw.d = *(global_half_word)(uintptr_t)(block + 208u);
+        };
+        // the run as it lies: nothing to do on a word boundary, else every word takes its upper half from the next
+        auto placed = [](const u32x4 &low, uint32_t above, uint32_t shift) -> u32x4 {
+            return u32x4{__builtin_amdgcn_alignbit(low.y, low.x, shift), __builtin_amdgcn_alignbit(low.z, low.y, shift),
+                         __builtin_amdgcn_alignbit(low.w, low.z, shift), __builtin_amdgcn_alignbit(above, low.w, shift)};
+        };
+        u32x4 av[4][2];  // activations by slot = step % 4
+        auto fetch_activations = [&](int slot, uint32_t step) {
+            const _Float16 *at = arow + (size_t)min(step, steps - 1u) * 32u;
+#pragma unroll
+            for (int i = 0; i < 2; i++) av[slot][i] = *(global_uint4)(uintptr_t)(at + 8 * i);
+        };
+        const half2_t bias = {(_Float16)1056.0f, (_Float16)1056.0f};  // 0x6400 | q is the half 1024 + q; the weight is q - 32
+        Q6Raw raws[2];
+        fetch(raws[0], 0);
+        __builtin_amdgcn_sched_barrier(0);  // the first super-block goes out first: the loop waits for the oldest loads only
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) fetch_activations(slot, slot);
+        fetch(raws[1], 1);
+        __builtin_amdgcn_sched_barrier(0);
+        auto super_block = [&](Q6Raw &raw, const uint32_t sb) {
+            const uint32_t shift = (uint32_t)((uintptr_t)(wrow + (size_t)sb * 210u) & 2u) * 8u;  // 0 or 16: where the block starts in its word
+            const u32x4 scales = placed(raw.sc, raw.sce, shift);
+            const uint32_t scale_words[4] = {scales.x, scales.y, scales.z, scales.w};
+            u32x4 high_pairs = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const uint32_t buf = s & 1u, sbuf = (s >> 2) & 1u;  // steps are whole super-blocks: step 8 sb + s has parity s & 1
+                const int n = s >> 2, quarter = s & 3;
+                if (quarter == 0) high_pairs = placed(raw.qh[n], raw.qhe[n], shift);
+                // group 2 s + sh of the super-block: scale byte 2 (s & 1) + sh of word s / 2
+                const int sc = __builtin_amdgcn_sbfe((int)scale_words[s >> 1], 16u * (s & 1) + 8u * sh, 8u);
+                const _Float16 fine = (_Float16)(float)(sc & 15), coarse = (_Float16)(float)(16 * (sc >> 4));
+                const half2_t fine2 = {fine, fine}, coarse2 = {coarse, coarse};
+                const u32x4 nibbles = placed(raw.ql[2 * n + (quarter & 1)], raw.qle[2 * n + (quarter & 1)], shift);
+                const uint32_t nibble_words[4] = {nibbles.x, nibbles.y, nibbles.z, nibbles.w};
+                const uint32_t pair_words[4] = {high_pairs.x, high_pairs.y, high_pairs.z, high_pairs.w};
+                uint32_t one[8], two[8];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const uint32_t low4 = (quarter >= 2 ? nibble_words[w] >> 4 : nibble_words[w]) & 0x0f0f0f0fu;
+                    const uint32_t q4 = low4 | (((pair_words[w] >> (2 * quarter)) & 0x03030303u) << 4);  // four weights' six bits, one a byte
+                    // element order inside a word: 0, 2 then 1, 3, as the activations were packed
+                    const half2_t even = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, q4, 0x0c020c00u) | 0x64006400u) - bias;
+                    const half2_t odd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, q4, 0x0c030c01u) | 0x64006400u) - bias;
+                    one[2 * w] = __builtin_bit_cast(uint32_t, even * fine2), one[2 * w + 1] = __builtin_bit_cast(uint32_t, odd * fine2);
+                    two[2 * w] = __builtin_bit_cast(uint32_t, even * coarse2), two[2 * w + 1] = __builtin_bit_cast(uint32_t, odd * coarse2);
+                }
+                u32x4 *first = reinterpret_cast<u32x4 *>(&Bs[buf][srow][16u * sh]), *second = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u + 16u * sh]);
+                first[0] = u32x4{one[0], one[1], one[2], one[3]};
+                first[1] = u32x4{one[4], one[5], one[6], one[7]};
+                second[0] = u32x4{two[0], two[1], two[2], two[3]};
+                second[1] = u32x4{two[4], two[5], two[6], two[7]};
+                if (quarter == 0 && sh == 0) dds[sbuf][srow] = raw.d;  // (d, no dmin) of these four steps
+                u32x4 *once = reinterpret_cast<u32x4 *>(&As[buf][srow][16u * sh]), *again = reinterpret_cast<u32x4 *>(&As[buf][srow][32u + 16u * sh]);
+#pragma unroll
+                for (int i = 0; i < 2; i++) once[i] = av[s & 3][i], again[i] = av[s & 3][i];
+                fetch_activations(s & 3, 8u * sb + (uint32_t)s + 4u);
+                if (s == 7) fetch(raw, sb + 2u);  // these registers are free: the super-block after the next
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();  // step is staged; the multipliers are done with the step before it
+            }
+        };
+        uint32_t sb = 0;
+        for (; sb + 2u <= nsb; sb += 2u) {
+            super_block(raws[0], sb);
+            super_block(raws[1], sb + 1u);
+        }
+        if (sb < nsb) super_block(raws[0], sb);
+        return;
+    }
+    gemm_multiply<false>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 1.0f);
+}
+
 // bytes of device scratch a Q4_K wide product over M activation rows of K numbers packs into
 size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows) {
     const size_t rows = half_rows ? M : (size_t)2 * M;
@@ -666,27 +810,29 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
     if (!sized) {
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q8_LDS));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
     if (a.element == NH_Q8_0) hipLaunchKernelGGL(gemm_q8_0_mfma_kernel, grid, dim3(512), GEMM_Q8_LDS, d->stream, p);
+    else if (a.element == NH_Q6_K) hipLaunchKernelGGL(gemm_q6k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
 
-// the matrix-core forms take Q4_K rows of whole super-blocks and Q8_0 rows of whole pairs of blocks, read from 16-byte
-// aligned addresses (a Q8_0 matrix from a 4-byte one; its rows may start on any half word)
+// the matrix-core forms take Q4_K and Q6_K rows of whole super-blocks and Q8_0 rows of whole pairs of blocks, read from 16-byte
+// aligned addresses (a Q8_0 or Q6_K matrix from a 4-byte one; its rows may start on any half word)
 static bool mfma_takes(int32_t element, uint32_t K, const void *X, const void *W) {
     const char *held = getenv("NEURA_HIP_GEMM_MFMA");
     const bool wanted = !(held && held[0] == '0');
-    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q8_0 ? 3u : 15u)) == 0;
-    return wanted && aligned && K > 0 && ((element == NH_Q4_K && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
+    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q4_K ? 15u : 3u)) == 0;
+    return wanted && aligned && K > 0 && (((element == NH_Q4_K || element == NH_Q6_K) && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
 }
 
 bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1) {
     if (!mfma_takes(element, K, X, W0)) return false;
-    const uintptr_t loose = element == NH_Q8_0 ? 3u : 15u;
+    const uintptr_t loose = element == NH_Q4_K ? 15u : 3u;
     if (W1 && (((uintptr_t)W1 & loose) || end0 % GT)) return false;
     if (W2 && (((uintptr_t)W2 & loose) || end1 % GT || !W1)) return false;
     return true;
