@@ -363,7 +363,13 @@ __device__ __forceinline__ void gemm_multiply(const GemmQ4Params &p, _Float16 (*
 // activations four steps ahead into registers, unpack step s + 1 into LDS; waves 0..3 (the multipliers) do nothing
 // but read operands and drive the matrix cores over step s.  One stager and one multiplier share each SIMD, so
 // unpacking and memory latency hide behind the MFMAs instead of taking turns with them.
-__global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
+//
+// FIFTH: Q5_K.  The header is Q4_K's; behind it come 32 bytes of fifth bits (bit 2g of byte l belongs to weight l of group g's
+// low half, bit 2g + 1 to weight 32 + l) and then the nibbles.  A code of five bits times a scale of six stays below 2048, so
+// the operand is as exact as Q4_K's: the fifth bit is set beside the nibble before the one multiplication.
+template <bool FIFTH>
+__device__ __forceinline__ void gemm_q45k_mfma(const GemmQ4Params &p) {
+    constexpr uint32_t BLOCK = FIFTH ? 176u : 144u, NIBBLES = FIFTH ? 48u : 16u;
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);                                           // [2]
     _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);          // [2]
@@ -387,19 +393,23 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
                                                 : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
         const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
         u32x4 ahead, qs[4], av[4][4];  // the next super-block's header; groups and activations by slot = step % 4
+        u32x4 fifth_ahead = {0u, 0u, 0u, 0u};  // Q5_K: the fifth bits of this thread's sixteen columns, next super-block
         const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
         ahead = *(global_uint4)(uintptr_t)wrow;
+        if (FIFTH) fifth_ahead = *(global_uint4)(uintptr_t)(wrow + 16u + 16u * sh);
 #pragma unroll
         for (int g = 0; g < 4; g++) {  // steps 0..3 = super-block 0
-            qs[g] = *(global_uint4)(uintptr_t)(wrow + 16u + 32u * g + 16u * sh);
+            qs[g] = *(global_uint4)(uintptr_t)(wrow + NIBBLES + 32u * g + 16u * sh);
 #pragma unroll
             for (int i = 0; i < 4; i++) av[g][i] = *(global_uint4)(uintptr_t)(arow + (size_t)g * 64u + 8 * i);
             __builtin_amdgcn_sched_barrier(0);  // slot 0 goes out first: the loop waits for the oldest slot only
         }
         for (uint32_t first = 0; first < steps; first += 4) {
-            const u32x4 hdr = ahead;
+            const u32x4 hdr = ahead, fifth = fifth_ahead;
             const uint32_t next = min((first >> 2) + 1u, (steps >> 2) - 1u);
-            ahead = *(global_uint4)(uintptr_t)(wrow + (size_t)next * 144u);
+            ahead = *(global_uint4)(uintptr_t)(wrow + (size_t)next * BLOCK);
+            if (FIFTH) fifth_ahead = *(global_uint4)(uintptr_t)(wrow + (size_t)next * BLOCK + 16u + 16u * sh);
+            const uint32_t fifth_words[4] = {fifth.x, fifth.y, fifth.z, fifth.w};
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const uint32_t buf = g & 1u, sbuf = (first >> 2) & 1u;
@@ -416,10 +426,17 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
                 for (int w = 0; w < 4; w++) {
                     const uint32_t even = words[w], odd = words[w] >> 8;
                     // element order inside a word: 0, 2 then 1, 3 (the byte lanes); the activations were packed in the same order
-                    low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
-                    low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
-                    high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
-                    high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+                    uint32_t low_even = even & 0x000f000fu, low_odd = odd & 0x000f000fu, high_even = even & 0x00f000f0u, high_odd = odd & 0x00f000f0u;
+                    if (FIFTH) {
+                        // bit 2g of a byte to bit 4 of its lane (beside the low nibble), bit 2g + 1 to bit 8 (beside the high nibble's four)
+                        const uint32_t bits = fifth_words[w] >> (2 * g);
+                        low_even |= (bits & 0x00010001u) << 4, low_odd |= ((bits >> 8) & 0x00010001u) << 4;
+                        high_even |= (bits & 0x00020002u) << 7, high_odd |= ((bits >> 8) & 0x00020002u) << 7;
+                    }
+                    low[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, low_even) * low_scale);
+                    low[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, low_odd) * low_scale);
+                    high[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, high_even) * high_scale);
+                    high[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, high_odd) * high_scale);
                 }
                 u32x4 *blow = reinterpret_cast<u32x4 *>(&Bs[buf][srow][16u * sh]), *bhigh = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u + 16u * sh]);
                 blow[0] = u32x4{low[0], low[1], low[2], low[3]};
@@ -444,8 +461,8 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
                 // the slot is free: the same group of the next super-block goes out.  Past the end the last super-block is
                 // fetched again and dropped: with the same loads in every round the waits count exactly how many are newer
                 {
-                    const uint8_t *block = wrow + (size_t)next * 144u;
-                    qs[g] = *(global_uint4)(uintptr_t)(block + 16u + 32u * g + 16u * sh);
+                    const uint8_t *block = wrow + (size_t)next * BLOCK;
+                    qs[g] = *(global_uint4)(uintptr_t)(block + NIBBLES + 32u * g + 16u * sh);
                     const _Float16 *at = arow + (size_t)(4u * next + g) * 64u;
 #pragma unroll
                     for (int i = 0; i < 4; i++) av[g][i] = *(global_uint4)(uintptr_t)(at + 8 * i);
@@ -459,6 +476,9 @@ __global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
 
     gemm_multiply<true>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 16384.0f);  // the weights were staged * 2^-14
 }
+
+__global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) { gemm_q45k_mfma<false>(p); }
+__global__ __launch_bounds__(512) void gemm_q5k_mfma_kernel(GemmQ4Params p) { gemm_q45k_mfma<true>(p); }
 
 // ------------------------------------------------------------------- Q8_0 on MFMA --------
 //
@@ -811,11 +831,13 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q8_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q5k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
     if (a.element == NH_Q8_0) hipLaunchKernelGGL(gemm_q8_0_mfma_kernel, grid, dim3(512), GEMM_Q8_LDS, d->stream, p);
     else if (a.element == NH_Q6_K) hipLaunchKernelGGL(gemm_q6k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
+    else if (a.element == NH_Q5_K) hipLaunchKernelGGL(gemm_q5k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
@@ -826,13 +848,14 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
 static bool mfma_takes(int32_t element, uint32_t K, const void *X, const void *W) {
     const char *held = getenv("NEURA_HIP_GEMM_MFMA");
     const bool wanted = !(held && held[0] == '0');
-    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q4_K ? 15u : 3u)) == 0;
-    return wanted && aligned && K > 0 && (((element == NH_Q4_K || element == NH_Q6_K) && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
+    const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q4_K || element == NH_Q5_K ? 15u : 3u)) == 0;
+    return wanted && aligned && K > 0 &&
+           (((element == NH_Q4_K || element == NH_Q5_K || element == NH_Q6_K) && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
 }
 
 bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1) {
     if (!mfma_takes(element, K, X, W0)) return false;
-    const uintptr_t loose = element == NH_Q4_K ? 15u : 3u;
+    const uintptr_t loose = element == NH_Q4_K || element == NH_Q5_K ? 15u : 3u;
     if (W1 && (((uintptr_t)W1 & loose) || end0 % GT)) return false;
     if (W2 && (((uintptr_t)W2 & loose) || end1 % GT || !W1)) return false;
     return true;

@@ -387,9 +387,10 @@ def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
 
 
 @pytest.mark.parametrize("element,M,N,K,half", [(NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q4_K, 70, 130, 512, True),
-                                                (NH_Q4_K, 33, 64, 256, False), (NH_Q6_K, 70, 130, 512, True), (NH_Q6_K, 33, 64, 256, False)])
+                                                (NH_Q4_K, 33, 64, 256, False), (NH_Q6_K, 70, 130, 512, True), (NH_Q6_K, 33, 64, 256, False),
+                                                (NH_Q5_K, 70, 130, 512, False)])
 def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N, K, half):
-    """NEURA_HIP_GEMM_MFMA=0 keeps Q8_0, Q4_K and Q6_K wide products on the tiled vector kernel that serves the shapes the matrix
+    """NEURA_HIP_GEMM_MFMA=0 keeps Q8_0, Q4_K, Q5_K and Q6_K wide products on the tiled vector kernel that serves the shapes the matrix
     cores do not take (rows that are not whole steps, unaligned operands)."""
     monkeypatch.setenv("NEURA_HIP_GEMM_MFMA", "0")
     rng = np.random.default_rng(M + N + K)
@@ -398,26 +399,34 @@ def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N,
     close(device.gemm(element, raw, N, K, X), oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8))
 
 
+@pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K])
 @pytest.mark.parametrize("M,N,K,half", [(70, 130, 512, False), (40, 64, 3584, True), (512, 256, 1280, True), (33, 200, 256, False),
                                         (130, 128, 768, True), (64, 256, 18944, False), (512, 512, 3584, False)])
-def test_q6_k_wide_product_on_the_matrix_cores(device, M, N, K, half):
-    """Q6_K rows as two exact half planes on the matrix cores ((q - 32) * (sc & 15) and 16 * (q - 32) * (sc >> 4)): against
-    the oracle at the wide product's bar and against the exact product far inside it, for scales at both ends of a signed
-    byte, blocks that start on either half of a word (210-byte blocks: every other one does), ragged tiles, half and fp32
-    activations, and a residual."""
-    rng = np.random.default_rng(M + N + K)
-    raw = np.array(synth.RANDOM[NH_Q6_K](rng, N * K), dtype=np.uint8).reshape(-1, 210)
-    hard = rng.random(raw.shape[0]) < 0.25  # a quarter of the blocks: scales from the ends and the seams of the split
-    raw[hard, 192:208] = rng.choice(np.array([-128, 127, -1, 15, 16, -16, -17, 0], np.int8).view(np.uint8), (int(hard.sum()), 16))
+def test_q6_k_and_q5_k_wide_products_on_the_matrix_cores(device, element, M, N, K, half):
+    """Q6_K rows as two exact half planes on the matrix cores ((q - 32) * (sc & 15) and 16 * (q - 32) * (sc >> 4)), Q5_K rows
+    as Q4_K's with the fifth bit beside the nibble: against the oracle at the wide product's bar and against the exact
+    product far inside it -- for Q6_K scales at both ends of a signed byte and at the seams of the split, blocks that start
+    on either half of a word (210-byte blocks: every other one does); for Q5_K scales, minimums and codes at their largest;
+    ragged tiles, half and fp32 activations, and a residual."""
+    rng = np.random.default_rng(M + N + K + element)
+    if element == NH_Q6_K:
+        raw = np.array(synth.RANDOM[NH_Q6_K](rng, N * K), dtype=np.uint8).reshape(-1, 210)
+        hard = rng.random(raw.shape[0]) < 0.25
+        raw[hard, 192:208] = rng.choice(np.array([-128, 127, -1, 15, 16, -16, -17, 0], np.int8).view(np.uint8), (int(hard.sum()), 16))
+    else:
+        raw = np.array(synth.RANDOM[NH_Q5_K](rng, N * K), dtype=np.uint8).reshape(-1, 176)
+        hard = rng.random(raw.shape[0]) < 0.25
+        raw[hard, 4:16] = 0xFF   # every scale and minimum 63
+        raw[hard, 16:176] = 0xFF  # every code 31
     raw = raw.reshape(-1)
     X = rng.standard_normal((M, K)).astype(np.float16 if half else np.float32)
-    want = oracle.gemm(NH_Q6_K, raw, N, K, X.astype(np.float32), threads=8)
-    got = device.gemm(NH_Q6_K, raw, N, K, X)
+    want = oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8)
+    got = device.gemm(element, raw, N, K, X)
     close(got, want)
-    exact = X.astype(np.float64) @ oracle.unpack(NH_Q6_K, raw, N * K).reshape(N, K).astype(np.float64).T
+    exact = X.astype(np.float64) @ oracle.unpack(element, raw, N * K).reshape(N, K).astype(np.float64).T
     assert np.abs(got - exact).max() <= max(4 * np.abs(want - exact).max(), 2e-6 * max(1.0, np.abs(exact).max()))
     r = rng.standard_normal((M, N)).astype(np.float32)
-    close(device.gemm(NH_Q6_K, raw, N, K, X, residual=r), want + r)
+    close(device.gemm(element, raw, N, K, X, residual=r), want + r)
 
 
 def test_q8_0_wide_product_of_the_small_decoder_s_shapes(device):
