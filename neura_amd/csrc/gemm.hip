@@ -782,6 +782,128 @@ __global__ __launch_bounds__(512) void gemm_q6k_mfma_kernel(GemmQ4Params p) {
     gemm_multiply<false>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 1.0f);
 }
 
+// ------------------------------------------------------------------- Q3_K on MFMA --------
+//
+// A Q3_K weight is d * (sc - 32) * c with c in -4..3 (two bits less 4 unless the third bit is set) and sc of six bits a 16
+// weights (crates/neura-precision/src/ggml.rs:224-229, 291-306): (sc - 32) * c stays within +-128 and is an exact half, so the
+// weights are one operand plane, a step is 64 k as in the Q4_K kernel (a stager's 32 weights are two scale groups), a
+// super-block's four steps are weighed by d together, and there are no minimums.  Blocks are 110 bytes and start on any
+// half word; they are read as the Q6_K kernel reads its own.
+struct Q3Raw {
+    u32x4 hm[2], qs[4], sc;           // the third bits of the 32 columns, the bit pairs of both halves, bytes 94..109 (scales, d)
+    uint32_t hme[2], qse[4], sce;     // the half word above each run
+};
+
+__global__ __launch_bounds__(512) void gemm_q3k_mfma_kernel(GemmQ4Params p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);
+    _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);
+    _Float16(*mns)[GT][8] = reinterpret_cast<_Float16(*)[GT][8]>(gemm_lds + sizeof(_Float16) * 4 * GT * GS);  // unused: no minimums
+    uint32_t(*dds)[GT] = reinterpret_cast<uint32_t(*)[GT]>(gemm_lds + sizeof(_Float16) * (4 * GT * GS + 2 * GT * 8));
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
+    const uint32_t steps = p.K / 64u;  // a multiple of 4: K is whole super-blocks
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    typedef const __attribute__((address_space(1))) uint16_t *global_half_word;
+
+    if (wave >= 4) {
+        // ------------------------------------------------------------------ stagers
+        // one row of each tile, one half (32 k: two scales) of the step
+        const uint32_t tid = threadIdx.x - 256u;
+        const uint32_t srow = tid >> 1, sh = tid & 1u;
+        const uint32_t column = min(n0 + srow, p.N - 1u);
+        const uint8_t *wrow = column < p.end0   ? p.W + (size_t)column * p.row_bytes
+                              : column < p.end1 ? p.W1 + (size_t)(column - p.end0) * p.row_bytes
+                                                : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
+        const _Float16 *arow = p.A + (size_t)min(m0 + srow, p.rows - 1u) * p.K + 32u * sh;
+        const uint32_t nsb = steps >> 2;
+        auto run = [&](const uint8_t *at, u32x4 &low, uint32_t &above) {
+            low = *(global_uint4)((uintptr_t)at & ~(uintptr_t)3);
+            above = *(global_half_word)(uintptr_t)(at + 14u);
+        };
+        auto fetch = [&](Q3Raw &raw, uint32_t sb) {
+            const uint8_t *block = wrow + (size_t)min(sb, nsb - 1u) * 110u;  // past the end the last super-block again, dropped
+#pragma unroll
+            for (int r = 0; r < 2; r++) run(block + 16u * r, raw.hm[r], raw.hme[r]);
+#pragma unroll
+            for (int r = 0; r < 4; r++) run(block + 32u + 16u * r, raw.qs[r], raw.qse[r]);
+            run(block + 94u, raw.sc, raw.sce);
+        };
+        auto placed = [](const u32x4 &low, uint32_t above, uint32_t shift) -> u32x4 {
+            return u32x4{__builtin_amdgcn_alignbit(low.y, low.x, shift), __builtin_amdgcn_alignbit(low.z, low.y, shift),
+                         __builtin_amdgcn_alignbit(low.w, low.z, shift), __builtin_amdgcn_alignbit(above, low.w, shift)};
+        };
+        u32x4 av[4][4];  // activations by slot = step % 4
+        auto fetch_activations = [&](int slot, uint32_t step) {
+            const _Float16 *at = arow + (size_t)min(step, steps - 1u) * 64u;
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[slot][i] = *(global_uint4)(uintptr_t)(at + 8 * i);
+        };
+        const half2_t scale_bias = {(_Float16)1056.0f, (_Float16)1056.0f};  // 0x6400 | v is the half 1024 + v; a scale is stored 32 too large
+        const half2_t code_bias = {(_Float16)1028.0f, (_Float16)1028.0f};   // and a code 4 too large
+        Q3Raw raws[2];
+        fetch(raws[0], 0);
+        __builtin_amdgcn_sched_barrier(0);  // the first super-block goes out first: the loop waits for the oldest loads only
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) fetch_activations(slot, slot);
+        fetch(raws[1], 1);
+        __builtin_amdgcn_sched_barrier(0);
+        auto super_block = [&](Q3Raw &raw, const uint32_t sb) {
+            const uint32_t shift = (uint32_t)((uintptr_t)(wrow + (size_t)sb * 110u) & 2u) * 8u;  // 0 or 16: where the block starts in its word
+            const u32x4 tail = placed(raw.sc, raw.sce, shift ^ 16u);  // bytes 94..109: this run starts on the other half of a word
+            // bytes 96..107: the scales' nibbles (two words) and their top bit pairs (one)
+            const uint32_t nibble_words[2] = {__builtin_amdgcn_alignbit(tail.y, tail.x, 16u), __builtin_amdgcn_alignbit(tail.z, tail.y, 16u)};
+            const uint32_t tops = __builtin_amdgcn_alignbit(tail.w, tail.z, 16u);
+            const u32x4 third0 = placed(raw.hm[0], raw.hme[0], shift), third1 = placed(raw.hm[1], raw.hme[1], shift);
+            const uint32_t third_words[8] = {third0.x, third0.y, third0.z, third0.w, third1.x, third1.y, third1.z, third1.w};
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const uint32_t buf = g & 1u, sbuf = sb & 1u;
+                const int n = g >> 1;
+                // scales 4 g + 2 sh and the one after: nibble 2 sh + t of word g & 1 (low nibbles for the first eight scales), top
+                // bits from byte 2 sh + t of the third word at 2 g
+                const uint32_t two = (nibble_words[g & 1] >> (16u * sh)) & 0xffffu, top = (tops >> (16u * sh)) & 0xffffu;
+                const uint32_t pair = ((g < 2 ? two : two >> 4) & 0x0f0fu) | (((top >> (2 * g)) & 0x0303u) << 4);
+                const half2_t scales = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, pair, 0x0c010c00u) | 0x64006400u) - scale_bias;
+                const half2_t first_scale = {scales.x, scales.x}, second_scale = {scales.y, scales.y};
+                const u32x4 pairs0 = placed(raw.qs[2 * n], raw.qse[2 * n], shift), pairs1 = placed(raw.qs[2 * n + 1], raw.qse[2 * n + 1], shift);
+                const uint32_t pair_words[8] = {pairs0.x, pairs0.y, pairs0.z, pairs0.w, pairs1.x, pairs1.y, pairs1.z, pairs1.w};
+                const uint32_t j = 2u * (g & 1) + sh;  // which bit pair of a byte, and with 4 n which third bit
+                uint32_t out[16];
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    const uint32_t v = ((pair_words[w] >> (2u * j)) & 0x03030303u) | (((third_words[w] >> (4u * n + j)) & 0x01010101u) << 2);  // code + 4, one a byte
+                    // element order inside a word: 0, 2 then 1, 3, as the activations were packed
+                    const half2_t even = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, v, 0x0c020c00u) | 0x64006400u) - code_bias;
+                    const half2_t odd = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, v, 0x0c030c01u) | 0x64006400u) - code_bias;
+                    const half2_t scale = w < 4 ? first_scale : second_scale;
+                    out[2 * w] = __builtin_bit_cast(uint32_t, even * scale), out[2 * w + 1] = __builtin_bit_cast(uint32_t, odd * scale);
+                }
+                u32x4 *to = reinterpret_cast<u32x4 *>(&Bs[buf][srow][32u * sh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) to[i] = u32x4{out[4 * i], out[4 * i + 1], out[4 * i + 2], out[4 * i + 3]};
+                if (g == 0 && sh == 0) dds[sbuf][srow] = tail.w >> 16;  // (d, no dmin)
+                u32x4 *adst = reinterpret_cast<u32x4 *>(&As[buf][srow][32u * sh]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) adst[i] = av[g][i];
+                fetch_activations(g, 4u * sb + (uint32_t)g + 4u);
+                if (g == 3) fetch(raw, sb + 2u);  // these registers are free: the super-block after the next
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();  // step is staged; the multipliers are done with the step before it
+            }
+        };
+        uint32_t sb = 0;
+        for (; sb + 2u <= nsb; sb += 2u) {
+            super_block(raws[0], sb);
+            super_block(raws[1], sb + 1u);
+        }
+        if (sb < nsb) super_block(raws[0], sb);
+        return;
+    }
+    gemm_multiply<false>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 1.0f);
+}
+
 // bytes of device scratch a Q4_K wide product over M activation rows of K numbers packs into
 size_t gemm_q4k_scratch_bytes(uint32_t M, uint32_t K, bool half_rows) {
     const size_t rows = half_rows ? M : (size_t)2 * M;
@@ -832,25 +954,27 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q8_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q5k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q3k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         sized = true;
     }
     dim3 grid((a.N + GT - 1) / GT, (p.rows + GT - 1) / GT);
     if (a.element == NH_Q8_0) hipLaunchKernelGGL(gemm_q8_0_mfma_kernel, grid, dim3(512), GEMM_Q8_LDS, d->stream, p);
     else if (a.element == NH_Q6_K) hipLaunchKernelGGL(gemm_q6k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else if (a.element == NH_Q5_K) hipLaunchKernelGGL(gemm_q5k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
+    else if (a.element == NH_Q3_K) hipLaunchKernelGGL(gemm_q3k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
 
-// the matrix-core forms take Q4_K and Q6_K rows of whole super-blocks and Q8_0 rows of whole pairs of blocks, read from 16-byte
-// aligned addresses (a Q8_0 or Q6_K matrix from a 4-byte one; its rows may start on any half word)
+// the matrix-core forms take Q4_K, Q5_K, Q6_K and Q3_K rows of whole super-blocks and Q8_0 rows of whole pairs of blocks, read
+// from 16-byte aligned addresses (a Q8_0, Q6_K or Q3_K matrix from a 4-byte one; its rows may start on any half word)
 static bool mfma_takes(int32_t element, uint32_t K, const void *X, const void *W) {
     const char *held = getenv("NEURA_HIP_GEMM_MFMA");
     const bool wanted = !(held && held[0] == '0');
     const bool aligned = ((uintptr_t)X & 15u) == 0 && ((uintptr_t)W & (element == NH_Q4_K || element == NH_Q5_K ? 15u : 3u)) == 0;
     return wanted && aligned && K > 0 &&
-           (((element == NH_Q4_K || element == NH_Q5_K || element == NH_Q6_K) && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
+           (((element == NH_Q4_K || element == NH_Q5_K || element == NH_Q6_K || element == NH_Q3_K) && K % 256u == 0) || (element == NH_Q8_0 && K % 64u == 0));
 }
 
 bool gemm_stacks(int32_t element, uint32_t K, const void *X, const void *W0, const void *W1, const void *W2, uint32_t end0, uint32_t end1) {

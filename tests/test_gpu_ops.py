@@ -388,9 +388,9 @@ def test_gemm_matches_fp32_accumulation(device, element, M, N, K, half):
 
 @pytest.mark.parametrize("element,M,N,K,half", [(NH_Q8_0, 100, 96, 896, False), (NH_Q8_0, 64, 64, 64, True), (NH_Q4_K, 70, 130, 512, True),
                                                 (NH_Q4_K, 33, 64, 256, False), (NH_Q6_K, 70, 130, 512, True), (NH_Q6_K, 33, 64, 256, False),
-                                                (NH_Q5_K, 70, 130, 512, False)])
+                                                (NH_Q5_K, 70, 130, 512, False), (NH_Q3_K, 70, 130, 512, True)])
 def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N, K, half):
-    """NEURA_HIP_GEMM_MFMA=0 keeps Q8_0, Q4_K, Q5_K and Q6_K wide products on the tiled vector kernel that serves the shapes the matrix
+    """NEURA_HIP_GEMM_MFMA=0 keeps Q8_0 and K-quant wide products on the tiled vector kernel that serves the shapes the matrix
     cores do not take (rows that are not whole steps, unaligned operands)."""
     monkeypatch.setenv("NEURA_HIP_GEMM_MFMA", "0")
     rng = np.random.default_rng(M + N + K)
@@ -399,20 +399,25 @@ def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N,
     close(device.gemm(element, raw, N, K, X), oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8))
 
 
-@pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K])
+@pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K, NH_Q3_K])
 @pytest.mark.parametrize("M,N,K,half", [(70, 130, 512, False), (40, 64, 3584, True), (512, 256, 1280, True), (33, 200, 256, False),
                                         (130, 128, 768, True), (64, 256, 18944, False), (512, 512, 3584, False)])
-def test_q6_k_and_q5_k_wide_products_on_the_matrix_cores(device, element, M, N, K, half):
+def test_q6_k_q5_k_and_q3_k_wide_products_on_the_matrix_cores(device, element, M, N, K, half):
     """Q6_K rows as two exact half planes on the matrix cores ((q - 32) * (sc & 15) and 16 * (q - 32) * (sc >> 4)), Q5_K rows
-    as Q4_K's with the fifth bit beside the nibble: against the oracle at the wide product's bar and against the exact
+    as Q4_K's with the fifth bit beside the nibble, Q3_K rows as the one exact plane (sc - 32) * code: against the oracle at the wide product's bar and against the exact
     product far inside it -- for Q6_K scales at both ends of a signed byte and at the seams of the split, blocks that start
-    on either half of a word (210-byte blocks: every other one does); for Q5_K scales, minimums and codes at their largest;
+    on either half of a word (210-byte blocks: every other one does; Q3_K's 110-byte blocks too); for Q5_K scales, minimums
+    and codes at their largest; for Q3_K scales and codes at both ends;
     ragged tiles, half and fp32 activations, and a residual."""
     rng = np.random.default_rng(M + N + K + element)
     if element == NH_Q6_K:
         raw = np.array(synth.RANDOM[NH_Q6_K](rng, N * K), dtype=np.uint8).reshape(-1, 210)
         hard = rng.random(raw.shape[0]) < 0.25
         raw[hard, 192:208] = rng.choice(np.array([-128, 127, -1, 15, 16, -16, -17, 0], np.int8).view(np.uint8), (int(hard.sum()), 16))
+    elif element == NH_Q3_K:
+        raw = np.array(synth.RANDOM[NH_Q3_K](rng, N * K), dtype=np.uint8).reshape(-1, 110)
+        hard = rng.random(raw.shape[0]) < 0.25
+        raw[hard, 0:108] = rng.choice(np.array([0x00, 0xFF], np.uint8), (int(hard.sum()), 1))  # scales -32 and codes -4, or +31 and +3
     else:
         raw = np.array(synth.RANDOM[NH_Q5_K](rng, N * K), dtype=np.uint8).reshape(-1, 176)
         hard = rng.random(raw.shape[0]) < 0.25
