@@ -1854,26 +1854,42 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
     const bool gated = p.swiglu != 0;
     const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
     const uint32_t shift = 16u * (kq >> 1);  // the group's pair of 6-bit fields inside its scale words
-    for (uint32_t base = blockIdx.x * TPW; base < p.tiles; base += gridDim.x * TPW) {
-        const uint32_t tile = base + ts;
-        const bool live = tile < p.tiles;
-        const uint32_t at_tile = live ? tile : p.tiles - 1u;
+    // Rounds of tiles: in round i the workgroup's tile slot ts takes tile (blockIdx.x + i * gridDim.x) * TPW + ts.  A wave's loads
+    // run two super-blocks ahead across rounds (the first blocks of the next tile are on their way while this tile's sums meet),
+    // and every fetch issues its three loads: past the last round the last block again, dropped.
+    const uint32_t rounds = (p.tiles > blockIdx.x * TPW) ? (p.tiles - blockIdx.x * TPW + gridDim.x * TPW - 1u) / (gridDim.x * TPW) : 0u;
+    const uint32_t first_round = blockIdx.x, hop = gridDim.x, tiles = p.tiles, row_bytes = p.row_bytes;
+    auto tile_of = [first_round, hop, ts](uint32_t round) __attribute__((always_inline)) -> uint32_t { return (first_round + round * hop) * TPW + ts; };
+    // written with selects over scalars captured by value: nothing here may end up indexed
+    const int64_t to_w1 = w1 - w0, to_w2 = w2 - w0;
+    auto row_of = [w0, to_w1, to_w2, end0, end1, gated, n, tiles, row_bytes, blk0, tile_of](uint32_t round) __attribute__((always_inline)) -> const uint8_t * {
+        const uint32_t at_tile = min(tile_of(round), tiles - 1u);
         const uint32_t r0 = at_tile * 16u;
         const bool in0 = r0 < end0, in1 = r0 < end1;
-        const uint8_t *row = gated ? (n < 8u ? w0 : w1) + (size_t)(at_tile * 8u + (n & 7u)) * p.row_bytes
-                                   : (in0 ? w0 : (in1 ? w1 : w2)) + (size_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1)) + n) * p.row_bytes;
-        row += (size_t)blk0 * 144u;
-        // two super-blocks in flight a wave: the loads of step s + 2 go out as step s is taken up
-        u32x4 even[3], odd[3];
-        auto fetch = [&](u32x4 (&ahead)[3], uint32_t step) {
-            // past the wave's last super-block the last one is fetched again: the waits count on every step issuing its loads
-            const uint8_t *block = row + (size_t)min(ks + KS * min(step, last_step), nb - 1u) * 144u;
-            ahead[0] = *(global_uint4)(uintptr_t)block;
-            ahead[1] = *(global_uint4)(uintptr_t)(block + 16u + 16u * kq);
-            ahead[2] = *(global_uint4)(uintptr_t)(block + 80u + 16u * kq);
-        };
+        const int64_t offset = gated ? (n < 8u ? (int64_t)0 : to_w1) + (int64_t)(at_tile * 8u + (n & 7u)) * row_bytes
+                                     : (in0 ? (int64_t)0 : (in1 ? to_w1 : to_w2)) + (int64_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1)) + n) * row_bytes;
+        return w0 + offset + (size_t)blk0 * 144u;
+    };
+    const uint32_t walked = max(count, 1u);  // a wave with no super-block of its own still keeps the ring's rhythm
+    uint32_t ahead_round = 0, ahead_step = 0;
+    const uint8_t *ahead_row = row_of(0);
+    u32x4 even[3], odd[3];
+    auto fetch = [&](u32x4 (&ahead)[3]) __attribute__((always_inline)) {
+        const uint8_t *block = ahead_row + (size_t)min(ks + KS * min(ahead_step, last_step), nb - 1u) * 144u;
+        ahead[0] = *(global_uint4)(uintptr_t)block;
+        ahead[1] = *(global_uint4)(uintptr_t)(block + 16u + 16u * kq);
+        ahead[2] = *(global_uint4)(uintptr_t)(block + 80u + 16u * kq);
+        if (++ahead_step >= walked) {
+            ahead_step = 0;
+            if (ahead_round + 1u < rounds) ahead_row = row_of(++ahead_round);
+        }
+    };
+    constexpr uint32_t parity = 0;  // one set of partial sums: 16 super-blocks of operands leave no room for two
+    {
         f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        auto take = [&](const u32x4 (&ahead)[3], uint32_t step) {
+        uint32_t tile = 0;
+        bool live = false;
+        auto take = [&](const u32x4 (&ahead)[3], uint32_t step) __attribute__((always_inline)) {
             const uint32_t b = min(ks + KS * step, nb - 1u);
             const u32x4 hdr = ahead[0], q0 = ahead[1], q1 = ahead[2];
             const u32x4 *a_block = pieces + (size_t)b * F16_BLOCK_PIECES + kq * 16u + n;
@@ -1886,6 +1902,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
                 const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;
                 const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;  // (sc0 * 2^10, sc1 * 2^6)
                 const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
+                // the four operands of the activations are asked for before the weights are unpacked: the unpacking hides LDS
+                u32x4 rows[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) rows[i] = a_block[(4u * j + i) * 64u];
+                __builtin_amdgcn_sched_barrier(0);
                 const u32x4 q = j == 0 ? q0 : q1;
                 const uint32_t words[4] = {q.x, q.y, q.z, q.w};
                 uint32_t low[8], high[8];
@@ -1901,8 +1922,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
                 for (int i = 0; i < 4; i++) {
                     const uint32_t *from = (i < 2 ? low : high) + 4 * (i & 1);
                     const half8_t weights = __builtin_bit_cast(half8_t, u32x4{from[0], from[1], from[2], from[3]});
-                    const half8_t rows = __builtin_bit_cast(half8_t, a_block[(4u * j + i) * 64u]);
-                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(rows, weights, tmp, 0, 0, 0);
+                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, rows[i]), weights, tmp, 0, 0, 0);
                 }
             }
             // ---- the super-block is complete: weigh by d, take the minimums off
@@ -1930,23 +1950,14 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[e] = fmaf(mscale, floors[e], fmaf(dscale, tmp[e], acc[e]));
         };
-        fetch(even, 0);
-        fetch(odd, 1);
-        uint32_t step = 0;
-        for (; step + 1u < count; step += 2u) {
-            take(even, step);
-            fetch(even, step + 2u);
-            take(odd, step + 1u);
-            fetch(odd, step + 3u);
-        }
-        if (step < count) take(even, step);
+        auto tile_end = [&]() __attribute__((always_inline)) {
         // ---- the waves of the tile meet lane by lane
-        float *mine = part + ((size_t)ts * KS + ks) * 4u * 64u;
+        float *mine = part + (((size_t)parity * TPW + ts) * KS + ks) * 4u * 64u;
 #pragma unroll
         for (int e = 0; e < 4; e++) mine[e * 64 + lane] = acc[e];
         __syncthreads();
         if (ks == 0) {
-            const float *from = part + (size_t)ts * KS * 4u * 64u;
+            const float *from = part + ((size_t)parity * TPW + ts) * KS * 4u * 64u;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 float total = 0.0f;
@@ -1969,7 +1980,30 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
                 }
             }
         }
-        __syncthreads();  // the next tile's partial sums take the same places
+            __syncthreads();  // the next tile's partial sums take the same places
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] = 0.0f;
+        };
+        fetch(even);
+        fetch(odd);
+        // every wave walks whole pairs of steps; a tile ends wherever its last step falls, and the steps past the last round
+        // multiply what was fetched again and publish nothing
+        uint32_t round = 0, step = 0;
+        tile = tile_of(0), live = rounds > 0 && tile < p.tiles;
+        const uint32_t steps = rounds * walked;
+        auto unit = [&](u32x4 (&held)[3]) __attribute__((always_inline)) {
+            if (count) take(held, step);
+            fetch(held);
+            if (++step >= walked) {
+                if (round < rounds) tile_end();
+                step = 0, round++;
+                tile = tile_of(round), live = round < rounds && tile < p.tiles;
+            }
+        };
+        for (uint32_t s0 = 0; s0 < steps; s0 += 2u) {
+            unit(even);
+            unit(odd);
+        }
     }
 }
 
