@@ -163,7 +163,8 @@ def cpu_baseline(shape, element, host_tensors, context, layers, seconds_budget=1
 def gemm_config3(device, rng, repeats=10):
     """The wide-product configuration of the benchmark: the Q4_K product M=512, K=3584, N=18944 (the 7B-shape FFN up projection), with half
     activations as the configuration states them and with fp32 activations as the decoder's fill passes them; and the same shape in
-    Q8_0 blocks (the element of the small decoder's fill), half activations."""
+    Q8_0 blocks (the element of the small decoder's fill) and in Q6_K, Q5_K and Q3_K blocks (what a K-quant mix stores beside Q4_K),
+    half activations."""
     from neura_amd import synth
 
     M, K, N = 512, 3584, 18944
@@ -171,7 +172,8 @@ def gemm_config3(device, rng, repeats=10):
     out = {"workload": "Q4_K wide product M=%d K=%d N=%d, random blocks, N(0,1) activations" % (M, K, N), "flop": 2.0 * M * N * K,
            "mfma_peak_tflops": 2500.0}
     for name, element, dtype, code in (("half_activations", 12, np.float16, 1), ("fp32_activations", 12, np.float32, 0),
-                                       ("q8_0_half_activations", 8, np.float16, 1)):
+                                       ("q8_0_half_activations", 8, np.float16, 1), ("q6_k_half_activations", 14, np.float16, 1),
+                                       ("q5_k_half_activations", 13, np.float16, 1), ("q3_k_half_activations", 11, np.float16, 1)):
         raw = device.upload(synth.RANDOM[element](rng, N * K))
         x = device.upload(rng.standard_normal((M, K)).astype(dtype))
         for timed in (False, True):
