@@ -127,13 +127,15 @@ MIXED_3 = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.ffn_
            "blk.2.attn_q.weight": NH_Q4_K, "blk.2.attn_k.weight": NH_Q4_K, "blk.2.attn_v.weight": NH_Q4_K, "blk.2.ffn_up.weight": NH_Q5_K}
 
 
-@pytest.mark.parametrize("base,mixed", [(NH_Q4_K, MIXED), (NH_Q3_K, MIXED_3)], ids=["q4_k_m", "q3_k_m"])
+@pytest.mark.parametrize("base,mixed", [(NH_Q4_K, MIXED), (NH_Q3_K, MIXED_3), (NH_Q6_K, {}), (NH_Q5_K, {}), (NH_Q3_K, {})],
+                         ids=["q4_k_m", "q3_k_m", "q6_k", "q5_k", "q3_k"])
 @pytest.mark.parametrize("batch", [1, 2])
 def test_mixed_elements_and_projection_biases(device, batch, base, mixed):
     """A decoder stored the way Q4_K_M files are (Q6_K for some matrices, Q4_K for the rest) whose q, k and v projections
     carry Qwen2's biases: layer 0 (a Q6_K value projection, biases) takes one product per matrix, layer 1 (one element,
     biases) folds rotation and biases into the stacked product at batch 1, layer 2 (gate and up stored differently) runs
-    the two halves apart.  Decode steps, a 16-row fill and the caches against the oracle."""
+    the two halves apart.  Decode steps, a 16-row fill and the caches against the oracle.  The same for decoders stored in
+    one K-quant throughout (the fill's q|k|v is then one stacked wide product of that element on the matrix cores)."""
     shape = SMALL_Q4
     rng = np.random.default_rng(21)
     tensors = list(synth.model_tensors(shape, base, rng, mode="normal", elements=mixed, biases=(0, 1)))
