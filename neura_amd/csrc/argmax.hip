@@ -39,6 +39,7 @@ __device__ void block_choice(float &value, uint32_t &index, float *values, uint3
 
 __global__ __launch_bounds__(256) void argmax_sections_kernel(const float *__restrict__ values, uint32_t n, uint32_t sections,
                                                               float *__restrict__ best_values, uint32_t *__restrict__ best_indices) {
+    NH_FETCH(values, n, sections, best_values, best_indices, gridDim.x);
     __shared__ float held_values[4];
     __shared__ uint32_t held_indices[4];
     const uint32_t row = blockIdx.y, section = blockIdx.x;
@@ -60,6 +61,7 @@ __global__ __launch_bounds__(256) void argmax_sections_kernel(const float *__res
 
 __global__ __launch_bounds__(256) void argmax_fold_kernel(const float *__restrict__ best_values, const uint32_t *__restrict__ best_indices,
                                                           uint32_t sections, uint32_t *__restrict__ out) {
+    NH_FETCH(best_values, best_indices, sections, out);
     __shared__ float held_values[4];
     __shared__ uint32_t held_indices[4];
     const uint32_t row = blockIdx.x;

@@ -34,6 +34,11 @@ struct AttentionParams {
     uint32_t reach;  // 0, or the span of a ring of `keys` slots
 };
 
+__device__ __forceinline__ void fetch_parameters(const AttentionParams &p) {
+    NH_FETCH(p.q, p.out, p.partial, p.q_sh, p.q_sb, p.q_sr, p.o_sh, p.o_sb, p.o_sr, p.cache_k, p.cache_v, p.heads, p.kv_heads, p.groups, p.batch, p.rows,
+             p.capacity, p.keys, p.sections, p.cursor, p.scale, p.refusal, p.reach);
+}
+
 // A ring cache (Cache::windowed, crates/neura-decoder/src/cache.rs:311-317, :391-394): once `written` positions have gone
 // in, slot `at` holds the latest position below `written` that lands on it (key_position,
 // crates/neura-kernel/src/task/attention.rs:103-108), and a query weighs the `reach` positions up to its own
@@ -104,6 +109,7 @@ __device__ __forceinline__ void fetch_tile(u32x4 (&kraw)[T], u32x4 (&vraw)[T], c
 
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
+    fetch_parameters(p);
     constexpr int LPK = WIDTH / 8;                       // lanes per key in the score pass
     constexpr int KPW = 64 / LPK, STEP = 4 * KPW;        // keys per wave and per workgroup step
     constexpr int TK = 64, T = TK / STEP;                // keys and steps per tile
@@ -277,6 +283,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 // section s into its weight; then thread (channel, stripe) sums its channel over every eighth
 // section -- all of its loads in flight at once -- and the eight stripes meet in LDS.
 __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, uint32_t width) {
+    fetch_parameters(p);
     __shared__ float weights[256], masses[256], held[256], stripes[8][32];
     const uint32_t G = p.groups, tid = threadIdx.x;
     const uint32_t blocks = (width + 31u) / 32u;
@@ -346,6 +353,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, uint32_t rows_per_wave) {
+    fetch_parameters(p);
     constexpr int TK = 32;                       // keys per tile
     constexpr int STEPS = WIDTH / 16;            // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 32;           // 32-channel blocks of the output
@@ -518,6 +526,7 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionParams p) {
+    fetch_parameters(p);
     constexpr int TK = 32;                  // keys per tile
     constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output
@@ -726,6 +735,7 @@ constexpr uint32_t ANY_KEYS = 256;  // keys a section holds at most: 16 query he
 
 template <int CE>
 __global__ __launch_bounds__(256) void attention_any_kernel(AttentionParams p, uint32_t width) {
+    fetch_parameters(p);
     __shared__ float scores[16 * ANY_KEYS];
     __shared__ float tops[16], masses[16];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;

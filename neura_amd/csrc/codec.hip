@@ -105,6 +105,7 @@ template <int ELEMENT>
 __global__ __launch_bounds__(256) void gather_kernel(const uint8_t *__restrict__ table, uint32_t vocab, uint32_t width, uint64_t row_bytes,
                                                      const uint32_t *__restrict__ tokens, uint32_t batch,
                                                      const uint8_t *__restrict__ mask, float *__restrict__ out, uint32_t *refusal) {
+    NH_FETCH(table, vocab, width, row_bytes, tokens, batch, mask, out, refusal);
     uint32_t t = blockIdx.x;
     uint32_t token = tokens[t];
     float keep = (mask == nullptr || mask[t % batch]) ? 1.0f : 0.0f;

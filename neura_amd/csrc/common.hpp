@@ -122,6 +122,47 @@ struct RopeFusion {
     uint32_t ring;       // 0, or the span of a ring cache: position p is written to slot p % ring
 };
 
+// NH_FETCH(p.a, p.b, ...): every scalar load of the named kernel parameters goes out at once, before the kernel's first
+// wait.  Left alone the compiler loads each parameter where it is first used: a parameter block that spans several cache
+// lines then costs one round trip to memory after another (about 0.3 us each) before the kernel's first vector load is
+// issued.  At most thirty names a statement; statements that follow one another still share one wait.
+#define NH_FETCH_1(a) "s"(a)
+#define NH_FETCH_2(a, ...) "s"(a), NH_FETCH_1(__VA_ARGS__)
+#define NH_FETCH_3(a, ...) "s"(a), NH_FETCH_2(__VA_ARGS__)
+#define NH_FETCH_4(a, ...) "s"(a), NH_FETCH_3(__VA_ARGS__)
+#define NH_FETCH_5(a, ...) "s"(a), NH_FETCH_4(__VA_ARGS__)
+#define NH_FETCH_6(a, ...) "s"(a), NH_FETCH_5(__VA_ARGS__)
+#define NH_FETCH_7(a, ...) "s"(a), NH_FETCH_6(__VA_ARGS__)
+#define NH_FETCH_8(a, ...) "s"(a), NH_FETCH_7(__VA_ARGS__)
+#define NH_FETCH_9(a, ...) "s"(a), NH_FETCH_8(__VA_ARGS__)
+#define NH_FETCH_10(a, ...) "s"(a), NH_FETCH_9(__VA_ARGS__)
+#define NH_FETCH_11(a, ...) "s"(a), NH_FETCH_10(__VA_ARGS__)
+#define NH_FETCH_12(a, ...) "s"(a), NH_FETCH_11(__VA_ARGS__)
+#define NH_FETCH_13(a, ...) "s"(a), NH_FETCH_12(__VA_ARGS__)
+#define NH_FETCH_14(a, ...) "s"(a), NH_FETCH_13(__VA_ARGS__)
+#define NH_FETCH_15(a, ...) "s"(a), NH_FETCH_14(__VA_ARGS__)
+#define NH_FETCH_16(a, ...) "s"(a), NH_FETCH_15(__VA_ARGS__)
+#define NH_FETCH_17(a, ...) "s"(a), NH_FETCH_16(__VA_ARGS__)
+#define NH_FETCH_18(a, ...) "s"(a), NH_FETCH_17(__VA_ARGS__)
+#define NH_FETCH_19(a, ...) "s"(a), NH_FETCH_18(__VA_ARGS__)
+#define NH_FETCH_20(a, ...) "s"(a), NH_FETCH_19(__VA_ARGS__)
+#define NH_FETCH_21(a, ...) "s"(a), NH_FETCH_20(__VA_ARGS__)
+#define NH_FETCH_22(a, ...) "s"(a), NH_FETCH_21(__VA_ARGS__)
+#define NH_FETCH_23(a, ...) "s"(a), NH_FETCH_22(__VA_ARGS__)
+#define NH_FETCH_24(a, ...) "s"(a), NH_FETCH_23(__VA_ARGS__)
+#define NH_FETCH_25(a, ...) "s"(a), NH_FETCH_24(__VA_ARGS__)
+#define NH_FETCH_26(a, ...) "s"(a), NH_FETCH_25(__VA_ARGS__)
+#define NH_FETCH_27(a, ...) "s"(a), NH_FETCH_26(__VA_ARGS__)
+#define NH_FETCH_28(a, ...) "s"(a), NH_FETCH_27(__VA_ARGS__)
+#define NH_FETCH_29(a, ...) "s"(a), NH_FETCH_28(__VA_ARGS__)
+#define NH_FETCH_30(a, ...) "s"(a), NH_FETCH_29(__VA_ARGS__)
+#define NH_FETCH_COUNT(_1, _2, _3, _4, _5, _6, _7, _8, _9, _10, _11, _12, _13, _14, _15, _16, _17, _18, _19, _20, _21, _22, _23, _24, _25, _26, _27, _28, _29, _30, N, ...) N
+#define NH_FETCH_PASTE(a, b) a##b
+#define NH_FETCH_PICK(n) NH_FETCH_PASTE(NH_FETCH_, n)
+#define NH_FETCH(...)                                                                                                                                    \
+    asm volatile("" ::NH_FETCH_PICK(NH_FETCH_COUNT(__VA_ARGS__, 30, 29, 28, 27, 26, 25, 24, 23, 22, 21, 20, 19, 18, 17, 16, 15, 14, 13, 12, 11, 10, 9, 8, 7, 6, 5, 4, \
+                                                   3, 2, 1))(__VA_ARGS__))
+
 struct GemvArgs {
     int32_t element;
     const void *W[3];  // up to three matrices stacked along N; unused entries are nullptr
@@ -137,8 +178,15 @@ struct GemvArgs {
     float eps;
     const RopeFusion *rope = nullptr;  // only where gemv_fuses_rope() says so
     const float *bias[3] = {nullptr, nullptr, nullptr};  // one per stacked matrix, added before the rotation: only together with `rope`
+    // Only where gemv_hands_digits() says so: a SwiGLU product leaves its outputs as digit planes (digits_out, in place of y)
+    // and the product that follows reads them (digits_in, in place of x) instead of turning floats into digits again.
+    uint8_t *digits_out = nullptr;
+    const uint8_t *digits_in = nullptr;
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
+// whether `producer` (a SwiGLU product of one row) can hand its outputs to `consumer` as digit planes, and the bytes they take
+bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer);
+size_t gemv_digit_bytes(uint32_t K);
 // whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)
 bool gemv_fuses_rope(const GemvArgs &args, const RopeFusion &rope);
 

@@ -135,6 +135,10 @@ struct GemmQ4Params {
     const float *unscale;  // [M] with split: undoes the row scale
 };
 
+__device__ __forceinline__ void fetch_parameters(const GemmQ4Params &p) {
+    NH_FETCH(p.W, p.W1, p.W2, p.end0, p.end1, p.N, p.K, p.row_bytes, p.A, p.S, p.rows, p.Y, p.residual, p.ldy, p.M, p.split, p.unscale);
+}
+
 // One workgroup per activation row: the row as MFMA-ready halves (and, for fp32 rows, its residue row and scale).
 // PRELUDE: what a row is before it is packed -- 0: X as it lies; 1: X normalised (rmsnorm_kernel's arithmetic, so the same
 // fp32 numbers: thread t adds the squares of columns t, t + 256, ..., then a 256-wide tree); 2: silu(gate) * X as
@@ -477,8 +481,193 @@ __device__ __forceinline__ void gemm_q45k_mfma(const GemmQ4Params &p) {
     gemm_multiply<true>(p, As, Bs, mns, dds, wave, lane, n0, m0, steps, 16384.0f);  // the weights were staged * 2^-14
 }
 
-__global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) { gemm_q45k_mfma<false>(p); }
-__global__ __launch_bounds__(512) void gemm_q5k_mfma_kernel(GemmQ4Params p) { gemm_q45k_mfma<true>(p); }
+__global__ __launch_bounds__(512) void gemm_q4k_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
+    gemm_q45k_mfma<false>(p);
+}
+__global__ __launch_bounds__(512) void gemm_q5k_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
+    gemm_q45k_mfma<true>(p);
+}
+
+// ------------------------------------------------------------------- Q4_K, weights through registers --------
+//
+// LDS is what bounds the kernel above (it takes a workgroup's writes at 64 B a clock and serves its reads at 128: a step moves
+// 32 KB in and 64 KB out, twice the time its MFMAs take).  Here the weights never touch it: eight multiplier waves own
+// 64 x 32 of the 128 x 128 tile each, and lane (l32, part) of one loads, unpacks and feeds the matrix cores the weights of ITS
+// row 32 wn + l32 -- per 64-k step one 16-byte load (bytes 16 part .. of the step's 32: the low nibbles are k = 16 part .. + 15,
+// the high nibbles k = 32 + 16 part ..), whose four 8-weight pieces are the B operands of the step's four MFMA depths; the
+// activation operand of depth kk is read from the matching 16-byte chunk of the staged row (chunk (kk >> 1) * 4 + 2 part +
+// (kk & 1)), so the k order inside a step is the weights', not the natural one, and nothing has to move.  The header of a
+// lane's row is in its registers, so d, dmin and the minimums need no LDS either.  Two multipliers share a SIMD (one unpacks
+// while the other's MFMAs run) beside one of the four stagers, which only copy packed activation rows: whole 128-byte
+// lines, eight lanes a row.  A stage of LDS is a whole super-block of k (256 columns of the 128 rows, 66 KB; two stages), so
+// the twelve waves meet at one barrier a super-block, not one a step.
+constexpr int GSB = 256 + 8;  // LDS row stride of a stage in halves: 528 B keeps 128-bit reads of 8 neighbouring rows on distinct banks
+constexpr size_t GEMM_Q4K_REGB_LDS = sizeof(_Float16) * 2 * GT * GSB;
+
+__global__ __launch_bounds__(768) void gemm_q4k_regb_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
+    _Float16(*As)[GT][GSB] = reinterpret_cast<_Float16(*)[GT][GSB]>(gemm_lds);  // [2]
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n0 = blockIdx.x * GT, m0 = blockIdx.y * GT;
+    const uint32_t steps = p.K / 64u;  // a multiple of 4: K is whole super-blocks
+    const uint32_t nsb = steps >> 2;
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+
+    if (wave >= 8) {
+        // ------------------------------------------------------------------ stagers: rows abase + 32 j, 16-byte chunks achunk + 8 c
+        const uint32_t tid = threadIdx.x - 512u;
+        const uint32_t abase = tid >> 3, achunk = tid & 7u;
+        const _Float16 *asrc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) asrc[j] = p.A + (size_t)min(m0 + abase + 32u * j, p.rows - 1u) * p.K + 8u * achunk;
+        u32x4 av[4][4];  // the super-block on its way: [64-k step][row]
+        auto fetch = [&](uint32_t sb) {
+            const size_t at = (size_t)min(sb, nsb - 1u) * 256u;  // past the end the last super-block again, dropped
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) av[c][j] = *(global_uint4)(uintptr_t)(asrc[j] + at + 64u * c);
+        };
+        fetch(0);
+        for (uint32_t sb = 0; sb < nsb; sb++) {
+            const uint32_t buf = sb & 1u;
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) *reinterpret_cast<u32x4 *>(&As[buf][abase + 32u * j][64u * c + 8u * achunk]) = av[c][j];
+            fetch(sb + 1u);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();  // the super-block is staged; the multipliers are done with the one before it
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- multipliers
+    const uint32_t wm = wave >> 2, wn = wave & 3u, l32 = lane & 31u, part = lane >> 5;
+    // a tile lies in one matrix: the boundaries between stacked matrices are multiples of the tile
+    const uint32_t column = min(n0 + 32u * wn + l32, p.N - 1u);
+    const uint8_t *wrow = column < p.end0   ? p.W + (size_t)column * p.row_bytes
+                          : column < p.end1 ? p.W1 + (size_t)(column - p.end0) * p.row_bytes
+                                            : p.W2 + (size_t)(column - p.end1) * p.row_bytes;
+    const _Float16 *sums[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) sums[i] = p.S + (size_t)min(m0 + 64u * wm + 32u * i + l32, p.rows - 1u) * nsb * 16u + 8u * part;
+    const half2_t offset = {(_Float16)1024.0f, (_Float16)1024.0f}, powers = {(_Float16)1024.0f, (_Float16)64.0f};
+
+    f32x16 acc[2], tmp[2], zero;
+#pragma unroll
+    for (int e = 0; e < 16; e++) zero[e] = 0.0f;
+    acc[0] = acc[1] = tmp[0] = tmp[1] = zero;
+
+    // the lane's weights: a super-block's header and its four 16-byte runs, one super-block ahead
+    u32x4 ahead, qs[4];
+    ahead = *(global_uint4)(uintptr_t)wrow;
+#pragma unroll
+    for (int g = 0; g < 4; g++) qs[g] = *(global_uint4)(uintptr_t)(wrow + 16u + 32u * g + 16u * part);
+    for (uint32_t first = 0; first < steps; first += 4) {
+        const u32x4 hdr = ahead;
+        const uint32_t next = min((first >> 2) + 1u, nsb - 1u);  // past the end the last super-block again, dropped
+        ahead = *(global_uint4)(uintptr_t)(wrow + (size_t)next * 144u);
+        u32x4 sraw[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) sraw[i] = *(global_uint4)(uintptr_t)(sums[i] + (size_t)(first >> 2) * 16u);  // wanted at the end of the super-block
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t sbuf = (first >> 2) & 1u;
+            // 6-bit fields of sub-blocks 2g, 2g+1 (crates/neura-precision/src/ggml.rs:127-136); 0x6400 | v is the half 1024 + v
+            const uint32_t shift = 16u * (g & 1u);
+            const uint32_t ya = (hdr.y >> shift) & 0xffffu, wa = (hdr.w >> shift) & 0xffffu;
+            const uint32_t sc = g < 2 ? (ya & 0x3f3fu) : ((wa & 0x0f0fu) | ((ya >> 2) & 0x3030u));
+            const uint32_t both = __builtin_amdgcn_perm(0u, sc, 0x0c010c00u) | 0x64006400u;  // (1024 + sc0, 1024 + sc1)
+            const half2_t scales = (__builtin_bit_cast(half2_t, both) - offset) * powers;     // (sc0 * 2^10, sc1 * 2^6)
+            const half2_t low_scale = {scales.x, scales.x}, high_scale = {scales.y, scales.y};
+            const uint32_t words[4] = {qs[g].x, qs[g].y, qs[g].z, qs[g].w};
+            // the slot is free once its words are copied out: the same run of the next super-block goes out
+            qs[g] = *(global_uint4)(uintptr_t)(wrow + (size_t)next * 144u + 16u + 32u * g + 16u * part);
+            if (g == 0) __syncthreads();  // the super-block's activations are staged
+            const _Float16 *arow0 = &As[sbuf][64u * wm + l32][64u * g], *arow1 = &As[sbuf][64u * wm + 32u + l32][64u * g];
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                // depth kk: words 2 (kk & 1), + 1 of the run, low nibbles for kk < 2; element order inside a word: 0, 2 then 1, 3
+                // (the byte lanes), the order the activations were packed in
+                uint32_t b[4];
+#pragma unroll
+                for (int w = 0; w < 2; w++) {
+                    const uint32_t even = words[2 * (kk & 1) + w], odd = even >> 8;
+                    if (kk < 2) {
+                        b[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x000f000fu) * low_scale);
+                        b[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x000f000fu) * low_scale);
+                    } else {
+                        b[2 * w] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, even & 0x00f000f0u) * high_scale);
+                        b[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, odd & 0x00f000f0u) * high_scale);
+                    }
+                }
+                const half8_t weights = __builtin_bit_cast(half8_t, u32x4{b[0], b[1], b[2], b[3]});
+                const uint32_t chunk = 8u * ((kk >> 1) * 4u + 2u * part + (kk & 1));  // where those eight k lie in the staged row
+                const half8_t a0 = *reinterpret_cast<const half8_t *>(arow0 + chunk), a1 = *reinterpret_cast<const half8_t *>(arow1 + chunk);
+                tmp[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0, weights, (g == 0 && kk == 0) ? zero : tmp[0], 0, 0, 0);
+                tmp[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, weights, (g == 0 && kk == 0) ? zero : tmp[1], 0, 0, 0);
+            }
+        }
+        // ---- the super-block is complete: weigh by d, then take the minimums off (the eight minimums as halves, k 8..15 * 2^-11
+        // against the sums' residues * 2^11)
+        const half2_t dd = __builtin_bit_cast(half2_t, hdr.x);
+        const float dscale = (float)dd.x * 16384.0f;  // the weights were unpacked * 2^-14
+        const float mscale = (float)dd.y * -64.0f;    // the sums were packed / 64
+        const uint32_t lo4 = hdr.z & 0x3f3f3f3fu;                                         // m0..m3
+        const uint32_t hi4 = ((hdr.w >> 4) & 0x0f0f0f0fu) | ((hdr.z >> 2) & 0x30303030u);  // m4..m7
+        half2_t m01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c010c00u) | 0x64006400u) - offset;
+        half2_t m23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, lo4, 0x0c030c02u) | 0x64006400u) - offset;
+        half2_t m45 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c010c00u) | 0x64006400u) - offset;
+        half2_t m67 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0u, hi4, 0x0c030c02u) | 0x64006400u) - offset;
+        if (part) {
+            const half2_t down = {(_Float16)0.00048828125f, (_Float16)0.00048828125f};
+            m01 = m01 * down, m23 = m23 * down, m45 = m45 * down, m67 = m67 * down;
+        }
+        const half8_t b2 = __builtin_bit_cast(half8_t, u32x4{__builtin_bit_cast(uint32_t, m01), __builtin_bit_cast(uint32_t, m23),
+                                                             __builtin_bit_cast(uint32_t, m45), __builtin_bit_cast(uint32_t, m67)});
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const f32x16 mins = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sraw[i]), b2, zero, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][e] = fmaf(dscale, tmp[i][e], acc[i][e]);
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][e] = fmaf(mscale, mins[e], acc[i][e]);
+        }
+    }
+    // ---- out: lane (l32, part) holds column n = l32 of a 32 x 32 block; register 4q + e is row 8q + 4 part + e
+    const uint32_t n = n0 + 32u * wn + l32;
+    if (n >= p.N) return;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t row = m0 + 64u * wm + 32u * i + 8u * q + 4u * part;  // first of four rows of A'
+            if (p.split) {
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const uint32_t m = (row >> 1) + e;
+                    if (m >= p.M) continue;
+                    float value = fmaf(acc[i][4 * q + 2 * e + 1], 0.00048828125f, acc[i][4 * q + 2 * e]) * p.unscale[m];
+                    const size_t at = (size_t)m * p.ldy + n;
+                    p.Y[at] = p.residual ? p.residual[at] + value : value;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t m = row + e;
+                    if (m >= p.M) continue;
+                    const size_t at = (size_t)m * p.ldy + n;
+                    p.Y[at] = p.residual ? p.residual[at] + acc[i][4 * q + e] : acc[i][4 * q + e];
+                }
+            }
+        }
+    }
+}
 
 // ------------------------------------------------------------------- Q8_0 on MFMA --------
 //
@@ -497,6 +686,7 @@ typedef uint32_t u32x4_loose __attribute__((ext_vector_type(4), aligned(4)));
 constexpr size_t GEMM_Q8_LDS = sizeof(_Float16) * (4 * GT * GS) + sizeof(float) * 2 * 2 * GT;
 
 __global__ __launch_bounds__(512) void gemm_q8_0_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);                                   // [2]
     _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);  // [2]
@@ -672,6 +862,7 @@ struct Q6Raw {
 };
 
 __global__ __launch_bounds__(512) void gemm_q6k_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);
     _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);
@@ -795,6 +986,7 @@ struct Q3Raw {
 };
 
 __global__ __launch_bounds__(512) void gemm_q3k_mfma_kernel(GemmQ4Params p) {
+    fetch_parameters(p);
     extern __shared__ __attribute__((aligned(16))) uint8_t gemm_lds[];
     _Float16(*As)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds);
     _Float16(*Bs)[GT][GS] = reinterpret_cast<_Float16(*)[GT][GS]>(gemm_lds + sizeof(_Float16) * 2 * GT * GS);
@@ -952,6 +1144,7 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
     if (!sized) {
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q8_0_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q8_LDS));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q4k_regb_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_REGB_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q6k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q5k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
         NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_q3k_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMM_Q4K_LDS));
@@ -962,7 +1155,9 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
     else if (a.element == NH_Q6_K) hipLaunchKernelGGL(gemm_q6k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else if (a.element == NH_Q5_K) hipLaunchKernelGGL(gemm_q5k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
     else if (a.element == NH_Q3_K) hipLaunchKernelGGL(gemm_q3k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
-    else hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
+    else if (const char *held = getenv("NEURA_HIP_GEMM_REGB"); held && held[0] == '0')  // the form that unpacks the weights into LDS
+        hipLaunchKernelGGL(gemm_q4k_mfma_kernel, grid, dim3(512), GEMM_Q4K_LDS, d->stream, p);
+    else hipLaunchKernelGGL(gemm_q4k_regb_mfma_kernel, grid, dim3(768), GEMM_Q4K_REGB_LDS, d->stream, p);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }

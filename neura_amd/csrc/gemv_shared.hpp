@@ -34,7 +34,21 @@ struct GemvParams {
     uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
     uint32_t *refusal;
     const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
+    // 16-row tile kernel: activations handed from one product to the next as the digit planes the matrix cores take
+    // (gemv_digit_bytes() of them): written by a SwiGLU epilogue in place of y, read by a plain product in place of x
+    uint8_t *digits_out;
+    const uint8_t *digits_in;
 };
+
+// the parameters a product reads before its first vector load, and the rotation's where it is folded in
+__device__ __forceinline__ void fetch_parameters(const GemvParams &p, bool rope = false) {
+    NH_FETCH(p.W[0], p.W[1], p.W[2], p.end[0], p.end[1], p.end[2], p.x, p.y, p.residual, p.norm_w, p.partial, p.N, p.K, p.row_bytes, p.nblk,
+             p.blocks_per_split, p.splits, p.group, p.row_groups, p.tile_rows, p.rows, p.chunks_per_row, p.swiglu, p.eps, p.rope_width, p.digits_in,
+             p.digits_out);
+    if (rope)
+        NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions, p.rope_ring,
+                 p.bias[0], p.bias[1], p.bias[2], p.refusal);
+}
 
 __device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
 

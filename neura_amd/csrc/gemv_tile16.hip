@@ -28,8 +28,11 @@ constexpr uint32_t TILE16_BLOCK_DIGITS = 768;  // 16 chunks of 16 activations x 
 constexpr uint32_t TILE16_ZERO_BYTES = 208;    // what an idle A lane reads: four chunk offsets (0, 48, 96, 144) + 16 bytes
 enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2 };
 
-static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R) {
-    return (size_t)R * nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + (size_t)R * nblk * 64u + (size_t)2 * NW * R * 16u * 4u + (size_t)NW * R * 4u + 64u;
+constexpr uint32_t TILE16_BLOCK_PAIRS = 128;   // handed-over activations: a (sum, scale) pair of floats per chunk of 16
+constexpr uint32_t TILE16_BLOCK_HANDED = 1024;  // in memory a chunk is one 64-byte piece: three planes, its pair, eight idle bytes
+static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R, bool handed = false) {
+    const size_t sums = handed ? (size_t)nblk * TILE16_BLOCK_PAIRS : (size_t)R * nblk * 64u;
+    return (size_t)R * nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + sums + (size_t)2 * NW * R * 16u * 4u + (size_t)NW * R * 4u + 64u;
 }
 
 struct Tile16Unit {
@@ -40,9 +43,17 @@ struct Tile16Unit {
 // R > 1: up to R activation rows (p.rows of them) meet the weights in one pass.  Every row has its own digit planes and sums in
 // LDS; a step unpacks its weights once and runs the four MFMAs and the weighing once a row, so the weights are read once for
 // all rows where one launch a row read them `rows` times.
-template <int NW, int D, int MODE, int R>
+//
+// HANDED: the activations arrive as digit planes already (p.digits_in: per chunk of 16 one 64-byte piece -- three planes of
+// 16 bytes, then the chunk's (sum, scale) pair), left there by the SwiGLU epilogue of the product before (p.digits_out),
+// which holds a chunk's sixteen outputs in sixteen lanes of one wave when it is done and writes the piece as one whole,
+// aligned 64 bytes (pieces smaller than the 32 bytes the memory checks as one cost a read-modify-write each).  The scale
+// is then a chunk's own, not a group's, so the four MFMAs of a step keep their sums apart and each is weighed by its
+// chunk's scale; the staging pass shrinks to a copy.
+template <int NW, int D, int MODE, int R, bool HANDED = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
+    static_assert(!HANDED || (R == 1 && MODE == TILE16_PLAIN), "handed-over digit planes feed a plain product of one row");
     extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
     constexpr uint32_t NT = NW * 64;
     typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -55,9 +66,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     const uint32_t row_digits = nblk * TILE16_BLOCK_DIGITS;  // digit planes of one activation row
     uint8_t *const zeros = tile16_lds_bytes + (size_t)R * row_digits + wave * TILE16_ZERO_BYTES;  // a wave's own zeros
     f32x4 *const sums = reinterpret_cast<f32x4 *>(tile16_lds_bytes + (size_t)R * row_digits + NW * TILE16_ZERO_BYTES);  // [row][block][group]
-    float *const part = reinterpret_cast<float *>(sums + (size_t)R * nblk * 4u);  // [parity][wave][row][16]
+    float *const part = reinterpret_cast<float *>(sums + (HANDED ? (size_t)nblk * (TILE16_BLOCK_PAIRS / 16u) : (size_t)R * nblk * 4u));  // [parity][wave][row][16]
     float *const red = part + 2u * NW * R * 16u;                                  // [wave][row]
 
+    fetch_parameters(p, MODE == TILE16_ROPE);
+    asm volatile("" ::"s"(gridDim.x));
     const uint32_t r = lane & 15u, q = lane >> 4;
     // tiles of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
     const uint32_t tiles = p.row_groups;
@@ -175,7 +188,36 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             if ((e4 & 7u) == 0) s[(e4 >> 3) & 1u] = total * unscale;
             if ((e4 & 15u) == 0) s[2] = unscale;
         };
-        if constexpr (R > 1) {
+        if constexpr (HANDED) {
+            // a wave copies the super-blocks it walks, one 16-byte load a lane and block: lane 4 c + part holds plane `part` of
+            // chunk c, or with part 3 the chunk's pair
+            constexpr int MAXB = 5;
+            uint8_t *const pairs = reinterpret_cast<uint8_t *>(sums);
+            const uint32_t chunk = lane >> 2, piece = lane & 3u;
+            for (uint32_t j0 = 0; j0 < count; j0 += MAXB) {
+                u32x4 held[MAXB];
+#pragma unroll
+                for (int j = 0; j < MAXB; j++) {
+                    uint32_t b = min(wave + NW * (j0 + j), nblk - 1u);
+                    held[j] = *(global_uint4)(uintptr_t)(p.digits_in + (size_t)b * TILE16_BLOCK_HANDED + lane * 16u);
+                }
+                if (j0 == 0) {
+#pragma unroll
+                    for (int i = 0; i < D; i++) fetch(ring[i]);
+                }
+#pragma unroll
+                for (int j = 0; j < MAXB; j++) {
+                    const uint32_t b = wave + NW * (j0 + j);
+                    if (b >= nblk) continue;
+                    if (piece < 3u) *reinterpret_cast<u32x4 *>(digits + (size_t)b * TILE16_BLOCK_DIGITS + chunk * 48u + piece * 16u) = held[j];
+                    else *reinterpret_cast<uint2 *>(pairs + (size_t)b * TILE16_BLOCK_PAIRS + chunk * 8u) = uint2{held[j].x, held[j].y};
+                }
+            }
+            if (count == 0) {
+#pragma unroll
+                for (int i = 0; i < D; i++) fetch(ring[i]);
+            }
+        } else if constexpr (R > 1) {
             // the weights' loads go out first; every row's activations follow (twice where the norm is folded in: once for
             // the row's sum of squares, once for the digits -- the second pass finds them in the cache)
 #pragma unroll
@@ -324,6 +366,41 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         const float d24 = (float)dd.x * (16777216.0f * st.s.z), m24 = (float)dd.y * -16777216.0f;
         acc[0] = fmaf(d24, weighed, fmaf(m24, floor_, acc[0]));
     };
+    // handed-over planes: a chunk of 16 has its own scale, so the four MFMAs keep their sums apart
+    struct HandedStep {
+        i32x4 c[4];
+        f32x4 low, high;  // (sum, scale) of chunks 0, 1 and of chunks 2, 3 of the lane's group
+        uint32_t sc, mn, dd;
+    };
+    auto multiply_handed = [&](const Tile16Unit &u, uint32_t b, HandedStep &st) {
+        const uint8_t *at = abase + (size_t)b * astride;
+        const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
+        const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
+        st.low = sums[b * 8u + 2u * q], st.high = sums[b * 8u + 2u * q + 1u];
+        const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+        const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
+        const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
+        half2_t sc, mn;
+        scale_pairs(u.hdr, lane_scales, sc, mn);
+        st.sc = __builtin_bit_cast(uint32_t, sc), st.mn = __builtin_bit_cast(uint32_t, mn), st.dd = u.hdr.x;
+        const i32x4 none = {0, 0, 0, 0};
+        st.c[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a00, la, none, 0, 0, 0);
+        st.c[2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a10, ha, none, 0, 0, 0);
+        st.c[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a01, lb, none, 0, 0, 0);
+        st.c[3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a11, hb, none, 0, 0, 0);
+        asm volatile("" : "+v"(st.sc), "+v"(st.mn), "+v"(st.dd));  // the header is read by here
+    };
+    auto weigh_handed = [&](const HandedStep &st) {
+        const half2_t sc = __builtin_bit_cast(half2_t, st.sc), mn = __builtin_bit_cast(half2_t, st.mn), dd = __builtin_bit_cast(half2_t, st.dd);
+        float f[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) f[i] = fmaf((float)((st.c[i][0] << 8) + st.c[i][1]), 256.0f, (float)st.c[i][2]);
+        const float fl = fmaf(st.low.y, f[0], st.low.w * f[1]), fh = fmaf(st.high.y, f[2], st.high.w * f[3]);  // scales are powers of two
+        const float weighed = fmaf((float)sc.x, fl, (float)sc.y * fh);
+        const float floor_ = fmaf((float)mn.x, st.low.x + st.low.z, (float)mn.y * (st.high.x + st.high.z));
+        const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * -16777216.0f;
+        acc[0] = fmaf(d24, weighed, fmaf(m24, floor_, acc[0]));
+    };
     // R > 1: the weights are unpacked once, the next fetch goes out, and every row then runs its four MFMAs and its weighing
     auto step_rows = [&](Tile16Unit &u, uint32_t b) {
         const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
@@ -359,7 +436,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             s += nblk * 4u;
         }
     };
-    auto tile_end = [&](uint32_t tile) {
+    // The wave that finishes a tile (sums the waves' parts, runs the epilogue) changes from tile to tile (with SwiGLU from pair
+    // to pair: the gate sum waits in its registers), so that no wave falls behind the others by an epilogue a tile.
+    auto tile_end = [&](uint32_t tile, uint32_t index) {
+        const uint32_t finisher = MODE == TILE16_ROPE ? 0u : (MODE == TILE16_SWIGLU ? index >> 1 : index) % NW;
 #pragma unroll
         for (int row = 0; row < R; row++) {
             float v = acc[row];
@@ -369,7 +449,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             acc[row] = 0.0f;
         }
         __syncthreads();
-        if (wave == 0) {
+        if (wave == finisher) {
 #pragma unroll
           for (int i = 0; i < RQ; i++) {
             // lane (r, q) finishes output r of activation rows q, q + 4, ...
@@ -379,8 +459,40 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
 #pragma unroll
             for (int w = 0; w < NW; w++) total += part[((parity * NW + w) * R + row) * 16u + r];
             if (MODE == TILE16_SWIGLU) {
-                if (tile & 1u) p.y[(size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r] = silu(gate[i]) * total;
-                else gate[i] = total;
+                if (!(tile & 1u)) {
+                    gate[i] = total;
+                } else if (R == 1 && p.digits_out) {
+                    // the sixteen outputs of this pair are chunk tile / 2 of the next product's activations: lanes 0..15 turn them
+                    // into the three digit planes below a power-of-two scale of their own, as `stage` does for a group
+                    const float value = silu(gate[i]) * total;
+                    uint32_t top = __builtin_bit_cast(uint32_t, value) & 0x7fffffffu;
+                    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+                    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+                    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
+                    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
+                    const uint32_t raw = top >> 23;
+                    const uint32_t exponent = min(max(raw, 22u), 254u);
+                    const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);
+                    const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
+                    const float rounded = rintf(value * scale);
+                    float chunk_sum = rounded;
+                    chunk_sum += dpp<DPP_QUAD_XOR1>(chunk_sum);
+                    chunk_sum += dpp<DPP_QUAD_XOR2>(chunk_sum);
+                    chunk_sum += dpp<DPP_ROW_ROR4>(chunk_sum);
+                    chunk_sum += dpp<DPP_ROW_ROR8>(chunk_sum);
+                    const int dg = (int)signed_digits((int)rounded);
+                    // lane l writes word l of the chunk's 64 bytes: words 0..3 the most significant digits of elements 4 l ..,
+                    // 4..7 the middle ones, 8..11 the least significant, 12 and 13 the pair
+                    const int first = (int)(r & 3u) * 4;
+                    const uint32_t d0 = (uint32_t)__shfl(dg, first, 16), d1 = (uint32_t)__shfl(dg, first + 1, 16);
+                    const uint32_t d2 = (uint32_t)__shfl(dg, first + 2, 16), d3 = (uint32_t)__shfl(dg, first + 3, 16);
+                    const uint32_t plane = r >> 2, shift = 16u - 8u * min(plane, 2u);
+                    uint32_t word = ((d0 >> shift) & 0xffu) | (((d1 >> shift) & 0xffu) << 8) | (((d2 >> shift) & 0xffu) << 16) | (((d3 >> shift) & 0xffu) << 24);
+                    if (plane == 3u) word = r == 12u ? __builtin_bit_cast(uint32_t, chunk_sum * unscale) : (r == 13u ? __builtin_bit_cast(uint32_t, unscale) : 0u);
+                    reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u)[r] = word;
+                } else {
+                    p.y[(size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r] = silu(gate[i]) * total;
+                }
             } else if (MODE == TILE16_ROPE) {
                 uint32_t c;
                 const uint32_t n = rope_row(tile, c);
@@ -400,7 +512,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         parity ^= 1u;
     };
     if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
-        for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t));
+        for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t), t);
         return;
     }
     // Every wave walks whole rounds of D steps: the steps past its last tile multiply what was fetched again and publish nothing.
@@ -411,6 +523,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         for (int slot = 0; slot < D; slot++) {
             if constexpr (R > 1) {
                 step_rows(ring[slot], at_b);
+            } else if constexpr (HANDED) {
+                HandedStep st;
+                multiply_handed(ring[slot], at_b, st);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(ring[slot]);
+                __builtin_amdgcn_sched_barrier(0);
+                weigh_handed(st);
             } else {
                 Step st;
                 multiply(ring[slot], at_b, st);
@@ -421,7 +540,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             }
             at_b += NW;
             if (at_b >= nblk) {
-                if (at_tile < walked) tile_end(tile_at(at_tile));
+                if (at_tile < walked) tile_end(tile_at(at_tile), at_tile);
                 at_b = wave;
                 at_tile++;
             }
@@ -454,20 +573,46 @@ bool tile16_takes(const GemvArgs &a) {
     } else if (a.end[0] % 16u != 0 || a.end[1] % 16u != 0) {
         return false;
     }
+    if (a.digits_out && (!a.swiglu || a.rows != 1 || a.N % 512u != 0 || ((uintptr_t)a.digits_out & 63u))) return false;
+    if (a.digits_in && (a.swiglu || a.rope || a.norm_w || a.rows != 1 || ((uintptr_t)a.digits_in & 15u))) return false;
     const uint32_t nblk = a.K / 256u;
-    return tile16_lds(nblk, nblk > 32u ? 16u : 8u, tile16_row_form(a.rows)) <= 160u * 1024u;
+    return tile16_lds(nblk, nblk > 32u ? 16u : 8u, tile16_row_form(a.rows), a.digits_in != nullptr) <= 160u * 1024u;
 }
 
-template <int NW, int D, int MODE, int R>
+// A SwiGLU product of one row ends with a chunk's sixteen outputs in sixteen lanes of one wave: it can leave them as the digit
+// planes the product behind it would otherwise make of them again (NEURA_HIP_TILE16_HANDED=0 keeps the floats).
+size_t gemv_digit_bytes(uint32_t K) { return (size_t)(K / 256u) * TILE16_BLOCK_HANDED; }
+
+bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer) {
+    if (env_int("NEURA_HIP_TILE16_HANDED", 1) == 0) return false;
+    if (!producer.swiglu || producer.rows != 1 || consumer.rows != 1 || consumer.K != producer.N / 2u || consumer.K % 256u != 0) return false;
+    if (consumer.swiglu || consumer.rope || consumer.norm_w) return false;
+    GemvArgs from = producer, to = consumer;
+    from.digits_out = nullptr, to.digits_in = nullptr;
+    if (!tile16_takes(from) || !tile16_takes(to)) return false;
+    const uint32_t nblk = to.K / 256u;
+    return tile16_lds(nblk, nblk > 32u ? 16u : 8u, 1u, true) <= 160u * 1024u;
+}
+
+template <int NW, int D, int MODE, int R, bool HANDED = false>
 static hipError_t launch_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
     static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE, R>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
     return hipGetLastError();
+}
+
+// a plain product of one row whose activations arrive as digit planes
+static hipError_t launch_tile16_handed(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
+    switch (waves) {
+    case 4: return launch_tile16_instance<4, 2, TILE16_PLAIN, 1, true>(d, p, grid, lds);
+    case 7: return launch_tile16_instance<7, 2, TILE16_PLAIN, 1, true>(d, p, grid, lds);
+    default: return launch_tile16_instance<8, 2, TILE16_PLAIN, 1, true>(d, p, grid, lds);
+    }
 }
 
 template <int MODE, int R>
@@ -500,6 +645,8 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     }
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
     p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps, p.rows = a.rows;
+    p.digits_out = a.digits_out, p.digits_in = a.digits_in;
+
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     p.nblk = a.K / 256u;
     p.rope_width = 16;  // the kernel derives a tile's rows from it only where the rotation is folded in
@@ -511,7 +658,9 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
         for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
     }
     // waves of a workgroup share a tile and split its super-blocks: about two steps a wave
-    const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u ? 8u : 16u));
+    // (sixteen on deep rows, where turning the activations into digits is the larger part of a wave's work; eight where the
+    // digits arrive ready: fewer loads in flight a compute unit stream faster, as the shallow products show)
+    const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u || a.digits_in ? 8u : 16u));
     // units of work: tiles, or with SwiGLU pairs (a gate tile and the up tile behind it); every workgroup takes the same
     // number of them, one workgroup a compute unit when there are that many
     // A plain tile holds the number of rows, 16 down to 12, that leaves the fewest compute units idle in the last round.
@@ -531,9 +680,10 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     p.row_groups = units;
     const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
     const uint32_t grid = (units + rounds - 1u) / rounds;
-    const size_t lds = tile16_lds(p.nblk, waves, tile16_row_form(a.rows));
+    const size_t lds = tile16_lds(p.nblk, waves, tile16_row_form(a.rows), a.digits_in != nullptr);
     profile_mark(d);
-    hipError_t launched = a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
+    hipError_t launched = a.digits_in ? launch_tile16_handed(d, p, waves, grid, lds)
+                          : a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
                           : a.rope ? launch_tile16_mode<TILE16_ROPE>(d, p, waves, grid, lds)
                                    : launch_tile16_mode<TILE16_PLAIN>(d, p, waves, grid, lds);
     NH_HIP(launched);

@@ -248,11 +248,17 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             GemvArgs o = narrow(m, element_at(m, L, O), m->attn_o[L], H, QW, m->att, T, m->h);
             o.residual = m->h;
             if ((status = launch_gemv(d, o)) != NH_OK) return status;
+            GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
+            dn.residual = m->h;
             if (element_at(m, L, GATE) == element_at(m, L, UP)) {
                 GemvArgs gu = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
                 gu.W[1] = m->ffn_up[L];
                 gu.end[0] = F, gu.end[1] = gu.end[2] = 2 * F;
                 gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
+                // one row: silu(gate) * up goes to the down projection as the digit planes it multiplies (they fit the up
+                // projection's idle buffer), not as floats it would turn into digits again
+                if (gemv_hands_digits(gu, dn) && gemv_digit_bytes(F) <= (size_t)F * sizeof(float))
+                    gu.digits_out = reinterpret_cast<uint8_t *>(m->up), dn.digits_in = reinterpret_cast<const uint8_t *>(m->up);
                 if ((status = launch_gemv(d, gu)) != NH_OK) return status;
             } else {
                 GemvArgs g = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], F, H, m->h, T, m->act);
@@ -262,8 +268,6 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 if ((status = launch_gemv(d, u)) != NH_OK) return status;
                 if ((status = launch_silu_mul(d, m->act, m->up, (uint64_t)T * F, m->act)) != NH_OK) return status;
             }
-            GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
-            dn.residual = m->h;
             if ((status = launch_gemv(d, dn)) != NH_OK) return status;
         }
         if (!products_only && mask && (status = launch_mask_rows(d, m->h, rows, B, H, mask)) != NH_OK) return status;

@@ -134,6 +134,7 @@ template <int CE>
 __global__ __launch_bounds__(256) void value_append_kernel(const float *__restrict__ v, const float *__restrict__ bias, void *__restrict__ cache_v,
                                                            uint32_t kv_heads, uint32_t width, uint32_t capacity, const uint32_t *__restrict__ cursor,
                                                            uint32_t *refusal, uint32_t ring) {
+    NH_FETCH(v, bias, cache_v, kv_heads, width, capacity, cursor, refusal, ring, blockDim.x);
     const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
     if (index >= kv_heads * width) return;
     const uint32_t slot = ring ? cursor[0] % ring : cursor[0];
@@ -190,6 +191,7 @@ __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qk
                                                           void *__restrict__ cache_v, uint32_t capacity, uint32_t window,
                                                           const uint32_t *__restrict__ cursor, const uint8_t *__restrict__ mask,
                                                           const float *__restrict__ table, uint32_t *refusal, bool ring) {
+    NH_FETCH(qkv, heads, kv_heads, width, batch, rows, cache_k, cache_v, capacity, window, cursor, mask, table, refusal);
     const uint32_t half = width / 2;
     const uint32_t vectors = heads + 2 * kv_heads;  // per token: q heads, k heads, v heads
     const uint32_t stride = vectors * width;

@@ -143,6 +143,7 @@ constexpr int SECTION_WAVES = 8;  // 512 threads: four columns a thread
 __global__ __launch_bounds__(SECTION_WAVES * 64) void sample_sections_kernel(const float *__restrict__ logits, uint32_t n, uint32_t sections,
                                                                              const nh_draw *__restrict__ draws, uint64_t *__restrict__ kept,
                                                                              float *__restrict__ stats) {
+    NH_FETCH(logits, n, sections, draws, kept, stats);
     __shared__ uint64_t keys[SECTION_WAVES][CANDIDATES];
     __shared__ float room[SECTION_WAVES];
     const uint32_t row = blockIdx.y, section = blockIdx.x, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;

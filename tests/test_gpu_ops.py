@@ -399,6 +399,17 @@ def test_gemm_on_the_vector_unit_matches_too(device, monkeypatch, element, M, N,
     close(device.gemm(element, raw, N, K, X), oracle.gemm(element, raw, N, K, X.astype(np.float32), threads=8))
 
 
+@pytest.mark.parametrize("M,N,K,half", [(70, 130, 512, True), (512, 256, 3584, True), (33, 64, 256, False), (130, 300, 1024, False)])
+def test_q4_k_wide_product_with_weights_unpacked_into_lds(device, monkeypatch, M, N, K, half):
+    """NEURA_HIP_GEMM_REGB=0: the Q4_K wide product whose stager waves unpack the weights into LDS (the default form keeps a
+    lane's weight row in its registers); both are held to the same bar."""
+    monkeypatch.setenv("NEURA_HIP_GEMM_REGB", "0")
+    rng = np.random.default_rng(M * N + K)
+    raw = synth.RANDOM[NH_Q4_K](rng, N * K)
+    X = rng.standard_normal((M, K)).astype(np.float16 if half else np.float32)
+    close(device.gemm(NH_Q4_K, raw, N, K, X), oracle.gemm(NH_Q4_K, raw, N, K, X.astype(np.float32), threads=8))
+
+
 @pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K, NH_Q3_K])
 @pytest.mark.parametrize("M,N,K,half", [(70, 130, 512, False), (40, 64, 3584, True), (512, 256, 1280, True), (33, 200, 256, False),
                                         (130, 128, 768, True), (64, 256, 18944, False), (512, 512, 3584, False)])
