@@ -109,7 +109,6 @@ __device__ __forceinline__ void fetch_tile(u32x4 (&kraw)[T], u32x4 (&vraw)[T], c
 
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
-    fetch_parameters(p);
     constexpr int LPK = WIDTH / 8;                       // lanes per key in the score pass
     constexpr int KPW = 64 / LPK, STEP = 4 * KPW;        // keys per wave and per workgroup step
     constexpr int TK = 64, T = TK / STEP;                // keys and steps per tile
@@ -283,7 +282,6 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 // section s into its weight; then thread (channel, stripe) sums its channel over every eighth
 // section -- all of its loads in flight at once -- and the eight stripes meet in LDS.
 __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, uint32_t width) {
-    fetch_parameters(p);
     __shared__ float weights[256], masses[256], held[256], stripes[8][32];
     const uint32_t G = p.groups, tid = threadIdx.x;
     const uint32_t blocks = (width + 31u) / 32u;
@@ -526,7 +524,6 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 template <int WIDTH>
 __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionParams p) {
-    fetch_parameters(p);
     constexpr int TK = 32;                  // keys per tile
     constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output

@@ -285,7 +285,6 @@ struct DecodeTile {
 // once; scales: * 2^-24, undone once per pass), so a weight costs 1.6 vector instructions.
 template <int R, int G, bool PIPE, int NW, bool ROPE = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_decode_kernel(GemvParams p) {
-    fetch_parameters(p, ROPE);
     extern __shared__ float xs[];  // skew64(slice)
     __shared__ float red[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -632,7 +631,6 @@ struct Q8Tile {
 // 64 w + 63, and meet in LDS once a pass.
 template <int R, int G, bool DEEP = false, bool ROPE = false>
 __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
-    fetch_parameters(p, ROPE);
     static_assert(!DEEP || G == 64, "a deep row fills every wave");
     static_assert(!ROPE || (R == 2 && !DEEP), "the rotation pairs the two rows of a pass");
     extern __shared__ float xs[];  // skew32(K)
@@ -1052,11 +1050,6 @@ struct MfmaParams {
     float eps;
 };
 
-__device__ __forceinline__ void fetch_parameters(const MfmaParams &p) {
-    NH_FETCH(p.W[0], p.W[1], p.W[2], p.end[0], p.end[1], p.end[2], p.x, p.y, p.residual, p.norm_w, p.partial, p.N, p.K, p.row_bytes, p.nblk, p.slice_blocks,
-             p.splits, p.rows, p.tiles, p.swiglu, p.eps);
-}
-
 struct MfmaUnit {
     u32x4 hdr, qa, qb;
 };
@@ -1078,7 +1071,6 @@ __device__ __forceinline__ void digit_planes(uint32_t d0, uint32_t d1, uint32_t 
 
 template <int KS, int NW, int P, int D>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
-    fetch_parameters(p);
     extern __shared__ uint32_t xop[];  // [block][16 steps][4 groups][4 P digit columns] of 4 bytes; then sums; then tile partials
     __shared__ float red[256];
     __shared__ uint32_t wave_top[NW];
@@ -1387,7 +1379,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
 // waits count exactly how many loads are newer than the one needed.
 template <int NW, int D>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MfmaParams p) {
-    fetch_parameters(p);
     static_assert(D % 2 == 0, "the activation ring alternates between two slots");
     __shared__ __attribute__((aligned(16))) uint32_t digits[NW][256];  // [step][group][digit plane] per wave
     __shared__ float sums[NW][16];                                    // per wave: 8 sub-block sums, 8 sub-block unscales
@@ -1518,7 +1509,6 @@ struct Tile32Unit {
 
 template <int J, int NW, int KS>
 __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_kernel(MfmaParams p) {  // second bound: waves per SIMD
-    fetch_parameters(p);
 
     constexpr uint32_t M8 = 8 * J, R2 = 2 * J, TPW = NW / KS, NT = NW * 64;
     constexpr bool STAGED = J == 1;  // raw blocks through LDS; with eight activation rows the digits leave no room for them
@@ -1755,7 +1745,6 @@ constexpr uint32_t F16_BLOCK_PIECES = 8u * 4u * 16u + 2u * 16u;  // 16-byte piec
 
 template <int NW, int KS>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
-    fetch_parameters(p);
     constexpr uint32_t TPW = NW / KS, NT = NW * 64;
     static_assert(NT == 1024, "eight row groups of 128 threads stage the activations");
     extern __shared__ __attribute__((aligned(16))) uint32_t staged[];  // [block][F16_BLOCK_PIECES] pieces
@@ -2570,6 +2559,7 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
 
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (rows4_takes(a)) return launch_rows4(d, a);
     if (tile16_takes(a)) return launch_tile16(d, a);
     if (a.digits_out || a.digits_in) return fail(NH_E_ARGUMENT, "this product hands over no digit planes (ask gemv_hands_digits first)");
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");

@@ -159,5 +159,8 @@ inline int env_int(const char *name, int fallback) {
 // the 16-row tile kernel (gemv_tile16.hip): whether it serves this product, and its launch
 bool tile16_takes(const GemvArgs &args);
 int32_t launch_tile16(nh_device *d, const GemvArgs &args);
+// the same for two to eight activation rows, four rows to an MFMA
+bool rows4_takes(const GemvArgs &args);
+int32_t launch_rows4(nh_device *d, const GemvArgs &args);
 
 }  // namespace nh

@@ -401,7 +401,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * -16777216.0f;
         acc[0] = fmaf(d24, weighed, fmaf(m24, floor_, acc[0]));
     };
-    // R > 1: the weights are unpacked once, the next fetch goes out, and every row then runs its four MFMAs and its weighing
+    // R > 1: the weights are unpacked once, the next fetch goes out, and every row then runs its four MFMAs and its weighing.
+    // Only the twelve lanes that feed the matrix cores read their operands from LDS; the other lanes' operand registers are
+    // cleared once and never written again (a read by all 64 lanes costs LDS eight clocks a time, most of them for zeros).
+    constexpr int G = R < 4 ? R : (NW > 8 ? 2 : 4);  // rows a phase; sixteen waves a workgroup leave a wave 128 registers
+    i32x4 a[G][4];
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) a[g][k] = i32x4{0, 0, 0, 0};
     auto step_rows = [&](Tile16Unit &u, uint32_t b) {
         const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
         const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
@@ -415,25 +423,48 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
         __builtin_amdgcn_sched_barrier(0);
         fetch(u);
         __builtin_amdgcn_sched_barrier(0);
-        const uint8_t *at = abase + (size_t)b * astride;
-        const f32x4 *s = sums + b * 4u + q;
+        // Rows go four at a time through three phases -- every operand read from LDS, every MFMA, every weighing -- so that
+        // a row's reads and matrix-core results are waited for behind the other rows' work, not one row after another.
 #pragma unroll
-        for (int row = 0; row < R; row++) {
-            const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
-            const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
-            const f32x4 rs = *s;
-            i32x4 cl = {0, 0, 0, 0}, ch = {0, 0, 0, 0};
-            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a00, la, cl, 0, 0, 0);
-            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a10, ha, ch, 0, 0, 0);
-            cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a01, lb, cl, 0, 0, 0);
-            ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a11, hb, ch, 0, 0, 0);
-            const float fl = fmaf((float)((cl[0] << 8) + cl[1]), 256.0f, (float)cl[2]);
-            const float fh = fmaf((float)((ch[0] << 8) + ch[1]), 256.0f, (float)ch[2]);
-            const float weighed = fmaf(scx, fl, scy * fh);
-            const float floor_ = fmaf(mnx, rs.x, mny * rs.y);
-            acc[row] = fmaf(d24 * rs.z, weighed, fmaf(m24, floor_, acc[row]));
-            at += arow;
-            s += nblk * 4u;
+        for (int first = 0; first < R; first += G) {
+            const uint8_t *at = abase + (size_t)b * astride + (size_t)first * arow;
+            const f32x4 *s = sums + b * 4u + q + (size_t)first * nblk * 4u;
+            i32x4 cl[G], ch[G];
+            f32x4 rs[G];
+            if (feeds) {
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    const uint8_t *from = at + (size_t)g * arow;
+                    a[g][0] = *reinterpret_cast<const i32x4 *>(from), a[g][1] = *reinterpret_cast<const i32x4 *>(from + 48);
+                    a[g][2] = *reinterpret_cast<const i32x4 *>(from + 96), a[g][3] = *reinterpret_cast<const i32x4 *>(from + 144);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                rs[g] = *s;
+                s += nblk * 4u;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const i32x4 none = {0, 0, 0, 0};
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                cl[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g][0], la, none, 0, 0, 0);
+                ch[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g][2], ha, none, 0, 0, 0);
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                cl[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g][1], lb, cl[g], 0, 0, 0);
+                ch[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g][3], hb, ch[g], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float fl = fmaf((float)((cl[g][0] << 8) + cl[g][1]), 256.0f, (float)cl[g][2]);
+                const float fh = fmaf((float)((ch[g][0] << 8) + ch[g][1]), 256.0f, (float)ch[g][2]);
+                const float weighed = fmaf(scx, fl, scy * fh);
+                const float floor_ = fmaf(mnx, rs[g].x, mny * rs[g].y);
+                acc[first + g] = fmaf(d24 * rs[g].z, weighed, fmaf(m24, floor_, acc[first + g]));
+            }
         }
     };
     // The wave that finishes a tile (sums the waves' parts, runs the epilogue) changes from tile to tile (with SwiGLU from pair
@@ -548,6 +579,356 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Two to eight activation rows against a Q4_K matrix, four rows to an MFMA, the sub-block scales inside the operand.
+//
+// The block-diagonal operand above spends a whole MFMA on one activation row (its A rows are slices of that row), so every
+// further row costs four more of them: measured, 4.7 us a row on gate|up, all of it matrix-core time.  Here the sixteen A rows
+// are (activation row, digit plane) pairs -- row m = 4 i + plane, four activation rows an instruction -- and an MFMA's K runs
+// over a whole 64-element group, which it may because the weights enter already multiplied by their sub-block's scale: a six-
+// bit scale is sc = 8 hi + lo with hi, lo < 8, and nibble * hi and nibble * lo (at most 105) are both bytes, so two MFMAs a
+// group, accumulated over the four groups of a super-block, leave 8 * C_hi + C_lo = sum of digit * nibble * sc in integers, exact.
+// One multiplication makes four such bytes (a word of nibbles times hi or lo: no byte carries into the next).  What is left to
+// fp32 per super-block and activation row is one conversion of the three plane sums, the activation scale and d; the minimums
+// come off against sub-block sums as in the one-row kernel.  The activations' power-of-two scale is a super-block's here, not
+// a 64-element group's (the digits of a super-block meet in one integer sum): 22 bits below the largest magnitude of 256.
+// Lane (r, s) = (lane % 16, lane / 16) supplies, for every group, the eight bytes 8 s .. 8 s + 7 of weight row r -- low nibbles
+// elements 8 s .., high nibbles elements 32 + 8 s .. -- and the digit planes are staged in that order (slot 16 s + 8 half + t of
+// a group's 64), so an operand is one aligned 16-byte read; it receives C column r, rows 4 s .. 4 s + 3: the three plane sums
+// of activation row s against ITS weight row, so again no sum crosses lanes.  A wave turns into digits exactly the
+// super-blocks it walks, all rows' activations asked for at once.  Launched for three and four rows (P = 1): there it beats
+// the block-diagonal form by 13 % a layer (gate|up 25.9 against 30.7 us); at two rows that form is ahead (21.8 against 23.7),
+// and two passes over the unpacked weights (P = 2, rows 0..3 then 4..7) tie with the 32-row and half-precision tiles at five
+// to eight rows (gate|up 34 against 36 us, the plain products 16 against 14) -- turning eight rows into digits in every
+// workgroup (6.6 us) is what bounds them -- so those keep their kernels.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+struct Rows4Unit {
+    u32x4 hdr;
+    u32x2 w[4];
+};
+
+static size_t rows4_row_stride(uint32_t nblk) {
+    const size_t bytes = (size_t)nblk * TILE16_BLOCK_DIGITS + 64u;  // the idle A rows (plane 3) read 64 bytes past a group
+    return (bytes + 255u) / 256u * 256u + 64u;  // rows 64 bytes apart modulo the banks' 256: the four rows of an operand read spread over them
+}
+static size_t rows4_lds(uint32_t nblk, uint32_t NW, uint32_t rows) {
+    return rows * rows4_row_stride(nblk) + (size_t)rows * nblk * 48u + (size_t)2 * NW * 64u * (rows / 4u) * 4u + (size_t)NW * rows * 4u + 64u;
+}
+
+template <int NW, int D, int MODE, int P>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_rows4_kernel(GemvParams p) {
+    static_assert(MODE == TILE16_PLAIN || MODE == TILE16_SWIGLU, "no rotation is folded into a product of several rows");
+    extern __shared__ __attribute__((aligned(16))) uint8_t rows4_lds_bytes[];
+    constexpr uint32_t NT = NW * 64, ROWS = 4 * P;
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+    typedef const __attribute__((address_space(1))) u32x2 *global_uint2;
+    fetch_parameters(p);
+    asm volatile("" ::"s"(gridDim.x));
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t nblk = p.nblk;
+    const uint32_t row_stride = (uint32_t)(((size_t)nblk * TILE16_BLOCK_DIGITS + 64u + 255u) / 256u * 256u + 64u);
+    uint8_t *const digits = rows4_lds_bytes;
+    float *const sums = reinterpret_cast<float *>(rows4_lds_bytes + (size_t)ROWS * row_stride);  // [row][block][8 sums, 4 scales]
+    float *const part = sums + (size_t)ROWS * nblk * 12u;                                          // [parity][wave][pass][lane]
+    float *const red = part + 2u * NW * P * 64u;                                                   // [wave][row]
+    const uint32_t r = lane & 15u, s = lane >> 4;
+    const uint32_t tiles = p.row_groups;
+    if (blockIdx.x >= tiles) return;
+    const uint32_t ntiles = (tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;
+    const uint32_t rows = min(p.rows, ROWS);
+
+    const uint8_t *const w0 = p.W[0];
+    const int64_t to_w1 = p.W[1] - p.W[0], to_w2 = p.W[2] - p.W[0];
+    const uint32_t end0 = p.end[0], end1 = p.end[1], row_bytes = p.row_bytes;
+    const uint32_t first_tile = blockIdx.x, hop = gridDim.x;
+    const uint32_t tile_rows = MODE == TILE16_PLAIN ? p.tile_rows : 16u;
+    auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, tile_rows, r, s](uint32_t tile) -> const uint8_t * {
+        (void)tile_rows;
+        int64_t offset;
+        if (MODE == TILE16_SWIGLU) {
+            offset = ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((tile >> 1) * 16u + r) * row_bytes;
+        } else {
+            const uint32_t n = tile * tile_rows + min(r, tile_rows - 1u);
+            const bool in0 = n < end0, in1 = n < end1;
+            const int64_t matrix = in0 ? (int64_t)0 : (in1 ? to_w1 : to_w2);
+            const uint32_t before = in0 ? 0u : (in1 ? end0 : end1);
+            offset = matrix + (int64_t)(n - before) * row_bytes;
+        }
+        return w0 + offset + s * 8u;
+    };
+    auto tile_at = [first_tile, hop](uint32_t i) -> uint32_t {
+        if (MODE == TILE16_SWIGLU) return 2u * (first_tile + (i >> 1) * hop) + (i & 1u);
+        return first_tile + i * hop;
+    };
+    const uint32_t walked = MODE == TILE16_SWIGLU ? 2u * ntiles : ntiles;
+
+    Rows4Unit ring[D];
+    uint32_t ahead_tile = 0, ahead_b = wave;
+    const uint8_t *ahead_row = lane_row(tile_at(0));
+    auto fetch = [&](Rows4Unit &u) {
+        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * 144u;
+        u.hdr = *(global_uint4)(uintptr_t)(at - s * 8u);
+#pragma unroll
+        for (int g = 0; g < 4; g++) u.w[g] = *(global_uint2)(uintptr_t)(at + 16u + 32u * g);
+        if (ahead_b + NW < nblk) {
+            ahead_b += NW;
+        } else if (ahead_tile + 1u < walked) {
+            ahead_b = wave;
+            ahead_tile++;
+            ahead_row = lane_row(tile_at(ahead_tile));
+        }
+    };
+#pragma unroll
+    for (int i = 0; i < D; i++) fetch(ring[i]);
+
+    // ---- activations -> digit planes: unit e4 = tid + NT * j (four consecutive activations) lies in super-block wave + NW * j
+    {
+        const uint32_t units = p.K / 4u;
+        auto stage = [&](uint32_t row, uint32_t e4, f32x4 v, f32x4 w, float rms) {
+            if (p.norm_w) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
+            }
+            uint32_t top = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float element = v[i];
+                top = max(top, __builtin_bit_cast(uint32_t, element) & 0x7fffffffu);
+            }
+            // the largest magnitude of the super-block: its 64 units are the 64 lanes of this wave
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
+            top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
+            top = max(top, (uint32_t)__builtin_amdgcn_ds_swizzle((int)top, 0x401F));  // lane ^ 16
+            top = max(top, (uint32_t)__shfl_xor((int)top, 32, 64));
+            const uint32_t raw = top >> 23;
+            const uint32_t exponent = min(max(raw, 22u), 254u);
+            const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);
+            const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
+            float total = 0.0f;
+            uint32_t dg[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float rounded = rintf(v[i] * scale);
+                total += rounded;
+                dg[i] = signed_digits((int)rounded);
+            }
+            const uint32_t lo01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(dg[1], dg[0], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(dg[3], dg[2], 0x07030602u);
+            const uint32_t plane2 = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);  // least significant digits
+            const uint32_t plane1 = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+            const uint32_t plane0 = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  // most significant
+            total += dpp<DPP_QUAD_XOR1>(total);
+            total += dpp<DPP_QUAD_XOR2>(total);
+            total += dpp<0x141>(total);  // the other quad of the eight lanes of a sub-block
+            // unit e4: 64 a super-block, 16 a group, 8 a sub-block.  Elements e = 4 (e4 % 16) .. + 3 of their group sit in slot
+            // 16 ((e % 32) / 8) + 8 (e / 32) + e % 8 of the group's 64: the order the weights' bytes unpack in
+            const uint32_t e = 4u * (e4 & 15u);
+            const uint32_t seat = 16u * ((e & 31u) >> 3) + 8u * (e >> 5) + (e & 7u);
+            uint8_t *group = digits + (size_t)row * row_stride + (size_t)(e4 >> 6) * TILE16_BLOCK_DIGITS + ((e4 >> 4) & 3u) * 192u + seat;
+            *reinterpret_cast<uint32_t *>(group) = plane0, *reinterpret_cast<uint32_t *>(group + 64) = plane1, *reinterpret_cast<uint32_t *>(group + 128) = plane2;
+            float *held = sums + (size_t)row * nblk * 12u + (size_t)(e4 >> 6) * 12u;
+            if ((e4 & 7u) == 0) held[(e4 >> 3) & 7u] = total * unscale;
+            if ((e4 & 63u) == 0) held[8] = unscale;
+        };
+        constexpr int MAXJ = 2;
+        if (units <= MAXJ * NT) {
+            // every row's activations are asked for at once and wait in registers: a row at a time pays a round trip to the
+            // cache a row
+            f32x4 held[ROWS][MAXJ], weight[MAXJ];
+#pragma unroll
+            for (int row = 0; row < (int)ROWS; row++)
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    held[row][j] = (uint32_t)row < rows && e4 < units ? *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            float rms[ROWS];
+#pragma unroll
+            for (int row = 0; row < (int)ROWS; row++) rms[row] = 1.0f;
+            if (p.norm_w) {
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    weight[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+#pragma unroll
+                for (int row = 0; row < (int)ROWS; row++) {
+                    float square = 0.0f;  // the row's sum of squares, thread by thread in the order the row-at-a-time loop adds them
+#pragma unroll
+                    for (int j = 0; j < MAXJ; j++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(held[row][j][i], held[row][j][i]));
+                    square = wave_sum(square);
+                    if (lane == 0) red[wave * ROWS + row] = square;
+                }
+                __syncthreads();
+#pragma unroll
+                for (int row = 0; row < (int)ROWS; row++) {
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < NW; w++) total += red[w * ROWS + row];
+                    rms[row] = rms_scale_of(total, p.K, p.eps);
+                }
+            }
+#pragma unroll
+            for (int row = 0; row < (int)ROWS; row++) {
+                if ((uint32_t)row >= rows) break;
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    if (e4 < units) stage(row, e4, held[row][j], weight[j], rms[row]);  // whole groups of 16 lanes are in or out together
+                }
+            }
+        } else {
+            if (p.norm_w) {
+                for (uint32_t row = 0; row < rows; row++) {
+                    float square = 0.0f;
+                    for (uint32_t e4 = tid; e4 < units; e4 += NT) {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
+                    }
+                    square = wave_sum(square);
+                    if (lane == 0) red[wave * ROWS + row] = square;
+                }
+                __syncthreads();
+            }
+            for (uint32_t row = 0; row < rows; row++) {
+                float rms = 1.0f;
+                if (p.norm_w) {
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < NW; w++) total += red[w * ROWS + row];
+                    rms = rms_scale_of(total, p.K, p.eps);
+                }
+                for (uint32_t e4 = tid; e4 < units; e4 += NT)
+                    stage(row, e4, *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4),
+                          p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms);
+            }
+        }
+    }
+    __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see this wave's writes
+
+    // ---- the walk.  A row m = 4 i + plane of pass `pass` is activation row 4 pass + i; lane (m, s) reads digits 16 s .. of a group
+    const uint32_t m = lane & 15u;
+    const uint8_t *const abase = digits + (size_t)(m >> 2) * row_stride + (m & 3u) * 64u + s * 16u;
+    const float *const sbase = sums + (size_t)s * nblk * 12u;  // this lane's activation row of pass 0 is row s
+    float acc[P], gate[P];
+#pragma unroll
+    for (int i = 0; i < P; i++) acc[i] = 0.0f, gate[i] = 0.0f;
+    uint32_t parity = 0;
+    auto step = [&](Rows4Unit &u, uint32_t b) {
+        // the eight scales and minimums of the row (crates/neura-precision/src/ggml.rs:127-136), four to a word
+        const uint32_t sc_words[2] = {u.hdr.y & 0x3f3f3f3fu, (u.hdr.w & 0x0f0f0f0fu) | ((u.hdr.y >> 2) & 0x30303030u)};
+        const uint32_t mn_words[2] = {u.hdr.z & 0x3f3f3f3fu, ((u.hdr.w >> 4) & 0x0f0f0f0fu) | ((u.hdr.z >> 2) & 0x30303030u)};
+        // the lane's weights times their scale's two digits, a group an operand: bytes 0..7 the low nibbles (sub-block 2 g),
+        // bytes 8..15 the high ones (sub-block 2 g + 1)
+        i32x4 high_part[4], low_part[4];
+        float mn[8];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t word = sc_words[g >> 1], shift = 16u * (g & 1u);
+            const uint32_t hi_a = (word >> (shift + 3u)) & 7u, lo_a = (word >> shift) & 7u;            // sub-block 2 g
+            const uint32_t hi_b = (word >> (shift + 11u)) & 7u, lo_b = (word >> (shift + 8u)) & 7u;    // sub-block 2 g + 1
+            const uint32_t n0 = u.w[g].x & 0x0f0f0f0fu, n1 = u.w[g].y & 0x0f0f0f0fu;
+            const uint32_t n2 = (u.w[g].x >> 4) & 0x0f0f0f0fu, n3 = (u.w[g].y >> 4) & 0x0f0f0f0fu;
+            // a word of four nibbles times a digit below 8, as two packed 16-bit products: no byte carries into the next
+            // (a full 32-bit multiplication runs at a quarter of the rate)
+            typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+            auto times = [](uint32_t nibbles, uint32_t digit) -> int {
+                const u16x2 both = {(uint16_t)digit, (uint16_t)digit};
+                return __builtin_bit_cast(int, __builtin_bit_cast(u16x2, nibbles) * both);
+            };
+            high_part[g] = i32x4{times(n0, hi_a), times(n1, hi_a), times(n2, hi_b), times(n3, hi_b)};
+            low_part[g] = i32x4{times(n0, lo_a), times(n1, lo_a), times(n2, lo_b), times(n3, lo_b)};
+            mn[2 * g] = (float)((mn_words[g >> 1] >> shift) & 0xffu), mn[2 * g + 1] = (float)((mn_words[g >> 1] >> (shift + 8u)) & 0xffu);
+        }
+        const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);
+        float scale_d = (float)dd.x, scale_m = -(float)dd.y;
+        asm volatile("" : "+v"(scale_d), "+v"(scale_m));  // the header is read by here
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(u);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pass = 0; pass < P; pass++) {
+            const uint8_t *at = abase + (size_t)pass * 4u * row_stride + (size_t)b * TILE16_BLOCK_DIGITS;
+            const float *held = sbase + (size_t)pass * 4u * nblk * 12u + (size_t)b * 12u;
+            i32x4 a[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) a[g] = *reinterpret_cast<const i32x4 *>(at + 192 * g);
+            const f32x4 s0 = *reinterpret_cast<const f32x4 *>(held), s1 = *reinterpret_cast<const f32x4 *>(held + 4);
+            const float unscale = held[8];
+            i32x4 ch = {0, 0, 0, 0}, cl = {0, 0, 0, 0};
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                ch = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g], high_part[g], ch, 0, 0, 0);
+                cl = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[g], low_part[g], cl, 0, 0, 0);
+            }
+            // plane sums of digit * nibble * scale, below 2^25 each; the three planes meet in fp32
+            const float t0 = (float)(8 * ch[0] + cl[0]), t1 = (float)(8 * ch[1] + cl[1]), t2 = (float)(8 * ch[2] + cl[2]);
+            const float weighed = fmaf(fmaf(t0, 256.0f, t1), 256.0f, t2) * unscale;
+            float floor_ = mn[0] * s0[0];
+            floor_ = fmaf(mn[1], s0[1], floor_), floor_ = fmaf(mn[2], s0[2], floor_), floor_ = fmaf(mn[3], s0[3], floor_);
+            floor_ = fmaf(mn[4], s1[0], floor_), floor_ = fmaf(mn[5], s1[1], floor_), floor_ = fmaf(mn[6], s1[2], floor_), floor_ = fmaf(mn[7], s1[3], floor_);
+            acc[pass] = fmaf(scale_d, weighed, fmaf(scale_m, floor_, acc[pass]));
+        }
+    };
+    // lane (r, s) holds output r of activation rows s (pass 0) and 4 + s (pass 1): the waves' parts meet in LDS, and the wave
+    // whose turn it is sums them and runs the epilogue
+    auto tile_end = [&](uint32_t tile, uint32_t index) {
+        const uint32_t finisher = (MODE == TILE16_SWIGLU ? index >> 1 : index) % NW;
+#pragma unroll
+        for (int pass = 0; pass < P; pass++) {
+            part[((parity * NW + wave) * P + pass) * 64u + lane] = acc[pass];
+            acc[pass] = 0.0f;
+        }
+        __syncthreads();
+        if (wave == finisher) {
+#pragma unroll
+            for (int pass = 0; pass < P; pass++) {
+                const uint32_t row = 4u * pass + s;
+                float total = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NW; w++) total += part[((parity * NW + w) * P + pass) * 64u + lane];
+                if (row >= rows) continue;
+                if (MODE == TILE16_SWIGLU) {
+                    if (tile & 1u) p.y[(size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r] = silu(gate[pass]) * total;
+                    else gate[pass] = total;
+                } else if (r < tile_rows) {
+                    const size_t n = (size_t)row * p.N + tile * tile_rows + r;
+                    if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);
+                    else p.y[n] = p.residual ? p.residual[n] + total : total;
+                }
+            }
+        }
+        parity ^= 1u;
+    };
+    if (count == 0) {
+        for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t), t);
+        return;
+    }
+    uint32_t at_tile = 0, at_b = wave;
+    const uint32_t steps = walked * count;
+    for (uint32_t s0 = 0; s0 < steps; s0 += D) {
+#pragma unroll
+        for (int slot = 0; slot < D; slot++) {
+            step(ring[slot], at_b);
+            at_b += NW;
+            if (at_b >= nblk) {
+                if (at_tile < walked) tile_end(tile_at(at_tile), at_tile);
+                at_b = wave;
+                at_tile++;
+            }
+        }
+    }
+}
+
 // ---- the 16-row tile kernel (one activation row, Q4_K)
 // NEURA_HIP_TILE16=0 keeps it out (the vector and the other matrix-core forms then take one row as before), as does a forced
 // NEURA_HIP_MFMA form.  Otherwise it takes every Q4_K product of one row whose matrices end on tile boundaries, and of two
@@ -592,6 +973,79 @@ bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer) {
     if (!tile16_takes(from) || !tile16_takes(to)) return false;
     const uint32_t nblk = to.K / 256u;
     return tile16_lds(nblk, nblk > 32u ? 16u : 8u, 1u, true) <= 160u * 1024u;
+}
+
+// ---- three and four rows, four to an MFMA.  NEURA_HIP_ROWS4=0 keeps the kernel out, as does any other form forced by its switch.
+bool rows4_takes(const GemvArgs &a) {
+    if (a.element != NH_Q4_K || a.rows < 3 || a.rows > 4 || a.K % 256u != 0 || a.K == 0 || a.rope || a.digits_in || a.digits_out) return false;
+    if (env_int("NEURA_HIP_ROWS4", 1) == 0 || env_int("NEURA_HIP_TILE16", 1) == 0 || env_int("NEURA_HIP_MFMA", 1) != 1) return false;
+    if (env_int("NEURA_HIP_MFMA32", 1) == 2 || env_int("NEURA_HIP_F16_TILES", 1) == 2 || env_int("NEURA_HIP_TILE16_ROWS", 8) < (int)a.rows) return false;
+    if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
+    if (a.N < 16u || a.N % 16u != 0) return false;
+    if (a.swiglu) {
+        if (a.residual || a.end[0] != a.N / 2 || (a.N / 2) % 16u != 0) return false;
+    } else if (a.end[0] % 16u != 0 || a.end[1] % 16u != 0) {
+        return false;
+    }
+    return rows4_lds(a.K / 256u, 8u, 4u) <= 160u * 1024u;
+}
+
+template <int NW, int MODE, int P>
+static hipError_t launch_rows4_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
+    static bool raised = false;
+    if (!raised && lds > 64u * 1024u) {
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_rows4_kernel<NW, 2, MODE, P>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (error != hipSuccess) return error;
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemv_q4k_rows4_kernel<NW, 2, MODE, P>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    return hipGetLastError();
+}
+
+template <int MODE, int P>
+static hipError_t launch_rows4_waves(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
+    switch (waves) {
+    case 4: return launch_rows4_instance<4, MODE, P>(d, p, grid, lds);
+    case 7: return launch_rows4_instance<7, MODE, P>(d, p, grid, lds);
+    default: return launch_rows4_instance<8, MODE, P>(d, p, grid, lds);
+    }
+}
+
+int32_t launch_rows4(nh_device *d, const GemvArgs &a) {
+    GemvParams p{};
+    for (int s = 0; s < 3; s++) {
+        p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
+        p.end[s] = a.end[s];
+    }
+    p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
+    p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps, p.rows = a.rows;
+    p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
+    p.nblk = a.K / 256u;
+    const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : 8u);
+    // tiles and rounds as the one-row kernel deals them: a plain tile holds the number of rows, 16 down to 12, that leaves the
+    // fewest compute units idle in the last round
+    p.tile_rows = 16;
+    if (!a.swiglu) {
+        auto idle = [&](uint32_t rows) {
+            const uint32_t tiles = a.N / rows, rounds = (tiles + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
+            return 65536u - (uint32_t)((uint64_t)tiles * 65536u / ((uint64_t)rounds * (uint32_t)d->compute_units));
+        };
+        for (uint32_t rows = 15; rows >= 12; rows--) {
+            if (a.N % rows || a.end[0] % rows || a.end[1] % rows) continue;
+            if (idle(rows) + 3277u < idle(p.tile_rows)) p.tile_rows = rows;
+        }
+    }
+    const uint32_t units = a.swiglu ? a.N / 32u : a.N / p.tile_rows;
+    p.row_groups = units;
+    const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
+    const uint32_t grid = (units + rounds - 1u) / rounds;
+    const size_t lds = rows4_lds(p.nblk, waves, 4u);
+    profile_mark(d);
+    hipError_t launched = a.swiglu ? launch_rows4_waves<TILE16_SWIGLU, 1>(d, p, waves, grid, lds) : launch_rows4_waves<TILE16_PLAIN, 1>(d, p, waves, grid, lds);
+    NH_HIP(launched);
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
 }
 
 template <int NW, int D, int MODE, int R, bool HANDED = false>

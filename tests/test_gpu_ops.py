@@ -255,11 +255,13 @@ def test_q4_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K)
 
 @pytest.mark.parametrize("N,K,rows", [(16, 256, 2), (64, 3584, 4), (4608, 3584, 4), (3584, 3584, 3), (4608, 3584, 2), (1040, 768, 4), (48, 2048, 3),
                                       (272, 8960, 4), (96, 18944, 2), (37888, 3584, 4), (64, 10240, 3), (152064, 3584, 2)])
-def test_q4_k_products_of_a_few_rows_on_16_row_tiles(device, N, K, rows):
-    """Two to four activation rows against Q4_K rows in one pass of the 16-row tiles (every row its own digit planes, the
+def test_q4_k_products_of_a_few_rows_on_16_row_tiles(device, monkeypatch, N, K, rows):
+    """(NEURA_HIP_ROWS4=0: the form that serves where the kernel with four rows to an MFMA does not fit.)
+    Two to four activation rows against Q4_K rows in one pass of the 16-row tiles (every row its own digit planes, the
     weights unpacked once a step): each row is, bit for bit, what the one-row product gives for it alone, plain, with a
     residual and with SwiGLU (the decoders' batches run it with the norm folded in); and the whole sits as close to the exact
     product as the oracle does.  A non-finite number stays in its own row."""
+    monkeypatch.setenv("NEURA_HIP_ROWS4", "0")
     rng = np.random.default_rng(N + K + rows)
     raw = synth.q4_k_random(rng, N * K)
     x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-2, 2, (rows, K)))).astype(np.float32)
@@ -283,6 +285,49 @@ def test_q4_k_products_of_a_few_rows_on_16_row_tiles(device, N, K, rows):
     x[0, 5] = np.inf
     spoilt = device.gemv(NH_Q4_K, raw, N, K, x)
     assert not np.isfinite(spoilt[0]).any() and np.array_equal(spoilt[1:], got[1:])
+
+
+@pytest.mark.parametrize("N,K,rows", [(16, 256, 3), (64, 3584, 4), (4608, 3584, 4), (3584, 3584, 3), (4608, 3584, 3), (1040, 768, 4), (48, 2048, 3),
+                                      (272, 8960, 4), (37888, 3584, 4), (37888, 3584, 3), (64, 10240, 3), (152064, 3584, 3)])
+def test_q4_k_products_of_several_rows_four_rows_to_an_mfma(device, N, K, rows):
+    """Three and four activation rows against Q4_K rows, four activation rows in an MFMA's sixteen operand rows and the
+    sub-block scales inside the weight operand: within the product's bar of the oracle and as close to the exact product as the oracle is, plain, with a residual
+    and with SwiGLU; a row's numbers do not depend on the rows beside it (bit for bit what it gives next to rows of zeros),
+    and a non-finite number stays in its own row."""
+    rng = np.random.default_rng(N + K + rows)
+    raw = synth.q4_k_random(rng, N * K)
+    x = (rng.standard_normal((rows, K)) * np.exp(rng.uniform(-2, 2, (rows, K)))).astype(np.float32)
+    r = rng.standard_normal((rows, N)).astype(np.float32)
+    small = N * K <= 4608 * 3584
+    if small:
+        plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+        close(device.gemv(NH_Q4_K, raw, N, K, x), plain)
+        tight(device.gemv(NH_Q4_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    x[rows - 1, rng.integers(0, K, 8)] *= 1e3  # with outliers the oracle's own fp32 sums are the looser side: the exact product judges
+    got = device.gemv(NH_Q4_K, raw, N, K, x)
+    if small:
+        plain = oracle.gemv(NH_Q4_K, raw, N, K, x, threads=8)
+        exact = oracle.unpack(NH_Q4_K, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64).T
+        # the digits' scale is a super-block's here: an outlier costs its 255 neighbours the bits it stands above them
+        assert np.abs(got - exact.T).max() <= max(4 * np.abs(plain - exact.T).max(), 8e-6 * max(1.0, np.abs(exact).max()))
+        if N % 32 == 0:
+            gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2 :].astype(np.float64)
+            want = gate / (1.0 + np.exp(-gate)) * up
+            close(device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
+    with_residual = device.gemv(NH_Q4_K, raw, N, K, x, residual=r)
+    gated = device.gemv(NH_Q4_K, raw, N, K, x, swiglu=True) if N % 32 == 0 else None
+    for row in range(rows):
+        beside_zeros = np.concatenate([x[row : row + 1], np.zeros((2, K), np.float32)])
+        assert np.array_equal(got[row], device.gemv(NH_Q4_K, raw, N, K, beside_zeros)[0]), row
+        assert np.array_equal(with_residual[row], device.gemv(NH_Q4_K, raw, N, K, beside_zeros, residual=np.stack([r[row], r[row], r[row]]))[0]), row
+        if gated is not None:
+            assert np.array_equal(gated[row], device.gemv(NH_Q4_K, raw, N, K, beside_zeros, swiglu=True)[0]), row
+    # one row through the one-row kernel: the same numbers to the last few bits
+    tight(got[0:1], device.gemv(NH_Q4_K, raw, N, K, x[0:1]), 8e-6)
+    x[0, 5] = np.inf
+    spoilt = device.gemv(NH_Q4_K, raw, N, K, x)
+    assert not np.isfinite(spoilt[0]).any() and np.array_equal(spoilt[1:], got[1:])
+    assert np.array_equal(device.gemv(NH_Q4_K, raw, N, K, np.zeros((rows, K), np.float32)), np.zeros((rows, N), np.float32))
 
 
 def test_q4_k_product_on_the_matrix_cores_keeps_non_finite_inputs_visible(device, monkeypatch):
