@@ -508,6 +508,32 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         held.release()
 
 
+def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch):
+    """At batch 1 the gate|up product of a Q4_K decoder leaves silu(gate) * up as the digit planes ffn_down multiplies (a
+    power-of-two scale per 16 outputs where ffn_down's own staging takes one per 64); NEURA_HIP_TILE16_HANDED=0 hands the
+    floats on instead.  Both stay within the decoder's bar of the oracle and of each other (a difference in the last bits of
+    a key now and then flips its rounding to half, 5e-4 of it) and choose the same tokens."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    handed, ref, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11)
+    floats, _, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11)
+    token = 7
+    for step in range(8):
+        monkeypatch.setenv("NEURA_HIP_TILE16_HANDED", "1")
+        got_a = handed.decode_step([token], [step])
+        logits_a = handed.logits()
+        monkeypatch.setenv("NEURA_HIP_TILE16_HANDED", "0")
+        got_b = floats.decode_step([token], [step])
+        logits_b = floats.logits()
+        want_logits, want = ref.forward([token], 1, [step])
+        scale = np.abs(want_logits).max()
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * scale and np.abs(logits_b - want_logits).max() <= 1e-3 * scale, step
+        assert np.abs(logits_a - logits_b).max() <= 1e-3 * scale, step
+        assert list(got_a) == list(got_b) == list(want), (step, margins(want_logits))
+        token = int(got_a[0])
+    for held in (handed, floats, weights_a, weights_b):
+        held.release()
+
+
 def test_decoders_of_different_rope_bases_step_in_turn(device):
     """Two decoders of different rope bases and head widths stepping alternately at batch 2 (the rotation as its own
     kernel, read from the device's table of inverse frequencies): each keeps answering from its own recorded step as the
