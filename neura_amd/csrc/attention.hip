@@ -281,29 +281,33 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 // One workgroup per (unit, group, block of 32 channels).  Thread s first turns the statistics of
 // section s into its weight; then thread (channel, stripe) sums its channel over every eighth
 // section -- all of its loads in flight at once -- and the eight stripes meet in LDS.
-__global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, uint32_t width) {
+// (The leading arguments are what the first loads need: the hardware hands them to a wave in scalar registers as it starts.)
+__global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_partial, uint32_t lead_sections, uint32_t lead_groups, uint32_t width,
+                                                             AttentionParams p) {
     __shared__ float weights[256], masses[256], held[256], stripes[8][32];
-    const uint32_t G = p.groups, tid = threadIdx.x;
+    const uint32_t G = lead_groups, tid = threadIdx.x, sections = lead_sections;
     const uint32_t blocks = (width + 31u) / 32u;
     const uint32_t cblock = blockIdx.x % blocks, ug = blockIdx.x / blocks;
     const uint32_t unit = ug / G, g = ug % G;
-    const uint32_t row = unit % p.rows;
-    const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
-    const float *src = p.partial + ((uint64_t)unit * p.sections * G + g) * (width + 2);
-    const uint64_t hop = (uint64_t)G * (width + 2);  // one section further
+    const float *src = lead_partial + ((uint64_t)unit * sections * G + g) * (width + 2);
+    const uint32_t hop = G * (width + 2u);  // one section further (a unit's partials are far fewer than 2^32 numbers)
     float top = -INFINITY, mass = 0.0f;
-    if (tid < p.sections) {
-        top = src[tid * hop + width];
-        mass = src[tid * hop + width + 1];
+    {
+        const float *stats = src + min(tid, sections - 1u) * hop + width;
+        const float read_top = stats[0], read_mass = stats[1];
+        if (tid < sections) top = read_top, mass = read_mass;
     }
-    // the channel sums do not wait for the weights: fetch first
+    // the channel sums do not wait for the weights: fetch first.  Every load is issued whatever its section (past the last
+    // one it reads the last again and is dropped): loads under a condition each got a branch of their own, and the address
+    // arithmetic between them waited for the loads before -- eight round trips one after another where one is enough.
     const uint32_t c = cblock * 32u + (tid & 31u), stripe = tid >> 5;
+    const float *column = src + min(c, width - 1u);
     float values[32];
 #pragma unroll
-    for (int j = 0; j < 32; j++) {
-        const uint32_t s = stripe + 8u * j;
-        values[j] = (s < p.sections && c < width) ? src[s * hop + c] : 0.0f;
-    }
+    for (int j = 0; j < 32; j++) values[j] = column[min(stripe + 8u * j, sections - 1u) * hop];
+#pragma unroll
+    for (int j = 0; j < 32; j++)
+        if (stripe + 8u * j >= sections || c >= width) values[j] = 0.0f;
     // the largest top and the weighed mass: a wave each, then the four waves' words
     const float wave_top = wave_max(top);
     if ((tid & 63u) == 0) held[tid >> 6] = wave_top;
@@ -320,11 +324,14 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(AttentionParams p, 
 #pragma unroll
     for (int j = 0; j < 32; j++) {
         const uint32_t s = stripe + 8u * j;
-        if (s < p.sections) sum = fmaf(values[j], weights[s], sum);
+        if (s < sections) sum = fmaf(values[j], weights[s], sum);
     }
     stripes[stripe][tid & 31u] = sum;
     __syncthreads();
     if (tid < 32 && c < width) {
+        // where the row goes is worked out here, behind the loads: it needs parameters the first loads do not wait for
+        const uint32_t row = unit % p.rows;
+        const uint32_t b = (unit / p.rows) % p.batch, kvh = unit / p.rows / p.batch;
         float value = ((stripes[0][tid] + stripes[1][tid]) + (stripes[2][tid] + stripes[3][tid])) +
                       ((stripes[4][tid] + stripes[5][tid]) + (stripes[6][tid] + stripes[7][tid]));
         p.out[(uint64_t)(kvh * G + g) * p.o_sh + (uint64_t)b * p.o_sb + (uint64_t)row * p.o_sr + c] = value * normalized;
@@ -522,8 +529,12 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
 //           that same key order (two 8-byte reads a lane).
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+// The leading arguments are what the first loads (cursor, queries, the first key and value tile) need: plain words that the
+// hardware hands to a wave in scalar registers as it starts (batch and query heads a group share a word); the rest is in `p`.
 template <int WIDTH>
-__global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionParams p) {
+__global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32_t *lead_cursor, const float *lead_q, const uint16_t *lead_k, const uint16_t *lead_v,
+                                                                    uint32_t lead_q_sh, uint32_t lead_q_sb, uint32_t lead_keys, uint32_t lead_sections,
+                                                                    uint32_t lead_capacity, uint32_t lead_batch_groups, AttentionParams p) {
     constexpr int TK = 32;                  // keys per tile
     constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output
@@ -538,22 +549,23 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t n = lane & 15u, kq = lane >> 4;
-    const uint32_t G = p.groups;
+    const uint32_t G = lead_batch_groups & 0xffffu, batch = lead_batch_groups >> 16;
+    const uint32_t keys_held = lead_keys, sections = lead_sections, capacity = lead_capacity;
     const uint32_t unit = blockIdx.x, section = blockIdx.y;
-    const uint32_t b = unit % p.batch, kvh = unit / p.batch;
-    const uint64_t plane = ((uint64_t)kvh * p.batch + b) * p.capacity;
+    const uint32_t b = unit % batch, kvh = unit / batch;
+    const uint64_t plane = ((uint64_t)kvh * batch + b) * capacity;
 
     // what does not need the cursor comes first: the cursor's load, the queries' and the first tile's are then all in flight
     // together instead of one round trip to memory behind the other
-    const uint32_t origin_read = p.cursor ? p.cursor[b] : 0u;
-    const uint32_t chunk = (p.keys + p.sections - 1u) / p.sections;
-    const uint32_t begin = min(p.keys, section * chunk);
+    const uint32_t origin_read = lead_cursor ? lead_cursor[b] : 0u;
+    const uint32_t chunk = (keys_held + sections - 1u) / sections;
+    const uint32_t begin = min(keys_held, section * chunk);
     const bool held = n < G;
 
     // the queries of this lane's column, as they lie; they become two half planes once the first tile has been asked for
     float q_raw[STEPS][8];
     {
-        const float *src = p.q + (uint64_t)(kvh * G + min(n, G - 1u)) * p.q_sh + (uint64_t)b * p.q_sb;
+        const float *src = lead_q + (uint64_t)(kvh * G + min(n, G - 1u)) * lead_q_sh + (uint64_t)b * lead_q_sb;
         // a column past the group reads the group's last head: its scores are masked, and no column reaches another's sums
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
@@ -573,21 +585,21 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
-                const uint64_t at = (plane + min(tile + 16u * kb + n, p.capacity - 1u)) * WIDTH + 32u * s + 8u * kq;
-                kraw[kb][s] = *reinterpret_cast<const u32x4 *>(p.cache_k + at);
+                const uint64_t at = (plane + min(tile + 16u * kb + n, capacity - 1u)) * WIDTH + 32u * s + 8u * kq;
+                kraw[kb][s] = *reinterpret_cast<const u32x4 *>(lead_k + at);
             }
     };
     auto fetch_values = [&](uint32_t tile) {
 #pragma unroll
         for (int i = 0; i < PIECES; i++) {
             const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
-            vraw[i] = *reinterpret_cast<const u32x4 *>(p.cache_v + (plane + min(tile + key, p.capacity - 1u)) * WIDTH + part * 8u);
+            vraw[i] = *reinterpret_cast<const u32x4 *>(lead_v + (plane + min(tile + key, capacity - 1u)) * WIDTH + part * 8u);
         }
     };
     // the first tile's rows are asked for whether or not the cursor has reached them (the addresses are clamped to the cache)
     uint32_t tile = begin + wave * TK;
     __builtin_amdgcn_sched_barrier(0);  // the queries' loads stay ahead of the tile's, their first use behind them
-    if (tile < min(p.keys, begin + chunk)) fetch_keys(tile), fetch_values(tile);
+    if (tile < min(keys_held, begin + chunk)) fetch_keys(tile), fetch_values(tile);
     __builtin_amdgcn_sched_barrier(0);
     half8_t q_value[STEPS], q_residue[STEPS];
 #pragma unroll
@@ -599,12 +611,12 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
             q_residue[s][i] = (_Float16)((q_raw[s][i] - (float)high) * 2048.0f);
         }
     uint32_t origin = origin_read;
-    if (!p.reach && origin + 1u > p.keys) {  // refusal::ORIGIN (attention.rs:250-252)
+    if (!p.reach && origin + 1u > keys_held) {  // refusal::ORIGIN (attention.rs:250-252)
         if (tid == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-        origin = p.keys - 1u;
+        origin = keys_held - 1u;
     }
-    const Ring ring(p.keys, origin + 1u, p.reach);
-    const uint32_t visible = min(p.keys, origin + 1u);  // a ring too: the slots written so far
+    const Ring ring(keys_held, origin + 1u, p.reach);
+    const uint32_t visible = min(keys_held, origin + 1u);  // a ring too: the slots written so far
     const uint32_t last = min(visible, begin + chunk);
     for (; tile < last; tile += 4 * TK) {
         // ---- scores
@@ -702,14 +714,14 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(AttentionPar
         const uint32_t g = index / WIDTH, c = index % WIDTH;
         const float value = (merged[0][g][c] + merged[1][g][c]) + (merged[2][g][c] + merged[3][g][c]);
         float total = 0.0f, highest = -INFINITY;
-        if (c == 0 || p.sections == 1) {
+        if (c == 0 || sections == 1) {
 #pragma unroll
             for (int w = 0; w < 4; w++) highest = fmaxf(highest, tops[w][g]);
 #pragma unroll
             for (int w = 0; w < 4; w++) total = fmaf(masses[w][g], tops[w][g] == -INFINITY ? 0.0f : softmax_exp(tops[w][g] - highest), total);
         }
-        if (p.sections > 1) {
-            float *dst = p.partial + (((uint64_t)unit * p.sections + section) * G + g) * (WIDTH + 2);
+        if (sections > 1) {
+            float *dst = p.partial + (((uint64_t)unit * sections + section) * G + g) * (WIDTH + 2);
             dst[c] = value;
             if (c == 0) dst[WIDTH] = highest, dst[WIDTH + 1] = total;
         } else {
@@ -833,7 +845,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
         else hipLaunchKernelGGL(attention_any_kernel<NH_BF16>, grid, dim3(256), 0, d->stream, p, a.width);
         NH_HIP(hipGetLastError());
         if (p.sections > 1) {
-            hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
+            hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
             NH_HIP(hipGetLastError());
         }
         return NH_OK;
@@ -870,11 +882,17 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
                 if (!p.partial) return NH_E_MEMORY;
             }
             dim3 grid(planes, p.sections);
-            if (a.width == 64) hipLaunchKernelGGL(attention_decode_tile_kernel<64>, grid, dim3(256), 0, d->stream, p);
-            else hipLaunchKernelGGL(attention_decode_tile_kernel<128>, grid, dim3(256), 0, d->stream, p);
+            if (p.q_sh > UINT32_MAX || p.q_sb > UINT32_MAX || p.batch > 0xffffu) return fail(NH_E_ARGUMENT, "query strides and planes past what the decode attention takes");
+            const uint32_t batch_groups = (p.batch << 16) | p.groups;
+            if (a.width == 64)
+                hipLaunchKernelGGL(attention_decode_tile_kernel<64>, grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh,
+                                   (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p);
+            else
+                hipLaunchKernelGGL(attention_decode_tile_kernel<128>, grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh,
+                                   (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p);
             NH_HIP(hipGetLastError());
             if (p.sections > 1) {
-                hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
+                hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
                 NH_HIP(hipGetLastError());
             }
             return NH_OK;
@@ -901,7 +919,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     NH_HIP(hipGetLastError());
     if (p.sections > 1) {
-        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p, a.width);
+        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
         NH_HIP(hipGetLastError());
     }
     return NH_OK;

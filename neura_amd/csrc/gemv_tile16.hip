@@ -50,8 +50,15 @@ struct Tile16Unit {
 // aligned 64 bytes (pieces smaller than the 32 bytes the memory checks as one cost a read-modify-write each).  The scale
 // is then a chunk's own, not a group's, so the four MFMAs of a step keep their sums apart and each is weighed by its
 // chunk's scale; the staging pass shrinks to a copy.
+//
+// The leading arguments are what a wave needs before it can ask for its first activations and weights.  They are plain words
+// so that the hardware can hand them over in scalar registers when it starts the wave (the file is built with
+// -amdgpu-kernarg-preload-count): the wave's first loads then go out without waiting for a load of its parameters
+// (about 0.5 us); everything else sits in `p` and is fetched meanwhile.  `input` is x, or the digit planes with HANDED.
 template <int NW, int D, int MODE, int R, bool HANDED = false>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) {
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, int32_t lead_to_w1,
+                                                                  int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
+                                                                  uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
     static_assert(!HANDED || (R == 1 && MODE == TILE16_PLAIN), "handed-over digit planes feed a plain product of one row");
     extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
@@ -61,7 +68,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nblk = p.nblk;
+    const uint32_t nblk = lead_row_bytes / 144u;  // super-blocks a row
+    const float *const x = static_cast<const float *>(lead_input);
     uint8_t *const digits = tile16_lds_bytes;
     const uint32_t row_digits = nblk * TILE16_BLOCK_DIGITS;  // digit planes of one activation row
     uint8_t *const zeros = tile16_lds_bytes + (size_t)R * row_digits + wave * TILE16_ZERO_BYTES;  // a wave's own zeros
@@ -69,26 +77,34 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     float *const part = reinterpret_cast<float *>(sums + (HANDED ? (size_t)nblk * (TILE16_BLOCK_PAIRS / 16u) : (size_t)R * nblk * 4u));  // [parity][wave][row][16]
     float *const red = part + 2u * NW * R * 16u;                                  // [wave][row]
 
-    fetch_parameters(p, MODE == TILE16_ROPE);
-    asm volatile("" ::"s"(gridDim.x));
+    // everything else a wave reads from `p` is asked for in one go once its first loads are out
+    auto fetch_the_rest = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        NH_FETCH(p.y, p.residual, p.N, p.K, p.rows, p.eps, p.digits_out);
+        if (MODE == TILE16_ROPE)
+            NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_width, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions,
+                     p.rope_ring, p.bias[0], p.bias[1], p.bias[2], p.refusal, p.end[0], p.end[1]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
     const uint32_t r = lane & 15u, q = lane >> 4;
-    // tiles of this workgroup: blockIdx.x, blockIdx.x + gridDim.x, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
-    const uint32_t tiles = p.row_groups;
+    // tiles of this workgroup: blockIdx.x, blockIdx.x + lead_grid, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
+    const uint32_t tiles = lead_tiles;
     if (blockIdx.x >= tiles) return;  // the whole workgroup: no barrier has been reached
-    const uint32_t ntiles = (tiles - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    const uint32_t ntiles = (tiles - blockIdx.x + lead_grid - 1u) / lead_grid;
     const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;  // super-blocks of one tile this wave walks
 
     // the weight row lane r reads in tile `tile`; with the rotation folded in a tile holds channels c0 .. c0 + 7 of a head and
     // their partners half a head further (written with selects over scalars captured by value: nothing here may end up indexed)
-    const uint8_t *const w0 = p.W[0];
-    const int64_t to_w1 = p.W[1] - p.W[0], to_w2 = p.W[2] - p.W[0];
-    const uint32_t end0 = p.end[0], end1 = p.end[1];
-    const uint32_t row_bytes = p.row_bytes;
-    const uint32_t half_width = p.rope_width >> 1, tiles_per_head = max(half_width >> 3, 1u);
-    const uint32_t first_tile = blockIdx.x, hop = gridDim.x;
+    const uint8_t *const w0 = lead_w0;
+    const int64_t to_w1 = (int64_t)lead_to_w1 * 16, to_w2 = (int64_t)lead_to_w2 * 16;  // handed over in units of 16 bytes
+    const uint32_t end0 = lead_end0, end1 = lead_end1;
+    const uint32_t row_bytes = lead_row_bytes;
+    // (with the rotation folded in the tile rows' word carries the rotation's width: such tiles are always whole)
+    const uint32_t half_width = (MODE == TILE16_ROPE ? lead_tile_rows : 16u) >> 1, tiles_per_head = max(half_width >> 3, 1u);
+    const uint32_t first_tile = blockIdx.x, hop = lead_grid;
     // a plain tile may hold fewer than 16 rows (a matrix of 3584 rows is 256 tiles of 14, one a compute unit, where it is 224
     // of 16): the columns past them walk the tile's last row again and are never written
-    const uint32_t tile_rows = MODE == TILE16_PLAIN ? p.tile_rows : 16u;
+    const uint32_t tile_rows = MODE == TILE16_PLAIN ? lead_tile_rows : 16u;
     auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, tile_rows, r, q](uint32_t tile) -> const uint8_t * {
         (void)tile_rows;  // the SwiGLU form's tiles are whole
         int64_t offset;
@@ -144,10 +160,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
     // Unit e4 = tid + NT * j (four consecutive activations) lies in super-block wave + NW * j: a wave turns into digits
     // exactly the super-blocks it multiplies.
     {
-        const uint32_t units = p.K / 4u;
+        const uint32_t units = nblk * 64u;
         if (lane < TILE16_ZERO_BYTES / 4u) reinterpret_cast<uint32_t *>(zeros)[lane] = 0u;
         auto stage = [&](uint32_t e4, f32x4 v, f32x4 w, float rms, uint8_t *row_planes, f32x4 *row_sums) {
-            if (p.norm_w) {
+            if (lead_norm_w) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) v[i] = __fmul_rn(__fmul_rn(v[i], rms), w[i]);
             }
@@ -199,11 +215,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
 #pragma unroll
                 for (int j = 0; j < MAXB; j++) {
                     uint32_t b = min(wave + NW * (j0 + j), nblk - 1u);
-                    held[j] = *(global_uint4)(uintptr_t)(p.digits_in + (size_t)b * TILE16_BLOCK_HANDED + lane * 16u);
+                    held[j] = *(global_uint4)(uintptr_t)(static_cast<const uint8_t *>(lead_input) + (size_t)b * TILE16_BLOCK_HANDED + lane * 16u);
                 }
                 if (j0 == 0) {
 #pragma unroll
                     for (int i = 0; i < D; i++) fetch(ring[i]);
+                    fetch_the_rest();
                 }
 #pragma unroll
                 for (int j = 0; j < MAXB; j++) {
@@ -216,18 +233,20 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             if (count == 0) {
 #pragma unroll
                 for (int i = 0; i < D; i++) fetch(ring[i]);
+                fetch_the_rest();
             }
         } else if constexpr (R > 1) {
             // the weights' loads go out first; every row's activations follow (twice where the norm is folded in: once for
             // the row's sum of squares, once for the digits -- the second pass finds them in the cache)
 #pragma unroll
             for (int i = 0; i < D; i++) fetch(ring[i]);
+            fetch_the_rest();
             const uint32_t rows = min(p.rows, (uint32_t)R);
-            if (p.norm_w) {
+            if (lead_norm_w) {
                 for (uint32_t row = 0; row < rows; row++) {
                     float square = 0.0f;
                     for (uint32_t e4 = tid; e4 < units; e4 += NT) {
-                        const f32x4 v = *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4);
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(x + (size_t)row * p.K + 4u * e4);
 #pragma unroll
                         for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
                     }
@@ -238,15 +257,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             }
             for (uint32_t row = 0; row < rows; row++) {
                 float rms = 1.0f;
-                if (p.norm_w) {
+                if (lead_norm_w) {
                     float total = 0.0f;
 #pragma unroll
                     for (int w = 0; w < NW; w++) total += red[w * R + row];
                     rms = rms_scale_of(total, p.K, p.eps);
                 }
                 for (uint32_t e4 = tid; e4 < units; e4 += NT)
-                    stage(e4, *reinterpret_cast<const f32x4 *>(p.x + (size_t)row * p.K + 4u * e4),
-                          p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms, digits + (size_t)row * row_digits,
+                    stage(e4, *reinterpret_cast<const f32x4 *>(x + (size_t)row * p.K + 4u * e4),
+                          lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms, digits + (size_t)row * row_digits,
                           sums + (size_t)row * nblk * 4u);
             }
         } else {
@@ -258,21 +277,22 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
 #pragma unroll
             for (int j = 0; j < MAXJ; j++) {
                 const uint32_t e4 = tid + NT * j;
-                held[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(p.x + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                held[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(x + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
-            if (p.norm_w) {
+            if (lead_norm_w) {
 #pragma unroll
                 for (int j = 0; j < MAXJ; j++) {
                     const uint32_t e4 = tid + NT * j;
-                    weight[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                    weight[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
                 }
             }
         }
-        if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
         // the weights' loads go out behind the activations', which everything waits for first
 #pragma unroll
         for (int i = 0; i < D; i++) fetch(ring[i]);
-        if (p.norm_w) {
+        fetch_the_rest();
+        if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
+        if (lead_norm_w) {
             // sum of squares of the whole row (crates/neura-kernel/src/task/norm.rs:69-83; the same fp32 adds in another order)
             float square = 0.0f;
             if (resident) {
@@ -282,7 +302,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(held[j][i], held[j][i]));
             } else {
                 for (uint32_t e4 = tid; e4 < units; e4 += NT) {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(p.x + 4u * e4);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(x + 4u * e4);
 #pragma unroll
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
                 }
@@ -304,7 +324,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(GemvParams p) 
             }
         } else {
             for (uint32_t e4 = tid; e4 < units; e4 += NT)
-                stage(e4, *reinterpret_cast<const f32x4 *>(p.x + 4u * e4), p.norm_w ? *reinterpret_cast<const f32x4 *>(p.norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
+                stage(e4, *reinterpret_cast<const f32x4 *>(x + 4u * e4), lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
                       digits, sums);
         }
         }
@@ -954,6 +974,11 @@ bool tile16_takes(const GemvArgs &a) {
     } else if (a.end[0] % 16u != 0 || a.end[1] % 16u != 0) {
         return false;
     }
+    for (int m = 1; m < 3; m++) {  // the matrices stacked behind the first are named by their distance from it in 16-byte units
+        if (!a.W[m]) continue;
+        const int64_t apart = static_cast<const uint8_t *>(a.W[m]) - static_cast<const uint8_t *>(a.W[0]);
+        if (apart % 16 != 0 || apart / 16 > INT32_MAX || apart / 16 < INT32_MIN) return false;
+    }
     if (a.digits_out && (!a.swiglu || a.rows != 1 || a.N % 512u != 0 || ((uintptr_t)a.digits_out & 63u))) return false;
     if (a.digits_in && (a.swiglu || a.rope || a.norm_w || a.rows != 1 || ((uintptr_t)a.digits_in & 15u))) return false;
     const uint32_t nblk = a.K / 256u;
@@ -1056,7 +1081,9 @@ static hipError_t launch_tile16_instance(nh_device *d, const GemvParams &p, uint
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
+                       HANDED ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x), p.norm_w, (int32_t)((p.W[1] - p.W[0]) / 16),
+                       (int32_t)((p.W[2] - p.W[0]) / 16), p.row_bytes, grid, p.row_groups, MODE == TILE16_ROPE ? p.rope_width : p.tile_rows, p.end[0], p.end[1], p);
     return hipGetLastError();
 }
 
