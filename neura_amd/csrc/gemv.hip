@@ -629,8 +629,18 @@ struct Q8Tile {
 
 // DEEP (rows of 65 to 256 blocks, K <= 8192): the four waves of a workgroup walk the same rows, wave w the blocks 64 w ..
 // 64 w + 63, and meet in LDS once a pass.
+// The leading arguments are what the first weight loads and the activations' need: plain words the hardware hands to a wave in
+// scalar registers as it starts (Q8_LEAD packs them: the rotation's width rides above the blocks a row, the SwiGLU flag above
+// N); they take the place of the same members of the parameter block, whose other members are loaded as they come to use.
+#define Q8_LEAD(p) (p).W[0], (p).W[1], (p).W[2], (p).x, (p).row_bytes, (p).nblk | ((p).rope_width << 16), (p).row_groups, (p).N | ((p).swiglu ? 0x80000000u : 0u), (p).end[0], (p).end[1], (p)
 template <int R, int G, bool DEEP = false, bool ROPE = false>
-__global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(GemvParams p) {
+__global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(const uint8_t *lead_w0, const uint8_t *lead_w1, const uint8_t *lead_w2, const float *lead_x,
+                                                               uint32_t lead_row_bytes, uint32_t lead_nblk_width, uint32_t lead_row_groups, uint32_t lead_n_swiglu,
+                                                               uint32_t lead_end0, uint32_t lead_end1, GemvParams rest) {
+    GemvParams p = rest;
+    p.W[0] = lead_w0, p.W[1] = lead_w1, p.W[2] = lead_w2, p.x = lead_x, p.row_bytes = lead_row_bytes, p.row_groups = lead_row_groups;
+    p.nblk = lead_nblk_width & 0xffffu, p.rope_width = lead_nblk_width >> 16, p.K = 32u * (lead_nblk_width & 0xffffu);
+    p.N = lead_n_swiglu & 0x7fffffffu, p.swiglu = (int32_t)(lead_n_swiglu >> 31), p.end[0] = lead_end0, p.end[1] = lead_end1;
     static_assert(!DEEP || G == 64, "a deep row fills every wave");
     static_assert(!ROPE || (R == 2 && !DEEP), "the rotation pairs the two rows of a pass");
     extern __shared__ float xs[];  // skew32(K)
@@ -2154,14 +2164,14 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         if (wgs > resident) wgs = resident;
         const size_t staged = (size_t)(a.K + a.K / 32u * 4u) * sizeof(float);
         const dim3 wide(wgs);
-#define NH_Q8(RR, GG) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<RR, GG>), wide, block, staged, d->stream, p)
+#define NH_Q8(RR, GG) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<RR, GG>), wide, block, staged, d->stream, Q8_LEAD(p))
         if (a.rope) {
-            if (p.group == 64) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, false, true>), wide, block, staged, d->stream, p);
-            else if (p.group == 32) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 32, false, true>), wide, block, staged, d->stream, p);
-            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 16, false, true>), wide, block, staged, d->stream, p);
+            if (p.group == 64) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+            else if (p.group == 32) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 32, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 16, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
         } else if (deep) {
-            if (R == 4) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<4, 64, true>), wide, block, staged, d->stream, p);
-            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, true>), wide, block, staged, d->stream, p);
+            if (R == 4) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<4, 64, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, true>), wide, block, staged, d->stream, Q8_LEAD(p));
         } else if (R == 4) {
             if (p.group == 64) NH_Q8(4, 64);
             else if (p.group == 32) NH_Q8(4, 32);
