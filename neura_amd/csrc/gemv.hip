@@ -875,8 +875,8 @@ __device__ __noinline__ u32x4 piece_before(const uint8_t *at, const uint8_t *end
 }
 
 template <int ELEMENT, int RB>
-__global__ __launch_bounds__(256) void gemv_staged_kernel(GemvParams p) {
-    fetch_parameters(p);
+__global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) {
+    GEMV_TAKE_LEAD;
     typedef Staged<ELEMENT> Format;
     extern __shared__ float xs[];  // [RB][slice]; the sums per eight activations; then the raw row slices, two per wave
     __shared__ float red[256];
@@ -1060,6 +1060,20 @@ struct MfmaParams {
     float eps;
 };
 
+// What a wave of the matrix-core products needs before its first loads, as leading plain arguments the hardware hands over in
+// scalar registers when it starts the wave (the activation rows ride above the blocks a row, the K slices above the blocks a
+// slice); they take the place of the same members of the parameter block, whose other members are loaded as they come to use.
+#define MFMA_LEAD_PARAMETERS                                                                                                                          \
+    const uint8_t *lead_w0, const uint8_t *lead_w1, const uint8_t *lead_w2, const float *lead_x, uint32_t lead_row_bytes, uint32_t lead_nblk_rows,      \
+        uint32_t lead_slice_splits, uint32_t lead_tiles, uint32_t lead_end0, uint32_t lead_end1, MfmaParams rest
+#define MFMA_LEAD(p)                                                                                                                                   \
+    (p).W[0], (p).W[1], (p).W[2], (p).x, (p).row_bytes, (p).nblk | ((p).rows << 16), (p).slice_blocks | ((p).splits << 16), (p).tiles, (p).end[0], (p).end[1], (p)
+#define MFMA_TAKE_LEAD                                                                                                                                 \
+    MfmaParams p = rest;                                                                                                                               \
+    p.W[0] = lead_w0, p.W[1] = lead_w1, p.W[2] = lead_w2, p.x = lead_x, p.row_bytes = lead_row_bytes, p.tiles = lead_tiles;                             \
+    p.nblk = lead_nblk_rows & 0xffffu, p.rows = lead_nblk_rows >> 16, p.K = 256u * (lead_nblk_rows & 0xffffu);                                          \
+    p.slice_blocks = lead_slice_splits & 0xffffu, p.splits = lead_slice_splits >> 16, p.end[0] = lead_end0, p.end[1] = lead_end1
+
 struct MfmaUnit {
     u32x4 hdr, qa, qb;
 };
@@ -1080,7 +1094,8 @@ __device__ __forceinline__ void digit_planes(uint32_t d0, uint32_t d1, uint32_t 
 }
 
 template <int KS, int NW, int P, int D>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MFMA_LEAD_PARAMETERS) {
+    MFMA_TAKE_LEAD;
     extern __shared__ uint32_t xop[];  // [block][16 steps][4 groups][4 P digit columns] of 4 bytes; then sums; then tile partials
     __shared__ float red[256];
     __shared__ uint32_t wave_top[NW];
@@ -1388,7 +1403,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MfmaParams p) {
 // Loads are issued whether or not a super-block is left (the last one again, its product dropped), so that the
 // waits count exactly how many loads are newer than the one needed.
 template <int NW, int D>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MfmaParams p) {
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MFMA_LEAD_PARAMETERS) {
+    MFMA_TAKE_LEAD;
     static_assert(D % 2 == 0, "the activation ring alternates between two slots");
     __shared__ __attribute__((aligned(16))) uint32_t digits[NW][256];  // [step][group][digit plane] per wave
     __shared__ float sums[NW][16];                                    // per wave: 8 sub-block sums, 8 sub-block unscales
@@ -1518,7 +1534,8 @@ struct Tile32Unit {
 };
 
 template <int J, int NW, int KS>
-__global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_kernel(MfmaParams p) {  // second bound: waves per SIMD
+__global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_kernel(MFMA_LEAD_PARAMETERS) {  // second bound: waves per SIMD
+    MFMA_TAKE_LEAD;
 
     constexpr uint32_t M8 = 8 * J, R2 = 2 * J, TPW = NW / KS, NT = NW * 64;
     constexpr bool STAGED = J == 1;  // raw blocks through LDS; with eight activation rows the digits leave no room for them
@@ -1754,7 +1771,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 constexpr uint32_t F16_BLOCK_PIECES = 8u * 4u * 16u + 2u * 16u;  // 16-byte pieces of LDS per staged super-block: operands, then sums
 
 template <int NW, int KS>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MfmaParams p) {
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MFMA_LEAD_PARAMETERS) {
+    MFMA_TAKE_LEAD;
     constexpr uint32_t TPW = NW / KS, NT = NW * 64;
     static_assert(NT == 1024, "eight row groups of 128 threads stage the activations");
     extern __shared__ __attribute__((aligned(16))) uint32_t staged[];  // [block][F16_BLOCK_PIECES] pieces
@@ -2227,7 +2245,7 @@ static hipError_t launch_mfma_instance(nh_device *d, const MfmaParams &p, uint32
         if (status != hipSuccess) return status;
         widened = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<KS, NW, P, D>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_mfma_kernel<KS, NW, P, D>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, MFMA_LEAD(p));
     return hipGetLastError();
 }
 
@@ -2261,7 +2279,7 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
         p.x = a.x, p.y = a.y, p.residual = a.residual;
         p.N = a.N, p.K = a.K, p.row_bytes = nblk * 144u, p.nblk = nblk, p.rows = 1, p.tiles = a.N / 16u;
         profile_mark(d);
-        hipLaunchKernelGGL((gemv_q4k_mfma_deep_kernel<16, 2>), dim3(p.tiles), dim3(1024), 0, d->stream, p);
+        hipLaunchKernelGGL((gemv_q4k_mfma_deep_kernel<16, 2>), dim3(p.tiles), dim3(1024), 0, d->stream, MFMA_LEAD(p));
         NH_HIP(hipGetLastError());
         profile_mark(d);
         if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
@@ -2405,7 +2423,7 @@ static int32_t launch_mfma32_instance(nh_device *d, const MfmaParams &p, size_t 
     uint32_t most = (uint32_t)d->compute_units * resident / p.splits;
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
-    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, MFMA_LEAD(p));
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -2484,7 +2502,7 @@ static int32_t launch_f16_tiles_instance(nh_device *d, const MfmaParams &p, size
     uint32_t most = (uint32_t)d->compute_units * resident / p.splits;
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
-    hipLaunchKernelGGL((gemv_q4k_f16_kernel<NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_f16_kernel<NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, MFMA_LEAD(p));
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -2554,7 +2572,7 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
     profile_mark(d);
-    hipLaunchKernelGGL((gemv_staged_kernel<ELEMENT, RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_staged_kernel<ELEMENT, RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, GEMV_LEAD(p));
     NH_HIP(hipGetLastError());
     if (p.splits > 1) {
         uint32_t outputs = (a.swiglu ? a.N / 2 : a.N) * RB;

@@ -50,6 +50,21 @@ __device__ __forceinline__ void fetch_parameters(const GemvParams &p, bool rope 
                  p.bias[0], p.bias[1], p.bias[2], p.refusal);
 }
 
+// What a wave of a K-quant product needs before its first loads, as leading plain arguments the hardware hands over in scalar
+// registers when it starts the wave (the activation rows and a tile's rows ride above the super-blocks a row, the SwiGLU flag
+// above N); they take the place of the same members of the parameter block, whose other members are loaded as they come to use.
+#define GEMV_LEAD_PARAMETERS                                                                                                                          \
+    const uint8_t *lead_w0, const uint8_t *lead_w1, const uint8_t *lead_w2, const float *lead_x, uint32_t lead_row_bytes, uint32_t lead_nblk_rows,      \
+        uint32_t lead_row_groups, uint32_t lead_n_swiglu, uint32_t lead_end0, uint32_t lead_end1, GemvParams rest
+#define GEMV_LEAD(p)                                                                                                                                   \
+    (p).W[0], (p).W[1], (p).W[2], (p).x, (p).row_bytes, (p).nblk | ((p).rows << 16) | ((p).tile_rows << 24), (p).row_groups,                           \
+        (p).N | ((p).swiglu ? 0x80000000u : 0u), (p).end[0], (p).end[1], (p)
+#define GEMV_TAKE_LEAD                                                                                                                                 \
+    GemvParams p = rest;                                                                                                                               \
+    p.W[0] = lead_w0, p.W[1] = lead_w1, p.W[2] = lead_w2, p.x = lead_x, p.row_bytes = lead_row_bytes, p.row_groups = lead_row_groups;                   \
+    p.nblk = lead_nblk_rows & 0xffffu, p.rows = (lead_nblk_rows >> 16) & 0xffu, p.tile_rows = lead_nblk_rows >> 24, p.K = 256u * (lead_nblk_rows & 0xffffu); \
+    p.N = lead_n_swiglu & 0x7fffffffu, p.swiglu = (int32_t)(lead_n_swiglu >> 31), p.end[0] = lead_end0, p.end[1] = lead_end1
+
 __device__ __forceinline__ float silu(float a) { return a * (1.0f / (1.0f + expf(-a))); }
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));

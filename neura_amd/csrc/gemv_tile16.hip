@@ -636,7 +636,8 @@ static size_t rows4_lds(uint32_t nblk, uint32_t NW, uint32_t rows) {
 }
 
 template <int NW, int D, int MODE, int P>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_rows4_kernel(GemvParams p) {
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_rows4_kernel(GEMV_LEAD_PARAMETERS) {
+    GEMV_TAKE_LEAD;
     static_assert(MODE == TILE16_PLAIN || MODE == TILE16_SWIGLU, "no rotation is folded into a product of several rows");
     extern __shared__ __attribute__((aligned(16))) uint8_t rows4_lds_bytes[];
     constexpr uint32_t NT = NW * 64, ROWS = 4 * P;
@@ -644,8 +645,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_rows4_kernel(GemvParams p) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
     typedef const __attribute__((address_space(1))) u32x2 *global_uint2;
-    fetch_parameters(p);
-    asm volatile("" ::"s"(gridDim.x));
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t nblk = p.nblk;
@@ -1023,7 +1022,7 @@ static hipError_t launch_rows4_instance(nh_device *d, const GemvParams &p, uint3
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_rows4_kernel<NW, 2, MODE, P>), dim3(grid), dim3(NW * 64), lds, d->stream, p);
+    hipLaunchKernelGGL((gemv_q4k_rows4_kernel<NW, 2, MODE, P>), dim3(grid), dim3(NW * 64), lds, d->stream, GEMV_LEAD(p));
     return hipGetLastError();
 }
 
