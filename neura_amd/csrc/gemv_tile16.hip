@@ -207,7 +207,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
         if constexpr (HANDED) {
             // a wave copies the super-blocks it walks, one 16-byte load a lane and block: lane 4 c + part holds plane `part` of
             // chunk c, or with part 3 the chunk's pair
-            constexpr int MAXB = 5;
+            constexpr int MAXB = NW <= 8 ? 10 : 5;  // super-blocks a wave copies at once: ffn_down at eight waves has ten, all asked for together
             uint8_t *const pairs = reinterpret_cast<uint8_t *>(sums);
             const uint32_t chunk = lane >> 2, piece = lane & 3u;
             for (uint32_t j0 = 0; j0 < count; j0 += MAXB) {
