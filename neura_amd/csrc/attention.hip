@@ -531,11 +531,13 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // The leading arguments are what the first loads (cursor, queries, the first key and value tile) need: plain words that the
 // hardware hands to a wave in scalar registers as it starts (batch and query heads a group share a word); the rest is in `p`.
-template <int WIDTH>
+// TK = 16 (one plane a kv head: a decode step of few planes): tiles of sixteen keys, so that sections of 64 keys give every
+// compute unit a workgroup and a wave half the work; the value product then runs on v_mfma_f32_16x16x16_f16 (K = the tile's keys).
+template <int WIDTH, int TK = 32>
 __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32_t *lead_cursor, const float *lead_q, const uint16_t *lead_k, const uint16_t *lead_v,
                                                                     uint32_t lead_q_sh, uint32_t lead_q_sb, uint32_t lead_keys, uint32_t lead_sections,
                                                                     uint32_t lead_capacity, uint32_t lead_batch_groups, AttentionParams p) {
-    constexpr int TK = 32;                  // keys per tile
+    constexpr int KB = TK / 16;             // 16-key blocks of a tile
     constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output
     constexpr int VPITCH = TK + 4;          // halves per staged value channel
@@ -579,10 +581,10 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
     for (int d = 0; d < BLOCKS; d++) acc[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float top = -INFINITY, mass = 0.0f;
 
-    u32x4 kraw[2][STEPS], vraw[PIECES];
+    u32x4 kraw[KB][STEPS], vraw[PIECES];
     auto fetch_keys = [&](uint32_t tile) {
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
                 const uint64_t at = (plane + min(tile + 16u * kb + n, capacity - 1u)) * WIDTH + 32u * s + 8u * kq;
@@ -620,9 +622,9 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
     const uint32_t last = min(visible, begin + chunk);
     for (; tile < last; tile += 4 * TK) {
         // ---- scores
-        f32x4_t scores[2], fine[2];
+        f32x4_t scores[KB], fine[KB];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int kb = 0; kb < KB; kb++) {
             scores[kb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, fine[kb] = scores[kb];
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
@@ -636,7 +638,7 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
         // ---- weights: register e of block kb is key 16 kb + 4 kq + e of the tile, for this lane's column
         float tile_top = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const uint32_t key = tile + 16u * kb + 4u * kq + e;
@@ -649,9 +651,11 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
         const float newer = fmaxf(top, tile_top);
         const float rescale = top == -INFINITY ? 0.0f : softmax_exp(top - newer);
         float tile_mass = 0.0f;
-        half8_t w_value, w_residue;
+        half8_t w_value, w_residue;  // with sixteen keys a tile the low four slots only
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int i = 0; i < 8; i++) w_value[i] = (_Float16)0.0f, w_residue[i] = (_Float16)0.0f;
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const float weight = scores[kb][e] == -INFINITY ? 0.0f : softmax_exp(scores[kb][e] - newer);
@@ -688,10 +692,18 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
             for (int e = 0; e < 4; e++) acc[d][e] *= rescale;
             // channels 16 d + n lie in parts 2 d and 2 d + 1: their key groups sit d / 2 places off
             const uint2 low = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * (kq ^ (d >> 1))]);
-            const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
-            const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_value, acc[d], 0, 0, 0);
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_residue, acc[d], 0, 0, 0);
+            if constexpr (TK == 32) {
+                const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
+                const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
+                acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_value, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_residue, acc[d], 0, 0, 0);
+            } else {
+                typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+                const half4_t values = __builtin_bit_cast(half4_t, low);
+                const half4_t first = {w_value[0], w_value[1], w_value[2], w_value[3]}, second = {w_residue[0], w_residue[1], w_residue[2], w_residue[3]};
+                acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(values, first, acc[d], 0, 0, 0);
+                acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(values, second, acc[d], 0, 0, 0);
+            }
         }
         __builtin_amdgcn_wave_barrier();  // the next tile overwrites the corner
     }
@@ -870,9 +882,12 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
                              a.q_sb % 4 == 0;
         const uint32_t planes = a.kv_heads * a.batch;
         if (aligned && a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16) {
-            // sections of at least 256 keys (two tiles a wave) where the planes alone fill the chip, of 128 (one tile a wave)
-            // where they do not; enough workgroups to fill the chip twice over
-            const uint32_t thinnest = planes >= 8 ? 256u : 128u;
+            // sections of at least 256 keys (two tiles a wave) where the planes alone fill the chip; where they do not (eight
+            // planes and fewer: measured even at twelve, slower from sixteen on), of 64 (one tile of sixteen keys a wave);
+            // enough workgroups to fill the chip twice over.  NEURA_HIP_ATTENTION_TK16=<planes> moves the line (0: never).
+            static const uint32_t thin_below = [] { const char *v = getenv("NEURA_HIP_ATTENTION_TK16"); return v ? (uint32_t)atoi(v) : 12u; }();
+            const bool thin = planes < thin_below;
+            const uint32_t thinnest = thin ? 64u : planes >= 8 ? 256u : 128u;
             uint32_t wanted_sections = ((uint32_t)d->compute_units * 2 + planes - 1) / planes;
             const uint32_t most = (a.keys + thinnest - 1) / thinnest;
             p.sections = wanted_sections < 1 ? 1 : (wanted_sections > most ? most : wanted_sections);
@@ -884,12 +899,17 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             dim3 grid(planes, p.sections);
             if (p.q_sh > UINT32_MAX || p.q_sb > UINT32_MAX || p.batch > 0xffffu) return fail(NH_E_ARGUMENT, "query strides and planes past what the decode attention takes");
             const uint32_t batch_groups = (p.batch << 16) | p.groups;
-            if (a.width == 64)
-                hipLaunchKernelGGL(attention_decode_tile_kernel<64>, grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh,
-                                   (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p);
-            else
-                hipLaunchKernelGGL(attention_decode_tile_kernel<128>, grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh,
-                                   (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p);
+#define DECODE_TILE(WIDTH, TK)                                                                                                                                   \
+    hipLaunchKernelGGL((attention_decode_tile_kernel<WIDTH, TK>), grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh, \
+                       (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p)
+            if (a.width == 64) {
+                if (thin) DECODE_TILE(64, 16);
+                else DECODE_TILE(64, 32);
+            } else {
+                if (thin) DECODE_TILE(128, 16);
+                else DECODE_TILE(128, 32);
+            }
+#undef DECODE_TILE
             NH_HIP(hipGetLastError());
             if (p.sections > 1) {
                 hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);

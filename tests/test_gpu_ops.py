@@ -593,6 +593,8 @@ def test_cache_write_casts_and_scatters(device):
     (12, 2, 1, 17, 300, 128, [200]),       # a fill chunk
     (8, 8, 2, 5, 40, 256, [35, 0]),
     (6, 1, 1, 2, 70, 64, [3]),
+    (8, 1, 1, 1, 333, 128, [331]),         # one plane, eight query heads a group: sections of 64 keys, tiles of sixteen
+    (7, 7, 1, 1, 90, 64, [17]),            # seven planes of one query head; the cursor inside the second tile
 ])
 def test_attention_matches_oracle_and_f64(device, heads, kv_heads, batch, rows, keys, width, origins):
     rng = np.random.default_rng(17)  # runtime.rs:594-605 draws seeds 17 / 29 / 43
