@@ -70,18 +70,6 @@ __device__ __forceinline__ void unpack8(const u32x4 &raw, float (&out)[8]) {
     }
 }
 
-// exp(max(argument, -104)) (crates/neura-kernel/src/substrate.rs:110-116)
-// e^argument for the arguments a running softmax meets (never above zero; -inf gives 0, below -104 the result is zero in
-// single precision anyway).  One hardware exp2 of argument * log2(e), the product carried in two parts so the result keeps
-// the accuracy of the instruction; no branches, so a lane's eight weights of a tile stay one straight run of instructions.
-__device__ __forceinline__ float softmax_exp(float argument) {
-    const float x = fmaxf(argument, -104.0f);
-    const float scaled = x * 1.44269502e+00f;
-    const float rest = fmaf(x, 1.44269502e+00f, -scaled) + x * 1.92596299e-08f;  // what the rounded product left out
-    const float power = __builtin_amdgcn_exp2f(scaled);
-    return fmaf(power, rest * 6.93147182e-01f, power);
-}
-
 // sum over the LPK lanes that share a key: DPP adds inside a row of 16 lanes
 template <int LPK>
 __device__ __forceinline__ float key_sum(float v) {
@@ -834,6 +822,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     p.heads = a.heads, p.kv_heads = a.kv_heads, p.groups = a.heads / a.kv_heads;
     p.batch = a.batch, p.rows = a.rows, p.capacity = a.capacity, p.keys = a.keys;
     p.cursor = a.cursor, p.scale = a.scale, p.refusal = d->refusal, p.reach = a.reach;
+    if (a.unmerged) *a.unmerged = SectionSums{nullptr, 0u, 0u, 0u};
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
@@ -892,6 +881,10 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             const uint32_t most = (a.keys + thinnest - 1) / thinnest;
             p.sections = wanted_sections < 1 ? 1 : (wanted_sections > most ? most : wanted_sections);
             if (p.sections > 256) p.sections = 256;
+            // the caller's next product merges the sections itself: no more of them than it takes, and only where sections that
+            // few stay under 128 keys (two tiles a wave)
+            const bool leave = a.unmerged && a.batch == 1 && thin && most <= 2u * MERGED_SECTIONS_MOST;
+            if (leave && p.sections > MERGED_SECTIONS_MOST) p.sections = MERGED_SECTIONS_MOST;
             if (p.sections > 1) {
                 p.partial = static_cast<float *>(scratch(d, (size_t)p.sections * a.heads * a.batch * (a.width + 2) * sizeof(float)));
                 if (!p.partial) return NH_E_MEMORY;
@@ -911,7 +904,9 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             }
 #undef DECODE_TILE
             NH_HIP(hipGetLastError());
-            if (p.sections > 1) {
+            if (p.sections > 1 && leave) {
+                *a.unmerged = SectionSums{p.partial, p.sections, p.groups, a.width};
+            } else if (p.sections > 1) {
                 hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
                 NH_HIP(hipGetLastError());
             }

@@ -19,6 +19,18 @@ __device__ __forceinline__ uint16_t float_to_half(float value) {
     return __builtin_bit_cast(uint16_t, (_Float16)value);
 }
 
+// exp(max(argument, -104)) (crates/neura-kernel/src/substrate.rs:110-116)
+// e^argument for the arguments a running softmax meets (never above zero; -inf gives 0, below -104 the result is zero in
+// single precision anyway).  One hardware exp2 of argument * log2(e), the product carried in two parts so the result keeps
+// the accuracy of the instruction; no branches, so a lane's eight weights of a tile stay one straight run of instructions.
+__device__ __forceinline__ float softmax_exp(float argument) {
+    const float x = fmaxf(argument, -104.0f);
+    const float scaled = x * 1.44269502e+00f;
+    const float rest = fmaf(x, 1.44269502e+00f, -scaled) + x * 1.92596299e-08f;  // what the rounded product left out
+    const float power = __builtin_amdgcn_exp2f(scaled);
+    return fmaf(power, rest * 6.93147182e-01f, power);
+}
+
 // round to nearest even, as the reference's device casts (crates/neura-kernel/src/task/convert.rs:86-89)
 __device__ __forceinline__ uint16_t float_to_bfloat16(float value) {
     const uint32_t bits = __builtin_bit_cast(uint32_t, value);

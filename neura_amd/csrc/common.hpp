@@ -163,6 +163,13 @@ struct RopeFusion {
     asm volatile("" ::NH_FETCH_PICK(NH_FETCH_COUNT(__VA_ARGS__, 30, 29, 28, 27, 26, 25, 24, 23, 22, 21, 20, 19, 18, 17, 16, 15, 14, 13, 12, 11, 10, 9, 8, 7, 6, 5, 4, \
                                                    3, 2, 1))(__VA_ARGS__))
 
+// The sums a decode attention left a section of the keys each, not merged yet: per (unit, section, query head of the group)
+// `width` weighed channel sums, then the section's largest score and its mass (what attention_fold_kernel reads).
+struct SectionSums {
+    const float *partial;
+    uint32_t sections, groups, width;
+};
+
 struct GemvArgs {
     int32_t element;
     const void *W[3];  // up to three matrices stacked along N; unused entries are nullptr
@@ -182,8 +189,14 @@ struct GemvArgs {
     // and the product that follows reads them (digits_in, in place of x) instead of turning floats into digits again.
     uint8_t *digits_out = nullptr;
     const uint8_t *digits_in = nullptr;
+    // Only where gemv_merges_sections() says so: the activation row is the attention output these sections merge into
+    // (x is not read); the product merges them as it stages its row, and the attention's own fold launch falls away.
+    const SectionSums *merge = nullptr;
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
+// whether launch_gemv can merge attention sections of `width` channels a head into the activation row of this product
+bool gemv_merges_sections(const GemvArgs &args, uint32_t width);
+constexpr uint32_t MERGED_SECTIONS_MOST = 16;  // sections such a product merges at most
 // whether `producer` (a SwiGLU product of one row) can hand its outputs to `consumer` as digit planes, and the bytes they take
 bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer);
 size_t gemv_digit_bytes(uint32_t K);
@@ -240,6 +253,10 @@ struct AttentionArgs {
     float scale;
     uint32_t reach = 0;  // 0, or the span of a ring cache of `keys` slots (Cache::windowed): the last `reach` positions are weighed
     int32_t cache_element = NH_F16;  // what the caches hold: NH_F16 (the matrix-core kernels), NH_BF16 or NH_F32 (the kernel for any element)
+    // Where the caller's next product merges the sections itself (gemv_merges_sections): a decode step of one plane may leave
+    // its sections unmerged (at most MERGED_SECTIONS_MOST of them) and say here where they are; sections == 0 on return
+    // means `out` holds the merged rows as always.
+    SectionSums *unmerged = nullptr;
 };
 int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 

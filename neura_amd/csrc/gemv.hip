@@ -613,6 +613,80 @@ __global__ __launch_bounds__(256) void gemv_q8_0_kernel(GemvParams p) {
     }
 }
 
+// The activation row of the product behind a decode attention, merged from the sums the attention left a section of the keys
+// each (SectionSums; crates/neura-kernel/src/task/attention.rs:619-671 is the merge): element (head, channel) is the sections'
+// channel sums weighed by e^(section's largest score - the largest of all) over the masses weighed the same way.  Every load
+// a thread needs -- the statistics of two (head, section) pairs, sixteen channel sums of each of its four elements -- is asked
+// for before the first is used (sections past the last read the last again and are dropped).  The statistics cross in LDS:
+// the thread of a pair turns its section's largest score into the section's weight, the thread of an element then reads
+// sixteen weights and masses.  `width` is a power of two (the decode attention's 64 or 128).
+template <typename Skew>
+__device__ __forceinline__ void stage_merged(const float *__restrict__ partial, uint32_t sections, uint32_t G, uint32_t width, uint32_t K, float *xs, Skew skew) {
+    constexpr uint32_t MOST = MERGED_SECTIONS_MOST, HEADS_MOST = 32;
+    __shared__ __attribute__((aligned(16))) float tops[HEADS_MOST * MOST], masses[HEADS_MOST * MOST], weights[HEADS_MOST * MOST];
+    const uint32_t tid = threadIdx.x, shift = 31u - __builtin_clz(width), heads = K >> shift, hop = G * (width + 2u), pairs = heads * sections;
+    const uint32_t by_groups = 65536u / G + 1u, by_sections = 65536u / sections + 1u;  // x / G = x * by_groups >> 16 for the few heads and pairs here
+    auto sums_of = [&](uint32_t head) {
+        const uint32_t unit = head * by_groups >> 16;
+        return partial + ((uint64_t)unit * sections * G + (head - unit * G)) * (width + 2u);
+    };
+    float top[2], mass[2];
+    uint32_t seat[2];  // head * MOST + section of this thread's pairs
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const uint32_t pair = min(tid + 256u * j, pairs - 1u), head = pair * by_sections >> 16, section = pair - head * sections;
+        const float *stats = sums_of(head) + section * hop + width;
+        top[j] = stats[0], mass[j] = stats[1];
+        seat[j] = head * MOST + section;
+    }
+    for (uint32_t base = 0; base < K; base += 1024u) {
+        float values[4][MOST];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t i = min(base + tid + 256u * e, K - 1u);
+            const float *column = sums_of(i >> shift) + (i & (width - 1u));
+#pragma unroll
+            for (uint32_t s = 0; s < MOST; s++) values[e][s] = column[min(s, sections - 1u) * hop];
+        }
+        if (base == 0) {
+            // a head's seats past its sections hold no score and no mass
+            for (uint32_t at = tid; at < heads * MOST; at += 256u) tops[at] = -INFINITY, masses[at] = 0.0f;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                if (tid + 256u * j < pairs) tops[seat[j]] = top[j], masses[seat[j]] = mass[j];
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float4 *row = reinterpret_cast<const float4 *>(tops + (seat[j] & ~(MOST - 1u)));
+                float largest = -INFINITY;
+#pragma unroll
+                for (uint32_t q = 0; q < MOST / 4u; q++) largest = fmaxf(fmaxf(largest, fmaxf(row[q].x, row[q].y)), fmaxf(row[q].z, row[q].w));
+                if (tid + 256u * j < pairs) weights[seat[j]] = top[j] == -INFINITY ? 0.0f : softmax_exp(top[j] - largest);
+            }
+            for (uint32_t at = tid; at < heads * MOST; at += 256u)
+                if ((at & (MOST - 1u)) >= sections) weights[at] = 0.0f;
+            __syncthreads();
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t i = base + tid + 256u * e;
+            if (i >= K) continue;
+            const float4 *head_weights = reinterpret_cast<const float4 *>(weights + (i >> shift) * MOST);
+            const float4 *head_masses = reinterpret_cast<const float4 *>(masses + (i >> shift) * MOST);
+            float total = 0.0f, sum = 0.0f;
+#pragma unroll
+            for (uint32_t q = 0; q < MOST / 4u; q++) {
+                const float4 w = head_weights[q], m = head_masses[q];
+                total = fmaf(m.x, w.x, total), total = fmaf(m.y, w.y, total), total = fmaf(m.z, w.z, total), total = fmaf(m.w, w.w, total);
+                sum = fmaf(values[e][4 * q], w.x, sum), sum = fmaf(values[e][4 * q + 1], w.y, sum);
+                sum = fmaf(values[e][4 * q + 2], w.z, sum), sum = fmaf(values[e][4 * q + 3], w.w, sum);
+            }
+            xs[skew(i)] = total > 0.0f ? sum * (1.0f / total) : 0.0f;
+        }
+    }
+}
+
 // Q8_0, one activation row, rows of at most 64 blocks (K <= 2048): the shape of the Q4_K decode kernel.  A lane owns one
 // block column for the whole kernel and keeps its 32 activations in registers; the 34 bytes of a block sit on a 2-byte
 // boundary, so a lane reads the nine words that cover it from the 4-byte boundary below it (the reference's own reading,
@@ -633,7 +707,8 @@ struct Q8Tile {
 // scalar registers as it starts (Q8_LEAD packs them: the rotation's width rides above the blocks a row, the SwiGLU flag above
 // N); they take the place of the same members of the parameter block, whose other members are loaded as they come to use.
 #define Q8_LEAD(p) (p).W[0], (p).W[1], (p).W[2], (p).x, (p).row_bytes, (p).nblk | ((p).rope_width << 16), (p).row_groups, (p).N | ((p).swiglu ? 0x80000000u : 0u), (p).end[0], (p).end[1], (p)
-template <int R, int G, bool DEEP = false, bool ROPE = false>
+// MERGE: the activation row is merged from a decode attention's section sums (x points at them) as it is staged.
+template <int R, int G, bool DEEP = false, bool ROPE = false, bool MERGE = false>
 __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(const uint8_t *lead_w0, const uint8_t *lead_w1, const uint8_t *lead_w2, const float *lead_x,
                                                                uint32_t lead_row_bytes, uint32_t lead_nblk_width, uint32_t lead_row_groups, uint32_t lead_n_swiglu,
                                                                uint32_t lead_end0, uint32_t lead_end1, GemvParams rest) {
@@ -694,7 +769,8 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(const uint8_t *le
     Q8Tile<R> held;
     if (rg < p.row_groups) load(held, rg);  // in flight while the activations are staged
 
-    stage_row(p.x, p.K, 0u, p.K, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew32(i); });
+    if constexpr (MERGE) stage_merged(p.x, p.merge_sections, p.merge_groups, p.merge_width, p.K, xs, [](uint32_t i) { return skew32(i); });
+    else stage_row(p.x, p.K, 0u, p.K, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew32(i); });
     __syncthreads();
 
     float xr[32];
@@ -2078,6 +2154,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
         p.end[s] = a.end[s];
     }
     p.x = x;
+    if (a.merge) p.x = a.merge->partial, p.merge_sections = a.merge->sections, p.merge_groups = a.merge->groups, p.merge_width = a.merge->width;
     p.y = y;
     p.residual = residual;
     p.norm_w = a.norm_w;
@@ -2150,6 +2227,8 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
 #define NH_LAUNCH(KERNEL, RR) hipLaunchKernelGGL((KERNEL<RR, RB>), grid, block, lds, d->stream, p)
 #define NH_DECODE(RR, GG) hipLaunchKernelGGL((gemv_q4k_decode_kernel<RR, GG, false, 4>), grid, block, lds, d->stream, p)
     const bool q8_direct = !q4 && RB == 1 && fast && p.nblk <= 256u;
+    if (a.merge && !(q8_direct && R == 2 && p.nblk <= 64u && !a.rope))
+        return fail(NH_E_ARGUMENT, "this product merges no attention sections (ask gemv_merges_sections first)");
     if (a.rope && !(q4 && RB == 1 && fast && R == 2 && p.splits == 1) && !(q8_direct && R == 2 && p.nblk <= 64u))
         return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (q4 && RB == 1 && fast && a.rope) {
@@ -2187,6 +2266,10 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
             if (p.group == 64) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
             else if (p.group == 32) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 32, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
             else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 16, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+        } else if (a.merge) {
+            if (p.group == 64) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, false, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+            else if (p.group == 32) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 32, false, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
+            else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 16, false, false, true>), wide, block, staged, d->stream, Q8_LEAD(p));
         } else if (deep) {
             if (R == 4) hipLaunchKernelGGL((gemv_q8_0_decode_kernel<4, 64, true>), wide, block, staged, d->stream, Q8_LEAD(p));
             else hipLaunchKernelGGL((gemv_q8_0_decode_kernel<2, 64, true>), wide, block, staged, d->stream, Q8_LEAD(p));
@@ -2585,8 +2668,21 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
     return NH_OK;
 }
 
+// What the Q8_0 decode kernel of two rows a lane group takes (launch_rows<1> sends such a product there), and the merge's own
+// bounds: whole heads, no more of them than the statistics' corner of LDS holds.
+bool gemv_merges_sections(const GemvArgs &a, uint32_t width) {
+    if (!env_int("NEURA_HIP_MERGE_IN_PRODUCT", 1) || a.element != NH_Q8_0 || a.rows != 1 || a.rope || a.swiglu || a.norm_w || a.digits_in || a.digits_out) return false;
+    if (!width || (width & (width - 1u)) || a.K % 32u || a.K / 32u > 64u || a.K % width || a.K / width > 32u) return false;
+    if (a.N < 2u || a.N >= 16384u || a.N % 2u || a.end[0] % 2u || a.end[1] % 2u) return false;
+    return (uint64_t)a.N * payload_bytes(a.element, a.K) < (1ull << 32);
+}
+
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (a.merge && (!gemv_merges_sections(a, a.merge->width) || a.merge->sections < 2u || a.merge->sections > MERGED_SECTIONS_MOST || !a.merge->groups ||
+                    (a.K / a.merge->width) % a.merge->groups))
+        return fail(NH_E_ARGUMENT, "this product merges no attention sections (ask gemv_merges_sections first)");
+    if (a.merge) return launch_rows<1>(d, a, a.x, a.y, a.residual);
     if (rows4_takes(a)) return launch_rows4(d, a);
     if (tile16_takes(a)) return launch_tile16(d, a);
     if (a.digits_out || a.digits_in) return fail(NH_E_ARGUMENT, "this product hands over no digit planes (ask gemv_hands_digits first)");

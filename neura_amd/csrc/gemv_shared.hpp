@@ -38,6 +38,8 @@ struct GemvParams {
     // (gemv_digit_bytes() of them): written by a SwiGLU epilogue in place of y, read by a plain product in place of x
     uint8_t *digits_out;
     const uint8_t *digits_in;
+    // Q8_0 decode kernel: x is the unmerged section sums of a decode attention (SectionSums), merged as the row is staged
+    uint32_t merge_sections, merge_groups, merge_width;
 };
 
 // the parameters a product reads before its first vector load, and the rotation's where it is folded in

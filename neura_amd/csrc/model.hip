@@ -223,6 +223,14 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
         at.heads = c.heads, at.kv_heads = c.kv_heads, at.batch = B, at.rows = rows, at.width = hd;
         at.capacity = m->capacity, at.keys = m->window, at.cursor = dev_cursor(m), at.scale = scale;
         at.reach = m->ring ? m->window : 0u;
+        // one row through a product that merges the attention's sections as it stages its row: the attention leaves them unmerged
+        SectionSums sums{};
+        GemvArgs o{};
+        if (!wide) {
+            o = narrow(m, element_at(m, L, O), m->attn_o[L], H, QW, m->att, T, m->h);
+            o.residual = m->h;
+            if (gemv_merges_sections(o, hd)) at.unmerged = &sums;
+        }
         if (!products_only && (status = launch_attention(d, at)) != NH_OK) return status;
         if (wide) {
             GemmArgs o{element_at(m, L, O), m->attn_o[L], H, QW, m->att, NH_F32, T, m->h, m->h, H};
@@ -245,8 +253,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             if (gated) dn.gate = m->act;
             if ((status = launch_gemm(d, dn)) != NH_OK) return status;
         } else {
-            GemvArgs o = narrow(m, element_at(m, L, O), m->attn_o[L], H, QW, m->att, T, m->h);
-            o.residual = m->h;
+            if (sums.sections) o.merge = &sums;
             if ((status = launch_gemv(d, o)) != NH_OK) return status;
             GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
             dn.residual = m->h;

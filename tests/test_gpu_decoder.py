@@ -534,6 +534,32 @@ def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monke
         held.release()
 
 
+def test_attention_sections_merged_by_the_output_projection_match_the_fold(device, monkeypatch):
+    """At batch 1 the attention of a Q8_0 decoder leaves the sums of its sections unmerged and the output projection merges
+    them as it stages its row (one launch fewer a layer); NEURA_HIP_MERGE_IN_PRODUCT=0 keeps the fold's own launch.  The
+    window is three sections of 54 keys: the steps walk from one section seen (the others empty: no mass) into the second.
+    Both twins stay within the decoder's bar of the oracle and choose its tokens."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    merged, ref, weights_a = build(device, TINY, NH_Q8_0, batch=1, context=160, seed=31)
+    folded, _, weights_b = build(device, TINY, NH_Q8_0, batch=1, context=160, seed=31)
+    token = 5
+    for step in range(70):
+        monkeypatch.setenv("NEURA_HIP_MERGE_IN_PRODUCT", "1")
+        got_a = merged.decode_step([token], [step])
+        logits_a = merged.logits()
+        monkeypatch.setenv("NEURA_HIP_MERGE_IN_PRODUCT", "0")
+        got_b = folded.decode_step([token], [step])
+        logits_b = folded.logits()
+        want_logits, want = ref.forward([token], 1, [step])
+        scale = np.abs(want_logits).max()
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * scale and np.abs(logits_b - want_logits).max() <= 1e-3 * scale, step
+        assert np.abs(logits_a - logits_b).max() <= 1e-4 * scale, step
+        assert list(got_a) == list(got_b) == list(want), (step, margins(want_logits))
+        token = int(got_a[0])
+    for held in (merged, folded, weights_a, weights_b):
+        held.release()
+
+
 def test_decoders_of_different_rope_bases_step_in_turn(device):
     """Two decoders of different rope bases and head widths stepping alternately at batch 2 (the rotation as its own
     kernel, read from the device's table of inverse frequencies): each keeps answering from its own recorded step as the
