@@ -37,6 +37,7 @@ struct nh_model {
     uint32_t *chosen_dev = nullptr;
     uint8_t *inputs_host = nullptr;  // pinned mirror of inputs_dev
     uint32_t *chosen_host = nullptr; // pinned [B + 1]: chosen tokens, then the refusal word
+    uint32_t *chosen_mapped = nullptr;  // the same words as the device addresses them: a step's last kernel writes them there
     uint32_t max_tokens = 0;
     // the decode step captured as a HIP graph: [0] all planes active, [1] some plane masked, [2], [3] the same with a sampled choice
     hipGraphExec_t decode_graph[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -282,6 +283,10 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
     return NH_OK;
 }
 
+__global__ __launch_bounds__(64) void publish_kernel(const uint32_t *chosen, const uint32_t *refusal, uint32_t batch, uint32_t *host) {
+    for (uint32_t i = threadIdx.x; i <= batch; i += 64u) host[i] = i < batch ? chosen[i] : *refusal;
+}
+
 // every kernel of one decode step: the layers, then logits = rms(hidden) . head^T and the greedy
 // choice (examples/qwen/model.rs:81-84, crates/neura-generate/src/sampling.rs:69-71)
 int32_t decode_kernels(nh_model *m, bool any_inactive, bool sampled) {
@@ -290,8 +295,14 @@ int32_t decode_kernels(nh_model *m, bool any_inactive, bool sampled) {
     GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
     head.norm_w = m->output_norm, head.eps = m->c.eps;
     if ((status = launch_gemv(m->d, head)) != NH_OK) return status;
-    if (sampled) return launch_sample(m->d, m->logits, m->c.batch, m->c.vocab, dev_draws(m), m->chosen_dev);
-    return launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
+    status = sampled ? launch_sample(m->d, m->logits, m->c.batch, m->c.vocab, dev_draws(m), m->chosen_dev)
+                     : launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
+    if (status != NH_OK || !m->chosen_mapped) return status;
+    // the choices and the refusal word go to the host's pinned words from a kernel of the step (part of the recorded graph): the
+    // two device-to-host copies they would otherwise take are two more operations behind every step
+    hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, m->d->stream, m->chosen_dev, m->d->refusal, m->c.batch, m->chosen_mapped);
+    NH_HIP(hipGetLastError());
+    return NH_OK;
 }
 
 }  // namespace
@@ -426,6 +437,7 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
     }
     ok = ok && hipHostMalloc((void **)&m->inputs_host, (T + 6 * c.batch + 4) * 4, hipHostMallocDefault) == hipSuccess &&
          hipHostMalloc((void **)&m->chosen_host, ((size_t)c.batch + 1) * 4, hipHostMallocDefault) == hipSuccess;
+    if (const char *held = getenv("NEURA_HIP_PUBLISH"); ok && !(held && held[0] == '0')) ok = hipHostGetDevicePointer((void **)&m->chosen_mapped, m->chosen_host, 0) == hipSuccess;
     // everything a captured step touches exists before the capture: the split partials of the
     // products (at most 5 slices x 4 rows), of the attention (at most 256 sections) and of the
     // greedy choice, and the rope table
@@ -517,8 +529,10 @@ static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *
         if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) return status;
         m->graph_warmed[variant] = true;
     }
-    NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
-    NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
+    if (!m->chosen_mapped) {
+        NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
+        NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
+    }
     NH_HIP(hipStreamSynchronize(d->stream));
     if (m->chosen_host[batch] != REFUSAL_NONE) return check_refusal(d, "a decode step");
     memcpy(chosen_out, m->chosen_host, (size_t)batch * 4);
