@@ -59,12 +59,15 @@ __global__ __launch_bounds__(256) void argmax_sections_kernel(const float *__res
     }
 }
 
+// `published`, where given: the host's pinned words [rows + 1] -- every row's choice again, then the word at `refusal`
 __global__ __launch_bounds__(256) void argmax_fold_kernel(const float *__restrict__ best_values, const uint32_t *__restrict__ best_indices,
-                                                          uint32_t sections, uint32_t *__restrict__ out) {
-    NH_FETCH(best_values, best_indices, sections, out);
+                                                          uint32_t sections, uint32_t *__restrict__ out, uint32_t *__restrict__ published,
+                                                          const uint32_t *__restrict__ refusal) {
+    NH_FETCH(best_values, best_indices, sections, out, published, refusal);
     __shared__ float held_values[4];
     __shared__ uint32_t held_indices[4];
     const uint32_t row = blockIdx.x;
+    const uint32_t refused = published && row == 0 && threadIdx.x == 0 ? *refusal : 0u;
     float value = -INFINITY;
     uint32_t index = 0xffffffffu;
     for (uint32_t s = threadIdx.x; s < sections; s += 256) {
@@ -73,7 +76,14 @@ __global__ __launch_bounds__(256) void argmax_fold_kernel(const float *__restric
         if (index == 0xffffffffu || precedes(value, index, held, at)) value = held, index = at;
     }
     block_choice(value, index, held_values, held_indices);
-    if (threadIdx.x == 0) out[row] = index == 0xffffffffu ? 0u : index;
+    if (threadIdx.x == 0) {
+        const uint32_t chosen = index == 0xffffffffu ? 0u : index;
+        out[row] = chosen;
+        if (published) {
+            published[row] = chosen;
+            if (row == 0) published[gridDim.x] = refused;
+        }
+    }
 }
 
 static uint32_t argmax_sections(uint32_t n) {
@@ -83,23 +93,25 @@ static uint32_t argmax_sections(uint32_t n) {
     return sections;
 }
 
-static int32_t launch_argmax_over(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out, uint8_t *held) {
+static int32_t launch_argmax_over(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out, uint8_t *held, uint32_t *published = nullptr,
+                                  const uint32_t *refusal = nullptr) {
     const uint32_t sections = argmax_sections(n);
     float *best_values = reinterpret_cast<float *>(held);
     uint32_t *best_indices = reinterpret_cast<uint32_t *>(held + (size_t)rows * sections * sizeof(float));
     hipLaunchKernelGGL(argmax_sections_kernel, dim3(sections, rows), dim3(256), 0, d->stream, values, n, sections, best_values, best_indices);
     NH_HIP(hipGetLastError());
-    hipLaunchKernelGGL(argmax_fold_kernel, dim3(rows), dim3(256), 0, d->stream, best_values, best_indices, sections, out);
+    hipLaunchKernelGGL(argmax_fold_kernel, dim3(rows), dim3(256), 0, d->stream, best_values, best_indices, sections, out, published, refusal);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
 
-int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out) {
+int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out, uint32_t *published, const uint32_t *refusal) {
     if (!rows) return NH_OK;
+    if (published && !refusal) return fail(NH_E_ARGUMENT, "choices published to the host go with the refusal word");
     const size_t bytes = (size_t)rows * argmax_sections(n) * (sizeof(float) + sizeof(uint32_t));
     uint8_t *held = static_cast<uint8_t *>(scratch(d, bytes));
     if (!held) return NH_E_MEMORY;
-    return launch_argmax_over(d, values, rows, n, out, held);
+    return launch_argmax_over(d, values, rows, n, out, held, published, refusal);
 }
 
 // ---- the greedy choice for callers that cannot allocate ----------------------------------------------------------

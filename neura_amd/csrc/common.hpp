@@ -276,7 +276,10 @@ int32_t launch_columns(nh_device *d, const float *src, uint32_t lds, const float
 int32_t launch_pack_q8_0(nh_device *d, const float *src, uint64_t elements, uint8_t *dst);
 int32_t launch_gather(nh_device *d, int32_t element, const void *table, uint32_t vocab, uint32_t width, const uint32_t *tokens,
                       uint32_t count, uint32_t batch, const uint8_t *mask, float *out);
-int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);
+// `published`, where given: pinned host words [rows + 1] as the device addresses them; the last kernel writes every row's choice
+// there too, and behind them the word at `refusal` (what a decode step's caller reads once the stream has drained)
+int32_t launch_argmax(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out, uint32_t *published = nullptr,
+                      const uint32_t *refusal = nullptr);
 // the same choice with its partials in a file-scope device array: no allocation, at most 64 rows
 int32_t argmax_static_setup(nh_device *d);
 int32_t launch_argmax_static(nh_device *d, const float *values, uint32_t rows, uint32_t n, uint32_t *out);

@@ -295,11 +295,12 @@ int32_t decode_kernels(nh_model *m, bool any_inactive, bool sampled) {
     GemvArgs head = narrow(m, m->output == m->token_embd ? m->elements[EMBD] : m->elements[HEAD], m->output, m->c.vocab, m->c.hidden, m->h, m->c.batch, m->logits);
     head.norm_w = m->output_norm, head.eps = m->c.eps;
     if ((status = launch_gemv(m->d, head)) != NH_OK) return status;
-    status = sampled ? launch_sample(m->d, m->logits, m->c.batch, m->c.vocab, dev_draws(m), m->chosen_dev)
-                     : launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev);
-    if (status != NH_OK || !m->chosen_mapped) return status;
     // the choices and the refusal word go to the host's pinned words from a kernel of the step (part of the recorded graph): the
-    // two device-to-host copies they would otherwise take are two more operations behind every step
+    // two device-to-host copies they would otherwise take are two more operations behind every step.  The greedy choice's
+    // last kernel writes them itself; a sampled step has a kernel for it.
+    if (!sampled) return launch_argmax(m->d, m->logits, m->c.batch, m->c.vocab, m->chosen_dev, m->chosen_mapped, m->d->refusal);
+    status = launch_sample(m->d, m->logits, m->c.batch, m->c.vocab, dev_draws(m), m->chosen_dev);
+    if (status != NH_OK || !m->chosen_mapped) return status;
     hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, m->d->stream, m->chosen_dev, m->d->refusal, m->c.batch, m->chosen_mapped);
     NH_HIP(hipGetLastError());
     return NH_OK;
