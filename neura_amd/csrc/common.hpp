@@ -192,6 +192,10 @@ struct GemvArgs {
     // Only where gemv_merges_sections() says so: the activation row is the attention output these sections merge into
     // (x is not read); the product merges them as it stages its row, and the attention's own fold launch falls away.
     const SectionSums *merge = nullptr;
+    // Only for a one-row product of a staged K-quant (Q6_K, Q5_K, Q3_K) over one K slice (K <= 4096): the value projection of a
+    // token whose q|k went out rotated from their own product -- its rows (+ bias[0]) are also cast into the value state
+    // (cache_v, cursor, width, capacity and ring of this RopeFusion; halves), what launch_value_append does from y.
+    const RopeFusion *append_value = nullptr;
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
 // whether launch_gemv can merge attention sections of `width` channels a head into the activation row of this product

@@ -962,6 +962,7 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) 
     const uint32_t blk0 = split * p.blocks_per_split;
     const uint32_t nb = min(p.blocks_per_split, p.nblk - blk0);
     const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
+    const uint32_t append_cursor = RB == 1 && p.append_value ? p.rope_cursor[0] : 0u;  // asked for here, wanted at the very end
     // halves of 128 activations sit 16 bytes apart: the lanes of a wave read eight of them at once
     const uint32_t xstride = skew128(p.blocks_per_split * 256u);
     for (uint32_t b = 0; b < RB; b++) {
@@ -1092,6 +1093,16 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) 
 #pragma unroll
             for (int b = 0; b < RB; b++) acc[r][b] = wave_sum(acc[r][b]);
         if (lane == 0) publish<2, RB>(p, first, split, acc);
+        if (RB == 1 && p.append_value && lane < 2 && first + lane < p.N) {
+            // a value projection of one token: its rows (+ bias) go into the value state at the cursor as halves, as
+            // value_append_kernel would cast them
+            const uint32_t n = first + lane;
+            const float sum = lane ? acc[1][0] : acc[0][0];
+            const float value = p.bias[0] ? sum + p.bias[0][n] : sum;
+            const uint32_t slot = p.rope_ring ? append_cursor % p.rope_ring : append_cursor;
+            if (slot >= p.rope_capacity) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+            else p.rope_v[((uint64_t)(n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + n % p.rope_width] = float_to_half(value);
+        }
         __builtin_amdgcn_wave_barrier();  // the next rows overwrite the staged ones
     }
 }
@@ -2638,6 +2649,12 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
     p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps;
     p.row_bytes = (uint32_t)payload_bytes(ELEMENT, a.K);
     p.nblk = a.K / 256u;
+    if (a.append_value) {
+        if (RB != 1 || a.swiglu || residual || p.nblk > 16u || !a.append_value->width || a.N % a.append_value->width)
+            return fail(NH_E_ARGUMENT, "this product appends no value rows (one row, one K slice, whole heads, no other epilogue)");
+        p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
+        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.bias[0] = a.bias[0], p.refusal = d->refusal;
+    }
     const uint32_t most_blocks = 16u;
     p.splits = (p.nblk + most_blocks - 1) / most_blocks;
     p.blocks_per_split = (p.nblk + p.splits - 1) / p.splits;
@@ -2678,7 +2695,10 @@ bool gemv_merges_sections(const GemvArgs &a, uint32_t width) {
 }
 
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
-    if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
+    if (!a.rope && !a.append_value && (a.bias[0] || a.bias[1] || a.bias[2]))
+        return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in or appends value rows");
+    if (a.append_value && !(staged_super_block(a.element) && a.rows == 1 && !a.rope))
+        return fail(NH_E_ARGUMENT, "only a one-row product of a staged K-quant appends its rows to the value state");
     if (a.merge && (!gemv_merges_sections(a, a.merge->width) || a.merge->sections < 2u || a.merge->sections > MERGED_SECTIONS_MOST || !a.merge->groups ||
                     (a.K / a.merge->width) % a.merge->groups))
         return fail(NH_E_ARGUMENT, "this product merges no attention sections (ask gemv_merges_sections first)");
@@ -2687,7 +2707,6 @@ int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (tile16_takes(a)) return launch_tile16(d, a);
     if (a.digits_out || a.digits_in) return fail(NH_E_ARGUMENT, "this product hands over no digit planes (ask gemv_hands_digits first)");
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
-    if (!a.rope && (a.bias[0] || a.bias[1] || a.bias[2])) return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in");
     if (f16_tiles_take(d, a)) return launch_f16_tiles(d, a);
     if (mfma32_takes(d, a)) return launch_mfma32(d, a);
     if (mfma_takes(a)) return launch_mfma(d, a);

@@ -40,6 +40,8 @@ struct GemvParams {
     const uint8_t *digits_in;
     // Q8_0 decode kernel: x is the unmerged section sums of a decode attention (SectionSums), merged as the row is staged
     uint32_t merge_sections, merge_groups, merge_width;
+    // staged K-quant kernel, one row: the outputs (+ bias[0]) also go into the value state rope_v at rope_cursor as halves
+    uint32_t append_value;
 };
 
 // the parameters a product reads before its first vector load, and the rotation's where it is folded in

@@ -560,6 +560,35 @@ def test_attention_sections_merged_by_the_output_projection_match_the_fold(devic
         held.release()
 
 
+def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, monkeypatch):
+    """Where q|k go out rotated from one product and the value projection is stored otherwise (layer 0 of the Q4_K_M-like
+    mix: Q6_K), the value product casts its rows (+ bias) into the value state itself; NEURA_HIP_APPEND_VALUE=0 leaves that
+    to the append kernel.  The same sums either way: states and logits equal bit for bit, and the oracle's tokens."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    shape = SMALL_Q4
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, np.random.default_rng(21), mode="normal", elements=MIXED, biases=(0, 1)))
+    host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
+    weights = Weights(device, tensors)
+    fused, apart = Model(device, weights, shape, NH_Q4_K, 1, 24, 1), Model(device, weights, shape, NH_Q4_K, 1, 24, 1)
+    ref = oracle.Model(shape, NH_Q4_K, host, 1, 24, 1, elements=MIXED)
+    token = 11
+    for step in range(6):
+        monkeypatch.setenv("NEURA_HIP_APPEND_VALUE", "1")
+        got_a = fused.decode_step([token], [step])
+        logits_a = fused.logits()
+        monkeypatch.setenv("NEURA_HIP_APPEND_VALUE", "0")
+        got_b = apart.decode_step([token], [step])
+        assert np.array_equal(logits_a, apart.logits()), step
+        want_logits, want = ref.forward([token], 1, [step])
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got_a) == list(got_b) == list(want), (step, margins(want_logits))
+        token = int(got_a[0])
+    for layer in range(shape["layers"]):
+        assert np.array_equal(fused.cache_read(layer, 1), apart.cache_read(layer, 1)), layer
+    assert np.any(fused.cache_read(0, 1)[:, 0, :6])
+    fused.release(), apart.release(), weights.release()
+
+
 def test_decoders_of_different_rope_bases_step_in_turn(device):
     """Two decoders of different rope bases and head widths stepping alternately at batch 2 (the rotation as its own
     kernel, read from the device's table of inverse frequencies): each keeps answering from its own recorded step as the
