@@ -43,38 +43,53 @@ __device__ float rms_scale(const float *__restrict__ x, uint32_t K, float eps, f
 }
 
 // Stages x[k0 .. k0 + kn) of one activation row into LDS at dst[skew(i)], RMS-normalised over the whole row and
-// weighed when norm_w is given.  With 256 threads and at most 16 values per thread every load goes out before the
+// weighed when norm_w is given.  With 256 threads and at most 32 values per thread every load goes out before the
 // first value is used and the row is read once: a loop that handles each value as it arrives spends one memory
 // round trip per value (6 us on a 3584-wide row).  Deeper slices take the looped form.
+template <int PER, typename Skew>
+__device__ __forceinline__ void stage_row_at_once(const float *__restrict__ x, uint32_t K, uint32_t k0, uint32_t kn, const float *__restrict__ norm_w,
+                                                  float eps, float *dst, float *red, Skew skew) {
+    const uint32_t tid = threadIdx.x;
+    float held[PER], weight[PER];
+    // every load is issued whatever its column (past the slice it reads the slice's last value, dropped below): loads
+    // under a condition wait for one another
+#pragma unroll
+    for (int j = 0; j < PER; j++) held[j] = x[k0 + min(tid + 256u * j, kn - 1u)];
+    if (norm_w) {
+#pragma unroll
+        for (int j = 0; j < PER; j++) weight[j] = norm_w[k0 + min(tid + 256u * j, kn - 1u)];
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+        if (tid + 256u * j >= kn) held[j] = 0.0f;
+    if (norm_w) {
+        float square = 0.0f;  // thread t adds columns t, t + 256, ... in order (crates/neura-kernel/src/task/norm.rs:69-83)
+#pragma unroll
+        for (int j = 0; j < PER; j++) square = __fadd_rn(square, __fmul_rn(held[j], held[j]));
+        square = wave_sum(square);
+        if ((tid & 63u) == 0) red[tid >> 6] = square;
+        __syncthreads();
+        const float scale = rms_scale_of((red[0] + red[1]) + (red[2] + red[3]), K, eps);
+        __syncthreads();  // red is reused by the next row
+#pragma unroll
+        for (int j = 0; j < PER; j++) held[j] = __fmul_rn(__fmul_rn(held[j], scale), weight[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+        const uint32_t c = tid + 256u * j;
+        if (c < kn) dst[skew(c)] = held[j];
+    }
+}
+
 template <typename Skew>
 __device__ __forceinline__ void stage_row(const float *__restrict__ x, uint32_t K, uint32_t k0, uint32_t kn, const float *__restrict__ norm_w,
                                           float eps, float *dst, float *red, Skew skew) {
     const uint32_t tid = threadIdx.x;
-    if (blockDim.x == 256 && kn <= 4096u && (!norm_w || (k0 == 0 && kn == K))) {
-        float held[16], weight[16];
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t c = tid + 256u * j;
-            held[j] = c < kn ? x[k0 + c] : 0.0f;
-            weight[j] = (norm_w && c < kn) ? norm_w[k0 + c] : 0.0f;
-        }
-        if (norm_w) {
-            float square = 0.0f;  // thread t adds columns t, t + 256, ... in order (crates/neura-kernel/src/task/norm.rs:69-83)
-#pragma unroll
-            for (int j = 0; j < 16; j++) square = __fadd_rn(square, __fmul_rn(held[j], held[j]));
-            square = wave_sum(square);
-            if ((tid & 63u) == 0) red[tid >> 6] = square;
-            __syncthreads();
-            const float scale = rms_scale_of((red[0] + red[1]) + (red[2] + red[3]), K, eps);
-            __syncthreads();  // red is reused by the next row
-#pragma unroll
-            for (int j = 0; j < 16; j++) held[j] = __fmul_rn(__fmul_rn(held[j], scale), weight[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t c = tid + 256u * j;
-            if (c < kn) dst[skew(c)] = held[j];
-        }
+    const bool at_once = blockDim.x == 256 && kn > 0 && (!norm_w || (k0 == 0 && kn == K));
+    if (at_once && kn <= 4096u) {
+        stage_row_at_once<16>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (at_once && kn <= 8192u) {
+        stage_row_at_once<32>(x, K, k0, kn, norm_w, eps, dst, red, skew);
     } else {
         float scale = 1.0f;
         if (norm_w) scale = rms_scale(x, K, eps, red);
