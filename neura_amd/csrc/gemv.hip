@@ -86,7 +86,11 @@ __device__ __forceinline__ void stage_row(const float *__restrict__ x, uint32_t 
                                           float eps, float *dst, float *red, Skew skew) {
     const uint32_t tid = threadIdx.x;
     const bool at_once = blockDim.x == 256 && kn > 0 && (!norm_w || (k0 == 0 && kn == K));
-    if (at_once && kn <= 4096u) {
+    if (at_once && kn <= 1024u) {  // no more loads than the slice needs, to the next power of two
+        stage_row_at_once<4>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (at_once && kn <= 2048u) {
+        stage_row_at_once<8>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (at_once && kn <= 4096u) {
         stage_row_at_once<16>(x, K, k0, kn, norm_w, eps, dst, red, skew);
     } else if (at_once && kn <= 8192u) {
         stage_row_at_once<32>(x, K, k0, kn, norm_w, eps, dst, red, skew);
