@@ -81,19 +81,20 @@ __device__ __forceinline__ void stage_row_at_once(const float *__restrict__ x, u
     }
 }
 
-template <typename Skew>
+// MOST: the values a thread holds at most (a kernel pays for its widest form in registers whether or not a launch takes it)
+template <int MOST = 16, typename Skew>
 __device__ __forceinline__ void stage_row(const float *__restrict__ x, uint32_t K, uint32_t k0, uint32_t kn, const float *__restrict__ norm_w,
                                           float eps, float *dst, float *red, Skew skew) {
     const uint32_t tid = threadIdx.x;
     const bool at_once = blockDim.x == 256 && kn > 0 && (!norm_w || (k0 == 0 && kn == K));
     if (at_once && kn <= 1024u) {  // no more loads than the slice needs, to the next power of two
         stage_row_at_once<4>(x, K, k0, kn, norm_w, eps, dst, red, skew);
-    } else if (at_once && kn <= 2048u) {
-        stage_row_at_once<8>(x, K, k0, kn, norm_w, eps, dst, red, skew);
-    } else if (at_once && kn <= 4096u) {
-        stage_row_at_once<16>(x, K, k0, kn, norm_w, eps, dst, red, skew);
-    } else if (at_once && kn <= 8192u) {
-        stage_row_at_once<32>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (MOST >= 8 && at_once && kn <= 2048u) {
+        stage_row_at_once<MOST >= 8 ? 8 : 4>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (MOST >= 16 && at_once && kn <= 4096u) {
+        stage_row_at_once<MOST >= 16 ? 16 : 4>(x, K, k0, kn, norm_w, eps, dst, red, skew);
+    } else if (MOST >= 32 && at_once && kn <= 8192u) {
+        stage_row_at_once<MOST >= 32 ? 32 : 4>(x, K, k0, kn, norm_w, eps, dst, red, skew);
     } else {
         float scale = 1.0f;
         if (norm_w) scale = rms_scale(x, K, eps, red);
@@ -789,7 +790,7 @@ __global__ __launch_bounds__(256) void gemv_q8_0_decode_kernel(const uint8_t *le
     if (rg < p.row_groups) load(held, rg);  // in flight while the activations are staged
 
     if constexpr (MERGE) stage_merged(p.x, p.merge_sections, p.merge_groups, p.merge_width, p.K, xs, [](uint32_t i) { return skew32(i); });
-    else stage_row(p.x, p.K, 0u, p.K, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew32(i); });
+    else stage_row<DEEP ? 32 : 8>(p.x, p.K, 0u, p.K, p.norm_w, p.eps, xs, red, [](uint32_t i) { return skew32(i); });  // rows of 256 blocks, or of 64
     __syncthreads();
 
     float xr[32];
