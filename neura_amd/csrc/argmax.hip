@@ -48,9 +48,17 @@ __global__ __launch_bounds__(256) void argmax_sections_kernel(const float *__res
     const float *src = values + (size_t)row * n;
     float value = -INFINITY;
     uint32_t index = first < n ? first : 0u;
-    for (uint32_t i = first + threadIdx.x; i < last; i += 256) {
-        float held = src[i];
-        if (precedes(value, index, held, i)) value = held, index = i;
+    // eight values a thread at a time, all asked for before the first is compared (past the section its last value again,
+    // dropped): a loop that compares each value as it arrives spends a memory round trip on every one
+    for (uint32_t base = first; base < last; base += 2048u) {
+        float held[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) held[j] = src[min(base + threadIdx.x + 256u * j, last - 1u)];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t i = base + threadIdx.x + 256u * j;
+            if (i < last && precedes(value, index, held[j], i)) value = held[j], index = i;
+        }
     }
     block_choice(value, index, held_values, held_indices);
     if (threadIdx.x == 0) {
