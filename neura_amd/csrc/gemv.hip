@@ -983,29 +983,6 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) 
     const uint32_t nb = min(p.blocks_per_split, p.nblk - blk0);
     const uint32_t k0 = blk0 * 256u, kn = nb * 256u;
     const uint32_t append_cursor = RB == 1 && p.append_value ? p.rope_cursor[0] : 0u;  // asked for here, wanted at the very end
-    // halves of 128 activations sit 16 bytes apart: the lanes of a wave read eight of them at once
-    const uint32_t xstride = skew128(p.blocks_per_split * 256u);
-    for (uint32_t b = 0; b < RB; b++) {
-        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew128(i); });
-    }
-    __syncthreads();
-    // what the codes' offset (or a run's minimum) multiplies, once for all rows: per unit and run the sum of the eight
-    // activations, times the offset where the format has one
-    float *const sums = xs + RB * xstride;
-    const uint32_t sstride = p.blocks_per_split * 32u;
-    for (uint32_t b = 0; b < RB; b++)
-        for (uint32_t q = tid; q < nb * 32u; q += 256u) {
-            const uint32_t u = q >> 2, g = q & 3u;
-            const float4 *at = reinterpret_cast<const float4 *>(xs + b * xstride + skew128((u >> 2) * 128u) + g * 32u + 8u * (u & 3u));
-            const float4 lo = at[0], hi = at[1];
-            const float total = ((lo.x + lo.y) + (lo.z + lo.w)) + ((hi.x + hi.y) + (hi.z + hi.w));
-            sums[b * sstride + q] = Format::FLOORS ? total : -Format::OFFSET * total;
-        }
-    __syncthreads();
-    const uint32_t raw_stride = p.chunks_per_row * 16u;  // bytes of one staged row slice
-    uint8_t *const mine = reinterpret_cast<uint8_t *>(sums + RB * sstride) + (size_t)wave * 2u * raw_stride;
-    const uint32_t units = nb * 8u;
-
     // the 16-byte pieces of the two rows `first`, `first + 1` this lane copies: fetched one pair of rows ahead, so the copy
     // of the next pair is in flight while this pair is multiplied (a slice is at most 16 blocks: four pieces a lane and row)
     typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
@@ -1042,7 +1019,30 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) 
     };
     const uint32_t stride = 2u * gridDim.x * 4u;
     uint32_t first = 2u * (blockIdx.x * 4u + wave);
-    if (first < p.N) fetch(first);
+    if (first < p.N) fetch(first);  // on its way while the activations are staged
+    // halves of 128 activations sit 16 bytes apart: the lanes of a wave read eight of them at once
+    const uint32_t xstride = skew128(p.blocks_per_split * 256u);
+    for (uint32_t b = 0; b < RB; b++) {
+        stage_row(p.x + (size_t)b * p.K, p.K, k0, kn, p.norm_w, p.eps, xs + b * xstride, red, [](uint32_t i) { return skew128(i); });
+    }
+    __syncthreads();
+    // what the codes' offset (or a run's minimum) multiplies, once for all rows: per unit and run the sum of the eight
+    // activations, times the offset where the format has one
+    float *const sums = xs + RB * xstride;
+    const uint32_t sstride = p.blocks_per_split * 32u;
+    for (uint32_t b = 0; b < RB; b++)
+        for (uint32_t q = tid; q < nb * 32u; q += 256u) {
+            const uint32_t u = q >> 2, g = q & 3u;
+            const float4 *at = reinterpret_cast<const float4 *>(xs + b * xstride + skew128((u >> 2) * 128u) + g * 32u + 8u * (u & 3u));
+            const float4 lo = at[0], hi = at[1];
+            const float total = ((lo.x + lo.y) + (lo.z + lo.w)) + ((hi.x + hi.y) + (hi.z + hi.w));
+            sums[b * sstride + q] = Format::FLOORS ? total : -Format::OFFSET * total;
+        }
+    __syncthreads();
+    const uint32_t raw_stride = p.chunks_per_row * 16u;  // bytes of one staged row slice
+    uint8_t *const mine = reinterpret_cast<uint8_t *>(sums + RB * sstride) + (size_t)wave * 2u * raw_stride;
+    const uint32_t units = nb * 8u;
+
     for (; first < p.N; first += stride) {
         uint32_t lead[2];
 #pragma unroll
@@ -2155,11 +2155,23 @@ __global__ __launch_bounds__(256) void gemv_fold_kernel(const float *__restrict_
     uint32_t outputs = swiglu ? N / 2 : N;
     for (uint32_t index = blockIdx.x * blockDim.x + threadIdx.x; index < rows * outputs; index += gridDim.x * blockDim.x) {
         uint32_t b = index / outputs, n = index % outputs;
-        float total = 0.0f;
-        for (uint32_t s = 0; s < splits; s++) total += partial[((size_t)s * rows + b) * N + n];
+        // eight slices at a time, every load asked for before the first is added (past the last slice the last again,
+        // dropped): the sum still runs in slice order
+        auto sum_of = [&](uint32_t column) {
+            float total = 0.0f;
+            for (uint32_t s0 = 0; s0 < splits; s0 += 8u) {
+                float held[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) held[j] = partial[((size_t)min(s0 + j, splits - 1u) * rows + b) * N + column];
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (s0 + j < splits) total += held[j];
+            }
+            return total;
+        };
+        float total = sum_of(n);
         if (swiglu) {
-            float up = 0.0f;
-            for (uint32_t s = 0; s < splits; s++) up += partial[((size_t)s * rows + b) * N + N / 2 + n];
+            const float up = sum_of(N / 2 + n);
             total = silu(total) * up;
         } else if (residual) {
             total = residual[(size_t)b * N + n] + total;
