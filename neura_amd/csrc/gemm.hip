@@ -139,6 +139,42 @@ __device__ __forceinline__ void fetch_parameters(const GemmQ4Params &p) {
     NH_FETCH(p.W, p.W1, p.W2, p.end0, p.end1, p.N, p.K, p.row_bytes, p.A, p.S, p.rows, p.Y, p.residual, p.ldy, p.M, p.split, p.unscale);
 }
 
+// Four neighbouring numbers of a row (`hi`: as halves; `lo`, with SPLIT: their residues * 2^11) into the packed rows, and their
+// share of the sub-block sums: eight neighbouring lanes hold the 32 numbers of a sub-block.
+template <bool SPLIT>
+__device__ __forceinline__ void pack_piece(const _Float16 (&hi)[4], const _Float16 (&lo)[4], uint32_t row, uint32_t k, uint32_t K, uint32_t nsb,
+                                           _Float16 *__restrict__ A, _Float16 *__restrict__ S) {
+    // the nibbles of four weight bytes unpack as bytes 0, 2, 1, 3
+    const half4_t out_hi = {hi[0], hi[2], hi[1], hi[3]}, out_lo = {lo[0], lo[2], lo[1], lo[3]};
+    *reinterpret_cast<half4_t *>(A + (size_t)row * K + k) = out_hi;
+    if (SPLIT) *reinterpret_cast<half4_t *>(A + (size_t)(row + 1u) * K + k) = out_lo;
+    // sums of the 32 halves of a sub-block: eight neighbouring lanes
+    float sum_hi = ((float)hi[0] + (float)hi[1]) + ((float)hi[2] + (float)hi[3]);
+    float sum_lo = ((float)lo[0] + (float)lo[1]) + ((float)lo[2] + (float)lo[3]);
+#pragma unroll
+    for (int offset = 1; offset < 8; offset <<= 1) {
+        sum_hi += __shfl_xor(sum_hi, offset, 64);
+        sum_lo += __shfl_xor(sum_lo, offset, 64);
+    }
+    if ((threadIdx.x & 7u) == 0) {
+        const uint32_t sb = k >> 8, slot = (k >> 5) & 7u;
+        {
+            const float v = sum_hi * 0.015625f;
+            const _Float16 h = (_Float16)v;
+            _Float16 *dst = S + ((size_t)row * nsb + sb) * 16u;
+            dst[slot] = h;
+            dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
+        }
+        if (SPLIT) {
+            const float v = sum_lo * 0.015625f;
+            const _Float16 h = (_Float16)v;
+            _Float16 *dst = S + ((size_t)(row + 1u) * nsb + sb) * 16u;
+            dst[slot] = h;
+            dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
+        }
+    }
+}
+
 // One workgroup per activation row: the row as MFMA-ready halves (and, for fp32 rows, its residue row and scale).
 // PRELUDE: what a row is before it is packed -- 0: X as it lies; 1: X normalised (rmsnorm_kernel's arithmetic, so the same
 // fp32 numbers: thread t adds the squares of columns t, t + 256, ..., then a 256-wide tree); 2: silu(gate) * X as
@@ -213,38 +249,101 @@ __global__ __launch_bounds__(256) void gemm_pack_rows_kernel(const void *__restr
                 lo[e] = (_Float16)((t[e] - (float)hi[e]) * 2048.0f);
             }
         }
-        // the nibbles of four weight bytes unpack as bytes 0, 2, 1, 3
-        const half4_t out_hi = {hi[0], hi[2], hi[1], hi[3]}, out_lo = {lo[0], lo[2], lo[1], lo[3]};
-        *reinterpret_cast<half4_t *>(A + (size_t)row * K + k) = out_hi;
-        if (!HALF_IN) *reinterpret_cast<half4_t *>(A + (size_t)(row + 1u) * K + k) = out_lo;
-        // sums of the 32 halves of a sub-block: eight neighbouring lanes
-        float sum_hi = ((float)hi[0] + (float)hi[1]) + ((float)hi[2] + (float)hi[3]);
-        float sum_lo = ((float)lo[0] + (float)lo[1]) + ((float)lo[2] + (float)lo[3]);
-#pragma unroll
-        for (int offset = 1; offset < 8; offset <<= 1) {
-            sum_hi += __shfl_xor(sum_hi, offset, 64);
-            sum_lo += __shfl_xor(sum_lo, offset, 64);
-        }
-        if ((tid & 7u) == 0) {
-            const uint32_t sb = k >> 8, slot = (k >> 5) & 7u;
-            {
-                const float v = sum_hi * 0.015625f;
-                const _Float16 h = (_Float16)v;
-                _Float16 *dst = S + ((size_t)row * nsb + sb) * 16u;
-                dst[slot] = h;
-                dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
-            }
-            if (!HALF_IN) {
-                const float v = sum_lo * 0.015625f;
-                const _Float16 h = (_Float16)v;
-                _Float16 *dst = S + ((size_t)(row + 1u) * nsb + sb) * 16u;
-                dst[slot] = h;
-                dst[8u + slot] = (_Float16)((v - (float)h) * 2048.0f);
-            }
-        }
+        pack_piece<!HALF_IN>(hi, lo, row, k, K, nsb, A, S);
     }
 }
 
+// The same for fp32 rows, through LDS: the kernel above walks a row three times (the norm's squares, the largest magnitude,
+// the packing) and meets every value as it arrives -- a memory round trip a value and walk, 22 in a row on a 3584-wide row
+// with the norm, 37 on an 18944-wide gated one.  Here a row crosses memory once, four 16-byte loads a thread in flight at a
+// time, and waits in LDS as the prelude left it: the squares are added from LDS in the same thread order, the packing reads
+// LDS.  The same arithmetic on the same numbers: the packed rows are the kernel above's bit for bit.  K is a multiple of 4.
+template <int PRELUDE>
+__global__ __launch_bounds__(256) void gemm_pack_rows_staged_kernel(const float *__restrict__ X, uint32_t K, _Float16 *__restrict__ A,
+                                                                    _Float16 *__restrict__ S, float *__restrict__ unscale,
+                                                                    const float *__restrict__ aux, float eps) {
+    extern __shared__ __attribute__((aligned(16))) float staged_row[];  // [K]
+    __shared__ uint32_t wave_top[4];
+    __shared__ float red[256];
+    const uint32_t m = blockIdx.x, tid = threadIdx.x;
+    const uint32_t nsb = (K + 255u) / 256u;
+    const float *xr = X + (size_t)m * K;
+    const float *other = PRELUDE == PACK_NORM ? aux : (PRELUDE == PACK_SWIGLU ? aux + (size_t)m * K : nullptr);
+    float norm = 1.0f;
+    if (PRELUDE == PACK_NORM) {
+        for (uint32_t k0 = tid * 4u; k0 < K; k0 += 4096u) {
+            float4 held[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) held[j] = *reinterpret_cast<const float4 *>(xr + min(k0 + 1024u * j, K - 4u));
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (k0 + 1024u * j < K) *reinterpret_cast<float4 *>(staged_row + k0 + 1024u * j) = held[j];
+        }
+        __syncthreads();
+        float square = 0.0f;  // thread t adds the squares of columns t, t + 256, ... as rmsnorm_kernel does
+        for (uint32_t c = tid; c < K; c += 256) square = __fadd_rn(square, __fmul_rn(staged_row[c], staged_row[c]));
+        red[tid] = square;
+        __syncthreads();
+        for (uint32_t stride = 128; stride > 0; stride >>= 1) {
+            if (tid < stride) red[tid] = __fadd_rn(red[tid], red[tid + stride]);
+            __syncthreads();
+        }
+        norm = rms_scale_of(red[0], K, eps);
+    }
+    uint32_t top = 0;
+    for (uint32_t k0 = tid * 4u; k0 < K; k0 += 4096u) {
+        float4 held[4], with[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t k = min(k0 + 1024u * j, K - 4u);
+            held[j] = PRELUDE == PACK_NORM ? *reinterpret_cast<const float4 *>(staged_row + k) : *reinterpret_cast<const float4 *>(xr + k);
+            if (PRELUDE != PACK_PLAIN) with[j] = *reinterpret_cast<const float4 *>(other + k);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (k0 + 1024u * j >= K) continue;
+            float4 v = held[j];
+            if (PRELUDE == PACK_NORM) {
+                const float4 w = with[j];
+                v.x = __fmul_rn(__fmul_rn(v.x, norm), w.x), v.y = __fmul_rn(__fmul_rn(v.y, norm), w.y);
+                v.z = __fmul_rn(__fmul_rn(v.z, norm), w.z), v.w = __fmul_rn(__fmul_rn(v.w, norm), w.w);
+            } else if (PRELUDE == PACK_SWIGLU) {
+                const float4 g = with[j];
+                v.x = g.x * (1.0f / (1.0f + expf(-g.x))) * v.x, v.y = g.y * (1.0f / (1.0f + expf(-g.y))) * v.y;
+                v.z = g.z * (1.0f / (1.0f + expf(-g.z))) * v.z, v.w = g.w * (1.0f / (1.0f + expf(-g.w))) * v.w;
+            }
+            top = max(max(top, __builtin_bit_cast(uint32_t, v.x) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.y) & 0x7fffffffu);
+            top = max(max(top, __builtin_bit_cast(uint32_t, v.z) & 0x7fffffffu), __builtin_bit_cast(uint32_t, v.w) & 0x7fffffffu);
+            *reinterpret_cast<float4 *>(staged_row + k0 + 1024u * j) = v;  // the thread that packs these four wrote them
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) top = max(top, (uint32_t)__shfl_xor((int)top, offset, 64));
+    if ((tid & 63u) == 0) wave_top[tid >> 6] = top;
+    __syncthreads();
+    top = max(max(wave_top[0], wave_top[1]), max(wave_top[2], wave_top[3]));
+    // a power of two that puts the largest magnitude in [2^13, 2^14)
+    const uint32_t raw = top >> 23, exponent = min(max(raw, 27u), 254u);
+    const float scale = __builtin_bit_cast(float, (267u - exponent) << 23);
+    if (tid == 0) unscale[m] = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 13u) << 23);
+    for (uint32_t k = tid * 4u; k < K; k += 1024u) {
+        const float4 v = *reinterpret_cast<const float4 *>(staged_row + k);
+        const float t[4] = {v.x * scale, v.y * scale, v.z * scale, v.w * scale};
+        _Float16 hi[4], lo[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            hi[e] = (_Float16)t[e];
+            lo[e] = (_Float16)((t[e] - (float)hi[e]) * 2048.0f);
+        }
+        pack_piece<true>(hi, lo, 2u * m, k, K, nsb, A, S);
+    }
+}
+
+static bool pack_unstaged() {  // NEURA_HIP_PACK_STAGED=0: the packing that walks a row in memory
+    const char *held = getenv("NEURA_HIP_PACK_STAGED");
+    return held && held[0] == '0';
+}
+constexpr size_t PACK_STAGED_LDS_MOST = 152 * 1024;  // the widest row the staged packing holds: 38912 numbers
 constexpr size_t GEMM_Q4K_LDS = sizeof(_Float16) * (2 * GT * GS + 2 * GT * GS + 2 * GT * 8) + sizeof(uint32_t) * 2 * GT;
 
 // What the multiplier waves of a super-block wide product do (waves 0..3 of the workgroup; the stagers fill As, Bs, mns and dds).
@@ -1131,6 +1230,20 @@ static int32_t launch_gemm_mfma(nh_device *d, const GemmArgs &a) {
         // what the launch before left in the scratch is this launch's operand
     } else if (half_rows) {
         hipLaunchKernelGGL(gemm_pack_rows_kernel<true>, dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, nullptr, 0.0f);
+    } else if (a.K % 4u == 0 && a.K >= 4u && (size_t)a.K * sizeof(float) <= PACK_STAGED_LDS_MOST && !pack_unstaged()) {
+        // a row of fp32 numbers crosses memory once and waits in LDS
+        const size_t lds = (size_t)a.K * sizeof(float);
+        static bool roomy = false;
+        if (!roomy) {
+            NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pack_rows_staged_kernel<PACK_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)PACK_STAGED_LDS_MOST));
+            NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pack_rows_staged_kernel<PACK_NORM>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)PACK_STAGED_LDS_MOST));
+            NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pack_rows_staged_kernel<PACK_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)PACK_STAGED_LDS_MOST));
+            roomy = true;
+        }
+        const float *rows = static_cast<const float *>(a.X);
+        if (a.norm_w) hipLaunchKernelGGL(gemm_pack_rows_staged_kernel<PACK_NORM>, dim3(a.M), dim3(256), lds, d->stream, rows, a.K, A, S, unscale, a.norm_w, a.eps);
+        else if (a.gate) hipLaunchKernelGGL(gemm_pack_rows_staged_kernel<PACK_SWIGLU>, dim3(a.M), dim3(256), lds, d->stream, rows, a.K, A, S, unscale, a.gate, 0.0f);
+        else hipLaunchKernelGGL(gemm_pack_rows_staged_kernel<PACK_PLAIN>, dim3(a.M), dim3(256), lds, d->stream, rows, a.K, A, S, unscale, static_cast<const float *>(nullptr), 0.0f);
     } else if (a.norm_w) {
         hipLaunchKernelGGL((gemm_pack_rows_kernel<false, PACK_NORM>), dim3(a.M), dim3(256), 0, d->stream, a.X, a.K, A, S, unscale, a.norm_w, a.eps);
     } else if (a.gate) {

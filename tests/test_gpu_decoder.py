@@ -589,6 +589,31 @@ def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, m
     fused.release(), apart.release(), weights.release()
 
 
+def test_rows_packed_through_lds_equal_the_rows_packed_from_memory(device, monkeypatch):
+    """A fill's wide products take their fp32 rows (as they lie, normalised, or gated by silu) packed into half rows; the
+    packing stages a row in LDS and crosses memory once, NEURA_HIP_PACK_STAGED=0 walks the row in memory three times.  The
+    same arithmetic on the same numbers: states and the next step's logits equal bit for bit, and within the oracle's bar."""
+    staged, ref, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=2, context=48, max_rows=20, seed=41)
+    walked, _, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=2, context=48, max_rows=20, seed=41)
+    prompt = np.random.default_rng(42).integers(0, SMALL_Q4["vocab"], (20, 2))
+    monkeypatch.setenv("NEURA_HIP_PACK_STAGED", "1")
+    staged.prefill(prompt.reshape(-1), 20, [0, 0])
+    monkeypatch.setenv("NEURA_HIP_PACK_STAGED", "0")
+    walked.prefill(prompt.reshape(-1), 20, [0, 0])
+    monkeypatch.delenv("NEURA_HIP_PACK_STAGED")
+    ref.forward(prompt.reshape(-1), 20, [0, 0], want_logits=False)
+    for layer in range(SMALL_Q4["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(staged.cache_read(layer, which), walked.cache_read(layer, which)), (layer, which)
+    want_logits, want = ref.forward([3, 4], 1, [20, 20])
+    got_a, got_b = staged.decode_step([3, 4], [20, 20]), walked.decode_step([3, 4], [20, 20])
+    assert np.array_equal(staged.logits(), walked.logits())
+    assert np.abs(staged.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max()
+    assert list(got_a) == list(got_b) == list(want), margins(want_logits)
+    for held in (staged, walked, weights_a, weights_b):
+        held.release()
+
+
 def test_decoders_of_different_rope_bases_step_in_turn(device):
     """Two decoders of different rope bases and head widths stepping alternately at batch 2 (the rotation as its own
     kernel, read from the device's table of inverse frequencies): each keeps answering from its own recorded step as the
