@@ -231,6 +231,29 @@ def test_a_windowed_model_keeps_a_ring_of_its_last_tokens(device, shape, element
     model.release(), weights.release()
 
 
+def test_a_ring_of_several_sections_merged_by_the_output_projection(device):
+    """A Q8_0 decoder of one plane whose window is a ring of 140 keys: three attention sections, left unmerged for the output
+    projection to merge as it stages its row.  Filled to four keys short of a full ring, then decode steps that wrap it:
+    logits and tokens as the oracle's."""
+    window, rows = 140, 8
+    model, ref, weights = build(device, TINY, NH_Q8_0, batch=1, context=400, max_rows=rows, seed=9, window=window)
+    rng = np.random.default_rng(10)
+    cursor = 0
+    for chunk in range(17):
+        prompt = rng.integers(0, TINY["vocab"], (rows, 1))
+        model.prefill(prompt.reshape(-1), rows, [cursor])
+        ref.forward(prompt.reshape(-1), rows, [cursor], want_logits=False)
+        cursor += rows
+    tokens = [7]
+    for step in range(12):
+        want_logits, want = ref.forward(tokens, 1, [cursor])
+        got = model.decode_step(tokens, [cursor])
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), (step, margins(want_logits))
+        tokens, cursor = got, cursor + 1
+    model.release(), weights.release()
+
+
 def test_a_window_as_wide_as_what_was_fed_changes_nothing(device):
     """Until the ring wraps a windowed model holds every key an unbounded one holds: the same tokens."""
     shape = TINY
