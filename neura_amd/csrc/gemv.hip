@@ -644,20 +644,22 @@ template <typename Skew>
 __device__ __forceinline__ void stage_merged(const float *__restrict__ partial, uint32_t sections, uint32_t G, uint32_t width, uint32_t K, float *xs, Skew skew) {
     constexpr uint32_t MOST = MERGED_SECTIONS_MOST, HEADS_MOST = 32;
     __shared__ __attribute__((aligned(16))) float tops[HEADS_MOST * MOST], masses[HEADS_MOST * MOST], weights[HEADS_MOST * MOST];
-    const uint32_t tid = threadIdx.x, shift = 31u - __builtin_clz(width), heads = K >> shift, hop = G * (width + 2u), pairs = heads * sections;
-    const uint32_t by_groups = 65536u / G + 1u, by_sections = 65536u / sections + 1u;  // x / G = x * by_groups >> 16 for the few heads and pairs here
+    const uint32_t tid = threadIdx.x, shift = 31u - __builtin_clz(width), heads = K >> shift, hop = G * (width + 2u);
+    const uint32_t by_groups = 65536u / G + 1u;  // x / G = x * by_groups >> 16 for the few heads here
     auto sums_of = [&](uint32_t head) {
         const uint32_t unit = head * by_groups >> 16;
         return partial + ((uint64_t)unit * sections * G + (head - unit * G)) * (width + 2u);
     };
+    // seat tid + 256 j of the statistics: head seat / MOST, section seat % MOST; a seat past the heads or the sections holds
+    // no score and no mass (its loads read the last head's, the last section's, and are dropped)
     float top[2], mass[2];
-    uint32_t seat[2];  // head * MOST + section of this thread's pairs
+    bool seated[2];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const uint32_t pair = min(tid + 256u * j, pairs - 1u), head = pair * by_sections >> 16, section = pair - head * sections;
-        const float *stats = sums_of(head) + section * hop + width;
+        const uint32_t seat = tid + 256u * j, head = seat / MOST, section = seat % MOST;
+        seated[j] = head < heads && section < sections;
+        const float *stats = sums_of(min(head, heads - 1u)) + min(section, sections - 1u) * hop + width;
         top[j] = stats[0], mass[j] = stats[1];
-        seat[j] = head * MOST + section;
     }
     for (uint32_t base = 0; base < K; base += 1024u) {
         float values[4][MOST];
@@ -669,23 +671,17 @@ __device__ __forceinline__ void stage_merged(const float *__restrict__ partial, 
             for (uint32_t s = 0; s < MOST; s++) values[e][s] = column[min(s, sections - 1u) * hop];
         }
         if (base == 0) {
-            // a head's seats past its sections hold no score and no mass
-            for (uint32_t at = tid; at < heads * MOST; at += 256u) tops[at] = -INFINITY, masses[at] = 0.0f;
-            __syncthreads();
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-                if (tid + 256u * j < pairs) tops[seat[j]] = top[j], masses[seat[j]] = mass[j];
+            for (int j = 0; j < 2; j++) tops[tid + 256u * j] = seated[j] ? top[j] : -INFINITY, masses[tid + 256u * j] = seated[j] ? mass[j] : 0.0f;
             __syncthreads();
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const float4 *row = reinterpret_cast<const float4 *>(tops + (seat[j] & ~(MOST - 1u)));
+                const float4 *row = reinterpret_cast<const float4 *>(tops + ((tid + 256u * j) & ~(MOST - 1u)));
                 float largest = -INFINITY;
 #pragma unroll
                 for (uint32_t q = 0; q < MOST / 4u; q++) largest = fmaxf(fmaxf(largest, fmaxf(row[q].x, row[q].y)), fmaxf(row[q].z, row[q].w));
-                if (tid + 256u * j < pairs) weights[seat[j]] = top[j] == -INFINITY ? 0.0f : softmax_exp(top[j] - largest);
+                weights[tid + 256u * j] = !seated[j] || top[j] == -INFINITY ? 0.0f : softmax_exp(top[j] - largest);
             }
-            for (uint32_t at = tid; at < heads * MOST; at += 256u)
-                if ((at & (MOST - 1u)) >= sections) weights[at] = 0.0f;
             __syncthreads();
         }
 #pragma unroll
