@@ -1660,24 +1660,34 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
     constexpr uint32_t GROUPS = NT / 256u;
     const uint32_t chunks = nb * 16u;
     const uint32_t rg = tid >> 8, t = tid & 255u;
+    // a thread's sixteen numbers of row `row0 + rg`, asked for whatever the row and the chunk (past them the last row's, the
+    // last chunk's, dropped by the caller): the next rows' are on their way while these rows become digits
+    auto fetch_rows = [&](uint32_t row0, float4 (&into)[4]) {
+        const float *xr = p.x + (size_t)min(row0 + rg, p.rows - 1u) * p.K + k0 + 16u * min(t, chunks - 1u);
+#pragma unroll
+        for (int c = 0; c < 4; c++) into[c] = *reinterpret_cast<const float4 *>(xr + 4u * c);
+    };
+    float4 ahead[4], w[4];
+    fetch_rows(0u, ahead);
+    if (p.norm_w) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) w[c] = *reinterpret_cast<const float4 *>(p.norm_w + k0 + 16u * min(t, chunks - 1u) + 4u * c);
+    }
+#pragma unroll
     for (uint32_t row0 = 0; row0 < R2; row0 += GROUPS) {
         const uint32_t row = row0 + rg;  // groups past the staged rows only keep the barriers company
         const bool real = row < p.rows;
-        const float *xr = p.x + (size_t)min(row, p.rows - 1u) * p.K;
         {
             const bool held = t < chunks && row < R2;
             float v[16];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (held && real) a = *reinterpret_cast<const float4 *>(xr + k0 + 16u * t + 4u * c);
+                const float4 a = held && real ? ahead[c] : make_float4(0.f, 0.f, 0.f, 0.f);
                 v[4 * c] = a.x, v[4 * c + 1] = a.y, v[4 * c + 2] = a.z, v[4 * c + 3] = a.w;
             }
+            if (row0 + GROUPS < R2) fetch_rows(row0 + GROUPS, ahead);
             if (p.norm_w) {
                 // the whole row is in registers across its 256 threads
-                float4 w[4];
-#pragma unroll
-                for (int c = 0; c < 4; c++) w[c] = held ? *reinterpret_cast<const float4 *>(p.norm_w + k0 + 16u * t + 4u * c) : make_float4(0.f, 0.f, 0.f, 0.f);
                 float square = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 16; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
