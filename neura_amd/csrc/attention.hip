@@ -270,6 +270,8 @@ __global__ __launch_bounds__(256) void attention_kernel(AttentionParams p) {
 // section s into its weight; then thread (channel, stripe) sums its channel over every eighth
 // section -- all of its loads in flight at once -- and the eight stripes meet in LDS.
 // (The leading arguments are what the first loads need: the hardware hands them to a wave in scalar registers as it starts.)
+// J: sections a stripe sums at most (8 J >= sections): no more loads than the sections ask for, to the next power of two.
+template <int J>
 __global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_partial, uint32_t lead_sections, uint32_t lead_groups, uint32_t width,
                                                              AttentionParams p) {
     __shared__ float weights[256], masses[256], held[256], stripes[8][32];
@@ -290,11 +292,11 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_p
     // arithmetic between them waited for the loads before -- eight round trips one after another where one is enough.
     const uint32_t c = cblock * 32u + (tid & 31u), stripe = tid >> 5;
     const float *column = src + min(c, width - 1u);
-    float values[32];
+    float values[J];
 #pragma unroll
-    for (int j = 0; j < 32; j++) values[j] = column[min(stripe + 8u * j, sections - 1u) * hop];
+    for (int j = 0; j < J; j++) values[j] = column[min(stripe + 8u * j, sections - 1u) * hop];
 #pragma unroll
-    for (int j = 0; j < 32; j++)
+    for (int j = 0; j < J; j++)
         if (stripe + 8u * j >= sections || c >= width) values[j] = 0.0f;
     // the largest top and the weighed mass: a wave each, then the four waves' words
     const float wave_top = wave_max(top);
@@ -310,7 +312,7 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_p
     const float normalized = total > 0.0f ? 1.0f / total : 0.0f;
     float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < 32; j++) {
+    for (int j = 0; j < J; j++) {
         const uint32_t s = stripe + 8u * j;
         if (s < sections) sum = fmaf(values[j], weights[s], sum);
     }
@@ -814,6 +816,15 @@ __global__ __launch_bounds__(256) void attention_any_kernel(AttentionParams p, u
     }
 }
 
+// the fold with as many loads a thread as the sections ask for
+template <typename... Args>
+static void launch_fold(uint32_t sections, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+    if (sections <= 32u) hipLaunchKernelGGL(attention_fold_kernel<4>, grid, block, lds, stream, args...);
+    else if (sections <= 64u) hipLaunchKernelGGL(attention_fold_kernel<8>, grid, block, lds, stream, args...);
+    else if (sections <= 128u) hipLaunchKernelGGL(attention_fold_kernel<16>, grid, block, lds, stream, args...);
+    else hipLaunchKernelGGL(attention_fold_kernel<32>, grid, block, lds, stream, args...);
+}
+
 int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     AttentionParams p{};
     p.q = a.q, p.out = a.out;
@@ -846,7 +857,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
         else hipLaunchKernelGGL(attention_any_kernel<NH_BF16>, grid, dim3(256), 0, d->stream, p, a.width);
         NH_HIP(hipGetLastError());
         if (p.sections > 1) {
-            hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
+            launch_fold(p.sections, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
             NH_HIP(hipGetLastError());
         }
         return NH_OK;
@@ -907,7 +918,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             if (p.sections > 1 && leave) {
                 *a.unmerged = SectionSums{p.partial, p.sections, p.groups, a.width};
             } else if (p.sections > 1) {
-                hipLaunchKernelGGL(attention_fold_kernel, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
+                launch_fold(p.sections, dim3(planes * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
                 NH_HIP(hipGetLastError());
             }
             return NH_OK;
@@ -934,7 +945,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     }
     NH_HIP(hipGetLastError());
     if (p.sections > 1) {
-        hipLaunchKernelGGL(attention_fold_kernel, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
+        launch_fold(p.sections, dim3(units * p.groups * ((a.width + 31) / 32)), dim3(256), 0, d->stream, p.partial, p.sections, p.groups, a.width, p);
         NH_HIP(hipGetLastError());
     }
     return NH_OK;
