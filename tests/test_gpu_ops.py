@@ -139,7 +139,8 @@ def test_reference_narrow_product_test(device, element, rows):
     tight(got, want, 2e-6)
 
 
-@pytest.mark.parametrize("element,N,K", [(NH_Q8_0, 5, 32), (NH_Q8_0, 33, 96), (NH_Q8_0, 1, 2048 + 32), (NH_Q8_0, 130, 4864), (NH_Q4_K, 3, 256),
+@pytest.mark.parametrize("element,N,K", [(NH_Q8_0, 5, 32), (NH_Q8_0, 33, 96), (NH_Q8_0, 1, 2048 + 32), (NH_Q8_0, 130, 4864), (NH_Q8_0, 20, 8192), (NH_Q8_0, 6, 8160),
+                                         (NH_Q8_0, 4, 1056), (NH_Q4_K, 3, 256),
                                          (NH_Q4_K, 17, 512), (NH_Q4_K, 1, 4096 + 256), (NH_Q4_K, 66, 18944), (NH_Q4_K, 9, 3584)])
 def test_gemv_ragged_shapes(device, element, N, K):
     rng = np.random.default_rng(N * 7 + K)
