@@ -351,6 +351,13 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         fail(NH_E_ARGUMENT, "a batch keeps a window of %u tokens over a context of %u", c.window, c.context);
         return nullptr;
     }
+    // states of another element than half are read by the plain attention kernel, in at most 256 sections of 256 keys, and
+    // by more than 16 query heads a key head not at all: refused here, not at the first step
+    if (c.cache_element != NH_F16 && ((c.window ? c.window : c.context) > 256u * 256u || c.heads / c.kv_heads > 16u)) {
+        fail(NH_E_ARGUMENT, "single and bfloat16 states are attended over at most %u keys by at most 16 query heads a key head, not %u keys by %u",
+             256u * 256u, c.window ? c.window : c.context, c.heads / c.kv_heads);
+        return nullptr;
+    }
     if (c.window && (c.max_rows ? c.max_rows : 1u) > c.window) {
         fail(NH_E_ARGUMENT, "a batch fills chunks of %u rows into a window of %u tokens", c.max_rows, c.window);
         return nullptr;
@@ -466,7 +473,14 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
         // same address in every such run) once a few thousand packets had gone through the queue, where eager launches of
         // the same kernels trace cleanly.  Kernel durations are the same either way, so traced runs step eagerly.
         const char *held = getenv("NEURA_HIP_GRAPH");
-        m->use_graph = !(held && held[0] == '0') && !(held == nullptr && traced_by_rocprofiler());
+        const bool traced = traced_by_rocprofiler();
+        if (held && held[0] == '1' && traced) {
+            fail(NH_E_ARGUMENT, "NEURA_HIP_GRAPH=1 asks for recorded decode steps in a process traced by rocprofv3: that combination has crashed "
+                                "inside hipGraphLaunch; traced processes step eagerly");
+            release(m);
+            return nullptr;
+        }
+        m->use_graph = !(held && held[0] == '0') && !traced;
     }
     ok = ok && hipStreamSynchronize(device->stream) == hipSuccess;
     if (!ok) {
@@ -502,8 +516,9 @@ static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *
     // Profiled steps run eagerly (event records do not belong in a graph).
     const int variant = (any_inactive ? 1 : 0) + (draws ? 2 : 0);
     hipGraphExec_t &graph = m->decode_graph[variant];
-    // The first step of a variant runs eagerly: its launchers grow the device scratch to what the variant needs (a
-    // synchronize, a free and an allocation), none of which belongs inside a stream capture.
+    // The first step of a variant runs eagerly: its launchers grow the device scratch to what the variant needs (an
+    // allocation, which does not belong inside a stream capture; the outgrown block is kept until nh_close).
+    if (m->use_graph && traced_by_rocprofiler()) return fail(NH_E_DEVICE, "a recorded decode step is never launched in a process traced by rocprofv3");
     if (m->use_graph && !d->profile && m->graph_warmed[variant]) {
         if (graph && m->graph_moved[variant] != d->moved) {
             // the device scratch or rope table moved since the capture (another model or operator call grew it)

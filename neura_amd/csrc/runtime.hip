@@ -28,7 +28,9 @@ void *scratch(nh_device *device, size_t bytes) {
     // The block that is outgrown is kept until nh_close: work already queued on the stream, and any recorded
     // decode step that has not been recorded again yet, still holds its address, and nothing is released
     // in the middle of a process (no synchronize, no free).
+    // It grows to at least twice its size, so that all the retired blocks together stay smaller than the live one.
     size_t wanted = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    if (wanted < 2 * device->scratch_bytes) wanted = 2 * device->scratch_bytes;
     void *held = nullptr;
     if (hipMalloc(&held, wanted) != hipSuccess) {
         fail(NH_E_MEMORY, "device %d holds no %zu bytes of scratch", device->index, wanted);

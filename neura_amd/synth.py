@@ -348,14 +348,44 @@ def layer_matrices(shape):
             ("ffn_down", H, F)]
 
 
-def model_tensors(shape, element, rng, mode="blocks", layers=None, elements=None, biases=()):
+def _normal_matrix(held, rows, columns, seed, threads):
+    """N(0, 0.02) weights of one matrix quantized chunk by chunk on `threads` threads: every chunk of rows draws from its own
+    generator (seeded by the matrix's seed and the chunk's index, so the bytes do not depend on the thread count) and is packed
+    by the host layer's encoder where that is the reference's (Q8_0, Q4_K, Q5_K, Q3_K) and by the numpy one for Q6_K."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    pack = None
+    if held != 14:
+        from . import host  # the C++ packer, byte for byte the numpy one and some ten times faster
+
+        pack = lambda values: np.asarray(host.pack(held, values.reshape(-1))).view(np.uint8).reshape(-1)
+    else:
+        pack = QUANTIZE[held]
+    out = np.empty(matrix_bytes(held, rows, columns), dtype=np.uint8)
+    row_bytes = matrix_bytes(held, 1, columns)
+    step = max(1, (1 << 22) // columns)
+
+    def chunk(index):
+        first = index * step
+        n = min(step, rows - first)
+        values = np.random.default_rng([seed, index]).standard_normal((n, columns), dtype=np.float32) * np.float32(0.02)
+        out[first * row_bytes:(first + n) * row_bytes] = pack(values)
+
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        list(pool.map(chunk, range((rows + step - 1) // step)))
+    return out
+
+
+def model_tensors(shape, element, rng, mode="blocks", layers=None, elements=None, biases=(), threads=None):
     """Yields (name, element, dims (GGUF order: K first), raw bytes) of a random-init decoder.
 
     `elements`: name -> element of the matrices stored otherwise than `element` (a Q4_K_M file keeps some in Q6_K);
     `biases`: layers whose q, k and v projections carry an fp32 bias (Qwen2 checkpoints do).
 
     mode "blocks": matrices are random raw blocks (the Q4_K distribution of the GEMV
-    configurations); mode "normal": N(0, 0.02) weights quantized with the reference's encoder.
+    configurations); mode "normal": N(0, 0.02) weights quantized with the reference's encoder
+    (`threads`: on that many threads, a generator per chunk of rows -- the way to build the 7B shape in seconds;
+    without it one generator draws everything in order).
     Norm weights are fp32.
     """
     H = shape["hidden"]
@@ -367,6 +397,8 @@ def model_tensors(shape, element, rng, mode="blocks", layers=None, elements=None
         held = elements.get(name, element)
         if mode == "blocks":
             return held, RANDOM[held](rng, rows * columns)
+        if threads:
+            return held, _normal_matrix(held, rows, columns, int(rng.integers(0, 1 << 62)), threads)
         out = np.empty(matrix_bytes(held, rows, columns), dtype=np.uint8)
         step = max(1, (1 << 24) // columns)
         row_bytes = matrix_bytes(held, 1, columns)

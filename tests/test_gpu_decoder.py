@@ -1,7 +1,11 @@
 """GPU parity of the decoder (decode step, fill, greedy loop) against the CPU oracle."""
+import json
+import os
+
 import numpy as np
 import pytest
 
+import cases
 import oracle
 from neura_amd import NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K, NH_Q8_0, NeuraError, synth
 from neura_amd.loader import Model, Weights
@@ -300,22 +304,23 @@ def test_decode_refuses_what_the_reference_refuses(device):
     model.release(), weights.release()
 
 
+def golden_ids(name):
+    """the ids the oracle chose when tests/golden/make_fixtures.py wrote the fixture"""
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)) as held:
+        return json.load(held)["ids"]
+
+
 def test_config4_greedy_64_steps_qwen2_5_0_5b_shape_q8_0(device):
     """Random-init 0.5B-shape Q8_0 decoder, fp16 caches prefilled to 1024 random tokens' worth
     of N(0,1) halves, 64 greedy steps from a random prompt id: token ids identical to the
-    oracle.  The oracle follows the reference's summation order; identity against the
-    reference binary itself is unpinned (it cannot be run here)."""
-    shape = synth.SHAPES["qwen2.5-0.5b"]
+    oracle's, and the oracle's identical to the committed ids.  The oracle follows the reference's summation order;
+    identity against the reference binary itself is unpinned (it cannot be run here)."""
+    shape, tensors, host, halves, token = cases.config4_case(threads=16)
     context, filled, steps = 1024 + 64, 1024, 64
-    model, ref, weights = build(device, shape, NH_Q8_0, batch=1, context=context, seed=0)
-    rng = np.random.default_rng(40)
-    for layer in range(shape["layers"]):
-        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-            halves = np.zeros(model.cache_shape, dtype=np.float16)
-            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
-            held[layer][:] = halves.view(np.uint16).reshape(-1)
-            model.cache_write(layer, which, halves.view(np.uint16))
-    token = int(rng.integers(0, shape["vocab"]))
+    weights = Weights(device, tensors)
+    model = Model(device, weights, shape, NH_Q8_0, 1, context, 1)
+    ref = oracle.Model(shape, NH_Q8_0, host, 1, context, 1)
+    cases.hold(halves, model.cache_shape, ref, model)
     got_tokens, want_tokens, gaps = [], [], []
     got = want = token
     for step in range(steps):
@@ -328,33 +333,76 @@ def test_config4_greedy_64_steps_qwen2_5_0_5b_shape_q8_0(device):
             break
     print("greedy margins (top1 - top2): min %.3g median %.3g" % (min(gaps), float(np.median(gaps))))
     assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
+    assert want_tokens == golden_ids("config4_greedy_ids.json")
+    same_cache_rows(model, ref, shape["layers"], [list(range(filled, filled + steps))], "rows the 64 steps appended")
     model.release(), weights.release()
 
 
-def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
-    """The 7B shape itself (hidden 3584, 28 query heads over 4 key heads of 128, ffn 18944, vocabulary 152064, random Q4_K
-    blocks, separate head) cut to two layers, at context 4096: decode steps at batch 1 on caches filled with N(0,1) halves
+def fill_caches(model, ref, rng, shape, layers, batch, filled):
+    """positions below `filled` of every state of both decoders hold the same N(0,1) halves"""
+    for layer in range(layers):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            halves = np.zeros(model.cache_shape, dtype=np.float16)
+            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], batch, filled, shape["head_dim"])).astype(np.float16)
+            held[layer][:] = halves.view(np.uint16).reshape(-1)
+            model.cache_write(layer, which, halves.view(np.uint16))
+
+
+def same_cache_rows(model, ref, layers, rows_of_plane, what):
+    """the key and value rows at the given positions (a list per plane) hold the oracle's halves: what a decode step or a
+    fill appended, rotation included"""
+    for layer in range(layers):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            got_all = model.cache_read(layer, which)
+            want_all = held[layer].reshape(model.cache_shape)
+            for plane, positions in enumerate(rows_of_plane):
+                got_rows = oracle.f16_to_f32(np.ascontiguousarray(got_all[:, plane, positions]).reshape(-1))
+                want_rows = oracle.f16_to_f32(np.ascontiguousarray(want_all[:, plane, positions]).reshape(-1))
+                assert np.any(want_rows), (what, layer, which, plane)
+                assert np.abs(got_rows - want_rows).max() <= 2e-3 * max(1.0, np.abs(want_rows).max()), (what, layer, which, plane)
+
+
+def input_moves_the_logits(ref, batch, cursors, vocab, least=1e-2):
+    """A test network must not be degenerate: another input token moves the oracle's logits by more than `least` of the
+    largest (random Q4_K blocks have a large positive mean: every matrix is all ones plus noise, the network collapses onto
+    one direction and its logits hardly depend on the token -- parity of ids proves nothing there).  Both passes write the
+    same cache rows, which the step under test then writes again."""
+    first, _ = ref.forward([1234 % vocab] * batch, 1, cursors, threads=16)
+    first = first.copy()
+    second, _ = ref.forward([7] * batch, 1, cursors, threads=16)
+    moved = float(np.abs(first - second).max() / np.abs(first).max())
+    print("another input token moves the oracle's logits by %.3g of the largest" % moved, flush=True)
+    return moved > least
+
+
+@pytest.mark.parametrize("mode", ["blocks", "normal"])
+def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device, mode):
+    """The 7B shape itself (hidden 3584, 28 query heads over 4 key heads of 128, ffn 18944, vocabulary 152064, separate head)
+    cut to two layers, at context 4096: decode steps at batch 1 on caches filled with N(0,1) halves
     (the products at their real depths and row counts, the rotation folded in, attention over 4000 keys in sections), a
     512-row fill, the prompt chunk of the benchmark (wide products with stacked q|k|v and fused packing passes, attention
-    over a chunk), and a step of eight planes (the half-precision tiles on gate|up and the head, the integer tiles on the
-    rest), each against the oracle: logits within 1e-3 of the largest, the greedy token identical at every step."""
+    over a chunk), and steps of eight planes (the half-precision tiles on gate|up and the head, the integer tiles on the
+    rest), each against the oracle: logits within 1e-3 of the largest, the greedy token identical at every step, and the key
+    and value rows the steps and the fill appended equal to the oracle's.
+
+    "blocks": random Q4_K blocks, the distribution BASELINE's product configurations name -- a degenerate network (its
+    logits do not depend on the token), which holds the products' bulk accuracy and nothing else.  "normal": N(0, 0.02)
+    weights packed by the reference's Q4_K encoder -- a network whose logits, tokens and appended rows depend on every
+    input-dependent piece (embedding row, rotation at the cursor, cache append, attention over the appended rows)."""
     shape = synth.SHAPES["qwen2.5-7b"]
     layers, context, filled, rows = 2, 4096, 3500, 512
     rng = np.random.default_rng(50)
-    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks", layers=layers))
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode=mode, layers=layers, threads=16))
     host = {name: raw for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
 
     def pair(batch, max_rows):
         model = Model(device, weights, shape, NH_Q4_K, batch, context, max_rows, layers=layers)
         ref = oracle.Model(shape, NH_Q4_K, host, batch, context, max_rows, layers=layers)
-        for layer in range(layers):
-            for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-                halves = np.zeros(model.cache_shape, dtype=np.float16)
-                halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], batch, filled, shape["head_dim"])).astype(np.float16)
-                held[layer][:] = halves.view(np.uint16).reshape(-1)
-                model.cache_write(layer, which, halves.view(np.uint16))
+        fill_caches(model, ref, rng, shape, layers, batch, filled)
         return model, ref
+
+    seen = []
 
     def same(model, ref, tokens, cursors, what):
         want_logits, want = ref.forward(tokens, 1, cursors, threads=16)
@@ -363,54 +411,58 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device):
         scale = np.abs(want_logits).max()
         assert np.abs(logits - want_logits).max() <= 1e-3 * scale, what
         gaps = margins(want_logits)
-        print("%s: top-2 margins min %.3g of a largest logit of %.3g, logits within %.3g" % (what, gaps.min(), scale, np.abs(logits - want_logits).max()))
+        print("%s (%s): tokens %s, top-2 margins min %.3g of a largest logit of %.3g, logits within %.3g" %
+              (what, mode, [int(t) for t in want], gaps.min(), scale, np.abs(logits - want_logits).max()), flush=True)
         assert [int(t) for t in got] == [int(t) for t in want], (what, gaps)
+        seen.extend(int(t) for t in want)
         return [int(t) for t in want]
 
     model, ref = pair(1, rows)
+    assert input_moves_the_logits(ref, 1, [filled], shape["vocab"]) or mode == "blocks"
     token = [int(rng.integers(0, shape["vocab"]))]
     for step in range(3):
         token = same(model, ref, token, [filled + step], "batch 1, step %d" % step)
+    # what the three steps appended: the rotated key rows and the value rows at the stepped cursors (the epilogue of the
+    # q|k|v product at 4608 x 3584)
+    same_cache_rows(model, ref, layers, [[filled, filled + 1, filled + 2]], "rows the batch-1 steps appended")
     # a fill of 512 rows behind the keys already held (positions 3503 .. 4014), then a step that weighs what it wrote
     prompt = rng.integers(0, shape["vocab"], rows)
     first = filled + 3
     model.prefill(prompt, rows, [first])
     ref.forward(prompt, rows, [first], want_logits=False, threads=16)
-    for layer in range(layers):
-        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-            got_rows = oracle.f16_to_f32(model.cache_read(layer, which)[:, :, first:first + rows].reshape(-1))
-            want_rows = oracle.f16_to_f32(held[layer].reshape(model.cache_shape)[:, :, first:first + rows].reshape(-1))
-            assert np.abs(got_rows - want_rows).max() <= 2e-3 * max(1.0, np.abs(want_rows).max()), (layer, which)
+    same_cache_rows(model, ref, layers, [list(range(first, first + rows))], "rows the fill appended")
     same(model, ref, token, [first + rows], "batch 1 after the 512-row fill")
+    same_cache_rows(model, ref, layers, [[first + rows]], "the row behind the fill")
     model.release()
     model, ref = pair(8, 1)
     tokens = [int(t) for t in rng.integers(0, shape["vocab"], 8)]
     for step in range(2):
         tokens = same(model, ref, tokens, [filled - 7 * plane + step for plane in range(8)], "batch 8, step %d" % step)
+    same_cache_rows(model, ref, layers, [[filled - 7 * plane, filled - 7 * plane + 1] for plane in range(8)], "rows the batch-8 steps appended")
+    if mode == "normal":
+        assert len(set(seen)) > len(seen) // 2, seen  # the chosen tokens differ from step to step and plane to plane
     model.release(), weights.release()
 
 
-def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device):
-    """The model the benchmark times, whole: 28 layers of the 7B shape, random Q4_K blocks, a separate head, fp16 caches
+@pytest.mark.parametrize("mode", ["blocks", "normal"])
+def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device, mode):
+    """The model the benchmark times, whole: 28 layers of the 7B shape, a separate head, fp16 caches
     holding 4032 positions of N(0,1) halves, then 64 greedy steps up to the end of the context of 4096 -- every token
-    identical to the oracle's, with no allowance for close calls.  The oracle follows the reference's summation order;
-    identity against the reference binary itself is unpinned (it cannot be run here)."""
+    identical to the oracle's, with no allowance for close calls.  "blocks": the benchmark's random Q4_K blocks (a
+    degenerate network: one token, margins in the hundreds -- the products' bulk accuracy); "normal": N(0, 0.02) weights
+    packed by the reference's encoder (tokens vary, margins are small and printed; nothing is gated on them).  The
+    oracle follows the reference's summation order; identity against the reference binary itself is unpinned (it cannot
+    be run here)."""
     shape = synth.SHAPES["qwen2.5-7b"]
     context, steps = 4096, 64
     filled = context - steps
-    rng = np.random.default_rng(52)
-    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks"))
-    host = {name: raw for name, _, _, raw in tensors}
+    tensors, host, halves, token = cases.decoder_case(shape, NH_Q4_K, mode, 52, None, 1, filled)
     weights = Weights(device, tensors)
     model = Model(device, weights, shape, NH_Q4_K, 1, context, 1)
     ref = oracle.Model(shape, NH_Q4_K, host, 1, context, 1)
-    for layer in range(shape["layers"]):
-        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-            halves = np.zeros(model.cache_shape, dtype=np.float16)
-            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
-            held[layer][:] = halves.view(np.uint16).reshape(-1)
-            model.cache_write(layer, which, halves.view(np.uint16))
-    got = want = int(rng.integers(0, shape["vocab"]))
+    cases.hold(halves, model.cache_shape, ref, model)
+    del halves
+    got = want = token
     got_tokens, want_tokens, gaps, apart = [], [], [], []
     for step in range(steps):
         want_logits, chosen = ref.forward([want], 1, [filled + step], threads=16)
@@ -420,44 +472,69 @@ def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device):
         gaps.append(float(margins(want_logits)[0]))
         apart.append(float(np.abs(model.logits() - want_logits).max() / np.abs(want_logits).max()))
         if step % 8 == 7:
-            print("step %d: tokens identical so far, smallest top-2 margin %.3g" % (step, min(gaps)), flush=True)
+            print("step %d (%s): tokens identical so far, smallest top-2 margin %.3g" % (step, mode, min(gaps)), flush=True)
         if got != want:
             break
+    print("greedy tokens (%s): %s" % (mode, want_tokens))
     print("greedy margins (top1 - top2) over %d steps: min %.3g median %.3g; logits within %.3g of the largest" %
           (len(gaps), min(gaps), float(np.median(gaps)), max(apart)))
     assert max(apart) <= 1e-3
     assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
+    if mode == "normal":
+        assert len(set(want_tokens)) > steps // 2, want_tokens
+        same_cache_rows(model, ref, shape["layers"], [list(range(filled, filled + steps))], "rows the 64 steps appended")
+        assert want_tokens == golden_ids("config5_normal_greedy_ids.json")
     model.release(), weights.release()
 
 
-def test_config5_shape_stored_as_a_q4_k_m_file_stores_it(device):
+@pytest.mark.parametrize("mode", ["blocks", "normal"])
+def test_config5_shape_stored_as_a_q4_k_m_file_stores_it(device, mode):
     """The 7B shape cut to two layers, stored the way llama.cpp's Q4_K_M recipe stores Qwen2.5-7B: the head and the first
     layer's value and down projections in Q6_K, q, k and v biases on every layer.  Batch-1 steps at context 4096: the
-    staged Q6_K products at their real shapes (a 152064-row head, a down projection in K slices), q|k rotated from one
-    product with the value row appended behind it, the layer of one element with biases in the folded rotation."""
+    Q6_K products at their real shapes (a 152064-row head, a down projection), q|k rotated from one
+    product with the value row appended behind it, the layer of one element with biases in the folded rotation.  Random
+    blocks and N(0, 0.02) weights (Q6_K through the symmetric numpy quantizer), as above."""
     shape = synth.SHAPES["qwen2.5-7b"]
     layers, context, filled = 2, 4096, 4000
     mixed = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.0.ffn_down.weight": NH_Q6_K}
     rng = np.random.default_rng(51)
-    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="blocks", layers=layers, elements=mixed, biases=(0, 1)))
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode=mode, layers=layers, elements=mixed, biases=(0, 1), threads=16))
     host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
     model = Model(device, weights, shape, NH_Q4_K, 1, context, 1, layers=layers)
     ref = oracle.Model(shape, NH_Q4_K, host, 1, context, 1, layers=layers, elements=mixed)
-    for layer in range(layers):
-        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
-            halves = np.zeros(model.cache_shape, dtype=np.float16)
-            halves[:, :, :filled] = rng.standard_normal((shape["kv_heads"], 1, filled, shape["head_dim"])).astype(np.float16)
-            held[layer][:] = halves.view(np.uint16).reshape(-1)
-            model.cache_write(layer, which, halves.view(np.uint16))
+    fill_caches(model, ref, rng, shape, layers, 1, filled)
+    assert input_moves_the_logits(ref, 1, [filled], shape["vocab"]) or mode == "blocks"
     token = [int(rng.integers(0, shape["vocab"]))]
+    chosen = []
     for step in range(3):
         want_logits, want = ref.forward(token, 1, [filled + step], threads=16)
         got = model.decode_step(token, [filled + step])
         scale = np.abs(want_logits).max()
+        print("step %d (%s): token %d, margin %.3g, logits within %.3g of %.3g" % (step, mode, int(want[0]), margins(want_logits)[0],
+                                                                                 np.abs(model.logits() - want_logits).max(), scale), flush=True)
         assert np.abs(model.logits() - want_logits).max() <= 1e-3 * scale, step
         assert int(got[0]) == int(want[0]), (step, margins(want_logits))
         token = [int(want[0])]
+        chosen.append(token[0])
+    same_cache_rows(model, ref, layers, [[filled, filled + 1, filled + 2]], "rows the steps appended")
+    if mode == "normal":
+        assert len(set(chosen)) > 1, chosen
+    model.release(), weights.release()
+
+
+def test_recorded_steps_are_refused_in_a_traced_process(device, monkeypatch):
+    """rocprofv3 names its tool library in the environment of what it runs; hipGraphLaunch has crashed under it, so a traced
+    process steps eagerly and NEURA_HIP_GRAPH=1 there is an error at nh_model_create, not a crash later.  (No graph is
+    launched here: the environment alone is what the library looks at.)"""
+    monkeypatch.setenv("ROCP_TOOL_LIBRARIES", "librocprofiler-sdk-tool.so")
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "1")
+    with pytest.raises(NeuraError, match="traced"):
+        build(device, TINY, NH_Q8_0, batch=1, context=8)
+    monkeypatch.delenv("NEURA_HIP_GRAPH")
+    model, ref, weights = build(device, TINY, NH_Q8_0, batch=1, context=8)  # without the switch: eager steps, same answers
+    for step in range(3):
+        assert model.decode_step([5], [step])[0] == ref.forward([5], 1, [step])[1][0]
     model.release(), weights.release()
 
 

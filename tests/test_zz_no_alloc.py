@@ -42,6 +42,37 @@ def test_the_static_choice_answers_as_the_allocating_one(device):
     assert np.array_equal(static, plain)
 
 
+def test_the_static_choice_allocates_nothing_on_a_device_that_has_chosen_nothing_yet():
+    """A handle opened here has no scratch yet and never calls nh_argmax: nh_argmax_static must answer from the static array
+    alone.  The device's free memory (hipMemGetInfo) is the same before and after the calls, and the second call's values
+    differ from the first's, so that partials left in the array cannot pass for fresh ones."""
+    import neura_amd
+
+    fresh = neura_amd.Device(0)
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    rng = np.random.default_rng(78)
+    first = rng.standard_normal((8, 152064)).astype(np.float32)
+    second = rng.standard_normal((8, 152064)).astype(np.float32)
+    held_first, held_second, out = fresh.upload(first), fresh.upload(second), fresh.alloc(8 * 4)
+    fresh.sync()
+    before = free_bytes()
+    _check(fresh.lib.nh_argmax_static(fresh.handle, held_first.pointer, 8, 152064, out.pointer))
+    assert np.array_equal(out.numpy(np.uint32), first.argmax(axis=1))
+    _check(fresh.lib.nh_argmax_static(fresh.handle, held_second.pointer, 8, 152064, out.pointer))
+    assert np.array_equal(out.numpy(np.uint32), second.argmax(axis=1))
+    fresh.sync()
+    assert free_bytes() == before
+    for buffer in (held_first, held_second, out):
+        buffer.release()
+    fresh.close()
+
+
 def test_the_static_choice_refuses_what_its_array_cannot_hold(device):
     values = device.upload(np.zeros((65, 16), dtype=np.float32))
     out = device.alloc(65 * 4)
