@@ -267,6 +267,11 @@ int32_t nh_model_logits(nh_model *model, float *host_out);
 int32_t nh_model_cache_write(nh_model *model, uint32_t layer, int32_t value_not_key, const void *host_src);
 int32_t nh_model_cache_read(nh_model *model, uint32_t layer, int32_t value_not_key, void *host_dst);
 uint32_t nh_model_capacity(const nh_model *model);
+/* A decode step of one plane runs the products between two attentions as one launch with seams between them, the way the
+ * reference runs a whole program as one persistent kernel (crates/neura-kernel/src/scheduler.rs:110-166).  A seam's wait is
+ * bounded; where one gave up, the step was run again one launch a product and the model stays on that path.  This counts
+ * those steps (0 in a healthy process). */
+uint32_t nh_model_seam_fallbacks(const nh_model *model);
 /* The shared prefix of a batch that declares one (Cache::with_shared / Cache::shared, crates/neura-decoder/src/cache.rs:71-90,
  * :138-161; Batch::prefix, crates/neura-generate/src/batch.rs:885-994): one more plane of keys and values per layer,
  * fp16 [kv_heads][1][capacity][head_dim], zero until kept.

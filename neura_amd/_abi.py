@@ -88,6 +88,7 @@ SIGNATURES = {
     "nh_model_shared_write": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
     "nh_model_shared_read": (c_int32, [c_void_p, c_uint32, c_int32, c_void_p]),
     "nh_model_capacity": (c_uint32, [c_void_p]),
+    "nh_model_seam_fallbacks": (c_uint32, [c_void_p]),
 }
 
 _library = None

@@ -78,6 +78,7 @@ struct nh_device {
     // recorded again when this no longer matches the count at its capture
     uint64_t moved = 0;
     uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
+    uint32_t *chain_flags = nullptr;  // 256 words: one a workgroup of a chained launch (launch_chain), cleared by a step's first kernel
     uint8_t *static_scratch = nullptr;  // this device's copy of the file-scope array nh_argmax_static works in (argmax.hip)
     struct RopeTable {
         float base;
@@ -104,7 +105,9 @@ int32_t check_refusal(nh_device *device, const char *what);
 // records the next profiling event on the stream (no-op unless profiling is on)
 void profile_mark(nh_device *device);
 
-enum Refusal : uint32_t { REFUSAL_NONE = 0, REFUSAL_INDEX = 1, REFUSAL_ORIGIN = 2 };
+// REFUSAL_SEAM: a workgroup of a chained launch gave up waiting for the others (launch_chain); it ranks below the refusals of an
+// input, which atomicMax keeps
+enum Refusal : uint32_t { REFUSAL_NONE = 0, REFUSAL_SEAM = 1, REFUSAL_INDEX = 2, REFUSAL_ORIGIN = 3 };
 
 // ---- launchers (each validates nothing: the C ABI layer checks shapes first) ----
 int32_t launch_dequant(nh_device *d, int32_t element, const void *src, uint64_t elements, float *dst);
@@ -204,6 +207,15 @@ constexpr uint32_t MERGED_SECTIONS_MOST = 16;  // sections such a product merges
 // whether `producer` (a SwiGLU product of one row) can hand its outputs to `consumer` as digit planes, and the bytes they take
 bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer);
 size_t gemv_digit_bytes(uint32_t K);
+// Several dependent one-row Q4_K products as one launch with seams between them: attn_output (`lead`, or nullptr), gate|up
+// handing its digit planes to ffn_down, and behind them the next q|k|v with the rotation folded in or the head (`trail`, or
+// nullptr).  gemv_chains() says whether launch_chain takes them.  `epoch`: the first of the three flag values the launch may
+// publish (they only grow between two launch_chain_clear); `spin`: the reads of the flag words a workgroup's wait may take
+// before it gives up with REFUSAL_SEAM.
+bool gemv_chains(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail);
+int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t epoch, uint32_t spin);
+int32_t launch_chain_clear(nh_device *d);
+constexpr uint32_t CHAIN_EPOCHS_A_LAUNCH = 3;
 // whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)
 bool gemv_fuses_rope(const GemvArgs &args, const RopeFusion &rope);
 

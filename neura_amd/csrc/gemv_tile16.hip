@@ -51,17 +51,49 @@ struct Tile16Unit {
 // is then a chunk's own, not a group's, so the four MFMAs of a step keep their sums apart and each is weighed by its
 // chunk's scale; the staging pass shrinks to a copy.
 //
-// The leading arguments are what a wave needs before it can ask for its first activations and weights.  They are plain words
-// so that the hardware can hand them over in scalar registers when it starts the wave (the file is built with
-// -amdgpu-kernarg-preload-count): the wave's first loads then go out without waiting for a load of its parameters
-// (about 0.5 us); everything else sits in `p` and is fetched meanwhile.  `input` is x, or the digit planes with HANDED.
-template <int NW, int D, int MODE, int R, bool HANDED = false>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, int32_t lead_to_w1,
-                                                                  int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
-                                                                  uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p) {
+// A seam stands between two products of one launch (gemv_q4k_chain_kernel below): the product behind it may ask for its
+// first weights at once -- they depend on nothing -- but reads its activations only when every workgroup has finished the
+// product before.  What crosses a seam crosses it between compute units of different dies, whose L2 caches do not see each
+// other's writes inside a launch: it is stored and loaded at device scope (sc1: written through to memory, read past the
+// L2), with no cache write-back or invalidation.  NoSeam is a product that is a launch of its own.
+struct NoSeam {
+    static constexpr bool WAITS = false;         // the activations wait for the seam
+    static constexpr bool SHARED_IN = false;     // activations (and the residual) were written by this launch
+    static constexpr bool SHARED_OUT = false;    // outputs are read by a later product of this launch
+    __device__ __forceinline__ bool wait(uint32_t) const { return true; }
+};
+
+typedef float tile16_f32x4 __attribute__((ext_vector_type(4)));
+// 16 bytes at `base + offset` (base uniform over the wave); SHARED: at device scope
+template <bool SHARED>
+__device__ __forceinline__ u32x4 tile16_load16(const void *base, uint32_t offset) {
+    if constexpr (SHARED) {
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0xffffffff, 0x00020000);
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, offset, 0, 16);  // aux 16: sc1
+    } else {
+        typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
+        return *(global_uint4)(uintptr_t)(static_cast<const uint8_t *>(base) + offset);
+    }
+}
+template <bool SHARED>
+__device__ __forceinline__ tile16_f32x4 tile16_load4(const float *base, uint32_t element) {
+    if constexpr (SHARED) return __builtin_bit_cast(tile16_f32x4, tile16_load16<true>(base, element * 4u));
+    else return *reinterpret_cast<const tile16_f32x4 *>(base + element);
+}
+template <bool SHARED>
+__device__ __forceinline__ void tile16_store_word(uint32_t *at, uint32_t word) {
+    if constexpr (SHARED) __hip_atomic_store(at, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *at = word;
+}
+
+// The product itself; `block` of `lead_grid` workgroups.  Returns false where the seam gave up (the whole workgroup leaves).
+template <int NW, int D, int MODE, int R, bool HANDED, class SEAM>
+__device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const uint32_t block, const SEAM seam, const uint8_t *lead_w0, const void *lead_input,
+                                               const float *lead_norm_w, int32_t lead_to_w1, int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid,
+                                               uint32_t lead_tiles, uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, const GemvParams &p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
     static_assert(!HANDED || (R == 1 && MODE == TILE16_PLAIN), "handed-over digit planes feed a plain product of one row");
-    extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
+    static_assert(!(SEAM::WAITS || SEAM::SHARED_IN || SEAM::SHARED_OUT) || R == 1, "products of one row are chained");
     constexpr uint32_t NT = NW * 64;
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -89,8 +121,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
     const uint32_t r = lane & 15u, q = lane >> 4;
     // tiles of this workgroup: blockIdx.x, blockIdx.x + lead_grid, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
     const uint32_t tiles = lead_tiles;
-    if (blockIdx.x >= tiles) return;  // the whole workgroup: no barrier has been reached
-    const uint32_t ntiles = (tiles - blockIdx.x + lead_grid - 1u) / lead_grid;
+    if (block >= tiles || block >= lead_grid) return true;  // the whole workgroup: no barrier has been reached
+    const uint32_t ntiles = (tiles - block + lead_grid - 1u) / lead_grid;
     const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;  // super-blocks of one tile this wave walks
 
     // the weight row lane r reads in tile `tile`; with the rotation folded in a tile holds channels c0 .. c0 + 7 of a head and
@@ -101,7 +133,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
     const uint32_t row_bytes = lead_row_bytes;
     // (with the rotation folded in the tile rows' word carries the rotation's width: such tiles are always whole)
     const uint32_t half_width = (MODE == TILE16_ROPE ? lead_tile_rows : 16u) >> 1, tiles_per_head = max(half_width >> 3, 1u);
-    const uint32_t first_tile = blockIdx.x, hop = lead_grid;
+    const uint32_t first_tile = block, hop = lead_grid;
     // a plain tile may hold fewer than 16 rows (a matrix of 3584 rows is 256 tiles of 14, one a compute unit, where it is 224
     // of 16): the columns past them walk the tile's last row again and are never written
     const uint32_t tile_rows = MODE == TILE16_PLAIN ? lead_tile_rows : 16u;
@@ -151,6 +183,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
     // the cursor with the activations, a tile's operands a tile early
     uint32_t rope_position = 0;
     RopeOperands rope_held{0.0f, 1.0f, 0.0f};
+    constexpr bool CHAINED = SEAM::SHARED_IN || SEAM::SHARED_OUT;  // one of several products of a launch
+    float residual_held = 0.0f;  // chained: the residual of this workgroup's first tile (lanes 0..15), asked for ahead
     auto rope_row = [half_width, tiles_per_head, lane](uint32_t tile, uint32_t &c) -> uint32_t {
         c = (tile % tiles_per_head) * 8u + (lane & 7u);
         return (tile / tiles_per_head) * (2u * half_width) + c + ((lane >> 3) & 1u) * half_width;
@@ -210,14 +244,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
             constexpr int MAXB = NW <= 8 ? 10 : 5;  // super-blocks a wave copies at once: ffn_down at eight waves has ten, all asked for together
             uint8_t *const pairs = reinterpret_cast<uint8_t *>(sums);
             const uint32_t chunk = lane >> 2, piece = lane & 3u;
+            if constexpr (SEAM::WAITS) {
+                // behind a seam: the first weights are asked for, then the planes wait for the product that writes them
+#pragma unroll
+                for (int i = 0; i < D; i++) fetch(ring[i]);
+                fetch_the_rest();
+                if (!seam.wait(tid)) return false;
+            }
             for (uint32_t j0 = 0; j0 < count; j0 += MAXB) {
                 u32x4 held[MAXB];
 #pragma unroll
                 for (int j = 0; j < MAXB; j++) {
                     uint32_t b = min(wave + NW * (j0 + j), nblk - 1u);
-                    held[j] = *(global_uint4)(uintptr_t)(static_cast<const uint8_t *>(lead_input) + (size_t)b * TILE16_BLOCK_HANDED + lane * 16u);
+                    held[j] = tile16_load16<SEAM::SHARED_IN>(lead_input, b * TILE16_BLOCK_HANDED + lane * 16u);
                 }
-                if (j0 == 0) {
+                if (!SEAM::WAITS && j0 == 0) {
 #pragma unroll
                     for (int i = 0; i < D; i++) fetch(ring[i]);
                     fetch_the_rest();
@@ -230,11 +271,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
                     else *reinterpret_cast<uint2 *>(pairs + (size_t)b * TILE16_BLOCK_PAIRS + chunk * 8u) = uint2{held[j].x, held[j].y};
                 }
             }
-            if (count == 0) {
+            if (!SEAM::WAITS && count == 0) {
 #pragma unroll
                 for (int i = 0; i < D; i++) fetch(ring[i]);
                 fetch_the_rest();
             }
+            if (CHAINED && p.residual && q == 0 && r < tile_rows)
+                residual_held = __hip_atomic_load(p.residual + first_tile * tile_rows + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else if constexpr (R > 1) {
             // the weights' loads go out first; every row's activations follow (twice where the norm is folded in: once for
             // the row's sum of squares, once for the digits -- the second pass finds them in the cache)
@@ -273,11 +316,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
         f32x4 held[MAXJ], weight[MAXJ];
         const bool resident = units <= MAXJ * NT;
         float rms = 1.0f;
+        if constexpr (SEAM::WAITS) {
+            // behind a seam: the first weights are asked for, then the activations wait for the product that writes them
+#pragma unroll
+            for (int i = 0; i < D; i++) fetch(ring[i]);
+            fetch_the_rest();
+            if (!seam.wait(tid)) return false;
+        }
         if (resident) {
 #pragma unroll
             for (int j = 0; j < MAXJ; j++) {
                 const uint32_t e4 = tid + NT * j;
-                held[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(x + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                held[j] = e4 < units ? tile16_load4<SEAM::SHARED_IN>(x, 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
             if (lead_norm_w) {
 #pragma unroll
@@ -288,10 +338,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
             }
         }
         // the weights' loads go out behind the activations', which everything waits for first
+        if constexpr (!SEAM::WAITS) {
 #pragma unroll
-        for (int i = 0; i < D; i++) fetch(ring[i]);
-        fetch_the_rest();
+            for (int i = 0; i < D; i++) fetch(ring[i]);
+            fetch_the_rest();
+        }
         if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
+        // the first tile's residual, where this launch wrote it or reads what is written here: asked for now, added at the tile's end
+        if (CHAINED && MODE == TILE16_PLAIN && p.residual && q == 0 && r < tile_rows)
+            residual_held = __hip_atomic_load(p.residual + first_tile * tile_rows + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (lead_norm_w) {
             // sum of squares of the whole row (crates/neura-kernel/src/task/norm.rs:69-83; the same fp32 adds in another order)
             float square = 0.0f;
@@ -302,7 +357,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(held[j][i], held[j][i]));
             } else {
                 for (uint32_t e4 = tid; e4 < units; e4 += NT) {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(x + 4u * e4);
+                    const f32x4 v = tile16_load4<SEAM::SHARED_IN>(x, 4u * e4);
 #pragma unroll
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
                 }
@@ -324,7 +379,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
             }
         } else {
             for (uint32_t e4 = tid; e4 < units; e4 += NT)
-                stage(e4, *reinterpret_cast<const f32x4 *>(x + 4u * e4), lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
+                stage(e4, tile16_load4<SEAM::SHARED_IN>(x, 4u * e4), lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
                       digits, sums);
         }
         }
@@ -540,9 +595,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
                     const uint32_t plane = r >> 2, shift = 16u - 8u * min(plane, 2u);
                     uint32_t word = ((d0 >> shift) & 0xffu) | (((d1 >> shift) & 0xffu) << 8) | (((d2 >> shift) & 0xffu) << 16) | (((d3 >> shift) & 0xffu) << 24);
                     if (plane == 3u) word = r == 12u ? __builtin_bit_cast(uint32_t, chunk_sum * unscale) : (r == 13u ? __builtin_bit_cast(uint32_t, unscale) : 0u);
-                    reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u)[r] = word;
+                    tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u) + r, word);
                 } else {
-                    p.y[(size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r] = silu(gate[i]) * total;
+                    tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.y + (size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r),
+                                                        __builtin_bit_cast(uint32_t, silu(gate[i]) * total));
                 }
             } else if (MODE == TILE16_ROPE) {
                 uint32_t c;
@@ -554,9 +610,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
                 }
             } else if (r < tile_rows) {
                 const size_t n = (size_t)row * p.N + tile * tile_rows + r;
-                // in place (the decoder's residual stream): one add per element, nothing to wait for
-                if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);
-                else p.y[n] = p.residual ? p.residual[n] + total : total;
+                if constexpr (CHAINED) {
+                    // what another die wrote or will read inside this launch goes past the L2: no add in the cache, the
+                    // residual read at device scope (the first tile's was asked for ahead) and the sum stored at device scope
+                    float old = 0.0f;
+                    if (p.residual) old = index == 0 ? residual_held : __hip_atomic_load(p.residual + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    tile16_store_word<true>(reinterpret_cast<uint32_t *>(p.y + n), __builtin_bit_cast(uint32_t, old + total));
+                } else if (p.residual == p.y) {
+                    // in place (the decoder's residual stream): one add per element, nothing to wait for
+                    unsafeAtomicAdd(p.y + n, total);
+                } else {
+                    p.y[n] = p.residual ? p.residual[n] + total : total;
+                }
             }
           }
         }
@@ -564,7 +629,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
     };
     if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
         for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t), t);
-        return;
+        return true;
     }
     // Every wave walks whole rounds of D steps: the steps past its last tile multiply what was fetched again and publish nothing.
     uint32_t at_tile = 0, at_b = wave;
@@ -597,6 +662,20 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
             }
         }
     }
+    return true;
+}
+
+// The leading arguments are what a wave needs before it can ask for its first activations and weights.  They are plain words
+// so that the hardware can hand them over in scalar registers when it starts the wave (the file is built with
+// -amdgpu-kernarg-preload-count): the wave's first loads then go out without waiting for a load of its parameters
+// (about 0.5 us); everything else sits in `p` and is fetched meanwhile.  `input` is x, or the digit planes with HANDED.
+template <int NW, int D, int MODE, int R, bool HANDED = false>
+__global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, int32_t lead_to_w1,
+                                                                  int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
+                                                                  uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
+    tile16_product<NW, D, MODE, R, HANDED>(tile16_lds_bytes, blockIdx.x, NoSeam{}, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes, lead_grid,
+                                           lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -1117,8 +1196,16 @@ static hipError_t launch_tile16_mode(nh_device *d, const GemvParams &p, uint32_t
     return launch_tile16_rows<MODE, 1>(d, p, waves, grid, lds);
 }
 
-int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
-    GemvParams p{};
+// what a launch of the 16-row tile product is made of: the parameter block, waves a workgroup, workgroups, LDS
+struct Tile16Launch {
+    GemvParams p;
+    uint32_t waves, grid;
+    size_t lds;
+};
+
+static Tile16Launch tile16_plan(nh_device *d, const GemvArgs &a, uint32_t fixed_waves = 0) {
+    Tile16Launch plan{};
+    GemvParams &p = plan.p;
     for (int s = 0; s < 3; s++) {
         p.W[s] = static_cast<const uint8_t *>(a.W[s] ? a.W[s] : a.W[0]);
         p.end[s] = a.end[s];
@@ -1140,7 +1227,7 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     // waves of a workgroup share a tile and split its super-blocks: about two steps a wave
     // (sixteen on deep rows, where turning the activations into digits is the larger part of a wave's work; eight where the
     // digits arrive ready: fewer loads in flight a compute unit stream faster, as the shallow products show)
-    const uint32_t waves = p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u || a.digits_in ? 8u : 16u));
+    plan.waves = fixed_waves ? fixed_waves : (p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u || a.digits_in ? 8u : 16u)));
     // units of work: tiles, or with SwiGLU pairs (a gate tile and the up tile behind it); every workgroup takes the same
     // number of them, one workgroup a compute unit when there are that many
     // A plain tile holds the number of rows, 16 down to 12, that leaves the fewest compute units idle in the last round.
@@ -1159,8 +1246,16 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     const uint32_t units = a.swiglu ? a.N / 32u : a.N / p.tile_rows;
     p.row_groups = units;
     const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
-    const uint32_t grid = (units + rounds - 1u) / rounds;
-    const size_t lds = tile16_lds(p.nblk, waves, tile16_row_form(a.rows), a.digits_in != nullptr);
+    plan.grid = (units + rounds - 1u) / rounds;
+    plan.lds = tile16_lds(p.nblk, plan.waves, tile16_row_form(a.rows), a.digits_in != nullptr);
+    return plan;
+}
+
+int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
+    const Tile16Launch plan = tile16_plan(d, a);
+    const GemvParams &p = plan.p;
+    const uint32_t waves = plan.waves, grid = plan.grid;
+    const size_t lds = plan.lds;
     profile_mark(d);
     hipError_t launched = a.digits_in ? launch_tile16_handed(d, p, waves, grid, lds)
                           : a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
@@ -1169,6 +1264,201 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     NH_HIP(launched);
     profile_mark(d);
     if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    return NH_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Several dependent one-row products in one launch (crates/neura-kernel/src/scheduler.rs:110-166 runs a whole program as one
+// persistent kernel; here it is the products between two attentions of a decode step: attn_output, gate|up, ffn_down and the
+// q|k|v product of the layer behind, or the head).  One workgroup of eight waves a compute unit, all resident at once; every
+// stage is the 16-row tile product above.  At a seam a workgroup
+//   - waits until its own stores of the stage before have been acknowledged (s_waitcnt vmcnt(0); they went out at device
+//     scope, so they are in memory by then), meets at a barrier and publishes `epoch` in its own flag word;
+//   - asks for its first weights of the next stage -- they depend on nothing, so HBM streams through the wait;
+//   - wave 0 reads all the flag words (sixteen bytes a lane) until every one holds the epoch, at most `spin` times: a wait
+//     that runs out writes REFUSAL_SEAM and the whole workgroup leaves, as then does every other one (the host runs the step
+//     again, one launch a product);
+//   - reads its activations at device scope and walks.
+// Flag words only grow within a step; the step's first kernel clears them.
+struct ChainStage {
+    const uint8_t *w0;
+    const void *input;
+    const float *norm_w;
+    int32_t to_w1, to_w2;
+    uint32_t row_bytes, grid, tiles, tile_rows, end0, end1;
+    GemvParams p;
+};
+constexpr int CHAIN_STAGES_MOST = 4;
+struct ChainParams {
+    ChainStage stage[CHAIN_STAGES_MOST];
+    uint32_t *flags;    // one word a workgroup
+    uint32_t *refusal;
+    uint32_t epoch;     // what the first seam of this launch publishes; the next one epoch + 1, ...
+    uint32_t spin;      // reads of the flag words a wait may take
+    uint32_t lds_bytes; // of the launch: the seam's word sits in its last sixteen bytes
+};
+
+template <bool WAITS_, bool IN_, bool OUT_>
+struct ChainSeam {
+    static constexpr bool WAITS = WAITS_, SHARED_IN = IN_, SHARED_OUT = OUT_;
+    const uint32_t *flags;
+    uint32_t *refusal;
+    uint32_t *word;  // in LDS
+    uint32_t epoch, spin, workgroups;
+    __device__ __forceinline__ bool wait(uint32_t tid) const {
+        if constexpr (!WAITS_) return true;
+        if (tid < 64u) {
+            bool met = false;
+            for (uint32_t turn = 0; turn < spin && !met; turn++) {
+                const u32x4 held = tile16_load16<true>(flags, tid * 16u);
+                bool here = true;
+#pragma unroll
+                for (int i = 0; i < 4; i++) here = here && (4u * tid + i >= workgroups || held[i] >= epoch);
+                met = __builtin_amdgcn_ballot_w64(!here) == 0;
+                if (!met) __builtin_amdgcn_s_sleep(2);
+            }
+            if (tid == 0) *word = met ? 1u : 0u;
+        }
+        __syncthreads();
+        const bool met = *word != 0u;
+        if (!met && tid == 0) atomicMax(refusal, (uint32_t)REFUSAL_SEAM);
+        return met;
+    }
+};
+
+// a workgroup's stores of the stage before are in memory, and it says so
+__device__ __forceinline__ void chain_arrive(uint32_t *flags, uint32_t block, uint32_t epoch) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(flags + block, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+enum ChainProgram { CHAIN_FFN = 0, CHAIN_O_FFN = 1, CHAIN_O_FFN_QKV = 2, CHAIN_O_FFN_HEAD = 3 };
+
+#define CHAIN_STAGE_ARGUMENTS(s) (s).w0, (s).input, (s).norm_w, (s).to_w1, (s).to_w2, (s).row_bytes, (s).grid, (s).tiles, (s).tile_rows, (s).end0, (s).end1, (s).p
+
+template <int PROGRAM>
+__global__ __launch_bounds__(512) void gemv_q4k_chain_kernel(ChainParams c) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t chain_lds_bytes[];
+    constexpr bool LEADS = PROGRAM != CHAIN_FFN;                               // attn_output in front
+    constexpr bool TRAILS = PROGRAM == CHAIN_O_FFN_QKV || PROGRAM == CHAIN_O_FFN_HEAD;  // a product behind ffn_down
+    const uint32_t block = blockIdx.x, workgroups = gridDim.x;
+    uint32_t *const word = reinterpret_cast<uint32_t *>(chain_lds_bytes + c.lds_bytes - 16u);
+    uint32_t epoch = c.epoch;
+    int at = 0;
+    if constexpr (LEADS) {
+        // attn_output: x is the attention's output (the launch before), y = h += ... is read by gate|up
+        const ChainSeam<false, false, true> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
+        tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]));
+        chain_arrive(c.flags, block, epoch);
+        at++;
+    }
+    {
+        // gate|up with SwiGLU: reads h, leaves digit planes
+        const ChainSeam<LEADS, LEADS, true> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
+        if (!tile16_product<8, 2, TILE16_SWIGLU, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
+        if (LEADS) epoch++;
+        chain_arrive(c.flags, block, epoch);
+        at++;
+    }
+    {
+        // ffn_down over the digit planes, h += ...
+        const ChainSeam<true, true, TRAILS> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
+        if (!tile16_product<8, 2, TILE16_PLAIN, 1, true>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
+        at++;
+    }
+    if constexpr (TRAILS) {
+        epoch++;
+        chain_arrive(c.flags, block, epoch);
+        const ChainSeam<true, true, false> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
+        if constexpr (PROGRAM == CHAIN_O_FFN_QKV) {
+            if (!tile16_product<8, 2, TILE16_ROPE, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
+        } else {
+            if (!tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
+        }
+    }
+}
+
+static bool chain_stage_takes(const GemvArgs &a) {
+    if (!tile16_takes(a) || a.rows != 1) return false;
+    return tile16_lds(a.K / 256u, 8u, 1u, a.digits_in != nullptr) + 16u <= 160u * 1024u;
+}
+
+// Whether launch_chain takes these products as one launch: attn_output (or none), gate|up handing its digits to ffn_down, and
+// behind them the next q|k|v with the rotation folded in, or the head (or none).  NEURA_HIP_CHAIN: 0 keeps one launch a product,
+// 1 chains gate|up and ffn_down, 2 (the default) attn_output in front of them, 3 the product behind them as well.
+bool gemv_chains(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail) {
+    const int wanted = env_int("NEURA_HIP_CHAIN", 2);
+    if (wanted <= 0 || !d->chain_flags || d->compute_units > 256 || d->compute_units < 1) return false;
+    if (lead && wanted < 2) return false;
+    if (trail && wanted < 3) return false;
+    if (!gate_up.digits_out || !down.digits_in || gate_up.digits_out != down.digits_in) return false;
+    if (!chain_stage_takes(gate_up) || !chain_stage_takes(down)) return false;
+    if (lead && (!chain_stage_takes(*lead) || lead->swiglu || lead->rope || lead->digits_in || lead->digits_out)) return false;
+    if (trail && (!chain_stage_takes(*trail) || trail->swiglu || trail->digits_in || trail->digits_out || trail->residual)) return false;
+    return true;
+}
+
+template <int PROGRAM>
+static hipError_t launch_chain_program(nh_device *d, const ChainParams &c, uint32_t grid) {
+    static bool raised = false;
+    if (!raised) {
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_chain_kernel<PROGRAM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (error != hipSuccess) return error;
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemv_q4k_chain_kernel<PROGRAM>), dim3(grid), dim3(512), c.lds_bytes, d->stream, c);
+    return hipGetLastError();
+}
+
+int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t epoch, uint32_t spin) {
+    ChainParams c{};
+    const GemvArgs *stages[CHAIN_STAGES_MOST] = {nullptr, nullptr, nullptr, nullptr};
+    int count = 0;
+    if (lead) stages[count++] = lead;
+    stages[count++] = &gate_up;
+    stages[count++] = &down;
+    if (trail) stages[count++] = trail;
+    size_t lds = 0;
+    uint64_t bytes = 0;
+    for (int s = 0; s < count; s++) {
+        const Tile16Launch plan = tile16_plan(d, *stages[s], 8u);
+        const GemvParams &p = plan.p;
+        ChainStage &stage = c.stage[s];
+        stage.w0 = p.W[0];
+        stage.input = p.digits_in ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x);
+        stage.norm_w = p.norm_w;
+        stage.to_w1 = (int32_t)((p.W[1] - p.W[0]) / 16), stage.to_w2 = (int32_t)((p.W[2] - p.W[0]) / 16);
+        stage.row_bytes = p.row_bytes, stage.grid = plan.grid, stage.tiles = p.row_groups;
+        stage.tile_rows = stages[s]->rope ? p.rope_width : p.tile_rows;
+        stage.end0 = p.end[0], stage.end1 = p.end[1];
+        stage.p = p;
+        if (plan.lds > lds) lds = plan.lds;
+        bytes += (uint64_t)stages[s]->N * p.row_bytes;
+    }
+    // one workgroup a compute unit: more LDS than two of them could share
+    lds += 16u;
+    if (lds < 84u * 1024u) lds = 84u * 1024u;
+    c.flags = d->chain_flags, c.refusal = d->refusal, c.epoch = epoch, c.spin = spin, c.lds_bytes = (uint32_t)lds;
+    const uint32_t grid = (uint32_t)d->compute_units;
+    profile_mark(d);
+    hipError_t launched;
+    if (!lead) launched = launch_chain_program<CHAIN_FFN>(d, c, grid);
+    else if (!trail) launched = launch_chain_program<CHAIN_O_FFN>(d, c, grid);
+    else if (trail->rope) launched = launch_chain_program<CHAIN_O_FFN_QKV>(d, c, grid);
+    else launched = launch_chain_program<CHAIN_O_FFN_HEAD>(d, c, grid);
+    NH_HIP(launched);
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += bytes;
+    return NH_OK;
+}
+
+__global__ __launch_bounds__(256) void chain_clear_kernel(uint32_t *flags) { flags[threadIdx.x] = 0u; }
+
+int32_t launch_chain_clear(nh_device *d) {
+    if (!d->chain_flags) return NH_OK;
+    hipLaunchKernelGGL(chain_clear_kernel, dim3(1), dim3(256), 0, d->stream, d->chain_flags);
+    NH_HIP(hipGetLastError());
     return NH_OK;
 }
 

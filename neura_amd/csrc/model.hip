@@ -44,6 +44,11 @@ struct nh_model {
     uint64_t graph_moved[4] = {0, 0, 0, 0};  // nh_device::moved when each graph was recorded
     bool graph_warmed[4] = {false, false, false, false};  // the variant has run once outside a capture
     bool use_graph = true;
+    // Dependent products of a decode step as one launch with seams between them (launch_chain) until a seam's wait runs out
+    // once: the step is then run again one launch a product, and so is every later one.
+    bool chain = true;
+    uint32_t chain_spin = 1u << 18;  // reads of the flag words a seam's wait may take (NEURA_HIP_CHAIN_SPIN)
+    uint32_t seam_fallbacks = 0;     // steps run again because a seam gave up
 };
 
 namespace {
@@ -126,6 +131,9 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
     const uint8_t *mask = any_inactive ? dev_mask(m) : nullptr;
     const bool wide = T > 8;  // more rows than the narrow product takes
     int32_t status;
+    uint32_t chain_launches = 0;
+    const bool chains = m->chain && T == 1 && !mask;
+    if (chains && (status = launch_chain_clear(d)) != NH_OK) return status;
     if (!products_only && (status = launch_gather(d, m->elements[EMBD], m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK)
         return status;
     const float scale = 1.0f / sqrtf((float)hd);
@@ -258,9 +266,30 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             if ((status = launch_gemm(d, dn)) != NH_OK) return status;
         } else {
             if (sums.sections) o.merge = &sums;
-            if ((status = launch_gemv(d, o)) != NH_OK) return status;
             GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
             dn.residual = m->h;
+            bool chained = false;
+            if (chains && !o.merge && element_at(m, L, GATE) == element_at(m, L, UP)) {
+                GemvArgs gu = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
+                gu.W[1] = m->ffn_up[L];
+                gu.end[0] = F, gu.end[1] = gu.end[2] = 2 * F;
+                gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
+                if (gemv_hands_digits(gu, dn) && gemv_digit_bytes(F) <= (size_t)F * sizeof(float)) {
+                    gu.digits_out = reinterpret_cast<uint8_t *>(m->up), dn.digits_in = reinterpret_cast<const uint8_t *>(m->up);
+                    const uint32_t epoch = 1u + CHAIN_EPOCHS_A_LAUNCH * chain_launches;
+                    if (gemv_chains(d, &o, gu, dn, nullptr)) {
+                        if ((status = launch_chain(d, &o, gu, dn, nullptr, epoch, m->chain_spin)) != NH_OK) return status;
+                        chained = true, chain_launches++;
+                    } else if (gemv_chains(d, nullptr, gu, dn, nullptr)) {
+                        if ((status = launch_gemv(d, o)) != NH_OK) return status;
+                        if ((status = launch_chain(d, nullptr, gu, dn, nullptr, epoch, m->chain_spin)) != NH_OK) return status;
+                        chained = true, chain_launches++;
+                    }
+                    dn.digits_in = nullptr;
+                }
+            }
+            if (chained) continue;
+            if ((status = launch_gemv(d, o)) != NH_OK) return status;
             if (element_at(m, L, GATE) == element_at(m, L, UP)) {
                 GemvArgs gu = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
                 gu.W[1] = m->ffn_up[L];
@@ -481,6 +510,9 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
             return nullptr;
         }
         m->use_graph = !(held && held[0] == '0') && !traced;
+        // NEURA_HIP_CHAIN_SPIN: the reads of the flag words a seam's wait may take (0: every wait gives up at once, which is how
+        // the tests reach the step that is run again)
+        if (const char *spin = getenv("NEURA_HIP_CHAIN_SPIN"); spin && spin[0]) m->chain_spin = (uint32_t)strtoul(spin, nullptr, 10);
     }
     ok = ok && hipStreamSynchronize(device->stream) == hipSuccess;
     if (!ok) {
@@ -494,6 +526,8 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
 void nh_model_destroy(nh_model *model) { release(model); }
 
 uint32_t nh_model_capacity(const nh_model *model) { return model ? model->capacity : 0; }
+
+uint32_t nh_model_seam_fallbacks(const nh_model *model) { return model ? model->seam_fallbacks : 0; }
 
 static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *cursors, const uint8_t *mask, uint32_t batch,
                            const nh_draw *draws, uint32_t *chosen_out) {
@@ -515,44 +549,59 @@ static int32_t decode_step(nh_model *m, const uint32_t *tokens, const uint32_t *
     // shape depends on them, so the step is captured once per mask variant and replayed.
     // Profiled steps run eagerly (event records do not belong in a graph).
     const int variant = (any_inactive ? 1 : 0) + (draws ? 2 : 0);
-    hipGraphExec_t &graph = m->decode_graph[variant];
-    // The first step of a variant runs eagerly: its launchers grow the device scratch to what the variant needs (an
-    // allocation, which does not belong inside a stream capture; the outgrown block is kept until nh_close).
-    if (m->use_graph && traced_by_rocprofiler()) return fail(NH_E_DEVICE, "a recorded decode step is never launched in a process traced by rocprofv3");
-    if (m->use_graph && !d->profile && m->graph_warmed[variant]) {
-        if (graph && m->graph_moved[variant] != d->moved) {
-            // the device scratch or rope table moved since the capture (another model or operator call grew it)
-            (void)hipGraphExecDestroy(graph);
-            graph = nullptr;
-        }
-        if (!graph) {
-            m->graph_moved[variant] = d->moved;
-            NH_HIP(hipStreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal));
-            status = decode_kernels(m, any_inactive, draws != nullptr);
-            hipGraph_t recorded = nullptr;
-            hipError_t ended = hipStreamEndCapture(d->stream, &recorded);
-            if (status != NH_OK) {
-                if (recorded) (void)hipGraphDestroy(recorded);
-                return status;
-            }
-            if (ended != hipSuccess) return hip_fail(ended, "hipStreamEndCapture");
-            hipError_t built = hipGraphInstantiate(&graph, recorded, nullptr, nullptr, 0);
-            (void)hipGraphDestroy(recorded);
-            if (built != hipSuccess) {
+    for (int attempt = 0;; attempt++) {
+        hipGraphExec_t &graph = m->decode_graph[variant];
+        // The first step of a variant runs eagerly: its launchers grow the device scratch to what the variant needs (an
+        // allocation, which does not belong inside a stream capture; the outgrown block is kept until nh_close).
+        if (m->use_graph && traced_by_rocprofiler()) return fail(NH_E_DEVICE, "a recorded decode step is never launched in a process traced by rocprofv3");
+        if (m->use_graph && !d->profile && m->graph_warmed[variant]) {
+            if (graph && m->graph_moved[variant] != d->moved) {
+                // the device scratch or rope table moved since the capture (another model or operator call grew it)
+                (void)hipGraphExecDestroy(graph);
                 graph = nullptr;
-                return hip_fail(built, "hipGraphInstantiate");
             }
+            if (!graph) {
+                m->graph_moved[variant] = d->moved;
+                NH_HIP(hipStreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal));
+                status = decode_kernels(m, any_inactive, draws != nullptr);
+                hipGraph_t recorded = nullptr;
+                hipError_t ended = hipStreamEndCapture(d->stream, &recorded);
+                if (status != NH_OK) {
+                    if (recorded) (void)hipGraphDestroy(recorded);
+                    return status;
+                }
+                if (ended != hipSuccess) return hip_fail(ended, "hipStreamEndCapture");
+                hipError_t built = hipGraphInstantiate(&graph, recorded, nullptr, nullptr, 0);
+                (void)hipGraphDestroy(recorded);
+                if (built != hipSuccess) {
+                    graph = nullptr;
+                    return hip_fail(built, "hipGraphInstantiate");
+                }
+            }
+            NH_HIP(hipGraphLaunch(graph, d->stream));
+        } else {
+            if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) return status;
+            m->graph_warmed[variant] = true;
         }
-        NH_HIP(hipGraphLaunch(graph, d->stream));
-    } else {
-        if ((status = decode_kernels(m, any_inactive, draws != nullptr)) != NH_OK) return status;
-        m->graph_warmed[variant] = true;
+        if (!m->chosen_mapped) {
+            NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
+            NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
+        }
+        NH_HIP(hipStreamSynchronize(d->stream));
+        if (m->chosen_host[batch] != REFUSAL_SEAM || attempt > 0) break;
+        // A seam of a chained launch gave up (not every workgroup was resident, or one was held up past the wait's bound):
+        // what the step wrote behind it is not to be trusted.  Every kernel of a step reads its inputs from where the host
+        // staged them and writes the same cache rows again, so the step is simply run once more, one launch a product, and
+        // the model stays that way; recorded steps hold chained launches and are dropped.
+        NH_HIP(hipMemsetAsync(d->refusal, 0, sizeof(uint32_t), d->stream));
+        NH_HIP(hipStreamSynchronize(d->stream));
+        m->chain = false;
+        m->seam_fallbacks++;
+        for (hipGraphExec_t &held : m->decode_graph) {
+            if (held) (void)hipGraphExecDestroy(held);
+            held = nullptr;
+        }
     }
-    if (!m->chosen_mapped) {
-        NH_HIP(hipMemcpyAsync(m->chosen_host, m->chosen_dev, (size_t)batch * 4, hipMemcpyDeviceToHost, d->stream));
-        NH_HIP(hipMemcpyAsync(m->chosen_host + batch, d->refusal, 4, hipMemcpyDeviceToHost, d->stream));
-    }
-    NH_HIP(hipStreamSynchronize(d->stream));
     if (m->chosen_host[batch] != REFUSAL_NONE) return check_refusal(d, "a decode step");
     memcpy(chosen_out, m->chosen_host, (size_t)batch * 4);
     return NH_OK;

@@ -101,6 +101,10 @@ class Model:
             self.lib.nh_model_destroy(self.handle)
             self.handle = None
 
+    def seam_fallbacks(self):
+        """decode steps that were run again, one launch a product, because a seam of a chained launch gave up"""
+        return int(self.lib.nh_model_seam_fallbacks(self.handle))
+
     @staticmethod
     def _u32(values):
         return np.ascontiguousarray(values, dtype=np.uint32)

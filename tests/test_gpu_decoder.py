@@ -608,6 +608,74 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         held.release()
 
 
+CHAIN_SHAPES = [SMALL_Q4, dict(layers=2, hidden=3584, heads=28, kv_heads=4, head_dim=128, ffn=18944, vocab=2048, tied=False)]
+
+
+@pytest.mark.parametrize("shape", CHAIN_SHAPES, ids=["small", "7b-layers"])
+@pytest.mark.parametrize("chain", ["1", "2"])
+def test_products_chained_into_one_launch_match_one_launch_a_product(device, monkeypatch, shape, chain):
+    """At batch 1 the products between two attentions run as one launch with seams between them (NEURA_HIP_CHAIN=1: gate|up
+    and ffn_down; 2: attn_output in front): what crosses a seam crosses it at device scope, behind a flag every workgroup
+    publishes.  The same steps one launch a product (NEURA_HIP_CHAIN=0) give the same logits to the last few bits (the chained
+    stages split a row's super-blocks over eight waves where the launches of their own take four or seven, so sums associate
+    differently), the same tokens and the same cache rows; both sit within the decoder's bar of the oracle.  No step fell
+    back."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    tensors = list(synth.model_tensors(shape, NH_Q4_K, np.random.default_rng(21), mode="normal", threads=16))
+    weights = Weights(device, tensors)
+    chained, apart = Model(device, weights, shape, NH_Q4_K, 1, 40), Model(device, weights, shape, NH_Q4_K, 1, 40)
+    ref = oracle.Model(shape, NH_Q4_K, {name: raw for name, _, _, raw in tensors}, 1, 40)
+    token_a = token_b = 11
+    for step in range(6):
+        monkeypatch.setenv("NEURA_HIP_CHAIN", chain)
+        got_a = chained.decode_step([token_a], [step])
+        logits_a = chained.logits()
+        monkeypatch.setenv("NEURA_HIP_CHAIN", "0")
+        got_b = apart.decode_step([token_b], [step])
+        logits_b = apart.logits()
+        want_logits, want = ref.forward([token_a], 1, [step], threads=16)
+        scale = np.abs(want_logits).max()
+        assert np.abs(logits_a - logits_b).max() <= 2e-5 * scale, step
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * scale, step
+        assert list(got_a) == list(got_b) == list(want), (step, margins(want_logits))
+        token_a = token_b = int(got_a[0])
+    same_cache_rows(chained, ref, shape["layers"], [list(range(6))], "rows the chained steps appended")
+    assert chained.seam_fallbacks() == 0 and apart.seam_fallbacks() == 0
+    for held in (chained, apart, weights):
+        held.release()
+
+
+@pytest.mark.parametrize("graph", ["0", "1"])
+def test_a_seam_that_gives_up_sends_the_step_down_the_path_of_one_launch_a_product(device, monkeypatch, graph):
+    """NEURA_HIP_CHAIN_SPIN=0: every wait at a seam gives up before its first look (the kernels all end; no wait is ever
+    unbounded).  The step that met it is run again one launch a product and answers as the oracle does, the model counts one
+    fallback and stays on that path, eager or recorded."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", graph)
+    monkeypatch.setenv("NEURA_HIP_CHAIN_SPIN", "0")
+    model, ref, weights = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=40, seed=22)
+    monkeypatch.delenv("NEURA_HIP_CHAIN_SPIN")
+    token = 5
+    for step in range(5):
+        want_logits, want = ref.forward([token], 1, [step])
+        got = model.decode_step([token], [step])
+        assert np.abs(model.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), step
+        assert model.seam_fallbacks() == 1, step
+        token = int(got[0])
+    # a model built without the hook chains, and never falls back
+    healthy, ref, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=40, seed=22)
+    token = 5
+    for step in range(5):
+        want_logits, want = ref.forward([token], 1, [step])
+        got = healthy.decode_step([token], [step])
+        assert np.abs(healthy.logits() - want_logits).max() <= 1e-3 * np.abs(want_logits).max(), step
+        assert list(got) == list(want), step
+        token = int(got[0])
+    assert healthy.seam_fallbacks() == 0
+    for held in (model, healthy, weights, weights_b):
+        held.release()
+
+
 def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch):
     """At batch 1 the gate|up product of a Q4_K decoder leaves silu(gate) * up as the digit planes ffn_down multiplies (a
     power-of-two scale per 16 outputs where ffn_down's own staging takes one per 64); NEURA_HIP_TILE16_HANDED=0 hands the
