@@ -78,7 +78,7 @@ struct nh_device {
     // recorded again when this no longer matches the count at its capture
     uint64_t moved = 0;
     uint32_t *refusal = nullptr;  // device word: 0 = none, else a refusal code
-    uint32_t *chain_flags = nullptr;  // 256 words: one a workgroup of a chained launch (launch_chain), cleared by a step's first kernel
+    uint32_t *tick = nullptr;  // device word that launch_tick moves on at the start of every pass over a decoder's layers: part of every tag word
     uint8_t *static_scratch = nullptr;  // this device's copy of the file-scope array nh_argmax_static works in (argmax.hip)
     struct RopeTable {
         float base;
@@ -199,6 +199,12 @@ struct GemvArgs {
     // token whose q|k went out rotated from their own product -- its rows (+ bias[0]) are also cast into the value state
     // (cache_v, cursor, width, capacity and ring of this RopeFusion; halves), what launch_value_append does from y.
     const RopeFusion *append_value = nullptr;
+    // Products chained into one launch (launch_chain), and a SwiGLU product that hands digit planes on: the numbers (1..127) of
+    // the seams this product reads and writes across -- what is handed over carries them as tag words -- and, for a plain
+    // product whose outputs another product of the same launch reads, where it leaves them as (value, tag) pairs beside y;
+    // then x of the product behind it is that same array.
+    uint32_t tag_in = 0, tag_out = 0;
+    void *pairs_out = nullptr;
 };
 int32_t launch_gemv(nh_device *d, const GemvArgs &args);
 // whether launch_gemv can merge attention sections of `width` channels a head into the activation row of this product
@@ -209,13 +215,13 @@ bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer);
 size_t gemv_digit_bytes(uint32_t K);
 // Several dependent one-row Q4_K products as one launch with seams between them: attn_output (`lead`, or nullptr), gate|up
 // handing its digit planes to ffn_down, and behind them the next q|k|v with the rotation folded in or the head (`trail`, or
-// nullptr).  gemv_chains() says whether launch_chain takes them.  `epoch`: the first of the three flag values the launch may
-// publish (they only grow between two launch_chain_clear); `spin`: the reads of the flag words a workgroup's wait may take
-// before it gives up with REFUSAL_SEAM.
+// nullptr).  gemv_chains() says whether launch_chain takes them.
+// `spin`: how often a reader may read a piece again whose tag is not the seam's before it gives up with REFUSAL_SEAM.
+int gemv_chain_level();  // NEURA_HIP_CHAIN: 0 (the default) one launch a product, 1 gate|up with ffn_down, 2 attn_output in front, 3 a product behind
 bool gemv_chains(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail);
-int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t epoch, uint32_t spin);
-int32_t launch_chain_clear(nh_device *d);
-constexpr uint32_t CHAIN_EPOCHS_A_LAUNCH = 3;
+int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t spin);
+// moves the device's tick word on: once at the start of every pass over a decoder's layers, before anything that writes tags
+int32_t launch_tick(nh_device *d);
 // whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)
 bool gemv_fuses_rope(const GemvArgs &args, const RopeFusion &rope);
 

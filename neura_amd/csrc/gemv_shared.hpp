@@ -42,6 +42,13 @@ struct GemvParams {
     uint32_t merge_sections, merge_groups, merge_width;
     // staged K-quant kernel, one row: the outputs (+ bias[0]) also go into the value state rope_v at rope_cursor as halves
     uint32_t append_value;
+    // 16-row tile kernel: what is handed to another product carries tag words (gemv_tile16.hip): `tick` is the device word a
+    // step's first kernel moves on, tag_in / tag_out the numbers (1..127) of the seams this product reads and writes across,
+    // pairs_out where a plain product of a chained launch leaves its outputs as (value, tag) pairs beside y
+    const uint32_t *tick;
+    uint32_t tag_in, tag_out;
+    uint2 *pairs_out;
+    uint32_t late_from;  // handed planes behind a seam: the first super-block whose chunks the product before writes in its last round
 };
 
 // the parameters a product reads before its first vector load, and the rotation's where it is folded in

@@ -51,16 +51,24 @@ struct Tile16Unit {
 // is then a chunk's own, not a group's, so the four MFMAs of a step keep their sums apart and each is weighed by its
 // chunk's scale; the staging pass shrinks to a copy.
 //
-// A seam stands between two products of one launch (gemv_q4k_chain_kernel below): the product behind it may ask for its
-// first weights at once -- they depend on nothing -- but reads its activations only when every workgroup has finished the
-// product before.  What crosses a seam crosses it between compute units of different dies, whose L2 caches do not see each
-// other's writes inside a launch: it is stored and loaded at device scope (sc1: written through to memory, read past the
-// L2), with no cache write-back or invalidation.  NoSeam is a product that is a launch of its own.
+// A seam stands between two products of one launch (gemv_q4k_chain_kernel below).  The product behind it asks for its first
+// weights at once -- they depend on nothing -- and then for its activations, which the product before may still be writing.
+// What crosses a seam crosses it between compute units of different dies, whose L2 caches do not see each other's writes
+// inside a launch, so it is stored and loaded at device scope (sc1: written through to memory, read past the L2) -- and it
+// carries its own proof of arrival: every piece the memory writes as one (a 32-byte sector of a chunk of digit planes, an
+// 8-byte (value, tag) pair of a float) ends in a tag word that names the launch's step and the seam, and a reader that
+// finds another tag reads the piece again, `spin` times at most.  No flag, no barrier between workgroups and no wait for a
+// store's acknowledgement: a workgroup that is done with one product walks into the next, and waits only where the very
+// numbers it needs are not there yet.  A reader that runs out of turns writes REFUSAL_SEAM and goes on with what it has
+// (every wave still reaches every barrier and the kernel ends); the host then runs the step again, one launch a product.
+// NoSeam is a product that is a launch of its own.
 struct NoSeam {
-    static constexpr bool WAITS = false;         // the activations wait for the seam
+    static constexpr bool WAITS = false;         // the first weights are asked for before the activations
     static constexpr bool SHARED_IN = false;     // activations (and the residual) were written by this launch
     static constexpr bool SHARED_OUT = false;    // outputs are read by a later product of this launch
-    __device__ __forceinline__ bool wait(uint32_t) const { return true; }
+    static constexpr bool HANDS_RING = false;    // past its last unit the ring fetches the first units of the product behind the seam
+    static constexpr bool TAKES_RING = false;    // the ring arrives with this product's first units in flight
+    uint32_t spin = 0;
 };
 
 typedef float tile16_f32x4 __attribute__((ext_vector_type(4)));
@@ -75,6 +83,11 @@ __device__ __forceinline__ u32x4 tile16_load16(const void *base, uint32_t offset
         return *(global_uint4)(uintptr_t)(static_cast<const uint8_t *>(base) + offset);
     }
 }
+// the same, past the L2 (device scope) only where `past` says so: a reader's first look may be served by the L2 of its die --
+// whatever it finds there carries its tag -- and only a piece found stale is read again from memory
+__device__ __forceinline__ u32x4 tile16_load16_either(const void *base, uint32_t offset, bool past) {
+    return past ? tile16_load16<true>(base, offset) : tile16_load16<false>(base, offset);
+}
 template <bool SHARED>
 __device__ __forceinline__ tile16_f32x4 tile16_load4(const float *base, uint32_t element) {
     if constexpr (SHARED) return __builtin_bit_cast(tile16_f32x4, tile16_load16<true>(base, element * 4u));
@@ -86,9 +99,13 @@ __device__ __forceinline__ void tile16_store_word(uint32_t *at, uint32_t word) {
     else *at = word;
 }
 
-// The product itself; `block` of `lead_grid` workgroups.  Returns false where the seam gave up (the whole workgroup leaves).
+// The product itself; `block` of `lead_grid` workgroups.
+// `ring`: the units in flight, the caller's (a chained launch hands them from one product to the next: with HANDS_RING the
+// fetches past this product's last unit ask for super-blocks wave, wave + NW, ... of `next_row`, this lane's weight row in
+// the first tile the workgroup walks of the product behind the seam (nullptr: it walks none), which then TAKES_RING).
 template <int NW, int D, int MODE, int R, bool HANDED, class SEAM>
-__device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const uint32_t block, const SEAM seam, const uint8_t *lead_w0, const void *lead_input,
+__device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const uint32_t block, const SEAM seam, Tile16Unit (&ring)[D], const uint8_t *next_row,
+                                               uint32_t next_nblk, const uint8_t *lead_w0, const void *lead_input,
                                                const float *lead_norm_w, int32_t lead_to_w1, int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid,
                                                uint32_t lead_tiles, uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, const GemvParams &p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
@@ -121,7 +138,22 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
     const uint32_t r = lane & 15u, q = lane >> 4;
     // tiles of this workgroup: blockIdx.x, blockIdx.x + lead_grid, ... (with SwiGLU a pair of tiles: gate rows, then the up rows)
     const uint32_t tiles = lead_tiles;
-    if (block >= tiles || block >= lead_grid) return true;  // the whole workgroup: no barrier has been reached
+    // what a wave with nothing (more) to fetch here asks for on behalf of the product behind the seam
+    auto hand_on = [&]() {
+        if constexpr (SEAM::HANDS_RING) {
+#pragma unroll
+            for (int i = 0; i < D; i++) {
+                const uint8_t *at = (next_row ? next_row : lead_w0 + q * 32u) + (size_t)(next_row ? min(wave + NW * (uint32_t)i, next_nblk - 1u) : 0u) * 144u;
+                ring[i].hdr = *(global_uint4)(uintptr_t)(at - q * 32u);
+                ring[i].qa = *(global_uint4)(uintptr_t)(at + 16u);
+                ring[i].qb = *(global_uint4)(uintptr_t)(at + 32u);
+            }
+        }
+    };
+    if (block >= tiles || block >= lead_grid) {  // the whole workgroup: no barrier has been reached
+        hand_on();
+        return;
+    }
     const uint32_t ntiles = (tiles - block + lead_grid - 1u) / lead_grid;
     const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;  // super-blocks of one tile this wave walks
 
@@ -162,20 +194,41 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
     // Loads run D steps ahead of the arithmetic, across tile boundaries.  Every fetch issues its three loads: past the last
     // step the last unit is fetched again and dropped, so that every path issues the same loads in the same order and the
     // waits count exactly how many loads are newer than the one needed.
-    Tile16Unit ring[D];
     uint32_t ahead_tile = 0, ahead_b = wave;
     const uint8_t *ahead_row = lane_row(tile_at(0));
-    auto fetch = [&](Tile16Unit &u) {
-        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * 144u;
-        u.hdr = *(global_uint4)(uintptr_t)(at - q * 32u);
-        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
-        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+    // HANDS_RING: once this wave's last unit is asked for, the fetches that would ask for it again ask for units 0, 1, ... of the
+    // product behind the seam instead (the first `pad` of them still are fillers: the walk below runs whole rounds of D steps,
+    // and the last D fetches are the ones whose units stay in the ring)
+    bool exhausted = count == 0;
+    int32_t beyond = -(int32_t)((D - (walked * count) % D) % D);
+    auto advance = [&]() {
         if (ahead_b + NW < nblk) {
             ahead_b += NW;
         } else if (ahead_tile + 1u < walked) {
             ahead_b = wave;
             ahead_tile++;
             ahead_row = lane_row(tile_at(ahead_tile));
+        } else {
+            exhausted = true;
+        }
+    };
+    auto fetch = [&](Tile16Unit &u) {
+        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * 144u;
+        if constexpr (SEAM::HANDS_RING) {
+            if (exhausted && next_row) at = next_row + (size_t)min(wave + NW * (uint32_t)max(beyond, 0), next_nblk - 1u) * 144u;
+            if (exhausted) beyond++;
+        }
+        u.hdr = *(global_uint4)(uintptr_t)(at - q * 32u);
+        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
+        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+        advance();
+    };
+    // TAKES_RING: the product before asked for this wave's first D units; the fetches here go on behind them
+    auto first_fetches = [&]() {
+#pragma unroll
+        for (int i = 0; i < D; i++) {
+            if constexpr (SEAM::TAKES_RING) advance();
+            else fetch(ring[i]);
         }
     };
 
@@ -184,10 +237,61 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
     uint32_t rope_position = 0;
     RopeOperands rope_held{0.0f, 1.0f, 0.0f};
     constexpr bool CHAINED = SEAM::SHARED_IN || SEAM::SHARED_OUT;  // one of several products of a launch
+    // the tag words of what this product reads and writes across a seam: the seam's number below the step's (a device word
+    // that the step's first kernel moves on, so that what the step before left in the same place never passes for fresh)
+    uint32_t tag_in = 0, tag_out = 0;
     float residual_held = 0.0f;  // chained: the residual of this workgroup's first tile (lanes 0..15), asked for ahead
     auto rope_row = [half_width, tiles_per_head, lane](uint32_t tile, uint32_t &c) -> uint32_t {
         c = (tile % tiles_per_head) * 8u + (lane & 7u);
         return (tile / tiles_per_head) * (2u * half_width) + c + ((lane >> 3) & 1u) * half_width;
+    };
+
+    // ---- handed-over planes (HANDED): one 16-byte piece a lane and super-block, into the LDS layout the walk reads
+    constexpr int LATE = HANDED && SEAM::SHARED_IN ? 3 : 0;  // super-blocks a wave may look at only when its walk reaches them
+    u32x4 late_held[LATE > 0 ? LATE : 1];
+    uint32_t late_count = 0, early_count = 0;
+    const uint32_t chunk = lane >> 2, piece = lane & 3u;
+    auto handed_load = [&](uint32_t b, bool past) -> u32x4 {
+        if constexpr (SEAM::SHARED_IN) return tile16_load16_either(lead_input, b * TILE16_BLOCK_HANDED + lane * 16u, past);
+        else return tile16_load16<false>(lead_input, b * TILE16_BLOCK_HANDED + lane * 16u);
+    };
+    auto handed_put = [&](uint32_t b, const u32x4 &held) {
+        uint8_t *planes = digits + (size_t)b * TILE16_BLOCK_DIGITS + chunk * 48u;
+        uint8_t *const pairs = reinterpret_cast<uint8_t *>(sums);
+        if (piece == 0u) {
+            *reinterpret_cast<u32x4 *>(planes) = held;
+        } else if (piece == 1u) {
+            *reinterpret_cast<uint2 *>(planes + 16u) = uint2{held.x, held.y};
+            *reinterpret_cast<uint32_t *>(planes + 24u) = held.z;
+        } else if (piece == 2u) {
+            *reinterpret_cast<uint32_t *>(planes + 28u) = held.x;
+            *reinterpret_cast<uint2 *>(planes + 32u) = uint2{held.y, held.z};
+            *reinterpret_cast<uint32_t *>(planes + 40u) = held.w;
+        } else {
+            *reinterpret_cast<uint32_t *>(planes + 44u) = held.x;
+            *reinterpret_cast<uint2 *>(pairs + (size_t)b * TILE16_BLOCK_PAIRS + chunk * 8u) = uint2{held.y, held.z};
+        }
+    };
+    // the late super-blocks' planes: read again past the L2 while any is stale, then put where the walk reads them
+    auto late_stage = [&]() {
+        if constexpr (LATE > 0) {
+            for (uint32_t turn = 0;; turn++) {
+                bool stale = false;
+#pragma unroll
+                for (int l = 0; l < LATE; l++) stale = stale || ((uint32_t)l < late_count && (piece & 1u) && late_held[l].w != tag_in);
+                if (__builtin_amdgcn_ballot_w64(stale) == 0 && seam.spin) break;
+                if (turn >= seam.spin) {
+                    if (lane == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_SEAM);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+                for (int l = 0; l < LATE; l++) late_held[l] = handed_load(min(wave + NW * (early_count + l), nblk - 1u), true);
+            }
+#pragma unroll
+            for (int l = 0; l < LATE; l++)
+                if ((uint32_t)l < late_count) handed_put(wave + NW * (early_count + l), late_held[l]);
+        }
     };
 
     // ---- activations -> three signed base-256 digit planes per 16 elements, a power-of-two scale per 64-element group.
@@ -239,41 +343,63 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
             if ((e4 & 15u) == 0) s[2] = unscale;
         };
         if constexpr (HANDED) {
-            // a wave copies the super-blocks it walks, one 16-byte load a lane and block: lane 4 c + part holds plane `part` of
-            // chunk c, or with part 3 the chunk's pair
+            // a wave copies the super-blocks it walks, one 16-byte load a lane and block.
+            // A chunk of 16 activations is 64 bytes in memory, two sectors that each end in a tag word:
+            //   words 0..3 plane 0 | 4..6 plane 1, first twelve | 7 tag || 8 plane 1, last four | 9..11 plane 2, first twelve |
+            //   12 plane 2, last four | 13, 14 the (sum, scale) pair | 15 tag
+            // lane 4 c + piece holds words 4 piece .. 4 piece + 3 of chunk c
             constexpr int MAXB = NW <= 8 ? 10 : 5;  // super-blocks a wave copies at once: ffn_down at eight waves has ten, all asked for together
-            uint8_t *const pairs = reinterpret_cast<uint8_t *>(sums);
-            const uint32_t chunk = lane >> 2, piece = lane & 3u;
             if constexpr (SEAM::WAITS) {
-                // behind a seam: the first weights are asked for, then the planes wait for the product that writes them
-#pragma unroll
-                for (int i = 0; i < D; i++) fetch(ring[i]);
+                // behind a seam: the first weights are asked for before the planes, which may not be there yet
+                first_fetches();
                 fetch_the_rest();
-                if (!seam.wait(tid)) return false;
             }
-            for (uint32_t j0 = 0; j0 < count; j0 += MAXB) {
+            if constexpr (SEAM::SHARED_IN) tag_in = p.tag_in + 128u * *p.tick;
+            // Behind a seam the planes of a wave's last super-blocks may be the ones the product before writes last (p.late_from:
+            // the first such super-block): they are asked for with the others and looked at only when the walk reaches them,
+            // by which time they have long arrived -- the walk does not wait at its start for what it needs at its end.
+            if constexpr (LATE > 0) {
+                uint32_t late = 0;
+                for (uint32_t j = 0; j < count; j++) late += wave + NW * j >= p.late_from ? 1u : 0u;
+                late_count = min(late, (uint32_t)LATE);
+            }
+            const uint32_t early = count - late_count;
+            early_count = early;
+            for (uint32_t j0 = 0; j0 < early || (j0 == 0 && LATE > 0); j0 += MAXB) {
                 u32x4 held[MAXB];
+                for (uint32_t turn = 0;; turn++) {
 #pragma unroll
-                for (int j = 0; j < MAXB; j++) {
-                    uint32_t b = min(wave + NW * (j0 + j), nblk - 1u);
-                    held[j] = tile16_load16<SEAM::SHARED_IN>(lead_input, b * TILE16_BLOCK_HANDED + lane * 16u);
-                }
-                if (!SEAM::WAITS && j0 == 0) {
+                    for (int j = 0; j < MAXB; j++) {
+                        const uint32_t b = min(wave + NW * min(j0 + j, early ? early - 1u : 0u), nblk - 1u);
+                        held[j] = handed_load(b, turn > 0);
+                    }
+                    if (j0 == 0 && turn == 0) {
+                        if constexpr (LATE > 0) {
 #pragma unroll
-                    for (int i = 0; i < D; i++) fetch(ring[i]);
-                    fetch_the_rest();
+                            for (int l = 0; l < LATE; l++) late_held[l] = handed_load(min(wave + NW * (early + l), nblk - 1u), false);
+                        }
+                        if constexpr (!SEAM::WAITS) {
+                            first_fetches();
+                            fetch_the_rest();
+                        }
+                    }
+                    if constexpr (!SEAM::SHARED_IN) break;
+                    bool stale = false;
+#pragma unroll
+                    for (int j = 0; j < MAXB; j++) stale = stale || ((piece & 1u) && held[j].w != tag_in);
+                    if ((__builtin_amdgcn_ballot_w64(stale) == 0 || early == 0) && seam.spin) break;  // (no turns at all: the tests' way to the refusal)
+                    if (turn >= seam.spin) {
+                        if (lane == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_SEAM);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
                 }
 #pragma unroll
-                for (int j = 0; j < MAXB; j++) {
-                    const uint32_t b = wave + NW * (j0 + j);
-                    if (b >= nblk) continue;
-                    if (piece < 3u) *reinterpret_cast<u32x4 *>(digits + (size_t)b * TILE16_BLOCK_DIGITS + chunk * 48u + piece * 16u) = held[j];
-                    else *reinterpret_cast<uint2 *>(pairs + (size_t)b * TILE16_BLOCK_PAIRS + chunk * 8u) = uint2{held[j].x, held[j].y};
-                }
+                for (int j = 0; j < MAXB; j++)
+                    if (j0 + j < early) handed_put(wave + NW * (j0 + j), held[j]);
             }
-            if (!SEAM::WAITS && count == 0) {
-#pragma unroll
-                for (int i = 0; i < D; i++) fetch(ring[i]);
+            if (!SEAM::WAITS && LATE == 0 && count == 0) {
+                first_fetches();
                 fetch_the_rest();
             }
             if (CHAINED && p.residual && q == 0 && r < tile_rows)
@@ -281,8 +407,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
         } else if constexpr (R > 1) {
             // the weights' loads go out first; every row's activations follow (twice where the norm is folded in: once for
             // the row's sum of squares, once for the digits -- the second pass finds them in the cache)
-#pragma unroll
-            for (int i = 0; i < D; i++) fetch(ring[i]);
+            first_fetches();
             fetch_the_rest();
             const uint32_t rows = min(p.rows, (uint32_t)R);
             if (lead_norm_w) {
@@ -317,17 +442,48 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
         const bool resident = units <= MAXJ * NT;
         float rms = 1.0f;
         if constexpr (SEAM::WAITS) {
-            // behind a seam: the first weights are asked for, then the activations wait for the product that writes them
-#pragma unroll
-            for (int i = 0; i < D; i++) fetch(ring[i]);
+            // behind a seam: the first weights are asked for before the activations, which may not be there yet
+            first_fetches();
             fetch_the_rest();
-            if (!seam.wait(tid)) return false;
         }
-        if (resident) {
+        if constexpr (SEAM::SHARED_IN) {
+            tag_in = p.tag_in + 128u * *p.tick;
+            // the row arrives as (value, tag) pairs of eight bytes, written as one by the product before: four activations
+            // are two 16-byte loads, read again until every pair of the wave carries this seam's tag (launch_chain takes no
+            // row that does not fit the registers)
+            if (lead_norm_w) {
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    weight[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            for (uint32_t turn = 0;; turn++) {
+                bool stale = false;
+#pragma unroll
+                for (int j = 0; j < MAXJ; j++) {
+                    const uint32_t e4 = tid + NT * j;
+                    held[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    if (e4 < units) {
+                        const u32x4 low = tile16_load16_either(lead_input, 32u * e4, turn > 0), high = tile16_load16_either(lead_input, 32u * e4 + 16u, turn > 0);
+                        // (each word is copied to a scalar first: the bits of a vector element taken in place read element 0 every time)
+                        const uint32_t v0 = low.x, v1 = low.z, v2 = high.x, v3 = high.z;
+                        held[j] = f32x4{__builtin_bit_cast(float, v0), __builtin_bit_cast(float, v1), __builtin_bit_cast(float, v2), __builtin_bit_cast(float, v3)};
+                        stale = stale || low.y != tag_in || low.w != tag_in || high.y != tag_in || high.w != tag_in;
+                    }
+                }
+                if (__builtin_amdgcn_ballot_w64(stale) == 0 && seam.spin) break;  // (no turns at all: the tests' way to the refusal)
+                if (turn >= seam.spin) {
+                    if (lane == 0) atomicMax(p.refusal, (uint32_t)REFUSAL_SEAM);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        } else if (resident) {
 #pragma unroll
             for (int j = 0; j < MAXJ; j++) {
                 const uint32_t e4 = tid + NT * j;
-                held[j] = e4 < units ? tile16_load4<SEAM::SHARED_IN>(x, 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                held[j] = e4 < units ? *reinterpret_cast<const f32x4 *>(x + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
             if (lead_norm_w) {
 #pragma unroll
@@ -339,8 +495,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
         }
         // the weights' loads go out behind the activations', which everything waits for first
         if constexpr (!SEAM::WAITS) {
-#pragma unroll
-            for (int i = 0; i < D; i++) fetch(ring[i]);
+            first_fetches();
             fetch_the_rest();
         }
         if (MODE == TILE16_ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
@@ -357,7 +512,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(held[j][i], held[j][i]));
             } else {
                 for (uint32_t e4 = tid; e4 < units; e4 += NT) {
-                    const f32x4 v = tile16_load4<SEAM::SHARED_IN>(x, 4u * e4);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(x + 4u * e4);
 #pragma unroll
                     for (int i = 0; i < 4; i++) square = __fadd_rn(square, __fmul_rn(v[i], v[i]));
                 }
@@ -379,7 +534,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
             }
         } else {
             for (uint32_t e4 = tid; e4 < units; e4 += NT)
-                stage(e4, tile16_load4<SEAM::SHARED_IN>(x, 4u * e4), lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
+                stage(e4, *reinterpret_cast<const f32x4 *>(x + 4u * e4), lead_norm_w ? *reinterpret_cast<const f32x4 *>(lead_norm_w + 4u * e4) : f32x4{0.f, 0.f, 0.f, 0.f}, rms,
                       digits, sums);
         }
         }
@@ -390,6 +545,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
         const uint32_t n = rope_row(tile_at(0), c);
         rope_held = rope_operands(p, n, c, rope_position);
     }
+    if (SEAM::SHARED_OUT || (MODE == TILE16_SWIGLU && R == 1)) tag_out = p.tag_out + (p.tick ? 128u * *p.tick : 0u);
 
     // ---- the walk
     const ScaleLane lane_scales = scale_lane(q);
@@ -587,14 +743,17 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
                     chunk_sum += dpp<DPP_ROW_ROR4>(chunk_sum);
                     chunk_sum += dpp<DPP_ROW_ROR8>(chunk_sum);
                     const int dg = (int)signed_digits((int)rounded);
-                    // lane l writes word l of the chunk's 64 bytes: words 0..3 the most significant digits of elements 4 l ..,
-                    // 4..7 the middle ones, 8..11 the least significant, 12 and 13 the pair
-                    const int first = (int)(r & 3u) * 4;
+                    // lane l writes word l of the chunk's 64 bytes (the layout the reader of handed planes states): four digits of
+                    // one plane, a word of the pair, or -- words 7 and 15, the last of each 32-byte sector -- the tag
+                    const uint32_t plane = r < 4u ? 0u : (r < 9u ? 1u : 2u);
+                    const int first = (int)(r < 4u ? 4u * r : (r < 7u ? 4u * (r - 4u) : (r == 8u || r == 12u ? 12u : 4u * (r - 9u)))) & 15;
                     const uint32_t d0 = (uint32_t)__shfl(dg, first, 16), d1 = (uint32_t)__shfl(dg, first + 1, 16);
                     const uint32_t d2 = (uint32_t)__shfl(dg, first + 2, 16), d3 = (uint32_t)__shfl(dg, first + 3, 16);
-                    const uint32_t plane = r >> 2, shift = 16u - 8u * min(plane, 2u);
+                    const uint32_t shift = 16u - 8u * plane;
                     uint32_t word = ((d0 >> shift) & 0xffu) | (((d1 >> shift) & 0xffu) << 8) | (((d2 >> shift) & 0xffu) << 16) | (((d3 >> shift) & 0xffu) << 24);
-                    if (plane == 3u) word = r == 12u ? __builtin_bit_cast(uint32_t, chunk_sum * unscale) : (r == 13u ? __builtin_bit_cast(uint32_t, unscale) : 0u);
+                    if (r == 13u) word = __builtin_bit_cast(uint32_t, chunk_sum * unscale);
+                    if (r == 14u) word = __builtin_bit_cast(uint32_t, unscale);
+                    if (r == 7u || r == 15u) word = tag_out;
                     tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u) + r, word);
                 } else {
                     tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.y + (size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r),
@@ -615,7 +774,13 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
                     // residual read at device scope (the first tile's was asked for ahead) and the sum stored at device scope
                     float old = 0.0f;
                     if (p.residual) old = index == 0 ? residual_held : __hip_atomic_load(p.residual + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    tile16_store_word<true>(reinterpret_cast<uint32_t *>(p.y + n), __builtin_bit_cast(uint32_t, old + total));
+                    const float value = old + total;
+                    tile16_store_word<true>(reinterpret_cast<uint32_t *>(p.y + n), __builtin_bit_cast(uint32_t, value));
+                    // for the product behind the seam: the number with the seam's tag beside it, eight bytes stored as one
+                    if (SEAM::SHARED_OUT && p.pairs_out)
+                        __hip_atomic_store(reinterpret_cast<unsigned long long *>(p.pairs_out) + n,
+                                           (unsigned long long)__builtin_bit_cast(uint32_t, value) | ((unsigned long long)tag_out << 32), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
                 } else if (p.residual == p.y) {
                     // in place (the decoder's residual stream): one add per element, nothing to wait for
                     unsafeAtomicAdd(p.y + n, total);
@@ -629,7 +794,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
     };
     if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
         for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t), t);
-        return true;
+        return;
     }
     // Every wave walks whole rounds of D steps: the steps past its last tile multiply what was fetched again and publish nothing.
     uint32_t at_tile = 0, at_b = wave;
@@ -640,6 +805,7 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
             if constexpr (R > 1) {
                 step_rows(ring[slot], at_b);
             } else if constexpr (HANDED) {
+                if (LATE > 0 && late_count && s0 + slot == early_count) late_stage();
                 HandedStep st;
                 multiply_handed(ring[slot], at_b, st);
                 __builtin_amdgcn_sched_barrier(0);
@@ -662,7 +828,6 @@ __device__ __forceinline__ bool tile16_product(uint8_t *tile16_lds_bytes, const 
             }
         }
     }
-    return true;
 }
 
 // The leading arguments are what a wave needs before it can ask for its first activations and weights.  They are plain words
@@ -674,7 +839,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t 
                                                                   int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
                                                                   uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
-    tile16_product<NW, D, MODE, R, HANDED>(tile16_lds_bytes, blockIdx.x, NoSeam{}, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes, lead_grid,
+    Tile16Unit ring[D];
+    tile16_product<NW, D, MODE, R, HANDED>(tile16_lds_bytes, blockIdx.x, NoSeam{}, ring, nullptr, 0u, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes, lead_grid,
                                            lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
 }
 
@@ -1213,6 +1379,9 @@ static Tile16Launch tile16_plan(nh_device *d, const GemvArgs &a, uint32_t fixed_
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
     p.N = a.N, p.K = a.K, p.swiglu = a.swiglu, p.eps = a.eps, p.rows = a.rows;
     p.digits_out = a.digits_out, p.digits_in = a.digits_in;
+    p.tick = d->tick, p.tag_in = a.tag_in, p.tag_out = a.tag_out, p.pairs_out = static_cast<uint2 *>(a.pairs_out);
+    p.late_from = 0xffffffffu;
+    p.refusal = d->refusal;
 
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     p.nblk = a.K / 256u;
@@ -1271,15 +1440,9 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
 // Several dependent one-row products in one launch (crates/neura-kernel/src/scheduler.rs:110-166 runs a whole program as one
 // persistent kernel; here it is the products between two attentions of a decode step: attn_output, gate|up, ffn_down and the
 // q|k|v product of the layer behind, or the head).  One workgroup of eight waves a compute unit, all resident at once; every
-// stage is the 16-row tile product above.  At a seam a workgroup
-//   - waits until its own stores of the stage before have been acknowledged (s_waitcnt vmcnt(0); they went out at device
-//     scope, so they are in memory by then), meets at a barrier and publishes `epoch` in its own flag word;
-//   - asks for its first weights of the next stage -- they depend on nothing, so HBM streams through the wait;
-//   - wave 0 reads all the flag words (sixteen bytes a lane) until every one holds the epoch, at most `spin` times: a wait
-//     that runs out writes REFUSAL_SEAM and the whole workgroup leaves, as then does every other one (the host runs the step
-//     again, one launch a product);
-//   - reads its activations at device scope and walks.
-// Flag words only grow within a step; the step's first kernel clears them.
+// stage is the 16-row tile product above, with the seams its comment describes: a workgroup walks from one product into the
+// next with nothing between them but a barrier of its own waves (they share LDS), asks for the next product's first
+// weights, and reads its activations as tagged pieces until they are this step's.
 struct ChainStage {
     const uint8_t *w0;
     const void *input;
@@ -1291,127 +1454,120 @@ struct ChainStage {
 constexpr int CHAIN_STAGES_MOST = 4;
 struct ChainParams {
     ChainStage stage[CHAIN_STAGES_MOST];
-    uint32_t *flags;    // one word a workgroup
-    uint32_t *refusal;
-    uint32_t epoch;     // what the first seam of this launch publishes; the next one epoch + 1, ...
-    uint32_t spin;      // reads of the flag words a wait may take
-    uint32_t lds_bytes; // of the launch: the seam's word sits in its last sixteen bytes
+    uint32_t spin;  // times a reader may read a stale piece again
+    uint32_t stages;  // bit s: stage s runs (all of them, unless a test splits a chain over several launches)
+    uint32_t second_lds;  // where ffn_down's part of LDS begins, behind the other products'
 };
 
-template <bool WAITS_, bool IN_, bool OUT_>
+template <bool WAITS_, bool IN_, bool OUT_, bool HANDS_ = false, bool TAKES_ = false>
 struct ChainSeam {
-    static constexpr bool WAITS = WAITS_, SHARED_IN = IN_, SHARED_OUT = OUT_;
-    const uint32_t *flags;
-    uint32_t *refusal;
-    uint32_t *word;  // in LDS
-    uint32_t epoch, spin, workgroups;
-    __device__ __forceinline__ bool wait(uint32_t tid) const {
-        if constexpr (!WAITS_) return true;
-        if (tid < 64u) {
-            bool met = false;
-            for (uint32_t turn = 0; turn < spin && !met; turn++) {
-                const u32x4 held = tile16_load16<true>(flags, tid * 16u);
-                bool here = true;
-#pragma unroll
-                for (int i = 0; i < 4; i++) here = here && (4u * tid + i >= workgroups || held[i] >= epoch);
-                met = __builtin_amdgcn_ballot_w64(!here) == 0;
-                if (!met) __builtin_amdgcn_s_sleep(2);
-            }
-            if (tid == 0) *word = met ? 1u : 0u;
-        }
-        __syncthreads();
-        const bool met = *word != 0u;
-        if (!met && tid == 0) atomicMax(refusal, (uint32_t)REFUSAL_SEAM);
-        return met;
-    }
+    static constexpr bool WAITS = WAITS_, SHARED_IN = IN_, SHARED_OUT = OUT_, HANDS_RING = HANDS_, TAKES_RING = TAKES_;
+    uint32_t spin;
 };
-
-// a workgroup's stores of the stage before are in memory, and it says so
-__device__ __forceinline__ void chain_arrive(uint32_t *flags, uint32_t block, uint32_t epoch) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_store(flags + block, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 enum ChainProgram { CHAIN_FFN = 0, CHAIN_O_FFN = 1, CHAIN_O_FFN_QKV = 2, CHAIN_O_FFN_HEAD = 3 };
 
 #define CHAIN_STAGE_ARGUMENTS(s) (s).w0, (s).input, (s).norm_w, (s).to_w1, (s).to_w2, (s).row_bytes, (s).grid, (s).tiles, (s).tile_rows, (s).end0, (s).end1, (s).p
 
+// this lane's weight row in the first tile workgroup `block` walks of a plain one-matrix stage (nullptr: it walks none)
+__device__ __forceinline__ const uint8_t *chain_first_row(const ChainStage &stage, uint32_t block) {
+    if (block >= stage.tiles || block >= stage.grid) return nullptr;
+    const uint32_t lane = threadIdx.x & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t n = block * stage.tile_rows + min(r, stage.tile_rows - 1u);
+    return stage.w0 + (size_t)n * stage.row_bytes + q * 32u;
+}
+
 template <int PROGRAM>
 __global__ __launch_bounds__(512) void gemv_q4k_chain_kernel(ChainParams c) {
     extern __shared__ __attribute__((aligned(16))) uint8_t chain_lds_bytes[];
-    constexpr bool LEADS = PROGRAM != CHAIN_FFN;                               // attn_output in front
+    constexpr bool LEADS = PROGRAM != CHAIN_FFN;                                        // attn_output in front
     constexpr bool TRAILS = PROGRAM == CHAIN_O_FFN_QKV || PROGRAM == CHAIN_O_FFN_HEAD;  // a product behind ffn_down
-    const uint32_t block = blockIdx.x, workgroups = gridDim.x;
-    uint32_t *const word = reinterpret_cast<uint32_t *>(chain_lds_bytes + c.lds_bytes - 16u);
-    uint32_t epoch = c.epoch;
+    const uint32_t block = blockIdx.x;
+    Tile16Unit ring[2];
     int at = 0;
     if constexpr (LEADS) {
-        // attn_output: x is the attention's output (the launch before), y = h += ... is read by gate|up
-        const ChainSeam<false, false, true> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
-        tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]));
-        chain_arrive(c.flags, block, epoch);
+        // attn_output: x is the attention's output (the launch before); y = h + ..., which gate|up reads as tagged pairs
+        if (c.stages & 1u)
+            tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, ChainSeam<false, false, true>{c.spin}, ring, nullptr, 0u,
+                                                         CHAIN_STAGE_ARGUMENTS(c.stage[at]));
+        __syncthreads();  // these two products stage their activations in the same part of LDS
         at++;
     }
-    {
-        // gate|up with SwiGLU: reads h, leaves digit planes
-        const ChainSeam<LEADS, LEADS, true> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
-        if (!tile16_product<8, 2, TILE16_SWIGLU, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
-        if (LEADS) epoch++;
-        chain_arrive(c.flags, block, epoch);
-        at++;
+    // gate|up with SwiGLU: leaves tagged digit planes; past its last unit its ring asks for ffn_down's first weights
+    const ChainStage &down = c.stage[at + 1];
+    if (c.stages & (1u << at))
+        tile16_product<8, 2, TILE16_SWIGLU, 1, false>(chain_lds_bytes, block, ChainSeam<LEADS, LEADS, true, true, false>{c.spin}, ring,
+                                                      chain_first_row(down, block), down.row_bytes / 144u, CHAIN_STAGE_ARGUMENTS(c.stage[at]));
+    at++;
+    // ffn_down over the digit planes, h += ...: in a part of LDS of its own (no wave waits for another between the two
+    // products), its first weights in flight, the planes of its last super-blocks looked at when the walk reaches them
+    if (c.stages & (1u << at)) {
+        if (c.stages & (1u << (at - 1)))
+            tile16_product<8, 2, TILE16_PLAIN, 1, true>(chain_lds_bytes + c.second_lds, block, ChainSeam<false, true, TRAILS, false, true>{c.spin}, ring, nullptr, 0u,
+                                                        CHAIN_STAGE_ARGUMENTS(c.stage[at]));
+        else  // (a launch of this stage alone: nothing handed it a ring)
+            tile16_product<8, 2, TILE16_PLAIN, 1, true>(chain_lds_bytes + c.second_lds, block, ChainSeam<false, true, TRAILS, false, false>{c.spin}, ring, nullptr, 0u,
+                                                        CHAIN_STAGE_ARGUMENTS(c.stage[at]));
     }
-    {
-        // ffn_down over the digit planes, h += ...
-        const ChainSeam<true, true, TRAILS> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
-        if (!tile16_product<8, 2, TILE16_PLAIN, 1, true>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
-        at++;
-    }
+    at++;
     if constexpr (TRAILS) {
-        epoch++;
-        chain_arrive(c.flags, block, epoch);
-        const ChainSeam<true, true, false> seam{c.flags, c.refusal, word, epoch, c.spin, workgroups};
-        if constexpr (PROGRAM == CHAIN_O_FFN_QKV) {
-            if (!tile16_product<8, 2, TILE16_ROPE, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
-        } else {
-            if (!tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, seam, CHAIN_STAGE_ARGUMENTS(c.stage[at]))) return;
-        }
+        // (every wave that gets here has passed ffn_down's barrier, which none reaches before it is done with gate|up's LDS)
+        if constexpr (PROGRAM == CHAIN_O_FFN_QKV)
+            tile16_product<8, 2, TILE16_ROPE, 1, false>(chain_lds_bytes, block, ChainSeam<true, true, false>{c.spin}, ring, nullptr, 0u, CHAIN_STAGE_ARGUMENTS(c.stage[at]));
+        else
+            tile16_product<8, 2, TILE16_PLAIN, 1, false>(chain_lds_bytes, block, ChainSeam<true, true, false>{c.spin}, ring, nullptr, 0u, CHAIN_STAGE_ARGUMENTS(c.stage[at]));
     }
 }
 
 static bool chain_stage_takes(const GemvArgs &a) {
     if (!tile16_takes(a) || a.rows != 1) return false;
-    return tile16_lds(a.K / 256u, 8u, 1u, a.digits_in != nullptr) + 16u <= 160u * 1024u;
+    return tile16_lds(a.K / 256u, 8u, 1u, a.digits_in != nullptr) <= 160u * 1024u;
 }
 
 // Whether launch_chain takes these products as one launch: attn_output (or none), gate|up handing its digits to ffn_down, and
-// behind them the next q|k|v with the rotation folded in, or the head (or none).  NEURA_HIP_CHAIN: 0 keeps one launch a product,
-// 1 chains gate|up and ffn_down, 2 (the default) attn_output in front of them, 3 the product behind them as well.
+// behind them the next q|k|v with the rotation folded in, or the head (or none).  NEURA_HIP_CHAIN: 0 (the default: measured, the
+// chained launch takes as long as its products one by one and a little more) keeps one launch a product, 1 chains gate|up and
+// ffn_down, 2 attn_output in front of them, 3 the product behind them as well.
+int gemv_chain_level() { return env_int("NEURA_HIP_CHAIN", 0); }
+
 bool gemv_chains(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail) {
-    const int wanted = env_int("NEURA_HIP_CHAIN", 2);
-    if (wanted <= 0 || !d->chain_flags || d->compute_units > 256 || d->compute_units < 1) return false;
+    const int wanted = gemv_chain_level();
+    if (wanted <= 0 || !d->tick || d->compute_units < 1) return false;
     if (lead && wanted < 2) return false;
     if (trail && wanted < 3) return false;
-    if (!gate_up.digits_out || !down.digits_in || gate_up.digits_out != down.digits_in) return false;
+    if (!gate_up.digits_out || !down.digits_in || gate_up.digits_out != down.digits_in || !gate_up.tag_out || gate_up.tag_out != down.tag_in) return false;
     if (!chain_stage_takes(gate_up) || !chain_stage_takes(down)) return false;
-    if (lead && (!chain_stage_takes(*lead) || lead->swiglu || lead->rope || lead->digits_in || lead->digits_out)) return false;
-    if (trail && (!chain_stage_takes(*trail) || trail->swiglu || trail->digits_in || trail->digits_out || trail->residual)) return false;
+    // the ring handed across the seam holds the first two units of every wave of ffn_down's first tile
+    if (down.K / 256u < 16u) return false;
+    if (tile16_lds(gate_up.K / 256u, 8u, 1u, false) + 256u + tile16_lds(down.K / 256u, 8u, 1u, true) > 160u * 1024u) return false;
+    if (lead && tile16_lds(lead->K / 256u, 8u, 1u, false) + 256u + tile16_lds(down.K / 256u, 8u, 1u, true) > 160u * 1024u) return false;
+    if (trail && tile16_lds(trail->K / 256u, 8u, 1u, false) + 256u + tile16_lds(down.K / 256u, 8u, 1u, true) > 160u * 1024u) return false;
+    // a row handed on as (value, tag) pairs is held in registers while its reader looks at the tags: five units of four a thread
+    constexpr uint32_t HELD_MOST = 5u * 512u * 4u;
+    if (lead) {
+        if (!chain_stage_takes(*lead) || lead->swiglu || lead->rope || lead->digits_in || lead->digits_out) return false;
+        if (!lead->pairs_out || lead->pairs_out != (const void *)gate_up.x || !lead->tag_out || lead->tag_out != gate_up.tag_in || gate_up.K > HELD_MOST) return false;
+    }
+    if (trail) {
+        if (!chain_stage_takes(*trail) || trail->swiglu || trail->digits_in || trail->digits_out || trail->residual) return false;
+        if (!down.pairs_out || down.pairs_out != (const void *)trail->x || !down.tag_out || down.tag_out != trail->tag_in || trail->K > HELD_MOST) return false;
+    }
     return true;
 }
 
 template <int PROGRAM>
-static hipError_t launch_chain_program(nh_device *d, const ChainParams &c, uint32_t grid) {
+static hipError_t launch_chain_program(nh_device *d, const ChainParams &c, uint32_t grid, size_t lds) {
     static bool raised = false;
     if (!raised) {
         hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_chain_kernel<PROGRAM>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_chain_kernel<PROGRAM>), dim3(grid), dim3(512), c.lds_bytes, d->stream, c);
+    hipLaunchKernelGGL((gemv_q4k_chain_kernel<PROGRAM>), dim3(grid), dim3(512), lds, d->stream, c);
     return hipGetLastError();
 }
 
-int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t epoch, uint32_t spin) {
+int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t spin) {
     ChainParams c{};
     const GemvArgs *stages[CHAIN_STAGES_MOST] = {nullptr, nullptr, nullptr, nullptr};
     int count = 0;
@@ -1419,10 +1575,17 @@ int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up
     stages[count++] = &gate_up;
     stages[count++] = &down;
     if (trail) stages[count++] = trail;
-    size_t lds = 0;
+    size_t lds = 0, lds_down = 0;
     uint64_t bytes = 0;
+    uint32_t late_from = 0xffffffffu;
     for (int s = 0; s < count; s++) {
-        const Tile16Launch plan = tile16_plan(d, *stages[s], 8u);
+        Tile16Launch plan = tile16_plan(d, *stages[s], 8u);
+        if (stages[s] == &gate_up) {
+            // the first of ffn_down's super-blocks that holds an output of gate|up's last round of pairs
+            const uint32_t pairs = plan.p.row_groups, last_round = (pairs - 1u) / plan.grid;
+            late_from = last_round * plan.grid / 16u;
+        }
+        if (stages[s] == &down) plan.p.late_from = late_from;
         const GemvParams &p = plan.p;
         ChainStage &stage = c.stage[s];
         stage.w0 = p.W[0];
@@ -1433,31 +1596,41 @@ int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up
         stage.tile_rows = stages[s]->rope ? p.rope_width : p.tile_rows;
         stage.end0 = p.end[0], stage.end1 = p.end[1];
         stage.p = p;
-        if (plan.lds > lds) lds = plan.lds;
+        if (stages[s] == &down) lds_down = plan.lds;
+        else if (plan.lds > lds) lds = plan.lds;
         bytes += (uint64_t)stages[s]->N * p.row_bytes;
     }
-    // one workgroup a compute unit: more LDS than two of them could share
-    lds += 16u;
+    // ffn_down stages its planes behind the other products' part of LDS; one workgroup a compute unit: more LDS than two of
+    // them could share
+    c.second_lds = (uint32_t)((lds + 255u) / 256u * 256u);
+    lds = c.second_lds + lds_down;
     if (lds < 84u * 1024u) lds = 84u * 1024u;
-    c.flags = d->chain_flags, c.refusal = d->refusal, c.epoch = epoch, c.spin = spin, c.lds_bytes = (uint32_t)lds;
+    c.spin = spin;
     const uint32_t grid = (uint32_t)d->compute_units;
     profile_mark(d);
-    hipError_t launched;
-    if (!lead) launched = launch_chain_program<CHAIN_FFN>(d, c, grid);
-    else if (!trail) launched = launch_chain_program<CHAIN_O_FFN>(d, c, grid);
-    else if (trail->rope) launched = launch_chain_program<CHAIN_O_FFN_QKV>(d, c, grid);
-    else launched = launch_chain_program<CHAIN_O_FFN_HEAD>(d, c, grid);
+    hipError_t launched = hipSuccess;
+    // NEURA_HIP_CHAIN_SPLIT=1 (a test's switch): every stage a launch of its own of the same kernel, the seams' tags unchanged
+    const bool split = env_int("NEURA_HIP_CHAIN_SPLIT", 0) == 1;
+    for (int part = 0; part < (split ? count : 1) && launched == hipSuccess; part++) {
+        c.stages = split ? 1u << part : 0xffu;
+        if (!lead) launched = launch_chain_program<CHAIN_FFN>(d, c, grid, lds);
+        else if (!trail) launched = launch_chain_program<CHAIN_O_FFN>(d, c, grid, lds);
+        else if (trail->rope) launched = launch_chain_program<CHAIN_O_FFN_QKV>(d, c, grid, lds);
+        else launched = launch_chain_program<CHAIN_O_FFN_HEAD>(d, c, grid, lds);
+    }
     NH_HIP(launched);
     profile_mark(d);
     if (d->profile) d->profile_bytes += bytes;
     return NH_OK;
 }
 
-__global__ __launch_bounds__(256) void chain_clear_kernel(uint32_t *flags) { flags[threadIdx.x] = 0u; }
+__global__ __launch_bounds__(64) void tick_kernel(uint32_t *tick) {
+    if (threadIdx.x == 0) *tick = *tick + 1u;
+}
 
-int32_t launch_chain_clear(nh_device *d) {
-    if (!d->chain_flags) return NH_OK;
-    hipLaunchKernelGGL(chain_clear_kernel, dim3(1), dim3(256), 0, d->stream, d->chain_flags);
+int32_t launch_tick(nh_device *d) {
+    if (!d->tick) return NH_OK;
+    hipLaunchKernelGGL(tick_kernel, dim3(1), dim3(64), 0, d->stream, d->tick);
     NH_HIP(hipGetLastError());
     return NH_OK;
 }

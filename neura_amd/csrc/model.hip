@@ -47,7 +47,8 @@ struct nh_model {
     // Dependent products of a decode step as one launch with seams between them (launch_chain) until a seam's wait runs out
     // once: the step is then run again one launch a product, and so is every later one.
     bool chain = true;
-    uint32_t chain_spin = 1u << 18;  // reads of the flag words a seam's wait may take (NEURA_HIP_CHAIN_SPIN)
+    uint32_t chain_spin = 1u << 18;  // times a reader at a seam may read a stale piece again (NEURA_HIP_CHAIN_SPIN)
+    uint2 *pairs = nullptr;          // [hidden] (value, tag): the residual stream as a chained launch hands it from product to product
     uint32_t seam_fallbacks = 0;     // steps run again because a seam gave up
 };
 
@@ -75,6 +76,7 @@ void release(nh_model *m) {
     float *buffers[] = {m->h, m->xn, m->qkv, m->att, m->act, m->up, m->logits, m->rope_cos, m->rope_sin};
     for (float *p : buffers)
         if (p) (void)hipFree(p);
+    if (m->pairs) (void)hipFree(m->pairs);
     if (m->inputs_dev) (void)hipFree(m->inputs_dev);
     if (m->chosen_dev) (void)hipFree(m->chosen_dev);
     if (m->inputs_host) (void)hipHostFree(m->inputs_host);
@@ -131,9 +133,10 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
     const uint8_t *mask = any_inactive ? dev_mask(m) : nullptr;
     const bool wide = T > 8;  // more rows than the narrow product takes
     int32_t status;
-    uint32_t chain_launches = 0;
-    const bool chains = m->chain && T == 1 && !mask;
-    if (chains && (status = launch_chain_clear(d)) != NH_OK) return status;
+    const bool chains = m->chain && T == 1 && !mask && gemv_chain_level() > 0;
+    // what one product of a chained launch hands another carries tag words that name the pass: the device's tick moves on
+    // before any is written
+    if (chains && (status = launch_tick(d)) != NH_OK) return status;
     if (!products_only && (status = launch_gather(d, m->elements[EMBD], m->token_embd, c.vocab, H, dev_tokens(m), T, B, mask, m->h)) != NH_OK)
         return status;
     const float scale = 1.0f / sqrtf((float)hd);
@@ -269,6 +272,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             GemvArgs dn = narrow(m, element_at(m, L, DOWN), m->ffn_down[L], H, F, m->act, T, m->h);
             dn.residual = m->h;
             bool chained = false;
+            const uint32_t seam = 1u + 4u * (L % 31u);  // the numbers of this layer's seams: seam (h), seam + 1 (digit planes), ...
             if (chains && !o.merge && element_at(m, L, GATE) == element_at(m, L, UP)) {
                 GemvArgs gu = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], 2 * F, H, m->h, T, m->act);
                 gu.W[1] = m->ffn_up[L];
@@ -276,16 +280,20 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 gu.swiglu = 1, gu.norm_w = m->ffn_norm[L], gu.eps = c.eps;
                 if (gemv_hands_digits(gu, dn) && gemv_digit_bytes(F) <= (size_t)F * sizeof(float)) {
                     gu.digits_out = reinterpret_cast<uint8_t *>(m->up), dn.digits_in = reinterpret_cast<const uint8_t *>(m->up);
-                    const uint32_t epoch = 1u + CHAIN_EPOCHS_A_LAUNCH * chain_launches;
-                    if (gemv_chains(d, &o, gu, dn, nullptr)) {
-                        if ((status = launch_chain(d, &o, gu, dn, nullptr, epoch, m->chain_spin)) != NH_OK) return status;
-                        chained = true, chain_launches++;
+                    gu.tag_out = dn.tag_in = seam + 1u;
+                    // with attn_output in front, gate|up reads the residual stream as the pairs attn_output leaves beside it
+                    GemvArgs lead = o, behind = gu;
+                    lead.pairs_out = m->pairs, lead.tag_out = seam;
+                    behind.x = reinterpret_cast<const float *>(m->pairs), behind.tag_in = seam;
+                    if (gemv_chains(d, &lead, behind, dn, nullptr)) {
+                        if ((status = launch_chain(d, &lead, behind, dn, nullptr, m->chain_spin)) != NH_OK) return status;
+                        chained = true;
                     } else if (gemv_chains(d, nullptr, gu, dn, nullptr)) {
                         if ((status = launch_gemv(d, o)) != NH_OK) return status;
-                        if ((status = launch_chain(d, nullptr, gu, dn, nullptr, epoch, m->chain_spin)) != NH_OK) return status;
-                        chained = true, chain_launches++;
+                        if ((status = launch_chain(d, nullptr, gu, dn, nullptr, m->chain_spin)) != NH_OK) return status;
+                        chained = true;
                     }
-                    dn.digits_in = nullptr;
+                    dn.digits_in = nullptr, dn.tag_in = 0;
                 }
             }
             if (chained) continue;
@@ -298,7 +306,7 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 // one row: silu(gate) * up goes to the down projection as the digit planes it multiplies (they fit the up
                 // projection's idle buffer), not as floats it would turn into digits again
                 if (gemv_hands_digits(gu, dn) && gemv_digit_bytes(F) <= (size_t)F * sizeof(float))
-                    gu.digits_out = reinterpret_cast<uint8_t *>(m->up), dn.digits_in = reinterpret_cast<const uint8_t *>(m->up);
+                    gu.digits_out = reinterpret_cast<uint8_t *>(m->up), dn.digits_in = reinterpret_cast<const uint8_t *>(m->up), gu.tag_out = dn.tag_in = seam + 1u;
                 if ((status = launch_gemv(d, gu)) != NH_OK) return status;
             } else {
                 GemvArgs g = narrow(m, element_at(m, L, GATE), m->ffn_gate[L], F, H, m->h, T, m->act);
@@ -465,7 +473,9 @@ nh_model *nh_model_create(nh_device *device, const nh_model_config *config, nh_w
          device_array(m->att, T * QW) && device_array(m->act, T * F) && device_array(m->up, T * F) &&
          device_array(m->logits, (size_t)c.batch * c.vocab) && device_array(m->inputs_dev, T + 6 * c.batch + 4) &&
          device_array(m->chosen_dev, c.batch) && device_array(m->rope_cos, (size_t)m->positions * (c.head_dim / 2)) &&
-         device_array(m->rope_sin, (size_t)m->positions * (c.head_dim / 2));
+         device_array(m->rope_sin, (size_t)m->positions * (c.head_dim / 2)) && device_array(m->pairs, (size_t)H) &&
+         hipMemsetAsync(m->pairs, 0, (size_t)H * sizeof(uint2), device->stream) == hipSuccess &&
+         hipMemsetAsync(m->up, 0, T * F * sizeof(float), device->stream) == hipSuccess;
     for (uint32_t L = 0; ok && L < c.layers; L++) {
         uint8_t *k = nullptr, *v = nullptr;
         ok = device_array(k, m->cache_elements * m->eb);

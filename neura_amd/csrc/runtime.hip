@@ -73,7 +73,7 @@ int32_t check_refusal(nh_device *device, const char *what) {
     NH_HIP(hipMemsetAsync(device->refusal, 0, sizeof(word), device->stream));
     NH_HIP(hipStreamSynchronize(device->stream));
     switch (word) {
-    case REFUSAL_SEAM: return fail(NH_E_DEVICE, "%s: a workgroup of a chained launch gave up waiting for the others", what);
+    case REFUSAL_SEAM: return fail(NH_E_DEVICE, "%s: a product of a chained launch gave up waiting for the numbers of the product before", what);
     case REFUSAL_INDEX: return fail(NH_E_REFUSAL, "%s: a token id walks past the rows its table holds", what);
     case REFUSAL_ORIGIN: return fail(NH_E_REFUSAL, "%s: a cursor walks past the keys its cache holds", what);
     default: return fail(NH_E_REFUSAL, "%s: the device refused with code %u", what, word);
@@ -123,7 +123,7 @@ nh_device *nh_open(int32_t device_index) {
     bool ok = hipStreamCreateWithFlags(&device->stream, hipStreamNonBlocking) == hipSuccess &&
               hipEventCreate(&device->started) == hipSuccess && hipEventCreate(&device->stopped) == hipSuccess &&
               hipMalloc((void **)&device->refusal, 256) == hipSuccess && hipMemset(device->refusal, 0, 256) == hipSuccess &&
-              hipMalloc((void **)&device->chain_flags, 1024) == hipSuccess && hipMemset(device->chain_flags, 0, 1024) == hipSuccess;
+              hipMalloc((void **)&device->tick, 256) == hipSuccess && hipMemset(device->tick, 0, 256) == hipSuccess;
     if (!ok) {
         fail(NH_E_DEVICE, "device %d opens no stream, events or refusal word", device_index);
         nh_close(device);
@@ -143,7 +143,7 @@ void nh_close(nh_device *device) {
     if (device->scratch) (void)hipFree(device->scratch);
     for (void *block : device->retired) (void)hipFree(block);
     if (device->refusal) (void)hipFree(device->refusal);
-    if (device->chain_flags) (void)hipFree(device->chain_flags);
+    if (device->tick) (void)hipFree(device->tick);
     for (const nh_device::RopeTable &known : device->rope_tables) (void)hipFree(known.table);
     for (hipEvent_t event : device->profile_events) (void)hipEventDestroy(event);
     if (device->started) (void)hipEventDestroy(device->started);

@@ -608,18 +608,20 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         held.release()
 
 
-CHAIN_SHAPES = [SMALL_Q4, dict(layers=2, hidden=3584, heads=28, kv_heads=4, head_dim=128, ffn=18944, vocab=2048, tied=False)]
+# (a chained launch hands ffn_down's first weights across the seam: it takes rows of sixteen super-blocks and more)
+CHAIN_SMALL = dict(layers=2, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=4096, vocab=1000, tied=False)
+CHAIN_SHAPES = [CHAIN_SMALL, dict(layers=2, hidden=3584, heads=28, kv_heads=4, head_dim=128, ffn=18944, vocab=2048, tied=False)]
 
 
 @pytest.mark.parametrize("shape", CHAIN_SHAPES, ids=["small", "7b-layers"])
 @pytest.mark.parametrize("chain", ["1", "2"])
 def test_products_chained_into_one_launch_match_one_launch_a_product(device, monkeypatch, shape, chain):
-    """At batch 1 the products between two attentions run as one launch with seams between them (NEURA_HIP_CHAIN=1: gate|up
-    and ffn_down; 2: attn_output in front): what crosses a seam crosses it at device scope, behind a flag every workgroup
-    publishes.  The same steps one launch a product (NEURA_HIP_CHAIN=0) give the same logits to the last few bits (the chained
-    stages split a row's super-blocks over eight waves where the launches of their own take four or seven, so sums associate
-    differently), the same tokens and the same cache rows; both sit within the decoder's bar of the oracle.  No step fell
-    back."""
+    """At batch 1 the products between two attentions can run as one launch with seams between them (NEURA_HIP_CHAIN=1: gate|up
+    and ffn_down; 2: attn_output in front; the default is one launch a product).  What crosses a seam crosses it at device
+    scope and carries tag words: a reader that finds a piece without this step's tag reads it again.  The same steps one launch
+    a product (NEURA_HIP_CHAIN=0) give the same logits to the last few bits (the chained stages split a row's super-blocks over
+    eight waves where the launches of their own take four or seven, so sums associate differently), the same tokens and the
+    same cache rows; both sit within the decoder's bar of the oracle.  No step fell back."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
     tensors = list(synth.model_tensors(shape, NH_Q4_K, np.random.default_rng(21), mode="normal", threads=16))
     weights = Weights(device, tensors)
@@ -647,12 +649,13 @@ def test_products_chained_into_one_launch_match_one_launch_a_product(device, mon
 
 @pytest.mark.parametrize("graph", ["0", "1"])
 def test_a_seam_that_gives_up_sends_the_step_down_the_path_of_one_launch_a_product(device, monkeypatch, graph):
-    """NEURA_HIP_CHAIN_SPIN=0: every wait at a seam gives up before its first look (the kernels all end; no wait is ever
-    unbounded).  The step that met it is run again one launch a product and answers as the oracle does, the model counts one
-    fallback and stays on that path, eager or recorded."""
+    """NEURA_HIP_CHAIN_SPIN=0: every reader at a seam gives up before it looks twice (the kernels all end; no wait is ever
+    unbounded, and no wave leaves early).  The step that met it is run again one launch a product and answers as the oracle
+    does, the model counts one fallback and stays on that path, eager or recorded."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", graph)
+    monkeypatch.setenv("NEURA_HIP_CHAIN", "2")
     monkeypatch.setenv("NEURA_HIP_CHAIN_SPIN", "0")
-    model, ref, weights = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=40, seed=22)
+    model, ref, weights = build(device, CHAIN_SMALL, NH_Q4_K, batch=1, context=40, seed=22)
     monkeypatch.delenv("NEURA_HIP_CHAIN_SPIN")
     token = 5
     for step in range(5):
@@ -663,7 +666,7 @@ def test_a_seam_that_gives_up_sends_the_step_down_the_path_of_one_launch_a_produ
         assert model.seam_fallbacks() == 1, step
         token = int(got[0])
     # a model built without the hook chains, and never falls back
-    healthy, ref, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=40, seed=22)
+    healthy, ref, weights_b = build(device, CHAIN_SMALL, NH_Q4_K, batch=1, context=40, seed=22)
     token = 5
     for step in range(5):
         want_logits, want = ref.forward([token], 1, [step])
