@@ -191,6 +191,28 @@ def gemm_config3(device, rng, repeats=10):
     return out
 
 
+def decode_batch8(device, weights, shape, element, context, layers):
+    """Eight sequences at the end of their context stepping together: 4 warm-up steps, then 16 timed."""
+    from neura_amd.loader import Model
+
+    batch = 8
+    model = Model(device, weights, shape, element, batch=batch, context=context, layers=layers)
+    steps, warm = 16, 4
+    tokens = list(range(1, batch + 1))
+    first = context - (steps + warm)
+    for step in range(warm):
+        tokens = [int(t) for t in model.decode_step(tokens, [first + step] * batch)]
+    device.sync()
+    began = time.perf_counter()
+    for step in range(steps):
+        tokens = [int(t) for t in model.decode_step(tokens, [first + warm + step] * batch)]
+    device.sync()
+    elapsed = time.perf_counter() - began
+    model.release()
+    return {"value": batch * steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
+            "note": "8 planes, caches not pre-filled (zeros), cursors at the end of context %d" % context}
+
+
 def extras(device, weights, shape, element, context, layers, rng):
     """The other two measurements the workload names, on the same resident weights: decode at
     batch 8 (eight sequences at the end of their context) and a 512-token prompt fill."""
@@ -216,22 +238,7 @@ def extras(device, weights, shape, element, context, layers, rng):
                                     "note": "as the headline step with the greedy choice replaced by the sampled one; caches not pre-filled (zeros)"}
     model.release()
     note("extras: decode, batch 8")
-    batch = 8
-    model = Model(device, weights, shape, element, batch=batch, context=context, layers=layers)
-    steps, warm = 16, 4
-    tokens = list(range(1, batch + 1))
-    first = context - (steps + warm)
-    for step in range(warm):
-        tokens = [int(t) for t in model.decode_step(tokens, [first + step] * batch)]
-    device.sync()
-    began = time.perf_counter()
-    for step in range(steps):
-        tokens = [int(t) for t in model.decode_step(tokens, [first + warm + step] * batch)]
-    device.sync()
-    elapsed = time.perf_counter() - began
-    out["decode_batch8"] = {"value": batch * steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
-                            "note": "8 planes, caches not pre-filled (zeros), cursors at the end of context %d" % context}
-    model.release()
+    out["decode_batch8"] = decode_batch8(device, weights, shape, element, context, layers)
     note("extras: 512-token fill")
     out["prefill_512"] = fill_512(device, weights, shape, element, context, layers, rng)
     note("extras: wide product of configuration 3")
@@ -340,6 +347,7 @@ def main():
     parser.add_argument("--no-extras", action="store_true", help="skip the batch-8 decode, 512-token fill and wide-product measurements")
     parser.add_argument("--gemm-only", action="store_true", help="run only the wide product (M=512, K=3584, N=18944) and print its line")
     parser.add_argument("--fill-only", action="store_true", help="run only the 512-token fill of the workload and print its line")
+    parser.add_argument("--batch8-only", action="store_true", help="run only the 8-plane decode of the workload and print its line")
     parser.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                         help="also run one plain device-to-device copy of MIB MiB (a known-size reference for HBM byte counters)")
     args = parser.parse_args()
@@ -366,6 +374,11 @@ def main():
     note("weights resident")
     if args.fill_only:
         print(json.dumps({"prefill_512": fill_512(device, weights, shape, element, context, layers, rng)}))
+        weights.release()
+        device.close()
+        return
+    if args.batch8_only:
+        print(json.dumps({"decode_batch8": decode_batch8(device, weights, shape, element, context, layers)}))
         weights.release()
         device.close()
         return
@@ -433,6 +446,11 @@ def main():
                         (args.workload, layers, context, ("Q4_K" if element == 12 else "Q8_0") + (" and Q6_K" if mixed else ""),
                          ", sampled choice" if args.sampled else ""),
             "weight_bytes_per_token": weight_bytes_per_token(shape, element, layers, mixed),
+            "arithmetic": "dtype f32 = what activations, sums, logits and every scale are held and joined in; inside a Q4_K product "
+                          "the 4-bit codes meet each activation as three signed base-256 digit planes (22 bits below a power-of-two "
+                          "scale of its 64-element group, of its 16-element chunk where ffn_down takes them from the SwiGLU epilogue) "
+                          "on v_mfma_i32_16x16x64_i8 -- exact integer sums, weighed by d * sc and dmin * m in fp32; keys and values "
+                          "are stored as fp16 and attention multiplies them on v_mfma_f32_16x16x{32,16}_f16 with fp32 sums",
         },
         "roofline": {
             "bound": "hbm",

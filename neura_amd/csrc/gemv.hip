@@ -1,6 +1,27 @@
 // Narrow products (1..8 activation rows) over raw GGUF blocks: y[r][n] = sum_k x[r][k] * W[n][k].
 //
-// Q4_K: a super-block is 144 B = a 16 B header (d, dmin, 12 scale bytes) + 128 B of nibbles.
+// Which Q4_K form a product reaches with no switch set (launch_gemv asks them in this order; the 16-row tile product and
+// the four-rows-to-an-MFMA kernel live in gemv_tile16.hip):
+//
+//   gemv_q4k_rows4_kernel      3 or 4 activation rows whose digit planes fit LDS (K up to about 10240), matrices that end on 16-row tiles
+//                              (batch 3 and 4: q|k|v, attn_output, gate|up, the head)
+//   gemv_q4k_tile16_kernel     1 row, any K of whole super-blocks, matrices that end on 16-row tiles: every product of a
+//                              batch-1 decode step of the 0.5B .. 7B shapes; 2 rows the same (ffn_down's 18944 columns
+//                              included); 3 and 4 rows where the kernel above refuses and the digits still fit LDS
+//   gemv_q4k_f16_kernel        5 to 8 rows, K <= 4096, at least 4 x 256 tiles of 16 rows (gate|up and the head at batch 5-8)
+//   gemv_q4k_mfma32_kernel     5 to 8 rows otherwise (q|k|v, attn_output; ffn_down in K slices with gemv_fold_kernel), matrices
+//                              that end on 32-row tiles; 3 and 4 rows of short (<= 8192 rows) or very tall (>= 65536) matrices that the
+//                              two kernels on top refused
+//   gemv_q4k_mfma_kernel       what is left with matrices on 16-row tiles and either several rows or K > 4096: ffn_down at
+//                              batch 3 and 4 (K = 18944 does not fit the LDS of the forms above at four rows)
+//   gemv_q4k_decode_kernel     1 row, K <= 4096, matrices that do NOT end on 16-row tiles or activations off a 16-byte
+//                              boundary (odd vocabularies and widths: the small decoders of the tests); the vector form
+//   gemv_q4k_kernel            the same refusals with K > 4096 or 2 to 4 rows: the LDS-tile vector form
+//
+// NEURA_HIP_TILE16=0, NEURA_HIP_ROWS4=0, NEURA_HIP_MFMA=0|2, NEURA_HIP_MFMA32=0|2 and NEURA_HIP_F16_TILES=0|2 push a product
+// down (or up) this list so that the tests can hold the forms to each other on the same shapes.
+//
+// The vector form, Q4_K: a super-block is 144 B = a 16 B header (d, dmin, 12 scale bytes) + 128 B of nibbles.
 // One lane owns one 64-element group of one super-block: it loads the header and its 32
 // nibble bytes with three 128-bit loads, keeps its 64 activations in registers for the whole
 // kernel and walks the output rows, so every weight byte is read from HBM exactly once and
@@ -1497,130 +1518,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_kernel(MFMA_LEAD_PARAME
     }
 }
 
-// One activation row against a short, deep matrix (a down projection: few output rows, long rows).  One 16-row tile
-// per workgroup, its super-blocks dealt to the NW waves in turn, and no shared staging at all: a wave turns the 256
-// activations of a super-block into digits itself, right before it multiplies them, in a corner of LDS nobody else
-// reads.  The digits are scaled per sub-block of 32 (a power of two that puts the sub-block's largest magnitude in
-// [2^29, 2^30)), which is exact, finer than one scale per row, and needs no pass over the whole row first: nothing
-// in the kernel waits for anything but its own loads until the sixteen partial sums of a row meet at the end.
-// Loads are issued whether or not a super-block is left (the last one again, its product dropped), so that the
-// waits count exactly how many loads are newer than the one needed.
-template <int NW, int D>
-__global__ __launch_bounds__(NW * 64) void gemv_q4k_mfma_deep_kernel(MFMA_LEAD_PARAMETERS) {
-    MFMA_TAKE_LEAD;
-    static_assert(D % 2 == 0, "the activation ring alternates between two slots");
-    __shared__ __attribute__((aligned(16))) uint32_t digits[NW][256];  // [step][group][digit plane] per wave
-    __shared__ float sums[NW][16];                                    // per wave: 8 sub-block sums, 8 sub-block unscales
-    __shared__ float part[NW][16];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t tile = blockIdx.x;
-    const uint32_t r = lane & 15u, g = lane >> 4;
-    const uint32_t nb = p.nblk;
-    const uint32_t count = wave < nb ? (nb - wave + NW - 1u) / NW : 0u;  // super-blocks wave, wave + NW, ...
-    const uint32_t last = count ? count - 1u : 0u;
-    typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    typedef const __attribute__((address_space(1))) f32x4 *global_float4;
-
-    float residual = 0.0f;
-    if (wave == 0 && lane < 16u && p.residual) residual = p.residual[(size_t)tile * 16u + lane];
-
-    const uint8_t *const rowp = p.W[0] + (size_t)(tile * 16u + r) * p.row_bytes + g * 32u;
-    const float *const xp = p.x + 4u * lane;
-    auto block_of = [&](uint32_t i) { return min(wave + NW * min(i, last), nb - 1u); };
-    MfmaUnit ring[D];
-    f32x4 xring[2];
-    auto fetch_x = [&](f32x4 &x, uint32_t i) { x = *(global_float4)(uintptr_t)(xp + (size_t)block_of(i) * 256u); };
-    auto fetch_w = [&](MfmaUnit &u, uint32_t i) {
-        const uint8_t *at = rowp + (size_t)block_of(i) * 144u;
-        u.hdr = *(global_uint4)(uintptr_t)(at - g * 32u);
-        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
-        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
-    };
-    fetch_x(xring[0], 0);
-    fetch_x(xring[1], 1);
-#pragma unroll
-    for (int i = 0; i < D; i++) fetch_w(ring[i], i);
-
-    const ScaleLane lane_scales = scale_lane(g);
-    uint32_t *const mine = digits[wave];
-    float *const mysums = sums[wave];
-    const uint32_t *const xlane = mine + g * 4u + (lane & 3u);
-    float acc = 0.0f;
-    for (uint32_t first = 0; first < count; first += D) {
-#pragma unroll
-        for (int slot = 0; slot < D; slot++) {
-            const uint32_t i = first + slot;
-            // ---- this super-block's 256 activations -> digits: lane l holds elements 4l..4l+3, eight lanes a sub-block
-            const f32x4 xv = xring[slot & 1];
-            fetch_x(xring[slot & 1], i + 2u);
-            const float v[4] = {xv.x, xv.y, xv.z, xv.w};
-            uint32_t top = 0;  // largest magnitude as bits: infinities and NaNs sort above every finite value
-#pragma unroll
-            for (int e = 0; e < 4; e++) top = max(top, __builtin_bit_cast(uint32_t, v[e]) & 0x7fffffffu);
-            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
-            top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
-            top = max(top, (uint32_t)dpp_int<0x141>((int)top));  // half mirror: the other quad of the eight
-            const uint32_t raw_exponent = top >> 23;
-            const uint32_t exponent = min(max(raw_exponent, 30u), 254u);
-            const float scale = __builtin_bit_cast(float, (283u - exponent) << 23);
-            const float unscale = raw_exponent == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 29u) << 23);
-            float total = 0.0f;
-            uint32_t word[4], each[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float rounded = rintf(v[e] * scale);
-                total += rounded;
-                each[e] = signed_digits((int)rounded);
-            }
-            digit_planes(each[0], each[1], each[2], each[3], word);
-            total += dpp<DPP_QUAD_XOR1>(total);
-            total += dpp<DPP_QUAD_XOR2>(total);
-            total += dpp<0x141>(total);
-            // elements 4l..4l+3 are nibble word l % 16 of group l / 16 (words 0..7: the low sub-block, 8..15: the high one)
-            *reinterpret_cast<u32x4 *>(mine + ((lane & 15u) * 4u + (lane >> 4)) * 4u) = u32x4{word[0], word[1], word[2], word[3]};
-            if ((lane & 7u) == 0) mysums[lane >> 3] = total, mysums[8u + (lane >> 3)] = unscale;
-            __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
-
-            // ---- the super-block against them
-            const MfmaUnit &u = ring[slot];
-            const uint32_t words[8] = {u.qa.x, u.qa.y, u.qa.z, u.qa.w, u.qb.x, u.qb.y, u.qb.z, u.qb.w};
-            i32x4 cl = {0, 0, 0, 0}, ch = {0, 0, 0, 0};
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-                const int low = (int)(words[w] & 0x0f0f0f0fu), high = (int)((words[w] >> 4) & 0x0f0f0f0fu);
-                const int xl = (int)xlane[w * 16], xh = (int)xlane[(8 + w) * 16];
-                cl = __builtin_amdgcn_mfma_i32_4x4x4i8(xl, low, cl, 0, 0, 0);
-                ch = __builtin_amdgcn_mfma_i32_4x4x4i8(xh, high, ch, 0, 0, 0);
-            }
-            half2_t sc, mn;
-            scale_pairs(u.hdr, lane_scales, sc, mn);                  // integers as half subnormals: value * 2^-24
-            const half2_t dd = __builtin_bit_cast(half2_t, u.hdr.x);  // (d, dmin)
-            const float ul = mysums[8u + 2u * g], uh = mysums[9u + 2u * g];
-            const float d24 = (float)dd.x * 16777216.0f, m24 = (float)dd.y * 16777216.0f;
-            const float s0 = d24 * (float)sc.x * ul, s1 = d24 * (float)sc.y * uh, m0 = m24 * (float)mn.x * ul, m1 = m24 * (float)mn.y * uh;
-            const float fl = fmaf(fmaf(fmaf((float)cl[0], 256.0f, (float)cl[1]), 256.0f, (float)cl[2]), 256.0f, (float)cl[3]);
-            const float fh = fmaf(fmaf(fmaf((float)ch[0], 256.0f, (float)ch[1]), 256.0f, (float)ch[2]), 256.0f, (float)ch[3]);
-            const float product = fmaf(s0, fl, s1 * fh) - fmaf(m0, mysums[2u * g], m1 * mysums[2u * g + 1u]);
-            acc += i < count ? product : 0.0f;
-            __builtin_amdgcn_wave_barrier();  // the next super-block's digits overwrite these
-            fetch_w(ring[slot], i + D);
-        }
-    }
-    // lane (r, g) holds group g's share of output row r: the four groups, then the waves
-    acc += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, acc), 0x401F));  // lane ^ 16
-    acc += __shfl_xor(acc, 32, 64);
-    if (g == 0) part[wave][r] = acc;
-    __syncthreads();
-    if (wave == 0 && lane < 16u) {
-        float total = 0.0f;
-#pragma unroll
-        for (int k = 0; k < NW; k++) total += part[k][lane];
-        p.y[(size_t)tile * 16u + lane] = p.residual ? residual + total : total;
-    }
-}
-
 // The Q4_K product on 32 x 32 x 32 integer MFMAs (v_mfma_i32_32x32x32_i8): weights are the B operand -- lane (n, q) =
 // (lane % 32, lane / 32) supplies 16 nibbles of row n, one per byte, straight from its 16-byte load of half a group --
 // and the digit planes of up to eight activation rows are the A operand (row m = 4 * activation row + plane, read from
@@ -2395,28 +2292,9 @@ static hipError_t launch_mfma_kernel(nh_device *d, const MfmaParams &p, uint32_t
 // LDS bytes of the staged activations of `blocks` super-blocks for P activation rows: digits + sums
 static size_t mfma_staged(uint32_t blocks, uint32_t P) { return (size_t)blocks * (1024u + 32u) * P; }
 
-// whether the deep kernel (one tile per workgroup, sixteen waves along K) serves this product
-static bool mfma_goes_deep(const nh_device *d, const GemvArgs &a) {
-    if (a.rows != 1 || a.swiglu || a.norm_w || a.W[1] || a.W[2]) return false;
-    // a matrix short enough that its tiles do not even fill the device once, and rows deep enough to feed sixteen waves
-    return a.N / 16u <= (uint32_t)d->compute_units && a.K / 256u >= 32u;
-}
-
 static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
     const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
     const uint32_t nblk = a.K / 256u;
-    if (mfma_goes_deep(d, a)) {
-        MfmaParams p{};
-        p.W[0] = static_cast<const uint8_t *>(a.W[0]);
-        p.x = a.x, p.y = a.y, p.residual = a.residual;
-        p.N = a.N, p.K = a.K, p.row_bytes = nblk * 144u, p.nblk = nblk, p.rows = 1, p.tiles = a.N / 16u;
-        profile_mark(d);
-        hipLaunchKernelGGL((gemv_q4k_mfma_deep_kernel<16, 2>), dim3(p.tiles), dim3(1024), 0, d->stream, MFMA_LEAD(p));
-        NH_HIP(hipGetLastError());
-        profile_mark(d);
-        if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
-        return NH_OK;
-    }
     const size_t room = 140 * 1024;  // a gfx950 workgroup may take all 160 KiB of a compute unit; tile partials and static arrays need the rest
     for (uint32_t done = 0; done < a.rows;) {
         // activation rows per launch: 4, 2 or 1 (the kernel's instantiations); rows too deep to stage whole are cut into K slices
