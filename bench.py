@@ -454,7 +454,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": ("all narrow products: gemv_q4k_tile16_kernel, gemv_staged_kernel<Q6_K>" if mixed else
+            "kernel": ("all narrow products: gemv_q4k_tile16_kernel, gemv_q6k_tile16_kernel" if mixed else
                        "gemv_q4k_tile16_kernel (q|k|v with the rotation, attn_output, gate|up with SwiGLU, ffn_down, output head)" if element == 12
                        else "gemv_q8_0_decode_kernel"),
             "achieved": achieved,

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBRARY = os.path.join(HERE, "libneura_hip.so")
-SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemv_tile16.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "sample.hip", "model.hip"]
+SOURCES = ["runtime.hip", "codec.hip", "gemv.hip", "gemv_tile16.hip", "gemv_q6k_tile16.hip", "gemm.hip", "rowops.hip", "attention.hip", "argmax.hip", "sample.hip", "model.hip"]
 # -amdgpu-kernarg-preload-count: the hardware hands a kernel's leading plain arguments (up to 14 words) to every wave in scalar
 # registers as it starts it, so a kernel's first loads need not wait for a load of its arguments (about 0.5 us a launch);
 # kernels that take a parameter struct name what they need first as leading arguments for this
@@ -31,7 +31,7 @@ def hipcc():
 
 
 # per file: the 16-row tile product and the attention kernels work on their matrix-core sums where they land, in vector registers
-EXTRA_FLAGS = {"gemv_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+EXTRA_FLAGS = {"gemv_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "gemv_q6k_tile16.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"], "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def _compile(source):

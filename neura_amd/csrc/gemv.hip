@@ -2621,6 +2621,7 @@ int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (a.merge) return launch_rows<1>(d, a, a.x, a.y, a.residual);
     if (rows4_takes(a)) return launch_rows4(d, a);
     if (tile16_takes(a)) return launch_tile16(d, a);
+    if (q6k_tile16_takes(a)) return launch_q6k_tile16(d, a);
     if (a.digits_out || a.digits_in) return fail(NH_E_ARGUMENT, "this product hands over no digit planes (ask gemv_hands_digits first)");
     if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (f16_tiles_take(d, a)) return launch_f16_tiles(d, a);

@@ -182,11 +182,21 @@ inline int env_int(const char *name, int fallback) {
     return held && *held ? atoi(held) : fallback;
 }
 
+// Activations as the 16x16x64 integer MFMA takes them (gemv_tile16.hip, gemv_q6k_tile16.hip): per super-block of 256, sixteen
+// chunks of 16 activations, each three signed base-256 digit planes of 16 bytes; where a chunk has a scale of its own, a
+// (sum, scale) pair of floats beside it; in memory (handed from one product to the next) a chunk is one 64-byte piece
+constexpr uint32_t TILE16_BLOCK_DIGITS = 768;
+constexpr uint32_t TILE16_BLOCK_PAIRS = 128;
+constexpr uint32_t TILE16_BLOCK_HANDED = 1024;
+
 // the 16-row tile kernel (gemv_tile16.hip): whether it serves this product, and its launch
 bool tile16_takes(const GemvArgs &args);
 int32_t launch_tile16(nh_device *d, const GemvArgs &args);
 // the same for two to eight activation rows, four rows to an MFMA
 bool rows4_takes(const GemvArgs &args);
 int32_t launch_rows4(nh_device *d, const GemvArgs &args);
+// one activation row against a Q6_K matrix on the same tiles (gemv_q6k_tile16.hip)
+bool q6k_tile16_takes(const GemvArgs &args);
+int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &args);
 
 }  // namespace nh

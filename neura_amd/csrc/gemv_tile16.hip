@@ -24,12 +24,9 @@ namespace nh {
 // 0.9 vector instructions a weight (the vector kernel above: 2.4) with the multiply-adds on the matrix cores.
 // Epilogues: y (+ in-place residual by one fire-and-forget add), SwiGLU over a gate tile and the up tile behind it, or the
 // rotation with the cache append (tile rows = 8 channels c.. and their partners c + width/2.. of one head).
-constexpr uint32_t TILE16_BLOCK_DIGITS = 768;  // 16 chunks of 16 activations x 3 planes x 16 bytes
 constexpr uint32_t TILE16_ZERO_BYTES = 208;    // what an idle A lane reads: four chunk offsets (0, 48, 96, 144) + 16 bytes
 enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2 };
 
-constexpr uint32_t TILE16_BLOCK_PAIRS = 128;   // handed-over activations: a (sum, scale) pair of floats per chunk of 16
-constexpr uint32_t TILE16_BLOCK_HANDED = 1024;  // in memory a chunk is one 64-byte piece: three planes, its pair, eight idle bytes
 static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R, bool handed = false) {
     const size_t sums = handed ? (size_t)nblk * TILE16_BLOCK_PAIRS : (size_t)R * nblk * 64u;
     return (size_t)R * nblk * TILE16_BLOCK_DIGITS + (size_t)NW * TILE16_ZERO_BYTES + sums + (size_t)2 * NW * R * 16u * 4u + (size_t)NW * R * 4u + 64u;
@@ -1239,7 +1236,14 @@ bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer) {
     if (consumer.swiglu || consumer.rope || consumer.norm_w) return false;
     GemvArgs from = producer, to = consumer;
     from.digits_out = nullptr, to.digits_in = nullptr;
-    if (!tile16_takes(from) || !tile16_takes(to)) return false;
+    if (!tile16_takes(from)) return false;
+    if (consumer.element == NH_Q6_K) {
+        // the Q6_K tiles read the same pieces in the same chunk order
+        alignas(16) static const uint8_t somewhere[16] = {};
+        to.digits_in = somewhere;
+        return q6k_tile16_takes(to);
+    }
+    if (!tile16_takes(to)) return false;
     const uint32_t nblk = to.K / 256u;
     return tile16_lds(nblk, nblk > 32u ? 16u : 8u, 1u, true) <= 160u * 1024u;
 }

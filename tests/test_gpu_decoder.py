@@ -16,13 +16,13 @@ TINY = dict(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512, voc
 SMALL_Q4 = dict(layers=3, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=1000, tied=False)
 
 
-def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None, window=None, cache_element=1):
+def build(device, shape, element, batch, context, max_rows=1, seed=0, mode="normal", layers=None, window=None, cache_element=1, elements=None):
     rng = np.random.default_rng(seed)
-    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers))
+    tensors = list(synth.model_tensors(shape, element, rng, mode=mode, layers=layers, elements=elements))
     host = {name: raw for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
     model = Model(device, weights, shape, element, batch, context, max_rows, layers=layers, window=window, cache_element=cache_element)
-    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers, window=window, cache_element=cache_element)
+    ref = oracle.Model(shape, element, host, batch, context, max_rows, layers=layers, window=window, cache_element=cache_element, elements=elements)
     return model, ref, weights
 
 
@@ -679,14 +679,17 @@ def test_a_seam_that_gives_up_sends_the_step_down_the_path_of_one_launch_a_produ
         held.release()
 
 
-def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch):
+@pytest.mark.parametrize("down", [NH_Q4_K, NH_Q6_K], ids=["q4_k ffn_down", "q6_k ffn_down"])
+def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch, down):
     """At batch 1 the gate|up product of a Q4_K decoder leaves silu(gate) * up as the digit planes ffn_down multiplies (a
     power-of-two scale per 16 outputs where ffn_down's own staging takes one per 64); NEURA_HIP_TILE16_HANDED=0 hands the
     floats on instead.  Both stay within the decoder's bar of the oracle and of each other (a difference in the last bits of
-    a key now and then flips its rounding to half, 5e-4 of it) and choose the same tokens."""
+    a key now and then flips its rounding to half, 5e-4 of it) and choose the same tokens.  With Q6_K down projections (a
+    Q4_K_M file's) the planes feed the Q6_K tiles, which read the same pieces."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
-    handed, ref, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11)
-    floats, _, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11)
+    elements = {"blk.%d.ffn_down.weight" % layer: down for layer in range(SMALL_Q4["layers"])} if down != NH_Q4_K else None
+    handed, ref, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11, elements=elements)
+    floats, _, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11, elements=elements)
     token = 7
     for step in range(8):
         monkeypatch.setenv("NEURA_HIP_TILE16_HANDED", "1")

@@ -403,6 +403,36 @@ def test_staged_super_block_products(device, element, N, K, rows):
         close(device.gemv(element, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
 
 
+@pytest.mark.parametrize("tile16", ["1", "0"])
+@pytest.mark.parametrize("N,K", [(16, 256), (64, 3584), (3584, 18944), (4608, 3584), (1040, 768), (48, 2048), (272, 8960), (37888, 3584)])
+def test_q6_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K):
+    """One activation row against Q6_K rows on the 16 x 16 x 64 integer MFMA (the stored 6-bit codes as bytes, a scale per
+    lane slice, the activation as three signed digit planes with a sum and a scale per 16 numbers), and with
+    NEURA_HIP_Q6K_TILE16=0 the staged kernel that served before it.  Rows of 210-byte blocks start on every alignment of a
+    half word; activations over many orders of magnitude, with outliers at any seat; plain and with a residual (added in
+    place); non-finite inputs stay visible and zeros give zeros."""
+    monkeypatch.setenv("NEURA_HIP_Q6K_TILE16", tile16)
+    rng = np.random.default_rng(N + K + 6)
+    raw = synth.RANDOM[NH_Q6_K](rng, N * K)
+    weights = oracle.unpack(NH_Q6_K, raw, N * K).reshape(N, K).astype(np.float64)
+    r = rng.standard_normal((1, N)).astype(np.float32)
+    for spread, outliers in ((0.0, False), (2.0, False), (6.0, False), (6.0, True)):
+        x = (rng.standard_normal((1, K)) * np.exp(rng.uniform(-spread, spread, (1, K)))).astype(np.float32)
+        if outliers:
+            x[0, rng.integers(0, K, 24)] *= 1e4  # at any seat of a group
+        plain = oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8)
+        exact = weights @ x.astype(np.float64).T
+        got = device.gemv(NH_Q6_K, raw, N, K, x)
+        if spread <= 2.0:
+            close(got, plain)  # past this spread the oracle's own fp32 sums are the looser side: the exact product judges
+        as_exact_as_the_oracle(got, plain, exact.T, 2e-6)
+        tight(device.gemv(NH_Q6_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    x[0, 5] = np.inf
+    assert not np.isfinite(device.gemv(NH_Q6_K, raw, N, K, x)).any()
+    assert not np.isfinite(device.gemv(NH_Q6_K, raw, N, K, np.full((1, K), np.nan, np.float32))).any()
+    assert np.array_equal(device.gemv(NH_Q6_K, raw, N, K, np.zeros((1, K), np.float32)), np.zeros((1, N), np.float32))
+
+
 @pytest.mark.parametrize("element", [NH_Q6_K, NH_Q5_K, NH_Q3_K])
 def test_staged_super_block_product_reads_packed_weights(device, element):
     N, K = 96, 2048
