@@ -394,7 +394,7 @@ bool q6k_tile16_takes(const GemvArgs &a) {
     } else if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) {
         return false;
     }
-    if ((uintptr_t)a.W[0] & 1u) return false;
+    if ((uintptr_t)a.W[0] & 3u) return false;  // the first block on a 4-byte boundary: no load starts before the matrix
     const uint32_t nblk = a.K / 256u;
     return q6k_tile16_lds(nblk, nblk > 32u && !a.digits_in ? 16u : 8u) <= 160u * 1024u;
 }
