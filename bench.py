@@ -58,6 +58,8 @@ def workload(name):
         return synth.SHAPES["qwen2.5-7b"], 12, 4096, {}, ()
     if name == "qwen2.5-0.5b-q8_0":
         return synth.SHAPES["qwen2.5-0.5b"], 8, 1088, {}, ()
+    if name == "qwen2.5-1.5b-q4k":  # the shape whose layer products are BASELINE's second configuration
+        return synth.SHAPES["qwen2.5-1.5b"], 12, 1088, {}, ()
     if name == "qwen2.5-7b-q4_k_m":
         # the mix llama.cpp's Q4_K_M recipe gives a Qwen2.5-7B file: the head and, in the first and last eighth of the layers
         # and every third between, the value and down projections in Q6_K, the rest Q4_K; q, k and v biases everywhere

@@ -34,7 +34,8 @@ namespace nh {
 // The rest is the Q4_K product's: NW waves share a tile and split its super-blocks, each turning into digits exactly the
 // activations it multiplies (or copying them, HANDED: the 64-byte pieces a SwiGLU epilogue left, whose chunk order is this
 // kernel's too); loads run two units ahead across tile boundaries, every wave walks whole rounds of two steps; the finishing
-// wave changes from tile to tile; plain epilogue (+ residual, in place by one fire-and-forget add).
+// wave changes from tile to tile; epilogues: plain (+ residual, in place by one fire-and-forget add), SwiGLU over a gate tile
+// and the up tile behind it, or the cast of a value projection's rows into the value state.
 constexpr uint32_t Q6K_BLOCK_BYTES = 210;
 constexpr uint32_t Q6K_ZERO_BYTES = 304;  // what an idle A lane reads: four chunk offsets (0, 96, 192, 288) + 16 bytes
 
@@ -53,9 +54,12 @@ static size_t q6k_tile16_lds(uint32_t nblk, uint32_t NW) {
 
 // The leading arguments are what a wave needs before its first loads: plain words, handed over in scalar registers as the wave
 // starts (-amdgpu-kernarg-preload-count).  `input` is x, or the digit planes with HANDED.
-template <int NW, bool HANDED>
+// SWIGLU: the matrix is a gate matrix with the up matrix `lead_to_w1` * 16 bytes further; a workgroup's unit of work is a pair of
+// tiles (gate rows, then the same rows of up) and the pair's finishing wave writes silu(gate) * up.
+template <int NW, bool HANDED, bool SWIGLU = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, uint32_t lead_row_bytes,
-                                                                  uint32_t lead_grid, uint32_t lead_tiles, uint32_t lead_tile_rows, GemvParams p) {
+                                                                  uint32_t lead_grid, uint32_t lead_tiles, uint32_t lead_tile_rows, int32_t lead_to_w1, GemvParams p) {
+    static_assert(!(HANDED && SWIGLU), "handed-over digit planes feed a plain product");
     extern __shared__ __attribute__((aligned(16))) uint8_t q6k_lds_bytes[];
     constexpr uint32_t NT = NW * 64;
     constexpr int D = 2;
@@ -86,8 +90,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
     const uint32_t tile_rows = lead_tile_rows, row_bytes = lead_row_bytes;
     const uint8_t *const w0 = lead_w0;
     // a tile may hold fewer than 16 rows: the columns past them walk the tile's last row again and are never written
-    auto lane_row = [w0, row_bytes, tile_rows, r](uint32_t tile) -> const uint8_t * { return w0 + (size_t)(tile * tile_rows + min(r, tile_rows - 1u)) * row_bytes; };
+    const int64_t to_w1 = (int64_t)lead_to_w1 * 16;
+    auto lane_row = [w0, row_bytes, tile_rows, r, to_w1](uint32_t tile) -> const uint8_t * {
+        if (SWIGLU) return w0 + ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((size_t)((tile >> 1) * 16u + r) * row_bytes);
+        return w0 + (size_t)(tile * tile_rows + min(r, tile_rows - 1u)) * row_bytes;
+    };
     const uint32_t first_tile = block, hop = lead_grid;
+    // with SwiGLU the workgroup's unit of work is a pair: tiles 2 t (gate) and 2 t + 1 (up)
+    auto tile_at = [first_tile, hop](uint32_t i) -> uint32_t {
+        if (SWIGLU) return 2u * (first_tile + (i >> 1) * hop) + (i & 1u);
+        return first_tile + i * hop;
+    };
+    const uint32_t walked = SWIGLU ? 2u * ntiles : ntiles;  // tiles this workgroup walks
     typedef const __attribute__((address_space(1))) q6_u32x3_a4 *global_uint3;
     const uint32_t at_low = 64u * h + 16u * j, at_high = 128u + 32u * h + 16u * j, at_scales = 192u + 8u * h;
 
@@ -95,7 +109,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
     // the last unit is fetched again and dropped, so that the waits count exactly how many loads are newer than the one needed.
     Q6Unit ring[D];
     uint32_t ahead_tile = 0, ahead_b = wave;
-    const uint8_t *ahead_row = lane_row(first_tile);
+    const uint8_t *ahead_row = lane_row(tile_at(0));
     auto fetch = [&](Q6Unit &u) {
         const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * Q6K_BLOCK_BYTES;
         const uint8_t *down = reinterpret_cast<const uint8_t *>(reinterpret_cast<uintptr_t>(at) & ~(uintptr_t)3);
@@ -106,10 +120,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
         u.shift = ((uint32_t)reinterpret_cast<uintptr_t>(at) & 2u) * 8u;
         if (ahead_b + NW < nblk) {
             ahead_b += NW;
-        } else if (ahead_tile + 1u < ntiles) {
+        } else if (ahead_tile + 1u < walked) {
             ahead_b = wave;
             ahead_tile++;
-            ahead_row = lane_row(first_tile + ahead_tile * hop);
+            ahead_row = lane_row(tile_at(ahead_tile));
         }
     };
     auto first_fetches = [&]() {
@@ -270,7 +284,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
     const f32x2 *const pbase = pairs + 8u * h + j;
     const uint32_t pick = j ? 0x07050301u : 0x06040200u;  // the scales of chunks 8 h + 2 g + j out of the eight of half h
     const int beside = (int)((lane ^ 16u) * 4u), above = (int)(((lane + 16u) & 63u) * 4u), across = (int)((lane ^ 32u) * 4u);  // lanes of the same row
-    float acc = 0.0f;
+    float acc = 0.0f, gate = 0.0f;
     uint32_t parity = 0;
     struct Step {
         i32x4 c[4];
@@ -321,9 +335,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
         }
         acc = fmaf(half_to_float((uint16_t)st.d), whole, acc);
     };
-    // The wave that finishes a tile (sums the waves' parts, runs the epilogue) changes from tile to tile
+    // The wave that finishes a tile (sums the waves' parts, runs the epilogue) changes from tile to tile (with SwiGLU from pair to
+    // pair: the gate sum waits in its registers)
     auto tile_end = [&](uint32_t tile, uint32_t index) {
-        const uint32_t finisher = index % NW;
+        const uint32_t finisher = (SWIGLU ? index >> 1 : index) % NW;
         float v = acc;
         v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
         v += __shfl_xor(v, 32, 64);
@@ -335,9 +350,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
 #pragma unroll
             for (int w = 0; w < NW; w++) total += part[(parity * NW + w) * 16u + r];
             const size_t n = (size_t)tile * tile_rows + r;
-            if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);  // in place: one add per element, nothing to wait for
+            if (SWIGLU) {
+                if (!(tile & 1u)) gate = total;
+                else p.y[(size_t)(tile >> 1) * 16u + r] = silu(gate) * total;
+            } else if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);  // in place: one add per element, nothing to wait for
             else p.y[n] = p.residual ? p.residual[n] + total : total;
-            if (p.append_value) {
+            if (!SWIGLU && p.append_value) {
                 // a value projection of one token: its rows (+ bias) go into the value state at the cursor as halves, as
                 // value_append_kernel would cast them
                 const uint32_t cursor = p.rope_cursor[0];
@@ -350,12 +368,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
         parity ^= 1u;
     };
     if (count == 0) {  // more waves than super-blocks: this one only keeps the barriers
-        for (uint32_t t = 0; t < ntiles; t++) tile_end(first_tile + t * hop, t);
+        for (uint32_t t = 0; t < walked; t++) tile_end(tile_at(t), t);
         return;
     }
     // Every wave walks whole rounds of D steps: the steps past its last tile multiply what was fetched again and publish nothing.
     uint32_t at_tile = 0, at_b = wave;
-    const uint32_t steps = ntiles * count;
+    const uint32_t steps = walked * count;
     for (uint32_t s0 = 0; s0 < steps; s0 += D) {
 #pragma unroll
         for (int slot = 0; slot < D; slot++) {
@@ -367,7 +385,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
             weigh(st);
             at_b += NW;
             if (at_b >= nblk) {
-                if (at_tile < ntiles) tile_end(first_tile + at_tile * hop, at_tile);
+                if (at_tile < walked) tile_end(tile_at(at_tile), at_tile);
                 at_b = wave;
                 at_tile++;
             }
@@ -376,12 +394,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
 }
 
 // NEURA_HIP_Q6K_TILE16=0 keeps the kernel out (the staged kernel then takes Q6_K as before).  Otherwise it takes every Q6_K product
-// of one row and one matrix that ends on a tile boundary, with no epilogue but the residual or the cast of a value
-// projection's rows into the value state: the head, ffn_down, attn_v and attn_output of a k-quant mix.
+// of one row and one matrix that ends on a tile boundary (or a gate and an up matrix with SwiGLU), with no other epilogue than the
+// residual or the cast of a value projection's rows into the value state: the head, ffn_down, attn_v and attn_output of a k-quant
+// mix, gate|up of a file stored in Q6_K throughout.  What folds the rotation in stays with the staged kernel.
 bool q6k_tile16_takes(const GemvArgs &a) {
-    if (a.element != NH_Q6_K || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.swiglu || a.rope || a.merge || a.digits_out) return false;
+    if (a.element != NH_Q6_K || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.rope || a.merge || a.digits_out) return false;
     if (env_int("NEURA_HIP_Q6K_TILE16", 1) == 0) return false;
-    if (a.W[1] || a.W[2] || a.end[0] != a.N) return false;
+    if (a.swiglu) {  // gate and up stacked: pairs of whole tiles, no other epilogue
+        if (!a.W[1] || a.W[2] || a.residual || a.append_value || a.digits_in || a.end[0] != a.N / 2u || a.N % 32u != 0) return false;
+        const int64_t apart = static_cast<const uint8_t *>(a.W[1]) - static_cast<const uint8_t *>(a.W[0]);
+        if (apart % 16 != 0 || apart / 16 > INT32_MAX || apart / 16 < INT32_MIN) return false;
+    } else if (a.W[1] || a.W[2] || a.end[0] != a.N) {
+        return false;
+    }
     if (a.append_value) {  // a value projection that casts its rows into the value state: whole heads, no other epilogue
         if (a.residual || a.digits_in || !a.append_value->width || a.N % a.append_value->width) return false;
     } else if (a.bias[0]) {
@@ -399,16 +424,17 @@ bool q6k_tile16_takes(const GemvArgs &a) {
     return q6k_tile16_lds(nblk, nblk > 32u && !a.digits_in ? 16u : 8u) <= 160u * 1024u;
 }
 
-template <int NW, bool HANDED>
+template <int NW, bool HANDED, bool SWIGLU = false>
 static hipError_t launch_q6k_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
     static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q6k_tile16_kernel<NW, HANDED>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q6k_tile16_kernel<NW, HANDED>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
-                       HANDED ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x), p.norm_w, p.row_bytes, grid, p.row_groups, p.tile_rows, p);
+    hipLaunchKernelGGL((gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
+                       HANDED ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x), p.norm_w, p.row_bytes, grid, p.row_groups, p.tile_rows,
+                       (int32_t)((p.W[1] - p.W[0]) / 16), p);
     return hipGetLastError();
 }
 
@@ -418,8 +444,9 @@ int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &a) {
         p.W[s] = static_cast<const uint8_t *>(a.W[0]);
         p.end[s] = a.N;
     }
+    if (a.swiglu) p.W[1] = static_cast<const uint8_t *>(a.W[1]), p.end[0] = a.N / 2u;
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
-    p.N = a.N, p.K = a.K, p.eps = a.eps, p.rows = 1;
+    p.N = a.N, p.K = a.K, p.eps = a.eps, p.rows = 1, p.swiglu = a.swiglu;
     p.digits_in = a.digits_in;
     if (a.append_value) {
         p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
@@ -436,18 +463,23 @@ int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &a) {
         const uint32_t tiles = a.N / rows, rounds = (tiles + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
         return 65536u - (uint32_t)((uint64_t)tiles * 65536u / ((uint64_t)rounds * (uint32_t)d->compute_units));
     };
-    for (uint32_t rows = 15; rows >= 12; rows--) {
+    for (uint32_t rows = 15; rows >= 12 && !a.swiglu; rows--) {
         if (a.N % rows) continue;
         if (idle(rows) + 3277u < idle(p.tile_rows)) p.tile_rows = rows;
     }
-    const uint32_t units = a.N / p.tile_rows;
+    const uint32_t units = a.swiglu ? a.N / 32u : a.N / p.tile_rows;
     p.row_groups = units;
     const uint32_t rounds = (units + (uint32_t)d->compute_units - 1u) / (uint32_t)d->compute_units;
     const uint32_t grid = (units + rounds - 1u) / rounds;
     const size_t lds = q6k_tile16_lds(p.nblk, waves);
     profile_mark(d);
     hipError_t launched;
-    if (a.digits_in) {
+    if (a.swiglu) {
+        launched = waves == 4u ? launch_q6k_tile16_instance<4, false, true>(d, p, grid, lds)
+                   : waves == 7u ? launch_q6k_tile16_instance<7, false, true>(d, p, grid, lds)
+                   : waves == 8u ? launch_q6k_tile16_instance<8, false, true>(d, p, grid, lds)
+                                 : launch_q6k_tile16_instance<16, false, true>(d, p, grid, lds);
+    } else if (a.digits_in) {
         launched = waves == 4u ? launch_q6k_tile16_instance<4, true>(d, p, grid, lds)
                    : waves == 7u ? launch_q6k_tile16_instance<7, true>(d, p, grid, lds)
                                  : launch_q6k_tile16_instance<8, true>(d, p, grid, lds);

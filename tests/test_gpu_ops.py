@@ -255,7 +255,8 @@ def test_q4_k_product_on_32_row_tiles(device, monkeypatch, forced, N, K, rows):
 
 
 @pytest.mark.parametrize("tile16", ["1", "0"])
-@pytest.mark.parametrize("N,K", [(16, 256), (64, 3584), (4608, 3584), (3584, 18944), (37888, 3584), (1040, 768), (48, 2048), (272, 8960)])
+@pytest.mark.parametrize("N,K", [(16, 256), (64, 3584), (4608, 3584), (3584, 18944), (37888, 3584), (1040, 768), (48, 2048), (272, 8960), (2048, 1536),
+                                 (17920, 1536), (1536, 1280)])
 def test_q4_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K):
     """One activation row against Q4_K rows: the 16-row tiles on the 16 x 16 x 64 integer MFMA (weights as nibbles, the
     activation as three signed digit planes scaled per 64 numbers), and with NEURA_HIP_TILE16=0 the kernels that served
@@ -409,8 +410,8 @@ def test_q6_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K)
     """One activation row against Q6_K rows on the 16 x 16 x 64 integer MFMA (the stored 6-bit codes as bytes, a scale per
     lane slice, the activation as three signed digit planes with a sum and a scale per 16 numbers), and with
     NEURA_HIP_Q6K_TILE16=0 the staged kernel that served before it.  Rows of 210-byte blocks start on every alignment of a
-    half word; activations over many orders of magnitude, with outliers at any seat; plain and with a residual (added in
-    place); non-finite inputs stay visible and zeros give zeros."""
+    half word; activations over many orders of magnitude, with outliers at any seat; plain, with a residual (added in
+    place) and with SwiGLU; non-finite inputs stay visible and zeros give zeros."""
     monkeypatch.setenv("NEURA_HIP_Q6K_TILE16", tile16)
     rng = np.random.default_rng(N + K + 6)
     raw = synth.RANDOM[NH_Q6_K](rng, N * K)
@@ -427,6 +428,14 @@ def test_q6_k_one_row_product_on_16_row_tiles(device, monkeypatch, tile16, N, K)
             close(got, plain)  # past this spread the oracle's own fp32 sums are the looser side: the exact product judges
         as_exact_as_the_oracle(got, plain, exact.T, 2e-6)
         tight(device.gemv(NH_Q6_K, raw, N, K, x, residual=r), r + plain, 1e-5)
+    if N % 32 == 0:
+        x = rng.standard_normal((1, K)).astype(np.float32)
+        x[0, rng.integers(0, K, 8)] *= 50.0
+        plain = oracle.gemv(NH_Q6_K, raw, N, K, x, threads=8)
+        gate, up = plain[:, : N // 2].astype(np.float64), plain[:, N // 2:].astype(np.float64)
+        with np.errstate(over="ignore"):
+            want = gate / (1.0 + np.exp(-gate)) * up
+        close(device.gemv(NH_Q6_K, raw, N, K, x, swiglu=True), want, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(want).max()))
     x[0, 5] = np.inf
     assert not np.isfinite(device.gemv(NH_Q6_K, raw, N, K, x)).any()
     assert not np.isfinite(device.gemv(NH_Q6_K, raw, N, K, np.full((1, K), np.nan, np.float32))).any()
