@@ -239,6 +239,21 @@ def extras(device, weights, shape, element, context, layers, rng):
     out["decode_sampled_batch1"] = {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
                                     "note": "as the headline step with the greedy choice replaced by the sampled one; caches not pre-filled (zeros)"}
     model.release()
+    note("extras: decode, batch 1, single precision states")
+    model = Model(device, weights, shape, element, batch=1, context=context, layers=layers, cache_element=0)
+    steps, warm = 32, 4
+    first, token = context - (steps + warm), 1
+    for step in range(warm + steps):
+        if step == warm:
+            device.sync()
+            began = time.perf_counter()
+        token = int(model.decode_step([token], [first + step])[0])
+    device.sync()
+    elapsed = time.perf_counter() - began
+    out["decode_single_states_batch1"] = {"value": steps / elapsed, "unit": "tokens/s", "ms_per_step": elapsed / steps * 1e3,
+                                          "note": "as the headline step with the key and value states in single precision (the element the "
+                                                  "reference's example keeps); caches not pre-filled (zeros)"}
+    model.release()
     note("extras: decode, batch 8")
     out["decode_batch8"] = decode_batch8(device, weights, shape, element, context, layers)
     note("extras: 512-token fill")

@@ -158,7 +158,8 @@ int32_t nh_attention(nh_device *device, const float *dev_q, const uint16_t *dev_
                      const uint32_t *dev_cursor, float scale, float *dev_out);
 /* nh_cache_write and nh_attention over states of another element (Cache::new(.., Element::Single | Half | Bfloat16),
  * crates/neura-decoder/src/cache.rs:130-134; the reference's cache tests run Single and Half, tests/cache.rs:17): the caches
- * are arrays of `cache_element` (NH_F16, NH_BF16 or NH_F32), everything else as above.  NH_F16 takes the kernels above. */
+ * are arrays of `cache_element` (NH_F16, NH_BF16 or NH_F32), everything else as above.  Chunks of one row and of four and more rows at head widths 64 and 128 ride the
+ * same matrix-core kernels whatever the element (bfloat16 as the halves they equal, single as two half planes). */
 int32_t nh_cache_write_element(nh_device *device, const float *dev_k, const float *dev_v, void *dev_cache_k, void *dev_cache_v,
                                uint32_t kv_heads, uint32_t batch, uint32_t rows, uint32_t width, uint32_t capacity, uint32_t window,
                                const uint32_t *dev_cursor, const uint8_t *dev_mask, int32_t ring, int32_t cache_element);
@@ -212,7 +213,9 @@ typedef struct nh_model_config {
     int32_t cache_element; /* what the key and value states hold (Cache::new(.., element), crates/neura-decoder/src/cache.rs:63,
                               :130-134): NH_F16, NH_BF16 or NH_F32 -- NH_F32 is 0, so a config that never names it keeps single
                               precision states as the reference's own example does (examples/qwen/main.rs:107); the headline
-                              workload names NH_F16.  Keys and values are cast on their way in (graph.cast, cache.rs:347-348;
+                              workload names NH_F16.  Every element takes the fused kernels (single and bfloat16 states are
+                              read onto the matrix cores as halves: magnitudes past 65504 overflow as in half states).
+                              Keys and values are cast on their way in (graph.cast, cache.rs:347-348;
                               bfloat16 rounds to nearest even, crates/neura-kernel/src/task/convert.rs:86-89) */
 } nh_model_config;
 

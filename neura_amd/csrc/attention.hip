@@ -329,6 +329,42 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_p
 }
 
 
+// Eight numbers of a key or value state as eight halves (four words) for the matrix cores, and for single states the eight
+// residues * 2^11 beside them.  Halves go as they lie.  bfloat16 numbers become the halves they equal (every bfloat16 between
+// 2^-17 and 65504 in magnitude is a half; smaller ones land within 2^-25).  Single numbers enter as two half planes, the value
+// rounded to half and its residue * 2^11 -- 22 bits of each, as the queries and the weights do.  States past the halves' range
+// (65504) overflow here as they would in half states.
+template <int CE, int WORDS>
+__device__ __forceinline__ void states_as_halves(const u32x4 (&raw)[WORDS], u32x4 &value, u32x4 &residue) {
+    if constexpr (CE == NH_F16) {
+        value = raw[0];
+    } else if constexpr (CE == NH_BF16) {
+        const uint32_t words[4] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w};
+        uint32_t out[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t word = words[i];
+            const _Float16 low = (_Float16)__builtin_bit_cast(float, word << 16), high = (_Float16)__builtin_bit_cast(float, word & 0xffff0000u);
+            out[i] = (uint32_t)__builtin_bit_cast(uint16_t, low) | ((uint32_t)__builtin_bit_cast(uint16_t, high) << 16);
+        }
+        value = u32x4{out[0], out[1], out[2], out[3]};
+    } else {
+        const uint32_t words[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[WORDS - 1].x, raw[WORDS - 1].y, raw[WORDS - 1].z, raw[WORDS - 1].w};
+        uint32_t out[4], fine_out[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t first = words[2 * i], second = words[2 * i + 1];
+            const float a = __builtin_bit_cast(float, first), b = __builtin_bit_cast(float, second);
+            const _Float16 a_high = (_Float16)a, b_high = (_Float16)b;
+            const _Float16 a_low = (_Float16)((a - (float)a_high) * 2048.0f), b_low = (_Float16)((b - (float)b_high) * 2048.0f);
+            out[i] = (uint32_t)__builtin_bit_cast(uint16_t, a_high) | ((uint32_t)__builtin_bit_cast(uint16_t, b_high) << 16);
+            fine_out[i] = (uint32_t)__builtin_bit_cast(uint16_t, a_low) | ((uint32_t)__builtin_bit_cast(uint16_t, b_low) << 16);
+        }
+        value = u32x4{out[0], out[1], out[2], out[3]};
+        residue = u32x4{fine_out[0], fine_out[1], fine_out[2], fine_out[3]};
+    }
+}
+
 // ---------------------------------------------------------------- several query rows: the matrix cores --------
 //
 // A chunk of query rows (a fill) against the same cache, on v_mfma_f32_32x32x16_f16.  One workgroup serves one
@@ -346,7 +382,9 @@ __global__ __launch_bounds__(256) void attention_fold_kernel(const float *lead_p
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-template <int WIDTH>
+// CE: what the states hold (states_as_halves above); single states stage a second plane of key and value residues and cost
+// one more MFMA a product.
+template <int WIDTH, int CE = NH_F16>
 __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, uint32_t rows_per_wave) {
     fetch_parameters(p);
     constexpr int TK = 32;                       // keys per tile
@@ -354,8 +392,15 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
     constexpr int BLOCKS = WIDTH / 32;           // 32-channel blocks of the output
     constexpr int KPITCH = WIDTH + 8;            // halves per staged key row (the pad spreads the banks)
     constexpr int VPITCH = TK + 4;               // halves per staged value channel
-    __shared__ __attribute__((aligned(16))) uint16_t kt[TK][KPITCH];
-    __shared__ __attribute__((aligned(16))) uint16_t vt[WIDTH][VPITCH];
+    constexpr int PLANES = CE == NH_F32 ? 2 : 1;  // values, and for single states their residues * 2^11
+    constexpr int WORDS = CE == NH_F32 ? 2 : 1;   // 16-byte loads that hold eight stored numbers
+    constexpr uint32_t STORED = CE == NH_F32 ? 4u : 2u;
+    __shared__ __attribute__((aligned(16))) uint16_t kt_planes[PLANES][TK][KPITCH];
+    __shared__ __attribute__((aligned(16))) uint16_t vt_planes[PLANES][WIDTH][VPITCH];
+    uint16_t(*const kt)[KPITCH] = kt_planes[0];
+    uint16_t(*const vt)[VPITCH] = vt_planes[0];
+    uint16_t(*const kt_fine)[KPITCH] = kt_planes[PLANES - 1];
+    uint16_t(*const vt_fine)[VPITCH] = vt_planes[PLANES - 1];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n = lane & 31u, h = lane >> 5;
     const uint32_t G = p.groups;
@@ -403,14 +448,18 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
 
     // the pieces of a tile this thread stages: 16 bytes of a key row and of a value row each
     constexpr int PIECES = TK * WIDTH / 8 / 256;  // per thread and tile
-    u32x4 kraw[PIECES], vraw[PIECES];
+    u32x4 kraw[PIECES][WORDS], vraw[PIECES][WORDS];
+    const uint8_t *const k_bytes = reinterpret_cast<const uint8_t *>(p.cache_k), *const v_bytes = reinterpret_cast<const uint8_t *>(p.cache_v);
     auto fetch = [&](uint32_t tile) {
 #pragma unroll
         for (int k = 0; k < PIECES; k++) {
             const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
             const uint64_t at = (plane + min(tile + key, p.capacity - 1u)) * WIDTH + chunk * 8u;
-            kraw[k] = *reinterpret_cast<const u32x4 *>(p.cache_k + at);
-            vraw[k] = *reinterpret_cast<const u32x4 *>(p.cache_v + at);
+#pragma unroll
+            for (int w = 0; w < WORDS; w++) {
+                kraw[k][w] = *reinterpret_cast<const u32x4 *>(k_bytes + at * STORED + 16u * w);
+                vraw[k][w] = *reinterpret_cast<const u32x4 *>(v_bytes + at * STORED + 16u * w);
+            }
         }
     };
     fetch(0);
@@ -419,14 +468,25 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
 #pragma unroll
         for (int k = 0; k < PIECES; k++) {
             const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
-            *reinterpret_cast<u32x4 *>(&kt[key][chunk * 8u]) = kraw[k];
+            u32x4 k_words, k_fine = {0u, 0u, 0u, 0u}, v_words, v_fine = {0u, 0u, 0u, 0u};
+            states_as_halves<CE, WORDS>(kraw[k], k_words, k_fine);
+            states_as_halves<CE, WORDS>(vraw[k], v_words, v_fine);
+            *reinterpret_cast<u32x4 *>(&kt[key][chunk * 8u]) = k_words;
+            if constexpr (CE == NH_F32) *reinterpret_cast<u32x4 *>(&kt_fine[key][chunk * 8u]) = k_fine;
             // rows past the written keys may hold anything, and a weight of zero does not silence a NaN
             const uint32_t keep = tile + key < span ? 0xffffffffu : 0u;
-            const uint32_t words[4] = {vraw[k].x & keep, vraw[k].y & keep, vraw[k].z & keep, vraw[k].w & keep};
             // groups of four keys change places by the channel block (chunk / 4), or the chunks a store instruction touches share four banks
             const uint32_t column = (((key >> 2) ^ (chunk >> 2)) << 2) | (key & 3u);
+            {
+                const uint32_t words[4] = {v_words.x & keep, v_words.y & keep, v_words.z & keep, v_words.w & keep};
 #pragma unroll
-            for (int i = 0; i < 8; i++) vt[chunk * 8u + i][column] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
+                for (int i = 0; i < 8; i++) vt[chunk * 8u + i][column] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
+            }
+            if constexpr (CE == NH_F32) {
+                const uint32_t words[4] = {v_fine.x & keep, v_fine.y & keep, v_fine.z & keep, v_fine.w & keep};
+#pragma unroll
+                for (int i = 0; i < 8; i++) vt_fine[chunk * 8u + i][column] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
+            }
         }
         if (tile + TK < span) fetch(tile + TK);  // in flight while this tile is multiplied
         __syncthreads();
@@ -441,6 +501,8 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             const half8_t keys = *reinterpret_cast<const half8_t *>(&kt[n][16 * s + 8 * h]);
             scores = __builtin_amdgcn_mfma_f32_32x32x16_f16(keys, q_value[s], scores, 0, 0, 0);
             fine = __builtin_amdgcn_mfma_f32_32x32x16_f16(keys, q_residue[s], fine, 0, 0, 0);
+            if constexpr (CE == NH_F32)
+                fine = __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const half8_t *>(&kt_fine[n][16 * s + 8 * h]), q_value[s], fine, 0, 0, 0);
         }
         // ---- weights: register 4j + e of lane (column, h) is key 8j + 4h + e of the tile
         float tile_top = -INFINITY;
@@ -455,7 +517,7 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
         const float next = fmaxf(top, tile_top);
         const float rescale = top == -INFINITY ? 0.0f : softmax_exp(top - next);
         float tile_mass = 0.0f;
-        half8_t w_value[2], w_residue[2];
+        half8_t w_value[2], w_residue[2], w_small[2];  // w_small: the weights * 2^-11, for the values' residues (single states)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const float weight = scores[r] == -INFINITY ? 0.0f : softmax_exp(scores[r] - next);
@@ -466,6 +528,7 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             // key slots of the second product: step t takes registers 8t .. 8t + 7 in order
             w_value[r >> 3][r & 7] = high;
             w_residue[r >> 3][r & 7] = (_Float16)(raised - (float)high);
+            w_small[r >> 3][r & 7] = (_Float16)(CE == NH_F32 ? raised * (1.0f / 2048.0f) : 0.0f);
         }
         tile_mass += __shfl_xor(tile_mass, 32, 64);
         mass = fmaf(mass, rescale, tile_mass);
@@ -486,6 +549,12 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
                 values = __builtin_bit_cast(half8_t, joined);
                 acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(values, w_value[t], acc[d], 0, 0, 0);
                 acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(values, w_residue[t], acc[d], 0, 0, 0);
+                if constexpr (CE == NH_F32) {
+                    const uint2 low_fine = *reinterpret_cast<const uint2 *>(&vt_fine[32 * d + n][4 * ((4 * t + h) ^ d)]);
+                    const uint2 high_fine = *reinterpret_cast<const uint2 *>(&vt_fine[32 * d + n][4 * ((4 * t + 2 + h) ^ d)]);
+                    const half8_t residues = __builtin_bit_cast(half8_t, u32x4{low_fine.x, low_fine.y, high_fine.x, high_fine.y});
+                    acc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(residues, w_small[t], acc[d], 0, 0, 0);
+                }
             }
         }
     }
@@ -523,7 +592,9 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // hardware hands to a wave in scalar registers as it starts (batch and query heads a group share a word); the rest is in `p`.
 // TK = 16 (one plane a kv head: a decode step of few planes): tiles of sixteen keys, so that sections of 64 keys give every
 // compute unit a workgroup and a wave half the work; the value product then runs on v_mfma_f32_16x16x16_f16 (K = the tile's keys).
-template <int WIDTH, int TK = 32>
+// CE: what the states hold (states_as_halves above): single states cost one more MFMA a product -- the key residues against the
+// query values, the value residues against the weights * 2^-11.
+template <int WIDTH, int TK = 32, int CE = NH_F16>
 __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32_t *lead_cursor, const float *lead_q, const uint16_t *lead_k, const uint16_t *lead_v,
                                                                     uint32_t lead_q_sh, uint32_t lead_q_sb, uint32_t lead_keys, uint32_t lead_sections,
                                                                     uint32_t lead_capacity, uint32_t lead_batch_groups, AttentionParams p) {
@@ -571,21 +642,27 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
     for (int d = 0; d < BLOCKS; d++) acc[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float top = -INFINITY, mass = 0.0f;
 
-    u32x4 kraw[KB][STEPS], vraw[PIECES];
+    constexpr int WORDS = CE == NH_F32 ? 2 : 1;              // 16-byte loads that hold eight stored numbers
+    constexpr uint32_t STORED = CE == NH_F32 ? 4u : 2u;      // bytes a stored number
+    const uint8_t *const k_bytes = reinterpret_cast<const uint8_t *>(lead_k), *const v_bytes = reinterpret_cast<const uint8_t *>(lead_v);
+    u32x4 kraw[KB][STEPS][WORDS], vraw[PIECES][WORDS];
     auto fetch_keys = [&](uint32_t tile) {
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
                 const uint64_t at = (plane + min(tile + 16u * kb + n, capacity - 1u)) * WIDTH + 32u * s + 8u * kq;
-                kraw[kb][s] = *reinterpret_cast<const u32x4 *>(lead_k + at);
+#pragma unroll
+                for (int w = 0; w < WORDS; w++) kraw[kb][s][w] = *reinterpret_cast<const u32x4 *>(k_bytes + at * STORED + 16u * w);
             }
     };
     auto fetch_values = [&](uint32_t tile) {
 #pragma unroll
         for (int i = 0; i < PIECES; i++) {
             const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
-            vraw[i] = *reinterpret_cast<const u32x4 *>(lead_v + (plane + min(tile + key, capacity - 1u)) * WIDTH + part * 8u);
+            const uint64_t at = (plane + min(tile + key, capacity - 1u)) * WIDTH + part * 8u;
+#pragma unroll
+            for (int w = 0; w < WORDS; w++) vraw[i][w] = *reinterpret_cast<const u32x4 *>(v_bytes + at * STORED + 16u * w);
         }
     };
     // the first tile's rows are asked for whether or not the cursor has reached them (the addresses are clamped to the cache)
@@ -618,9 +695,12 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
             scores[kb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, fine[kb] = scores[kb];
 #pragma unroll
             for (int s = 0; s < STEPS; s++) {
-                const half8_t keys = __builtin_bit_cast(half8_t, kraw[kb][s]);
+                u32x4 key_words, key_residues = {0u, 0u, 0u, 0u};
+                states_as_halves<CE, WORDS>(kraw[kb][s], key_words, key_residues);
+                const half8_t keys = __builtin_bit_cast(half8_t, key_words);
                 scores[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(keys, q_value[s], scores[kb], 0, 0, 0);
                 fine[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(keys, q_residue[s], fine[kb], 0, 0, 0);
+                if constexpr (CE == NH_F32) fine[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, key_residues), q_value[s], fine[kb], 0, 0, 0);
             }
         }
         const uint32_t next = tile + 4 * TK;
@@ -641,9 +721,9 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
         const float newer = fmaxf(top, tile_top);
         const float rescale = top == -INFINITY ? 0.0f : softmax_exp(top - newer);
         float tile_mass = 0.0f;
-        half8_t w_value, w_residue;  // with sixteen keys a tile the low four slots only
+        half8_t w_value, w_residue, w_small;  // with sixteen keys a tile the low four slots only; w_small: the weights * 2^-11, for the values' residues
 #pragma unroll
-        for (int i = 0; i < 8; i++) w_value[i] = (_Float16)0.0f, w_residue[i] = (_Float16)0.0f;
+        for (int i = 0; i < 8; i++) w_value[i] = (_Float16)0.0f, w_residue[i] = (_Float16)0.0f, w_small[i] = (_Float16)0.0f;
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
 #pragma unroll
@@ -655,24 +735,35 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
                 const _Float16 high = (_Float16)raised;
                 w_value[4 * kb + e] = high;
                 w_residue[4 * kb + e] = (_Float16)(raised - (float)high);
+                if constexpr (CE == NH_F32) w_small[4 * kb + e] = (_Float16)(raised * (1.0f / 2048.0f));
             }
         tile_mass += __shfl_xor(tile_mass, 16, 64);
         tile_mass += __shfl_xor(tile_mass, 32, 64);
         mass = fmaf(mass, rescale, tile_mass);
         top = newer;
-        // ---- the tile's value rows, transposed, into this wave's corner of LDS
+        // ---- the tile's value rows, transposed, into this wave's corner of LDS (single states: the values' plane, then their
+        // residues' plane through the same corner)
+        u32x4 v_words[PIECES], v_fine[PIECES];
 #pragma unroll
         for (int i = 0; i < PIECES; i++) {
-            const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
-            // rows past the walked keys may hold anything, and a weight of zero does not silence a NaN
-            const uint32_t keep = tile + key < last ? 0xffffffffu : 0u;
-            const uint32_t words[4] = {vraw[i].x & keep, vraw[i].y & keep, vraw[i].z & keep, vraw[i].w & keep};
-            // groups of four keys change places by the channel block (part / 4): the sixteen parts a store instruction
-            // touches would otherwise share four banks
-            const uint32_t column = (((key >> 2) ^ (part >> 2)) << 2) | (key & 3u);
-#pragma unroll
-            for (int j = 0; j < 8; j++) vt[wave][part * 8u + j][column] = (uint16_t)(words[j >> 1] >> (16 * (j & 1)));
+            v_fine[i] = u32x4{0u, 0u, 0u, 0u};
+            states_as_halves<CE, WORDS>(vraw[i], v_words[i], v_fine[i]);
         }
+        auto stage_plane = [&](const u32x4 (&plane_words)[PIECES]) {
+#pragma unroll
+            for (int i = 0; i < PIECES; i++) {
+                const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
+                // rows past the walked keys may hold anything, and a weight of zero does not silence a NaN
+                const uint32_t keep = tile + key < last ? 0xffffffffu : 0u;
+                const uint32_t words[4] = {plane_words[i].x & keep, plane_words[i].y & keep, plane_words[i].z & keep, plane_words[i].w & keep};
+                // groups of four keys change places by the channel block (part / 4): the sixteen parts a store instruction
+                // touches would otherwise share four banks
+                const uint32_t column = (((key >> 2) ^ (part >> 2)) << 2) | (key & 3u);
+#pragma unroll
+                for (int j = 0; j < 8; j++) vt[wave][part * 8u + j][column] = (uint16_t)(words[j >> 1] >> (16 * (j & 1)));
+            }
+        };
+        stage_plane(v_words);
         if (next < last) fetch_values(next);
         __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see these writes
         // ---- values
@@ -695,7 +786,25 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
                 acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(values, second, acc[d], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_wave_barrier();  // the next tile overwrites the corner
+        __builtin_amdgcn_wave_barrier();  // the next plane, or the next tile, overwrites the corner
+        if constexpr (CE == NH_F32) {
+            stage_plane(v_fine);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int d = 0; d < BLOCKS; d++) {
+                const uint2 low = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * (kq ^ (d >> 1))]);
+                if constexpr (TK == 32) {
+                    const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
+                    const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
+                    acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_small, acc[d], 0, 0, 0);
+                } else {
+                    typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+                    const half4_t third = {w_small[0], w_small[1], w_small[2], w_small[3]};
+                    acc[d] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, low), third, acc[d], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
     }
     // ---- the four waves meet: register e of block d is channel 16 d + 4 kq + e of this lane's column
     // a wave's sums are weighed by e^(its top - the largest of the four) before they leave its registers: the four tops and
@@ -837,9 +946,16 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
     if (p.groups > (uint32_t)MAX_GROUPS) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides %d", p.groups, MAX_GROUPS);
     uint32_t units = a.kv_heads * a.batch * a.rows;
     if (!units) return NH_OK;
-    if (a.cache_element != NH_F16) {
-        if (a.cache_element != NH_F32 && a.cache_element != NH_BF16)
-            return fail(NH_E_ARGUMENT, "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid", a.cache_element);
+    if (a.cache_element != NH_F16 && a.cache_element != NH_F32 && a.cache_element != NH_BF16)
+        return fail(NH_E_ARGUMENT, "a cache holds keys and values in single, half or bfloat16 storage, and element %d carries another grid", a.cache_element);
+    // one query row a plane over single or bfloat16 states rides the matrix cores too (NEURA_HIP_ATTENTION_ANY=1: the plain fp32 kernel)
+    const char *const asked = a.cache_element != NH_F16 ? getenv("NEURA_HIP_ATTENTION_ANY") : nullptr;  // read at every launch: the tests switch it
+    const bool plain_states = asked && asked[0] == '1';
+    const bool decode_tiles = a.rows == 1 && (a.width == 64 || a.width == 128) && p.groups <= 16 && ((uintptr_t)a.cache_k & 15u) == 0 &&
+                              ((uintptr_t)a.cache_v & 15u) == 0 && ((uintptr_t)a.q & 15u) == 0 && a.q_sh % 4 == 0 && a.q_sb % 4 == 0;
+    const bool fill_tiles = a.rows >= 4 && (a.width == 64 || a.width == 128) && p.groups >= 1 && ((uintptr_t)a.out & 15u) == 0 && a.o_sh % 4 == 0 &&
+                            a.o_sb % 4 == 0 && a.o_sr % 4 == 0 && ((uintptr_t)a.cache_k & 15u) == 0 && ((uintptr_t)a.cache_v & 15u) == 0;
+    if (a.cache_element != NH_F16 && (plain_states || !(decode_tiles || fill_tiles))) {
         if (p.groups > 16u) return fail(NH_E_ARGUMENT, "%u query heads share a key head where this kernel rides 16", p.groups);
         // sections of at most ANY_KEYS keys, enough of them to fill the device where the units alone do not
         uint32_t sections = (a.keys + ANY_KEYS - 1u) / ANY_KEYS;
@@ -863,18 +979,21 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
         return NH_OK;
     }
     // a chunk of query rows goes to the matrix cores
-    {
-        const bool aligned = ((uintptr_t)a.out & 15u) == 0 && a.o_sh % 4 == 0 && a.o_sb % 4 == 0 && a.o_sr % 4 == 0 && ((uintptr_t)a.cache_k & 15u) == 0 &&
-                             ((uintptr_t)a.cache_v & 15u) == 0;
-        if (aligned && a.rows >= 4 && (a.width == 64 || a.width == 128) && p.groups >= 1) {
-            const uint32_t rows_per_wave = 32u / p.groups;
-            dim3 grid(a.kv_heads * a.batch, (a.rows + 4u * rows_per_wave - 1u) / (4u * rows_per_wave));
-            p.sections = 1;
-            if (a.width == 64) hipLaunchKernelGGL(attention_tile_kernel<64>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
-            else hipLaunchKernelGGL(attention_tile_kernel<128>, grid, dim3(256), 0, d->stream, p, rows_per_wave);
-            NH_HIP(hipGetLastError());
-            return NH_OK;
-        }
+    if (fill_tiles) {
+        const uint32_t rows_per_wave = 32u / p.groups;
+        dim3 grid(a.kv_heads * a.batch, (a.rows + 4u * rows_per_wave - 1u) / (4u * rows_per_wave));
+        p.sections = 1;
+#define FILL_TILE(WIDTH)                                                                                                                           \
+    do {                                                                                                                                           \
+        if (a.cache_element == NH_F16) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F16>), grid, dim3(256), 0, d->stream, p, rows_per_wave);   \
+        else if (a.cache_element == NH_BF16) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_BF16>), grid, dim3(256), 0, d->stream, p, rows_per_wave); \
+        else hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F32>), grid, dim3(256), 0, d->stream, p, rows_per_wave);                             \
+    } while (0)
+        if (a.width == 64) FILL_TILE(64);
+        else FILL_TILE(128);
+#undef FILL_TILE
+        NH_HIP(hipGetLastError());
+        return NH_OK;
     }
     // one query row a plane: the group's query heads are the columns of the matrix cores
     {
@@ -903,9 +1022,15 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
             dim3 grid(planes, p.sections);
             if (p.q_sh > UINT32_MAX || p.q_sb > UINT32_MAX || p.batch > 0xffffu) return fail(NH_E_ARGUMENT, "query strides and planes past what the decode attention takes");
             const uint32_t batch_groups = (p.batch << 16) | p.groups;
-#define DECODE_TILE(WIDTH, TK)                                                                                                                                   \
-    hipLaunchKernelGGL((attention_decode_tile_kernel<WIDTH, TK>), grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh, \
+#define DECODE_TILE_OF(WIDTH, TK, CE)                                                                                                                            \
+    hipLaunchKernelGGL((attention_decode_tile_kernel<WIDTH, TK, CE>), grid, dim3(256), 0, d->stream, p.cursor, p.q, p.cache_k, p.cache_v, (uint32_t)p.q_sh, \
                        (uint32_t)p.q_sb, p.keys, p.sections, p.capacity, batch_groups, p)
+#define DECODE_TILE(WIDTH, TK)                                                                                                                                   \
+    do {                                                                                                                                                         \
+        if (a.cache_element == NH_F16) DECODE_TILE_OF(WIDTH, TK, NH_F16);                                                                                        \
+        else if (a.cache_element == NH_BF16) DECODE_TILE_OF(WIDTH, TK, NH_BF16);                                                                                 \
+        else DECODE_TILE_OF(WIDTH, TK, NH_F32);                                                                                                                  \
+    } while (0)
             if (a.width == 64) {
                 if (thin) DECODE_TILE(64, 16);
                 else DECODE_TILE(64, 32);
@@ -914,6 +1039,7 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
                 else DECODE_TILE(128, 32);
             }
 #undef DECODE_TILE
+#undef DECODE_TILE_OF
             NH_HIP(hipGetLastError());
             if (p.sections > 1 && leave) {
                 *a.unmerged = SectionSums{p.partial, p.sections, p.groups, a.width};

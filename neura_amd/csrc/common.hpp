@@ -123,6 +123,7 @@ struct RopeFusion {
     uint32_t width, q_rows, k_rows, capacity;
     uint32_t positions;  // rows of the two tables
     uint32_t ring;       // 0, or the span of a ring cache: position p is written to slot p % ring
+    int32_t element = NH_F16;  // what the two states hold (NH_F16, NH_BF16 or NH_F32: cache_k and cache_v then point at numbers of that size)
 };
 
 // NH_FETCH(p.a, p.b, ...): every scalar load of the named kernel parameters goes out at once, before the kernel's first

@@ -306,7 +306,7 @@ __device__ __forceinline__ void rotate_and_store(const GemvParams &p, float tota
             const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
             uint16_t *cache = key ? p.rope_k : p.rope_v;
             const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
-            cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
+            state_store(cache, p.rope_element, ((uint64_t)head * p.rope_capacity + slot) * p.rope_width + channel, value);
         }
     }
 }
@@ -1138,7 +1138,7 @@ __global__ __launch_bounds__(256) void gemv_staged_kernel(GEMV_LEAD_PARAMETERS) 
             const float value = p.bias[0] ? sum + p.bias[0][n] : sum;
             const uint32_t slot = p.rope_ring ? append_cursor % p.rope_ring : append_cursor;
             if (slot >= p.rope_capacity) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-            else p.rope_v[((uint64_t)(n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + n % p.rope_width] = float_to_half(value);
+            else state_store(p.rope_v, p.rope_element, ((uint64_t)(n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + n % p.rope_width, value);
         }
         __builtin_amdgcn_wave_barrier();  // the next rows overwrite the staged ones
     }
@@ -2111,7 +2111,7 @@ static int32_t launch_rows(nh_device *d, const GemvArgs &a, const float *x, floa
     if (a.rope) {
         p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
         p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
-        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring;
+        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring, p.rope_element = a.rope->element;
         p.refusal = d->refusal;
         for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
     } else if (a.bias[0] || a.bias[1] || a.bias[2]) {
@@ -2569,7 +2569,7 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
         if (RB != 1 || a.swiglu || residual || p.nblk > 16u || !a.append_value->width || a.N % a.append_value->width)
             return fail(NH_E_ARGUMENT, "this product appends no value rows (one row, one K slice, whole heads, no other epilogue)");
         p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
-        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.bias[0] = a.bias[0], p.refusal = d->refusal;
+        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.rope_element = a.append_value->element, p.bias[0] = a.bias[0], p.refusal = d->refusal;
     }
     const uint32_t most_blocks = 16u;
     p.splits = (p.nblk + most_blocks - 1) / most_blocks;

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
 
     auto fetch_the_rest = [&]() {
         __builtin_amdgcn_sched_barrier(0);
-        NH_FETCH(p.y, p.residual, p.N, p.K, p.eps, p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.bias[0], p.refusal);
+        NH_FETCH(p.y, p.residual, p.N, p.K, p.eps, p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
         __builtin_amdgcn_sched_barrier(0);
     };
     const uint32_t r = lane & 15u, q = lane >> 4, h = q >> 1, j = q & 1u;
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
                 const float value = p.bias[0] ? total + p.bias[0][n] : total;
                 const uint32_t slot = p.rope_ring ? cursor % p.rope_ring : cursor;
                 if (slot >= p.rope_capacity) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
-                else p.rope_v[((uint64_t)((uint32_t)n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + (uint32_t)n % p.rope_width] = float_to_half(value);
+                else state_store(p.rope_v, p.rope_element, ((uint64_t)((uint32_t)n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + (uint32_t)n % p.rope_width, value);
             }
         }
         parity ^= 1u;
@@ -450,7 +450,7 @@ int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &a) {
     p.digits_in = a.digits_in;
     if (a.append_value) {
         p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
-        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.bias[0] = a.bias[0], p.refusal = d->refusal;
+        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.rope_element = a.append_value->element, p.bias[0] = a.bias[0], p.refusal = d->refusal;
     }
     p.row_bytes = (uint32_t)payload_bytes(a.element, a.K);
     p.nblk = a.K / 256u;

@@ -32,6 +32,7 @@ struct GemvParams {
     const uint32_t *rope_cursor;
     uint16_t *rope_k, *rope_v;
     uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
+    int32_t rope_element;  // what the states hold: NH_F16 (0 is NH_F32: launchers always name it), NH_BF16 or NH_F32
     uint32_t *refusal;
     const float *bias[3];  // per stacked matrix or nullptr (decode kernel with the rotation folded in only)
     // 16-row tile kernel: activations handed from one product to the next as the digit planes the matrix cores take
@@ -58,7 +59,7 @@ __device__ __forceinline__ void fetch_parameters(const GemvParams &p, bool rope 
              p.digits_out);
     if (rope)
         NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions, p.rope_ring,
-                 p.bias[0], p.bias[1], p.bias[2], p.refusal);
+                 p.rope_element, p.bias[0], p.bias[1], p.bias[2], p.refusal);
 }
 
 // What a wave of a K-quant product needs before its first loads, as leading plain arguments the hardware hands over in scalar
@@ -119,6 +120,12 @@ __device__ __forceinline__ void scale_pairs(const u32x4 &hdr, const ScaleLane &s
     mn = __builtin_bit_cast(half2_t, (p_mn & s.mask_p) | ((q_mn >> 2) & s.mask_q));
 }
 
+// one number into a key or value state of `element` (crates/neura-decoder/src/cache.rs:347-348 casts as it appends)
+__device__ __forceinline__ void state_store(uint16_t *state, int32_t element, uint64_t at, float value) {
+    if (element == NH_F32) reinterpret_cast<float *>(state)[at] = value;
+    else state[at] = element == NH_BF16 ? float_to_bfloat16(value) : float_to_half(value);
+}
+
 // One rotated output of a q|k|v product that folds the rotation in: `total` is output row n (channel c of its head's first
 // half, or c + width/2 when `second`), the lane 8 further round its row of 16 holds the partner channel.  The projection's
 // bias, if it has one, comes before the rotation; q rows go to y, k rows rotated and v rows as they are to the caches as
@@ -163,7 +170,7 @@ __device__ __forceinline__ void rope_store(const GemvParams &p, float total, uin
         const uint32_t head = within / p.rope_width, channel = within % p.rope_width;
         uint16_t *cache = key ? p.rope_k : p.rope_v;
         const uint32_t slot = p.rope_ring ? position % p.rope_ring : position;  // a ring seats position p at p mod its span
-        cache[((size_t)head * p.rope_capacity + slot) * p.rope_width + channel] = float_to_half(value);
+        state_store(cache, p.rope_element, ((uint64_t)head * p.rope_capacity + slot) * p.rope_width + channel, value);
     }
 }
 

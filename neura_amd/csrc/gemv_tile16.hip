@@ -129,7 +129,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
         NH_FETCH(p.y, p.residual, p.N, p.K, p.rows, p.eps, p.digits_out);
         if (MODE == TILE16_ROPE)
             NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_width, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions,
-                     p.rope_ring, p.bias[0], p.bias[1], p.bias[2], p.refusal, p.end[0], p.end[1]);
+                     p.rope_ring, p.rope_element, p.bias[0], p.bias[1], p.bias[2], p.refusal, p.end[0], p.end[1]);
         __builtin_amdgcn_sched_barrier(0);
     };
     const uint32_t r = lane & 15u, q = lane >> 4;
@@ -1396,7 +1396,7 @@ static Tile16Launch tile16_plan(nh_device *d, const GemvArgs &a, uint32_t fixed_
     if (a.rope) {
         p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
         p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
-        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring;
+        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring, p.rope_element = a.rope->element;
         p.refusal = d->refusal;
         for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
     }

@@ -177,10 +177,10 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             a.end[0] = QW, a.end[1] = QW + KW, a.end[2] = QKV;
             a.norm_w = m->attn_norm[L], a.eps = c.eps;
             // one token of one active plane: the rotation, the biases and the cache append ride in the product's epilogue
-            // (the folded rotation appends halves: states of another element take the rotation's own kernel)
-            const bool halves = c.cache_element == NH_F16;
+            // (the epilogue casts what it appends into the states' element)
+            const bool halves = true;
             RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), reinterpret_cast<uint16_t *>(m->cache_k[L]), reinterpret_cast<uint16_t *>(m->cache_v[L]),
-                            hd, QW, QW + KW, m->capacity, m->positions, m->ring ? m->window : 0u};
+                            hd, QW, QW + KW, m->capacity, m->positions, m->ring ? m->window : 0u, c.cache_element};
             if (halves && alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
                 a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];

@@ -90,6 +90,47 @@ def test_decoders_keep_their_states_in_single_or_bfloat16(device, shape, element
     model.release(), weights.release()
 
 
+@pytest.mark.parametrize("cache_element", [0, 30], ids=["single", "bfloat16"])
+@pytest.mark.parametrize("shape,element", [(TINY, NH_Q8_0), (SMALL_Q4, NH_Q4_K)])
+def test_one_plane_steps_over_single_or_bfloat16_states_ride_the_fused_kernels(device, monkeypatch, shape, element, cache_element):
+    """One plane, one token a step: the rotation and the append ride in the q|k|v product's epilogue, which casts what it
+    appends into the states' element, and the attention walks single and bfloat16 states on the matrix cores.  Logits and
+    tokens as the oracle's over the same states, the appended rows equal to its rows, and the same steps with the rotation in
+    a kernel of its own and the plain fp32 attention (the forms these replaced) within the same bar."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # the twins launch eagerly, so the switches below are read at every step
+    fused, ref, weights_a = build(device, shape, element, batch=1, context=40, max_rows=8, seed=5, cache_element=cache_element)
+    plain, _, weights_b = build(device, shape, element, batch=1, context=40, max_rows=8, seed=5, cache_element=cache_element)
+    rng = np.random.default_rng(6)
+    prompt = rng.integers(0, shape["vocab"], 8)
+    for model in (fused, plain):
+        model.prefill(prompt, 8, [0])
+    ref.forward(prompt, 8, [0], want_logits=False)
+    token = int(rng.integers(0, shape["vocab"]))
+    for step in range(6):
+        want_logits, want = ref.forward([token], 1, [8 + step])
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1"), monkeypatch.setenv("NEURA_HIP_ATTENTION_ANY", "0")
+        got = fused.decode_step([token], [8 + step])
+        logits = fused.logits()
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "0"), monkeypatch.setenv("NEURA_HIP_ATTENTION_ANY", "1")
+        got_plain = plain.decode_step([token], [8 + step])
+        scale = np.abs(want_logits).max()
+        assert np.abs(logits - want_logits).max() <= 1e-3 * scale and np.abs(plain.logits() - want_logits).max() <= 1e-3 * scale, step
+        assert list(got) == list(got_plain) == list(want), (step, margins(want_logits))
+        token = int(got[0])
+    for layer in range(shape["layers"]):
+        for which, held in ((0, ref.cache_k), (1, ref.cache_v)):
+            rows = []
+            for model in (fused, plain):
+                got_cache = model.cache_read(layer, which).reshape(-1)
+                rows.append((got_cache.astype(np.uint32) << 16).view(np.float32) if cache_element == 30 else got_cache)
+            want_cache = (held[layer].astype(np.uint32) << 16).view(np.float32) if cache_element == 30 else held[layer]
+            bar = 1e-2 * max(1.0, np.abs(want_cache).max())
+            assert np.abs(rows[0] - want_cache).max() <= bar and np.abs(rows[1] - want_cache).max() <= bar
+            assert np.any(rows[0].reshape(fused.cache_shape)[:, 0, 8:14])  # the decode steps' rows are there
+    for held in (fused, plain, weights_a, weights_b):
+        held.release()
+
+
 def test_a_decoder_names_the_element_of_its_states(device):
     with pytest.raises(NeuraError, match="single, half or bfloat16"):
         build(device, TINY, NH_Q8_0, batch=1, context=8, cache_element=12)
