@@ -35,6 +35,33 @@ static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R, bool handed = f
 struct Tile16Unit {
     u32x4 hdr, qa, qb;
 };
+// Q5_K: a super-block is Q4_K's with the codes' fifth bits between the header and the nibbles (176 bytes: 16 of header, 32 of
+// fifth bits, 128 of nibbles; crates/neura-precision/src/ggml.rs:321-335).  Byte l of the 32 carries, in bits 2 g and 2 g + 1,
+// the fifth bits of codes l and 32 + l of group g: lane (r, q) fetches all 32 bytes beside its group's nibbles (the four lanes
+// of a row ask for the same bytes in one instruction) and sets bit 4 of its sixteen-code operands from them.  Scales,
+// minimums, digit planes and the weighing are Q4_K's.
+struct Tile16UnitFifth {
+    u32x4 hdr, qa, qb, fa, fb;  // fa, fb: the fifth bits of codes l = 0..15 and 16..31 of every group
+};
+template <bool FIFTH>
+struct Tile16UnitOf {
+    typedef Tile16Unit type;
+};
+template <>
+struct Tile16UnitOf<true> {
+    typedef Tile16UnitFifth type;
+};
+// the B operands of a step: low and high nibbles of the unit's two nibble loads, with the fifth bit where the element has one
+template <bool FIFTH, class UNIT>
+__device__ __forceinline__ void tile16_codes(const UNIT &u, uint32_t q, u32x4 &la, u32x4 &ha, u32x4 &lb, u32x4 &hb) {
+    const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
+    la = u.qa & mask, ha = (u.qa >> 4) & mask, lb = u.qb & mask, hb = (u.qb >> 4) & mask;
+    if constexpr (FIFTH) {
+        const u32x4 bit = {0x10101010u, 0x10101010u, 0x10101010u, 0x10101010u};
+        const u32x4 fa = u.fa >> (2u * q), fb = u.fb >> (2u * q);  // bit 0: the low nibble's fifth bit, bit 1: the high nibble's
+        la |= (fa << 4) & bit, ha |= (fa << 3) & bit, lb |= (fb << 4) & bit, hb |= (fb << 3) & bit;
+    }
+}
 
 //
 // R > 1: up to R activation rows (p.rows of them) meet the weights in one pass.  Every row has its own digit planes and sums in
@@ -100,21 +127,24 @@ __device__ __forceinline__ void tile16_store_word(uint32_t *at, uint32_t word) {
 // `ring`: the units in flight, the caller's (a chained launch hands them from one product to the next: with HANDS_RING the
 // fetches past this product's last unit ask for super-blocks wave, wave + NW, ... of `next_row`, this lane's weight row in
 // the first tile the workgroup walks of the product behind the seam (nullptr: it walks none), which then TAKES_RING).
-template <int NW, int D, int MODE, int R, bool HANDED, class SEAM>
-__device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const uint32_t block, const SEAM seam, Tile16Unit (&ring)[D], const uint8_t *next_row,
+template <int NW, int D, int MODE, int R, bool HANDED, class SEAM, bool FIFTH = false>
+__device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const uint32_t block, const SEAM seam, typename Tile16UnitOf<FIFTH>::type (&ring)[D], const uint8_t *next_row,
                                                uint32_t next_nblk, const uint8_t *lead_w0, const void *lead_input,
                                                const float *lead_norm_w, int32_t lead_to_w1, int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid,
                                                uint32_t lead_tiles, uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, const GemvParams &p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
     static_assert(!HANDED || (R == 1 && MODE == TILE16_PLAIN), "handed-over digit planes feed a plain product of one row");
     static_assert(!(SEAM::WAITS || SEAM::SHARED_IN || SEAM::SHARED_OUT) || R == 1, "products of one row are chained");
+    static_assert(!FIFTH || (R == 1 && !SEAM::HANDS_RING && !SEAM::TAKES_RING), "Q5_K: one row, a launch of its own");
+    typedef typename Tile16UnitOf<FIFTH>::type Unit;
+    constexpr uint32_t BLOCK_BYTES = FIFTH ? 176u : 144u, TO_NIBBLES = FIFTH ? 48u : 16u;  // a super-block, and from its start to its nibbles
     constexpr uint32_t NT = NW * 64;
     typedef int i32x4 __attribute__((ext_vector_type(4)));
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     typedef const __attribute__((address_space(1))) u32x4 *global_uint4;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nblk = lead_row_bytes / 144u;  // super-blocks a row
+    const uint32_t nblk = lead_row_bytes / BLOCK_BYTES;  // super-blocks a row
     const float *const x = static_cast<const float *>(lead_input);
     uint8_t *const digits = tile16_lds_bytes;
     const uint32_t row_digits = nblk * TILE16_BLOCK_DIGITS;  // digit planes of one activation row
@@ -209,15 +239,19 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
             exhausted = true;
         }
     };
-    auto fetch = [&](Tile16Unit &u) {
-        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * 144u;
+    auto fetch = [&](Unit &u) {
+        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * BLOCK_BYTES;
         if constexpr (SEAM::HANDS_RING) {
             if (exhausted && next_row) at = next_row + (size_t)min(wave + NW * (uint32_t)max(beyond, 0), next_nblk - 1u) * 144u;
             if (exhausted) beyond++;
         }
         u.hdr = *(global_uint4)(uintptr_t)(at - q * 32u);
-        u.qa = *(global_uint4)(uintptr_t)(at + 16u);
-        u.qb = *(global_uint4)(uintptr_t)(at + 32u);
+        u.qa = *(global_uint4)(uintptr_t)(at + TO_NIBBLES);
+        u.qb = *(global_uint4)(uintptr_t)(at + TO_NIBBLES + 16u);
+        if constexpr (FIFTH) {
+            u.fa = *(global_uint4)(uintptr_t)(at - q * 32u + 16u);
+            u.fb = *(global_uint4)(uintptr_t)(at - q * 32u + 32u);
+        }
         advance();
     };
     // TAKES_RING: the product before asked for this wave's first D units; the fetches here go on behind them
@@ -565,14 +599,14 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
         f32x4 s;
         uint32_t sc, mn, dd;
     };
-    auto multiply = [&](const Tile16Unit &u, uint32_t b, Step &st) {
+    auto multiply = [&](const Unit &u, uint32_t b, Step &st) {
         const uint8_t *at = abase + (size_t)b * astride;
         const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
         const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
         st.s = sums[b * 4u + q];
-        const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
-        const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
-        const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
+        u32x4 la_, ha_, lb_, hb_;
+        tile16_codes<FIFTH>(u, q, la_, ha_, lb_, hb_);
+        const i32x4 la = (i32x4)la_, ha = (i32x4)ha_, lb = (i32x4)lb_, hb = (i32x4)hb_;
         half2_t sc, mn;
         scale_pairs(u.hdr, lane_scales, sc, mn);
         st.sc = __builtin_bit_cast(uint32_t, sc), st.mn = __builtin_bit_cast(uint32_t, mn), st.dd = u.hdr.x;
@@ -600,14 +634,14 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
         f32x4 low, high;  // (sum, scale) of chunks 0, 1 and of chunks 2, 3 of the lane's group
         uint32_t sc, mn, dd;
     };
-    auto multiply_handed = [&](const Tile16Unit &u, uint32_t b, HandedStep &st) {
+    auto multiply_handed = [&](const Unit &u, uint32_t b, HandedStep &st) {
         const uint8_t *at = abase + (size_t)b * astride;
         const i32x4 a00 = *reinterpret_cast<const i32x4 *>(at), a01 = *reinterpret_cast<const i32x4 *>(at + 48);
         const i32x4 a10 = *reinterpret_cast<const i32x4 *>(at + 96), a11 = *reinterpret_cast<const i32x4 *>(at + 144);
         st.low = sums[b * 8u + 2u * q], st.high = sums[b * 8u + 2u * q + 1u];
-        const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
-        const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
-        const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
+        u32x4 la_, ha_, lb_, hb_;
+        tile16_codes<FIFTH>(u, q, la_, ha_, lb_, hb_);
+        const i32x4 la = (i32x4)la_, ha = (i32x4)ha_, lb = (i32x4)lb_, hb = (i32x4)hb_;
         half2_t sc, mn;
         scale_pairs(u.hdr, lane_scales, sc, mn);
         st.sc = __builtin_bit_cast(uint32_t, sc), st.mn = __builtin_bit_cast(uint32_t, mn), st.dd = u.hdr.x;
@@ -638,7 +672,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
     for (int g = 0; g < G; g++)
 #pragma unroll
         for (int k = 0; k < 4; k++) a[g][k] = i32x4{0, 0, 0, 0};
-    auto step_rows = [&](Tile16Unit &u, uint32_t b) {
+    auto step_rows = [&](Unit &u, uint32_t b) {
         const u32x4 mask = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu};
         const i32x4 la = (i32x4)(u.qa & mask), ha = (i32x4)((u.qa >> 4) & mask);
         const i32x4 lb = (i32x4)(u.qb & mask), hb = (i32x4)((u.qb >> 4) & mask);
@@ -831,14 +865,14 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
 // so that the hardware can hand them over in scalar registers when it starts the wave (the file is built with
 // -amdgpu-kernarg-preload-count): the wave's first loads then go out without waiting for a load of its parameters
 // (about 0.5 us); everything else sits in `p` and is fetched meanwhile.  `input` is x, or the digit planes with HANDED.
-template <int NW, int D, int MODE, int R, bool HANDED = false>
+template <int NW, int D, int MODE, int R, bool HANDED = false, bool FIFTH = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, int32_t lead_to_w1,
                                                                   int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
                                                                   uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t tile16_lds_bytes[];
-    Tile16Unit ring[D];
-    tile16_product<NW, D, MODE, R, HANDED>(tile16_lds_bytes, blockIdx.x, NoSeam{}, ring, nullptr, 0u, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes, lead_grid,
-                                           lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
+    typename Tile16UnitOf<FIFTH>::type ring[D];
+    tile16_product<NW, D, MODE, R, HANDED, NoSeam, FIFTH>(tile16_lds_bytes, blockIdx.x, NoSeam{}, ring, nullptr, 0u, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2,
+                                                          lead_row_bytes, lead_grid, lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
@@ -1199,8 +1233,12 @@ constexpr uint32_t TILE16_MOST_ROWS = 4;
 static uint32_t tile16_row_form(uint32_t rows) { return rows <= 1u ? 1u : (rows <= 2u ? 2u : 4u); }
 
 bool tile16_takes(const GemvArgs &a) {
-    if (a.element != NH_Q4_K || a.rows < 1 || a.rows > TILE16_MOST_ROWS || a.K % 256u != 0 || a.K == 0) return false;
+    if ((a.element != NH_Q4_K && a.element != NH_Q5_K) || a.rows < 1 || a.rows > TILE16_MOST_ROWS || a.K % 256u != 0 || a.K == 0) return false;
     if (env_int("NEURA_HIP_TILE16", 1) == 0 || env_int("NEURA_HIP_MFMA", 1) != 1) return false;
+    // Q5_K (one row): the same tiles with the fifth bit beside the nibble; NEURA_HIP_Q5K_TILE16=0 leaves it to the staged kernel
+    if (a.element == NH_Q5_K && (a.rows != 1 || a.append_value || a.merge || env_int("NEURA_HIP_Q5K_TILE16", 1) == 0)) return false;
+    for (int m = 0; m < 3; m++)
+        if (a.W[m] && ((uintptr_t)a.W[m] & 15u)) return false;
     if (a.rows > 1 && (a.rope || a.rows > (uint32_t)env_int("NEURA_HIP_TILE16_ROWS", (int)TILE16_MOST_ROWS))) return false;
     if (a.rows > 1 && (env_int("NEURA_HIP_MFMA32", 1) == 2 || env_int("NEURA_HIP_F16_TILES", 1) == 2)) return false;  // another form is forced
     if (((uintptr_t)a.x & 15u) || (a.norm_w && ((uintptr_t)a.norm_w & 15u))) return false;
@@ -1321,15 +1359,15 @@ int32_t launch_rows4(nh_device *d, const GemvArgs &a) {
     return NH_OK;
 }
 
-template <int NW, int D, int MODE, int R, bool HANDED = false>
+template <int NW, int D, int MODE, int R, bool HANDED = false, bool FIFTH = false>
 static hipError_t launch_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
     static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED, FIFTH>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
+    hipLaunchKernelGGL((gemv_q4k_tile16_kernel<NW, D, MODE, R, HANDED, FIFTH>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
                        HANDED ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x), p.norm_w, (int32_t)((p.W[1] - p.W[0]) / 16),
                        (int32_t)((p.W[2] - p.W[0]) / 16), p.row_bytes, grid, p.row_groups, MODE == TILE16_ROPE ? p.rope_width : p.tile_rows, p.end[0], p.end[1], p);
     return hipGetLastError();
@@ -1367,6 +1405,18 @@ static hipError_t launch_tile16_mode(nh_device *d, const GemvParams &p, uint32_t
         }
     }
     return launch_tile16_rows<MODE, 1>(d, p, waves, grid, lds);
+}
+
+// Q5_K: one row, every mode
+template <int MODE, bool HANDED>
+static hipError_t launch_tile16_fifth(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
+    switch (waves) {
+    case 4: return launch_tile16_instance<4, 2, MODE, 1, HANDED, true>(d, p, grid, lds);
+    case 6: return launch_tile16_instance<6, 2, MODE, 1, HANDED, true>(d, p, grid, lds);
+    case 7: return launch_tile16_instance<7, 2, MODE, 1, HANDED, true>(d, p, grid, lds);
+    case 8: return launch_tile16_instance<8, 2, MODE, 1, HANDED, true>(d, p, grid, lds);
+    default: return launch_tile16_instance<16, 2, MODE, 1, HANDED, true>(d, p, grid, lds);
+    }
 }
 
 // what a launch of the 16-row tile product is made of: the parameter block, waves a workgroup, workgroups, LDS
@@ -1436,10 +1486,17 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     const uint32_t waves = plan.waves, grid = plan.grid;
     const size_t lds = plan.lds;
     profile_mark(d);
-    hipError_t launched = a.digits_in ? launch_tile16_handed(d, p, waves, grid, lds)
-                          : a.swiglu ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
-                          : a.rope ? launch_tile16_mode<TILE16_ROPE>(d, p, waves, grid, lds)
-                                   : launch_tile16_mode<TILE16_PLAIN>(d, p, waves, grid, lds);
+    hipError_t launched;
+    if (a.element == NH_Q5_K)
+        launched = a.digits_in ? launch_tile16_fifth<TILE16_PLAIN, true>(d, p, waves, grid, lds)
+                   : a.swiglu  ? launch_tile16_fifth<TILE16_SWIGLU, false>(d, p, waves, grid, lds)
+                   : a.rope    ? launch_tile16_fifth<TILE16_ROPE, false>(d, p, waves, grid, lds)
+                               : launch_tile16_fifth<TILE16_PLAIN, false>(d, p, waves, grid, lds);
+    else
+        launched = a.digits_in ? launch_tile16_handed(d, p, waves, grid, lds)
+                   : a.swiglu  ? launch_tile16_mode<TILE16_SWIGLU>(d, p, waves, grid, lds)
+                   : a.rope    ? launch_tile16_mode<TILE16_ROPE>(d, p, waves, grid, lds)
+                               : launch_tile16_mode<TILE16_PLAIN>(d, p, waves, grid, lds);
     NH_HIP(launched);
     profile_mark(d);
     if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
@@ -1530,7 +1587,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_chain_kernel(ChainParams c) {
 }
 
 static bool chain_stage_takes(const GemvArgs &a) {
-    if (!tile16_takes(a) || a.rows != 1) return false;
+    if (a.element != NH_Q4_K || !tile16_takes(a) || a.rows != 1) return false;
     return tile16_lds(a.K / 256u, 8u, 1u, a.digits_in != nullptr) <= 160u * 1024u;
 }
 
