@@ -214,6 +214,10 @@ constexpr uint32_t MERGED_SECTIONS_MOST = 16;  // sections such a product merges
 // whether `producer` (a SwiGLU product of one row) can hand its outputs to `consumer` as digit planes, and the bytes they take
 bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer);
 size_t gemv_digit_bytes(uint32_t K);
+// A Q4_K q|k product that folds the rotation in and the Q6_K value projection that appends its own rows, both over the same
+// activation row, as one launch (a layer of a Q4_K_M file whose value projection is stored in Q6_K): gemv_pairs() says whether.
+bool gemv_pairs(nh_device *d, const GemvArgs &rotated, const GemvArgs &value);
+int32_t launch_gemv_pair(nh_device *d, const GemvArgs &rotated, const GemvArgs &value);
 // Several dependent one-row Q4_K products as one launch with seams between them: attn_output (`lead`, or nullptr), gate|up
 // handing its digit planes to ffn_down, and behind them the next q|k|v with the rotation folded in or the head (`trail`, or
 // nullptr).  gemv_chains() says whether launch_chain takes them.

@@ -205,5 +205,11 @@ int32_t launch_rows4(nh_device *d, const GemvArgs &args);
 // one activation row against a Q6_K matrix on the same tiles (gemv_q6k_tile16.hip)
 bool q6k_tile16_takes(const GemvArgs &args);
 int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &args);
+struct Q6kLaunch {  // what a launch of it is made of: the parameter block, waves a workgroup, workgroups, LDS
+    GemvParams p;
+    uint32_t waves, grid;
+    size_t lds;
+};
+Q6kLaunch q6k_tile16_plan(nh_device *d, const GemvArgs &args);
 
 }  // namespace nh

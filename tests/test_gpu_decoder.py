@@ -775,11 +775,14 @@ def test_attention_sections_merged_by_the_output_projection_match_the_fold(devic
         held.release()
 
 
-def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, monkeypatch):
+@pytest.mark.parametrize("pair", ["1", "0"], ids=["one launch", "two launches"])
+def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, monkeypatch, pair):
     """Where q|k go out rotated from one product and the value projection is stored otherwise (layer 0 of the Q4_K_M-like
-    mix: Q6_K), the value product casts its rows (+ bias) into the value state itself; NEURA_HIP_APPEND_VALUE=0 leaves that
-    to the append kernel.  The same sums either way: states and logits equal bit for bit, and the oracle's tokens."""
+    mix: Q6_K), the value product casts its rows (+ bias) into the value state itself -- beside the q|k product in one
+    launch, or (NEURA_HIP_PAIR=0) in a launch of its own; NEURA_HIP_APPEND_VALUE=0 leaves the cast to the append kernel.
+    The same sums either way: states and logits equal bit for bit, and the oracle's tokens."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    monkeypatch.setenv("NEURA_HIP_PAIR", pair)
     shape = SMALL_Q4
     tensors = list(synth.model_tensors(shape, NH_Q4_K, np.random.default_rng(21), mode="normal", elements=MIXED, biases=(0, 1)))
     host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
