@@ -1387,9 +1387,7 @@ template <int MODE, int R>
 static hipError_t launch_tile16_rows(nh_device *d, const GemvParams &p, uint32_t waves, uint32_t grid, size_t lds) {
     switch (waves) {
     case 4: return launch_tile16_instance<4, 2, MODE, R>(d, p, grid, lds);
-    case 6:
-        if constexpr (R == 1) return launch_tile16_instance<6, 2, MODE, 1>(d, p, grid, lds);
-        else return launch_tile16_instance<7, 2, MODE, R>(d, p, grid, lds);
+    case 6: return launch_tile16_instance<6, 2, MODE, R>(d, p, grid, lds);
     case 7: return launch_tile16_instance<7, 2, MODE, R>(d, p, grid, lds);
     case 8: return launch_tile16_instance<8, 2, MODE, R>(d, p, grid, lds);
     default: return launch_tile16_instance<16, 2, MODE, R>(d, p, grid, lds);
@@ -1457,7 +1455,8 @@ static Tile16Launch tile16_plan(nh_device *d, const GemvArgs &a, uint32_t fixed_
     plan.waves = fixed_waves ? fixed_waves : (p.nblk <= 8u ? 4u : (p.nblk <= 14u ? 7u : (p.nblk <= 32u || a.digits_in ? 8u : 16u)));
     // one row against short rows (the 1.5B shape's 1536 columns are six super-blocks): a wave a super-block keeps more bytes in
     // flight a compute unit than four waves of two steps -- measured on that shape, a decode step 0.963 -> 0.898 ms
-    if (!fixed_waves && a.rows == 1 && !a.digits_in && p.nblk > 4u && p.nblk <= 8u) plan.waves = p.nblk <= 6u ? 6u : 8u;
+    // (two to four rows take the same waves: a row of theirs is then, bit for bit, what the one-row product gives)
+    if (!fixed_waves && !a.digits_in && p.nblk > 4u && p.nblk <= 8u) plan.waves = p.nblk <= 6u ? 6u : 8u;
     // units of work: tiles, or with SwiGLU pairs (a gate tile and the up tile behind it); every workgroup takes the same
     // number of them, one workgroup a compute unit when there are that many
     // A plain tile holds the number of rows, 16 down to 12, that leaves the fewest compute units idle in the last round.
