@@ -1,22 +1,22 @@
-// The Q6_K product of one activation row on 16-row tiles of the 16x16x64 integer MFMA: kernel and launcher.
+// The Q6_K and Q3_K products of one activation row on 16-row tiles of the 16x16x64 integer MFMA: kernel and launcher.
 // Built with the matrix-core results in vector registers (-amdgpu-mfma-vgpr-form).
 #include "gemv_q6k_tile16.hpp"
 
 namespace nh {
 
-template <int NW, bool HANDED, bool SWIGLU = false>
+template <int NW, bool HANDED, bool SWIGLU = false, int ELEMENT = NH_Q6_K>
 __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, uint32_t lead_row_bytes,
                                                                   uint32_t lead_grid, uint32_t lead_tiles, uint32_t lead_tile_rows, int32_t lead_to_w1, GemvParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t q6k_lds_bytes[];
-    q6k_tile16_product<NW, HANDED, SWIGLU>(q6k_lds_bytes, blockIdx.x, lead_w0, lead_input, lead_norm_w, lead_row_bytes, lead_grid, lead_tiles, lead_tile_rows, lead_to_w1, p);
+    q6k_tile16_product<NW, HANDED, SWIGLU, ELEMENT>(q6k_lds_bytes, blockIdx.x, lead_w0, lead_input, lead_norm_w, lead_row_bytes, lead_grid, lead_tiles, lead_tile_rows, lead_to_w1, p);
 }
 
-// NEURA_HIP_Q6K_TILE16=0 keeps the kernel out (the staged kernel then takes Q6_K as before).  Otherwise it takes every Q6_K product
+// NEURA_HIP_Q6K_TILE16=0 keeps the kernel out (the staged kernel then takes Q6_K and Q3_K as before).  Otherwise it takes every such product
 // of one row and one matrix that ends on a tile boundary (or a gate and an up matrix with SwiGLU), with no other epilogue than the
 // residual or the cast of a value projection's rows into the value state: the head, ffn_down, attn_v and attn_output of a k-quant
 // mix, gate|up of a file stored in Q6_K throughout.  What folds the rotation in stays with the staged kernel.
 bool q6k_tile16_takes(const GemvArgs &a) {
-    if (a.element != NH_Q6_K || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.rope || a.merge || a.digits_out) return false;
+    if ((a.element != NH_Q6_K && a.element != NH_Q3_K) || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.rope || a.merge || a.digits_out) return false;
     if (env_int("NEURA_HIP_Q6K_TILE16", 1) == 0) return false;
     if (a.swiglu) {  // gate and up stacked: pairs of whole tiles, no other epilogue
         if (!a.W[1] || a.W[2] || a.residual || a.append_value || a.digits_in || a.end[0] != a.N / 2u || a.N % 32u != 0) return false;
@@ -42,15 +42,15 @@ bool q6k_tile16_takes(const GemvArgs &a) {
     return q6k_tile16_lds(nblk, nblk > 32u && !a.digits_in ? 16u : 8u) <= 160u * 1024u;
 }
 
-template <int NW, bool HANDED, bool SWIGLU = false>
+template <int NW, bool HANDED, bool SWIGLU = false, int ELEMENT = NH_Q6_K>
 static hipError_t launch_q6k_tile16_instance(nh_device *d, const GemvParams &p, uint32_t grid, size_t lds) {
     static bool raised = false;  // a workgroup may hold more than the default 64 KiB of LDS once the kernel says so
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU, ELEMENT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
+    hipLaunchKernelGGL((gemv_q6k_tile16_kernel<NW, HANDED, SWIGLU, ELEMENT>), dim3(grid), dim3(NW * 64), lds, d->stream, p.W[0],
                        HANDED ? static_cast<const void *>(p.digits_in) : static_cast<const void *>(p.x), p.norm_w, p.row_bytes, grid, p.row_groups, p.tile_rows,
                        (int32_t)((p.W[1] - p.W[0]) / 16), p);
     return hipGetLastError();
@@ -94,31 +94,34 @@ Q6kLaunch q6k_tile16_plan(nh_device *d, const GemvArgs &a) {
     return plan;
 }
 
-int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &a) {
-    const Q6kLaunch plan = q6k_tile16_plan(d, a);
+template <int ELEMENT>
+static hipError_t launch_q6k_tile16_of(nh_device *d, const GemvArgs &a, const Q6kLaunch &plan) {
     const GemvParams &p = plan.p;
     const uint32_t waves = plan.waves, grid = plan.grid;
     const size_t lds = plan.lds;
-    profile_mark(d);
-    hipError_t launched;
     if (a.swiglu) {
-        launched = waves == 4u ? launch_q6k_tile16_instance<4, false, true>(d, p, grid, lds)
-                   : waves == 7u ? launch_q6k_tile16_instance<7, false, true>(d, p, grid, lds)
-                   : waves == 8u ? launch_q6k_tile16_instance<8, false, true>(d, p, grid, lds)
-                                 : launch_q6k_tile16_instance<16, false, true>(d, p, grid, lds);
-    } else if (a.digits_in) {
-        launched = waves == 4u ? launch_q6k_tile16_instance<4, true>(d, p, grid, lds)
-                   : waves == 7u ? launch_q6k_tile16_instance<7, true>(d, p, grid, lds)
-                                 : launch_q6k_tile16_instance<8, true>(d, p, grid, lds);
-    } else {
-        launched = waves == 4u ? launch_q6k_tile16_instance<4, false>(d, p, grid, lds)
-                   : waves == 7u ? launch_q6k_tile16_instance<7, false>(d, p, grid, lds)
-                   : waves == 8u ? launch_q6k_tile16_instance<8, false>(d, p, grid, lds)
-                                 : launch_q6k_tile16_instance<16, false>(d, p, grid, lds);
+        return waves == 4u   ? launch_q6k_tile16_instance<4, false, true, ELEMENT>(d, p, grid, lds)
+               : waves == 7u ? launch_q6k_tile16_instance<7, false, true, ELEMENT>(d, p, grid, lds)
+               : waves == 8u ? launch_q6k_tile16_instance<8, false, true, ELEMENT>(d, p, grid, lds)
+                             : launch_q6k_tile16_instance<16, false, true, ELEMENT>(d, p, grid, lds);
     }
-    NH_HIP(launched);
+    if (a.digits_in) {
+        return waves == 4u   ? launch_q6k_tile16_instance<4, true, false, ELEMENT>(d, p, grid, lds)
+               : waves == 7u ? launch_q6k_tile16_instance<7, true, false, ELEMENT>(d, p, grid, lds)
+                             : launch_q6k_tile16_instance<8, true, false, ELEMENT>(d, p, grid, lds);
+    }
+    return waves == 4u   ? launch_q6k_tile16_instance<4, false, false, ELEMENT>(d, p, grid, lds)
+           : waves == 7u ? launch_q6k_tile16_instance<7, false, false, ELEMENT>(d, p, grid, lds)
+           : waves == 8u ? launch_q6k_tile16_instance<8, false, false, ELEMENT>(d, p, grid, lds)
+                         : launch_q6k_tile16_instance<16, false, false, ELEMENT>(d, p, grid, lds);
+}
+
+int32_t launch_q6k_tile16(nh_device *d, const GemvArgs &a) {
+    const Q6kLaunch plan = q6k_tile16_plan(d, a);
     profile_mark(d);
-    if (d->profile) d->profile_bytes += (uint64_t)a.N * p.row_bytes;
+    NH_HIP(a.element == NH_Q3_K ? launch_q6k_tile16_of<NH_Q3_K>(d, a, plan) : launch_q6k_tile16_of<NH_Q6_K>(d, a, plan));
+    profile_mark(d);
+    if (d->profile) d->profile_bytes += (uint64_t)a.N * plan.p.row_bytes;
     return NH_OK;
 }
 

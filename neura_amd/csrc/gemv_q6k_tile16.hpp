@@ -37,17 +37,35 @@ namespace nh {
 // kernel's too); loads run two units ahead across tile boundaries, every wave walks whole rounds of two steps; the finishing
 // wave changes from tile to tile; epilogues: plain (+ residual, in place by one fire-and-forget add), SwiGLU over a gate tile
 // and the up tile behind it, or the cast of a value projection's rows into the value state.
+//
+// Q3_K (ELEMENT = NH_Q3_K; crates/neura-precision/src/ggml.rs:291-306) has the same sixteen scale groups of 16 in a super-block
+// of 110 bytes: 32 bytes of third bits, 64 of bit pairs, twelve bytes of 6-bit scales and d.  Lane (r, q) takes the 16 bytes of
+// bit pairs 32 h + 16 j .. and the 16 third-bit bytes 16 j .., and its four B operands are the codes 0..7
+//     ((pairs >> 2 g) & 3) | (((third >> (4 h + g)) & 1) << 2)     of elements 128 h + 32 g + 16 j .. + 15, g = 0..3
+// whose offset of 4 comes off against the activations' sums; the scales (stored 32 too large) and d come as one 16-byte load
+// every lane issues.  Blocks of 110 bytes sit on odd half words as often as Q6_K's: the loads start at the 4-byte boundary
+// below and two exchanges a step bring the pieces' last half words.
 constexpr uint32_t Q6K_BLOCK_BYTES = 210;
+constexpr uint32_t Q3K_BLOCK_BYTES = 110;
 constexpr uint32_t Q6K_ZERO_BYTES = 304;  // what an idle A lane reads: four chunk offsets (0, 96, 192, 288) + 16 bytes
 
 typedef uint32_t q6_u32x3 __attribute__((ext_vector_type(3)));
 typedef q6_u32x3 q6_u32x3_a4 __attribute__((aligned(4)));
 typedef u32x4 q6_u32x4_a4 __attribute__((aligned(4)));
-struct Q6Unit {
+template <int ELEMENT>
+struct KqUnit;
+template <>
+struct KqUnit<NH_Q6_K> {
     u32x4 la, lb, qh;
     q6_u32x3 sc;
     uint32_t shift;  // 16 where the block sits on an odd half word (the loads then start two bytes early), else 0
 };
+template <>
+struct KqUnit<NH_Q3_K> {
+    u32x4 qs, hm, sc;  // bit pairs, third bits, the twelve scale bytes and d
+    uint32_t shift;
+};
+typedef KqUnit<NH_Q6_K> Q6Unit;
 
 static inline size_t q6k_tile16_lds(uint32_t nblk, uint32_t NW) {
     return (size_t)nblk * (TILE16_BLOCK_DIGITS + TILE16_BLOCK_PAIRS) + (size_t)NW * Q6K_ZERO_BYTES + (size_t)2 * NW * 16u * 4u + (size_t)NW * 4u + 64u;
@@ -58,11 +76,15 @@ static inline size_t q6k_tile16_lds(uint32_t nblk, uint32_t NW) {
 // SWIGLU: the matrix is a gate matrix with the up matrix `lead_to_w1` * 16 bytes further; a workgroup's unit of work is a pair of
 // tiles (gate rows, then the same rows of up) and the pair's finishing wave writes silu(gate) * up.
 // The product itself, `block` of `lead_grid` workgroups, its LDS at `q6k_lds_bytes` (q6k_tile16_lds() of it).
-template <int NW, bool HANDED, bool SWIGLU = false>
+template <int NW, bool HANDED, bool SWIGLU = false, int ELEMENT = NH_Q6_K>
 __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const uint32_t block, const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w,
                                                    uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles, uint32_t lead_tile_rows, int32_t lead_to_w1,
                                                    const GemvParams &p) {
     static_assert(!(HANDED && SWIGLU), "handed-over digit planes feed a plain product");
+    static_assert(ELEMENT == NH_Q6_K || ELEMENT == NH_Q3_K, "super-blocks of sixteen scale groups of 16");
+    constexpr bool Q3 = ELEMENT == NH_Q3_K;
+    constexpr uint32_t BLOCK_BYTES = Q3 ? Q3K_BLOCK_BYTES : Q6K_BLOCK_BYTES;
+    typedef KqUnit<ELEMENT> Unit;
     constexpr uint32_t NT = NW * 64;
     constexpr int D = 2;
     typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -71,7 +93,7 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
     typedef const __attribute__((address_space(1))) q6_u32x4_a4 *global_uint4;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t nblk = lead_row_bytes / Q6K_BLOCK_BYTES;
+    const uint32_t nblk = lead_row_bytes / BLOCK_BYTES;
     const float *const x = static_cast<const float *>(lead_input);
     uint8_t *const digits = q6k_lds_bytes;
     uint8_t *const zeros = q6k_lds_bytes + (size_t)nblk * TILE16_BLOCK_DIGITS + wave * Q6K_ZERO_BYTES;
@@ -109,16 +131,22 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
 
     // Loads run D steps ahead of the arithmetic, across tile boundaries.  Every fetch issues its four loads: past the last step
     // the last unit is fetched again and dropped, so that the waits count exactly how many loads are newer than the one needed.
-    Q6Unit ring[D];
+    Unit ring[D];
     uint32_t ahead_tile = 0, ahead_b = wave;
     const uint8_t *ahead_row = lane_row(tile_at(0));
-    auto fetch = [&](Q6Unit &u) {
-        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * Q6K_BLOCK_BYTES;
+    auto fetch = [&](Unit &u) {
+        const uint8_t *at = ahead_row + (size_t)min(ahead_b, nblk - 1u) * BLOCK_BYTES;
         const uint8_t *down = reinterpret_cast<const uint8_t *>(reinterpret_cast<uintptr_t>(at) & ~(uintptr_t)3);
-        u.la = *(global_uint4)(uintptr_t)(down + at_low);
-        u.lb = *(global_uint4)(uintptr_t)(down + at_low + 32u);
-        u.qh = *(global_uint4)(uintptr_t)(down + at_high);
-        u.sc = *(global_uint3)(uintptr_t)(down + at_scales);
+        if constexpr (Q3) {
+            u.qs = *(global_uint4)(uintptr_t)(down + 32u + 32u * h + 16u * j);
+            u.hm = *(global_uint4)(uintptr_t)(down + 16u * j);
+            u.sc = *(global_uint4)(uintptr_t)(down + 96u);
+        } else {
+            u.la = *(global_uint4)(uintptr_t)(down + at_low);
+            u.lb = *(global_uint4)(uintptr_t)(down + at_low + 32u);
+            u.qh = *(global_uint4)(uintptr_t)(down + at_high);
+            u.sc = *(global_uint3)(uintptr_t)(down + at_scales);
+        }
         u.shift = ((uint32_t)reinterpret_cast<uintptr_t>(at) & 2u) * 8u;
         if (ahead_b + NW < nblk) {
             ahead_b += NW;
@@ -293,33 +321,56 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
         f32x2 pr[4];
         uint32_t scales, d;
     };
-    auto multiply = [&](const Q6Unit &u, uint32_t b, Step &st) {
+    auto multiply = [&](const Unit &u, uint32_t b, Step &st) {
         const uint8_t *at = abase + (size_t)b * astride;
         const i32x4 a0 = *reinterpret_cast<const i32x4 *>(at), a1 = *reinterpret_cast<const i32x4 *>(at + 96);
         const i32x4 a2 = *reinterpret_cast<const i32x4 *>(at + 192), a3 = *reinterpret_cast<const i32x4 *>(at + 288);
 #pragma unroll
         for (int g = 0; g < 4; g++) st.pr[g] = pbase[b * 16u + 2u * g];
-        // The word that follows each of the lane's three pieces in memory is the first word of another piece of the row:
-        //   first nibble piece:  lane (h, 0) <- first piece of (h, 1);  lane (h, 1) <- second piece of (h, 0)
-        //   second nibble piece: (0, 0) <- second of (0, 1);  (0, 1) <- first of (1, 0);  (1, 0) <- second of (1, 1);  (1, 1) <- bit pairs of (0, 0)
-        //   bit pairs:           (h, j) <- bit pairs of the lane 16 further;  (1, 1) <- the scales of (0, 0)
-        // every lane offers what its reader wants and takes part in every exchange
-        const uint32_t la0 = u.la.x, lb0 = u.lb.x, qh0 = u.qh.x, sc0 = u.sc.x, sc2 = u.sc.z;
-        const uint32_t after_la = (uint32_t)__builtin_amdgcn_ds_bpermute(beside, (int)(j ? la0 : lb0));
-        const uint32_t after_lb = (uint32_t)__builtin_amdgcn_ds_bpermute(above, (int)(q == 0u ? qh0 : (q == 2u ? la0 : lb0)));
-        const uint32_t after_qh = (uint32_t)__builtin_amdgcn_ds_bpermute(above, (int)(q == 0u ? sc0 : qh0));
-        const uint32_t from_upper = (uint32_t)__builtin_amdgcn_ds_bpermute(across, (int)sc2);
         const uint32_t shift = u.shift;
         auto placed = [shift](const u32x4 &piece, uint32_t after) -> u32x4 {
             return u32x4{__builtin_amdgcn_alignbit(piece.y, piece.x, shift), __builtin_amdgcn_alignbit(piece.z, piece.y, shift),
                          __builtin_amdgcn_alignbit(piece.w, piece.z, shift), __builtin_amdgcn_alignbit(after, piece.w, shift)};
         };
-        const u32x4 la = placed(u.la, after_la), lb = placed(u.lb, after_lb), qh = placed(u.qh, after_qh);
-        const u32x4 low = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu}, high = {0x30303030u, 0x30303030u, 0x30303030u, 0x30303030u};
-        const i32x4 b0 = (i32x4)((la & low) | ((qh << 4) & high)), b1 = (i32x4)((lb & low) | ((qh << 2) & high));
-        const i32x4 b2 = (i32x4)(((la >> 4) & low) | (qh & high)), b3 = (i32x4)(((lb >> 4) & low) | ((qh >> 2) & high));
-        st.scales = __builtin_amdgcn_perm(__builtin_amdgcn_alignbit(u.sc.z, u.sc.y, shift), __builtin_amdgcn_alignbit(u.sc.y, u.sc.x, shift), pick);
-        st.d = ((h ? sc2 : from_upper) >> shift) & 0xffffu;  // d follows the sixteen scales: the third word of the upper lanes' twelve bytes
+        i32x4 b0, b1, b2, b3;
+        if constexpr (Q3) {
+            // The word that follows a piece in memory:
+            //   bit pairs:  lane (h, j) <- the bit pairs of the lane 16 further;  (1, 1) <- its own scales' first word
+            //   third bits: (h, 0) <- the third bits of (h, 1);  (h, 1) <- the bit pairs of (0, 0)
+            const uint32_t qs0 = u.qs.x, hm0 = u.hm.x;
+            const uint32_t got_qs = (uint32_t)__builtin_amdgcn_ds_bpermute(above, (int)qs0);
+            const uint32_t after_hm = (uint32_t)__builtin_amdgcn_ds_bpermute(q == 1u ? beside : above, (int)(j ? hm0 : qs0));
+            const uint32_t after_qs = q == 3u ? u.sc.x : got_qs;
+            const u32x4 qs = placed(u.qs, after_qs), hm = placed(u.hm, after_hm) >> (4u * h);
+            const u32x4 two = {0x03030303u, 0x03030303u, 0x03030303u, 0x03030303u}, third = {0x04040404u, 0x04040404u, 0x04040404u, 0x04040404u};
+            b0 = (i32x4)((qs & two) | ((hm << 2) & third)), b1 = (i32x4)(((qs >> 2) & two) | ((hm << 1) & third));
+            b2 = (i32x4)(((qs >> 4) & two) | (hm & third)), b3 = (i32x4)(((qs >> 6) & two) | ((hm >> 1) & third));
+            // sixteen 6-bit scales: low nibbles in the first eight bytes (scales 0..7, then 8..15 in the high nibbles), bit pairs in
+            // the last four; this lane's are 8 h + 2 g + j
+            const uint32_t s0 = __builtin_amdgcn_alignbit(u.sc.y, u.sc.x, shift), s1 = __builtin_amdgcn_alignbit(u.sc.z, u.sc.y, shift);
+            const uint32_t s2 = __builtin_amdgcn_alignbit(u.sc.w, u.sc.z, shift);
+            const uint32_t first = ((s0 >> (4u * h)) & 0x0f0f0f0fu) | (((s2 >> (4u * h)) & 0x03030303u) << 4);
+            const uint32_t second = ((s1 >> (4u * h)) & 0x0f0f0f0fu) | (((s2 >> (4u * h + 2u)) & 0x03030303u) << 4);
+            st.scales = __builtin_amdgcn_perm(second, first, pick);
+            st.d = (u.sc.w >> shift) & 0xffffu;
+        } else {
+            // The word that follows each of the lane's three pieces in memory is the first word of another piece of the row:
+            //   first nibble piece:  lane (h, 0) <- first piece of (h, 1);  lane (h, 1) <- second piece of (h, 0)
+            //   second nibble piece: (0, 0) <- second of (0, 1);  (0, 1) <- first of (1, 0);  (1, 0) <- second of (1, 1);  (1, 1) <- bit pairs of (0, 0)
+            //   bit pairs:           (h, j) <- bit pairs of the lane 16 further;  (1, 1) <- the scales of (0, 0)
+            // every lane offers what its reader wants and takes part in every exchange
+            const uint32_t la0 = u.la.x, lb0 = u.lb.x, qh0 = u.qh.x, sc0 = u.sc.x, sc2 = u.sc.z;
+            const uint32_t after_la = (uint32_t)__builtin_amdgcn_ds_bpermute(beside, (int)(j ? la0 : lb0));
+            const uint32_t after_lb = (uint32_t)__builtin_amdgcn_ds_bpermute(above, (int)(q == 0u ? qh0 : (q == 2u ? la0 : lb0)));
+            const uint32_t after_qh = (uint32_t)__builtin_amdgcn_ds_bpermute(above, (int)(q == 0u ? sc0 : qh0));
+            const uint32_t from_upper = (uint32_t)__builtin_amdgcn_ds_bpermute(across, (int)sc2);
+            const u32x4 la = placed(u.la, after_la), lb = placed(u.lb, after_lb), qh = placed(u.qh, after_qh);
+            const u32x4 low = {0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu, 0x0f0f0f0fu}, high = {0x30303030u, 0x30303030u, 0x30303030u, 0x30303030u};
+            b0 = (i32x4)((la & low) | ((qh << 4) & high)), b1 = (i32x4)((lb & low) | ((qh << 2) & high));
+            b2 = (i32x4)(((la >> 4) & low) | (qh & high)), b3 = (i32x4)(((lb >> 4) & low) | ((qh >> 2) & high));
+            st.scales = __builtin_amdgcn_perm(__builtin_amdgcn_alignbit(u.sc.z, u.sc.y, shift), __builtin_amdgcn_alignbit(u.sc.y, u.sc.x, shift), pick);
+            st.d = ((h ? sc2 : from_upper) >> shift) & 0xffffu;  // d follows the sixteen scales: the third word of the upper lanes' twelve bytes
+        }
         const i32x4 none = {0, 0, 0, 0};
         st.c[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, none, 0, 0, 0);
         st.c[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, none, 0, 0, 0);
@@ -332,8 +383,8 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const float planes = fmaf(fmaf((float)st.c[g][0], 256.0f, (float)st.c[g][1]), 256.0f, (float)st.c[g][2]);
-            const float scale = (float)(int8_t)(st.scales >> (8 * g));
-            whole = fmaf(scale, fmaf(st.pr[g].y, planes, -32.0f * st.pr[g].x), whole);
+            const float scale = Q3 ? (float)((st.scales >> (8 * g)) & 0xffu) - 32.0f : (float)(int8_t)(st.scales >> (8 * g));
+            whole = fmaf(scale, fmaf(st.pr[g].y, planes, (Q3 ? -4.0f : -32.0f) * st.pr[g].x), whole);
         }
         acc = fmaf(half_to_float((uint16_t)st.d), whole, acc);
     };

@@ -1276,8 +1276,8 @@ bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer) {
     GemvArgs from = producer, to = consumer;
     from.digits_out = nullptr, to.digits_in = nullptr;
     if (!tile16_takes(from)) return false;
-    if (consumer.element == NH_Q6_K) {
-        // the Q6_K tiles read the same pieces in the same chunk order
+    if (consumer.element == NH_Q6_K || consumer.element == NH_Q3_K) {
+        // the Q6_K and Q3_K tiles read the same pieces in the same chunk order
         alignas(16) static const uint8_t somewhere[16] = {};
         to.digits_in = somewhere;
         return q6k_tile16_takes(to);

@@ -405,13 +405,15 @@ def test_staged_super_block_products(device, element, N, K, rows):
 
 
 @pytest.mark.parametrize("tile16", ["1", "0"])
-@pytest.mark.parametrize("element,switch", [(NH_Q6_K, "NEURA_HIP_Q6K_TILE16"), (NH_Q5_K, "NEURA_HIP_Q5K_TILE16")], ids=["q6_k", "q5_k"])
+@pytest.mark.parametrize("element,switch", [(NH_Q6_K, "NEURA_HIP_Q6K_TILE16"), (NH_Q5_K, "NEURA_HIP_Q5K_TILE16"), (NH_Q3_K, "NEURA_HIP_Q6K_TILE16")],
+                         ids=["q6_k", "q5_k", "q3_k"])
 @pytest.mark.parametrize("N,K", [(16, 256), (64, 3584), (3584, 18944), (4608, 3584), (1040, 768), (48, 2048), (272, 8960), (37888, 3584), (2048, 1536)])
 def test_q6_k_and_q5_k_one_row_products_on_16_row_tiles(device, monkeypatch, tile16, element, switch, N, K):
     """One activation row against Q6_K rows on the 16 x 16 x 64 integer MFMA (the stored 6-bit codes as bytes, a scale per
-    lane slice, the activation as three signed digit planes with a sum and a scale per 16 numbers) and against Q5_K rows on
-    the Q4_K tiles with the fifth bit beside the nibble; with NEURA_HIP_Q6K_TILE16=0 / NEURA_HIP_Q5K_TILE16=0 the staged
-    kernel that served before them.  Rows of 210-byte blocks start on every alignment of a half word; activations over many
+    lane slice, the activation as three signed digit planes with a sum and a scale per 16 numbers), against Q3_K rows the
+    same way (3-bit codes, 6-bit scales) and against Q5_K rows on the Q4_K tiles with the fifth bit beside the nibble; with
+    NEURA_HIP_Q6K_TILE16=0 / NEURA_HIP_Q5K_TILE16=0 the staged kernel that served before them.  Rows of 210- and 110-byte
+    blocks start on every alignment of a half word; activations over many
     orders of magnitude, with outliers at any seat; plain, with a residual (added in place) and with SwiGLU; non-finite
     inputs stay visible and zeros give zeros."""
     monkeypatch.setenv(switch, tile16)
