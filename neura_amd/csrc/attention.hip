@@ -584,8 +584,8 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
 //           C hands lane (column, kq) the keys 4 kq + e and 16 + 4 kq + e of the tile: a column's statistics live in four lanes.
 //   values  O^T[channel][column] += V^T[channel][key] . P^T[key][column]: the weights (* 2^10, value and residue planes) go
 //           back in as the B operand from the registers C left them in -- slots 0..3 the keys 4 kq + e, slots 4..7 the keys
-//           16 + 4 kq + e -- and the value rows, which the wave wrote to its own corner of LDS transposed, are the A operand in
-//           that same key order (two 8-byte reads a lane).
+//           16 + 4 kq + e -- and the value rows, which the wave wrote to its own corner of LDS as they lie, are the A operand in
+//           that same key order, transposed by the read (ds_read_b64_tr_b16, two a lane).
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // The leading arguments are what the first loads (cursor, queries, the first key and value tile) need: plain words that the
@@ -601,13 +601,13 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
     constexpr int KB = TK / 16;             // 16-key blocks of a tile
     constexpr int STEPS = WIDTH / 32;       // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 16;      // 16-channel blocks of the output
-    constexpr int VPITCH = TK + 4;          // halves per staged value channel
+    constexpr int VROW = WIDTH + 16;        // halves per staged value row: the four rows a read's sixteen lanes touch fall into different banks
     constexpr int PIECES = TK * WIDTH / 8 / 64;  // 16-byte pieces of a value tile per lane
     // the waves' value corners and, once every wave has left the walk, their sums share one buffer
-    constexpr size_t VT_BYTES = sizeof(uint16_t) * 4 * WIDTH * VPITCH, MERGED_BYTES = sizeof(float) * 4 * 16 * (WIDTH + 4), STATS_BYTES = sizeof(float) * 8 * 16;
+    constexpr size_t VT_BYTES = sizeof(uint16_t) * 4 * TK * VROW, MERGED_BYTES = sizeof(float) * 4 * 16 * (WIDTH + 4), STATS_BYTES = sizeof(float) * 8 * 16;
     constexpr size_t ROWS_BYTES = VT_BYTES > MERGED_BYTES ? VT_BYTES : MERGED_BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t shared_rows[ROWS_BYTES + STATS_BYTES];
-    uint16_t(*vt)[WIDTH][VPITCH] = reinterpret_cast<uint16_t(*)[WIDTH][VPITCH]>(shared_rows);
+    uint16_t(*vt)[TK][VROW] = reinterpret_cast<uint16_t(*)[TK][VROW]>(shared_rows);
     float(*merged)[16][WIDTH + 4] = reinterpret_cast<float(*)[16][WIDTH + 4]>(shared_rows);  // per wave and column: the weighed channel sums (rows 16 bytes apart in phase)
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -755,13 +755,16 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
                 const uint32_t piece = lane + 64u * i, key = piece / (WIDTH / 8), part = piece % (WIDTH / 8);
                 // rows past the walked keys may hold anything, and a weight of zero does not silence a NaN
                 const uint32_t keep = tile + key < last ? 0xffffffffu : 0u;
-                const uint32_t words[4] = {plane_words[i].x & keep, plane_words[i].y & keep, plane_words[i].z & keep, plane_words[i].w & keep};
-                // groups of four keys change places by the channel block (part / 4): the sixteen parts a store instruction
-                // touches would otherwise share four banks
-                const uint32_t column = (((key >> 2) ^ (part >> 2)) << 2) | (key & 3u);
-#pragma unroll
-                for (int j = 0; j < 8; j++) vt[wave][part * 8u + j][column] = (uint16_t)(words[j >> 1] >> (16 * (j & 1)));
+                *reinterpret_cast<u32x4 *>(&vt[wave][key][part * 8u]) = u32x4{plane_words[i].x & keep, plane_words[i].y & keep, plane_words[i].z & keep, plane_words[i].w & keep};
             }
+        };
+        // ds_read_b64_tr_b16 hands lane 4 k + a of a group of sixteen, which points at four halves, element (lane % 4) of the pieces
+        // its lanes a, a + 4, a + 8, a + 12 point at: with lane (k, a) of group kq at key 4 kq + k, channels 16 d + 4 a .., lane n
+        // receives channel 16 d + n of keys 4 kq .. 4 kq + 3 -- the A operand, transposed on the way out of LDS
+        typedef short short4_t __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) short4_t *lds_short4;
+        auto transposed = [&](uint32_t first_key, int d) -> uint2 {
+            return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4)&vt[wave][first_key + 4u * kq + (n >> 2)][16 * d + 4 * (n & 3u)]));
         };
         stage_plane(v_words);
         if (next < last) fetch_values(next);
@@ -771,10 +774,9 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
         for (int d = 0; d < BLOCKS; d++) {
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[d][e] *= rescale;
-            // channels 16 d + n lie in parts 2 d and 2 d + 1: their key groups sit d / 2 places off
-            const uint2 low = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * (kq ^ (d >> 1))]);
+            const uint2 low = transposed(0u, d);
             if constexpr (TK == 32) {
-                const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
+                const uint2 high = transposed(16u, d);
                 const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
                 acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_value, acc[d], 0, 0, 0);
                 acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_residue, acc[d], 0, 0, 0);
@@ -792,9 +794,9 @@ __global__ __launch_bounds__(256) void attention_decode_tile_kernel(const uint32
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
             for (int d = 0; d < BLOCKS; d++) {
-                const uint2 low = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * (kq ^ (d >> 1))]);
+                const uint2 low = transposed(0u, d);
                 if constexpr (TK == 32) {
-                    const uint2 high = *reinterpret_cast<const uint2 *>(&vt[wave][16 * d + n][4 * ((4 + kq) ^ (d >> 1))]);
+                    const uint2 high = transposed(16u, d);
                     const half8_t values = __builtin_bit_cast(half8_t, u32x4{low.x, low.y, high.x, high.y});
                     acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(values, w_small, acc[d], 0, 0, 0);
                 } else {
