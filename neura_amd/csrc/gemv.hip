@@ -8,7 +8,7 @@
 //   gemv_q4k_tile16_kernel     1 row, any K of whole super-blocks, matrices that end on 16-row tiles: every product of a
 //                              batch-1 decode step of the 0.5B .. 7B shapes; 2 rows the same (ffn_down's 18944 columns
 //                              included); 3 and 4 rows where the kernel above refuses and the digits still fit LDS
-//                              (with FIFTH the same for one row of Q5_K; gemv_q6k_tile16_kernel is its Q6_K sibling)
+//                              (with FIFTH the same for one row of Q5_K; gemv_q6k_tile16_kernel is its sibling for one row of Q6_K or Q3_K)
 //   gemv_q4k_f16_kernel        5 to 8 rows, K <= 4096, at least 4 x 256 tiles of 16 rows (gate|up and the head at batch 5-8)
 //   gemv_q4k_mfma32_kernel     5 to 8 rows otherwise (q|k|v, attn_output; ffn_down in K slices with gemv_fold_kernel), matrices
 //                              that end on 32-row tiles; 3 and 4 rows of short (<= 8192 rows) or very tall (>= 65536) matrices that the
