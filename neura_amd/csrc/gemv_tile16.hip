@@ -577,7 +577,10 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
         const uint32_t n = rope_row(tile_at(0), c);
         rope_held = rope_operands(p, n, c, rope_position);
     }
-    if (SEAM::SHARED_OUT || (MODE == TILE16_SWIGLU && R == 1)) tag_out = p.tag_out + (p.tick ? 128u * *p.tick : 0u);
+    // (planes that leave through a kernel boundary carry the seam's number alone: their reader does not look at tags, and the
+    // step's word would be a load from memory that the walk's start waits for)
+    if constexpr (SEAM::SHARED_OUT) tag_out = p.tag_out + (p.tick ? 128u * *p.tick : 0u);
+    else if (MODE == TILE16_SWIGLU && R == 1) tag_out = p.tag_out;
 
     // ---- the walk
     const ScaleLane lane_scales = scale_lane(q);
