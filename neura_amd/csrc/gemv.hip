@@ -2371,7 +2371,7 @@ bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     {
         GemvArgs folded = a;
         folded.rope = &rope;
-        if (tile16_takes(folded)) return true;
+        if (tile16_takes(folded) || q6k_tile16_takes(folded)) return true;
     }
     if (a.element == NH_Q8_0) {
         // the direct Q8_0 decode kernel, a row of blocks inside one wave

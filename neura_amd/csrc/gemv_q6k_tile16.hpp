@@ -75,12 +75,17 @@ static inline size_t q6k_tile16_lds(uint32_t nblk, uint32_t NW) {
 // starts (-amdgpu-kernarg-preload-count).  `input` is x, or the digit planes with HANDED.
 // SWIGLU: the matrix is a gate matrix with the up matrix `lead_to_w1` * 16 bytes further; a workgroup's unit of work is a pair of
 // tiles (gate rows, then the same rows of up) and the pair's finishing wave writes silu(gate) * up.
+// ROPE: a q|k|v product (up to three matrices stacked, the second `lead_to_w1` * 16 bytes and the third `lead_to_w2` * 16 bytes
+// behind the first, ending at rows `lead_end0`, `lead_end1` and N) whose epilogue rotates the q and k rows and writes k and v
+// into the states (rope_store): `lead_tile_rows` is then the rotation's width, and a tile holds channels c .. c + 7 of a head
+// and their partners half a head further.
 // The product itself, `block` of `lead_grid` workgroups, its LDS at `q6k_lds_bytes` (q6k_tile16_lds() of it).
-template <int NW, bool HANDED, bool SWIGLU = false, int ELEMENT = NH_Q6_K>
+template <int NW, bool HANDED, bool SWIGLU = false, int ELEMENT = NH_Q6_K, bool ROPE = false>
 __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const uint32_t block, const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w,
                                                    uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles, uint32_t lead_tile_rows, int32_t lead_to_w1,
-                                                   const GemvParams &p) {
+                                                   int32_t lead_to_w2, uint32_t lead_end0, uint32_t lead_end1, const GemvParams &p) {
     static_assert(!(HANDED && SWIGLU), "handed-over digit planes feed a plain product");
+    static_assert(!ROPE || (!HANDED && !SWIGLU), "the rotation is folded into a product of floats with no other epilogue");
     static_assert(ELEMENT == NH_Q6_K || ELEMENT == NH_Q3_K, "super-blocks of sixteen scale groups of 16");
     constexpr bool Q3 = ELEMENT == NH_Q3_K;
     constexpr uint32_t BLOCK_BYTES = Q3 ? Q3K_BLOCK_BYTES : Q6K_BLOCK_BYTES;
@@ -104,6 +109,7 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
     auto fetch_the_rest = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         NH_FETCH(p.y, p.residual, p.N, p.K, p.eps, p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
+        if (ROPE) NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_k, p.rope_q_rows, p.rope_k_rows, p.rope_positions, p.bias[1], p.bias[2], p.end[0], p.end[1]);
         __builtin_amdgcn_sched_barrier(0);
     };
     const uint32_t r = lane & 15u, q = lane >> 4, h = q >> 1, j = q & 1u;
@@ -111,13 +117,27 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
     if (block >= tiles || block >= lead_grid) return;  // the whole workgroup: no barrier has been reached
     const uint32_t ntiles = (tiles - block + lead_grid - 1u) / lead_grid;
     const uint32_t count = wave < nblk ? (nblk - wave + NW - 1u) / NW : 0u;  // super-blocks of one tile this wave walks
-    const uint32_t tile_rows = lead_tile_rows, row_bytes = lead_row_bytes;
+    const uint32_t tile_rows = ROPE ? 16u : lead_tile_rows, row_bytes = lead_row_bytes;
     const uint8_t *const w0 = lead_w0;
     // a tile may hold fewer than 16 rows: the columns past them walk the tile's last row again and are never written
-    const int64_t to_w1 = (int64_t)lead_to_w1 * 16;
-    auto lane_row = [w0, row_bytes, tile_rows, r, to_w1](uint32_t tile) -> const uint8_t * {
+    const int64_t to_w1 = (int64_t)lead_to_w1 * 16, to_w2 = (int64_t)lead_to_w2 * 16;
+    const uint32_t end0 = lead_end0, end1 = lead_end1;
+    const uint32_t half_width = (ROPE ? lead_tile_rows : 16u) >> 1, tiles_per_head = max(half_width >> 3, 1u);
+    auto lane_row = [w0, row_bytes, tile_rows, r, to_w1, to_w2, end0, end1, half_width, tiles_per_head](uint32_t tile) -> const uint8_t * {
         if (SWIGLU) return w0 + ((tile & 1u) ? to_w1 : (int64_t)0) + (int64_t)((size_t)((tile >> 1) * 16u + r) * row_bytes);
+        if (ROPE) {
+            const uint32_t n = (tile / tiles_per_head) * (2u * half_width) + (tile % tiles_per_head) * 8u + (r & 7u) + (r >> 3) * half_width;
+            const bool in0 = n < end0, in1 = n < end1;
+            return w0 + (in0 ? (int64_t)0 : (in1 ? to_w1 : to_w2)) + (int64_t)((size_t)(n - (in0 ? 0u : (in1 ? end0 : end1))) * row_bytes);
+        }
         return w0 + (size_t)(tile * tile_rows + min(r, tile_rows - 1u)) * row_bytes;
+    };
+    // what the rotation's epilogue reads (the cursor, then cos, sin and bias of a tile's sixteen outputs) is fetched ahead
+    uint32_t rope_position = 0;
+    RopeOperands rope_held{0.0f, 1.0f, 0.0f};
+    auto rope_row = [half_width, tiles_per_head, lane](uint32_t tile, uint32_t &c) -> uint32_t {
+        c = (tile % tiles_per_head) * 8u + (lane & 7u);
+        return (tile / tiles_per_head) * (2u * half_width) + c + ((lane >> 3) & 1u) * half_width;
     };
     const uint32_t first_tile = block, hop = lead_grid;
     // with SwiGLU the workgroup's unit of work is a pair: tiles 2 t (gate) and 2 t + 1 (up)
@@ -267,6 +287,7 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
             // the weights' loads go out behind the activations', which everything waits for first
             first_fetches();
             fetch_the_rest();
+            if (ROPE && wave == 0 && lane < 16u) rope_position = p.rope_cursor[0];
             if (lead_norm_w) {
                 // sum of squares of the whole row (crates/neura-kernel/src/task/norm.rs:69-83; the same fp32 adds in another order)
                 float square = 0.0f;
@@ -305,6 +326,11 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
         }
     }
     __builtin_amdgcn_wave_barrier();  // LDS serves a wave's accesses in order: the reads below see this wave's writes
+    if (ROPE && wave == 0 && lane < 16u) {
+        uint32_t c;
+        const uint32_t n = rope_row(tile_at(0), c);
+        rope_held = rope_operands(p, n, c, rope_position);
+    }
 
     // ---- the walk
     const uint32_t m = lane & 15u;
@@ -391,7 +417,7 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
     // The wave that finishes a tile (sums the waves' parts, runs the epilogue) changes from tile to tile (with SwiGLU from pair to
     // pair: the gate sum waits in its registers)
     auto tile_end = [&](uint32_t tile, uint32_t index) {
-        const uint32_t finisher = (SWIGLU ? index >> 1 : index) % NW;
+        const uint32_t finisher = ROPE ? 0u : (SWIGLU ? index >> 1 : index) % NW;
         float v = acc;
         v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
         v += __shfl_xor(v, 32, 64);
@@ -403,12 +429,20 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
 #pragma unroll
             for (int w = 0; w < NW; w++) total += part[(parity * NW + w) * 16u + r];
             const size_t n = (size_t)tile * tile_rows + r;
-            if (SWIGLU) {
+            if (ROPE) {
+                uint32_t c;
+                const uint32_t row = rope_row(tile, c);
+                rope_store(p, total, row, lane >= 8u, rope_position, rope_held);
+                if (tile + hop < tiles) {  // the next tile of this workgroup
+                    const uint32_t next = rope_row(tile + hop, c);
+                    rope_held = rope_operands(p, next, c, rope_position);
+                }
+            } else if (SWIGLU) {
                 if (!(tile & 1u)) gate = total;
                 else p.y[(size_t)(tile >> 1) * 16u + r] = silu(gate) * total;
             } else if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);  // in place: one add per element, nothing to wait for
             else p.y[n] = p.residual ? p.residual[n] + total : total;
-            if (!SWIGLU && p.append_value) {
+            if (!SWIGLU && !ROPE && p.append_value) {
                 // a value projection of one token: its rows (+ bias) go into the value state at the cursor as halves, as
                 // value_append_kernel would cast them
                 const uint32_t cursor = p.rope_cursor[0];

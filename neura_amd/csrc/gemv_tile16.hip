@@ -1529,7 +1529,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_rope_beside_q6k_kernel(const
                                                      lead_grid, lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
     } else {
         q6k_tile16_product<NW, false, false>(pair_lds_bytes, blockIdx.x - lead_grid, beside.w0, lead_input, beside.norm_w, beside.row_bytes, beside.grid, beside.tiles,
-                                             beside.tile_rows, 0, beside.p);
+                                             beside.tile_rows, 0, 0, 0u, 0u, beside.p);
     }
 }
 
