@@ -19,7 +19,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q6k_tile16_kernel(const uint8_t 
 // mix, gate|up of a file stored in Q6_K or Q3_K; or up to three matrices stacked with the rotation folded in (the q|k or q|k|v
 // product of such a file).
 bool q6k_tile16_takes(const GemvArgs &a) {
-    if ((a.element != NH_Q6_K && a.element != NH_Q3_K) || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.merge || a.digits_out) return false;
+    if ((a.element != NH_Q6_K && a.element != NH_Q3_K) || a.rows != 1 || a.K % 256u != 0 || a.K == 0 || a.merge) return false;
+    if (a.digits_out && (!a.swiglu || a.N % 512u != 0 || ((uintptr_t)a.digits_out & 63u))) return false;  // whole super-blocks of planes
     if (env_int("NEURA_HIP_Q6K_TILE16", 1) == 0) return false;
     auto stacked = [&a](int m) {  // a matrix behind the first is named by its distance from it in 16-byte units
         const int64_t apart = static_cast<const uint8_t *>(a.W[m]) - static_cast<const uint8_t *>(a.W[0]);
@@ -86,7 +87,7 @@ Q6kLaunch q6k_tile16_plan(nh_device *d, const GemvArgs &a) {
     }
     p.x = a.x, p.y = a.y, p.residual = a.residual, p.norm_w = a.norm_w;
     p.N = a.N, p.K = a.K, p.eps = a.eps, p.rows = 1, p.swiglu = a.swiglu;
-    p.digits_in = a.digits_in;
+    p.digits_in = a.digits_in, p.digits_out = a.digits_out, p.tag_out = a.tag_out;
     if (a.append_value) {
         p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
         p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.rope_element = a.append_value->element, p.bias[0] = a.bias[0], p.refusal = d->refusal;

@@ -109,6 +109,7 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
     auto fetch_the_rest = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         NH_FETCH(p.y, p.residual, p.N, p.K, p.eps, p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
+        if (SWIGLU) NH_FETCH(p.digits_out, p.tag_out);
         if (ROPE) NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_k, p.rope_q_rows, p.rope_k_rows, p.rope_positions, p.bias[1], p.bias[2], p.end[0], p.end[1]);
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -438,7 +439,9 @@ __device__ __forceinline__ void q6k_tile16_product(uint8_t *q6k_lds_bytes, const
                     rope_held = rope_operands(p, next, c, rope_position);
                 }
             } else if (SWIGLU) {
+                // (the pair's sixteen outputs either as floats or as chunk tile / 2 of the digit planes the product behind takes)
                 if (!(tile & 1u)) gate = total;
+                else if (p.digits_out) reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u)[r] = handed_piece_word(silu(gate) * total, r, p.tag_out);
                 else p.y[(size_t)(tile >> 1) * 16u + r] = silu(gate) * total;
             } else if (p.residual == p.y) unsafeAtomicAdd(p.y + n, total);  // in place: one add per element, nothing to wait for
             else p.y[n] = p.residual ? p.residual[n] + total : total;

@@ -184,6 +184,41 @@ __device__ __forceinline__ int dpp_int(int v) {
 // signed digits need), and flipping bit 7 takes the 128 off again.
 __device__ __forceinline__ uint32_t signed_digits(int whole) { return ((uint32_t)whole + 0x00808080u) ^ 0x00808080u; }
 
+// Sixteen outputs of a product as a chunk of the next product's activations: lanes 0..15 of a wave, each holding one output, turn
+// them into three signed base-256 digit planes below a power-of-two scale of their own (the chunk's largest magnitude lands in
+// [2^21, 2^22)) and return the word each writes of the chunk's 64-byte piece:
+//   words 0..3 plane 0 | 4..6 plane 1, first twelve | 7 tag || 8 plane 1, last four | 9..11 plane 2, first twelve |
+//   12 plane 2, last four | 13, 14 the (sum, scale) pair | 15 tag
+// (the tag words end the piece's two 32-byte sectors: a reader behind a seam of one launch knows by them that a sector has arrived).
+__device__ __forceinline__ uint32_t handed_piece_word(float value, uint32_t r, uint32_t tag) {
+    uint32_t top = __builtin_bit_cast(uint32_t, value) & 0x7fffffffu;
+    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
+    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
+    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
+    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
+    const uint32_t raw = top >> 23;
+    const uint32_t exponent = min(max(raw, 22u), 254u);
+    const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);
+    const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
+    const float rounded = rintf(value * scale);
+    float chunk_sum = rounded;
+    chunk_sum += dpp<DPP_QUAD_XOR1>(chunk_sum);
+    chunk_sum += dpp<DPP_QUAD_XOR2>(chunk_sum);
+    chunk_sum += dpp<DPP_ROW_ROR4>(chunk_sum);
+    chunk_sum += dpp<DPP_ROW_ROR8>(chunk_sum);
+    const int dg = (int)signed_digits((int)rounded);
+    const uint32_t plane = r < 4u ? 0u : (r < 9u ? 1u : 2u);
+    const int first = (int)(r < 4u ? 4u * r : (r < 7u ? 4u * (r - 4u) : (r == 8u || r == 12u ? 12u : 4u * (r - 9u)))) & 15;
+    const uint32_t d0 = (uint32_t)__shfl(dg, first, 16), d1 = (uint32_t)__shfl(dg, first + 1, 16);
+    const uint32_t d2 = (uint32_t)__shfl(dg, first + 2, 16), d3 = (uint32_t)__shfl(dg, first + 3, 16);
+    const uint32_t shift = 16u - 8u * plane;
+    uint32_t word = ((d0 >> shift) & 0xffu) | (((d1 >> shift) & 0xffu) << 8) | (((d2 >> shift) & 0xffu) << 16) | (((d3 >> shift) & 0xffu) << 24);
+    if (r == 13u) word = __builtin_bit_cast(uint32_t, chunk_sum * unscale);
+    if (r == 14u) word = __builtin_bit_cast(uint32_t, unscale);
+    if (r == 7u || r == 15u) word = tag;
+    return word;
+}
+
 inline int env_int(const char *name, int fallback) {
     const char *held = getenv(name);
     return held && *held ? atoi(held) : fallback;

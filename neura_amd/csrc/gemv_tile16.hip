@@ -759,36 +759,8 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
                 if (!(tile & 1u)) {
                     gate[i] = total;
                 } else if (R == 1 && p.digits_out) {
-                    // the sixteen outputs of this pair are chunk tile / 2 of the next product's activations: lanes 0..15 turn them
-                    // into the three digit planes below a power-of-two scale of their own, as `stage` does for a group
-                    const float value = silu(gate[i]) * total;
-                    uint32_t top = __builtin_bit_cast(uint32_t, value) & 0x7fffffffu;
-                    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR1>((int)top));
-                    top = max(top, (uint32_t)dpp_int<DPP_QUAD_XOR2>((int)top));
-                    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR4>((int)top));
-                    top = max(top, (uint32_t)dpp_int<DPP_ROW_ROR8>((int)top));
-                    const uint32_t raw = top >> 23;
-                    const uint32_t exponent = min(max(raw, 22u), 254u);
-                    const float scale = __builtin_bit_cast(float, (275u - exponent) << 23);
-                    const float unscale = raw == 255u ? __builtin_bit_cast(float, 0x7fc00000u) : __builtin_bit_cast(float, (exponent - 21u) << 23);
-                    const float rounded = rintf(value * scale);
-                    float chunk_sum = rounded;
-                    chunk_sum += dpp<DPP_QUAD_XOR1>(chunk_sum);
-                    chunk_sum += dpp<DPP_QUAD_XOR2>(chunk_sum);
-                    chunk_sum += dpp<DPP_ROW_ROR4>(chunk_sum);
-                    chunk_sum += dpp<DPP_ROW_ROR8>(chunk_sum);
-                    const int dg = (int)signed_digits((int)rounded);
-                    // lane l writes word l of the chunk's 64 bytes (the layout the reader of handed planes states): four digits of
-                    // one plane, a word of the pair, or -- words 7 and 15, the last of each 32-byte sector -- the tag
-                    const uint32_t plane = r < 4u ? 0u : (r < 9u ? 1u : 2u);
-                    const int first = (int)(r < 4u ? 4u * r : (r < 7u ? 4u * (r - 4u) : (r == 8u || r == 12u ? 12u : 4u * (r - 9u)))) & 15;
-                    const uint32_t d0 = (uint32_t)__shfl(dg, first, 16), d1 = (uint32_t)__shfl(dg, first + 1, 16);
-                    const uint32_t d2 = (uint32_t)__shfl(dg, first + 2, 16), d3 = (uint32_t)__shfl(dg, first + 3, 16);
-                    const uint32_t shift = 16u - 8u * plane;
-                    uint32_t word = ((d0 >> shift) & 0xffu) | (((d1 >> shift) & 0xffu) << 8) | (((d2 >> shift) & 0xffu) << 16) | (((d3 >> shift) & 0xffu) << 24);
-                    if (r == 13u) word = __builtin_bit_cast(uint32_t, chunk_sum * unscale);
-                    if (r == 14u) word = __builtin_bit_cast(uint32_t, unscale);
-                    if (r == 7u || r == 15u) word = tag_out;
+                    // the sixteen outputs of this pair are chunk tile / 2 of the next product's activations
+                    const uint32_t word = handed_piece_word(silu(gate[i]) * total, r, tag_out);
                     tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.digits_out + (size_t)(tile >> 1) * 64u) + r, word);
                 } else {
                     tile16_store_word<SEAM::SHARED_OUT>(reinterpret_cast<uint32_t *>(p.y + (size_t)row * (p.N / 2u) + (tile >> 1) * 16u + r),
@@ -1278,7 +1250,7 @@ bool gemv_hands_digits(const GemvArgs &producer, const GemvArgs &consumer) {
     if (consumer.swiglu || consumer.rope || consumer.norm_w) return false;
     GemvArgs from = producer, to = consumer;
     from.digits_out = nullptr, to.digits_in = nullptr;
-    if (!tile16_takes(from)) return false;
+    if (!tile16_takes(from) && !q6k_tile16_takes(from)) return false;  // (both leave the same pieces)
     if (consumer.element == NH_Q6_K || consumer.element == NH_Q3_K) {
         // the Q6_K and Q3_K tiles read the same pieces in the same chunk order
         alignas(16) static const uint8_t somewhere[16] = {};

@@ -739,17 +739,19 @@ def test_a_seam_that_gives_up_sends_the_step_down_the_path_of_one_launch_a_produ
         held.release()
 
 
-@pytest.mark.parametrize("down", [NH_Q4_K, NH_Q6_K], ids=["q4_k ffn_down", "q6_k ffn_down"])
-def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch, down):
-    """At batch 1 the gate|up product of a Q4_K decoder leaves silu(gate) * up as the digit planes ffn_down multiplies (a
+@pytest.mark.parametrize("base,down", [(NH_Q4_K, NH_Q4_K), (NH_Q4_K, NH_Q6_K), (NH_Q6_K, NH_Q6_K), (NH_Q3_K, NH_Q3_K), (NH_Q3_K, NH_Q4_K), (NH_Q5_K, NH_Q6_K)],
+                         ids=["q4_k ffn_down", "q6_k ffn_down", "q6_k throughout", "q3_k throughout", "q3_k into q4_k", "q5_k into q6_k"])
+def test_swiglu_outputs_handed_on_as_digit_planes_match_the_floats(device, monkeypatch, base, down):
+    """At batch 1 the gate|up product of a decoder leaves silu(gate) * up as the digit planes ffn_down multiplies (a
     power-of-two scale per 16 outputs where ffn_down's own staging takes one per 64); NEURA_HIP_TILE16_HANDED=0 hands the
     floats on instead.  Both stay within the decoder's bar of the oracle and of each other (a difference in the last bits of
     a key now and then flips its rounding to half, 5e-4 of it) and choose the same tokens.  With Q6_K down projections (a
-    Q4_K_M file's) the planes feed the Q6_K tiles, which read the same pieces."""
+    Q4_K_M file's) the planes feed the Q6_K tiles, which read the same pieces; gate|up products of Q6_K, Q3_K and Q5_K leave
+    the same pieces, for down projections of any K-quant."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
-    elements = {"blk.%d.ffn_down.weight" % layer: down for layer in range(SMALL_Q4["layers"])} if down != NH_Q4_K else None
-    handed, ref, weights_a = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11, elements=elements)
-    floats, _, weights_b = build(device, SMALL_Q4, NH_Q4_K, batch=1, context=24, seed=11, elements=elements)
+    elements = {"blk.%d.ffn_down.weight" % layer: down for layer in range(SMALL_Q4["layers"])} if down != base else None
+    handed, ref, weights_a = build(device, SMALL_Q4, base, batch=1, context=24, seed=11, elements=elements)
+    floats, _, weights_b = build(device, SMALL_Q4, base, batch=1, context=24, seed=11, elements=elements)
     token = 7
     for step in range(8):
         monkeypatch.setenv("NEURA_HIP_TILE16_HANDED", "1")
