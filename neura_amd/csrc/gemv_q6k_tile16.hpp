@@ -1,4 +1,4 @@
-// The Q6_K product of one activation row on 16-row tiles of the 16x16x64 integer MFMA: the product as a device function (the
+// The Q6_K and Q3_K products of one activation row on 16-row tiles of the 16x16x64 integer MFMA: the product as a device function (the
 // kernel of its own is in gemv_q6k_tile16.hip; gemv_tile16.hip runs it beside a Q4_K product in one launch).
 #pragma once
 #include "gemv_shared.hpp"
@@ -36,7 +36,8 @@ namespace nh {
 // activations it multiplies (or copying them, HANDED: the 64-byte pieces a SwiGLU epilogue left, whose chunk order is this
 // kernel's too); loads run two units ahead across tile boundaries, every wave walks whole rounds of two steps; the finishing
 // wave changes from tile to tile; epilogues: plain (+ residual, in place by one fire-and-forget add), SwiGLU over a gate tile
-// and the up tile behind it, or the cast of a value projection's rows into the value state.
+// and the up tile behind it (as floats, or as the digit planes the product behind takes), the cast of a value projection's
+// rows into the value state, or the rotation of a q|k|v product with its cache append (ROPE).
 //
 // Q3_K (ELEMENT = NH_Q3_K; crates/neura-precision/src/ggml.rs:291-306) has the same sixteen scale groups of 16 in a super-block
 // of 110 bytes: 32 bytes of third bits, 64 of bit pairs, twelve bytes of 6-bit scales and d.  Lane (r, q) takes the 16 bytes of
