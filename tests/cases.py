@@ -40,6 +40,16 @@ def config1():
     return N, K, raw, x
 
 
+def kquant_products(element):
+    """A narrow product of each K-quant at a shape every one-row form takes (48 rows of three super-blocks: whole 16-row tiles,
+    rows of 210- and 110-byte blocks on both alignments): seeded random blocks, activations over a few orders of magnitude."""
+    N, K = 48, 768
+    rng = np.random.default_rng(900 + element)
+    raw = synth.RANDOM[element](rng, N * K)
+    x = (rng.standard_normal(K) * np.exp(rng.uniform(-2.0, 2.0, K))).astype(np.float32)
+    return N, K, raw, x
+
+
 def sha256(array):
     return hashlib.sha256(np.ascontiguousarray(array).view(np.uint8).tobytes()).hexdigest()
 

@@ -1,6 +1,6 @@
 """Writes the committed fixtures of tests/golden/ from the CPU oracle (run from the repository root):
 
-    python tests/golden/make_fixtures.py [blocks] [config1] [config4] [config5]
+    python tests/golden/make_fixtures.py [blocks] [config1] [kquants] [config4] [config5]
 
 A fixture is data -- inputs and the outputs the oracle gave for them on the day it was written -- so that an oracle and a
 kernel that drift together no longer agree with what is stored here.  The tests that read them:
@@ -10,6 +10,8 @@ tests/test_oracle_golden.py (CPU: the oracle against the files) and the GPU test
                                they unpack to                                  (test_gpu_ops.py::test_dequant_of_the_committed_blocks)
   config1_q8_0_gemv.npz/.json  BASELINE configuration 1: the first 64 rows of W, x, every output, and SHA-256 of the whole W
                                and of the outputs                              (test_gpu_ops.py::test_config1_against_the_committed_outputs)
+  kquant_gemv.npz              a one-row product of Q3_K, Q4_K, Q5_K and Q6_K each (48 x 768): blocks, activations and the
+                               oracle's outputs, plain and as silu(gate) * up  (test_gpu_ops.py::test_k_quant_products_against_the_committed_outputs)
   config4_greedy_ids.json      the 64 greedy ids of configuration 4            (test_gpu_decoder.py::test_config4_...)
   config5_normal_greedy_ids.json  the 64 greedy ids of the whole 7B shape with N(0, 0.02) weights packed to Q4_K
                                                                                (test_gpu_decoder.py::test_config5_full_depth_...[normal])
@@ -53,6 +55,17 @@ def config1():
         out.write("\n")
 
 
+def kquants():
+    held = {}
+    for element in (cases.Q3_K, cases.Q4_K, cases.Q5_K, cases.Q6_K):
+        N, K, raw, x = cases.kquant_products(element)
+        y = oracle.gemv(element, raw, N, K, x, threads=THREADS)[0]
+        exact = oracle.unpack(element, raw, N * K).reshape(N, K).astype(np.float64) @ x.astype(np.float64)
+        assert np.abs(y - exact).max() <= 2e-5 * np.abs(exact).max()
+        held["raw_%d" % element], held["x_%d" % element], held["y_bits_%d" % element] = raw, x, y.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "kquant_gemv.npz"), **held)
+
+
 def greedy(shape, element, host, halves, token, context, filled, steps, name, note):
     ref = oracle.Model(shape, element, host, 1, context, 1)
     cache_shape = (shape["kv_heads"], 1, context + 1, shape["head_dim"])
@@ -84,6 +97,6 @@ def config5():
 
 
 if __name__ == "__main__":
-    wanted = sys.argv[1:] or ["blocks", "config1", "config4", "config5"]
+    wanted = sys.argv[1:] or ["blocks", "config1", "kquants", "config4", "config5"]
     for name in wanted:
-        {"blocks": blocks, "config1": config1, "config4": config4, "config5": config5}[name]()
+        {"blocks": blocks, "config1": config1, "kquants": kquants, "config4": config4, "config5": config5}[name]()

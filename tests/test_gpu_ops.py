@@ -150,6 +150,19 @@ def test_config1_against_the_committed_outputs(device):
     tight(device.gemv(NH_Q8_0, held["w_first_64_rows"], 64, K, held["x"])[0], want[:64], 2e-6)
 
 
+@pytest.mark.parametrize("element", [NH_Q3_K, NH_Q4_K, NH_Q5_K, NH_Q6_K])
+def test_k_quant_products_against_the_committed_outputs(device, element):
+    """a one-row product of each K-quant (the 16-row tiles take all four) against the outputs the oracle gave when the fixture
+    was written, plain and with SwiGLU over the stored outputs' halves"""
+    held = np.load(os.path.join(GOLDEN, "kquant_gemv.npz"))
+    N, K, _, _ = cases.kquant_products(element)
+    raw, x, want = held["raw_%d" % element], held["x_%d" % element], held["y_bits_%d" % element].view(np.float32)
+    tight(device.gemv(element, raw, N, K, x)[0], want, 3e-6)
+    gate, up = want[: N // 2].astype(np.float64), want[N // 2:].astype(np.float64)
+    gated = gate / (1.0 + np.exp(-gate)) * up
+    close(device.gemv(element, raw, N, K, x, swiglu=True)[0], gated, rel=1e-3, abs_=1e-4 * max(1.0, np.abs(gated).max()))
+
+
 @pytest.mark.parametrize("name,N,K,seed", [("q", 1536, 1536, 201), ("k", 256, 1536, 202), ("o", 1536, 1536, 203), ("gate", 8960, 1536, 204),
                                            ("down", 1536, 8960, 205)])
 def test_config2_q4_k_gemvs_of_a_1_5b_layer(device, name, N, K, seed):

@@ -40,6 +40,18 @@ def test_the_oracle_answers_configuration_1_as_committed():
     assert np.abs(first - exact).max() <= 2e-5 * np.abs(exact).max()
 
 
+@pytest.mark.parametrize("element", [cases.Q3_K, cases.Q4_K, cases.Q5_K, cases.Q6_K])
+def test_the_oracle_answers_the_k_quant_products_as_committed(element):
+    held = np.load(os.path.join(GOLDEN, "kquant_gemv.npz"))
+    N, K, raw, x = cases.kquant_products(element)
+    assert np.array_equal(raw, held["raw_%d" % element]) and np.array_equal(x, held["x_%d" % element])  # the seeded inputs are the ones stored
+    y = oracle.gemv(element, held["raw_%d" % element], N, K, held["x_%d" % element], threads=4)[0]
+    assert np.array_equal(y.view(np.uint32), held["y_bits_%d" % element])
+    # and the stored outputs are the fp64 product of ggml's published walk (in numpy) to the rounding of fp32 sums
+    exact = synth.DEQUANT[element](held["raw_%d" % element], N * K).reshape(N, K).astype(np.float64) @ held["x_%d" % element].astype(np.float64)
+    assert np.abs(held["y_bits_%d" % element].view(np.float32) - exact).max() <= 2e-5 * np.abs(exact).max()
+
+
 SMALL_Q4 = dict(layers=3, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=1024, vocab=1000, tied=False)
 TINY = dict(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=320, tied=True)
 CUT_7B = dict(synth.SHAPES["qwen2.5-7b"], vocab=4096)  # the 7B shape's layers behind a short vocabulary
