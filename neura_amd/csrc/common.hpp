@@ -225,6 +225,8 @@ int32_t launch_gemv_pair(nh_device *d, const GemvArgs &rotated, const GemvArgs &
 int gemv_chain_level();  // NEURA_HIP_CHAIN: 0 (the default) one launch a product, 1 gate|up with ffn_down, 2 attn_output in front, 3 a product behind
 bool gemv_chains(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail);
 int32_t launch_chain(nh_device *d, const GemvArgs *lead, const GemvArgs &gate_up, const GemvArgs &down, const GemvArgs *trail, uint32_t spin);
+// whether a one-row product with `append_value` set casts its rows into the value state from its own epilogue
+bool gemv_appends_value(const GemvArgs &a);
 // moves the device's tick word on: once at the start of every pass over a decoder's layers, before anything that writes tags
 int32_t launch_tick(nh_device *d);
 // whether launch_gemv can fold `rope` into this product (else the caller runs the rotation as its own kernel)

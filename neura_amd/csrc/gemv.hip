@@ -2611,11 +2611,19 @@ bool gemv_merges_sections(const GemvArgs &a, uint32_t width) {
     return (uint64_t)a.N * payload_bytes(a.element, a.K) < (1ull << 32);
 }
 
+// Whether a product with `append_value` set casts its rows into the value state itself: one row of a K-quant on the 16-row
+// tiles, or on the staged kernel where a row is one K slice.
+bool gemv_appends_value(const GemvArgs &a) {
+    if (!a.append_value || a.rows != 1 || a.rope || a.swiglu || a.residual) return false;
+    if (tile16_takes(a) || q6k_tile16_takes(a)) return true;
+    return staged_super_block(a.element) && a.K <= 4096u && a.append_value->width && a.N % a.append_value->width == 0;
+}
+
 int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (!a.rope && !a.append_value && (a.bias[0] || a.bias[1] || a.bias[2]))
         return fail(NH_E_ARGUMENT, "a product adds a bias only where it folds the rotation in or appends value rows");
-    if (a.append_value && !(staged_super_block(a.element) && a.rows == 1 && !a.rope))
-        return fail(NH_E_ARGUMENT, "only a one-row product of a staged K-quant appends its rows to the value state");
+    if (a.append_value && !gemv_appends_value(a))
+        return fail(NH_E_ARGUMENT, "this product does not append its rows to the value state (ask gemv_appends_value first)");
     if (a.merge && (!gemv_merges_sections(a, a.merge->width) || a.merge->sections < 2u || a.merge->sections > MERGED_SECTIONS_MOST || !a.merge->groups ||
                     (a.K / a.merge->width) % a.merge->groups))
         return fail(NH_E_ARGUMENT, "this product merges no attention sections (ask gemv_merges_sections first)");

@@ -158,6 +158,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
     auto fetch_the_rest = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         NH_FETCH(p.y, p.residual, p.N, p.K, p.rows, p.eps, p.digits_out);
+        if (MODE == TILE16_PLAIN && R == 1) NH_FETCH(p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
         if (MODE == TILE16_ROPE)
             NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_width, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions,
                      p.rope_ring, p.rope_element, p.bias[0], p.bias[1], p.bias[2], p.refusal, p.end[0], p.end[1]);
@@ -794,6 +795,15 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
                 } else {
                     p.y[n] = p.residual ? p.residual[n] + total : total;
                 }
+                if (!CHAINED && R == 1 && MODE == TILE16_PLAIN && p.append_value) {
+                    // a value projection of one token: its rows (+ bias) go into the value state at the cursor, as
+                    // value_append_kernel would cast them
+                    const uint32_t cursor = p.rope_cursor[0];
+                    const float value = p.bias[0] ? total + p.bias[0][n] : total;
+                    const uint32_t slot = p.rope_ring ? cursor % p.rope_ring : cursor;
+                    if (slot >= p.rope_capacity) atomicMax(p.refusal, (uint32_t)REFUSAL_ORIGIN);
+                    else state_store(p.rope_v, p.rope_element, ((uint64_t)((uint32_t)n / p.rope_width) * p.rope_capacity + slot) * p.rope_width + (uint32_t)n % p.rope_width, value);
+                }
             }
           }
         }
@@ -1212,7 +1222,11 @@ bool tile16_takes(const GemvArgs &a) {
     if ((a.element != NH_Q4_K && a.element != NH_Q5_K) || a.rows < 1 || a.rows > TILE16_MOST_ROWS || a.K % 256u != 0 || a.K == 0) return false;
     if (env_int("NEURA_HIP_TILE16", 1) == 0 || env_int("NEURA_HIP_MFMA", 1) != 1) return false;
     // Q5_K (one row): the same tiles with the fifth bit beside the nibble; NEURA_HIP_Q5K_TILE16=0 leaves it to the staged kernel
-    if (a.element == NH_Q5_K && (a.rows != 1 || a.append_value || a.merge || env_int("NEURA_HIP_Q5K_TILE16", 1) == 0)) return false;
+    if (a.element == NH_Q5_K && (a.rows != 1 || a.merge || env_int("NEURA_HIP_Q5K_TILE16", 1) == 0)) return false;
+    // a value projection that casts its rows into the value state: one row, whole heads, no other epilogue
+    if (a.append_value && (a.rows != 1 || a.swiglu || a.rope || a.residual || a.digits_in || a.digits_out || a.W[1] || a.W[2] || !a.append_value->width ||
+                           a.N % a.append_value->width))
+        return false;
     for (int m = 0; m < 3; m++)
         if (a.W[m] && ((uintptr_t)a.W[m] & 15u)) return false;
     if (a.rows > 1 && (a.rope || a.rows > (uint32_t)env_int("NEURA_HIP_TILE16_ROWS", (int)TILE16_MOST_ROWS))) return false;
@@ -1423,6 +1437,10 @@ static Tile16Launch tile16_plan(nh_device *d, const GemvArgs &a, uint32_t fixed_
         p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring, p.rope_element = a.rope->element;
         p.refusal = d->refusal;
         for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
+    }
+    if (a.append_value) {  // (a plain product: the width here is the value heads', not a tile's)
+        p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
+        p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.rope_element = a.append_value->element, p.bias[0] = a.bias[0];
     }
     // waves of a workgroup share a tile and split its super-blocks: about two steps a wave
     // (sixteen on deep rows, where turning the activations into digits is the larger part of a wave's work; eight where the

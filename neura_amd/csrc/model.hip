@@ -202,9 +202,11 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
                 qk.bias[0] = m->bias_q[L], qk.bias[1] = m->bias_k[L];
                 GemvArgs value = narrow(m, element_at(m, L, V), m->attn_v[L], KW, H, m->h, T, m->xn);
                 value.norm_w = m->attn_norm[L], value.eps = c.eps;
-                // a staged K-quant product of one K slice casts its rows into the value state itself; others leave that to a small kernel
-                const bool appends = staged_super_block(value.element) && H <= 4096u && KW % hd == 0 && !(getenv("NEURA_HIP_APPEND_VALUE") && getenv("NEURA_HIP_APPEND_VALUE")[0] == '0');
-                if (appends) value.append_value = &rope_qk, value.bias[0] = m->bias_v[L];
+                // a K-quant product on the tiles (or on the staged kernel, of one K slice) casts its rows into the value state itself;
+                // others leave that to a small kernel
+                value.append_value = &rope_qk, value.bias[0] = m->bias_v[L];
+                const bool appends = gemv_appends_value(value) && !(getenv("NEURA_HIP_APPEND_VALUE") && getenv("NEURA_HIP_APPEND_VALUE")[0] == '0');
+                if (!appends) value.append_value = nullptr, value.bias[0] = nullptr;
                 if (gemv_pairs(d, qk, value)) {  // both in one launch: neither waits for the other
                     if ((status = launch_gemv_pair(d, qk, value)) != NH_OK) return status;
                 } else {

@@ -168,7 +168,7 @@ def test_masked_planes_and_chunked_fill(device):
 
 MIXED = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q6_K, "blk.2.ffn_down.weight": NH_Q6_K, "blk.2.ffn_gate.weight": NH_Q6_K}
 # the way Q3_K_M files are: Q3_K for most, Q5_K and Q4_K for some projections, a Q6_K head
-MIXED_3 = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.ffn_down.weight": NH_Q5_K, "blk.1.attn_output.weight": NH_Q4_K,
+MIXED_3 = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.attn_v.weight": NH_Q4_K, "blk.1.ffn_down.weight": NH_Q5_K, "blk.1.attn_output.weight": NH_Q4_K,
            "blk.2.attn_q.weight": NH_Q4_K, "blk.2.attn_k.weight": NH_Q4_K, "blk.2.attn_v.weight": NH_Q4_K, "blk.2.ffn_up.weight": NH_Q5_K}
 
 
@@ -180,7 +180,9 @@ def test_mixed_elements_and_projection_biases(device, batch, base, mixed):
     carry Qwen2's biases: layer 0 (a Q6_K value projection, biases) takes one product per matrix, layer 1 (one element,
     biases) folds rotation and biases into the stacked product at batch 1, layer 2 (gate and up stored differently) runs
     the two halves apart.  Decode steps, a 16-row fill and the caches against the oracle.  The same for decoders stored in
-    one K-quant throughout (the fill's q|k|v is then one stacked wide product of that element on the matrix cores)."""
+    one K-quant throughout (the fill's q|k|v is then one stacked wide product of that element on the matrix cores).  In the
+    Q3_K_M mix layers 0 and 1 rotate q|k in a Q3_K product and cast the rows of a Q5_K and a Q4_K value projection into the
+    value state from those products' own epilogues."""
     shape = SMALL_Q4
     rng = np.random.default_rng(21)
     tensors = list(synth.model_tensors(shape, base, rng, mode="normal", elements=mixed, biases=(0, 1)))
