@@ -1497,9 +1497,9 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
-// Two independent one-row products over the same activation row in one launch: a Q4_K q|k product with the rotation folded in
-// and the Q6_K value projection that casts its rows into the value state -- what a layer of a Q4_K_M file asks for where the
-// value projection is stored in Q6_K.  The first `lead_grid` workgroups run the Q4_K product, the others the Q6_K one; neither
+// Two independent one-row products over the same activation row in one launch: a Q4_K (FIFTH: Q5_K) q|k product with the rotation
+// folded in and the Q6_K value projection that casts its rows into the value state -- what a layer of a Q4_K_M or Q5_K_M file asks
+// for where the value projection is stored in Q6_K.  The first `lead_grid` workgroups run the Q4_K product, the others the Q6_K one; neither
 // waits for the other.  As two launches the pair takes 6.1 + 6.5 us, and nearly all of either is the launch and the first
 // round trips.
 struct Q6kBeside {
@@ -1508,14 +1508,14 @@ struct Q6kBeside {
     uint32_t row_bytes, grid, tiles, tile_rows;
     GemvParams p;
 };
-template <int NW>
+template <int NW, bool FIFTH = false>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_rope_beside_q6k_kernel(const uint8_t *lead_w0, const void *lead_input, const float *lead_norm_w, int32_t lead_to_w1,
                                                                            int32_t lead_to_w2, uint32_t lead_row_bytes, uint32_t lead_grid, uint32_t lead_tiles,
                                                                            uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, GemvParams p, Q6kBeside beside) {
     extern __shared__ __attribute__((aligned(16))) uint8_t pair_lds_bytes[];
     if (blockIdx.x < lead_grid) {
-        Tile16Unit ring[2];
-        tile16_product<NW, 2, TILE16_ROPE, 1, false>(pair_lds_bytes, blockIdx.x, NoSeam{}, ring, nullptr, 0u, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes,
+        typename Tile16UnitOf<FIFTH>::type ring[2];
+        tile16_product<NW, 2, TILE16_ROPE, 1, false, NoSeam, FIFTH>(pair_lds_bytes, blockIdx.x, NoSeam{}, ring, nullptr, 0u, lead_w0, lead_input, lead_norm_w, lead_to_w1, lead_to_w2, lead_row_bytes,
                                                      lead_grid, lead_tiles, lead_tile_rows, lead_end0, lead_end1, p);
     } else {
         q6k_tile16_product<NW, false, false>(pair_lds_bytes, blockIdx.x - lead_grid, beside.w0, lead_input, beside.norm_w, beside.row_bytes, beside.grid, beside.tiles,
@@ -1523,18 +1523,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_rope_beside_q6k_kernel(const
     }
 }
 
-template <int NW>
+template <int NW, bool FIFTH>
 static hipError_t launch_pair_instance(nh_device *d, const Tile16Launch &first, const Q6kLaunch &second) {
     const size_t lds = first.lds > second.lds ? first.lds : second.lds;
     static bool raised = false;
     if (!raised && lds > 64u * 1024u) {
-        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_rope_beside_q6k_kernel<NW>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t error = hipFuncSetAttribute((const void *)gemv_q4k_rope_beside_q6k_kernel<NW, FIFTH>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (error != hipSuccess) return error;
         raised = true;
     }
     const GemvParams &p = first.p;
     Q6kBeside beside{second.p.W[0], second.p.norm_w, second.p.row_bytes, second.grid, second.p.row_groups, second.p.tile_rows, second.p};
-    hipLaunchKernelGGL((gemv_q4k_rope_beside_q6k_kernel<NW>), dim3(first.grid + second.grid), dim3(NW * 64), lds, d->stream, p.W[0], static_cast<const void *>(p.x), p.norm_w,
+    hipLaunchKernelGGL((gemv_q4k_rope_beside_q6k_kernel<NW, FIFTH>), dim3(first.grid + second.grid), dim3(NW * 64), lds, d->stream, p.W[0], static_cast<const void *>(p.x), p.norm_w,
                        (int32_t)((p.W[1] - p.W[0]) / 16), (int32_t)((p.W[2] - p.W[0]) / 16), p.row_bytes, first.grid, p.row_groups, p.rope_width, p.end[0], p.end[1], p, beside);
     return hipGetLastError();
 }
@@ -1542,7 +1542,7 @@ static hipError_t launch_pair_instance(nh_device *d, const Tile16Launch &first, 
 // NEURA_HIP_PAIR=0 keeps the two launches
 bool gemv_pairs(nh_device *d, const GemvArgs &rotated, const GemvArgs &value) {
     if (env_int("NEURA_HIP_PAIR", 1) == 0) return false;
-    if (rotated.element != NH_Q4_K || !rotated.rope || rotated.rows != 1 || !tile16_takes(rotated)) return false;
+    if ((rotated.element != NH_Q4_K && rotated.element != NH_Q5_K) || !rotated.rope || rotated.rows != 1 || !tile16_takes(rotated)) return false;
     if (value.element != NH_Q6_K || !value.append_value || value.rows != 1 || value.digits_in || !q6k_tile16_takes(value)) return false;
     if (rotated.x != value.x || rotated.norm_w != value.norm_w || rotated.K != value.K || rotated.eps != value.eps) return false;
     const uint32_t waves = tile16_plan(d, rotated).waves;
@@ -1554,7 +1554,11 @@ int32_t launch_gemv_pair(nh_device *d, const GemvArgs &rotated, const GemvArgs &
     const Tile16Launch first = tile16_plan(d, rotated);
     const Q6kLaunch second = q6k_tile16_plan(d, value);
     profile_mark(d);
-    hipError_t launched = first.waves == 4u ? launch_pair_instance<4>(d, first, second) : first.waves == 7u ? launch_pair_instance<7>(d, first, second) : launch_pair_instance<8>(d, first, second);
+    hipError_t launched;
+    if (rotated.element == NH_Q5_K)
+        launched = first.waves == 4u ? launch_pair_instance<4, true>(d, first, second) : first.waves == 7u ? launch_pair_instance<7, true>(d, first, second) : launch_pair_instance<8, true>(d, first, second);
+    else
+        launched = first.waves == 4u ? launch_pair_instance<4, false>(d, first, second) : first.waves == 7u ? launch_pair_instance<7, false>(d, first, second) : launch_pair_instance<8, false>(d, first, second);
     NH_HIP(launched);
     profile_mark(d);
     if (d->profile) d->profile_bytes += (uint64_t)rotated.N * first.p.row_bytes + (uint64_t)value.N * second.p.row_bytes;

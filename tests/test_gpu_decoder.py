@@ -798,20 +798,22 @@ def test_attention_sections_merged_by_the_output_projection_match_the_fold(devic
         held.release()
 
 
+@pytest.mark.parametrize("base,mixed", [(NH_Q4_K, MIXED), (NH_Q5_K, MIXED), (NH_Q3_K, MIXED_3)], ids=["q4_k_m", "q5_k_m", "q3_k_m"])
 @pytest.mark.parametrize("pair", ["1", "0"], ids=["one launch", "two launches"])
-def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, monkeypatch, pair):
+def test_value_rows_appended_by_their_product_equal_the_append_kernels(device, monkeypatch, pair, base, mixed):
     """Where q|k go out rotated from one product and the value projection is stored otherwise (layer 0 of the Q4_K_M-like
-    mix: Q6_K), the value product casts its rows (+ bias) into the value state itself -- beside the q|k product in one
-    launch, or (NEURA_HIP_PAIR=0) in a launch of its own; NEURA_HIP_APPEND_VALUE=0 leaves the cast to the append kernel.
+    mix: Q6_K; the same mix over Q5_K; layers 0 and 1 of the Q3_K_M-like mix: Q5_K and Q4_K), the value product casts its
+    rows (+ bias) into the value state itself -- beside a Q4_K or Q5_K q|k product in one launch, or (NEURA_HIP_PAIR=0, and
+    wherever no pair is built) in a launch of its own; NEURA_HIP_APPEND_VALUE=0 leaves the cast to the append kernel.
     The same sums either way: states and logits equal bit for bit, and the oracle's tokens."""
     monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
     monkeypatch.setenv("NEURA_HIP_PAIR", pair)
     shape = SMALL_Q4
-    tensors = list(synth.model_tensors(shape, NH_Q4_K, np.random.default_rng(21), mode="normal", elements=MIXED, biases=(0, 1)))
+    tensors = list(synth.model_tensors(shape, base, np.random.default_rng(21), mode="normal", elements=mixed, biases=(0, 1)))
     host = {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
     weights = Weights(device, tensors)
-    fused, apart = Model(device, weights, shape, NH_Q4_K, 1, 24, 1), Model(device, weights, shape, NH_Q4_K, 1, 24, 1)
-    ref = oracle.Model(shape, NH_Q4_K, host, 1, 24, 1, elements=MIXED)
+    fused, apart = Model(device, weights, shape, base, 1, 24, 1), Model(device, weights, shape, base, 1, 24, 1)
+    ref = oracle.Model(shape, base, host, 1, 24, 1, elements=mixed)
     token = 11
     for step in range(6):
         monkeypatch.setenv("NEURA_HIP_APPEND_VALUE", "1")
