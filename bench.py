@@ -60,17 +60,23 @@ def workload(name):
         return synth.SHAPES["qwen2.5-0.5b"], 8, 1088, {}, ()
     if name == "qwen2.5-1.5b-q4k":  # the shape whose layer products are BASELINE's second configuration
         return synth.SHAPES["qwen2.5-1.5b"], 12, 1088, {}, ()
-    if name == "qwen2.5-7b-q4_k_m":
+    if name in ("qwen2.5-7b-q4_k_m", "qwen2.5-7b-q5_k_m", "qwen2.5-7b-q3_k_m"):
         # the mix llama.cpp's Q4_K_M recipe gives a Qwen2.5-7B file: the head and, in the first and last eighth of the layers
-        # and every third between, the value and down projections in Q6_K, the rest Q4_K; q, k and v biases everywhere
+        # and every third between, the value and down projections in Q6_K, the rest Q4_K; q, k and v biases everywhere.
+        # Q5_K_M: the same over Q5_K.  Q3_K_M: Q3_K for q, k, gate and up, Q4_K for o, Q5_K for v and down in those
+        # layers and Q4_K in the others.
         shape = synth.SHAPES["qwen2.5-7b"]
         count = shape["layers"]
         more_bits = [i for i in range(count) if i < count // 8 or i >= 7 * count // 8 or (i - count // 8) % 3 == 2]
         mixed = {"output.weight": 14}
-        for i in more_bits:
-            mixed["blk.%d.attn_v.weight" % i] = 14
-            mixed["blk.%d.ffn_down.weight" % i] = 14
-        return shape, 12, 4096, mixed, tuple(range(count))
+        base = {"qwen2.5-7b-q4_k_m": 12, "qwen2.5-7b-q5_k_m": 13, "qwen2.5-7b-q3_k_m": 11}[name]
+        for i in range(count):
+            if base == 11:
+                mixed["blk.%d.attn_output.weight" % i] = 12
+                mixed["blk.%d.attn_v.weight" % i] = mixed["blk.%d.ffn_down.weight" % i] = 13 if i in more_bits else 12
+            elif i in more_bits:
+                mixed["blk.%d.attn_v.weight" % i] = mixed["blk.%d.ffn_down.weight" % i] = 14
+        return shape, base, 4096, mixed, tuple(range(count))
     raise SystemExit("unknown workload %s" % name)
 
 
