@@ -473,19 +473,26 @@ def test_staged_super_block_product_reads_packed_weights(device, element):
     tight(device.gemv(element, raw, N, K, x), oracle.gemv(element, raw, N, K, x, threads=8), 2e-6)
 
 
-def test_gemv_is_linear_and_matches_at_full_size(device):
+@pytest.mark.parametrize("element", [NH_Q4_K, NH_Q6_K, NH_Q5_K, NH_Q3_K])
+def test_gemv_is_linear_and_matches_at_full_size(device, element):
     # size-independent properties at the 7B FFN shape: W(a x + b z) = a W x + b W z
     rng = np.random.default_rng(6)
     N, K = 18944, 3584
-    raw = device.upload(synth.q4_k_random(rng, N * K))
+    host = synth.RANDOM[element](rng, N * K)
+    raw = device.upload(host)
     x, z = rng.standard_normal(K).astype(np.float32), rng.standard_normal(K).astype(np.float32)
-    yx, yz = device.gemv(NH_Q4_K, raw, N, K, x)[0], device.gemv(NH_Q4_K, raw, N, K, z)[0]
-    both = device.gemv(NH_Q4_K, raw, N, K, np.float32(0.5) * x - np.float32(2.0) * z)[0]
+    yx, yz = device.gemv(element, raw, N, K, x)[0], device.gemv(element, raw, N, K, z)[0]
+    both = device.gemv(element, raw, N, K, np.float32(0.5) * x - np.float32(2.0) * z)[0]
     tight(both, 0.5 * yx - 2.0 * yz, 1e-5)
-    batched = device.gemv(NH_Q4_K, raw, N, K, np.stack([x, z]))
-    tight(batched[0], yx, 2e-6)
-    tight(batched[1], yz, 2e-6)
-    assert np.array_equal(yx, device.gemv(NH_Q4_K, raw, N, K, x)[0])  # deterministic
+    batched = device.gemv(element, raw, N, K, np.stack([x, z]))
+    tight(batched[0], yx, 3e-6)  # (two rows of a K-quant other than Q4_K run the staged kernel: another order of the sums)
+    tight(batched[1], yz, 3e-6)
+    assert np.array_equal(yx, device.gemv(element, raw, N, K, x)[0])  # deterministic
+    # and a handful of rows against the exact product of the unpacked weights
+    row_bytes = host.nbytes // N
+    for n in rng.integers(0, N, 8):
+        weights = oracle.unpack(element, host[n * row_bytes:(n + 1) * row_bytes], K).astype(np.float64)
+        assert abs(float(yx[n]) - float(weights @ x.astype(np.float64))) <= 2e-5 * max(1.0, float(np.abs(yx).max()))
 
 
 def test_gemv_refuses_bad_shapes(device):
