@@ -26,7 +26,9 @@ namespace nh {
 // Epilogues: y (+ in-place residual by one fire-and-forget add), SwiGLU over a gate tile and the up tile behind it, or the
 // rotation with the cache append (tile rows = 8 channels c.. and their partners c + width/2.. of one head).
 constexpr uint32_t TILE16_ZERO_BYTES = 208;    // what an idle A lane reads: four chunk offsets (0, 48, 96, 144) + 16 bytes
-enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2 };
+// (TILE16_APPEND: a plain product of one row that also casts its outputs into the value state -- a form of its own, so that the
+// plain products of a step fetch and test nothing for it)
+enum Tile16Mode { TILE16_PLAIN = 0, TILE16_SWIGLU = 1, TILE16_ROPE = 2, TILE16_APPEND = 3 };
 
 static size_t tile16_lds(uint32_t nblk, uint32_t NW, uint32_t R, bool handed = false) {
     const size_t sums = handed ? (size_t)nblk * TILE16_BLOCK_PAIRS : (size_t)R * nblk * 64u;
@@ -135,6 +137,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
                                                uint32_t lead_tiles, uint32_t lead_tile_rows, uint32_t lead_end0, uint32_t lead_end1, const GemvParams &p) {
     static_assert(R == 1 || MODE != TILE16_ROPE, "the rotation is folded into the product of one row only");
     static_assert(!HANDED || (R == 1 && MODE == TILE16_PLAIN), "handed-over digit planes feed a plain product of one row");
+    static_assert(MODE != TILE16_APPEND || (R == 1 && !SEAM::SHARED_IN && !SEAM::SHARED_OUT), "a value projection's append rides a product of one row with a launch of its own");
     static_assert(!(SEAM::WAITS || SEAM::SHARED_IN || SEAM::SHARED_OUT) || R == 1, "products of one row are chained");
     static_assert(!FIFTH || (R == 1 && !SEAM::HANDS_RING && !SEAM::TAKES_RING), "Q5_K: one row, a launch of its own");
     typedef typename Tile16UnitOf<FIFTH>::type Unit;
@@ -158,7 +161,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
     auto fetch_the_rest = [&]() {
         __builtin_amdgcn_sched_barrier(0);
         NH_FETCH(p.y, p.residual, p.N, p.K, p.rows, p.eps, p.digits_out);
-        if (MODE == TILE16_PLAIN && R == 1) NH_FETCH(p.append_value, p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
+        if (MODE == TILE16_APPEND) NH_FETCH(p.rope_cursor, p.rope_v, p.rope_width, p.rope_capacity, p.rope_ring, p.rope_element, p.bias[0], p.refusal);
         if (MODE == TILE16_ROPE)
             NH_FETCH(p.rope_cosines, p.rope_sines, p.rope_cursor, p.rope_k, p.rope_v, p.rope_width, p.rope_q_rows, p.rope_k_rows, p.rope_capacity, p.rope_positions,
                      p.rope_ring, p.rope_element, p.bias[0], p.bias[1], p.bias[2], p.refusal, p.end[0], p.end[1]);
@@ -197,7 +200,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
     const uint32_t first_tile = block, hop = lead_grid;
     // a plain tile may hold fewer than 16 rows (a matrix of 3584 rows is 256 tiles of 14, one a compute unit, where it is 224
     // of 16): the columns past them walk the tile's last row again and are never written
-    const uint32_t tile_rows = MODE == TILE16_PLAIN ? lead_tile_rows : 16u;
+    const uint32_t tile_rows = MODE == TILE16_PLAIN || MODE == TILE16_APPEND ? lead_tile_rows : 16u;
     auto lane_row = [w0, to_w1, to_w2, end0, end1, row_bytes, half_width, tiles_per_head, tile_rows, r, q](uint32_t tile) -> const uint8_t * {
         (void)tile_rows;  // the SwiGLU form's tiles are whole
         int64_t offset;
@@ -795,7 +798,7 @@ __device__ __forceinline__ void tile16_product(uint8_t *tile16_lds_bytes, const 
                 } else {
                     p.y[n] = p.residual ? p.residual[n] + total : total;
                 }
-                if (!CHAINED && R == 1 && MODE == TILE16_PLAIN && p.append_value) {
+                if constexpr (MODE == TILE16_APPEND) {
                     // a value projection of one token: its rows (+ bias) go into the value state at the cursor, as
                     // value_append_kernel would cast them
                     const uint32_t cursor = p.rope_cursor[0];
@@ -1480,7 +1483,9 @@ int32_t launch_tile16(nh_device *d, const GemvArgs &a) {
     const size_t lds = plan.lds;
     profile_mark(d);
     hipError_t launched;
-    if (a.element == NH_Q5_K)
+    if (a.append_value)
+        launched = a.element == NH_Q5_K ? launch_tile16_fifth<TILE16_APPEND, false>(d, p, waves, grid, lds) : launch_tile16_rows<TILE16_APPEND, 1>(d, p, waves, grid, lds);
+    else if (a.element == NH_Q5_K)
         launched = a.digits_in ? launch_tile16_fifth<TILE16_PLAIN, true>(d, p, waves, grid, lds)
                    : a.swiglu  ? launch_tile16_fifth<TILE16_SWIGLU, false>(d, p, waves, grid, lds)
                    : a.rope    ? launch_tile16_fifth<TILE16_ROPE, false>(d, p, waves, grid, lds)
