@@ -96,9 +96,13 @@ def config4_case(threads=None):
     return shape, tensors, host, halves, token
 
 
-def config5_normal_case():
-    """BASELINE configuration 5 with weights a test can see through: the whole 7B shape, N(0, 0.02) weights packed to Q4_K by
-    the reference's encoder, states holding 4032 positions."""
+def config5_case(mode):
+    """BASELINE configuration 5, the whole 7B shape with states holding 4032 positions.  "normal": weights a test can see
+    through, N(0, 0.02) packed to Q4_K by the reference's encoder; "blocks": the benchmark's random Q4_K blocks."""
     shape = synth.SHAPES["qwen2.5-7b"]
-    tensors, host, halves, token = decoder_case(shape, Q4_K, "normal", 52, None, 1, 4096 - 64)
+    tensors, host, halves, token = decoder_case(shape, Q4_K, mode, 52, None, 1, 4096 - 64)
     return shape, tensors, host, halves, token
+
+
+def config5_normal_case():
+    return config5_case("normal")

@@ -1,6 +1,6 @@
 """Writes the committed fixtures of tests/golden/ from the CPU oracle (run from the repository root):
 
-    python tests/golden/make_fixtures.py [blocks] [config1] [kquants] [config4] [config5]
+    python tests/golden/make_fixtures.py [blocks] [config1] [kquants] [config4] [config5] [config5_blocks]
 
 A fixture is data -- inputs and the outputs the oracle gave for them on the day it was written -- so that an oracle and a
 kernel that drift together no longer agree with what is stored here.  The tests that read them:
@@ -15,6 +15,7 @@ tests/test_oracle_golden.py (CPU: the oracle against the files) and the GPU test
   config4_greedy_ids.json      the 64 greedy ids of configuration 4            (test_gpu_decoder.py::test_config4_...)
   config5_normal_greedy_ids.json  the 64 greedy ids of the whole 7B shape with N(0, 0.02) weights packed to Q4_K
                                                                                (test_gpu_decoder.py::test_config5_full_depth_...[normal])
+  config5_blocks_greedy_ids.json  the same with the benchmark's random Q4_K blocks (test_gpu_decoder.py::test_config5_full_depth_...[blocks])
 """
 import json
 import os
@@ -96,7 +97,13 @@ def config5():
            "cases.config5_normal_case: 7B shape, N(0, 0.02) weights packed to Q4_K, states holding 4032 positions, 64 greedy steps of the oracle")
 
 
+def config5_blocks():
+    shape, _, host, halves, token = cases.config5_case("blocks")
+    greedy(shape, cases.Q4_K, host, halves, token, 4096, 4096 - 64, 64, "config5_blocks_greedy_ids.json",
+           "cases.config5_case('blocks'): 7B shape, random Q4_K blocks (a degenerate network), states holding 4032 positions, 64 greedy steps of the oracle")
+
+
 if __name__ == "__main__":
-    wanted = sys.argv[1:] or ["blocks", "config1", "kquants", "config4", "config5"]
+    wanted = sys.argv[1:] or ["blocks", "config1", "kquants", "config4", "config5", "config5_blocks"]
     for name in wanted:
-        {"blocks": blocks, "config1": config1, "kquants": kquants, "config4": config4, "config5": config5}[name]()
+        {"blocks": blocks, "config1": config1, "kquants": kquants, "config4": config4, "config5": config5, "config5_blocks": config5_blocks}[name]()

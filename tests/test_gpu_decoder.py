@@ -433,7 +433,8 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device, mode):
     weights packed by the reference's Q4_K encoder -- a network whose logits, tokens and appended rows depend on every
     input-dependent piece (embedding row, rotation at the cursor, cache append, attention over the appended rows)."""
     shape = synth.SHAPES["qwen2.5-7b"]
-    layers, context, filled, rows = 2, 4096, 3500, 512
+    # (the degenerate twin fills 128 rows -- the same kernels over one tile of rows -- which spares the oracle half a minute)
+    layers, context, filled, rows = 2, 4096, 3500, 512 if mode == "normal" else 128
     rng = np.random.default_rng(50)
     tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode=mode, layers=layers, threads=16))
     host = {name: raw for name, _, _, raw in tensors}
@@ -468,13 +469,13 @@ def test_config5_shape_two_layers_qwen2_5_7b_q4_k(device, mode):
     # what the three steps appended: the rotated key rows and the value rows at the stepped cursors (the epilogue of the
     # q|k|v product at 4608 x 3584)
     same_cache_rows(model, ref, layers, [[filled, filled + 1, filled + 2]], "rows the batch-1 steps appended")
-    # a fill of 512 rows behind the keys already held (positions 3503 .. 4014), then a step that weighs what it wrote
+    # a fill of 512 (128) rows behind the keys already held (positions 3503 .. 4014), then a step that weighs what it wrote
     prompt = rng.integers(0, shape["vocab"], rows)
     first = filled + 3
     model.prefill(prompt, rows, [first])
     ref.forward(prompt, rows, [first], want_logits=False, threads=16)
     same_cache_rows(model, ref, layers, [list(range(first, first + rows))], "rows the fill appended")
-    same(model, ref, token, [first + rows], "batch 1 after the 512-row fill")
+    same(model, ref, token, [first + rows], "batch 1 after the %d-row fill" % rows)
     same_cache_rows(model, ref, layers, [[first + rows]], "the row behind the fill")
     model.release()
     model, ref = pair(8, 1)
@@ -493,13 +494,21 @@ def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device, mode):
     holding 4032 positions of N(0,1) halves, then 64 greedy steps up to the end of the context of 4096 -- every token
     identical to the oracle's, with no allowance for close calls.  "blocks": the benchmark's random Q4_K blocks (a
     degenerate network: one token, margins in the hundreds -- the products' bulk accuracy); "normal": N(0, 0.02) weights
-    packed by the reference's encoder (tokens vary, margins are small and printed; nothing is gated on them).  The
-    oracle follows the reference's summation order; identity against the reference binary itself is unpinned (it cannot
-    be run here)."""
+    packed by the reference's encoder (tokens vary, margins are small and printed; nothing is gated on them).
+
+    The oracle's 64 ids are the committed ones (tests/golden/make_fixtures.py wrote them from these same seeded inputs: two
+    minutes of host time a file).  Beside the device the oracle itself runs the first NEURA_TEST_ORACLE_STEPS steps (default 8;
+    64 runs it all the way): its ids must be the file's, the device's logits must lie within 1e-3 of its largest, and the key
+    and value rows those steps append must be its rows.  The oracle follows the reference's summation order; identity against
+    the reference binary itself is unpinned (it cannot be run here)."""
     shape = synth.SHAPES["qwen2.5-7b"]
     context, steps = 4096, 64
+    live = max(1, min(steps, int(os.environ.get("NEURA_TEST_ORACLE_STEPS", "8"))))
     filled = context - steps
-    tensors, host, halves, token = cases.decoder_case(shape, NH_Q4_K, mode, 52, None, 1, filled)
+    shape_, tensors, host, halves, token = cases.config5_case(mode)
+    assert shape_ is shape
+    stored = golden_ids("config5_%s_greedy_ids.json" % mode)
+    assert len(stored) == steps
     weights = Weights(device, tensors)
     model = Model(device, weights, shape, NH_Q4_K, 1, context, 1)
     ref = oracle.Model(shape, NH_Q4_K, host, 1, context, 1)
@@ -508,25 +517,25 @@ def test_config5_full_depth_greedy_64_steps_qwen2_5_7b_shape_q4_k(device, mode):
     got = want = token
     got_tokens, want_tokens, gaps, apart = [], [], [], []
     for step in range(steps):
-        want_logits, chosen = ref.forward([want], 1, [filled + step], threads=16)
-        want = int(chosen[0])
         got = int(model.decode_step([got], [filled + step])[0])
-        want_tokens.append(want), got_tokens.append(got)
-        gaps.append(float(margins(want_logits)[0]))
-        apart.append(float(np.abs(model.logits() - want_logits).max() / np.abs(want_logits).max()))
-        if step % 8 == 7:
-            print("step %d (%s): tokens identical so far, smallest top-2 margin %.3g" % (step, mode, min(gaps)), flush=True)
-        if got != want:
+        got_tokens.append(got)
+        if step < live:
+            want_logits, chosen = ref.forward([want], 1, [filled + step], threads=16)
+            want = int(chosen[0])
+            want_tokens.append(want)
+            gaps.append(float(margins(want_logits)[0]))
+            apart.append(float(np.abs(model.logits() - want_logits).max() / np.abs(want_logits).max()))
+        if got != stored[step]:
             break
-    print("greedy tokens (%s): %s" % (mode, want_tokens))
-    print("greedy margins (top1 - top2) over %d steps: min %.3g median %.3g; logits within %.3g of the largest" %
+    print("greedy tokens (%s): %s" % (mode, got_tokens))
+    print("the oracle beside the device over %d steps: top-2 margins min %.3g median %.3g; logits within %.3g of the largest" %
           (len(gaps), min(gaps), float(np.median(gaps)), max(apart)))
+    assert want_tokens == stored[:len(want_tokens)], "the oracle no longer chooses what it chose when the fixture was written"
     assert max(apart) <= 1e-3
-    assert got_tokens == want_tokens, "first divergence at step %d, margin %g" % (len(got_tokens) - 1, gaps[-1])
+    assert got_tokens == stored, "first divergence from the oracle's ids at step %d" % (len(got_tokens) - 1)
     if mode == "normal":
-        assert len(set(want_tokens)) > steps // 2, want_tokens
-        same_cache_rows(model, ref, shape["layers"], [list(range(filled, filled + steps))], "rows the 64 steps appended")
-        assert want_tokens == golden_ids("config5_normal_greedy_ids.json")
+        assert len(set(got_tokens)) > steps // 2, got_tokens
+        same_cache_rows(model, ref, shape["layers"], [list(range(filled, filled + live))], "rows the first steps appended")
     model.release(), weights.release()
 
 
