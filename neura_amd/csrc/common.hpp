@@ -295,7 +295,8 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &args);
 int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t positions, float *cosines, float *sines);
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            void *cache_k, void *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base, bool ring, int32_t cache_element = NH_F16);
+                           const uint8_t *mask, float base, bool ring, int32_t cache_element = NH_F16, const float *cosines = nullptr,
+                           const float *sines = nullptr, uint32_t positions = 0);  // (a model's table of cosines and sines, where it has one)
 
 // one token of one plane: v (+ bias) as halves into the value state at cursor[0] (at cursor[0] % ring when the cache is a ring)
 int32_t launch_value_append(nh_device *d, const float *v, const float *bias, void *cache_v, uint32_t kv_heads, uint32_t width, uint32_t capacity,

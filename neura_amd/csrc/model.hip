@@ -233,7 +233,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             }
         }
         if (!products_only && !roped && (status = launch_rope_append(d, m->qkv, c.heads, c.kv_heads, hd, B, rows, m->cache_k[L], m->cache_v[L],
-                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base, m->ring, c.cache_element)) != NH_OK)
+                                                           m->capacity, m->window, dev_cursor(m), mask, c.rope_base, m->ring, c.cache_element, m->rope_cos, m->rope_sin,
+                                                           m->positions)) != NH_OK)
             return status;
         AttentionArgs at{};
         at.q = m->qkv, at.out = m->att;

@@ -185,63 +185,70 @@ int32_t launch_rope_angles(nh_device *d, float base, uint32_t width, uint32_t po
 // The decoder's fused form of the two kernels above on a token-major buffer
 // qkv [T][(heads + 2 kv_heads) * width], t = row * batch + plane: q is roped in place, k is
 // roped, k and v are cast to the states' element and appended to the caches.
+// A token a blockIdx.y, its (vector, channel pair) items over blockIdx.x: no 64-bit division on the way to an item.  `cosines` /
+// `sines` [positions][width / 2] (may be null): what rotate() would compute for (position, channel pair), tabulated by
+// rope_angles_kernel with the same instructions, so a table entry is bit for bit the cosine and sine formed on the spot;
+// positions past the table are formed on the spot.
 template <int CE>
 __global__ __launch_bounds__(256) void rope_append_kernel(float *__restrict__ qkv, uint32_t heads, uint32_t kv_heads, uint32_t width,
                                                           uint32_t batch, uint32_t rows, void *__restrict__ cache_k,
                                                           void *__restrict__ cache_v, uint32_t capacity, uint32_t window,
                                                           const uint32_t *__restrict__ cursor, const uint8_t *__restrict__ mask,
-                                                          const float *__restrict__ table, uint32_t *refusal, bool ring) {
-    NH_FETCH(qkv, heads, kv_heads, width, batch, rows, cache_k, cache_v, capacity, window, cursor, mask, table, refusal);
+                                                          const float *__restrict__ table, uint32_t *refusal, bool ring,
+                                                          const float *__restrict__ cosines, const float *__restrict__ sines, uint32_t positions) {
+    NH_FETCH(qkv, heads, kv_heads, width, batch, rows, cache_k, cache_v, capacity, window, cursor, mask, table, refusal, cosines, sines, positions);
     const uint32_t half = width / 2;
     const uint32_t vectors = heads + 2 * kv_heads;  // per token: q heads, k heads, v heads
     const uint32_t stride = vectors * width;
-    const uint64_t total = (uint64_t)batch * rows * vectors * half;
-    for (uint64_t index = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; index < total; index += (uint64_t)gridDim.x * blockDim.x) {
-        uint32_t c = (uint32_t)(index % half);
-        uint32_t vector = (uint32_t)((index / half) % vectors);
-        uint32_t t = (uint32_t)(index / half / vectors);
-        uint32_t row = t / batch, b = t % batch;
+    const uint32_t items = vectors * half, tokens = batch * rows;
+    const uint32_t item = blockIdx.x * blockDim.x + threadIdx.x;
+    if (item >= items) return;
+    const uint32_t c = item % half, vector = item / half;
+    for (uint32_t t = blockIdx.y; t < tokens; t += gridDim.y) {
+        const uint32_t row = t / batch, b = t % batch;
         float *src = qkv + (size_t)t * stride + (size_t)vector * width;
-        uint32_t position = cursor[b] + row;
+        const uint32_t position = cursor[b] + row;
+        const bool key = vector >= heads && vector < heads + kv_heads;
+        float low = src[c], high = src[c + half];
+        if (vector < heads || key) {
+            if (cosines && position < positions) {
+                const float cosine = cosines[(size_t)position * half + c], sine = sines[(size_t)position * half + c];
+                const float turned_low = low * cosine - high * sine, turned_high = high * cosine + low * sine;
+                low = turned_low, high = turned_high;
+            } else {
+                rotate(low, high, position, table[c], low, high);
+            }
+        }
         if (vector < heads) {
-            float low, high;
-            rotate(src[c], src[c + half], position, table[c], low, high);
             src[c] = low;
             src[c + half] = high;
             continue;
         }
-        bool active = mask == nullptr || mask[b];
-        uint32_t slot = active ? (ring ? position % window : position) : window + row;
+        const bool active = mask == nullptr || mask[b];
+        const uint32_t slot = active ? (ring ? position % window : position) : window + row;
         if (slot >= capacity) {
             atomicMax(refusal, (uint32_t)REFUSAL_ORIGIN);
             continue;
         }
-        if (vector < heads + kv_heads) {
-            uint32_t head = vector - heads;
-            float low, high;
-            rotate(src[c], src[c + half], position, table[c], low, high);
-            uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
-            cache_store<CE>(cache_k, at + c, low);
-            cache_store<CE>(cache_k, at + c + half, high);
-        } else {
-            uint32_t head = vector - heads - kv_heads;
-            uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
-            cache_store<CE>(cache_v, at + c, src[c]);
-            cache_store<CE>(cache_v, at + c + half, src[c + half]);
-        }
+        const uint32_t head = key ? vector - heads : vector - heads - kv_heads;
+        const uint64_t at = (((uint64_t)head * batch + b) * capacity + slot) * width;
+        void *cache = key ? cache_k : cache_v;
+        cache_store<CE>(cache, at + c, low);
+        cache_store<CE>(cache, at + c + half, high);
     }
 }
 
 int32_t launch_rope_append(nh_device *d, float *qkv, uint32_t heads, uint32_t kv_heads, uint32_t width, uint32_t batch, uint32_t rows,
                            void *cache_k, void *cache_v, uint32_t capacity, uint32_t window, const uint32_t *cursor,
-                           const uint8_t *mask, float base, bool ring, int32_t cache_element) {
+                           const uint8_t *mask, float base, bool ring, int32_t cache_element, const float *cosines, const float *sines,
+                           uint32_t positions) {
     const float *table = rope_frequencies(d, base, width);
     if (!table) return NH_E_DEVICE;
-    uint64_t total = (uint64_t)batch * rows * (heads + 2 * kv_heads) * (width / 2);
-    if (!total) return NH_OK;
-    uint32_t grid = (uint32_t)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
-#define NH_ROPE(CE) hipLaunchKernelGGL(rope_append_kernel<CE>, dim3(grid), dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k, \
-                                       cache_v, capacity, window, cursor, mask, table, d->refusal, ring)
+    const uint32_t items = (heads + 2 * kv_heads) * (width / 2), tokens = batch * rows;
+    if (!items || !tokens) return NH_OK;
+    const dim3 grid((items + 255u) / 256u, tokens < 65535u ? tokens : 65535u);
+#define NH_ROPE(CE) hipLaunchKernelGGL(rope_append_kernel<CE>, grid, dim3(256), 0, d->stream, qkv, heads, kv_heads, width, batch, rows, cache_k, \
+                                       cache_v, capacity, window, cursor, mask, table, d->refusal, ring, cosines, sines, positions)
     if (cache_element == NH_F32) NH_ROPE(NH_F32);
     else if (cache_element == NH_BF16) NH_ROPE(NH_BF16);
     else NH_ROPE(NH_F16);
