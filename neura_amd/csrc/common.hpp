@@ -118,7 +118,7 @@ int32_t launch_convert_half(nh_device *d, const float *src, uint64_t elements, u
 // written to the key cache at the cursor, the rest are rounded to fp16 into the value cache.
 struct RopeFusion {
     const float *cosines, *sines;  // [positions][width / 2]: cos and sin of f32(position) * pow(base, -2c/width)
-    const uint32_t *cursor;        // device, one plane
+    const uint32_t *cursor;        // device: a word a plane (a product of one row reads the first)
     uint16_t *cache_k, *cache_v;
     uint32_t width, q_rows, k_rows, capacity;
     uint32_t positions;  // rows of the two tables

@@ -1183,6 +1183,14 @@ struct MfmaParams {
     uint32_t tiles;  // 16-row tiles
     int32_t swiglu;
     float eps;
+    // the rotation folded into a q|k|v product of several planes, one token each (gemv_q4k_mfma32_kernel<.., ROPE>): activation
+    // row b is plane b, whose token sits at rope_cursor[b]
+    const float *rope_cosines, *rope_sines, *bias[3];
+    const uint32_t *rope_cursor;
+    uint16_t *rope_k, *rope_v;
+    uint32_t *refusal;
+    uint32_t rope_width, rope_q_rows, rope_k_rows, rope_capacity, rope_positions, rope_ring;
+    int32_t rope_element;
 };
 
 // What a wave of the matrix-core products needs before its first loads, as leading plain arguments the hardware hands over in
@@ -1534,9 +1542,15 @@ struct Tile32Unit {
     u32x4 hdr, g[4];
 };
 
-template <int J, int NW, int KS>
+// ROPE: a q|k|v product of several planes, one token each, with the rotation, the biases and the cache append in its epilogue
+// (crates/neura-kernel/src/task/rope.rs:95-122, crates/neura-decoder/src/cache.rs:347-348).  A tile then holds sixteen
+// channels c.. of a head in its rows 0..15 and their partners c + width/2.. in its rows 16..31, so the lane 16 further holds the
+// number a rotated output needs beside its own; q rows go to y, k rows rotated and v rows as they are into the states at the
+// plane's cursor, as rope_append_kernel would leave them (the same table of cosines and sines, the same three roundings).
+template <int J, int NW, int KS, bool ROPE = false>
 __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_kernel(MFMA_LEAD_PARAMETERS) {  // second bound: waves per SIMD
     MFMA_TAKE_LEAD;
+    static_assert(!ROPE || J == 4, "the rotation is folded into the product of five to eight planes");
 
     constexpr uint32_t M8 = 8 * J, R2 = 2 * J, TPW = NW / KS, NT = NW * 64;
     constexpr bool STAGED = J == 1;  // raw blocks through LDS; with eight activation rows the digits leave no room for them
@@ -1655,8 +1669,15 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
         const uint32_t r0 = at_tile * 32u;
         const bool in0 = r0 < end0, in1 = r0 < end1;
         const uint8_t *const plain_base = (in0 ? w0 : (in1 ? w1 : w2)) + (size_t)(r0 - (in0 ? 0u : (in1 ? end0 : end1))) * p.row_bytes;
+        // ROPE: the tile's first output row -- channel c0 of a head -- and what its rows 16..31 lie further (half a head)
+        const uint32_t rope_tiles_a_head = ROPE ? rest.rope_width / 32u : 1u, rope_half = ROPE ? rest.rope_width / 2u : 0u;
+        const uint32_t rope_first = ROPE ? (at_tile / rope_tiles_a_head) * rest.rope_width + (at_tile % rope_tiles_a_head) * 16u : 0u;
+        // (a head never straddles two matrices: the tile's first row names the matrix of all its rows)
+        const uint8_t *const rope_base = (rope_first < end0 ? w0 : (rope_first < end1 ? w1 : w2)) +
+                                         (size_t)(rope_first - (rope_first < end0 ? 0u : (rope_first < end1 ? end0 : end1))) * p.row_bytes;
         auto row_base = [&](uint32_t r) -> const uint8_t * {
             if (gated) return (r < 16u ? w0 : w1) + (size_t)(at_tile * 16u + (r & 15u)) * p.row_bytes;
+            if constexpr (ROPE) return rope_base + (size_t)((r & 15u) + (r >= 16u ? rope_half : 0u)) * p.row_bytes;
             return plain_base + (size_t)r * p.row_bytes;
         };
         // A super-block of the tile is 32 rows x 144 bytes = 288 pieces of 16 bytes.  Lane l fetches pieces l, l + 64, ...: nine
@@ -1733,14 +1754,48 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 3) void gemv_q4k_mfma32_ker
 #pragma unroll
         for (int j = 0; j < J; j++) mine[j * 64 + lane] = acc[j];
         __syncthreads();
-        if (ks == 0) {
+        // (the first J waves of the tile take a pair of activation rows each: one wave's reads of the tile's parts do not queue
+        // behind another pair's, nor the rotation's loads; the sums and their order are the same)
+        static_assert(KS >= J, "a wave of the tile for every pair of activation rows");
+        if (ks < (uint32_t)J) {
             const float *from = part + (size_t)(parity * TPW + ts) * KS * J * 64u;
-#pragma unroll
-            for (int j = 0; j < J; j++) {
+            for (int once = 0; once < 1; once++) {  // (a loop for its `continue`s)
+                const uint32_t j = ks;
                 float total = 0.0f;
 #pragma unroll
-                for (int k = 0; k < KS; k++) total += from[(size_t)k * J * 64u + j * 64 + lane];
+                for (int k = 0; k < KS; k++) total += from[(size_t)k * J * 64u + j * 64u + lane];
                 const uint32_t arow = 2u * j + q;
+                if constexpr (ROPE) {
+                    // (what the rotation needs is read from the kernel's own argument block, `rest`: a member of the local copy
+                    // chosen by a number would put the whole copy into scratch memory)
+                    const uint32_t row_n = rope_first + (n & 15u) + (n >= 16u ? rope_half : 0u);  // the output row among q|k|v's
+                    const uint32_t c = (at_tile % rope_tiles_a_head) * 16u + (n & 15u);           // its channel pair
+                    const bool first0 = rope_first < end0, first1 = rope_first < end1;            // the tile's matrix: one for all its rows
+                    const float *bias = first0 ? rest.bias[0] : (first1 ? rest.bias[1] : rest.bias[2]);
+                    if (bias) total += bias[row_n - (first0 ? 0u : (first1 ? end0 : end1))];
+                    const float other = __shfl_xor(total, 16, 64);
+                    if (!live || arow >= p.rows) continue;
+                    const uint32_t position = rest.rope_cursor[arow];
+                    float value = total;
+                    if (row_n < rest.rope_k_rows) {
+                        const size_t at = (size_t)min(position, rest.rope_positions - 1u) * rope_half + c;
+                        const float cosine = rest.rope_cosines[at], sine = rest.rope_sines[at];
+                        value = n >= 16u ? total * cosine + other * sine : total * cosine - other * sine;
+                    }
+                    if (row_n < rest.rope_q_rows) {
+                        rest.y[(size_t)arow * rest.N + row_n] = value;
+                    } else if (position >= rest.rope_positions || (!rest.rope_ring && position >= rest.rope_capacity)) {
+                        atomicMax(rest.refusal, (uint32_t)REFUSAL_ORIGIN);
+                    } else {
+                        const bool key = row_n < rest.rope_k_rows;
+                        const uint32_t within = row_n - (key ? rest.rope_q_rows : rest.rope_k_rows);  // head * width + channel
+                        const uint32_t head = within / rest.rope_width, channel = within % rest.rope_width;
+                        const uint32_t slot = rest.rope_ring ? position % rest.rope_ring : position;  // a ring seats position p at p mod its span
+                        state_store(key ? rest.rope_k : rest.rope_v, rest.rope_element, (((uint64_t)head * p.rows + arow) * rest.rope_capacity + slot) * rest.rope_width + channel,
+                                    value);
+                    }
+                    continue;
+                }
                 const float up = __shfl_xor(total, 16, 64);
                 if (!live || arow >= p.rows) continue;
                 if (p.splits > 1) {
@@ -2365,8 +2420,15 @@ static int32_t launch_mfma(nh_device *d, const GemvArgs &a) {
 }
 
 // mirrors the conditions under which launch_rows<1> takes the decode kernel with two rows per pass
+static bool mfma32_takes(const nh_device *d, const GemvArgs &a);
+
 bool gemv_fuses_rope(const GemvArgs &a, const RopeFusion &rope) {
     if (env_int("NEURA_HIP_FUSE_ROPE", 1) == 0) return false;
+    if (a.rows >= 5 && a.rows <= 8) {  // one token of each of five to eight planes: the 32-row integer tiles
+        GemvArgs folded = a;
+        folded.rope = &rope;
+        return !((uintptr_t)rope.cosines & 3u) && rope.positions > 0 && mfma32_takes(nullptr, folded);
+    }
     if (a.rows != 1 || a.swiglu || a.residual) return false;
     {
         GemvArgs folded = a;
@@ -2399,7 +2461,14 @@ static size_t mfma32_lds(uint32_t nblk, uint32_t J, uint32_t NW) {
 // it measured faster -- several activation rows, or one row against a tall matrix
 static bool mfma32_takes(const nh_device *d, const GemvArgs &a) {
     const int mode = env_int("NEURA_HIP_MFMA32", 1);
-    if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.rows > 8) return false;
+    if (mode == 0 || a.element != NH_Q4_K || a.K % 256u != 0 || a.rows > 8) return false;
+    if (a.rope) {
+        // five to eight planes of one token each, rows of one K slice, heads of whole 32-row tiles that never straddle two matrices
+        const uint32_t width = a.rope->width;
+        if (a.rows < 5 || a.K > 3584u || a.swiglu || a.residual || width < 32u || width % 32u || a.N % width || a.end[0] % width || a.end[1] % width ||
+            a.end[2] != a.N || a.rope->q_rows % width || a.rope->k_rows % width || a.rope->q_rows > a.rope->k_rows || a.rope->k_rows > a.N)
+            return false;
+    }
     // deeper rows go in K slices with a fold behind them: worth it from five activation rows on, and never with a fused norm
     if (a.K > 4096u && (a.norm_w || (mode != 2 && a.rows < 5))) return false;
     if (a.swiglu) {
@@ -2418,11 +2487,11 @@ static bool mfma32_takes(const nh_device *d, const GemvArgs &a) {
     return a.rows >= 3 && (a.N >= 65536u || a.N <= 8192u);
 }
 
-template <int J, int NW, int KS>
+template <int J, int NW, int KS, bool ROPE = false>
 static int32_t launch_mfma32_instance(nh_device *d, const MfmaParams &p, size_t lds) {
     static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
     if (lds > 64 * 1024 && !widened) {
-        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma32_kernel<J, NW, KS>), hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024));
+        NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4k_mfma32_kernel<J, NW, KS, ROPE>), hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024));
         widened = true;
     }
     // one resident round of workgroups, as many as LDS and registers let a compute unit hold
@@ -2434,7 +2503,7 @@ static int32_t launch_mfma32_instance(nh_device *d, const MfmaParams &p, size_t 
     uint32_t most = (uint32_t)d->compute_units * resident / p.splits;
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
-    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, MFMA_LEAD(p));
+    hipLaunchKernelGGL((gemv_q4k_mfma32_kernel<J, NW, KS, ROPE>), dim3(blocks_x, p.splits), dim3(NW * 64), lds, d->stream, MFMA_LEAD(p));
     NH_HIP(hipGetLastError());
     return NH_OK;
 }
@@ -2449,6 +2518,13 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     p.N = a.N, p.K = a.K, p.nblk = a.K / 256u, p.row_bytes = p.nblk * 144u, p.rows = a.rows;
     p.swiglu = a.swiglu, p.eps = a.eps;
     p.tiles = a.N / 32u;
+    if (a.rope) {
+        p.rope_cosines = a.rope->cosines, p.rope_sines = a.rope->sines, p.rope_cursor = a.rope->cursor, p.rope_k = a.rope->cache_k, p.rope_v = a.rope->cache_v;
+        p.rope_width = a.rope->width, p.rope_q_rows = a.rope->q_rows, p.rope_k_rows = a.rope->k_rows, p.rope_capacity = a.rope->capacity;
+        p.rope_positions = a.rope->positions, p.rope_ring = a.rope->ring, p.rope_element = a.rope->element;
+        p.refusal = d->refusal;
+        for (int s = 0; s < 3; s++) p.bias[s] = a.bias[s];
+    }
     const uint32_t J = a.rows <= 2 ? 1u : 4u;  // a two-pair form spilled at 128 registers; three and four rows take the four-pair one
     // K slices: at most 14 super-blocks with eight staged rows (the digits of 3584 activations x 8 rows fill 112 KiB), 16 otherwise
     const uint32_t most_blocks = J == 4 ? 14u : 16u;
@@ -2463,7 +2539,8 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     int32_t status;
     // with eight staged rows, a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
     const bool few = p.tiles * p.splits < 2u * (uint32_t)d->compute_units;
-    if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.slice_blocks, 1, 4));
+    if (a.rope) status = few ? launch_mfma32_instance<4, 16, 16, true>(d, p, mfma32_lds(p.slice_blocks, 4, 16)) : launch_mfma32_instance<4, 16, 4, true>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
+    else if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.slice_blocks, 1, 4));
     else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
     else status = launch_mfma32_instance<4, 16, 4>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
     if (status != NH_OK) return status;
@@ -2632,7 +2709,11 @@ int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
     if (tile16_takes(a)) return launch_tile16(d, a);
     if (q6k_tile16_takes(a)) return launch_q6k_tile16(d, a);
     if (a.digits_out || a.digits_in) return fail(NH_E_ARGUMENT, "this product hands over no digit planes (ask gemv_hands_digits first)");
-    if (a.rope && (a.rows != 1 || mfma_takes(a))) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
+    if (a.rope && a.rows != 1) {  // several planes: the 32-row integer tiles or nothing
+        if (!mfma32_takes(d, a)) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
+        return launch_mfma32(d, a);
+    }
+    if (a.rope && mfma_takes(a)) return fail(NH_E_ARGUMENT, "this product cannot fold the rotation in (ask gemv_fuses_rope first)");
     if (f16_tiles_take(d, a)) return launch_f16_tiles(d, a);
     if (mfma32_takes(d, a)) return launch_mfma32(d, a);
     if (mfma_takes(a)) return launch_mfma(d, a);

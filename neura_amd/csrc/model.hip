@@ -181,7 +181,8 @@ int32_t forward(nh_model *m, uint32_t rows, bool any_inactive, bool products_onl
             const bool halves = true;
             RopeFusion rope{m->rope_cos, m->rope_sin, dev_cursor(m), reinterpret_cast<uint16_t *>(m->cache_k[L]), reinterpret_cast<uint16_t *>(m->cache_v[L]),
                             hd, QW, QW + KW, m->capacity, m->positions, m->ring ? m->window : 0u, c.cache_element};
-            if (halves && alike && !products_only && T == 1 && !mask && gemv_fuses_rope(a, rope)) {
+            // (five to eight planes of one token each: the same from the product of the 32-row tiles, every plane at its own cursor)
+            if (halves && alike && !products_only && rows == 1 && !mask && gemv_fuses_rope(a, rope)) {
                 a.rope = &rope;
                 a.bias[0] = m->bias_q[L], a.bias[1] = m->bias_k[L], a.bias[2] = m->bias_v[L];
                 roped = true;

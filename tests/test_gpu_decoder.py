@@ -679,6 +679,54 @@ def test_rotation_folded_into_the_product_matches_the_separate_kernel(device, mo
         held.release()
 
 
+@pytest.mark.parametrize("shape,biased", [(SMALL_Q4, False), (SMALL_Q4, True), (WIDE_CUT, False)], ids=["small", "small-biased", "3584"])
+@pytest.mark.parametrize("batch", [5, 8])
+def test_rotation_folded_into_the_product_of_several_planes(device, monkeypatch, shape, biased, batch):
+    """Five to eight planes of one token each: the q|k|v product of a Q4_K decoder (the 32-row integer tiles) rotates q and k
+    and appends k and v in its epilogue, every plane at its own cursor.  The twin with the rotation as a kernel of its own runs
+    the same product kernel and the same table of cosines and sines, so logits and caches agree bit for bit; both are held to
+    the oracle (logits, tokens, and the rows the steps appended).  With q, k and v biases the twin multiplies the three
+    matrices one by one: each row's sums are the same, and so are the bits."""
+    monkeypatch.setenv("NEURA_HIP_GRAPH", "0")  # both twins launch eagerly, so the switch below is read at every step
+    layers = list(range(shape["layers"])) if biased else []
+
+    def pair():
+        rng = np.random.default_rng(31)
+        tensors = list(synth.model_tensors(shape, NH_Q4_K, rng, mode="normal" if shape is not WIDE_CUT else "blocks", biases=layers))
+        weights = Weights(device, tensors)
+        return Model(device, weights, shape, NH_Q4_K, batch, 40, 1), weights, {name: (raw.view(np.float32) if name.endswith(".bias") else raw) for name, _, _, raw in tensors}
+
+    folded, weights_a, host = pair()
+    apart, weights_b, _ = pair()
+    ref = oracle.Model(shape, NH_Q4_K, host, batch, 40, 1)
+    tokens = [3 + 7 * plane for plane in range(batch)]
+    first = [3 * plane for plane in range(batch)]  # every plane at a cursor of its own
+    steps = 5
+    for step in range(steps):
+        cursors = [at + step for at in first]
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1")
+        got_a = folded.decode_step(tokens, cursors)
+        logits_a = folded.logits()
+        monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "0")
+        got_b = apart.decode_step(tokens, cursors)
+        logits_b = apart.logits()
+        want_logits, want = ref.forward(tokens, 1, cursors)
+        assert np.array_equal(logits_a, logits_b), step
+        assert np.abs(logits_a - want_logits).max() <= 1e-3 * np.abs(want_logits).max()
+        assert list(got_a) == list(got_b) == list(want), (step, margins(want_logits))
+        tokens = [int(t) for t in got_a]
+    for layer in range(shape["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(folded.cache_read(layer, which), apart.cache_read(layer, which)), (layer, which)
+    same_cache_rows(folded, ref, shape["layers"], [list(range(at, at + steps)) for at in first], "rows the planes' steps appended")
+    # a cursor past the window is refused by the folded form as by the separate kernel
+    monkeypatch.setenv("NEURA_HIP_FUSE_ROPE", "1")
+    with pytest.raises(NeuraError):
+        folded.decode_step(tokens, [folded.capacity + 3] * batch)
+    for held in (folded, apart, weights_a, weights_b):
+        held.release()
+
+
 # (a chained launch hands ffn_down's first weights across the seam: it takes rows of sixteen super-blocks and more)
 CHAIN_SMALL = dict(layers=2, hidden=512, heads=8, kv_heads=2, head_dim=128, ffn=4096, vocab=1000, tied=False)
 CHAIN_SHAPES = [CHAIN_SMALL, dict(layers=2, hidden=3584, heads=28, kv_heads=4, head_dim=128, ffn=18944, vocab=2048, tied=False)]
