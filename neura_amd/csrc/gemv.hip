@@ -2053,13 +2053,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MFMA_LEAD_PARAMET
 #pragma unroll
         for (int e = 0; e < 4; e++) mine[e * 64 + lane] = acc[e];
         __syncthreads();
-        if (ks == 0) {
+        // (the first four waves of the tile take one of the four C registers each -- a wave's reads of the tile's parts do not
+        // queue behind another register's, and every wave waits for them at the barrier below; the sums and their order are the same)
+        static_assert(KS >= 4, "a wave of the tile for every C register");
+        if (ks < 4u) {
             const float *from = part + ((size_t)parity * TPW + ts) * KS * 4u * 64u;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
+            for (int once = 0; once < 1; once++) {  // (a loop for its `continue`)
+                const uint32_t e = ks;
                 float total = 0.0f;
 #pragma unroll
-                for (int k = 0; k < KS; k++) total += from[(size_t)k * 4u * 64u + e * 64 + lane];
+                for (int k = 0; k < KS; k++) total += from[(size_t)k * 4u * 64u + e * 64u + lane];
                 // C row 4 kq + e: activation row 4 kq + e for kq < 2, its residue plane for kq >= 2 (32 lanes on)
                 const float residue = __shfl_xor(total, 32, 64);
                 const uint32_t arow = 4u * (kq & 1u) + e;
