@@ -1835,6 +1835,7 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t F16_BLOCK_PIECES = 8u * 4u * 16u + 2u * 16u;  // 16-byte pieces of LDS per staged super-block: operands, then sums
+constexpr uint32_t F16_TWO_SETS_BLOCKS = 14;  // up to so many staged super-blocks leave LDS room for two sets of the waves' partial sums
 
 template <int NW, int KS>
 __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MFMA_LEAD_PARAMETERS) {
@@ -1981,7 +1982,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MFMA_LEAD_PARAMET
             if (ahead_round + 1u < rounds) ahead_row = row_of(++ahead_round);
         }
     };
-    constexpr uint32_t parity = 0;  // one set of partial sums: 16 super-blocks of operands leave no room for two
+    // Two sets of partial sums where the operands leave room (up to fourteen super-blocks staged: what the launcher asked LDS
+    // for says so): a tile's parts are read while the next tile's are written, and no wave waits for the readers.  Sixteen
+    // super-blocks of operands leave room for one set, and a barrier behind the readers.
+    const bool two_sets = nb <= F16_TWO_SETS_BLOCKS;
+    uint32_t parity = 0;
     {
         f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
         uint32_t tile = 0;
@@ -2080,7 +2085,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_q4k_f16_kernel(MFMA_LEAD_PARAMET
                 }
             }
         }
-            __syncthreads();  // the next tile's partial sums take the same places
+            if (two_sets) parity ^= 1u;  // (a wave gets no further than the next tile's barrier before the readers are done)
+            else __syncthreads();        // the next tile's partial sums take the same places
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[e] = 0.0f;
         };
@@ -2563,7 +2569,9 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
 // against a matrix of enough tiles to give every wave several super-blocks (gate|up 36.6 against 42 us, the head 91 against
 // 110, ffn_down 29 against 27 with its fold; q|k|v and the output projection, one super-block a wave, are slower: 16.2 and
 // 12.5 against 11.4 and 11.2)
-static size_t f16_tiles_lds(uint32_t blocks, uint32_t NW) { return (size_t)blocks * F16_BLOCK_PIECES * 16u + (size_t)NW * 4u * 64u * sizeof(float); }
+static size_t f16_tiles_lds(uint32_t blocks, uint32_t NW) {
+    return (size_t)blocks * F16_BLOCK_PIECES * 16u + (size_t)(blocks <= F16_TWO_SETS_BLOCKS ? 2u : 1u) * NW * 4u * 64u * sizeof(float);
+}
 static bool f16_tiles_take(const nh_device *d, const GemvArgs &a) {
     const int mode = env_int("NEURA_HIP_F16_TILES", 1);
     if (mode == 0 || a.element != NH_Q4_K || a.rope || a.K % 256u != 0 || a.rows < 2 || a.rows > 8) return false;
