@@ -2547,7 +2547,8 @@ static int32_t launch_mfma32(nh_device *d, const GemvArgs &a) {
     profile_mark(d);
     int32_t status;
     // with eight staged rows, a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
-    const bool few = p.tiles * p.splits < 2u * (uint32_t)d->compute_units;
+    // (ffn_down of the 7B shape at eight rows, 112 tiles in six slices, is among the few: 22.0 -> 21.0 us)
+    const bool few = p.tiles * p.splits < 3u * (uint32_t)d->compute_units;
     if (a.rope) status = few ? launch_mfma32_instance<4, 16, 16, true>(d, p, mfma32_lds(p.slice_blocks, 4, 16)) : launch_mfma32_instance<4, 16, 4, true>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
     else if (J == 1) status = launch_mfma32_instance<1, 4, 4>(d, p, mfma32_lds(p.slice_blocks, 1, 4));
     else if (few) status = launch_mfma32_instance<4, 16, 16>(d, p, mfma32_lds(p.slice_blocks, 4, 16));
@@ -2626,10 +2627,10 @@ static int32_t launch_f16_tiles(nh_device *d, const GemvArgs &a) {
         if (!p.partial) return NH_E_MEMORY;
     }
     profile_mark(d);
-    // a matrix of few tiles deals each tile's super-blocks to sixteen waves instead of four
-    const bool few = p.tiles * p.splits < 4u * (uint32_t)d->compute_units;
+    // sixteen waves a tile: a workgroup walks one tile at a time, so the tiles deal evenly over the compute units (with four waves
+    // a tile and four tiles a round, gate|up's 2368 tiles were 2.3 rounds a workgroup, walked as three: batch 8 2.90 -> 2.78 ms a step)
     const size_t lds = f16_tiles_lds(p.slice_blocks, 16);
-    int32_t status = few ? launch_f16_tiles_instance<16, 16>(d, p, lds) : launch_f16_tiles_instance<16, 4>(d, p, lds);
+    int32_t status = launch_f16_tiles_instance<16, 16>(d, p, lds);
     if (status != NH_OK) return status;
     if (p.splits > 1) {
         const uint32_t outputs = a.swiglu ? a.N / 2 : a.N;
