@@ -10,7 +10,8 @@
 //                              included); 3 and 4 rows where the kernel above refuses and the digits still fit LDS
 //                              (with FIFTH the same for one row of Q5_K; gemv_q6k_tile16_kernel is its sibling for one row of Q6_K or Q3_K)
 //   gemv_q4k_f16_kernel        5 to 8 rows, K <= 4096, at least 4 x 256 tiles of 16 rows (gate|up and the head at batch 5-8)
-//   gemv_q4k_mfma32_kernel     5 to 8 rows otherwise (q|k|v, attn_output; ffn_down in K slices with gemv_fold_kernel), matrices
+//   gemv_q4k_mfma32_kernel     5 to 8 rows otherwise (q|k|v -- with the rotation and the cache append in its epilogue where five to
+//                              eight planes step one token each --, attn_output; ffn_down in K slices with gemv_fold_kernel), matrices
 //                              that end on 32-row tiles; 3 and 4 rows of short (<= 8192 rows) or very tall (>= 65536) matrices that the
 //                              two kernels on top refused
 //   gemv_q4k_mfma_kernel       what is left with matrices on 16-row tiles and either several rows or K > 4096: ffn_down at
@@ -2643,7 +2644,7 @@ static int32_t launch_f16_tiles(nh_device *d, const GemvArgs &a) {
     return NH_OK;
 }
 
-// Q6_K, Q5_K, Q3_K: two activation rows at most per launch (their slices and the raw rows share 64 KiB of LDS)
+// Q6_K, Q5_K, Q3_K: one, two or four activation rows a launch (their slices and the raw rows share LDS: three workgroups a compute unit)
 template <int ELEMENT, int RB>
 static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *x, float *y, const float *residual) {
     GemvParams p{};
@@ -2661,7 +2662,8 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
         p.append_value = 1u, p.rope_v = a.append_value->cache_v, p.rope_cursor = a.append_value->cursor, p.rope_width = a.append_value->width;
         p.rope_capacity = a.append_value->capacity, p.rope_ring = a.append_value->ring, p.rope_element = a.append_value->element, p.bias[0] = a.bias[0], p.refusal = d->refusal;
     }
-    const uint32_t most_blocks = 16u;
+    // K slices of sixteen super-blocks at most; of eight with four activation rows, whose slices take the room of two rows' twice over
+    const uint32_t most_blocks = RB == 4 ? 8u : 16u;
     p.splits = (p.nblk + most_blocks - 1) / most_blocks;
     p.blocks_per_split = (p.nblk + p.splits - 1) / p.splits;
     p.splits = (p.nblk + p.blocks_per_split - 1) / p.blocks_per_split;
@@ -2678,6 +2680,13 @@ static int32_t launch_staged_rows(nh_device *d, const GemvArgs &a, const float *
     if (most < 1) most = 1;
     if (blocks_x > most) blocks_x = most;
     profile_mark(d);
+    if (lds > 64u * 1024u) {
+        static bool widened = false;  // past 64 KiB of dynamic LDS a kernel has to be told once
+        if (!widened) {
+            NH_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_staged_kernel<ELEMENT, RB>), hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024));
+            widened = true;
+        }
+    }
     hipLaunchKernelGGL((gemv_staged_kernel<ELEMENT, RB>), dim3(blocks_x, p.splits), dim3(256), lds, d->stream, GEMV_LEAD(p));
     NH_HIP(hipGetLastError());
     if (p.splits > 1) {
@@ -2739,15 +2748,19 @@ int32_t launch_gemv(nh_device *d, const GemvArgs &a) {
             float *y = a.y + (size_t)done * outputs;
             const float *residual = a.residual ? a.residual + (size_t)done * a.N : nullptr;
             const bool pair = a.rows - done >= 2;
+            const bool four = a.rows - done >= 4;  // (the Q4_K_M mix at eight planes: 5.77 -> 5.46 ms a step against two rows a pass)
             int32_t status;
             if (a.element == NH_Q6_K)
-                status = pair ? launch_staged_rows<NH_Q6_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q6_K, 1>(d, a, x, y, residual);
+                status = four ? launch_staged_rows<NH_Q6_K, 4>(d, a, x, y, residual)
+                         : pair ? launch_staged_rows<NH_Q6_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q6_K, 1>(d, a, x, y, residual);
             else if (a.element == NH_Q5_K)
-                status = pair ? launch_staged_rows<NH_Q5_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q5_K, 1>(d, a, x, y, residual);
+                status = four ? launch_staged_rows<NH_Q5_K, 4>(d, a, x, y, residual)
+                         : pair ? launch_staged_rows<NH_Q5_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q5_K, 1>(d, a, x, y, residual);
             else
-                status = pair ? launch_staged_rows<NH_Q3_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q3_K, 1>(d, a, x, y, residual);
+                status = four ? launch_staged_rows<NH_Q3_K, 4>(d, a, x, y, residual)
+                         : pair ? launch_staged_rows<NH_Q3_K, 2>(d, a, x, y, residual) : launch_staged_rows<NH_Q3_K, 1>(d, a, x, y, residual);
             if (status != NH_OK) return status;
-            done += pair ? 2 : 1;
+            done += four ? 4 : (pair ? 2 : 1);
         }
         return NH_OK;
     }

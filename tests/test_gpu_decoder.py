@@ -174,7 +174,7 @@ MIXED_3 = {"output.weight": NH_Q6_K, "blk.0.attn_v.weight": NH_Q5_K, "blk.1.attn
 
 @pytest.mark.parametrize("base,mixed", [(NH_Q4_K, MIXED), (NH_Q3_K, MIXED_3), (NH_Q6_K, {}), (NH_Q5_K, {}), (NH_Q3_K, {})],
                          ids=["q4_k_m", "q3_k_m", "q6_k", "q5_k", "q3_k"])
-@pytest.mark.parametrize("batch", [1, 2])
+@pytest.mark.parametrize("batch", [1, 2, 8])
 def test_mixed_elements_and_projection_biases(device, batch, base, mixed):
     """A decoder stored the way Q4_K_M files are (Q6_K for some matrices, Q4_K for the rest) whose q, k and v projections
     carry Qwen2's biases: layer 0 (a Q6_K value projection, biases) takes one product per matrix, layer 1 (one element,
