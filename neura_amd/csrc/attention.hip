@@ -384,9 +384,14 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // CE: what the states hold (states_as_halves above); single states stage a second plane of key and value residues and cost
 // one more MFMA a product.
-template <int WIDTH, int CE = NH_F16>
-__global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, uint32_t rows_per_wave) {
+// SPLIT: two sets of four waves share the block of query rows and take every other key tile each (the walk of a long row
+// block is a chain of tiles, each a chain of MFMAs and a softmax with one wave a SIMD: two sets halve it); the two meet in
+// LDS at the end, lane by lane, as two partial softmaxes do.  Single states stage twice the planes and keep one set.
+template <int WIDTH, int CE = NH_F16, bool SPLIT = false>
+__global__ __launch_bounds__(SPLIT ? 512 : 256) void attention_tile_kernel(AttentionParams p, uint32_t rows_per_wave) {
     fetch_parameters(p);
+    static_assert(!SPLIT || CE != NH_F32, "two sets of staged tiles of single states do not fit the static LDS");
+    constexpr int SETS = SPLIT ? 2 : 1;
     constexpr int TK = 32;                       // keys per tile
     constexpr int STEPS = WIDTH / 16;            // MFMA steps over the channels of a score
     constexpr int BLOCKS = WIDTH / 32;           // 32-channel blocks of the output
@@ -395,13 +400,16 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
     constexpr int PLANES = CE == NH_F32 ? 2 : 1;  // values, and for single states their residues * 2^11
     constexpr int WORDS = CE == NH_F32 ? 2 : 1;   // 16-byte loads that hold eight stored numbers
     constexpr uint32_t STORED = CE == NH_F32 ? 4u : 2u;
-    __shared__ __attribute__((aligned(16))) uint16_t kt_planes[PLANES][TK][KPITCH];
-    __shared__ __attribute__((aligned(16))) uint16_t vt_planes[PLANES][WIDTH][VPITCH];
-    uint16_t(*const kt)[KPITCH] = kt_planes[0];
-    uint16_t(*const vt)[VPITCH] = vt_planes[0];
-    uint16_t(*const kt_fine)[KPITCH] = kt_planes[PLANES - 1];
-    uint16_t(*const vt_fine)[VPITCH] = vt_planes[PLANES - 1];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    constexpr size_t KT_BYTES = sizeof(uint16_t) * SETS * PLANES * TK * KPITCH, VT_BYTES = sizeof(uint16_t) * SETS * PLANES * WIDTH * VPITCH;
+    __shared__ __attribute__((aligned(16))) uint8_t tile_lds[KT_BYTES + VT_BYTES];  // the staged key tiles, then the value tiles
+    uint16_t(*const kt_planes)[PLANES][TK][KPITCH] = reinterpret_cast<uint16_t(*)[PLANES][TK][KPITCH]>(tile_lds);
+    uint16_t(*const vt_planes)[PLANES][WIDTH][VPITCH] = reinterpret_cast<uint16_t(*)[PLANES][WIDTH][VPITCH]>(tile_lds + KT_BYTES);
+    const uint32_t set = SPLIT ? threadIdx.x >> 8 : 0u;  // which of the two sets of waves; tid, wave: within the set
+    uint16_t(*const kt)[KPITCH] = kt_planes[set][0];
+    uint16_t(*const vt)[VPITCH] = vt_planes[set][0];
+    uint16_t(*const kt_fine)[KPITCH] = kt_planes[set][PLANES - 1];
+    uint16_t(*const vt_fine)[VPITCH] = vt_planes[set][PLANES - 1];
+    const uint32_t tid = threadIdx.x & 255u, lane = tid & 63u, wave = tid >> 6;
     const uint32_t n = lane & 31u, h = lane >> 5;
     const uint32_t G = p.groups;
     const uint32_t b = blockIdx.x % p.batch, kvh = blockIdx.x / p.batch;
@@ -462,11 +470,15 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
             }
         }
     };
-    fetch(0);
-    for (uint32_t tile = 0; tile < span; tile += TK) {
+    // set s walks tiles s, s + SETS, ...; both sets meet every barrier of every round
+    if (set * TK < span) fetch(set * TK);
+    for (uint32_t first = 0; first < span; first += SETS * TK) {
+        const uint32_t tile = first + set * TK;
+        const bool have = tile < span;
         __syncthreads();  // the last tile's readers are done
 #pragma unroll
         for (int k = 0; k < PIECES; k++) {
+            if (!have) break;
             const uint32_t piece = tid + 256u * k, key = piece / (WIDTH / 8), chunk = piece % (WIDTH / 8);
             u32x4 k_words, k_fine = {0u, 0u, 0u, 0u}, v_words, v_fine = {0u, 0u, 0u, 0u};
             states_as_halves<CE, WORDS>(kraw[k], k_words, k_fine);
@@ -488,9 +500,9 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
                 for (int i = 0; i < 8; i++) vt_fine[chunk * 8u + i][column] = (uint16_t)(words[i >> 1] >> (16 * (i & 1)));
             }
         }
-        if (tile + TK < span) fetch(tile + TK);  // in flight while this tile is multiplied
+        if (tile + SETS * TK < span) fetch(tile + SETS * TK);  // in flight while this tile is multiplied
         __syncthreads();
-        if (tile >= wave_span) continue;  // keys none of this wave's rows see (every wave still meets the barriers)
+        if (!have || tile >= wave_span) continue;  // keys none of this wave's rows see (every wave still meets the barriers)
 
         // ---- scores
         f32x16 scores, fine;
@@ -557,6 +569,36 @@ __global__ __launch_bounds__(256) void attention_tile_kernel(AttentionParams p, 
                 }
             }
         }
+    }
+    if constexpr (SPLIT) {
+        // ---- the two sets meet lane by lane: the second leaves its maximum, its mass and its sums (a 32-channel block a
+        // round) where the tiles were staged, the first joins them as two partial softmaxes join
+        static_assert(KT_BYTES + VT_BYTES >= sizeof(float) * 256 * 18, "the staged tiles' LDS holds a round of the meeting");
+        float *const meet = reinterpret_cast<float *>(tile_lds);
+        float mine = 1.0f, theirs = 0.0f;
+#pragma unroll
+        for (int d = 0; d < BLOCKS; d++) {
+            __syncthreads();  // the walk (or the round before) is done with this LDS
+            if (set == 1u) {
+                if (d == 0) meet[16 * 256 + tid] = top, meet[17 * 256 + tid] = mass;
+#pragma unroll
+                for (int r = 0; r < 16; r++) meet[r * 256 + tid] = acc[d][r];
+            }
+            __syncthreads();
+            if (set == 0u) {
+                if (d == 0) {
+                    const float other_top = meet[16 * 256 + tid], other_mass = meet[17 * 256 + tid];
+                    const float next = fmaxf(top, other_top);
+                    mine = top == -INFINITY ? 0.0f : softmax_exp(top - next);
+                    theirs = other_top == -INFINITY ? 0.0f : softmax_exp(other_top - next);
+                    mass = fmaf(mass, mine, other_mass * theirs);
+                    top = next;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[d][r] = fmaf(acc[d][r], mine, meet[r * 256 + tid] * theirs);
+            }
+        }
+        if (set == 1u) return;
     }
     if (!held) return;
     // register 4j + e of block d is channel 32d + 8j + 4h + e of this lane's column
@@ -985,9 +1027,15 @@ int32_t launch_attention(nh_device *d, const AttentionArgs &a) {
         const uint32_t rows_per_wave = 32u / p.groups;
         dim3 grid(a.kv_heads * a.batch, (a.rows + 4u * rows_per_wave - 1u) / (4u * rows_per_wave));
         p.sections = 1;
+        // two sets of waves a workgroup where the block's walk is long enough to be worth their meeting (four tiles and more);
+        // NEURA_HIP_FILL_SPLIT=0 keeps one set
+        static const bool split_wanted = [] { const char *v = getenv("NEURA_HIP_FILL_SPLIT"); return !(v && v[0] == '0'); }();
+        const bool split = split_wanted && a.cache_element != NH_F32 && a.keys >= 128u;
 #define FILL_TILE(WIDTH)                                                                                                                           \
     do {                                                                                                                                           \
-        if (a.cache_element == NH_F16) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F16>), grid, dim3(256), 0, d->stream, p, rows_per_wave);   \
+        if (a.cache_element == NH_F16 && split) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F16, true>), grid, dim3(512), 0, d->stream, p, rows_per_wave);   \
+        else if (a.cache_element == NH_BF16 && split) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_BF16, true>), grid, dim3(512), 0, d->stream, p, rows_per_wave); \
+        else if (a.cache_element == NH_F16) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F16>), grid, dim3(256), 0, d->stream, p, rows_per_wave);   \
         else if (a.cache_element == NH_BF16) hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_BF16>), grid, dim3(256), 0, d->stream, p, rows_per_wave); \
         else hipLaunchKernelGGL((attention_tile_kernel<WIDTH, NH_F32>), grid, dim3(256), 0, d->stream, p, rows_per_wave);                             \
     } while (0)
